@@ -1,0 +1,130 @@
+"""ctypes binding of libaimet_amd.so (the C ABI declared in include/aimet_amd.h).
+
+The library is the only compute path of this package: if it is missing, or a tensor does not live on a HIP device,
+the callers raise -- there is no CPU or eager-PyTorch fallback.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+from typing import Optional, Sequence
+
+import torch
+
+AHQ_MAX_DIMS = 8
+
+AHQ_OK = 0
+AHQ_F32, AHQ_F16, AHQ_BF16 = 0, 1, 2
+AHQ_ARITH_ATEN, AHQ_ARITH_AUTOGRAD, AHQ_ARITH_DLQ = 1, 2, 3
+AHQ_OP_QDQ, AHQ_OP_QUANTIZE, AHQ_OP_DEQUANTIZE = 0, 1, 2
+
+DTYPE_CODE = {torch.float32: AHQ_F32, torch.float16: AHQ_F16, torch.bfloat16: AHQ_BF16}
+
+LIB_NAME = "libaimet_amd.so"
+LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), LIB_NAME)
+
+
+class Layout(ctypes.Structure):
+    _fields_ = [
+        ("ndim", ctypes.c_int32),
+        ("dims", ctypes.c_int64 * AHQ_MAX_DIMS),
+        ("block", ctypes.c_int64 * AHQ_MAX_DIMS),
+        ("enc_stride", ctypes.c_int64 * AHQ_MAX_DIMS),
+    ]
+
+
+class Grid(ctypes.Structure):
+    _fields_ = [
+        ("arith", ctypes.c_int32),
+        ("op", ctypes.c_int32),
+        ("io_dtype", ctypes.c_int32),
+        ("compute_dtype", ctypes.c_int32),
+        ("qmin", ctypes.c_int64),
+        ("qmax", ctypes.c_int64),
+        ("zero_point_shift", ctypes.c_double),
+    ]
+
+
+class HipLibraryError(RuntimeError):
+    """Raised when libaimet_amd.so is missing or one of its entry points reports an error."""
+
+
+_lib: Optional[ctypes.CDLL] = None
+
+# name -> (restype, argtypes); every symbol include/aimet_amd.h declares
+_P = ctypes.c_void_p
+_SIGNATURES = {
+    "ahq_last_error": (ctypes.c_char_p, []),
+    "ahq_version": (ctypes.c_int, []),
+    "ahq_qdq_forward": (ctypes.c_int, [ctypes.POINTER(Grid), ctypes.POINTER(Layout), _P, _P, _P, _P, _P, _P, _P, _P]),
+    "ahq_qdq_backward_workspace_bytes": (ctypes.c_size_t, [ctypes.POINTER(Grid), ctypes.POINTER(Layout), ctypes.c_int]),
+    "ahq_qdq_backward": (ctypes.c_int, [ctypes.POINTER(Grid), ctypes.POINTER(Layout), _P, _P, _P, _P, _P, _P, _P, _P,
+                                        ctypes.c_size_t, _P]),
+    "ahq_minmax_workspace_bytes": (ctypes.c_size_t, [ctypes.POINTER(Layout)]),
+    "ahq_minmax": (ctypes.c_int, [ctypes.c_int32, ctypes.POINTER(Layout), _P, _P, _P, ctypes.c_int, ctypes.c_int, _P,
+                                  ctypes.c_size_t, _P]),
+}
+
+
+def exported_symbols() -> Sequence[str]:
+    return tuple(_SIGNATURES)
+
+
+def load() -> ctypes.CDLL:
+    """Load the shared library (once).  Raises HipLibraryError if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise HipLibraryError(
+            f"{LIB_PATH} not found: build it with `python -m aimet_amd.csrc.build` "
+            "(this package has no fallback implementation)"
+        )
+    try:
+        lib = ctypes.CDLL(LIB_PATH)
+    except OSError as e:
+        raise HipLibraryError(f"cannot load {LIB_PATH}: {e}") from e
+    for name, (res, args) in _SIGNATURES.items():
+        try:
+            fn = getattr(lib, name)
+        except AttributeError as e:
+            raise HipLibraryError(f"{LIB_PATH} does not export {name}; rebuild it") from e
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def check(status: int, where: str) -> None:
+    if status != AHQ_OK:
+        msg = load().ahq_last_error()
+        raise HipLibraryError(f"{where} failed ({status}): {msg.decode() if msg else 'unknown error'}")
+
+
+def make_layout(dims: Sequence[int], block: Sequence[int], enc_stride: Sequence[int]) -> Layout:
+    n = len(dims)
+    if n > AHQ_MAX_DIMS:
+        raise HipLibraryError(f"tensors of more than {AHQ_MAX_DIMS} dimensions are not supported (got {n})")
+    lay = Layout()
+    lay.ndim = n
+    for i in range(n):
+        lay.dims[i] = int(dims[i])
+        lay.block[i] = int(block[i])
+        lay.enc_stride[i] = int(enc_stride[i])
+    return lay
+
+
+def require_device(t: torch.Tensor, what: str) -> None:
+    if not t.is_cuda:
+        raise HipLibraryError(
+            f"{what} lives on '{t.device}': the HIP backend only runs on GPU tensors and has no CPU fallback"
+        )
+
+
+def ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def current_stream(device: torch.device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream

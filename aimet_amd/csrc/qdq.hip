@@ -1,0 +1,597 @@
+// Fake-quantization kernels: quantize-dequantize / quantize / dequantize forward and straight-through backward.
+//
+// One streaming pass per tensor: every element is read once and written once (forward: x -> y [+ 1-byte mask];
+// backward: g, x -> gx [+ per-encoding scale/offset gradients]).  Threads move 16-byte vectors; a workgroup owns a
+// tile of kTileVec vectors and first stages the encodings its tile touches in LDS, so per-channel and blockwise scales
+// are fetched from memory once per tile with one coalesced load.
+//
+// Arithmetic reproduced (see include/aimet_amd.h for the reference locations):
+//   AHQ_ARITH_ATEN      reciprocal multiply, round-half-even, clamp on the code          (fp32 math)
+//   AHQ_ARITH_AUTOGRAD  true division, round-half-even, every intermediate rounded to the compute dtype
+//   AHQ_ARITH_DLQ       clamp on the value, true division, round-half-away-from-zero     (fp32 math)
+// Built with -ffp-contract=off: fusing a multiply into an add would change the rounding of any of them.
+
+#include <atomic>
+#include <cstdio>
+
+#include "ahq_device.h"
+#include "ahq_host.h"
+#include "layout.h"
+#include "tiling.h"
+
+namespace ahq {
+
+constexpr int kStage = kTileVec + 2;  // most encodings a tile can touch
+
+struct GridC {
+    float qmin, qmax, zps;
+};
+
+struct EncP {
+    float p0, p1, p2, p3;
+};
+
+// --------------------------------------------------------------------------------------------------- arithmetic --
+// Each Math type: kNP staged floats per encoding; prep() turns (scale, offset, min, max) into them; fwd() returns the
+// output value (already rounded to the compute dtype) and whether the code was in range; bwd() returns the three
+// per-element gradient terms.
+
+template <int CD>
+struct MathAutogradQdq {
+    static constexpr int kNP = 2;
+    static constexpr bool kHasBwd = true;
+    __device__ static EncP prep(float s, float off, float, float, const GridC&) { return {rnd<CD>(s), rnd<CD>(off), 0.f, 0.f}; }
+    __device__ static float fwd(float x, const EncP& e, const GridC& g, bool& inr) {
+        float t = rnd<CD>(x / e.p0);
+        if (g.zps != 0.f) t = rnd<CD>(t - g.zps);
+        const float r = rnd<CD>(__builtin_rintf(t) - e.p1);
+        inr = (r >= g.qmin) & (r <= g.qmax);
+        const float q = r < g.qmin ? g.qmin : (r > g.qmax ? g.qmax : r);
+        const float offp = g.zps != 0.f ? rnd<CD>(e.p1 + g.zps) : e.p1;
+        return rnd<CD>(rnd<CD>(q + offp) * e.p0);
+    }
+    __device__ static void bwd(float gr, float x, const EncP& e, const GridC& g, float& gx, float& gs, float& goff) {
+        const float t = rnd<CD>(rnd<CD>(x / e.p0) - g.zps);
+        const float xr = __builtin_rintf(t);
+        const float err = rnd<CD>(xr - t);
+        const float r = rnd<CD>(xr - e.p1);
+        const bool inr = (r >= g.qmin) & (r <= g.qmax);
+        const float lo = rnd<CD>(e.p1 + g.qmin), hi = rnd<CD>(e.p1 + g.qmax);
+        float xc = xr < lo ? lo : (xr > hi ? hi : xr);
+        if (g.zps != 0.f) xc = rnd<CD>(xc + g.zps);
+        gx = inr ? gr : 0.f;
+        gs = rnd<CD>(gr * (inr ? err : xc));
+        goff = inr ? 0.f : rnd<CD>(gr * e.p0);
+    }
+};
+
+template <int CD>
+struct MathAutogradQuantize {
+    static constexpr int kNP = 2;
+    static constexpr bool kHasBwd = true;
+    __device__ static EncP prep(float s, float off, float, float, const GridC&) { return {rnd<CD>(s), rnd<CD>(off), 0.f, 0.f}; }
+    __device__ static float fwd(float x, const EncP& e, const GridC& g, bool& inr) {
+        const float r = rnd<CD>(__builtin_rintf(rnd<CD>(x / e.p0)) - e.p1);
+        inr = (r >= g.qmin) & (r <= g.qmax);
+        return r < g.qmin ? g.qmin : (r > g.qmax ? g.qmax : r);
+    }
+    __device__ static void bwd(float gr, float x, const EncP& e, const GridC& g, float& gx, float& gs, float& goff) {
+        const float xs = rnd<CD>(x / e.p0);
+        const float r = rnd<CD>(__builtin_rintf(xs) - e.p1);
+        const bool inr = (r >= g.qmin) & (r <= g.qmax);
+        const float mg = rnd<CD>(gr * (inr ? 1.f : 0.f));
+        gx = rnd<CD>(mg / e.p0);
+        gs = rnd<CD>((-gx) * xs);
+        goff = -mg;
+    }
+};
+
+template <int CD>
+struct MathAutogradDequantize {
+    static constexpr int kNP = 2;
+    static constexpr bool kHasBwd = true;
+    __device__ static EncP prep(float s, float off, float, float, const GridC&) { return {rnd<CD>(s), rnd<CD>(off), 0.f, 0.f}; }
+    __device__ static float fwd(float x, const EncP& e, const GridC&, bool& inr) {
+        inr = true;
+        return rnd<CD>(rnd<CD>(x + e.p1) * e.p0);
+    }
+    __device__ static void bwd(float gr, float x, const EncP& e, const GridC&, float& gx, float& gs, float& goff) {
+        gx = rnd<CD>(gr * e.p0);
+        gs = rnd<CD>(gr * rnd<CD>(x + e.p1));
+        goff = gx;
+    }
+};
+
+struct MathAten {
+    static constexpr int kNP = 3;
+    static constexpr bool kHasBwd = true;
+    // p0 = scale, p1 = zero point as float, p2 = 1.0f/scale
+    __device__ static EncP prep(float s, float off, float, float, const GridC&) { return {s, (float)(-(int)off), 1.0f / s, 0.f}; }
+    __device__ static float fwd(float x, const EncP& e, const GridC& g, bool& inr) {
+        const float q = __builtin_rintf(x * e.p2) + e.p1;
+        inr = (q >= g.qmin) & (q <= g.qmax);
+        const float qc = fminf(fmaxf(q, g.qmin), g.qmax);
+        return (qc - e.p1) * e.p0;
+    }
+    __device__ static void bwd(float gr, float x, const EncP& e, const GridC& g, float& gx, float& gs, float& goff) {
+        const float q = __builtin_rintf(x * e.p2) + e.p1;
+        const bool inr = (q >= g.qmin) & (q <= g.qmax);
+        gx = gr * (inr ? 1.f : 0.f);
+        gs = 0.f;
+        goff = 0.f;
+    }
+};
+
+struct MathDlq {
+    static constexpr int kNP = 4;
+    static constexpr bool kHasBwd = false;
+    // p0 = delta, p1 = offset, p2 = min, p3 = max
+    __device__ static EncP prep(float s, float off, float mn, float mx, const GridC&) { return {s, off, mn, mx}; }
+    __device__ static float fwd(float x, const EncP& e, const GridC&, bool& inr) {
+        inr = true;
+        float v = (x != x) ? e.p2 : x;
+        v = fmaxf(fminf(v, e.p3), e.p2);
+        v = v / e.p0 - e.p1;
+        v = roundf(v);
+        return e.p0 * (v + e.p1);
+    }
+    __device__ static void bwd(float, float, const EncP&, const GridC&, float& gx, float& gs, float& goff) { gx = gs = goff = 0.f; }
+};
+
+// ------------------------------------------------------------------------------------------------ kernel arguments --
+struct QdqArgs : Geom {
+    const void* x;
+    void* y;
+    uint8_t* mask;
+    const void* g;
+    void* gx;
+    const float* scale;
+    const float* offset;
+    const float* emin;
+    const float* emax;
+    float* gscale;
+    float* goffset;
+    double* partials;  // kRedTile: [nblocks][2]; kRedAtomic: [num_enc][2]
+    GridC gc;
+    int32_t red;
+    int32_t ticket;
+    int32_t out_cd;  // compute dtype the reduced gradients are rounded through
+};
+
+template <typename M>
+__device__ __forceinline__ void stage_encodings(const QdqArgs& a, const Tile& t, float (*sp)[kStage]) {
+    for (int i = threadIdx.x; i < t.nstage; i += kBlock) {
+        int64_t e = t.e0 + i;
+        if (e >= a.J) e %= a.J;
+        const float s = a.scale[e];
+        const float off = a.offset ? a.offset[e] : 0.f;
+        const float mn = a.emin ? a.emin[e] : 0.f;
+        const float mx = a.emax ? a.emax[e] : 0.f;
+        const EncP p = M::prep(s, off, mn, mx, a.gc);
+        sp[0][i] = p.p0;
+        sp[1][i] = p.p1;
+        if (M::kNP > 2) sp[2][i] = p.p2;
+        if (M::kNP > 3) sp[3][i] = p.p3;
+    }
+}
+
+template <typename M>
+__device__ __forceinline__ EncP staged(float (*sp)[kStage], int i) {
+    EncP e;
+    e.p0 = sp[0][i];
+    e.p1 = sp[1][i];
+    e.p2 = M::kNP > 2 ? sp[2][i] : 0.f;
+    e.p3 = M::kNP > 3 ? sp[3][i] : 0.f;
+    return e;
+}
+
+template <typename M>
+__device__ __forceinline__ EncP load_enc(const QdqArgs& a, int64_t e) {
+    return M::prep(a.scale[e], a.offset ? a.offset[e] : 0.f, a.emin ? a.emin[e] : 0.f, a.emax ? a.emax[e] : 0.f, a.gc);
+}
+
+// -------------------------------------------------------------------------------------------------------- forward --
+template <typename IO, int VEC, typename M>
+__global__ __launch_bounds__(kBlock) void qdq_fwd_kernel(const QdqArgs a) {
+    __shared__ float sp[M::kNP][kStage];
+    const Tile t = make_tile(a);
+    stage_encodings<M>(a, t, sp);
+    __syncthreads();
+
+    const IO* __restrict__ x = static_cast<const IO*>(a.x);
+    IO* __restrict__ y = static_cast<IO*>(a.y);
+    Pack<IO, VEC> in[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+        const int lv = u * kBlock + threadIdx.x;
+        if (lv < t.nv) in[u] = load_pack<IO, VEC>(x + (t.v0 + lv) * VEC);
+    }
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+        const int lv = u * kBlock + threadIdx.x;
+        if (lv < t.nv) {
+            const EncP e = staged<M>(sp, stage_index(a, t, lv));
+            Pack<IO, VEC> out;
+            Pack<uint8_t, VEC> mk;
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) {
+                bool inr;
+                const float r = M::fwd(load_f32(in[u].v[k]), e, a.gc, inr);
+                out.v[k] = store_cast<IO>(r);
+                mk.v[k] = inr ? 1 : 0;
+            }
+            store_pack<IO, VEC>(y + (t.v0 + lv) * VEC, out);
+            if (a.mask) store_pack<uint8_t, VEC>(a.mask + (t.v0 + lv) * VEC, mk);
+        }
+    }
+    // elements past the last full vector (only possible with a single encoding)
+    if (VEC > 1 && blockIdx.x == 0) {
+        const int64_t i = a.nvec * VEC + threadIdx.x;
+        if (i < a.numel) {
+            const EncP e = staged<M>(sp, 0);
+            bool inr;
+            const float r = M::fwd(load_f32(x[i]), e, a.gc, inr);
+            y[i] = store_cast<IO>(r);
+            if (a.mask) a.mask[i] = inr ? 1 : 0;
+        }
+    }
+}
+
+template <typename IO, typename M>
+__global__ __launch_bounds__(kBlock) void qdq_fwd_generic_kernel(const QdqArgs a) {
+    const IO* __restrict__ x = static_cast<const IO*>(a.x);
+    IO* __restrict__ y = static_cast<IO*>(a.y);
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < a.numel; i += (int64_t)gridDim.x * kBlock) {
+        const EncP e = load_enc<M>(a, generic_enc_index(a, i));
+        bool inr;
+        const float r = M::fwd(load_f32(x[i]), e, a.gc, inr);
+        y[i] = store_cast<IO>(r);
+        if (a.mask) a.mask[i] = inr ? 1 : 0;
+    }
+}
+
+// ------------------------------------------------------------------------------------------------------- backward --
+template <int CD>
+__device__ __forceinline__ float finish_sum(double s) {
+    return rnd<CD>((float)s);
+}
+__device__ __forceinline__ float finish_sum_rt(double s, int cd) {
+    if (cd == AHQ_BF16) return rnd<AHQ_BF16>((float)s);
+    if (cd == AHQ_F16) return rnd<AHQ_F16>((float)s);
+    return (float)s;
+}
+
+template <typename IO, int VEC, typename M, int RED>
+__global__ __launch_bounds__(kBlock) void qdq_bwd_kernel(const QdqArgs a) {
+    __shared__ float sp[M::kNP][kStage];
+    __shared__ double red_smem[kBlock / kWave];
+    __shared__ int flag_smem;
+    const Tile t = make_tile(a);
+    stage_encodings<M>(a, t, sp);
+    __syncthreads();
+
+    const IO* __restrict__ x = static_cast<const IO*>(a.x);
+    const IO* __restrict__ g = static_cast<const IO*>(a.g);
+    IO* __restrict__ gxp = static_cast<IO*>(a.gx);
+    Pack<IO, VEC> xin[kUnroll], gin[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+        const int lv = u * kBlock + threadIdx.x;
+        if (lv < t.nv) {
+            xin[u] = load_pack<IO, VEC>(x + (t.v0 + lv) * VEC);
+            gin[u] = load_pack<IO, VEC>(g + (t.v0 + lv) * VEC);
+        }
+    }
+    double acc_s = 0.0, acc_o = 0.0;  // kRedTile: per-thread totals
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+        const int lv = u * kBlock + threadIdx.x;
+        float vs = 0.f, vo = 0.f;
+        int si = 0;
+        if (lv < t.nv) {
+            si = stage_index(a, t, lv);
+            const EncP e = staged<M>(sp, si);
+            Pack<IO, VEC> out;
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) {
+                float gx, gs, go;
+                M::bwd(load_f32(gin[u].v[k]), load_f32(xin[u].v[k]), e, a.gc, gx, gs, go);
+                out.v[k] = store_cast<IO>(gx);
+                vs += gs;
+                vo += go;
+            }
+            if (gxp) store_pack<IO, VEC>(gxp + (t.v0 + lv) * VEC, out);
+        }
+        if (RED == kRedTile) {
+            acc_s += (double)vs;
+            acc_o += (double)vo;
+        } else if (RED == kRedSeg) {
+            // runs of Kv (power of two <= 64) neighbouring lanes share an encoding; runs never straddle a wave
+            double ds = (double)vs, dofs = (double)vo;
+            const int kv = (int)a.Kv;
+            for (int m = 1; m < kv; m <<= 1) {
+                ds += __shfl_xor(ds, m, kWave);
+                dofs += __shfl_xor(dofs, m, kWave);
+            }
+            if (lv < t.nv && (threadIdx.x & (kv - 1)) == 0) {
+                const int64_t e = t.e0 + si;
+                a.gscale[e] = finish_sum_rt(ds, a.out_cd);
+                a.goffset[e] = finish_sum_rt(dofs, a.out_cd);
+            }
+        } else if (RED == kRedAtomic) {
+            if (lv < t.nv) {
+                int64_t e = t.e0 + si;
+                if (e >= a.J) e %= a.J;
+                atomicAdd(&a.partials[2 * e], (double)vs);
+                atomicAdd(&a.partials[2 * e + 1], (double)vo);
+            }
+        }
+    }
+    if (VEC > 1 && blockIdx.x == 0) {  // tail elements, single encoding only
+        const int64_t i = a.nvec * VEC + threadIdx.x;
+        if (i < a.numel) {
+            const EncP e = staged<M>(sp, 0);
+            float gx, gs, go;
+            M::bwd(load_f32(g[i]), load_f32(x[i]), e, a.gc, gx, gs, go);
+            if (gxp) gxp[i] = store_cast<IO>(gx);
+            if (RED == kRedTile) {
+                acc_s += (double)gs;
+                acc_o += (double)go;
+            } else if (RED == kRedAtomic) {
+                atomicAdd(&a.partials[0], (double)gs);
+                atomicAdd(&a.partials[1], (double)go);
+            }
+        }
+    }
+    if (RED == kRedTile) {
+        const double bs = block_reduce(acc_s, OpAddD(), red_smem);
+        const double bo = block_reduce(acc_o, OpAddD(), red_smem);
+        // number of tiles that feed one encoding
+        const int64_t per_enc = a.mode == kRows ? a.I * (int64_t)a.tpr : (int64_t)a.nblocks;
+        if (per_enc == 1) {
+            if (threadIdx.x == 0) {
+                a.gscale[t.e0] = finish_sum_rt(bs, a.out_cd);
+                a.goffset[t.e0] = finish_sum_rt(bo, a.out_cd);
+            }
+            return;
+        }
+        if (threadIdx.x == 0) {
+            a.partials[2 * (int64_t)blockIdx.x] = bs;
+            a.partials[2 * (int64_t)blockIdx.x + 1] = bo;
+        }
+        if (!last_block_done(a.ticket, a.nblocks, &flag_smem)) return;
+        // the last workgroup adds the partials of every encoding in a fixed order
+        if (a.mode != kRows) {
+            double s = 0.0, o = 0.0;
+            for (int64_t q = threadIdx.x; q < per_enc; q += kBlock) {
+                s += a.partials[2 * q];
+                o += a.partials[2 * q + 1];
+            }
+            s = block_reduce(s, OpAddD(), red_smem);
+            o = block_reduce(o, OpAddD(), red_smem);
+            if (threadIdx.x == 0) {
+                a.gscale[0] = finish_sum_rt(s, a.out_cd);
+                a.goffset[0] = finish_sum_rt(o, a.out_cd);
+            }
+        } else {
+            // one wave per encoding, lanes stride over that encoding's tiles
+            const int lane = threadIdx.x & (kWave - 1);
+            for (int64_t j = threadIdx.x / kWave; j < a.J; j += kBlock / kWave) {
+                double s = 0.0, o = 0.0;
+                for (int64_t q = lane; q < per_enc; q += kWave) {
+                    const int64_t i = q / a.tpr, tt = q - i * a.tpr;
+                    const int64_t blk = (i * a.J + j) * a.tpr + tt;
+                    s += a.partials[2 * blk];
+                    o += a.partials[2 * blk + 1];
+                }
+                s = wave_reduce(s, OpAddD());
+                o = wave_reduce(o, OpAddD());
+                if (lane == 0) {
+                    a.gscale[j] = finish_sum_rt(s, a.out_cd);
+                    a.goffset[j] = finish_sum_rt(o, a.out_cd);
+                }
+            }
+        }
+    }
+}
+
+template <typename IO, typename M>
+__global__ __launch_bounds__(kBlock) void qdq_bwd_generic_kernel(const QdqArgs a) {
+    const IO* __restrict__ x = static_cast<const IO*>(a.x);
+    const IO* __restrict__ g = static_cast<const IO*>(a.g);
+    IO* __restrict__ gxp = static_cast<IO*>(a.gx);
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < a.numel; i += (int64_t)gridDim.x * kBlock) {
+        const int64_t ei = generic_enc_index(a, i);
+        const EncP e = load_enc<M>(a, ei);
+        float gx, gs, go;
+        M::bwd(load_f32(g[i]), load_f32(x[i]), e, a.gc, gx, gs, go);
+        if (gxp) gxp[i] = store_cast<IO>(gx);
+        if (a.partials) {
+            atomicAdd(&a.partials[2 * ei], (double)gs);
+            atomicAdd(&a.partials[2 * ei + 1], (double)go);
+        }
+    }
+}
+
+__global__ void zero_f64_kernel(double* p, int64_t n) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) p[i] = 0.0;
+}
+
+__global__ void finish_atomic_kernel(const double* acc, float* gscale, float* goffset, int64_t nenc, int cd) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < nenc; i += (int64_t)gridDim.x * blockDim.x) {
+        gscale[i] = finish_sum_rt(acc[2 * i], cd);
+        goffset[i] = finish_sum_rt(acc[2 * i + 1], cd);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------ host dispatch --
+static void fill_args(const ahq_grid& grid, const Plan& p, QdqArgs* a) {
+    fill_geom(p, a);
+    a->gc.qmin = (float)grid.qmin;
+    a->gc.qmax = (float)grid.qmax;
+    a->gc.zps = (float)grid.zero_point_shift;
+    a->red = p.red;
+    a->ticket = next_ticket();
+    a->out_cd = grid.compute_dtype;
+}
+
+static bool validate_grid(const ahq_grid* g, bool backward) {
+    if (!g) return set_error("grid is null"), false;
+    if (g->io_dtype < AHQ_F32 || g->io_dtype > AHQ_BF16) return set_error("bad io_dtype"), false;
+    if (g->compute_dtype != g->io_dtype && g->compute_dtype != AHQ_F32) return set_error("compute_dtype must equal io_dtype or be fp32"), false;
+    if (g->arith < AHQ_ARITH_ATEN || g->arith > AHQ_ARITH_DLQ) return set_error("bad arith"), false;
+    if (g->op < AHQ_OP_QDQ || g->op > AHQ_OP_DEQUANTIZE) return set_error("bad op"), false;
+    if (g->arith != AHQ_ARITH_AUTOGRAD && g->op != AHQ_OP_QDQ) return set_error("only quantize-dequantize exists for this arithmetic"), false;
+    if (g->op != AHQ_OP_DEQUANTIZE && g->qmin > g->qmax) return set_error("qmin must not exceed qmax"), false;
+    if (g->op == AHQ_OP_DEQUANTIZE && g->compute_dtype != g->io_dtype) return set_error("dequantize computes in the io dtype"), false;
+    if (g->zero_point_shift != 0.0 && g->zero_point_shift != 0.5) return set_error("zero_point_shift must be 0.0 or 0.5"), false;
+    if (g->zero_point_shift != 0.0 && (g->arith != AHQ_ARITH_AUTOGRAD || g->op != AHQ_OP_QDQ)) return set_error("zero_point_shift needs the autograd quantize-dequantize arithmetic"), false;
+    if (g->qmax - g->qmin >= (1ll << 24) || g->qmin < -(1ll << 24) || g->qmax > (1ll << 24)) return set_error("grid wider than fp32 can represent exactly"), false;
+    if (backward && g->arith == AHQ_ARITH_DLQ) return set_error("no backward exists for the DlQuantization arithmetic"), false;
+    return true;
+}
+
+// Expands to a call of F<IO, ...> for the io dtype at run time.
+#define AHQ_IO_SWITCH(dtype, CALL)                                      \
+    switch (dtype) {                                                    \
+        case AHQ_F32: { using IO = float; CALL; } break;                \
+        case AHQ_F16: { using IO = f16_t; CALL; } break;                \
+        default: { using IO = bf16_t; CALL; } break;                    \
+    }
+
+template <typename IO, typename M>
+static void launch_fwd(const Plan& p, const QdqArgs& a, hipStream_t st) {
+    if (p.cl.kind == kGeneric) {
+        hipLaunchKernelGGL((qdq_fwd_generic_kernel<IO, M>), dim3(p.nblocks), dim3(kBlock), 0, st, a);
+    } else if (p.vec == 1) {
+        hipLaunchKernelGGL((qdq_fwd_kernel<IO, 1, M>), dim3(p.nblocks), dim3(kBlock), 0, st, a);
+    } else {
+        hipLaunchKernelGGL((qdq_fwd_kernel<IO, IoTraits<IO>::kVec, M>), dim3(p.nblocks), dim3(kBlock), 0, st, a);
+    }
+}
+
+template <typename IO, typename M, int RED>
+static void launch_bwd_red(const Plan& p, const QdqArgs& a, hipStream_t st) {
+    if (p.vec == 1) {
+        hipLaunchKernelGGL((qdq_bwd_kernel<IO, 1, M, RED>), dim3(p.nblocks), dim3(kBlock), 0, st, a);
+    } else {
+        hipLaunchKernelGGL((qdq_bwd_kernel<IO, IoTraits<IO>::kVec, M, RED>), dim3(p.nblocks), dim3(kBlock), 0, st, a);
+    }
+}
+
+template <typename IO, typename M>
+static void launch_bwd(const Plan& p, const QdqArgs& a, hipStream_t st) {
+    if (p.cl.kind == kGeneric) {
+        hipLaunchKernelGGL((qdq_bwd_generic_kernel<IO, M>), dim3(p.nblocks), dim3(kBlock), 0, st, a);
+        return;
+    }
+    switch (p.red) {
+        case kRedNone: launch_bwd_red<IO, M, kRedNone>(p, a, st); break;
+        case kRedTile: launch_bwd_red<IO, M, kRedTile>(p, a, st); break;
+        case kRedSeg: launch_bwd_red<IO, M, kRedSeg>(p, a, st); break;
+        default: launch_bwd_red<IO, M, kRedAtomic>(p, a, st); break;
+    }
+}
+
+// Calls F with the Math type selected by (arith, op, compute dtype).
+#define AHQ_MATH_SWITCH(grid, CALL)                                                                  \
+    do {                                                                                             \
+        if ((grid).arith == AHQ_ARITH_ATEN) { using M = MathAten; CALL; }                            \
+        else if ((grid).arith == AHQ_ARITH_DLQ) { using M = MathDlq; CALL; }                         \
+        else if ((grid).op == AHQ_OP_QDQ) {                                                          \
+            if ((grid).compute_dtype == AHQ_F32) { using M = MathAutogradQdq<AHQ_F32>; CALL; }       \
+            else if ((grid).compute_dtype == AHQ_F16) { using M = MathAutogradQdq<AHQ_F16>; CALL; }  \
+            else { using M = MathAutogradQdq<AHQ_BF16>; CALL; }                                      \
+        } else if ((grid).op == AHQ_OP_QUANTIZE) {                                                   \
+            if ((grid).compute_dtype == AHQ_F32) { using M = MathAutogradQuantize<AHQ_F32>; CALL; }  \
+            else if ((grid).compute_dtype == AHQ_F16) { using M = MathAutogradQuantize<AHQ_F16>; CALL; } \
+            else { using M = MathAutogradQuantize<AHQ_BF16>; CALL; }                                 \
+        } else {                                                                                     \
+            if ((grid).compute_dtype == AHQ_F32) { using M = MathAutogradDequantize<AHQ_F32>; CALL; } \
+            else if ((grid).compute_dtype == AHQ_F16) { using M = MathAutogradDequantize<AHQ_F16>; CALL; } \
+            else { using M = MathAutogradDequantize<AHQ_BF16>; CALL; }                               \
+        }                                                                                            \
+    } while (0)
+
+}  // namespace ahq
+
+using namespace ahq;
+
+extern "C" int ahq_qdq_forward(const ahq_grid* grid, const ahq_layout* layout, const void* x, void* y, uint8_t* mask_out,
+                               const float* scale, const float* offset, const float* enc_min, const float* enc_max,
+                               void* stream) {
+    if (!validate_grid(grid, false)) return AHQ_ERR_INVALID;
+    if (!layout) return set_error("layout is null"), AHQ_ERR_INVALID;
+    if (!scale) return set_error("scale is null"), AHQ_ERR_INVALID;
+    if (grid->arith == AHQ_ARITH_DLQ && (!enc_min || !enc_max || !offset)) return set_error("DlQuantization arithmetic needs offset, enc_min and enc_max"), AHQ_ERR_INVALID;
+    if (grid->arith != AHQ_ARITH_DLQ && (enc_min || enc_max)) return set_error("enc_min/enc_max only apply to the DlQuantization arithmetic"), AHQ_ERR_INVALID;
+    Plan p;
+    const bool al = aligned16(x) && aligned16(y) && (!mask_out || (reinterpret_cast<uintptr_t>(mask_out) & 7u) == 0);
+    if (!make_plan(grid->io_dtype, *layout, al, false, &p)) return AHQ_ERR_INVALID;
+    if (p.cl.numel == 0) return AHQ_OK;
+    if (!x || !y) return set_error("x or y is null"), AHQ_ERR_INVALID;
+    QdqArgs a{};
+    a.x = x;
+    a.y = y;
+    a.mask = mask_out;
+    a.scale = scale;
+    a.offset = offset;
+    a.emin = enc_min;
+    a.emax = enc_max;
+    fill_args(*grid, p, &a);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    AHQ_IO_SWITCH(grid->io_dtype, AHQ_MATH_SWITCH(*grid, (launch_fwd<IO, M>(p, a, st))));
+    return check_launch("ahq_qdq_forward");
+}
+
+extern "C" size_t ahq_qdq_backward_workspace_bytes(const ahq_grid* grid, const ahq_layout* layout, int want_param_grads) {
+    if (!grid || !layout) return 0;
+    Plan p;
+    if (!make_plan(grid->io_dtype, *layout, true, want_param_grads != 0, &p)) return 0;
+    size_t a = p.ws_elems * 2 * sizeof(double);
+    // an unaligned tensor falls back to the scalar path whose strategy may need a different amount
+    Plan q;
+    if (make_plan(grid->io_dtype, *layout, false, want_param_grads != 0, &q) && q.ws_elems * 2 * sizeof(double) > a) a = q.ws_elems * 2 * sizeof(double);
+    return a;
+}
+
+extern "C" int ahq_qdq_backward(const ahq_grid* grid, const ahq_layout* layout, const void* g, const void* x, void* gx,
+                                float* gscale, float* goffset, const float* scale, const float* offset, void* workspace,
+                                size_t workspace_bytes, void* stream) {
+    if (!validate_grid(grid, true)) return AHQ_ERR_INVALID;
+    if (!layout) return set_error("layout is null"), AHQ_ERR_INVALID;
+    if (!scale) return set_error("scale is null"), AHQ_ERR_INVALID;
+    if ((gscale == nullptr) != (goffset == nullptr)) return set_error("gscale and goffset must be given together"), AHQ_ERR_INVALID;
+    const bool want_pg = gscale != nullptr;
+    if (want_pg && grid->arith == AHQ_ARITH_ATEN) return set_error("the ATen arithmetic has no scale/offset gradient"), AHQ_ERR_INVALID;
+    Plan p;
+    const bool al = aligned16(x) && aligned16(g) && (!gx || aligned16(gx));
+    if (!make_plan(grid->io_dtype, *layout, al, want_pg, &p)) return AHQ_ERR_INVALID;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (p.cl.numel == 0) return AHQ_OK;  // nothing to read: outputs are left untouched
+    if (!x || !g) return set_error("x or g is null"), AHQ_ERR_INVALID;
+    if (!gx && !want_pg) return AHQ_OK;
+    const size_t ws_need = p.ws_elems * 2 * sizeof(double);
+    if (ws_need > 0 && (!workspace || workspace_bytes < ws_need)) return set_error("workspace too small"), AHQ_ERR_WORKSPACE;
+    QdqArgs a{};
+    a.x = x;
+    a.g = g;
+    a.gx = gx;
+    a.scale = scale;
+    a.offset = offset;
+    a.gscale = gscale;
+    a.goffset = goffset;
+    a.partials = ws_need ? static_cast<double*>(workspace) : nullptr;
+    fill_args(*grid, p, &a);
+    if (p.red == kRedAtomic) {
+        const int64_t n = p.cl.num_enc * 2;
+        hipLaunchKernelGGL(zero_f64_kernel, dim3((unsigned)((n + 255) / 256 > 1024 ? 1024 : (n + 255) / 256)), dim3(256), 0, st, a.partials, n);
+    }
+    AHQ_IO_SWITCH(grid->io_dtype, AHQ_MATH_SWITCH(*grid, (launch_bwd<IO, M>(p, a, st))));
+    if (p.red == kRedAtomic) {
+        const int64_t n = p.cl.num_enc;
+        hipLaunchKernelGGL(finish_atomic_kernel, dim3((unsigned)((n + 255) / 256 > 1024 ? 1024 : (n + 255) / 256)), dim3(256), 0, st,
+                           (const double*)a.partials, gscale, goffset, n, (int)grid->compute_dtype);
+    }
+    return check_launch("ahq_qdq_backward");
+}

@@ -1,0 +1,287 @@
+// Minimum / maximum statistics in one pass over the tensor (both extrema from the same read).
+//
+// Per-lane running min/max over 16-byte vectors -> wave64 shuffle tree -> LDS across the four waves of a workgroup ->
+// per-tile partials that the last workgroup to finish folds together, so a calibration call is a single launch.
+// NaN handling follows torch.amin/amax (any NaN in a slice makes that slice's result NaN) unless `finite_only`, which
+// reproduces the histogram observer's range (non-finite values ignored).
+
+#include "ahq_device.h"
+#include "ahq_host.h"
+#include "layout.h"
+#include "tiling.h"
+
+namespace ahq {
+
+struct MmArgs : Geom {
+    const void* x;
+    void* out_min;
+    void* out_max;
+    float* part_min;      // kRedTile: [nblocks]
+    float* part_max;
+    int* part_nan;
+    unsigned int* key_min;  // kRedAtomic: [num_enc] order-preserving keys
+    unsigned int* key_max;
+    int32_t red;
+    int32_t ticket;
+    int32_t finite_only;
+    int32_t running;
+};
+
+struct MinMax {
+    float mn, mx;
+    int nan;
+};
+
+__device__ __forceinline__ MinMax mm_identity() { return {__builtin_inff(), -__builtin_inff(), 0}; }
+
+__device__ __forceinline__ void mm_add(MinMax& m, float v, bool finite_only) {
+    if (finite_only) {
+        const bool fin = __builtin_fabsf(v) < __builtin_inff();
+        m.mn = fminf(m.mn, fin ? v : __builtin_inff());
+        m.mx = fmaxf(m.mx, fin ? v : -__builtin_inff());
+    } else {
+        m.nan |= (v != v) ? 1 : 0;
+        m.mn = fminf(m.mn, v);
+        m.mx = fmaxf(m.mx, v);
+    }
+}
+
+__device__ __forceinline__ MinMax mm_merge(const MinMax& a, const MinMax& b) {
+    return {fminf(a.mn, b.mn), fmaxf(a.mx, b.mx), a.nan | b.nan};
+}
+
+__device__ __forceinline__ MinMax mm_shfl_xor(const MinMax& a, int m) {
+    return {__shfl_xor(a.mn, m, kWave), __shfl_xor(a.mx, m, kWave), __shfl_xor(a.nan, m, kWave)};
+}
+
+__device__ __forceinline__ MinMax mm_block_reduce(MinMax v, MinMax* smem) {
+#pragma unroll
+    for (int m = kWave / 2; m >= 1; m >>= 1) v = mm_merge(v, mm_shfl_xor(v, m));
+    __syncthreads();
+    if ((threadIdx.x & (kWave - 1)) == 0) smem[threadIdx.x / kWave] = v;
+    __syncthreads();
+    MinMax r = smem[0];
+#pragma unroll
+    for (int w = 1; w < kBlock / kWave; ++w) r = mm_merge(r, smem[w]);
+    return r;
+}
+
+template <typename IO>
+__device__ __forceinline__ void mm_write(const MmArgs& a, int64_t e, MinMax m) {
+    IO* omn = static_cast<IO*>(a.out_min);
+    IO* omx = static_cast<IO*>(a.out_max);
+    const float qnan = __builtin_nanf("");
+    float mn = m.nan ? qnan : m.mn;
+    float mx = m.nan ? qnan : m.mx;
+    if (a.running) {
+        // torch.minimum / torch.maximum: NaN in either operand wins
+        const float pmn = load_f32(omn[e]), pmx = load_f32(omx[e]);
+        mn = (pmn != pmn || mn != mn) ? qnan : fminf(pmn, mn);
+        mx = (pmx != pmx || mx != mx) ? qnan : fmaxf(pmx, mx);
+    }
+    omn[e] = store_cast<IO>(mn);
+    omx[e] = store_cast<IO>(mx);
+}
+
+__device__ __forceinline__ unsigned int f32_key(float f) {
+    const unsigned int b = f32_to_bits(f);
+    return b ^ ((b >> 31) ? 0xffffffffu : 0x80000000u);
+}
+__device__ __forceinline__ float key_f32(unsigned int k) {
+    return bits_to_f32(k ^ ((k >> 31) ? 0x80000000u : 0xffffffffu));
+}
+
+template <typename IO, int VEC, int RED>
+__global__ __launch_bounds__(kBlock) void minmax_kernel(const MmArgs a) {
+    __shared__ MinMax red_smem[kBlock / kWave];
+    __shared__ int flag_smem;
+    const Tile t = make_tile(a);
+    const IO* __restrict__ x = static_cast<const IO*>(a.x);
+    const bool fo = a.finite_only != 0;
+
+    Pack<IO, VEC> in[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+        const int lv = u * kBlock + threadIdx.x;
+        if (lv < t.nv) in[u] = load_pack<IO, VEC>(x + (t.v0 + lv) * VEC);
+    }
+    MinMax acc = mm_identity();
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+        const int lv = u * kBlock + threadIdx.x;
+        MinMax v = mm_identity();
+        int si = 0;
+        if (lv < t.nv) {
+            si = stage_index(a, t, lv);
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) mm_add(v, load_f32(in[u].v[k]), fo);
+        }
+        if (RED == kRedTile) {
+            acc = mm_merge(acc, v);
+        } else if (RED == kRedSeg) {
+            const int kv = (int)a.Kv;
+            for (int m = 1; m < kv; m <<= 1) v = mm_merge(v, mm_shfl_xor(v, m));
+            if (lv < t.nv && (threadIdx.x & (kv - 1)) == 0) mm_write<IO>(a, t.e0 + si, v);
+        } else if (RED == kRedAtomic) {
+            if (lv < t.nv) {
+                int64_t e = t.e0 + si;
+                if (e >= a.J) e %= a.J;
+                atomicMin(&a.key_min[e], f32_key(v.mn));
+                atomicMax(&a.key_max[e], f32_key(v.mx));
+                if (v.nan) atomicOr(&a.part_nan[e], 1);
+            }
+        }
+    }
+    if (VEC > 1 && blockIdx.x == 0) {  // elements past the last full vector (single encoding only)
+        const int64_t i = a.nvec * VEC + threadIdx.x;
+        if (i < a.numel) {
+            MinMax v = mm_identity();
+            mm_add(v, load_f32(x[i]), fo);
+            if (RED == kRedTile) acc = mm_merge(acc, v);
+            if (RED == kRedAtomic) {
+                atomicMin(&a.key_min[0], f32_key(v.mn));
+                atomicMax(&a.key_max[0], f32_key(v.mx));
+                if (v.nan) atomicOr(&a.part_nan[0], 1);
+            }
+        }
+    }
+    if (RED == kRedTile) {
+        const MinMax b = mm_block_reduce(acc, red_smem);
+        const int64_t per_enc = a.mode == kRows ? a.I * (int64_t)a.tpr : (int64_t)a.nblocks;
+        if (per_enc == 1) {
+            if (threadIdx.x == 0) mm_write<IO>(a, t.e0, b);
+            return;
+        }
+        if (threadIdx.x == 0) {
+            a.part_min[blockIdx.x] = b.mn;
+            a.part_max[blockIdx.x] = b.mx;
+            a.part_nan[blockIdx.x] = b.nan;
+        }
+        if (!last_block_done(a.ticket, a.nblocks, &flag_smem)) return;
+        if (a.mode != kRows) {
+            MinMax s = mm_identity();
+            for (int64_t q = threadIdx.x; q < per_enc; q += kBlock) s = mm_merge(s, MinMax{a.part_min[q], a.part_max[q], a.part_nan[q]});
+            s = mm_block_reduce(s, red_smem);
+            if (threadIdx.x == 0) mm_write<IO>(a, 0, s);
+        } else {
+            const int lane = threadIdx.x & (kWave - 1);
+            for (int64_t j = threadIdx.x / kWave; j < a.J; j += kBlock / kWave) {
+                MinMax s = mm_identity();
+                for (int64_t q = lane; q < per_enc; q += kWave) {
+                    const int64_t i = q / a.tpr, tt = q - i * a.tpr;
+                    const int64_t blk = (i * a.J + j) * a.tpr + tt;
+                    s = mm_merge(s, MinMax{a.part_min[blk], a.part_max[blk], a.part_nan[blk]});
+                }
+#pragma unroll
+                for (int m = kWave / 2; m >= 1; m >>= 1) s = mm_merge(s, mm_shfl_xor(s, m));
+                if (lane == 0) mm_write<IO>(a, j, s);
+            }
+        }
+    }
+}
+
+template <typename IO>
+__global__ __launch_bounds__(kBlock) void minmax_generic_kernel(const MmArgs a) {
+    const IO* __restrict__ x = static_cast<const IO*>(a.x);
+    const bool fo = a.finite_only != 0;
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < a.numel; i += (int64_t)gridDim.x * kBlock) {
+        const int64_t e = generic_enc_index(a, i);
+        MinMax v = mm_identity();
+        mm_add(v, load_f32(x[i]), fo);
+        atomicMin(&a.key_min[e], f32_key(v.mn));
+        atomicMax(&a.key_max[e], f32_key(v.mx));
+        if (v.nan) atomicOr(&a.part_nan[e], 1);
+    }
+}
+
+__global__ void minmax_keys_init_kernel(unsigned int* kmn, unsigned int* kmx, int* nan, int64_t n) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+        kmn[i] = 0xff800000u;  // key of +inf
+        kmx[i] = 0x007fffffu;  // key of -inf
+        nan[i] = 0;
+    }
+}
+
+template <typename IO>
+__global__ void minmax_keys_finish_kernel(const MmArgs a, int64_t n) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+        mm_write<IO>(a, i, MinMax{key_f32(a.key_min[i]), key_f32(a.key_max[i]), a.part_nan[i]});
+}
+
+template <typename IO, int RED>
+static void launch_mm_red(const Plan& p, const MmArgs& a, hipStream_t st) {
+    if (p.vec == 1) hipLaunchKernelGGL((minmax_kernel<IO, 1, RED>), dim3(p.nblocks), dim3(kBlock), 0, st, a);
+    else hipLaunchKernelGGL((minmax_kernel<IO, IoTraits<IO>::kVec, RED>), dim3(p.nblocks), dim3(kBlock), 0, st, a);
+}
+
+template <typename IO>
+static void launch_mm(const Plan& p, const MmArgs& a, hipStream_t st) {
+    const int64_t ne = p.cl.num_enc;
+    const unsigned gb = (unsigned)((ne + 255) / 256 > 1024 ? 1024 : (ne + 255) / 256);
+    if (p.red == kRedAtomic) hipLaunchKernelGGL(minmax_keys_init_kernel, dim3(gb), dim3(256), 0, st, a.key_min, a.key_max, a.part_nan, ne);
+    if (p.cl.kind == kGeneric) {
+        hipLaunchKernelGGL((minmax_generic_kernel<IO>), dim3(p.nblocks), dim3(kBlock), 0, st, a);
+    } else if (p.red == kRedTile) {
+        launch_mm_red<IO, kRedTile>(p, a, st);
+    } else if (p.red == kRedSeg) {
+        launch_mm_red<IO, kRedSeg>(p, a, st);
+    } else {
+        launch_mm_red<IO, kRedAtomic>(p, a, st);
+    }
+    if (p.red == kRedAtomic) hipLaunchKernelGGL((minmax_keys_finish_kernel<IO>), dim3(gb), dim3(256), 0, st, a, ne);
+}
+
+}  // namespace ahq
+
+using namespace ahq;
+
+extern "C" size_t ahq_minmax_workspace_bytes(const ahq_layout* layout) {
+    if (!layout) return 0;
+    // the widest plan over dtypes and alignments decides; 12 bytes per tile or per encoding
+    size_t need = 0;
+    for (int dt = AHQ_F32; dt <= AHQ_BF16; ++dt)
+        for (int al = 0; al < 2; ++al) {
+            Plan p;
+            if (make_plan(dt, *layout, al != 0, true, &p) && p.ws_elems * 12 > need) need = p.ws_elems * 12;
+        }
+    return need;
+}
+
+extern "C" int ahq_minmax(int32_t dtype, const ahq_layout* layout, const void* x, void* out_min, void* out_max,
+                          int finite_only, int running, void* workspace, size_t workspace_bytes, void* stream) {
+    if (dtype < AHQ_F32 || dtype > AHQ_BF16) return set_error("bad dtype"), AHQ_ERR_INVALID;
+    if (!layout) return set_error("layout is null"), AHQ_ERR_INVALID;
+    if (!out_min || !out_max) return set_error("out_min or out_max is null"), AHQ_ERR_INVALID;
+    Plan p;
+    if (!make_plan(dtype, *layout, aligned16(x), true, &p)) return AHQ_ERR_INVALID;
+    if (p.cl.numel == 0) return set_error("cannot reduce an empty tensor"), AHQ_ERR_INVALID;
+    if (!x) return set_error("x is null"), AHQ_ERR_INVALID;
+    const size_t need = p.ws_elems * 12;
+    const int64_t per_enc = p.red == kRedTile ? (p.mode == kRows ? p.cl.I * (int64_t)p.tpr : (int64_t)p.nblocks) : 0;
+    const bool uses_ws = p.red == kRedAtomic || (p.red == kRedTile && per_enc > 1);
+    if (uses_ws && (!workspace || workspace_bytes < need)) return set_error("workspace too small"), AHQ_ERR_WORKSPACE;
+    MmArgs a{};
+    fill_geom(p, &a);
+    a.x = x;
+    a.out_min = out_min;
+    a.out_max = out_max;
+    a.red = p.red;
+    a.ticket = next_ticket();
+    a.finite_only = finite_only;
+    a.running = running;
+    if (uses_ws) {
+        char* w = static_cast<char*>(workspace);
+        a.part_min = reinterpret_cast<float*>(w);
+        a.part_max = reinterpret_cast<float*>(w + p.ws_elems * 4);
+        a.part_nan = reinterpret_cast<int*>(w + p.ws_elems * 8);
+        a.key_min = reinterpret_cast<unsigned int*>(w);
+        a.key_max = reinterpret_cast<unsigned int*>(w + p.ws_elems * 4);
+    }
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    switch (dtype) {
+        case AHQ_F32: launch_mm<float>(p, a, st); break;
+        case AHQ_F16: launch_mm<f16_t>(p, a, st); break;
+        default: launch_mm<bf16_t>(p, a, st); break;
+    }
+    return check_launch("ahq_minmax");
+}

@@ -1,0 +1,189 @@
+// How a flat tensor is cut into workgroup tiles and how a tile finds the encodings it touches.
+// Shared by the fake-quantization kernels and the statistics kernels.
+#pragma once
+
+#include <atomic>
+
+#include "ahq_device.h"
+#include "ahq_host.h"
+#include "layout.h"
+
+namespace ahq {
+
+enum TileMode : int { kFlat = 0, kRows = 1 };
+// How per-encoding reductions leave the kernel:
+//   kRedTile    every tile lies inside one run; workgroup totals go to a partials array (or straight to the output
+//               when one tile covers the whole encoding) and the last workgroup adds them in a fixed order
+//   kRedSeg     a run is a power-of-two number (<= 64) of neighbouring lanes: shuffle reduction, direct store
+//   kRedAtomic  anything else: atomics into a per-encoding scratch array, finished by a second tiny kernel
+enum RedMode : int { kRedNone = 0, kRedTile = 1, kRedSeg = 2, kRedAtomic = 3 };
+
+// Geometry every tiled kernel receives (flat index = (i*J + j)*K + k, encoding index = j).
+struct Geom {
+    int64_t numel;
+    int64_t nvec;  // numel / VEC
+    int64_t I, J, K;
+    int64_t Kv;    // vectors per run of one encoding (K / VEC); 2^62 when J == 1
+    int32_t mode;
+    int32_t tpr;   // tiles per row (kRows)
+    uint32_t nblocks;
+    // generic layout (per-element coordinate walk)
+    int32_t nseg;
+    int64_t seg_extent[2 * AHQ_MAX_DIMS];
+    int64_t seg_flat_stride[2 * AHQ_MAX_DIMS];
+    int64_t seg_enc_stride[2 * AHQ_MAX_DIMS];
+};
+
+struct Tile {
+    int64_t v0;    // first vector of the tile
+    int nv;        // vectors in the tile
+    int64_t rem0;  // position of v0 inside its run, in vectors
+    int64_t e0;    // encoding index of the first run
+    int nstage;    // runs touched
+};
+
+__device__ __forceinline__ Tile make_tile(const Geom& a) {
+    Tile t;
+    if (a.mode == kRows) {
+        const int64_t row = blockIdx.x / (uint32_t)a.tpr;
+        const int64_t tt = blockIdx.x - row * a.tpr;
+        t.v0 = row * a.Kv + tt * kTileVec;
+        const int64_t left = a.Kv - tt * kTileVec;
+        t.nv = (int)(left < kTileVec ? left : kTileVec);
+        t.rem0 = tt * kTileVec;
+        t.e0 = a.I == 1 ? row : row % a.J;
+        t.nstage = 1;
+    } else {
+        t.v0 = (int64_t)blockIdx.x * kTileVec;
+        const int64_t left = a.nvec - t.v0;
+        t.nv = (int)(left < kTileVec ? left : kTileVec);
+        if (t.nv < 0) t.nv = 0;
+        if (a.J == 1) {
+            t.rem0 = 0;
+            t.e0 = 0;
+            t.nstage = 1;
+        } else {
+            const int64_t row0 = t.v0 / a.Kv;
+            t.rem0 = t.v0 - row0 * a.Kv;
+            t.e0 = a.I == 1 ? row0 : row0 % a.J;
+            t.nstage = t.nv > 0 ? (int)((t.rem0 + t.nv - 1) / a.Kv) + 1 : 0;
+        }
+    }
+    return t;
+}
+
+// index of local vector lv's run among the runs the tile touches
+__device__ __forceinline__ int stage_index(const Geom& a, const Tile& t, int lv) {
+    if (t.nstage == 1) return 0;
+    const int64_t p = t.rem0 + lv;
+    if (a.Kv >= kTileVec) return p >= a.Kv ? 1 : 0;
+    return (int)((uint32_t)p / (uint32_t)a.Kv);
+}
+
+__device__ __forceinline__ int64_t generic_enc_index(const Geom& a, int64_t idx) {
+    int64_t e = 0;
+    for (int s = 0; s < a.nseg; ++s) {
+        const int64_t c = (idx / a.seg_flat_stride[s]) % a.seg_extent[s];
+        e += c * a.seg_enc_stride[s];
+    }
+    return e;
+}
+
+// ------------------------------------------------------------------------------------------------------ host side --
+struct Plan {
+    CanonLayout cl;
+    int vec;       // element vector width used (16 bytes worth, or 1)
+    int mode;
+    int tpr;
+    int red;
+    uint32_t nblocks;
+    int64_t Kv, nvec;
+    size_t ws_elems;  // kRedTile: number of tiles; kRedAtomic: number of encodings; else 0
+};
+
+inline int io_vec(int dtype) { return dtype == AHQ_F32 ? 4 : 8; }
+inline size_t io_size(int dtype) { return dtype == AHQ_F32 ? 4 : 2; }
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+inline bool is_pow2(int64_t v) { return v > 0 && (v & (v - 1)) == 0; }
+
+inline int next_ticket() {
+    static std::atomic<unsigned> rr{0};
+    return (int)(rr.fetch_add(1) % kTicketSlots);
+}
+
+// Decide tiling and reduction strategy.  `ptr_aligned`: every tensor pointer is 16-byte aligned.
+inline bool make_plan(int io_dtype, const ahq_layout& layout, bool ptr_aligned, bool want_red, Plan* p) {
+    const char* err = nullptr;
+    if (!canonicalize(layout, &p->cl, &err)) {
+        set_error(err);
+        return false;
+    }
+    const CanonLayout& c = p->cl;
+    p->mode = kFlat;
+    p->tpr = 0;
+    p->red = kRedNone;
+    p->ws_elems = 0;
+    if (c.kind == kGeneric) {
+        p->vec = 1;
+        p->Kv = 1;
+        p->nvec = c.numel;
+        int64_t nb = (c.numel + kBlock - 1) / kBlock;
+        if (nb > 65536) nb = 65536;
+        p->nblocks = (uint32_t)(nb < 1 ? 1 : nb);
+        if (want_red) {
+            p->red = kRedAtomic;
+            p->ws_elems = (size_t)c.num_enc;
+        }
+        return true;
+    }
+    const int V = io_vec(io_dtype);
+    const bool shared = ptr_aligned && (c.J == 1 || c.K % V == 0);
+    p->vec = shared ? V : 1;
+    p->nvec = c.numel / p->vec;
+    p->Kv = c.J == 1 ? ((int64_t)1 << 62) : c.K / p->vec;
+    int64_t nb = (p->nvec + kTileVec - 1) / kTileVec;
+    if (want_red) {
+        if (c.J == 1) {
+            p->red = kRedTile;
+        } else if (c.I == 1 && is_pow2(p->Kv) && p->Kv <= kWave) {
+            p->red = kRedSeg;
+        } else if (p->Kv >= kTileVec / 2) {
+            p->red = kRedTile;
+            p->mode = kRows;
+            p->tpr = (int)((p->Kv + kTileVec - 1) / kTileVec);
+            nb = c.I * c.J * (int64_t)p->tpr;
+        } else {
+            p->red = kRedAtomic;
+        }
+        if (p->red == kRedTile) p->ws_elems = (size_t)(nb < 1 ? 1 : nb);
+        if (p->red == kRedAtomic) p->ws_elems = (size_t)c.num_enc;
+    }
+    if (nb < 1) nb = 1;
+    if (nb > 0x7fffffff) {
+        set_error("tensor too large for one launch");
+        return false;
+    }
+    p->nblocks = (uint32_t)nb;
+    return true;
+}
+
+inline void fill_geom(const Plan& p, Geom* g) {
+    const CanonLayout& c = p.cl;
+    g->numel = c.numel;
+    g->nvec = p.nvec;
+    g->I = c.I;
+    g->J = c.J;
+    g->K = c.K;
+    g->Kv = p.Kv;
+    g->mode = p.mode;
+    g->tpr = p.tpr;
+    g->nblocks = p.nblocks;
+    g->nseg = c.kind == kGeneric ? c.nseg : 0;
+    for (int i = 0; i < g->nseg; ++i) {
+        g->seg_extent[i] = c.seg_extent[i];
+        g->seg_flat_stride[i] = c.seg_flat_stride[i];
+        g->seg_enc_stride[i] = c.seg_enc_stride[i];
+    }
+}
+
+}  // namespace ahq

@@ -1,0 +1,62 @@
+"""Thin Python wrappers over the statistics entry points of libaimet_amd.so."""
+
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+
+from aimet_amd import _lib
+from aimet_amd._lib import HipLibraryError
+from aimet_amd.quantization._utils import _is_expandable
+from aimet_amd.quantization.affine.backends.hip import _prepare
+
+
+def _check_reducible(x: torch.Tensor, shape: Tuple[int, ...], block_size) -> None:
+    if block_size is not None:
+        if len(block_size) != len(shape):
+            raise RuntimeError(f"Length of shape {shape} must equal length of block size {block_size}")
+        if x.dim() < len(shape):
+            raise RuntimeError(f"Input of shape {list(x.shape)} can't be reduced to shape {list(shape)}")
+        for i in range(1, len(shape) + 1):
+            b, s, d = block_size[-i], shape[-i], x.shape[-i]
+            ok = (d % s == 0) if b == -1 else (b * s == d)
+            if not ok:
+                raise RuntimeError(f"Input of shape {list(x.shape)} can't be reduced to shape {list(shape)}")
+    elif not _is_expandable(shape, x.shape):
+        raise RuntimeError(f"Input of shape {list(x.shape)} can't be reduced to shape {list(shape)}")
+
+
+def reduce_min_max(x: torch.Tensor, shape: Tuple[int, ...], block_size=None, *, finite_only: bool = False,
+                   running: Optional[Tuple[torch.Tensor, torch.Tensor]] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Per-encoding minimum and maximum of ``x`` in one pass (both extrema from a single read of the tensor).
+
+    Equivalent of ``reduce(x, shape, torch.amin, block_size)`` and ``reduce(x, shape, torch.amax, block_size)``
+    (aimet_torch/utils.py:1115-1148, aimet_torch/quantization/encoding_analyzer.py:80-94).  With ``running`` the
+    results are folded into the given (min, max) tensors in place, as ``_MinMaxObserver.merge_stats`` does.
+    """
+    _lib.require_device(x, "input tensor")
+    if x.dtype not in _lib.DTYPE_CODE:
+        raise HipLibraryError(f"min/max statistics support float32, float16 and bfloat16; got {x.dtype}")
+    shape = tuple(shape)
+    _check_reducible(x, shape, block_size)
+    if x.numel() == 0:
+        raise RuntimeError("cannot reduce an empty tensor")
+    lib = _lib.load()
+    xd, layout = _prepare(x.detach(), shape, block_size)
+    if running is not None:
+        mn, mx = running
+        if mn.dtype != x.dtype or not mn.is_contiguous() or not mx.is_contiguous() or tuple(mn.shape) != shape:
+            raise RuntimeError("running statistics must be contiguous tensors of the observer shape and input dtype")
+    else:
+        mn = torch.empty(shape, dtype=x.dtype, device=x.device)
+        mx = torch.empty(shape, dtype=x.dtype, device=x.device)
+    nbytes = lib.ahq_minmax_workspace_bytes(layout)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device) if nbytes else None
+    _lib.check(
+        lib.ahq_minmax(_lib.DTYPE_CODE[x.dtype], layout, xd.data_ptr(), mn.data_ptr(), mx.data_ptr(),
+                       1 if finite_only else 0, 1 if running is not None else 0, _lib.ptr(ws), nbytes,
+                       _lib.current_stream(x.device)),
+        "ahq_minmax",
+    )
+    return mn, mx

@@ -1,0 +1,128 @@
+/*
+ * aimet_amd.h -- C ABI of libaimet_amd.so: MI355X (gfx950) kernels for AIMET's quantization-simulation hot path.
+ *
+ * Conventions
+ *   - every tensor pointer is a DEVICE pointer; tensors are dense and contiguous in the dimension order given
+ *   - every function enqueues work on `stream` (a hipStream_t passed as void*) and returns without synchronising
+ *   - return value: AHQ_OK or an ahq_status error code; ahq_last_error() returns a thread-local message
+ *   - the library never allocates device memory: scratch is a caller-provided `workspace` whose required size is
+ *     returned by the matching *_workspace_bytes() query (the buffer does not need to be cleared by the caller)
+ *
+ * Reference interfaces each entry point stands in for (paths relative to the AIMET checkout):
+ *   AT  = TrainingExtensions/torch/src/python/aimet_torch
+ *   DLQ = ModelOptimizations/DlQuantization
+ */
+#ifndef AIMET_AMD_H
+#define AIMET_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define AHQ_MAX_DIMS 8
+
+typedef enum {
+    AHQ_OK              = 0,
+    AHQ_ERR_INVALID     = 1, /* malformed argument (null pointer, negative size, bad enum, ...) */
+    AHQ_ERR_UNSUPPORTED = 2, /* well-formed request this library has no kernel for */
+    AHQ_ERR_LAUNCH      = 3, /* HIP runtime reported an error */
+    AHQ_ERR_WORKSPACE   = 4  /* workspace missing or too small */
+} ahq_status;
+
+typedef enum { AHQ_F32 = 0, AHQ_F16 = 1, AHQ_BF16 = 2 } ahq_dtype;
+
+/* Which of the reference's three quantize-dequantize arithmetics to reproduce. */
+typedef enum {
+    /* ATen fake_quantize_per_{tensor,channel}_affine as called from AT/quantization/affine/backends/torch_builtins.py:485-491,526-533:
+       inv = 1.0f/scale; q = rint(float(x)*inv) + zp; y = T((clamp(q,qmin,qmax) - zp) * scale); zp = -int32(offset) */
+    AHQ_ARITH_ATEN = 1,
+    /* QuantDequantFunc / QuantizeFunc / DequantizeFunc, torch_builtins.py:588-831: every intermediate rounded to the
+       compute dtype; t = x/scale [- zps]; r = rint(t) - offset; y = (clamp(r,qmin,qmax) + offset [+ zps]) * scale */
+    AHQ_ARITH_AUTOGRAD = 2,
+    /* DlQuantization quantizeValueCpu/dequantizeValueCpu, DLQ/src/trim_functions.cpp:177-209:
+       v = isnan(x) ? min : x; v = fmax(fmin(v,max),min); v = round(v/delta - offset); y = delta*(v + offset) */
+    AHQ_ARITH_DLQ = 3
+} ahq_arith;
+
+typedef enum {
+    AHQ_OP_QDQ = 0,       /* quantize-dequantize */
+    AHQ_OP_QUANTIZE = 1,  /* integer codes stored as floating point */
+    AHQ_OP_DEQUANTIZE = 2 /* (x + offset) * scale */
+} ahq_op;
+
+/*
+ * How encodings map onto a dense tensor.  The tensor has `ndim` dimensions `dims[]` (row-major, dims[ndim-1]
+ * fastest).  Along dimension d, `block[d]` consecutive coordinates share an encoding, and moving to the next block
+ * advances the encoding index by `enc_stride[d]` (0 = the encoding is broadcast along d).  The encoding index of an
+ * element with coordinates c[] is  sum_d (c[d] / block[d]) * enc_stride[d].
+ *   per-tensor:               ndim=1, dims={N}, block={N}, enc_stride={0}
+ *   per-channel axis 0 of RxC: dims={R,C}, block={1,C}, enc_stride={1,0}
+ *   blockwise (1,B) on RxC:    dims={R,C}, block={1,B}, enc_stride={C/B,1}
+ * This is the flattened form of the interleaved reshape in torch_builtins.py:285-289 and of
+ * getBroadcastableShapes/shapeToStrides in DLQ/src/tensor_utils.cpp:28-77.
+ */
+typedef struct {
+    int32_t ndim;
+    int64_t dims[AHQ_MAX_DIMS];
+    int64_t block[AHQ_MAX_DIMS];
+    int64_t enc_stride[AHQ_MAX_DIMS];
+} ahq_layout;
+
+/* Parameters of one quantization grid. */
+typedef struct {
+    int32_t arith;           /* ahq_arith */
+    int32_t op;              /* ahq_op */
+    int32_t io_dtype;        /* ahq_dtype of x / y / g / gx */
+    int32_t compute_dtype;   /* ahq_dtype every intermediate is rounded to (torch_builtins.py:268-277); == io_dtype or AHQ_F32 */
+    int64_t qmin;
+    int64_t qmax;
+    double  zero_point_shift; /* 0.0 or 0.5 (AT/quantization/affine/quantizer.py:170-174) */
+} ahq_grid;
+
+const char* ahq_last_error(void);
+int         ahq_version(void);
+
+/* ---------------------------------------------------------------- QDQ forward / backward --------------------------
+ * Replaces: torch_builtins.quantize / quantize_dequantize / dequantize (torch_builtins.py:166-302, 537-571), the ATen
+ * fast path (torch_builtins.py:335-431), and for AHQ_ARITH_DLQ DlQuantization::quantizeDequantize /
+ * quantizeDequantizeBroadcast (DLQ/src/trim_functions.cpp:108-128, 909-948).
+ *
+ * scale/offset: fp32 arrays with one entry per encoding (AHQ_ARITH_ATEN/AUTOGRAD).  For AHQ_ARITH_DLQ pass
+ * enc_min/enc_max as well (the float-narrowed TfEncoding fields, DLQ/src/trim_functions.cpp:211-226); otherwise
+ * they must be NULL.
+ * mask_out: optional (may be NULL) one byte per element, 1 where the code was inside [qmin,qmax]
+ * (torch_builtins.py:743-746).
+ */
+int ahq_qdq_forward(const ahq_grid* grid, const ahq_layout* layout, const void* x, void* y, uint8_t* mask_out,
+                    const float* scale, const float* offset, const float* enc_min, const float* enc_max,
+                    void* stream);
+
+/* Backward of the above with the straight-through estimator (torch_builtins.py:637-655, 691-701, 779-831).  The mask
+ * is recomputed from x.  gx may be NULL; gscale/goffset may be NULL (both or neither); when given they receive the
+ * gradient already reduced to one fp32 value per encoding (what autograd's sum-to-size produces in the reference).
+ */
+size_t ahq_qdq_backward_workspace_bytes(const ahq_grid* grid, const ahq_layout* layout, int want_param_grads);
+int    ahq_qdq_backward(const ahq_grid* grid, const ahq_layout* layout, const void* g, const void* x, void* gx,
+                        float* gscale, float* goffset, const float* scale, const float* offset, void* workspace,
+                        size_t workspace_bytes, void* stream);
+
+/* ---------------------------------------------------------------- min / max statistics ----------------------------
+ * Replaces: _MinMaxObserver.collect_stats = utils.reduce(amin/amax) (AT/quantization/encoding_analyzer.py:80-94,
+ * AT/utils.py:1115-1148), _HistogramObserver._get_min_max (encoding_analyzer.py:213-219, finite_only=1) and
+ * DlQuantization GetMinMax (DLQ/src/math_functions.cpp:72-117).
+ * out_min/out_max: one value per encoding in the tensor's own dtype.  NaN propagates like torch.amin/amax unless
+ * finite_only, where non-finite values are ignored (an all-non-finite slice yields +inf / -inf).
+ * If running != 0, out_min/out_max are combined with their current contents (minimum/maximum,
+ * encoding_analyzer.py:96-112) instead of being overwritten.
+ */
+size_t ahq_minmax_workspace_bytes(const ahq_layout* layout);
+int    ahq_minmax(int32_t dtype, const ahq_layout* layout, const void* x, void* out_min, void* out_max,
+                  int finite_only, int running, void* workspace, size_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* AIMET_AMD_H */

@@ -1,0 +1,275 @@
+"""Parity of the HIP quantize / dequantize / quantize-dequantize kernels with the CPU oracle.
+
+Bar: outputs and input gradients bit-exact; scale/offset gradients (order-sensitive sums) within 1e-5 relative in
+fp32 arithmetic and within one unit in the last place of the compute dtype for 16-bit arithmetic.
+"""
+
+import math
+
+import pytest
+import torch
+
+from oracle import torch_ref as O
+from tests.helpers import assert_same_bits, assert_close_rel
+
+pytestmark = pytest.mark.gpu
+
+# (tensor shape, encoding shape, block_size)
+LAYOUTS = [
+    ((37, 129), (), None),                 # per-tensor, ragged tail
+    ((4, 8, 16, 16), (1,), None),          # per-tensor, shape (1,)
+    ((1024, 1030), (), None),              # per-tensor, many tiles (last-workgroup reduction)
+    ((64, 4096), (64, 1), None),           # per-channel, one tile per row
+    ((16, 5000), (16, 1), None),           # per-channel, two tiles per row
+    ((8, 100), (8, 1), None),              # per-channel, rows shorter than a tile (atomic reduction)
+    ((8, 128), (8, 1), None),              # per-channel, power-of-two run inside a wave
+    ((4, 6, 10, 10), (6, 1, 1), None),     # activation per-channel (I > 1)
+    ((2, 3, 64, 64), (3, 1, 1), None),     # activation per-channel, long runs
+    ((32, 256), (32, 4), (1, 64)),         # blockwise along the input dimension
+    ((3, 32, 256), (32, 4), (1, 64)),      # blockwise with a leading broadcast dimension
+    ((8, 16), (2, 4), (4, 4)),             # two-dimensional blocks (generic walk)
+    ((10, 12), (12,), None),               # per-channel on the fastest axis
+    ((6, 10), (6, 1), None),               # run length not a multiple of the vector width
+    ((5, 7, 64), (5, 1, 2), (1, -1, -1)),  # wildcard block sizes
+]
+
+DTYPES = [torch.float32, torch.bfloat16, torch.float16]
+
+
+def _grid(bitwidth, symmetric):
+    n = 2 ** bitwidth - 1
+    if symmetric:
+        return -math.ceil(n / 2), math.floor(n / 2)
+    return 0, n
+
+
+def _make_case(shape, enc_shape, dtype, qmin, qmax, symmetric, seed):
+    g = torch.Generator().manual_seed(seed)
+    scale = (torch.rand(enc_shape, generator=g) * 0.05 + 0.002).to(torch.float32)
+    if symmetric:
+        offset = torch.full(enc_shape, float(-round((qmin + qmax) / 2)))
+    else:
+        offset = torch.randint(-qmax, -qmin + 1, enc_shape, generator=g).to(torch.float32)
+    span = float(qmax - qmin)
+    x = torch.randn(shape, generator=g) * 0.04 * span * 0.4
+    flat = x.flatten()
+    # exact half-way points and a few far outliers
+    k = torch.arange(min(flat.numel() // 3, 600), dtype=torch.float32)
+    flat[: k.numel()] = (k - k.numel() // 2 + 0.5) * 0.01
+    if flat.numel() > 8:
+        flat[-1] = 1e30
+        flat[-2] = -1e30
+        flat[-3] = 0.0
+    x = flat.view(shape).to(dtype)
+    grad = torch.randn(shape, generator=g).to(dtype)
+    return x, scale, offset, grad
+
+
+def _tol(compute_dtype):
+    if compute_dtype == torch.float32:
+        return 1e-5
+    return float(torch.finfo(compute_dtype).eps)  # one unit in the last place of the rounded sum
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=lambda d: str(d).split(".")[-1])
+@pytest.mark.parametrize("layout", LAYOUTS, ids=lambda l: "x".join(map(str, l[0])) + "_" + "x".join(map(str, l[1])))
+@pytest.mark.parametrize("bitwidth,symmetric", [(4, True), (8, False), (8, True), (16, False)])
+def test_quantize_dequantize_learnable(device, layout, dtype, bitwidth, symmetric):
+    """Composed autograd arithmetic (scale/offset require grad): forward, gx, gscale, goffset."""
+    from aimet_amd.quantization import affine
+
+    shape, enc_shape, block = layout
+    qmin, qmax = _grid(bitwidth, symmetric)
+    x, scale, offset, grad = _make_case(shape, enc_shape, dtype, qmin, qmax, symmetric, seed=bitwidth * 7 + len(shape))
+
+    tr = O.qdq_v2_forward(x, scale, offset, qmin, qmax, block)
+    gx_ref, gs_ref, go_ref = O.qdq_v2_backward(grad, x, scale, offset, qmin, qmax, block)
+
+    xd = x.to(device).requires_grad_(True)
+    sd = scale.to(device).requires_grad_(True)
+    od = offset.to(device).requires_grad_(True)
+    y = affine.quantize_dequantize(xd, sd, od, qmin, qmax, block_size=block)
+    assert y.dtype == dtype and y.shape == x.shape
+    assert_same_bits(y, tr.y, "output")
+    y.backward(grad.to(device))
+    assert_same_bits(xd.grad, gx_ref, "input gradient")
+    tol = _tol(tr.dtype)
+    assert_close_rel(sd.grad, gs_ref, tol, "scale gradient", abs_floor=1e-30)
+    assert_close_rel(od.grad, go_ref, tol, "offset gradient", abs_floor=1e-30)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=lambda d: str(d).split(".")[-1])
+@pytest.mark.parametrize("layout", [l for l in LAYOUTS if l[2] is None],
+                         ids=lambda l: "x".join(map(str, l[0])) + "_" + "x".join(map(str, l[1])))
+@pytest.mark.parametrize("bitwidth,symmetric", [(4, False), (8, False), (8, True), (16, False)])
+def test_quantize_dequantize_frozen(device, layout, dtype, bitwidth, symmetric):
+    """Frozen encodings take the ATen fake-quantize arithmetic where the reference does."""
+    from aimet_amd.quantization import affine
+
+    shape, enc_shape, _ = layout
+    qmin, qmax = _grid(bitwidth, symmetric)
+    x, scale, offset, grad = _make_case(shape, enc_shape, dtype, qmin, qmax, symmetric, seed=bitwidth * 11 + 3)
+    # the ATen kernels have undefined behaviour for inf * inv_scale: keep the outliers finite after scaling
+    x = torch.where(x.abs() > 1e20, torch.sign(x) * 1e4, x.float()).to(dtype)
+
+    ref = O.qdq_v1(x, scale, offset, qmin, qmax)
+    if ref is None:
+        tr = O.qdq_v2_forward(x, scale, offset, qmin, qmax)
+        y_ref, mask_ref = tr.y, tr.mask
+    else:
+        y_ref, mask_ref = ref
+
+    xd = x.to(device).requires_grad_(True)
+    y = affine.quantize_dequantize(xd, scale.to(device), offset.to(device), qmin, qmax)
+    assert_same_bits(y, y_ref, "output")
+    y.backward(grad.to(device))
+    assert_same_bits(xd.grad, (grad * mask_ref).to(dtype), "input gradient")
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=lambda d: str(d).split(".")[-1])
+@pytest.mark.parametrize("layout", LAYOUTS[:1] + LAYOUTS[3:4] + LAYOUTS[9:12],
+                         ids=lambda l: "x".join(map(str, l[0])) + "_" + "x".join(map(str, l[1])))
+def test_zero_point_shift(device, layout, dtype):
+    """zero_point_shift = 0.5 (symmetric 4-bit) including the gradient correction of the scale term."""
+    from aimet_amd.quantization import affine
+
+    shape, enc_shape, block = layout
+    qmin, qmax = -8, 7
+    x, scale, offset, grad = _make_case(shape, enc_shape, dtype, qmin, qmax, True, seed=5)
+    tr = O.qdq_v2_forward(x, scale, offset, qmin, qmax, block, 0.5)
+    gx_ref, gs_ref, go_ref = O.qdq_v2_backward(grad, x, scale, offset, qmin, qmax, block, 0.5)
+    xd = x.to(device).requires_grad_(True)
+    sd = scale.to(device).requires_grad_(True)
+    od = offset.to(device).requires_grad_(True)
+    y = affine.quantize_dequantize(xd, sd, od, qmin, qmax, block_size=block, zero_point_shift=0.5)
+    assert_same_bits(y, tr.y, "output")
+    y.backward(grad.to(device))
+    assert_same_bits(xd.grad, gx_ref, "input gradient")
+    assert_close_rel(sd.grad, gs_ref, _tol(tr.dtype), "scale gradient", abs_floor=1e-30)
+    assert_close_rel(od.grad, go_ref, _tol(tr.dtype), "offset gradient", abs_floor=1e-30)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=lambda d: str(d).split(".")[-1])
+@pytest.mark.parametrize("layout", LAYOUTS[:1] + LAYOUTS[3:4] + LAYOUTS[7:8] + LAYOUTS[9:10] + LAYOUTS[11:12],
+                         ids=lambda l: "x".join(map(str, l[0])) + "_" + "x".join(map(str, l[1])))
+@pytest.mark.parametrize("bitwidth,symmetric", [(4, True), (8, False)])
+def test_quantize_and_dequantize(device, layout, dtype, bitwidth, symmetric):
+    from aimet_amd.quantization import affine
+
+    shape, enc_shape, block = layout
+    qmin, qmax = _grid(bitwidth, symmetric)
+    x, scale, offset, grad = _make_case(shape, enc_shape, dtype, qmin, qmax, symmetric, seed=17)
+
+    q_ref, _ = O.quantize_forward(x, scale, offset, qmin, qmax, block)
+    gx_ref, gs_ref, go_ref = O.quantize_backward(grad, x, scale, offset, qmin, qmax, block)
+    D = O.internal_dtype(dtype, qmin, qmax)
+    xd = x.to(device).requires_grad_(True)
+    sd = scale.to(device).requires_grad_(True)
+    od = offset.to(device).requires_grad_(True)
+    q = affine.quantize(xd, sd, od, qmin, qmax, block_size=block)
+    assert_same_bits(q, q_ref, "codes")
+    q.backward(grad.to(device))
+    assert_same_bits(xd.grad, gx_ref, "quantize input gradient")
+    # the scale gradient multiplies two quotients: outliers make it huge, compare relative to its own magnitude
+    assert_close_rel(sd.grad, gs_ref, max(_tol(D), 1e-5), "quantize scale gradient", abs_floor=1e-30)
+    assert_close_rel(od.grad, go_ref, max(_tol(D), 1e-5), "quantize offset gradient", abs_floor=1e-30)
+
+    # dequantize the codes again
+    codes = q_ref
+    dq_ref = O.dequantize_forward(codes, scale, offset, block)
+    gx2, gs2, go2 = O.dequantize_backward(grad, codes, scale, offset, block)
+    cd = codes.to(device).requires_grad_(True)
+    sd2 = scale.to(device).requires_grad_(True)
+    od2 = offset.to(device).requires_grad_(True)
+    dq = affine.dequantize(cd, sd2, od2, block_size=block)
+    assert_same_bits(dq, dq_ref, "dequantized")
+    dq.backward(grad.to(device))
+    assert_same_bits(cd.grad, gx2, "dequantize input gradient")
+    assert_close_rel(sd2.grad, gs2, max(_tol(dtype), 1e-5), "dequantize scale gradient", abs_floor=1e-30)
+    assert_close_rel(od2.grad, go2, max(_tol(dtype), 1e-5), "dequantize offset gradient", abs_floor=1e-30)
+
+
+def test_non_finite_inputs(device):
+    """NaN propagates, +-inf saturates (composed arithmetic); gradients of NaN inputs are zero."""
+    from aimet_amd.quantization import affine
+
+    x = torch.tensor([float("nan"), float("inf"), -float("inf"), 0.3, -0.0, 1e-45, -1e-45, 3.4e38])
+    scale = torch.tensor(0.01)
+    offset = torch.tensor(-128.0)
+    grad = torch.ones_like(x)
+    tr = O.qdq_v2_forward(x, scale, offset, 0, 255)
+    gx_ref, gs_ref, go_ref = O.qdq_v2_backward(grad, x, scale, offset, 0, 255)
+    xd = x.to(device).requires_grad_(True)
+    sd = scale.to(device).requires_grad_(True)
+    od = offset.to(device).requires_grad_(True)
+    y = affine.quantize_dequantize(xd, sd, od, 0, 255)
+    assert_same_bits(y, tr.y, "output")
+    y.backward(grad.to(device))
+    assert_same_bits(xd.grad, gx_ref, "input gradient")
+
+
+@pytest.mark.parametrize("memory_format", [torch.channels_last, torch.channels_last_3d])
+def test_memory_format_is_preserved(device, memory_format):
+    """Dense non-contiguous inputs keep their memory format (reference: test_backend.py:410-448)."""
+    from aimet_amd.quantization import affine
+
+    shape = (2, 3, 4, 5) if memory_format == torch.channels_last else (2, 3, 4, 5, 2)
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(shape, generator=g)
+    scale = torch.rand(3, *([1] * (len(shape) - 2)), generator=g) * 0.05 + 0.01
+    offset = torch.randint(-255, 1, scale.shape, generator=g).float()
+    tr = O.qdq_v2_forward(x, scale, offset, 0, 255)
+    xd = x.to(device).to(memory_format=memory_format)
+    sd = scale.to(device).requires_grad_(True)
+    y = affine.quantize_dequantize(xd, sd, offset.to(device), 0, 255)
+    assert y.is_contiguous(memory_format=memory_format)
+    assert_same_bits(y, tr.y, "output")
+    q = affine.quantize(xd, scale.to(device), offset.to(device), 0, 255)
+    assert q.is_contiguous(memory_format=memory_format)
+    assert_same_bits(q, O.quantize_forward(x, scale, offset, 0, 255)[0], "codes")
+
+
+def test_non_dense_and_misaligned_inputs(device):
+    from aimet_amd.quantization import affine
+
+    g = torch.Generator().manual_seed(4)
+    base = torch.randn(64, 130, generator=g)
+    scale = torch.tensor(0.02)
+    offset = torch.tensor(-100.0)
+    bd = base.to(device)
+    # strided view (not dense) and a view whose storage offset breaks 16-byte alignment
+    for cpu_view, dev_view in [(base[:, ::2], bd[:, ::2]), (base.flatten()[1:], bd.flatten()[1:])]:
+        tr = O.qdq_v2_forward(cpu_view, scale, offset, 0, 255)
+        sd = scale.to(device).requires_grad_(True)
+        y = affine.quantize_dequantize(dev_view, sd, offset.to(device), 0, 255)
+        assert_same_bits(y, tr.y, "output")
+
+
+def test_errors(device):
+    from aimet_amd.quantization import affine
+
+    x = torch.randn(2, 3, 4, 5, device=device)
+    off = torch.zeros((), device=device)
+    for bad in [(4,), (2,), (3, 1), (2, 1, 1)]:
+        s = torch.rand(bad, device=device) + 0.1
+        with pytest.raises(RuntimeError):
+            affine.quantize_dequantize(x, s, off, 0, 255)
+        with pytest.raises(RuntimeError):
+            affine.quantize(x, s, off, 0, 255)
+        with pytest.raises(RuntimeError):
+            affine.dequantize(x, s, off)
+    s = torch.tensor(0.1, device=device)
+    with pytest.raises(RuntimeError):  # mixed devices
+        affine.quantize_dequantize(x, s.cpu(), off, 0, 255)
+    with pytest.raises(RuntimeError):  # CPU tensors have no path here
+        affine.quantize_dequantize(x.cpu(), s.cpu(), off.cpu(), 0, 255)
+    with pytest.raises(RuntimeError):  # qmin > qmax
+        affine.quantize_dequantize(x, s, off, 5, 1)
+    with pytest.raises(RuntimeError):  # bf16 cannot hold a 16-bit grid
+        affine.quantize(x.bfloat16(), s, off, 0, 65535)
+    with pytest.raises(RuntimeError):  # block size that does not tile the tensor
+        affine.quantize_dequantize(x, torch.ones(4, 2, device=device), torch.zeros(4, 2, device=device), 0, 255,
+                                   block_size=(1, 3))
+    # empty tensors pass through
+    e = torch.empty(0, 4, device=device)
+    assert affine.quantize_dequantize(e, s, off, 0, 255).shape == (0, 4)
