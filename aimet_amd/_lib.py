@@ -46,6 +46,36 @@ class Grid(ctypes.Structure):
     ]
 
 
+class HistState(ctypes.Structure):
+    _fields_ = [
+        ("num_slots", ctypes.c_int32),
+        ("num_bins", ctypes.c_int32),
+        ("growth_limit", ctypes.c_float),
+        ("hist", ctypes.c_void_p),
+        ("edges", ctypes.c_void_p),
+        ("minmax", ctypes.c_void_p),
+        ("limits", ctypes.c_void_p),
+        ("new_hist", ctypes.c_void_p),
+        ("new_edges", ctypes.c_void_p),
+        ("new_minmax", ctypes.c_void_p),
+    ]
+
+
+class SqnrParams(ctypes.Structure):
+    _fields_ = [
+        ("num_slots", ctypes.c_int32),
+        ("num_bins", ctypes.c_int32),
+        ("num_deltas", ctypes.c_int32),
+        ("num_offsets", ctypes.c_int32),
+        ("symmetric", ctypes.c_int32),
+        ("stat_dtype", ctypes.c_int32),
+        ("num_steps", ctypes.c_int64),
+        ("minimum_scale", ctypes.c_double),
+        ("gamma", ctypes.c_double),
+        ("p", ctypes.c_double),
+    ]
+
+
 class HipLibraryError(RuntimeError):
     """Raised when libaimet_amd.so is missing or one of its entry points reports an error."""
 
@@ -62,8 +92,12 @@ _SIGNATURES = {
     "ahq_qdq_backward": (ctypes.c_int, [ctypes.POINTER(Grid), ctypes.POINTER(Layout), _P, _P, _P, _P, _P, _P, _P, _P,
                                         ctypes.c_size_t, _P]),
     "ahq_minmax_workspace_bytes": (ctypes.c_size_t, [ctypes.POINTER(Layout)]),
-    "ahq_minmax": (ctypes.c_int, [ctypes.c_int32, ctypes.POINTER(Layout), _P, _P, _P, ctypes.c_int, ctypes.c_int, _P,
+    "ahq_minmax": (ctypes.c_int, [ctypes.c_int32, ctypes.POINTER(Layout), _P, _P, _P, _P, _P, ctypes.c_int, _P,
                                   ctypes.c_size_t, _P]),
+    "ahq_hist_update_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int32, ctypes.POINTER(Layout), ctypes.c_int32]),
+    "ahq_hist_update": (ctypes.c_int, [ctypes.c_int32, ctypes.POINTER(Layout), _P, ctypes.POINTER(HistState),
+                                       ctypes.c_int, _P, ctypes.c_size_t, _P]),
+    "ahq_sqnr_search": (ctypes.c_int, [ctypes.POINTER(SqnrParams), _P, _P, _P, _P, _P, _P, _P, _P, _P, _P]),
 }
 
 

@@ -83,27 +83,4 @@ struct OpMinF { __device__ __forceinline__ float operator()(float a, float b) co
 struct OpMaxF { __device__ __forceinline__ float operator()(float a, float b) const { return fmaxf(a, b); } };
 struct OpOrI { __device__ __forceinline__ int operator()(int a, int b) const { return a | b; } };
 
-// ------------------------------------------------------------------------------- "last workgroup finishes" ticket --
-// Self-resetting counters living in the library's own device memory (one array per translation unit); a launch takes
-// one slot (chosen round-robin on the host) so that launches in flight on different streams do not share a counter.
-constexpr int kTicketSlots = 1024;
-static __device__ unsigned int g_tickets[kTicketSlots];
-
-// Returns true in every thread of the workgroup that arrived last.  Earlier global writes of all workgroups are
-// visible to that workgroup afterwards.
-__device__ __forceinline__ bool last_block_done(int slot, unsigned int nblocks, int* smem_flag) {
-    __threadfence();
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        unsigned int prev = atomicAdd(&g_tickets[slot], 1u);
-        int last = (prev == nblocks - 1);
-        if (last) g_tickets[slot] = 0;  // only the last arrival touches it again: safe to reset here
-        *smem_flag = last;
-    }
-    __syncthreads();
-    const bool last = *smem_flag != 0;
-    if (last) __threadfence();
-    return last;
-}
-
 }  // namespace ahq

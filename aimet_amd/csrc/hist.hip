@@ -1,0 +1,548 @@
+// Histogram statistics of the histogram observer (aimet_torch/quantization/encoding_analyzer.py:121-338).
+//
+// One ahq_hist_update() call folds a batch into the running per-encoding histogram:
+//   1. finite min/max of the batch                     (ahq_minmax with finite_only, reduce.hip)
+//   2. hist_prepare_kernel (one workgroup per slot):   bin edges of the batch's own histogram, the updated range
+//      clamped to the growth limit, and the running counts re-binned onto that range (same fp32 operations in the
+//      same order as the reference, encoding_analyzer.py:221-310)
+//   3. hist_bin_kernel:                                one pass over the batch that bins every element against BOTH
+//      ranges (the batch's own and the updated one) into wave-private LDS sub-histograms, merged per workgroup
+//   4. hist_finish_kernel:                             integer counts -> fp32, plus carried counts and the
+//      below/above-range counts, in the reference's order of additions (encoding_analyzer.py:198-207, 313-323)
+//
+// Bin index formula = torch.histc on CPU:  pos = int64(((x - lo) * B) / (hi - lo)) in fp32, the top edge belongs to the
+// last bin, values outside [lo, hi] and NaN are not counted.
+
+#include "ahq_device.h"
+#include "ahq_host.h"
+#include "layout.h"
+#include "tiling.h"
+
+extern "C" int ahq_minmax(int32_t dtype, const ahq_layout* layout, const void* x, void* out_min, void* out_max,
+                          void* run_min, void* run_max, int finite_only, void* workspace, size_t workspace_bytes,
+                          void* stream);
+extern "C" size_t ahq_minmax_workspace_bytes(const ahq_layout* layout);
+
+namespace ahq {
+
+constexpr int kHistBlocksMax = 1024;  // persistent workgroups of the binning pass (4 per CU)
+constexpr int kRng = 8;               // floats per slot in `ranges`
+
+// ranges[slot]: lo1, hi1, thr_lo1, thr_hi1 (batch's own range), lo2, hi2, thr_lo2, thr_hi2 (updated range).
+// thr_* are the edges rounded to the tensor dtype: the reference compares `x < edge` in the tensor's dtype.
+
+template <typename IO>
+__device__ __forceinline__ float round_io(float v) { return load_f32(store_cast<IO>(v)); }
+
+struct PrepArgs {
+    int32_t num_slots, num_bins, first;
+    float growth;
+    const void* bmin;  // [S] io dtype
+    const void* bmax;
+    float* hist;       // [S][B] running
+    float* edges;      // [S][B+1]
+    float* minmax;     // [S][2] stored min / max
+    float* limits;     // [S][2]
+    float* new_edges;  // [S][B+1]
+    float* new_minmax; // [S][2]
+    float* carried;    // [S][B]
+    float* upd_edges;  // [S][B+1]
+    float* ranges;     // [S][8]
+    int32_t* scratch;  // [S][2][B] destination indices
+};
+
+// _create_bin_edges (encoding_analyzer.py:221-229).  `lo`/`hi` already hold the min==max adjustment.
+__device__ __forceinline__ float edge_at(float lo, float step, int i) { return (float)i * step + lo; }
+
+template <typename IO>
+__global__ void hist_prepare_kernel(const PrepArgs a) {
+    const int s = blockIdx.x;
+    const int B = a.num_bins;
+    const float Bf = (float)B;
+    const float mn = load_f32(static_cast<const IO*>(a.bmin)[s]);
+    const float mx = load_f32(static_cast<const IO*>(a.bmax)[s]);
+    // the batch's own bin edges; "min - 0.5" happens in the tensor dtype before the cast to float
+    const bool eq = mn == mx;
+    const float lo1 = eq ? round_io<IO>(mn - 0.5f) : mn;
+    const float hi1 = eq ? round_io<IO>(mx + 0.5f) : mx;
+    const float step1 = (hi1 - lo1) / Bf;
+    float* ne = a.new_edges + (size_t)s * (B + 1);
+    for (int i = threadIdx.x; i <= B; i += blockDim.x) ne[i] = edge_at(lo1, step1, i);
+    const float e1_first = edge_at(lo1, step1, 0), e1_last = edge_at(lo1, step1, B);
+    float* rg = a.ranges + (size_t)s * kRng;
+    float* mmx = a.minmax + (size_t)s * 2;
+    float* lim = a.limits + (size_t)s * 2;
+    if (threadIdx.x == 0) {
+        a.new_minmax[2 * s] = mn;
+        a.new_minmax[2 * s + 1] = mx;
+        rg[0] = e1_first;
+        rg[1] = e1_last;
+        rg[2] = round_io<IO>(e1_first);
+        rg[3] = round_io<IO>(e1_last);
+    }
+    if (a.first) {
+        // the first batch becomes the running statistics; the growth limit is fixed from its edge range
+        if (threadIdx.x == 0) {
+            const float range = e1_last - e1_first;
+            lim[0] = e1_first - (range * a.growth) / 2.0f;
+            lim[1] = e1_last + (range * a.growth) / 2.0f;
+            mmx[0] = mn;
+            mmx[1] = mx;
+            rg[4] = rg[0];
+            rg[5] = rg[1];
+            rg[6] = rg[2];
+            rg[7] = rg[3];
+        }
+        float* ue = a.upd_edges + (size_t)s * (B + 1);
+        for (int i = threadIdx.x; i <= B; i += blockDim.x) ue[i] = edge_at(lo1, step1, i);
+        return;
+    }
+    const float* ce = a.edges + (size_t)s * (B + 1);
+    const float* ch = a.hist + (size_t)s * B;
+    float* carried = a.carried + (size_t)s * B;
+    const float c_first = ce[0], c_last = ce[B];
+    // clamp(min=left, max=edge0) == min(max(x, left), edge0)
+    const float umin = fminf(fmaxf(mn, lim[0]), c_first);
+    const float umax = fminf(fmaxf(mx, c_last), lim[1]);
+    const bool same = (umin == mmx[0]) && (umax == mmx[1]);
+    if (same) {
+        for (int i = threadIdx.x; i < B; i += blockDim.x) carried[i] = ch[i];
+    } else {
+        const float dst_w = (umax - umin) / Bf;
+        const float src_w = ce[1] - ce[0];
+        int32_t* di = a.scratch + (size_t)s * 2 * B;
+        int32_t* oi = di + B;
+        for (int i = threadIdx.x; i < B; i += blockDim.x) {
+            const float start = ce[i];
+            int d = (int)((start - umin) / dst_w);
+            di[i] = d < B - 1 ? d : B - 1;
+            int o = (int)(((start + dst_w) - umin) / dst_w);
+            oi[i] = o < B - 1 ? o : B - 1;
+        }
+        __syncthreads();
+        // index_add_ runs over the source bins in order: reproduce that order for every destination bin
+        for (int d = threadIdx.x; d < B; d += blockDim.x) {
+            float acc = 0.f;
+            for (int i = 0; i < B; ++i) {
+                if (di[i] == d) {
+                    const float start = ce[i];
+                    const float dst_end = umin + dst_w * (float)(di[i] + 1);
+                    const float part = __builtin_rintf(((dst_end - start) / src_w) * ch[i]);
+                    acc += fminf(part, ch[i]);
+                }
+            }
+            for (int i = 0; i < B; ++i) {
+                if (oi[i] == d) {
+                    const float start = ce[i];
+                    const float dst_end = umin + dst_w * (float)(di[i] + 1);
+                    const float part = __builtin_rintf(((dst_end - start) / src_w) * ch[i]);
+                    const float first = fminf(part, ch[i]);
+                    if (first < ch[i]) acc += ch[i] - first;
+                }
+            }
+            carried[d] = acc;
+        }
+    }
+    // bin edges of the updated range (with the min == max adjustment, in fp32 here)
+    const bool ueq = umin == umax;
+    const float lo2 = ueq ? umin - 0.5f : umin;
+    const float hi2 = ueq ? umax + 0.5f : umax;
+    const float step2 = (hi2 - lo2) / Bf;
+    float* ue = a.upd_edges + (size_t)s * (B + 1);
+    for (int i = threadIdx.x; i <= B; i += blockDim.x) ue[i] = edge_at(lo2, step2, i);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        rg[4] = umin;
+        rg[5] = umax;
+        rg[6] = round_io<IO>(umin);
+        rg[7] = round_io<IO>(umax);
+        mmx[0] = umin;
+        mmx[1] = umax;
+    }
+}
+
+// ------------------------------------------------------------------------------------------------ binning pass --
+struct BinArgs : Geom {
+    const void* x;
+    const float* ranges;   // [S][8]
+    uint32_t* partials;    // single slot: [nblocks][NH][B + 2]  (bins, below, above)
+    uint32_t* counts;      // several slots: [S][NH][B + 2], zero-initialised
+    int32_t num_bins;
+    int32_t nhist;
+    int32_t copies;        // wave-private LDS copies (1..4)
+    int64_t ntiles;
+};
+
+struct RangeC {
+    float lo, hi, width, thr_lo, thr_hi;
+};
+
+__device__ __forceinline__ RangeC load_range(const float* rg, int h) {
+    RangeC r;
+    r.lo = rg[4 * h];
+    r.hi = rg[4 * h + 1];
+    // torch.histc widens an empty range by one on each side
+    if (r.lo == r.hi) {
+        r.lo -= 1.f;
+        r.hi += 1.f;
+    }
+    r.width = r.hi - r.lo;
+    r.thr_lo = rg[4 * h + 2];
+    r.thr_hi = rg[4 * h + 3];
+    return r;
+}
+
+// returns the bin of v in range r or -1
+__device__ __forceinline__ int bin_of(float v, const RangeC& r, float Bf, int B) {
+    if (!(v >= r.lo && v <= r.hi)) return -1;
+    int p = (int)(((v - r.lo) * Bf) / r.width);
+    return p >= B ? B - 1 : p;
+}
+
+// Single-slot fast path: persistent workgroups, wave-private LDS sub-histograms, one partial per workgroup.
+template <typename IO, int VEC, int NH>
+__global__ __launch_bounds__(kBlock) void hist_bin_kernel(const BinArgs a) {
+    extern __shared__ uint32_t lds[];  // [copies][NH][B]
+    __shared__ uint32_t cnt_smem[kBlock / kWave][NH][2];
+    const int B = a.num_bins;
+    const float Bf = (float)B;
+    const int copies = a.copies;
+    for (int i = threadIdx.x; i < copies * NH * B; i += kBlock) lds[i] = 0;
+    RangeC r[NH];
+#pragma unroll
+    for (int h = 0; h < NH; ++h) r[h] = load_range(a.ranges, h);
+    __syncthreads();
+    const int wave = threadIdx.x / kWave;
+    uint32_t* mine = lds + (size_t)(wave % copies) * NH * B;
+    const IO* __restrict__ x = static_cast<const IO*>(a.x);
+    uint32_t below[NH], above[NH];
+#pragma unroll
+    for (int h = 0; h < NH; ++h) below[h] = above[h] = 0;
+
+    for (int64_t tile = blockIdx.x; tile < a.ntiles; tile += gridDim.x) {
+        const int64_t v0 = tile * kTileVec;
+        const int64_t left = a.nvec - v0;
+        const int nv = (int)(left < kTileVec ? left : kTileVec);
+        Pack<IO, VEC> in[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            const int lv = u * kBlock + threadIdx.x;
+            if (lv < nv) in[u] = load_pack<IO, VEC>(x + (v0 + lv) * VEC);
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            const int lv = u * kBlock + threadIdx.x;
+            if (lv < nv) {
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) {
+                    const float v = load_f32(in[u].v[k]);
+#pragma unroll
+                    for (int h = 0; h < NH; ++h) {
+                        const int b = bin_of(v, r[h], Bf, B);
+                        if (b >= 0) atomicAdd(&mine[h * B + b], 1u);
+                        below[h] += v < r[h].thr_lo ? 1u : 0u;
+                        above[h] += v > r[h].thr_hi ? 1u : 0u;
+                    }
+                }
+            }
+        }
+    }
+    if (VEC > 1 && blockIdx.x == 0) {  // elements past the last full vector
+        const int64_t i = a.nvec * VEC + threadIdx.x;
+        if (i < a.numel) {
+            const float v = load_f32(x[i]);
+#pragma unroll
+            for (int h = 0; h < NH; ++h) {
+                const int b = bin_of(v, r[h], Bf, B);
+                if (b >= 0) atomicAdd(&mine[h * B + b], 1u);
+                below[h] += v < r[h].thr_lo ? 1u : 0u;
+                above[h] += v > r[h].thr_hi ? 1u : 0u;
+            }
+        }
+    }
+    // below / above: wave reduce, then across waves
+#pragma unroll
+    for (int h = 0; h < NH; ++h) {
+        uint32_t bl = below[h], ab = above[h];
+#pragma unroll
+        for (int m = kWave / 2; m >= 1; m >>= 1) {
+            bl += __shfl_xor(bl, m, kWave);
+            ab += __shfl_xor(ab, m, kWave);
+        }
+        if ((threadIdx.x & (kWave - 1)) == 0) {
+            cnt_smem[wave][h][0] = bl;
+            cnt_smem[wave][h][1] = ab;
+        }
+    }
+    __syncthreads();
+    uint32_t* out = a.partials + (size_t)blockIdx.x * NH * (B + 2);
+    for (int i = threadIdx.x; i < NH * B; i += kBlock) {
+        const int h = i / B, b = i - h * B;
+        uint32_t c = 0;
+        for (int cp = 0; cp < copies; ++cp) c += lds[(size_t)cp * NH * B + i];
+        out[h * (B + 2) + b] = c;
+    }
+    if (threadIdx.x < NH * 2) {
+        const int h = threadIdx.x / 2, w = threadIdx.x & 1;
+        uint32_t c = 0;
+        for (int wv = 0; wv < kBlock / kWave; ++wv) c += cnt_smem[wv][h][w];
+        out[h * (B + 2) + B + w] = c;
+    }
+}
+
+// Several slots (or histograms too large for LDS): every element adds to its slot's counters in global memory.
+template <typename IO>
+__global__ __launch_bounds__(kBlock) void hist_bin_generic_kernel(const BinArgs a) {
+    const int B = a.num_bins;
+    const float Bf = (float)B;
+    const IO* __restrict__ x = static_cast<const IO*>(a.x);
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < a.numel; i += (int64_t)gridDim.x * kBlock) {
+        int64_t e;
+        if (a.nseg > 0) e = generic_enc_index(a, i);
+        else e = a.J == 1 ? 0 : (i / a.K) % a.J;
+        const float v = load_f32(x[i]);
+        const float* rg = a.ranges + e * kRng;
+        uint32_t* c = a.counts + (size_t)e * a.nhist * (B + 2);
+        for (int h = 0; h < a.nhist; ++h) {
+            const RangeC r = load_range(rg, h);
+            const int b = bin_of(v, r, Bf, B);
+            if (b >= 0) atomicAdd(&c[h * (B + 2) + b], 1u);
+            if (v < r.thr_lo) atomicAdd(&c[h * (B + 2) + B], 1u);
+            if (v > r.thr_hi) atomicAdd(&c[h * (B + 2) + B + 1], 1u);
+        }
+    }
+}
+
+__global__ void zero_u32_kernel(uint32_t* p, int64_t n) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) p[i] = 0;
+}
+
+// ----------------------------------------------------------------------------------------------------- finish --
+struct FinArgs {
+    int32_t num_slots, num_bins, nhist, first;
+    int32_t nparts;            // partial histograms per slot (1 when `counts` is used)
+    const uint32_t* counts;    // [S][nparts][NH][B + 2]
+    const float* carried;      // [S][B]
+    const float* upd_edges;    // [S][B+1]
+    float* hist;               // [S][B] running (out)
+    float* edges;              // [S][B+1] running (out)
+    float* new_hist;           // [S][B] (out)
+};
+
+__global__ __launch_bounds__(kBlock) void hist_finish_kernel(const FinArgs a) {
+    // grid: (ceil(B/64), S); thread = (bin within 64, group of partials)
+    __shared__ unsigned long long sm[4][2][64];
+    __shared__ unsigned long long edge_cnt[2][2];
+    const int B = a.num_bins, NH = a.nhist;
+    const int s = blockIdx.y;
+    const int bl = threadIdx.x & 63, grp = threadIdx.x >> 6;
+    const int b = blockIdx.x * 64 + bl;
+    const uint32_t* base = a.counts + (size_t)s * a.nparts * NH * (B + 2);
+    unsigned long long c[2] = {0, 0};
+    if (b < B) {
+        for (int p = grp; p < a.nparts; p += 4)
+            for (int h = 0; h < NH; ++h) c[h] += base[((size_t)p * NH + h) * (B + 2) + b];
+    }
+    sm[grp][0][bl] = c[0];
+    sm[grp][1][bl] = c[1];
+    // below/above totals (needed by the workgroups that own bin 0 and bin B-1; cheap enough to do everywhere)
+    if (threadIdx.x < 4) {
+        const int h = threadIdx.x >> 1, w = threadIdx.x & 1;
+        unsigned long long t = 0;
+        if (h < NH)
+            for (int p = 0; p < a.nparts; ++p) t += base[((size_t)p * NH + h) * (B + 2) + B + w];
+        edge_cnt[h][w] = t;
+    }
+    __syncthreads();
+    if (grp != 0 || b >= B) return;
+    unsigned long long tot[2];
+    for (int h = 0; h < 2; ++h) tot[h] = sm[0][h][bl] + sm[1][h][bl] + sm[2][h][bl] + sm[3][h][bl];
+    // the batch's own histogram: counts, then "+= below" on bin 0 and "+= above" on the last bin
+    float nh = (float)tot[0];
+    if (b == 0) nh += (float)edge_cnt[0][0];
+    if (b == B - 1) nh += (float)edge_cnt[0][1];
+    a.new_hist[(size_t)s * B + b] = nh;
+    float uh;
+    if (a.first) {
+        uh = nh;
+    } else {
+        const int h = NH - 1;
+        uh = (float)tot[h] + a.carried[(size_t)s * B + b];
+        if (b == 0) uh += (float)edge_cnt[h][0];
+        if (b == B - 1) uh += (float)edge_cnt[h][1];
+    }
+    a.hist[(size_t)s * B + b] = uh;
+    a.edges[(size_t)s * (B + 1) + b] = a.upd_edges[(size_t)s * (B + 1) + b];
+    if (b == B - 1) a.edges[(size_t)s * (B + 1) + B] = a.upd_edges[(size_t)s * (B + 1) + B];
+}
+
+}  // namespace ahq
+
+using namespace ahq;
+
+namespace {
+
+struct HistPlan {
+    Plan plan;
+    bool fast;       // single slot through LDS
+    int copies;
+    int nblocks;
+    int64_t ntiles;
+    size_t off_mm_ws, off_bmin, off_bmax, off_ranges, off_carried, off_upd_edges, off_scratch, off_counts, total;
+};
+
+size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
+
+bool make_hist_plan(int dtype, const ahq_layout& layout, const void* x, int num_bins, HistPlan* hp) {
+    if (!make_plan(dtype, layout, aligned16(x), false, &hp->plan)) return false;
+    const CanonLayout& c = hp->plan.cl;
+    const int64_t S = c.num_enc;
+    hp->fast = false;
+    hp->copies = 0;
+    if (c.kind == kIJK && c.J == 1) {
+        int copies = (int)((65536 - 512) / ((size_t)2 * num_bins * 4));
+        if (copies > 4) copies = 4;
+        if (copies >= 1) {
+            hp->fast = true;
+            hp->copies = copies;
+        }
+    }
+    hp->ntiles = (hp->plan.nvec + kTileVec - 1) / kTileVec;
+    int64_t nb = hp->fast ? hp->ntiles : (c.numel + kBlock - 1) / kBlock;
+    if (nb > kHistBlocksMax) nb = kHistBlocksMax;
+    if (nb < 1) nb = 1;
+    hp->nblocks = (int)nb;
+    const size_t B = (size_t)num_bins;
+    size_t o = 0;
+    hp->off_mm_ws = o;     o = align_up(o + ahq_minmax_workspace_bytes(&layout));
+    hp->off_bmin = o;      o = align_up(o + (size_t)S * 4);
+    hp->off_bmax = o;      o = align_up(o + (size_t)S * 4);
+    hp->off_ranges = o;    o = align_up(o + (size_t)S * kRng * 4);
+    hp->off_carried = o;   o = align_up(o + (size_t)S * B * 4);
+    hp->off_upd_edges = o; o = align_up(o + (size_t)S * (B + 1) * 4);
+    hp->off_scratch = o;   o = align_up(o + (size_t)S * 2 * B * 4);
+    hp->off_counts = o;
+    const size_t nparts = hp->fast ? (size_t)hp->nblocks : 1;
+    o = align_up(o + (size_t)S * nparts * 2 * (B + 2) * 4);
+    hp->total = o;
+    return true;
+}
+
+}  // namespace
+
+extern "C" size_t ahq_hist_update_workspace_bytes(int32_t dtype, const ahq_layout* layout, int32_t num_bins) {
+    if (!layout || num_bins <= 0) return 0;
+    HistPlan hp;
+    size_t need = 0;
+    // the plan depends on pointer alignment only through the vector width; take the larger of the two
+    if (make_hist_plan(dtype, *layout, nullptr, num_bins, &hp)) need = hp.total;
+    if (make_hist_plan(dtype, *layout, reinterpret_cast<const void*>(4), num_bins, &hp) && hp.total > need) need = hp.total;
+    return need;
+}
+
+extern "C" int ahq_hist_update(int32_t dtype, const ahq_layout* layout, const void* x, const ahq_hist_state* st,
+                               int first_batch, void* workspace, size_t workspace_bytes, void* stream) {
+    if (dtype < AHQ_F32 || dtype > AHQ_BF16) return set_error("bad dtype"), AHQ_ERR_INVALID;
+    if (!layout || !st || !x) return set_error("null argument"), AHQ_ERR_INVALID;
+    if (st->num_bins <= 0) return set_error("num_bins must be positive"), AHQ_ERR_INVALID;
+    if (!st->hist || !st->edges || !st->minmax || !st->limits || !st->new_hist || !st->new_edges || !st->new_minmax)
+        return set_error("histogram state has a null buffer"), AHQ_ERR_INVALID;
+    if (!(st->growth_limit >= 1.0f)) return set_error("growth limit must be at least 1"), AHQ_ERR_INVALID;
+    HistPlan hp;
+    if (!make_hist_plan(dtype, *layout, x, st->num_bins, &hp)) return AHQ_ERR_INVALID;
+    const CanonLayout& c = hp.plan.cl;
+    if (c.numel == 0) return set_error("cannot observe an empty tensor"), AHQ_ERR_INVALID;
+    if (c.num_enc != st->num_slots) return set_error("layout does not have num_slots encodings"), AHQ_ERR_INVALID;
+    if (!workspace || workspace_bytes < hp.total) return set_error("workspace too small"), AHQ_ERR_WORKSPACE;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    char* w = static_cast<char*>(workspace);
+    const int S = st->num_slots, B = st->num_bins;
+    const int NH = first_batch ? 1 : 2;
+
+    // 1. finite range of the batch, in the tensor's dtype
+    int rc = ahq_minmax(dtype, layout, x, w + hp.off_bmin, w + hp.off_bmax, nullptr, nullptr, 1, w + hp.off_mm_ws,
+                        hp.off_bmin - hp.off_mm_ws, stream);
+    if (rc != AHQ_OK) return rc;
+
+    // 2. edges, updated range, re-binned running counts
+    PrepArgs pa{};
+    pa.num_slots = S;
+    pa.num_bins = B;
+    pa.first = first_batch ? 1 : 0;
+    pa.growth = st->growth_limit;
+    pa.bmin = w + hp.off_bmin;
+    pa.bmax = w + hp.off_bmax;
+    pa.hist = st->hist;
+    pa.edges = st->edges;
+    pa.minmax = st->minmax;
+    pa.limits = st->limits;
+    pa.new_edges = st->new_edges;
+    pa.new_minmax = st->new_minmax;
+    pa.carried = reinterpret_cast<float*>(w + hp.off_carried);
+    pa.upd_edges = reinterpret_cast<float*>(w + hp.off_upd_edges);
+    pa.ranges = reinterpret_cast<float*>(w + hp.off_ranges);
+    pa.scratch = reinterpret_cast<int32_t*>(w + hp.off_scratch);
+    const int pthreads = B >= 512 ? 512 : (B >= 64 ? ((B + 63) / 64) * 64 : 64);
+    switch (dtype) {
+        case AHQ_F32: hipLaunchKernelGGL((hist_prepare_kernel<float>), dim3(S), dim3(pthreads), 0, s, pa); break;
+        case AHQ_F16: hipLaunchKernelGGL((hist_prepare_kernel<f16_t>), dim3(S), dim3(pthreads), 0, s, pa); break;
+        default: hipLaunchKernelGGL((hist_prepare_kernel<bf16_t>), dim3(S), dim3(pthreads), 0, s, pa); break;
+    }
+
+    // 3. binning pass
+    BinArgs ba{};
+    fill_geom(hp.plan, &ba);
+    ba.x = x;
+    ba.ranges = pa.ranges;
+    ba.num_bins = B;
+    ba.nhist = NH;
+    ba.copies = hp.copies;
+    ba.ntiles = hp.ntiles;
+    uint32_t* counts = reinterpret_cast<uint32_t*>(w + hp.off_counts);
+    if (hp.fast) {
+        ba.partials = counts;
+        const size_t lds = (size_t)hp.copies * NH * B * 4;
+        const dim3 g(hp.nblocks), b(kBlock);
+#define AHQ_LAUNCH_BIN(IO)                                                                                          \
+    do {                                                                                                            \
+        if (hp.plan.vec == 1) {                                                                                     \
+            if (NH == 1) hipLaunchKernelGGL((hist_bin_kernel<IO, 1, 1>), g, b, lds, s, ba);                         \
+            else hipLaunchKernelGGL((hist_bin_kernel<IO, 1, 2>), g, b, lds, s, ba);                                 \
+        } else {                                                                                                    \
+            if (NH == 1) hipLaunchKernelGGL((hist_bin_kernel<IO, IoTraits<IO>::kVec, 1>), g, b, lds, s, ba);        \
+            else hipLaunchKernelGGL((hist_bin_kernel<IO, IoTraits<IO>::kVec, 2>), g, b, lds, s, ba);                \
+        }                                                                                                           \
+    } while (0)
+        switch (dtype) {
+            case AHQ_F32: AHQ_LAUNCH_BIN(float); break;
+            case AHQ_F16: AHQ_LAUNCH_BIN(f16_t); break;
+            default: AHQ_LAUNCH_BIN(bf16_t); break;
+        }
+#undef AHQ_LAUNCH_BIN
+    } else {
+        ba.counts = counts;
+        const int64_t n = (int64_t)S * NH * (B + 2);
+        hipLaunchKernelGGL(zero_u32_kernel, dim3((unsigned)((n + 255) / 256 > 1024 ? 1024 : (n + 255) / 256)), dim3(256), 0, s, counts, n);
+        switch (dtype) {
+            case AHQ_F32: hipLaunchKernelGGL((hist_bin_generic_kernel<float>), dim3(hp.nblocks), dim3(kBlock), 0, s, ba); break;
+            case AHQ_F16: hipLaunchKernelGGL((hist_bin_generic_kernel<f16_t>), dim3(hp.nblocks), dim3(kBlock), 0, s, ba); break;
+            default: hipLaunchKernelGGL((hist_bin_generic_kernel<bf16_t>), dim3(hp.nblocks), dim3(kBlock), 0, s, ba); break;
+        }
+    }
+
+    // 4. counts -> fp32 statistics
+    FinArgs fa{};
+    fa.num_slots = S;
+    fa.num_bins = B;
+    fa.nhist = NH;
+    fa.first = first_batch ? 1 : 0;
+    fa.nparts = hp.fast ? hp.nblocks : 1;
+    fa.counts = counts;
+    fa.carried = pa.carried;
+    fa.upd_edges = pa.upd_edges;
+    fa.hist = st->hist;
+    fa.edges = st->edges;
+    fa.new_hist = st->new_hist;
+    hipLaunchKernelGGL(hist_finish_kernel, dim3((B + 63) / 64, S), dim3(kBlock), 0, s, fa);
+    return check_launch("ahq_hist_update");
+}

@@ -11,7 +11,6 @@
 //   AHQ_ARITH_DLQ       clamp on the value, true division, round-half-away-from-zero     (fp32 math)
 // Built with -ffp-contract=off: fusing a multiply into an add would change the rounding of any of them.
 
-#include <atomic>
 #include <cstdio>
 
 #include "ahq_device.h"
@@ -154,7 +153,6 @@ struct QdqArgs : Geom {
     double* partials;  // kRedTile: [nblocks][2]; kRedAtomic: [num_enc][2]
     GridC gc;
     int32_t red;
-    int32_t ticket;
     int32_t out_cd;  // compute dtype the reduced gradients are rounded through
 };
 
@@ -265,7 +263,6 @@ template <typename IO, int VEC, typename M, int RED>
 __global__ __launch_bounds__(kBlock) void qdq_bwd_kernel(const QdqArgs a) {
     __shared__ float sp[M::kNP][kStage];
     __shared__ double red_smem[kBlock / kWave];
-    __shared__ int flag_smem;
     const Tile t = make_tile(a);
     stage_encodings<M>(a, t, sp);
     __syncthreads();
@@ -359,38 +356,44 @@ __global__ __launch_bounds__(kBlock) void qdq_bwd_kernel(const QdqArgs a) {
             a.partials[2 * (int64_t)blockIdx.x] = bs;
             a.partials[2 * (int64_t)blockIdx.x + 1] = bo;
         }
-        if (!last_block_done(a.ticket, a.nblocks, &flag_smem)) return;
-        // the last workgroup adds the partials of every encoding in a fixed order
-        if (a.mode != kRows) {
-            double s = 0.0, o = 0.0;
-            for (int64_t q = threadIdx.x; q < per_enc; q += kBlock) {
-                s += a.partials[2 * q];
-                o += a.partials[2 * q + 1];
-            }
-            s = block_reduce(s, OpAddD(), red_smem);
-            o = block_reduce(o, OpAddD(), red_smem);
-            if (threadIdx.x == 0) {
-                a.gscale[0] = finish_sum_rt(s, a.out_cd);
-                a.goffset[0] = finish_sum_rt(o, a.out_cd);
-            }
-        } else {
-            // one wave per encoding, lanes stride over that encoding's tiles
-            const int lane = threadIdx.x & (kWave - 1);
-            for (int64_t j = threadIdx.x / kWave; j < a.J; j += kBlock / kWave) {
-                double s = 0.0, o = 0.0;
-                for (int64_t q = lane; q < per_enc; q += kWave) {
-                    const int64_t i = q / a.tpr, tt = q - i * a.tpr;
-                    const int64_t blk = (i * a.J + j) * a.tpr + tt;
-                    s += a.partials[2 * blk];
-                    o += a.partials[2 * blk + 1];
-                }
-                s = wave_reduce(s, OpAddD());
-                o = wave_reduce(o, OpAddD());
-                if (lane == 0) {
-                    a.gscale[j] = finish_sum_rt(s, a.out_cd);
-                    a.goffset[j] = finish_sum_rt(o, a.out_cd);
-                }
-            }
+    }
+}
+
+// Adds the per-tile partial sums of every encoding in a fixed order (second launch: a kernel boundary makes the
+// partials visible without any in-kernel fence, which on a multi-die GPU would flush the L2 once per workgroup).
+__global__ __launch_bounds__(kBlock) void qdq_bwd_finish_kernel(const QdqArgs a) {
+    __shared__ double red_smem[kBlock / kWave];
+    const int64_t per_enc = a.mode == kRows ? a.I * (int64_t)a.tpr : (int64_t)a.nblocks;
+    if (a.mode != kRows) {
+        double s = 0.0, o = 0.0;
+        for (int64_t q = threadIdx.x; q < per_enc; q += kBlock) {
+            s += a.partials[2 * q];
+            o += a.partials[2 * q + 1];
+        }
+        s = block_reduce(s, OpAddD(), red_smem);
+        o = block_reduce(o, OpAddD(), red_smem);
+        if (threadIdx.x == 0) {
+            a.gscale[0] = finish_sum_rt(s, a.out_cd);
+            a.goffset[0] = finish_sum_rt(o, a.out_cd);
+        }
+        return;
+    }
+    // one wave per encoding, lanes stride over that encoding's tiles
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t wave0 = (int64_t)blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
+    for (int64_t j = wave0; j < a.J; j += (int64_t)gridDim.x * (kBlock / kWave)) {
+        double s = 0.0, o = 0.0;
+        for (int64_t q = lane; q < per_enc; q += kWave) {
+            const int64_t i = q / a.tpr, tt = q - i * a.tpr;
+            const int64_t blk = (i * a.J + j) * a.tpr + tt;
+            s += a.partials[2 * blk];
+            o += a.partials[2 * blk + 1];
+        }
+        s = wave_reduce(s, OpAddD());
+        o = wave_reduce(o, OpAddD());
+        if (lane == 0) {
+            a.gscale[j] = finish_sum_rt(s, a.out_cd);
+            a.goffset[j] = finish_sum_rt(o, a.out_cd);
         }
     }
 }
@@ -431,7 +434,6 @@ static void fill_args(const ahq_grid& grid, const Plan& p, QdqArgs* a) {
     a->gc.qmax = (float)grid.qmax;
     a->gc.zps = (float)grid.zero_point_shift;
     a->red = p.red;
-    a->ticket = next_ticket();
     a->out_cd = grid.compute_dtype;
 }
 
@@ -588,6 +590,13 @@ extern "C" int ahq_qdq_backward(const ahq_grid* grid, const ahq_layout* layout, 
         hipLaunchKernelGGL(zero_f64_kernel, dim3((unsigned)((n + 255) / 256 > 1024 ? 1024 : (n + 255) / 256)), dim3(256), 0, st, a.partials, n);
     }
     AHQ_IO_SWITCH(grid->io_dtype, AHQ_MATH_SWITCH(*grid, (launch_bwd<IO, M>(p, a, st))));
+    if (p.red == kRedTile) {
+        const int64_t per_enc = p.mode == kRows ? p.cl.I * (int64_t)p.tpr : (int64_t)p.nblocks;
+        if (per_enc > 1) {
+            const int64_t nb = p.mode == kRows ? (p.cl.J + 3) / 4 : 1;
+            hipLaunchKernelGGL(qdq_bwd_finish_kernel, dim3((unsigned)(nb > 4096 ? 4096 : nb)), dim3(kBlock), 0, st, a);
+        }
+    }
     if (p.red == kRedAtomic) {
         const int64_t n = p.cl.num_enc;
         hipLaunchKernelGGL(finish_atomic_kernel, dim3((unsigned)((n + 255) / 256 > 1024 ? 1024 : (n + 255) / 256)), dim3(256), 0, st,

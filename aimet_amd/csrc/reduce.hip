@@ -1,7 +1,7 @@
 // Minimum / maximum statistics in one pass over the tensor (both extrema from the same read).
 //
 // Per-lane running min/max over 16-byte vectors -> wave64 shuffle tree -> LDS across the four waves of a workgroup ->
-// per-tile partials that the last workgroup to finish folds together, so a calibration call is a single launch.
+// per-tile partials that a second, one-workgroup launch folds together.
 // NaN handling follows torch.amin/amax (any NaN in a slice makes that slice's result NaN) unless `finite_only`, which
 // reproduces the histogram observer's range (non-finite values ignored).
 
@@ -22,9 +22,9 @@ struct MmArgs : Geom {
     unsigned int* key_min;  // kRedAtomic: [num_enc] order-preserving keys
     unsigned int* key_max;
     int32_t red;
-    int32_t ticket;
+    void* run_min;          // optional running statistics folded with torch.minimum / torch.maximum semantics
+    void* run_max;
     int32_t finite_only;
-    int32_t running;
 };
 
 struct MinMax {
@@ -71,16 +71,18 @@ __device__ __forceinline__ void mm_write(const MmArgs& a, int64_t e, MinMax m) {
     IO* omn = static_cast<IO*>(a.out_min);
     IO* omx = static_cast<IO*>(a.out_max);
     const float qnan = __builtin_nanf("");
-    float mn = m.nan ? qnan : m.mn;
-    float mx = m.nan ? qnan : m.mx;
-    if (a.running) {
-        // torch.minimum / torch.maximum: NaN in either operand wins
-        const float pmn = load_f32(omn[e]), pmx = load_f32(omx[e]);
-        mn = (pmn != pmn || mn != mn) ? qnan : fminf(pmn, mn);
-        mx = (pmx != pmx || mx != mx) ? qnan : fmaxf(pmx, mx);
-    }
+    const float mn = m.nan ? qnan : m.mn;
+    const float mx = m.nan ? qnan : m.mx;
     omn[e] = store_cast<IO>(mn);
     omx[e] = store_cast<IO>(mx);
+    if (a.run_min) {
+        // torch.minimum / torch.maximum: NaN in either operand wins
+        IO* rmn = static_cast<IO*>(a.run_min);
+        IO* rmx = static_cast<IO*>(a.run_max);
+        const float pmn = load_f32(rmn[e]), pmx = load_f32(rmx[e]);
+        rmn[e] = store_cast<IO>((pmn != pmn || mn != mn) ? qnan : fminf(pmn, mn));
+        rmx[e] = store_cast<IO>((pmx != pmx || mx != mx) ? qnan : fmaxf(pmx, mx));
+    }
 }
 
 __device__ __forceinline__ unsigned int f32_key(float f) {
@@ -94,7 +96,6 @@ __device__ __forceinline__ float key_f32(unsigned int k) {
 template <typename IO, int VEC, int RED>
 __global__ __launch_bounds__(kBlock) void minmax_kernel(const MmArgs a) {
     __shared__ MinMax red_smem[kBlock / kWave];
-    __shared__ int flag_smem;
     const Tile t = make_tile(a);
     const IO* __restrict__ x = static_cast<const IO*>(a.x);
     const bool fo = a.finite_only != 0;
@@ -157,26 +158,33 @@ __global__ __launch_bounds__(kBlock) void minmax_kernel(const MmArgs a) {
             a.part_max[blockIdx.x] = b.mx;
             a.part_nan[blockIdx.x] = b.nan;
         }
-        if (!last_block_done(a.ticket, a.nblocks, &flag_smem)) return;
-        if (a.mode != kRows) {
-            MinMax s = mm_identity();
-            for (int64_t q = threadIdx.x; q < per_enc; q += kBlock) s = mm_merge(s, MinMax{a.part_min[q], a.part_max[q], a.part_nan[q]});
-            s = mm_block_reduce(s, red_smem);
-            if (threadIdx.x == 0) mm_write<IO>(a, 0, s);
-        } else {
-            const int lane = threadIdx.x & (kWave - 1);
-            for (int64_t j = threadIdx.x / kWave; j < a.J; j += kBlock / kWave) {
-                MinMax s = mm_identity();
-                for (int64_t q = lane; q < per_enc; q += kWave) {
-                    const int64_t i = q / a.tpr, tt = q - i * a.tpr;
-                    const int64_t blk = (i * a.J + j) * a.tpr + tt;
-                    s = mm_merge(s, MinMax{a.part_min[blk], a.part_max[blk], a.part_nan[blk]});
-                }
-#pragma unroll
-                for (int m = kWave / 2; m >= 1; m >>= 1) s = mm_merge(s, mm_shfl_xor(s, m));
-                if (lane == 0) mm_write<IO>(a, j, s);
-            }
+    }
+}
+
+// Folds the per-tile partials of every encoding (second launch; see the note on fences in qdq.hip).
+template <typename IO>
+__global__ __launch_bounds__(kBlock) void minmax_finish_kernel(const MmArgs a) {
+    __shared__ MinMax red_smem[kBlock / kWave];
+    const int64_t per_enc = a.mode == kRows ? a.I * (int64_t)a.tpr : (int64_t)a.nblocks;
+    if (a.mode != kRows) {
+        MinMax s = mm_identity();
+        for (int64_t q = threadIdx.x; q < per_enc; q += kBlock) s = mm_merge(s, MinMax{a.part_min[q], a.part_max[q], a.part_nan[q]});
+        s = mm_block_reduce(s, red_smem);
+        if (threadIdx.x == 0) mm_write<IO>(a, 0, s);
+        return;
+    }
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t wave0 = (int64_t)blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
+    for (int64_t j = wave0; j < a.J; j += (int64_t)gridDim.x * (kBlock / kWave)) {
+        MinMax s = mm_identity();
+        for (int64_t q = lane; q < per_enc; q += kWave) {
+            const int64_t i = q / a.tpr, tt = q - i * a.tpr;
+            const int64_t blk = (i * a.J + j) * a.tpr + tt;
+            s = mm_merge(s, MinMax{a.part_min[blk], a.part_max[blk], a.part_nan[blk]});
         }
+#pragma unroll
+        for (int m = kWave / 2; m >= 1; m >>= 1) s = mm_merge(s, mm_shfl_xor(s, m));
+        if (lane == 0) mm_write<IO>(a, j, s);
     }
 }
 
@@ -223,6 +231,11 @@ static void launch_mm(const Plan& p, const MmArgs& a, hipStream_t st) {
         hipLaunchKernelGGL((minmax_generic_kernel<IO>), dim3(p.nblocks), dim3(kBlock), 0, st, a);
     } else if (p.red == kRedTile) {
         launch_mm_red<IO, kRedTile>(p, a, st);
+        const int64_t per_enc = p.mode == kRows ? p.cl.I * (int64_t)p.tpr : (int64_t)p.nblocks;
+        if (per_enc > 1) {
+            const int64_t nb = p.mode == kRows ? (p.cl.J + 3) / 4 : 1;
+            hipLaunchKernelGGL((minmax_finish_kernel<IO>), dim3((unsigned)(nb > 4096 ? 4096 : nb)), dim3(kBlock), 0, st, a);
+        }
     } else if (p.red == kRedSeg) {
         launch_mm_red<IO, kRedSeg>(p, a, st);
     } else {
@@ -248,10 +261,12 @@ extern "C" size_t ahq_minmax_workspace_bytes(const ahq_layout* layout) {
 }
 
 extern "C" int ahq_minmax(int32_t dtype, const ahq_layout* layout, const void* x, void* out_min, void* out_max,
-                          int finite_only, int running, void* workspace, size_t workspace_bytes, void* stream) {
+                          void* run_min, void* run_max, int finite_only, void* workspace, size_t workspace_bytes,
+                          void* stream) {
     if (dtype < AHQ_F32 || dtype > AHQ_BF16) return set_error("bad dtype"), AHQ_ERR_INVALID;
     if (!layout) return set_error("layout is null"), AHQ_ERR_INVALID;
     if (!out_min || !out_max) return set_error("out_min or out_max is null"), AHQ_ERR_INVALID;
+    if ((run_min == nullptr) != (run_max == nullptr)) return set_error("run_min and run_max must be given together"), AHQ_ERR_INVALID;
     Plan p;
     if (!make_plan(dtype, *layout, aligned16(x), true, &p)) return AHQ_ERR_INVALID;
     if (p.cl.numel == 0) return set_error("cannot reduce an empty tensor"), AHQ_ERR_INVALID;
@@ -266,9 +281,9 @@ extern "C" int ahq_minmax(int32_t dtype, const ahq_layout* layout, const void* x
     a.out_min = out_min;
     a.out_max = out_max;
     a.red = p.red;
-    a.ticket = next_ticket();
+    a.run_min = run_min;
+    a.run_max = run_max;
     a.finite_only = finite_only;
-    a.running = running;
     if (uses_ws) {
         char* w = static_cast<char*>(workspace);
         a.part_min = reinterpret_cast<float*>(w);

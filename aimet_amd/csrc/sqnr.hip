@@ -1,0 +1,203 @@
+// SQNR / TF-enhanced encoding search over a histogram (aimet_torch/quantization/encoding_analyzer.py:695-899).
+//
+// The (histogram, delta, offset, bin) tensor of the reference is never materialised: one workgroup owns one
+// (histogram, delta) row, its waves take the offset candidates in turn, lanes stride over the bins with the histogram
+// and bin mid-points held in LDS, and the clipping/quantisation noise of a candidate is accumulated in fp64.  A second
+// single-workgroup launch per histogram picks the first minimum and writes the encoding.
+//
+// Candidate generation repeats the reference's fp32 operations one by one (encoding_analyzer.py:728-820); the only
+// host-made input is the rounded offset grid, because torch.arange computes it in double precision on the CPU.
+
+#include "ahq_device.h"
+#include "ahq_host.h"
+
+namespace ahq {
+
+struct SqnrArgs {
+    int32_t num_slots, num_bins, num_deltas, num_offsets;  // num_offsets counts the observed offset (asymmetric)
+    int32_t symmetric;
+    int32_t stat_dtype;     // dtype the stored min/max live in (arithmetic on them happens in that dtype)
+    float num_steps;
+    float min_scale;        // minimum_scale as float
+    float min_range;        // float(minimum_scale * num_steps)
+    float sym_offset;       // (-num_steps) // 2
+    float gamma;
+    float p;
+    const float* hist;      // [S][B]
+    const float* edges;     // [S][B+1]
+    const float* minmax;    // [S][2]
+    const float* offset_grid;  // [num_offsets - 1] rounded offsets (asymmetric)
+    float* noise;           // [S][D][O]
+    float* deltas;          // [S][D][O] clamped candidates
+    float* offsets;         // [S][D][O]
+    float* out;             // [S][4]: best delta, best offset, encoding min, encoding max
+    long long* best_index;  // [S]
+};
+
+__device__ __forceinline__ float rnd_rt(float v, int dt) {
+    if (dt == AHQ_BF16) return rnd<AHQ_BF16>(v);
+    if (dt == AHQ_F16) return rnd<AHQ_F16>(v);
+    return v;
+}
+
+struct Cand {
+    float delta, offset;
+};
+
+// (delta, offset) of candidate (d, o) for histogram s, after clamping to the observed range.
+__device__ __forceinline__ Cand candidate(const SqnrArgs& a, int s, int d, int o) {
+    const int dt = a.stat_dtype;
+    float lo = a.minmax[2 * s], hi = a.minmax[2 * s + 1];
+    lo = fminf(lo, 0.f);
+    hi = fmaxf(hi, 0.f);
+    hi = fmaxf(hi, rnd_rt(lo + a.min_range, dt));
+    Cand c;
+    if (a.symmetric) {
+        const float dmax = (2.f * fmaxf(hi, -lo)) / a.num_steps;
+        c.delta = fmaxf((dmax * (float)(d + 1)) / (float)(a.num_deltas - 1), a.min_scale);
+        c.offset = a.sym_offset;
+        return c;
+    }
+    const float dmax = rnd_rt(hi - lo, dt) / a.num_steps;
+    const float obs_off = __builtin_rintf(lo / dmax);
+    const float obs_min = dmax * obs_off;
+    const float obs_max = obs_min + dmax * a.num_steps;
+    const float td = (dmax * (float)(d + 1)) / (float)(a.num_deltas - 1);
+    const float to = o < a.num_offsets - 1 ? a.offset_grid[o] : obs_off;
+    float tmin = td * to;
+    float tmax = tmin + td * a.num_steps;
+    tmin = fmaxf(obs_min, tmin);
+    tmax = fminf(obs_max, tmax);
+    c.delta = fmaxf((tmax - tmin) / a.num_steps, a.min_scale);
+    c.offset = __builtin_rintf(tmin / c.delta);
+    return c;
+}
+
+constexpr int kSqnrMaxBins = 4096;
+
+__global__ __launch_bounds__(kBlock) void sqnr_noise_kernel(const SqnrArgs a) {
+    __shared__ float h_lds[kSqnrMaxBins];
+    __shared__ float m_lds[kSqnrMaxBins];
+    const int s = blockIdx.y, d = blockIdx.x;
+    const int B = a.num_bins, O = a.num_offsets;
+    const float* e = a.edges + (size_t)s * (B + 1);
+    const float w = e[1] - e[0];
+    const float first_mid = e[0] + w / 2.f;
+    for (int b = threadIdx.x; b < B; b += kBlock) {
+        h_lds[b] = a.hist[(size_t)s * B + b];
+        m_lds[b] = first_mid + w * (float)b;
+    }
+    __syncthreads();
+    const int lane = threadIdx.x & (kWave - 1);
+    const bool use_gamma = a.gamma != 1.0f;
+    for (int o = threadIdx.x / kWave; o < O; o += kBlock / kWave) {
+        const Cand c = candidate(a, s, d, o);
+        double acc = 0.0;
+        for (int b = lane; b < B; b += kWave) {
+            const float mid = m_lds[b];
+            float q = __builtin_rintf(mid / c.delta - c.offset);
+            const bool clipped = (q < 0.f) | (q > a.num_steps);
+            q = q < 0.f ? 0.f : (q > a.num_steps ? a.num_steps : q);
+            const float y = (q + c.offset) * c.delta;
+            const float ad = __builtin_fabsf(y - mid);
+            float err = (a.p == 2.0f ? ad * ad : __builtin_powf(ad, a.p)) * h_lds[b];
+            if (use_gamma && clipped) err = err * a.gamma;
+            acc += (double)err;
+        }
+        acc = wave_reduce(acc, OpAddD());
+        if (lane == 0) {
+            const size_t i = ((size_t)s * a.num_deltas + d) * O + o;
+            a.noise[i] = (float)acc;
+            a.deltas[i] = c.delta;
+            a.offsets[i] = c.offset;
+        }
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void sqnr_select_kernel(const SqnrArgs a) {
+    __shared__ float v_sm[kBlock];
+    __shared__ int i_sm[kBlock];
+    const int s = blockIdx.x;
+    const int n = a.num_deltas * a.num_offsets;
+    const float* noise = a.noise + (size_t)s * n;
+    // first minimum; NaN never wins unless everything is NaN
+    float best = __builtin_inff();
+    int bi = n;
+    for (int i = threadIdx.x; i < n; i += kBlock) {
+        const float v = noise[i];
+        if (v < best) {
+            best = v;
+            bi = i;
+        }
+    }
+    v_sm[threadIdx.x] = best;
+    i_sm[threadIdx.x] = bi;
+    __syncthreads();
+    for (int st = kBlock / 2; st >= 1; st >>= 1) {
+        if (threadIdx.x < st) {
+            const float ov = v_sm[threadIdx.x + st];
+            const int oi = i_sm[threadIdx.x + st];
+            if (ov < v_sm[threadIdx.x] || (ov == v_sm[threadIdx.x] && oi < i_sm[threadIdx.x])) {
+                v_sm[threadIdx.x] = ov;
+                i_sm[threadIdx.x] = oi;
+            }
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        int idx = i_sm[0];
+        if (idx >= n) idx = 0;
+        const float delta = a.deltas[(size_t)s * n + idx];
+        const float off = a.offsets[(size_t)s * n + idx];
+        const float mn = off * delta;
+        const float mx = mn + a.num_steps * delta;
+        a.out[4 * s] = delta;
+        a.out[4 * s + 1] = off;
+        a.out[4 * s + 2] = mn;
+        a.out[4 * s + 3] = mx;
+        a.best_index[s] = idx;
+    }
+}
+
+}  // namespace ahq
+
+using namespace ahq;
+
+extern "C" int ahq_sqnr_search(const ahq_sqnr_params* p, const float* hist, const float* edges, const float* minmax,
+                               const float* offset_grid, float* noise, float* deltas, float* offsets, float* out,
+                               long long* best_index, void* stream) {
+    if (!p || !hist || !edges || !minmax || !noise || !deltas || !offsets || !out || !best_index)
+        return set_error("null argument"), AHQ_ERR_INVALID;
+    if (p->num_slots <= 0 || p->num_deltas <= 1 || p->num_offsets <= 0) return set_error("bad candidate grid"), AHQ_ERR_INVALID;
+    if (p->num_bins <= 1 || p->num_bins > kSqnrMaxBins) return set_error("num_bins must be in [2, 4096]"), AHQ_ERR_UNSUPPORTED;
+    if (p->num_steps <= 0) return set_error("num_steps must be positive"), AHQ_ERR_INVALID;
+    if (!p->symmetric && (p->num_offsets < 2 || !offset_grid)) return set_error("asymmetric search needs an offset grid"), AHQ_ERR_INVALID;
+    if (p->stat_dtype < AHQ_F32 || p->stat_dtype > AHQ_BF16) return set_error("bad stat_dtype"), AHQ_ERR_INVALID;
+    SqnrArgs a{};
+    a.num_slots = p->num_slots;
+    a.num_bins = p->num_bins;
+    a.num_deltas = p->num_deltas;
+    a.num_offsets = p->symmetric ? 1 : p->num_offsets;
+    a.symmetric = p->symmetric;
+    a.stat_dtype = p->stat_dtype;
+    a.num_steps = (float)p->num_steps;
+    a.min_scale = (float)p->minimum_scale;
+    a.min_range = (float)(p->minimum_scale * (double)p->num_steps);
+    // Python floor division of -num_steps by 2
+    a.sym_offset = (float)(-((p->num_steps + 1) / 2));
+    a.gamma = (float)p->gamma;
+    a.p = (float)p->p;
+    a.hist = hist;
+    a.edges = edges;
+    a.minmax = minmax;
+    a.offset_grid = offset_grid;
+    a.noise = noise;
+    a.deltas = deltas;
+    a.offsets = offsets;
+    a.out = out;
+    a.best_index = best_index;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    hipLaunchKernelGGL(sqnr_noise_kernel, dim3(a.num_deltas, a.num_slots), dim3(kBlock), 0, st, a);
+    hipLaunchKernelGGL(sqnr_select_kernel, dim3(a.num_slots), dim3(kBlock), 0, st, a);
+    return check_launch("ahq_sqnr_search");
+}

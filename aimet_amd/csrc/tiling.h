@@ -2,8 +2,6 @@
 // Shared by the fake-quantization kernels and the statistics kernels.
 #pragma once
 
-#include <atomic>
-
 #include "ahq_device.h"
 #include "ahq_host.h"
 #include "layout.h"
@@ -12,8 +10,8 @@ namespace ahq {
 
 enum TileMode : int { kFlat = 0, kRows = 1 };
 // How per-encoding reductions leave the kernel:
-//   kRedTile    every tile lies inside one run; workgroup totals go to a partials array (or straight to the output
-//               when one tile covers the whole encoding) and the last workgroup adds them in a fixed order
+//   kRedTile    every tile lies inside one run; workgroup totals go straight to the output when one tile covers the
+//               whole encoding, else to a partials array that a second small launch adds in a fixed order
 //   kRedSeg     a run is a power-of-two number (<= 64) of neighbouring lanes: shuffle reduction, direct store
 //   kRedAtomic  anything else: atomics into a per-encoding scratch array, finished by a second tiny kernel
 enum RedMode : int { kRedNone = 0, kRedTile = 1, kRedSeg = 2, kRedAtomic = 3 };
@@ -105,11 +103,6 @@ inline int io_vec(int dtype) { return dtype == AHQ_F32 ? 4 : 8; }
 inline size_t io_size(int dtype) { return dtype == AHQ_F32 ? 4 : 2; }
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 inline bool is_pow2(int64_t v) { return v > 0 && (v & (v - 1)) == 0; }
-
-inline int next_ticket() {
-    static std::atomic<unsigned> rr{0};
-    return (int)(rr.fetch_add(1) % kTicketSlots);
-}
 
 // Decide tiling and reduction strategy.  `ptr_aligned`: every tensor pointer is 16-byte aligned.
 inline bool make_plan(int io_dtype, const ahq_layout& layout, bool ptr_aligned, bool want_red, Plan* p) {

@@ -32,8 +32,9 @@ def reduce_min_max(x: torch.Tensor, shape: Tuple[int, ...], block_size=None, *, 
     """Per-encoding minimum and maximum of ``x`` in one pass (both extrema from a single read of the tensor).
 
     Equivalent of ``reduce(x, shape, torch.amin, block_size)`` and ``reduce(x, shape, torch.amax, block_size)``
-    (aimet_torch/utils.py:1115-1148, aimet_torch/quantization/encoding_analyzer.py:80-94).  With ``running`` the
-    results are folded into the given (min, max) tensors in place, as ``_MinMaxObserver.merge_stats`` does.
+    (aimet_torch/utils.py:1115-1148, aimet_torch/quantization/encoding_analyzer.py:80-94).  The batch result is
+    returned; with ``running`` it is also folded into the given (min, max) tensors in place, as
+    ``_MinMaxObserver.merge_stats`` does.
     """
     _lib.require_device(x, "input tensor")
     if x.dtype not in _lib.DTYPE_CODE:
@@ -44,18 +45,20 @@ def reduce_min_max(x: torch.Tensor, shape: Tuple[int, ...], block_size=None, *, 
         raise RuntimeError("cannot reduce an empty tensor")
     lib = _lib.load()
     xd, layout = _prepare(x.detach(), shape, block_size)
+    rmn = rmx = None
     if running is not None:
-        mn, mx = running
-        if mn.dtype != x.dtype or not mn.is_contiguous() or not mx.is_contiguous() or tuple(mn.shape) != shape:
-            raise RuntimeError("running statistics must be contiguous tensors of the observer shape and input dtype")
-    else:
-        mn = torch.empty(shape, dtype=x.dtype, device=x.device)
-        mx = torch.empty(shape, dtype=x.dtype, device=x.device)
+        rmn, rmx = running
+        for r in (rmn, rmx):
+            if r.dtype != x.dtype or not r.is_contiguous() or tuple(r.shape) != shape or r.device != x.device:
+                raise RuntimeError("running statistics must be contiguous tensors of the observer shape, on the "
+                                   "input's device and of its dtype")
+    mn = torch.empty(shape, dtype=x.dtype, device=x.device)
+    mx = torch.empty(shape, dtype=x.dtype, device=x.device)
     nbytes = lib.ahq_minmax_workspace_bytes(layout)
     ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device) if nbytes else None
     _lib.check(
         lib.ahq_minmax(_lib.DTYPE_CODE[x.dtype], layout, xd.data_ptr(), mn.data_ptr(), mx.data_ptr(),
-                       1 if finite_only else 0, 1 if running is not None else 0, _lib.ptr(ws), nbytes,
+                       _lib.ptr(rmn), _lib.ptr(rmx), 1 if finite_only else 0, _lib.ptr(ws), nbytes,
                        _lib.current_stream(x.device)),
         "ahq_minmax",
     )

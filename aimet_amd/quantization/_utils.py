@@ -125,3 +125,16 @@ class _RoundSTE(torch.autograd.Function):
 def ste_round(x: torch.Tensor) -> torch.Tensor:
     """round() whose gradient is the identity."""
     return _RoundSTE.apply(x)
+
+
+def true_divide(t: torch.Tensor, value: float) -> torch.Tensor:
+    """``t / value`` with IEEE division on any device.
+
+    Dividing a GPU tensor by a Python number is evaluated by torch as a multiplication with the reciprocal, which is
+    one unit in the last place off for some operands; dividing by a 0-dim device tensor is a true division.  16-bit
+    tensors are divided in float32 and rounded once, which is what the CPU path does for ``tensor / number``.
+    """
+    divisor = torch.full((), float(value), dtype=torch.float32, device=t.device)
+    if t.dtype == torch.float32:
+        return t / divisor
+    return (t.to(torch.float32) / divisor).to(t.dtype)

@@ -1,0 +1,492 @@
+"""Affine quantizer modules: ``Quantize``, ``QuantizeDequantize``, ``Dequantize``, ``GroupedBlockQuantizeDequantize``.
+
+API-compatible counterparts of aimet_torch/quantization/affine/quantizer.py (constructor overloads, learnable
+``min`` / ``max`` parameters, ``get_scale`` / ``get_offset`` / ``get_min`` / ``get_max`` / ``set_range`` /
+``get_encodings``, the ``compute_encodings()`` context manager, ``allow_overwrite``, extra state for checkpoints).
+Tensor work is done by the HIP backend and the HIP encoding analyzers.  Quantizers here are parametrised by min/max;
+the reference's alternative scale/offset parametrisation is not part of this package.
+"""
+
+# pylint: disable=redefined-builtin
+
+from __future__ import annotations
+
+import functools
+from contextlib import contextmanager, nullcontext
+from typing import Optional, Tuple
+
+import torch
+from torch import nn
+
+from aimet_amd.quantization._utils import (
+    StatisticsNotFoundError,
+    _get_minimum_scale,
+    _is_expandable,
+    concretize_block_size,
+    interleave,
+    patch_attr,
+    ste_round,
+    true_divide,
+)
+from aimet_amd.quantization.affine._utils import _GridMixin
+from aimet_amd.quantization.affine.backends import quantize, quantize_dequantize, dequantize, _derive_qmin_qmax
+from aimet_amd.quantization.affine.encoding import AffineEncoding, GroupedBlockEncoding
+from aimet_amd.quantization.base.quantizer import QuantizerBase
+from aimet_amd.quantization.encoding_analyzer import EncodingAnalyzer, MinMaxEncodingAnalyzer, _flag_extreme_min_max
+from aimet_amd.quantization.tensor import QuantizedTensor, DequantizedTensor
+
+__all__ = ["AffineQuantizerBase", "Quantize", "QuantizeDequantize", "Dequantize", "GroupedBlockQuantizeDequantize"]
+
+
+def _symmetric_offset(qmin: int, qmax: int, shape, dtype, device) -> torch.Tensor:
+    """Constant offset of a symmetric grid (quantizer.py:843-850).  The value is also attached as a Python attribute
+    so that the backend can reason about it without reading device memory."""
+    value = -round((qmin + qmax) / 2)
+    off = torch.full(tuple(shape), fill_value=value, requires_grad=False, dtype=dtype, device=device)
+    off._ahq_constant = value  # pylint: disable=protected-access
+    return off
+
+
+def _get_scale_offset(min: torch.Tensor, max: torch.Tensor, qmin: int, qmax: int, symmetric: bool):
+    """scale = (max - min) / (qmax - qmin); offset = round(min / scale) - qmin, or the symmetric constant
+    (quantizer.py:876-900)."""
+    num_steps = qmax - qmin
+    if not isinstance(min, torch.Tensor):
+        min = torch.tensor(min, dtype=torch.float32)
+    if not isinstance(max, torch.Tensor):
+        max = torch.tensor(max, dtype=torch.float32)
+    out_dtype = min.dtype
+    min = min.to(torch.float32)
+    max = max.to(torch.float32)
+    scale = true_divide(max - min, num_steps)
+    if symmetric:
+        offset = _symmetric_offset(qmin, qmax, min.shape, min.dtype, min.device)
+    else:
+        offset = ste_round(min / scale) - qmin
+    return scale.to(out_dtype), offset.to(out_dtype)
+
+
+class AffineQuantizerBase(QuantizerBase, _GridMixin):
+    """Base class of the affine quantizers.
+
+    ``(shape, bitwidth, symmetric, encoding_analyzer=None, block_size=None, zero_point_shift=None)`` or
+    ``(shape, qmin, qmax, symmetric, encoding_analyzer=None, block_size=None, zero_point_shift=None)``.
+    """
+
+    def __init__(self, shape, *args, **kwargs):
+        super().__init__()
+        if isinstance(shape, int):
+            shape = (shape,)
+        self.shape = tuple(shape)
+        pos = tuple(args) + (None,) * (6 - len(args))
+        first = kwargs.pop("qmin", kwargs.pop("bitwidth", pos[0]))
+        second = kwargs.pop("qmax", pos[1])
+        if second is not None and not isinstance(second, bool):
+            qmin, qmax = first, second
+            symmetric = kwargs.pop("symmetric", pos[2])
+            rest = pos[3:6]
+        else:
+            symmetric = kwargs.pop("symmetric", pos[1])
+            if first is None or symmetric is None:
+                raise TypeError("expected (shape, bitwidth, symmetric, ...) or (shape, qmin, qmax, symmetric, ...)")
+            qmin, qmax = _derive_qmin_qmax(bitwidth=first, signed=symmetric)
+            rest = pos[2:5]
+        if qmin is None or qmax is None or symmetric is None:
+            raise TypeError("expected (shape, bitwidth, symmetric, ...) or (shape, qmin, qmax, symmetric, ...)")
+        encoding_analyzer = kwargs.pop("encoding_analyzer", rest[0])
+        block_size = kwargs.pop("block_size", rest[1])
+        zero_point_shift = kwargs.pop("zero_point_shift", rest[2])
+        if kwargs:
+            raise TypeError(f"{type(self).__qualname__}.__init__ got unexpected keyword argument: {', '.join(kwargs)}")
+        if qmin >= qmax:
+            raise ValueError(f"qmax should be strictly larger than qmin. Got qmax={qmax}, qmin={qmin}")
+
+        self.qmin = qmin
+        self.qmax = qmax
+        self._symmetric = symmetric
+        self.block_size = block_size
+        self.zero_point_shift = zero_point_shift or 0.0
+        if self.zero_point_shift not in (0.0, 0.5):
+            raise ValueError(f"zero_point_shift should be 0.0 or 0.5. Got {self.zero_point_shift}")
+
+        self.encoding_analyzer: EncodingAnalyzer = encoding_analyzer or MinMaxEncodingAnalyzer(
+            shape=self.shape, block_size=self.block_size
+        )
+        if not _is_expandable(self.encoding_analyzer.observer.shape, self.shape):
+            raise RuntimeError(
+                f"Encoding analyzer of shape {self.encoding_analyzer.observer.shape} "
+                f"is incompatible with quantizer of shape {self.shape}."
+            )
+
+        self.register_quantization_parameter("min", nn.Parameter(-torch.ones(self.shape)))
+        self.register_quantization_parameter("max", nn.Parameter(torch.ones(self.shape)))
+        self._is_overwrite_allowed.update({"min": True, "max": True})
+
+    # ------------------------------------------------------------------------------------- derived quantities --
+    def get_scale(self, dtype=None) -> Optional[torch.Tensor]:
+        """|max - min| / (qmax - qmin), floored at the minimum scale; None before initialisation
+        (quantizer.py:319-342)."""
+        if not self.is_initialized():
+            return None
+        dtype = dtype or torch.float32
+        num_steps = self.qmax - self.qmin
+        scale = true_divide(self.max.to(dtype) - self.min.to(dtype), num_steps)
+        return scale.abs().clamp_min_(_get_minimum_scale(num_steps)).to(dtype)
+
+    def get_offset(self, dtype=None) -> Optional[torch.Tensor]:
+        return self._get_offset(dtype=dtype)
+
+    def _get_offset(self, scale=None, dtype=None) -> Optional[torch.Tensor]:
+        """clamp(round(min / scale) - qmin, -qmax, -qmin), or the symmetric constant (quantizer.py:357-376)."""
+        if not self.is_initialized():
+            return None
+        dtype = dtype or torch.float32
+        if self.symmetric:
+            device = next(p.device for p in self.parameters())
+            return _symmetric_offset(self.qmin, self.qmax, self.shape, dtype, device)
+        scale = scale if scale is not None else self.get_scale(dtype)
+        offset = torch.clamp(ste_round(self.min / scale) - self.qmin, -self.qmax, -self.qmin)
+        return offset.to(dtype)
+
+    def get_min(self, dtype=None) -> Optional[torch.Tensor]:
+        if not self.is_initialized():
+            return None
+        return self.get_scale(dtype) * (self.get_offset(dtype) + self.qmin + self.zero_point_shift)
+
+    def get_max(self, dtype=None) -> Optional[torch.Tensor]:
+        if not self.is_initialized():
+            return None
+        return self.get_scale(dtype) * (self.get_offset(dtype) + self.qmax + self.zero_point_shift)
+
+    @torch.no_grad()
+    def set_range(self, min, max):
+        """Assign the encoding range; ``None`` leaves that end untouched (quantizer.py:378-438)."""
+        if min is None and max is None:
+            return
+        if min is not None:
+            self.min.copy_(min if isinstance(min, torch.Tensor) else torch.tensor(min))
+        if max is not None:
+            self.max.copy_(max if isinstance(max, torch.Tensor) else torch.tensor(max))
+
+    def get_encodings(self) -> Optional[AffineEncoding]:
+        scale = self.get_scale(dtype=torch.float32)
+        offset = self._get_offset(scale=scale, dtype=torch.float32)
+        if scale is None or offset is None:
+            return None
+        return AffineEncoding(scale, offset, self.qmin, self.qmax, self._symmetric, self.block_size,
+                              self.zero_point_shift, producer=self)
+
+    @classmethod
+    def from_encodings(cls, encodings: AffineEncoding) -> "AffineQuantizerBase":
+        if not isinstance(encodings, AffineEncoding):
+            raise TypeError(f"Expected {AffineEncoding}; got {type(encodings)}")
+        qtzr = cls(shape=encodings.scale.shape, qmin=encodings.qmin, qmax=encodings.qmax,
+                   symmetric=encodings.symmetry, block_size=encodings.block_size,
+                   zero_point_shift=encodings.zero_point_shift)
+        qtzr.to(encodings.scale.device)
+        qtzr.set_range(encodings.min, encodings.max)
+        return qtzr
+
+    def extra_repr(self) -> str:
+        parts = [f"shape={self.shape}"]
+        if self.block_size:
+            parts.append(f"block_size={self.block_size}")
+        parts += [f"qmin={self.qmin}", f"qmax={self.qmax}", f"symmetric={self.symmetric}"]
+        if self.zero_point_shift:
+            parts.append(f"zero_point_shift={self.zero_point_shift}")
+        return ", ".join(parts)
+
+    @property
+    def symmetric(self) -> bool:
+        return self._symmetric
+
+    @symmetric.setter
+    def symmetric(self, symmetric: bool):
+        self._symmetric = symmetric
+
+    @property
+    def bitwidth(self) -> int:
+        return self._get_bitwidth()
+
+    @bitwidth.setter
+    def bitwidth(self, bitwidth: int):
+        self._set_bitwidth(bitwidth)
+
+    @property
+    def signed(self) -> bool:
+        return self._get_signed()
+
+    @signed.setter
+    def signed(self, signed: bool):
+        self._set_signed(signed)
+
+    # --------------------------------------------------------------------------------------------- calibration --
+    @contextmanager
+    def compute_encodings(self):
+        """Observe inputs and set min/max from their statistics on exit.  Inside the context the forward pass
+        quantizes dynamically with the statistics of the current input (quantizer.py:591-599)."""
+        with self._compute_encodings(passthrough=False):
+            yield
+
+    def _num_steps_for_calibration(self) -> int:
+        n = self.qmax - self.qmin
+        return n - 1 if self.zero_point_shift == 0.5 else n
+
+    @contextmanager
+    def _compute_encodings(self, passthrough: bool = False):
+        """passthrough=True: inputs are observed and returned unquantized (what a whole-model calibration uses)
+        (quantizer.py:601-698)."""
+        if not any(self._is_overwrite_allowed.values()):
+            yield
+            return
+        inner_forward = torch.Tensor.clone if passthrough else self.forward
+        shape = self.shape
+        try:
+            dtype, device = next((p.dtype, p.device) for p in self.parameters())
+        except StopIteration as e:
+            raise RuntimeError from e
+
+        @functools.wraps(inner_forward)
+        def observing_forward(input: torch.Tensor) -> torch.Tensor:
+            if type(input) != torch.Tensor:  # pylint: disable=unidiomatic-typecheck
+                input = input.as_subclass(torch.Tensor)
+            if input.numel() == 0:
+                return inner_forward(input)
+            batch_stats = self.encoding_analyzer.update_stats(input)
+            lo, hi = self.encoding_analyzer.compute_encodings_from_stats(
+                batch_stats, self._num_steps_for_calibration(), self.symmetric
+            )
+            if self.block_size is not None:
+                lo, hi = lo.view(shape), hi.view(shape)
+            lo = lo.to(dtype=dtype, device=device).expand(shape)
+            hi = hi.to(dtype=dtype, device=device).expand(shape)
+            scale, offset = _get_scale_offset(lo.to(torch.float32), hi.to(torch.float32), qmin=self.qmin,
+                                              qmax=self.qmax, symmetric=self.symmetric)
+            encoding = AffineEncoding(scale, offset, self.qmin, self.qmax, self.symmetric, self.block_size,
+                                      self.zero_point_shift, producer=self)
+            with self._set_encodings(encoding):
+                ret = inner_forward(input)
+            if not hasattr(ret, "encoding"):
+                ret.encoding = encoding
+            return ret
+
+        self.encoding_analyzer.reset_stats()
+        with patch_attr(self, "forward", observing_forward):
+            yield
+
+        try:
+            lo, hi = self.encoding_analyzer.compute_encodings(self._num_steps_for_calibration(), self.symmetric)
+            if self.block_size is not None:
+                lo, hi = lo.view(shape), hi.view(shape)
+            _flag_extreme_min_max(lo, hi)
+        except StatisticsNotFoundError:
+            return
+        if not self._is_overwrite_allowed["min"]:
+            lo = None
+        if not self._is_overwrite_allowed["max"]:
+            hi = None
+        self.set_range(lo, hi)
+
+    @contextmanager
+    def _set_encodings(self, enc: Optional[AffineEncoding]):
+        """Temporarily make ``get_encodings()`` return ``enc`` (quantizer.py:806-821)."""
+        with (
+            patch_attr(self, "get_encodings", lambda *a, **k: enc),
+            patch_attr(self, "is_initialized", lambda *a, **k: enc is not None),
+        ):
+            yield
+
+    @contextmanager
+    def _precompute_encodings(self, dtype: Optional[torch.dtype] = None):
+        """Evaluate the encodings once and reuse them for every forward inside the context (quantizer.py:790-804)."""
+        enc = self.get_encodings()
+        if enc is not None:
+            with torch.no_grad():
+                enc = enc.to(dtype=dtype) if dtype is not None else enc
+                const = getattr(enc.offset, "_ahq_constant", None)
+                enc.scale = enc.scale.detach()
+                enc.offset = enc.offset.detach()
+                if const is not None:
+                    enc.offset._ahq_constant = const  # pylint: disable=protected-access
+        with self._set_encodings(enc) if enc is not None else nullcontext():
+            yield
+
+    def _get_dummy_encoding(self) -> AffineEncoding:
+        device = next(p.device for p in self.parameters())
+        return AffineEncoding(torch.ones((), device=device), torch.zeros((), device=device), self.qmin, self.qmax,
+                              self._symmetric, block_size=None, zero_point_shift=self.zero_point_shift, producer=self)
+
+    def _forward_encoding(self, input: torch.Tensor, what: str) -> AffineEncoding:
+        encoding = self.get_encodings()
+        if encoding is None:
+            if input.numel() == 0:
+                return self._get_dummy_encoding()
+            raise RuntimeError(
+                f"Failed to run {what} since quantization parameters are not initialized."
+                " Please initialize the quantization parameters using `compute_encodings()`."
+            )
+        return encoding
+
+    # ----------------------------------------------------------------------------------------- checkpointing --
+    def get_extra_state(self):
+        state = super().get_extra_state()
+        state.update({
+            "qmin": torch.tensor(self.qmin),
+            "qmax": torch.tensor(self.qmax),
+            "symmetric": torch.tensor(self.symmetric),
+            "block_size": torch.tensor(self.block_size or ()),
+            "zero_point_shift": torch.tensor(self.zero_point_shift),
+        })
+        return state
+
+    def set_extra_state(self, state):
+        state = dict(state)
+        grid = {k: state.pop(k) for k in ("qmin", "qmax", "symmetric", "block_size", "zero_point_shift") if k in state}
+        super().set_extra_state(state)
+        if "qmin" in grid:
+            self.qmin = grid["qmin"].item()
+        if "qmax" in grid:
+            self.qmax = grid["qmax"].item()
+        if "symmetric" in grid:
+            self.symmetric = grid["symmetric"].item()
+        if "block_size" in grid:
+            self.block_size = tuple(int(b) for b in grid["block_size"]) or None
+        if "zero_point_shift" in grid:
+            self.zero_point_shift = grid["zero_point_shift"].item()
+        self.shape = tuple(self.min.shape)
+
+    def load_state_dict(self, state_dict, strict: bool = True, **kwargs):  # pylint: disable=arguments-differ
+        if not strict:
+            # a non-strict load may change the shape of the encodings (quantizer.py:700-751)
+            for name in ("min", "max"):
+                new = state_dict.get(name)
+                cur = getattr(self, name)
+                if new is not None and new.shape != cur.shape:
+                    setattr(self, name, nn.Parameter(new.clone().to(device=cur.device, dtype=cur.dtype)))
+        return super().load_state_dict(state_dict, strict, **kwargs)
+
+
+class Quantize(AffineQuantizerBase):
+    r"""out = clamp(round(input / scale) - offset, qmin, qmax), returned as a :class:`QuantizedTensor`."""
+
+    def __init__(self, shape, *args, **kwargs):
+        super().__init__(shape, *args, **kwargs)
+        if self.zero_point_shift != 0.0:
+            raise RuntimeError("Nonzero quant shift not supported for Quantize")
+
+    def forward(self, input: torch.Tensor) -> QuantizedTensor:
+        encoding = self._forward_encoding(input, "Quantize")
+        if type(input) != torch.Tensor:  # pylint: disable=unidiomatic-typecheck
+            input = input.as_subclass(torch.Tensor)
+        output = quantize(input, encoding.scale, encoding.offset, encoding.qmin, encoding.qmax,
+                          block_size=encoding.block_size)
+        output = output.as_subclass(QuantizedTensor)
+        output.encoding = encoding
+        return output
+
+
+class QuantizeDequantize(AffineQuantizerBase):
+    r"""out = (clamp(round(input / scale) - offset, qmin, qmax) + offset) * scale, returned as a
+    :class:`DequantizedTensor`; scale and offset derive from the learnable ``min`` / ``max``."""
+
+    def __init__(self, shape, *args, **kwargs):  # pylint: disable=useless-parent-delegation
+        super().__init__(shape, *args, **kwargs)
+
+    def forward(self, input: torch.Tensor) -> DequantizedTensor:
+        encoding = self._forward_encoding(input, "QuantizeDequantize")
+        if type(input) != torch.Tensor:  # pylint: disable=unidiomatic-typecheck
+            input = input.as_subclass(torch.Tensor)
+        output = quantize_dequantize(input, encoding.scale, encoding.offset, encoding.qmin, encoding.qmax,
+                                     block_size=encoding.block_size, zero_point_shift=encoding.zero_point_shift)
+        output = output.as_subclass(DequantizedTensor)
+        output.encoding = encoding
+        return output
+
+
+class Dequantize(AffineQuantizerBase):
+    r"""out = (input + offset) * scale"""
+
+    def forward(self, input):
+        if self.zero_point_shift != 0.0:
+            raise RuntimeError("Nonzero quant shift not supported for Dequantize")
+        encoding = self._forward_encoding(input, "Dequantize")
+        if type(input) != torch.Tensor:  # pylint: disable=unidiomatic-typecheck
+            input = input.as_subclass(torch.Tensor)
+        output = dequantize(input, encoding.scale, encoding.offset, block_size=encoding.block_size)
+        output = output.as_subclass(DequantizedTensor)
+        output.encoding = encoding
+        return output
+
+
+class GroupedBlockQuantizeDequantize(QuantizeDequantize):
+    """Blockwise quantize-dequantize whose block scales are snapped to integer multiples (1 .. 2^(decompressed_bw -
+    bitwidth)) of a scale shared by each group of blocks -- LPBQ (quantizer.py:1270-1440)."""
+
+    def __init__(self, shape, bitwidth: int, symmetric: bool, decompressed_bw: int,
+                 encoding_analyzer: EncodingAnalyzer = None, block_size: Optional[Tuple[int, ...]] = None,
+                 block_grouping: Optional[Tuple[int, ...]] = None):
+        super().__init__(shape, bitwidth, symmetric, encoding_analyzer, block_size)
+        self.decompressed_bw = decompressed_bw
+        self.block_grouping = block_grouping
+        if self.block_grouping is None:
+            self.block_grouping = tuple(1 for _ in self.shape)
+        if block_grouping is not None:
+            if len(block_grouping) != len(self.shape):
+                raise RuntimeError(f"Length of block grouping {block_grouping} must equal length of shape {shape}.")
+            for dim, group in zip(self.shape, block_grouping):
+                if group != -1 and dim % group != 0:
+                    raise RuntimeError(
+                        f"Quantizer shape dimensions must divide evenly with corresponding block "
+                        f"grouping values for shapes {shape} and block grouping {block_grouping}."
+                    )
+        if self.decompressed_bw < self.bitwidth:
+            raise RuntimeError(
+                f"Decompressed bitwidth {decompressed_bw} cannot be smaller than self.bitwidth {bitwidth}"
+            )
+        if not symmetric:
+            raise RuntimeError("GroupedBlockQuantizeDequantize only supports symmetric quantization.")
+
+    def get_scale(self, dtype=None) -> Optional[torch.Tensor]:
+        return self._get_scale(dtype)[0]
+
+    def get_per_channel_scale(self, dtype=None) -> Optional[torch.Tensor]:
+        raw = super().get_scale(dtype)
+        return None if raw is None else self._get_per_channel_scale(raw)
+
+    def _get_scale(self, dtype=None):
+        raw = super().get_scale(dtype)
+        if raw is None:
+            return None, None
+        per_channel = self._get_per_channel_scale(raw)
+        snapped = quantize_dequantize(raw, per_channel, torch.zeros_like(per_channel), 1,
+                                      2 ** (self.decompressed_bw - self.bitwidth), block_size=self.block_grouping)
+        return snapped, per_channel
+
+    def _get_per_channel_scale(self, raw_scale: torch.Tensor) -> torch.Tensor:
+        """Largest block scale of each group divided by the number of integer multipliers (quantizer.py:1382-1399)."""
+        group_shape = [d // g if g != -1 else 1 for d, g in zip(raw_scale.shape, self.block_grouping)]
+        grouping = concretize_block_size(raw_scale.shape, group_shape, self.block_grouping)
+        view = raw_scale.reshape(*interleave(group_shape, grouping))
+        largest = torch.amax(view, dim=tuple(range(1, view.dim(), 2)))
+        return true_divide(largest, 2 ** (self.decompressed_bw - self.bitwidth))
+
+    def get_encodings(self) -> Optional[GroupedBlockEncoding]:
+        if not self.is_initialized():
+            return None
+        scale, per_channel = self._get_scale(dtype=torch.float32)
+        return GroupedBlockEncoding(scale=scale, offset=self.get_offset(dtype=torch.float32), bitwidth=self.bitwidth,
+                                    signed=self.signed, symmetry=self.symmetric, block_size=self.block_size,
+                                    block_grouping=self.block_grouping, decompressed_bw=self.decompressed_bw,
+                                    per_channel_scale=per_channel, zero_point_shift=self.zero_point_shift,
+                                    producer=self)
+
+    @classmethod
+    def from_encodings(cls, encodings: GroupedBlockEncoding) -> "GroupedBlockQuantizeDequantize":
+        if not isinstance(encodings, GroupedBlockEncoding):
+            raise TypeError(f"Expected {GroupedBlockEncoding}; got {type(encodings)}")
+        qtzr = cls(shape=encodings.scale.shape, bitwidth=encodings.bitwidth, symmetric=encodings.symmetry,
+                   decompressed_bw=encodings.decompressed_bw, block_size=encodings.block_size,
+                   block_grouping=encodings.block_grouping)
+        qtzr.to(encodings.scale.device)
+        qtzr.set_range(encodings.min, encodings.max)
+        return qtzr

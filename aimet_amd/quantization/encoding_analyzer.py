@@ -1,0 +1,481 @@
+"""Encoding analyzers: observe tensors on the GPU and turn the statistics into (min, max) encodings.
+
+Same classes, constructor signatures and methods as aimet_torch/quantization/encoding_analyzer.py:
+``MinMaxEncodingAnalyzer``, ``PercentileEncodingAnalyzer``, ``SqnrEncodingAnalyzer``, ``TfEnhancedEncodingAnalyzer``
+(``update_stats``, ``reset_stats``, ``compute_encodings``, ``compute_encodings_from_stats``,
+``compute_dynamic_encodings``, ``.observer.shape``).  Every pass over a tensor (min/max, histogram binning) and the
+SQNR candidate search run in HIP kernels; only arithmetic on encoding-shaped tensors is left to torch ops on the
+device, where each operation is a single IEEE operation and therefore reproduces the reference bit for bit.
+"""
+
+# pylint: disable=redefined-builtin, missing-docstring
+
+from __future__ import annotations
+
+import math
+import warnings
+from abc import ABC, abstractmethod
+from dataclasses import dataclass
+from typing import Generic, List, Optional, Tuple, TypeVar
+
+import torch
+
+from aimet_amd import _lib
+from aimet_amd._lib import HipLibraryError
+from aimet_amd.quantization._utils import StatisticsNotFoundError, _get_minimum_scale, _is_expandable, true_divide
+from aimet_amd.quantization._stats import reduce_min_max, _check_reducible
+from aimet_amd.quantization.affine.backends.hip import _prepare
+
+
+@dataclass
+class _MinMaxRange:
+    min: Optional[torch.Tensor] = None
+    max: Optional[torch.Tensor] = None
+
+
+@dataclass
+class _Histogram:
+    histogram: torch.Tensor = None
+    bin_edges: torch.Tensor = None
+    min: Optional[torch.Tensor] = None
+    max: Optional[torch.Tensor] = None
+
+
+_Statistics = TypeVar("_Statistics", _MinMaxRange, _Histogram)
+
+
+class _Observer(Generic[_Statistics], ABC):
+    """Observes tensors and accumulates statistics of a given shape."""
+
+    def __init__(self, shape, block_size=None):
+        if isinstance(shape, int):
+            shape = (shape,)
+        self.shape = tuple(shape)
+        self.block_size = block_size
+
+    @abstractmethod
+    def collect_stats(self, input_tensor: torch.Tensor) -> _Statistics: ...
+
+    @abstractmethod
+    def merge_stats(self, stats: _Statistics): ...
+
+    @abstractmethod
+    def reset_stats(self): ...
+
+    @abstractmethod
+    def get_stats(self) -> _Statistics: ...
+
+
+class _MinMaxObserver(_Observer[_MinMaxRange]):
+    """Running per-encoding minimum and maximum (reference: encoding_analyzer.py:69-118).  One fused kernel reads the
+    tensor once for both extrema and folds them into the running statistics."""
+
+    def __init__(self, shape, block_size=None):
+        super().__init__(shape, block_size)
+        self.stats = _MinMaxRange()
+
+    @torch.no_grad()
+    def collect_stats(self, input_tensor: torch.Tensor) -> _MinMaxRange:
+        mn, mx = reduce_min_max(input_tensor, self.shape, self.block_size)
+        return _MinMaxRange(mn, mx)
+
+    @torch.no_grad()
+    def merge_stats(self, stats: _MinMaxRange):
+        new_min, new_max = self.stats.min, self.stats.max
+        if stats.min is not None:
+            new_min = stats.min.clone() if new_min is None else torch.minimum(new_min, stats.min)
+        if stats.max is not None:
+            new_max = stats.max.clone() if new_max is None else torch.maximum(new_max, stats.max)
+        self.stats = _MinMaxRange(new_min, new_max)
+
+    @torch.no_grad()
+    def update(self, input_tensor: torch.Tensor) -> _MinMaxRange:
+        """collect + merge in one launch: the running fold happens where the reduction finishes."""
+        cur = self.stats
+        fused = (
+            cur.min is not None and cur.max is not None
+            and cur.min.dtype == input_tensor.dtype and cur.min.device == input_tensor.device
+            and cur.min.is_contiguous() and cur.max.is_contiguous()
+        )
+        if fused:
+            mn, mx = reduce_min_max(input_tensor, self.shape, self.block_size, running=(cur.min, cur.max))
+            return _MinMaxRange(mn, mx)
+        new = self.collect_stats(input_tensor)
+        self.merge_stats(new)
+        return new
+
+    def reset_stats(self):
+        self.stats = _MinMaxRange()
+
+    def get_stats(self) -> _MinMaxRange:
+        return self.stats
+
+
+class _HistogramObserver(_Observer[_Histogram]):
+    """Running per-encoding histograms (reference: encoding_analyzer.py:121-338).
+
+    State lives in fp32 device tensors: ``hist [S, B]``, ``edges [S, B+1]``, ``minmax [S, 2]``, ``limits [S, 2]``.
+    One library call per batch produces the batch's own histogram and folds the batch into the running one."""
+
+    def __init__(self, shape, *, block_size=None, num_bins: int, growth_limit: Optional[float] = None):
+        super().__init__(shape, block_size)
+        self.num_bins = num_bins
+        self.num_slots = int(math.prod(self.shape))
+        if growth_limit is None:
+            growth_limit = float("inf")
+        if growth_limit < 1.0:
+            raise RuntimeError(f"Growth limit must be at least 1.0. Got {growth_limit}")
+        self.growth_limit = growth_limit
+        self._state = None          # dict of device tensors
+        self._has_stats = False
+        self._stat_dtype = None     # dtype of stats.min / stats.max as the reference would hold them
+        self._stats_cache = None
+
+    # ---------------------------------------------------------------------------------------------- internals --
+    def _alloc(self, device) -> dict:
+        S, B = self.num_slots, self.num_bins
+        f = dict(dtype=torch.float32, device=device)
+        return {
+            "hist": torch.zeros(S, B, **f), "edges": torch.zeros(S, B + 1, **f),
+            "minmax": torch.zeros(S, 2, **f), "limits": torch.zeros(S, 2, **f),
+        }
+
+    def _run(self, x: torch.Tensor, state: dict, first: bool):
+        """One ahq_hist_update call.  Returns (new_hist, new_edges, new_minmax)."""
+        _lib.require_device(x, "input tensor")
+        if x.dtype not in _lib.DTYPE_CODE:
+            raise HipLibraryError(f"histogram statistics support float32, float16 and bfloat16; got {x.dtype}")
+        try:
+            _check_reducible(x, self.shape, self.block_size)
+        except RuntimeError as e:
+            raise RuntimeError(f"Shape {self.shape} is incompatible with input of shape {x.shape}") from e
+        if x.numel() == 0:
+            raise RuntimeError("cannot observe an empty tensor")
+        lib = _lib.load()
+        S, B = self.num_slots, self.num_bins
+        xd, layout = _prepare(x.detach(), self.shape, self.block_size)
+        f = dict(dtype=torch.float32, device=x.device)
+        new_hist = torch.empty(S, B, **f)
+        new_edges = torch.empty(S, B + 1, **f)
+        new_minmax = torch.empty(S, 2, **f)
+        st = _lib.HistState()
+        st.num_slots, st.num_bins, st.growth_limit = S, B, self.growth_limit
+        st.hist, st.edges = state["hist"].data_ptr(), state["edges"].data_ptr()
+        st.minmax, st.limits = state["minmax"].data_ptr(), state["limits"].data_ptr()
+        st.new_hist, st.new_edges, st.new_minmax = new_hist.data_ptr(), new_edges.data_ptr(), new_minmax.data_ptr()
+        code = _lib.DTYPE_CODE[x.dtype]
+        nbytes = lib.ahq_hist_update_workspace_bytes(code, layout, B)
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
+        _lib.check(
+            lib.ahq_hist_update(code, layout, xd.data_ptr(), st, 1 if first else 0, ws.data_ptr(), nbytes,
+                                _lib.current_stream(x.device)),
+            "ahq_hist_update",
+        )
+        return new_hist, new_edges, new_minmax
+
+    @staticmethod
+    def _as_list(hist, edges, minmax, dtype) -> List[_Histogram]:
+        mm = minmax if dtype == torch.float32 else minmax.to(dtype)
+        return [_Histogram(hist[s], edges[s], mm[s, 0], mm[s, 1]) for s in range(hist.shape[0])]
+
+    # --------------------------------------------------------------------------------------------------- API --
+    @torch.no_grad()
+    def collect_stats(self, input_tensor: torch.Tensor) -> List[_Histogram]:
+        scratch = self._alloc(input_tensor.device)
+        h, e, mm = self._run(input_tensor, scratch, first=True)
+        return self._as_list(h, e, mm, input_tensor.dtype)
+
+    @torch.no_grad()
+    def update(self, input_tensor: torch.Tensor) -> List[_Histogram]:
+        """collect_stats + merge_stats with a single binning pass over the tensor."""
+        first = not self._has_stats
+        if first or self._state["hist"].device != input_tensor.device:
+            if not first:
+                raise RuntimeError("histogram statistics live on a different device than the input")
+            self._state = self._alloc(input_tensor.device)
+        h, e, mm = self._run(input_tensor, self._state, first)
+        # the reference keeps the first batch's min/max in the tensor dtype; after a merge they are float32
+        self._stat_dtype = input_tensor.dtype if first else torch.promote_types(self._stat_dtype, torch.float32)
+        self._has_stats = True
+        self._stats_cache = None
+        return self._as_list(h, e, mm, input_tensor.dtype)
+
+    @torch.no_grad()
+    def merge_stats(self, new_stats_list: List[_Histogram], input_tensor: torch.Tensor):  # pylint: disable=arguments-differ
+        # the fused update recomputes the batch statistics while it bins the batch onto the running range
+        del new_stats_list
+        self.update(input_tensor)
+
+    def reset_stats(self):
+        self._state = None
+        self._has_stats = False
+        self._stat_dtype = None
+        self._stats_cache = None
+
+    def get_stats(self) -> List[_Histogram]:
+        if not self._has_stats:
+            return [_Histogram() for _ in range(self.num_slots)]
+        if self._stats_cache is None:
+            s = self._state
+            self._stats_cache = self._as_list(s["hist"], s["edges"], s["minmax"], self._stat_dtype)
+        return self._stats_cache
+
+    @property
+    def stats(self) -> List[_Histogram]:
+        return self.get_stats()
+
+
+class EncodingAnalyzer(Generic[_Statistics], ABC):
+    """Gathers statistics of input data and computes encodings from them."""
+
+    def __init__(self, observer: _Observer):
+        self.observer = observer
+
+    @torch.no_grad()
+    def update_stats(self, input_tensor: torch.Tensor):
+        """Update the running statistics with ``input_tensor``; returns the statistics of this tensor alone."""
+        return self.observer.update(input_tensor)
+
+    def reset_stats(self):
+        self.observer.reset_stats()
+
+    def compute_encodings(self, num_steps: int, is_symmetric: bool):
+        """(min, max) of the encoding for a grid of ``num_steps`` steps."""
+        return self.compute_encodings_from_stats(self.observer.get_stats(), num_steps, is_symmetric)
+
+    def compute_dynamic_encodings(self, input_tensor: torch.Tensor, num_steps: int, is_symmetric: bool):
+        return self.compute_encodings_from_stats(self.observer.collect_stats(input_tensor), num_steps, is_symmetric)
+
+    @abstractmethod
+    def compute_encodings_from_stats(self, stats, num_steps: int, is_symmetric: bool): ...
+
+
+class MinMaxEncodingAnalyzer(EncodingAnalyzer[_MinMaxRange]):
+    """Min-max calibration: the encoding range is [min(input), max(input)], widened to contain zero and to be
+    representable (reference: encoding_analyzer.py:397-481)."""
+
+    def __init__(self, shape, block_size=None):
+        super().__init__(_MinMaxObserver(shape, block_size))
+
+    @torch.no_grad()
+    def compute_encodings_from_stats(self, stats: _MinMaxRange, num_steps: int, is_symmetric: bool):
+        if num_steps <= 0:
+            raise ValueError("The number of quantization bins cannot be less than or equal to 0.")
+        if stats.min is None or stats.max is None:
+            raise StatisticsNotFoundError("No statistics present to compute encodings.")
+
+        tiny = _get_minimum_scale(num_steps)
+        lo = torch.clamp(stats.min, max=0)
+        hi = torch.clamp(stats.max, min=0)
+        # ranges narrower than the minimum scale are widened by it (this fp32 term promotes 16-bit statistics)
+        widen = tiny * (true_divide(hi - lo, num_steps) < tiny)
+        if is_symmetric:
+            pos, neg = math.floor(num_steps / 2), math.ceil(num_steps / 2)
+            hi = hi + pos * widen
+            lo = lo - neg * widen
+            # a 2-bit signed grid would waste a level on the negative side: calibrate as if it had one more
+            extra = 1 if num_steps == 3 else 0
+            delta = torch.maximum(true_divide(hi, pos + extra), true_divide(-lo, neg))
+            lo = (-1 * neg) * delta
+            hi = pos * delta
+        else:
+            hi = hi + num_steps * widen
+        hi = torch.clamp(hi, max=torch.finfo(stats.min.dtype).max).to(stats.min.dtype)
+        lo = torch.clamp(lo, min=torch.finfo(stats.max.dtype).min).to(stats.max.dtype)
+        return lo, hi
+
+
+def _flag_extreme_min_max(curr_min, curr_max):
+    """Warn about non-finite or near-overflow encodings (reference: encoding_analyzer.py:484-498)."""
+    if not (torch.all(torch.isfinite(curr_min)) and torch.all(torch.isfinite(curr_max))):
+        warnings.warn("Infinite or NaN values detected within input! This may skew the associated encodings")
+    big = torch.full_like(curr_min, torch.finfo(curr_min.dtype).max)
+    if torch.any(torch.isclose(torch.abs(curr_min), big, rtol=0.05)) or torch.any(
+        torch.isclose(torch.abs(curr_max), big, rtol=0.05)
+    ):
+        warnings.warn("Extreme values detected within input! This may skew the associated encodings")
+
+
+def adjust_min_max(curr_min, curr_max, num_steps, is_symmetric):
+    """Make a (min, max) pair contain zero, finite and at least minimum_scale wide; symmetric grids are re-centred
+    (reference: encoding_analyzer.py:501-534).  Works on tensors of any shape."""
+    tiny = _get_minimum_scale(num_steps)
+    curr_min = torch.minimum(curr_min, torch.zeros_like(curr_min))
+    curr_max = torch.maximum(curr_max, torch.zeros_like(curr_max))
+    curr_min = curr_min.clamp(min=torch.finfo(curr_max.dtype).min, max=0)
+    curr_max = curr_max.clamp(min=0, max=torch.finfo(curr_max.dtype).max)
+    narrow = true_divide(curr_max - curr_min, num_steps) < tiny
+    if is_symmetric:
+        curr_min = torch.where(narrow, curr_min - tiny * math.ceil(num_steps / 2), curr_min)
+        curr_max = torch.where(narrow, curr_max + tiny * math.floor(num_steps / 2), curr_max)
+        pos, neg = math.floor(num_steps / 2), math.ceil(num_steps / 2)
+        delta = torch.maximum(true_divide(curr_max, pos), true_divide(-curr_min, neg))
+        curr_min = (-1 * neg) * delta
+        curr_max = pos * delta
+    else:
+        curr_max = torch.where(narrow, curr_max + tiny * num_steps, curr_max)
+    return curr_min, curr_max
+
+
+class _HistogramAnalyzer(EncodingAnalyzer[_Histogram]):
+    def _stack(self, stats: List[_Histogram]):
+        """(hist [S,B], edges [S,B+1], minmax [S,2] fp32, dtype of min/max) from a list of per-slot statistics."""
+        obs = self.observer
+        if stats is obs.get_stats() and obs._has_stats:  # pylint: disable=protected-access
+            s = obs._state  # pylint: disable=protected-access
+            return s["hist"], s["edges"], s["minmax"], obs._stat_dtype  # pylint: disable=protected-access
+        hist = torch.stack([s.histogram for s in stats]).contiguous()
+        edges = torch.stack([s.bin_edges for s in stats]).contiguous()
+        dtype = stats[0].min.dtype
+        mm = torch.stack([torch.stack((s.min, s.max)) for s in stats]).to(torch.float32).contiguous()
+        return hist, edges, mm, dtype
+
+
+class PercentileEncodingAnalyzer(_HistogramAnalyzer):
+    """Percentile calibration: clip (100 - p)% of the largest and smallest observed values
+    (reference: encoding_analyzer.py:538-650)."""
+
+    def __init__(self, shape, num_bins: int = 2048, percentile: float = 100, block_size=None):
+        if num_bins <= 0:
+            raise ValueError("Number of bins cannot be less than or equal to 0.")
+        super().__init__(_HistogramObserver(shape=shape, num_bins=num_bins, block_size=block_size))
+        self.set_percentile(percentile)
+
+    def set_percentile(self, percentile):
+        if percentile < 50 or percentile > 100:
+            raise ValueError("Percentile value must be within 50-100 range")
+        self.percentile = percentile
+
+    @torch.no_grad()
+    def compute_encodings_from_stats(self, stats: List[_Histogram], num_steps: int, is_symmetric: bool):
+        if num_steps <= 0:
+            raise ValueError("The number of quantization bins cannot be less than or equal to 0.")
+        if stats[0].histogram is None:
+            raise StatisticsNotFoundError("No statistics present to compute encodings.")
+        hist, edges, _, dtype = self._stack(stats)
+        B = hist.shape[1]
+        if self.percentile == 100:
+            lo, hi = edges[:, 0], edges[:, B]
+        else:
+            cs = torch.cumsum(hist, dim=1)
+            total = cs[:, -1:]
+            hi_i = torch.searchsorted(cs, total * self.percentile / 100).clamp_(max=B)
+            lo_i = torch.searchsorted(cs, total * (1 - self.percentile / 100)).clamp_(max=B)
+            lo = torch.gather(edges, 1, lo_i).squeeze(1)
+            hi = torch.gather(edges, 1, hi_i).squeeze(1)
+        lo, hi = adjust_min_max(lo, hi, num_steps, is_symmetric)
+        return lo.to(dtype).reshape(self.observer.shape), hi.to(dtype).reshape(self.observer.shape)
+
+
+class _LpNormEncodingAnalyzer(_HistogramAnalyzer):
+    """Searches (delta, offset) candidates for the lowest expected p-norm quantization + gamma * clipping noise
+    over the histogram (reference: encoding_analyzer.py:653-899).  The whole search is one library call."""
+
+    def __init__(self, shape, num_bins: int, *, p: float, asymmetric_delta_candidates: int,
+                 symmetric_delta_candidates: int, offset_candidates: int, max_parallelism: int, gamma: float,
+                 histogram_growth_limit: Optional[float] = None, block_size=None):
+        if num_bins <= 0:
+            raise ValueError("Number of bins cannot be less than or equal to 0.")
+        super().__init__(_HistogramObserver(shape=shape, num_bins=num_bins, growth_limit=histogram_growth_limit,
+                                            block_size=block_size))
+        self.p = p
+        self.asym_delta_candidates = asymmetric_delta_candidates
+        self.sym_delta_candidates = symmetric_delta_candidates
+        self.num_offset_candidates = offset_candidates
+        self.gamma = gamma
+        self.max_parallelism = max_parallelism  # kept for signature compatibility; the kernel needs no chunking
+        self._offset_grid_cache = {}
+        self.last_search = None
+
+    def _offset_grid(self, num_steps: int, device) -> torch.Tensor:
+        """round(arange(-num_steps, step, step)) evaluated on the CPU (torch.arange computes in double there),
+        then kept on the device."""
+        key = (num_steps, self.num_offset_candidates, str(device))
+        grid = self._offset_grid_cache.get(key)
+        if grid is None:
+            n_off = min(num_steps + 2, self.num_offset_candidates)
+            step = num_steps / (n_off - 2)
+            grid = torch.round(torch.arange(start=-num_steps, end=step, step=step, dtype=torch.float32)).to(device)
+            self._offset_grid_cache[key] = grid
+        return grid
+
+    @torch.no_grad()
+    def compute_encodings_from_stats(self, stats: List[_Histogram], num_steps: int, is_symmetric: bool):
+        if stats[0].histogram is None:
+            raise StatisticsNotFoundError("No statistics present to compute encodings.")
+        if num_steps <= 0:
+            raise ValueError("The number of quantization bins cannot be less than or equal to 0.")
+        num_steps = int(num_steps)
+        hist, edges, minmax, dtype = self._stack(stats)
+        device = hist.device
+        lib = _lib.load()
+        S, B = hist.shape
+        prm = _lib.SqnrParams()
+        prm.num_slots, prm.num_bins = S, B
+        prm.symmetric = 1 if is_symmetric else 0
+        prm.stat_dtype = _lib.DTYPE_CODE[dtype]
+        prm.num_steps = num_steps
+        prm.minimum_scale = _get_minimum_scale(num_steps)
+        prm.gamma, prm.p = float(self.gamma), float(self.p)
+        grid = None
+        if is_symmetric:
+            prm.num_deltas, prm.num_offsets = self.sym_delta_candidates, 1
+        else:
+            grid = self._offset_grid(num_steps, device)
+            prm.num_deltas, prm.num_offsets = self.asym_delta_candidates, grid.numel() + 1
+        D, O = prm.num_deltas, prm.num_offsets
+        f = dict(dtype=torch.float32, device=device)
+        noise = torch.empty(S, D, O, **f)
+        deltas = torch.empty(S, D, O, **f)
+        offsets = torch.empty(S, D, O, **f)
+        out = torch.empty(S, 4, **f)
+        best = torch.empty(S, dtype=torch.int64, device=device)
+        _lib.check(
+            lib.ahq_sqnr_search(prm, hist.data_ptr(), edges.data_ptr(), minmax.data_ptr(), _lib.ptr(grid),
+                                noise.data_ptr(), deltas.data_ptr(), offsets.data_ptr(), out.data_ptr(),
+                                best.data_ptr(), _lib.current_stream(device)),
+            "ahq_sqnr_search",
+        )
+        self.last_search = {"noise": noise, "deltas": deltas, "offsets": offsets, "best_index": best,
+                            "best_delta": out[:, 0], "best_offset": out[:, 1]}
+        shape = self.observer.shape
+        return out[:, 2].to(dtype).view(shape), out[:, 3].to(dtype).view(shape)
+
+
+class SqnrEncodingAnalyzer(_LpNormEncodingAnalyzer):
+    """SQNR calibration (p = 2) (reference: encoding_analyzer.py:902-953)."""
+
+    def __init__(self, shape, num_bins: int = 2048, *, asymmetric_delta_candidates=17, symmetric_delta_candidates=101,
+                 offset_candidates=21, max_parallelism=64, gamma=3.0, histogram_growth_limit: Optional[float] = None,
+                 block_size=None):
+        super().__init__(shape=shape, num_bins=num_bins, p=2.0,
+                         asymmetric_delta_candidates=asymmetric_delta_candidates,
+                         symmetric_delta_candidates=symmetric_delta_candidates, offset_candidates=offset_candidates,
+                         max_parallelism=max_parallelism, gamma=gamma, histogram_growth_limit=histogram_growth_limit,
+                         block_size=block_size)
+
+
+class TfEnhancedEncodingAnalyzer(SqnrEncodingAnalyzer):
+    """SQNR analyzer with the fixed hyper-parameters of the legacy tf-enhanced scheme: 512 bins, 17 / 101 delta
+    candidates, 21 offsets, gamma 3, histogram range limited to 3x the first input's range
+    (reference: encoding_analyzer.py:956-1002)."""
+
+    _V1_HISTOGRAM_NUM_BINS = 512
+    _V1_ASYMMETRIC_DELTA_CANDIDATES = 17
+    _V1_SYMMETRIC_DELTA_CANDIDATES = 101
+    _V1_OFFSET_CANDIDATES = 21
+    _V1_GAMMA = 3.0
+    _V1_HISTOGRAM_MAX_GROWTH_RATE = 3.0
+
+    def __init__(self, shape, block_size=None):
+        super().__init__(shape=shape, num_bins=self._V1_HISTOGRAM_NUM_BINS,
+                         asymmetric_delta_candidates=self._V1_ASYMMETRIC_DELTA_CANDIDATES,
+                         symmetric_delta_candidates=self._V1_SYMMETRIC_DELTA_CANDIDATES,
+                         offset_candidates=self._V1_OFFSET_CANDIDATES, gamma=self._V1_GAMMA,
+                         histogram_growth_limit=self._V1_HISTOGRAM_MAX_GROWTH_RATE, block_size=block_size)
+
+    @classmethod
+    def set_growth_limit(cls, growth_limit: float):
+        if growth_limit < 1.0:
+            raise RuntimeError(f"Growth limit must be at least 1.0. Got {growth_limit}")
+        cls._V1_HISTOGRAM_MAX_GROWTH_RATE = growth_limit

@@ -1,0 +1,238 @@
+#!/usr/bin/env python3
+"""Benchmark of the fake-quant hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2]
+
+Default workload ("c2"): per-output-channel 8-bit symmetric weight quantize-dequantize forward + straight-through
+backward (input, scale and offset gradients) on an fp32 [4096, 4096] weight.  A step is one forward plus one backward
+launched through the C ABI on tensors already resident in HBM.  Prints ONE JSON line.
+
+`value` = algorithmic bytes per step (5 * sizeof(dtype) per element: forward reads x and writes y, backward reads g
+and x and writes gx) divided by the wall time per step, in GB/s.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+
+def _ensure_built():
+    from aimet_amd import _lib
+
+    if not os.path.exists(_lib.LIB_PATH):
+        from aimet_amd.csrc.build import build
+
+        build(verbose=False)
+    return _lib.load()
+
+
+# ----------------------------------------------------------------------------------------------------- workloads --
+def _make_c1(dev):
+    g = torch.Generator().manual_seed(0)
+    x = torch.relu(torch.randn(32, 64, 112, 112, generator=g))
+    g1 = torch.Generator().manual_seed(1)
+    grad = torch.randn(x.shape, generator=g1)
+    return dict(name="c1_per_tensor_8b_asym_fp32_32x64x112x112", x=x, grad=grad, enc_shape=(), block=None,
+                bitwidth=8, symmetric=False)
+
+
+def _make_c2(dev):
+    g = torch.Generator().manual_seed(0)
+    w = torch.randn(4096, 4096, generator=g) * 0.02
+    rows = torch.randperm(4096, generator=torch.Generator().manual_seed(1))[:41]
+    w[rows] *= 10
+    grad = torch.randn(4096, 4096, generator=torch.Generator().manual_seed(2)) * 1e-3
+    return dict(name="c2_per_channel_8b_sym_fp32_4096x4096", x=w, grad=grad, enc_shape=(4096, 1), block=None,
+                bitwidth=8, symmetric=True)
+
+
+def _make_c4(dev):
+    g = torch.Generator().manual_seed(0)
+    w = (torch.randn(14336, 4096, generator=g) * 0.02).bfloat16()
+    grad = torch.randn(14336, 4096, generator=torch.Generator().manual_seed(1)).bfloat16()
+    return dict(name="c4_blockwise64_4b_sym_bf16_14336x4096", x=w, grad=grad, enc_shape=(14336, 64), block=(1, 64),
+                bitwidth=4, symmetric=True)
+
+
+WORKLOADS = {"c1": _make_c1, "c2": _make_c2, "c4": _make_c4}
+
+
+def _encodings_cpu(w):
+    """Min/max calibration + scale/offset derivation on the CPU oracle (same arithmetic as the product path)."""
+    from oracle import torch_ref as O
+
+    import math
+
+    n = 2 ** w["bitwidth"] - 1
+    qmin, qmax = (-math.ceil(n / 2), math.floor(n / 2)) if w["symmetric"] else (0, n)
+    mn, mx = O.reduce_minmax(w["x"], w["enc_shape"], w["block"])
+    emin, emax = O.minmax_encodings(mn, mx, n, w["symmetric"])
+    scale = O.scale_from_minmax(emin, emax, qmin, qmax)
+    offset = O.offset_from_minmax(emin.float(), scale, qmin, qmax, w["symmetric"])
+    return scale, offset, qmin, qmax
+
+
+def run_qdq_workload(key, steps, warmup, dev, with_cpu_baseline=True):
+    from aimet_amd import _lib
+    from aimet_amd.quantization.affine.backends import hip
+    from oracle import torch_ref as O
+
+    lib = _ensure_built()
+    w = WORKLOADS[key](dev)
+    scale_c, offset_c, qmin, qmax = _encodings_cpu(w)
+    x = w["x"].to(dev)
+    grad = w["grad"].to(dev)
+    scale = scale_c.to(dev).contiguous()
+    offset = offset_c.to(dev).contiguous()
+    cd = hip._internal_dtype(x.dtype, qmin, qmax)
+    grid = hip._grid(_lib.AHQ_ARITH_AUTOGRAD, _lib.AHQ_OP_QDQ, x.dtype, cd, qmin, qmax, 0.0)
+    _, layout = hip._prepare(x, scale.shape, w["block"])
+    y = torch.empty_like(x)
+    gx = torch.empty_like(x)
+    gs = torch.empty_like(scale)
+    go = torch.empty_like(scale)
+    nbytes = lib.ahq_qdq_backward_workspace_bytes(grid, layout, 1)
+    ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=dev)
+    stream = _lib.current_stream(dev)
+
+    def fwd():
+        _lib.check(lib.ahq_qdq_forward(grid, layout, x.data_ptr(), y.data_ptr(), None, scale.data_ptr(),
+                                       offset.data_ptr(), None, None, stream), "fwd")
+
+    def bwd():
+        _lib.check(lib.ahq_qdq_backward(grid, layout, grad.data_ptr(), x.data_ptr(), gx.data_ptr(), gs.data_ptr(),
+                                        go.data_ptr(), scale.data_ptr(), offset.data_ptr(), ws.data_ptr(), nbytes,
+                                        stream), "bwd")
+
+    for _ in range(warmup):
+        fwd()
+        bwd()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fwd()
+        bwd()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+
+    # per-kernel durations from events on the launch stream
+    def event_time(fn, reps):
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        fn()
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / reps * 1e-3
+
+    reps = max(steps, 20)
+    t_fwd = event_time(fwd, reps)
+    t_bwd = event_time(bwd, reps)
+
+    n = x.numel()
+    S = x.element_size()
+    enc_bytes = 8 * scale.numel()
+    bytes_fwd = 2 * S * n + enc_bytes
+    bytes_bwd = 3 * S * n + enc_bytes + 8 * scale.numel()
+    bytes_step = bytes_fwd + bytes_bwd
+    ms_per_step = wall / steps * 1e3
+    value = bytes_step / (wall / steps) / 1e9
+
+    # parity spot check against the oracle (same seeded inputs)
+    tr = O.qdq_v2_forward(w["x"], scale_c, offset_c, qmin, qmax, w["block"])
+    gx_ref, gs_ref, go_ref = O.qdq_v2_backward(w["grad"], w["x"], scale_c, offset_c, qmin, qmax, w["block"])
+    exact_y = bool(torch.equal(y.cpu(), tr.y))
+    exact_gx = bool(torch.equal(gx.cpu(), gx_ref))
+    gs_err = float(((gs.cpu() - gs_ref).abs().max() / gs_ref.abs().max().clamp_min(1e-30)))
+
+    dom = ("qdq_bwd_kernel", t_bwd, bytes_bwd) if t_bwd >= t_fwd else ("qdq_fwd_kernel", t_fwd, bytes_fwd)
+    out = {
+        "metric": "QDQ fwd+bwd GB/s (% of HBM peak); calibration elems/s; vs host-CPU ref",
+        "value": round(value, 2),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": steps,
+        "warmup": warmup,
+        "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": {torch.float32: "f32", torch.bfloat16: "bf16", torch.float16: "f16"}[x.dtype],
+        "data": "synthetic",
+        "config": {"workload": w["name"], "elements": n, "algorithmic_bytes_per_step": bytes_step,
+                   "arithmetic": "autograd (learnable min/max)", "compute_dtype": str(cd).split(".")[-1]},
+        "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
+        "elements_per_s": round(n / (wall / steps), 1),
+        "kernels": {
+            "qdq_fwd_kernel": {"us": round(t_fwd * 1e6, 2), "GBps": round(bytes_fwd / t_fwd / 1e9, 1)},
+            "qdq_bwd_kernel": {"us": round(t_bwd * 1e6, 2), "GBps": round(bytes_bwd / t_bwd / 1e9, 1)},
+        },
+        "parity": {"y_bit_exact": exact_y, "gx_bit_exact": exact_gx, "gscale_max_rel_err": gs_err},
+        "roofline": {"bound": "hbm", "kernel": dom[0], "achieved": round(dom[2] / dom[1] / 1e9, 1),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(dom[2] / dom[1] / 1e9 / HBM_PEAK_GBS, 4),
+                     "traffic": None},
+    }
+    if with_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline_qdq(w, scale_c, offset_c, qmin, qmax, bytes_step)
+    return out
+
+
+def cpu_baseline_qdq(w, scale, offset, qmin, qmax, bytes_step, budget_s=12.0):
+    """The oracle (the reference's own sequence of torch CPU operations) timed on this host, full-size workload."""
+    from oracle import torch_ref as O
+
+    def step():
+        O.qdq_v2_forward(w["x"], scale, offset, qmin, qmax, w["block"])
+        O.qdq_v2_backward(w["grad"], w["x"], scale, offset, qmin, qmax, w["block"])
+
+    step()
+    t0 = time.perf_counter()
+    reps = 0
+    while True:
+        step()
+        reps += 1
+        if time.perf_counter() - t0 > budget_s or reps >= 20:
+            break
+    dt = (time.perf_counter() - t0) / reps
+    return {"value": round(bytes_step / dt / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(),
+            "kind": "port", "sample": f"{reps} full-size fwd+bwd steps of {w['name']} with torch CPU ops "
+                                      f"({dt * 1e3:.1f} ms/step)"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (no collectives exist on this path); use --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: no HIP device visible", file=sys.stderr)
+        sys.exit(1)
+    dev = torch.device("cuda:0")
+    out = run_qdq_workload(args.workload, args.steps, args.warmup, dev, with_cpu_baseline=not args.no_cpu_baseline)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

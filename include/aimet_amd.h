@@ -115,12 +115,60 @@ int    ahq_qdq_backward(const ahq_grid* grid, const ahq_layout* layout, const vo
  * DlQuantization GetMinMax (DLQ/src/math_functions.cpp:72-117).
  * out_min/out_max: one value per encoding in the tensor's own dtype.  NaN propagates like torch.amin/amax unless
  * finite_only, where non-finite values are ignored (an all-non-finite slice yields +inf / -inf).
- * If running != 0, out_min/out_max are combined with their current contents (minimum/maximum,
- * encoding_analyzer.py:96-112) instead of being overwritten.
+ * run_min/run_max (optional, both or neither): running statistics of the same shape and dtype that the batch result is
+ * folded into with torch.minimum / torch.maximum semantics (_MinMaxObserver.merge_stats, encoding_analyzer.py:96-112).
  */
 size_t ahq_minmax_workspace_bytes(const ahq_layout* layout);
 int    ahq_minmax(int32_t dtype, const ahq_layout* layout, const void* x, void* out_min, void* out_max,
-                  int finite_only, int running, void* workspace, size_t workspace_bytes, void* stream);
+                  void* run_min, void* run_max, int finite_only, void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---------------------------------------------------------------- histogram statistics ----------------------------
+ * Replaces: _HistogramObserver.collect_stats + merge_stats (AT/quantization/encoding_analyzer.py:189-332), i.e. what
+ * PercentileEncodingAnalyzer / SqnrEncodingAnalyzer / TfEnhancedEncodingAnalyzer.update_stats do per batch.
+ * One call: finite min/max of the batch, the batch's own num_bins-bin histogram over its own range (returned as
+ * new_*), the running range widened to cover the batch (clamped to growth_limit x the first batch's range), the
+ * running counts re-binned onto that range, and the batch binned onto it and added.  Bin index formula and
+ * out-of-range handling are torch.histc's on CPU; counts are fp32 like the reference's.
+ * All buffers are fp32 device arrays owned by the caller; hist/edges/minmax/limits persist between calls.
+ */
+typedef struct {
+    int32_t num_slots;     /* number of histograms = number of encodings of the layout */
+    int32_t num_bins;
+    float   growth_limit;  /* >= 1; +inf for no limit (encoding_analyzer.py:138-145) */
+    float*  hist;          /* [num_slots][num_bins]     running histogram */
+    float*  edges;         /* [num_slots][num_bins+1]   running bin edges */
+    float*  minmax;        /* [num_slots][2]            running stats.min / stats.max */
+    float*  limits;        /* [num_slots][2]            range limits fixed by the first batch */
+    float*  new_hist;      /* [num_slots][num_bins]     out: this batch's own histogram */
+    float*  new_edges;     /* [num_slots][num_bins+1]   out */
+    float*  new_minmax;    /* [num_slots][2]            out: this batch's finite min / max */
+} ahq_hist_state;
+
+size_t ahq_hist_update_workspace_bytes(int32_t dtype, const ahq_layout* layout, int32_t num_bins);
+int    ahq_hist_update(int32_t dtype, const ahq_layout* layout, const void* x, const ahq_hist_state* state,
+                       int first_batch, void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---------------------------------------------------------------- SQNR / TF-enhanced search ------------------------
+ * Replaces: _LpNormEncodingAnalyzer._pick_test_candidates / _clamp_delta_offset_values /
+ * _estimate_clip_and_quant_noise / _select_best_candidates (encoding_analyzer.py:728-899).
+ * offset_grid: the rounded offsets `round(arange(-num_steps, step, step))` (encoding_analyzer.py:763-770), made by the
+ * caller; num_offsets = len(offset_grid) + 1 (the observed offset is appended).  Ignored when symmetric.
+ * noise/deltas/offsets: [num_slots][num_deltas][num_offsets] fp32 outputs (every candidate, for inspection).
+ * out: [num_slots][4] = best delta, best offset, encoding min, encoding max; best_index: flat argmin (first minimum).
+ */
+typedef struct {
+    int32_t num_slots, num_bins, num_deltas, num_offsets;
+    int32_t symmetric;
+    int32_t stat_dtype;      /* ahq_dtype the running min/max are stored in (their arithmetic happens in it) */
+    int64_t num_steps;
+    double  minimum_scale;   /* _get_minimum_scale(num_steps) */
+    double  gamma;
+    double  p;
+} ahq_sqnr_params;
+
+int ahq_sqnr_search(const ahq_sqnr_params* params, const float* hist, const float* edges, const float* minmax,
+                    const float* offset_grid, float* noise, float* deltas, float* offsets, float* out,
+                    long long* best_index, void* stream);
 
 #ifdef __cplusplus
 }

@@ -150,7 +150,7 @@ def qdq_v1(x: torch.Tensor, scale: torch.Tensor, offset: torch.Tensor, qmin: int
     if len(axes) != 1:
         return None
     zp = -offset.to(torch.int32)
-    y, mask = torch.fake_quantize_per_channel_affine_cachemask(
+    y, mask = torch.ops.aten.fake_quantize_per_channel_affine_cachemask(
         x, scale.flatten(), zp.flatten(), axes[0], qmin, qmax
     )
     return y, mask

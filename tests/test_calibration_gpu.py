@@ -1,0 +1,229 @@
+"""Parity of the HIP calibration path (histogram observer, SQNR / TF-enhanced search, percentile, min-max encodings)
+with the CPU oracle.
+
+Bar: histogram bin counts, bin edges, stored min/max and min-max encodings bit-exact; SQNR-selected candidate index
+identical and the selected delta/offset/min/max bit-exact (the candidates are produced by the same fp32 operations);
+per-candidate noise sums within 1e-5 relative (fp64 accumulation here, fp32 cascade sums in the reference).
+"""
+
+import math
+
+import pytest
+import torch
+
+from oracle import torch_ref as O
+from tests.helpers import assert_same_bits, assert_close_rel
+
+pytestmark = pytest.mark.gpu
+
+
+def _laplace_with_outliers(shape, seed, frac=0.001):
+    g = torch.Generator().manual_seed(seed)
+    u = torch.rand(shape, generator=g) - 0.5
+    x = -torch.sign(u) * torch.log1p(-2 * u.abs())
+    n = x.numel()
+    k = max(1, int(n * frac))
+    idx = torch.randperm(n, generator=g)[:k]
+    out = (torch.rand(k, generator=g) * 40 + 20) * torch.sign(torch.rand(k, generator=g) - 0.5)
+    x.view(-1)[idx] = out
+    return x
+
+
+def _check_hist_lists(got, ref, what):
+    assert len(got) == len(ref)
+    for s, (a, b) in enumerate(zip(got, ref)):
+        assert_same_bits(a.histogram, b.histogram, f"{what}[{s}].histogram")
+        assert_same_bits(a.bin_edges, b.bin_edges, f"{what}[{s}].bin_edges")
+        assert a.min.dtype == b.min.dtype, f"{what}[{s}].min dtype {a.min.dtype} vs {b.min.dtype}"
+        assert_same_bits(a.min, b.min, f"{what}[{s}].min")
+        assert_same_bits(a.max, b.max, f"{what}[{s}].max")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=lambda d: str(d).split(".")[-1])
+@pytest.mark.parametrize("num_bins", [512, 10, 2048, 3])
+@pytest.mark.parametrize("growth", [None, 3.0, 1.0])
+def test_histogram_stream_single_slot(device, dtype, num_bins, growth):
+    """Five batches with drifting ranges (growth, shrink, identical range, clamped growth)."""
+    from aimet_amd.quantization.encoding_analyzer import _HistogramObserver
+
+    obs = _HistogramObserver((1,), num_bins=num_bins, growth_limit=growth)
+    ref = O.HistObserver((1,), num_bins, growth)
+    g = torch.Generator().manual_seed(11)
+    batches = [
+        torch.randn(3, 4099, generator=g),
+        torch.randn(3, 4099, generator=g) * 2.5 + 1.0,        # wider
+        torch.randn(3, 4099, generator=g) * 0.3,              # inside
+        torch.randn(3, 4099, generator=g) * 40.0 - 5.0,       # far beyond the growth limit
+        torch.cat([torch.randn(3, 4096, generator=g), torch.tensor([[float("inf"), -float("inf"), float("nan")]] * 3)], dim=1),
+    ]
+    for k, b in enumerate(batches):
+        b = b.to(dtype)
+        new_ref = ref.update(b)
+        new = obs.update(b.to(device))
+        _check_hist_lists(new, new_ref, f"batch {k} own statistics")
+        _check_hist_lists(obs.get_stats(), ref.stats, f"running statistics after batch {k}")
+
+
+@pytest.mark.parametrize("case", [((4, 1), None, (4, 300)), ((2, 3), (2, 5), (4, 15)), ((3, 1, 1), None, (2, 3, 5, 7))],
+                         ids=["per_channel", "blockwise", "activation_channels"])
+def test_histogram_several_slots(device, case):
+    from aimet_amd.quantization.encoding_analyzer import _HistogramObserver
+
+    shape, block, xshape = case
+    obs = _HistogramObserver(shape, num_bins=16, block_size=block)
+    ref = O.HistObserver(shape, 16, None, block)
+    g = torch.Generator().manual_seed(2)
+    for k in range(3):
+        x = torch.randn(xshape, generator=g) * (1 + k)
+        new_ref = ref.update(x)
+        new = obs.update(x.to(device))
+        _check_hist_lists(new, new_ref, f"batch {k}")
+        _check_hist_lists(obs.get_stats(), ref.stats, f"running {k}")
+
+
+def test_histogram_large_counts_round_like_fp32(device):
+    """Running totals above 2^24 are rounded once per batch, as the reference's fp32 accumulation does."""
+    from aimet_amd.quantization.encoding_analyzer import _HistogramObserver
+
+    obs = _HistogramObserver((1,), num_bins=4)
+    ref = O.HistObserver((1,), 4)
+    n = 9_000_001
+    for k in range(3):
+        x = torch.zeros(n)
+        x[0] = -1.0
+        x[1] = 1.0 + k * 1e-3 * 0  # same range every batch
+        ref.update(x)
+        obs.update(x.to(device))
+    _check_hist_lists(obs.get_stats(), ref.stats, "running")
+    assert ref.stats[0].histogram.max() > 2 ** 24
+
+
+@pytest.mark.parametrize("symmetric", [False, True])
+@pytest.mark.parametrize("cfg", [dict(num_bins=512, asymmetric_delta_candidates=100, offset_candidates=64, gamma=3.0),
+                                 dict(num_bins=2048), dict(num_bins=64, gamma=1.0, offset_candidates=300)],
+                         ids=["c3_grid", "defaults", "gamma1_many_offsets"])
+@pytest.mark.parametrize("num_steps", [255, 15, 65535])
+def test_sqnr_search(device, cfg, symmetric, num_steps):
+    from aimet_amd.quantization.encoding_analyzer import SqnrEncodingAnalyzer
+
+    an = SqnrEncodingAnalyzer((1,), **cfg)
+    ref = O.HistObserver((1,), cfg["num_bins"])
+    for k in range(3):
+        x = _laplace_with_outliers((64, 1024), seed=k)
+        ref.update(x)
+        an.update_stats(x.to(device))
+    lo, hi = an.compute_encodings(num_steps, symmetric)
+    kw = dict(asym_deltas=cfg.get("asymmetric_delta_candidates", 17), sym_deltas=101,
+              num_offsets=cfg.get("offset_candidates", 21), gamma=cfg.get("gamma", 3.0))
+    d_ref, o_ref = O.sqnr_candidates(ref.stats, num_steps, symmetric, kw["asym_deltas"], kw["sym_deltas"], kw["num_offsets"])
+    noise_ref = O.sqnr_noise(ref.stats, d_ref, o_ref, num_steps, 2.0, kw["gamma"])
+    lo_ref, hi_ref, bd, bo, bi = O.sqnr_encodings(ref.stats, (1,), num_steps, symmetric, **kw)
+    ls = an.last_search
+    assert_same_bits(ls["deltas"].expand_as(ls["noise"]), d_ref.expand(noise_ref.shape), "candidate deltas")
+    assert_same_bits(ls["offsets"].expand_as(ls["noise"]), o_ref.expand(noise_ref.shape), "candidate offsets")
+    assert_close_rel(ls["noise"], noise_ref, 1e-5, "noise")
+    assert int(ls["best_index"].item()) == int(bi.item()), "argmin"
+    assert_same_bits(lo, lo_ref, "encoding min")
+    assert_same_bits(hi, hi_ref, "encoding max")
+
+
+def test_tf_enhanced_preset_and_per_channel(device):
+    from aimet_amd.quantization.encoding_analyzer import TfEnhancedEncodingAnalyzer
+
+    an = TfEnhancedEncodingAnalyzer((4, 1))
+    ref = O.HistObserver((4, 1), 512, 3.0)
+    g = torch.Generator().manual_seed(9)
+    for k in range(3):
+        x = torch.randn(4, 5000, generator=g) * torch.tensor([[1.0], [0.1], [10.0], [3.0]]) * (1 + 2 * k)
+        ref.update(x)
+        an.update_stats(x.to(device))
+    for sym in (False, True):
+        lo, hi = an.compute_encodings(255, sym)
+        lo_ref, hi_ref, _, _, bi = O.sqnr_encodings(ref.stats, (4, 1), 255, sym, asym_deltas=17, sym_deltas=101,
+                                                    num_offsets=21, gamma=3.0)
+        assert torch.equal(an.last_search["best_index"].cpu(), bi)
+        assert_same_bits(lo, lo_ref, "encoding min")
+        assert_same_bits(hi, hi_ref, "encoding max")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=lambda d: str(d).split(".")[-1])
+@pytest.mark.parametrize("case", [((), None, (37, 129)), ((8, 1), None, (8, 300)), ((4, 4), (1, 32), (4, 128))],
+                         ids=["per_tensor", "per_channel", "blockwise"])
+@pytest.mark.parametrize("num_steps,symmetric", [(255, False), (255, True), (15, True), (3, True), (65535, False)])
+def test_minmax_analyzer(device, case, dtype, num_steps, symmetric):
+    from aimet_amd.quantization.encoding_analyzer import MinMaxEncodingAnalyzer
+
+    shape, block, xshape = case
+    an = MinMaxEncodingAnalyzer(shape, block)
+    g = torch.Generator().manual_seed(5)
+    mn_ref = mx_ref = None
+    for k in range(3):
+        x = (torch.randn(xshape, generator=g) * (k + 1) * 0.5).to(dtype)
+        a, b = O.reduce_minmax(x, shape, block)
+        mn_ref = a if mn_ref is None else torch.minimum(mn_ref, a)
+        mx_ref = b if mx_ref is None else torch.maximum(mx_ref, b)
+        st = an.update_stats(x.to(device))
+        assert_same_bits(st.min, a, "batch min")
+        assert_same_bits(st.max, b, "batch max")
+    lo_ref, hi_ref = O.minmax_encodings(mn_ref, mx_ref, num_steps, symmetric)
+    lo, hi = an.compute_encodings(num_steps, symmetric)
+    assert lo.dtype == dtype
+    assert_same_bits(lo, lo_ref, "encoding min")
+    assert_same_bits(hi, hi_ref, "encoding max")
+
+
+def test_minmax_degenerate_ranges(device):
+    from aimet_amd.quantization.encoding_analyzer import MinMaxEncodingAnalyzer
+
+    for x in [torch.zeros(100), torch.full((100,), 3.0), torch.full((100,), -2.0), torch.tensor([3.4e38, -3.4e38]),
+              torch.tensor([1e-12, -1e-12])]:
+        for sym in (False, True):
+            an = MinMaxEncodingAnalyzer(())
+            an.update_stats(x.to(device))
+            lo, hi = an.compute_encodings(255, sym)
+            lo_ref, hi_ref = O.minmax_encodings(x.min(), x.max(), 255, sym)
+            assert_same_bits(lo, lo_ref, "min")
+            assert_same_bits(hi, hi_ref, "max")
+
+
+@pytest.mark.parametrize("percentile", [100, 99, 80, 50])
+@pytest.mark.parametrize("symmetric", [False, True])
+def test_percentile_analyzer(device, percentile, symmetric):
+    from aimet_amd.quantization.encoding_analyzer import PercentileEncodingAnalyzer
+
+    an = PercentileEncodingAnalyzer((2, 1), num_bins=100, percentile=percentile)
+    ref = O.HistObserver((2, 1), 100)
+    g = torch.Generator().manual_seed(6)
+    for k in range(2):
+        x = torch.randn(2, 3000, generator=g) * (k + 1)
+        ref.update(x)
+        an.update_stats(x.to(device))
+    lo, hi = an.compute_encodings(255, symmetric)
+    lo_ref, hi_ref = O.percentile_encodings(ref.stats, (2, 1), percentile, 255, symmetric)
+    assert_same_bits(lo, lo_ref, "min")
+    assert_same_bits(hi, hi_ref, "max")
+
+
+def test_analyzer_errors(device):
+    from aimet_amd.quantization.encoding_analyzer import (MinMaxEncodingAnalyzer, SqnrEncodingAnalyzer,
+                                                          PercentileEncodingAnalyzer, TfEnhancedEncodingAnalyzer)
+    from aimet_amd.quantization._utils import StatisticsNotFoundError
+
+    for an in [MinMaxEncodingAnalyzer((1,)), SqnrEncodingAnalyzer((1,)), PercentileEncodingAnalyzer((1,)),
+               TfEnhancedEncodingAnalyzer((1,))]:
+        with pytest.raises(StatisticsNotFoundError):
+            an.compute_encodings(255, False)
+        an.update_stats(torch.randn(100, device=device))
+        with pytest.raises(ValueError):
+            an.compute_encodings(0, False)
+        an.reset_stats()
+        with pytest.raises(StatisticsNotFoundError):
+            an.compute_encodings(255, False)
+    with pytest.raises(ValueError):
+        SqnrEncodingAnalyzer((1,), num_bins=0)
+    with pytest.raises(ValueError):
+        PercentileEncodingAnalyzer((1,), percentile=40)
+    with pytest.raises(RuntimeError):
+        SqnrEncodingAnalyzer((1,), histogram_growth_limit=0.5)
+    with pytest.raises(RuntimeError):
+        SqnrEncodingAnalyzer((3,)).update_stats(torch.randn(4, 4, device=device))

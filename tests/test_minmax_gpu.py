@@ -45,7 +45,9 @@ def test_min_max(device, case, dtype):
     # running update == torch.minimum / torch.maximum with the previous statistics
     x2 = (torch.randn(shape, generator=g) * 2 + 0.5).to(dtype)
     mn2_ref, mx2_ref = O.reduce_minmax(x2, enc_shape, block)
-    reduce_min_max(x2.to(device), enc_shape, block, running=(mn, mx))
+    b_mn, b_mx = reduce_min_max(x2.to(device), enc_shape, block, running=(mn, mx))
+    assert_same_bits(b_mn, mn2_ref, "batch min")
+    assert_same_bits(b_mx, mx2_ref, "batch max")
     assert_same_bits(mn, torch.minimum(mn_ref, mn2_ref), "running min")
     assert_same_bits(mx, torch.maximum(mx_ref, mx2_ref), "running max")
 

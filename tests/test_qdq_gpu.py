@@ -110,7 +110,8 @@ def test_quantize_dequantize_frozen(device, layout, dtype, bitwidth, symmetric):
     qmin, qmax = _grid(bitwidth, symmetric)
     x, scale, offset, grad = _make_case(shape, enc_shape, dtype, qmin, qmax, symmetric, seed=bitwidth * 11 + 3)
     # the ATen kernels have undefined behaviour for inf * inv_scale: keep the outliers finite after scaling
-    x = torch.where(x.abs() > 1e20, torch.sign(x) * 1e4, x.float()).to(dtype)
+    xf = x.float()
+    x = torch.where(xf.abs() > 1e20, torch.sign(xf) * 1e4, xf).to(dtype)
 
     ref = O.qdq_v1(x, scale, offset, qmin, qmax)
     if ref is None:

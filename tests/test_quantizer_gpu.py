@@ -1,0 +1,250 @@
+"""End-to-end parity of the quantizer modules (calibrate -> forward -> backward) with the CPU oracle, plus the
+closed-form expectations the reference's own quantizer tests hold
+(TrainingExtensions/torch/test/python/v2/quantization/affine/test_affine_quantizer.py)."""
+
+import math
+
+import pytest
+import torch
+
+from oracle import torch_ref as O
+from tests.helpers import assert_same_bits, assert_close_rel
+
+pytestmark = pytest.mark.gpu
+
+
+class _OracleQdq(torch.autograd.Function):
+    """CPU autograd node around the oracle's quantize-dequantize so that torch's CPU autograd can carry gradients on
+    to min/max through the same scale/offset expressions the quantizer uses."""
+
+    @staticmethod
+    def forward(ctx, x, scale, offset, qmin, qmax, block, zps):
+        ctx.args = (qmin, qmax, block, zps)
+        ctx.save_for_backward(x, scale, offset)
+        return O.qdq_v2_forward(x, scale, offset, qmin, qmax, block, zps).y
+
+    @staticmethod
+    def backward(ctx, g):
+        x, scale, offset = ctx.saved_tensors
+        qmin, qmax, block, zps = ctx.args
+        gx, gs, go = O.qdq_v2_backward(g, x, scale, offset, qmin, qmax, block, zps)
+        return gx, gs, go, None, None, None, None
+
+
+class _RoundSTE(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, v):
+        return torch.round(v)
+
+    @staticmethod
+    def backward(ctx, g):
+        return g
+
+
+def _oracle_pipeline(x, grad, shape, qmin, qmax, symmetric, block, zps=0.0):
+    """min/max calibration -> parameters -> scale/offset -> QDQ forward/backward, all on the CPU."""
+    n = qmax - qmin
+    cal_steps = n - 1 if zps == 0.5 else n
+    mn, mx = O.reduce_minmax(x, shape, block)
+    emin, emax = O.minmax_encodings(mn, mx, cal_steps, symmetric)
+    pmin = emin.view(shape).float().clone().requires_grad_(True)
+    pmax = emax.view(shape).float().clone().requires_grad_(True)
+    ms = O.minimum_scale(n)
+    scale = ((pmax - pmin) / n).abs().clamp_min(ms)
+    if symmetric:
+        offset = torch.full(shape, float(-round((qmin + qmax) / 2)))
+    else:
+        offset = torch.clamp(_RoundSTE.apply(pmin / scale) - qmin, -qmax, -qmin)
+    xr = x.clone().requires_grad_(True)
+    y = _OracleQdq.apply(xr, scale, offset, qmin, qmax, block, zps)
+    y.backward(grad)
+    return dict(min=pmin.detach(), max=pmax.detach(), scale=scale.detach(), offset=offset.detach(), y=y.detach(),
+                gx=xr.grad, gmin=pmin.grad, gmax=pmax.grad)
+
+
+CASES = [
+    # name, x shape, dtype, quantizer shape, bitwidth, symmetric, block_size
+    ("c1_like", (4, 8, 28, 28), torch.float32, (), 8, False, None),
+    ("c2_like", (64, 512), torch.float32, (64, 1), 8, True, None),
+    ("blockwise_bf16", (48, 256), torch.bfloat16, (48, 4), 4, True, (1, 64)),
+    ("a16_bf16", (2, 64, 128), torch.bfloat16, (), 16, False, None),
+    ("per_channel_fp16", (16, 3, 3, 3), torch.float16, (16, 1, 1, 1), 8, True, None),
+]
+
+
+@pytest.mark.parametrize("case", CASES, ids=lambda c: c[0])
+def test_calibrate_forward_backward(device, case):
+    from aimet_amd.quantization.affine import QuantizeDequantize
+
+    _, xshape, dtype, qshape, bw, sym, block = case
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(xshape, generator=g)
+    if not sym:
+        x = torch.relu(x)
+    x = x.to(dtype)
+    grad = torch.randn(xshape, generator=g).to(dtype)
+    n = 2 ** bw - 1
+    qmin, qmax = (-math.ceil(n / 2), math.floor(n / 2)) if sym else (0, n)
+    ref = _oracle_pipeline(x, grad, qshape, qmin, qmax, sym, block)
+
+    q = QuantizeDequantize(qshape, bw, sym, block_size=block).to(device)
+    xd = x.to(device)
+    with q.compute_encodings():
+        out_dyn = q(xd)
+    assert_same_bits(q.min, ref["min"], "calibrated min")
+    assert_same_bits(q.max, ref["max"], "calibrated max")
+    assert_same_bits(q.get_scale(), ref["scale"], "scale")
+    assert_same_bits(q.get_offset(), ref["offset"], "offset")
+    xd = xd.clone().requires_grad_(True)
+    y = q(xd)
+    assert type(y).__name__ == "DequantizedTensor" and y.encoding is not None
+    assert_same_bits(y, ref["y"], "forward")
+    # inside compute_encodings the output is quantized with the batch's own encodings; those do not require grad,
+    # so the reference (and this backend) take the ATen arithmetic wherever it applies
+    dyn_ref = None if block is not None else O.qdq_v1(x, ref["scale"], ref["offset"], qmin, qmax)
+    dyn_y = ref["y"] if dyn_ref is None else dyn_ref[0]
+    assert_same_bits(out_dyn, dyn_y, "dynamic forward")
+    y.backward(grad.to(device))
+    assert_same_bits(xd.grad, ref["gx"], "input gradient")
+    D = O.internal_dtype(dtype, qmin, qmax)
+    tol = 1e-5 if D == torch.float32 else float(torch.finfo(D).eps)
+    assert_close_rel(q.min.grad, ref["gmin"], tol, "min gradient", abs_floor=1e-30)
+    assert_close_rel(q.max.grad, ref["gmax"], tol, "max gradient", abs_floor=1e-30)
+
+
+def test_frozen_quantizer_takes_aten_arithmetic(device):
+    """requires_grad_(False) on the quantizer selects the ATen fake-quantize arithmetic, as in the reference."""
+    from aimet_amd.quantization.affine import QuantizeDequantize
+
+    g = torch.Generator().manual_seed(1)
+    x = torch.relu(torch.randn(3, 1000, generator=g))
+    q = QuantizeDequantize((), 8, False).to(device)
+    with q.compute_encodings():
+        q(x.to(device))
+    scale, offset = q.get_scale().detach().cpu(), q.get_offset().detach().cpu()
+    q.requires_grad_(False)
+    y = q(x.to(device))
+    y_ref, _ = O.qdq_v1(x, scale, offset, 0, 255)
+    assert_same_bits(y, y_ref, "frozen forward")
+    with torch.no_grad():
+        q.requires_grad_(True)
+        assert_same_bits(q(x.to(device)), y_ref, "no_grad forward")
+
+
+@pytest.mark.parametrize("bw,symmetric,expected_scale", [(2, True, 5.25), (2, False, 7.0), (3, True, 3.5), (3, False, 3.0)])
+def test_compute_encodings_low_bw(device, bw, symmetric, expected_scale):
+    """Reference expectation: test_affine_quantizer.py:397-406."""
+    from aimet_amd.quantization.affine import QuantizeDequantize
+
+    qdq = QuantizeDequantize(shape=(), bitwidth=bw, symmetric=symmetric).to(device)
+    with qdq.compute_encodings():
+        qdq(torch.tensor([-10.5, 10.5], device=device))
+    assert qdq.get_scale().item() == expected_scale
+
+
+@pytest.mark.parametrize("bitwidth,decompressed_bw", [[4, 8], [4, 16], [4, 12], [3, 5], [5, 9], [6, 6]])
+def test_gbbq_per_block_sanity(device, bitwidth, decompressed_bw):
+    """Reference expectation: test_affine_quantizer.py:1426-1474 -- every LPBQ block scale equals
+    max(1, round(scale / gamma)) * gamma with gamma = (largest block scale of the group) / 2^(decompressed_bw - bw)."""
+    from aimet_amd.quantization.affine import GroupedBlockQuantizeDequantize, QuantizeDequantize
+
+    g = torch.Generator().manual_seed(0)
+    tensor = torch.randn(4, 8, 12, generator=g).to(device)
+    gbbq = GroupedBlockQuantizeDequantize(shape=(2, 4, 6), bitwidth=bitwidth, symmetric=True, block_size=(2, 2, 2),
+                                          decompressed_bw=decompressed_bw, block_grouping=(2, 2, 3)).to(device)
+    qdq = QuantizeDequantize(shape=(2, 4, 6), bitwidth=bitwidth, symmetric=True, block_size=(2, 2, 2)).to(device)
+    with gbbq.compute_encodings():
+        gbbq(tensor)
+    with qdq.compute_encodings():
+        qdq(tensor)
+    gs, qs = gbbq.get_scale().detach().cpu(), qdq.get_scale().detach().cpu()
+    for j in range(2):
+        for k in range(2):
+            grp_g = gs[0:2, 2 * j:2 * j + 2, 3 * k:3 * k + 3]
+            grp_q = qs[0:2, 2 * j:2 * j + 2, 3 * k:3 * k + 3]
+            gamma = torch.max(grp_q) / 2 ** (decompressed_bw - bitwidth)
+            expect = torch.maximum(torch.tensor([1.0]), torch.round(grp_q / gamma)) * gamma
+            assert torch.equal(expect, grp_g)
+
+
+def test_zero_point_shift_equals_nearest_of_four_levels(device):
+    """Reference expectation: test_affine_quantizer.py:2679-2711."""
+    from aimet_amd.quantization.affine import QuantizeDequantize
+
+    g = torch.Generator().manual_seed(0)
+    for _ in range(10):
+        quantizer = QuantizeDequantize(shape=(), bitwidth=2, symmetric=True, zero_point_shift=0.5).to(device)
+        t = torch.rand(5, 10, generator=g) * 10.0 - 5
+        with quantizer.compute_encodings():
+            quantizer(t.to(device))
+        scale = torch.max(torch.abs(t)) / 1.5
+        assert quantizer.get_scale().item() == scale.item()
+        levels = torch.tensor([scale * -1.5, scale * -0.5, scale * 0.5, scale * 1.5])
+        nearest = levels[torch.cdist(t.flatten().unsqueeze(1), levels.unsqueeze(1)).argmin(dim=1)].reshape(t.shape)
+        assert torch.equal(nearest, quantizer(t.to(device)).detach().cpu())
+
+
+def test_lpbq_c4_like(device):
+    """Blockwise 4-bit weights with 8-bit per-channel scale (LPBQ) on bf16, forward + backward vs the oracle."""
+    from aimet_amd.quantization.affine import GroupedBlockQuantizeDequantize
+
+    g = torch.Generator().manual_seed(0)
+    w = (torch.randn(96, 512, generator=g) * 0.02).bfloat16()
+    grad = torch.randn(96, 512, generator=g).bfloat16()
+    q = GroupedBlockQuantizeDequantize(shape=(96, 8), bitwidth=4, symmetric=True, decompressed_bw=8,
+                                       block_size=(1, 64), block_grouping=(1, -1)).to(device)
+    with q.compute_encodings():
+        q(w.to(device))
+    mn, mx = O.reduce_minmax(w, (96, 8), (1, 64))
+    emin, emax = O.minmax_encodings(mn, mx, 15, True)
+    assert_same_bits(q.min, emin.float(), "min")
+    assert_same_bits(q.max, emax.float(), "max")
+    raw = O.scale_from_minmax(emin, emax, -8, 7)
+    scale, pcs = O.lpbq_scale(raw, 4, 8, (1, -1))
+    enc = q.get_encodings()
+    assert_same_bits(enc.per_channel_scale, pcs, "per-channel scale")
+    assert_same_bits(enc.scale, scale, "LPBQ scale")
+    mult = enc.per_block_int_scale.detach().cpu()
+    assert mult.min() >= 1 and mult.max() <= 16 and torch.equal(mult, mult.round())
+    offset = torch.zeros(96, 8)
+    wd = w.to(device).requires_grad_(True)
+    y = q(wd)
+    assert_same_bits(y, O.qdq_v2_forward(w, scale, offset, -8, 7, (1, 64)).y, "forward")
+    y.backward(grad.to(device))
+    gx_ref, _, _ = O.qdq_v2_backward(grad, w, scale, offset, -8, 7, (1, 64))
+    assert_same_bits(wd.grad, gx_ref, "input gradient")
+    assert q.min.grad is not None and q.max.grad is not None
+
+
+def test_quantize_module_and_state_dict(device):
+    from aimet_amd.quantization.affine import Quantize, QuantizeDequantize, Dequantize
+
+    x = torch.randn(8, 32, generator=torch.Generator().manual_seed(3))
+    q = Quantize((8, 1), 8, False).to(device)
+    with pytest.raises(RuntimeError):
+        q(x.to(device))
+    with q.compute_encodings():
+        q(x.to(device))
+    out = q(x.to(device))
+    assert type(out).__name__ == "QuantizedTensor"
+    codes_ref, _ = O.quantize_forward(x, q.get_scale().detach().cpu(), q.get_offset().detach().cpu(), 0, 255)
+    assert_same_bits(out, codes_ref, "codes")
+    assert_same_bits(out.dequantize(), O.dequantize_forward(codes_ref, q.get_scale().detach().cpu(),
+                                                            q.get_offset().detach().cpu()), "dequantize()")
+    # checkpoint round trip keeps values and initialised-ness
+    q2 = Quantize((8, 1), 8, False).to(device)
+    assert not q2.is_initialized()
+    q2.load_state_dict(q.state_dict())
+    assert q2.is_initialized()
+    assert_same_bits(q2(x.to(device)), codes_ref, "codes after load")
+    # frozen parameters are not overwritten
+    q2.allow_overwrite(False)
+    before = q2.min.detach().clone()
+    with q2.compute_encodings():
+        q2(10 * x.to(device))
+    assert torch.equal(before, q2.min.detach())
+    # empty input passes through an uninitialised quantizer
+    q3 = QuantizeDequantize((), 8, False).to(device)
+    assert q3(torch.empty(0, 3, device=device)).shape == (0, 3)
+    with pytest.raises(RuntimeError):
+        Dequantize((), 8, False).to(device)(x.to(device))
