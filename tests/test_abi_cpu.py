@@ -1,0 +1,178 @@
+"""Host-side checks that need no GPU: the shared library loads and exports the C ABI of include/aimet_amd.h, argument
+validation answers with error codes before anything is launched, workspace queries and layout planning are pure host
+code, and the Python front end keeps the reference's registry / overload / error behaviour."""
+
+import ctypes
+import os
+import re
+import subprocess
+import sys
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from aimet_amd import _lib
+
+    if not os.path.exists(_lib.LIB_PATH):
+        from aimet_amd.csrc.build import build
+
+        build(verbose=False)
+    return _lib.load()
+
+
+def test_every_declared_symbol_is_exported_and_bound(lib):
+    from aimet_amd import _lib
+
+    header = open(os.path.join(ROOT, "include", "aimet_amd.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    declared = set(re.findall(r"\b(ahq_[a-z0-9_]+)\s*\(", header))
+    assert declared, "no declarations found"
+    for name in declared:
+        assert hasattr(lib, name), f"{name} is declared in include/aimet_amd.h but not exported"
+    assert declared == set(_lib.exported_symbols()), "ctypes bindings and header disagree"
+    assert lib.ahq_version() >= 1
+
+
+def test_argument_validation_without_a_gpu(lib):
+    from aimet_amd import _lib
+
+    g = _lib.Grid()
+    g.arith, g.op, g.io_dtype, g.compute_dtype, g.qmin, g.qmax = _lib.AHQ_ARITH_AUTOGRAD, 0, 0, 0, 0, 255
+    lay = _lib.make_layout([16], [16], [0])
+    assert lib.ahq_qdq_forward(None, lay, None, None, None, None, None, None, None, None) == 1
+    assert b"grid" in lib.ahq_last_error()
+    assert lib.ahq_qdq_forward(g, lay, None, None, None, None, None, None, None, None) == 1  # scale is null
+    g.qmin, g.qmax = 5, 1
+    assert lib.ahq_qdq_forward(g, lay, None, None, None, 1, None, None, None, None) == 1
+    assert b"qmin" in lib.ahq_last_error()
+    g.qmin, g.qmax, g.compute_dtype = 0, 255, _lib.AHQ_BF16  # fp32 tensors cannot compute in bf16
+    assert lib.ahq_qdq_forward(g, lay, None, None, None, 1, None, None, None, None) == 1
+    g.compute_dtype, g.zero_point_shift = 0, 0.25
+    assert lib.ahq_qdq_forward(g, lay, None, None, None, 1, None, None, None, None) == 1
+    g.zero_point_shift = 0.0
+    g.arith = _lib.AHQ_ARITH_DLQ
+    assert lib.ahq_qdq_backward(g, lay, None, None, None, None, None, 1, None, None, 0, None) == 1
+    bad = _lib.make_layout([16], [5], [0])  # block does not divide the dimension
+    g.arith = _lib.AHQ_ARITH_AUTOGRAD
+    assert lib.ahq_qdq_forward(g, bad, None, None, None, 1, None, None, None, None) == 1
+    assert lib.ahq_minmax(7, lay, None, 1, 1, None, None, 0, None, 0, None) == 1
+    assert lib.ahq_minmax(0, lay, None, None, None, None, None, 0, None, 0, None) == 1
+    assert lib.ahq_hist_update(0, lay, None, None, 1, None, 0, None) == 1
+    assert lib.ahq_sqnr_search(None, None, None, None, None, None, None, None, None, None, None) == 1
+
+
+def test_workspace_queries_and_planning(lib):
+    from aimet_amd import _lib
+
+    g = _lib.Grid()
+    g.arith, g.op, g.io_dtype, g.compute_dtype, g.qmin, g.qmax = _lib.AHQ_ARITH_AUTOGRAD, 0, 0, 0, -128, 127
+    per_tensor = _lib.make_layout([32 * 64 * 112 * 112], [32 * 64 * 112 * 112], [0])
+    per_channel = _lib.make_layout([4096, 4096], [1, 4096], [1, 0])
+    blockwise = _lib.make_layout([14336, 4096], [1, 64], [64, 1])
+    assert lib.ahq_qdq_backward_workspace_bytes(g, per_tensor, 0) == 0
+    # per-tensor: one (gscale, goffset) pair of doubles per 16 KiB tile
+    tiles = -(-32 * 64 * 112 * 112 // 4096)
+    assert lib.ahq_qdq_backward_workspace_bytes(g, per_tensor, 1) >= tiles * 16
+    # one tile per row / one wave segment per block: written directly (only the unaligned fallback needs scratch)
+    assert lib.ahq_qdq_backward_workspace_bytes(g, per_channel, 1) <= 4096 * 4 * 16
+    assert lib.ahq_minmax_workspace_bytes(per_tensor) >= tiles * 12
+    assert lib.ahq_hist_update_workspace_bytes(0, per_tensor, 512) > 1024 * 2 * 514 * 4
+    assert lib.ahq_qdq_backward_workspace_bytes(g, blockwise, 1) >= 0
+
+
+def test_backend_registry():
+    import aimet_amd.quantization as Q
+    from aimet_amd.quantization.affine.backends import hip
+
+    assert Q.get_backend() is hip
+
+    class Dummy:
+        quantize = dequantize = quantize_dequantize = staticmethod(lambda *a, **k: "dummy")
+
+    assert Q.add_backend("dummy", Dummy) is None
+    assert isinstance(Q.add_backend("dummy", Dummy), RuntimeError)  # returned, not raised
+    with Q.set_backend("dummy"):
+        assert Q.get_backend() is Dummy
+        assert Q.affine.quantize_dequantize(torch.zeros(1), torch.ones(()), torch.zeros(()), 8) == "dummy"
+    assert Q.get_backend() is hip
+    with pytest.raises(RuntimeError):
+        Q.set_backend("no-such-backend")
+
+
+def test_overload_parsing():
+    from aimet_amd.quantization.affine.backends import _parse_args, _derive_qmin_qmax
+
+    assert _parse_args((8,), {}) == (0, 255, None, 0.0)
+    assert _parse_args((8, True), {}) == (-128, 127, None, 0.0)
+    assert _parse_args((), {"bitwidth": 4, "signed": True, "block_size": (1, 64)}) == (-8, 7, (1, 64), 0.0)
+    assert _parse_args((), {"num_steps": 15, "signed": False}) == (0, 15, None, 0.0)
+    assert _parse_args((-7, 7), {"zero_point_shift": 0.5}) == (-7, 7, None, 0.5)
+    assert _parse_args((0, 255, (2, 2)), {}) == (0, 255, (2, 2), 0.0)
+    assert _derive_qmin_qmax(num_steps=3, signed=True) == (-2, 1)
+    with pytest.raises(RuntimeError):
+        import aimet_amd.quantization as Q
+        Q.affine.quantize(torch.zeros(1), torch.ones(()), torch.zeros(()), 8, zero_point_shift=0.5)
+
+
+def test_cpu_tensors_fail_loudly():
+    """There is no CPU or eager-PyTorch fallback: the product path raises on tensors that are not on the GPU."""
+    import aimet_amd.quantization as Q
+    from aimet_amd.quantization.encoding_analyzer import MinMaxEncodingAnalyzer, SqnrEncodingAnalyzer
+
+    x = torch.randn(4, 4)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        Q.affine.quantize_dequantize(x, torch.tensor(0.1), torch.tensor(0.0), 8)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        MinMaxEncodingAnalyzer(()).update_stats(x)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        SqnrEncodingAnalyzer(()).update_stats(x)
+    # shape errors are reported before the device check, like the reference's validation
+    with pytest.raises(RuntimeError, match="cannot be expanded"):
+        Q.affine.quantize_dequantize(torch.randn(2, 3, 4, 5), torch.ones(4), torch.zeros(()), 0, 255)
+
+
+def test_quantizer_construction_and_bookkeeping_on_cpu():
+    from aimet_amd.quantization.affine import QuantizeDequantize, GroupedBlockQuantizeDequantize, Quantize
+
+    q = QuantizeDequantize((3, 1), 8, True)
+    assert (q.qmin, q.qmax, q.bitwidth, q.signed, q.symmetric) == (-128, 127, 8, True, True)
+    assert not q.is_initialized() and q.get_scale() is None and q.get_encodings() is None
+    q.set_range(-torch.ones(3, 1), torch.ones(3, 1))
+    assert q.is_initialized()
+    assert torch.equal(q.get_offset(), torch.zeros(3, 1))
+    q2 = QuantizeDequantize((), qmin=0, qmax=15, symmetric=False)
+    assert q2.bitwidth == 4 and not q2.signed
+    q2.bitwidth = 8
+    assert (q2.qmin, q2.qmax) == (0, 255)
+    with pytest.raises(ValueError):
+        QuantizeDequantize((), qmin=3, qmax=3, symmetric=False)
+    with pytest.raises(ValueError):
+        QuantizeDequantize((), 8, True, zero_point_shift=0.3)
+    with pytest.raises(RuntimeError):
+        Quantize((), 8, True, zero_point_shift=0.5)
+    with pytest.raises(RuntimeError):
+        GroupedBlockQuantizeDequantize((4, 2), 4, False, 8, None, (1, 8), (1, -1))
+    with pytest.raises(RuntimeError):
+        GroupedBlockQuantizeDequantize((4, 2), 8, True, 4, None, (1, 8), (1, -1))
+    with pytest.raises(TypeError):
+        QuantizeDequantize((), 8, True, bogus=1)
+    sd = q.state_dict()
+    q3 = QuantizeDequantize((3, 1), 8, True)
+    q3.load_state_dict(sd)
+    assert q3.is_initialized() and torch.equal(q3.max, q.max)
+    import copy
+    assert copy.deepcopy(q).is_initialized() and not copy.deepcopy(QuantizeDequantize((), 8, True)).is_initialized()
+
+
+def test_product_never_imports_the_oracle():
+    out = subprocess.run(["grep", "-rIl", "--include=*.py", "--include=*.hip", "--include=*.h", "-e", "oracle",
+                          os.path.join(ROOT, "aimet_amd")], capture_output=True, text=True).stdout.split()
+    assert out == [], f"product files mention the oracle: {out}"
+    code = "import sys; import aimet_amd.quantization, aimet_amd.quantization.affine, aimet_amd.quantization.encoding_analyzer; print(any(m.startswith('oracle') for m in sys.modules))"
+    res = subprocess.run([sys.executable, "-c", code], cwd=ROOT, capture_output=True, text=True)
+    assert res.stdout.strip() == "False", res.stdout + res.stderr
