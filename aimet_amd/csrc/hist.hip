@@ -27,6 +27,7 @@ namespace ahq {
 
 constexpr int kHistBlocksMax = 1024;  // persistent workgroups of the binning pass (4 per CU)
 constexpr int kRng = 8;               // floats per slot in `ranges`
+constexpr int kFoldGroups = 32;       // partial histograms left after the first fold
 
 // ranges[slot]: lo1, hi1, thr_lo1, thr_hi1 (batch's own range), lo2, hi2, thr_lo2, thr_hi2 (updated range).
 // thr_* are the edges rounded to the tensor dtype: the reference compares `x < edge` in the tensor's dtype.
@@ -120,24 +121,25 @@ __global__ void hist_prepare_kernel(const PrepArgs a) {
             oi[i] = o < B - 1 ? o : B - 1;
         }
         __syncthreads();
-        // index_add_ runs over the source bins in order: reproduce that order for every destination bin
+        // index_add_ runs over the source bins in order.  Both index arrays are non-decreasing, so the sources of a
+        // destination bin form one contiguous run: find it by bisection and add it up in source order.
         for (int d = threadIdx.x; d < B; d += blockDim.x) {
             float acc = 0.f;
-            for (int i = 0; i < B; ++i) {
-                if (di[i] == d) {
-                    const float start = ce[i];
-                    const float dst_end = umin + dst_w * (float)(di[i] + 1);
-                    const float part = __builtin_rintf(((dst_end - start) / src_w) * ch[i]);
-                    acc += fminf(part, ch[i]);
+            for (int pass = 0; pass < 2; ++pass) {
+                const int32_t* idx = pass == 0 ? di : oi;
+                int lo = 0, hi = B;
+                while (lo < hi) {  // first i with idx[i] >= d
+                    const int mid = (lo + hi) >> 1;
+                    if (idx[mid] < d) lo = mid + 1;
+                    else hi = mid;
                 }
-            }
-            for (int i = 0; i < B; ++i) {
-                if (oi[i] == d) {
+                for (int i = lo; i < B && idx[i] == d; ++i) {
                     const float start = ce[i];
                     const float dst_end = umin + dst_w * (float)(di[i] + 1);
                     const float part = __builtin_rintf(((dst_end - start) / src_w) * ch[i]);
                     const float first = fminf(part, ch[i]);
-                    if (first < ch[i]) acc += ch[i] - first;
+                    if (pass == 0) acc += first;
+                    else if (first < ch[i]) acc += ch[i] - first;
                 }
             }
             carried[d] = acc;
@@ -169,12 +171,13 @@ struct BinArgs : Geom {
     uint32_t* counts;      // several slots: [S][NH][B + 2], zero-initialised
     int32_t num_bins;
     int32_t nhist;
-    int32_t copies;        // wave-private LDS copies (1..4)
+    int32_t copies;        // interleaved LDS copies of each histogram (power of two, 1..8)
+    int32_t copy_shift;    // log2(copies)
     int64_t ntiles;
 };
 
 struct RangeC {
-    float lo, hi, width, thr_lo, thr_hi;
+    float lo, hi, width, rwidth, thr_lo, thr_hi;
 };
 
 __device__ __forceinline__ RangeC load_range(const float* rg, int h) {
@@ -187,22 +190,43 @@ __device__ __forceinline__ RangeC load_range(const float* rg, int h) {
         r.hi += 1.f;
     }
     r.width = r.hi - r.lo;
+    r.rwidth = 1.0f / r.width;
     r.thr_lo = rg[4 * h + 2];
     r.thr_hi = rg[4 * h + 3];
     return r;
 }
 
-// returns the bin of v in range r or -1
-__device__ __forceinline__ int bin_of(float v, const RangeC& r, float Bf, int B) {
-    if (!(v >= r.lo && v <= r.hi)) return -1;
-    int p = (int)(((v - r.lo) * Bf) / r.width);
-    return p >= B ? B - 1 : p;
+// Reference bin index: trunc(((v - lo) * B) / width) with a correctly rounded fp32 division, capped at B - 1.
+__device__ __forceinline__ int bin_exact(float v, const RangeC& r, float Bf, int B) {
+    const int p = (int)(((v - r.lo) * Bf) / r.width);
+    return p > B - 1 ? B - 1 : p;
 }
 
-// Single-slot fast path: persistent workgroups, wave-private LDS sub-histograms, one partial per workgroup.
+// Division-free estimate of the same index.  q1 = q0 + (t - q0*w) * (1/w) with fused multiply-adds differs from the
+// correctly rounded quotient by at most one unit in the last place (the residual is evaluated without rounding of
+// the product, so q0 + e/w is the true quotient to ~2^-46 and rounds to the quotient or to its neighbour).  The two
+// can only truncate differently when q1 is an integer or the float just below one.  `fast` is true when
+//   * q1 is not within q1 * 2^-23 (>= one ulp) of an integer, and
+//   * 0 <= q1 < B - 4 ulp, tested on the bit pattern (negative values, -0, NaN and +inf all compare above the limit).
+// v < lo gives q1 <= 0 with the sign bit set; v > hi gives a quotient of at least B - 2 ulp; so a `fast` element is
+// inside the range and its truncated estimate is the reference bin.  Everything else is redone with bin_exact().
+__device__ __forceinline__ int bin_estimate(float v, const RangeC& r, float Bf, uint32_t limit_bits, bool& fast) {
+    const float t = (v - r.lo) * Bf;
+    const float q0 = t * r.rwidth;
+    const float e = __builtin_fmaf(-q0, r.width, t);
+    const float q1 = __builtin_fmaf(e, r.rwidth, q0);
+    const bool safe = __builtin_fabsf(__builtin_rintf(q1) - q1) > q1 * 1.1920929e-7f;
+    fast = safe & (f32_to_bits(q1) < limit_bits);
+    return (int)q1;
+}
+
+// Single-slot fast path: persistent workgroups, lane-interleaved LDS sub-histograms, one partial per workgroup.
+// The kernel is bound by instruction issue, not by LDS or HBM, so the per-element path is kept free of branches:
+// elements that need the exact division or lie outside the range are only flagged, and one wave-uniform branch per
+// tile revisits them.
 template <typename IO, int VEC, int NH>
 __global__ __launch_bounds__(kBlock) void hist_bin_kernel(const BinArgs a) {
-    extern __shared__ uint32_t lds[];  // [copies][NH][B]
+    extern __shared__ uint32_t lds[];  // [NH][B][copies]: lane l adds to copy l % copies, neighbouring copies sit in neighbouring banks
     __shared__ uint32_t cnt_smem[kBlock / kWave][NH][2];
     const int B = a.num_bins;
     const float Bf = (float)B;
@@ -213,52 +237,75 @@ __global__ __launch_bounds__(kBlock) void hist_bin_kernel(const BinArgs a) {
     for (int h = 0; h < NH; ++h) r[h] = load_range(a.ranges, h);
     __syncthreads();
     const int wave = threadIdx.x / kWave;
-    uint32_t* mine = lds + (size_t)(wave % copies) * NH * B;
+    const int cshift = a.copy_shift;  // copies == 1 << cshift
+    const int bshift = cshift + 2;    // bin index -> byte offset inside one histogram
+    const uint32_t limit_bits = f32_to_bits(Bf) - 4u;
+    uint32_t* mine[NH];
+#pragma unroll
+    for (int h = 0; h < NH; ++h) mine[h] = lds + (size_t)h * B * copies + (threadIdx.x & (copies - 1));
     const IO* __restrict__ x = static_cast<const IO*>(a.x);
     uint32_t below[NH], above[NH];
 #pragma unroll
     for (int h = 0; h < NH; ++h) below[h] = above[h] = 0;
 
-    for (int64_t tile = blockIdx.x; tile < a.ntiles; tile += gridDim.x) {
-        const int64_t v0 = tile * kTileVec;
-        const int64_t left = a.nvec - v0;
-        const int nv = (int)(left < kTileVec ? left : kTileVec);
+    // every element, exactly (ragged tile, tail elements and the revisit of flagged elements)
+    auto bin_slow = [&](float v, bool only_flagged) {
+#pragma unroll
+        for (int h = 0; h < NH; ++h) {
+            const bool inr = (v >= r[h].lo) & (v <= r[h].hi);
+            bool fast = false;
+            if (only_flagged) (void)bin_estimate(v, r[h], Bf, limit_bits, fast);
+            if (inr & !fast) atomicAdd(&mine[h][bin_exact(v, r[h], Bf, B) << cshift], 1u);
+            // values below/above the edges (rounded to the tensor dtype) are necessarily outside the fp32 range
+            if (!inr) {
+                below[h] += v < r[h].thr_lo ? 1u : 0u;
+                above[h] += v > r[h].thr_hi ? 1u : 0u;
+            }
+        }
+    };
+
+    const int64_t full_tiles = a.nvec / kTileVec;
+    for (int64_t tile = blockIdx.x; tile < full_tiles; tile += gridDim.x) {
         Pack<IO, VEC> in[kUnroll];
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
-            const int lv = u * kBlock + threadIdx.x;
-            if (lv < nv) in[u] = load_pack<IO, VEC>(x + (v0 + lv) * VEC);
-        }
+        for (int u = 0; u < kUnroll; ++u) in[u] = load_pack<IO, VEC>(x + (tile * kTileVec + u * kBlock + threadIdx.x) * VEC);
+        uint32_t binned = 0;  // this lane's elements that took the fast path
 #pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) {
+                const float v = load_f32(in[u].v[k]);
+#pragma unroll
+                for (int h = 0; h < NH; ++h) {
+                    bool fast;
+                    const int b = bin_estimate(v, r[h], Bf, limit_bits, fast);
+                    if (fast) {
+                        atomicAdd(reinterpret_cast<uint32_t*>(reinterpret_cast<char*>(mine[h]) + ((uint32_t)b << bshift)), 1u);
+                        ++binned;
+                    }
+                }
+            }
+        }
+        if (__builtin_amdgcn_ballot_w64(binned != (uint32_t)(kUnroll * VEC * NH)) != 0) {
+            for (int u = 0; u < kUnroll; ++u)
+                for (int k = 0; k < VEC; ++k) bin_slow(load_f32(in[u].v[k]), true);
+        }
+    }
+    // the ragged last tile
+    if (blockIdx.x == 0 && full_tiles * kTileVec < a.nvec) {
+        const int64_t v0 = full_tiles * kTileVec;
+        const int nv = (int)(a.nvec - v0);
         for (int u = 0; u < kUnroll; ++u) {
             const int lv = u * kBlock + threadIdx.x;
             if (lv < nv) {
-#pragma unroll
-                for (int k = 0; k < VEC; ++k) {
-                    const float v = load_f32(in[u].v[k]);
-#pragma unroll
-                    for (int h = 0; h < NH; ++h) {
-                        const int b = bin_of(v, r[h], Bf, B);
-                        if (b >= 0) atomicAdd(&mine[h * B + b], 1u);
-                        below[h] += v < r[h].thr_lo ? 1u : 0u;
-                        above[h] += v > r[h].thr_hi ? 1u : 0u;
-                    }
-                }
+                const Pack<IO, VEC> pk = load_pack<IO, VEC>(x + (v0 + lv) * VEC);
+                for (int k = 0; k < VEC; ++k) bin_slow(load_f32(pk.v[k]), false);
             }
         }
     }
     if (VEC > 1 && blockIdx.x == 0) {  // elements past the last full vector
         const int64_t i = a.nvec * VEC + threadIdx.x;
-        if (i < a.numel) {
-            const float v = load_f32(x[i]);
-#pragma unroll
-            for (int h = 0; h < NH; ++h) {
-                const int b = bin_of(v, r[h], Bf, B);
-                if (b >= 0) atomicAdd(&mine[h * B + b], 1u);
-                below[h] += v < r[h].thr_lo ? 1u : 0u;
-                above[h] += v > r[h].thr_hi ? 1u : 0u;
-            }
-        }
+        if (i < a.numel) bin_slow(load_f32(x[i]), false);
     }
     // below / above: wave reduce, then across waves
 #pragma unroll
@@ -279,7 +326,7 @@ __global__ __launch_bounds__(kBlock) void hist_bin_kernel(const BinArgs a) {
     for (int i = threadIdx.x; i < NH * B; i += kBlock) {
         const int h = i / B, b = i - h * B;
         uint32_t c = 0;
-        for (int cp = 0; cp < copies; ++cp) c += lds[(size_t)cp * NH * B + i];
+        for (int cp = 0; cp < copies; ++cp) c += lds[(size_t)i * copies + cp];
         out[h * (B + 2) + b] = c;
     }
     if (threadIdx.x < NH * 2) {
@@ -305,8 +352,7 @@ __global__ __launch_bounds__(kBlock) void hist_bin_generic_kernel(const BinArgs 
         uint32_t* c = a.counts + (size_t)e * a.nhist * (B + 2);
         for (int h = 0; h < a.nhist; ++h) {
             const RangeC r = load_range(rg, h);
-            const int b = bin_of(v, r, Bf, B);
-            if (b >= 0) atomicAdd(&c[h * (B + 2) + b], 1u);
+            if ((v >= r.lo) & (v <= r.hi)) atomicAdd(&c[h * (B + 2) + bin_exact(v, r, Bf, B)], 1u);
             if (v < r.thr_lo) atomicAdd(&c[h * (B + 2) + B], 1u);
             if (v > r.thr_hi) atomicAdd(&c[h * (B + 2) + B + 1], 1u);
         }
@@ -315,6 +361,18 @@ __global__ __launch_bounds__(kBlock) void hist_bin_generic_kernel(const BinArgs 
 
 __global__ void zero_u32_kernel(uint32_t* p, int64_t n) {
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) p[i] = 0;
+}
+
+// ------------------------------------------------------------------------------------ fold of the partial counts --
+// partial[p][l] (p < nparts, l < len) -> folded[g][l] = sum of the partials p with p % groups == g
+__global__ __launch_bounds__(kBlock) void hist_fold_kernel(const uint32_t* partial, uint32_t* folded, int nparts, int len, int groups) {
+    const int l = blockIdx.x * kBlock + threadIdx.x;
+    const int g = blockIdx.y;
+    if (l >= len) return;
+    uint32_t acc = 0;
+#pragma unroll 4
+    for (int p = g; p < nparts; p += groups) acc += partial[(size_t)p * len + l];
+    folded[(size_t)g * len + l] = acc;
 }
 
 // ----------------------------------------------------------------------------------------------------- finish --
@@ -346,12 +404,16 @@ __global__ __launch_bounds__(kBlock) void hist_finish_kernel(const FinArgs a) {
     sm[grp][0][bl] = c[0];
     sm[grp][1][bl] = c[1];
     // below/above totals (needed by the workgroups that own bin 0 and bin B-1; cheap enough to do everywhere)
-    if (threadIdx.x < 4) {
-        const int h = threadIdx.x >> 1, w = threadIdx.x & 1;
+    {
+        // wave w (0..3) owns edge counter (h = w / 2, side = w % 2); its lanes stride over the partials
+        const int w4 = threadIdx.x >> 6, lane = threadIdx.x & 63;
+        const int h = w4 >> 1, side = w4 & 1;
         unsigned long long t = 0;
         if (h < NH)
-            for (int p = 0; p < a.nparts; ++p) t += base[((size_t)p * NH + h) * (B + 2) + B + w];
-        edge_cnt[h][w] = t;
+            for (int p = lane; p < a.nparts; p += 64) t += base[((size_t)p * NH + h) * (B + 2) + B + side];
+#pragma unroll
+        for (int m = 32; m >= 1; m >>= 1) t += __shfl_xor(t, m, kWave);
+        if (lane == 0) edge_cnt[h][side] = t;
     }
     __syncthreads();
     if (grp != 0 || b >= B) return;
@@ -388,7 +450,7 @@ struct HistPlan {
     int copies;
     int nblocks;
     int64_t ntiles;
-    size_t off_mm_ws, off_bmin, off_bmax, off_ranges, off_carried, off_upd_edges, off_scratch, off_counts, total;
+    size_t off_mm_ws, off_bmin, off_bmax, off_ranges, off_carried, off_upd_edges, off_scratch, off_counts, off_folded, total;
 };
 
 size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
@@ -400,8 +462,13 @@ bool make_hist_plan(int dtype, const ahq_layout& layout, const void* x, int num_
     hp->fast = false;
     hp->copies = 0;
     if (c.kind == kIJK && c.J == 1) {
-        int copies = (int)((65536 - 512) / ((size_t)2 * num_bins * 4));
-        if (copies > 4) copies = 4;
+        const int fit = (int)((65536 - 512) / ((size_t)2 * num_bins * 4));
+        int copies = 0;
+        for (int c = 8; c >= 1; c >>= 1)
+            if (c <= fit) {
+                copies = c;
+                break;
+            }
         if (copies >= 1) {
             hp->fast = true;
             hp->copies = copies;
@@ -424,6 +491,8 @@ bool make_hist_plan(int dtype, const ahq_layout& layout, const void* x, int num_
     hp->off_counts = o;
     const size_t nparts = hp->fast ? (size_t)hp->nblocks : 1;
     o = align_up(o + (size_t)S * nparts * 2 * (B + 2) * 4);
+    hp->off_folded = o;
+    o = align_up(o + (size_t)kFoldGroups * 2 * (B + 2) * 4);
     hp->total = o;
     return true;
 }
@@ -497,6 +566,8 @@ extern "C" int ahq_hist_update(int32_t dtype, const ahq_layout* layout, const vo
     ba.num_bins = B;
     ba.nhist = NH;
     ba.copies = hp.copies;
+    ba.copy_shift = 0;
+    while ((1 << ba.copy_shift) < hp.copies) ++ba.copy_shift;
     ba.ntiles = hp.ntiles;
     uint32_t* counts = reinterpret_cast<uint32_t*>(w + hp.off_counts);
     if (hp.fast) {
@@ -538,6 +609,14 @@ extern "C" int ahq_hist_update(int32_t dtype, const ahq_layout* layout, const vo
     fa.first = first_batch ? 1 : 0;
     fa.nparts = hp.fast ? hp.nblocks : 1;
     fa.counts = counts;
+    if (hp.fast && hp.nblocks > kFoldGroups) {
+        uint32_t* folded = reinterpret_cast<uint32_t*>(w + hp.off_folded);
+        const int len = NH * (B + 2);
+        hipLaunchKernelGGL(hist_fold_kernel, dim3((len + kBlock - 1) / kBlock, kFoldGroups), dim3(kBlock), 0, s, counts,
+                           folded, hp.nblocks, len, kFoldGroups);
+        fa.nparts = kFoldGroups;
+        fa.counts = folded;
+    }
     fa.carried = pa.carried;
     fa.upd_edges = pa.upd_edges;
     fa.hist = st->hist;

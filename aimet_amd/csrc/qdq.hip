@@ -189,25 +189,22 @@ __device__ __forceinline__ EncP load_enc(const QdqArgs& a, int64_t e) {
 }
 
 // -------------------------------------------------------------------------------------------------------- forward --
-template <typename IO, int VEC, typename M>
-__global__ __launch_bounds__(kBlock) void qdq_fwd_kernel(const QdqArgs a) {
-    __shared__ float sp[M::kNP][kStage];
-    const Tile t = make_tile(a);
-    stage_encodings<M>(a, t, sp);
-    __syncthreads();
-
-    const IO* __restrict__ x = static_cast<const IO*>(a.x);
-    IO* __restrict__ y = static_cast<IO*>(a.y);
+// FULL: every lane of the tile has work, so loads and stores carry no per-lane bounds checks (all tiles but the last).
+template <typename IO, int VEC, typename M, bool FULL>
+__device__ __forceinline__ void fwd_tile(const QdqArgs& a, const Tile& t, float (*sp)[kStage]) {
+    const IO* __restrict__ x = static_cast<const IO*>(a.x) + t.v0 * VEC;
+    IO* __restrict__ y = static_cast<IO*>(a.y) + t.v0 * VEC;
+    uint8_t* __restrict__ mask = a.mask ? a.mask + t.v0 * VEC : nullptr;
     Pack<IO, VEC> in[kUnroll];
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
         const int lv = u * kBlock + threadIdx.x;
-        if (lv < t.nv) in[u] = load_pack<IO, VEC>(x + (t.v0 + lv) * VEC);
+        if (FULL || lv < t.nv) in[u] = load_pack<IO, VEC>(x + (int64_t)lv * VEC);
     }
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
         const int lv = u * kBlock + threadIdx.x;
-        if (lv < t.nv) {
+        if (FULL || lv < t.nv) {
             const EncP e = staged<M>(sp, stage_index(a, t, lv));
             Pack<IO, VEC> out;
             Pack<uint8_t, VEC> mk;
@@ -218,14 +215,26 @@ __global__ __launch_bounds__(kBlock) void qdq_fwd_kernel(const QdqArgs a) {
                 out.v[k] = store_cast<IO>(r);
                 mk.v[k] = inr ? 1 : 0;
             }
-            store_pack<IO, VEC>(y + (t.v0 + lv) * VEC, out);
-            if (a.mask) store_pack<uint8_t, VEC>(a.mask + (t.v0 + lv) * VEC, mk);
+            store_pack<IO, VEC>(y + (int64_t)lv * VEC, out);
+            if (mask) store_pack<uint8_t, VEC>(mask + (int64_t)lv * VEC, mk);
         }
     }
+}
+
+template <typename IO, int VEC, typename M>
+__global__ __launch_bounds__(kBlock) void qdq_fwd_kernel(const QdqArgs a) {
+    __shared__ float sp[M::kNP][kStage];
+    const Tile t = make_tile(a, blockIdx.x);
+    stage_encodings<M>(a, t, sp);
+    __syncthreads();
+    if (t.nv == kTileVec) fwd_tile<IO, VEC, M, true>(a, t, sp);
+    else fwd_tile<IO, VEC, M, false>(a, t, sp);
     // elements past the last full vector (only possible with a single encoding)
     if (VEC > 1 && blockIdx.x == 0) {
         const int64_t i = a.nvec * VEC + threadIdx.x;
         if (i < a.numel) {
+            const IO* x = static_cast<const IO*>(a.x);
+            IO* y = static_cast<IO*>(a.y);
             const EncP e = staged<M>(sp, 0);
             bool inr;
             const float r = M::fwd(load_f32(x[i]), e, a.gc, inr);
@@ -249,43 +258,32 @@ __global__ __launch_bounds__(kBlock) void qdq_fwd_generic_kernel(const QdqArgs a
 }
 
 // ------------------------------------------------------------------------------------------------------- backward --
-template <int CD>
-__device__ __forceinline__ float finish_sum(double s) {
-    return rnd<CD>((float)s);
-}
 __device__ __forceinline__ float finish_sum_rt(double s, int cd) {
     if (cd == AHQ_BF16) return rnd<AHQ_BF16>((float)s);
     if (cd == AHQ_F16) return rnd<AHQ_F16>((float)s);
     return (float)s;
 }
 
-template <typename IO, int VEC, typename M, int RED>
-__global__ __launch_bounds__(kBlock) void qdq_bwd_kernel(const QdqArgs a) {
-    __shared__ float sp[M::kNP][kStage];
-    __shared__ double red_smem[kBlock / kWave];
-    const Tile t = make_tile(a);
-    stage_encodings<M>(a, t, sp);
-    __syncthreads();
-
-    const IO* __restrict__ x = static_cast<const IO*>(a.x);
-    const IO* __restrict__ g = static_cast<const IO*>(a.g);
-    IO* __restrict__ gxp = static_cast<IO*>(a.gx);
+template <typename IO, int VEC, typename M, int RED, bool FULL>
+__device__ __forceinline__ void bwd_tile(const QdqArgs& a, const Tile& t, float (*sp)[kStage], double& acc_s, double& acc_o) {
+    const IO* __restrict__ x = static_cast<const IO*>(a.x) + t.v0 * VEC;
+    const IO* __restrict__ g = static_cast<const IO*>(a.g) + t.v0 * VEC;
+    IO* __restrict__ gxp = a.gx ? static_cast<IO*>(a.gx) + t.v0 * VEC : nullptr;
     Pack<IO, VEC> xin[kUnroll], gin[kUnroll];
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
         const int lv = u * kBlock + threadIdx.x;
-        if (lv < t.nv) {
-            xin[u] = load_pack<IO, VEC>(x + (t.v0 + lv) * VEC);
-            gin[u] = load_pack<IO, VEC>(g + (t.v0 + lv) * VEC);
+        if (FULL || lv < t.nv) {
+            xin[u] = load_pack<IO, VEC>(x + (int64_t)lv * VEC);
+            gin[u] = load_pack<IO, VEC>(g + (int64_t)lv * VEC);
         }
     }
-    double acc_s = 0.0, acc_o = 0.0;  // kRedTile: per-thread totals
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
         const int lv = u * kBlock + threadIdx.x;
         float vs = 0.f, vo = 0.f;
         int si = 0;
-        if (lv < t.nv) {
+        if (FULL || lv < t.nv) {
             si = stage_index(a, t, lv);
             const EncP e = staged<M>(sp, si);
             Pack<IO, VEC> out;
@@ -297,7 +295,7 @@ __global__ __launch_bounds__(kBlock) void qdq_bwd_kernel(const QdqArgs a) {
                 vs += gs;
                 vo += go;
             }
-            if (gxp) store_pack<IO, VEC>(gxp + (t.v0 + lv) * VEC, out);
+            if (gxp) store_pack<IO, VEC>(gxp + (int64_t)lv * VEC, out);
         }
         if (RED == kRedTile) {
             acc_s += (double)vs;
@@ -310,13 +308,13 @@ __global__ __launch_bounds__(kBlock) void qdq_bwd_kernel(const QdqArgs a) {
                 ds += __shfl_xor(ds, m, kWave);
                 dofs += __shfl_xor(dofs, m, kWave);
             }
-            if (lv < t.nv && (threadIdx.x & (kv - 1)) == 0) {
+            if ((FULL || lv < t.nv) && (threadIdx.x & (kv - 1)) == 0) {
                 const int64_t e = t.e0 + si;
                 a.gscale[e] = finish_sum_rt(ds, a.out_cd);
                 a.goffset[e] = finish_sum_rt(dofs, a.out_cd);
             }
         } else if (RED == kRedAtomic) {
-            if (lv < t.nv) {
+            if (FULL || lv < t.nv) {
                 int64_t e = t.e0 + si;
                 if (e >= a.J) e %= a.J;
                 atomicAdd(&a.partials[2 * e], (double)vs);
@@ -324,9 +322,24 @@ __global__ __launch_bounds__(kBlock) void qdq_bwd_kernel(const QdqArgs a) {
             }
         }
     }
+}
+
+template <typename IO, int VEC, typename M, int RED>
+__global__ __launch_bounds__(kBlock) void qdq_bwd_kernel(const QdqArgs a) {
+    __shared__ float sp[M::kNP][kStage];
+    __shared__ double red_smem[kBlock / kWave];
+    const Tile t = make_tile(a, blockIdx.x);
+    stage_encodings<M>(a, t, sp);
+    __syncthreads();
+    double acc_s = 0.0, acc_o = 0.0;  // kRedTile: per-thread totals
+    if (t.nv == kTileVec) bwd_tile<IO, VEC, M, RED, true>(a, t, sp, acc_s, acc_o);
+    else bwd_tile<IO, VEC, M, RED, false>(a, t, sp, acc_s, acc_o);
     if (VEC > 1 && blockIdx.x == 0) {  // tail elements, single encoding only
         const int64_t i = a.nvec * VEC + threadIdx.x;
         if (i < a.numel) {
+            const IO* x = static_cast<const IO*>(a.x);
+            const IO* g = static_cast<const IO*>(a.g);
+            IO* gxp = static_cast<IO*>(a.gx);
             const EncP e = staged<M>(sp, 0);
             float gx, gs, go;
             M::bwd(load_f32(g[i]), load_f32(x[i]), e, a.gc, gx, gs, go);
@@ -361,27 +374,40 @@ __global__ __launch_bounds__(kBlock) void qdq_bwd_kernel(const QdqArgs a) {
 
 // Adds the per-tile partial sums of every encoding in a fixed order (second launch: a kernel boundary makes the
 // partials visible without any in-kernel fence, which on a multi-die GPU would flush the L2 once per workgroup).
-__global__ __launch_bounds__(kBlock) void qdq_bwd_finish_kernel(const QdqArgs a) {
-    __shared__ double red_smem[kBlock / kWave];
+constexpr int kFinishThreads = 1024;
+__global__ __launch_bounds__(kFinishThreads) void qdq_bwd_finish_kernel(const QdqArgs a) {
+    __shared__ double red_smem[2][kFinishThreads / kWave];
     const int64_t per_enc = a.mode == kRows ? a.I * (int64_t)a.tpr : (int64_t)a.nblocks;
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     if (a.mode != kRows) {
+        // single encoding: independent loads per thread, then one tree
         double s = 0.0, o = 0.0;
-        for (int64_t q = threadIdx.x; q < per_enc; q += kBlock) {
+#pragma unroll 4
+        for (int64_t q = threadIdx.x; q < per_enc; q += kFinishThreads) {
             s += a.partials[2 * q];
             o += a.partials[2 * q + 1];
         }
-        s = block_reduce(s, OpAddD(), red_smem);
-        o = block_reduce(o, OpAddD(), red_smem);
+        s = wave_reduce(s, OpAddD());
+        o = wave_reduce(o, OpAddD());
+        if (lane == 0) {
+            red_smem[0][wave] = s;
+            red_smem[1][wave] = o;
+        }
+        __syncthreads();
         if (threadIdx.x == 0) {
-            a.gscale[0] = finish_sum_rt(s, a.out_cd);
-            a.goffset[0] = finish_sum_rt(o, a.out_cd);
+            double ts = 0.0, to = 0.0;
+            for (int w = 0; w < kFinishThreads / kWave; ++w) {
+                ts += red_smem[0][w];
+                to += red_smem[1][w];
+            }
+            a.gscale[0] = finish_sum_rt(ts, a.out_cd);
+            a.goffset[0] = finish_sum_rt(to, a.out_cd);
         }
         return;
     }
     // one wave per encoding, lanes stride over that encoding's tiles
-    const int lane = threadIdx.x & (kWave - 1);
-    const int64_t wave0 = (int64_t)blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
-    for (int64_t j = wave0; j < a.J; j += (int64_t)gridDim.x * (kBlock / kWave)) {
+    const int64_t wave0 = (int64_t)blockIdx.x * (kFinishThreads / kWave) + wave;
+    for (int64_t j = wave0; j < a.J; j += (int64_t)gridDim.x * (kFinishThreads / kWave)) {
         double s = 0.0, o = 0.0;
         for (int64_t q = lane; q < per_enc; q += kWave) {
             const int64_t i = q / a.tpr, tt = q - i * a.tpr;
@@ -593,8 +619,9 @@ extern "C" int ahq_qdq_backward(const ahq_grid* grid, const ahq_layout* layout, 
     if (p.red == kRedTile) {
         const int64_t per_enc = p.mode == kRows ? p.cl.I * (int64_t)p.tpr : (int64_t)p.nblocks;
         if (per_enc > 1) {
-            const int64_t nb = p.mode == kRows ? (p.cl.J + 3) / 4 : 1;
-            hipLaunchKernelGGL(qdq_bwd_finish_kernel, dim3((unsigned)(nb > 4096 ? 4096 : nb)), dim3(kBlock), 0, st, a);
+            const int64_t waves = kFinishThreads / kWave;
+            const int64_t nb = p.mode == kRows ? (p.cl.J + waves - 1) / waves : 1;
+            hipLaunchKernelGGL(qdq_bwd_finish_kernel, dim3((unsigned)(nb > 4096 ? 4096 : nb)), dim3(kFinishThreads), 0, st, a);
         }
     }
     if (p.red == kRedAtomic) {

@@ -93,38 +93,34 @@ __device__ __forceinline__ float key_f32(unsigned int k) {
     return bits_to_f32(k ^ ((k >> 31) ? 0x80000000u : 0xffffffffu));
 }
 
-template <typename IO, int VEC, int RED>
-__global__ __launch_bounds__(kBlock) void minmax_kernel(const MmArgs a) {
-    __shared__ MinMax red_smem[kBlock / kWave];
-    const Tile t = make_tile(a);
-    const IO* __restrict__ x = static_cast<const IO*>(a.x);
-    const bool fo = a.finite_only != 0;
-
+// FULL: every lane of the tile has work (all tiles but the last).  FINITE: ignore non-finite values.
+template <typename IO, int VEC, int RED, bool FINITE, bool FULL>
+__device__ __forceinline__ void mm_tile(const MmArgs& a, const Tile& t, MinMax& acc) {
+    const IO* __restrict__ x = static_cast<const IO*>(a.x) + t.v0 * VEC;
     Pack<IO, VEC> in[kUnroll];
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
         const int lv = u * kBlock + threadIdx.x;
-        if (lv < t.nv) in[u] = load_pack<IO, VEC>(x + (t.v0 + lv) * VEC);
+        if (FULL || lv < t.nv) in[u] = load_pack<IO, VEC>(x + (int64_t)lv * VEC);
     }
-    MinMax acc = mm_identity();
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
         const int lv = u * kBlock + threadIdx.x;
         MinMax v = mm_identity();
         int si = 0;
-        if (lv < t.nv) {
+        if (FULL || lv < t.nv) {
             si = stage_index(a, t, lv);
 #pragma unroll
-            for (int k = 0; k < VEC; ++k) mm_add(v, load_f32(in[u].v[k]), fo);
+            for (int k = 0; k < VEC; ++k) mm_add(v, load_f32(in[u].v[k]), FINITE);
         }
         if (RED == kRedTile) {
             acc = mm_merge(acc, v);
         } else if (RED == kRedSeg) {
             const int kv = (int)a.Kv;
             for (int m = 1; m < kv; m <<= 1) v = mm_merge(v, mm_shfl_xor(v, m));
-            if (lv < t.nv && (threadIdx.x & (kv - 1)) == 0) mm_write<IO>(a, t.e0 + si, v);
+            if ((FULL || lv < t.nv) && (threadIdx.x & (kv - 1)) == 0) mm_write<IO>(a, t.e0 + si, v);
         } else if (RED == kRedAtomic) {
-            if (lv < t.nv) {
+            if (FULL || lv < t.nv) {
                 int64_t e = t.e0 + si;
                 if (e >= a.J) e %= a.J;
                 atomicMin(&a.key_min[e], f32_key(v.mn));
@@ -133,19 +129,15 @@ __global__ __launch_bounds__(kBlock) void minmax_kernel(const MmArgs a) {
             }
         }
     }
-    if (VEC > 1 && blockIdx.x == 0) {  // elements past the last full vector (single encoding only)
-        const int64_t i = a.nvec * VEC + threadIdx.x;
-        if (i < a.numel) {
-            MinMax v = mm_identity();
-            mm_add(v, load_f32(x[i]), fo);
-            if (RED == kRedTile) acc = mm_merge(acc, v);
-            if (RED == kRedAtomic) {
-                atomicMin(&a.key_min[0], f32_key(v.mn));
-                atomicMax(&a.key_max[0], f32_key(v.mx));
-                if (v.nan) atomicOr(&a.part_nan[0], 1);
-            }
-        }
-    }
+}
+
+template <typename IO, int VEC, int RED, bool FINITE>
+__global__ __launch_bounds__(kBlock) void minmax_kernel(const MmArgs a) {
+    __shared__ MinMax red_smem[kBlock / kWave];
+    const Tile t = make_tile(a, blockIdx.x);
+    MinMax acc = mm_identity();
+    if (t.nv == kTileVec) mm_tile<IO, VEC, RED, FINITE, true>(a, t, acc);
+    else mm_tile<IO, VEC, RED, FINITE, false>(a, t, acc);
     if (RED == kRedTile) {
         const MinMax b = mm_block_reduce(acc, red_smem);
         const int64_t per_enc = a.mode == kRows ? a.I * (int64_t)a.tpr : (int64_t)a.nblocks;
@@ -161,21 +153,76 @@ __global__ __launch_bounds__(kBlock) void minmax_kernel(const MmArgs a) {
     }
 }
 
-// Folds the per-tile partials of every encoding (second launch; see the note on fences in qdq.hip).
-template <typename IO>
-__global__ __launch_bounds__(kBlock) void minmax_finish_kernel(const MmArgs a) {
+// Single encoding (per-tensor statistics): a lean streaming kernel without any encoding lookup.  A workgroup reads
+// kFlatUnroll 16-byte vectors per lane, all issued before the first use, and leaves one partial.
+constexpr int kFlatUnroll = 4;
+constexpr int kFlatTileVec = kBlock * kFlatUnroll;
+
+template <typename IO, int VEC, bool FINITE>
+__global__ __launch_bounds__(kBlock) void minmax_flat_kernel(const MmArgs a) {
     __shared__ MinMax red_smem[kBlock / kWave];
-    const int64_t per_enc = a.mode == kRows ? a.I * (int64_t)a.tpr : (int64_t)a.nblocks;
+    const int64_t v0 = (int64_t)blockIdx.x * kFlatTileVec;
+    const int64_t left = a.nvec - v0;
+    const IO* __restrict__ x = static_cast<const IO*>(a.x) + v0 * VEC;
+    MinMax acc = mm_identity();
+    Pack<IO, VEC> in[kFlatUnroll];
+    if (left >= kFlatTileVec) {
+#pragma unroll
+        for (int u = 0; u < kFlatUnroll; ++u) in[u] = load_pack<IO, VEC>(x + (int64_t)(u * kBlock + threadIdx.x) * VEC);
+#pragma unroll
+        for (int u = 0; u < kFlatUnroll; ++u)
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) mm_add(acc, load_f32(in[u].v[k]), FINITE);
+    } else {
+        for (int u = 0; u < kFlatUnroll; ++u) {
+            const int lv = u * kBlock + threadIdx.x;
+            if (lv < left) {
+                const Pack<IO, VEC> p = load_pack<IO, VEC>(x + (int64_t)lv * VEC);
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) mm_add(acc, load_f32(p.v[k]), FINITE);
+            }
+        }
+    }
+    if (VEC > 1 && blockIdx.x == 0) {  // elements past the last full vector
+        const int64_t i = a.nvec * VEC + threadIdx.x;
+        if (i < a.numel) mm_add(acc, load_f32(static_cast<const IO*>(a.x)[i]), FINITE);
+    }
+    const MinMax b = mm_block_reduce(acc, red_smem);
+    if (threadIdx.x == 0) {
+        if (gridDim.x == 1) {
+            mm_write<IO>(a, 0, b);
+        } else {
+            a.part_min[blockIdx.x] = b.mn;
+            a.part_max[blockIdx.x] = b.mx;
+            a.part_nan[blockIdx.x] = b.nan;
+        }
+    }
+}
+
+// Folds the per-tile partials of every encoding (second launch; see the note on fences in qdq.hip).
+constexpr int kFinishThreads = 1024;
+template <typename IO>
+__global__ __launch_bounds__(kFinishThreads) void minmax_finish_kernel(const MmArgs a, int64_t nparts) {
+    __shared__ MinMax red_smem[kFinishThreads / kWave];
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     if (a.mode != kRows) {
         MinMax s = mm_identity();
-        for (int64_t q = threadIdx.x; q < per_enc; q += kBlock) s = mm_merge(s, MinMax{a.part_min[q], a.part_max[q], a.part_nan[q]});
-        s = mm_block_reduce(s, red_smem);
-        if (threadIdx.x == 0) mm_write<IO>(a, 0, s);
+#pragma unroll 4
+        for (int64_t q = threadIdx.x; q < nparts; q += kFinishThreads) s = mm_merge(s, MinMax{a.part_min[q], a.part_max[q], a.part_nan[q]});
+#pragma unroll
+        for (int m = kWave / 2; m >= 1; m >>= 1) s = mm_merge(s, mm_shfl_xor(s, m));
+        if (lane == 0) red_smem[wave] = s;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            MinMax r = red_smem[0];
+            for (int w = 1; w < kFinishThreads / kWave; ++w) r = mm_merge(r, red_smem[w]);
+            mm_write<IO>(a, 0, r);
+        }
         return;
     }
-    const int lane = threadIdx.x & (kWave - 1);
-    const int64_t wave0 = (int64_t)blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
-    for (int64_t j = wave0; j < a.J; j += (int64_t)gridDim.x * (kBlock / kWave)) {
+    const int64_t per_enc = a.I * (int64_t)a.tpr;
+    const int64_t wave0 = (int64_t)blockIdx.x * (kFinishThreads / kWave) + wave;
+    for (int64_t j = wave0; j < a.J; j += (int64_t)gridDim.x * (kFinishThreads / kWave)) {
         MinMax s = mm_identity();
         for (int64_t q = lane; q < per_enc; q += kWave) {
             const int64_t i = q / a.tpr, tt = q - i * a.tpr;
@@ -216,30 +263,40 @@ __global__ void minmax_keys_finish_kernel(const MmArgs a, int64_t n) {
         mm_write<IO>(a, i, MinMax{key_f32(a.key_min[i]), key_f32(a.key_max[i]), a.part_nan[i]});
 }
 
-template <typename IO, int RED>
+template <typename IO, int RED, bool FINITE>
 static void launch_mm_red(const Plan& p, const MmArgs& a, hipStream_t st) {
-    if (p.vec == 1) hipLaunchKernelGGL((minmax_kernel<IO, 1, RED>), dim3(p.nblocks), dim3(kBlock), 0, st, a);
-    else hipLaunchKernelGGL((minmax_kernel<IO, IoTraits<IO>::kVec, RED>), dim3(p.nblocks), dim3(kBlock), 0, st, a);
+    if (p.vec == 1) hipLaunchKernelGGL((minmax_kernel<IO, 1, RED, FINITE>), dim3(p.nblocks), dim3(kBlock), 0, st, a);
+    else hipLaunchKernelGGL((minmax_kernel<IO, IoTraits<IO>::kVec, RED, FINITE>), dim3(p.nblocks), dim3(kBlock), 0, st, a);
 }
 
-template <typename IO>
+static int64_t flat_blocks(const Plan& p) { return p.nvec > 0 ? (p.nvec + kFlatTileVec - 1) / kFlatTileVec : 1; }
+
+template <typename IO, bool FINITE>
 static void launch_mm(const Plan& p, const MmArgs& a, hipStream_t st) {
     const int64_t ne = p.cl.num_enc;
     const unsigned gb = (unsigned)((ne + 255) / 256 > 1024 ? 1024 : (ne + 255) / 256);
+    if (p.cl.kind == kIJK && p.cl.J == 1) {
+        const int64_t nb = flat_blocks(p);
+        if (p.vec == 1) hipLaunchKernelGGL((minmax_flat_kernel<IO, 1, FINITE>), dim3((unsigned)nb), dim3(kBlock), 0, st, a);
+        else hipLaunchKernelGGL((minmax_flat_kernel<IO, IoTraits<IO>::kVec, FINITE>), dim3((unsigned)nb), dim3(kBlock), 0, st, a);
+        if (nb > 1) hipLaunchKernelGGL((minmax_finish_kernel<IO>), dim3(1), dim3(kFinishThreads), 0, st, a, nb);
+        return;
+    }
     if (p.red == kRedAtomic) hipLaunchKernelGGL(minmax_keys_init_kernel, dim3(gb), dim3(256), 0, st, a.key_min, a.key_max, a.part_nan, ne);
     if (p.cl.kind == kGeneric) {
         hipLaunchKernelGGL((minmax_generic_kernel<IO>), dim3(p.nblocks), dim3(kBlock), 0, st, a);
     } else if (p.red == kRedTile) {
-        launch_mm_red<IO, kRedTile>(p, a, st);
-        const int64_t per_enc = p.mode == kRows ? p.cl.I * (int64_t)p.tpr : (int64_t)p.nblocks;
+        launch_mm_red<IO, kRedTile, FINITE>(p, a, st);
+        const int64_t per_enc = p.cl.I * (int64_t)p.tpr;
         if (per_enc > 1) {
-            const int64_t nb = p.mode == kRows ? (p.cl.J + 3) / 4 : 1;
-            hipLaunchKernelGGL((minmax_finish_kernel<IO>), dim3((unsigned)(nb > 4096 ? 4096 : nb)), dim3(kBlock), 0, st, a);
+            const int64_t waves = kFinishThreads / kWave;
+            const int64_t nb = (p.cl.J + waves - 1) / waves;
+            hipLaunchKernelGGL((minmax_finish_kernel<IO>), dim3((unsigned)(nb > 4096 ? 4096 : nb)), dim3(kFinishThreads), 0, st, a, per_enc);
         }
     } else if (p.red == kRedSeg) {
-        launch_mm_red<IO, kRedSeg>(p, a, st);
+        launch_mm_red<IO, kRedSeg, FINITE>(p, a, st);
     } else {
-        launch_mm_red<IO, kRedAtomic>(p, a, st);
+        launch_mm_red<IO, kRedAtomic, FINITE>(p, a, st);
     }
     if (p.red == kRedAtomic) hipLaunchKernelGGL((minmax_keys_finish_kernel<IO>), dim3(gb), dim3(256), 0, st, a, ne);
 }
@@ -293,10 +350,12 @@ extern "C" int ahq_minmax(int32_t dtype, const ahq_layout* layout, const void* x
         a.key_max = reinterpret_cast<unsigned int*>(w + p.ws_elems * 4);
     }
     hipStream_t st = static_cast<hipStream_t>(stream);
+#define AHQ_MM(IO) do { if (finite_only) launch_mm<IO, true>(p, a, st); else launch_mm<IO, false>(p, a, st); } while (0)
     switch (dtype) {
-        case AHQ_F32: launch_mm<float>(p, a, st); break;
-        case AHQ_F16: launch_mm<f16_t>(p, a, st); break;
-        default: launch_mm<bf16_t>(p, a, st); break;
+        case AHQ_F32: AHQ_MM(float); break;
+        case AHQ_F16: AHQ_MM(f16_t); break;
+        default: AHQ_MM(bf16_t); break;
     }
+#undef AHQ_MM
     return check_launch("ahq_minmax");
 }

@@ -25,6 +25,7 @@ struct Geom {
     int32_t mode;
     int32_t tpr;   // tiles per row (kRows)
     uint32_t nblocks;
+    int64_t ntiles;  // tiles in total (== nblocks: one tile per workgroup)
     // generic layout (per-element coordinate walk)
     int32_t nseg;
     int64_t seg_extent[2 * AHQ_MAX_DIMS];
@@ -40,11 +41,11 @@ struct Tile {
     int nstage;    // runs touched
 };
 
-__device__ __forceinline__ Tile make_tile(const Geom& a) {
+__device__ __forceinline__ Tile make_tile(const Geom& a, int64_t tile) {
     Tile t;
     if (a.mode == kRows) {
-        const int64_t row = blockIdx.x / (uint32_t)a.tpr;
-        const int64_t tt = blockIdx.x - row * a.tpr;
+        const int64_t row = tile / a.tpr;
+        const int64_t tt = tile - row * a.tpr;
         t.v0 = row * a.Kv + tt * kTileVec;
         const int64_t left = a.Kv - tt * kTileVec;
         t.nv = (int)(left < kTileVec ? left : kTileVec);
@@ -52,7 +53,7 @@ __device__ __forceinline__ Tile make_tile(const Geom& a) {
         t.e0 = a.I == 1 ? row : row % a.J;
         t.nstage = 1;
     } else {
-        t.v0 = (int64_t)blockIdx.x * kTileVec;
+        t.v0 = tile * kTileVec;
         const int64_t left = a.nvec - t.v0;
         t.nv = (int)(left < kTileVec ? left : kTileVec);
         if (t.nv < 0) t.nv = 0;
@@ -96,6 +97,7 @@ struct Plan {
     int red;
     uint32_t nblocks;
     int64_t Kv, nvec;
+    int64_t ntiles;
     size_t ws_elems;  // kRedTile: number of tiles; kRedAtomic: number of encodings; else 0
 };
 
@@ -123,6 +125,7 @@ inline bool make_plan(int io_dtype, const ahq_layout& layout, bool ptr_aligned, 
         int64_t nb = (c.numel + kBlock - 1) / kBlock;
         if (nb > 65536) nb = 65536;
         p->nblocks = (uint32_t)(nb < 1 ? 1 : nb);
+        p->ntiles = p->nblocks;
         if (want_red) {
             p->red = kRedAtomic;
             p->ws_elems = (size_t)c.num_enc;
@@ -156,6 +159,7 @@ inline bool make_plan(int io_dtype, const ahq_layout& layout, bool ptr_aligned, 
         set_error("tensor too large for one launch");
         return false;
     }
+    p->ntiles = nb;
     p->nblocks = (uint32_t)nb;
     return true;
 }
@@ -171,6 +175,7 @@ inline void fill_geom(const Plan& p, Geom* g) {
     g->mode = p.mode;
     g->tpr = p.tpr;
     g->nblocks = p.nblocks;
+    g->ntiles = p.ntiles;
     g->nseg = c.kind == kGeneric ? c.nseg : 0;
     for (int i = 0; i < g->nseg; ++i) {
         g->seg_extent[i] = c.seg_extent[i];

@@ -144,6 +144,21 @@ def run_qdq_workload(key, steps, warmup, dev, with_cpu_baseline=True):
     t_fwd = event_time(fwd, reps)
     t_bwd = event_time(bwd, reps)
 
+    # min/max calibration of the same tensor (one fused pass for both extrema)
+    mm_ws_bytes = lib.ahq_minmax_workspace_bytes(layout)
+    mm_ws = torch.empty(max(mm_ws_bytes, 16), dtype=torch.uint8, device=dev)
+    mn_out = torch.empty(scale.shape, dtype=x.dtype, device=dev)
+    mx_out = torch.empty(scale.shape, dtype=x.dtype, device=dev)
+    code = _lib.DTYPE_CODE[x.dtype]
+
+    def minmax():
+        _lib.check(lib.ahq_minmax(code, layout, x.data_ptr(), mn_out.data_ptr(), mx_out.data_ptr(), None, None, 0,
+                                  mm_ws.data_ptr(), mm_ws_bytes, stream), "minmax")
+
+    t_mm = event_time(minmax, reps)
+    mn_ref, mx_ref = O.reduce_minmax(w["x"], w["enc_shape"], w["block"])
+    exact_mm = bool(torch.equal(mn_out.cpu(), mn_ref) and torch.equal(mx_out.cpu(), mx_ref))
+
     n = x.numel()
     S = x.element_size()
     enc_bytes = 8 * scale.numel()
@@ -182,7 +197,12 @@ def run_qdq_workload(key, steps, warmup, dev, with_cpu_baseline=True):
             "qdq_fwd_kernel": {"us": round(t_fwd * 1e6, 2), "GBps": round(bytes_fwd / t_fwd / 1e9, 1)},
             "qdq_bwd_kernel": {"us": round(t_bwd * 1e6, 2), "GBps": round(bytes_bwd / t_bwd / 1e9, 1)},
         },
-        "parity": {"y_bit_exact": exact_y, "gx_bit_exact": exact_gx, "gscale_max_rel_err": gs_err},
+        "calibration": {"kernel": "minmax_kernel", "us": round(t_mm * 1e6, 2),
+                        "GBps": round((S * n + 2 * S * scale.numel()) / t_mm / 1e9, 1),
+                        "elements_per_s": round(n / t_mm, 1),
+                        "frac_of_hbm_peak": round((S * n) / t_mm / 1e9 / HBM_PEAK_GBS, 4)},
+        "parity": {"y_bit_exact": exact_y, "gx_bit_exact": exact_gx, "gscale_max_rel_err": gs_err,
+                   "minmax_bit_exact": exact_mm},
         "roofline": {"bound": "hbm", "kernel": dom[0], "achieved": round(dom[2] / dom[1] / 1e9, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(dom[2] / dom[1] / 1e9 / HBM_PEAK_GBS, 4),
                      "traffic": None},
@@ -214,12 +234,115 @@ def cpu_baseline_qdq(w, scale, offset, qmin, qmax, bytes_step, budget_s=12.0):
                                       f"({dt * 1e3:.1f} ms/step)"}
 
 
+def _laplace_batch(shape, seed, dev):
+    """Laplace(0, 1) with 0.1 % of the elements replaced by +-U(20, 60), generated on the device."""
+    g = torch.Generator(device=dev).manual_seed(seed)
+    u = torch.rand(shape, generator=g, device=dev) - 0.5
+    x = -torch.sign(u) * torch.log1p(-2 * u.abs())
+    n = x.numel()
+    k = n // 1000
+    idx = torch.randint(0, n, (k,), generator=g, device=dev)
+    out = (torch.rand(k, generator=g, device=dev) * 40 + 20) * torch.sign(torch.rand(k, generator=g, device=dev) - 0.5)
+    x.view(-1)[idx] = out
+    return x
+
+
+def run_hist_workload(steps, warmup, dev, with_cpu_baseline=True, batches=16, shape=(8, 2048, 4096)):
+    """c3: 16 batches folded into a 512-bin histogram, then the 100 x 64 candidate SQNR search (8-bit asymmetric)."""
+    from aimet_amd.quantization.encoding_analyzer import SqnrEncodingAnalyzer
+    from oracle import torch_ref as O
+
+    _ensure_built()
+    xs = [_laplace_batch(shape, b, dev) for b in range(batches)]
+    an = SqnrEncodingAnalyzer((1,), num_bins=512, asymmetric_delta_candidates=100, offset_candidates=64, gamma=3.0)
+
+    def step():
+        an.reset_stats()
+        for x in xs:
+            an.update_stats(x)
+        return an.compute_encodings(255, False)
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        lo, hi = step()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) / steps
+
+    def event_time(fn, reps):
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        fn()
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / reps * 1e-3
+
+    # one histogram update of a later batch (range pass + binning pass against two ranges) and the search alone
+    t_upd = event_time(lambda: an.update_stats(xs[1]), 20)
+    t_search = event_time(lambda: an.compute_encodings(255, False), 20)
+    n_b = xs[0].numel()
+    n = n_b * batches
+    bytes_step = 8 * n
+    bytes_upd = 8 * n_b
+
+    # parity on a bounded sample: the first two batches through the CPU oracle
+    ref = O.HistObserver((1,), 512)
+    t_cpu0 = time.perf_counter()
+    cpu_batches = [xs[0].cpu(), xs[1].cpu()]
+    t_cpu1 = time.perf_counter()
+    for xb in cpu_batches:
+        ref.update(xb)
+    lo_r, hi_r, _, _, bi = O.sqnr_encodings(ref.stats, (1,), 255, False, asym_deltas=100, num_offsets=64, gamma=3.0)
+    cpu_dt = time.perf_counter() - t_cpu1
+    an.reset_stats()
+    for xb in xs[:2]:
+        an.update_stats(xb)
+    lo2, hi2 = an.compute_encodings(255, False)
+    st = an.observer.get_stats()[0]
+    parity = {
+        "hist_bit_exact": bool(torch.equal(st.histogram.cpu(), ref.stats[0].histogram)),
+        "edges_bit_exact": bool(torch.equal(st.bin_edges.cpu(), ref.stats[0].bin_edges)),
+        "argmin_identical": bool(int(an.last_search["best_index"].item()) == int(bi.item())),
+        "encoding_bit_exact": bool(torch.equal(lo2.cpu(), lo_r) and torch.equal(hi2.cpu(), hi_r)),
+        "sample": "first 2 of 16 batches",
+    }
+    out = {
+        "metric": "QDQ fwd+bwd GB/s (% of HBM peak); calibration elems/s; vs host-CPU ref",
+        "value": round(bytes_step / wall / 1e9, 2),
+        "unit": "GB/s",
+        "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": round(wall * 1e3, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "c3_hist512_sqnr100x64_fp32_16x8x2048x4096", "elements": n,
+                   "algorithmic_bytes_per_step": bytes_step, "batches": batches},
+        "pct_of_hbm_peak": round(100.0 * bytes_step / wall / 1e9 / HBM_PEAK_GBS, 2),
+        "elements_per_s": round(n / wall, 1),
+        "kernels": {"hist_update(batch>=2)": {"us": round(t_upd * 1e6, 2), "GBps": round(bytes_upd / t_upd / 1e9, 1)},
+                    "sqnr_search": {"us": round(t_search * 1e6, 2), "candidates": 6400, "bins": 512}},
+        "encoding": {"min": float(lo.item()), "max": float(hi.item())},
+        "parity": parity,
+        "roofline": {"bound": "hbm", "kernel": "hist_update (minmax_kernel + hist_bin_kernel)",
+                     "achieved": round(bytes_upd / t_upd / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(bytes_upd / t_upd / 1e9 / HBM_PEAK_GBS, 4), "traffic": None},
+    }
+    if with_cpu_baseline:
+        out["cpu_baseline"] = {"value": round(2 * n_b / cpu_dt, 1), "unit": "elements/s", "cores": torch.get_num_threads(),
+                               "kind": "port", "sample": f"2 of 16 batches folded + SQNR search with torch CPU ops "
+                                                         f"({cpu_dt:.2f} s)"}
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["c3"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -230,7 +353,10 @@ def main():
         print("bench.py: no HIP device visible", file=sys.stderr)
         sys.exit(1)
     dev = torch.device("cuda:0")
-    out = run_qdq_workload(args.workload, args.steps, args.warmup, dev, with_cpu_baseline=not args.no_cpu_baseline)
+    if args.workload == "c3":
+        out = run_hist_workload(min(args.steps, 10), min(args.warmup, 2), dev, with_cpu_baseline=not args.no_cpu_baseline)
+    else:
+        out = run_qdq_workload(args.workload, args.steps, args.warmup, dev, with_cpu_baseline=not args.no_cpu_baseline)
     print(json.dumps(out))
 
 
