@@ -26,6 +26,15 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+COPY_REF_ELEMS = 1 << 26
+# HBM bytes per launch of each workload's dominant kernel(s): rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE averages per
+# dispatch, scaled by what the same counters read for _copy_reference() (x2.000 for FETCH_SIZE, x1.000 for WRITE_SIZE);
+# the counter summary is profiles/hbm_traffic_pmc__c2_qdq__c3_hist.txt.  None where no counter run has been made.
+MEASURED_TRAFFIC_BYTES = {
+    ("c2", "qdq_bwd_kernel"): int((131490.1 + 65795.8) * 1024),
+    ("c2", "qdq_fwd_kernel"): int((65942.9 + 65536.0) * 1024),
+    ("c3", "hist_update"): int((262160.2 + 1542.6 + 262299.5 + 4128.0 + 4564.8 + 127.2 + 284.9 + 199.2) * 1024),
+}
 
 
 def _ensure_built():
@@ -84,12 +93,22 @@ def _encodings_cpu(w):
     return scale, offset, qmin, qmax
 
 
+def _copy_reference(dev):
+    """One plain elementwise pass of known size (256 MiB read, 256 MiB written), outside every timed region: hardware
+    counter runs of this script scale FETCH_SIZE / WRITE_SIZE of the kernels below by what they read for this one."""
+    src = torch.ones(COPY_REF_ELEMS, dtype=torch.float32, device=dev)
+    dst = torch.empty_like(src)
+    torch.mul(src, 1.0, out=dst)
+    torch.cuda.synchronize()
+
+
 def run_qdq_workload(key, steps, warmup, dev, with_cpu_baseline=True):
     from aimet_amd import _lib
     from aimet_amd.quantization.affine.backends import hip
     from oracle import torch_ref as O
 
     lib = _ensure_built()
+    _copy_reference(dev)
     w = WORKLOADS[key](dev)
     scale_c, offset_c, qmin, qmax = _encodings_cpu(w)
     x = w["x"].to(dev)
@@ -205,7 +224,7 @@ def run_qdq_workload(key, steps, warmup, dev, with_cpu_baseline=True):
                    "minmax_bit_exact": exact_mm},
         "roofline": {"bound": "hbm", "kernel": dom[0], "achieved": round(dom[2] / dom[1] / 1e9, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(dom[2] / dom[1] / 1e9 / HBM_PEAK_GBS, 4),
-                     "traffic": None},
+                     "algorithmic_bytes": dom[2], "traffic": MEASURED_TRAFFIC_BYTES.get((key, dom[0]))},
     }
     if with_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline_qdq(w, scale_c, offset_c, qmin, qmax, bytes_step)
@@ -253,6 +272,7 @@ def run_hist_workload(steps, warmup, dev, with_cpu_baseline=True, batches=16, sh
     from oracle import torch_ref as O
 
     _ensure_built()
+    _copy_reference(dev)
     xs = [_laplace_batch(shape, b, dev) for b in range(batches)]
     an = SqnrEncodingAnalyzer((1,), num_bins=512, asymmetric_delta_candidates=100, offset_candidates=64, gamma=3.0)
 
@@ -328,7 +348,8 @@ def run_hist_workload(steps, warmup, dev, with_cpu_baseline=True, batches=16, sh
         "parity": parity,
         "roofline": {"bound": "hbm", "kernel": "hist_update (minmax_kernel + hist_bin_kernel)",
                      "achieved": round(bytes_upd / t_upd / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(bytes_upd / t_upd / 1e9 / HBM_PEAK_GBS, 4), "traffic": None},
+                     "frac": round(bytes_upd / t_upd / 1e9 / HBM_PEAK_GBS, 4), "algorithmic_bytes": bytes_upd,
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(("c3", "hist_update"))},
     }
     if with_cpu_baseline:
         out["cpu_baseline"] = {"value": round(2 * n_b / cpu_dt, 1), "unit": "elements/s", "cores": torch.get_num_threads(),
