@@ -76,6 +76,20 @@ class SqnrParams(ctypes.Structure):
     ]
 
 
+class DlqPdfState(ctypes.Structure):
+    """ahq_dlq_pdf_state"""
+
+    _fields_ = [
+        ("num_slots", ctypes.c_int32),
+        ("xleft", ctypes.c_void_p),
+        ("pdf", ctypes.c_void_p),
+        ("meta", ctypes.c_void_p),
+    ]
+
+
+DLQ_PDF_SIZE = 1536
+
+
 class HipLibraryError(RuntimeError):
     """Raised when libaimet_amd.so is missing or one of its entry points reports an error."""
 
@@ -98,6 +112,14 @@ _SIGNATURES = {
     "ahq_hist_update": (ctypes.c_int, [ctypes.c_int32, ctypes.POINTER(Layout), _P, ctypes.POINTER(HistState),
                                        ctypes.c_int, _P, ctypes.c_size_t, _P]),
     "ahq_sqnr_search": (ctypes.c_int, [ctypes.POINTER(SqnrParams), _P, _P, _P, _P, _P, _P, _P, _P, _P, _P]),
+    "ahq_dlq_minmax_encodings": (ctypes.c_int, [_P, _P, ctypes.c_int64, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32,
+                                                ctypes.c_int32, ctypes.c_double, _P, _P]),
+    "ahq_dlq_pdf_update_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int32, ctypes.POINTER(Layout)]),
+    "ahq_dlq_pdf_update": (ctypes.c_int, [ctypes.c_int32, ctypes.POINTER(Layout), _P, ctypes.POINTER(DlqPdfState),
+                                          ctypes.c_int32, _P, _P, ctypes.c_size_t, _P]),
+    "ahq_dlq_tfe_encodings_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int32]),
+    "ahq_dlq_tfe_encodings": (ctypes.c_int, [ctypes.POINTER(DlqPdfState), ctypes.c_int32, ctypes.c_int32, ctypes.c_int32,
+                                             ctypes.c_int32, _P, _P, _P, ctypes.c_size_t, _P]),
 }
 
 

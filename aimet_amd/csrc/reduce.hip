@@ -71,8 +71,15 @@ __device__ __forceinline__ void mm_write(const MmArgs& a, int64_t e, MinMax m) {
     IO* omn = static_cast<IO*>(a.out_min);
     IO* omx = static_cast<IO*>(a.out_max);
     const float qnan = __builtin_nanf("");
-    const float mn = m.nan ? qnan : m.mn;
-    const float mx = m.nan ? qnan : m.mx;
+    float mn = m.nan ? qnan : m.mn;
+    float mx = m.nan ? qnan : m.mx;
+    if (a.finite_only == 2) {
+        // std::min / std::max folds that start from the largest / lowest finite float: NaN never wins a comparison
+        // and the minimum cannot exceed FLT_MAX (DlQuantization GetMin_cpu / GetMax_cpu)
+        const float big = 3.402823466e+38f;
+        mn = fminf(m.mn, big);
+        mx = fmaxf(m.mx, -big);
+    }
     omn[e] = store_cast<IO>(mn);
     omx[e] = store_cast<IO>(mx);
     if (a.run_min) {
@@ -80,8 +87,13 @@ __device__ __forceinline__ void mm_write(const MmArgs& a, int64_t e, MinMax m) {
         IO* rmn = static_cast<IO*>(a.run_min);
         IO* rmx = static_cast<IO*>(a.run_max);
         const float pmn = load_f32(rmn[e]), pmx = load_f32(rmx[e]);
-        rmn[e] = store_cast<IO>((pmn != pmn || mn != mn) ? qnan : fminf(pmn, mn));
-        rmx[e] = store_cast<IO>((pmx != pmx || mx != mx) ? qnan : fmaxf(pmx, mx));
+        if (a.finite_only == 2) {
+            rmn[e] = store_cast<IO>(mn < pmn ? mn : pmn);
+            rmx[e] = store_cast<IO>(pmx < mx ? mx : pmx);
+        } else {
+            rmn[e] = store_cast<IO>((pmn != pmn || mn != mn) ? qnan : fminf(pmn, mn));
+            rmx[e] = store_cast<IO>((pmx != pmx || mx != mx) ? qnan : fmaxf(pmx, mx));
+        }
     }
 }
 
@@ -238,7 +250,7 @@ __global__ __launch_bounds__(kFinishThreads) void minmax_finish_kernel(const MmA
 template <typename IO>
 __global__ __launch_bounds__(kBlock) void minmax_generic_kernel(const MmArgs a) {
     const IO* __restrict__ x = static_cast<const IO*>(a.x);
-    const bool fo = a.finite_only != 0;
+    const bool fo = a.finite_only == 1;
     for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < a.numel; i += (int64_t)gridDim.x * kBlock) {
         const int64_t e = generic_enc_index(a, i);
         MinMax v = mm_identity();
@@ -350,7 +362,7 @@ extern "C" int ahq_minmax(int32_t dtype, const ahq_layout* layout, const void* x
         a.key_max = reinterpret_cast<unsigned int*>(w + p.ws_elems * 4);
     }
     hipStream_t st = static_cast<hipStream_t>(stream);
-#define AHQ_MM(IO) do { if (finite_only) launch_mm<IO, true>(p, a, st); else launch_mm<IO, false>(p, a, st); } while (0)
+#define AHQ_MM(IO) do { if (finite_only == 1) launch_mm<IO, true>(p, a, st); else launch_mm<IO, false>(p, a, st); } while (0)
     switch (dtype) {
         case AHQ_F32: AHQ_MM(float); break;
         case AHQ_F16: AHQ_MM(f16_t); break;

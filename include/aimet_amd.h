@@ -113,8 +113,11 @@ int    ahq_qdq_backward(const ahq_grid* grid, const ahq_layout* layout, const vo
  * Replaces: _MinMaxObserver.collect_stats = utils.reduce(amin/amax) (AT/quantization/encoding_analyzer.py:80-94,
  * AT/utils.py:1115-1148), _HistogramObserver._get_min_max (encoding_analyzer.py:213-219, finite_only=1) and
  * DlQuantization GetMinMax (DLQ/src/math_functions.cpp:72-117).
- * out_min/out_max: one value per encoding in the tensor's own dtype.  NaN propagates like torch.amin/amax unless
- * finite_only, where non-finite values are ignored (an all-non-finite slice yields +inf / -inf).
+ * out_min/out_max: one value per encoding in the tensor's own dtype.  finite_only selects the NaN / infinity rule:
+ *   0  NaN propagates like torch.amin/amax
+ *   1  non-finite values are ignored (an all-non-finite slice yields +inf / -inf)
+ *   2  DlQuantization's std::min / std::max folds: NaN is skipped, the minimum starts from FLT_MAX and the maximum
+ *      from -FLT_MAX (math_functions.cpp:324-345); run_min/run_max are folded the same way
  * run_min/run_max (optional, both or neither): running statistics of the same shape and dtype that the batch result is
  * folded into with torch.minimum / torch.maximum semantics (_MinMaxObserver.merge_stats, encoding_analyzer.py:96-112).
  */
@@ -169,6 +172,53 @@ typedef struct {
 int ahq_sqnr_search(const ahq_sqnr_params* params, const float* hist, const float* edges, const float* minmax,
                     const float* offset_grid, float* noise, float* deltas, float* offsets, float* out,
                     long long* best_index, void* stream);
+
+/* ---------------------------------------------------------------- DlQuantization calibration ----------------------
+ * Encodings are rows of five doubles: min, max, delta, offset, bw (DLQ TfEncoding, QuantizationType.hpp).
+ *
+ * ahq_dlq_minmax_encodings replaces MinMaxEncodingAnalyzer::computeEncoding -> getComputedEncodings
+ * (DLQ/src/MinMaxEncodingAnalyzer.cpp:97-119, DLQ/src/quantization_utils.cpp:23-99): stat_min/stat_max are the running
+ * per-block float statistics (ahq_minmax with finite_only = 2); out is [num_encodings][5].  A non-zero
+ * zero_point_shift with a mode the reference rejects returns AHQ_ERR_UNSUPPORTED with the reference's message.
+ */
+int ahq_dlq_minmax_encodings(const float* stat_min, const float* stat_max, int64_t num_encodings, int32_t bw,
+                             int32_t symmetric, int32_t strict, int32_t unsigned_sym, double zero_point_shift,
+                             double* out, void* stream);
+
+/* TF-enhanced statistics: one 1536-bucket PDF per encoding block (DLQ/src/math_functions.hpp:28-49).
+ * xleft/pdf: [num_slots][AHQ_DLQ_PDF_SIZE] doubles; meta: [num_slots][4] int32 = iterations, initialized (xLeft not
+ * empty), stats_updated, reserved.  All zero = a freshly constructed analyzer; resetStats zeroes everything but
+ * stats_updated (DLQ/src/TfEnhancedEncodingAnalyzer.cpp:44-50).
+ */
+#define AHQ_DLQ_PDF_SIZE 1536
+typedef struct {
+    int32_t  num_slots;
+    double*  xleft;
+    double*  pdf;
+    int32_t* meta;
+} ahq_dlq_pdf_state;
+
+/* Replaces TfEnhancedEncodingAnalyzer::updateStats -> UpdatePdf / InitializePdf / GetHistogram
+ * (DLQ/src/TfEnhancedEncodingAnalyzer.cpp:26-42, DLQ/src/math_functions.cpp:190-285, 364-381) for every block of the
+ * layout (EncodingAnalyzerWrapper::updateStats, DLQ/src/EncodingAnalyzerWrapper.cpp:27-46).
+ * with_init: non-zero adds the pass that finds the batch's range, needed while any slot is still uninitialised (a
+ * slot stays uninitialised while it has only seen all-zero batches); callers pass 1 until meta says every slot is
+ * initialised, 0 afterwards (one read of the tensor instead of two).  With 0, an uninitialised slot ignores the batch.
+ * hist_out (optional): [num_slots][AHQ_DLQ_PDF_SIZE] counts of this batch alone.
+ */
+size_t ahq_dlq_pdf_update_workspace_bytes(int32_t dtype, const ahq_layout* layout);
+int    ahq_dlq_pdf_update(int32_t dtype, const ahq_layout* layout, const void* x, const ahq_dlq_pdf_state* state,
+                          int32_t with_init, uint32_t* hist_out, void* workspace, size_t workspace_bytes, void* stream);
+
+/* Replaces TfEnhancedEncodingAnalyzer::computeEncoding (DLQ/src/TfEnhancedEncodingAnalyzer.cpp:52-377): range of the
+ * aggregate statistics, the 17 x 21 + 1 asymmetric or 101 symmetric (delta, offset) candidates, the quantization +
+ * 3 x saturation cost of each over the PDF, first minimum.  out: [num_slots][5]; best_index (optional):
+ * [num_slots][2] = position of the chosen candidate in the reference's candidate list, length of that list.
+ */
+size_t ahq_dlq_tfe_encodings_workspace_bytes(int32_t num_slots);
+int    ahq_dlq_tfe_encodings(const ahq_dlq_pdf_state* state, int32_t bw, int32_t symmetric, int32_t strict,
+                             int32_t unsigned_sym, double* out, int32_t* best_index, void* workspace,
+                             size_t workspace_bytes, void* stream);
 
 #ifdef __cplusplus
 }

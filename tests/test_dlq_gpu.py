@@ -1,0 +1,282 @@
+"""DlQuantization rows on the GPU: the HIP path against the reference's own expected outputs (shared checks) and,
+bit for bit, against the plain-C oracle on seeded inputs.  Everything goes through the C ABI (aimet_amd.dlq)."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import dlq as OD
+from tests import dlq_checks as C
+from tests.dlq_adapters import QUANTIZATION_TF, QUANTIZATION_TF_ENHANCED, HipQuantizer, OracleQuantizer
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture()
+def make(device):
+    return lambda shape, bw, scheme: HipQuantizer(shape, bw, scheme, device)
+
+
+# ------------------------------------------------------------------------------ the reference's expected outputs --
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_broadcast_qdq_vectors(make, dtype):
+    C.check_broadcast_qdq(make, dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+def test_per_tensor_qdq(make, dtype):
+    C.check_per_tensor_qdq(make, dtype)
+
+
+def test_minmax_quantizer_vectors(make):
+    C.check_minmax_quantizer(make)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_block_minmax_vectors(make, dtype):
+    C.check_block_minmax(make, dtype)
+
+
+def test_tfe_all_zero_vector(make):
+    C.check_tfe_all_zero(make)
+
+
+def test_tfe_reference_bounds(make):
+    C.check_tfe_properties(make)
+
+
+# ------------------------------------------------------------------------------------- bit-exact against the oracle --
+def _data(shape, seed, dtype=torch.float32, special=True):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(shape, generator=g) * 3 + 0.25
+    if special and x.numel() >= 16:
+        f = x.view(-1)
+        f[1] = float("nan")
+        f[5] = float("inf")
+        f[7] = float("-inf")
+        f[11] = 1e30
+        f[13] = 0.0
+    return x.to(dtype)
+
+
+QDQ_CASES = [
+    ((1000,), ()),
+    ((4099,), ()),
+    ((64, 256), (64, 1)),
+    ((64, 256), (1, 256)),
+    ((48, 512), (48, 8)),
+    ((2, 6, 10, 12), (2, 3, 1, 4)),
+    ((4, 2, 3), (2, 3)),
+    ((3, 5, 7), (5, 1)),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("shape,enc_shape", QDQ_CASES)
+def test_qdq_bit_exact(device, dtype, shape, enc_shape):
+    x = _data(shape, 3, dtype)
+    E = int(np.prod(enc_shape)) if enc_shape else 1
+    g = torch.Generator().manual_seed(4)
+    encs = []
+    for e in range(E):
+        lo = -float(torch.rand((), generator=g)) * 8 - 0.1
+        hi = float(torch.rand((), generator=g)) * 8 + 0.1
+        bw = [4, 8, 16][e % 3]
+        encs.append(tuple(OD.computed_encodings(bw, lo, hi, e % 2 == 1)))
+    a = OracleQuantizer(enc_shape, 8, QUANTIZATION_TF)
+    b = HipQuantizer(enc_shape, 8, QUANTIZATION_TF, device)
+    a.setEncodings(encs)
+    b.setEncodings(encs)
+    ya, yb = a.quantizeDequantize(x), b.quantizeDequantize(x)
+    assert ya.dtype == yb.dtype == dtype and ya.shape == yb.shape
+    assert torch.equal(ya.view(torch.int16 if dtype != torch.float32 else torch.int32),
+                       yb.view(torch.int16 if dtype != torch.float32 else torch.int32))
+
+
+def test_qdq_requires_encodings_and_matching_length(device):
+    q = HipQuantizer((4,), 8, QUANTIZATION_TF, device)
+    with pytest.raises(RuntimeError, match="before computing encodings"):
+        q.quantizeDequantize(torch.zeros(8, 4))
+    with pytest.raises(RuntimeError, match="did not match"):
+        q.setEncodings([(0.0, 1.0, 1 / 255, 0.0, 8)])
+    q = HipQuantizer((3,), 8, QUANTIZATION_TF, device)
+    q.setEncodings([(0.0, 1.0, 1 / 255, 0.0, 8)] * 3)
+    with pytest.raises(RuntimeError, match="broadcastable"):
+        q.quantizeDequantize(torch.zeros(8, 4))
+
+
+MM_CASES = [((4099,), ()), ((64, 256), (64, 1)), ((48, 512), (48, 8)), ((2, 6, 10, 12), (2, 3, 1, 4)), ((3, 5, 7), (5, 1))]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("shape,enc_shape", MM_CASES)
+def test_minmax_stats_and_encodings_bit_exact(device, dtype, shape, enc_shape):
+    a = OracleQuantizer(enc_shape, 8, QUANTIZATION_TF)
+    b = HipQuantizer(enc_shape, 8, QUANTIZATION_TF, device)
+    for seed in (1, 2, 3):
+        x = _data(shape, seed, dtype)
+        if dtype != torch.float32:
+            x = torch.nan_to_num(x, posinf=6e4, neginf=-6e4)  # keep infinities out of the encodings for 16-bit ranges
+        a.updateStats(x)
+        b.updateStats(x)
+        sa, sb = a.stats(), b.stats()
+        assert np.array_equal(sa[0], sb[0]) and np.array_equal(sa[1], sb[1])
+    for bw in (2, 4, 8, 16):
+        a.bitwidth = bw
+        b.q.bitwidth = bw
+        for sym, strict, uns in ((False, False, False), (True, False, False), (True, True, False), (True, False, True)):
+            for q in (a, b):
+                q.setStrictSymmetric(strict)
+                q.setUnsignedSymmetric(uns)
+            ea, eb = a.computeEncodings(sym), b.computeEncodings(sym)
+            assert np.array_equal(np.array(ea), np.array(eb)), (bw, sym, strict, uns)
+
+
+def test_minmax_all_nan_block_keeps_float_limits(device):
+    x = torch.full((2, 8), float("nan"))
+    x[1] = torch.arange(8.0)
+    a = OracleQuantizer((2, 1), 8, QUANTIZATION_TF)
+    b = HipQuantizer((2, 1), 8, QUANTIZATION_TF, device)
+    a.updateStats(x)
+    b.updateStats(x)
+    assert np.array_equal(a.stats()[0], b.stats()[0]) and np.array_equal(a.stats()[1], b.stats()[1])
+    assert b.stats()[0][0] == np.finfo(np.float32).max and b.stats()[1][0] == -np.finfo(np.float32).max
+
+
+def _same_pdf(a, b):
+    xa, pa, ma = a.stats()
+    xb, pb, mb = b.stats()
+    assert np.array_equal(ma, mb), (ma, mb)
+    assert np.array_equal(xa, xb)
+    assert np.array_equal(pa, pb)
+
+
+PDF_CASES = [((6000,), ()), ((70001,), ()), ((1 << 20,), ()), ((8, 4096), (8, 1)), ((6, 2, 512), (3, 2, 1)), ((4, 2, 3), (2, 3))]
+
+
+@pytest.mark.parametrize("shape,enc_shape", PDF_CASES)
+def test_pdf_update_bit_exact(device, shape, enc_shape):
+    a = OracleQuantizer(enc_shape, 8, QUANTIZATION_TF_ENHANCED)
+    b = HipQuantizer(enc_shape, 8, QUANTIZATION_TF_ENHANCED, device)
+    for seed in (1, 2, 3, 4):
+        x = _data(shape, seed) * (1.0 if seed < 3 else 2.5)  # later batches reach past the fixed range
+        ha = a.updateStats(x, return_histogram=True)
+        hb = b.updateStats(x, return_histogram=True)
+        assert torch.equal(ha, hb), (seed, (ha != hb).sum())
+        _same_pdf(a, b)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_pdf_update_16bit_inputs(device, dtype):
+    a = OracleQuantizer((), 8, QUANTIZATION_TF_ENHANCED)
+    b = HipQuantizer((), 8, QUANTIZATION_TF_ENHANCED, device)
+    for seed in (1, 2):
+        x = torch.nan_to_num(_data((33000,), seed, dtype), posinf=6e4, neginf=-6e4)
+        assert torch.equal(a.updateStats(x, True), b.updateStats(x, True))
+        _same_pdf(a, b)
+
+
+def test_pdf_zero_and_empty_batches(device):
+    a = OracleQuantizer((2, 1), 8, QUANTIZATION_TF_ENHANCED)
+    b = HipQuantizer((2, 1), 8, QUANTIZATION_TF_ENHANCED, device)
+    z = torch.zeros(2, 100)
+    for q in (a, b):
+        q.updateStats(z)
+    _same_pdf(a, b)
+    ea, eb = a.computeEncodings(False), b.computeEncodings(False)
+    assert np.array_equal(np.array(ea), np.array(eb))
+    x = z.clone()
+    x[1] = torch.linspace(-1, 3, 100)  # block 0 still all zero: stays uninitialised while block 1 gets its range
+    for q in (a, b):
+        q.updateStats(x)
+    _same_pdf(a, b)
+    assert b.stats()[2][:, 1].tolist() == [0, 1]
+    x[0] = torch.linspace(-2, 0.5, 100)
+    for q in (a, b):
+        q.updateStats(x)
+    _same_pdf(a, b)
+    for sym in (False, True):
+        assert np.array_equal(np.array(a.computeEncodings(sym)), np.array(b.computeEncodings(sym)))
+    for q in (a, b):
+        q.resetEncodingStats()
+    _same_pdf(a, b)
+
+
+def test_empty_tensors_do_not_broadcast(device):
+    # a zero-sized dimension is neither equal to nor a multiple of the encoding dimension (tensor_utils.cpp:28-58)
+    for shape, t in (((), torch.zeros(0)), ((2, 1), torch.zeros(2, 0))):
+        for scheme in (QUANTIZATION_TF, QUANTIZATION_TF_ENHANCED):
+            for q in (OracleQuantizer(shape, 8, scheme), HipQuantizer(shape, 8, scheme, device)):
+                with pytest.raises(RuntimeError, match="broadcastable"):
+                    q.updateStats(t)
+
+
+def test_pdf_update_of_an_empty_tensor_through_the_c_abi(device):
+    """UpdatePdf returns at once for cnt == 0 (math_functions.cpp:240-243): only the updated flag changes."""
+    from aimet_amd import _lib
+
+    lib = _lib.load()
+    xl = torch.zeros(1, 1536, dtype=torch.float64, device=device)
+    pdf = torch.zeros_like(xl)
+    meta = torch.zeros(1, 4, dtype=torch.int32, device=device)
+    st = _lib.DlqPdfState()
+    st.num_slots, st.xleft, st.pdf, st.meta = 1, xl.data_ptr(), pdf.data_ptr(), meta.data_ptr()
+    lay = _lib.make_layout([0], [1], [0])
+    _lib.check(lib.ahq_dlq_pdf_update(_lib.AHQ_F32, lay, None, st, 1, None, None, 0, _lib.current_stream(device)), "update")
+    assert meta.cpu().tolist() == [[0, 0, 1, 0]] and float(pdf.abs().sum()) == 0.0
+
+
+TFE_MODES = [(False, False, False), (True, False, False), (True, True, False), (True, False, True)]
+
+
+@pytest.mark.parametrize("bw", [4, 8, 16])
+@pytest.mark.parametrize("kind", ["normal", "positive", "laplace_outliers", "two_values"])
+def test_tfe_encodings_bit_exact(device, kind, bw):
+    g = torch.Generator().manual_seed(11)
+    if kind == "normal":
+        batches = [torch.randn(50000, generator=g) * 2 + 2 for _ in range(3)]
+    elif kind == "positive":
+        batches = [torch.randn(50000, generator=g).abs() * 1.5 for _ in range(2)]
+    elif kind == "laplace_outliers":
+        u = torch.rand(100000, generator=g) - 0.5
+        x = -torch.sign(u) * torch.log1p(-2 * u.abs())
+        x[::1000] = 40.0
+        batches = [x, x * 0.5]
+    else:
+        batches = [torch.tensor([0.0, 1.0] * 500)]
+    a = OracleQuantizer((), bw, QUANTIZATION_TF_ENHANCED)
+    b = HipQuantizer((), bw, QUANTIZATION_TF_ENHANCED, device)
+    for x in batches:
+        a.updateStats(x)
+        b.updateStats(x)
+    _same_pdf(a, b)
+    for sym, strict, uns in TFE_MODES:
+        for q in (a, b):
+            q.setStrictSymmetric(strict)
+            q.setUnsignedSymmetric(uns)
+        ea, eb = a.computeEncodings(sym), b.computeEncodings(sym)
+        assert np.array_equal(np.array(ea), np.array(eb)), (sym, strict, uns, ea, eb)
+        assert a.last_best == b.last_best, (sym, strict, uns, a.last_best, b.last_best)
+
+
+def test_tfe_encodings_per_block(device):
+    x = _data((6, 2, 512), 5, special=False)
+    a = OracleQuantizer((3, 2, 1), 8, QUANTIZATION_TF_ENHANCED)
+    b = HipQuantizer((3, 2, 1), 8, QUANTIZATION_TF_ENHANCED, device)
+    for q in (a, b):
+        q.updateStats(x)
+        q.updateStats(x * 0.5 + 1)
+    for sym in (False, True):
+        ea, eb = a.computeEncodings(sym), b.computeEncodings(sym)
+        assert np.array_equal(np.array(ea), np.array(eb))
+        assert a.last_best == b.last_best
+
+
+def test_end_to_end_tf_enhanced_then_qdq(device):
+    x = torch.from_numpy(C.INPUTS["normal_mean2_std2"].copy())
+    a = OracleQuantizer((), 8, QUANTIZATION_TF_ENHANCED)
+    b = HipQuantizer((), 8, QUANTIZATION_TF_ENHANCED, device)
+    for q in (a, b):
+        q.updateStats(x)
+        q.setEncodings(q.computeEncodings(False))
+    assert torch.equal(a.quantizeDequantize(x), b.quantizeDequantize(x))
