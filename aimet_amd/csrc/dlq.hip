@@ -80,7 +80,7 @@ struct PdfPrepArgs {
     double* xleft;
     double* pdf;
     int32_t* meta;
-    float* params;  // [S][4]: inv_bucket, float(pdf_offset), active, unused
+    float* params;  // [S][4]: inv_bucket, float(pdf_offset), active, iterations so far (int bits)
 };
 
 __device__ __forceinline__ float load_stat(const void* p, int dtype, int s) {
@@ -143,7 +143,7 @@ __global__ __launch_bounds__(kBlock) void dlq_pdf_prepare_kernel(const PdfPrepAr
             p[1] = 0.f;
             p[2] = 0.f;
         }
-        p[3] = 0.f;
+        p[3] = __int_as_float(meta[0]);  // iterations before this batch, for the running average
     }
 }
 
@@ -164,13 +164,20 @@ __device__ __forceinline__ bool pdf_index(float v, float inv, float off, int& id
     return (f >= 0.f) & (f < (float)kPdf);
 }
 
-template <typename IO, int VEC>
-__global__ __launch_bounds__(kBlock) void dlq_pdf_bin_kernel(const PdfBinArgs a) {
+// THREADS lanes share one workgroup-wide histogram in LDS.  Bucket i of copy c sits at word i * copies + c and lane l
+// adds to copy l % copies, so with many copies the lanes of a wave land in different banks whatever the data looks
+// like: real activations put most elements into a few dozen buckets, and with few copies the wave's 64 atomic adds
+// pile onto a handful of banks and are replayed bank conflict by bank conflict.
+constexpr int kPdfUnroll = 4;  // 16-byte loads in flight per lane: the workgroups are persistent, so this sets the bytes in flight
+
+template <typename IO, int VEC, int THREADS>
+__global__ __launch_bounds__(THREADS) void dlq_pdf_bin_kernel(const PdfBinArgs a) {
     extern __shared__ uint32_t lds[];  // [kPdf][copies]
     if (a.params[2] == 0.f) return;    // histogram not initialised (only all-zero batches so far): nothing to count
+    constexpr int kTile = THREADS * kPdfUnroll;  // vectors per workgroup and iteration
     const float inv = a.params[0], off = a.params[1];
     const int copies = a.copies;
-    for (int i = threadIdx.x; i < copies * kPdf; i += kBlock) lds[i] = 0;
+    for (int i = threadIdx.x; i < copies * kPdf; i += THREADS) lds[i] = 0;
     __syncthreads();
     const int bshift = a.copy_shift + 2;
     char* mine = reinterpret_cast<char*>(lds + (threadIdx.x & (copies - 1)));
@@ -179,26 +186,44 @@ __global__ __launch_bounds__(kBlock) void dlq_pdf_bin_kernel(const PdfBinArgs a)
         int idx;
         if (pdf_index(v, inv, off, idx)) atomicAdd(reinterpret_cast<uint32_t*>(mine + ((uint32_t)idx << bshift)), 1u);
     };
-    const int64_t full_tiles = a.nvec / kTileVec;
-    for (int64_t tile = blockIdx.x; tile < full_tiles; tile += gridDim.x) {
-        Pack<IO, VEC> in[kUnroll];
+    const int64_t full_tiles = a.nvec / kTile;
+    // software pipeline with two register buffers used alternately (no copies between them, which would force a full
+    // wait): the next tile's loads are in flight while the current tile is binned
+    Pack<IO, VEC> bufa[kPdfUnroll], bufb[kPdfUnroll];
+    auto load_tile = [&](Pack<IO, VEC>* buf, int64_t t) {
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u) in[u] = load_pack<IO, VEC>(x + (tile * kTileVec + u * kBlock + threadIdx.x) * VEC);
+        for (int u = 0; u < kPdfUnroll; ++u) buf[u] = load_pack<IO, VEC>(x + (t * kTile + u * THREADS + threadIdx.x) * VEC);
+    };
+    auto bin_tile = [&](const Pack<IO, VEC>* buf) {
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u)
+        for (int u = 0; u < kPdfUnroll; ++u)
 #pragma unroll
-            for (int k = 0; k < VEC; ++k) add(load_f32(in[u].v[k]));
+            for (int k = 0; k < VEC; ++k) add(load_f32(buf[u].v[k]));
+    };
+    const int64_t step = gridDim.x;
+    int64_t tile = blockIdx.x;
+    if (tile < full_tiles) load_tile(bufa, tile);
+    // the prefetch is unconditional (past the end it re-reads the current tile, an L2 hit, and the data is dropped):
+    // a conditional load would leave the number of loads in flight unknown and force a full wait before every use
+    while (tile < full_tiles) {
+        load_tile(bufb, tile + step < full_tiles ? tile + step : tile);
+        bin_tile(bufa);
+        tile += step;
+        if (tile >= full_tiles) break;
+        load_tile(bufa, tile + step < full_tiles ? tile + step : tile);
+        bin_tile(bufb);
+        tile += step;
     }
     if (blockIdx.x == 0) {  // ragged last tile and the elements past the last full vector
-        for (int64_t v = full_tiles * kTileVec + threadIdx.x; v < a.nvec; v += kBlock) {
+        for (int64_t v = full_tiles * kTile + threadIdx.x; v < a.nvec; v += THREADS) {
             const Pack<IO, VEC> pk = load_pack<IO, VEC>(x + v * VEC);
             for (int k = 0; k < VEC; ++k) add(load_f32(pk.v[k]));
         }
-        for (int64_t i = a.nvec * VEC + threadIdx.x; i < a.numel; i += kBlock) add(load_f32(x[i]));
+        for (int64_t i = a.nvec * VEC + threadIdx.x; i < a.numel; i += THREADS) add(load_f32(x[i]));
     }
     __syncthreads();
     uint32_t* out = a.partials + (size_t)blockIdx.x * kPdf;
-    for (int i = threadIdx.x; i < kPdf; i += kBlock) {
+    for (int i = threadIdx.x; i < kPdf; i += THREADS) {
         uint32_t c = 0;
         for (int cp = 0; cp < copies; ++cp) c += lds[(size_t)i * copies + cp];
         out[i] = c;
@@ -256,17 +281,14 @@ __global__ __launch_bounds__(kBlock) void dlq_pdf_finish_kernel(const PdfFinArgs
     if (active) {
         const uint32_t* c = a.counts + (size_t)s * a.nparts * kPdf;
         for (int p = 0; p < a.nparts; ++p) h += c[(size_t)p * kPdf + i];
-        const int it = a.meta[4 * s];
+        const int it = __float_as_int(a.params[4 * s + 3]);
         const double prob = (double)h / (double)a.cnt;
         double* pdf = a.pdf + (size_t)s * kPdf;
         pdf[i] = (pdf[i] * it + prob) / (it + 1);
     }
     if (a.hist_out) a.hist_out[(size_t)s * kPdf + i] = h;
-}
-
-__global__ void dlq_pdf_bump_kernel(const float* params, int32_t* meta, int S) {
-    const int s = blockIdx.x * blockDim.x + threadIdx.x;
-    if (s < S && params[4 * s + 2] != 0.f) meta[4 * s] += 1;
+    // pdf.iterations++ ; every thread above took the old count from `params`, so nothing else reads this word here
+    if (active && i == 0) a.meta[4 * s] = __float_as_int(a.params[4 * s + 3]) + 1;
 }
 
 __global__ void dlq_pdf_mark_kernel(int32_t* meta, int S) {
@@ -524,7 +546,9 @@ __global__ __launch_bounds__(kWave) void dlq_tfe_select_kernel(const TfeArgs a) 
 // -------------------------------------------------------------------------------------------------- host side ---
 namespace {
 
-constexpr int kPdfBlocksMax = 1024;
+constexpr int kPdfThreads = 1024;  // one workgroup per compute unit: 16 copies x 1536 buckets x 4 B = 96 KB of LDS
+constexpr int kPdfCopies = 8;
+constexpr int kPdfBlocksMax = 512;
 
 size_t up256(size_t v) { return (v + 255) & ~(size_t)255; }
 
@@ -540,8 +564,8 @@ bool make_pdf_plan(int dtype, const ahq_layout& layout, const void* x, PdfPlan* 
     const CanonLayout& c = pp->plan.cl;
     const size_t S = (size_t)c.num_enc;
     pp->fast = c.kind == kIJK && c.J == 1;
-    pp->copies = 8;  // 8 x 1536 x 4 B = 48 KB of LDS
-    const int64_t ntiles = (pp->plan.nvec + kTileVec - 1) / kTileVec;
+    pp->copies = kPdfCopies;
+    const int64_t ntiles = (pp->plan.nvec + kPdfThreads * kPdfUnroll - 1) / (kPdfThreads * kPdfUnroll);
     int64_t nb = pp->fast ? ntiles : (c.numel + kBlock - 1) / kBlock;
     if (nb > kPdfBlocksMax) nb = kPdfBlocksMax;
     if (nb < 1) nb = 1;
@@ -649,7 +673,8 @@ extern "C" int ahq_dlq_pdf_update(int32_t dtype, const ahq_layout* layout, const
     ba.x = x;
     ba.params = params;
     ba.copies = pp.copies;
-    ba.copy_shift = 3;
+    ba.copy_shift = 0;
+    while ((1 << ba.copy_shift) < pp.copies) ++ba.copy_shift;
     uint32_t* counts = reinterpret_cast<uint32_t*>(w + pp.off_counts);
     PdfFinArgs fa{};
     fa.params = params;
@@ -660,11 +685,22 @@ extern "C" int ahq_dlq_pdf_update(int32_t dtype, const ahq_layout* layout, const
     if (pp.fast) {
         ba.partials = counts;
         const size_t lds = (size_t)pp.copies * kPdf * 4;
-        const dim3 g(pp.nblocks), b(kBlock);
+        const dim3 g(pp.nblocks), b(kPdfThreads);
+#define AHQ_LAUNCH_PDF_K(K)                                                                                    \
+    do {                                                                                                       \
+        static bool attr_set = false; /* more than 64 KB of dynamic LDS has to be allowed once per kernel */     \
+        if (!attr_set) {                                                                                       \
+            if (hipFuncSetAttribute(reinterpret_cast<const void*>(&K), hipFuncAttributeMaxDynamicSharedMemorySize, \
+                                    (int)lds) != hipSuccess)                                                   \
+                return set_error("cannot reserve LDS for the PDF kernel"), AHQ_ERR_LAUNCH;                     \
+            attr_set = true;                                                                                   \
+        }                                                                                                      \
+        hipLaunchKernelGGL(K, g, b, lds, s, ba);                                                               \
+    } while (0)
 #define AHQ_LAUNCH_PDF(IO)                                                                                     \
     do {                                                                                                       \
-        if (pp.plan.vec == 1) hipLaunchKernelGGL((dlq_pdf_bin_kernel<IO, 1>), g, b, lds, s, ba);               \
-        else hipLaunchKernelGGL((dlq_pdf_bin_kernel<IO, IoTraits<IO>::kVec>), g, b, lds, s, ba);               \
+        if (pp.plan.vec == 1) AHQ_LAUNCH_PDF_K((dlq_pdf_bin_kernel<IO, 1, kPdfThreads>));                      \
+        else AHQ_LAUNCH_PDF_K((dlq_pdf_bin_kernel<IO, IoTraits<IO>::kVec, kPdfThreads>));                      \
     } while (0)
         switch (dtype) {
             case AHQ_F32: AHQ_LAUNCH_PDF(float); break;
@@ -672,6 +708,7 @@ extern "C" int ahq_dlq_pdf_update(int32_t dtype, const ahq_layout* layout, const
             default: AHQ_LAUNCH_PDF(bf16_t); break;
         }
 #undef AHQ_LAUNCH_PDF
+#undef AHQ_LAUNCH_PDF_K
         fa.counts = counts;
         fa.nparts = pp.nblocks;
         if (pp.nblocks > kPdfFoldGroups) {
@@ -695,7 +732,6 @@ extern "C" int ahq_dlq_pdf_update(int32_t dtype, const ahq_layout* layout, const
         fa.nparts = 1;
     }
     hipLaunchKernelGGL(dlq_pdf_finish_kernel, dim3(kPdf / kBlock, S), dim3(kBlock), 0, s, fa);
-    hipLaunchKernelGGL(dlq_pdf_bump_kernel, dim3((S + 255) / 256), dim3(256), 0, s, params, st->meta, S);
     return check_launch("dlq_pdf_update");
 }
 

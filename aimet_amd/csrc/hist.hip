@@ -25,7 +25,7 @@ extern "C" size_t ahq_minmax_workspace_bytes(const ahq_layout* layout);
 
 namespace ahq {
 
-constexpr int kHistBlocksMax = 1024;  // persistent workgroups of the binning pass (4 per CU)
+constexpr int kHistBlocksMax = 1536;  // persistent workgroups of the binning pass (6 per CU)
 constexpr int kRng = 8;               // floats per slot in `ranges`
 constexpr int kFoldGroups = 32;       // partial histograms left after the first fold
 
@@ -225,7 +225,7 @@ __device__ __forceinline__ int bin_estimate(float v, const RangeC& r, float Bf, 
 // elements that need the exact division or lie outside the range are only flagged, and one wave-uniform branch per
 // tile revisits them.
 template <typename IO, int VEC, int NH>
-__global__ __launch_bounds__(kBlock) void hist_bin_kernel(const BinArgs a) {
+__global__ __launch_bounds__(kBlock, 6) void hist_bin_kernel(const BinArgs a) {
     extern __shared__ uint32_t lds[];  // [NH][B][copies]: lane l adds to copy l % copies, neighbouring copies sit in neighbouring banks
     __shared__ uint32_t cnt_smem[kBlock / kWave][NH][2];
     const int B = a.num_bins;
@@ -462,7 +462,8 @@ bool make_hist_plan(int dtype, const ahq_layout& layout, const void* x, int num_
     hp->fast = false;
     hp->copies = 0;
     if (c.kind == kIJK && c.J == 1) {
-        const int fit = (int)((65536 - 512) / ((size_t)2 * num_bins * 4));
+        // at most 16 KB of LDS per workgroup of four waves, so that eight workgroups (32 waves) fit a compute unit
+        const int fit = (int)(16384 / ((size_t)2 * num_bins * 4));
         int copies = 0;
         for (int c = 8; c >= 1; c >>= 1)
             if (c <= fit) {

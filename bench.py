@@ -256,7 +256,8 @@ def cpu_baseline_qdq(w, scale, offset, qmin, qmax, bytes_step, budget_s=12.0):
 def _laplace_batch(shape, seed, dev):
     """Laplace(0, 1) with 0.1 % of the elements replaced by +-U(20, 60), generated on the device."""
     g = torch.Generator(device=dev).manual_seed(seed)
-    u = torch.rand(shape, generator=g, device=dev) - 0.5
+    # u = +-0.5 would give an infinite sample; rand() does return 0 a few times in 67 M draws
+    u = (torch.rand(shape, generator=g, device=dev) - 0.5).clamp_(-0.4999999, 0.4999999)
     x = -torch.sign(u) * torch.log1p(-2 * u.abs())
     n = x.numel()
     k = n // 1000
@@ -358,12 +359,124 @@ def run_hist_workload(steps, warmup, dev, with_cpu_baseline=True, batches=16, sh
     return out
 
 
+def run_dlq_workload(steps, warmup, dev, with_cpu_baseline=True, batches=16, shape=(8, 2048, 4096)):
+    """dlq: DlQuantization TF-enhanced calibration of the c3 stream (1536-bucket PDF per batch, then the 17 x 21 + 1
+    candidate search for an 8-bit asymmetric encoding) followed by one per-tensor quantize-dequantize of a batch."""
+    from aimet_amd import dlq
+    from oracle import dlq as OD
+
+    _ensure_built()
+    _copy_reference(dev)
+    xs = [_laplace_batch(shape, b, dev) for b in range(batches)]
+    q = dlq.BlockTensorQuantizer((), 8, dlq.QUANTIZATION_TF_ENHANCED, device=dev)
+    y = torch.empty_like(xs[0])
+
+    def step():
+        q.resetEncodingStats()
+        for x in xs:
+            q.updateStats(x)
+        enc = q.computeEncodings(False)
+        q.setEncodings(enc)
+        q.quantizeDequantize(xs[0], y)
+        return enc
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        enc = step()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) / steps
+
+    def event_time(fn, reps):
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        fn()
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / reps * 1e-3
+
+    t_upd = event_time(lambda: q.updateStats(xs[1]), 20)   # range already fixed: one read of the batch
+    t_qdq = event_time(lambda: q.quantizeDequantize(xs[0], y), 20)
+    t_enc = event_time(lambda: q.computeEncodings(False), 5)
+    n_b = xs[0].numel()
+    n = n_b * batches
+    bytes_upd = 4 * n_b
+    bytes_qdq = 8 * n_b
+    bytes_step = batches * bytes_upd + bytes_qdq
+
+    # parity on the first two batches and a bounded sample of the quantize-dequantize, against the C oracle
+    q.resetEncodingStats()
+    ref = OD.Pdf()
+    hist_ok = True
+    for b in range(2):
+        h = q.updateStats(xs[b], return_histogram=True)
+        hr = ref.update(xs[b].cpu().numpy())
+        hist_ok = hist_ok and bool((h.cpu().numpy().astype("int64")[0] == hr.astype("int64")).all())
+    pdf_ok = bool((q._pdf.cpu().numpy()[0] == ref.pdf).all() and (q._xleft.cpu().numpy()[0] == ref.xleft).all())
+    enc_gpu = q.computeEncodings(False)[0]
+    enc_ref = ref.compute_encoding(8, False)
+    enc_ok = tuple(enc_gpu) == tuple(float(v) for v in enc_ref[:4]) + (8,)
+    q.setEncodings([enc_gpu])
+    sample = xs[0].view(-1)[: 1 << 22]
+    y_s = q.quantizeDequantize(sample).cpu().numpy()
+    y_ok = bool((y_s.view("int32") == OD.qdq(sample.cpu().numpy(), enc_ref[:4]).view("int32")).all())
+
+    out = {
+        "metric": "QDQ fwd+bwd GB/s (% of HBM peak); calibration elems/s; vs host-CPU ref",
+        "value": round(bytes_step / wall / 1e9, 2),
+        "unit": "GB/s",
+        "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": round(wall * 1e3, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "dlq_tf_enhanced_pdf1536_search17x21_qdq_fp32_16x8x2048x4096", "elements": n,
+                   "algorithmic_bytes_per_step": bytes_step, "batches": batches},
+        "pct_of_hbm_peak": round(100.0 * bytes_step / wall / 1e9 / HBM_PEAK_GBS, 2),
+        "elements_per_s": round(n / wall, 1),
+        "kernels": {"pdf_update(range fixed)": {"us": round(t_upd * 1e6, 2), "GBps": round(bytes_upd / t_upd / 1e9, 1)},
+                    "dlq_qdq_forward": {"us": round(t_qdq * 1e6, 2), "GBps": round(bytes_qdq / t_qdq / 1e9, 1)},
+                    "tfe_search(with host read-back)": {"us": round(t_enc * 1e6, 2), "candidates": 358, "buckets": 1536}},
+        "encoding": {"min": enc[0].min, "max": enc[0].max, "delta": enc[0].delta, "offset": enc[0].offset},
+        "parity": {"hist_bit_exact": hist_ok, "pdf_bit_exact": pdf_ok, "encoding_bit_exact": bool(enc_ok),
+                   "qdq_bit_exact": y_ok, "sample": "first 2 of 16 batches; 4M-element quantize-dequantize"},
+        "roofline": {"bound": "hbm", "kernel": "dlq_pdf_bin_kernel", "achieved": round(bytes_upd / t_upd / 1e9, 1),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(bytes_upd / t_upd / 1e9 / HBM_PEAK_GBS, 4),
+                     "algorithmic_bytes": bytes_upd, "traffic": None},
+    }
+    if with_cpu_baseline:
+        # the scalar C restatement of the reference's loops, one thread, on a bounded slice of one batch
+        m = 1 << 24
+        xc = xs[0].view(-1)[:m].cpu().numpy()
+        p = OD.Pdf()
+        p.update(xc[:1024])
+        t0 = time.perf_counter()
+        p.update(xc)
+        t_pdf = time.perf_counter() - t0
+        t0 = time.perf_counter()
+        OD.qdq(xc, enc_ref[:4])
+        t_q = time.perf_counter() - t0
+        t0 = time.perf_counter()
+        p.compute_encoding(8, False)
+        t_s = time.perf_counter() - t0
+        cpu_step = (t_pdf * batches + t_q) * (n_b / m) + t_s
+        out["cpu_baseline"] = {"value": round(bytes_step / cpu_step / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+                               "sample": f"{m} elements of one batch through the scalar C loops (pdf update "
+                                         f"{t_pdf * 1e3:.1f} ms, quantize-dequantize {t_q * 1e3:.1f} ms), search "
+                                         f"{t_s * 1e3:.2f} ms, scaled to the full step",
+                               "elements_per_s": round(n / cpu_step, 1)}
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["c3"])
+    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["c3", "dlq"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -376,6 +489,8 @@ def main():
     dev = torch.device("cuda:0")
     if args.workload == "c3":
         out = run_hist_workload(min(args.steps, 10), min(args.warmup, 2), dev, with_cpu_baseline=not args.no_cpu_baseline)
+    elif args.workload == "dlq":
+        out = run_dlq_workload(min(args.steps, 10), min(args.warmup, 2), dev, with_cpu_baseline=not args.no_cpu_baseline)
     else:
         out = run_qdq_workload(args.workload, args.steps, args.warmup, dev, with_cpu_baseline=not args.no_cpu_baseline)
     print(json.dumps(out))
