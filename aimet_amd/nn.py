@@ -1,0 +1,152 @@
+"""The quantized-module glue a whole-model calibration needs, for ``nn.Linear`` only.
+
+Counterpart of the reference's ``BaseQuantizationMixin`` as used by ``QuantizedLinear``
+(aimet_torch/nn/base.py:228-427, aimet_torch/nn/fake_quant.py): one input quantizer, one output quantizer, a weight
+quantizer; ``compute_encodings()`` calibrates the weight quantizer from the weight once and puts the activation
+quantizers into observe-and-pass-through mode (nn/base.py:392-427); outside that context the forward pass
+quantize-dequantizes input, weight and output.  The GEMM itself is ``torch.nn.functional.linear``.
+
+Not reproduced: the lossless decomposition of an already-quantized weight (``_decompose_prequantized_tensor``,
+aimet_torch/utils.py:2024-2300).  Only its early exit is -- a weight whose first blocks hold more distinct magnitudes
+than the grid has levels goes straight to min/max calibration, which is what happens for every trained or random
+weight; a weight that passes the early exit raises NotImplementedError rather than being calibrated differently.
+"""
+
+from __future__ import annotations
+
+import contextlib
+import math
+from typing import Iterable, Optional
+
+import torch
+from torch import nn
+from torch.nn import functional as F
+
+from aimet_amd.quantization._utils import concretize_block_size
+from aimet_amd.quantization.affine.quantizer import AffineQuantizerBase, GroupedBlockQuantizeDequantize
+from aimet_amd.quantization.base.quantizer import QuantizerBase
+
+__all__ = ["QuantizedLinear", "compute_encodings", "quantized_linears"]
+
+
+def _may_be_prequantized(param: torch.Tensor, qtzr: AffineQuantizerBase) -> bool:
+    """The early exit of _decompose_prequantized_tensor (aimet_torch/utils.py:2098-2118): the first 64 blocks, first
+    2 * num_levels elements each; more distinct magnitudes than grid levels means the tensor is not on a grid."""
+    num_levels = max(abs(qtzr.qmax), abs(qtzr.qmin)) + 1
+    shape = tuple(qtzr.shape)
+    block = concretize_block_size(tuple(param.shape), shape, qtzr.block_size or tuple(-1 for _ in shape))
+    block = (*param.shape[: param.dim() - len(block)], *block)
+    split = []
+    for d, b in zip(param.shape, block):
+        split += [d // b, b]
+    nd = len(split)
+    x = param.reshape(split).permute(*range(0, nd, 2), *range(1, nd, 2))
+    nblocks = math.prod(split[0::2])
+    x = x.reshape(nblocks, -1)
+    if x.shape[1] <= num_levels:
+        return True
+    xs = x[:64, : num_levels * 2].float().abs().sort(dim=1).values
+    distinct = (xs[:, 1:] != xs[:, :-1]).sum(dim=1) + 1
+    return not bool(torch.any(distinct > num_levels))
+
+
+class QuantizedLinear(nn.Linear):
+    """``nn.Linear`` with quantizers at its input, weight and output (any of them may be None)."""
+
+    def __init__(self, *args, **kwargs):
+        super().__init__(*args, **kwargs)
+        self.input_quantizers = nn.ModuleList([None])
+        self.output_quantizers = nn.ModuleList([None])
+        self.param_quantizers = nn.ModuleDict({"weight": None, "bias": None})
+
+    @classmethod
+    def from_module(cls, linear: nn.Linear) -> "QuantizedLinear":
+        """Wraps an existing layer; the parameters are shared, not copied."""
+        q = cls.__new__(cls)
+        nn.Module.__init__(q)
+        q.in_features, q.out_features = linear.in_features, linear.out_features
+        q.weight, q.bias = linear.weight, linear.bias
+        q.input_quantizers = nn.ModuleList([None])
+        q.output_quantizers = nn.ModuleList([None])
+        q.param_quantizers = nn.ModuleDict({"weight": None, "bias": None})
+        return q
+
+    def __call__(self, *args, **kwargs):
+        self._compute_param_encodings(overwrite=False)  # nn/base.py:262-265
+        return super().__call__(*args, **kwargs)
+
+    def forward(self, input: torch.Tensor) -> torch.Tensor:  # pylint: disable=redefined-builtin
+        iq, oq = self.input_quantizers[0], self.output_quantizers[0]
+        wq, bq = self.param_quantizers["weight"], self.param_quantizers["bias"]
+        if iq is not None:
+            input = iq(input)
+        weight = self.weight if wq is None else wq(self.weight)
+        bias = self.bias if (bq is None or self.bias is None) else bq(self.bias)
+        out = F.linear(input.as_subclass(torch.Tensor), weight.as_subclass(torch.Tensor),
+                       None if bias is None else bias.as_subclass(torch.Tensor))
+        if oq is not None:
+            out = oq(out)
+        return out
+
+    def _compute_param_encodings(self, overwrite: bool):
+        """nn/base.py:331-383"""
+        for name, qtzr in self.param_quantizers.items():
+            if qtzr is None or not qtzr.is_overwrite_allowed():
+                continue
+            if qtzr.is_initialized() and not overwrite:
+                continue
+            param = getattr(self, name)
+            if param is None:
+                continue
+            if (isinstance(qtzr, AffineQuantizerBase) and not isinstance(qtzr, GroupedBlockQuantizeDequantize)
+                    and qtzr.symmetric and math.ceil((qtzr.qmin + qtzr.qmax) / 2) == 0):
+                if _may_be_prequantized(param.detach(), qtzr):
+                    raise NotImplementedError(
+                        f"parameter '{name}' looks like an already-quantized tensor; recovering its grid "
+                        "(lossless decomposition) is not implemented here"
+                    )
+            with qtzr._compute_encodings(passthrough=True):  # pylint: disable=protected-access
+                _ = qtzr(param)
+
+    @contextlib.contextmanager
+    def compute_encodings(self):
+        """nn/base.py:392-427: weights are calibrated on entry; activation quantizers observe their inputs and pass
+        them through unquantized, and set their ranges on exit."""
+        self._compute_param_encodings(overwrite=True)
+        with contextlib.ExitStack() as stack:
+            for qtzr in list(self.input_quantizers) + list(self.output_quantizers):
+                if not isinstance(qtzr, QuantizerBase) or not qtzr.is_overwrite_allowed():
+                    continue
+                stack.enter_context(qtzr._compute_encodings(passthrough=True))  # pylint: disable=protected-access
+            yield
+
+
+def quantized_linears(model: nn.Module) -> Iterable[QuantizedLinear]:
+    return (m for m in model.modules() if isinstance(m, QuantizedLinear))
+
+
+@contextlib.contextmanager
+def compute_encodings(model: nn.Module):
+    """aimet_torch.nn.compute_encodings (nn/base.py): the compute_encodings context of every quantized module."""
+    with contextlib.ExitStack() as stack:
+        for m in quantized_linears(model):
+            stack.enter_context(m.compute_encodings())
+        yield
+
+
+def wrap_linears(model: nn.Module, make_quantizers) -> int:
+    """Replaces every nn.Linear in ``model`` by a QuantizedLinear sharing its parameters.  ``make_quantizers(name,
+    linear)`` returns (input quantizer, weight quantizer, output quantizer), any of them None."""
+    count = 0
+    for parent_name, parent in list(model.named_modules()):
+        for child_name, child in list(parent.named_children()):
+            if type(child) is nn.Linear:  # pylint: disable=unidiomatic-typecheck
+                q = QuantizedLinear.from_module(child)
+                full = f"{parent_name}.{child_name}" if parent_name else child_name
+                iq, wq, oq = make_quantizers(full, child)
+                q.input_quantizers[0] = iq
+                q.param_quantizers["weight"] = wq
+                q.output_quantizers[0] = oq
+                setattr(parent, child_name, q)
+                count += 1
+    return count

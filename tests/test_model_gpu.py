@@ -1,0 +1,135 @@
+"""Whole-model calibration and quantized forward of a small Llama-style decoder: every quantizer's statistics,
+encodings and quantize-dequantize output are checked, bit for bit, against the CPU oracle applied to the very tensors
+that quantizer saw on the GPU (the GEMMs in between are PyTorch's and are not under test)."""
+
+import pytest
+import torch
+
+import llama_harness as LH
+from aimet_amd import nn as qnn
+from aimet_amd.quantization.affine import QuantizeDequantize
+from oracle import torch_ref as O
+
+pytestmark = pytest.mark.gpu
+
+CFG = LH.LlamaConfig(layers=2, hidden=128, ffn=256, heads=4, vocab=512)
+
+
+def _bits(t):
+    return t.contiguous().view(torch.int16 if t.element_size() == 2 else torch.int32)
+
+
+@pytest.fixture(scope="module")
+def calibrated(device):
+    torch.manual_seed(0)
+    model = LH.build(CFG, device, seed=0)
+    n = LH.quantize(model)
+    assert n == 2 * 7 + 1
+    seen = {}   # quantizer -> list of CPU copies of its inputs during calibration
+    passed = {}  # quantizer -> True while every calibration-time output had its input's bits
+    hooks = []
+
+    def record(key):
+        def hook(mod, args, out):
+            x = args[0].detach()
+            seen[key].append(x.cpu())
+            passed[key] = passed.get(key, True) and torch.equal(_bits(out.detach().as_subclass(torch.Tensor)), _bits(x))
+        return hook
+
+    for name, m in model.named_modules():
+        if isinstance(m, QuantizeDequantize):
+            seen[name] = []
+            hooks.append(m.register_forward_hook(record(name)))
+    batches = LH.calibration_batches(CFG, device, batches=3, seq=64)
+    with torch.no_grad(), qnn.compute_encodings(model):
+        for ids in batches:
+            out = model(ids)
+            assert out.shape == (1, 64, CFG.vocab)
+    for h in hooks:
+        h.remove()
+    return model, seen, batches, passed
+
+
+def test_every_quantizer_is_calibrated_like_the_oracle(calibrated):
+    model, seen, _, _ = calibrated
+    quantizers = {n: m for n, m in model.named_modules() if isinstance(m, QuantizeDequantize)}
+    assert len(quantizers) == 3 * 15
+    for name, q in quantizers.items():
+        xs = seen[name]
+        assert q.is_initialized()
+        is_weight = name.endswith("param_quantizers.weight")
+        # a weight quantizer sees its weight once for calibration (on entry) and once per forward pass after that
+        assert len(xs) == (4 if is_weight else 3), name
+        if is_weight:
+            xs = xs[:1]
+        mn = mx = None
+        for x in xs:
+            a, b = O.reduce_minmax(x, tuple(q.shape), q.block_size)
+            mn = a if mn is None else torch.minimum(mn, a)
+            mx = b if mx is None else torch.maximum(mx, b)
+        lo, hi = O.minmax_encodings(mn, mx, q.qmax - q.qmin, q.symmetric)
+        assert lo.dtype == torch.bfloat16
+        assert torch.equal(q.min.detach().cpu(), lo.view(q.shape).to(torch.float32)), name
+        assert torch.equal(q.max.detach().cpu(), hi.view(q.shape).to(torch.float32)), name
+        scale = O.scale_from_minmax(q.min.detach().cpu(), q.max.detach().cpu(), q.qmin, q.qmax)
+        offset = O.offset_from_minmax(q.min.detach().cpu(), scale, q.qmin, q.qmax, q.symmetric)
+        assert torch.equal(q.get_scale().detach().cpu(), scale), name
+        assert torch.equal(q.get_offset().detach().cpu(), offset), name
+
+
+def test_calibration_passes_activations_through_unquantized(calibrated):
+    _, _, _, passed = calibrated
+    acts = [k for k in passed if "param_quantizers" not in k]
+    assert len(acts) == 30 and all(passed[k] for k in acts)
+    # weights are quantized during the calibration passes (their quantizers are calibrated on entry)
+    assert not any(passed[k] for k in passed if "param_quantizers" in k)
+
+
+def test_quantized_forward_matches_the_oracle_per_quantizer(calibrated):
+    model, _, batches, _ = calibrated
+    quantizers = {n: m for n, m in model.named_modules() if isinstance(m, QuantizeDequantize)}
+    io = {}
+    hooks = [m.register_forward_hook(lambda mod, args, out, key=n: io.__setitem__(key, (args[0].detach().cpu(),
+                                                                                      out.detach().cpu())))
+             for n, m in quantizers.items()]
+    with torch.no_grad():
+        logits = model(batches[0])
+    for h in hooks:
+        h.remove()
+    assert torch.isfinite(logits.float()).all()
+    assert len(io) == len(quantizers)
+    changed = 0
+    for name, q in quantizers.items():
+        x, y = io[name]
+        scale, offset = q.get_scale().detach().cpu(), q.get_offset().detach().cpu()
+        if q.block_size is None:
+            # no gradients needed: the ATen fake-quantize arithmetic (torch_builtins.py:243-260)
+            ref = O.qdq_v1(x, scale, offset, q.qmin, q.qmax)[0]
+        else:
+            ref = O.qdq_v2_forward(x, scale, offset, q.qmin, q.qmax, q.block_size).y
+        assert ref.dtype == y.dtype == torch.bfloat16
+        assert torch.equal(_bits(y.as_subclass(torch.Tensor)), _bits(ref)), name
+        changed += int(not torch.equal(_bits(y.as_subclass(torch.Tensor)), _bits(x)))
+    assert changed >= 15  # at least every 4-bit weight actually moved
+
+
+def test_param_encodings_are_computed_lazily_on_first_call(device):
+    model = LH.build(CFG, device, seed=3)
+    LH.quantize(model)
+    lin = model.blocks[0].attn.q_proj
+    lin.input_quantizers[0] = None
+    lin.output_quantizers[0] = None
+    wq = lin.param_quantizers["weight"]
+    assert not wq.is_initialized()
+    with torch.no_grad():
+        lin(torch.randn(4, CFG.hidden, device=device, dtype=torch.bfloat16))
+    assert wq.is_initialized()
+
+
+def test_prequantized_weight_is_reported(device):
+    lin = qnn.QuantizedLinear(64, 8, bias=False).to(device)
+    with torch.no_grad():
+        lin.weight.copy_(torch.randint(-8, 8, (8, 64)).float() * 0.125)
+    lin.param_quantizers["weight"] = QuantizeDequantize((8, 1), 4, symmetric=True).to(device)
+    with pytest.raises(NotImplementedError):
+        lin(torch.randn(2, 64, device=device))
