@@ -193,24 +193,30 @@ def _workspace(nbytes: int, device) -> Optional[torch.Tensor]:
     return torch.empty(nbytes, dtype=torch.uint8, device=device)
 
 
+def _launch_forward(tensor, scale, offset, arith, op, compute_dtype, qmin, qmax, block_size, zps):
+    lib = _lib.load()
+    x, layout = _prepare(tensor.detach(), scale.shape, block_size)
+    s = _enc_f32(scale)
+    o = _enc_f32(offset)
+    grid = _grid(arith, op, x.dtype, compute_dtype, qmin, qmax, zps)
+    y = torch.empty_like(x)
+    if x.numel():
+        _lib.check(
+            lib.ahq_qdq_forward(grid, layout, x.data_ptr(), y.data_ptr(), None, s.data_ptr(), o.data_ptr(),
+                                None, None, _lib.current_stream(x.device)),
+            "ahq_qdq_forward",
+        )
+    return y, x, s, o, grid, layout
+
+
 # ---------------------------------------------------------------------------------------------- autograd function --
 class _HipAffineFunction(torch.autograd.Function):
     """One fused kernel forward, one fused kernel backward (input, scale and offset gradients together)."""
 
     @staticmethod
     def forward(ctx, tensor, scale, offset, arith, op, compute_dtype, qmin, qmax, block_size, zps):
-        lib = _lib.load()
-        x, layout = _prepare(tensor.detach(), scale.shape, block_size)
-        s = _enc_f32(scale)
-        o = _enc_f32(offset)
-        grid = _grid(arith, op, x.dtype, compute_dtype, qmin, qmax, zps)
-        y = torch.empty_like(x)
-        if x.numel():
-            _lib.check(
-                lib.ahq_qdq_forward(grid, layout, x.data_ptr(), y.data_ptr(), None, s.data_ptr(), o.data_ptr(),
-                                    None, None, _lib.current_stream(x.device)),
-                "ahq_qdq_forward",
-            )
+        y, x, s, o, grid, layout = _launch_forward(tensor, scale, offset, arith, op, compute_dtype, qmin, qmax,
+                                                   block_size, zps)
         ctx.grid = grid
         ctx.layout = layout
         ctx.save_for_backward(x, s, o)
@@ -253,6 +259,9 @@ class _HipAffineFunction(torch.autograd.Function):
 
 def _apply(tensor, scale, offset, arith, op, compute_dtype, qmin, qmax, block_size, zps):
     bs = tuple(block_size) if block_size else None
+    if not torch.is_grad_enabled() or not (tensor.requires_grad or scale.requires_grad or offset.requires_grad):
+        # nothing to differentiate: skip the autograd bookkeeping (a whole-model forward makes hundreds of these calls)
+        return _launch_forward(tensor, scale, offset, arith, op, compute_dtype, qmin, qmax, bs, zps)[0]
     return _HipAffineFunction.apply(tensor, scale, offset, arith, op, compute_dtype, qmin, qmax, bs, zps)
 
 

@@ -169,6 +169,27 @@ class AffineQuantizerBase(QuantizerBase, _GridMixin):
             self.max.copy_(max if isinstance(max, torch.Tensor) else torch.tensor(max))
 
     def get_encodings(self) -> Optional[AffineEncoding]:
+        # When no gradient can flow into min/max, scale and offset are constants of the current parameter values:
+        # they are derived once and reused until min or max is written again (their version counters change) or
+        # moved.  A whole-model forward calls this once per quantizer, and the half-dozen tiny kernels behind
+        # get_scale()/get_offset() would otherwise cost more than the quantize-dequantize kernel itself.
+        # (Writes through `.data` do not bump the version counter and are not seen; the reference's own
+        # is_initialized() bookkeeping has the same blind spot.)
+        if torch.is_grad_enabled() and (self.min.requires_grad or self.max.requires_grad):
+            return self._derive_encodings()
+        mn, mx = self.min, self.max
+        key = (id(mn), mn._version, mn.data_ptr(), id(mx), mx._version, mx.data_ptr(),  # pylint: disable=protected-access
+               self.qmin, self.qmax, self._symmetric, self.block_size, self.zero_point_shift)
+        cached = self.__dict__.get("_encoding_cache")
+        if cached is not None and cached[0] == key:
+            return cached[1]
+        with torch.no_grad():
+            enc = self._derive_encodings()
+        if enc is not None:
+            self.__dict__["_encoding_cache"] = (key, enc)
+        return enc
+
+    def _derive_encodings(self) -> Optional[AffineEncoding]:
         scale = self.get_scale(dtype=torch.float32)
         offset = self._get_offset(scale=scale, dtype=torch.float32)
         if scale is None or offset is None:
@@ -253,6 +274,9 @@ class AffineQuantizerBase(QuantizerBase, _GridMixin):
             if input.numel() == 0:
                 return inner_forward(input)
             batch_stats = self.encoding_analyzer.update_stats(input)
+            if passthrough:
+                # the input is only observed; the dynamic encodings of this batch would go unused
+                return inner_forward(input)
             lo, hi = self.encoding_analyzer.compute_encodings_from_stats(
                 batch_stats, self._num_steps_for_calibration(), self.symmetric
             )

@@ -287,12 +287,14 @@ class MinMaxEncodingAnalyzer(EncodingAnalyzer[_MinMaxRange]):
 
 def _flag_extreme_min_max(curr_min, curr_max):
     """Warn about non-finite or near-overflow encodings (reference: encoding_analyzer.py:484-498)."""
-    if not (torch.all(torch.isfinite(curr_min)) and torch.all(torch.isfinite(curr_max))):
-        warnings.warn("Infinite or NaN values detected within input! This may skew the associated encodings")
     big = torch.full_like(curr_min, torch.finfo(curr_min.dtype).max)
-    if torch.any(torch.isclose(torch.abs(curr_min), big, rtol=0.05)) or torch.any(
-        torch.isclose(torch.abs(curr_max), big, rtol=0.05)
-    ):
+    finite = torch.all(torch.isfinite(curr_min)) & torch.all(torch.isfinite(curr_max))
+    extreme = torch.any(torch.isclose(torch.abs(curr_min), big, rtol=0.05)) | torch.any(
+        torch.isclose(torch.abs(curr_max), big, rtol=0.05))
+    finite, extreme = torch.stack([finite, extreme]).tolist()  # both answers in one device-to-host read
+    if not finite:
+        warnings.warn("Infinite or NaN values detected within input! This may skew the associated encodings")
+    if extreme:
         warnings.warn("Extreme values detected within input! This may skew the associated encodings")
 
 

@@ -471,12 +471,151 @@ def run_dlq_workload(steps, warmup, dev, with_cpu_baseline=True, batches=16, sha
     return out
 
 
+def run_model_workload(steps, warmup, dev, with_cpu_baseline=True, batches=8, seq=2048):
+    """c5: whole-model calibration (8 batches through compute_encodings) and one quantized forward of the random-init
+    bf16 Llama-style decoder; the GEMMs are PyTorch-ROCm's, the quantize-dequantize and min/max kernels are ours."""
+    import llama_harness as LH
+    from aimet_amd import nn as qnn
+    from aimet_amd.quantization.affine import QuantizeDequantize
+    from oracle import torch_ref as O
+
+    _ensure_built()
+    _copy_reference(dev)
+    cfg = LH.LlamaConfig()
+    model = LH.build(cfg, dev, seed=0)
+    nlin = LH.quantize(model)
+    ids = LH.calibration_batches(cfg, dev, batches=batches, seq=seq)
+
+    def calibrate():
+        with torch.no_grad(), qnn.compute_encodings(model):
+            for b in ids:
+                model(b)
+
+    def forward():
+        with torch.no_grad():
+            return model(ids[0])
+
+    def step():
+        calibrate()
+        return forward()
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) / steps
+
+    def timed(fn, reps):
+        fn()
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        for _ in range(reps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t) / reps
+
+    t_cal = timed(calibrate, 2)
+    t_fwd = timed(forward, 3)
+    plain = LH.build(cfg, dev, seed=0)
+    t_plain = timed(lambda: torch.no_grad()(plain)(ids[0]), 3)
+    del plain
+
+    # elements that pass through our kernels per step
+    tokens = seq
+    wel = LH.weight_elements(cfg)
+    act_in = cfg.layers * (4 * cfg.hidden + 2 * cfg.hidden + cfg.ffn) * tokens + cfg.hidden * tokens
+    act_out = cfg.layers * (4 * cfg.hidden + 2 * cfg.ffn + cfg.hidden) * tokens + cfg.vocab * tokens
+    act = act_in + act_out
+    S = 2
+    # calibration: weights min/max once + QDQ per batch; activations min/max once per batch
+    bytes_cal = wel * S + batches * (wel * 2 * S + act * S)
+    bytes_fwd = wel * 2 * S + act * 2 * S
+    bytes_step = bytes_cal + bytes_fwd
+    elems_step = wel * (1 + batches + 1) + act * (batches + 1)
+
+    # parity: three quantizers of different kinds against the oracle on the tensors they see in one forward
+    io = {}
+    names = ["blocks.0.attn.q_proj.input_quantizers.0", "blocks.0.mlp.down_proj.param_quantizers.weight",
+             "blocks.15.mlp.down_proj.output_quantizers.0"]
+    mods = dict(model.named_modules())
+    hooks = [mods[n].register_forward_hook(lambda m, a, o, k=n: io.__setitem__(k, (a[0].detach().cpu(), o.detach().cpu())))
+             for n in names]
+    forward()
+    for h in hooks:
+        h.remove()
+    parity = {}
+    for n in names:
+        q = mods[n]
+        x, y = io[n]
+        sc, off = q.get_scale().detach().cpu(), q.get_offset().detach().cpu()
+        ref = (O.qdq_v1(x, sc, off, q.qmin, q.qmax)[0] if q.block_size is None
+               else O.qdq_v2_forward(x, sc, off, q.qmin, q.qmax, q.block_size).y)
+        parity[n.split(".")[-3] + "." + n.split(".")[-2]] = bool(
+            torch.equal(y.as_subclass(torch.Tensor).view(torch.int16), ref.view(torch.int16)))
+    wq = mods[names[1]]
+    w = mods["blocks.0.mlp.down_proj"].weight.detach().cpu()
+    mn, mx = O.reduce_minmax(w, tuple(wq.shape), wq.block_size)
+    lo, hi = O.minmax_encodings(mn, mx, wq.qmax - wq.qmin, True)
+    parity["weight_encodings_bit_exact"] = bool(torch.equal(wq.min.detach().cpu(), lo.view(wq.shape).float())
+                                                and torch.equal(wq.max.detach().cpu(), hi.view(wq.shape).float()))
+
+    out = {
+        "metric": "QDQ fwd+bwd GB/s (% of HBM peak); calibration elems/s; vs host-CPU ref",
+        "value": round(bytes_step / wall / 1e9, 2),
+        "unit": "GB/s",
+        "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": round(wall * 1e3, 3),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "c5_llama16x2048_ffn8192_w4b64_a16_calib8x2048_plus_forward", "linear_layers": nlin,
+                   "weight_elements": wel, "activation_elements_per_forward": act,
+                   "algorithmic_bytes_per_step": bytes_step, "quantizer_elements_per_step": elems_step},
+        "pct_of_hbm_peak": round(100.0 * bytes_step / wall / 1e9 / HBM_PEAK_GBS, 2),
+        "elements_per_s": round(elems_step / wall, 1),
+        "phases": {"calibration_8_batches_ms": round(t_cal * 1e3, 2), "quantized_forward_ms": round(t_fwd * 1e3, 2),
+                   "unquantized_forward_ms": round(t_plain * 1e3, 2),
+                   "linear_tflops_unquantized": round(LH.linear_flops(cfg, tokens) / t_plain / 1e12, 1)},
+        "parity": parity,
+        "roofline": {"bound": "hbm", "kernel": "qdq_fwd_kernel (weights) inside the quantized forward",
+                     "achieved": round(bytes_fwd / t_fwd / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(bytes_fwd / t_fwd / 1e9 / HBM_PEAK_GBS, 4), "algorithmic_bytes": bytes_fwd,
+                     "traffic": None,
+                     "note": "whole forward including PyTorch GEMMs and attention; the per-kernel figure is in profiles/"},
+    }
+    if with_cpu_baseline:
+        # the reference's CPU path for the same quantizers on a bounded sample: one weight and one activation tensor
+        w = mods["blocks.0.mlp.down_proj"].weight.detach().cpu()
+        wq = mods[names[1]]
+        sc, off = wq.get_scale().detach().cpu(), wq.get_offset().detach().cpu()
+        x, _ = io[names[2]]
+        aq = mods[names[2]]
+        asc, aoff = aq.get_scale().detach().cpu(), aq.get_offset().detach().cpu()
+        reps = 0
+        t0 = time.perf_counter()
+        while time.perf_counter() - t0 < 10.0:
+            O.reduce_minmax(w, tuple(wq.shape), wq.block_size)
+            O.qdq_v2_forward(w, sc, off, wq.qmin, wq.qmax, wq.block_size)
+            O.reduce_minmax(x, ())
+            O.qdq_v1(x, asc, aoff, aq.qmin, aq.qmax)
+            reps += 1
+        dt = (time.perf_counter() - t0) / reps
+        el = 2 * w.numel() + 2 * x.numel()
+        out["cpu_baseline"] = {"value": round(el / dt * (bytes_step / elems_step) / 1e9, 3), "unit": "GB/s",
+                               "cores": torch.get_num_threads(), "kind": "port",
+                               "sample": "min/max + quantize-dequantize of one 2048x8192 bf16 weight (block 64, 4 bit) and "
+                                         "one 2048x2048 bf16 activation (16 bit) with the reference's torch CPU calls, "
+                                         f"{reps} repetitions; quantizer work only, no GEMMs",
+                               "elements_per_s": round(el / dt, 1)}
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["c3", "dlq"])
+    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["c3", "c5", "dlq"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -489,6 +628,8 @@ def main():
     dev = torch.device("cuda:0")
     if args.workload == "c3":
         out = run_hist_workload(min(args.steps, 10), min(args.warmup, 2), dev, with_cpu_baseline=not args.no_cpu_baseline)
+    elif args.workload == "c5":
+        out = run_model_workload(min(args.steps, 3), min(args.warmup, 1), dev, with_cpu_baseline=not args.no_cpu_baseline)
     elif args.workload == "dlq":
         out = run_dlq_workload(min(args.steps, 10), min(args.warmup, 2), dev, with_cpu_baseline=not args.no_cpu_baseline)
     else:
