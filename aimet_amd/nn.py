@@ -29,9 +29,10 @@ from aimet_amd.quantization.base.quantizer import QuantizerBase
 __all__ = ["QuantizedLinear", "compute_encodings", "quantized_linears"]
 
 
-def _may_be_prequantized(param: torch.Tensor, qtzr: AffineQuantizerBase) -> bool:
+def _may_be_prequantized(param: torch.Tensor, qtzr: AffineQuantizerBase):
     """The early exit of _decompose_prequantized_tensor (aimet_torch/utils.py:2098-2118): the first 64 blocks, first
-    2 * num_levels elements each; more distinct magnitudes than grid levels means the tensor is not on a grid."""
+    2 * num_levels elements each; more distinct magnitudes than grid levels means the tensor is not on a grid.
+    Returns True, or a 0-dim bool tensor on the parameter's device (not yet read back)."""
     num_levels = max(abs(qtzr.qmax), abs(qtzr.qmin)) + 1
     shape = tuple(qtzr.shape)
     block = concretize_block_size(tuple(param.shape), shape, qtzr.block_size or tuple(-1 for _ in shape))
@@ -47,7 +48,7 @@ def _may_be_prequantized(param: torch.Tensor, qtzr: AffineQuantizerBase) -> bool
         return True
     xs = x[:64, : num_levels * 2].float().abs().sort(dim=1).values
     distinct = (xs[:, 1:] != xs[:, :-1]).sum(dim=1) + 1
-    return not bool(torch.any(distinct > num_levels))
+    return ~torch.any(distinct > num_levels)
 
 
 class QuantizedLinear(nn.Linear):
@@ -88,31 +89,46 @@ class QuantizedLinear(nn.Linear):
             out = oq(out)
         return out
 
-    def _compute_param_encodings(self, overwrite: bool):
-        """nn/base.py:331-383"""
+    def _params_to_calibrate(self, overwrite: bool):
         for name, qtzr in self.param_quantizers.items():
             if qtzr is None or not qtzr.is_overwrite_allowed():
                 continue
             if qtzr.is_initialized() and not overwrite:
                 continue
             param = getattr(self, name)
-            if param is None:
-                continue
+            if param is not None:
+                yield name, qtzr, param
+
+    def _prequantized_verdicts(self, overwrite: bool):
+        """name -> True / device flag for the parameters whose grid the reference would first try to recover."""
+        out = {}
+        for name, qtzr, param in self._params_to_calibrate(overwrite):
             if (isinstance(qtzr, AffineQuantizerBase) and not isinstance(qtzr, GroupedBlockQuantizeDequantize)
                     and qtzr.symmetric and math.ceil((qtzr.qmin + qtzr.qmax) / 2) == 0):
-                if _may_be_prequantized(param.detach(), qtzr):
-                    raise NotImplementedError(
-                        f"parameter '{name}' looks like an already-quantized tensor; recovering its grid "
-                        "(lossless decomposition) is not implemented here"
-                    )
+                out[name] = _may_be_prequantized(param.detach(), qtzr)
+        return out
+
+    def _compute_param_encodings(self, overwrite: bool, verdicts=None):
+        """nn/base.py:331-383.  ``verdicts``: already read-back results of _prequantized_verdicts()."""
+        todo = list(self._params_to_calibrate(overwrite))
+        if not todo:
+            return
+        if verdicts is None:
+            verdicts = {k: bool(v) for k, v in self._prequantized_verdicts(overwrite).items()}
+        for name, qtzr, param in todo:
+            if verdicts.get(name, False):
+                raise NotImplementedError(
+                    f"parameter '{name}' looks like an already-quantized tensor; recovering its grid "
+                    "(lossless decomposition) is not implemented here"
+                )
             with qtzr._compute_encodings(passthrough=True):  # pylint: disable=protected-access
                 _ = qtzr(param)
 
     @contextlib.contextmanager
-    def compute_encodings(self):
+    def compute_encodings(self, _verdicts=None):
         """nn/base.py:392-427: weights are calibrated on entry; activation quantizers observe their inputs and pass
         them through unquantized, and set their ranges on exit."""
-        self._compute_param_encodings(overwrite=True)
+        self._compute_param_encodings(overwrite=True, verdicts=_verdicts)
         with contextlib.ExitStack() as stack:
             for qtzr in list(self.input_quantizers) + list(self.output_quantizers):
                 if not isinstance(qtzr, QuantizerBase) or not qtzr.is_overwrite_allowed():
@@ -128,9 +144,18 @@ def quantized_linears(model: nn.Module) -> Iterable[QuantizedLinear]:
 @contextlib.contextmanager
 def compute_encodings(model: nn.Module):
     """aimet_torch.nn.compute_encodings (nn/base.py): the compute_encodings context of every quantized module."""
-    with contextlib.ExitStack() as stack:
-        for m in quantized_linears(model):
-            stack.enter_context(m.compute_encodings())
+    from aimet_amd.quantization.encoding_analyzer import deferred_range_warnings
+
+    modules = list(quantized_linears(model))
+    # the "is this weight already quantized" tests of all layers are evaluated on the device and read back together
+    pending = [(m, m._prequantized_verdicts(True)) for m in modules]  # pylint: disable=protected-access
+    flags = [v for _, d in pending for v in d.values() if isinstance(v, torch.Tensor)]
+    answers = iter(torch.stack(flags).tolist()) if flags else iter(())
+    verdicts = {id(m): {k: (next(answers) if isinstance(v, torch.Tensor) else bool(v)) for k, v in d.items()}
+                for m, d in pending}
+    with deferred_range_warnings(), contextlib.ExitStack() as stack:
+        for m in modules:
+            stack.enter_context(m.compute_encodings(_verdicts=verdicts[id(m)]))
         yield
 
 

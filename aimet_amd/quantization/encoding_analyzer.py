@@ -13,6 +13,7 @@ device, where each operation is a single IEEE operation and therefore reproduces
 from __future__ import annotations
 
 import math
+import contextlib
 import warnings
 from abc import ABC, abstractmethod
 from dataclasses import dataclass
@@ -285,17 +286,50 @@ class MinMaxEncodingAnalyzer(EncodingAnalyzer[_MinMaxRange]):
         return lo, hi
 
 
-def _flag_extreme_min_max(curr_min, curr_max):
-    """Warn about non-finite or near-overflow encodings (reference: encoding_analyzer.py:484-498)."""
-    big = torch.full_like(curr_min, torch.finfo(curr_min.dtype).max)
-    finite = torch.all(torch.isfinite(curr_min)) & torch.all(torch.isfinite(curr_max))
-    extreme = torch.any(torch.isclose(torch.abs(curr_min), big, rtol=0.05)) | torch.any(
-        torch.isclose(torch.abs(curr_max), big, rtol=0.05))
-    finite, extreme = torch.stack([finite, extreme]).tolist()  # both answers in one device-to-host read
-    if not finite:
+_deferred_range_flags = None  # list of device flag pairs while deferred_range_warnings() is active
+
+
+@contextlib.contextmanager
+def deferred_range_warnings():
+    """Inside this context the non-finite / near-overflow checks of every quantizer are gathered on the device and
+    read back once on exit, instead of one host synchronisation per quantizer (a whole-model calibration ends
+    hundreds of quantizer contexts at once).  The same warnings are issued, at the end."""
+    global _deferred_range_flags  # pylint: disable=global-statement
+    if _deferred_range_flags is not None:
+        yield
+        return
+    _deferred_range_flags = []
+    try:
+        yield
+    finally:
+        flags, _deferred_range_flags = _deferred_range_flags, None
+        if flags:
+            by_device = {}
+            for f in flags:
+                by_device.setdefault(f.device, []).append(f)
+            for group in by_device.values():
+                _warn_range_flags(*torch.stack(group).any(dim=0).tolist())
+
+
+def _warn_range_flags(nonfinite: bool, extreme: bool):
+    if nonfinite:
         warnings.warn("Infinite or NaN values detected within input! This may skew the associated encodings")
     if extreme:
         warnings.warn("Extreme values detected within input! This may skew the associated encodings")
+
+
+def _flag_extreme_min_max(curr_min, curr_max):
+    """Warn about non-finite or near-overflow encodings (reference: encoding_analyzer.py:484-498)."""
+    big = torch.finfo(curr_min.dtype).max
+    both = torch.stack([curr_min.reshape(-1), curr_max.reshape(-1)]).abs()
+    nonfinite = ~torch.isfinite(both).all()
+    # torch.isclose(|x|, big, rtol=0.05) with its default atol of 1e-8: | |x| - big | <= 1e-8 + 0.05 * big
+    extreme = ((both - big).abs() <= 1e-8 + 0.05 * big).any()
+    flags = torch.stack([nonfinite, extreme])
+    if _deferred_range_flags is not None:
+        _deferred_range_flags.append(flags)
+        return
+    _warn_range_flags(*flags.tolist())  # both answers in one device-to-host read
 
 
 def adjust_min_max(curr_min, curr_max, num_steps, is_symmetric):
