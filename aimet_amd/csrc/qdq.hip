@@ -28,36 +28,69 @@ struct GridC {
 
 struct EncP {
     float p0, p1, p2, p3;
+    float rs;  // 1 / scale correctly rounded, or 0 when the division-free path must not be used for this encoding
 };
+
+// x / s, correctly rounded.  FAST: two residual corrections of x * (1/s) with fused multiply-adds.  With rs = RN(1/s)
+// the first correction leaves a quotient that is off by at most a few 2^-47 relative, and the second is then the
+// correctly rounded one (Markstein's division theorem); the residuals are exact as long as nothing under- or
+// overflows, which the callers guarantee by taking this path only for |x| <= 2^60 and 2^-60 <= |s| <= 2^60 (a
+// quotient below 2^-120 cannot arise there, and one too small to matter rounds to code 0 either way).  Five
+// instructions instead of the thirteen of the general IEEE sequence, whose divisor scaling, reciprocal refinement and
+// fix-up are work per element that does not depend on the element.
+template <bool FAST>
+__device__ __forceinline__ float divide(float x, float s, float rs) {
+    if (!FAST) return x / s;
+    const float q0 = x * rs;
+    const float r0 = __builtin_fmaf(-q0, s, x);
+    const float q1 = __builtin_fmaf(r0, rs, q0);
+    const float r1 = __builtin_fmaf(-q1, s, x);
+    return __builtin_fmaf(r1, rs, q1);
+}
+
+constexpr float kFastDivMax = 1.152921504606846976e18f;     // 2^60
+constexpr float kFastDivMin = 8.673617379884035472e-19f;    // 2^-60
+
+__device__ __forceinline__ float safe_reciprocal(float s) {
+    const float m = __builtin_fabsf(s);
+    return (m >= kFastDivMin && m <= kFastDivMax) ? 1.0f / s : 0.f;
+}
 
 // --------------------------------------------------------------------------------------------------- arithmetic --
 // Each Math type: kNP staged floats per encoding; prep() turns (scale, offset, min, max) into them; fwd() returns the
 // output value (already rounded to the compute dtype) and whether the code was in range; bwd() returns the three
 // per-element gradient terms.
 
-template <int CD>
+template <int CD, bool ZPS>
 struct MathAutogradQdq {
     static constexpr int kNP = 2;
+    static constexpr bool kDiv = true;
     static constexpr bool kHasBwd = true;
-    __device__ static EncP prep(float s, float off, float, float, const GridC&) { return {rnd<CD>(s), rnd<CD>(off), 0.f, 0.f}; }
+    __device__ static EncP prep(float s, float off, float, float, const GridC&) {
+        const float sr = rnd<CD>(s);
+        return {sr, rnd<CD>(off), 0.f, 0.f, safe_reciprocal(sr)};
+    }
+    template <bool FAST>
     __device__ static float fwd(float x, const EncP& e, const GridC& g, bool& inr) {
-        float t = rnd<CD>(x / e.p0);
-        if (g.zps != 0.f) t = rnd<CD>(t - g.zps);
+        float t = rnd<CD>(divide<FAST>(x, e.p0, e.rs));
+        if (ZPS) t = rnd<CD>(t - g.zps);
         const float r = rnd<CD>(__builtin_rintf(t) - e.p1);
         inr = (r >= g.qmin) & (r <= g.qmax);
         const float q = r < g.qmin ? g.qmin : (r > g.qmax ? g.qmax : r);
-        const float offp = g.zps != 0.f ? rnd<CD>(e.p1 + g.zps) : e.p1;
+        const float offp = ZPS ? rnd<CD>(e.p1 + g.zps) : e.p1;
         return rnd<CD>(rnd<CD>(q + offp) * e.p0);
     }
+    template <bool FAST>
     __device__ static void bwd(float gr, float x, const EncP& e, const GridC& g, float& gx, float& gs, float& goff) {
-        const float t = rnd<CD>(rnd<CD>(x / e.p0) - g.zps);
+        float t = rnd<CD>(divide<FAST>(x, e.p0, e.rs));
+        if (ZPS) t = rnd<CD>(t - g.zps);
         const float xr = __builtin_rintf(t);
         const float err = rnd<CD>(xr - t);
         const float r = rnd<CD>(xr - e.p1);
         const bool inr = (r >= g.qmin) & (r <= g.qmax);
         const float lo = rnd<CD>(e.p1 + g.qmin), hi = rnd<CD>(e.p1 + g.qmax);
         float xc = xr < lo ? lo : (xr > hi ? hi : xr);
-        if (g.zps != 0.f) xc = rnd<CD>(xc + g.zps);
+        if (ZPS) xc = rnd<CD>(xc + g.zps);
         gx = inr ? gr : 0.f;
         gs = rnd<CD>(gr * (inr ? err : xc));
         goff = inr ? 0.f : rnd<CD>(gr * e.p0);
@@ -67,19 +100,25 @@ struct MathAutogradQdq {
 template <int CD>
 struct MathAutogradQuantize {
     static constexpr int kNP = 2;
+    static constexpr bool kDiv = true;
     static constexpr bool kHasBwd = true;
-    __device__ static EncP prep(float s, float off, float, float, const GridC&) { return {rnd<CD>(s), rnd<CD>(off), 0.f, 0.f}; }
+    __device__ static EncP prep(float s, float off, float, float, const GridC&) {
+        const float sr = rnd<CD>(s);
+        return {sr, rnd<CD>(off), 0.f, 0.f, safe_reciprocal(sr)};
+    }
+    template <bool FAST>
     __device__ static float fwd(float x, const EncP& e, const GridC& g, bool& inr) {
-        const float r = rnd<CD>(__builtin_rintf(rnd<CD>(x / e.p0)) - e.p1);
+        const float r = rnd<CD>(__builtin_rintf(rnd<CD>(divide<FAST>(x, e.p0, e.rs))) - e.p1);
         inr = (r >= g.qmin) & (r <= g.qmax);
         return r < g.qmin ? g.qmin : (r > g.qmax ? g.qmax : r);
     }
+    template <bool FAST>
     __device__ static void bwd(float gr, float x, const EncP& e, const GridC& g, float& gx, float& gs, float& goff) {
-        const float xs = rnd<CD>(x / e.p0);
+        const float xs = rnd<CD>(divide<FAST>(x, e.p0, e.rs));
         const float r = rnd<CD>(__builtin_rintf(xs) - e.p1);
         const bool inr = (r >= g.qmin) & (r <= g.qmax);
         const float mg = rnd<CD>(gr * (inr ? 1.f : 0.f));
-        gx = rnd<CD>(mg / e.p0);
+        gx = rnd<CD>(mg / e.p0);  // the gradient's magnitude is not bounded like x: general division
         gs = rnd<CD>((-gx) * xs);
         goff = -mg;
     }
@@ -88,12 +127,15 @@ struct MathAutogradQuantize {
 template <int CD>
 struct MathAutogradDequantize {
     static constexpr int kNP = 2;
+    static constexpr bool kDiv = false;
     static constexpr bool kHasBwd = true;
-    __device__ static EncP prep(float s, float off, float, float, const GridC&) { return {rnd<CD>(s), rnd<CD>(off), 0.f, 0.f}; }
+    __device__ static EncP prep(float s, float off, float, float, const GridC&) { return {rnd<CD>(s), rnd<CD>(off), 0.f, 0.f, 0.f}; }
+    template <bool FAST>
     __device__ static float fwd(float x, const EncP& e, const GridC&, bool& inr) {
         inr = true;
         return rnd<CD>(rnd<CD>(x + e.p1) * e.p0);
     }
+    template <bool FAST>
     __device__ static void bwd(float gr, float x, const EncP& e, const GridC&, float& gx, float& gs, float& goff) {
         gx = rnd<CD>(gr * e.p0);
         gs = rnd<CD>(gr * rnd<CD>(x + e.p1));
@@ -103,15 +145,18 @@ struct MathAutogradDequantize {
 
 struct MathAten {
     static constexpr int kNP = 3;
+    static constexpr bool kDiv = false;
     static constexpr bool kHasBwd = true;
     // p0 = scale, p1 = zero point as float, p2 = 1.0f/scale
-    __device__ static EncP prep(float s, float off, float, float, const GridC&) { return {s, (float)(-(int)off), 1.0f / s, 0.f}; }
+    __device__ static EncP prep(float s, float off, float, float, const GridC&) { return {s, (float)(-(int)off), 1.0f / s, 0.f, 0.f}; }
+    template <bool FAST>
     __device__ static float fwd(float x, const EncP& e, const GridC& g, bool& inr) {
         const float q = __builtin_rintf(x * e.p2) + e.p1;
         inr = (q >= g.qmin) & (q <= g.qmax);
         const float qc = fminf(fmaxf(q, g.qmin), g.qmax);
         return (qc - e.p1) * e.p0;
     }
+    template <bool FAST>
     __device__ static void bwd(float gr, float x, const EncP& e, const GridC& g, float& gx, float& gs, float& goff) {
         const float q = __builtin_rintf(x * e.p2) + e.p1;
         const bool inr = (q >= g.qmin) & (q <= g.qmax);
@@ -123,17 +168,24 @@ struct MathAten {
 
 struct MathDlq {
     static constexpr int kNP = 4;
+    static constexpr bool kDiv = true;
     static constexpr bool kHasBwd = false;
-    // p0 = delta, p1 = offset, p2 = min, p3 = max
-    __device__ static EncP prep(float s, float off, float mn, float mx, const GridC&) { return {s, off, mn, mx}; }
+    // p0 = delta, p1 = offset, p2 = min, p3 = max.  The value is clamped to [min, max] before it is divided, so the
+    // division-free path only needs the encoding itself to be in range.
+    __device__ static EncP prep(float s, float off, float mn, float mx, const GridC&) {
+        const bool bounded = __builtin_fabsf(mn) <= kFastDivMax && __builtin_fabsf(mx) <= kFastDivMax;
+        return {s, off, mn, mx, bounded ? safe_reciprocal(s) : 0.f};
+    }
+    template <bool FAST>
     __device__ static float fwd(float x, const EncP& e, const GridC&, bool& inr) {
         inr = true;
         float v = (x != x) ? e.p2 : x;
         v = fmaxf(fminf(v, e.p3), e.p2);
-        v = v / e.p0 - e.p1;
+        v = divide<FAST>(v, e.p0, e.rs) - e.p1;
         v = roundf(v);
         return e.p0 * (v + e.p1);
     }
+    template <bool FAST>
     __device__ static void bwd(float, float, const EncP&, const GridC&, float& gx, float& gs, float& goff) { gx = gs = goff = 0.f; }
 };
 
@@ -170,6 +222,7 @@ __device__ __forceinline__ void stage_encodings(const QdqArgs& a, const Tile& t,
         sp[1][i] = p.p1;
         if (M::kNP > 2) sp[2][i] = p.p2;
         if (M::kNP > 3) sp[3][i] = p.p3;
+        if (M::kDiv) sp[M::kNP][i] = p.rs;
     }
 }
 
@@ -180,6 +233,7 @@ __device__ __forceinline__ EncP staged(float (*sp)[kStage], int i) {
     e.p1 = sp[1][i];
     e.p2 = M::kNP > 2 ? sp[2][i] : 0.f;
     e.p3 = M::kNP > 3 ? sp[3][i] : 0.f;
+    e.rs = M::kDiv ? sp[M::kNP][i] : 0.f;
     return e;
 }
 
@@ -189,6 +243,48 @@ __device__ __forceinline__ EncP load_enc(const QdqArgs& a, int64_t e) {
 }
 
 // -------------------------------------------------------------------------------------------------------- forward --
+// FULL: every lane of the tile has work, so loads and stores carry no per-lane bounds checks (all tiles but the last).
+// True when every element and encoding this lane handles allows the division-free path (see divide()).
+template <typename IO, int VEC, typename M, bool FULL>
+__device__ __forceinline__ bool lane_can_divide_fast(const QdqArgs& a, const Tile& t, float (*sp)[kStage],
+                                                     const Pack<IO, VEC>* in) {
+    if (!M::kDiv) return true;
+    bool ok = true;
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+        const int lv = u * kBlock + threadIdx.x;
+        if (FULL || lv < t.nv) {
+            ok &= sp[M::kNP][stage_index(a, t, lv)] != 0.f;
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) ok &= !(__builtin_fabsf(load_f32(in[u].v[k])) > kFastDivMax);
+        }
+    }
+    return ok;
+}
+
+template <typename IO, int VEC, typename M, bool FULL, bool FAST>
+__device__ __forceinline__ void fwd_math(const QdqArgs& a, const Tile& t, float (*sp)[kStage], const Pack<IO, VEC>* in,
+                                         IO* __restrict__ y, uint8_t* __restrict__ mask) {
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+        const int lv = u * kBlock + threadIdx.x;
+        if (FULL || lv < t.nv) {
+            const EncP e = staged<M>(sp, stage_index(a, t, lv));
+            Pack<IO, VEC> out;
+            Pack<uint8_t, VEC> mk;
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) {
+                bool inr;
+                const float r = M::template fwd<FAST>(load_f32(in[u].v[k]), e, a.gc, inr);
+                out.v[k] = store_cast<IO>(r);
+                mk.v[k] = inr ? 1 : 0;
+            }
+            store_pack<IO, VEC>(y + (int64_t)lv * VEC, out);
+            if (mask) store_pack<uint8_t, VEC>(mask + (int64_t)lv * VEC, mk);
+        }
+    }
+}
+
 // FULL: every lane of the tile has work, so loads and stores carry no per-lane bounds checks (all tiles but the last).
 template <typename IO, int VEC, typename M, bool FULL>
 __device__ __forceinline__ void fwd_tile(const QdqArgs& a, const Tile& t, float (*sp)[kStage]) {
@@ -201,29 +297,16 @@ __device__ __forceinline__ void fwd_tile(const QdqArgs& a, const Tile& t, float 
         const int lv = u * kBlock + threadIdx.x;
         if (FULL || lv < t.nv) in[u] = load_pack<IO, VEC>(x + (int64_t)lv * VEC);
     }
-#pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
-        const int lv = u * kBlock + threadIdx.x;
-        if (FULL || lv < t.nv) {
-            const EncP e = staged<M>(sp, stage_index(a, t, lv));
-            Pack<IO, VEC> out;
-            Pack<uint8_t, VEC> mk;
-#pragma unroll
-            for (int k = 0; k < VEC; ++k) {
-                bool inr;
-                const float r = M::fwd(load_f32(in[u].v[k]), e, a.gc, inr);
-                out.v[k] = store_cast<IO>(r);
-                mk.v[k] = inr ? 1 : 0;
-            }
-            store_pack<IO, VEC>(y + (int64_t)lv * VEC, out);
-            if (mask) store_pack<uint8_t, VEC>(mask + (int64_t)lv * VEC, mk);
-        }
-    }
+    // one wave-uniform choice per tile: huge or infinite inputs and out-of-range scales take the general division
+    if (!M::kDiv || __builtin_amdgcn_ballot_w64(!lane_can_divide_fast<IO, VEC, M, FULL>(a, t, sp, in)) == 0)
+        fwd_math<IO, VEC, M, FULL, true>(a, t, sp, in, y, mask);
+    else
+        fwd_math<IO, VEC, M, FULL, false>(a, t, sp, in, y, mask);
 }
 
 template <typename IO, int VEC, typename M>
 __global__ __launch_bounds__(kBlock) void qdq_fwd_kernel(const QdqArgs a) {
-    __shared__ float sp[M::kNP][kStage];
+    __shared__ float sp[M::kNP + (M::kDiv ? 1 : 0)][kStage];
     const Tile t = make_tile(a, blockIdx.x);
     stage_encodings<M>(a, t, sp);
     __syncthreads();
@@ -237,7 +320,7 @@ __global__ __launch_bounds__(kBlock) void qdq_fwd_kernel(const QdqArgs a) {
             IO* y = static_cast<IO*>(a.y);
             const EncP e = staged<M>(sp, 0);
             bool inr;
-            const float r = M::fwd(load_f32(x[i]), e, a.gc, inr);
+            const float r = M::template fwd<false>(load_f32(x[i]), e, a.gc, inr);
             y[i] = store_cast<IO>(r);
             if (a.mask) a.mask[i] = inr ? 1 : 0;
         }
@@ -251,7 +334,7 @@ __global__ __launch_bounds__(kBlock) void qdq_fwd_generic_kernel(const QdqArgs a
     for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < a.numel; i += (int64_t)gridDim.x * kBlock) {
         const EncP e = load_enc<M>(a, generic_enc_index(a, i));
         bool inr;
-        const float r = M::fwd(load_f32(x[i]), e, a.gc, inr);
+        const float r = M::template fwd<false>(load_f32(x[i]), e, a.gc, inr);
         y[i] = store_cast<IO>(r);
         if (a.mask) a.mask[i] = inr ? 1 : 0;
     }
@@ -264,20 +347,9 @@ __device__ __forceinline__ float finish_sum_rt(double s, int cd) {
     return (float)s;
 }
 
-template <typename IO, int VEC, typename M, int RED, bool FULL>
-__device__ __forceinline__ void bwd_tile(const QdqArgs& a, const Tile& t, float (*sp)[kStage], double& acc_s, double& acc_o) {
-    const IO* __restrict__ x = static_cast<const IO*>(a.x) + t.v0 * VEC;
-    const IO* __restrict__ g = static_cast<const IO*>(a.g) + t.v0 * VEC;
-    IO* __restrict__ gxp = a.gx ? static_cast<IO*>(a.gx) + t.v0 * VEC : nullptr;
-    Pack<IO, VEC> xin[kUnroll], gin[kUnroll];
-#pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
-        const int lv = u * kBlock + threadIdx.x;
-        if (FULL || lv < t.nv) {
-            xin[u] = load_pack<IO, VEC>(x + (int64_t)lv * VEC);
-            gin[u] = load_pack<IO, VEC>(g + (int64_t)lv * VEC);
-        }
-    }
+template <typename IO, int VEC, typename M, int RED, bool FULL, bool FAST>
+__device__ __forceinline__ void bwd_math(const QdqArgs& a, const Tile& t, float (*sp)[kStage], const Pack<IO, VEC>* xin,
+                                         const Pack<IO, VEC>* gin, IO* __restrict__ gxp, double& acc_s, double& acc_o) {
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
         const int lv = u * kBlock + threadIdx.x;
@@ -290,7 +362,7 @@ __device__ __forceinline__ void bwd_tile(const QdqArgs& a, const Tile& t, float 
 #pragma unroll
             for (int k = 0; k < VEC; ++k) {
                 float gx, gs, go;
-                M::bwd(load_f32(gin[u].v[k]), load_f32(xin[u].v[k]), e, a.gc, gx, gs, go);
+                M::template bwd<FAST>(load_f32(gin[u].v[k]), load_f32(xin[u].v[k]), e, a.gc, gx, gs, go);
                 out.v[k] = store_cast<IO>(gx);
                 vs += gs;
                 vo += go;
@@ -324,9 +396,29 @@ __device__ __forceinline__ void bwd_tile(const QdqArgs& a, const Tile& t, float 
     }
 }
 
+template <typename IO, int VEC, typename M, int RED, bool FULL>
+__device__ __forceinline__ void bwd_tile(const QdqArgs& a, const Tile& t, float (*sp)[kStage], double& acc_s, double& acc_o) {
+    const IO* __restrict__ x = static_cast<const IO*>(a.x) + t.v0 * VEC;
+    const IO* __restrict__ g = static_cast<const IO*>(a.g) + t.v0 * VEC;
+    IO* __restrict__ gxp = a.gx ? static_cast<IO*>(a.gx) + t.v0 * VEC : nullptr;
+    Pack<IO, VEC> xin[kUnroll], gin[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+        const int lv = u * kBlock + threadIdx.x;
+        if (FULL || lv < t.nv) {
+            xin[u] = load_pack<IO, VEC>(x + (int64_t)lv * VEC);
+            gin[u] = load_pack<IO, VEC>(g + (int64_t)lv * VEC);
+        }
+    }
+    if (!M::kDiv || __builtin_amdgcn_ballot_w64(!lane_can_divide_fast<IO, VEC, M, FULL>(a, t, sp, xin)) == 0)
+        bwd_math<IO, VEC, M, RED, FULL, true>(a, t, sp, xin, gin, gxp, acc_s, acc_o);
+    else
+        bwd_math<IO, VEC, M, RED, FULL, false>(a, t, sp, xin, gin, gxp, acc_s, acc_o);
+}
+
 template <typename IO, int VEC, typename M, int RED>
 __global__ __launch_bounds__(kBlock) void qdq_bwd_kernel(const QdqArgs a) {
-    __shared__ float sp[M::kNP][kStage];
+    __shared__ float sp[M::kNP + (M::kDiv ? 1 : 0)][kStage];
     __shared__ double red_smem[kBlock / kWave];
     const Tile t = make_tile(a, blockIdx.x);
     stage_encodings<M>(a, t, sp);
@@ -342,7 +434,7 @@ __global__ __launch_bounds__(kBlock) void qdq_bwd_kernel(const QdqArgs a) {
             IO* gxp = static_cast<IO*>(a.gx);
             const EncP e = staged<M>(sp, 0);
             float gx, gs, go;
-            M::bwd(load_f32(g[i]), load_f32(x[i]), e, a.gc, gx, gs, go);
+            M::template bwd<false>(load_f32(g[i]), load_f32(x[i]), e, a.gc, gx, gs, go);
             if (gxp) gxp[i] = store_cast<IO>(gx);
             if (RED == kRedTile) {
                 acc_s += (double)gs;
@@ -433,7 +525,7 @@ __global__ __launch_bounds__(kBlock) void qdq_bwd_generic_kernel(const QdqArgs a
         const int64_t ei = generic_enc_index(a, i);
         const EncP e = load_enc<M>(a, ei);
         float gx, gs, go;
-        M::bwd(load_f32(g[i]), load_f32(x[i]), e, a.gc, gx, gs, go);
+        M::template bwd<false>(load_f32(g[i]), load_f32(x[i]), e, a.gc, gx, gs, go);
         if (gxp) gxp[i] = store_cast<IO>(gx);
         if (a.partials) {
             atomicAdd(&a.partials[2 * ei], (double)gs);
@@ -527,9 +619,13 @@ static void launch_bwd(const Plan& p, const QdqArgs& a, hipStream_t st) {
         if ((grid).arith == AHQ_ARITH_ATEN) { using M = MathAten; CALL; }                            \
         else if ((grid).arith == AHQ_ARITH_DLQ) { using M = MathDlq; CALL; }                         \
         else if ((grid).op == AHQ_OP_QDQ) {                                                          \
-            if ((grid).compute_dtype == AHQ_F32) { using M = MathAutogradQdq<AHQ_F32>; CALL; }       \
-            else if ((grid).compute_dtype == AHQ_F16) { using M = MathAutogradQdq<AHQ_F16>; CALL; }  \
-            else { using M = MathAutogradQdq<AHQ_BF16>; CALL; }                                      \
+            if ((grid).zero_point_shift != 0.0) {                                                    \
+                if ((grid).compute_dtype == AHQ_F32) { using M = MathAutogradQdq<AHQ_F32, true>; CALL; }       \
+                else if ((grid).compute_dtype == AHQ_F16) { using M = MathAutogradQdq<AHQ_F16, true>; CALL; }  \
+                else { using M = MathAutogradQdq<AHQ_BF16, true>; CALL; }                            \
+            } else if ((grid).compute_dtype == AHQ_F32) { using M = MathAutogradQdq<AHQ_F32, false>; CALL; }   \
+            else if ((grid).compute_dtype == AHQ_F16) { using M = MathAutogradQdq<AHQ_F16, false>; CALL; }     \
+            else { using M = MathAutogradQdq<AHQ_BF16, false>; CALL; }                               \
         } else if ((grid).op == AHQ_OP_QUANTIZE) {                                                   \
             if ((grid).compute_dtype == AHQ_F32) { using M = MathAutogradQuantize<AHQ_F32>; CALL; }  \
             else if ((grid).compute_dtype == AHQ_F16) { using M = MathAutogradQuantize<AHQ_F16>; CALL; } \
