@@ -38,12 +38,18 @@ struct EncP {
 // quotient below 2^-120 cannot arise there, and one too small to matter rounds to code 0 either way).  Five
 // instructions instead of the thirteen of the general IEEE sequence, whose divisor scaling, reciprocal refinement and
 // fix-up are work per element that does not depend on the element.
-template <bool FAST>
+//
+// CD = the dtype the caller rounds the quotient to next.  For the 16-bit dtypes one correction is enough: x and s then
+// have p <= 11 significant bits, so an exact quotient that is not itself a rounding tie of that dtype lies at least
+// 2^-(2p+1) >= 2^-23 (relative) away from every tie, while the once-corrected quotient is exact whenever the true
+// quotient is a float (every tie is) and within 2^-24 otherwise: both round to the same 16-bit value.
+template <bool FAST, int CD>
 __device__ __forceinline__ float divide(float x, float s, float rs) {
     if (!FAST) return x / s;
     const float q0 = x * rs;
     const float r0 = __builtin_fmaf(-q0, s, x);
     const float q1 = __builtin_fmaf(r0, rs, q0);
+    if (CD != AHQ_F32) return q1;
     const float r1 = __builtin_fmaf(-q1, s, x);
     return __builtin_fmaf(r1, rs, q1);
 }
@@ -72,7 +78,7 @@ struct MathAutogradQdq {
     }
     template <bool FAST>
     __device__ static float fwd(float x, const EncP& e, const GridC& g, bool& inr) {
-        float t = rnd<CD>(divide<FAST>(x, e.p0, e.rs));
+        float t = rnd<CD>(divide<FAST, CD>(x, e.p0, e.rs));
         if (ZPS) t = rnd<CD>(t - g.zps);
         const float r = rnd<CD>(__builtin_rintf(t) - e.p1);
         inr = (r >= g.qmin) & (r <= g.qmax);
@@ -82,7 +88,7 @@ struct MathAutogradQdq {
     }
     template <bool FAST>
     __device__ static void bwd(float gr, float x, const EncP& e, const GridC& g, float& gx, float& gs, float& goff) {
-        float t = rnd<CD>(divide<FAST>(x, e.p0, e.rs));
+        float t = rnd<CD>(divide<FAST, CD>(x, e.p0, e.rs));
         if (ZPS) t = rnd<CD>(t - g.zps);
         const float xr = __builtin_rintf(t);
         const float err = rnd<CD>(xr - t);
@@ -108,13 +114,13 @@ struct MathAutogradQuantize {
     }
     template <bool FAST>
     __device__ static float fwd(float x, const EncP& e, const GridC& g, bool& inr) {
-        const float r = rnd<CD>(__builtin_rintf(rnd<CD>(divide<FAST>(x, e.p0, e.rs))) - e.p1);
+        const float r = rnd<CD>(__builtin_rintf(rnd<CD>(divide<FAST, CD>(x, e.p0, e.rs))) - e.p1);
         inr = (r >= g.qmin) & (r <= g.qmax);
         return r < g.qmin ? g.qmin : (r > g.qmax ? g.qmax : r);
     }
     template <bool FAST>
     __device__ static void bwd(float gr, float x, const EncP& e, const GridC& g, float& gx, float& gs, float& goff) {
-        const float xs = rnd<CD>(divide<FAST>(x, e.p0, e.rs));
+        const float xs = rnd<CD>(divide<FAST, CD>(x, e.p0, e.rs));
         const float r = rnd<CD>(__builtin_rintf(xs) - e.p1);
         const bool inr = (r >= g.qmin) & (r <= g.qmax);
         const float mg = rnd<CD>(gr * (inr ? 1.f : 0.f));
@@ -181,7 +187,7 @@ struct MathDlq {
         inr = true;
         float v = (x != x) ? e.p2 : x;
         v = fmaxf(fminf(v, e.p3), e.p2);
-        v = divide<FAST>(v, e.p0, e.rs) - e.p1;
+        v = divide<FAST, AHQ_F32>(v, e.p0, e.rs) - e.p1;
         v = roundf(v);
         return e.p0 * (v + e.p1);
     }

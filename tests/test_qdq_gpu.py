@@ -315,19 +315,22 @@ def test_division_free_quotients_are_correctly_rounded_fp32(device, op):
     assert_same_bits(got, ref)
 
 
-def test_division_free_quotients_bf16_exhaustive(device):
-    """Every finite bf16 value against a set of bf16 scales, in bf16 arithmetic (4-bit grid)."""
-    allv = torch.arange(-32768, 32768, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+@pytest.mark.parametrize("dtype,qmin,qmax", [(torch.bfloat16, -8, 7), (torch.float16, -128, 127), (torch.float16, 0, 15)])
+def test_division_free_quotients_16bit_exhaustive(device, dtype, qmin, qmax):
+    """Every finite 16-bit value against a set of scales of the same dtype, in that dtype's arithmetic."""
+    allv = torch.arange(-32768, 32768, dtype=torch.int32).to(torch.int16).view(dtype)
     allv = allv[torch.isfinite(allv.float())]
-    scales = _awkward_scales(256, 7).to(torch.bfloat16).float().reshape(-1, 1)
+    scales = _awkward_scales(256, 7)
+    if dtype == torch.float16:
+        scales = scales.clamp(6.2e-5, 6e4)
+    scales = scales.to(dtype).float().reshape(-1, 1)
     x = allv.reshape(1, -1).repeat(scales.shape[0], 1).contiguous()
     offset = torch.zeros_like(scales)
-    qmin, qmax = -8, 7
     from aimet_amd.quantization import affine
     sd = scales.to(device).requires_grad_(True)
     got = affine.quantize_dequantize(x.to(device), sd, offset.to(device), qmin, qmax).detach().cpu()
     ref = O.qdq_v2_forward(x, scales, offset, qmin, qmax).y
-    assert ref.dtype == torch.bfloat16
+    assert ref.dtype == dtype
     assert_same_bits(got, ref)
 
 
