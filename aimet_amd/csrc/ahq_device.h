@@ -57,6 +57,40 @@ __device__ __forceinline__ void store_pack(T* p, const Pack<T, N>& v) {
 }
 
 // ------------------------------------------------------------------------------------------- wave / block reduce --
+// ------------------------------------------------------------------------------------------ segment exchange --
+// Value of the lane whose index differs by XOR-ing `m` inside runs of `kv` lanes (kv a power of two, m < kv).
+// Inside a row of 16 lanes the exchange is a data-parallel-primitive move in the vector ALU (quad permutes for m = 1
+// and 2; for m = 4 and 8 the mirrored lane, which after the earlier steps holds the other half's partial result, so
+// these are only valid as steps of a full butterfly over operands that are symmetric within the halves already
+// combined); wider exchanges go through the LDS permute network.
+template <int CTRL>
+__device__ __forceinline__ int dpp_int(int v) {
+    return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xf, 0xf, false);
+}
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) { return __builtin_bit_cast(float, dpp_int<CTRL>(__builtin_bit_cast(int, v))); }
+template <int CTRL>
+__device__ __forceinline__ int dpp_move(int v) { return dpp_int<CTRL>(v); }
+template <int CTRL>
+__device__ __forceinline__ double dpp_move(double v) {
+    const long long b = __builtin_bit_cast(long long, v);
+    const int lo = dpp_int<CTRL>((int)(b & 0xffffffffll)), hi = dpp_int<CTRL>((int)(b >> 32));
+    return __builtin_bit_cast(double, ((long long)hi << 32) | (unsigned int)lo);
+}
+
+// All-lanes butterfly reduction over runs of kv lanes (kv a power of two <= 64, uniform across the wave), written as
+// straight-line steps so that each exchange is a compile-time DPP pattern.
+template <typename T, typename Op>
+__device__ __forceinline__ T segment_reduce(T v, int kv, Op op) {
+    if (kv > 1) v = op(v, dpp_move<0xB1>(v));   // quad_perm [1,0,3,2]
+    if (kv > 2) v = op(v, dpp_move<0x4E>(v));   // quad_perm [2,3,0,1]
+    if (kv > 4) v = op(v, dpp_move<0x141>(v));  // row_half_mirror: lane i <-> 7 - i of each 8
+    if (kv > 8) v = op(v, dpp_move<0x140>(v));  // row_mirror: lane i <-> 15 - i of each 16
+    if (kv > 16) v = op(v, __shfl_xor(v, 16, kWave));
+    if (kv > 32) v = op(v, __shfl_xor(v, 32, kWave));
+    return v;
+}
+
 template <typename T, typename Op>
 __device__ __forceinline__ T wave_reduce(T v, Op op) {
 #pragma unroll
@@ -78,6 +112,7 @@ __device__ __forceinline__ T block_reduce(T v, Op op, T* smem) {
     return r;
 }
 
+struct OpAddF { __device__ __forceinline__ float operator()(float a, float b) const { return a + b; } };
 struct OpAddD { __device__ __forceinline__ double operator()(double a, double b) const { return a + b; } };
 struct OpMinF { __device__ __forceinline__ float operator()(float a, float b) const { return fminf(a, b); } };
 struct OpMaxF { __device__ __forceinline__ float operator()(float a, float b) const { return fmaxf(a, b); } };

@@ -379,17 +379,15 @@ __device__ __forceinline__ void bwd_math(const QdqArgs& a, const Tile& t, float 
             acc_s += (double)vs;
             acc_o += (double)vo;
         } else if (RED == kRedSeg) {
-            // runs of Kv (power of two <= 64) neighbouring lanes share an encoding; runs never straddle a wave
-            double ds = (double)vs, dofs = (double)vo;
+            // runs of Kv (power of two <= 64) neighbouring lanes share an encoding; runs never straddle a wave.  At most
+            // 64 x VEC terms per encoding, so single precision (what the reference's own sum accumulates in) is enough
             const int kv = (int)a.Kv;
-            for (int m = 1; m < kv; m <<= 1) {
-                ds += __shfl_xor(ds, m, kWave);
-                dofs += __shfl_xor(dofs, m, kWave);
-            }
+            const float fs = segment_reduce(vs, kv, OpAddF());
+            const float fo = segment_reduce(vo, kv, OpAddF());
             if ((FULL || lv < t.nv) && (threadIdx.x & (kv - 1)) == 0) {
                 const int64_t e = t.e0 + si;
-                a.gscale[e] = finish_sum_rt(ds, a.out_cd);
-                a.goffset[e] = finish_sum_rt(dofs, a.out_cd);
+                a.gscale[e] = finish_sum_rt((double)fs, a.out_cd);
+                a.goffset[e] = finish_sum_rt((double)fo, a.out_cd);
             }
         } else if (RED == kRedAtomic) {
             if (FULL || lv < t.nv) {

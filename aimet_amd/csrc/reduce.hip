@@ -129,7 +129,9 @@ __device__ __forceinline__ void mm_tile(const MmArgs& a, const Tile& t, MinMax& 
             acc = mm_merge(acc, v);
         } else if (RED == kRedSeg) {
             const int kv = (int)a.Kv;
-            for (int m = 1; m < kv; m <<= 1) v = mm_merge(v, mm_shfl_xor(v, m));
+            v.mn = segment_reduce(v.mn, kv, OpMinF());
+            v.mx = segment_reduce(v.mx, kv, OpMaxF());
+            v.nan = segment_reduce(v.nan, kv, OpOrI());
             if ((FULL || lv < t.nv) && (threadIdx.x & (kv - 1)) == 0) mm_write<IO>(a, t.e0 + si, v);
         } else if (RED == kRedAtomic) {
             if (FULL || lv < t.nv) {
