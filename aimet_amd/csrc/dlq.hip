@@ -543,6 +543,64 @@ __global__ __launch_bounds__(kWave) void dlq_tfe_select_kernel(const TfeArgs a) 
     }
 }
 
+// --------------------------------------------------------------------------------------------------- percentile ---
+// PercentileEncodingAnalyzer::computeEncoding (PercentileEncodingAnalyzer.cpp:52-169).  One workgroup per slot; the
+// cumulative distribution is a sequential sum in the reference, so one lane forms it (1536 additions).
+__global__ __launch_bounds__(kWave) void dlq_percentile_kernel(const double* xleft, const double* pdfs, const int32_t* meta,
+                                                               float percentile, int bw, int symmetric, int strict,
+                                                               int unsigned_sym, double* outs) {
+    const int s = blockIdx.x;
+    const double* xl = xleft + (size_t)s * kPdf;
+    const double* pdf = pdfs + (size_t)s * kPdf;
+    double* out = outs + 5 * s;
+    __shared__ double cdf[kPdf];
+    if (threadIdx.x != 0) return;
+    float num_steps = (float)((double)(1ull << bw) - 1);
+    if (symmetric && strict) num_steps -= 1;
+    if (meta[4 * s + 1] == 0) {
+        if (meta[4 * s + 2]) {
+            double mn = -1, mx = 1;
+            const double delta = (mx - mn) / (int)num_steps;
+            const double offset = floor(mn / delta);
+            mn = offset * delta;
+            mx = mn + (int)num_steps * delta;
+            out[0] = mn; out[1] = mx; out[2] = delta; out[3] = offset; out[4] = bw;
+        } else {
+            out[0] = out[1] = out[2] = out[3] = out[4] = 0.0;
+        }
+        return;
+    }
+    // findOriginalRange (math_functions.cpp:401-435)
+    float lo = (float)xl[0], hi = (float)xl[kPdf - 1];
+    for (int i = 0; i < kPdf; ++i)
+        if (pdf[i] > 0) { lo = (float)xl[i]; break; }
+    for (int i = kPdf - 1; i > 0; --i)
+        if (pdf[i] > 0) { hi = (float)xl[i]; break; }
+    lo = std_min(lo, 0.0f);
+    hi = std_max(hi, 0.0f);
+    hi = std_max(hi, lo + (float)0.01);
+    float a_min = lo, a_max = hi;
+    if (percentile != 100.0f) {
+        const float bin_width = (float)(xl[1] - xl[0]);
+        float pmin = (float)xl[0];
+        float pmax = (float)(xl[kPdf - 1] + bin_width);
+        cdf[0] = pdf[0];
+        for (int i = 1; i < kPdf; ++i) cdf[i] = pdf[i] + cdf[i - 1];
+        const float left = 1 - percentile / 100;
+        for (int i = 0; i < kPdf; ++i)
+            if (cdf[i] >= left) { pmin = (float)xl[i]; break; }
+        const float right = percentile / 100;
+        for (int i = kPdf - 1; i >= 0; --i)
+            if (cdf[i] < right && xl[i] < hi) { pmax = (float)(xl[i] + bin_width); break; }
+        if (pmin == pmax) pmax += bin_width;
+        a_min = pmin;
+        a_max = pmax;
+    }
+    a_min = std_min(a_min, 0.f);
+    a_max = std_max(a_max, 0.f);
+    computed_encodings(bw, a_min, a_max, symmetric != 0, strict != 0, unsigned_sym != 0, 0.0, out);
+}
+
 // -------------------------------------------------------------------------------------------------- host side ---
 namespace {
 
@@ -774,4 +832,14 @@ extern "C" int ahq_dlq_tfe_encodings(const ahq_dlq_pdf_state* st, int32_t bw, in
     hipLaunchKernelGGL(dlq_tfe_cost_kernel, dim3(kMaxCand / kWave, st->num_slots), dim3(kWave), 0, s, a);
     hipLaunchKernelGGL(dlq_tfe_select_kernel, dim3(st->num_slots), dim3(kWave), 0, s, a);
     return check_launch("dlq_tfe_encodings");
+}
+
+extern "C" int ahq_dlq_percentile_encodings(const ahq_dlq_pdf_state* st, float percentile, int32_t bw, int32_t symmetric,
+                                            int32_t strict, int32_t unsigned_sym, double* out, void* stream) {
+    if (!check_pdf_state(st)) return AHQ_ERR_INVALID;
+    if (!out) return set_error("out is null"), AHQ_ERR_INVALID;
+    if (bw < 1 || bw > 31) return set_error("bitwidth must be in 1..31"), AHQ_ERR_INVALID;
+    hipLaunchKernelGGL(dlq_percentile_kernel, dim3(st->num_slots), dim3(kWave), 0, static_cast<hipStream_t>(stream),
+                       st->xleft, st->pdf, st->meta, percentile, bw, symmetric, strict, unsigned_sym, out);
+    return check_launch("dlq_percentile_encodings");
 }

@@ -19,6 +19,8 @@ from .quantization.affine.backends import hip as _hip
 
 QUANTIZATION_TF = 0           # DlQuantization::QuantizationMode (Quantization.hpp)
 QUANTIZATION_TF_ENHANCED = 1
+QUANTIZATION_PERCENTILE = 3
+_SCHEMES = (QUANTIZATION_TF, QUANTIZATION_TF_ENHANCED, QUANTIZATION_PERCENTILE)
 PDF_SIZE = _lib.DLQ_PDF_SIZE
 
 TfEncoding = namedtuple("TfEncoding", ["min", "max", "delta", "offset", "bw"])
@@ -38,8 +40,9 @@ class BlockTensorQuantizer:
     quantizer shape being right-aligned against the tensor shape (tensor_utils.cpp:28-58)."""
 
     def __init__(self, shape: Sequence[int], bitwidth: int, quantScheme: int, device="cuda"):
-        if quantScheme not in (QUANTIZATION_TF, QUANTIZATION_TF_ENHANCED):
-            raise ValueError("only QUANTIZATION_TF and QUANTIZATION_TF_ENHANCED are implemented")
+        if quantScheme not in _SCHEMES:
+            raise ValueError("only QUANTIZATION_TF, QUANTIZATION_TF_ENHANCED and QUANTIZATION_PERCENTILE are implemented")
+        self._percentile = 100.0  # PercentileEncodingAnalyzer.h:71
         self._shape = tuple(int(d) for d in shape)
         self.bitwidth = int(bitwidth)
         self.isEncodingValid = False
@@ -158,10 +161,14 @@ class BlockTensorQuantizer:
         return out
 
     def setPercentileValue(self, percentile: float):
-        raise RuntimeError("percentile is only used by the percentile quantization scheme")
+        if self._quantScheme != QUANTIZATION_PERCENTILE:
+            raise RuntimeError("percentile is only used by the percentile quantization scheme")
+        self._percentile = float(percentile)
 
     def getPercentileValue(self) -> float:
-        raise RuntimeError("percentile is only used by the percentile quantization scheme")
+        if self._quantScheme != QUANTIZATION_PERCENTILE:
+            raise RuntimeError("percentile is only used by the percentile quantization scheme")
+        return self._percentile
 
     # ------------------------------------------------------------------------------------------------- encodings --
     def computeEncodings(self, useSymmetricEncodings: bool) -> List[TfEncoding]:
@@ -178,6 +185,12 @@ class BlockTensorQuantizer:
                                                   float(self._zeroPointShift), out.data_ptr(), stream)
             if status != _lib.AHQ_OK:
                 raise RuntimeError(lib.ahq_last_error().decode())
+        elif self._quantScheme == QUANTIZATION_PERCENTILE:
+            if self._zeroPointShift != 0.0:
+                raise RuntimeError("Non-zero zeroPointShift is only supported for min-max quant scheme.")
+            _lib.check(lib.ahq_dlq_percentile_encodings(self._pdf_state(), self._percentile, self.bitwidth, sym,
+                                                        int(self._useStrictSymmetric), int(self._useUnsignedSymmetric),
+                                                        out.data_ptr(), stream), "ahq_dlq_percentile_encodings")
         else:
             if self._zeroPointShift != 0.0:
                 raise RuntimeError("Non-zero zeroPointShift is only supported for min-max quant scheme.")
@@ -224,8 +237,8 @@ class BlockTensorQuantizer:
 
     # --------------------------------------------------------------------------------------------------- settings --
     def setQuantScheme(self, quantScheme: int):
-        if quantScheme not in (QUANTIZATION_TF, QUANTIZATION_TF_ENHANCED):
-            raise ValueError("only QUANTIZATION_TF and QUANTIZATION_TF_ENHANCED are implemented")
+        if quantScheme not in _SCHEMES:
+            raise ValueError("only QUANTIZATION_TF, QUANTIZATION_TF_ENHANCED and QUANTIZATION_PERCENTILE are implemented")
         self._quantScheme = quantScheme
         self._allocate_stats()
         self._validStats = False

@@ -220,6 +220,13 @@ int    ahq_dlq_tfe_encodings(const ahq_dlq_pdf_state* state, int32_t bw, int32_t
                              int32_t unsigned_sym, double* out, int32_t* best_index, void* workspace,
                              size_t workspace_bytes, void* stream);
 
+/* Replaces PercentileEncodingAnalyzer::computeEncoding (DLQ/src/PercentileEncodingAnalyzer.cpp:52-169) on the same PDF
+ * statistics: the range that keeps `percentile` percent of the probability mass on each side, widened to contain
+ * zero, then getComputedEncodings.  out: [num_slots][5].
+ */
+int ahq_dlq_percentile_encodings(const ahq_dlq_pdf_state* state, float percentile, int32_t bw, int32_t symmetric,
+                                 int32_t strict, int32_t unsigned_sym, double* out, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

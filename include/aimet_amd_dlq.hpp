@@ -1,6 +1,6 @@
 // aimet_amd_dlq.hpp -- header-only C++ facade over the C ABI of libaimet_amd.so with the interface of
 // DlQuantization::BlockTensorQuantizer (ModelOptimizations/DlQuantization/include/DlQuantization/TensorQuantizer.h:34-199,
-// src/TensorQuantizer.cpp), for the integer QUANTIZATION_TF and QUANTIZATION_TF_ENHANCED schemes.
+// src/TensorQuantizer.cpp), for the integer QUANTIZATION_TF, QUANTIZATION_TF_ENHANCED and QUANTIZATION_PERCENTILE schemes.
 //
 // Differences from the reference class, all forced by "device only":
 //   * useCuda must be true: tensors are device pointers (the reference's CPU path has no counterpart here);
@@ -27,7 +27,8 @@ namespace aimet_amd
 enum QuantizationMode
 {
     QUANTIZATION_TF          = 0,
-    QUANTIZATION_TF_ENHANCED = 1
+    QUANTIZATION_TF_ENHANCED = 1,
+    QUANTIZATION_PERCENTILE  = 3
 };
 
 struct TfEncoding
@@ -152,6 +153,14 @@ public:
                                                       _numEncodings, bitwidth, useSymmetricEncodings, _useStrictSymmetric,
                                                       _useUnsignedSymmetric, _zeroPointShift, out, stream));
         }
+        else if (_quantScheme == QUANTIZATION_PERCENTILE)
+        {
+            if (_zeroPointShift != 0.0)
+                throw std::runtime_error("Non-zero zeroPointShift is only supported for min-max quant scheme.");
+            ahq_dlq_pdf_state st = pdfState();
+            detail::ahqCheck(ahq_dlq_percentile_encodings(&st, _percentile, bitwidth, useSymmetricEncodings,
+                                                          _useStrictSymmetric, _useUnsignedSymmetric, out, stream));
+        }
         else
         {
             if (_zeroPointShift != 0.0)
@@ -256,8 +265,18 @@ public:
         isEncodingValid       = false;
         _useUnsignedSymmetric = v;
     }
-    void setPercentileValue(float) { throw std::runtime_error("percentile is only used by the percentile quantization scheme"); }
-    float getPercentileValue() const { throw std::runtime_error("percentile is only used by the percentile quantization scheme"); }
+    void setPercentileValue(float percentile)
+    {
+        if (_quantScheme != QUANTIZATION_PERCENTILE)
+            throw std::runtime_error("percentile is only used by the percentile quantization scheme");
+        _percentile = percentile;
+    }
+    float getPercentileValue() const
+    {
+        if (_quantScheme != QUANTIZATION_PERCENTILE)
+            throw std::runtime_error("percentile is only used by the percentile quantization scheme");
+        return _percentile;
+    }
     bool hasValidStats() const { return _validStats; }
     TensorDims getShape() const { return _shape; }
     Encodings getEncodings() const { return _encodings; }
@@ -354,6 +373,7 @@ private:
     bool _validStats           = false;
     bool _allInitialized       = false;
     double _zeroPointShift     = 0.0;
+    float _percentile          = 100;
     Encodings _encodings;
     TensorDims _shape;
     int64_t _numEncodings = 1;

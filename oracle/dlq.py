@@ -46,6 +46,9 @@ def lib():
         L.dlq_tfe_compute_encoding.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                                _f64p, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int)]
         L.dlq_tfe_compute_encoding.restype = None
+        L.dlq_percentile_compute_encoding.argtypes = [ctypes.c_void_p, ctypes.c_float, ctypes.c_int, ctypes.c_int,
+                                                      ctypes.c_int, ctypes.c_int, _f64p]
+        L.dlq_percentile_compute_encoding.restype = None
         _lib = L
     return _lib
 
@@ -152,3 +155,9 @@ class Pdf:
         lib().dlq_tfe_compute_encoding(self._buf, bw, int(symmetric), int(strict), int(unsigned_sym), out,
                                        ctypes.byref(n), ctypes.byref(best))
         return (out, n.value, best.value) if with_index else out
+
+    def percentile_encoding(self, percentile, bw, symmetric, strict=False, unsigned_sym=False):
+        out = np.zeros(5)
+        lib().dlq_percentile_compute_encoding(self._buf, float(percentile), bw, int(symmetric), int(strict),
+                                              int(unsigned_sym), out)
+        return out

@@ -364,5 +364,50 @@ void dlq_tfe_compute_encoding(const dlq_pdf* p, int bw, int symmetric, int stric
     if (best_out) *best_out = best;
 }
 
+/* ------------------------------------------------------------------ percentile --------------------------------------
+ * PercentileEncodingAnalyzer::computeEncoding / _computePercentileRange (PercentileEncodingAnalyzer.cpp:52-169) with
+ * findOriginalRange (math_functions.cpp:401-435).  The statistics are the same PDF as the TF-enhanced analyzer's. */
+void dlq_percentile_compute_encoding(const dlq_pdf* p, float percentile, int bw, int symmetric, int strict,
+                                     int unsigned_sym, double* out) {
+    float num_steps = (float)(pow(2, bw) - 1);
+    if (symmetric && strict) num_steps -= 1;
+    memset(out, 0, 5 * sizeof(double));
+    if (!p->initialized) {
+        if (p->stats_updated) {
+            double mn = -1, mx = 1;
+            const double delta = (mx - mn) / (int)num_steps;
+            const double offset = floor(mn / delta);
+            mn = offset * delta;
+            mx = mn + (int)num_steps * delta;
+            out[0] = mn; out[1] = mx; out[2] = delta; out[3] = offset; out[4] = bw;
+        }
+        return;
+    }
+    float min_val, max_val;
+    find_range(p, &min_val, &max_val); /* findOriginalRange is the same search as _findRangeOfAggregateStats */
+    float a_min = min_val, a_max = max_val;
+    if (percentile != 100.0f) {
+        const float bin_width = (float)(p->xleft[1] - p->xleft[0]);
+        const float hist_min = (float)p->xleft[0];
+        const float hist_max = (float)(p->xleft[DLQ_PDF_SIZE - 1] + bin_width);
+        float pmin = hist_min, pmax = hist_max;
+        double cdf[DLQ_PDF_SIZE];
+        cdf[0] = p->pdf[0];
+        for (int i = 1; i < DLQ_PDF_SIZE; ++i) cdf[i] = p->pdf[i] + cdf[i - 1];
+        const float left = 1 - percentile / 100;
+        for (int i = 0; i < DLQ_PDF_SIZE; ++i)
+            if (cdf[i] >= left) { pmin = (float)p->xleft[i]; break; }
+        const float right = percentile / 100;
+        for (int i = DLQ_PDF_SIZE - 1; i >= 0; --i)
+            if (cdf[i] < right && p->xleft[i] < max_val) { pmax = (float)(p->xleft[i] + bin_width); break; }
+        if (pmin == pmax) pmax += bin_width;
+        a_min = pmin;
+        a_max = pmax;
+    }
+    a_min = fmin_std(a_min, 0.f);
+    a_max = fmax_std(a_max, 0.f);
+    dlq_computed_encodings(bw, a_min, a_max, symmetric, strict, unsigned_sym, 0.0, out);
+}
+
 /* size of dlq_pdf, for callers that allocate it from another language */
 uint64_t dlq_pdf_sizeof(void) { return sizeof(dlq_pdf); }

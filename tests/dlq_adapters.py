@@ -8,6 +8,7 @@ from oracle import dlq as OD
 
 QUANTIZATION_TF = 0
 QUANTIZATION_TF_ENHANCED = 1
+QUANTIZATION_PERCENTILE = 3
 
 
 def _widen(x: torch.Tensor) -> np.ndarray:
@@ -25,6 +26,7 @@ class OracleQuantizer:
         self.strict = False
         self.unsigned = False
         self.zps = 0.0
+        self.percentile = 100.0
         self.valid_stats = False
         self.isEncodingValid = False
         self.encodings = None
@@ -67,6 +69,9 @@ class OracleQuantizer:
                                              self.zps)) for e in range(self.E)]
         if self.zps != 0.0:
             raise RuntimeError("Non-zero zeroPointShift is only supported for min-max quant scheme.")
+        if self.scheme == QUANTIZATION_PERCENTILE:
+            return [tuple(p.percentile_encoding(self.percentile, self.bitwidth, symmetric, self.strict, self.unsigned))
+                    for p in self.pdfs]
         out = []
         self.last_best = []
         for p in self.pdfs:
@@ -100,6 +105,9 @@ class OracleQuantizer:
 
     def setZeroPointShift(self, v):
         self.zps = float(v)
+
+    def setPercentileValue(self, v):
+        self.percentile = float(np.float32(v))
 
     def stats(self):
         """(min, max) arrays or (xleft, pdf, meta) arrays, for comparisons between implementations."""
@@ -150,6 +158,9 @@ class HipQuantizer:
 
     def setZeroPointShift(self, v):
         self.q.setZeroPointShift(v)
+
+    def setPercentileValue(self, v):
+        self.q.setPercentileValue(v)
 
     def stats(self):
         if self.scheme == QUANTIZATION_TF:

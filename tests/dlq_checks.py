@@ -12,7 +12,7 @@ import torch
 HERE = os.path.dirname(os.path.abspath(__file__))
 V = json.load(open(os.path.join(HERE, "golden", "dlq_vectors.json")))
 INPUTS = np.load(os.path.join(HERE, "golden", "dlq_inputs.npz"))
-TF, TFE = 0, 1
+TF, TFE, PCT = 0, 1, 3
 
 
 def _t(v, dtype=torch.float32):
@@ -289,3 +289,61 @@ def check_tfe_properties(make):
         pass
     else:
         raise AssertionError("TF-enhanced must reject a zero-point shift")
+
+
+def check_percentile(make):
+    """test/TestPercentileEncodingAnalyzer.cpp:21-296: the reference's bounds and exact expectations."""
+    d100k = torch.from_numpy(INPUTS["normal_mean2_std2_100k"].copy())
+    dm21 = torch.from_numpy(INPUTS["normal_meanm2_std1"].copy())
+    # Asymmetric, 99.9999 %, 100000 samples of N(2, 2): between 2 and 6 standard deviations each side
+    q = make((), 8, PCT)
+    q.setPercentileValue(99.9999)
+    q.updateStats(d100k)
+    (e,) = q.computeEncodings(False)
+    assert 2 - 12 < e[0] < 2 - 4 and 2 + 4 < e[1] < 2 + 12
+    amax = float(dm21.abs().max())
+    for strict, steps, off in ((False, 255, -128), (True, 254, -127)):
+        q = make((), 8, PCT)
+        q.setPercentileValue(99.9)
+        q.setStrictSymmetric(strict)
+        q.updateStats(dm21)
+        (e,) = q.computeEncodings(True)
+        assert e[0] > -amax and e[1] < amax
+        assert abs(e[2] - (e[1] - e[0]) / steps) <= 4e-7 * abs(e[2])
+        assert abs(e[3] - e[0] / e[2]) <= 4e-7 * abs(e[3])
+        assert e[3] == off and e[4] == 8
+        if strict:
+            assert e[0] == -e[1]
+    # SymmetricUnsigned, 99.9999 %
+    clipped = dm21.clamp_min(0.0)
+    q = make((), 8, PCT)
+    q.setPercentileValue(99.9999)
+    q.setUnsignedSymmetric(True)
+    q.updateStats(clipped)
+    (e,) = q.computeEncodings(True)
+    assert e[0] == 0 and abs(e[1] - float(clipped.max())) <= 0.015
+    assert abs(e[2] - (e[1] - e[0]) / 255) <= 4e-7 * abs(e[2])
+    # percentile 100: the full observed range
+    q = make((), 8, PCT)
+    q.setPercentileValue(100)
+    q.updateStats(dm21)
+    (e,) = q.computeEncodings(True)
+    assert e[1] < amax + 1536 and e[3] == -128 and e[4] == 8
+    assert abs(e[2] - (e[1] - e[0]) / 255) <= 4e-7 * abs(e[2])
+    # constant tensors
+    q = make((), 8, PCT)
+    q.setPercentileValue(99.9999)
+    q.updateStats(torch.full((6000,), 4.0))
+    (e,) = q.computeEncodings(False)
+    assert e[0] <= 0 and e[1] >= 3.99006
+    q = make((), 8, PCT)
+    q.setPercentileValue(99.9999)
+    q.updateStats(torch.full((6000,), -5.0))
+    (e,) = q.computeEncodings(False)
+    assert e[0] <= -4.99992 and e[1] >= 0
+    # all zeros
+    q = make((), 8, PCT)
+    q.setPercentileValue(99.9999)
+    q.updateStats(torch.zeros(6000))
+    (e,) = q.computeEncodings(False)
+    assert abs(e[0] + 1.00392) <= 1e-4 and abs(e[1] - 0.996078) <= 1e-4 and e[3] == -128 and e[4] == 8

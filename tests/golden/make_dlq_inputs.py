@@ -16,9 +16,10 @@ def main():
         exe = os.path.join(tmp, "make_dlq_inputs")
         subprocess.run(["g++", "-O1", "-o", exe, os.path.join(HERE, "make_dlq_inputs.cpp")], check=True)
         out = {}
-        for name, mean, std in (("normal_mean2_std2", 2, 2), ("normal_meanm2_std1", -2, 1)):
+        for name, mean, std, count in (("normal_mean2_std2", 2, 2, 6000), ("normal_meanm2_std1", -2, 1, 6000),
+                                       ("normal_mean2_std2_100k", 2, 2, 100000)):
             path = os.path.join(tmp, name + ".f32")
-            subprocess.run([exe, str(mean), str(std), "6000", path], check=True)
+            subprocess.run([exe, str(mean), str(std), str(count), path], check=True)
             out[name] = np.fromfile(path, dtype=np.float32)
         np.savez_compressed(os.path.join(HERE, "dlq_inputs.npz"), **out)
         for k, v in out.items():

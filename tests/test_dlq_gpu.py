@@ -7,7 +7,8 @@ import torch
 
 from oracle import dlq as OD
 from tests import dlq_checks as C
-from tests.dlq_adapters import QUANTIZATION_TF, QUANTIZATION_TF_ENHANCED, HipQuantizer, OracleQuantizer
+from tests.dlq_adapters import (QUANTIZATION_PERCENTILE, QUANTIZATION_TF, QUANTIZATION_TF_ENHANCED, HipQuantizer,
+                                OracleQuantizer)
 
 pytestmark = pytest.mark.gpu
 
@@ -43,6 +44,10 @@ def test_tfe_all_zero_vector(make):
 
 def test_tfe_reference_bounds(make):
     C.check_tfe_properties(make)
+
+
+def test_percentile_reference_expectations(make):
+    C.check_percentile(make)
 
 
 # ------------------------------------------------------------------------------------- bit-exact against the oracle --
@@ -280,3 +285,37 @@ def test_end_to_end_tf_enhanced_then_qdq(device):
         q.updateStats(x)
         q.setEncodings(q.computeEncodings(False))
     assert torch.equal(a.quantizeDequantize(x), b.quantizeDequantize(x))
+
+
+@pytest.mark.parametrize("percentile", [100.0, 99.9999, 99.9, 99.0, 90.0, 50.0])
+@pytest.mark.parametrize("enc_shape,shape", [((), (100000,)), ((4, 1), (4, 30000))])
+def test_percentile_encodings_bit_exact(device, percentile, enc_shape, shape):
+    g = torch.Generator().manual_seed(21)
+    a = OracleQuantizer(enc_shape, 8, QUANTIZATION_PERCENTILE)
+    b = HipQuantizer(enc_shape, 8, QUANTIZATION_PERCENTILE, device)
+    for q in (a, b):
+        q.setPercentileValue(percentile)
+    for k in range(3):
+        x = torch.randn(shape, generator=g) * (1.0 + k) + 0.5
+        x.view(-1)[::997] = 25.0  # a thin tail of outliers for the percentile to cut
+        a.updateStats(x)
+        b.updateStats(x)
+    _same_pdf(a, b)
+    for bw in (4, 8, 16):
+        a.bitwidth = bw
+        b.q.bitwidth = bw
+        for sym, strict, uns in TFE_MODES:
+            for q in (a, b):
+                q.setStrictSymmetric(strict)
+                q.setUnsignedSymmetric(uns)
+            ea, eb = a.computeEncodings(sym), b.computeEncodings(sym)
+            assert np.array_equal(np.array(ea), np.array(eb)), (bw, sym, strict, uns, ea, eb)
+
+
+def test_percentile_value_only_exists_for_the_percentile_scheme(device):
+    q = HipQuantizer((), 8, QUANTIZATION_TF_ENHANCED, device)
+    with pytest.raises(RuntimeError):
+        q.setPercentileValue(90.0)
+    q = HipQuantizer((), 8, QUANTIZATION_PERCENTILE, device)
+    q.setPercentileValue(90.0)
+    assert q.q.getPercentileValue() == 90.0

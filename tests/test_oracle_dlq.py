@@ -43,6 +43,26 @@ def test_tfe_reference_bounds():
     C.check_tfe_properties(make)
 
 
+def test_percentile_reference_expectations():
+    C.check_percentile(make)
+
+
+def test_percentile_matches_numpy_quantiles():
+    """Closed form: the chosen range brackets the empirical quantiles to within two buckets."""
+    x = C.INPUTS["normal_mean2_std2_100k"]
+    p = OD.Pdf()
+    p.update(x)
+    width = p.xleft[1] - p.xleft[0]
+    for pct in (99.0, 99.9, 90.0):
+        e = p.percentile_encoding(pct, 16, False)
+        lo, hi = np.quantile(x.astype(np.float64), [1 - pct / 100, pct / 100])
+        assert abs(e[0] - min(lo, 0.0)) <= 2 * width + e[2], (pct, e, lo)
+        assert abs(e[1] - max(hi, 0.0)) <= 2 * width + e[2], (pct, e, hi)
+    # 100 % keeps the whole observed range
+    e = p.percentile_encoding(100.0, 16, False)
+    assert e[0] <= x.min() + width and e[1] >= x.max() - width
+
+
 # ------------------------------------------------------------------------------------------------ closed forms ----
 def test_qdq_is_identity_on_grid_points_and_saturates():
     enc = C.tf_encoding(-4.0, 3.96875, 8)  # delta = 1/32: every grid point is exact in float
