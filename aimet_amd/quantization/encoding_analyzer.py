@@ -12,6 +12,7 @@ device, where each operation is a single IEEE operation and therefore reproduces
 
 from __future__ import annotations
 
+import functools
 import math
 import contextlib
 import warnings
@@ -265,6 +266,10 @@ class MinMaxEncodingAnalyzer(EncodingAnalyzer[_MinMaxRange]):
         if stats.min is None or stats.max is None:
             raise StatisticsNotFoundError("No statistics present to compute encodings.")
 
+        fused = self._fused_encodings(stats, num_steps, is_symmetric)
+        if fused is not None:
+            return fused
+
         tiny = _get_minimum_scale(num_steps)
         lo = torch.clamp(stats.min, max=0)
         hi = torch.clamp(stats.max, min=0)
@@ -284,6 +289,37 @@ class MinMaxEncodingAnalyzer(EncodingAnalyzer[_MinMaxRange]):
         hi = torch.clamp(hi, max=torch.finfo(stats.min.dtype).max).to(stats.min.dtype)
         lo = torch.clamp(lo, min=torch.finfo(stats.max.dtype).min).to(stats.max.dtype)
         return lo, hi
+
+
+    @staticmethod
+    def _fused_encodings(stats: _MinMaxRange, num_steps: int, is_symmetric: bool):
+        """The arithmetic below in one kernel launch (ahq_minmax_to_encodings); None when the statistics are not a
+        pair of same-shaped 16/32-bit float tensors, in which case the elementwise formulation runs."""
+        mn, mx = stats.min, stats.max
+        if (mn.dtype not in _lib.DTYPE_CODE or mx.dtype != mn.dtype or mn.shape != mx.shape or not mn.is_cuda
+                or num_steps > (1 << 24)):
+            return None
+        dt = mn.dtype
+        tiny = _get_minimum_scale(num_steps)
+        consts = _scalar_constants(dt, tiny)
+        mn, mx = mn.contiguous(), mx.contiguous()
+        lo, hi = torch.empty_like(mn), torch.empty_like(mx)
+        flags = torch.zeros(2, dtype=torch.int32, device=mn.device)
+        lib = _lib.load()
+        _lib.check(lib.ahq_minmax_to_encodings(_lib.DTYPE_CODE[dt], mn.data_ptr(), mx.data_ptr(), mn.numel(), num_steps,
+                                               1 if is_symmetric else 0, consts[0], consts[1], consts[2], consts[3],
+                                               lo.data_ptr(), hi.data_ptr(), flags.data_ptr(),
+                                               _lib.current_stream(mn.device)), "ahq_minmax_to_encodings")
+        lo._ahq_range_flags = hi._ahq_range_flags = flags  # pylint: disable=protected-access
+        return lo, hi
+
+
+@functools.lru_cache(maxsize=256)
+def _scalar_constants(dtype: torch.dtype, tiny: float):
+    """(minimum scale as `dtype` sees it, as float32, finfo(dtype).max, the near-overflow threshold in `dtype`)."""
+    big = torch.finfo(dtype).max
+    return (float(torch.tensor(tiny, dtype=dtype)), float(torch.tensor(tiny, dtype=torch.float32)), float(big),
+            float(torch.tensor(1e-8 + 0.05 * big, dtype=dtype)))
 
 
 _deferred_range_flags = None  # list of device flag pairs while deferred_range_warnings() is active
@@ -320,6 +356,14 @@ def _warn_range_flags(nonfinite: bool, extreme: bool):
 
 def _flag_extreme_min_max(curr_min, curr_max):
     """Warn about non-finite or near-overflow encodings (reference: encoding_analyzer.py:484-498)."""
+    flags = getattr(curr_min, "_ahq_range_flags", None)
+    if flags is not None and getattr(curr_max, "_ahq_range_flags", None) is flags:
+        flags = flags != 0  # already evaluated by the kernel that produced this pair
+        if _deferred_range_flags is not None:
+            _deferred_range_flags.append(flags)
+            return
+        _warn_range_flags(*flags.tolist())
+        return
     big = torch.finfo(curr_min.dtype).max
     both = torch.stack([curr_min.reshape(-1), curr_max.reshape(-1)]).abs()
     nonfinite = ~torch.isfinite(both).all()

@@ -125,6 +125,20 @@ size_t ahq_minmax_workspace_bytes(const ahq_layout* layout);
 int    ahq_minmax(int32_t dtype, const ahq_layout* layout, const void* x, void* out_min, void* out_max,
                   void* run_min, void* run_max, int finite_only, void* workspace, size_t workspace_bytes, void* stream);
 
+/* Replaces MinMaxEncodingAnalyzer.compute_encodings_from_stats (AT/quantization/encoding_analyzer.py:425-481) and the
+ * checks of _flag_extreme_min_max (:484-498): zero forced into the range, ranges narrower than the minimum scale
+ * widened, symmetric grids re-centred, the result clamped to the statistics dtype.  stat_min / stat_max / out_min /
+ * out_max hold num_encodings values of `dtype`.  The three thresholds are passed the way torch's scalar handling
+ * produces them: minimum_scale_in_dtype = the minimum scale rounded to `dtype` (the comparison), minimum_scale = the
+ * same as float32 (the widening term), near_max_threshold = dtype(1e-8 + 0.05 * dtype_max).
+ * flags (optional, int32[2], accumulated with OR, cleared by the caller): [0] a result is NaN or infinite, [1] a
+ * result lies within 5 % of dtype_max.
+ */
+int ahq_minmax_to_encodings(int32_t dtype, const void* stat_min, const void* stat_max, int64_t num_encodings,
+                            int64_t num_steps, int32_t symmetric, float minimum_scale_in_dtype, float minimum_scale,
+                            float dtype_max, float near_max_threshold, void* out_min, void* out_max, int32_t* flags,
+                            void* stream);
+
 /* ---------------------------------------------------------------- histogram statistics ----------------------------
  * Replaces: _HistogramObserver.collect_stats + merge_stats (AT/quantization/encoding_analyzer.py:189-332), i.e. what
  * PercentileEncodingAnalyzer / SqnrEncodingAnalyzer / TfEnhancedEncodingAnalyzer.update_stats do per batch.
