@@ -21,6 +21,9 @@ class _GridMixin:
             f"{what} only exists for grids [0, 2^B - 1] and [-2^(B-1), 2^(B-1) - 1]"
         )
 
+    def _get_centroid(self) -> int:
+        return math.ceil((self.qmax + self.qmin) / 2)
+
     def _get_bitwidth(self) -> int:
         """B such that the grid is [0, 2^B - 1] or [-2^(B-1), 2^(B-1) - 1]; RuntimeError otherwise."""
         if self._is_standard_grid():

@@ -1,12 +1,13 @@
 """Affine encodings: the (scale, offset, grid) description attached to quantizer outputs.
 
-Counterpart of aimet_torch/quantization/affine/encoding.py:33-331 and :579-619 (the export formats are not part of
-this package).
+Counterpart of aimet_torch/quantization/affine/encoding.py:33-458 and :579-684, including the export of an encoding to
+the dictionary formats "0.6.1", "1.0.0", "2.0.0" and "2.1.0" (`to_qnn_encoding_dict`).
 """
 
 from __future__ import annotations
 
-from typing import Optional, Tuple
+import math
+from typing import Dict, List, Optional, Tuple, Union
 
 import torch
 
@@ -24,6 +25,7 @@ class AffineEncoding(EncodingBase, _GridMixin):
     def __init__(self, scale: torch.Tensor, offset: torch.Tensor, *args, **kwargs):
         self.scale = scale
         self.offset = offset
+        self._input_shape_hint = None
         pos = tuple(args) + (None,) * (5 - len(args))
         first = kwargs.pop("qmin", kwargs.pop("bitwidth", pos[0]))
         second = kwargs.pop("qmax", kwargs.pop("signed", pos[1]))
@@ -105,6 +107,120 @@ class AffineEncoding(EncodingBase, _GridMixin):
         return AffineEncoding(scale, offset, self.qmin, self.qmax, self._symmetry, self.block_size,
                               self._zero_point_shift, producer=self.producer)
 
+    # ------------------------------------------------------------------------------------------------ export --
+    def _hint_input_shape(self, input_shape: Tuple[int, ...]) -> "AffineEncoding":
+        """Shape of the tensor this encoding quantizes; needed to tell channel axes from block axes
+        (aimet_torch/quantization/base/encoding.py:130-140)."""
+        self._input_shape_hint = tuple(input_shape)
+        return self
+
+    def _safe_get_channel_and_block_axis(self):
+        """(channel axis, block axis) as negative indices into the scale's dimensions, None where there is none
+        (base/encoding.py:142-213).  An axis with several blocks of more than one element is a block axis; an axis
+        with several blocks of one element is a channel axis."""
+        from aimet_amd.quantization._utils import concretize_block_size
+
+        if self._input_shape_hint is None:
+            raise RuntimeError("Could not safely infer channel and block axes because input shape hint is not provided. "
+                               "Call `_hint_input_shape` before calling this function.")
+        concrete = concretize_block_size(self._input_shape_hint, self.scale.shape, self.block_size or ())
+        channel_axes, block_axes = [], []
+        for axis, (n_blocks, blk) in enumerate(zip(self.scale.shape, concrete)):
+            if n_blocks > 1:
+                (block_axes if blk > 1 else channel_axes).append(axis)
+        if len(block_axes) > 1:
+            raise RuntimeError(f"Multiple non-trivial block axes found: {block_axes}. Cannot determine a unique block axis.")
+        block_axis = block_axes[0] if block_axes else None
+        if not channel_axes and block_axis is not None:
+            # a singleton dimension is still the channel axis when its block size is 1
+            channel_axes = [axis for axis, blk in enumerate(concrete) if blk == 1]
+        if len(channel_axes) > 1:
+            raise RuntimeError(f"Multiple non-trivial channel axes found: {channel_axes}. "
+                               "Cannot determine a unique channel axis.")
+        channel_axis = channel_axes[0] if channel_axes else None
+        if channel_axis is None and block_axis is not None:
+            raise RuntimeError(f"Block axis {block_axis} found without a corresponding channel axis. "
+                               "Cannot determine a unique channel axis.")
+        nd = self.scale.dim()
+        return (None if channel_axis is None else channel_axis - nd, None if block_axis is None else block_axis - nd)
+
+    def _get_export_dtype(self) -> str:
+        nbits = math.ceil(math.log2(self.qmax - self.qmin + 1))
+        return f"int{nbits}" if self.qmin < 0 <= self.qmax else f"uint{nbits}"
+
+    def _to_legacy_format(self) -> List[Dict]:
+        """One dictionary per encoding; the offset counts from qmin (encoding.py:333-357)."""
+        offset = self.offset.flatten() + self.qmin
+        out = []
+        for mn, mx, sc, off in zip(self.min.flatten(), self.max.flatten(), self.scale.flatten(), offset):
+            enc = {"min": float(mn), "max": float(mx), "scale": float(sc), "offset": int(off),
+                   "bitwidth": self.bitwidth, "dtype": "int", "is_symmetric": str(self.symmetry)}
+            if self.zero_point_shift:
+                enc["zero_point_shift"] = self.zero_point_shift
+            out.append(enc)
+        return out
+
+    def to_qnn_encoding_dict(self, encoding_version=None) -> Union[List, Dict]:
+        """The encoding as a dictionary of the given format version (encoding.py:362-458)."""
+        if encoding_version == "0.6.1":
+            return self._to_legacy_format()
+
+        if encoding_version == "1.0.0":
+            offset = self.offset
+            if self.signed:
+                offset = offset - 2 ** (self.bitwidth - 1)
+            enc = {"dtype": "INT", "bw": self.bitwidth, "is_sym": self.symmetry,
+                   "scale": self.scale.flatten().tolist(), "offset": offset.to(torch.int).flatten().tolist()}
+            if self.zero_point_shift != 0.0:
+                assert self.zero_point_shift == 0.5 and self.symmetry
+                enc["zero_point_shift"] = [self.zero_point_shift] * len(enc["offset"])
+            granularity = self.granularity
+            assert granularity != "unknown"
+            if granularity == "pertensor":
+                enc["enc_type"] = "PER_TENSOR"
+            elif granularity == "perchannel":
+                enc["enc_type"] = "PER_CHANNEL"
+            else:
+                _, block_axis = self._safe_get_channel_and_block_axis()
+                enc["enc_type"] = "PER_BLOCK"
+                enc["block_size"] = self.block_size[block_axis]
+                if enc["block_size"] == -1:
+                    raise NotImplementedError("Exporting encodings to 1.0.0 format with block size -1 is not supported yet. "
+                                              "Export using sim.export() instead.")
+            return enc
+
+        if encoding_version in ("2.0.0", "2.1.0"):
+            y_scale = self.scale
+            if self.symmetry:
+                y_zero_point = torch.full_like(y_scale, self._get_centroid(), dtype=torch.int32)
+            else:
+                y_zero_point = -self.offset.to(torch.int32)
+            if self.zero_point_shift:
+                y_zero_point = y_zero_point - self.zero_point_shift
+            channel_axis = block_axis = block_size = None
+            if self.granularity != "pertensor":
+                channel_axis, block_axis = self._safe_get_channel_and_block_axis()
+            if block_axis is not None:
+                axis = block_axis
+                block_size = self.block_size[block_axis]
+            elif channel_axis is not None:
+                axis = channel_axis
+                y_scale, y_zero_point = y_scale.flatten(), y_zero_point.flatten()
+            else:
+                axis = None
+                y_scale, y_zero_point = y_scale.squeeze(), y_zero_point.squeeze()
+            ret = {"output_dtype": self._get_export_dtype(), "y_scale": y_scale.tolist()}
+            if not bool(torch.all(y_zero_point == 0)):
+                ret["y_zero_point"] = y_zero_point.tolist()
+            if axis is not None:
+                ret["axis"] = axis
+            if block_size is not None:
+                ret["block_size"] = block_size
+            return ret
+
+        raise AssertionError(f"Export encoding version {encoding_version} not supported."
+                             "Expected one of: ['0.6.1', '1.0.0', '2.0.0', '2.1.0']")
+
     def quantize(self, input: torch.Tensor) -> torch.Tensor:  # pylint: disable=redefined-builtin
         return quantize(input, self.scale, self.offset, self.qmin, self.qmax, block_size=self.block_size)
 
@@ -132,6 +248,37 @@ class GroupedBlockEncoding(AffineEncoding):
         """Integer multipliers m with scale = m * per_channel_scale (1 <= m <= 2^(decompressed_bw - bitwidth))."""
         return quantize(self.scale, scale=self.per_channel_scale, offset=torch.zeros_like(self.per_channel_scale),
                         qmin=1, qmax=2 ** (self.decompressed_bw - self.bitwidth), block_size=self.block_grouping)
+
+    def to_qnn_encoding_dict(self, encoding_version=None) -> Union[List, Dict]:
+        """encoding.py:621-684: the per-block integer multipliers and the per-channel float scale replace the
+        blockwise scale, unless no blocks are grouped or the legacy format is asked for."""
+        enc = super().to_qnn_encoding_dict(encoding_version)
+        if all(g == 1 for g in self.block_grouping) or encoding_version == "0.6.1":
+            return enc
+        if encoding_version == "1.0.0":
+            enc["bw"] = self.decompressed_bw
+            enc["compressed_bw"] = self.bitwidth
+            enc["scale"] = self.per_channel_scale.flatten().tolist()
+            enc["offset"] = [-(2 ** (self.decompressed_bw - 1)) for _ in enc["scale"]]
+            enc["enc_type"] = "LPBQ"
+            enc["per_block_int_scale"] = self.per_block_int_scale.to(torch.int32).flatten().tolist()
+            return enc
+        y_zero_point = enc.pop("y_zero_point", None)
+        if y_zero_point is not None and bool(torch.any(torch.tensor(y_zero_point) != 0)):
+            raise RuntimeError(f"LPBQ only supports symmetric quantization; got non-zero y_zero_point {y_zero_point}")
+        output_dtype = f"int{self.bitwidth}" if self.signed else f"uint{self.bitwidth}"
+        int_scale = self.per_block_int_scale.to(torch.int32).tolist()
+        if encoding_version == "2.0.0":
+            del enc["y_scale"]
+            del enc["output_dtype"]
+            enc.update({"per_block_int_scale": int_scale, "per_channel_float_scale": self.per_channel_scale.tolist(),
+                        "output_dtype": output_dtype})
+        else:
+            channel_axis, _ = self._safe_get_channel_and_block_axis()
+            enc.update({"y_scale": {"x": int_scale, "x_scale": self.per_channel_scale.flatten().tolist(),
+                                    "axis": channel_axis},
+                        "output_dtype": output_dtype})
+        return enc
 
     def _rebuilt(self, scale, offset):
         return GroupedBlockEncoding(scale, offset, self.bitwidth, self.signed, self._symmetry, self.block_size,

@@ -248,3 +248,52 @@ def test_quantize_module_and_state_dict(device):
     assert q3(torch.empty(0, 3, device=device)).shape == (0, 3)
     with pytest.raises(RuntimeError):
         Dequantize((), 8, False).to(device)(x.to(device))
+
+
+@torch.no_grad()
+@pytest.mark.parametrize("shape,block_size,block_grouping,axis", [
+    ((10, 64, 1, 1), (1, 8, 1, 1), (1, 64, 1, 1), 1),
+    ((64, 10, 1, 1), (8, 1, 1, 1), (64, 1, 1, 1), 0),
+    ((10, 64), (1, 8), (1, 64), 1),
+    ((64, 10), (8, 1), (64, 1), 0),
+])
+@pytest.mark.parametrize("compressed_bw,decompressed_bw", [(4, 8), (8, 16)])
+@pytest.mark.parametrize("version", ["2.0.0", "2.1.0", "1.0.0"])
+def test_lpbq_encoding_export(device, shape, block_size, block_grouping, axis, compressed_bw, decompressed_bw, version):
+    """Parameter table and assertions of the reference's test_lpbq_encoding_schema_2_0_0
+    (test_affine_quantizer.py:2443-2535), extended to the other two formats."""
+    import numpy as np
+
+    from aimet_amd.quantization import affine
+    from aimet_amd.quantization.affine import GroupedBlockQuantizeDequantize
+
+    input_shape = tuple(1 if d == 10 else 64 if d == 64 else 10 for d in shape)
+    input_shape = tuple(s * b for s, b in zip(shape, block_size))
+    scale = (torch.arange(1, int(np.prod(shape)) + 1).view(shape) * 0.001).to(device)
+    qmin, qmax = -(2 ** (decompressed_bw - 1)), 2 ** (decompressed_bw - 1) - 1
+    qtzr = GroupedBlockQuantizeDequantize(shape=shape, bitwidth=compressed_bw, symmetric=True,
+                                          decompressed_bw=decompressed_bw, block_size=block_size,
+                                          block_grouping=block_grouping).to(device)
+    qtzr.set_range(scale * qmin, scale * qmax)
+    enc = qtzr.get_encodings()._hint_input_shape(input_shape).to_qnn_encoding_dict(version)
+    if version == "2.0.0":
+        int_scale = torch.tensor(enc["per_block_int_scale"])
+        ch_scale = torch.tensor(enc["per_channel_float_scale"])
+    elif version == "2.1.0":
+        int_scale = torch.tensor(enc["y_scale"]["x"])
+        ch_scale = torch.tensor(enc["y_scale"]["x_scale"]).view(qtzr.get_per_channel_scale().shape)
+        assert enc["y_scale"]["axis"] in (1 - axis, 1 - axis - len(shape))
+    else:
+        int_scale = torch.tensor(enc["per_block_int_scale"]).view(shape)
+        ch_scale = torch.tensor(enc["scale"]).view(qtzr.get_per_channel_scale().shape)
+        assert enc["enc_type"] == "LPBQ" and enc["bw"] == decompressed_bw and enc["compressed_bw"] == compressed_bw
+        assert enc["offset"] == [-(2 ** (decompressed_bw - 1))] * ch_scale.numel()
+    assert int_scale.min() >= 1 and int_scale.max() <= 2 ** (decompressed_bw - compressed_bw)
+    rebuilt = affine.dequantize(int_scale.to(torch.float32).to(device), ch_scale.to(device),
+                                torch.zeros_like(ch_scale).to(device), block_size=block_grouping)
+    assert torch.allclose(qtzr.get_scale(), rebuilt)
+    if version != "1.0.0":
+        assert "y_zero_point" not in enc
+        assert enc["axis"] in (axis, axis - len(shape))
+        assert enc["output_dtype"] == f"int{compressed_bw}"
+    assert enc["block_size"] == next(iter(b for b in block_size if b != 1))
