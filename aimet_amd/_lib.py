@@ -14,7 +14,7 @@ import torch
 
 AHQ_MAX_DIMS = 8
 
-AHQ_OK = 0
+AHQ_OK, AHQ_ERR_INVALID, AHQ_ERR_UNSUPPORTED, AHQ_ERR_LAUNCH, AHQ_ERR_WORKSPACE = 0, 1, 2, 3, 4
 AHQ_F32, AHQ_F16, AHQ_BF16 = 0, 1, 2
 AHQ_ARITH_ATEN, AHQ_ARITH_AUTOGRAD, AHQ_ARITH_DLQ = 1, 2, 3
 AHQ_OP_QDQ, AHQ_OP_QUANTIZE, AHQ_OP_DEQUANTIZE = 0, 1, 2
@@ -121,6 +121,8 @@ _SIGNATURES = {
     "ahq_dlq_pdf_update": (ctypes.c_int, [ctypes.c_int32, ctypes.POINTER(Layout), _P, ctypes.POINTER(DlqPdfState),
                                           ctypes.c_int32, _P, _P, ctypes.c_size_t, _P]),
     "ahq_dlq_tfe_encodings_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int32]),
+    "ahq_dlq_fp8_qdq": (ctypes.c_int, [ctypes.c_int32, ctypes.POINTER(Layout), _P, _P, _P, ctypes.c_int32, ctypes.c_int32,
+                                       ctypes.c_float, _P]),
     "ahq_dlq_percentile_encodings": (ctypes.c_int, [ctypes.POINTER(DlqPdfState), ctypes.c_float, ctypes.c_int32,
                                                     ctypes.c_int32, ctypes.c_int32, ctypes.c_int32, _P, _P]),
     "ahq_dlq_tfe_encodings": (ctypes.c_int, [ctypes.POINTER(DlqPdfState), ctypes.c_int32, ctypes.c_int32, ctypes.c_int32,

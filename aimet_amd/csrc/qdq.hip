@@ -195,6 +195,32 @@ struct MathDlq {
     __device__ static void bwd(float, float, const EncP&, const GridC&, float& gx, float& gs, float& goff) { gx = gs = goff = 0.f; }
 };
 
+// DlQuantization FP8 fake-cast (fakeCastToFp8 / quantizeDequantizeFp8Cpu, DLQ/src/trim_functions.cpp:49-67, 243-258):
+// v = clamp(x / scale, -max, max); e = max(frexp exponent of v - 1, exponent_min); step = 2^(e - mantissa bits);
+// y = rint(v / step) * step * scale.  The grid constants travel in GridC: qmin = exponent_min, qmax = max value,
+// zps = mantissa bits.  Dividing by a power of two is exact, so it is done by scaling the exponent.
+struct MathDlqFp8 {
+    static constexpr int kNP = 2;
+    static constexpr bool kDiv = true;
+    static constexpr bool kHasBwd = false;
+    __device__ static EncP prep(float s, float, float, float, const GridC&) { return {s, 0.f, 0.f, 0.f, safe_reciprocal(s)}; }
+    template <bool FAST>
+    __device__ static float fwd(float x, const EncP& e, const GridC& g, bool& inr) {
+        inr = true;
+        float v = divide<FAST, AHQ_F32>(x, e.p0, e.rs);
+        v = (v < -g.qmax) ? -g.qmax : (g.qmax < v) ? g.qmax : v;  // std::clamp: NaN passes through
+        int ex = __builtin_amdgcn_frexp_expf(v);                   // v = m * 2^ex, |m| in [0.5, 1); 0 for v == 0
+        ex = ex - 1 < (int)g.qmin ? (int)g.qmin : ex - 1;
+        const int sh = ex - (int)g.zps;
+        const float y = __builtin_ldexpf(__builtin_rintf(__builtin_ldexpf(v, -sh)), sh) * e.p0;
+        // a zero result carries the sign of x in the reference (quotient, rounding and product all keep it); the
+        // corrected quotient of divide<true> does not keep the sign of a zero
+        return y == 0.f ? __builtin_copysignf(0.f, x) : y;
+    }
+    template <bool FAST>
+    __device__ static void bwd(float, float, const EncP&, const GridC&, float& gx, float& gs, float& goff) { gx = gs = goff = 0.f; }
+};
+
 // ------------------------------------------------------------------------------------------------ kernel arguments --
 struct QdqArgs : Geom {
     const void* x;
@@ -670,6 +696,32 @@ extern "C" int ahq_qdq_forward(const ahq_grid* grid, const ahq_layout* layout, c
     hipStream_t st = static_cast<hipStream_t>(stream);
     AHQ_IO_SWITCH(grid->io_dtype, AHQ_MATH_SWITCH(*grid, (launch_fwd<IO, M>(p, a, st))));
     return check_launch("ahq_qdq_forward");
+}
+
+extern "C" int ahq_dlq_fp8_qdq(int32_t dtype, const ahq_layout* layout, const void* x, void* y, const float* scale,
+                               int32_t mantissa_bits, int32_t exponent_min, float max_value, void* stream) {
+    if (dtype != AHQ_F32) return set_error("FP8 quantize-dequantize supports float tensors only"), AHQ_ERR_UNSUPPORTED;
+    if (!layout) return set_error("layout is null"), AHQ_ERR_INVALID;
+    if (!scale) return set_error("scale is null"), AHQ_ERR_INVALID;
+    if (mantissa_bits < 0 || mantissa_bits > 23 || exponent_min < -126 || exponent_min > 127 || !(max_value > 0.f))
+        return set_error("bad FP8 format description"), AHQ_ERR_INVALID;
+    Plan p;
+    if (!make_plan(dtype, *layout, aligned16(x) && aligned16(y), false, &p)) return AHQ_ERR_INVALID;
+    if (p.cl.numel == 0) return AHQ_OK;
+    if (!x || !y) return set_error("x or y is null"), AHQ_ERR_INVALID;
+    QdqArgs a{};
+    a.x = x;
+    a.y = y;
+    a.scale = scale;
+    ahq_grid grid{};
+    grid.compute_dtype = AHQ_F32;
+    fill_args(grid, p, &a);
+    a.gc.qmin = (float)exponent_min;
+    a.gc.qmax = max_value;
+    a.gc.zps = (float)mantissa_bits;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    launch_fwd<float, MathDlqFp8>(p, a, st);
+    return check_launch("ahq_dlq_fp8_qdq");
 }
 
 extern "C" size_t ahq_qdq_backward_workspace_bytes(const ahq_grid* grid, const ahq_layout* layout, int want_param_grads) {

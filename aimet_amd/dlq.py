@@ -2,8 +2,9 @@
 
 Mirrors ``DlQuantization::BlockTensorQuantizer`` (ModelOptimizations/DlQuantization/include/DlQuantization/
 TensorQuantizer.h:34-199, src/TensorQuantizer.cpp) method for method, for the two integer calibration schemes on the
-hot path: ``QUANTIZATION_TF`` (running min/max per block) and ``QUANTIZATION_TF_ENHANCED`` (1536-bucket PDF per block
-and the (delta, offset) grid search).  Tensors are torch tensors on a HIP device; statistics stay on the device, and
+hot path: ``QUANTIZATION_TF`` (running min/max per block), ``QUANTIZATION_TF_ENHANCED`` (1536-bucket PDF per block
+and the (delta, offset) grid search) and ``QUANTIZATION_PERCENTILE`` (the same PDF, clipped at a percentile), on
+integer grids and on the FP8 formats (fake-cast with a per-block scale).  Tensors are torch tensors on a HIP device; statistics stay on the device, and
 ``computeEncodings`` returns host-side ``TfEncoding`` tuples like the reference.  There is no CPU path.
 """
 
@@ -25,6 +26,67 @@ PDF_SIZE = _lib.DLQ_PDF_SIZE
 
 TfEncoding = namedtuple("TfEncoding", ["min", "max", "delta", "offset", "bw"])
 
+
+class QuantizationType:
+    """DlQuantization::QuantizationType (include/DlQuantization/QuantizationType.hpp:36-186): an integer grid of a
+    given bitwidth, or a small floating-point format described by its exponent/mantissa layout."""
+
+    __slots__ = ("_float", "_bitwidth", "exponentBits", "mantissaBits", "exponentMin", "maxValue", "finite",
+                 "unsignedZero")
+
+    def __init__(self):
+        raise TypeError("use QuantizationType.Int / Float / Fp8E4M3FN / Fp8E5M2")
+
+    @classmethod
+    def Int(cls, bitwidth: int) -> "QuantizationType":
+        if bitwidth <= 0:
+            raise ValueError("Integer quantization bitwidth must be positive")
+        t = object.__new__(cls)
+        t._float, t._bitwidth = False, int(bitwidth)
+        t.exponentBits = t.mantissaBits = t.exponentMin = 0
+        t.maxValue, t.finite, t.unsignedZero = 0.0, False, False
+        return t
+
+    @classmethod
+    def Float(cls, exponentBits: int, mantissaBits: int, finite: bool, unsignedZero: bool) -> "QuantizationType":
+        """Bitwidth, minimum normal exponent and largest value follow from the layout
+        (QuantizationType.hpp:88-135): "fnuz" formats move the bias by one and use the whole top binade, "fn"
+        formats give up only the all-ones mantissa of the top binade, IEEE-like formats give up the top binade."""
+        if exponentBits <= 0:
+            raise ValueError("Floating-point quantization exponent bits must be positive")
+        if mantissaBits < 0:
+            raise ValueError("Floating-point quantization mantissa bits must be non-negative")
+        bias = (1 << (exponentBits - 1)) - 1 + (1 if unsignedZero else 0)
+        unit = 2.0 ** -mantissaBits
+        if unsignedZero:
+            max_exponent, max_mantissa = (1 << exponentBits) - 1 - bias, 2.0 - unit
+        elif finite:
+            max_exponent, max_mantissa = (1 << exponentBits) - 1 - bias, 2.0 - 2.0 * unit
+        else:
+            max_exponent, max_mantissa = (1 << exponentBits) - 2 - bias, 2.0 - unit
+        t = object.__new__(cls)
+        t._float, t._bitwidth = True, 1 + exponentBits + mantissaBits
+        t.exponentBits, t.mantissaBits, t.exponentMin = int(exponentBits), int(mantissaBits), 1 - bias
+        t.maxValue, t.finite, t.unsignedZero = max_mantissa * 2.0 ** max_exponent, bool(finite), bool(unsignedZero)
+        return t
+
+    @classmethod
+    def Fp8E4M3FN(cls) -> "QuantizationType":
+        return cls.Float(4, 3, True, False)
+
+    @classmethod
+    def Fp8E5M2(cls) -> "QuantizationType":
+        return cls.Float(5, 2, False, False)
+
+    def isInt(self) -> bool:
+        return not self._float
+
+    def isFloat(self) -> bool:
+        return self._float
+
+    def bitwidth(self) -> int:
+        return self._bitwidth
+
 _FLT_MAX = torch.finfo(torch.float32).max
 
 
@@ -39,12 +101,14 @@ class BlockTensorQuantizer:
     """Simulated blocked quantization: the block size along tensor dimension i is tensor_shape[i] / shape[i], the
     quantizer shape being right-aligned against the tensor shape (tensor_utils.cpp:28-58)."""
 
-    def __init__(self, shape: Sequence[int], bitwidth: int, quantScheme: int, device="cuda"):
+    def __init__(self, shape: Sequence[int], bitwidth, quantScheme: int, device="cuda"):
+        """``bitwidth``: an int (integer grid) or a QuantizationType (TensorQuantizer.cpp:17-29)."""
         if quantScheme not in _SCHEMES:
             raise ValueError("only QUANTIZATION_TF, QUANTIZATION_TF_ENHANCED and QUANTIZATION_PERCENTILE are implemented")
         self._percentile = 100.0  # PercentileEncodingAnalyzer.h:71
         self._shape = tuple(int(d) for d in shape)
-        self.bitwidth = int(bitwidth)
+        self._qtype = bitwidth if isinstance(bitwidth, QuantizationType) else QuantizationType.Int(int(bitwidth))
+        self.bitwidth = self._qtype.bitwidth()  # legacy field; setEncodings overwrites it, the qtype stays
         self.isEncodingValid = False
         self._quantScheme = quantScheme
         self._useStrictSymmetric = False
@@ -202,7 +266,31 @@ class BlockTensorQuantizer:
                                                  self._last_best.data_ptr(), ws.data_ptr(), nbytes, stream),
                        "ahq_dlq_tfe_encodings")
         rows = out.cpu().tolist()
+        if self._qtype.isFloat():
+            return self._fp8_encodings(rows)
         return [TfEncoding(r[0], r[1], r[2], r[3], int(r[4])) for r in rows]
+
+    def _fp8_encodings(self, rows) -> List[TfEncoding]:
+        """TensorQuantizer.cpp:182-224: scale = amax / maxValue, with the raw observed extrema in place of the
+        grid-snapped ones where the analyzer keeps them (min/max scheme only); delta carries the scale."""
+        if self._qtype.bitwidth() != 8:
+            raise RuntimeError("BlockTensorQuantizer floating-point encodings currently support FP8 qtypes only")
+        observed = None
+        if self._quantScheme == QUANTIZATION_TF:
+            observed = torch.stack([self._min, self._max], dim=1).double().cpu().tolist()
+        max_value = self._qtype.maxValue
+        out = []
+        for idx, r in enumerate(rows):
+            amax = max(abs(r[0]), abs(r[1]))
+            if observed is not None:
+                seen = max(abs(observed[idx][0]), abs(observed[idx][1]))
+                if seen > 0.0:
+                    amax = seen
+            if not amax > 0:
+                raise ValueError("FP8 amax must be positive")  # computeFp8Scale, quantization_utils.cpp:186-194
+            scale = amax / max_value
+            out.append(TfEncoding(-scale * max_value, scale * max_value, scale, 0.0, self._qtype.bitwidth()))
+        return out
 
     def setEncodings(self, encodings: Sequence[TfEncoding]):
         if len(encodings) != self._E:
@@ -224,11 +312,22 @@ class BlockTensorQuantizer:
         _lib.require_device(input, "input")
         if input.dtype not in _lib.DTYPE_CODE:
             raise TypeError("quantizeDequantize only supports float, half and bfloat16")
+        if self._qtype.isFloat():
+            if self._qtype.bitwidth() != 8:
+                raise RuntimeError("BlockTensorQuantizer floating-point QDQ currently supports FP8 qtypes only")
+            if input.dtype != torch.float32:
+                raise RuntimeError("BlockTensorQuantizer FP8 QDQ currently supports float tensors only")
         lib = _lib.load()
         x, layout = self._layout(input)
         y = torch.empty_like(x) if output is None else output
         if y.shape != x.shape or y.dtype != x.dtype or y.stride() != x.stride():
             raise RuntimeError("output must match the input's shape, dtype and memory layout")
+        if self._qtype.isFloat():
+            t = self._qtype
+            _lib.check(lib.ahq_dlq_fp8_qdq(_lib.DTYPE_CODE[x.dtype], layout, x.data_ptr(), y.data_ptr(),
+                                           self._enc_dev[0].data_ptr(), t.mantissaBits, t.exponentMin,
+                                           float(t.maxValue), _lib.current_stream(x.device)), "ahq_dlq_fp8_qdq")
+            return y
         grid = _hip._grid(_lib.AHQ_ARITH_DLQ, _lib.AHQ_OP_QDQ, x.dtype, torch.float32, 0, 0, 0.0)
         d, o, mn, mx = self._enc_dev
         _lib.check(lib.ahq_qdq_forward(grid, layout, x.data_ptr(), y.data_ptr(), None, d.data_ptr(), o.data_ptr(),
@@ -269,6 +368,9 @@ class BlockTensorQuantizer:
 
     def getShape(self):
         return self._shape
+
+    def getQuantizationType(self) -> QuantizationType:
+        return self._qtype
 
 
 def quantizeDequantizeBroadcast(input: torch.Tensor, encodings: Sequence[TfEncoding], encodingShape: Sequence[int]):

@@ -404,6 +404,12 @@ def run_dlq_workload(steps, warmup, dev, with_cpu_baseline=True, batches=16, sha
     t_upd = event_time(lambda: q.updateStats(xs[1]), 20)   # range already fixed: one read of the batch
     t_qdq = event_time(lambda: q.quantizeDequantize(xs[0], y), 20)
     t_enc = event_time(lambda: q.computeEncodings(False), 5)
+    # the FP8 fake-cast of the same batch (E4M3FN, scale = amax / 448 from a min/max calibration), timed beside it
+    q8 = dlq.BlockTensorQuantizer((), dlq.QuantizationType.Fp8E4M3FN(), dlq.QUANTIZATION_TF, device=dev)
+    q8.updateStats(xs[0])
+    enc8 = q8.computeEncodings(False)
+    q8.setEncodings(enc8)
+    t_fp8 = event_time(lambda: q8.quantizeDequantize(xs[0], y), 20)
     n_b = xs[0].numel()
     n = n_b * batches
     bytes_upd = 4 * n_b
@@ -426,6 +432,8 @@ def run_dlq_workload(steps, warmup, dev, with_cpu_baseline=True, batches=16, sha
     sample = xs[0].view(-1)[: 1 << 22]
     y_s = q.quantizeDequantize(sample).cpu().numpy()
     y_ok = bool((y_s.view("int32") == OD.qdq(sample.cpu().numpy(), enc_ref[:4]).view("int32")).all())
+    y8 = q8.quantizeDequantize(sample).cpu().numpy()
+    fp8_ok = bool((y8.view("int32") == OD.fp8_qdq(sample.cpu().numpy(), enc8[0].delta, OD.FP8_E4M3FN).view("int32")).all())
 
     out = {
         "metric": "QDQ fwd+bwd GB/s (% of HBM peak); calibration elems/s; vs host-CPU ref",
@@ -439,10 +447,12 @@ def run_dlq_workload(steps, warmup, dev, with_cpu_baseline=True, batches=16, sha
         "elements_per_s": round(n / wall, 1),
         "kernels": {"pdf_update(range fixed)": {"us": round(t_upd * 1e6, 2), "GBps": round(bytes_upd / t_upd / 1e9, 1)},
                     "dlq_qdq_forward": {"us": round(t_qdq * 1e6, 2), "GBps": round(bytes_qdq / t_qdq / 1e9, 1)},
+                    "dlq_fp8_qdq(e4m3fn, not part of the step)": {"us": round(t_fp8 * 1e6, 2),
+                                                                  "GBps": round(bytes_qdq / t_fp8 / 1e9, 1)},
                     "tfe_search(with host read-back)": {"us": round(t_enc * 1e6, 2), "candidates": 358, "buckets": 1536}},
         "encoding": {"min": enc[0].min, "max": enc[0].max, "delta": enc[0].delta, "offset": enc[0].offset},
         "parity": {"hist_bit_exact": hist_ok, "pdf_bit_exact": pdf_ok, "encoding_bit_exact": bool(enc_ok),
-                   "qdq_bit_exact": y_ok, "sample": "first 2 of 16 batches; 4M-element quantize-dequantize"},
+                   "qdq_bit_exact": y_ok, "fp8_qdq_bit_exact": fp8_ok, "sample": "first 2 of 16 batches; 4M-element quantize-dequantize"},
         "roofline": {"bound": "hbm", "kernel": "dlq_pdf_bin_kernel", "achieved": round(bytes_upd / t_upd / 1e9, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(bytes_upd / t_upd / 1e9 / HBM_PEAK_GBS, 4),
                      "algorithmic_bytes": bytes_upd, "traffic": None},

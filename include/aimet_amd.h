@@ -234,6 +234,16 @@ int    ahq_dlq_tfe_encodings(const ahq_dlq_pdf_state* state, int32_t bw, int32_t
                              int32_t unsigned_sym, double* out, int32_t* best_index, void* workspace,
                              size_t workspace_bytes, void* stream);
 
+/* Replaces quantizeDequantizeFp8 / quantizeDequantizeFp8Broadcast (DLQ/include/DlQuantization/Quantization.hpp,
+ * DLQ/src/trim_functions.cpp:49-67, 243-258, 791-900): y = fakeCastToFp8(x / scale) * scale under round-to-nearest-
+ * even, for the FP8 format given by its mantissa bits, minimum normal exponent and largest value
+ * (FloatQuantizationSpec, DLQ/include/DlQuantization/QuantizationType.hpp:24-33; E4M3FN = 3, -6, 448; E5M2 = 2, -14,
+ * 57344).  scale: one float per encoding of the layout (float(encoding.delta)).  Float tensors only, as in the
+ * reference.
+ */
+int ahq_dlq_fp8_qdq(int32_t dtype, const ahq_layout* layout, const void* x, void* y, const float* scale,
+                    int32_t mantissa_bits, int32_t exponent_min, float max_value, void* stream);
+
 /* Replaces PercentileEncodingAnalyzer::computeEncoding (DLQ/src/PercentileEncodingAnalyzer.cpp:52-169) on the same PDF
  * statistics: the range that keeps `percentile` percent of the probability mass on each side, widened to contain
  * zero, then getComputedEncodings.  out: [num_slots][5].

@@ -1,6 +1,6 @@
 // aimet_amd_dlq.hpp -- header-only C++ facade over the C ABI of libaimet_amd.so with the interface of
 // DlQuantization::BlockTensorQuantizer (ModelOptimizations/DlQuantization/include/DlQuantization/TensorQuantizer.h:34-199,
-// src/TensorQuantizer.cpp), for the integer QUANTIZATION_TF, QUANTIZATION_TF_ENHANCED and QUANTIZATION_PERCENTILE schemes.
+// src/TensorQuantizer.cpp), for the QUANTIZATION_TF, QUANTIZATION_TF_ENHANCED and QUANTIZATION_PERCENTILE schemes on integer grids and FP8 formats.
 //
 // Differences from the reference class, all forced by "device only":
 //   * useCuda must be true: tensors are device pointers (the reference's CPU path has no counterpart here);
@@ -13,6 +13,8 @@
 
 #include <hip/hip_runtime_api.h>
 
+#include <algorithm>
+#include <cmath>
 #include <cstdint>
 #include <stdexcept>
 #include <string>
@@ -35,6 +37,61 @@ struct TfEncoding
 {
     double min, max, delta, offset;
     int bw;
+};
+
+// QuantizationType (DlQuantization/include/DlQuantization/QuantizationType.hpp:36-186): an integer grid of a given
+// bitwidth, or a small floating-point format given by its exponent/mantissa layout.
+class QuantizationType
+{
+public:
+    static QuantizationType Int(int bitwidth)
+    {
+        if (bitwidth <= 0)
+            throw std::invalid_argument("Integer quantization bitwidth must be positive");
+        QuantizationType t;
+        t._bitwidth = bitwidth;
+        return t;
+    }
+
+    // "fnuz" formats move the bias by one and use the whole top binade; "fn" formats give up only the all-ones
+    // mantissa of the top binade; IEEE-like formats give up the top binade (QuantizationType.hpp:88-135).
+    static QuantizationType Float(int exponentBits, int mantissaBits, bool finite, bool unsignedZero)
+    {
+        if (exponentBits <= 0)
+            throw std::invalid_argument("Floating-point quantization exponent bits must be positive");
+        if (mantissaBits < 0)
+            throw std::invalid_argument("Floating-point quantization mantissa bits must be non-negative");
+        const int bias    = (1 << (exponentBits - 1)) - 1 + (unsignedZero ? 1 : 0);
+        const double unit = std::ldexp(1.0, -mantissaBits);
+        const int top     = (1 << exponentBits) - ((unsignedZero || finite) ? 1 : 2) - bias;
+        const double man  = (!unsignedZero && finite) ? 2.0 - 2.0 * unit : 2.0 - unit;
+        QuantizationType t;
+        t._isFloat     = true;
+        t._bitwidth    = 1 + exponentBits + mantissaBits;
+        t.exponentBits = exponentBits;
+        t.mantissaBits = mantissaBits;
+        t.exponentMin  = 1 - bias;
+        t.maxValue     = man * std::ldexp(1.0, top);
+        t.finite       = finite;
+        t.unsignedZero = unsignedZero;
+        return t;
+    }
+
+    static QuantizationType Fp8E4M3FN() { return Float(4, 3, true, false); }
+    static QuantizationType Fp8E5M2() { return Float(5, 2, false, false); }
+
+    bool isInt() const { return !_isFloat; }
+    bool isFloat() const { return _isFloat; }
+    int bitwidth() const { return _bitwidth; }
+
+    int exponentBits = 0, mantissaBits = 0, exponentMin = 0;
+    double maxValue  = 0.0;
+    bool finite = false, unsignedZero = false;
+
+private:
+    QuantizationType() = default;
+    bool _isFloat = false;
+    int _bitwidth = 0;
 };
 
 using TensorDim  = int64_t;
@@ -83,7 +140,14 @@ class BlockTensorQuantizer
 {
 public:
     BlockTensorQuantizer(TensorDims shape, int bitwidth, QuantizationMode quantScheme) :
-        isEncodingValid(false), bitwidth(bitwidth), _quantScheme(quantScheme), _shape(std::move(shape))
+        BlockTensorQuantizer(std::move(shape), QuantizationType::Int(bitwidth), quantScheme)
+    {
+    }
+
+    // TensorQuantizer.cpp:22-29.  `bitwidth` is the legacy field setEncodings overwrites; the type stays.
+    BlockTensorQuantizer(TensorDims shape, QuantizationType qtype, QuantizationMode quantScheme) :
+        isEncodingValid(false), bitwidth(qtype.bitwidth()), _quantScheme(quantScheme), _shape(std::move(shape)),
+        _qtype(qtype)
     {
         _numEncodings = 1;
         for (auto d: _shape)
@@ -179,6 +243,8 @@ public:
         Encodings encodings(_numEncodings);
         for (int64_t e = 0; e < _numEncodings; e++)
             encodings[e] = {host[5 * e], host[5 * e + 1], host[5 * e + 2], host[5 * e + 3], static_cast<int>(host[5 * e + 4])};
+        if (_qtype.isFloat())
+            toFp8Encodings(encodings, stream);
         return encodings;
     }
 
@@ -218,6 +284,17 @@ public:
         if (!isEncodingValid)
             throw std::runtime_error("Cannot perform quantization before computing encodings");
         const ahq_layout layout = makeLayout(tensorShape);
+        if (_qtype.isFloat())
+        {
+            if (_qtype.bitwidth() != 8)
+                throw std::runtime_error("BlockTensorQuantizer floating-point QDQ currently supports FP8 qtypes only");
+            if (dtype != AHQ_F32)
+                throw std::runtime_error("BlockTensorQuantizer FP8 QDQ currently supports float tensors only");
+            detail::ahqCheck(ahq_dlq_fp8_qdq(dtype, &layout, input, output, static_cast<const float*>(_encDevice.ptr),
+                                             _qtype.mantissaBits, _qtype.exponentMin, static_cast<float>(_qtype.maxValue),
+                                             stream));
+            return;
+        }
         ahq_grid grid{};
         grid.arith         = AHQ_ARITH_DLQ;
         grid.op            = AHQ_OP_QDQ;
@@ -280,6 +357,7 @@ public:
     bool hasValidStats() const { return _validStats; }
     TensorDims getShape() const { return _shape; }
     Encodings getEncodings() const { return _encodings; }
+    QuantizationType getQuantizationType() const { return _qtype; }
     double getZeroPointShift() const { return _zeroPointShift; }
     void setZeroPointShift(double v) { _zeroPointShift = v; }
 
@@ -287,6 +365,40 @@ public:
     int bitwidth;
 
 private:
+    // TensorQuantizer.cpp:182-224: scale = amax / maxValue, from the raw observed extrema where the analyzer keeps
+    // them (min/max scheme) and they are not all zero, from the analyzer's range otherwise; delta carries the scale.
+    void toFp8Encodings(Encodings& encodings, void* stream) const
+    {
+        if (_qtype.bitwidth() != 8)
+            throw std::runtime_error("BlockTensorQuantizer floating-point encodings currently support FP8 qtypes only");
+        std::vector<float> seenMin, seenMax;
+        if (_quantScheme == QUANTIZATION_TF)
+        {
+            seenMin.resize(_numEncodings);
+            seenMax.resize(_numEncodings);
+            detail::hipCheck(hipMemcpyAsync(seenMin.data(), _min.ptr, sizeof(float) * _numEncodings, hipMemcpyDeviceToHost,
+                                            static_cast<hipStream_t>(stream)), "hipMemcpyAsync");
+            detail::hipCheck(hipMemcpyAsync(seenMax.data(), _max.ptr, sizeof(float) * _numEncodings, hipMemcpyDeviceToHost,
+                                            static_cast<hipStream_t>(stream)), "hipMemcpyAsync");
+            detail::hipCheck(hipStreamSynchronize(static_cast<hipStream_t>(stream)), "hipStreamSynchronize");
+        }
+        for (int64_t e = 0; e < _numEncodings; e++)
+        {
+            TfEncoding& enc = encodings[e];
+            double amax     = std::max(std::abs(enc.min), std::abs(enc.max));
+            if (!seenMin.empty())
+            {
+                const double seen = std::max(std::abs(static_cast<double>(seenMin[e])), std::abs(static_cast<double>(seenMax[e])));
+                if (seen > 0.0)
+                    amax = seen;
+            }
+            if (!(amax > 0))
+                throw std::invalid_argument("FP8 amax must be positive");   // quantization_utils.cpp:186-194
+            const double scale = amax / _qtype.maxValue;
+            enc                = {-scale * _qtype.maxValue, scale * _qtype.maxValue, scale, 0.0, _qtype.bitwidth()};
+        }
+    }
+
     static void requireDevice(bool useCuda)
     {
         if (!useCuda)
@@ -376,6 +488,7 @@ private:
     float _percentile          = 100;
     Encodings _encodings;
     TensorDims _shape;
+    QuantizationType _qtype;
     int64_t _numEncodings = 1;
     detail::DeviceBuffer _min, _max, _xleft, _pdf, _meta, _encDevice;
     mutable detail::DeviceBuffer _workspace, _result;

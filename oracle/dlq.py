@@ -29,6 +29,8 @@ def lib():
         L.dlq_qdq.restype = None
         L.dlq_qdq_broadcast.argtypes = [_f32p, _f32p, _i64p, ctypes.c_int, _i64p, ctypes.c_int, _f64p]
         L.dlq_qdq_broadcast.restype = ctypes.c_int
+        L.dlq_fp8_qdq.argtypes = [_f32p, ctypes.c_uint64, ctypes.c_double, ctypes.c_int, ctypes.c_int, ctypes.c_double, _f32p]
+        L.dlq_fp8_qdq.restype = None
         L.dlq_minmax.argtypes = [_f32p, ctypes.c_uint64, ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_float)]
         L.dlq_minmax.restype = None
         L.dlq_computed_encodings.argtypes = [ctypes.c_int, ctypes.c_double, ctypes.c_double, ctypes.c_int, ctypes.c_int,
@@ -76,6 +78,64 @@ def qdq_broadcast(x, enc_shape, encs):
     if rc:
         raise RuntimeError("Cannot interpret tensor and encoding dimensions as broadcastable")
     return out.reshape(x.shape)
+
+
+def fp8_spec(exponent_bits, mantissa_bits, finite, unsigned_zero):
+    """QuantizationType::Float(exponentBits, mantissaBits, finite, unsignedZero) (QuantizationType.hpp:85-128):
+    returns (bitwidth, mantissa_bits, exponent_min, max_value)."""
+    bias = (1 << (exponent_bits - 1)) - 1 + (1 if unsigned_zero else 0)
+    unit = 2.0 ** -mantissa_bits
+    if unsigned_zero:
+        max_exp, max_man = (1 << exponent_bits) - 1 - bias, 2.0 - unit
+    elif finite:
+        max_exp, max_man = (1 << exponent_bits) - 1 - bias, 2.0 - 2.0 * unit
+    else:
+        max_exp, max_man = (1 << exponent_bits) - 2 - bias, 2.0 - unit
+    return 1 + exponent_bits + mantissa_bits, mantissa_bits, 1 - bias, max_man * 2.0 ** max_exp
+
+
+FP8_E4M3FN = fp8_spec(4, 3, True, False)
+FP8_E5M2 = fp8_spec(5, 2, False, False)
+
+
+def fp8_qdq(x, delta, spec):
+    x = np.asarray(x, dtype=np.float32)
+    out = np.empty(x.size, dtype=np.float32)
+    lib().dlq_fp8_qdq(_f32(x), x.size, float(delta), spec[1], spec[2], float(spec[3]), out)
+    return out.reshape(x.shape)
+
+
+def fp8_qdq_broadcast(x, enc_shape, deltas, spec):
+    """quantizeDequantizeFp8Broadcast (trim_functions.cpp:791-900): every block with its own scale."""
+    x = np.asarray(x, dtype=np.float32)
+    ts = list(x.shape)
+    es = [1] * (len(ts) - len(enc_shape)) + list(enc_shape)
+    split, enc_axes, blk_axes = [], [], []
+    for d, e in zip(ts, es):
+        enc_axes.append(len(split))
+        split.append(e)
+        blk_axes.append(len(split))
+        split.append(d // e)
+    perm = enc_axes + blk_axes
+    blocks = block_view(x, enc_shape)
+    out = np.stack([fp8_qdq(blocks[e], deltas[e], spec) for e in range(blocks.shape[0])])
+    out = out.reshape([split[a] for a in perm]).transpose(np.argsort(perm))
+    return np.ascontiguousarray(out).reshape(x.shape)
+
+
+def fp8_encoding(computed, observed, spec):
+    """The FP8 branch of BlockTensorQuantizer::computeEncodings (TensorQuantizer.cpp:182-224).  computed: the
+    analyzer's (min, max, ...); observed: (min, max) statistics where the analyzer keeps them (min/max scheme),
+    else None.  Returns (min, max, delta, offset, bw)."""
+    amax = max(abs(float(computed[0])), abs(float(computed[1])))
+    if observed is not None:
+        seen = max(abs(float(observed[0])), abs(float(observed[1])))
+        if seen > 0.0:
+            amax = seen
+    if not amax > 0:
+        raise ValueError("FP8 amax must be positive")
+    scale = amax / spec[3]
+    return (-scale * spec[3], scale * spec[3], scale, 0.0, spec[0])
 
 
 def minmax(x):

@@ -83,6 +83,25 @@ int dlq_qdq_broadcast(const float* in, float* out, const int64_t* tshape, int tn
     return 0;
 }
 
+/* ------------------------------------------------------------------ FP8 fake-cast ---------------------------------
+ * fakeCastToFp8<float> (trim_functions.cpp:49-67) under round-to-nearest-even, and quantizeDequantizeFp8Cpu
+ * (trim_functions.cpp:243-258): out = fakeCast(in / scale) * scale, scale = float(encoding.delta). */
+static float fake_cast_fp8(float value, int mantissa_bits, int exponent_min, float max_value) {
+    value = (value < -max_value) ? -max_value : (max_value < value) ? max_value : value; /* std::clamp */
+    int exponent;
+    frexpf(value, &exponent);
+    exponent = (exponent - 1 < exponent_min) ? exponent_min : exponent - 1;
+    const float step = ldexpf(1.0f, exponent - mantissa_bits);
+    return nearbyintf(value / step) * step;
+}
+
+void dlq_fp8_qdq(const float* in, uint64_t cnt, double delta, int mantissa_bits, int exponent_min, double max_value,
+                 float* out) {
+    const float scale = (float)delta;
+    for (uint64_t i = 0; i < cnt; ++i)
+        out[i] = fake_cast_fp8(in[i] / scale, mantissa_bits, exponent_min, (float)max_value) * scale;
+}
+
 /* ------------------------------------------------------------------ min/max statistics ----------------------------
  * GetMin_cpu / GetMax_cpu (math_functions.cpp:324-345): std::min / std::max folds, so NaN never replaces the running
  * value and the minimum starts from FLT_MAX */

@@ -90,7 +90,29 @@ int main()
         BlockTensorQuantizer strict({1, 1, 5, 1}, 8, QUANTIZATION_TF);
         strict.setStrictSymmetric(true);
         strict.updateStats(dIn, {1, 4, 5, 3}, true);
-        printEncodings("tf_strict_symmetric", strict.computeEncodings(true), true);
+        printEncodings("tf_strict_symmetric", strict.computeEncodings(true));
+
+        // FP8: calibrate per channel on the ramp (E4M3FN), quantize-dequantize; E5M2 per tensor with a fixed scale;
+        // the legacy bitwidth field follows setEncodings, the quantization type does not
+        BlockTensorQuantizer fp8({3}, QuantizationType::Fp8E4M3FN(), QUANTIZATION_TF);
+        fp8.updateStats(dIn, {1, 4, 5, 3}, true);
+        Encodings fp8Enc = fp8.computeEncodings(false);
+        fp8.setEncodings(fp8Enc);
+        fp8.quantizeDequantize(dIn, dOut, {1, 4, 5, 3}, true);
+        detail::hipCheck(hipMemcpy(out2.data(), dOut, sizeof(float) * 60, hipMemcpyDeviceToHost), "hipMemcpy");
+        printEncodings("fp8_e4m3_per_channel", fp8Enc);
+        printFloats("fp8_e4m3_per_channel_qdq", out2);
+
+        detail::hipCheck(hipMemcpy(dIn, data4.data(), sizeof(float) * 6000, hipMemcpyHostToDevice), "hipMemcpy");
+        BlockTensorQuantizer e5m2({}, QuantizationType::Fp8E5M2(), QUANTIZATION_TF);
+        e5m2.setEncodings({{-57344.0 * 0.3, 57344.0 * 0.3, 0.3, 0.0, 4}});
+        e5m2.quantizeDequantize(dIn, dOut, {6000}, true);
+        std::vector<float> out3(6000);
+        detail::hipCheck(hipMemcpy(out3.data(), dOut, sizeof(float) * 6000, hipMemcpyDeviceToHost), "hipMemcpy");
+        out3.resize(256);
+        printFloats("fp8_e5m2_qdq_head", out3);
+        std::printf("\"fp8_sticky\": [%d, %d, %d]\n", (int) e5m2.getQuantizationType().isFloat(),
+                    e5m2.getQuantizationType().bitwidth(), e5m2.bitwidth);
         std::printf("}\n");
         (void) hipFree(dIn);
         (void) hipFree(dOut);

@@ -10,6 +10,10 @@ QUANTIZATION_TF = 0
 QUANTIZATION_TF_ENHANCED = 1
 QUANTIZATION_PERCENTILE = 3
 
+# floating-point formats as (exponent bits, mantissa bits, finite, unsigned zero); an int stands for an integer grid
+FP8_E4M3FN = (4, 3, True, False)
+FP8_E5M2 = (5, 2, False, False)
+
 
 def _widen(x: torch.Tensor) -> np.ndarray:
     return x.detach().to(torch.float32).cpu().numpy()
@@ -20,7 +24,8 @@ class OracleQuantizer:
 
     def __init__(self, shape, bitwidth, scheme):
         self.shape = tuple(shape)
-        self.bitwidth = bitwidth
+        self.fp8 = OD.fp8_spec(*bitwidth) if isinstance(bitwidth, tuple) else None
+        self.bitwidth = self.fp8[0] if self.fp8 else bitwidth
         self.scheme = scheme
         self.E = int(np.prod(self.shape)) if self.shape else 1
         self.strict = False
@@ -64,6 +69,14 @@ class OracleQuantizer:
     def computeEncodings(self, symmetric):
         if not self.valid_stats:
             raise RuntimeError("Cannot compute encodings before updating stats")
+        if self.fp8:
+            fp8, self.fp8 = self.fp8, None
+            try:
+                computed = self.computeEncodings(symmetric)
+            finally:
+                self.fp8 = fp8
+            seen = list(zip(self.mn, self.mx)) if self.scheme == QUANTIZATION_TF else [None] * self.E
+            return [OD.fp8_encoding(c, o, fp8) for c, o in zip(computed, seen)]
         if self.scheme == QUANTIZATION_TF:
             return [tuple(OD.minmax_encoding(self.mn[e], self.mx[e], self.bitwidth, symmetric, self.strict, self.unsigned,
                                              self.zps)) for e in range(self.E)]
@@ -91,6 +104,13 @@ class OracleQuantizer:
         if not self.isEncodingValid:
             raise RuntimeError("Cannot perform quantization before computing encodings")
         encs = [[e[0], e[1], e[2], e[3]] for e in self.encodings]
+        if self.fp8:
+            if x.dtype != torch.float32:
+                raise RuntimeError("BlockTensorQuantizer FP8 QDQ currently supports float tensors only")
+            xf = x.numpy()
+            if self.E == 1:
+                return torch.from_numpy(OD.fp8_qdq(xf, encs[0][2], self.fp8))
+            return torch.from_numpy(OD.fp8_qdq_broadcast(xf, self.shape, [e[2] for e in encs], self.fp8))
         xf = _widen(x)
         y = OD.qdq(xf, encs[0]) if self.E == 1 else OD.qdq_broadcast(xf, self.shape, encs)
         return torch.from_numpy(y).to(x.dtype)  # static_cast<DTYPE>(val): round to nearest even
@@ -124,6 +144,8 @@ class HipQuantizer:
         from aimet_amd import dlq
 
         self.dev = torch.device(device)
+        if isinstance(bitwidth, tuple):
+            bitwidth = dlq.QuantizationType.Float(*bitwidth)
         self.q = dlq.BlockTensorQuantizer(shape, bitwidth, scheme, device=self.dev)
         self.scheme = scheme
 

@@ -2,11 +2,14 @@
 `make(shape, bitwidth, scheme)` returns an object with the BlockTensorQuantizer interface of tests/dlq_adapters.py; the
 same checks run on the CPU oracle (pinning it) and on the HIP path."""
 
+import bisect
 import json
 import math
 import os
+from fractions import Fraction
 
 import numpy as np
+import pytest
 import torch
 
 HERE = os.path.dirname(os.path.abspath(__file__))
@@ -347,3 +350,179 @@ def check_percentile(make):
     q.updateStats(torch.zeros(6000))
     (e,) = q.computeEncodings(False)
     assert abs(e[0] + 1.00392) <= 1e-4 and abs(e[1] - 0.996078) <= 1e-4 and e[3] == -128 and e[4] == 8
+
+
+# ------------------------------------------------------------------------------------------------ FP8 fake-cast ----
+# Formats as the adapters take them: (exponent bits, mantissa bits, finite, unsigned zero); torch's storage type of the
+# same format serves as an independent decoder of the 256 bit patterns.
+FP8_FORMATS = {
+    "e4m3fn": ((4, 3, True, False), torch.float8_e4m3fn, 448.0, 3, -6),
+    "e5m2": ((5, 2, False, False), torch.float8_e5m2, 57344.0, 2, -14),
+}
+
+
+def fp8_grid(f8dtype):
+    """The non-negative finite values of the format in increasing order; index == bit pattern."""
+    vals = torch.arange(128, dtype=torch.uint8).view(f8dtype).float()
+    vals = vals[torch.isfinite(vals)]
+    assert torch.all(vals[1:] > vals[:-1])
+    return [Fraction(v) for v in vals.tolist()]
+
+
+def fp8_brute(x, scale, f8dtype):
+    """x / scale and the product with scale in correctly rounded float arithmetic (numpy float32); the cast itself by
+    exact search on the enumerated grid, ties to the even bit pattern, saturating."""
+    grid = fp8_grid(f8dtype)
+    s = np.float32(scale)
+    with np.errstate(all="ignore"):
+        q = (np.asarray(x, dtype=np.float32) / s).astype(np.float32)
+    out = np.empty(q.shape, dtype=np.float32)
+    for i, v in enumerate(q.tolist()):
+        if math.isnan(v):
+            out[i] = np.nan
+            continue
+        a = grid[-1] if math.isinf(v) else min(Fraction(abs(v)), grid[-1])
+        hi = bisect.bisect_left(grid, a)
+        if grid[hi] == a:
+            pick = hi
+        else:
+            lo = hi - 1
+            dl, dh = a - grid[lo], grid[hi] - a
+            pick = lo if dl < dh else hi if dh < dl else (lo if lo % 2 == 0 else hi)
+        out[i] = np.float32(math.copysign(float(grid[pick]), v)) * s
+    return out
+
+
+def _fp8_encoding(scale, max_value):
+    return (-max_value * scale, max_value * scale, scale, 0.0, 8)
+
+
+def _same_floats(got, want):
+    """Bit-for-bit, signs of zero included; NaN matches NaN."""
+    got, want = np.asarray(got, dtype=np.float32).ravel(), np.asarray(want, dtype=np.float32).ravel()
+    nan = np.isnan(want)
+    assert np.array_equal(np.isnan(got), nan)
+    assert np.array_equal(got[~nan].view(np.uint32), want[~nan].view(np.uint32)), \
+        [(i, g, w) for i, (g, w) in enumerate(zip(got, want)) if g != w][:8]
+
+
+def check_fp8_against_torch_cast(make):
+    """Scale 1: inside the finite range the fake-cast is exactly torch's conversion to the storage type and back."""
+    rng = np.random.default_rng(11)
+    for fmt, f8, max_value, _, _ in FP8_FORMATS.values():
+        q = make((), fmt, TF)
+        q.setEncodings([_fp8_encoding(1.0, max_value)])
+        grid = np.array([float(g) for g in fp8_grid(f8)], dtype=np.float32)
+        mids = (grid[1:] + grid[:-1]) / 2  # exact ties
+        near = np.concatenate([np.nextafter(mids, np.float32(0)), np.nextafter(mids, np.float32(np.inf))])
+        rnd = (rng.standard_normal(20000) * np.exp(rng.uniform(-12, math.log(max_value), 20000))).astype(np.float32)
+        tiny = np.array([0.0, 1e-45, 1e-30, float(grid[1]) / 2, float(grid[1]) / 4], dtype=np.float32)
+        x = np.concatenate([grid, mids, near, rnd, tiny])
+        x = np.concatenate([x, -x])
+        x = x[np.abs(x) <= max_value]
+        y = q.quantizeDequantize(torch.from_numpy(x)).numpy()
+        want = torch.from_numpy(x).to(f8).float().numpy()
+        _same_floats(y, want)
+
+
+def check_fp8_edge_cases(make):
+    """The inputs of Fp8QdqCpuGpuBitExactAtEdgeCases (TestTensorQuantizer.cpp:439-510) at its scale 0.3f, against the
+    exact search on the enumerated grid; plus saturation and the sign of zero spelled out."""
+    for fmt, f8, max_value, mbits, emin in FP8_FORMATS.values():
+        f = np.float32
+        scale = f(0.3)
+        mx = f(max_value)
+        step1, sub = f(2.0 ** -mbits), f(2.0 ** (emin - mbits))
+        x = np.array([-np.inf, f(-2) * mx * scale, -mx * scale, -(f(1) + f(1.5) * step1) * scale,
+                      -(f(1) + f(0.5) * step1) * scale, f(-0.5) * sub * scale, -0.0, 0.0, f(0.5) * sub * scale,
+                      (f(1) + f(0.5) * step1) * scale, (f(1) + f(1.5) * step1) * scale, mx * scale, f(2) * mx * scale,
+                      np.inf, np.nan], dtype=np.float32)
+        q = make((), fmt, TF)
+        q.setEncodings([_fp8_encoding(float(scale), max_value)])
+        y = q.quantizeDequantize(torch.from_numpy(x)).numpy()
+        _same_floats(y, fp8_brute(x, scale, f8))
+        assert y[0] == y[1] == -mx * scale and y[-2] == y[-3] == mx * scale
+        assert np.signbit(y[6]) and not np.signbit(y[7]) and y[6] == 0 and y[7] == 0
+        assert np.isnan(y[-1])
+
+
+def check_fp8_reference_tensors(make):
+    """The tensors and encodings of Fp8PerTensorQdq... / Fp8PerChannelQdq... / their E5M2 twins
+    (TestTensorQuantizer.cpp:302-437) against the exact search."""
+    data4 = INPUTS["normal_mean2_std2"]
+    data1 = np.arange(24, dtype=np.float32).reshape(2, 3, 2, 2)
+    for fmt, f8, max_value, _, _ in FP8_FORMATS.values():
+        q = make((), fmt, TF)
+        q.setEncodings([_fp8_encoding(0.5, max_value)])
+        _same_floats(q.quantizeDequantize(torch.from_numpy(data4)).numpy(), fp8_brute(data4, 0.5, f8))
+        q = make((1, 3, 1, 1), fmt, TF)
+        q.setEncodings([_fp8_encoding(0.25 * (c + 1), max_value) for c in range(3)])
+        y = q.quantizeDequantize(torch.from_numpy(data1)).numpy()
+        for c in range(3):
+            _same_floats(y[:, c], fp8_brute(data1[:, c].ravel(), 0.25 * (c + 1), f8))
+        # scales that are not powers of two, blocks along two axes
+        x = (np.random.default_rng(5).standard_normal((4, 6, 8)) * 37).astype(np.float32)
+        q = make((2, 1, 4), fmt, TF)
+        scales = [0.013 * (k + 1) for k in range(8)]
+        q.setEncodings([_fp8_encoding(s, max_value) for s in scales])
+        y = q.quantizeDequantize(torch.from_numpy(x)).numpy()
+        for k in range(8):
+            i, j = divmod(k, 4)
+            blk = (slice(2 * i, 2 * i + 2), slice(None), slice(2 * j, 2 * j + 2))
+            _same_floats(y[blk], fp8_brute(x[blk].ravel(), scales[k], f8))
+
+
+def check_fp8_encodings(make):
+    """TensorQuantizer.cpp:182-224: scale = amax / maxValue from the raw observed extrema under the min/max scheme
+    (the example in the reference's comment: observed 7.25 must not become 7.307), from the analyzer's range
+    otherwise; delta carries the scale, offset is 0, bw 8, min/max = -/+ scale * maxValue."""
+    fmt, _, max_value, _, _ = FP8_FORMATS["e4m3fn"]
+    x = torch.tensor([[-7.25, 1.0, 0.5, 3.0], [0.25, 2.0, 5.5, -1.0]])
+    q = make((), fmt, TF)
+    q.updateStats(x)
+    (e,) = q.computeEncodings(False)
+    assert e[2] == 7.25 / max_value and e[3] == 0.0 and e[4] == 8
+    assert e[0] == -(7.25 / max_value) * max_value and e[1] == (7.25 / max_value) * max_value
+    # per block, E5M2
+    fmt5, _, max5, _, _ = FP8_FORMATS["e5m2"]
+    q = make((2, 1), fmt5, TF)
+    q.updateStats(x)
+    encs = q.computeEncodings(True)
+    assert [e[2] for e in encs] == [7.25 / max5, 5.5 / max5]
+    # all-zero statistics: the observed amax is 0, the analyzer's widened range (MIN_RANGE 0.01) decides
+    q = make((), fmt, TF)
+    q.updateStats(torch.zeros(16))
+    (e,) = q.computeEncodings(False)
+    twin = make((), 8, TF)
+    twin.updateStats(torch.zeros(16))
+    (t,) = twin.computeEncodings(False)
+    assert e[2] == max(abs(t[0]), abs(t[1])) / max_value > 0
+    # histogram schemes keep no raw extrema: the scale follows the searched range
+    data = torch.from_numpy(INPUTS["normal_mean2_std2"])
+    for scheme in (TFE, PCT):
+        q, twin = make((), fmt, scheme), make((), 8, scheme)
+        for z in (q, twin):
+            z.updateStats(data)
+        (e,), (t,) = q.computeEncodings(False), twin.computeEncodings(False)
+        assert e[2] == max(abs(t[0]), abs(t[1])) / max_value and e[3] == 0.0 and e[4] == 8
+    # end to end: calibrate, set, quantize; every output is on the scaled grid and the largest magnitude survives
+    q = make((), fmt, TF)
+    q.updateStats(data)
+    encs = q.computeEncodings(False)
+    q.setEncodings(encs)
+    y = q.quantizeDequantize(data).numpy()
+    amax = np.abs(data.numpy()).max()
+    assert np.abs(y).max() == np.float32(np.float32(448.0) * np.float32(encs[0][2]))
+    assert abs(float(np.abs(y).max()) - float(amax)) <= 1e-6 * float(amax)
+
+
+def check_fp8_qtype_is_sticky(make):
+    """SetEncodingsDoesNotChangeFp8QuantizationType (TestTensorQuantizer.cpp:74-90): the legacy bitwidth field follows
+    the encodings, the quantization type does not; and 16-bit tensors are refused."""
+    fmt, f8, max_value, _, _ = FP8_FORMATS["e4m3fn"]
+    q = make((), fmt, TF)
+    q.setEncodings([(-448.0, 448.0, 1.0, 0.0, 4)])
+    x = torch.tensor([0.3, 1.06, -17.4, 500.0])
+    _same_floats(q.quantizeDequantize(x).numpy(), fp8_brute(x.numpy(), 1.0, f8))
+    with pytest.raises(RuntimeError, match="float tensors only"):
+        q.quantizeDequantize(x.half())

@@ -10,7 +10,7 @@ import pytest
 import torch
 
 from tests import dlq_checks as C
-from tests.dlq_adapters import QUANTIZATION_TF, QUANTIZATION_TF_ENHANCED, OracleQuantizer
+from tests.dlq_adapters import FP8_E4M3FN, FP8_E5M2, QUANTIZATION_TF, QUANTIZATION_TF_ENHANCED, OracleQuantizer
 
 pytestmark = pytest.mark.gpu
 
@@ -50,3 +50,14 @@ def test_facade_program_matches_the_oracle(device):
     s.setStrictSymmetric(True)
     s.updateStats(ramp)
     assert np.array_equal(np.array(out["tf_strict_symmetric"]), np.array(s.computeEncodings(True)))
+
+    f = OracleQuantizer((3,), FP8_E4M3FN, QUANTIZATION_TF)
+    f.updateStats(ramp)
+    encs = f.computeEncodings(False)
+    assert np.array_equal(np.array(out["fp8_e4m3_per_channel"]), np.array(encs))
+    f.setEncodings(encs)
+    assert np.array_equal(np.array(out["fp8_e4m3_per_channel_qdq"], dtype=np.float32), f.quantizeDequantize(ramp).flatten().numpy())
+    g = OracleQuantizer((), FP8_E5M2, QUANTIZATION_TF)
+    g.setEncodings([(-57344.0 * 0.3, 57344.0 * 0.3, 0.3, 0.0, 4)])
+    assert np.array_equal(np.array(out["fp8_e5m2_qdq_head"], dtype=np.float32), g.quantizeDequantize(x)[:256].numpy())
+    assert out["fp8_sticky"] == [1, 8, 4]

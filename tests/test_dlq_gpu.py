@@ -319,3 +319,69 @@ def test_percentile_value_only_exists_for_the_percentile_scheme(device):
     q = HipQuantizer((), 8, QUANTIZATION_PERCENTILE, device)
     q.setPercentileValue(90.0)
     assert q.q.getPercentileValue() == 90.0
+
+
+# ---------------------------------------------------------------------------------------------------- FP8 fake-cast --
+def test_fp8_against_torch_cast(make):
+    C.check_fp8_against_torch_cast(make)
+
+
+def test_fp8_reference_edge_cases(make):
+    C.check_fp8_edge_cases(make)
+
+
+def test_fp8_reference_tensors(make):
+    C.check_fp8_reference_tensors(make)
+
+
+def test_fp8_encodings(make):
+    C.check_fp8_encodings(make)
+
+
+def test_fp8_qtype_is_sticky(make):
+    C.check_fp8_qtype_is_sticky(make)
+
+
+@pytest.mark.parametrize("fmt", ["e4m3fn", "e5m2"])
+@pytest.mark.parametrize("shape,enc_shape", [((1 << 20,), ()), ((1031,), ()), ((64, 3, 40, 9), (1, 3, 1, 1)),
+                                             ((256, 4096), (256, 64)), ((37, 130), (37, 1))])
+def test_fp8_qdq_bit_exact(device, fmt, shape, enc_shape):
+    """Magnitudes from far below the smallest subnormal to beyond saturation, scales of every size (tiny and huge ones
+    take the general division), NaN and infinities: identical bits to the plain-C restatement."""
+    layout = C.FP8_FORMATS[fmt][0]
+    g = torch.Generator().manual_seed(len(shape) * 131 + len(enc_shape))
+    x = torch.randn(shape, generator=g) * torch.exp(torch.rand(shape, generator=g) * 40 - 30)
+    f = x.view(-1)
+    f[1], f[5], f[7], f[11] = float("nan"), float("inf"), float("-inf"), -0.0
+    E = int(np.prod(enc_shape)) if enc_shape else 1
+    scales = torch.exp(torch.rand(E, generator=g, dtype=torch.float64) * 20 - 14).tolist()
+    if E >= 4:
+        scales[0], scales[1], scales[2], scales[3] = 1e-30, 3e25, 1.0, 2.0 ** -70
+    encs = [(-s, s, s, 0.0, 8) for s in scales]
+    hip, ora = HipQuantizer(enc_shape, layout, QUANTIZATION_TF, device), OracleQuantizer(enc_shape, layout, QUANTIZATION_TF)
+    hip.setEncodings(encs)
+    ora.setEncodings(encs)
+    C._same_floats(hip.quantizeDequantize(x).numpy(), ora.quantizeDequantize(x).numpy())
+
+
+def test_fp8_c_abi_rejects_bad_arguments(device):
+    from aimet_amd import _lib
+    from aimet_amd.quantization.affine.backends import hip as H
+
+    lib = _lib.load()
+    x = torch.randn(64, device=device)
+    s = torch.ones(1, device=device)
+    _, layout = H._prepare(x, (), None)
+    st = _lib.current_stream(x.device)
+    args = (x.data_ptr(), x.data_ptr(), s.data_ptr())
+    assert lib.ahq_dlq_fp8_qdq(_lib.DTYPE_CODE[torch.float16], layout, *args, 3, -6, 448.0, st) == _lib.AHQ_ERR_UNSUPPORTED
+    assert b"float tensors only" in lib.ahq_last_error()
+    assert lib.ahq_dlq_fp8_qdq(_lib.DTYPE_CODE[torch.float32], layout, *args, 3, -6, 0.0, st) == _lib.AHQ_ERR_INVALID
+    assert lib.ahq_dlq_fp8_qdq(_lib.DTYPE_CODE[torch.float32], layout, *args, 24, -6, 448.0, st) == _lib.AHQ_ERR_INVALID
+    assert lib.ahq_dlq_fp8_qdq(_lib.DTYPE_CODE[torch.float32], layout, x.data_ptr(), x.data_ptr(), None, 3, -6, 448.0,
+                               st) == _lib.AHQ_ERR_INVALID
+    # in place is allowed, like every element-wise entry point
+    y = x.clone()
+    assert lib.ahq_dlq_fp8_qdq(_lib.DTYPE_CODE[torch.float32], layout, y.data_ptr(), y.data_ptr(), s.data_ptr(), 3, -6,
+                               448.0, st) == _lib.AHQ_OK
+    assert torch.equal(y.cpu(), x.cpu().to(torch.float8_e4m3fn).float())

@@ -47,6 +47,40 @@ def test_percentile_reference_expectations():
     C.check_percentile(make)
 
 
+def test_fp8_against_torch_cast():
+    C.check_fp8_against_torch_cast(make)
+
+
+def test_fp8_reference_edge_cases():
+    C.check_fp8_edge_cases(make)
+
+
+def test_fp8_reference_tensors():
+    C.check_fp8_reference_tensors(make)
+
+
+def test_fp8_encodings():
+    C.check_fp8_encodings(make)
+
+
+def test_fp8_qtype_is_sticky():
+    C.check_fp8_qtype_is_sticky(make)
+
+
+def test_fp8_format_constants():
+    """QuantizationType::Float derives bitwidth, minimum normal exponent and largest value from the layout
+    (QuantizationType.hpp:88-135); the published constants of the four OCP / fnuz formats."""
+    assert OD.fp8_spec(4, 3, True, False) == (8, 3, -6, 448.0)
+    assert OD.fp8_spec(5, 2, False, False) == (8, 2, -14, 57344.0)
+    assert OD.fp8_spec(4, 3, True, True) == (8, 3, -7, 240.0)
+    assert OD.fp8_spec(5, 2, True, True) == (8, 2, -15, 57344.0)
+    for spec, dt in ((OD.FP8_E4M3FN, torch.float8_e4m3fn), (OD.FP8_E5M2, torch.float8_e5m2),
+                     (OD.fp8_spec(4, 3, True, True), torch.float8_e4m3fnuz),
+                     (OD.fp8_spec(5, 2, True, True), torch.float8_e5m2fnuz)):
+        info = torch.finfo(dt)
+        assert info.max == spec[3] and info.smallest_normal == 2.0 ** spec[2]
+
+
 def test_percentile_matches_numpy_quantiles():
     """Closed form: the chosen range brackets the empirical quantiles to within two buckets."""
     x = C.INPUTS["normal_mean2_std2_100k"]
