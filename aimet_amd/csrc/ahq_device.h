@@ -1,6 +1,7 @@
 // Device-side helpers shared by all kernels (gfx950, wave64).
 #pragma once
 
+#include <type_traits>
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -31,7 +32,12 @@ __device__ __forceinline__ float load_f32(bf16_t v) { return bits_to_f32((uint32
 
 // Round-to-nearest-even narrowing (one v_cvt_pk_bf16_f32 / v_cvt_f16_f32 each on gfx950).
 __device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) { return __builtin_bit_cast(uint16_t, (__bf16)f); }
-__device__ __forceinline__ uint16_t f32_to_f16_bits(float f) { return __builtin_bit_cast(uint16_t, (_Float16)f); }
+// The value passes through an empty asm statement first: without it the compiler merges a preceding multiplication
+// into v_fma_mixlo_f16 with a +0 addend, which turns a product of -0 into +0.
+__device__ __forceinline__ uint16_t f32_to_f16_bits(float f) {
+    asm("" : "+v"(f));
+    return __builtin_bit_cast(uint16_t, (_Float16)f);
+}
 
 template <typename T> __device__ __forceinline__ T store_cast(float v);
 template <> __device__ __forceinline__ float store_cast<float>(float v) { return v; }
@@ -41,8 +47,18 @@ template <> __device__ __forceinline__ bf16_t store_cast<bf16_t>(float v) { retu
 // Round a float to the compute dtype and widen it again ("every intermediate is rounded to D").
 template <int CD> __device__ __forceinline__ float rnd(float v);
 template <> __device__ __forceinline__ float rnd<AHQ_F32>(float v) { return v; }
-template <> __device__ __forceinline__ float rnd<AHQ_F16>(float v) { return (float)(_Float16)v; }
+template <> __device__ __forceinline__ float rnd<AHQ_F16>(float v) { return (float)__builtin_bit_cast(_Float16, f32_to_f16_bits(v)); }
 template <> __device__ __forceinline__ float rnd<AHQ_BF16>(float v) { return bits_to_f32((uint32_t)f32_to_bf16_bits(v) << 16); }
+
+// Round to the compute dtype CD, then narrow to the storage type: one conversion when the two formats coincide.
+template <typename IO, int CD>
+__device__ __forceinline__ IO store_rounded(float v) {
+    if constexpr (CD == AHQ_F32 || (CD == AHQ_BF16 && std::is_same<IO, bf16_t>::value) ||
+                  (CD == AHQ_F16 && std::is_same<IO, f16_t>::value))
+        return store_cast<IO>(v);
+    else
+        return store_cast<IO>(rnd<CD>(v));
+}
 
 // ------------------------------------------------------------------------------------------- 16-byte vector I/O --
 template <typename T, int N> struct alignas(sizeof(T) * N) Pack { T v[N]; };

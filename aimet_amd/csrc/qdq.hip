@@ -67,28 +67,69 @@ __device__ __forceinline__ float safe_reciprocal(float s) {
 // output value (already rounded to the compute dtype) and whether the code was in range; bwd() returns the three
 // per-element gradient terms.
 
+// Largest integer magnitude n such that every integer up to n + 1 is a value of the compute dtype.
+template <int CD> struct ExactInt { static constexpr float kMax = 16777215.f; };
+template <> struct ExactInt<AHQ_F16> { static constexpr float kMax = 2047.f; };
+template <> struct ExactInt<AHQ_BF16> { static constexpr float kMax = 255.f; };
+
+// The FAST form (no zero-point shift) needs more than a divisible scale: an integer offset, and grid bounds, offset
+// and shifted bounds lo = offset + qmin, hi = offset + qmax small enough that every integer the reference's
+// intermediate steps can produce near the grid is exact in the compute dtype.  Then
+//   r = rnd(rint(t) - offset) is in [qmin, qmax]  <=>  lo <= rint(t) <= hi        (integers, roundings monotone and
+//                                                                                   exact up to one past the bounds)
+//   rnd(clamp(r) + offset) = clamp(rint(t), lo, hi)
+// so the subtraction, the addition and two of the roundings drop out, and the clamp is one median-of-three.  The
+// median does not propagate NaN: tiles holding a NaN take the general form (lane_can_divide_fast).  Encodings that do
+// not qualify get rs = 0, which sends their tile to the general form too.
 template <int CD, bool ZPS>
 struct MathAutogradQdq {
     static constexpr int kNP = 2;
+    static constexpr int kCD = CD;
     static constexpr bool kDiv = true;
     static constexpr bool kHasBwd = true;
-    __device__ static EncP prep(float s, float off, float, float, const GridC&) {
-        const float sr = rnd<CD>(s);
-        return {sr, rnd<CD>(off), 0.f, 0.f, safe_reciprocal(sr)};
+    __device__ static EncP prep(float s, float off, float, float, const GridC& g) {
+        const float sr = rnd<CD>(s), offr = rnd<CD>(off);
+        float rs = safe_reciprocal(sr);
+        if (!ZPS) {
+            constexpr float K = ExactInt<CD>::kMax;
+            const float lo = offr + g.qmin, hi = offr + g.qmax;
+            const bool small = (offr == __builtin_rintf(offr)) & (__builtin_fabsf(offr) <= K) &
+                               (__builtin_fabsf(g.qmin) <= K) & (__builtin_fabsf(g.qmax) <= K) &
+                               (__builtin_fabsf(lo) <= K) & (__builtin_fabsf(hi) <= K);
+            if (!small) rs = 0.f;
+        }
+        return {sr, offr, 0.f, 0.f, rs};
     }
+    // Returns the output before its last rounding to the compute dtype (the caller rounds while storing).
     template <bool FAST>
     __device__ static float fwd(float x, const EncP& e, const GridC& g, bool& inr) {
         float t = rnd<CD>(divide<FAST, CD>(x, e.p0, e.rs));
+        if (FAST && !ZPS) {
+            const float xr = __builtin_rintf(t);
+            const float m = __builtin_amdgcn_fmed3f(xr, e.p1 + g.qmin, e.p1 + g.qmax);
+            inr = (m == xr);
+            return (m + 0.f) * e.p0;  // the reference's (q + offset) is never a negative zero
+        }
         if (ZPS) t = rnd<CD>(t - g.zps);
         const float r = rnd<CD>(__builtin_rintf(t) - e.p1);
         inr = (r >= g.qmin) & (r <= g.qmax);
         const float q = r < g.qmin ? g.qmin : (r > g.qmax ? g.qmax : r);
         const float offp = ZPS ? rnd<CD>(e.p1 + g.zps) : e.p1;
-        return rnd<CD>(rnd<CD>(q + offp) * e.p0);
+        return rnd<CD>(q + offp) * e.p0;
     }
     template <bool FAST>
     __device__ static void bwd(float gr, float x, const EncP& e, const GridC& g, float& gx, float& gs, float& goff) {
         float t = rnd<CD>(divide<FAST, CD>(x, e.p0, e.rs));
+        if (FAST && !ZPS) {
+            const float xr = __builtin_rintf(t);
+            const float m = __builtin_amdgcn_fmed3f(xr, e.p1 + g.qmin, e.p1 + g.qmax);
+            const bool in = (m == xr);
+            // rint(t) - t is a multiple of ulp(t) no larger than 1/2: exact in the compute dtype, no rounding needed
+            gx = in ? gr : 0.f;
+            gs = rnd<CD>(gr * (in ? xr - t : m));
+            goff = in ? 0.f : rnd<CD>(gr * e.p0);
+            return;
+        }
         if (ZPS) t = rnd<CD>(t - g.zps);
         const float xr = __builtin_rintf(t);
         const float err = rnd<CD>(xr - t);
@@ -106,6 +147,7 @@ struct MathAutogradQdq {
 template <int CD>
 struct MathAutogradQuantize {
     static constexpr int kNP = 2;
+    static constexpr int kCD = AHQ_F32;  // its outputs are already values of CD
     static constexpr bool kDiv = true;
     static constexpr bool kHasBwd = true;
     __device__ static EncP prep(float s, float off, float, float, const GridC&) {
@@ -133,13 +175,14 @@ struct MathAutogradQuantize {
 template <int CD>
 struct MathAutogradDequantize {
     static constexpr int kNP = 2;
+    static constexpr int kCD = CD;
     static constexpr bool kDiv = false;
     static constexpr bool kHasBwd = true;
     __device__ static EncP prep(float s, float off, float, float, const GridC&) { return {rnd<CD>(s), rnd<CD>(off), 0.f, 0.f, 0.f}; }
     template <bool FAST>
     __device__ static float fwd(float x, const EncP& e, const GridC&, bool& inr) {
         inr = true;
-        return rnd<CD>(rnd<CD>(x + e.p1) * e.p0);
+        return rnd<CD>(x + e.p1) * e.p0;  // last rounding by the caller
     }
     template <bool FAST>
     __device__ static void bwd(float gr, float x, const EncP& e, const GridC&, float& gx, float& gs, float& goff) {
@@ -150,6 +193,7 @@ struct MathAutogradDequantize {
 };
 
 struct MathAten {
+    static constexpr int kCD = AHQ_F32;
     static constexpr int kNP = 3;
     static constexpr bool kDiv = false;
     static constexpr bool kHasBwd = true;
@@ -173,6 +217,7 @@ struct MathAten {
 };
 
 struct MathDlq {
+    static constexpr int kCD = AHQ_F32;
     static constexpr int kNP = 4;
     static constexpr bool kDiv = true;
     static constexpr bool kHasBwd = false;
@@ -200,6 +245,7 @@ struct MathDlq {
 // y = rint(v / step) * step * scale.  The grid constants travel in GridC: qmin = exponent_min, qmax = max value,
 // zps = mantissa bits.  Dividing by a power of two is exact, so it is done by scaling the exponent.
 struct MathDlqFp8 {
+    static constexpr int kCD = AHQ_F32;
     static constexpr int kNP = 2;
     static constexpr bool kDiv = true;
     static constexpr bool kHasBwd = false;
@@ -288,7 +334,7 @@ __device__ __forceinline__ bool lane_can_divide_fast(const QdqArgs& a, const Til
         if (FULL || lv < t.nv) {
             ok &= sp[M::kNP][stage_index(a, t, lv)] != 0.f;
 #pragma unroll
-            for (int k = 0; k < VEC; ++k) ok &= !(__builtin_fabsf(load_f32(in[u].v[k])) > kFastDivMax);
+            for (int k = 0; k < VEC; ++k) ok &= __builtin_fabsf(load_f32(in[u].v[k])) <= kFastDivMax;  // NaN: general form
         }
     }
     return ok;
@@ -308,7 +354,7 @@ __device__ __forceinline__ void fwd_math(const QdqArgs& a, const Tile& t, float 
             for (int k = 0; k < VEC; ++k) {
                 bool inr;
                 const float r = M::template fwd<FAST>(load_f32(in[u].v[k]), e, a.gc, inr);
-                out.v[k] = store_cast<IO>(r);
+                out.v[k] = store_rounded<IO, M::kCD>(r);
                 mk.v[k] = inr ? 1 : 0;
             }
             store_pack<IO, VEC>(y + (int64_t)lv * VEC, out);
@@ -353,7 +399,7 @@ __global__ __launch_bounds__(kBlock) void qdq_fwd_kernel(const QdqArgs a) {
             const EncP e = staged<M>(sp, 0);
             bool inr;
             const float r = M::template fwd<false>(load_f32(x[i]), e, a.gc, inr);
-            y[i] = store_cast<IO>(r);
+            y[i] = store_rounded<IO, M::kCD>(r);
             if (a.mask) a.mask[i] = inr ? 1 : 0;
         }
     }
@@ -367,7 +413,7 @@ __global__ __launch_bounds__(kBlock) void qdq_fwd_generic_kernel(const QdqArgs a
         const EncP e = load_enc<M>(a, generic_enc_index(a, i));
         bool inr;
         const float r = M::template fwd<false>(load_f32(x[i]), e, a.gc, inr);
-        y[i] = store_cast<IO>(r);
+        y[i] = store_rounded<IO, M::kCD>(r);
         if (a.mask) a.mask[i] = inr ? 1 : 0;
     }
 }

@@ -4,12 +4,12 @@ import torch
 
 
 def assert_same_bits(actual: torch.Tensor, expected: torch.Tensor, what: str = ""):
-    """Bit-exact comparison (NaN == NaN, +0 == -0 as torch.equal treats them)."""
+    """Bit-exact comparison, signs of zero included (any NaN matches any NaN)."""
     a = actual.detach().cpu()
     e = expected.detach().cpu()
     assert a.shape == e.shape, f"{what}: shape {tuple(a.shape)} vs {tuple(e.shape)}"
     assert a.dtype == e.dtype, f"{what}: dtype {a.dtype} vs {e.dtype}"
-    same = (a == e) | (a.isnan() & e.isnan())
+    same = ((a == e) & (torch.signbit(a) == torch.signbit(e))) | (a.isnan() & e.isnan())
     if not bool(same.all()):
         bad = (~same).nonzero()
         i = tuple(bad[0].tolist())

@@ -344,3 +344,63 @@ def test_huge_inputs_and_scales_take_the_general_division(device):
     got = affine.quantize_dequantize(x.to(device), sd, offset.to(device), -128, 127).detach().cpu()
     ref = O.qdq_v2_forward(x, scale, offset, -128, 127).y
     assert_same_bits(got, ref)
+
+
+# (compute dtype, tensor dtype, qmin, qmax, offsets): grids and offsets on both sides of the limits up to which the
+# kernels may work on rint(x / scale) directly (integer offset; bounds, offset and shifted bounds at most 255 in
+# bfloat16, 2047 in float16, 2^24 - 1 in float32 arithmetic); rows that do not qualify take the step-by-step form
+_SHORTCUT_CASES = [
+    (torch.bfloat16, torch.bfloat16, 0, 255, [0.0, -100.0, -255.0, -254.0, 1.0, 0.5, -128.5, 37.0]),
+    (torch.bfloat16, torch.bfloat16, -128, 127, [-128.0, -127.0, 127.0, 128.0, 0.0, 0.25, 300.0, -300.0]),
+    (torch.bfloat16, torch.bfloat16, -256, 255, [0.0, 1.0, -1.0, 16.0]),
+    (torch.bfloat16, torch.bfloat16, -8, 7, [0.0, 247.0, 248.0, 249.0, -247.0, -248.0, 0.75, -8.0]),
+    (torch.float16, torch.float16, 0, 2047, [0.0, -2047.0, -1000.0, 1.0, -0.5, 3.0, -2046.0, 0.125]),
+    (torch.float16, torch.float16, -1024, 1023, [0.0, 1024.0, 1025.0, -1023.0, -1024.0, 512.5, 7.0, -7.0]),
+    (torch.float32, torch.bfloat16, -32768, 32767, [0.0, -32768.0, 0.5, 123.0, 16777215.0, 16744448.0, -16777216.0, 8.0]),
+    (torch.float32, torch.float32, 0, 65535, [0.0, -65535.0, 0.5, 16711680.0, 16711681.0, -0.25, 77.0, -16777215.0]),
+]
+
+
+@pytest.mark.parametrize("case", _SHORTCUT_CASES, ids=lambda c: f"{str(c[0])[6:]}_{str(c[1])[6:]}_{c[2]}_{c[3]}")
+def test_small_integer_grid_shortcut_limits(device, monkeypatch, case):
+    """Outputs, masks-as-gradients and parameter gradients with the arithmetic dtype forced, at codes one and two
+    steps either side of both grid ends, at rounding ties, far outside, and with NaN / infinities in some rows."""
+    from aimet_amd import _lib
+    from aimet_amd.quantization.affine.backends import hip as H
+
+    cd, dtype, qmin, qmax, offsets = case
+    monkeypatch.setattr(O, "internal_dtype", lambda *a: cd)
+    R, K = len(offsets), 4096
+    g = torch.Generator().manual_seed(R * 31 + qmax)
+    scale = (torch.rand(R, 1, generator=g) * 0.05 + 0.002).to(cd).float()
+    offset = torch.tensor(offsets).reshape(R, 1)
+    off_cd = offset.to(cd).float()
+    lo, hi = off_cd + qmin, off_cd + qmax
+    # codes around both ends of each row's grid, ties and near-ties, ordinary values, far outliers
+    j = torch.arange(K).reshape(1, K)
+    around = torch.where(j % 2 == 0, lo, hi) + ((j // 2) % 9 - 4).float()
+    frac = torch.tensor([0.0, 0.5, -0.5, 0.25, 0.499, -0.499, 0.75, 0.0])[(j // 18) % 8]
+    t = around + frac
+    t[:, K // 2:] = (torch.rand(R, K - K // 2, generator=g) - 0.5) * (hi - lo + 40) + (hi + lo) / 2
+    x = t * scale
+    x[:, -1], x[:, -2], x[:, -3] = 1e30, -1e30, 0.0
+    x[1, 5], x[1, 6], x[2, 7] = float("nan"), float("inf"), float("-inf")
+    x = x.to(dtype)
+    grad = torch.randn(R, K, generator=g).to(dtype)
+
+    tr = O.qdq_v2_forward(x, scale, offset, qmin, qmax)
+    gx_ref, gs_ref, go_ref = O.qdq_v2_backward(grad, x, scale, offset, qmin, qmax)
+    assert tr.dtype == cd
+
+    xd = x.to(device).requires_grad_(True)
+    sd = scale.to(device).requires_grad_(True)
+    od = offset.to(device).requires_grad_(True)
+    y = H._apply(xd, sd, od, _lib.AHQ_ARITH_AUTOGRAD, _lib.AHQ_OP_QDQ, cd, qmin, qmax, None, 0.0)
+    assert_same_bits(y, tr.y, "output")
+    y.backward(grad.to(device))
+    assert_same_bits(xd.grad, gx_ref, "input gradient")
+    tol = _tol(cd)
+    finite_rows = torch.tensor([r not in (1, 2) for r in range(R)])  # NaN / inf rows: the sums are NaN on both sides
+    assert_close_rel(sd.grad[finite_rows], gs_ref[finite_rows], tol, "scale gradient", abs_floor=1e-30)
+    assert_close_rel(od.grad[finite_rows], go_ref[finite_rows], tol, "offset gradient", abs_floor=1e-30)
+    assert bool((sd.grad[~finite_rows].cpu().isnan() == gs_ref[~finite_rows].isnan()).all())
