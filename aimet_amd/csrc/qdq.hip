@@ -24,7 +24,10 @@ constexpr int kStage = kTileVec + 2;  // most encodings a tile can touch
 
 struct GridC {
     float qmin, qmax, zps;
+    int flags;  // float fake-cast only: kCastOverflowNaN | kCastUnsignedZero
 };
+constexpr int kCastOverflowNaN = 1;    // a value that rounds past the largest one becomes NaN (else infinity)
+constexpr int kCastUnsignedZero = 2;   // the format has no negative zero
 
 struct EncP {
     float p0, p1, p2, p3;
@@ -265,6 +268,48 @@ struct MathDlqFp8 {
     }
     template <bool FAST>
     __device__ static void bwd(float, float, const EncP&, const GridC&, float& gx, float& gs, float& goff) { gx = gs = goff = 0.f; }
+};
+
+// aimet_torch's float fake-cast (quantization/float/quantizer.py:634-716): in the arithmetic dtype CD of the call,
+//   t = x / scale;  t = clamp(t, -max, max);  v = t rounded to the simulated format and brought back to CD;
+//   y = v * scale.
+// The simulated format is given by its mantissa bits, the exponent of its smallest normal binade and its largest
+// value (GridC: zps, qmin, qmax); rounding is to nearest even on that grid, exactly what a conversion to a storage
+// type of that layout does and what the reference's logarithm-based formula evaluates to
+// (fp_quantization.py:148-214).  The clamp bound is the largest value as CD holds it, like the Python scalar the
+// reference hands to torch.clamp; where that rounds upward (65504 in bfloat16) a clamped value can round past the
+// format's largest value and overflows like the conversion would.
+template <int CD>
+struct MathFloatCast {
+    static constexpr int kCD = CD;
+    static constexpr int kNP = 2;
+    static constexpr bool kDiv = true;
+    static constexpr bool kHasBwd = false;
+    // The scale stays a float whatever CD is: a float32 scale with one element per tensor is an operand torch keeps
+    // at full precision next to a 16-bit tensor (and any larger float32 scale widens the whole computation), so the
+    // quotient is the correctly rounded float one, rounded once more to CD.
+    __device__ static EncP prep(float s, float, float, float, const GridC&) { return {s, 0.f, 0.f, 0.f, safe_reciprocal(s)}; }
+    template <bool FAST>
+    __device__ static float fwd(float x, const EncP& e, const GridC& g, bool& inr) {
+        inr = true;
+        float t = rnd<CD>(divide<FAST, AHQ_F32>(x, e.p0, e.rs));
+        // the corrected quotient of divide<true> does not keep the sign of a zero
+        if (FAST && t == 0.f) t = bits_to_f32((f32_to_bits(x) ^ f32_to_bits(e.p0)) & 0x80000000u);
+        const float mx = rnd<CD>(g.qmax);
+        t = (t < -mx) ? -mx : (mx < t) ? mx : t;
+        int ex = __builtin_amdgcn_frexp_expf(t) - 1;
+        ex = ex < (int)g.qmin ? (int)g.qmin : ex;
+        const int sh = ex - (int)g.zps;
+        float v = __builtin_ldexpf(__builtin_rintf(__builtin_ldexpf(t, -sh)), sh);
+        if (__builtin_fabsf(v) > g.qmax)
+            v = (g.flags & kCastOverflowNaN) ? __builtin_nanf("") : __builtin_copysignf(__builtin_inff(), v);
+        if ((g.flags & kCastUnsignedZero) && v == 0.f) v = 0.f;
+        return rnd<CD>(v) * e.p0;  // last rounding by the caller
+    }
+    template <bool FAST>
+    __device__ static void bwd(float, float, const EncP&, const GridC&, float& gx, float& gs, float& goff) {
+        gx = gs = goff = 0.f;
+    }
 };
 
 // ------------------------------------------------------------------------------------------------ kernel arguments --
@@ -627,6 +672,7 @@ static void fill_args(const ahq_grid& grid, const Plan& p, QdqArgs* a) {
     a->gc.qmin = (float)grid.qmin;
     a->gc.qmax = (float)grid.qmax;
     a->gc.zps = (float)grid.zero_point_shift;
+    a->gc.flags = 0;
     a->red = p.red;
     a->out_cd = grid.compute_dtype;
 }
@@ -768,6 +814,36 @@ extern "C" int ahq_dlq_fp8_qdq(int32_t dtype, const ahq_layout* layout, const vo
     hipStream_t st = static_cast<hipStream_t>(stream);
     launch_fwd<float, MathDlqFp8>(p, a, st);
     return check_launch("ahq_dlq_fp8_qdq");
+}
+
+extern "C" int ahq_float_qdq(int32_t dtype, const ahq_layout* layout, const void* x, void* y, const float* scale,
+                             int32_t mantissa_bits, int32_t exponent_min, float max_value, int32_t overflow_to_nan,
+                             int32_t unsigned_zero, void* stream) {
+    if (dtype < AHQ_F32 || dtype > AHQ_BF16) return set_error("bad dtype"), AHQ_ERR_INVALID;
+    if (!layout) return set_error("layout is null"), AHQ_ERR_INVALID;
+    if (!scale) return set_error("scale is null"), AHQ_ERR_INVALID;
+    if (mantissa_bits < 0 || mantissa_bits > 23 || exponent_min < -126 || exponent_min > 127 || !(max_value > 0.f))
+        return set_error("bad float format description"), AHQ_ERR_INVALID;
+    Plan p;
+    if (!make_plan(dtype, *layout, aligned16(x) && aligned16(y), false, &p)) return AHQ_ERR_INVALID;
+    if (p.cl.numel == 0) return AHQ_OK;
+    if (!x || !y) return set_error("x or y is null"), AHQ_ERR_INVALID;
+    QdqArgs a{};
+    a.x = x;
+    a.y = y;
+    a.scale = scale;
+    ahq_grid grid{};
+    grid.compute_dtype = dtype;
+    fill_args(grid, p, &a);
+    a.gc.qmin = (float)exponent_min;
+    a.gc.qmax = max_value;
+    a.gc.zps = (float)mantissa_bits;
+    a.gc.flags = (overflow_to_nan ? kCastOverflowNaN : 0) | (unsigned_zero ? kCastUnsignedZero : 0);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (dtype == AHQ_F32) launch_fwd<float, MathFloatCast<AHQ_F32>>(p, a, st);
+    else if (dtype == AHQ_F16) launch_fwd<f16_t, MathFloatCast<AHQ_F16>>(p, a, st);
+    else launch_fwd<bf16_t, MathFloatCast<AHQ_BF16>>(p, a, st);
+    return check_launch("ahq_float_qdq");
 }
 
 extern "C" size_t ahq_qdq_backward_workspace_bytes(const ahq_grid* grid, const ahq_layout* layout, int want_param_grads) {

@@ -297,8 +297,9 @@ class MinMaxEncodingAnalyzer(EncodingAnalyzer[_MinMaxRange]):
         pair of same-shaped 16/32-bit float tensors, in which case the elementwise formulation runs."""
         mn, mx = stats.min, stats.max
         if (mn.dtype not in _lib.DTYPE_CODE or mx.dtype != mn.dtype or mn.shape != mx.shape or not mn.is_cuda
-                or num_steps > (1 << 24)):
+                or num_steps > (1 << 24) or num_steps != int(num_steps)):
             return None
+        num_steps = int(num_steps)  # callers may hand over 2.0 ** bitwidth - 1
         dt = mn.dtype
         tiny = _get_minimum_scale(num_steps)
         consts = _scalar_constants(dt, tiny)

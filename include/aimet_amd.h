@@ -244,6 +244,20 @@ int    ahq_dlq_tfe_encodings(const ahq_dlq_pdf_state* state, int32_t bw, int32_t
 int ahq_dlq_fp8_qdq(int32_t dtype, const ahq_layout* layout, const void* x, void* y, const float* scale,
                     int32_t mantissa_bits, int32_t exponent_min, float max_value, void* stream);
 
+/* Replaces _float_quantize_dequantize of aimet_torch (aimet_torch/quantization/float/quantizer.py:634-716, with
+ * _cast_decast :709-710 and fake_cast_to_ieee_float, aimet_torch/fp_quantization.py:148-214): in the arithmetic of
+ * `dtype` (x, y and every intermediate), y = cast(clamp(x / scale, -max_value, max_value)) * scale, where cast rounds
+ * to nearest even onto the floating-point grid with `mantissa_bits` explicit mantissa bits whose smallest normal
+ * binade starts at 2^exponent_min, and max_value is the largest value of the simulated format.  overflow_to_nan: what
+ * a value that still rounds past max_value becomes (1: NaN, as the "fn" / "fnuz" storage types do; 0: infinity).
+ * unsigned_zero: the format has no negative zero.  scale: one float per encoding of the layout, used at float
+ * precision (quotient and product are formed in float and rounded once to `dtype`), which is how torch treats a
+ * one-element float32 operand next to a 16-bit tensor.
+ */
+int ahq_float_qdq(int32_t dtype, const ahq_layout* layout, const void* x, void* y, const float* scale,
+                  int32_t mantissa_bits, int32_t exponent_min, float max_value, int32_t overflow_to_nan,
+                  int32_t unsigned_zero, void* stream);
+
 /* Replaces PercentileEncodingAnalyzer::computeEncoding (DLQ/src/PercentileEncodingAnalyzer.cpp:52-169) on the same PDF
  * statistics: the range that keeps `percentile` percent of the probability mass on each side, widened to contain
  * zero, then getComputedEncodings.  out: [num_slots][5].

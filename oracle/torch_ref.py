@@ -607,3 +607,66 @@ def sqnr_encodings(stats: List[Hist], shape, num_steps, symmetric, *, asym_delta
     lo = lo.to(stats[0].min.dtype)
     hi = hi.to(stats[0].max.dtype)
     return lo.view(shape), hi.view(shape), delta, off, torch.cat(bi)
+
+
+# --------------------------------------------------------------------------- #
+# Float fake-cast (quantization/float/quantizer.py:634-716, fp_quantization.py:148-214)
+# --------------------------------------------------------------------------- #
+FLOAT_TORCH_DTYPES = {
+    (5, 10, False, False): torch.float16,
+    (8, 7, False, False): torch.bfloat16,
+    (4, 3, True, False): torch.float8_e4m3fn,
+    (4, 3, True, True): torch.float8_e4m3fnuz,
+    (5, 2, False, False): torch.float8_e5m2,
+    (5, 2, True, True): torch.float8_e5m2fnuz,
+}
+
+
+def float_max(exponent_bits, mantissa_bits, finite, unsigned_zero) -> float:
+    """_finfo.max (float/_finfo.py:66-86)."""
+    key = (exponent_bits, mantissa_bits, finite, unsigned_zero)
+    if key in FLOAT_TORCH_DTYPES:
+        return torch.finfo(FLOAT_TORCH_DTYPES[key]).max
+    if key == (2, 1, True, False):
+        return 6.0
+    if not finite and not unsigned_zero:
+        exponent_max = 2 ** exponent_bits - 1
+        return (2 - 2 ** -mantissa_bits) * 2 ** (exponent_max - exponent_max // 2 - 1)
+    raise RuntimeError("Maximum representable value of this format is unknown")
+
+
+def fake_cast_to_ieee_float(x, maxval, exponent_bits, mantissa_bits, finite=True):
+    """fp_quantization.py:148-214, for a tensor x and a Python-float maxval."""
+    import numpy as np
+
+    maxval = torch.tensor(maxval, dtype=torch.float64)
+    bias = 2 ** exponent_bits - torch.log2(maxval) + np.log2(2 - 2 ** (-mantissa_bits)) - 1
+    xc = x.clamp(-maxval, maxval)
+    log_scales = torch.floor(torch.log2(torch.abs(xc)) + bias).detach()
+    log_scales = torch.clamp(log_scales, 1.0)
+    scales = 2.0 ** (log_scales - mantissa_bits - bias)
+    out = torch.round(xc / scales) * scales
+    if not finite:
+        out = torch.where(x.isinf(), x, out)
+    return out.to(x.dtype)
+
+
+def float_qdq(x, scale, exponent_bits, mantissa_bits, finite, unsigned_zero, block_size=None):
+    """_float_quantize_dequantize (float/quantizer.py:634-716): divide, clamp, fake-cast, multiply, every step a torch
+    op on the promoted dtype of (x, scale)."""
+    key = (exponent_bits, mantissa_bits, finite, unsigned_zero)
+    mx = float_max(*key)
+    shape = x.shape
+    xb, sb, _ = _blocked_views(x, scale, None, block_size)
+    t = torch.div(xb, sb).reshape(shape) if block_size else torch.div(x, scale)
+    t = t.clamp(-mx, mx)
+    if key in FLOAT_TORCH_DTYPES:
+        t = t.to(FLOAT_TORCH_DTYPES[key]).to(t.dtype)
+    elif not unsigned_zero:
+        t = fake_cast_to_ieee_float(t, mx, exponent_bits, mantissa_bits, finite=finite)
+    else:
+        raise NotImplementedError("Fake-casting to this format is not implemented")
+    if block_size:
+        tb, sb, _ = _blocked_views(t, scale, None, block_size)
+        return torch.mul(tb, sb).reshape(shape)
+    return torch.mul(t, scale)
