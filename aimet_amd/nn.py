@@ -6,6 +6,9 @@ quantizer; ``compute_encodings()`` calibrates the weight quantizer from the weig
 quantizers into observe-and-pass-through mode (nn/base.py:392-427); outside that context the forward pass
 quantize-dequantizes input, weight and output.  The GEMM itself is ``torch.nn.functional.linear``.
 
+``fold_param_quantizers`` / ``inference_mode`` are the two ways the reference avoids re-quantizing weights on every
+forward pass (nn/base.py:1103-1151, utils.py:1653-1684).
+
 Not reproduced: the lossless decomposition of an already-quantized weight (``_decompose_prequantized_tensor``,
 aimet_torch/utils.py:2024-2300).  Only its early exit is -- a weight whose first blocks hold more distinct magnitudes
 than the grid has levels goes straight to min/max calibration, which is what happens for every trained or random
@@ -22,11 +25,12 @@ import torch
 from torch import nn
 from torch.nn import functional as F
 
-from aimet_amd.quantization._utils import concretize_block_size
+from aimet_amd.quantization._utils import concretize_block_size, patch_attr
 from aimet_amd.quantization.affine.quantizer import AffineQuantizerBase, GroupedBlockQuantizeDequantize
 from aimet_amd.quantization.base.quantizer import QuantizerBase
 
-__all__ = ["QuantizedLinear", "compute_encodings", "quantized_linears"]
+__all__ = ["QuantizedLinear", "compute_encodings", "quantized_linears", "fold_param_quantizers", "inference_mode",
+           "remove_param_quantizers"]
 
 
 def _may_be_prequantized(param: torch.Tensor, qtzr: AffineQuantizerBase):
@@ -124,6 +128,49 @@ class QuantizedLinear(nn.Linear):
             with qtzr._compute_encodings(passthrough=True):  # pylint: disable=protected-access
                 _ = qtzr(param)
 
+    def _patch_quantized_parameters(self, param_names: Optional[Iterable[str]] = None):
+        """nn/base.py:296-324: a context in which the named parameters (all by default) hold their
+        quantize-dequantized values, computed once on entry."""
+        names = self.param_quantizers.keys() if param_names is None else param_names
+        stack = contextlib.ExitStack()
+        for name in names:
+            qtzr = self.param_quantizers[name]
+            param = getattr(self, name)
+            if qtzr is None or param is None:
+                continue
+            if qtzr.is_initialized():
+                param = qtzr(param)
+            stack.enter_context(patch_attr(self, name, param))
+        return stack
+
+    @contextlib.contextmanager
+    def _remove_param_quantizers(self, keys=None):
+        """nn/base.py:995-1005."""
+        keys = list(self.param_quantizers.keys()) if keys is None else ([keys] if isinstance(keys, str) else list(keys))
+        slots = self.param_quantizers._modules  # pylint: disable=protected-access
+        saved = {k: slots[k] for k in keys}
+        try:
+            for k in keys:
+                slots[k] = None
+            yield
+        finally:
+            slots.update(saved)
+
+    def fold_param_quantizers(self):
+        """nn/base.py:1103-1151: bake each parameter quantizer into its parameter (the parameter becomes the
+        quantize-dequantized tensor, the quantizer is dropped), so later forward passes skip that work."""
+        self._compute_param_encodings(overwrite=False)
+        for name, qtzr in self.param_quantizers.items():
+            if not qtzr:
+                continue
+            param = getattr(self, name)
+            if param is None:
+                continue
+            with torch.no_grad():
+                qdq = qtzr(param).dequantize()
+            setattr(self, name, nn.Parameter(qdq, requires_grad=param.requires_grad))
+            self.param_quantizers[name] = None
+
     @contextlib.contextmanager
     def compute_encodings(self, _verdicts=None):
         """nn/base.py:392-427: weights are calibrated on entry; activation quantizers observe their inputs and pass
@@ -156,6 +203,46 @@ def compute_encodings(model: nn.Module):
     with deferred_range_warnings(), contextlib.ExitStack() as stack:
         for m in modules:
             stack.enter_context(m.compute_encodings(_verdicts=verdicts[id(m)]))
+        yield
+
+
+def fold_param_quantizers(model: nn.Module):
+    """QuantizationSimModel.fold_param_quantizers (quantsim/quantsim.py:930-960)."""
+    for m in quantized_linears(model):
+        m.fold_param_quantizers()
+
+
+@contextlib.contextmanager
+def remove_param_quantizers(model: nn.Module):
+    """aimet_torch.utils.remove_param_quantizers (utils.py:1395-1437) for the quantized modules of ``model``."""
+    with contextlib.ExitStack() as stack:
+        for m in quantized_linears(model):
+            stack.enter_context(m._remove_param_quantizers())  # pylint: disable=protected-access
+        yield
+
+
+@contextlib.contextmanager
+def inference_mode(model: nn.Module, prequantize_parameters: bool = True):
+    """aimet_torch.utils._inference_mode (utils.py:1653-1684): every quantizer's encodings are evaluated once and
+    reused by all forward passes inside the context; with ``prequantize_parameters`` the parameters are
+    quantize-dequantized once on entry and their quantizers are skipped inside."""
+    with contextlib.ExitStack() as stack:
+        for q in model.modules():
+            if isinstance(q, QuantizerBase):
+                import itertools
+
+                dtype = next(p.dtype for p in itertools.chain(q.parameters(), q.buffers()))
+                stack.enter_context(q._precompute_encodings(dtype=dtype))  # pylint: disable=protected-access
+        if prequantize_parameters:
+            with torch.no_grad():
+                for m in quantized_linears(model):
+                    stack.enter_context(m._patch_quantized_parameters())  # pylint: disable=protected-access
+            stack.enter_context(remove_param_quantizers(model))
+        # quantized parameters enter the GEMM as plain tensors
+        for m in quantized_linears(model):
+            for name, param in list(m.named_parameters(recurse=False)):
+                if type(param) not in (torch.Tensor, nn.Parameter):
+                    stack.enter_context(patch_attr(m, name, param.as_subclass(torch.Tensor)))
         yield
 
 

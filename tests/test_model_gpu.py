@@ -133,3 +133,76 @@ def test_prequantized_weight_is_reported(device):
     lin.param_quantizers["weight"] = QuantizeDequantize((8, 1), 4, symmetric=True).to(device)
     with pytest.raises(NotImplementedError):
         lin(torch.randn(2, 64, device=device))
+
+
+def _calibrated_copy(device, seed=5):
+    model = LH.build(CFG, device, seed=seed)
+    LH.quantize(model)
+    batches = LH.calibration_batches(CFG, device, batches=2, seq=32)
+    with torch.no_grad(), qnn.compute_encodings(model):
+        for ids in batches:
+            model(ids)
+    return model, batches
+
+
+def _count_calls(modules):
+    counts = {id(m): 0 for m in modules}
+    hooks = [m.register_forward_hook(lambda mod, a, o: counts.__setitem__(id(mod), counts[id(mod)] + 1)) for m in modules]
+    return counts, hooks
+
+
+def test_inference_mode_quantizes_weights_once_and_changes_nothing(device):
+    """utils.py:1653-1684: encodings evaluated once, parameters quantize-dequantized once on entry; outputs keep
+    their bits."""
+    model, batches = _calibrated_copy(device)
+    with torch.no_grad():
+        want = [model(ids) for ids in batches]
+    wqs = [m.param_quantizers["weight"] for m in qnn.quantized_linears(model)]
+    counts, hooks = _count_calls(wqs)
+    with torch.no_grad(), qnn.inference_mode(model):
+        got = [model(ids) for ids in batches]
+        assert all(m.param_quantizers["weight"] is None for m in qnn.quantized_linears(model))
+        assert all(type(m.weight) is torch.Tensor for m in qnn.quantized_linears(model))
+    for h in hooks:
+        h.remove()
+    assert all(c == 1 for c in counts.values())  # once on entry, never inside the two forward passes
+    for g, w in zip(got, want):
+        assert torch.equal(_bits(g), _bits(w))
+    # everything is back in place afterwards
+    assert [m.param_quantizers["weight"] for m in qnn.quantized_linears(model)] == wqs
+    assert all(isinstance(m.weight, torch.nn.Parameter) for m in qnn.quantized_linears(model))
+    with torch.no_grad():
+        assert torch.equal(_bits(model(batches[0])), _bits(want[0]))
+
+
+def test_fold_param_quantizers(device):
+    """nn/base.py:1103-1151: the weight becomes its quantize-dequantized value, the quantizer goes away, outputs keep
+    their bits, and folding an uncalibrated layer calibrates it first."""
+    from aimet_amd.quantization.tensor import DequantizedTensor
+
+    model, batches = _calibrated_copy(device, seed=6)
+    with torch.no_grad():
+        want = model(batches[0])
+    lin = model.blocks[0].mlp.down_proj
+    wq = lin.param_quantizers["weight"]
+    with torch.no_grad():
+        w_qdq = wq(lin.weight)
+    qnn.fold_param_quantizers(model)
+    assert all(m.param_quantizers["weight"] is None for m in qnn.quantized_linears(model))
+    assert isinstance(lin.weight, torch.nn.Parameter) and isinstance(lin.weight.data, torch.Tensor)
+    assert torch.equal(_bits(lin.weight.detach().as_subclass(torch.Tensor)), _bits(w_qdq.as_subclass(torch.Tensor)))
+    with torch.no_grad():
+        assert torch.equal(_bits(model(batches[0])), _bits(want))
+    fresh = qnn.QuantizedLinear(512, 8, bias=False).to(device)  # rows longer than the grid has levels
+    fresh.param_quantizers["weight"] = QuantizeDequantize((8, 1), 8, symmetric=True).to(device)
+    ref = O.qdq_v2_forward(fresh.weight.detach().cpu(), *_absmax_encoding(fresh.weight.detach().cpu()), -128, 127).y
+    fresh.fold_param_quantizers()
+    assert fresh.param_quantizers["weight"] is None
+    assert torch.equal(fresh.weight.detach().cpu().as_subclass(torch.Tensor), ref)
+
+
+def _absmax_encoding(w):
+    """Symmetric 8-bit per-channel min/max encoding of a weight (encoding_analyzer.py:425-481 for num_steps 255)."""
+    lo, hi = O.minmax_encodings(w.amin(dim=1, keepdim=True), w.amax(dim=1, keepdim=True), 255, True)
+    scale = O.scale_from_minmax(lo, hi, -128, 127)
+    return scale, O.offset_from_minmax(lo, scale, -128, 127, True)
