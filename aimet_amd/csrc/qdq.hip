@@ -120,6 +120,19 @@ struct MathAutogradQdq {
         const float offp = ZPS ? rnd<CD>(e.p1 + g.zps) : e.p1;
         return rnd<CD>(q + offp) * e.p0;
     }
+    // The FAST backward in two steps, so that a caller can look at a whole vector's in-range flags before it spends
+    // work on the out-of-range terms (calibrated data is almost always inside the grid): pre() gives the rounded
+    // quotient t, rint(t) and its clamp; an element is in range when the clamp left rint(t) alone.
+    static constexpr bool kSplitBwd = !ZPS;
+    __device__ static void bwd_pre(float x, const EncP& e, float lo, float hi, float& t, float& xr, float& m) {
+        t = rnd<CD>(divide<true, CD>(x, e.p0, e.rs));
+        xr = __builtin_rintf(t);
+        m = __builtin_amdgcn_fmed3f(xr, lo, hi);
+    }
+    __device__ static float bwd_gs_in(float gr, float t, float xr) { return rnd<CD>(gr * (xr - t)); }
+    __device__ static float bwd_gs_out(float gr, float m) { return rnd<CD>(gr * m); }
+    __device__ static float bwd_goff_out(float gr, const EncP& e) { return rnd<CD>(gr * e.p0); }
+
     template <bool FAST>
     __device__ static void bwd(float gr, float x, const EncP& e, const GridC& g, float& gx, float& gs, float& goff) {
         float t = rnd<CD>(divide<FAST, CD>(x, e.p0, e.rs));
@@ -149,6 +162,7 @@ struct MathAutogradQdq {
 
 template <int CD>
 struct MathAutogradQuantize {
+    static constexpr bool kSplitBwd = false;
     static constexpr int kNP = 2;
     static constexpr int kCD = AHQ_F32;  // its outputs are already values of CD
     static constexpr bool kDiv = true;
@@ -177,6 +191,7 @@ struct MathAutogradQuantize {
 
 template <int CD>
 struct MathAutogradDequantize {
+    static constexpr bool kSplitBwd = false;
     static constexpr int kNP = 2;
     static constexpr int kCD = CD;
     static constexpr bool kDiv = false;
@@ -196,6 +211,7 @@ struct MathAutogradDequantize {
 };
 
 struct MathAten {
+    static constexpr bool kSplitBwd = false;
     static constexpr int kCD = AHQ_F32;
     static constexpr int kNP = 3;
     static constexpr bool kDiv = false;
@@ -220,6 +236,7 @@ struct MathAten {
 };
 
 struct MathDlq {
+    static constexpr bool kSplitBwd = false;
     static constexpr int kCD = AHQ_F32;
     static constexpr int kNP = 4;
     static constexpr bool kDiv = true;
@@ -248,6 +265,7 @@ struct MathDlq {
 // y = rint(v / step) * step * scale.  The grid constants travel in GridC: qmin = exponent_min, qmax = max value,
 // zps = mantissa bits.  Dividing by a power of two is exact, so it is done by scaling the exponent.
 struct MathDlqFp8 {
+    static constexpr bool kSplitBwd = false;
     static constexpr int kCD = AHQ_F32;
     static constexpr int kNP = 2;
     static constexpr bool kDiv = true;
@@ -281,6 +299,7 @@ struct MathDlqFp8 {
 // format's largest value and overflows like the conversion would.
 template <int CD>
 struct MathFloatCast {
+    static constexpr bool kSplitBwd = false;
     static constexpr int kCD = CD;
     static constexpr int kNP = 2;
     static constexpr bool kDiv = true;
@@ -478,7 +497,44 @@ __device__ __forceinline__ void bwd_math(const QdqArgs& a, const Tile& t, float 
         const int lv = u * kBlock + threadIdx.x;
         float vs = 0.f, vo = 0.f;
         int si = 0;
-        if (FULL || lv < t.nv) {
+        bool wave_all_in = false;  // only the split form below sets it
+        if constexpr (FAST && M::kSplitBwd) {
+            const bool work = FULL || lv < t.nv;
+            EncP e{};
+            float tq[VEC], xr[VEC], m[VEC];
+            bool all_in = true;
+            if (work) {
+                si = stage_index(a, t, lv);
+                e = staged<M>(sp, si);
+                const float lo = e.p1 + a.gc.qmin, hi = e.p1 + a.gc.qmax;
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) {
+                    M::bwd_pre(load_f32(xin[u].v[k]), e, lo, hi, tq[k], xr[k], m[k]);
+                    all_in &= (m[k] == xr[k]);
+                }
+            }
+            wave_all_in = __builtin_amdgcn_ballot_w64(!all_in) == 0;
+            if (wave_all_in) {
+                // every element of this vector, in every lane, is inside the grid: the input gradient is the output
+                // gradient, the offset gradient gets no term
+                if (work) {
+#pragma unroll
+                    for (int k = 0; k < VEC; ++k) vs += M::bwd_gs_in(load_f32(gin[u].v[k]), tq[k], xr[k]);
+                    if (gxp) store_pack<IO, VEC>(gxp + (int64_t)lv * VEC, gin[u]);
+                }
+            } else if (work) {
+                Pack<IO, VEC> out;
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) {
+                    const float gr = load_f32(gin[u].v[k]);
+                    const bool in = (m[k] == xr[k]);
+                    out.v[k] = store_cast<IO>(in ? gr : 0.f);
+                    vs += in ? M::bwd_gs_in(gr, tq[k], xr[k]) : M::bwd_gs_out(gr, m[k]);
+                    vo += in ? 0.f : M::bwd_goff_out(gr, e);
+                }
+                if (gxp) store_pack<IO, VEC>(gxp + (int64_t)lv * VEC, out);
+            }
+        } else if (FULL || lv < t.nv) {
             si = stage_index(a, t, lv);
             const EncP e = staged<M>(sp, si);
             Pack<IO, VEC> out;
@@ -500,7 +556,7 @@ __device__ __forceinline__ void bwd_math(const QdqArgs& a, const Tile& t, float 
             // 64 x VEC terms per encoding, so single precision (what the reference's own sum accumulates in) is enough
             const int kv = (int)a.Kv;
             const float fs = segment_reduce(vs, kv, OpAddF());
-            const float fo = segment_reduce(vo, kv, OpAddF());
+            const float fo = wave_all_in ? 0.f : segment_reduce(vo, kv, OpAddF());
             if ((FULL || lv < t.nv) && (threadIdx.x & (kv - 1)) == 0) {
                 const int64_t e = t.e0 + si;
                 a.gscale[e] = finish_sum_rt((double)fs, a.out_cd);

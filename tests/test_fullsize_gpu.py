@@ -1,0 +1,143 @@
+"""The kernels at the full sizes of the benchmark configurations, where the CPU oracle would take too long for a unit
+test: properties that do not depend on size (idempotence, consistency between the three operations, linearity of the
+backward pass in the upstream gradient, additivity of counts, agreement of a strided sample with the oracle)."""
+
+import pytest
+import torch
+
+from oracle import torch_ref as O
+from tests.helpers import assert_same_bits
+
+pytestmark = pytest.mark.gpu
+
+
+def _affine():
+    from aimet_amd.quantization import affine
+    return affine
+
+
+# (name, tensor shape, dtype, encoding shape, block size, qmin, qmax, symmetric)
+CONFIGS = [
+    ("c1", (32, 64, 112, 112), torch.float32, (), None, 0, 255, False),
+    ("c2", (4096, 4096), torch.float32, (4096, 1), None, -128, 127, True),
+    ("c4", (14336, 4096), torch.bfloat16, (14336, 64), (1, 64), -8, 7, True),
+]
+
+
+def _make(name, shape, dtype, enc_shape, block, qmin, qmax, symmetric, device):
+    g = torch.Generator(device=device).manual_seed(0)
+    if name == "c1":
+        x = torch.relu(torch.randn(shape, generator=g, device=device))
+    else:
+        x = torch.randn(shape, generator=g, device=device) * 0.02
+    x = x.to(dtype)
+    from aimet_amd.quantization._stats import reduce_min_max
+    mn, mx = reduce_min_max(x, enc_shape, block)
+    mn, mx = mn.float(), mx.float()
+    if symmetric:
+        amax = torch.maximum(mn.abs(), mx.abs()).clamp_min(1e-8)
+        scale = amax / qmax
+        offset = torch.zeros_like(scale)
+    else:
+        scale = ((mx - mn) / (qmax - qmin)).clamp_min(1e-8)
+        offset = torch.round(mn / scale) - qmin
+    grad = torch.randn(shape, generator=g, device=device).to(dtype)
+    return x, scale, offset, grad
+
+
+@pytest.mark.parametrize("cfg", CONFIGS, ids=lambda c: c[0])
+def test_qdq_properties_at_full_size(device, cfg):
+    A = _affine()
+    name, shape, dtype, enc_shape, block, qmin, qmax, symmetric = cfg
+    x, scale, offset, grad = _make(*cfg, device)
+    s_req = scale.clone().requires_grad_(True)   # learnable scale: the composed (true-division) arithmetic
+    y = A.quantize_dequantize(x, s_req, offset, qmin, qmax, block_size=block).detach()
+    # idempotence: a tensor that is already on the grid maps to itself
+    y2 = A.quantize_dequantize(y, s_req, offset, qmin, qmax, block_size=block).detach()
+    assert torch.equal(y.view(torch.int16 if dtype == torch.bfloat16 else torch.int32),
+                       y2.view(torch.int16 if dtype == torch.bfloat16 else torch.int32))
+    # the three operations agree: dequantize(quantize(x)) is quantize_dequantize(x), codes are integers on the grid
+    codes = A.quantize(x, s_req, offset, qmin, qmax, block_size=block).detach()
+    c = codes.as_subclass(torch.Tensor).float()
+    assert bool(((c >= qmin) & (c <= qmax) & (c == c.round())).all())
+    dq = A.dequantize(codes.as_subclass(torch.Tensor), s_req.detach(), offset, block_size=block)
+    assert torch.equal(dq.as_subclass(torch.Tensor), y.as_subclass(torch.Tensor))
+    # a strided sample against the oracle (elementwise operation: rows can be checked on their own)
+    rows = slice(0, shape[0], max(1, shape[0] // 16))
+    sub_scale = scale if scale.dim() == 0 else scale[rows]
+    sub_off = offset if offset.dim() == 0 else offset[rows]
+    ref = O.qdq_v2_forward(x[rows].cpu(), sub_scale.cpu(), sub_off.cpu(), qmin, qmax, block)
+    assert_same_bits(y[rows].as_subclass(torch.Tensor), ref.y, f"{name} sample")
+
+
+@pytest.mark.parametrize("cfg", CONFIGS, ids=lambda c: c[0])
+def test_backward_is_linear_in_the_upstream_gradient(device, cfg):
+    """gx, gscale and goffset of 2g are exactly twice those of g (a power of two commutes with every rounding), gx is
+    g or 0, and a strided sample of gx matches the oracle."""
+    A = _affine()
+    name, shape, dtype, enc_shape, block, qmin, qmax, symmetric = cfg
+    x, scale, offset, grad = _make(*cfg, device)
+
+    def run(g):
+        xd = x.clone().requires_grad_(True)
+        sd = scale.clone().requires_grad_(True)
+        od = offset.clone().requires_grad_(True)
+        A.quantize_dequantize(xd, sd, od, qmin, qmax, block_size=block).backward(g)
+        return xd.grad, sd.grad, od.grad
+
+    gx1, gs1, go1 = run(grad)
+    gx2, gs2, go2 = run(grad * 2)
+    assert torch.equal(gx2.float(), gx1.float() * 2)
+    assert torch.equal(gs2, gs1 * 2) and torch.equal(go2, go1 * 2)
+    assert bool(((gx1 == grad) | (gx1 == 0)).all())
+    rows = slice(0, shape[0], max(1, shape[0] // 16))
+    sub_scale = scale if scale.dim() == 0 else scale[rows]
+    sub_off = offset if offset.dim() == 0 else offset[rows]
+    gx_ref, _, _ = O.qdq_v2_backward(grad[rows].cpu(), x[rows].cpu(), sub_scale.cpu(), sub_off.cpu(), qmin, qmax, block)
+    assert_same_bits(gx1[rows], gx_ref, f"{name} gx sample")
+
+
+@pytest.mark.parametrize("cfg", CONFIGS, ids=lambda c: c[0])
+def test_minmax_at_full_size(device, cfg):
+    """Against torch's own reductions on the device, and: the extrema of the whole are the extrema of its halves."""
+    from aimet_amd.quantization._stats import reduce_min_max
+    name, shape, dtype, enc_shape, block, *_ = cfg
+    x = _make(*cfg, device)[0]
+    mn, mx = reduce_min_max(x, enc_shape, block)
+    if enc_shape == ():
+        assert mn == x.amin() and mx == x.amax()
+        h = shape[0] // 2
+        a, b = reduce_min_max(x[:h], (), None), reduce_min_max(x[h:], (), None)
+        assert mn == torch.minimum(a[0], b[0]) and mx == torch.maximum(a[1], b[1])
+    elif block is None:
+        assert torch.equal(mn, x.amin(dim=1, keepdim=True)) and torch.equal(mx, x.amax(dim=1, keepdim=True))
+    else:
+        v = x.view(shape[0], enc_shape[1], block[1])
+        assert torch.equal(mn, v.amin(dim=2)) and torch.equal(mx, v.amax(dim=2))
+
+
+def test_histogram_counts_are_additive_at_full_size(device):
+    """One batch of the calibration stream ([8, 2048, 4096] float32): every finite element is counted once; feeding
+    the same batch again leaves the range alone and doubles every count; a second, narrower batch only adds."""
+    from aimet_amd.quantization.encoding_analyzer import _HistogramObserver
+
+    g = torch.Generator(device=device).manual_seed(1)
+    u = (torch.rand((8, 2048, 4096), generator=g, device=device) - 0.5).clamp_(-0.4999999, 0.4999999)
+    x = -torch.sign(u) * torch.log1p(-2 * u.abs())
+    del u
+    obs = _HistogramObserver((1,), num_bins=512)
+    first = obs.update(x)[0]
+    n = x.numel()
+    assert float(first.histogram.double().sum()) == n
+    assert first.min == x.amin() and first.max == x.amax()
+    h1 = obs.get_stats()[0].histogram.clone()
+    obs.update(x)
+    h2 = obs.get_stats()[0].histogram
+    assert torch.equal(h2, h1 * 2)
+    obs.update(x * 0.5)
+    h3 = obs.get_stats()[0].histogram
+    assert float(h3.double().sum()) == 3 * n
+    assert bool((h3 >= h2).all())
+    # the batch's own histogram against torch.histc on the device (same formula, counts below 2^24 are exact)
+    lo, hi = float(first.min), float(first.max)
+    assert torch.equal(first.histogram.view(-1), torch.histc(x, 512, lo, hi))
