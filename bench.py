@@ -496,10 +496,10 @@ def run_model_workload(steps, warmup, dev, with_cpu_baseline=True, batches=8, se
     nlin = LH.quantize(model)
     ids = LH.calibration_batches(cfg, dev, batches=batches, seq=seq)
 
-    def calibrate():
-        with torch.no_grad(), qnn.compute_encodings(model):
-            for b in ids:
-                model(b)
+    def calibrate(use_graph=False):
+        # eager passes; the graph-replayed variant (llama_harness.calibrate) is timed beside it and must leave
+        # identical encodings -- with 8 batches its capture costs as much as the replays save
+        LH.calibrate(model, ids, use_graph=use_graph)
 
     def forward():
         with torch.no_grad():
@@ -527,8 +527,21 @@ def run_model_workload(steps, warmup, dev, with_cpu_baseline=True, batches=8, se
         torch.cuda.synchronize()
         return (time.perf_counter() - t) / reps
 
+    def all_ranges():
+        return [(m.min.detach().clone(), m.max.detach().clone()) for m in model.modules() if isinstance(m, QuantizeDequantize)]
+
+    t_cal_graph = timed(lambda: calibrate(True), 1)
+    graph_ranges = all_ranges()
     t_cal = timed(calibrate, 2)
+    eager_ranges = all_ranges()
+    same_ranges = all(torch.equal(a[0], b[0]) and torch.equal(a[1], b[1]) for a, b in zip(graph_ranges, eager_ranges))
     t_fwd = timed(forward, 3)
+
+    def inference_forward():
+        with torch.no_grad(), qnn.inference_mode(model):
+            return timed(lambda: model(ids[0]), 3)
+
+    t_fwd_inf = inference_forward()
     plain = LH.build(cfg, dev, seed=0)
     t_plain = timed(lambda: torch.no_grad()(plain)(ids[0]), 3)
     del plain
@@ -569,6 +582,7 @@ def run_model_workload(steps, warmup, dev, with_cpu_baseline=True, batches=8, se
     w = mods["blocks.0.mlp.down_proj"].weight.detach().cpu()
     mn, mx = O.reduce_minmax(w, tuple(wq.shape), wq.block_size)
     lo, hi = O.minmax_encodings(mn, mx, wq.qmax - wq.qmin, True)
+    parity["graph_replayed_calibration_equals_eager"] = bool(same_ranges)
     parity["weight_encodings_bit_exact"] = bool(torch.equal(wq.min.detach().cpu(), lo.view(wq.shape).float())
                                                 and torch.equal(wq.max.detach().cpu(), hi.view(wq.shape).float()))
 
@@ -583,7 +597,10 @@ def run_model_workload(steps, warmup, dev, with_cpu_baseline=True, batches=8, se
                    "algorithmic_bytes_per_step": bytes_step, "quantizer_elements_per_step": elems_step},
         "pct_of_hbm_peak": round(100.0 * bytes_step / wall / 1e9 / HBM_PEAK_GBS, 2),
         "elements_per_s": round(elems_step / wall, 1),
-        "phases": {"calibration_8_batches_ms": round(t_cal * 1e3, 2), "quantized_forward_ms": round(t_fwd * 1e3, 2),
+        "phases": {"calibration_8_batches_ms": round(t_cal * 1e3, 2),
+                   "calibration_8_batches_graph_replay_ms": round(t_cal_graph * 1e3, 2),
+                   "quantized_forward_ms": round(t_fwd * 1e3, 2),
+                   "quantized_forward_inference_mode_ms": round(t_fwd_inf * 1e3, 2),
                    "unquantized_forward_ms": round(t_plain * 1e3, 2),
                    "linear_tflops_unquantized": round(LH.linear_flops(cfg, tokens) / t_plain / 1e12, 1)},
         "parity": parity,
