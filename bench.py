@@ -410,6 +410,12 @@ def run_dlq_workload(steps, warmup, dev, with_cpu_baseline=True, batches=16, sha
     enc8 = q8.computeEncodings(False)
     q8.setEncodings(enc8)
     t_fp8 = event_time(lambda: q8.quantizeDequantize(xs[0], y), 20)
+    # aimet_torch's float fake-cast of the same batch (float8_e4m3fn, per-tensor scale), also outside the step
+    from aimet_amd.quantization.float import float_quantize_dequantize
+    from aimet_amd.quantization.float._finfo import _float8_e4m3fn
+    from oracle import torch_ref as O
+    fscale = torch.tensor(float(enc8[0].delta), device=dev)
+    t_fcast = event_time(lambda: float_quantize_dequantize(xs[0], _float8_e4m3fn, fscale), 20)
     n_b = xs[0].numel()
     n = n_b * batches
     bytes_upd = 4 * n_b
@@ -434,6 +440,8 @@ def run_dlq_workload(steps, warmup, dev, with_cpu_baseline=True, batches=16, sha
     y_ok = bool((y_s.view("int32") == OD.qdq(sample.cpu().numpy(), enc_ref[:4]).view("int32")).all())
     y8 = q8.quantizeDequantize(sample).cpu().numpy()
     fp8_ok = bool((y8.view("int32") == OD.fp8_qdq(sample.cpu().numpy(), enc8[0].delta, OD.FP8_E4M3FN).view("int32")).all())
+    yf = float_quantize_dequantize(sample, _float8_e4m3fn, fscale).cpu()
+    fcast_ok = bool(torch.equal(yf.view(torch.int32), O.float_qdq(sample.cpu(), fscale.cpu(), 4, 3, True, False).view(torch.int32)))
 
     out = {
         "metric": "QDQ fwd+bwd GB/s (% of HBM peak); calibration elems/s; vs host-CPU ref",
@@ -449,10 +457,12 @@ def run_dlq_workload(steps, warmup, dev, with_cpu_baseline=True, batches=16, sha
                     "dlq_qdq_forward": {"us": round(t_qdq * 1e6, 2), "GBps": round(bytes_qdq / t_qdq / 1e9, 1)},
                     "dlq_fp8_qdq(e4m3fn, not part of the step)": {"us": round(t_fp8 * 1e6, 2),
                                                                   "GBps": round(bytes_qdq / t_fp8 / 1e9, 1)},
+                    "float_qdq(float8_e4m3fn, not part of the step)": {"us": round(t_fcast * 1e6, 2),
+                                                                       "GBps": round(bytes_qdq / t_fcast / 1e9, 1)},
                     "tfe_search(with host read-back)": {"us": round(t_enc * 1e6, 2), "candidates": 358, "buckets": 1536}},
         "encoding": {"min": enc[0].min, "max": enc[0].max, "delta": enc[0].delta, "offset": enc[0].offset},
         "parity": {"hist_bit_exact": hist_ok, "pdf_bit_exact": pdf_ok, "encoding_bit_exact": bool(enc_ok),
-                   "qdq_bit_exact": y_ok, "fp8_qdq_bit_exact": fp8_ok, "sample": "first 2 of 16 batches; 4M-element quantize-dequantize"},
+                   "qdq_bit_exact": y_ok, "fp8_qdq_bit_exact": fp8_ok, "float_qdq_bit_exact": fcast_ok, "sample": "first 2 of 16 batches; 4M-element quantize-dequantize"},
         "roofline": {"bound": "hbm", "kernel": "dlq_pdf_bin_kernel", "achieved": round(bytes_upd / t_upd / 1e9, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(bytes_upd / t_upd / 1e9 / HBM_PEAK_GBS, 4),
                      "algorithmic_bytes": bytes_upd, "traffic": None},
