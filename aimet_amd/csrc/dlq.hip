@@ -149,7 +149,12 @@ __global__ __launch_bounds__(kBlock) void dlq_pdf_prepare_kernel(const PdfPrepAr
 
 struct PdfBinArgs : Geom {
     const void* x;
-    const float* params;  // [S][4]
+    float* params;        // [S][4]
+    // single slot, range already fixed: the kernel derives the binning parameters from the statistics itself and
+    // leaves them in `params` for the kernel that averages the counts in (no separate preparation launch)
+    const double* xleft;
+    const int32_t* meta;
+    int32_t from_state;
     uint32_t* partials;   // single slot: [nblocks][kPdf]
     uint32_t* counts;     // several slots: [S][kPdf], zero-initialised
     int32_t copies, copy_shift;
@@ -173,9 +178,28 @@ constexpr int kPdfUnroll = 4;  // 16-byte loads in flight per lane: the workgrou
 template <typename IO, int VEC, int THREADS>
 __global__ __launch_bounds__(THREADS) void dlq_pdf_bin_kernel(const PdfBinArgs a) {
     extern __shared__ uint32_t lds[];  // [kPdf][copies]
-    if (a.params[2] == 0.f) return;    // histogram not initialised (only all-zero batches so far): nothing to count
+    float inv, off;
+    if (a.from_state) {
+        // what dlq_pdf_prepare_kernel computes for an initialised slot, evaluated by every lane (a few dozen
+        // instructions once per workgroup); workgroup 0 also records it for the averaging kernel
+        const bool active = a.meta[1] != 0;
+        const double x0 = a.xleft[0], x1 = a.xleft[1];
+        const double bucket = x1 - x0;
+        inv = active ? (float)(1 / bucket) : 0.f;
+        off = active ? (float)to_int(round(x0 / bucket)) : 0.f;
+        if (blockIdx.x == 0 && threadIdx.x == 0) {
+            a.params[0] = inv;
+            a.params[1] = off;
+            a.params[2] = active ? 1.f : 0.f;
+            a.params[3] = __int_as_float(a.meta[0]);
+        }
+        if (!active) return;
+    } else {
+        if (a.params[2] == 0.f) return;  // histogram not initialised (only all-zero batches so far): nothing to count
+        inv = a.params[0];
+        off = a.params[1];
+    }
     constexpr int kTile = THREADS * kPdfUnroll;  // vectors per workgroup and iteration
-    const float inv = a.params[0], off = a.params[1];
     const int copies = a.copies;
     for (int i = threadIdx.x; i < copies * kPdf; i += THREADS) lds[i] = 0;
     __syncthreads();
@@ -289,6 +313,36 @@ __global__ __launch_bounds__(kBlock) void dlq_pdf_finish_kernel(const PdfFinArgs
     if (a.hist_out) a.hist_out[(size_t)s * kPdf + i] = h;
     // pdf.iterations++ ; every thread above took the old count from `params`, so nothing else reads this word here
     if (active && i == 0) a.meta[4 * s] = __float_as_int(a.params[4 * s + 3]) + 1;
+}
+
+// Single slot, many partial histograms: fold and average in one launch.  A workgroup owns kFfBins neighbouring
+// buckets; its lanes split the partials kFfGroups ways (64-byte segments per partial), then one lane per bucket adds
+// the group sums in a fixed order and does what dlq_pdf_finish_kernel does.
+constexpr int kFfBins = 16, kFfGroups = kBlock / kFfBins;
+__global__ __launch_bounds__(kBlock) void dlq_pdf_fold_finish_kernel(const PdfFinArgs a) {
+    __shared__ uint32_t sm[kFfGroups][kFfBins];
+    const int bl = threadIdx.x & (kFfBins - 1), grp = threadIdx.x / kFfBins;
+    const int i = blockIdx.x * kFfBins + bl;
+    const bool active = a.params[2] != 0.f;
+    uint32_t acc = 0;
+    if (active) {
+#pragma unroll 8
+        for (int p = grp; p < a.nparts; p += kFfGroups) acc += a.counts[(size_t)p * kPdf + i];
+    }
+    sm[grp][bl] = acc;
+    __syncthreads();
+    if (grp != 0) return;
+    uint32_t h = 0;
+#pragma unroll
+    for (int g = 0; g < kFfGroups; ++g) h += sm[g][bl];
+    if (active) {
+        const int it = __float_as_int(a.params[3]);
+        const double prob = (double)h / (double)a.cnt;
+        a.pdf[i] = (a.pdf[i] * it + prob) / (it + 1);
+        if (i == 0) a.meta[0] = it + 1;
+    }
+    if (a.hist_out) a.hist_out[i] = h;
+    if (i == 0) a.meta[2] = 1;  // _statsUpdated
 }
 
 __global__ void dlq_pdf_mark_kernel(int32_t* meta, int S) {
@@ -724,12 +778,17 @@ extern "C" int ahq_dlq_pdf_update(int32_t dtype, const ahq_layout* layout, const
     pa.pdf = st->pdf;
     pa.meta = st->meta;
     pa.params = params;
-    hipLaunchKernelGGL(dlq_pdf_prepare_kernel, dim3(S), dim3(kBlock), 0, s, pa);
+    // one slot whose range is already fixed: the binning kernel works the parameters out itself
+    const bool from_state = !with_init && S == 1 && pp.fast && pp.nblocks > kPdfFoldGroups;
+    if (!from_state) hipLaunchKernelGGL(dlq_pdf_prepare_kernel, dim3(S), dim3(kBlock), 0, s, pa);
 
     PdfBinArgs ba{};
     fill_geom(pp.plan, &ba);
     ba.x = x;
     ba.params = params;
+    ba.xleft = st->xleft;
+    ba.meta = st->meta;
+    ba.from_state = from_state ? 1 : 0;
     ba.copies = pp.copies;
     ba.copy_shift = 0;
     while ((1 << ba.copy_shift) < pp.copies) ++ba.copy_shift;
@@ -769,6 +828,10 @@ extern "C" int ahq_dlq_pdf_update(int32_t dtype, const ahq_layout* layout, const
 #undef AHQ_LAUNCH_PDF_K
         fa.counts = counts;
         fa.nparts = pp.nblocks;
+        if (S == 1 && pp.nblocks > kPdfFoldGroups) {
+            hipLaunchKernelGGL(dlq_pdf_fold_finish_kernel, dim3(kPdf / kFfBins), dim3(kBlock), 0, s, fa);
+            return check_launch("dlq_pdf_update");
+        }
         if (pp.nblocks > kPdfFoldGroups) {
             uint32_t* folded = reinterpret_cast<uint32_t*>(w + pp.off_folded);
             hipLaunchKernelGGL(dlq_pdf_fold_kernel, dim3(kPdf / kBlock, kPdfFoldGroups), dim3(kBlock), 0, s, counts, folded,

@@ -22,6 +22,9 @@ extern "C" int ahq_minmax(int32_t dtype, const ahq_layout* layout, const void* x
                           void* run_min, void* run_max, int finite_only, void* workspace, size_t workspace_bytes,
                           void* stream);
 extern "C" size_t ahq_minmax_workspace_bytes(const ahq_layout* layout);
+extern "C" int ahq_minmax_finite_partials(int32_t dtype, const ahq_layout* layout, const void* x, void* out_min,
+                                          void* out_max, void* workspace, size_t workspace_bytes, void* stream,
+                                          const float** part_min, const float** part_max, int64_t* nparts);
 
 namespace ahq {
 
@@ -40,6 +43,9 @@ struct PrepArgs {
     float growth;
     const void* bmin;  // [S] io dtype
     const void* bmax;
+    const float* part_min;  // single slot: per-workgroup partial extrema of the batch, folded here when nparts > 0
+    const float* part_max;
+    int64_t nparts;
     float* hist;       // [S][B] running
     float* edges;      // [S][B+1]
     float* minmax;     // [S][2] stored min / max
@@ -60,8 +66,38 @@ __global__ void hist_prepare_kernel(const PrepArgs a) {
     const int s = blockIdx.x;
     const int B = a.num_bins;
     const float Bf = (float)B;
-    const float mn = load_f32(static_cast<const IO*>(a.bmin)[s]);
-    const float mx = load_f32(static_cast<const IO*>(a.bmax)[s]);
+    float mn, mx;
+    if (a.nparts > 0) {
+        // fold the partial extrema of the min/max pass (saves that pass's own finishing launch); min and max are
+        // exact and order-independent, and the partials already are values of the tensor's dtype
+        __shared__ float red_mn[16], red_mx[16];
+        mn = __builtin_inff();
+        mx = -__builtin_inff();
+        for (int64_t q = threadIdx.x; q < a.nparts; q += blockDim.x) {
+            mn = fminf(mn, a.part_min[q]);
+            mx = fmaxf(mx, a.part_max[q]);
+        }
+#pragma unroll
+        for (int m = kWave / 2; m >= 1; m >>= 1) {
+            mn = fminf(mn, __shfl_xor(mn, m, kWave));
+            mx = fmaxf(mx, __shfl_xor(mx, m, kWave));
+        }
+        if ((threadIdx.x & (kWave - 1)) == 0) {
+            red_mn[threadIdx.x / kWave] = mn;
+            red_mx[threadIdx.x / kWave] = mx;
+        }
+        __syncthreads();
+        const int nw = (blockDim.x + kWave - 1) / kWave;
+        mn = red_mn[0];
+        mx = red_mx[0];
+        for (int w = 1; w < nw; ++w) {
+            mn = fminf(mn, red_mn[w]);
+            mx = fmaxf(mx, red_mx[w]);
+        }
+    } else {
+        mn = load_f32(static_cast<const IO*>(a.bmin)[s]);
+        mx = load_f32(static_cast<const IO*>(a.bmax)[s]);
+    }
     // the batch's own bin edges; "min - 0.5" happens in the tensor dtype before the cast to float
     const bool eq = mn == mx;
     const float lo1 = eq ? round_io<IO>(mn - 0.5f) : mn;
@@ -530,8 +566,10 @@ extern "C" int ahq_hist_update(int32_t dtype, const ahq_layout* layout, const vo
     const int NH = first_batch ? 1 : 2;
 
     // 1. finite range of the batch, in the tensor's dtype
-    int rc = ahq_minmax(dtype, layout, x, w + hp.off_bmin, w + hp.off_bmax, nullptr, nullptr, 1, w + hp.off_mm_ws,
-                        hp.off_bmin - hp.off_mm_ws, stream);
+    const float *part_min = nullptr, *part_max = nullptr;
+    int64_t nparts = 0;
+    int rc = ahq_minmax_finite_partials(dtype, layout, x, w + hp.off_bmin, w + hp.off_bmax, w + hp.off_mm_ws,
+                                        hp.off_bmin - hp.off_mm_ws, stream, &part_min, &part_max, &nparts);
     if (rc != AHQ_OK) return rc;
 
     // 2. edges, updated range, re-binned running counts
@@ -542,6 +580,9 @@ extern "C" int ahq_hist_update(int32_t dtype, const ahq_layout* layout, const vo
     pa.growth = st->growth_limit;
     pa.bmin = w + hp.off_bmin;
     pa.bmax = w + hp.off_bmax;
+    pa.part_min = part_min;
+    pa.part_max = part_max;
+    pa.nparts = S == 1 ? nparts : 0;
     pa.hist = st->hist;
     pa.edges = st->edges;
     pa.minmax = st->minmax;
@@ -552,7 +593,7 @@ extern "C" int ahq_hist_update(int32_t dtype, const ahq_layout* layout, const vo
     pa.upd_edges = reinterpret_cast<float*>(w + hp.off_upd_edges);
     pa.ranges = reinterpret_cast<float*>(w + hp.off_ranges);
     pa.scratch = reinterpret_cast<int32_t*>(w + hp.off_scratch);
-    const int pthreads = B >= 512 ? 512 : (B >= 64 ? ((B + 63) / 64) * 64 : 64);
+    const int pthreads = nparts > 0 ? 1024 : (B >= 512 ? 512 : (B >= 64 ? ((B + 63) / 64) * 64 : 64));
     switch (dtype) {
         case AHQ_F32: hipLaunchKernelGGL((hist_prepare_kernel<float>), dim3(S), dim3(pthreads), 0, s, pa); break;
         case AHQ_F16: hipLaunchKernelGGL((hist_prepare_kernel<f16_t>), dim3(S), dim3(pthreads), 0, s, pa); break;
@@ -610,6 +651,11 @@ extern "C" int ahq_hist_update(int32_t dtype, const ahq_layout* layout, const vo
     fa.first = first_batch ? 1 : 0;
     fa.nparts = hp.fast ? hp.nblocks : 1;
     fa.counts = counts;
+    fa.carried = pa.carried;
+    fa.upd_edges = pa.upd_edges;
+    fa.hist = st->hist;
+    fa.edges = st->edges;
+    fa.new_hist = st->new_hist;
     if (hp.fast && hp.nblocks > kFoldGroups) {
         uint32_t* folded = reinterpret_cast<uint32_t*>(w + hp.off_folded);
         const int len = NH * (B + 2);

@@ -319,6 +319,51 @@ static void launch_mm(const Plan& p, const MmArgs& a, hipStream_t st) {
 
 using namespace ahq;
 
+extern "C" int ahq_minmax(int32_t dtype, const ahq_layout* layout, const void* x, void* out_min, void* out_max,
+                          void* run_min, void* run_max, int finite_only, void* workspace, size_t workspace_bytes,
+                          void* stream);
+
+// Library-internal: the finite-only extrema for a caller that will fold the per-workgroup partials itself.  For a
+// single encoding over more than one workgroup only the streaming kernel is launched and the partial arrays are
+// handed back (*nparts > 0, out_min / out_max untouched); every other layout runs the complete reduction into
+// out_min / out_max (*nparts == 0).
+extern "C" __attribute__((visibility("hidden"))) int ahq_minmax_finite_partials(
+    int32_t dtype, const ahq_layout* layout, const void* x, void* out_min, void* out_max, void* workspace,
+    size_t workspace_bytes, void* stream, const float** part_min, const float** part_max, int64_t* nparts) {
+    *nparts = 0;
+    Plan p;
+    if (dtype < AHQ_F32 || dtype > AHQ_BF16 || !layout || !make_plan(dtype, *layout, aligned16(x), true, &p) ||
+        !(p.cl.kind == kIJK && p.cl.J == 1) || flat_blocks(p) <= 1 || !x || !workspace ||
+        workspace_bytes < p.ws_elems * 12)
+        return ahq_minmax(dtype, layout, x, out_min, out_max, nullptr, nullptr, 1, workspace, workspace_bytes, stream);
+    MmArgs a{};
+    fill_geom(p, &a);
+    a.x = x;
+    a.red = p.red;
+    a.finite_only = 1;
+    char* w = static_cast<char*>(workspace);
+    a.part_min = reinterpret_cast<float*>(w);
+    a.part_max = reinterpret_cast<float*>(w + p.ws_elems * 4);
+    a.part_nan = reinterpret_cast<int*>(w + p.ws_elems * 8);
+    const int64_t nb = flat_blocks(p);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+#define AHQ_FLAT(IO)                                                                                                  \
+    do {                                                                                                              \
+        if (p.vec == 1) hipLaunchKernelGGL((minmax_flat_kernel<IO, 1, true>), dim3((unsigned)nb), dim3(kBlock), 0, st, a); \
+        else hipLaunchKernelGGL((minmax_flat_kernel<IO, IoTraits<IO>::kVec, true>), dim3((unsigned)nb), dim3(kBlock), 0, st, a); \
+    } while (0)
+    switch (dtype) {
+        case AHQ_F32: AHQ_FLAT(float); break;
+        case AHQ_F16: AHQ_FLAT(f16_t); break;
+        default: AHQ_FLAT(bf16_t); break;
+    }
+#undef AHQ_FLAT
+    *part_min = a.part_min;
+    *part_max = a.part_max;
+    *nparts = nb;
+    return check_launch("ahq_minmax");
+}
+
 extern "C" size_t ahq_minmax_workspace_bytes(const ahq_layout* layout) {
     if (!layout) return 0;
     // the widest plan over dtypes and alignments decides; 12 bytes per tile or per encoding
