@@ -242,7 +242,7 @@ __device__ __forceinline__ int bin_exact(float v, const RangeC& r, float Bf, int
 // correctly rounded quotient by at most one unit in the last place (the residual is evaluated without rounding of
 // the product, so q0 + e/w is the true quotient to ~2^-46 and rounds to the quotient or to its neighbour).  The two
 // can only truncate differently when q1 is an integer or the float just below one.  `fast` is true when
-//   * q1 is not within q1 * 2^-23 (>= one ulp) of an integer, and
+//   * q1 is +0, or is not within q1 * 2^-23 (>= one ulp) of an integer, and
 //   * 0 <= q1 < B - 4 ulp, tested on the bit pattern (negative values, -0, NaN and +inf all compare above the limit).
 // v < lo gives q1 <= 0 with the sign bit set; v > hi gives a quotient of at least B - 2 ulp; so a `fast` element is
 // inside the range and its truncated estimate is the reference bin.  Everything else is redone with bin_exact().
@@ -251,7 +251,9 @@ __device__ __forceinline__ int bin_estimate(float v, const RangeC& r, float Bf, 
     const float q0 = t * r.rwidth;
     const float e = __builtin_fmaf(-q0, r.width, t);
     const float q1 = __builtin_fmaf(e, r.rwidth, q0);
-    const bool safe = __builtin_fabsf(__builtin_rintf(q1) - q1) > q1 * 1.1920929e-7f;
+    // ">=": an estimate of exactly +0 (v == lo, which is every zero of a rectified activation whose minimum is 0) is
+    // safe -- the quotient is exactly 0; for every other q1 equality needs q1 a power of two, where the left side is 0
+    const bool safe = __builtin_fabsf(__builtin_rintf(q1) - q1) >= q1 * 1.1920929e-7f;
     fast = safe & (f32_to_bits(q1) < limit_bits);
     return (int)q1;
 }
@@ -280,9 +282,9 @@ __global__ __launch_bounds__(kBlock, 6) void hist_bin_kernel(const BinArgs a) {
 #pragma unroll
     for (int h = 0; h < NH; ++h) mine[h] = lds + (size_t)h * B * copies + (threadIdx.x & (copies - 1));
     const IO* __restrict__ x = static_cast<const IO*>(a.x);
-    uint32_t below[NH], above[NH];
+    uint32_t below[NH], above[NH], zeros[NH];
 #pragma unroll
-    for (int h = 0; h < NH; ++h) below[h] = above[h] = 0;
+    for (int h = 0; h < NH; ++h) below[h] = above[h] = zeros[h] = 0;
 
     // every element, exactly (ragged tile, tail elements and the revisit of flagged elements)
     auto bin_slow = [&](float v, bool only_flagged) {
@@ -311,13 +313,18 @@ __global__ __launch_bounds__(kBlock, 6) void hist_bin_kernel(const BinArgs a) {
 #pragma unroll
             for (int k = 0; k < VEC; ++k) {
                 const float v = load_f32(in[u].v[k]);
+                // exact zeros (half of a rectified activation) would all add to one LDS word, which serialises the
+                // wave's atomics (161 instead of 126 us per batch on such data); they are counted in a register and
+                // added to their bin once, at the end.  Costs 4 % on data without zeros.
+                const bool zero = v == 0.f;
 #pragma unroll
                 for (int h = 0; h < NH; ++h) {
                     bool fast;
                     const int b = bin_estimate(v, r[h], Bf, limit_bits, fast);
                     if (fast) {
-                        atomicAdd(reinterpret_cast<uint32_t*>(reinterpret_cast<char*>(mine[h]) + ((uint32_t)b << bshift)), 1u);
                         ++binned;
+                        if (zero) ++zeros[h];
+                        else atomicAdd(reinterpret_cast<uint32_t*>(reinterpret_cast<char*>(mine[h]) + ((uint32_t)b << bshift)), 1u);
                     }
                 }
             }
@@ -343,6 +350,11 @@ __global__ __launch_bounds__(kBlock, 6) void hist_bin_kernel(const BinArgs a) {
         const int64_t i = a.nvec * VEC + threadIdx.x;
         if (i < a.numel) bin_slow(load_f32(x[i]), false);
     }
+    // the zeros counted in registers (a non-zero count means zero took the fast path, so it lies inside the range
+    // and its estimated bin is the exact one)
+#pragma unroll
+    for (int h = 0; h < NH; ++h)
+        if (zeros[h] != 0) atomicAdd(&mine[h][bin_exact(0.f, r[h], Bf, B) << cshift], zeros[h]);
     // below / above: wave reduce, then across waves
 #pragma unroll
     for (int h = 0; h < NH; ++h) {
