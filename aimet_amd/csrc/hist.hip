@@ -385,6 +385,107 @@ __global__ __launch_bounds__(kBlock, 6) void hist_bin_kernel(const BinArgs a) {
     }
 }
 
+// Several slots whose runs are long enough that a tile lies inside one run (per-channel weights, per-channel
+// activations with large feature maps): one workgroup per tile bins into LDS sub-histograms of its slot and adds the
+// non-empty bins to the slot's zero-initialised counters in global memory.
+template <typename IO, int VEC, int NH>
+__global__ __launch_bounds__(kBlock, 6) void hist_bin_rows_kernel(const BinArgs a, const Geom rows) {
+    extern __shared__ uint32_t lds[];  // [NH][B][copies]
+    __shared__ uint32_t cnt_smem[kBlock / kWave][NH][2];
+    const int B = a.num_bins;
+    const float Bf = (float)B;
+    const int copies = a.copies;
+    const Tile t = make_tile(rows, blockIdx.x);
+    for (int i = threadIdx.x; i < copies * NH * B; i += kBlock) lds[i] = 0;
+    RangeC r[NH];
+#pragma unroll
+    for (int h = 0; h < NH; ++h) r[h] = load_range(a.ranges + t.e0 * kRng, h);
+    __syncthreads();
+    const int cshift = a.copy_shift, bshift = cshift + 2;
+    const uint32_t limit_bits = f32_to_bits(Bf) - 4u;
+    uint32_t* mine[NH];
+#pragma unroll
+    for (int h = 0; h < NH; ++h) mine[h] = lds + (size_t)h * B * copies + (threadIdx.x & (copies - 1));
+    const IO* __restrict__ x = static_cast<const IO*>(a.x) + t.v0 * VEC;
+    uint32_t below[NH], above[NH];
+#pragma unroll
+    for (int h = 0; h < NH; ++h) below[h] = above[h] = 0;
+    auto bin_slow = [&](float v, bool only_flagged) {
+#pragma unroll
+        for (int h = 0; h < NH; ++h) {
+            const bool inr = (v >= r[h].lo) & (v <= r[h].hi);
+            bool fast = false;
+            if (only_flagged) (void)bin_estimate(v, r[h], Bf, limit_bits, fast);
+            if (inr & !fast) atomicAdd(&mine[h][bin_exact(v, r[h], Bf, B) << cshift], 1u);
+            if (!inr) {
+                below[h] += v < r[h].thr_lo ? 1u : 0u;
+                above[h] += v > r[h].thr_hi ? 1u : 0u;
+            }
+        }
+    };
+    if (t.nv == kTileVec) {
+        Pack<IO, VEC> in[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) in[u] = load_pack<IO, VEC>(x + (int64_t)(u * kBlock + threadIdx.x) * VEC);
+        uint32_t binned = 0;
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u)
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) {
+                const float v = load_f32(in[u].v[k]);
+#pragma unroll
+                for (int h = 0; h < NH; ++h) {
+                    bool fast;
+                    const int b = bin_estimate(v, r[h], Bf, limit_bits, fast);
+                    if (fast) {
+                        atomicAdd(reinterpret_cast<uint32_t*>(reinterpret_cast<char*>(mine[h]) + ((uint32_t)b << bshift)), 1u);
+                        ++binned;
+                    }
+                }
+            }
+        if (__builtin_amdgcn_ballot_w64(binned != (uint32_t)(kUnroll * VEC * NH)) != 0) {
+            for (int u = 0; u < kUnroll; ++u)
+                for (int k = 0; k < VEC; ++k) bin_slow(load_f32(in[u].v[k]), true);
+        }
+    } else {
+        for (int u = 0; u < kUnroll; ++u) {
+            const int lv = u * kBlock + threadIdx.x;
+            if (lv < t.nv) {
+                const Pack<IO, VEC> pk = load_pack<IO, VEC>(x + (int64_t)lv * VEC);
+                for (int k = 0; k < VEC; ++k) bin_slow(load_f32(pk.v[k]), false);
+            }
+        }
+    }
+    const int wave = threadIdx.x / kWave;
+#pragma unroll
+    for (int h = 0; h < NH; ++h) {
+        uint32_t bl = below[h], ab = above[h];
+#pragma unroll
+        for (int m = kWave / 2; m >= 1; m >>= 1) {
+            bl += __shfl_xor(bl, m, kWave);
+            ab += __shfl_xor(ab, m, kWave);
+        }
+        if ((threadIdx.x & (kWave - 1)) == 0) {
+            cnt_smem[wave][h][0] = bl;
+            cnt_smem[wave][h][1] = ab;
+        }
+    }
+    __syncthreads();
+    uint32_t* out = a.counts + (size_t)t.e0 * NH * (B + 2);
+    for (int i = threadIdx.x; i < NH * B; i += kBlock) {
+        const int h = i / B, b = i - h * B;
+        uint32_t c = 0;
+        for (int cp = 0; cp < copies; ++cp) c += lds[(size_t)i * copies + cp];
+        if (c) atomicAdd(&out[h * (B + 2) + b], c);
+    }
+    if (threadIdx.x < NH * 2) {
+        const int h = threadIdx.x / 2, w = threadIdx.x & 1;
+        uint32_t c = 0;
+        for (int wv = 0; wv < kBlock / kWave; ++wv) c += cnt_smem[wv][h][w];
+        if (c) atomicAdd(&out[h * (B + 2) + B + w], c);
+    }
+}
+
 // Several slots (or histograms too large for LDS): every element adds to its slot's counters in global memory.
 template <typename IO>
 __global__ __launch_bounds__(kBlock) void hist_bin_generic_kernel(const BinArgs a) {
@@ -494,7 +595,9 @@ namespace {
 
 struct HistPlan {
     Plan plan;
+    Plan rows_plan;  // tiling by runs (valid when `rows`)
     bool fast;       // single slot through LDS
+    bool rows;       // several slots, every tile inside one run: per-tile LDS histograms
     int copies;
     int nblocks;
     int64_t ntiles;
@@ -520,6 +623,20 @@ bool make_hist_plan(int dtype, const ahq_layout& layout, const void* x, int num_
             }
         if (copies >= 1) {
             hp->fast = true;
+            hp->copies = copies;
+        }
+    }
+    hp->rows = false;
+    if (c.kind == kIJK && c.J > 1) {
+        const int fit = (int)(16384 / ((size_t)2 * num_bins * 4));
+        int copies = 0;
+        for (int c2 = 8; c2 >= 1; c2 >>= 1)
+            if (c2 <= fit) {
+                copies = c2;
+                break;
+            }
+        if (copies >= 1 && make_plan(dtype, layout, aligned16(x), true, &hp->rows_plan) && hp->rows_plan.mode == kRows) {
+            hp->rows = true;
             hp->copies = copies;
         }
     }
@@ -648,6 +765,28 @@ extern "C" int ahq_hist_update(int32_t dtype, const ahq_layout* layout, const vo
         ba.counts = counts;
         const int64_t n = (int64_t)S * NH * (B + 2);
         hipLaunchKernelGGL(zero_u32_kernel, dim3((unsigned)((n + 255) / 256 > 1024 ? 1024 : (n + 255) / 256)), dim3(256), 0, s, counts, n);
+        if (hp.rows) {
+            Geom rg{};
+            fill_geom(hp.rows_plan, &rg);
+            const size_t lds = (size_t)hp.copies * NH * B * 4;
+            const dim3 g(hp.rows_plan.nblocks), b(kBlock);
+#define AHQ_LAUNCH_ROWS(IO)                                                                                         \
+    do {                                                                                                            \
+        if (hp.rows_plan.vec == 1) {                                                                                \
+            if (NH == 1) hipLaunchKernelGGL((hist_bin_rows_kernel<IO, 1, 1>), g, b, lds, s, ba, rg);                \
+            else hipLaunchKernelGGL((hist_bin_rows_kernel<IO, 1, 2>), g, b, lds, s, ba, rg);                        \
+        } else {                                                                                                    \
+            if (NH == 1) hipLaunchKernelGGL((hist_bin_rows_kernel<IO, IoTraits<IO>::kVec, 1>), g, b, lds, s, ba, rg); \
+            else hipLaunchKernelGGL((hist_bin_rows_kernel<IO, IoTraits<IO>::kVec, 2>), g, b, lds, s, ba, rg);       \
+        }                                                                                                           \
+    } while (0)
+            switch (dtype) {
+                case AHQ_F32: AHQ_LAUNCH_ROWS(float); break;
+                case AHQ_F16: AHQ_LAUNCH_ROWS(f16_t); break;
+                default: AHQ_LAUNCH_ROWS(bf16_t); break;
+            }
+#undef AHQ_LAUNCH_ROWS
+        } else
         switch (dtype) {
             case AHQ_F32: hipLaunchKernelGGL((hist_bin_generic_kernel<float>), dim3(hp.nblocks), dim3(kBlock), 0, s, ba); break;
             case AHQ_F16: hipLaunchKernelGGL((hist_bin_generic_kernel<f16_t>), dim3(hp.nblocks), dim3(kBlock), 0, s, ba); break;

@@ -18,6 +18,7 @@ import contextlib
 import warnings
 from abc import ABC, abstractmethod
 from dataclasses import dataclass
+from collections.abc import Sequence
 from typing import Generic, List, Optional, Tuple, TypeVar
 
 import torch
@@ -41,6 +42,45 @@ class _Histogram:
     bin_edges: torch.Tensor = None
     min: Optional[torch.Tensor] = None
     max: Optional[torch.Tensor] = None
+
+
+class _HistogramList(Sequence):
+    """``List[_Histogram]`` (one entry per encoding, what the reference's observer returns) as a view over the stacked
+    device tensors: entries are built when they are asked for.  A per-channel or blockwise observer has thousands of
+    slots, and materialising a Python object with four tensor views for each of them on every batch costs
+    milliseconds to seconds of host time that nothing reads during a calibration pass."""
+
+    def __init__(self, hist, edges, minmax, dtype, count: Optional[int] = None):
+        self._hist, self._edges, self._minmax, self._dtype = hist, edges, minmax, dtype
+        self._typed_minmax = None
+        self._count = hist.shape[0] if hist is not None else int(count)
+
+    def __len__(self) -> int:
+        return self._count
+
+    def stacked(self):
+        """(hist [S, B], bin edges [S, B + 1], min/max [S, 2] in float32, dtype the reference keeps min/max in)."""
+        return self._hist, self._edges, self._minmax, self._dtype
+
+    def _entry(self, i: int) -> _Histogram:
+        if self._hist is None:
+            return _Histogram()
+        if self._typed_minmax is None:
+            self._typed_minmax = self._minmax if self._dtype == torch.float32 else self._minmax.to(self._dtype)
+        mm = self._typed_minmax
+        return _Histogram(self._hist[i], self._edges[i], mm[i, 0], mm[i, 1])
+
+    def __getitem__(self, i):
+        if isinstance(i, slice):
+            return [self._entry(k) for k in range(*i.indices(self._count))]
+        if i < 0:
+            i += self._count
+        if not 0 <= i < self._count:
+            raise IndexError("histogram index out of range")
+        return self._entry(i)
+
+    def __iter__(self):
+        return (self._entry(i) for i in range(self._count))
 
 
 _Statistics = TypeVar("_Statistics", _MinMaxRange, _Histogram)
@@ -176,9 +216,8 @@ class _HistogramObserver(_Observer[_Histogram]):
         return new_hist, new_edges, new_minmax
 
     @staticmethod
-    def _as_list(hist, edges, minmax, dtype) -> List[_Histogram]:
-        mm = minmax if dtype == torch.float32 else minmax.to(dtype)
-        return [_Histogram(hist[s], edges[s], mm[s, 0], mm[s, 1]) for s in range(hist.shape[0])]
+    def _as_list(hist, edges, minmax, dtype) -> "_HistogramList":
+        return _HistogramList(hist, edges, minmax, dtype)
 
     # --------------------------------------------------------------------------------------------------- API --
     @torch.no_grad()
@@ -216,7 +255,7 @@ class _HistogramObserver(_Observer[_Histogram]):
 
     def get_stats(self) -> List[_Histogram]:
         if not self._has_stats:
-            return [_Histogram() for _ in range(self.num_slots)]
+            return _HistogramList(None, None, None, None, count=self.num_slots)
         if self._stats_cache is None:
             s = self._state
             self._stats_cache = self._as_list(s["hist"], s["edges"], s["minmax"], self._stat_dtype)
@@ -405,6 +444,8 @@ class _HistogramAnalyzer(EncodingAnalyzer[_Histogram]):
         if stats is obs.get_stats() and obs._has_stats:  # pylint: disable=protected-access
             s = obs._state  # pylint: disable=protected-access
             return s["hist"], s["edges"], s["minmax"], obs._stat_dtype  # pylint: disable=protected-access
+        if isinstance(stats, _HistogramList) and stats.stacked()[0] is not None:
+            return stats.stacked()
         hist = torch.stack([s.histogram for s in stats]).contiguous()
         edges = torch.stack([s.bin_edges for s in stats]).contiguous()
         dtype = stats[0].min.dtype
