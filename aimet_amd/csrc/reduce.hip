@@ -106,8 +106,10 @@ __device__ __forceinline__ float key_f32(unsigned int k) {
 }
 
 // FULL: every lane of the tile has work (all tiles but the last).  FINITE: ignore non-finite values.
+constexpr int kMmStage = kTileVec + 2;  // most runs a tile can touch
+
 template <typename IO, int VEC, int RED, bool FINITE, bool FULL>
-__device__ __forceinline__ void mm_tile(const MmArgs& a, const Tile& t, MinMax& acc) {
+__device__ __forceinline__ void mm_tile(const MmArgs& a, const Tile& t, MinMax& acc, unsigned int* stage_keys) {
     const IO* __restrict__ x = static_cast<const IO*>(a.x) + t.v0 * VEC;
     Pack<IO, VEC> in[kUnroll];
 #pragma unroll
@@ -134,12 +136,12 @@ __device__ __forceinline__ void mm_tile(const MmArgs& a, const Tile& t, MinMax& 
             v.nan = segment_reduce(v.nan, kv, OpOrI());
             if ((FULL || lv < t.nv) && (threadIdx.x & (kv - 1)) == 0) mm_write<IO>(a, t.e0 + si, v);
         } else if (RED == kRedAtomic) {
+            // first into the tile's own table in LDS (one entry per run the tile touches); the table goes to the
+            // global keys once per run and tile instead of once per vector
             if (FULL || lv < t.nv) {
-                int64_t e = t.e0 + si;
-                if (e >= a.J) e %= a.J;
-                atomicMin(&a.key_min[e], f32_key(v.mn));
-                atomicMax(&a.key_max[e], f32_key(v.mx));
-                if (v.nan) atomicOr(&a.part_nan[e], 1);
+                atomicMin(&stage_keys[si], f32_key(v.mn));
+                atomicMax(&stage_keys[kMmStage + si], f32_key(v.mx));
+                if (v.nan) atomicOr(&stage_keys[2 * kMmStage + si], 1u);
             }
         }
     }
@@ -148,10 +150,29 @@ __device__ __forceinline__ void mm_tile(const MmArgs& a, const Tile& t, MinMax& 
 template <typename IO, int VEC, int RED, bool FINITE>
 __global__ __launch_bounds__(kBlock) void minmax_kernel(const MmArgs a) {
     __shared__ MinMax red_smem[kBlock / kWave];
+    __shared__ unsigned int stage_keys[RED == kRedAtomic ? 3 * kMmStage : 1];  // min keys | max keys | NaN flags
     const Tile t = make_tile(a, blockIdx.x);
+    if (RED == kRedAtomic) {
+        for (int i = threadIdx.x; i < t.nstage; i += kBlock) {
+            stage_keys[i] = f32_key(__builtin_inff());
+            stage_keys[kMmStage + i] = f32_key(-__builtin_inff());
+            stage_keys[2 * kMmStage + i] = 0u;
+        }
+        __syncthreads();
+    }
     MinMax acc = mm_identity();
-    if (t.nv == kTileVec) mm_tile<IO, VEC, RED, FINITE, true>(a, t, acc);
-    else mm_tile<IO, VEC, RED, FINITE, false>(a, t, acc);
+    if (t.nv == kTileVec) mm_tile<IO, VEC, RED, FINITE, true>(a, t, acc, stage_keys);
+    else mm_tile<IO, VEC, RED, FINITE, false>(a, t, acc, stage_keys);
+    if (RED == kRedAtomic) {
+        __syncthreads();
+        for (int i = threadIdx.x; i < t.nstage; i += kBlock) {
+            int64_t e = t.e0 + i;
+            if (e >= a.J) e %= a.J;
+            atomicMin(&a.key_min[e], stage_keys[i]);
+            atomicMax(&a.key_max[e], stage_keys[kMmStage + i]);
+            if (stage_keys[2 * kMmStage + i]) atomicOr(&a.part_nan[e], 1);
+        }
+    }
     if (RED == kRedTile) {
         const MinMax b = mm_block_reduce(acc, red_smem);
         const int64_t per_enc = a.mode == kRows ? a.I * (int64_t)a.tpr : (int64_t)a.nblocks;
@@ -253,13 +274,62 @@ template <typename IO>
 __global__ __launch_bounds__(kBlock) void minmax_generic_kernel(const MmArgs a) {
     const IO* __restrict__ x = static_cast<const IO*>(a.x);
     const bool fo = a.finite_only == 1;
-    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < a.numel; i += (int64_t)gridDim.x * kBlock) {
-        const int64_t e = generic_enc_index(a, i);
+    const int lane = threadIdx.x & (kWave - 1);
+    // every lane of a wave runs the same number of iterations (inactive ones carry the identity), so the wave-level
+    // exchanges below are executed by whole waves
+    const int64_t stride = (int64_t)gridDim.x * kBlock;
+    const int64_t first = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    for (int64_t base = first - lane; base < a.numel; base += stride) {
+        const int64_t i = base + lane;
+        const bool active = i < a.numel;
+        const int64_t e = active ? generic_enc_index(a, i) : -1;
         MinMax v = mm_identity();
-        mm_add(v, load_f32(x[i]), fo);
-        atomicMin(&a.key_min[e], f32_key(v.mn));
-        atomicMax(&a.key_max[e], f32_key(v.mx));
-        if (v.nan) atomicOr(&a.part_nan[e], 1);
+        if (active) mm_add(v, load_f32(x[i]), fo);
+        // neighbouring elements mostly share an encoding: the lanes of each distinct encoding are combined first and
+        // one lane issues the atomics (64 times fewer of them when the whole wave lies in one block)
+        uint64_t todo = __builtin_amdgcn_ballot_w64(active);
+        while (todo != 0) {
+            const int lead = __builtin_ctzll(todo);
+            const int64_t el = __shfl(e, lead, kWave);
+            const bool mine = active && e == el;
+            MinMax m = mine ? v : mm_identity();
+#pragma unroll
+            for (int k = kWave / 2; k >= 1; k >>= 1) m = mm_merge(m, mm_shfl_xor(m, k));
+            if (lane == lead) {
+                atomicMin(&a.key_min[el], f32_key(m.mn));
+                atomicMax(&a.key_max[el], f32_key(m.mx));
+                if (m.nan) atomicOr(&a.part_nan[el], 1);
+            }
+            todo &= ~__builtin_amdgcn_ballot_w64(mine);
+        }
+    }
+}
+
+// Encodings that change with every element (run length 1, e.g. per-channel along the fastest axis): a lane owns VEC
+// neighbouring encodings and walks down the rows of its slab, so loads stay coalesced 16-byte vectors and each lane
+// ends with one pair of atomics per encoding instead of one per element.
+constexpr int kColRows = 64;  // rows per slab
+template <typename IO, int VEC, bool FINITE>
+__global__ __launch_bounds__(kBlock) void minmax_cols_kernel(const MmArgs a) {
+    const int64_t c0 = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * VEC;
+    if (c0 >= a.J) return;
+    const int64_t r0 = (int64_t)blockIdx.y * kColRows;
+    const int64_t r1 = r0 + kColRows < a.I ? r0 + kColRows : a.I;
+    const IO* __restrict__ x = static_cast<const IO*>(a.x);
+    MinMax m[VEC];
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) m[k] = mm_identity();
+#pragma unroll 4
+    for (int64_t r = r0; r < r1; ++r) {
+        const Pack<IO, VEC> pk = load_pack<IO, VEC>(x + r * a.J + c0);
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) mm_add(m[k], load_f32(pk.v[k]), FINITE);
+    }
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) {
+        atomicMin(&a.key_min[c0 + k], f32_key(m[k].mn));
+        atomicMax(&a.key_max[c0 + k], f32_key(m[k].mx));
+        if (m[k].nan) atomicOr(&a.part_nan[c0 + k], 1);
     }
 }
 
@@ -309,6 +379,11 @@ static void launch_mm(const Plan& p, const MmArgs& a, hipStream_t st) {
         }
     } else if (p.red == kRedSeg) {
         launch_mm_red<IO, kRedSeg, FINITE>(p, a, st);
+    } else if (p.cl.K == 1 && p.cl.J % IoTraits<IO>::kVec == 0 && aligned16(a.x) && p.cl.I > 1 &&
+               (p.cl.I + kColRows - 1) / kColRows <= 65535) {
+        constexpr int V = IoTraits<IO>::kVec;
+        const dim3 g((unsigned)((p.cl.J / V + kBlock - 1) / kBlock), (unsigned)((p.cl.I + kColRows - 1) / kColRows));
+        hipLaunchKernelGGL((minmax_cols_kernel<IO, V, FINITE>), g, dim3(kBlock), 0, st, a);
     } else {
         launch_mm_red<IO, kRedAtomic, FINITE>(p, a, st);
     }

@@ -25,6 +25,11 @@ CASES = [
     ((6, 10), (6, 1), None),
     ((5, 7, 64), (5, 1, 2), (1, -1, -1)),
     ((3, 5), (3, 5), None),
+    ((200, 2056), (2056,), None),          # one encoding per element of the fastest axis: lanes walk down columns
+    ((3, 70, 512), (512,), None),          # the same with several slabs of rows and leading dimensions folded in
+    ((256, 256), (2, 2), (128, 128)),      # two-dimensional blocks wider than a wave (generic walk, wave pre-reduction)
+    ((96, 100), (3, 4), (32, 25)),         # two-dimensional blocks narrower than a wave
+    ((32, 512, 14, 14), (512, 1, 1), None),  # short runs, many per tile (LDS table of the tile's runs)
 ]
 
 
@@ -89,3 +94,28 @@ def test_errors(device):
         reduce_min_max(x.cpu(), ())
     with pytest.raises(RuntimeError):
         reduce_min_max(torch.empty(0, 3, device=device), ())
+
+
+@pytest.mark.parametrize("case", [((64, 520), (520,), None), ((256, 256), (2, 2), (128, 128)), ((32, 64, 7, 7), (64, 1, 1), None)],
+                         ids=["columns", "blocks_2d", "short_runs"])
+def test_nan_and_inf_in_the_aggregating_paths(device, case):
+    """NaN wins, infinities count, and the finite-only variant skips both, on the layouts that pre-aggregate in LDS,
+    across a wave, or down columns before they touch the global keys."""
+    from aimet_amd.quantization._stats import reduce_min_max
+
+    shape, enc_shape, block = case
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(shape, generator=g)
+    f = x.view(-1)
+    f[3], f[1000], f[2001], f[-1] = float("nan"), float("inf"), float("-inf"), float("nan")
+    mn_ref, mx_ref = O.reduce_minmax(x, enc_shape, block)
+    mn, mx = reduce_min_max(x.to(device), enc_shape, block)
+    assert_same_bits(mn, mn_ref, "min")
+    assert_same_bits(mx, mx_ref, "max")
+    fin = torch.where(x.isfinite(), x, torch.zeros_like(x))  # the test data has finite values on both sides of zero
+    lo_ref, hi_ref = O.reduce_minmax(torch.where(x.isfinite(), x, torch.full_like(x, 1e30)), enc_shape, block)[0], \
+        O.reduce_minmax(torch.where(x.isfinite(), x, torch.full_like(x, -1e30)), enc_shape, block)[1]
+    lo, hi = reduce_min_max(x.to(device), enc_shape, block, finite_only=True)
+    assert_same_bits(lo, lo_ref, "finite min")
+    assert_same_bits(hi, hi_ref, "finite max")
+    del fin
