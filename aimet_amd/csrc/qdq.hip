@@ -491,7 +491,8 @@ __device__ __forceinline__ float finish_sum_rt(double s, int cd) {
 
 template <typename IO, int VEC, typename M, int RED, bool FULL, bool FAST>
 __device__ __forceinline__ void bwd_math(const QdqArgs& a, const Tile& t, float (*sp)[kStage], const Pack<IO, VEC>* xin,
-                                         const Pack<IO, VEC>* gin, IO* __restrict__ gxp, double& acc_s, double& acc_o) {
+                                         const Pack<IO, VEC>* gin, IO* __restrict__ gxp, double& acc_s, double& acc_o,
+                                         double* stage_sums) {
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
         const int lv = u * kBlock + threadIdx.x;
@@ -563,18 +564,19 @@ __device__ __forceinline__ void bwd_math(const QdqArgs& a, const Tile& t, float 
                 a.goffset[e] = finish_sum_rt((double)fo, a.out_cd);
             }
         } else if (RED == kRedAtomic) {
+            // into the tile's own table in LDS first (one entry per run the tile touches); the table is added to the
+            // global sums once per run and tile instead of once per vector
             if (FULL || lv < t.nv) {
-                int64_t e = t.e0 + si;
-                if (e >= a.J) e %= a.J;
-                atomicAdd(&a.partials[2 * e], (double)vs);
-                atomicAdd(&a.partials[2 * e + 1], (double)vo);
+                atomicAdd(&stage_sums[2 * si], (double)vs);
+                atomicAdd(&stage_sums[2 * si + 1], (double)vo);
             }
         }
     }
 }
 
 template <typename IO, int VEC, typename M, int RED, bool FULL>
-__device__ __forceinline__ void bwd_tile(const QdqArgs& a, const Tile& t, float (*sp)[kStage], double& acc_s, double& acc_o) {
+__device__ __forceinline__ void bwd_tile(const QdqArgs& a, const Tile& t, float (*sp)[kStage], double& acc_s, double& acc_o,
+                                         double* stage_sums) {
     const IO* __restrict__ x = static_cast<const IO*>(a.x) + t.v0 * VEC;
     const IO* __restrict__ g = static_cast<const IO*>(a.g) + t.v0 * VEC;
     IO* __restrict__ gxp = a.gx ? static_cast<IO*>(a.gx) + t.v0 * VEC : nullptr;
@@ -588,21 +590,33 @@ __device__ __forceinline__ void bwd_tile(const QdqArgs& a, const Tile& t, float 
         }
     }
     if (!M::kDiv || __builtin_amdgcn_ballot_w64(!lane_can_divide_fast<IO, VEC, M, FULL>(a, t, sp, xin)) == 0)
-        bwd_math<IO, VEC, M, RED, FULL, true>(a, t, sp, xin, gin, gxp, acc_s, acc_o);
+        bwd_math<IO, VEC, M, RED, FULL, true>(a, t, sp, xin, gin, gxp, acc_s, acc_o, stage_sums);
     else
-        bwd_math<IO, VEC, M, RED, FULL, false>(a, t, sp, xin, gin, gxp, acc_s, acc_o);
+        bwd_math<IO, VEC, M, RED, FULL, false>(a, t, sp, xin, gin, gxp, acc_s, acc_o, stage_sums);
 }
 
 template <typename IO, int VEC, typename M, int RED>
 __global__ __launch_bounds__(kBlock) void qdq_bwd_kernel(const QdqArgs a) {
     __shared__ float sp[M::kNP + (M::kDiv ? 1 : 0)][kStage];
     __shared__ double red_smem[kBlock / kWave];
+    __shared__ double stage_sums[RED == kRedAtomic ? 2 * kStage : 1];  // kRedAtomic: (scale, offset) sums per run
     const Tile t = make_tile(a, blockIdx.x);
     stage_encodings<M>(a, t, sp);
+    if (RED == kRedAtomic)
+        for (int i = threadIdx.x; i < 2 * t.nstage; i += kBlock) stage_sums[i] = 0.0;
     __syncthreads();
     double acc_s = 0.0, acc_o = 0.0;  // kRedTile: per-thread totals
-    if (t.nv == kTileVec) bwd_tile<IO, VEC, M, RED, true>(a, t, sp, acc_s, acc_o);
-    else bwd_tile<IO, VEC, M, RED, false>(a, t, sp, acc_s, acc_o);
+    if (t.nv == kTileVec) bwd_tile<IO, VEC, M, RED, true>(a, t, sp, acc_s, acc_o, stage_sums);
+    else bwd_tile<IO, VEC, M, RED, false>(a, t, sp, acc_s, acc_o, stage_sums);
+    if (RED == kRedAtomic) {
+        __syncthreads();
+        for (int i = threadIdx.x; i < t.nstage; i += kBlock) {
+            int64_t e = t.e0 + i;
+            if (e >= a.J) e %= a.J;
+            atomicAdd(&a.partials[2 * e], stage_sums[2 * i]);
+            atomicAdd(&a.partials[2 * e + 1], stage_sums[2 * i + 1]);
+        }
+    }
     if (VEC > 1 && blockIdx.x == 0) {  // tail elements, single encoding only
         const int64_t i = a.nvec * VEC + threadIdx.x;
         if (i < a.numel) {
@@ -698,15 +712,41 @@ __global__ __launch_bounds__(kBlock) void qdq_bwd_generic_kernel(const QdqArgs a
     const IO* __restrict__ x = static_cast<const IO*>(a.x);
     const IO* __restrict__ g = static_cast<const IO*>(a.g);
     IO* __restrict__ gxp = static_cast<IO*>(a.gx);
-    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < a.numel; i += (int64_t)gridDim.x * kBlock) {
-        const int64_t ei = generic_enc_index(a, i);
-        const EncP e = load_enc<M>(a, ei);
-        float gx, gs, go;
-        M::template bwd<false>(load_f32(g[i]), load_f32(x[i]), e, a.gc, gx, gs, go);
-        if (gxp) gxp[i] = store_cast<IO>(gx);
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t stride = (int64_t)gridDim.x * kBlock;
+    const int64_t first = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    // whole waves iterate together (lanes past the end carry zeros), so the exchanges below are wave-wide
+    for (int64_t base = first - lane; base < a.numel; base += stride) {
+        const int64_t i = base + lane;
+        const bool active = i < a.numel;
+        int64_t ei = -1;
+        float gx = 0.f, gs = 0.f, go = 0.f;
+        if (active) {
+            ei = generic_enc_index(a, i);
+            const EncP e = load_enc<M>(a, ei);
+            M::template bwd<false>(load_f32(g[i]), load_f32(x[i]), e, a.gc, gx, gs, go);
+            if (gxp) gxp[i] = store_cast<IO>(gx);
+        }
         if (a.partials) {
-            atomicAdd(&a.partials[2 * ei], (double)gs);
-            atomicAdd(&a.partials[2 * ei + 1], (double)go);
+            // neighbouring elements mostly share an encoding: the lanes of each distinct encoding are summed first
+            // and one lane issues the two atomics
+            uint64_t todo = __builtin_amdgcn_ballot_w64(active);
+            while (todo != 0) {
+                const int lead = __builtin_ctzll(todo);
+                const int64_t el = __shfl(ei, lead, kWave);
+                const bool mine = active && ei == el;
+                double ss = mine ? (double)gs : 0.0, so = mine ? (double)go : 0.0;
+#pragma unroll
+                for (int k = kWave / 2; k >= 1; k >>= 1) {
+                    ss += __shfl_xor(ss, k, kWave);
+                    so += __shfl_xor(so, k, kWave);
+                }
+                if (lane == lead) {
+                    atomicAdd(&a.partials[2 * el], ss);
+                    atomicAdd(&a.partials[2 * el + 1], so);
+                }
+                todo &= ~__builtin_amdgcn_ballot_w64(mine);
+            }
         }
     }
 }
