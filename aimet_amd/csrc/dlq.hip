@@ -522,6 +522,91 @@ __global__ __launch_bounds__(kWave) void dlq_tfe_cost_kernel(const TfeArgs a) {
     a.cost[(size_t)s * kMaxCand + k] = ok ? std_min(cost, kDblMax) : kDblMax;
 }
 
+// the value that lane j (a constant) holds, as a wave-uniform scalar
+__device__ __forceinline__ double lane_value(double v, int j) {
+    const long long b = __double_as_longlong(v);
+    const unsigned int lo = __builtin_amdgcn_readlane((int)(unsigned int)b, j);
+    const unsigned int hi = __builtin_amdgcn_readlane((int)(unsigned int)((unsigned long long)b >> 32), j);
+    return __longlong_as_double((long long)(((unsigned long long)hi << 32) | lo));
+}
+
+// The same costs with one wave per candidate, for few slots (a per-tensor search has 358 candidates: six waves of
+// the kernel above, each doing the arithmetic of all 1536 buckets for 64 candidates, leave the GPU idle).  The lanes
+// work out the terms of 64 buckets at a time; the additions into the three sums then run over those 64 terms in
+// bucket order on values read lane by lane, so every sum sees exactly the sequence of roundings of the serial loop
+// (a term that does not belong to a sum is +0, which leaves a non-negative sum unchanged).
+__global__ __launch_bounds__(kWave) void dlq_tfe_cost_wave_kernel(const TfeArgs a) {
+    const int s = blockIdx.y;
+    const int k = blockIdx.x;
+    if (a.meta[4 * s + 1] == 0) return;
+    const int lane = threadIdx.x;
+    const bool ok = a.cand_ok[(size_t)s * kMaxCand + k] != 0;
+    if (!ok) {
+        if (lane == 0) a.cost[(size_t)s * kMaxCand + k] = kDblMax;
+        return;
+    }
+    const float delta = a.cand_delta[(size_t)s * kMaxCand + k];
+    const int offset = a.cand_off[(size_t)s * kMaxCand + k];
+    const double* xl = a.xleft + (size_t)s * kPdf;
+    const double* pdf = a.pdf + (size_t)s * kPdf;
+    const float* centers = a.centers + (size_t)s * kPdf;
+    const float min_val = delta * offset;
+    const float step_size = (float)((double)(1ull << a.bw) - 1);
+    const float max_val = delta * (offset + step_size);
+    const float pdf_start = (float)xl[0];
+    const double pdf_step = xl[1] - xl[0];
+    int min_ind = to_int(floor((min_val - pdf_start) / pdf_step));
+    min_ind = min_ind < 0 ? 0 : (min_ind > kPdf - 1 ? kPdf - 1 : min_ind);
+    int max_ind = to_int(floor((max_val - pdf_start) / pdf_step));
+    max_ind = max_ind < 0 ? 0 : (max_ind > kPdf - 1 ? kPdf - 1 : max_ind);
+    const float min_mid = centers[min_ind], max_mid = centers[max_ind];
+    const float inv_delta = 1 / delta;
+    double sat_bottom = 0, sat_top = 0, quant = 0;
+    for (int i0 = 0; i0 < kPdf; i0 += kWave) {
+        const int i = i0 + lane;
+        const float c = centers[i];
+        const double p = pdf[i];
+        double tb = 0, tt = 0, tq = 0;
+        if (i < min_ind) {
+            const double d = (double)c - min_mid;
+            tb = p * (d * d);
+        }
+        if (i >= max_ind) {
+            const double d = (double)c - max_mid;
+            tt = p * (d * d);
+        }
+        if (i >= min_ind && i < max_ind) {
+            const float deq = __builtin_floorf(c * inv_delta + 0.5f) * delta;
+            const double d = (double)(c - deq);
+            tq = p * (d * d);
+        }
+        // The three sums take their buckets from three consecutive ranges, so a chunk of 64 buckets that lies within
+        // one range is a single chain of additions; only the (at most two) chunks that straddle a boundary feed all
+        // three sums.
+        const int last = i0 + kWave - 1;
+        const int phase = i0 < min_ind ? 0 : (i0 < max_ind ? 1 : 2);
+        const int phase_last = last < min_ind ? 0 : (last < max_ind ? 1 : 2);
+        if (phase == phase_last && min_ind <= max_ind) {
+            const double t = phase == 0 ? tb : (phase == 1 ? tq : tt);
+            double acc = phase == 0 ? sat_bottom : (phase == 1 ? quant : sat_top);
+#pragma unroll
+            for (int j = 0; j < kWave; ++j) acc += lane_value(t, j);
+            if (phase == 0) sat_bottom = acc;
+            else if (phase == 1) quant = acc;
+            else sat_top = acc;
+        } else {
+#pragma unroll
+            for (int j = 0; j < kWave; ++j) {
+                sat_bottom += lane_value(tb, j);
+                sat_top += lane_value(tt, j);
+                quant += lane_value(tq, j);
+            }
+        }
+    }
+    const double cost = 3.0 * (sat_bottom + sat_top) + quant;
+    if (lane == 0) a.cost[(size_t)s * kMaxCand + k] = std_min(cost, kDblMax);
+}
+
 // _findBestCandidate (first strictly smaller cost wins) and the final encoding (TfEnhancedEncodingAnalyzer.cpp:88-127,
 // 337-377); also the two cases without a histogram (TfEnhancedEncodingAnalyzer.cpp:58-80)
 __global__ __launch_bounds__(kWave) void dlq_tfe_select_kernel(const TfeArgs a) {
@@ -545,16 +630,24 @@ __global__ __launch_bounds__(kWave) void dlq_tfe_select_kernel(const TfeArgs a) 
         }
         return;
     }
-    // each lane scans a contiguous run of candidates, then the lanes are compared in order
+    // each lane scans every 64th candidate in rising order (all loads are issued before the first comparison), then
+    // the lanes are compared by (cost, index)
     constexpr int kPer = kMaxCand / kWave;
+    double cs[kPer];
+    int oks[kPer];
+#pragma unroll
+    for (int r = 0; r < kPer; ++r) {
+        cs[r] = a.cost[(size_t)s * kMaxCand + r * kWave + lane];
+        oks[r] = a.cand_ok[(size_t)s * kMaxCand + r * kWave + lane];
+    }
     double bc = kDblMax;
     int bi = -1, n = 0;
-    for (int k = lane * kPer; k < (lane + 1) * kPer; ++k) {
-        const double c = a.cost[(size_t)s * kMaxCand + k];
-        n += a.cand_ok[(size_t)s * kMaxCand + k];
-        if (c < bc) {
-            bc = c;
-            bi = k;
+#pragma unroll
+    for (int r = 0; r < kPer; ++r) {
+        n += oks[r];
+        if (cs[r] < bc) {
+            bc = cs[r];
+            bi = r * kWave + lane;
         }
     }
 #pragma unroll
@@ -569,6 +662,12 @@ __global__ __launch_bounds__(kWave) void dlq_tfe_select_kernel(const TfeArgs a) 
             bi = oi;
         }
     }
+    // index of the winner among the accepted candidates, as a host loop that skips rejected ones would count
+    int rank = 0;
+#pragma unroll
+    for (int r = 0; r < kPer; ++r) rank += (r * kWave + lane < bi) ? oks[r] : 0;
+#pragma unroll
+    for (int m = 1; m < kWave; m <<= 1) rank += __shfl_xor(rank, m, kWave);
     if (lane == 0) {
         float best_delta = -1;
         int best_offset = -1;
@@ -585,13 +684,7 @@ __global__ __launch_bounds__(kWave) void dlq_tfe_select_kernel(const TfeArgs a) 
         out[3] = best_offset;
         out[4] = a.bw;
         if (a.best) {
-            // index among the accepted candidates, as a host loop that skips rejected ones would count
-            int rank = -1;
-            if (bi >= 0) {
-                rank = 0;
-                for (int k = 0; k < bi; ++k) rank += a.cand_ok[(size_t)s * kMaxCand + k];
-            }
-            a.best[2 * s] = rank;
+            a.best[2 * s] = bi >= 0 ? rank : -1;
             a.best[2 * s + 1] = n;
         }
     }
@@ -892,7 +985,11 @@ extern "C" int ahq_dlq_tfe_encodings(const ahq_dlq_pdf_state* st, int32_t bw, in
     a.best = best_index;
     hipStream_t s = static_cast<hipStream_t>(stream);
     hipLaunchKernelGGL(dlq_tfe_candidates_kernel, dim3(st->num_slots), dim3(kMaxCand), 0, s, a);
-    hipLaunchKernelGGL(dlq_tfe_cost_kernel, dim3(kMaxCand / kWave, st->num_slots), dim3(kWave), 0, s, a);
+    // Few slots: one wave per candidate (the candidates beyond the list are marked invalid and cost nothing).  That
+    // form issues about eight times the instructions of the lane-per-candidate one, so it pays only while the latter
+    // cannot fill the GPU.
+    if (st->num_slots <= 16) hipLaunchKernelGGL(dlq_tfe_cost_wave_kernel, dim3(kMaxCand, st->num_slots), dim3(kWave), 0, s, a);
+    else hipLaunchKernelGGL(dlq_tfe_cost_kernel, dim3(kMaxCand / kWave, st->num_slots), dim3(kWave), 0, s, a);
     hipLaunchKernelGGL(dlq_tfe_select_kernel, dim3(st->num_slots), dim3(kWave), 0, s, a);
     return check_launch("dlq_tfe_encodings");
 }

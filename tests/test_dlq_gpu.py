@@ -264,10 +264,12 @@ def test_tfe_encodings_bit_exact(device, kind, bw):
         assert a.last_best == b.last_best, (sym, strict, uns, a.last_best, b.last_best)
 
 
-def test_tfe_encodings_per_block(device):
-    x = _data((6, 2, 512), 5, special=False)
-    a = OracleQuantizer((3, 2, 1), 8, QUANTIZATION_TF_ENHANCED)
-    b = HipQuantizer((3, 2, 1), 8, QUANTIZATION_TF_ENHANCED, device)
+@pytest.mark.parametrize("shape,enc_shape", [((6, 2, 512), (3, 2, 1)), ((48, 2, 256), (24, 2, 1))])
+def test_tfe_encodings_per_block(device, shape, enc_shape):
+    """6 slots are searched with one wave per candidate, 48 with one lane per candidate."""
+    x = _data(shape, 5, special=False)
+    a = OracleQuantizer(enc_shape, 8, QUANTIZATION_TF_ENHANCED)
+    b = HipQuantizer(enc_shape, 8, QUANTIZATION_TF_ENHANCED, device)
     for q in (a, b):
         q.updateStats(x)
         q.updateStats(x * 0.5 + 1)
