@@ -71,6 +71,23 @@ template <typename T, int N>
 __device__ __forceinline__ void store_pack(T* p, const Pack<T, N>& v) {
     *reinterpret_cast<Pack<T, N>*>(p) = v;
 }
+// Store of an output that this kernel never reads back: marked non-temporal, so the written lines do not displace the
+// inputs from the caches (a backward pass re-reads the tensor its forward pass has just read).
+template <typename T, int N>
+__device__ __forceinline__ void store_pack_stream(T* p, const Pack<T, N>& v) {
+    constexpr int kBytes = (int)sizeof(T) * N;
+    if constexpr (kBytes == 16) {
+        typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+        __builtin_nontemporal_store(__builtin_bit_cast(u32x4, v), reinterpret_cast<u32x4*>(p));
+    } else if constexpr (kBytes == 8) {
+        typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+        __builtin_nontemporal_store(__builtin_bit_cast(u32x2, v), reinterpret_cast<u32x2*>(p));
+    } else if constexpr (kBytes == 4) {
+        __builtin_nontemporal_store(__builtin_bit_cast(unsigned int, v), reinterpret_cast<unsigned int*>(p));
+    } else {
+        store_pack<T, N>(p, v);
+    }
+}
 
 // ------------------------------------------------------------------------------------------- wave / block reduce --
 // ------------------------------------------------------------------------------------------ segment exchange --

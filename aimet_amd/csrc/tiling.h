@@ -22,6 +22,8 @@ struct Geom {
     int64_t nvec;  // numel / VEC
     int64_t I, J, K;
     int64_t Kv;    // vectors per run of one encoding (K / VEC); 2^62 when J == 1
+    int32_t kv_shift;  // log2(Kv) when Kv is a power of two below the tile size, else -1
+    int32_t tile_vec;  // vectors per tile: kBlock x (vectors per thread, at most kUnroll)
     int32_t mode;
     int32_t tpr;   // tiles per row (kRows)
     uint32_t nblocks;
@@ -46,16 +48,16 @@ __device__ __forceinline__ Tile make_tile(const Geom& a, int64_t tile) {
     if (a.mode == kRows) {
         const int64_t row = tile / a.tpr;
         const int64_t tt = tile - row * a.tpr;
-        t.v0 = row * a.Kv + tt * kTileVec;
-        const int64_t left = a.Kv - tt * kTileVec;
-        t.nv = (int)(left < kTileVec ? left : kTileVec);
-        t.rem0 = tt * kTileVec;
+        t.v0 = row * a.Kv + tt * a.tile_vec;
+        const int64_t left = a.Kv - tt * a.tile_vec;
+        t.nv = (int)(left < a.tile_vec ? left : a.tile_vec);
+        t.rem0 = tt * a.tile_vec;
         t.e0 = a.I == 1 ? row : row % a.J;
         t.nstage = 1;
     } else {
-        t.v0 = tile * kTileVec;
+        t.v0 = tile * a.tile_vec;
         const int64_t left = a.nvec - t.v0;
-        t.nv = (int)(left < kTileVec ? left : kTileVec);
+        t.nv = (int)(left < a.tile_vec ? left : a.tile_vec);
         if (t.nv < 0) t.nv = 0;
         if (a.J == 1) {
             t.rem0 = 0;
@@ -75,7 +77,8 @@ __device__ __forceinline__ Tile make_tile(const Geom& a, int64_t tile) {
 __device__ __forceinline__ int stage_index(const Geom& a, const Tile& t, int lv) {
     if (t.nstage == 1) return 0;
     const int64_t p = t.rem0 + lv;
-    if (a.Kv >= kTileVec) return p >= a.Kv ? 1 : 0;
+    if (a.Kv >= a.tile_vec) return p >= a.Kv ? 1 : 0;
+    if (a.kv_shift >= 0) return (int)((uint32_t)p >> a.kv_shift);  // the usual block sizes: no per-lane division
     return (int)((uint32_t)p / (uint32_t)a.Kv);
 }
 
@@ -97,6 +100,7 @@ struct Plan {
     int red;
     uint32_t nblocks;
     int64_t Kv, nvec;
+    int tile_vec;  // vectors per tile
     int64_t ntiles;
     size_t ws_elems;  // kRedTile: number of tiles; kRedAtomic: number of encodings; else 0
 };
@@ -106,8 +110,12 @@ inline size_t io_size(int dtype) { return dtype == AHQ_F32 ? 4 : 2; }
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 inline bool is_pow2(int64_t v) { return v > 0 && (v & (v - 1)) == 0; }
 
-// Decide tiling and reduction strategy.  `ptr_aligned`: every tensor pointer is 16-byte aligned.
-inline bool make_plan(int io_dtype, const ahq_layout& layout, bool ptr_aligned, bool want_red, Plan* p) {
+// Decide tiling and reduction strategy.  `ptr_aligned`: every tensor pointer is 16-byte aligned; `unroll`: vectors per
+// thread and tile the kernel family works with (its register arrays hold that many).
+inline bool make_plan(int io_dtype, const ahq_layout& layout, bool ptr_aligned, bool want_red, Plan* p,
+                      int unroll = kUnroll) {
+    const int tile_vec = kBlock * unroll;
+    p->tile_vec = tile_vec;
     const char* err = nullptr;
     if (!canonicalize(layout, &p->cl, &err)) {
         set_error(err);
@@ -137,16 +145,16 @@ inline bool make_plan(int io_dtype, const ahq_layout& layout, bool ptr_aligned, 
     p->vec = shared ? V : 1;
     p->nvec = c.numel / p->vec;
     p->Kv = c.J == 1 ? ((int64_t)1 << 62) : c.K / p->vec;
-    int64_t nb = (p->nvec + kTileVec - 1) / kTileVec;
+    int64_t nb = (p->nvec + tile_vec - 1) / tile_vec;
     if (want_red) {
         if (c.J == 1) {
             p->red = kRedTile;
         } else if (c.I == 1 && is_pow2(p->Kv) && p->Kv <= kWave) {
             p->red = kRedSeg;
-        } else if (p->Kv >= kTileVec / 2) {
+        } else if (p->Kv >= tile_vec / 2) {
             p->red = kRedTile;
             p->mode = kRows;
-            p->tpr = (int)((p->Kv + kTileVec - 1) / kTileVec);
+            p->tpr = (int)((p->Kv + tile_vec - 1) / tile_vec);
             nb = c.I * c.J * (int64_t)p->tpr;
         } else {
             p->red = kRedAtomic;
@@ -172,6 +180,11 @@ inline void fill_geom(const Plan& p, Geom* g) {
     g->J = c.J;
     g->K = c.K;
     g->Kv = p.Kv;
+    g->kv_shift = -1;
+    g->tile_vec = p.tile_vec;
+    if (p.Kv < p.tile_vec && is_pow2(p.Kv))
+        for (int b = 0; b < 31; ++b)
+            if (((int64_t)1 << b) == p.Kv) g->kv_shift = b;
     g->mode = p.mode;
     g->tpr = p.tpr;
     g->nblocks = p.nblocks;
