@@ -572,7 +572,7 @@ __global__ __launch_bounds__(kBlock) void hist_finish_kernel(const FinArgs a) {
     float nh = (float)tot[0];
     if (b == 0) nh += (float)edge_cnt[0][0];
     if (b == B - 1) nh += (float)edge_cnt[0][1];
-    a.new_hist[(size_t)s * B + b] = nh;
+    if (a.new_hist) a.new_hist[(size_t)s * B + b] = nh;
     float uh;
     if (a.first) {
         uh = nh;
@@ -680,7 +680,7 @@ extern "C" int ahq_hist_update(int32_t dtype, const ahq_layout* layout, const vo
     if (dtype < AHQ_F32 || dtype > AHQ_BF16) return set_error("bad dtype"), AHQ_ERR_INVALID;
     if (!layout || !st || !x) return set_error("null argument"), AHQ_ERR_INVALID;
     if (st->num_bins <= 0) return set_error("num_bins must be positive"), AHQ_ERR_INVALID;
-    if (!st->hist || !st->edges || !st->minmax || !st->limits || !st->new_hist || !st->new_edges || !st->new_minmax)
+    if (!st->hist || !st->edges || !st->minmax || !st->limits || !st->new_edges || !st->new_minmax)
         return set_error("histogram state has a null buffer"), AHQ_ERR_INVALID;
     if (!(st->growth_limit >= 1.0f)) return set_error("growth limit must be at least 1"), AHQ_ERR_INVALID;
     HistPlan hp;
@@ -692,7 +692,10 @@ extern "C" int ahq_hist_update(int32_t dtype, const ahq_layout* layout, const vo
     hipStream_t s = static_cast<hipStream_t>(stream);
     char* w = static_cast<char*>(workspace);
     const int S = st->num_slots, B = st->num_bins;
-    const int NH = first_batch ? 1 : 2;
+    // Without new_hist only the running histogram is formed: one LDS update per element instead of two (a first batch
+    // forms a single histogram either way, its own one being the running one).
+    const bool merged_only = !first_batch && !st->new_hist;
+    const int NH = (first_batch || merged_only) ? 1 : 2;
 
     // 1. finite range of the batch, in the tensor's dtype
     const float *part_min = nullptr, *part_max = nullptr;
@@ -733,7 +736,7 @@ extern "C" int ahq_hist_update(int32_t dtype, const ahq_layout* layout, const vo
     BinArgs ba{};
     fill_geom(hp.plan, &ba);
     ba.x = x;
-    ba.ranges = pa.ranges;
+    ba.ranges = merged_only ? pa.ranges + 4 : pa.ranges;  // per slot: the batch's own range, then the running one
     ba.num_bins = B;
     ba.nhist = NH;
     ba.copies = hp.copies;

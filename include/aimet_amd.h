@@ -147,6 +147,9 @@ int ahq_minmax_to_encodings(int32_t dtype, const void* stat_min, const void* sta
  * running counts re-binned onto that range, and the batch binned onto it and added.  Bin index formula and
  * out-of-range handling are torch.histc's on CPU; counts are fp32 like the reference's.
  * All buffers are fp32 device arrays owned by the caller; hist/edges/minmax/limits persist between calls.
+ * new_hist may be NULL: the batch's own histogram is then not formed (new_edges and new_minmax still are), which
+ * leaves one histogram update per element instead of two for every batch after the first.  A caller that turns out to
+ * need it gets the same values from a first_batch call on a scratch state (collect_stats alone).
  */
 typedef struct {
     int32_t num_slots;     /* number of histograms = number of encodings of the layout */
@@ -156,7 +159,7 @@ typedef struct {
     float*  edges;         /* [num_slots][num_bins+1]   running bin edges */
     float*  minmax;        /* [num_slots][2]            running stats.min / stats.max */
     float*  limits;        /* [num_slots][2]            range limits fixed by the first batch */
-    float*  new_hist;      /* [num_slots][num_bins]     out: this batch's own histogram */
+    float*  new_hist;      /* [num_slots][num_bins]     out: this batch's own histogram (optional) */
     float*  new_edges;     /* [num_slots][num_bins+1]   out */
     float*  new_minmax;    /* [num_slots][2]            out: this batch's finite min / max */
 } ahq_hist_state;

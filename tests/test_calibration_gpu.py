@@ -86,6 +86,60 @@ def test_histogram_several_slots(device, case):
         _check_hist_lists(obs.get_stats(), ref.stats, f"running {k}")
 
 
+@pytest.mark.parametrize("case", [((1,), None, (3, 70001)), ((4, 1), None, (4, 5000)), ((2, 3), (2, 5), (4, 15))],
+                         ids=["single_slot", "rows", "blockwise"])
+def test_histogram_update_with_and_without_the_batch_histogram(device, case):
+    """ahq_hist_update with new_hist: both histograms in one pass (what the oracle's update returns and keeps);
+    without: only the running one, bit-identical, and the batch's own edges / min / max are still written."""
+    from aimet_amd.quantization.encoding_analyzer import _HistogramObserver
+
+    shape, block, xshape = case
+    both = _HistogramObserver(shape, num_bins=32, block_size=block)
+    only = _HistogramObserver(shape, num_bins=32, block_size=block)
+    ref = O.HistObserver(shape, 32, None, block)
+    g = torch.Generator().manual_seed(5)
+    for k in range(3):
+        x = torch.randn(xshape, generator=g) * (1 + 0.7 * k) + 0.1 * k
+        new_ref = ref.update(x)
+        xd = x.to(device)
+        for obs in (both, only):
+            if obs._state is None:
+                obs._state = obs._alloc(xd.device)
+        h2, e2, mm2 = both._run(xd, both._state, first=(k == 0), batch_hist=True)
+        h1, e1, mm1 = only._run(xd, only._state, first=(k == 0), batch_hist=(k == 0))
+        assert (h1 is None) == (k > 0)
+        for s_, r in enumerate(new_ref):
+            assert_same_bits(h2[s_], r.histogram, f"batch {k} slot {s_} own histogram")
+            assert_same_bits(e2[s_], r.bin_edges, f"batch {k} slot {s_} own edges")
+        assert_same_bits(e1, e2, f"batch {k} own edges")
+        assert_same_bits(mm1, mm2, f"batch {k} own min/max")
+        for key in ("hist", "edges", "minmax", "limits"):
+            assert_same_bits(only._state[key], both._state[key], f"running {key} after batch {k}")
+        for s_, r in enumerate(ref.stats):
+            assert_same_bits(only._state["hist"][s_], r.histogram, f"running histogram after batch {k} slot {s_}")
+
+
+def test_batch_histogram_is_formed_on_first_read(device):
+    from aimet_amd.quantization.encoding_analyzer import _HistogramObserver
+
+    obs = _HistogramObserver((1,), num_bins=64)
+    ref = O.HistObserver((1,), 64)
+    g = torch.Generator().manual_seed(9)
+    news = []
+    for k in range(3):
+        x = torch.randn(2, 9001, generator=g) * (k + 1)
+        want = ref.update(x)[0]  # the oracle's first list becomes its running statistics: keep the values, not the list
+        news.append((obs.update(x.to(device)), [t.clone() for t in (want.histogram, want.bin_edges, want.min, want.max)]))
+    # read in reverse order, after all updates: each list still describes its own batch
+    for k in (2, 1, 0):
+        got, (w_hist, w_edges, w_min, w_max) = news[k]
+        hist, edges, mm, _ = got.stacked()
+        assert_same_bits(hist[0], w_hist, f"batch {k} histogram")
+        assert_same_bits(edges[0], w_edges, f"batch {k} edges")
+        assert_same_bits(got[0].min, w_min, f"batch {k} min")
+        assert_same_bits(got[0].max, w_max, f"batch {k} max")
+
+
 def test_histogram_large_counts_round_like_fp32(device):
     """Running totals above 2^24 are rounded once per batch, as the reference's fp32 accumulation does."""
     from aimet_amd.quantization.encoding_analyzer import _HistogramObserver
