@@ -77,9 +77,70 @@ __global__ void minmax_to_encodings_kernel(const EncArgs a) {
     }
 }
 
+// ----------------------------------------------------------------------------------- range -> (scale, offset) --
+// AffineQuantizerBase.get_scale / _get_offset for min/max quantizers with dtype = float32
+// (aimet_torch/quantization/affine/quantizer.py:319-376):
+//   scale  = clamp_min(|float(max) - float(min)| / num_steps, minimum_scale)
+//   offset = clamp(round(min / scale) - qmin, -qmax, -qmin)          (asymmetric grids only)
+// in float32 throughout (a 16-bit min is promoted by the division with the float32 scale), division by num_steps an
+// IEEE division (what the CPU path does for tensor / number), round = half to even, NaN kept by both clamps.
+struct ScaleOffArgs {
+    const void* pmin;
+    const void* pmax;
+    float* scale;
+    float* offset;  // null: symmetric grid, the offset is a constant the caller knows
+    int64_t n;
+    float num_steps, minimum_scale, qmin, lo, hi;  // lo = -qmax, hi = -qmin
+};
+
+template <typename T>
+__global__ void range_to_scale_offset_kernel(const ScaleOffArgs a) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= a.n) return;
+    const float mn = load_f32(static_cast<const T*>(a.pmin)[i]);
+    const float mx = load_f32(static_cast<const T*>(a.pmax)[i]);
+    float s = __builtin_fabsf((mx - mn) / a.num_steps);
+    s = (s != s) ? s : fmaxf(s, a.minimum_scale);
+    a.scale[i] = s;
+    if (a.offset) {
+        const float r = __builtin_rintf(mn / s) - a.qmin;
+        a.offset[i] = (r != r) ? r : fminf(fmaxf(r, a.lo), a.hi);
+    }
+}
+
 }  // namespace ahq
 
 using namespace ahq;
+
+extern "C" int ahq_range_to_scale_offset(int32_t dtype, const void* range_min, const void* range_max,
+                                         int64_t num_encodings, int64_t qmin, int64_t qmax, double minimum_scale,
+                                         float* scale, float* offset, void* stream) {
+    if (dtype < AHQ_F32 || dtype > AHQ_BF16) return set_error("bad dtype"), AHQ_ERR_INVALID;
+    if (!range_min || !range_max || !scale) return set_error("null argument"), AHQ_ERR_INVALID;
+    if (num_encodings < 0) return set_error("negative encoding count"), AHQ_ERR_INVALID;
+    if (qmin >= qmax) return set_error("qmax must be larger than qmin"), AHQ_ERR_INVALID;
+    if (num_encodings == 0) return AHQ_OK;
+    ScaleOffArgs a{};
+    a.pmin = range_min;
+    a.pmax = range_max;
+    a.scale = scale;
+    a.offset = offset;
+    a.n = num_encodings;
+    // Python numbers reach torch's float32 kernels rounded once from double
+    a.num_steps = (float)(double)(qmax - qmin);
+    a.minimum_scale = (float)minimum_scale;
+    a.qmin = (float)(double)qmin;
+    a.lo = (float)(double)(-qmax);
+    a.hi = (float)(double)(-qmin);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const dim3 g((unsigned)((num_encodings + 255) / 256)), b(256);
+    switch (dtype) {
+        case AHQ_F32: hipLaunchKernelGGL((range_to_scale_offset_kernel<float>), g, b, 0, s, a); break;
+        case AHQ_F16: hipLaunchKernelGGL((range_to_scale_offset_kernel<f16_t>), g, b, 0, s, a); break;
+        default: hipLaunchKernelGGL((range_to_scale_offset_kernel<bf16_t>), g, b, 0, s, a); break;
+    }
+    return check_launch("range_to_scale_offset");
+}
 
 extern "C" int ahq_minmax_to_encodings(int32_t dtype, const void* stat_min, const void* stat_max, int64_t num_encodings,
                                        int64_t num_steps, int32_t symmetric, float minimum_scale_in_dtype,

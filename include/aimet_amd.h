@@ -139,6 +139,19 @@ int ahq_minmax_to_encodings(int32_t dtype, const void* stat_min, const void* sta
                             float dtype_max, float near_max_threshold, void* out_min, void* out_max, int32_t* flags,
                             void* stream);
 
+/* Replaces AffineQuantizerBase.get_scale / _get_offset with dtype = float32 for a quantizer that holds min / max
+ * (AT/quantization/affine/quantizer.py:319-376), the half-dozen elementwise launches a quantizer spends on its first
+ * forward after its range was written:
+ *   scale  = clamp_min(|float(max) - float(min)| / (qmax - qmin), minimum_scale)
+ *   offset = clamp(round(min / scale) - qmin, -qmax, -qmin)
+ * range_min / range_max: num_encodings values of `dtype`; scale / offset: float32 outputs.  offset may be NULL (a
+ * symmetric grid, whose offset is the constant -round((qmin + qmax) / 2)).  minimum_scale = _get_minimum_scale(qmax -
+ * qmin) as the Python float.
+ */
+int ahq_range_to_scale_offset(int32_t dtype, const void* range_min, const void* range_max, int64_t num_encodings,
+                              int64_t qmin, int64_t qmax, double minimum_scale, float* scale, float* offset,
+                              void* stream);
+
 /* ---------------------------------------------------------------- histogram statistics ----------------------------
  * Replaces: _HistogramObserver.collect_stats + merge_stats (AT/quantization/encoding_analyzer.py:189-332), i.e. what
  * PercentileEncodingAnalyzer / SqnrEncodingAnalyzer / TfEnhancedEncodingAnalyzer.update_stats do per batch.

@@ -297,3 +297,38 @@ def test_lpbq_encoding_export(device, shape, block_size, block_grouping, axis, c
         assert enc["axis"] in (axis, axis - len(shape))
         assert enc["output_dtype"] == f"int{compressed_bw}"
     assert enc["block_size"] == next(iter(b for b in block_size if b != 1))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16], ids=lambda d: str(d).split(".")[-1])
+@pytest.mark.parametrize("grid", [(0, 255, False), (-128, 127, True), (-8, 7, True), (0, 15, False), (0, 65535, False),
+                                  (-2 ** 31, 2 ** 31 - 1, False), (3, 11, False)], ids=str)
+def test_scale_and_offset_from_a_range_in_one_launch(device, dtype, grid):
+    """get_encodings() of a min/max quantizer derives scale and offset with ahq_range_to_scale_offset: bit-exact with
+    the reference's step-by-step float32 arithmetic (quantizer.py:319-376) on awkward ranges."""
+    from aimet_amd.quantization.affine import QuantizeDequantize
+
+    qmin, qmax, symmetric = grid
+    g = torch.Generator().manual_seed(3)
+    lo = -torch.rand(4096, generator=g) * torch.logspace(-12, 12, 4096)
+    hi = torch.rand(4096, generator=g) * torch.logspace(12, -12, 4096)
+    special = torch.tensor([0.0, -0.0, 1.0, -1.0, 1e-30, -1e-30, 3e38, -3e38, float("inf"), -float("inf"), float("nan"),
+                            0.1, -0.1, 65504.0, -65504.0, 2.5, -2.5])
+    lo = torch.cat([lo, special, special.flip(0), torch.zeros(17), -torch.ones(17)])
+    hi = torch.cat([hi, special, special, special, special])
+    lo, hi = lo.to(dtype), hi.to(dtype)
+    q = QuantizeDequantize((lo.numel(),), qmin=qmin, qmax=qmax, symmetric=symmetric).to(device=device, dtype=dtype)
+    with torch.no_grad():
+        q.set_range(lo.to(device), hi.to(device))
+    with torch.no_grad():
+        assert q._fused_scale_offset() is not None
+        enc = q.get_encodings()
+    scale = O.scale_from_minmax(lo, hi, qmin, qmax)
+    offset = O.offset_from_minmax(lo, scale, qmin, qmax, symmetric)
+    assert_same_bits(enc.scale, scale, "scale")
+    assert_same_bits(enc.offset, offset, "offset")
+    # the step-by-step form on the device gives the same answer
+    assert_same_bits(q.get_scale(), scale, "get_scale")
+    assert_same_bits(q.get_offset(), offset, "get_offset")
+    # gradients wanted: the step-by-step form runs
+    with torch.enable_grad():
+        assert q._fused_scale_offset() is None
