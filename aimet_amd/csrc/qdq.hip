@@ -480,6 +480,67 @@ __global__ __launch_bounds__(kBlock) void qdq_fwd_kernel(const QdqArgs a) {
     }
 }
 
+// Encodings that change with every element (run length 1: per-channel along the fastest axis).  The tiled kernel
+// would prepare one encoding per element; here a lane owns VEC neighbouring encodings, prepares them once and walks
+// down the rows, so loads and stores stay coalesced 16-byte vectors.  A workgroup is 64 lanes across x kColWaves waves
+// down; each wave takes kColUnroll rows per step.
+constexpr int kColWaves = 16;
+constexpr int kColThreads = kWave * kColWaves;
+constexpr int kColUnroll = 2;
+
+// the division-free form is allowed for this lane's VEC elements of one row
+template <typename IO, int VEC>
+__device__ __forceinline__ bool row_can_divide_fast(const Pack<IO, VEC>& p) {
+    float sum = 0.f;
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) sum += __builtin_fabsf(load_f32(p.v[k]));
+    return sum <= kFastDivMax;  // fails for NaN and infinity
+}
+
+template <typename IO, int VEC, typename M>
+__global__ __launch_bounds__(kColThreads) void qdq_fwd_cols_kernel(const QdqArgs a) {
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int64_t c0 = ((int64_t)blockIdx.x * kWave + lane) * VEC;
+    if (c0 >= a.J) return;
+    const IO* __restrict__ x = static_cast<const IO*>(a.x);
+    IO* __restrict__ y = static_cast<IO*>(a.y);
+    EncP e[VEC];
+    bool enc_fast = true;
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) {
+        e[k] = load_enc<M>(a, c0 + k);
+        enc_fast &= !M::kDiv || e[k].rs != 0.f;
+    }
+    const int64_t step = (int64_t)gridDim.y * kColWaves * kColUnroll;
+    for (int64_t r0 = ((int64_t)blockIdx.y * kColWaves + wave) * kColUnroll; r0 < a.I; r0 += step) {
+        Pack<IO, VEC> in[kColUnroll];
+        bool ok = enc_fast;
+#pragma unroll
+        for (int u = 0; u < kColUnroll; ++u)
+            if (r0 + u < a.I) in[u] = load_pack<IO, VEC>(x + (r0 + u) * a.J + c0);
+#pragma unroll
+        for (int u = 0; u < kColUnroll; ++u)
+            if (M::kDiv && r0 + u < a.I) ok &= row_can_divide_fast<IO, VEC>(in[u]);
+        const bool fast = !M::kDiv || __builtin_amdgcn_ballot_w64(!ok) == 0;  // wave-uniform, like the tiled kernel
+#pragma unroll
+        for (int u = 0; u < kColUnroll; ++u) {
+            if (r0 + u >= a.I) continue;
+            Pack<IO, VEC> out;
+            Pack<uint8_t, VEC> mk;
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) {
+                bool inr;
+                const float v = load_f32(in[u].v[k]);
+                const float r = fast ? M::template fwd<true>(v, e[k], a.gc, inr) : M::template fwd<false>(v, e[k], a.gc, inr);
+                out.v[k] = store_rounded<IO, M::kCD>(r);
+                mk.v[k] = inr ? 1 : 0;
+            }
+            store_pack_stream<IO, VEC>(y + (r0 + u) * a.J + c0, out);
+            if (a.mask) store_pack_stream<uint8_t, VEC>(a.mask + (r0 + u) * a.J + c0, mk);
+        }
+    }
+}
+
 template <typename IO, typename M>
 __global__ __launch_bounds__(kBlock) void qdq_fwd_generic_kernel(const QdqArgs a) {
     const IO* __restrict__ x = static_cast<const IO*>(a.x);
@@ -763,6 +824,82 @@ __global__ __launch_bounds__(kBlock) void qdq_bwd_generic_kernel(const QdqArgs a
     }
 }
 
+// Backward for run length 1 (see qdq_fwd_cols_kernel): every lane keeps the sums of its VEC encodings over the rows
+// it walks, the waves of a workgroup add theirs up in LDS, and one wave adds the workgroup's sums to the global ones.
+template <typename IO, int VEC, typename M>
+__global__ __launch_bounds__(kColThreads) void qdq_bwd_cols_kernel(const QdqArgs a) {
+    __shared__ double sums[2 * VEC * kWave];
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int64_t c0 = ((int64_t)blockIdx.x * kWave + lane) * VEC;
+    const bool live = c0 < a.J;
+    const bool want_pg = a.partials != nullptr;
+    if (want_pg) {
+        for (int i = threadIdx.x; i < 2 * VEC * kWave; i += kColThreads) sums[i] = 0.0;
+        __syncthreads();
+    }
+    if (live) {
+        const IO* __restrict__ x = static_cast<const IO*>(a.x);
+        const IO* __restrict__ g = static_cast<const IO*>(a.g);
+        IO* __restrict__ gxp = static_cast<IO*>(a.gx);
+        EncP e[VEC];
+        bool enc_fast = true;
+        double acc_s[VEC], acc_o[VEC];
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) {
+            e[k] = load_enc<M>(a, c0 + k);
+            enc_fast &= !M::kDiv || e[k].rs != 0.f;
+            acc_s[k] = acc_o[k] = 0.0;
+        }
+        const int64_t step = (int64_t)gridDim.y * kColWaves * kColUnroll;
+        for (int64_t r0 = ((int64_t)blockIdx.y * kColWaves + wave) * kColUnroll; r0 < a.I; r0 += step) {
+            Pack<IO, VEC> xin[kColUnroll], gin[kColUnroll];
+            bool ok = enc_fast;
+#pragma unroll
+            for (int u = 0; u < kColUnroll; ++u)
+                if (r0 + u < a.I) {
+                    xin[u] = load_pack<IO, VEC>(x + (r0 + u) * a.J + c0);
+                    gin[u] = load_pack<IO, VEC>(g + (r0 + u) * a.J + c0);
+                }
+#pragma unroll
+            for (int u = 0; u < kColUnroll; ++u)
+                if (M::kDiv && r0 + u < a.I) ok &= row_can_divide_fast<IO, VEC>(xin[u]);
+            const bool fast = !M::kDiv || __builtin_amdgcn_ballot_w64(!ok) == 0;
+#pragma unroll
+            for (int u = 0; u < kColUnroll; ++u) {
+                if (r0 + u >= a.I) continue;
+                Pack<IO, VEC> out;
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) {
+                    float gx, gs, go;
+                    const float gr = load_f32(gin[u].v[k]), v = load_f32(xin[u].v[k]);
+                    if (fast) M::template bwd<true>(gr, v, e[k], a.gc, gx, gs, go);
+                    else M::template bwd<false>(gr, v, e[k], a.gc, gx, gs, go);
+                    out.v[k] = store_cast<IO>(gx);
+                    acc_s[k] += (double)gs;
+                    acc_o[k] += (double)go;
+                }
+                if (gxp) store_pack_stream<IO, VEC>(gxp + (r0 + u) * a.J + c0, out);
+            }
+        }
+        if (want_pg) {
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) {
+                atomicAdd(&sums[(2 * k) * kWave + lane], acc_s[k]);
+                atomicAdd(&sums[(2 * k + 1) * kWave + lane], acc_o[k]);
+            }
+        }
+    }
+    if (!want_pg) return;
+    __syncthreads();
+    if (wave == 0 && live) {
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) {
+            atomicAdd(&a.partials[2 * (c0 + k)], sums[(2 * k) * kWave + lane]);
+            atomicAdd(&a.partials[2 * (c0 + k) + 1], sums[(2 * k + 1) * kWave + lane]);
+        }
+    }
+}
+
 __global__ void zero_f64_kernel(double* p, int64_t n) {
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) p[i] = 0.0;
 }
@@ -809,8 +946,32 @@ static bool validate_grid(const ahq_grid* g, bool backward) {
         default: { using IO = bf16_t; CALL; } break;                    \
     }
 
+// Run length 1 over several rows, whole 16-byte vectors per row: the column-walking kernels apply.
+template <typename IO>
+static bool cols_layout(const Plan& p, bool aligned) {
+    constexpr int V = IoTraits<IO>::kVec;
+    return aligned && p.cl.kind == kIJK && p.cl.K == 1 && p.cl.I > 1 && p.cl.J > 1 && p.cl.J % V == 0;
+}
+
+// grid of the column-walking kernels: x over groups of 64 lanes x VEC encodings, y over row groups; about `target`
+// workgroups, every wave with at least one step of rows
+template <typename IO>
+static dim3 cols_grid(const Plan& p, int64_t target) {
+    constexpr int V = IoTraits<IO>::kVec;
+    const int64_t gx = (p.cl.J / V + kWave - 1) / kWave;
+    const int64_t row_groups = (p.cl.I + (int64_t)kColWaves * kColUnroll - 1) / ((int64_t)kColWaves * kColUnroll);
+    int64_t gy = (target + gx - 1) / gx;
+    gy = gy < 1 ? 1 : (gy > row_groups ? row_groups : gy);
+    if (gy > 65535) gy = 65535;
+    return dim3((unsigned)gx, (unsigned)gy);
+}
+
 template <typename IO, typename M>
-static void launch_fwd(const Plan& p, const QdqArgs& a, hipStream_t st) {
+static void launch_fwd(const Plan& p, const QdqArgs& a, hipStream_t st, bool aligned) {
+    if (cols_layout<IO>(p, aligned) && (p.cl.J / IoTraits<IO>::kVec + kWave - 1) / kWave <= 0x7fffffff) {
+        hipLaunchKernelGGL((qdq_fwd_cols_kernel<IO, IoTraits<IO>::kVec, M>), cols_grid<IO>(p, 2048), dim3(kColThreads), 0, st, a);
+        return;
+    }
     if (p.cl.kind == kGeneric) {
         hipLaunchKernelGGL((qdq_fwd_generic_kernel<IO, M>), dim3(p.nblocks), dim3(kBlock), 0, st, a);
     } else if (p.vec == 1) {
@@ -830,7 +991,12 @@ static void launch_bwd_red(const Plan& p, const QdqArgs& a, hipStream_t st) {
 }
 
 template <typename IO, typename M>
-static void launch_bwd(const Plan& p, const QdqArgs& a, hipStream_t st) {
+static void launch_bwd(const Plan& p, const QdqArgs& a, hipStream_t st, bool aligned) {
+    if (cols_layout<IO>(p, aligned) && (p.red == kRedAtomic || p.red == kRedNone)) {
+        // few row groups: every workgroup ends with two global atomics per encoding
+        hipLaunchKernelGGL((qdq_bwd_cols_kernel<IO, IoTraits<IO>::kVec, M>), cols_grid<IO>(p, 512), dim3(kColThreads), 0, st, a);
+        return;
+    }
     if (p.cl.kind == kGeneric) {
         hipLaunchKernelGGL((qdq_bwd_generic_kernel<IO, M>), dim3(p.nblocks), dim3(kBlock), 0, st, a);
         return;
@@ -894,7 +1060,7 @@ extern "C" int ahq_qdq_forward(const ahq_grid* grid, const ahq_layout* layout, c
     a.emax = enc_max;
     fill_args(*grid, p, &a);
     hipStream_t st = static_cast<hipStream_t>(stream);
-    AHQ_IO_SWITCH(grid->io_dtype, AHQ_MATH_SWITCH(*grid, (launch_fwd<IO, M>(p, a, st))));
+    AHQ_IO_SWITCH(grid->io_dtype, AHQ_MATH_SWITCH(*grid, (launch_fwd<IO, M>(p, a, st, al))));
     return check_launch("ahq_qdq_forward");
 }
 
@@ -920,7 +1086,7 @@ extern "C" int ahq_dlq_fp8_qdq(int32_t dtype, const ahq_layout* layout, const vo
     a.gc.qmax = max_value;
     a.gc.zps = (float)mantissa_bits;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    launch_fwd<float, MathDlqFp8>(p, a, st);
+    launch_fwd<float, MathDlqFp8>(p, a, st, aligned16(x) && aligned16(y));
     return check_launch("ahq_dlq_fp8_qdq");
 }
 
@@ -948,9 +1114,9 @@ extern "C" int ahq_float_qdq(int32_t dtype, const ahq_layout* layout, const void
     a.gc.zps = (float)mantissa_bits;
     a.gc.flags = (overflow_to_nan ? kCastOverflowNaN : 0) | (unsigned_zero ? kCastUnsignedZero : 0);
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (dtype == AHQ_F32) launch_fwd<float, MathFloatCast<AHQ_F32>>(p, a, st);
-    else if (dtype == AHQ_F16) launch_fwd<f16_t, MathFloatCast<AHQ_F16>>(p, a, st);
-    else launch_fwd<bf16_t, MathFloatCast<AHQ_BF16>>(p, a, st);
+    if (dtype == AHQ_F32) launch_fwd<float, MathFloatCast<AHQ_F32>>(p, a, st, aligned16(x) && aligned16(y));
+    else if (dtype == AHQ_F16) launch_fwd<f16_t, MathFloatCast<AHQ_F16>>(p, a, st, aligned16(x) && aligned16(y));
+    else launch_fwd<bf16_t, MathFloatCast<AHQ_BF16>>(p, a, st, aligned16(x) && aligned16(y));
     return check_launch("ahq_float_qdq");
 }
 
@@ -997,7 +1163,7 @@ extern "C" int ahq_qdq_backward(const ahq_grid* grid, const ahq_layout* layout, 
         const int64_t n = p.cl.num_enc * 2;
         hipLaunchKernelGGL(zero_f64_kernel, dim3((unsigned)((n + 255) / 256 > 1024 ? 1024 : (n + 255) / 256)), dim3(256), 0, st, a.partials, n);
     }
-    AHQ_IO_SWITCH(grid->io_dtype, AHQ_MATH_SWITCH(*grid, (launch_bwd<IO, M>(p, a, st))));
+    AHQ_IO_SWITCH(grid->io_dtype, AHQ_MATH_SWITCH(*grid, (launch_bwd<IO, M>(p, a, st, al))));
     if (p.red == kRedTile) {
         const int64_t per_enc = p.mode == kRows ? p.cl.I * (int64_t)p.tpr : (int64_t)p.nblocks;
         if (per_enc > 1) {
