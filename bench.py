@@ -29,11 +29,18 @@ HBM_PEAK_GBS = 8000.0
 COPY_REF_ELEMS = 1 << 26
 # HBM bytes per launch of each workload's dominant kernel(s): rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE averages per
 # dispatch, scaled by what the same counters read for _copy_reference() (x2.000 for FETCH_SIZE, x1.000 for WRITE_SIZE);
-# the counter summary is profiles/hbm_traffic_pmc__c2_qdq__c3_hist.txt.  None where no counter run has been made.
+# the counter summary is profiles/hbm_traffic_pmc__qdq_c1_c2_c4__hist_c3__dlq.txt.  None where no counter run has been
+# made.
 MEASURED_TRAFFIC_BYTES = {
-    ("c2", "qdq_bwd_kernel"): int((131490.1 + 65795.8) * 1024),
-    ("c2", "qdq_fwd_kernel"): int((65942.9 + 65536.0) * 1024),
-    ("c3", "hist_update"): int((262160.2 + 1542.6 + 262299.5 + 4128.0 + 4564.8 + 127.2 + 284.9 + 199.2) * 1024),
+    ("c1", "qdq_bwd_kernel"): int((200909.2 + 100609.7) * 1024),
+    ("c1", "qdq_fwd_kernel"): int((100484.2 + 100570.7) * 1024),
+    ("c2", "qdq_bwd_kernel"): int((131547.2 + 65855.4) * 1024),
+    ("c2", "qdq_fwd_kernel"): int((65965.2 + 65950.1) * 1024),
+    ("c4", "qdq_bwd_kernel"): int((236860.2 + 121859.7) * 1024),
+    ("c4", "qdq_fwd_kernel"): int((122043.4 + 115082.2) * 1024),
+    # min/max + binning + the three small kernels between and after them
+    ("c3", "hist_update"): int((262202.4 + 1542.6 + 262290.8 + 3120.0 + 3650.0 + 127.2 + 171.6 + 139.4) * 1024),
+    ("dlq", "pdf_update"): int((262350.0 + 3072.0 + 6182.0) * 1024),
 }
 
 
@@ -465,7 +472,7 @@ def run_dlq_workload(steps, warmup, dev, with_cpu_baseline=True, batches=16, sha
                    "qdq_bit_exact": y_ok, "fp8_qdq_bit_exact": fp8_ok, "float_qdq_bit_exact": fcast_ok, "sample": "first 2 of 16 batches; 4M-element quantize-dequantize"},
         "roofline": {"bound": "hbm", "kernel": "dlq_pdf_bin_kernel", "achieved": round(bytes_upd / t_upd / 1e9, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(bytes_upd / t_upd / 1e9 / HBM_PEAK_GBS, 4),
-                     "algorithmic_bytes": bytes_upd, "traffic": None},
+                     "algorithmic_bytes": bytes_upd, "traffic": MEASURED_TRAFFIC_BYTES.get(("dlq", "pdf_update"))},
     }
     if with_cpu_baseline:
         # the scalar C restatement of the reference's loops, one thread, on a bounded slice of one batch
