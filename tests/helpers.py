@@ -33,3 +33,33 @@ def assert_close_rel(actual: torch.Tensor, expected: torch.Tensor, rel: float, w
     diff = torch.where(same, torch.zeros_like(a), (a - e).abs())
     err = diff.max().item()
     assert err <= rel * scale + abs_floor, f"{what}: max abs err {err:.3e} exceeds {rel:.1e} * {scale:.3e}"
+
+
+def histogram_merge_closed_forms():
+    """Two-batch histogram merges whose result is known without running the algorithm (every number below is an exact
+    binary fraction).  Each case: (num_bins, first batch, second batch, merged counts, (lo, hi) of the merged range).
+
+    nested    the range doubles, so every old bin lies inside one new bin: the merged histogram is the plain histogram
+              of all the data over the new range.
+    straddle  new bins of twice the width whose edges cut old bins 0 and 2 in the middle: an old bin of c values gives
+              round(c / 2) to the lower new bin (half to even: 3 -> 2, 5 -> 2) and the rest to the upper one.
+    """
+    import torch
+
+    def rep(pairs):
+        return torch.tensor([v for v, n in pairs for _ in range(n)], dtype=torch.float32)
+
+    # old range [0, 1], 8 bins of 1/8: counts 1, 2, 3, 4, 5, 6, 7, 8 (the extremes 0 and 1 are members of bins 0 and 7)
+    first = rep([(0.0, 1), (0.1875, 2), (0.3125, 3), (0.4375, 4), (0.5625, 5), (0.6875, 6), (0.8125, 7), (0.9375, 7), (1.0, 1)])
+    # new range [0, 2], 8 bins of 1/4
+    second = rep([(0.0, 1), (0.125, 2), (0.375, 1), (1.125, 3), (1.375, 2), (1.875, 4), (2.0, 1)])
+    nested = (8, first, second, [1 + 2 + 3, 3 + 4 + 1, 5 + 6, 7 + 8, 3, 2, 0, 5], (0.0, 2.0))
+
+    # old range [0, 1], 4 bins of 1/4 with counts 3, 4, 5, 6; new range [-0.375, 1.625], 4 bins of 1/2 with edges
+    # -0.375, 0.125, 0.625, 1.125, 1.625
+    first = rep([(0.0, 1), (0.0625, 2), (0.3125, 4), (0.5625, 5), (0.8125, 5), (1.0, 1)])
+    second = rep([(-0.375, 1), (0.0, 2), (0.5, 1), (1.0, 3), (1.625, 1)])
+    old = [2, (3 - 2) + 4 + 2, (5 - 2) + 6, 0]
+    new = [1 + 2, 1, 3, 1]
+    straddle = (4, first, second, [o + n for o, n in zip(old, new)], (-0.375, 1.625))
+    return {"nested": nested, "straddle": straddle}

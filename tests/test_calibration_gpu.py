@@ -119,6 +119,22 @@ def test_histogram_update_with_and_without_the_batch_histogram(device, case):
             assert_same_bits(only._state["hist"][s_], r.histogram, f"running histogram after batch {k} slot {s_}")
 
 
+@pytest.mark.parametrize("case", ["nested", "straddle"])
+def test_histogram_merge_closed_forms(device, case):
+    """The merges whose result is known by hand (tests/helpers.py), on the HIP path."""
+    from aimet_amd.quantization.encoding_analyzer import _HistogramObserver
+    from tests.helpers import histogram_merge_closed_forms
+
+    bins, first, second, counts, (lo, hi) = histogram_merge_closed_forms()[case]
+    obs = _HistogramObserver((1,), num_bins=bins)
+    obs.update(first.to(device))
+    obs.update(second.to(device))
+    st = obs.get_stats()[0]
+    assert st.histogram.tolist() == [float(c) for c in counts]
+    assert st.bin_edges[0].item() == lo and st.bin_edges[-1].item() == hi
+    assert st.min.item() == lo and st.max.item() == hi
+
+
 def test_batch_histogram_is_formed_on_first_read(device):
     from aimet_amd.quantization.encoding_analyzer import _HistogramObserver
 

@@ -8,7 +8,8 @@ against facts the mathematics fixes.  Which check pins which oracle function:
     internal_dtype             the dtype table of the reference's test_affine_quantizer.py:1761-1768
     reduce_minmax              torch.amin/amax on explicitly sliced blocks
     minmax_encodings           exact expected min/max of the reference's analyzer tests, zero / constant inputs
-    HistObserver               the reference's merge sequences (exact counts and edges), +-inf handling, count conservation
+    HistObserver               the reference's merge sequences (exact counts and edges), +-inf handling, count conservation,
+                               two merges with hand-derived results (nested bins; bins cut in half, rounding half to even)
     sqnr_encodings             uniform-distribution closed form, outlier optimum, brute-force enumeration in Python floats
     lpbq_scale                 closed form max(1, round(s / gamma)) * gamma
 """
@@ -172,6 +173,20 @@ def test_histogram_counts_are_conserved_and_finite_only():
         total += 9999  # everything but the NaN lands in some bin (infinities in the edge bins)
         assert abs(obs.stats[0].histogram.sum().item() - total) <= 2 * (k + 1)  # re-binning rounds per source bin
         assert math.isfinite(obs.stats[0].min.item()) and math.isfinite(obs.stats[0].max.item())
+
+
+@pytest.mark.parametrize("case", ["nested", "straddle"])
+def test_histogram_merge_closed_forms(case):
+    from tests.helpers import histogram_merge_closed_forms
+
+    bins, first, second, counts, (lo, hi) = histogram_merge_closed_forms()[case]
+    obs = O.HistObserver((1,), bins)
+    obs.update(first)
+    obs.update(second)
+    st = obs.stats[0]
+    assert st.histogram.tolist() == [float(c) for c in counts]
+    assert st.bin_edges[0].item() == lo and st.bin_edges[-1].item() == hi
+    assert st.min.item() == lo and st.max.item() == hi
 
 
 def test_lpbq_closed_form():
