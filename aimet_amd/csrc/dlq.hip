@@ -474,18 +474,25 @@ __global__ __launch_bounds__(kMaxCand) void dlq_tfe_candidates_kernel(const TfeA
 
 // _quantAndSatCost (TfEnhancedEncodingAnalyzer.cpp:273-335), one candidate per lane.  The three sums run over the
 // buckets in increasing order like the reference's three loops; pow(x, 2) is x*x.
-__global__ __launch_bounds__(kWave) void dlq_tfe_cost_kernel(const TfeArgs a) {
-    const int s = blockIdx.y;
+// One workgroup per slot: its waves share one staged copy of the slot's statistics (18 KB of LDS, so eight
+// workgroups = 64 waves fit a CU; with a workgroup per wave the LDS allowed two waves per SIMD and every wave staged
+// the statistics for itself).  Waves without a valid candidate leave at once.
+__global__ __launch_bounds__(kMaxCand) void dlq_tfe_cost_kernel(const TfeArgs a) {
+    const int s = blockIdx.x;
     if (a.meta[4 * s + 1] == 0) return;
     __shared__ double sh_pdf[kPdf];
     __shared__ float sh_c[kPdf];
-    for (int i = threadIdx.x; i < kPdf; i += kWave) {
+    for (int i = threadIdx.x; i < kPdf; i += kMaxCand) {
         sh_pdf[i] = a.pdf[(size_t)s * kPdf + i];
         sh_c[i] = a.centers[(size_t)s * kPdf + i];
     }
     __syncthreads();
-    const int k = blockIdx.x * kWave + threadIdx.x;
+    const int k = threadIdx.x;
     const bool ok = a.cand_ok[(size_t)s * kMaxCand + k] != 0;
+    if (__builtin_amdgcn_ballot_w64(ok) == 0) {
+        a.cost[(size_t)s * kMaxCand + k] = kDblMax;
+        return;
+    }
     const float delta = a.cand_delta[(size_t)s * kMaxCand + k];
     const int offset = a.cand_off[(size_t)s * kMaxCand + k];
     const double* xl = a.xleft + (size_t)s * kPdf;
@@ -989,7 +996,7 @@ extern "C" int ahq_dlq_tfe_encodings(const ahq_dlq_pdf_state* st, int32_t bw, in
     // form issues about eight times the instructions of the lane-per-candidate one, so it pays only while the latter
     // cannot fill the GPU.
     if (st->num_slots <= 16) hipLaunchKernelGGL(dlq_tfe_cost_wave_kernel, dim3(kMaxCand, st->num_slots), dim3(kWave), 0, s, a);
-    else hipLaunchKernelGGL(dlq_tfe_cost_kernel, dim3(kMaxCand / kWave, st->num_slots), dim3(kWave), 0, s, a);
+    else hipLaunchKernelGGL(dlq_tfe_cost_kernel, dim3(st->num_slots), dim3(kMaxCand), 0, s, a);
     hipLaunchKernelGGL(dlq_tfe_select_kernel, dim3(st->num_slots), dim3(kWave), 0, s, a);
     return check_launch("dlq_tfe_encodings");
 }
