@@ -17,6 +17,7 @@ struct SqnrArgs {
     int32_t num_slots, num_bins, num_deltas, num_offsets;  // num_offsets counts the observed offset (asymmetric)
     int32_t symmetric;
     int32_t stat_dtype;     // dtype the stored min/max live in (arithmetic on them happens in that dtype)
+    int32_t pairs_per_block;  // (delta, offset) candidates one workgroup prices
     float num_steps;
     float min_scale;        // minimum_scale as float
     float min_range;        // float(minimum_scale * num_steps)
@@ -75,11 +76,17 @@ __device__ __forceinline__ Cand candidate(const SqnrArgs& a, int s, int d, int o
 
 constexpr int kSqnrMaxBins = 4096;
 
+// A workgroup stages one slot's histogram and bin centres and prices kPairsPerBlock (delta, offset) candidates, one
+// wave per candidate at a time.  Candidates are numbered delta-major across the whole grid, so a symmetric search
+// (one offset) fills its workgroups as well as an asymmetric one.
+constexpr int kPairsPerBlock = 64;  // at most; fewer when that leaves the GPU short of workgroups
+
 __global__ __launch_bounds__(kBlock) void sqnr_noise_kernel(const SqnrArgs a) {
-    __shared__ float h_lds[kSqnrMaxBins];
-    __shared__ float m_lds[kSqnrMaxBins];
-    const int s = blockIdx.y, d = blockIdx.x;
+    extern __shared__ float sqnr_lds[];  // [2][num_bins]
+    const int s = blockIdx.y;
     const int B = a.num_bins, O = a.num_offsets;
+    float* h_lds = sqnr_lds;
+    float* m_lds = sqnr_lds + B;
     const float* e = a.edges + (size_t)s * (B + 1);
     const float w = e[1] - e[0];
     const float first_mid = e[0] + w / 2.f;
@@ -90,7 +97,11 @@ __global__ __launch_bounds__(kBlock) void sqnr_noise_kernel(const SqnrArgs a) {
     __syncthreads();
     const int lane = threadIdx.x & (kWave - 1);
     const bool use_gamma = a.gamma != 1.0f;
-    for (int o = threadIdx.x / kWave; o < O; o += kBlock / kWave) {
+    const int pairs = a.num_deltas * O;
+    const int p0 = blockIdx.x * a.pairs_per_block;
+    const int p1 = p0 + a.pairs_per_block < pairs ? p0 + a.pairs_per_block : pairs;
+    for (int p = p0 + threadIdx.x / kWave; p < p1; p += kBlock / kWave) {
+        const int d = p / O, o = p - d * O;
         const Cand c = candidate(a, s, d, o);
         double acc = 0.0;
         for (int b = lane; b < B; b += kWave) {
@@ -197,7 +208,14 @@ extern "C" int ahq_sqnr_search(const ahq_sqnr_params* p, const float* hist, cons
     a.out = out;
     a.best_index = best_index;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    hipLaunchKernelGGL(sqnr_noise_kernel, dim3(a.num_deltas, a.num_slots), dim3(kBlock), 0, st, a);
+    // a per-tensor search has a few thousand candidates in all: one per wave, so that its latency is that of a single
+    // candidate; with many slots a workgroup prices up to 64 per staged histogram
+    const int pairs = a.num_deltas * a.num_offsets;
+    int64_t ppb = ((int64_t)pairs * a.num_slots) / 2048;
+    ppb = ppb < kBlock / kWave ? kBlock / kWave : (ppb > kPairsPerBlock ? kPairsPerBlock : ppb);
+    a.pairs_per_block = (int)ppb;
+    hipLaunchKernelGGL(sqnr_noise_kernel, dim3((unsigned)((pairs + ppb - 1) / ppb), a.num_slots), dim3(kBlock),
+                       2 * (size_t)a.num_bins * sizeof(float), st, a);
     hipLaunchKernelGGL(sqnr_select_kernel, dim3(a.num_slots), dim3(kBlock), 0, st, a);
     return check_launch("ahq_sqnr_search");
 }
