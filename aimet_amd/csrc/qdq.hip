@@ -950,7 +950,8 @@ static bool validate_grid(const ahq_grid* g, bool backward) {
 template <typename IO>
 static bool cols_layout(const Plan& p, bool aligned) {
     constexpr int V = IoTraits<IO>::kVec;
-    return aligned && p.cl.kind == kIJK && p.cl.K == 1 && p.cl.I > 1 && p.cl.J > 1 && p.cl.J % V == 0;
+    // at least half a wave of lanes must own columns, or the tiled kernel's full waves win
+    return aligned && p.cl.kind == kIJK && p.cl.K == 1 && p.cl.I > 1 && p.cl.J % V == 0 && p.cl.J / V >= kWave / 2;
 }
 
 // grid of the column-walking kernels: x over groups of 64 lanes x VEC encodings, y over row groups; about `target`

@@ -379,7 +379,7 @@ static void launch_mm(const Plan& p, const MmArgs& a, hipStream_t st) {
         }
     } else if (p.red == kRedSeg) {
         launch_mm_red<IO, kRedSeg, FINITE>(p, a, st);
-    } else if (p.cl.K == 1 && p.cl.J % IoTraits<IO>::kVec == 0 && aligned16(a.x) && p.cl.I > 1 &&
+    } else if (p.cl.K == 1 && p.cl.J % IoTraits<IO>::kVec == 0 && p.cl.J / IoTraits<IO>::kVec >= kWave / 2 && aligned16(a.x) && p.cl.I > 1 &&
                (p.cl.I + kColRows - 1) / kColRows <= 65535) {
         constexpr int V = IoTraits<IO>::kVec;
         const dim3 g((unsigned)((p.cl.J / V + kBlock - 1) / kBlock), (unsigned)((p.cl.I + kColRows - 1) / kColRows));

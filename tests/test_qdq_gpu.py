@@ -31,8 +31,9 @@ LAYOUTS = [
     ((10, 12), (12,), None),               # per-channel on the fastest axis
     ((6, 10), (6, 1), None),               # run length not a multiple of the vector width
     ((5, 7, 64), (5, 1, 2), (1, -1, -1)),  # wildcard block sizes
-    ((70, 64), (64,), None),               # run length 1 over whole vectors: column-walking kernels
-    ((1100, 24), (1, 24), None),           # same, many rows per workgroup, lanes without columns
+    ((70, 256), (256,), None),             # run length 1 over whole vectors: column-walking kernels
+    ((1100, 264), (1, 264), None),         # same, many rows per workgroup, lanes without columns
+    ((1100, 24), (1, 24), None),           # too few columns for them: tiled kernel
     ((3, 40, 1536), (1536,), None),        # same, several groups of 64 lanes across
 ]
 
