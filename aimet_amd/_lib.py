@@ -108,6 +108,8 @@ _SIGNATURES = {
     "ahq_minmax_workspace_bytes": (ctypes.c_size_t, [ctypes.POINTER(Layout)]),
     "ahq_minmax": (ctypes.c_int, [ctypes.c_int32, ctypes.POINTER(Layout), _P, _P, _P, _P, _P, ctypes.c_int, _P,
                                   ctypes.c_size_t, _P]),
+    "ahq_minmax_copy": (ctypes.c_int, [ctypes.c_int32, ctypes.POINTER(Layout), _P, _P, _P, _P, _P, _P, ctypes.c_int, _P,
+                                       ctypes.c_size_t, _P]),
     "ahq_minmax_to_encodings": (ctypes.c_int, [ctypes.c_int32, _P, _P, ctypes.c_int64, ctypes.c_int64, ctypes.c_int32,
                                                ctypes.c_float, ctypes.c_float, ctypes.c_float, ctypes.c_float, _P, _P, _P,
                                                _P]),

@@ -25,6 +25,7 @@ struct MmArgs : Geom {
     void* run_min;          // optional running statistics folded with torch.minimum / torch.maximum semantics
     void* run_max;
     int32_t finite_only;
+    void* copy;             // optional: the tensor is also copied there by the pass that reads it (single encoding)
 };
 
 struct MinMax {
@@ -199,11 +200,16 @@ __global__ __launch_bounds__(kBlock) void minmax_flat_kernel(const MmArgs a) {
     const int64_t v0 = (int64_t)blockIdx.x * kFlatTileVec;
     const int64_t left = a.nvec - v0;
     const IO* __restrict__ x = static_cast<const IO*>(a.x) + v0 * VEC;
+    IO* __restrict__ cp = a.copy ? static_cast<IO*>(a.copy) + v0 * VEC : nullptr;
     MinMax acc = mm_identity();
     Pack<IO, VEC> in[kFlatUnroll];
     if (left >= kFlatTileVec) {
 #pragma unroll
         for (int u = 0; u < kFlatUnroll; ++u) in[u] = load_pack<IO, VEC>(x + (int64_t)(u * kBlock + threadIdx.x) * VEC);
+        if (cp) {
+#pragma unroll
+            for (int u = 0; u < kFlatUnroll; ++u) store_pack<IO, VEC>(cp + (int64_t)(u * kBlock + threadIdx.x) * VEC, in[u]);
+        }
 #pragma unroll
         for (int u = 0; u < kFlatUnroll; ++u)
 #pragma unroll
@@ -213,6 +219,7 @@ __global__ __launch_bounds__(kBlock) void minmax_flat_kernel(const MmArgs a) {
             const int lv = u * kBlock + threadIdx.x;
             if (lv < left) {
                 const Pack<IO, VEC> p = load_pack<IO, VEC>(x + (int64_t)lv * VEC);
+                if (cp) store_pack<IO, VEC>(cp + (int64_t)lv * VEC, p);
 #pragma unroll
                 for (int k = 0; k < VEC; ++k) mm_add(acc, load_f32(p.v[k]), FINITE);
             }
@@ -220,7 +227,11 @@ __global__ __launch_bounds__(kBlock) void minmax_flat_kernel(const MmArgs a) {
     }
     if (VEC > 1 && blockIdx.x == 0) {  // elements past the last full vector
         const int64_t i = a.nvec * VEC + threadIdx.x;
-        if (i < a.numel) mm_add(acc, load_f32(static_cast<const IO*>(a.x)[i]), FINITE);
+        if (i < a.numel) {
+            const IO v = static_cast<const IO*>(a.x)[i];
+            if (a.copy) static_cast<IO*>(a.copy)[i] = v;
+            mm_add(acc, load_f32(v), FINITE);
+        }
     }
     const MinMax b = mm_block_reduce(acc, red_smem);
     if (threadIdx.x == 0) {
@@ -451,15 +462,15 @@ extern "C" size_t ahq_minmax_workspace_bytes(const ahq_layout* layout) {
     return need;
 }
 
-extern "C" int ahq_minmax(int32_t dtype, const ahq_layout* layout, const void* x, void* out_min, void* out_max,
-                          void* run_min, void* run_max, int finite_only, void* workspace, size_t workspace_bytes,
-                          void* stream) {
+static int minmax_impl(int32_t dtype, const ahq_layout* layout, const void* x, void* copy, void* out_min, void* out_max,
+                       void* run_min, void* run_max, int finite_only, void* workspace, size_t workspace_bytes,
+                       void* stream) {
     if (dtype < AHQ_F32 || dtype > AHQ_BF16) return set_error("bad dtype"), AHQ_ERR_INVALID;
     if (!layout) return set_error("layout is null"), AHQ_ERR_INVALID;
     if (!out_min || !out_max) return set_error("out_min or out_max is null"), AHQ_ERR_INVALID;
     if ((run_min == nullptr) != (run_max == nullptr)) return set_error("run_min and run_max must be given together"), AHQ_ERR_INVALID;
     Plan p;
-    if (!make_plan(dtype, *layout, aligned16(x), true, &p)) return AHQ_ERR_INVALID;
+    if (!make_plan(dtype, *layout, aligned16(x) && aligned16(copy), true, &p)) return AHQ_ERR_INVALID;
     if (p.cl.numel == 0) return set_error("cannot reduce an empty tensor"), AHQ_ERR_INVALID;
     if (!x) return set_error("x is null"), AHQ_ERR_INVALID;
     const size_t need = p.ws_elems * 12;
@@ -484,6 +495,14 @@ extern "C" int ahq_minmax(int32_t dtype, const ahq_layout* layout, const void* x
         a.key_max = reinterpret_cast<unsigned int*>(w + p.ws_elems * 4);
     }
     hipStream_t st = static_cast<hipStream_t>(stream);
+    if (copy) {
+        // the streaming kernel of the single-encoding case writes the copy itself; other layouts copy separately
+        if (p.cl.kind == kIJK && p.cl.J == 1) {
+            a.copy = copy;
+        } else if (hipMemcpyAsync(copy, x, (size_t)p.cl.numel * io_size(dtype), hipMemcpyDeviceToDevice, st) != hipSuccess) {
+            return set_error("device-to-device copy failed"), AHQ_ERR_LAUNCH;
+        }
+    }
 #define AHQ_MM(IO) do { if (finite_only == 1) launch_mm<IO, true>(p, a, st); else launch_mm<IO, false>(p, a, st); } while (0)
     switch (dtype) {
         case AHQ_F32: AHQ_MM(float); break;
@@ -492,4 +511,20 @@ extern "C" int ahq_minmax(int32_t dtype, const ahq_layout* layout, const void* x
     }
 #undef AHQ_MM
     return check_launch("ahq_minmax");
+}
+
+extern "C" int ahq_minmax(int32_t dtype, const ahq_layout* layout, const void* x, void* out_min, void* out_max,
+                          void* run_min, void* run_max, int finite_only, void* workspace, size_t workspace_bytes,
+                          void* stream) {
+    return minmax_impl(dtype, layout, x, nullptr, out_min, out_max, run_min, run_max, finite_only, workspace,
+                       workspace_bytes, stream);
+}
+
+extern "C" int ahq_minmax_copy(int32_t dtype, const ahq_layout* layout, const void* x, void* y, void* out_min,
+                               void* out_max, void* run_min, void* run_max, int finite_only, void* workspace,
+                               size_t workspace_bytes, void* stream) {
+    if (!y) return set_error("y is null"), AHQ_ERR_INVALID;
+    if (y == x) return set_error("y must not alias x"), AHQ_ERR_INVALID;
+    return minmax_impl(dtype, layout, x, y, out_min, out_max, run_min, run_max, finite_only, workspace, workspace_bytes,
+                       stream);
 }

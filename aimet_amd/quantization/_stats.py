@@ -28,13 +28,15 @@ def _check_reducible(x: torch.Tensor, shape: Tuple[int, ...], block_size) -> Non
 
 
 def reduce_min_max(x: torch.Tensor, shape: Tuple[int, ...], block_size=None, *, finite_only: bool = False,
-                   running: Optional[Tuple[torch.Tensor, torch.Tensor]] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+                   running: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
+                   copy_to: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
     """Per-encoding minimum and maximum of ``x`` in one pass (both extrema from a single read of the tensor).
 
     Equivalent of ``reduce(x, shape, torch.amin, block_size)`` and ``reduce(x, shape, torch.amax, block_size)``
     (aimet_torch/utils.py:1115-1148, aimet_torch/quantization/encoding_analyzer.py:80-94).  The batch result is
     returned; with ``running`` it is also folded into the given (min, max) tensors in place, as
-    ``_MinMaxObserver.merge_stats`` does.
+    ``_MinMaxObserver.merge_stats`` does.  ``copy_to``: a contiguous tensor of ``x``'s shape and dtype that receives a
+    copy of ``x`` from the same pass (``ahq_minmax_copy``).
     """
     _lib.require_device(x, "input tensor")
     if x.dtype not in _lib.DTYPE_CODE:
@@ -56,6 +58,17 @@ def reduce_min_max(x: torch.Tensor, shape: Tuple[int, ...], block_size=None, *, 
     mx = torch.empty(shape, dtype=x.dtype, device=x.device)
     nbytes = lib.ahq_minmax_workspace_bytes(layout)
     ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device) if nbytes else None
+    if copy_to is not None:
+        if (copy_to.dtype != x.dtype or copy_to.device != x.device or copy_to.shape != x.shape
+                or not copy_to.is_contiguous()):
+            raise RuntimeError("copy_to must be a contiguous tensor of the input's shape, dtype and device")
+        _lib.check(
+            lib.ahq_minmax_copy(_lib.DTYPE_CODE[x.dtype], layout, xd.data_ptr(), copy_to.data_ptr(), mn.data_ptr(),
+                                mx.data_ptr(), _lib.ptr(rmn), _lib.ptr(rmx), 1 if finite_only else 0, _lib.ptr(ws),
+                                nbytes, _lib.current_stream(x.device)),
+            "ahq_minmax_copy",
+        )
+        return mn, mx
     _lib.check(
         lib.ahq_minmax(_lib.DTYPE_CODE[x.dtype], layout, xd.data_ptr(), mn.data_ptr(), mx.data_ptr(),
                        _lib.ptr(rmn), _lib.ptr(rmx), 1 if finite_only else 0, _lib.ptr(ws), nbytes,

@@ -307,10 +307,16 @@ class AffineQuantizerBase(QuantizerBase, _GridMixin):
                 input = input.as_subclass(torch.Tensor)
             if input.numel() == 0:
                 return inner_forward(input)
-            batch_stats = self.encoding_analyzer.update_stats(input)
             if passthrough:
-                # the input is only observed; the dynamic encodings of this batch would go unused
+                # the input is only observed; the dynamic encodings of this batch would go unused.  A min/max
+                # analyzer writes the clone from the pass that reads the tensor
+                fused = getattr(self.encoding_analyzer, "update_stats_and_clone", None)
+                if (fused is not None and input.is_cuda and input.dtype in _lib.DTYPE_CODE and input.is_contiguous()
+                        and not (torch.is_grad_enabled() and input.requires_grad)):
+                    return fused(input)[1]
+                self.encoding_analyzer.update_stats(input)
                 return inner_forward(input)
+            batch_stats = self.encoding_analyzer.update_stats(input)
             lo, hi = self.encoding_analyzer.compute_encodings_from_stats(
                 batch_stats, self._num_steps_for_calibration(), self.symmetric
             )

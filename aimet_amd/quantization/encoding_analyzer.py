@@ -137,8 +137,9 @@ class _MinMaxObserver(_Observer[_MinMaxRange]):
         self.stats = _MinMaxRange(new_min, new_max)
 
     @torch.no_grad()
-    def update(self, input_tensor: torch.Tensor) -> _MinMaxRange:
-        """collect + merge in one launch: the running fold happens where the reduction finishes."""
+    def update(self, input_tensor: torch.Tensor, copy_to: Optional[torch.Tensor] = None) -> _MinMaxRange:
+        """collect + merge in one launch: the running fold happens where the reduction finishes.  ``copy_to``
+        receives a copy of the input from the same pass (what pass-through calibration returns)."""
         cur = self.stats
         fused = (
             cur.min is not None and cur.max is not None
@@ -146,9 +147,11 @@ class _MinMaxObserver(_Observer[_MinMaxRange]):
             and cur.min.is_contiguous() and cur.max.is_contiguous()
         )
         if fused:
-            mn, mx = reduce_min_max(input_tensor, self.shape, self.block_size, running=(cur.min, cur.max))
+            mn, mx = reduce_min_max(input_tensor, self.shape, self.block_size, running=(cur.min, cur.max),
+                                    copy_to=copy_to)
             return _MinMaxRange(mn, mx)
-        new = self.collect_stats(input_tensor)
+        mn, mx = reduce_min_max(input_tensor, self.shape, self.block_size, copy_to=copy_to)
+        new = _MinMaxRange(mn, mx)
         self.merge_stats(new)
         return new
 
@@ -318,6 +321,12 @@ class MinMaxEncodingAnalyzer(EncodingAnalyzer[_MinMaxRange]):
 
     def __init__(self, shape, block_size=None):
         super().__init__(_MinMaxObserver(shape, block_size))
+
+    @torch.no_grad()
+    def update_stats_and_clone(self, input_tensor: torch.Tensor):
+        """update_stats(input) and input.clone() with one read of the tensor.  Returns (batch statistics, clone)."""
+        out = torch.empty(input_tensor.shape, dtype=input_tensor.dtype, device=input_tensor.device)
+        return self.observer.update(input_tensor, copy_to=out), out
 
     @torch.no_grad()
     def compute_encodings_from_stats(self, stats: _MinMaxRange, num_steps: int, is_symmetric: bool):

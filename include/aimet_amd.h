@@ -125,6 +125,15 @@ size_t ahq_minmax_workspace_bytes(const ahq_layout* layout);
 int    ahq_minmax(int32_t dtype, const ahq_layout* layout, const void* x, void* out_min, void* out_max,
                   void* run_min, void* run_max, int finite_only, void* workspace, size_t workspace_bytes, void* stream);
 
+/* ahq_minmax that also writes y = x (same dtype and layout, y not aliasing x).  Replaces the observe-then-clone of an
+ * input / output quantizer in pass-through calibration: AffineQuantizerBase._compute_encodings(passthrough=True)
+ * observes the tensor and returns torch.Tensor.clone(input) (AT/quantization/affine/quantizer.py:601-640).  With one
+ * encoding the pass that reads the tensor writes the copy; other layouts reduce and copy separately.
+ */
+int    ahq_minmax_copy(int32_t dtype, const ahq_layout* layout, const void* x, void* y, void* out_min, void* out_max,
+                       void* run_min, void* run_max, int finite_only, void* workspace, size_t workspace_bytes,
+                       void* stream);
+
 /* Replaces MinMaxEncodingAnalyzer.compute_encodings_from_stats (AT/quantization/encoding_analyzer.py:425-481) and the
  * checks of _flag_extreme_min_max (:484-498): zero forced into the range, ranges narrower than the minimum scale
  * widened, symmetric grids re-centred, the result clamped to the statistics dtype.  stat_min / stat_max / out_min /

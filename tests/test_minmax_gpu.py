@@ -119,3 +119,55 @@ def test_nan_and_inf_in_the_aggregating_paths(device, case):
     assert_same_bits(lo, lo_ref, "finite min")
     assert_same_bits(hi, hi_ref, "finite max")
     del fin
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=lambda d: str(d).split(".")[-1])
+@pytest.mark.parametrize("case", [((37, 129), (), None), ((3, 1024, 1027), (1,), None), ((5,), (), None),
+                                  ((64, 4096), (64, 1), None), ((200, 2056), (2056,), None)],
+                         ids=lambda c: "x".join(map(str, c[0])) + "_" + "x".join(map(str, c[1])))
+def test_min_max_with_copy(device, case, dtype):
+    """ahq_minmax_copy: the statistics of ahq_minmax and a bit-identical copy of the tensor (NaN payloads and signs of
+    zero included), with and without running statistics; layouts with several encodings copy separately."""
+    from aimet_amd.quantization._stats import reduce_min_max
+
+    shape, enc_shape, block = case
+    g = torch.Generator().manual_seed(sum(shape) + 1)
+    x = (torch.randn(shape, generator=g) * 3).to(dtype)
+    x.view(-1)[0] = -0.0
+    xd = x.to(device)
+    mn_ref, mx_ref = reduce_min_max(xd, enc_shape, block)
+    out = torch.full_like(xd, 7.0)
+    mn, mx = reduce_min_max(xd, enc_shape, block, copy_to=out)
+    assert_same_bits(mn, mn_ref.cpu(), "min")
+    assert_same_bits(mx, mx_ref.cpu(), "max")
+    assert_same_bits(out, x, "copy")
+    x2 = (torch.randn(shape, generator=g) * 2 + 0.5).to(dtype)
+    if x2.numel() > 3:
+        x2.view(-1)[2] = float("nan")
+    out2 = torch.empty_like(xd)
+    reduce_min_max(x2.to(device), enc_shape, block, running=(mn, mx), copy_to=out2)
+    rm, rx = mn_ref.clone(), mx_ref.clone()
+    reduce_min_max(x2.to(device), enc_shape, block, running=(rm, rx))
+    assert_same_bits(mn, rm.cpu(), "running min")
+    assert_same_bits(mx, rx.cpu(), "running max")
+    assert out2.view(torch.int16 if dtype != torch.float32 else torch.int32).cpu().equal(
+        x2.view(torch.int16 if dtype != torch.float32 else torch.int32)), "copy of a tensor holding NaN"
+
+
+def test_passthrough_calibration_returns_a_clone(device):
+    """Whole-model calibration observes and passes the input on as a new tensor with the same values."""
+    from aimet_amd.quantization.affine import QuantizeDequantize
+
+    q = QuantizeDequantize((), 8, False).to(device)
+    x = torch.randn(3, 1000, device=device, dtype=torch.bfloat16)
+    with torch.no_grad(), q._compute_encodings(passthrough=True):
+        y = q(x)
+        y2 = q(x.t())  # not contiguous: the step-by-step form
+    assert y.data_ptr() != x.data_ptr() and torch.equal(y, x)
+    assert torch.equal(y2, x.t()) and y2.stride() == x.t().clone().stride()
+    assert float(q.min.detach()) <= float(x.float().min()) and float(q.max.detach()) >= float(x.float().max())
+    xg = x.float().requires_grad_(True)
+    with q._compute_encodings(passthrough=True):
+        yg = q(xg)
+    yg.sum().backward()
+    assert torch.equal(xg.grad, torch.ones_like(xg))
