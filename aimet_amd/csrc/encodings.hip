@@ -9,6 +9,7 @@
 
 #include "ahq_device.h"
 #include "ahq_host.h"
+#include "layout.h"
 
 namespace ahq {
 
@@ -108,9 +109,121 @@ __global__ void range_to_scale_offset_kernel(const ScaleOffArgs a) {
     }
 }
 
+// --------------------------------------------------------------------- "is this tensor already on a grid" test --
+// The early exit of _decompose_prequantized_tensor (aimet_torch/utils.py:2098-2118), which runs on every weight at
+// the start of a calibration: of the first 64 blocks take the first 2 * num_levels elements each, as float
+// magnitudes; a block with more than num_levels distinct ones cannot lie on the grid.  The reference sorts each
+// sample and counts the places where neighbours differ (NaN differs from everything).  One workgroup does the same
+// with a bitonic sort in LDS over as many blocks at a time as fit, and writes the verdict: 1 = no sampled block rules
+// the grid out.
+constexpr int kProbeThreads = 1024;
+constexpr int kProbeKeys = 8192;   // sort keys held in LDS (32 KB)
+constexpr int kProbeBlocks = 64;   // blocks the reference samples
+
+struct ProbeArgs {
+    const void* x;
+    uint8_t* verdict;
+    int64_t I, J, K;     // flat = (i * J + j) * K + k, block index j
+    int32_t nblocks;     // min(J, 64)
+    int32_t n;           // sampled elements per block
+    int32_t padded;      // n rounded up to a power of two
+    int32_t num_levels;
+};
+
+template <typename T>
+__global__ __launch_bounds__(kProbeThreads) void grid_probe_kernel(const ProbeArgs a) {
+    __shared__ unsigned int keys[kProbeKeys];
+    __shared__ int exceeded;
+    if (threadIdx.x == 0) exceeded = 0;
+    const int P = a.padded, per_round = kProbeKeys / P;
+    const T* __restrict__ x = static_cast<const T*>(a.x);
+    for (int b0 = 0; b0 < a.nblocks; b0 += per_round) {
+        const int nb = a.nblocks - b0 < per_round ? a.nblocks - b0 : per_round;
+        const int total = nb * P;
+        __syncthreads();
+        // magnitudes as unsigned keys (their order is the order of the magnitudes; NaN above infinity); the padding
+        // sorts behind every element
+        for (int t = threadIdx.x; t < total; t += kProbeThreads) {
+            const int seg = t / P, m = t - seg * P;
+            unsigned int key = 0xffffffffu;
+            if (m < a.n) {
+                const int64_t i = m / a.K, k = m - i * a.K;
+                key = f32_to_bits(load_f32(x[(i * a.J + (b0 + seg)) * a.K + k])) & 0x7fffffffu;
+            }
+            keys[t] = key;
+        }
+        __syncthreads();
+        for (int k = 2; k <= P; k <<= 1) {
+            for (int j = k >> 1; j >= 1; j >>= 1) {
+                for (int t = threadIdx.x; t < total; t += kProbeThreads) {
+                    const int u = t ^ j;
+                    if (u > t) {
+                        const bool up = ((t & (P - 1)) & k) == 0;  // every segment ends ascending
+                        const unsigned int kt = keys[t], ku = keys[u];
+                        if ((kt > ku) == up) {
+                            keys[t] = ku;
+                            keys[u] = kt;
+                        }
+                    }
+                }
+                __syncthreads();
+            }
+        }
+        // distinct values of a segment = 1 + places where float neighbours differ; one wave per segment at a time
+        const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+        for (int seg = wave; seg < nb; seg += kProbeThreads / kWave) {
+            int differ = 0;
+            for (int m = 1 + lane; m < a.n; m += kWave) {
+                const float v0 = bits_to_f32(keys[seg * P + m - 1]), v1 = bits_to_f32(keys[seg * P + m]);
+                differ += (v1 != v0) ? 1 : 0;
+            }
+#pragma unroll
+            for (int s = kWave / 2; s >= 1; s >>= 1) differ += __shfl_xor(differ, s, kWave);
+            if (lane == 0 && differ + 1 > a.num_levels) atomicOr(&exceeded, 1);
+        }
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) *a.verdict = exceeded ? 0 : 1;
+}
+
 }  // namespace ahq
 
 using namespace ahq;
+
+extern "C" int ahq_grid_probe(int32_t dtype, const ahq_layout* layout, const void* x, int64_t num_levels,
+                              uint8_t* verdict, void* stream) {
+    if (dtype < AHQ_F32 || dtype > AHQ_BF16) return set_error("bad dtype"), AHQ_ERR_INVALID;
+    if (!layout || !x || !verdict) return set_error("null argument"), AHQ_ERR_INVALID;
+    if (num_levels < 1) return set_error("num_levels must be positive"), AHQ_ERR_INVALID;
+    CanonLayout c;
+    const char* err = nullptr;
+    if (!canonicalize(*layout, &c, &err)) return set_error(err), AHQ_ERR_INVALID;
+    if (c.kind != kIJK) return set_error("blocks along several dimensions are not supported by the grid test"), AHQ_ERR_UNSUPPORTED;
+    if (c.numel == 0) return set_error("empty tensor"), AHQ_ERR_INVALID;
+    const int64_t block_elems = c.I * c.K;
+    if (block_elems <= num_levels) return set_error("blocks no larger than the grid need no test"), AHQ_ERR_INVALID;
+    const int64_t n = block_elems < 2 * num_levels ? block_elems : 2 * num_levels;
+    int64_t padded = 1;
+    while (padded < n) padded <<= 1;
+    if (padded > kProbeKeys) return set_error("grid too wide for the on-device grid test"), AHQ_ERR_UNSUPPORTED;
+    ProbeArgs a{};
+    a.x = x;
+    a.verdict = verdict;
+    a.I = c.I;
+    a.J = c.J;
+    a.K = c.K;
+    a.nblocks = (int32_t)(c.J < kProbeBlocks ? c.J : kProbeBlocks);
+    a.n = (int32_t)n;
+    a.padded = (int32_t)(padded < 2 ? 2 : padded);
+    a.num_levels = (int32_t)(num_levels > 0x7fffffff ? 0x7fffffff : num_levels);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    switch (dtype) {
+        case AHQ_F32: hipLaunchKernelGGL((grid_probe_kernel<float>), dim3(1), dim3(kProbeThreads), 0, s, a); break;
+        case AHQ_F16: hipLaunchKernelGGL((grid_probe_kernel<f16_t>), dim3(1), dim3(kProbeThreads), 0, s, a); break;
+        default: hipLaunchKernelGGL((grid_probe_kernel<bf16_t>), dim3(1), dim3(kProbeThreads), 0, s, a); break;
+    }
+    return check_launch("grid_probe");
+}
 
 extern "C" int ahq_range_to_scale_offset(int32_t dtype, const void* range_min, const void* range_max,
                                          int64_t num_encodings, int64_t qmin, int64_t qmax, double minimum_scale,

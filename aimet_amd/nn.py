@@ -33,12 +33,39 @@ __all__ = ["QuantizedLinear", "compute_encodings", "quantized_linears", "fold_pa
            "remove_param_quantizers"]
 
 
-def _may_be_prequantized(param: torch.Tensor, qtzr: AffineQuantizerBase):
+def _grid_probe(param: torch.Tensor, qtzr: AffineQuantizerBase, num_levels: int):
+    """The same test in one launch (ahq_grid_probe) for a contiguous GPU parameter; None where the library does not
+    cover the case (blocks along several dimensions, grids above 13 bits) and the torch form has to run."""
+    from aimet_amd import _lib
+    from aimet_amd.quantization.affine.backends.hip import _prepare
+
+    if not (param.is_cuda and param.dtype in _lib.DTYPE_CODE and param.is_contiguous() and param.numel() > 0):
+        return None
+    shape = tuple(qtzr.shape)
+    block_elems = param.numel() // max(1, math.prod(shape))
+    if block_elems <= num_levels:
+        return True
+    if num_levels > 4096:
+        return None
+    xd, layout = _prepare(param, shape, qtzr.block_size)
+    out = torch.empty((), dtype=torch.bool, device=param.device)
+    status = _lib.load().ahq_grid_probe(_lib.DTYPE_CODE[param.dtype], layout, xd.data_ptr(), num_levels, out.data_ptr(),
+                                        _lib.current_stream(param.device))
+    if status == _lib.AHQ_ERR_UNSUPPORTED:
+        return None
+    _lib.check(status, "ahq_grid_probe")
+    return out
+
+
+def _may_be_prequantized(param: torch.Tensor, qtzr: AffineQuantizerBase, on_device: bool = True):
     """The early exit of _decompose_prequantized_tensor (aimet_torch/utils.py:2098-2118): the first 64 blocks, first
     2 * num_levels elements each; more distinct magnitudes than grid levels means the tensor is not on a grid.
     Returns True, or a 0-dim bool tensor on the parameter's device (not yet read back)."""
     num_levels = max(abs(qtzr.qmax), abs(qtzr.qmin)) + 1
     shape = tuple(qtzr.shape)
+    verdict = _grid_probe(param, qtzr, num_levels) if on_device else None
+    if verdict is not None:
+        return verdict
     block = concretize_block_size(tuple(param.shape), shape, qtzr.block_size or tuple(-1 for _ in shape))
     block = (*param.shape[: param.dim() - len(block)], *block)
     split = []

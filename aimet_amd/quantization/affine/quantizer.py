@@ -341,7 +341,12 @@ class AffineQuantizerBase(QuantizerBase, _GridMixin):
         try:
             lo, hi = self.encoding_analyzer.compute_encodings(self._num_steps_for_calibration(), self.symmetric)
             if self.block_size is not None:
+                # the views are new tensor objects: hand on the range flags the kernel has already evaluated
+                flags = getattr(lo, "_ahq_range_flags", None)
+                same = flags is not None and getattr(hi, "_ahq_range_flags", None) is flags
                 lo, hi = lo.view(shape), hi.view(shape)
+                if same:
+                    lo._ahq_range_flags = hi._ahq_range_flags = flags  # pylint: disable=protected-access
             _flag_extreme_min_max(lo, hi)
         except StatisticsNotFoundError:
             return

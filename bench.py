@@ -526,14 +526,21 @@ def run_model_workload(steps, warmup, dev, with_cpu_baseline=True, batches=8, se
         calibrate()
         return forward()
 
+    import gc
+
     for _ in range(warmup):
         step()
     torch.cuda.synchronize()
+    # the step is bound by the host interpreter (about 4000 launches): keep the cyclic garbage collector's pauses out
+    # of the few timed steps
+    gc.collect()
+    gc.disable()
     t0 = time.perf_counter()
     for _ in range(steps):
         step()
     torch.cuda.synchronize()
     wall = (time.perf_counter() - t0) / steps
+    gc.enable()
 
     def timed(fn, reps):
         fn()

@@ -161,6 +161,16 @@ int ahq_range_to_scale_offset(int32_t dtype, const void* range_min, const void* 
                               int64_t qmin, int64_t qmax, double minimum_scale, float* scale, float* offset,
                               void* stream);
 
+/* Replaces the early exit of _decompose_prequantized_tensor (AT/utils.py:2098-2118), the test every weight goes
+ * through when a calibration starts: of the first 64 blocks of the layout, the first 2 * num_levels elements each are
+ * taken as float magnitudes; *verdict = 0 if one of those samples holds more than num_levels distinct values (the
+ * tensor is not an already-quantized one), else 1.  verdict: one byte of device memory (a torch.bool element).
+ * The caller handles blocks of at most num_levels elements itself (the reference skips the test for them).
+ * AHQ_ERR_UNSUPPORTED: blocks along several dimensions, or num_levels above 4096.
+ */
+int ahq_grid_probe(int32_t dtype, const ahq_layout* layout, const void* x, int64_t num_levels, uint8_t* verdict,
+                   void* stream);
+
 /* ---------------------------------------------------------------- histogram statistics ----------------------------
  * Replaces: _HistogramObserver.collect_stats + merge_stats (AT/quantization/encoding_analyzer.py:189-332), i.e. what
  * PercentileEncodingAnalyzer / SqnrEncodingAnalyzer / TfEnhancedEncodingAnalyzer.update_stats do per batch.

@@ -229,3 +229,39 @@ def test_graph_replayed_calibration_equals_eager_calibration(device):
         for a, b in zip(eager_stats[name], graph_stats[name]):
             assert torch.equal(_bits(a), _bits(b)), name
     assert torch.equal(_bits(eager_out), _bits(graph_out))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=lambda d: str(d).split(".")[-1])
+@pytest.mark.parametrize("case", [
+    # weight shape, encoding shape, block size, bitwidth
+    ((96, 512), (96, 8), (1, 64), 4),
+    ((96, 512), (96, 1), None, 4),
+    ((40, 2048), (40, 1), None, 8),          # 258 sampled elements per block: several rounds of sorting
+    ((70, 1024), (), None, 8),
+    ((6, 5, 16, 16), (1, 5, 1, 1), None, 4),  # a block's elements are spread over the leading dimension
+    ((96, 512), (96, 8), (1, 64), 12),       # 64-element blocks are no larger than the 2049-level grid: no test
+], ids=lambda c: "x".join(map(str, c[0])) + f"_b{c[3]}")
+def test_grid_probe_matches_the_sorted_sample_test(device, case, dtype):
+    """ahq_grid_probe against the step-by-step form of the reference's early exit (utils.py:2098-2118) run on the
+    CPU: random weights, weights on the grid, a violation inside and one outside the sampled region, NaNs."""
+    from aimet_amd.nn import _may_be_prequantized
+    from aimet_amd.quantization.affine import QuantizeDequantize
+
+    shape, enc_shape, block, bw = case
+    q = QuantizeDequantize(enc_shape, bw, True, block_size=block)
+    levels = 2 ** (bw - 1)
+    g = torch.Generator().manual_seed(17)
+    rand = torch.randn(shape, generator=g)
+    grid = torch.randint(-levels, levels, shape, generator=g).float() * 0.0625
+    late = grid.clone()
+    late.view(-1)[-300:] = torch.randn(300, generator=g)  # far from the first blocks' samples
+    early = grid.clone()
+    early.view(-1)[: 3 * levels] = torch.randn(3 * levels, generator=g)
+    nans = grid.clone()
+    nans.view(-1)[: 2 * levels : 2] = float("nan")
+    for name, w in (("random", rand), ("grid", grid), ("violation outside the sample", late),
+                    ("violation in the first block", early), ("NaN in the sample", nans)):
+        w = w.to(dtype)
+        want = _may_be_prequantized(w, q, on_device=False)
+        got = _may_be_prequantized(w.to(device), q)
+        assert bool(got) == bool(want), (name, bool(got), bool(want))
