@@ -268,6 +268,36 @@ __global__ __launch_bounds__(kBlock) void dlq_pdf_bin_generic_kernel(const PdfBi
     }
 }
 
+// Several slots, each one contiguous run of the tensor (per-channel statistics of a weight): a workgroup bins its
+// slot's run into an LDS histogram and stores it as the slot's counts -- no global atomics, no zeroing pass.
+template <typename IO, int VEC>
+__global__ __launch_bounds__(kBlock) void dlq_pdf_bin_runs_kernel(const PdfBinArgs a) {
+    __shared__ uint32_t hist[kPdf];
+    const int64_t e = blockIdx.x;
+    for (int i = threadIdx.x; i < kPdf; i += kBlock) hist[i] = 0;
+    __syncthreads();
+    const float* p = a.params + 4 * e;
+    if (p[2] != 0.f) {
+        const float inv = p[0], off = p[1];
+        const IO* __restrict__ x = static_cast<const IO*>(a.x) + e * a.K;
+        const int64_t nv = a.K / VEC;
+        for (int64_t v = threadIdx.x; v < nv; v += kBlock) {
+            const Pack<IO, VEC> pk = load_pack<IO, VEC>(x + v * VEC);
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) {
+                int idx;
+                if (pdf_index(load_f32(pk.v[k]), inv, off, idx)) atomicAdd(&hist[idx], 1u);
+            }
+        }
+        for (int64_t i = nv * VEC + threadIdx.x; i < a.K; i += kBlock) {
+            int idx;
+            if (pdf_index(load_f32(x[i]), inv, off, idx)) atomicAdd(&hist[idx], 1u);
+        }
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < kPdf; i += kBlock) a.counts[(size_t)e * kPdf + i] = hist[i];
+}
+
 __global__ void dlq_zero_u32_kernel(uint32_t* p, int64_t n) {
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) p[i] = 0;
 }
@@ -939,6 +969,25 @@ extern "C" int ahq_dlq_pdf_update(int32_t dtype, const ahq_layout* layout, const
             fa.counts = folded;
             fa.nparts = kPdfFoldGroups;
         }
+    } else if (pp.plan.cl.kind == kIJK && pp.plan.cl.I == 1 && pp.plan.cl.J > 1 && pp.plan.cl.K >= kBlock &&
+               pp.plan.cl.J <= 0x7fffffff) {
+        // one run per slot
+        ba.counts = counts;
+        const bool vec = aligned16(x) && pp.plan.cl.K % io_vec(dtype) == 0;
+        const dim3 g((unsigned)pp.plan.cl.J), b(kBlock);
+#define AHQ_LAUNCH_RUNS(IO)                                                                                         \
+    do {                                                                                                            \
+        if (vec) hipLaunchKernelGGL((dlq_pdf_bin_runs_kernel<IO, IoTraits<IO>::kVec>), g, b, 0, s, ba);             \
+        else hipLaunchKernelGGL((dlq_pdf_bin_runs_kernel<IO, 1>), g, b, 0, s, ba);                                  \
+    } while (0)
+        switch (dtype) {
+            case AHQ_F32: AHQ_LAUNCH_RUNS(float); break;
+            case AHQ_F16: AHQ_LAUNCH_RUNS(f16_t); break;
+            default: AHQ_LAUNCH_RUNS(bf16_t); break;
+        }
+#undef AHQ_LAUNCH_RUNS
+        fa.counts = counts;
+        fa.nparts = 1;
     } else {
         ba.counts = counts;
         const int64_t n = (int64_t)S * kPdf;

@@ -156,7 +156,8 @@ def _same_pdf(a, b):
     assert np.array_equal(pa, pb)
 
 
-PDF_CASES = [((6000,), ()), ((70001,), ()), ((1 << 20,), ()), ((8, 4096), (8, 1)), ((6, 2, 512), (3, 2, 1)), ((4, 2, 3), (2, 3))]
+PDF_CASES = [((6000,), ()), ((70001,), ()), ((1 << 20,), ()), ((8, 4096), (8, 1)), ((6, 2, 512), (3, 2, 1)), ((4, 2, 3), (2, 3)),
+             ((5, 1001), (5, 1)), ((3, 300), (3, 1))]  # one run per slot, ragged and vector-aligned
 
 
 @pytest.mark.parametrize("shape,enc_shape", PDF_CASES)
@@ -214,6 +215,22 @@ def test_empty_tensors_do_not_broadcast(device):
             for q in (OracleQuantizer(shape, 8, scheme), HipQuantizer(shape, 8, scheme, device)):
                 with pytest.raises(RuntimeError, match="broadcastable"):
                     q.updateStats(t)
+
+
+def test_pdf_per_channel_rows_with_an_all_zero_row(device):
+    """One run per slot (a workgroup per row): a row of zeros stays uninitialised while its neighbours collect."""
+    a = OracleQuantizer((3, 1), 8, QUANTIZATION_TF_ENHANCED)
+    b = HipQuantizer((3, 1), 8, QUANTIZATION_TF_ENHANCED, device)
+    g = torch.Generator().manual_seed(4)
+    for k in range(3):
+        x = torch.randn(3, 2048, generator=g) * (1 + k)
+        if k < 2:
+            x[1] = 0.0
+        for q in (a, b):
+            q.updateStats(x)
+        _same_pdf(a, b)
+    ea, eb = a.computeEncodings(False), b.computeEncodings(False)
+    assert np.array_equal(np.array(ea), np.array(eb))
 
 
 def test_pdf_update_of_an_empty_tensor_through_the_c_abi(device):
