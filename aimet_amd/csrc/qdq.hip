@@ -178,7 +178,10 @@ struct MathAutogradQuantize {
     }
     template <bool FAST>
     __device__ static float fwd(float x, const EncP& e, const GridC& g, bool& inr) {
-        const float r = rnd<CD>(__builtin_rintf(rnd<CD>(divide<FAST, CD>(x, e.p0, e.rs))) - e.p1);
+        float t = divide<FAST, CD>(x, e.p0, e.rs);
+        // the division-free quotient of a zero comes out as +0; with a zero offset the code of -0 is -0 in the reference
+        if (FAST && t == 0.f) t = bits_to_f32((f32_to_bits(x) ^ f32_to_bits(e.p0)) & 0x80000000u);
+        const float r = rnd<CD>(__builtin_rintf(rnd<CD>(t)) - e.p1);
         inr = (r >= g.qmin) & (r <= g.qmax);
         return r < g.qmin ? g.qmin : (r > g.qmax ? g.qmax : r);
     }

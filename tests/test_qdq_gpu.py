@@ -408,3 +408,17 @@ def test_small_integer_grid_shortcut_limits(device, monkeypatch, case):
     assert_close_rel(sd.grad[finite_rows], gs_ref[finite_rows], tol, "scale gradient", abs_floor=1e-30)
     assert_close_rel(od.grad[finite_rows], go_ref[finite_rows], tol, "offset gradient", abs_floor=1e-30)
     assert bool((sd.grad[~finite_rows].cpu().isnan() == gs_ref[~finite_rows].isnan()).all())
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=lambda d: str(d).split(".")[-1])
+def test_quantize_keeps_the_sign_of_a_zero_code(device, dtype):
+    """With a zero offset, inputs in [-scale / 2, -0] have the code -0.0 in the reference (round(-0.2) - 0); the
+    division-free quotient must not lose the sign of an input that is exactly -0."""
+    from aimet_amd.quantization import affine
+
+    x = torch.tensor([-0.0, 0.0, -0.01, 0.01, -1e-30, 1e-30, -0.6, 0.6] * 40, dtype=torch.float32).to(dtype)
+    scale, offset = torch.tensor(1.0), torch.tensor(0.0)
+    codes_ref, _ = O.quantize_forward(x, scale, offset, -2, 1)
+    codes = affine.quantize(x.to(device), scale.to(device), offset.to(device), -2, 1)
+    assert_same_bits(codes.as_subclass(torch.Tensor), codes_ref, "codes")
+    assert torch.signbit(codes_ref[0]) and not torch.signbit(codes_ref[1])
