@@ -31,6 +31,7 @@ struct GridC {
 };
 constexpr int kCastOverflowNaN = 1;    // a value that rounds past the largest one becomes NaN (else infinity)
 constexpr int kCastUnsignedZero = 2;   // the format has no negative zero
+constexpr int kCastLogForm = 4;        // 16-bit tensors: the reference's logarithm formula, rounded step by step
 
 struct EncP {
     float p0, p1, p2, p3;
@@ -324,6 +325,24 @@ struct MathFloatCast {
         if (FAST && t == 0.f) t = bits_to_f32((f32_to_bits(x) ^ f32_to_bits(e.p0)) & 0x80000000u);
         const float mx = rnd<CD>(g.qmax);
         t = (t < -mx) ? -mx : (mx < t) ? mx : t;
+        if constexpr (CD != AHQ_F32) {
+            if (g.flags & kCastLogForm) {
+                // fake_cast_to_ieee_float (aimet_torch/fp_quantization.py:177-201) on a 16-bit tensor, every torch
+                // operation with its own rounding to that dtype:
+                //   log_scales = clamp(floor(log2|x| + bias), 1);  scales = 2 ** (log_scales - mantissa_bits - bias)
+                //   out = round(x / scales) * scales
+                // Near the top of a binade the rounded logarithm reaches the next integer, so such values land on the
+                // next binade's coarser grid, and a clamp bound that rounds upward in the tensor's dtype is returned
+                // as it is: this is what the reference computes, and it is reproduced rather than corrected.
+                const float bias = rnd<CD>(1.f - g.qmin);
+                float ls = __builtin_floorf(rnd<CD>(rnd<CD>(__builtin_log2f(__builtin_fabsf(t))) + bias));
+                ls = (ls != ls) ? ls : fmaxf(ls, 1.f);
+                const float ex2 = rnd<CD>(rnd<CD>(ls - g.zps) - bias);
+                const float sc = rnd<CD>(__builtin_exp2f(ex2));
+                const float q = rnd<CD>(t / sc);
+                return rnd<CD>(__builtin_rintf(q) * sc) * e.p0;  // last rounding by the caller
+            }
+        }
         int ex = __builtin_amdgcn_frexp_expf(t) - 1;
         ex = ex < (int)g.qmin ? (int)g.qmin : ex;
         const int sh = ex - (int)g.zps;
@@ -1096,7 +1115,7 @@ extern "C" int ahq_dlq_fp8_qdq(int32_t dtype, const ahq_layout* layout, const vo
 
 extern "C" int ahq_float_qdq(int32_t dtype, const ahq_layout* layout, const void* x, void* y, const float* scale,
                              int32_t mantissa_bits, int32_t exponent_min, float max_value, int32_t overflow_to_nan,
-                             int32_t unsigned_zero, void* stream) {
+                             int32_t unsigned_zero, int32_t logarithm_form, void* stream) {
     if (dtype < AHQ_F32 || dtype > AHQ_BF16) return set_error("bad dtype"), AHQ_ERR_INVALID;
     if (!layout) return set_error("layout is null"), AHQ_ERR_INVALID;
     if (!scale) return set_error("scale is null"), AHQ_ERR_INVALID;
@@ -1116,7 +1135,8 @@ extern "C" int ahq_float_qdq(int32_t dtype, const ahq_layout* layout, const void
     a.gc.qmin = (float)exponent_min;
     a.gc.qmax = max_value;
     a.gc.zps = (float)mantissa_bits;
-    a.gc.flags = (overflow_to_nan ? kCastOverflowNaN : 0) | (unsigned_zero ? kCastUnsignedZero : 0);
+    a.gc.flags = (overflow_to_nan ? kCastOverflowNaN : 0) | (unsigned_zero ? kCastUnsignedZero : 0) |
+                 (logarithm_form ? kCastLogForm : 0);
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (dtype == AHQ_F32) launch_fwd<float, MathFloatCast<AHQ_F32>>(p, a, st, aligned16(x) && aligned16(y));
     else if (dtype == AHQ_F16) launch_fwd<f16_t, MathFloatCast<AHQ_F16>>(p, a, st, aligned16(x) && aligned16(y));

@@ -37,8 +37,12 @@ def _launch(x: torch.Tensor, finfo: _finfo, scale: torch.Tensor, block_size) -> 
     if x.numel():
         mbits, emin, mx, overflow_nan, uz = finfo.kernel_format()
         s = _hip._enc_f32(scale)  # pylint: disable=protected-access
+        # a format without a storage type goes through the reference's logarithm formula, whose steps round to the
+        # tensor's dtype: on 16-bit tensors that differs from an exact cast next to binade boundaries
+        log_form = finfo.to_torch_dtype() is None and x.dtype != torch.float32
         _lib.check(lib.ahq_float_qdq(_lib.DTYPE_CODE[x.dtype], layout, x.data_ptr(), y.data_ptr(), s.data_ptr(), mbits,
-                                     emin, mx, int(overflow_nan), int(uz), _lib.current_stream(x.device)),
+                                     emin, mx, int(overflow_nan), int(uz), int(log_form),
+                                     _lib.current_stream(x.device)),
                    "ahq_float_qdq")
     return y
 

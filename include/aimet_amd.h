@@ -288,10 +288,15 @@ int ahq_dlq_fp8_qdq(int32_t dtype, const ahq_layout* layout, const void* x, void
  * unsigned_zero: the format has no negative zero.  scale: one float per encoding of the layout, used at float
  * precision (quotient and product are formed in float and rounded once to `dtype`), which is how torch treats a
  * one-element float32 operand next to a 16-bit tensor.
+ * logarithm_form (16-bit `dtype` only, ignored for float32): cast the way fake_cast_to_ieee_float does for a format
+ * without a torch storage type, scales = 2 ** (clamp(floor(log2|x| + bias), 1) - mantissa_bits - bias), out =
+ * round(x / scales) * scales with bias = 1 - exponent_min and every operation rounded to `dtype`: values within one
+ * unit of `dtype` below a power of two land on the next binade's grid and a clamp bound that `dtype` rounds upward is
+ * returned as it is, as in the reference; overflow_to_nan and unsigned_zero do not apply.
  */
 int ahq_float_qdq(int32_t dtype, const ahq_layout* layout, const void* x, void* y, const float* scale,
                   int32_t mantissa_bits, int32_t exponent_min, float max_value, int32_t overflow_to_nan,
-                  int32_t unsigned_zero, void* stream);
+                  int32_t unsigned_zero, int32_t logarithm_form, void* stream);
 
 /* Replaces PercentileEncodingAnalyzer::computeEncoding (DLQ/src/PercentileEncodingAnalyzer.cpp:52-169) on the same PDF
  * statistics: the range that keeps `percentile` percent of the probability mass on each side, widened to contain

@@ -34,6 +34,28 @@ def _data(shape, dtype, seed, span):
     return x.to(dtype)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=lambda d: str(d)[6:])
+@pytest.mark.parametrize("fmt", [(3, 9, False, False), (5, 9, False, False), (4, 6, False, False), (5, 3, False, False),
+                                 (2, 6, False, False), (6, 4, False, False), (2, 1, False, False)], ids=str)
+@pytest.mark.parametrize("scale", [1.0, 0.7451069355010986, 29.658720016479492])
+def test_every_16bit_value_through_a_format_without_a_storage_type(device, fmt, dtype, scale):
+    """Formats that torch has no dtype for go through the reference's logarithm formula, whose steps round to the
+    tensor's dtype: next to the top of a binade and at a clamp bound that the dtype rounds upward that is not the
+    exact cast.  Every bit pattern of the tensor dtype, against the CPU restatement."""
+    from aimet_amd.quantization.float._finfo import _finfo as FI
+
+    x = torch.arange(-32768, 32768, dtype=torch.int32).to(torch.int16).view(dtype)
+    sc = torch.tensor(scale)
+    mx = O.float_max(*fmt)
+    if mx > torch.finfo(dtype).max:
+        with pytest.raises(RuntimeError, match="without overflow"):
+            _fq().float_quantize_dequantize(x.to(device), FI(*fmt), sc.to(device))
+        return
+    want = O.float_qdq(x, sc, *fmt)
+    got = _fq().float_quantize_dequantize(x.to(device), FI(*fmt), sc.to(device))
+    assert_same_bits(got, want, str(fmt))
+
+
 # ------------------------------------------------------------------------------------- kernel against the oracle --
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=lambda d: str(d)[6:])
 @pytest.mark.parametrize("name", list(FORMATS))
