@@ -56,6 +56,7 @@ struct PrepArgs {
     float* upd_edges;  // [S][B+1]
     float* ranges;     // [S][8]
     int32_t* scratch;  // [S][2][B] destination indices
+    int32_t* rebin;    // optional [S]: set to 1 when the running range changed (the batch has to be binned again)
 };
 
 // _create_bin_edges (encoding_analyzer.py:221-229).  `lo`/`hi` already hold the min==max adjustment.
@@ -103,15 +104,19 @@ __global__ void hist_prepare_kernel(const PrepArgs a) {
     const float lo1 = eq ? round_io<IO>(mn - 0.5f) : mn;
     const float hi1 = eq ? round_io<IO>(mx + 0.5f) : mx;
     const float step1 = (hi1 - lo1) / Bf;
-    float* ne = a.new_edges + (size_t)s * (B + 1);
-    for (int i = threadIdx.x; i <= B; i += blockDim.x) ne[i] = edge_at(lo1, step1, i);
+    if (a.new_edges) {
+        float* ne = a.new_edges + (size_t)s * (B + 1);
+        for (int i = threadIdx.x; i <= B; i += blockDim.x) ne[i] = edge_at(lo1, step1, i);
+    }
     const float e1_first = edge_at(lo1, step1, 0), e1_last = edge_at(lo1, step1, B);
     float* rg = a.ranges + (size_t)s * kRng;
     float* mmx = a.minmax + (size_t)s * 2;
     float* lim = a.limits + (size_t)s * 2;
     if (threadIdx.x == 0) {
-        a.new_minmax[2 * s] = mn;
-        a.new_minmax[2 * s + 1] = mx;
+        if (a.new_minmax) {
+            a.new_minmax[2 * s] = mn;
+            a.new_minmax[2 * s + 1] = mx;
+        }
         rg[0] = e1_first;
         rg[1] = e1_last;
         rg[2] = round_io<IO>(e1_first);
@@ -142,6 +147,7 @@ __global__ void hist_prepare_kernel(const PrepArgs a) {
     const float umin = fminf(fmaxf(mn, lim[0]), c_first);
     const float umax = fminf(fmaxf(mx, c_last), lim[1]);
     const bool same = (umin == mmx[0]) && (umax == mmx[1]);
+    if (a.rebin && threadIdx.x == 0) a.rebin[s] = same ? 0 : 1;
     if (same) {
         for (int i = threadIdx.x; i < B; i += blockDim.x) carried[i] = ch[i];
     } else {
@@ -210,6 +216,11 @@ struct BinArgs : Geom {
     int32_t copies;        // interleaved LDS copies of each histogram (power of two, 1..8)
     int32_t copy_shift;    // log2(copies)
     int64_t ntiles;
+    // speculative pass (see hist_bin_kernel): the running range as the state holds it, and where the batch's extrema go
+    const float* state_minmax;
+    float* part_min;       // [nblocks]
+    float* part_max;
+    const int32_t* rebin;  // second pass: leave at once unless *rebin != 0
 };
 
 struct RangeC {
@@ -262,17 +273,47 @@ __device__ __forceinline__ int bin_estimate(float v, const RangeC& r, float Bf, 
 // The kernel is bound by instruction issue, not by LDS or HBM, so the per-element path is kept free of branches:
 // elements that need the exact division or lie outside the range are only flagged, and one wave-uniform branch per
 // tile revisits them.
-template <typename IO, int VEC, int NH>
+//
+// SPEC (one histogram): the speculative pass of a batch after the first, for a caller that wants the running
+// statistics only.  Most batches of a calibration stay inside the running range, and then the reference bins them on
+// exactly that range; so the batch is binned on the running range as the state holds it.  The running range can only
+// move because of finite elements outside it, and those already take the kernel's rare element-by-element path:
+// their extrema are collected there at no cost to the others (per-workgroup partials that the prepare kernel folds;
+// +-inf when nothing lies outside, which leaves the range where it is).  If the prepare kernel then finds the range
+// unchanged, these counts are the batch's contribution and the second read of the batch is skipped (the ordinary pass
+// is launched with `rebin` and leaves at once); if the range grew, the ordinary pass bins again on the new range and
+// overwrites the partial histograms.  A running range of zero width is binned on a widened one, so then every
+// element is looked at.
+template <typename IO, int VEC, int NH, bool SPEC = false>
 __global__ __launch_bounds__(kBlock, 6) void hist_bin_kernel(const BinArgs a) {
     extern __shared__ uint32_t lds[];  // [NH][B][copies]: lane l adds to copy l % copies, neighbouring copies sit in neighbouring banks
     __shared__ uint32_t cnt_smem[kBlock / kWave][NH][2];
+    __shared__ float ext_smem[kBlock / kWave][2];
+    if (!SPEC && a.rebin && *a.rebin == 0) return;
     const int B = a.num_bins;
     const float Bf = (float)B;
     const int copies = a.copies;
     for (int i = threadIdx.x; i < copies * NH * B; i += kBlock) lds[i] = 0;
     RangeC r[NH];
+    float run_lo = 0.f, run_hi = 0.f;  // SPEC: the running range itself
+    if (SPEC) {
+        run_lo = a.state_minmax[0];
+        run_hi = a.state_minmax[1];
+        const float rg[4] = {run_lo, run_hi, round_io<IO>(run_lo), round_io<IO>(run_hi)};
+        r[0] = load_range(rg, 0);
+    } else {
 #pragma unroll
-    for (int h = 0; h < NH; ++h) r[h] = load_range(a.ranges, h);
+        for (int h = 0; h < NH; ++h) r[h] = load_range(a.ranges, h);
+    }
+    float ext_min = __builtin_inff(), ext_max = -__builtin_inff();  // SPEC: finite extrema of this lane's elements
+    const bool degenerate = SPEC && run_lo == run_hi;
+    auto track = [&](float v) {  // finite elements outside the running range
+        if (SPEC) {
+            const bool fin = __builtin_fabsf(v) < __builtin_inff();
+            ext_min = fminf(ext_min, (fin & (v < run_lo)) ? v : __builtin_inff());
+            ext_max = fmaxf(ext_max, (fin & (v > run_hi)) ? v : -__builtin_inff());
+        }
+    };
     __syncthreads();
     const int wave = threadIdx.x / kWave;
     const int cshift = a.copy_shift;  // copies == 1 << cshift
@@ -288,6 +329,7 @@ __global__ __launch_bounds__(kBlock, 6) void hist_bin_kernel(const BinArgs a) {
 
     // every element, exactly (ragged tile, tail elements and the revisit of flagged elements)
     auto bin_slow = [&](float v, bool only_flagged) {
+        track(v);
 #pragma unroll
         for (int h = 0; h < NH; ++h) {
             const bool inr = (v >= r[h].lo) & (v <= r[h].hi);
@@ -307,6 +349,10 @@ __global__ __launch_bounds__(kBlock, 6) void hist_bin_kernel(const BinArgs a) {
         Pack<IO, VEC> in[kUnroll];
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) in[u] = load_pack<IO, VEC>(x + (tile * kTileVec + u * kBlock + threadIdx.x) * VEC);
+        if (degenerate) {
+            for (int u = 0; u < kUnroll; ++u)
+                for (int k = 0; k < VEC; ++k) track(load_f32(in[u].v[k]));
+        }
         uint32_t binned = 0;  // this lane's elements that took the fast path
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
@@ -369,7 +415,27 @@ __global__ __launch_bounds__(kBlock, 6) void hist_bin_kernel(const BinArgs a) {
             cnt_smem[wave][h][1] = ab;
         }
     }
+    if (SPEC) {
+#pragma unroll
+        for (int m = kWave / 2; m >= 1; m >>= 1) {
+            ext_min = fminf(ext_min, __shfl_xor(ext_min, m, kWave));
+            ext_max = fmaxf(ext_max, __shfl_xor(ext_max, m, kWave));
+        }
+        if ((threadIdx.x & (kWave - 1)) == 0) {
+            ext_smem[wave][0] = ext_min;
+            ext_smem[wave][1] = ext_max;
+        }
+    }
     __syncthreads();
+    if (SPEC && threadIdx.x == 0) {
+        float mn = ext_smem[0][0], mx = ext_smem[0][1];
+        for (int wv = 1; wv < kBlock / kWave; ++wv) {
+            mn = fminf(mn, ext_smem[wv][0]);
+            mx = fmaxf(mx, ext_smem[wv][1]);
+        }
+        a.part_min[blockIdx.x] = mn;
+        a.part_max[blockIdx.x] = mx;
+    }
     uint32_t* out = a.partials + (size_t)blockIdx.x * NH * (B + 2);
     for (int i = threadIdx.x; i < NH * B; i += kBlock) {
         const int h = i / B, b = i - h * B;
@@ -601,7 +667,7 @@ struct HistPlan {
     int copies;
     int nblocks;
     int64_t ntiles;
-    size_t off_mm_ws, off_bmin, off_bmax, off_ranges, off_carried, off_upd_edges, off_scratch, off_counts, off_folded, total;
+    size_t off_mm_ws, off_bmin, off_bmax, off_ranges, off_carried, off_upd_edges, off_scratch, off_rebin, off_counts, off_folded, total;
 };
 
 size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
@@ -654,6 +720,7 @@ bool make_hist_plan(int dtype, const ahq_layout& layout, const void* x, int num_
     hp->off_carried = o;   o = align_up(o + (size_t)S * B * 4);
     hp->off_upd_edges = o; o = align_up(o + (size_t)S * (B + 1) * 4);
     hp->off_scratch = o;   o = align_up(o + (size_t)S * 2 * B * 4);
+    hp->off_rebin = o;     o = align_up(o + (size_t)S * 4);
     hp->off_counts = o;
     const size_t nparts = hp->fast ? (size_t)hp->nblocks : 1;
     o = align_up(o + (size_t)S * nparts * 2 * (B + 2) * 4);
@@ -680,8 +747,10 @@ extern "C" int ahq_hist_update(int32_t dtype, const ahq_layout* layout, const vo
     if (dtype < AHQ_F32 || dtype > AHQ_BF16) return set_error("bad dtype"), AHQ_ERR_INVALID;
     if (!layout || !st || !x) return set_error("null argument"), AHQ_ERR_INVALID;
     if (st->num_bins <= 0) return set_error("num_bins must be positive"), AHQ_ERR_INVALID;
-    if (!st->hist || !st->edges || !st->minmax || !st->limits || !st->new_edges || !st->new_minmax)
+    if (!st->hist || !st->edges || !st->minmax || !st->limits)
         return set_error("histogram state has a null buffer"), AHQ_ERR_INVALID;
+    if ((st->new_edges == nullptr) != (st->new_minmax == nullptr) || (st->new_hist && !st->new_edges))
+        return set_error("new_edges and new_minmax go together, and new_hist needs them"), AHQ_ERR_INVALID;
     if (!(st->growth_limit >= 1.0f)) return set_error("growth limit must be at least 1"), AHQ_ERR_INVALID;
     HistPlan hp;
     if (!make_hist_plan(dtype, *layout, x, st->num_bins, &hp)) return AHQ_ERR_INVALID;
@@ -697,12 +766,51 @@ extern "C" int ahq_hist_update(int32_t dtype, const ahq_layout* layout, const vo
     const bool merged_only = !first_batch && !st->new_hist;
     const int NH = (first_batch || merged_only) ? 1 : 2;
 
+    // A batch after the first, one slot, only the running histogram wanted: bin on the running range while reading
+    // the batch for its extrema, and bin again only if the range turns out to have changed.
+    const bool speculative = merged_only && !st->new_edges && hp.fast && (size_t)hp.nblocks * 8 <= hp.off_bmin - hp.off_mm_ws;
+    BinArgs ba{};
+    fill_geom(hp.plan, &ba);
+    ba.x = x;
+    ba.num_bins = B;
+    ba.nhist = NH;
+    ba.copies = hp.copies;
+    ba.copy_shift = 0;
+    while ((1 << ba.copy_shift) < hp.copies) ++ba.copy_shift;
+    ba.ntiles = hp.ntiles;
+    uint32_t* counts = reinterpret_cast<uint32_t*>(w + hp.off_counts);
+    int32_t* rebin = reinterpret_cast<int32_t*>(w + hp.off_rebin);
+
     // 1. finite range of the batch, in the tensor's dtype
     const float *part_min = nullptr, *part_max = nullptr;
     int64_t nparts = 0;
-    int rc = ahq_minmax_finite_partials(dtype, layout, x, w + hp.off_bmin, w + hp.off_bmax, w + hp.off_mm_ws,
-                                        hp.off_bmin - hp.off_mm_ws, stream, &part_min, &part_max, &nparts);
-    if (rc != AHQ_OK) return rc;
+    if (speculative) {
+        ba.partials = counts;
+        ba.state_minmax = st->minmax;
+        ba.part_min = reinterpret_cast<float*>(w + hp.off_mm_ws);
+        ba.part_max = ba.part_min + hp.nblocks;
+        const size_t lds = (size_t)hp.copies * B * 4;
+        const dim3 g(hp.nblocks), b(kBlock);
+#define AHQ_LAUNCH_SPEC(IO)                                                                                         \
+    do {                                                                                                            \
+        if (hp.plan.vec == 1) hipLaunchKernelGGL((hist_bin_kernel<IO, 1, 1, true>), g, b, lds, s, ba);              \
+        else hipLaunchKernelGGL((hist_bin_kernel<IO, IoTraits<IO>::kVec, 1, true>), g, b, lds, s, ba);              \
+    } while (0)
+        switch (dtype) {
+            case AHQ_F32: AHQ_LAUNCH_SPEC(float); break;
+            case AHQ_F16: AHQ_LAUNCH_SPEC(f16_t); break;
+            default: AHQ_LAUNCH_SPEC(bf16_t); break;
+        }
+#undef AHQ_LAUNCH_SPEC
+        part_min = ba.part_min;
+        part_max = ba.part_max;
+        nparts = hp.nblocks;
+        ba.rebin = rebin;  // for the second pass
+    } else {
+        int rc = ahq_minmax_finite_partials(dtype, layout, x, w + hp.off_bmin, w + hp.off_bmax, w + hp.off_mm_ws,
+                                            hp.off_bmin - hp.off_mm_ws, stream, &part_min, &part_max, &nparts);
+        if (rc != AHQ_OK) return rc;
+    }
 
     // 2. edges, updated range, re-binned running counts
     PrepArgs pa{};
@@ -725,6 +833,7 @@ extern "C" int ahq_hist_update(int32_t dtype, const ahq_layout* layout, const vo
     pa.upd_edges = reinterpret_cast<float*>(w + hp.off_upd_edges);
     pa.ranges = reinterpret_cast<float*>(w + hp.off_ranges);
     pa.scratch = reinterpret_cast<int32_t*>(w + hp.off_scratch);
+    pa.rebin = speculative ? rebin : nullptr;
     const int pthreads = nparts > 0 ? 1024 : (B >= 512 ? 512 : (B >= 64 ? ((B + 63) / 64) * 64 : 64));
     switch (dtype) {
         case AHQ_F32: hipLaunchKernelGGL((hist_prepare_kernel<float>), dim3(S), dim3(pthreads), 0, s, pa); break;
@@ -732,18 +841,8 @@ extern "C" int ahq_hist_update(int32_t dtype, const ahq_layout* layout, const vo
         default: hipLaunchKernelGGL((hist_prepare_kernel<bf16_t>), dim3(S), dim3(pthreads), 0, s, pa); break;
     }
 
-    // 3. binning pass
-    BinArgs ba{};
-    fill_geom(hp.plan, &ba);
-    ba.x = x;
+    // 3. binning pass (after a speculative pass: only if the range changed)
     ba.ranges = merged_only ? pa.ranges + 4 : pa.ranges;  // per slot: the batch's own range, then the running one
-    ba.num_bins = B;
-    ba.nhist = NH;
-    ba.copies = hp.copies;
-    ba.copy_shift = 0;
-    while ((1 << ba.copy_shift) < hp.copies) ++ba.copy_shift;
-    ba.ntiles = hp.ntiles;
-    uint32_t* counts = reinterpret_cast<uint32_t*>(w + hp.off_counts);
     if (hp.fast) {
         ba.partials = counts;
         const size_t lds = (size_t)hp.copies * NH * B * 4;

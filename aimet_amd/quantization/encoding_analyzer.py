@@ -50,23 +50,25 @@ class _HistogramList(Sequence):
     slots, and materialising a Python object with four tensor views for each of them on every batch costs
     milliseconds to seconds of host time that nothing reads during a calibration pass."""
 
-    def __init__(self, hist, edges, minmax, dtype, count: Optional[int] = None, make_hist=None):
+    def __init__(self, hist, edges, minmax, dtype, count: Optional[int] = None, make=None):
         self._hist, self._edges, self._minmax, self._dtype = hist, edges, minmax, dtype
         self._typed_minmax = None
-        self._make_hist = make_hist  # forms the counts when they are first asked for (see _HistogramObserver.update)
+        # forms (counts, edges, min/max) when they are first asked for (see _HistogramObserver.update)
+        self._make = make
         self._count = int(count) if count is not None else hist.shape[0]
 
     def __len__(self) -> int:
         return self._count
 
     def _counts(self):
-        if self._hist is None and self._make_hist is not None:
-            self._hist, self._make_hist = self._make_hist(), None
+        if self._hist is None and self._make is not None:
+            (self._hist, self._edges, self._minmax), self._make = self._make(), None
         return self._hist
 
     def stacked(self):
         """(hist [S, B], bin edges [S, B + 1], min/max [S, 2] in float32, dtype the reference keeps min/max in)."""
-        return self._counts(), self._edges, self._minmax, self._dtype
+        hist = self._counts()
+        return hist, self._edges, self._minmax, self._dtype
 
     def _entry(self, i: int) -> _Histogram:
         if self._counts() is None:
@@ -191,8 +193,10 @@ class _HistogramObserver(_Observer[_Histogram]):
             "minmax": torch.zeros(S, 2, **f), "limits": torch.zeros(S, 2, **f),
         }
 
-    def _run(self, x: torch.Tensor, state: dict, first: bool, batch_hist: bool = True):
-        """One ahq_hist_update call.  Returns (new_hist, new_edges, new_minmax); new_hist is None if not asked for."""
+    def _run(self, x: torch.Tensor, state: dict, first: bool, batch_hist: bool = True, batch_stats: bool = True):
+        """One ahq_hist_update call.  Returns (new_hist, new_edges, new_minmax): the batch's own counts if
+        ``batch_hist``, its own edges and min / max if ``batch_stats`` (None otherwise)."""
+        batch_stats = batch_stats or batch_hist
         _lib.require_device(x, "input tensor")
         if x.dtype not in _lib.DTYPE_CODE:
             raise HipLibraryError(f"histogram statistics support float32, float16 and bfloat16; got {x.dtype}")
@@ -207,14 +211,15 @@ class _HistogramObserver(_Observer[_Histogram]):
         xd, layout = _prepare(x.detach(), self.shape, self.block_size)
         f = dict(dtype=torch.float32, device=x.device)
         new_hist = torch.empty(S, B, **f) if batch_hist else None
-        new_edges = torch.empty(S, B + 1, **f)
-        new_minmax = torch.empty(S, 2, **f)
+        new_edges = torch.empty(S, B + 1, **f) if batch_stats else None
+        new_minmax = torch.empty(S, 2, **f) if batch_stats else None
         st = _lib.HistState()
         st.num_slots, st.num_bins, st.growth_limit = S, B, self.growth_limit
         st.hist, st.edges = state["hist"].data_ptr(), state["edges"].data_ptr()
         st.minmax, st.limits = state["minmax"].data_ptr(), state["limits"].data_ptr()
         st.new_hist = new_hist.data_ptr() if batch_hist else None
-        st.new_edges, st.new_minmax = new_edges.data_ptr(), new_minmax.data_ptr()
+        st.new_edges = new_edges.data_ptr() if batch_stats else None
+        st.new_minmax = new_minmax.data_ptr() if batch_stats else None
         code = _lib.DTYPE_CODE[x.dtype]
         nbytes = lib.ahq_hist_update_workspace_bytes(code, layout, B)
         ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
@@ -240,18 +245,19 @@ class _HistogramObserver(_Observer[_Histogram]):
     def update(self, input_tensor: torch.Tensor) -> List[_Histogram]:
         """collect_stats + merge_stats with a single binning pass over the tensor.
 
-        After the first batch, the counts of the returned batch statistics (not their edges, minimum and maximum) are
-        formed when they are first read, from the tensor that was passed in: the running histogram never uses them
-        (reference: merge_stats, encoding_analyzer.py:260-331, bins the tensor itself onto the running range), a
-        calibration loop discards them, and leaving them out halves the histogram updates of the binning pass.  The
-        returned object keeps the tensor alive until then; a caller that modifies the tensor in place before reading
-        the counts gets the counts of the modified tensor."""
+        After the first batch, the returned batch statistics are formed when they are first read, from the tensor
+        that was passed in: the running histogram only needs to know whether the batch reaches beyond the running
+        range (reference: merge_stats, encoding_analyzer.py:260-331, bins the tensor itself onto the running range),
+        a calibration loop discards the batch statistics, and without them a batch inside the running range is read
+        once instead of twice, with one histogram update per element instead of two.  The returned object keeps the
+        tensor alive until then; a caller that modifies the tensor in place before reading the statistics gets those
+        of the modified tensor."""
         first = not self._has_stats
         if first or self._state["hist"].device != input_tensor.device:
             if not first:
                 raise RuntimeError("histogram statistics live on a different device than the input")
             self._state = self._alloc(input_tensor.device)
-        h, e, mm = self._run(input_tensor, self._state, first, batch_hist=first)
+        h, e, mm = self._run(input_tensor, self._state, first, batch_hist=first, batch_stats=first)
         # the reference keeps the first batch's min/max in the tensor dtype; after a merge they are float32
         self._stat_dtype = input_tensor.dtype if first else torch.promote_types(self._stat_dtype, torch.float32)
         self._has_stats = True
@@ -260,10 +266,10 @@ class _HistogramObserver(_Observer[_Histogram]):
             return self._as_list(h, e, mm, input_tensor.dtype)
         held = input_tensor.detach()
 
-        def counts():
-            return self._run(held, self._alloc(held.device), first=True)[0]
+        def collect():
+            return self._run(held, self._alloc(held.device), first=True)
 
-        return _HistogramList(None, e, mm, input_tensor.dtype, count=self.num_slots, make_hist=counts)
+        return _HistogramList(None, None, None, input_tensor.dtype, count=self.num_slots, make=collect)
 
     @torch.no_grad()
     def merge_stats(self, new_stats_list: List[_Histogram], input_tensor: torch.Tensor):  # pylint: disable=arguments-differ

@@ -179,9 +179,12 @@ int ahq_grid_probe(int32_t dtype, const ahq_layout* layout, const void* x, int64
  * running counts re-binned onto that range, and the batch binned onto it and added.  Bin index formula and
  * out-of-range handling are torch.histc's on CPU; counts are fp32 like the reference's.
  * All buffers are fp32 device arrays owned by the caller; hist/edges/minmax/limits persist between calls.
- * new_hist may be NULL: the batch's own histogram is then not formed (new_edges and new_minmax still are), which
- * leaves one histogram update per element instead of two for every batch after the first.  A caller that turns out to
- * need it gets the same values from a first_batch call on a scratch state (collect_stats alone).
+ * new_hist may be NULL: the batch's own histogram is then not formed, which leaves one histogram update per element
+ * instead of two for every batch after the first.  new_edges and new_minmax may be NULL as well (both, and then
+ * new_hist too): only the running statistics are kept up, and a batch after the first that stays inside the running
+ * range is read once instead of twice (it is binned on the running range while its out-of-range elements are looked
+ * for; only a batch that moves the range is binned again).  A caller that turns out to need a batch's own statistics
+ * gets the same values from a first_batch call on a scratch state (collect_stats alone).
  */
 typedef struct {
     int32_t num_slots;     /* number of histograms = number of encodings of the layout */
@@ -192,8 +195,8 @@ typedef struct {
     float*  minmax;        /* [num_slots][2]            running stats.min / stats.max */
     float*  limits;        /* [num_slots][2]            range limits fixed by the first batch */
     float*  new_hist;      /* [num_slots][num_bins]     out: this batch's own histogram (optional) */
-    float*  new_edges;     /* [num_slots][num_bins+1]   out */
-    float*  new_minmax;    /* [num_slots][2]            out: this batch's finite min / max */
+    float*  new_edges;     /* [num_slots][num_bins+1]   out (optional, with new_minmax) */
+    float*  new_minmax;    /* [num_slots][2]            out: this batch's finite min / max (optional) */
 } ahq_hist_state;
 
 size_t ahq_hist_update_workspace_bytes(int32_t dtype, const ahq_layout* layout, int32_t num_bins);

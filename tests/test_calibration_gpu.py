@@ -90,24 +90,30 @@ def test_histogram_several_slots(device, case):
                          ids=["single_slot", "rows", "blockwise"])
 def test_histogram_update_with_and_without_the_batch_histogram(device, case):
     """ahq_hist_update with new_hist: both histograms in one pass (what the oracle's update returns and keeps);
-    without: only the running one, bit-identical, and the batch's own edges / min / max are still written."""
+    without: only the running one, bit-identical, and the batch's own edges / min / max are still written; without
+    those either: the running statistics alone (a single slot is then binned speculatively on the running range)."""
     from aimet_amd.quantization.encoding_analyzer import _HistogramObserver
 
     shape, block, xshape = case
     both = _HistogramObserver(shape, num_bins=32, block_size=block)
     only = _HistogramObserver(shape, num_bins=32, block_size=block)
+    bare = _HistogramObserver(shape, num_bins=32, block_size=block)  # running statistics only
     ref = O.HistObserver(shape, 32, None, block)
     g = torch.Generator().manual_seed(5)
     for k in range(3):
         x = torch.randn(xshape, generator=g) * (1 + 0.7 * k) + 0.1 * k
         new_ref = ref.update(x)
         xd = x.to(device)
-        for obs in (both, only):
+        for obs in (both, only, bare):
             if obs._state is None:
                 obs._state = obs._alloc(xd.device)
         h2, e2, mm2 = both._run(xd, both._state, first=(k == 0), batch_hist=True)
         h1, e1, mm1 = only._run(xd, only._state, first=(k == 0), batch_hist=(k == 0))
         assert (h1 is None) == (k > 0)
+        h0, e0, mm0 = bare._run(xd, bare._state, first=(k == 0), batch_hist=(k == 0), batch_stats=(k == 0))
+        assert (e0 is None) == (k > 0) and (mm0 is None) == (k > 0)
+        for key in ("hist", "edges", "minmax", "limits"):
+            assert_same_bits(bare._state[key], both._state[key], f"running {key} after batch {k} (running statistics only)")
         for s_, r in enumerate(new_ref):
             assert_same_bits(h2[s_], r.histogram, f"batch {k} slot {s_} own histogram")
             assert_same_bits(e2[s_], r.bin_edges, f"batch {k} slot {s_} own edges")
