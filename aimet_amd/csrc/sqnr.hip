@@ -3,7 +3,8 @@
 // The (histogram, delta, offset, bin) tensor of the reference is never materialised: one workgroup owns one
 // (histogram, delta) row, its waves take the offset candidates in turn, lanes stride over the bins with the histogram
 // and bin mid-points held in LDS, and the clipping/quantisation noise of a candidate is accumulated in fp64.  A second
-// single-workgroup launch per histogram picks the first minimum and writes the encoding.
+// single-workgroup launch per histogram picks the first minimum and writes the encoding.  Searches over many histograms
+// (per-channel analyzers) price one candidate per lane instead (sqnr_noise_lanes_kernel).
 //
 // Candidate generation repeats the reference's fp32 operations one by one (encoding_analyzer.py:728-820); the only
 // host-made input is the rounded offset grid, because torch.arange computes it in double precision on the CPU.
@@ -125,6 +126,83 @@ __global__ __launch_bounds__(kBlock) void sqnr_noise_kernel(const SqnrArgs a) {
     }
 }
 
+// The same sums with one lane per candidate, for searches with enough candidates to fill the GPU that way (per-channel
+// and blockwise analyzers).  A lane walks every bin of its slot's staged histogram -- all lanes read the same LDS word,
+// a broadcast -- so a candidate is derived once instead of once per lane of a wave, no cross-lane sum is needed, and
+// the divisor of the bin loop is a per-lane constant: with its reciprocal at hand the quotient takes the
+// division-free form (two residual corrections, correctly rounded like the IEEE sequence as long as nothing under- or
+// overflows: bin centres up to 2^60 and a step in [2^-60, 2^60]; a wave with a lane outside that takes the plain
+// division).  The bins are summed in fp64 in two interleaved chains.
+constexpr float kSqnrFastDivMax = 1.152921504606846976e18f;   // 2^60
+constexpr float kSqnrFastDivMin = 8.673617379884035472e-19f;  // 2^-60
+constexpr int kLaneBlockMax = 512;
+
+template <bool FAST, bool P2>
+__device__ __forceinline__ double lane_noise(const SqnrArgs& a, const float2* hm, int B, Cand c, float rs) {
+    double acc0 = 0.0, acc1 = 0.0;
+    auto term = [&](float2 v) {
+        const float mid = v.y;
+        float t;
+        if (FAST) {
+            const float q0 = mid * rs;
+            const float q1 = __builtin_fmaf(__builtin_fmaf(-q0, c.delta, mid), rs, q0);
+            t = __builtin_fmaf(__builtin_fmaf(-q1, c.delta, mid), rs, q1);
+        } else {
+            t = mid / c.delta;
+        }
+        float q = __builtin_rintf(t - c.offset);
+        const bool clipped = (q < 0.f) | (q > a.num_steps);
+        q = q < 0.f ? 0.f : (q > a.num_steps ? a.num_steps : q);
+        const float y = (q + c.offset) * c.delta;
+        const float ad = __builtin_fabsf(y - mid);
+        const float err = (P2 ? ad * ad : __builtin_powf(ad, a.p)) * v.x;
+        // gamma == 1 leaves the term as it is, like the reference's skipped multiplication
+        return (double)(clipped ? err * a.gamma : err);
+    };
+    int b = 0;
+#pragma unroll 4
+    for (; b + 1 < B; b += 2) {
+        acc0 += term(hm[b]);
+        acc1 += term(hm[b + 1]);
+    }
+    if (b < B) acc0 += term(hm[b]);
+    return acc0 + acc1;
+}
+
+__global__ __launch_bounds__(kLaneBlockMax) void sqnr_noise_lanes_kernel(const SqnrArgs a) {
+    extern __shared__ float2 sqnr_hm[];  // [num_bins] (count, bin centre)
+    const int s = blockIdx.y;
+    const int B = a.num_bins, O = a.num_offsets;
+    const float* e = a.edges + (size_t)s * (B + 1);
+    const float w = e[1] - e[0];
+    const float first_mid = e[0] + w / 2.f;
+    for (int b = threadIdx.x; b < B; b += blockDim.x)
+        sqnr_hm[b] = make_float2(a.hist[(size_t)s * B + b], first_mid + w * (float)b);
+    __syncthreads();
+    const int pairs = a.num_deltas * O;
+    const int p = blockIdx.x * blockDim.x + threadIdx.x;
+    const bool live = p < pairs;
+    const int d = live ? p / O : 0, o = live ? p - d * O : 0;
+    const Cand c = candidate(a, s, d, o);
+    const float last_mid = first_mid + w * (float)(B - 1);
+    const float dm = __builtin_fabsf(c.delta);
+    const bool fast = __builtin_fabsf(first_mid) <= kSqnrFastDivMax && __builtin_fabsf(last_mid) <= kSqnrFastDivMax &&
+                      dm >= kSqnrFastDivMin && dm <= kSqnrFastDivMax;
+    const bool all_fast = __builtin_amdgcn_ballot_w64(!fast) == 0;
+    const float rs = all_fast ? 1.0f / c.delta : 0.f;
+    double acc;
+    if (a.p == 2.0f)
+        acc = all_fast ? lane_noise<true, true>(a, sqnr_hm, B, c, rs) : lane_noise<false, true>(a, sqnr_hm, B, c, rs);
+    else
+        acc = all_fast ? lane_noise<true, false>(a, sqnr_hm, B, c, rs) : lane_noise<false, false>(a, sqnr_hm, B, c, rs);
+    if (live) {
+        const size_t i = (size_t)s * pairs + p;
+        a.noise[i] = (float)acc;
+        a.deltas[i] = c.delta;
+        a.offsets[i] = c.offset;
+    }
+}
+
 __global__ __launch_bounds__(kBlock) void sqnr_select_kernel(const SqnrArgs a) {
     __shared__ float v_sm[kBlock];
     __shared__ int i_sm[kBlock];
@@ -208,14 +286,26 @@ extern "C" int ahq_sqnr_search(const ahq_sqnr_params* p, const float* hist, cons
     a.out = out;
     a.best_index = best_index;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    // a per-tensor search has a few thousand candidates in all: one per wave, so that its latency is that of a single
-    // candidate; with many slots a workgroup prices up to 64 per staged histogram
     const int pairs = a.num_deltas * a.num_offsets;
-    int64_t ppb = ((int64_t)pairs * a.num_slots) / 2048;
-    ppb = ppb < kBlock / kWave ? kBlock / kWave : (ppb > kPairsPerBlock ? kPairsPerBlock : ppb);
-    a.pairs_per_block = (int)ppb;
-    hipLaunchKernelGGL(sqnr_noise_kernel, dim3((unsigned)((pairs + ppb - 1) / ppb), a.num_slots), dim3(kBlock),
-                       2 * (size_t)a.num_bins * sizeof(float), st, a);
+    // One lane per candidate costs about 19 instructions per bin for a whole wave of candidates; one wave per candidate
+    // about 30 per 64 bins plus 150 for deriving the candidate and summing across lanes.  The first form also needs
+    // enough waves of candidates to occupy the GPU, which a per-tensor search does not have.
+    const int64_t cand_waves = (pairs + kWave - 1) / kWave;
+    const int64_t cost_lanes = cand_waves * a.num_bins * 19;
+    const int64_t cost_waves = (int64_t)pairs * ((int64_t)a.num_bins * 30 / kWave + 150);
+    if (cand_waves * a.num_slots >= 512 && cost_lanes < cost_waves) {
+        const int block = (int)(cand_waves * kWave < kLaneBlockMax ? cand_waves * kWave : kLaneBlockMax);
+        hipLaunchKernelGGL(sqnr_noise_lanes_kernel, dim3((unsigned)((pairs + block - 1) / block), a.num_slots), dim3(block),
+                           (size_t)a.num_bins * sizeof(float2), st, a);
+    } else {
+        // a per-tensor search has a few thousand candidates in all: one per wave, so that its latency is that of a
+        // single candidate; with many slots a workgroup prices up to 64 per staged histogram
+        int64_t ppb = ((int64_t)pairs * a.num_slots) / 2048;
+        ppb = ppb < kBlock / kWave ? kBlock / kWave : (ppb > kPairsPerBlock ? kPairsPerBlock : ppb);
+        a.pairs_per_block = (int)ppb;
+        hipLaunchKernelGGL(sqnr_noise_kernel, dim3((unsigned)((pairs + ppb - 1) / ppb), a.num_slots), dim3(kBlock),
+                           2 * (size_t)a.num_bins * sizeof(float), st, a);
+    }
     hipLaunchKernelGGL(sqnr_select_kernel, dim3(a.num_slots), dim3(kBlock), 0, st, a);
     return check_launch("ahq_sqnr_search");
 }

@@ -208,6 +208,62 @@ def test_sqnr_search(device, cfg, symmetric, num_steps):
     assert_same_bits(hi, hi_ref, "encoding max")
 
 
+@pytest.mark.parametrize("symmetric", [False, True])
+@pytest.mark.parametrize("cfg", [dict(num_bins=512), dict(num_bins=301, gamma=1.0), dict(num_bins=256, p=3.0)],
+                         ids=["bins512", "odd_bins_gamma1", "cubic_norm"])
+def test_sqnr_search_many_slots(device, cfg, symmetric):
+    """Per-channel searches price one candidate per lane; same candidates, noise sums and winners as the oracle.  A slot
+    whose winner differs must be a tie of the two noise sums to within the fp32 rounding of the reference's own sums."""
+    from aimet_amd.quantization.encoding_analyzer import SqnrEncodingAnalyzer, _LpNormEncodingAnalyzer
+
+    S = 300
+    p = cfg.get("p", 2.0)
+    kw = dict(asym_deltas=17, sym_deltas=101, num_offsets=21, gamma=cfg.get("gamma", 3.0))
+    if p == 2.0:
+        an = SqnrEncodingAnalyzer((S, 1), num_bins=cfg["num_bins"], gamma=kw["gamma"])
+    else:
+        an = _LpNormEncodingAnalyzer((S, 1), cfg["num_bins"], p=p, asymmetric_delta_candidates=17,
+                                     symmetric_delta_candidates=101, offset_candidates=21, max_parallelism=64,
+                                     gamma=kw["gamma"])
+    ref = O.HistObserver((S, 1), cfg["num_bins"])
+    g = torch.Generator().manual_seed(21)
+    scale = torch.logspace(-3, 3, S).reshape(S, 1)
+    for k in range(2):
+        x = torch.randn(S, 700, generator=g) * scale * (k + 1) + (torch.arange(S).reshape(S, 1) % 5 - 2) * scale
+        x[::7] = x[::7].abs()  # one-sided slots
+        # bin centres beyond 2^60: these slots take the plain division; squares stay finite, some sums overflow alike
+        if p == 2.0:
+            x[-10:] = 2e18 + torch.randn(10, 700, generator=g) * 1e15
+        ref.update(x)
+        an.update_stats(x.to(device))
+    lo, hi = an.compute_encodings(255, symmetric)
+    d_ref, o_ref = O.sqnr_candidates(ref.stats, 255, symmetric, kw["asym_deltas"], kw["sym_deltas"], kw["num_offsets"])
+    noise_ref = O.sqnr_noise(ref.stats, d_ref, o_ref, 255, p, kw["gamma"])
+    ls = an.last_search
+    assert_same_bits(ls["deltas"].expand_as(ls["noise"]), d_ref.expand(noise_ref.shape), "candidate deltas")
+    # one-sided slots clamp a candidate minimum of -0 against an observed +0: which zero max() keeps is an accident of
+    # torch's vectorised CPU kernel, so zeros are compared without their sign (adding +0 makes them all positive)
+    assert_same_bits(ls["offsets"].expand_as(ls["noise"]) + 0.0, o_ref.expand(noise_ref.shape) + 0.0, "candidate offsets")
+    got, want = ls["noise"].cpu().double(), noise_ref.double()
+    assert not want.isnan().any()
+    close = (got == want) | ((got - want).abs() <= 1e-5 * want.abs())  # every term is positive: relative per candidate
+    assert bool(close.all()), f"noise: {int((~close).sum())} candidates differ"
+    assert int(want[-10:].isfinite().sum()) > 0
+    lo_ref, hi_ref, _, _, bi_ref = O.sqnr_encodings(ref.stats, (S, 1), 255, symmetric, p=p, **kw)
+    flat_ref = noise_ref.reshape(S, -1)
+    bi_ref = bi_ref.reshape(S)
+    bi = ls["best_index"].cpu().reshape(S)
+    differ = (bi != bi_ref).nonzero().flatten().tolist()
+    assert len(differ) <= S // 50, differ
+    for s_ in differ:
+        a_, b_ = float(flat_ref[s_, bi[s_]]), float(flat_ref[s_, bi_ref[s_]])
+        assert abs(a_ - b_) <= 1e-6 * abs(b_), (s_, a_, b_)
+    same = torch.ones(S, dtype=torch.bool)
+    same[differ] = False
+    assert_same_bits(lo.cpu().reshape(S)[same] + 0.0, lo_ref.reshape(S)[same] + 0.0, "encoding min")
+    assert_same_bits(hi.cpu().reshape(S)[same], hi_ref.reshape(S)[same], "encoding max")
+
+
 def test_tf_enhanced_preset_and_per_channel(device):
     from aimet_amd.quantization.encoding_analyzer import TfEnhancedEncodingAnalyzer
 
