@@ -203,18 +203,25 @@ __global__ __launch_bounds__(kLaneBlockMax) void sqnr_noise_lanes_kernel(const S
     }
 }
 
+// torch.min over the flattened candidates (encoding_analyzer.py:822-839): the first minimum, and a NaN counts as
+// smaller than every number, so the first NaN wins when there is one.
+__device__ __forceinline__ bool sqnr_better(float v, int i, float bv, int bi) {
+    const bool vn = v != v, bn = bv != bv;
+    if (vn | bn) return vn && (!bn || i < bi);
+    return v < bv || (v == bv && i < bi);
+}
+
 __global__ __launch_bounds__(kBlock) void sqnr_select_kernel(const SqnrArgs a) {
     __shared__ float v_sm[kBlock];
     __shared__ int i_sm[kBlock];
     const int s = blockIdx.x;
     const int n = a.num_deltas * a.num_offsets;
     const float* noise = a.noise + (size_t)s * n;
-    // first minimum; NaN never wins unless everything is NaN
     float best = __builtin_inff();
     int bi = n;
     for (int i = threadIdx.x; i < n; i += kBlock) {
         const float v = noise[i];
-        if (v < best) {
+        if (sqnr_better(v, i, best, bi)) {
             best = v;
             bi = i;
         }
@@ -226,7 +233,7 @@ __global__ __launch_bounds__(kBlock) void sqnr_select_kernel(const SqnrArgs a) {
         if (threadIdx.x < st) {
             const float ov = v_sm[threadIdx.x + st];
             const int oi = i_sm[threadIdx.x + st];
-            if (ov < v_sm[threadIdx.x] || (ov == v_sm[threadIdx.x] && oi < i_sm[threadIdx.x])) {
+            if (sqnr_better(ov, oi, v_sm[threadIdx.x], i_sm[threadIdx.x])) {
                 v_sm[threadIdx.x] = ov;
                 i_sm[threadIdx.x] = oi;
             }

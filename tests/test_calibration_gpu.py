@@ -213,7 +213,9 @@ def test_sqnr_search(device, cfg, symmetric, num_steps):
                          ids=["bins512", "odd_bins_gamma1", "cubic_norm"])
 def test_sqnr_search_many_slots(device, cfg, symmetric):
     """Per-channel searches price one candidate per lane; same candidates, noise sums and winners as the oracle.  A slot
-    whose winner differs must be a tie of the two noise sums to within the fp32 rounding of the reference's own sums."""
+    whose winner differs must be a tie of the two noise sums to within the fp32 rounding of the reference's own sums.
+    The last ten slots hold values near 2e18: bin centres too large for the division-free quotient, sums that overflow
+    and, for the cubic norm, NaN sums."""
     from aimet_amd.quantization.encoding_analyzer import SqnrEncodingAnalyzer, _LpNormEncodingAnalyzer
 
     S = 300
@@ -232,8 +234,7 @@ def test_sqnr_search_many_slots(device, cfg, symmetric):
         x = torch.randn(S, 700, generator=g) * scale * (k + 1) + (torch.arange(S).reshape(S, 1) % 5 - 2) * scale
         x[::7] = x[::7].abs()  # one-sided slots
         # bin centres beyond 2^60: these slots take the plain division; squares stay finite, some sums overflow alike
-        if p == 2.0:
-            x[-10:] = 2e18 + torch.randn(10, 700, generator=g) * 1e15
+        x[-10:] = 2e18 + torch.randn(10, 700, generator=g) * 1e15
         ref.update(x)
         an.update_stats(x.to(device))
     lo, hi = an.compute_encodings(255, symmetric)
@@ -245,10 +246,11 @@ def test_sqnr_search_many_slots(device, cfg, symmetric):
     # torch's vectorised CPU kernel, so zeros are compared without their sign (adding +0 makes them all positive)
     assert_same_bits(ls["offsets"].expand_as(ls["noise"]) + 0.0, o_ref.expand(noise_ref.shape) + 0.0, "candidate offsets")
     got, want = ls["noise"].cpu().double(), noise_ref.double()
-    assert not want.isnan().any()
-    close = (got == want) | ((got - want).abs() <= 1e-5 * want.abs())  # every term is positive: relative per candidate
+    # every term is positive: relative per candidate.  The cubes of the huge slots overflow, and an infinite term times
+    # an empty bin makes the sum NaN on both sides; torch.min then returns the first NaN
+    close = (got == want) | ((got - want).abs() <= 1e-5 * want.abs()) | (got.isnan() & want.isnan())
     assert bool(close.all()), f"noise: {int((~close).sum())} candidates differ"
-    assert int(want[-10:].isfinite().sum()) > 0
+    assert bool(want[-10:].isnan().any()) == (p != 2.0) and (p != 2.0 or int(want[-10:].isfinite().sum()) > 0)
     lo_ref, hi_ref, _, _, bi_ref = O.sqnr_encodings(ref.stats, (S, 1), 255, symmetric, p=p, **kw)
     flat_ref = noise_ref.reshape(S, -1)
     bi_ref = bi_ref.reshape(S)
