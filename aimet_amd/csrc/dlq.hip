@@ -599,10 +599,17 @@ __global__ __launch_bounds__(kWave) void dlq_tfe_cost_wave_kernel(const TfeArgs 
     const float min_mid = centers[min_ind], max_mid = centers[max_ind];
     const float inv_delta = 1 / delta;
     double sat_bottom = 0, sat_top = 0, quant = 0;
+    // the next chunk's statistics are fetched before the additions of this one, whose chain hides the latency
+    float c_next = centers[lane];
+    double p_next = pdf[lane];
     for (int i0 = 0; i0 < kPdf; i0 += kWave) {
         const int i = i0 + lane;
-        const float c = centers[i];
-        const double p = pdf[i];
+        const float c = c_next;
+        const double p = p_next;
+        if (i0 + kWave < kPdf) {
+            c_next = centers[i + kWave];
+            p_next = pdf[i + kWave];
+        }
         double tb = 0, tt = 0, tq = 0;
         if (i < min_ind) {
             const double d = (double)c - min_mid;
