@@ -212,33 +212,47 @@ __device__ __forceinline__ bool sqnr_better(float v, int i, float bv, int bi) {
 }
 
 __global__ __launch_bounds__(kBlock) void sqnr_select_kernel(const SqnrArgs a) {
-    __shared__ float v_sm[kBlock];
-    __shared__ int i_sm[kBlock];
+    __shared__ float v_sm[kBlock / kWave];
+    __shared__ int i_sm[kBlock / kWave];
     const int s = blockIdx.x;
     const int n = a.num_deltas * a.num_offsets;
     const float* noise = a.noise + (size_t)s * n;
     float best = __builtin_inff();
     int bi = n;
-    for (int i = threadIdx.x; i < n; i += kBlock) {
-        const float v = noise[i];
-        if (sqnr_better(v, i, best, bi)) {
-            best = v;
-            bi = i;
-        }
-    }
-    v_sm[threadIdx.x] = best;
-    i_sm[threadIdx.x] = bi;
-    __syncthreads();
-    for (int st = kBlock / 2; st >= 1; st >>= 1) {
-        if (threadIdx.x < st) {
-            const float ov = v_sm[threadIdx.x + st];
-            const int oi = i_sm[threadIdx.x + st];
-            if (sqnr_better(ov, oi, v_sm[threadIdx.x], i_sm[threadIdx.x])) {
-                v_sm[threadIdx.x] = ov;
-                i_sm[threadIdx.x] = oi;
+    constexpr int kLoads = 4;  // loads in flight per lane
+    for (int i0 = threadIdx.x; i0 < n; i0 += kLoads * kBlock) {
+        float v[kLoads];
+#pragma unroll
+        for (int u = 0; u < kLoads; ++u) v[u] = i0 + u * kBlock < n ? noise[i0 + u * kBlock] : __builtin_inff();
+#pragma unroll
+        for (int u = 0; u < kLoads; ++u) {
+            const int i = i0 + u * kBlock < n ? i0 + u * kBlock : n;
+            if (sqnr_better(v[u], i, best, bi)) {
+                best = v[u];
+                bi = i;
             }
         }
-        __syncthreads();
+    }
+#pragma unroll
+    for (int m = kWave / 2; m >= 1; m >>= 1) {
+        const float ov = __shfl_xor(best, m, kWave);
+        const int oi = __shfl_xor(bi, m, kWave);
+        if (sqnr_better(ov, oi, best, bi)) {
+            best = ov;
+            bi = oi;
+        }
+    }
+    if ((threadIdx.x & (kWave - 1)) == 0) {
+        v_sm[threadIdx.x / kWave] = best;
+        i_sm[threadIdx.x / kWave] = bi;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < kBlock / kWave; ++w)
+            if (sqnr_better(v_sm[w], i_sm[w], v_sm[0], i_sm[0])) {
+                v_sm[0] = v_sm[w];
+                i_sm[0] = i_sm[w];
+            }
     }
     if (threadIdx.x == 0) {
         int idx = i_sm[0];
