@@ -324,12 +324,14 @@ struct PdfFinArgs {
     int32_t* meta;
     unsigned long long cnt;  // elements per slot in this batch
     uint32_t* hist_out;      // optional [S][kPdf]: this batch's integer histogram
+    int32_t num_slots;
 };
 
 // Average the batch into the running PDF (math_functions.cpp:274-284)
 __global__ __launch_bounds__(kBlock) void dlq_pdf_finish_kernel(const PdfFinArgs a) {
-    const int s = blockIdx.y;
     const int i = blockIdx.x * kBlock + threadIdx.x;
+    // the y dimension of a grid ends at 65535: slots beyond it are taken in further rounds
+    for (int s = blockIdx.y; s < a.num_slots; s += gridDim.y) {
     const bool active = a.params[4 * s + 2] != 0.f;
     uint32_t h = 0;
     if (active) {
@@ -343,6 +345,7 @@ __global__ __launch_bounds__(kBlock) void dlq_pdf_finish_kernel(const PdfFinArgs
     if (a.hist_out) a.hist_out[(size_t)s * kPdf + i] = h;
     // pdf.iterations++ ; every thread above took the old count from `params`, so nothing else reads this word here
     if (active && i == 0) a.meta[4 * s] = __float_as_int(a.params[4 * s + 3]) + 1;
+    }
 }
 
 // Single slot, many partial histograms: fold and average in one launch.  A workgroup owns kFfBins neighbouring
@@ -795,7 +798,7 @@ __global__ __launch_bounds__(kWave) void dlq_percentile_kernel(const double* xle
 // -------------------------------------------------------------------------------------------------- host side ---
 namespace {
 
-constexpr int kPdfThreads = 1024;  // one workgroup per compute unit: 16 copies x 1536 buckets x 4 B = 96 KB of LDS
+constexpr int kPdfThreads = 1024;  // two workgroups per compute unit: 8 copies x 1536 buckets x 4 B = 48 KB of LDS each
 constexpr int kPdfCopies = 8;
 constexpr int kPdfBlocksMax = 512;
 
@@ -936,21 +939,13 @@ extern "C" int ahq_dlq_pdf_update(int32_t dtype, const ahq_layout* layout, const
     fa.meta = st->meta;
     fa.cnt = (unsigned long long)(c.numel / S);
     fa.hist_out = hist_out;
+    fa.num_slots = S;
     if (pp.fast) {
         ba.partials = counts;
         const size_t lds = (size_t)pp.copies * kPdf * 4;
         const dim3 g(pp.nblocks), b(kPdfThreads);
-#define AHQ_LAUNCH_PDF_K(K)                                                                                    \
-    do {                                                                                                       \
-        static bool attr_set = false; /* more than 64 KB of dynamic LDS has to be allowed once per kernel */     \
-        if (!attr_set) {                                                                                       \
-            if (hipFuncSetAttribute(reinterpret_cast<const void*>(&K), hipFuncAttributeMaxDynamicSharedMemorySize, \
-                                    (int)lds) != hipSuccess)                                                   \
-                return set_error("cannot reserve LDS for the PDF kernel"), AHQ_ERR_LAUNCH;                     \
-            attr_set = true;                                                                                   \
-        }                                                                                                      \
-        hipLaunchKernelGGL(K, g, b, lds, s, ba);                                                               \
-    } while (0)
+        static_assert((size_t)kPdfCopies * kPdf * 4 <= 64 * 1024, "dynamic LDS beyond 64 KB needs hipFuncSetAttribute");
+#define AHQ_LAUNCH_PDF_K(K) hipLaunchKernelGGL(K, g, b, lds, s, ba)
 #define AHQ_LAUNCH_PDF(IO)                                                                                     \
     do {                                                                                                       \
         if (pp.plan.vec == 1) AHQ_LAUNCH_PDF_K((dlq_pdf_bin_kernel<IO, 1, kPdfThreads>));                      \
@@ -1008,7 +1003,7 @@ extern "C" int ahq_dlq_pdf_update(int32_t dtype, const ahq_layout* layout, const
         fa.counts = counts;
         fa.nparts = 1;
     }
-    hipLaunchKernelGGL(dlq_pdf_finish_kernel, dim3(kPdf / kBlock, S), dim3(kBlock), 0, s, fa);
+    hipLaunchKernelGGL(dlq_pdf_finish_kernel, dim3(kPdf / kBlock, S < 65535 ? S : 65535), dim3(kBlock), 0, s, fa);
     return check_launch("dlq_pdf_update");
 }
 

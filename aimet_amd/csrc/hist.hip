@@ -218,6 +218,7 @@ struct BinArgs : Geom {
     int64_t ntiles;
     // speculative pass (see hist_bin_kernel): the running range as the state holds it, and where the batch's extrema go
     const float* state_minmax;
+    const float* state_edges;  // running bin edges [B + 1]
     float* part_min;       // [nblocks]
     float* part_max;
     const int32_t* rebin;  // second pass: leave at once unless *rebin != 0
@@ -276,14 +277,19 @@ __device__ __forceinline__ int bin_estimate(float v, const RangeC& r, float Bf, 
 //
 // SPEC (one histogram): the speculative pass of a batch after the first, for a caller that wants the running
 // statistics only.  Most batches of a calibration stay inside the running range, and then the reference bins them on
-// exactly that range; so the batch is binned on the running range as the state holds it.  The running range can only
-// move because of finite elements outside it, and those already take the kernel's rare element-by-element path:
-// their extrema are collected there at no cost to the others (per-workgroup partials that the prepare kernel folds;
-// +-inf when nothing lies outside, which leaves the range where it is).  If the prepare kernel then finds the range
-// unchanged, these counts are the batch's contribution and the second read of the batch is skipped (the ordinary pass
-// is launched with `rebin` and leaves at once); if the range grew, the ordinary pass bins again on the new range and
-// overwrites the partial histograms.  A running range of zero width is binned on a widened one, so then every
-// element is looked at.
+// exactly that range; so the batch is binned on the running range as the state holds it.  The reference clamps the
+// batch's extrema with the outermost bin edges (updated_max = clamp(new.max, bin_edges[-1], limit),
+// encoding_analyzer.py:266-270), so the batch's own minimum / maximum matters only beyond those edges.  When the edges
+// coincide with the running range or lie outside it, such elements are outside the running range too and already take
+// the kernel's rare element-by-element path: their extrema are collected there at no cost to the others
+// (per-workgroup partials that the prepare kernel folds; +-inf when there are none, which the clamp turns into the
+// edge).  The last edge B * RN(width / B) + min can also round to a value BELOW the running maximum; a batch whose
+// maximum lies between the two (a repeated batch, a saturating activation) must then report it, so in that case the
+// kernel follows the extrema of every finite element (`track_all`, kernel-uniform).  If the prepare kernel then finds
+// the range unchanged, these counts are the batch's contribution and the second read of the batch is skipped (the
+// ordinary pass is launched with `rebin` and leaves at once); if the range moved, the ordinary pass bins again on the
+// new range and overwrites the partial histograms.  A running range of zero width is binned on a widened one, so then
+// every element is looked at.
 template <typename IO, int VEC, int NH, bool SPEC = false>
 __global__ __launch_bounds__(kBlock, 6) void hist_bin_kernel(const BinArgs a) {
     extern __shared__ uint32_t lds[];  // [NH][B][copies]: lane l adds to copy l % copies, neighbouring copies sit in neighbouring banks
@@ -306,12 +312,21 @@ __global__ __launch_bounds__(kBlock, 6) void hist_bin_kernel(const BinArgs a) {
         for (int h = 0; h < NH; ++h) r[h] = load_range(a.ranges, h);
     }
     float ext_min = __builtin_inff(), ext_max = -__builtin_inff();  // SPEC: finite extrema of this lane's elements
-    const bool degenerate = SPEC && run_lo == run_hi;
-    auto track = [&](float v) {  // finite elements outside the running range
+    // thresholds beyond which the batch's own extrema reach the reference's clamp
+    float thr_min = run_lo, thr_max = run_hi;
+    bool track_all = false;
+    if (SPEC) {
+        const float c_first = a.state_edges[0], c_last = a.state_edges[B];
+        thr_min = c_first;
+        thr_max = c_last;
+        // every element has to be followed when an edge lies strictly inside the running range (or the range is empty)
+        track_all = (run_lo == run_hi) | (c_last < run_hi) | (c_first > run_lo);
+    }
+    auto track = [&](float v) {  // finite elements beyond the outermost edges
         if (SPEC) {
             const bool fin = __builtin_fabsf(v) < __builtin_inff();
-            ext_min = fminf(ext_min, (fin & (v < run_lo)) ? v : __builtin_inff());
-            ext_max = fmaxf(ext_max, (fin & (v > run_hi)) ? v : -__builtin_inff());
+            ext_min = fminf(ext_min, (fin & (v < thr_min)) ? v : __builtin_inff());
+            ext_max = fmaxf(ext_max, (fin & (v > thr_max)) ? v : -__builtin_inff());
         }
     };
     __syncthreads();
@@ -349,7 +364,7 @@ __global__ __launch_bounds__(kBlock, 6) void hist_bin_kernel(const BinArgs a) {
         Pack<IO, VEC> in[kUnroll];
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) in[u] = load_pack<IO, VEC>(x + (tile * kTileVec + u * kBlock + threadIdx.x) * VEC);
-        if (degenerate) {
+        if (track_all) {
             for (int u = 0; u < kUnroll; ++u)
                 for (int k = 0; k < VEC; ++k) track(load_f32(in[u].v[k]));
         }
@@ -607,9 +622,11 @@ __global__ __launch_bounds__(kBlock) void hist_finish_kernel(const FinArgs a) {
     __shared__ unsigned long long sm[4][2][64];
     __shared__ unsigned long long edge_cnt[2][2];
     const int B = a.num_bins, NH = a.nhist;
-    const int s = blockIdx.y;
     const int bl = threadIdx.x & 63, grp = threadIdx.x >> 6;
     const int b = blockIdx.x * 64 + bl;
+    // the y dimension of a grid ends at 65535: slots beyond it are taken in further rounds
+    for (int s = blockIdx.y; s < a.num_slots; s += gridDim.y) {
+    if (s != (int)blockIdx.y) __syncthreads();  // the previous slot's sums in LDS are still being read
     const uint32_t* base = a.counts + (size_t)s * a.nparts * NH * (B + 2);
     unsigned long long c[2] = {0, 0};
     if (b < B) {
@@ -631,7 +648,7 @@ __global__ __launch_bounds__(kBlock) void hist_finish_kernel(const FinArgs a) {
         if (lane == 0) edge_cnt[h][side] = t;
     }
     __syncthreads();
-    if (grp != 0 || b >= B) return;
+    if (grp != 0 || b >= B) continue;
     unsigned long long tot[2];
     for (int h = 0; h < 2; ++h) tot[h] = sm[0][h][bl] + sm[1][h][bl] + sm[2][h][bl] + sm[3][h][bl];
     // the batch's own histogram: counts, then "+= below" on bin 0 and "+= above" on the last bin
@@ -651,6 +668,7 @@ __global__ __launch_bounds__(kBlock) void hist_finish_kernel(const FinArgs a) {
     a.hist[(size_t)s * B + b] = uh;
     a.edges[(size_t)s * (B + 1) + b] = a.upd_edges[(size_t)s * (B + 1) + b];
     if (b == B - 1) a.edges[(size_t)s * (B + 1) + B] = a.upd_edges[(size_t)s * (B + 1) + B];
+    }
 }
 
 }  // namespace ahq
@@ -787,6 +805,7 @@ extern "C" int ahq_hist_update(int32_t dtype, const ahq_layout* layout, const vo
     if (speculative) {
         ba.partials = counts;
         ba.state_minmax = st->minmax;
+        ba.state_edges = st->edges;
         ba.part_min = reinterpret_cast<float*>(w + hp.off_mm_ws);
         ba.part_max = ba.part_min + hp.nblocks;
         const size_t lds = (size_t)hp.copies * B * 4;
@@ -922,6 +941,6 @@ extern "C" int ahq_hist_update(int32_t dtype, const ahq_layout* layout, const vo
     fa.hist = st->hist;
     fa.edges = st->edges;
     fa.new_hist = st->new_hist;
-    hipLaunchKernelGGL(hist_finish_kernel, dim3((B + 63) / 64, S), dim3(kBlock), 0, s, fa);
+    hipLaunchKernelGGL(hist_finish_kernel, dim3((B + 63) / 64, S < 65535 ? S : 65535), dim3(kBlock), 0, s, fa);
     return check_launch("ahq_hist_update");
 }

@@ -76,6 +76,7 @@ __device__ __forceinline__ Cand candidate(const SqnrArgs& a, int s, int d, int o
 }
 
 constexpr int kSqnrMaxBins = 4096;
+constexpr int kMaxGridY = 65535;  // largest y dimension of a grid
 
 // A workgroup stages one slot's histogram and bin centres and prices kPairsPerBlock (delta, offset) candidates, one
 // wave per candidate at a time.  Candidates are numbered delta-major across the whole grid, so a symmetric search
@@ -84,10 +85,12 @@ constexpr int kPairsPerBlock = 64;  // at most; fewer when that leaves the GPU s
 
 __global__ __launch_bounds__(kBlock) void sqnr_noise_kernel(const SqnrArgs a) {
     extern __shared__ float sqnr_lds[];  // [2][num_bins]
-    const int s = blockIdx.y;
     const int B = a.num_bins, O = a.num_offsets;
     float* h_lds = sqnr_lds;
     float* m_lds = sqnr_lds + B;
+    // the y dimension of a grid ends at 65535: slots beyond it are taken in further rounds
+    for (int s = blockIdx.y; s < a.num_slots; s += gridDim.y) {
+    if (s != (int)blockIdx.y) __syncthreads();  // the previous slot's staged histogram is still being read
     const float* e = a.edges + (size_t)s * (B + 1);
     const float w = e[1] - e[0];
     const float first_mid = e[0] + w / 2.f;
@@ -123,6 +126,7 @@ __global__ __launch_bounds__(kBlock) void sqnr_noise_kernel(const SqnrArgs a) {
             a.deltas[i] = c.delta;
             a.offsets[i] = c.offset;
         }
+    }
     }
 }
 
@@ -171,8 +175,9 @@ __device__ __forceinline__ double lane_noise(const SqnrArgs& a, const float2* hm
 
 __global__ __launch_bounds__(kLaneBlockMax) void sqnr_noise_lanes_kernel(const SqnrArgs a) {
     extern __shared__ float2 sqnr_hm[];  // [num_bins] (count, bin centre)
-    const int s = blockIdx.y;
     const int B = a.num_bins, O = a.num_offsets;
+    for (int s = blockIdx.y; s < a.num_slots; s += gridDim.y) {  // slots beyond the y limit of a grid: further rounds
+    if (s != (int)blockIdx.y) __syncthreads();
     const float* e = a.edges + (size_t)s * (B + 1);
     const float w = e[1] - e[0];
     const float first_mid = e[0] + w / 2.f;
@@ -200,6 +205,7 @@ __global__ __launch_bounds__(kLaneBlockMax) void sqnr_noise_lanes_kernel(const S
         a.noise[i] = (float)acc;
         a.deltas[i] = c.delta;
         a.offsets[i] = c.offset;
+    }
     }
 }
 
@@ -312,11 +318,12 @@ extern "C" int ahq_sqnr_search(const ahq_sqnr_params* p, const float* hist, cons
     // about 30 per 64 bins plus 150 for deriving the candidate and summing across lanes.  The first form also needs
     // enough waves of candidates to occupy the GPU, which a per-tensor search does not have.
     const int64_t cand_waves = (pairs + kWave - 1) / kWave;
+    const unsigned grid_y = (unsigned)(a.num_slots < kMaxGridY ? a.num_slots : kMaxGridY);
     const int64_t cost_lanes = cand_waves * a.num_bins * 19;
     const int64_t cost_waves = (int64_t)pairs * ((int64_t)a.num_bins * 30 / kWave + 150);
     if (cand_waves * a.num_slots >= 512 && cost_lanes < cost_waves) {
         const int block = (int)(cand_waves * kWave < kLaneBlockMax ? cand_waves * kWave : kLaneBlockMax);
-        hipLaunchKernelGGL(sqnr_noise_lanes_kernel, dim3((unsigned)((pairs + block - 1) / block), a.num_slots), dim3(block),
+        hipLaunchKernelGGL(sqnr_noise_lanes_kernel, dim3((unsigned)((pairs + block - 1) / block), grid_y), dim3(block),
                            (size_t)a.num_bins * sizeof(float2), st, a);
     } else {
         // a per-tensor search has a few thousand candidates in all: one per wave, so that its latency is that of a
@@ -324,7 +331,7 @@ extern "C" int ahq_sqnr_search(const ahq_sqnr_params* p, const float* hist, cons
         int64_t ppb = ((int64_t)pairs * a.num_slots) / 2048;
         ppb = ppb < kBlock / kWave ? kBlock / kWave : (ppb > kPairsPerBlock ? kPairsPerBlock : ppb);
         a.pairs_per_block = (int)ppb;
-        hipLaunchKernelGGL(sqnr_noise_kernel, dim3((unsigned)((pairs + ppb - 1) / ppb), a.num_slots), dim3(kBlock),
+        hipLaunchKernelGGL(sqnr_noise_kernel, dim3((unsigned)((pairs + ppb - 1) / ppb), grid_y), dim3(kBlock),
                            2 * (size_t)a.num_bins * sizeof(float), st, a);
     }
     hipLaunchKernelGGL(sqnr_select_kernel, dim3(a.num_slots), dim3(kBlock), 0, st, a);

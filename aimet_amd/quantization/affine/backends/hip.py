@@ -257,8 +257,40 @@ class _HipAffineFunction(torch.autograd.Function):
         return (gx, gs_out, go_out) + none7
 
 
+def _broadcast_encodings(scale: torch.Tensor, offset: torch.Tensor, block_size):
+    """Scale and offset expanded to one common shape, the way the reference's elementwise arithmetic broadcasts them
+    against each other (torch_builtins.py:727-773: ``tensor / scale - offset``).  The kernels index both arrays with
+    the same encoding index, so a scalar offset next to a per-channel scale has to be materialised; ``expand`` is
+    differentiable, so autograd sums the gradient back to the operand's own shape."""
+    if offset.shape == scale.shape:
+        return scale, offset
+    try:
+        shape = torch.broadcast_shapes(scale.shape, offset.shape)
+    except RuntimeError as e:
+        raise RuntimeError(
+            f"Offset of shape {tuple(offset.shape)} cannot be broadcast with scale of shape {tuple(scale.shape)}"
+        ) from e
+    if block_size is not None and len(shape) != len(scale.shape):
+        raise RuntimeError(
+            f"Offset of shape {tuple(offset.shape)} has more dimensions than scale of shape {tuple(scale.shape)}, "
+            f"which block size {tuple(block_size)} describes"
+        )
+    if block_size is not None and tuple(shape) != tuple(scale.shape):
+        raise RuntimeError(
+            f"Offset of shape {tuple(offset.shape)} cannot be expanded to scale of shape {tuple(scale.shape)}"
+        )
+    return scale.expand(shape), offset.expand(shape)
+
+
 def _apply(tensor, scale, offset, arith, op, compute_dtype, qmin, qmax, block_size, zps):
     bs = tuple(block_size) if block_size else None
+    if offset.shape != scale.shape:
+        scale, offset = _broadcast_encodings(scale, offset, bs)
+        if bs is None and not _is_expandable(scale.shape, tensor.shape):
+            raise RuntimeError(
+                f"Encodings of shape {tuple(scale.shape)} cannot be expanded like input tensor of shape "
+                f"{tuple(tensor.shape)}"
+            )
     if not torch.is_grad_enabled() or not (tensor.requires_grad or scale.requires_grad or offset.requires_grad):
         # nothing to differentiate: skip the autograd bookkeeping (a whole-model forward makes hundreds of these calls)
         return _launch_forward(tensor, scale, offset, arith, op, compute_dtype, qmin, qmax, bs, zps)[0]

@@ -174,8 +174,10 @@ class AffineQuantizerBase(QuantizerBase, _GridMixin):
         # they are derived once and reused until min or max is written again (their version counters change) or
         # moved.  A whole-model forward calls this once per quantizer, and the half-dozen tiny kernels behind
         # get_scale()/get_offset() would otherwise cost more than the quantize-dequantize kernel itself.
-        # (Writes through `.data` do not bump the version counter and are not seen; the reference's own
-        # is_initialized() bookkeeping has the same blind spot.)
+        # Deviation from the reference, which recomputes scale and offset on every call: a write through `.data`
+        # (`q.min.data.copy_(...)`, `q.min.data.fill_(...)`) changes neither the version counter nor the address and
+        # is not seen here; such callers follow the write with invalidate_encoding_cache().  set_range(), copy_(),
+        # load_state_dict() and optimizer steps all bump the version counter and need nothing.
         if torch.is_grad_enabled() and (self.min.requires_grad or self.max.requires_grad):
             return self._derive_encodings()
         mn, mx = self.min, self.max
@@ -189,6 +191,11 @@ class AffineQuantizerBase(QuantizerBase, _GridMixin):
         if enc is not None:
             self.__dict__["_encoding_cache"] = (key, enc)
         return enc
+
+    def invalidate_encoding_cache(self) -> None:
+        """Forget the scale / offset derived from min / max.  Needed only after a write that bypasses torch's version
+        counter (through ``.data``); every tracked in-place write invalidates the cache by itself."""
+        self.__dict__.pop("_encoding_cache", None)
 
     def _fused_scale_offset(self):
         """get_scale(float32) and _get_offset(float32) of a quantizer that holds min / max on a GPU in one launch

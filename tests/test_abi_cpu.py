@@ -136,6 +136,52 @@ def test_cpu_tensors_fail_loudly():
         Q.affine.quantize_dequantize(torch.randn(2, 3, 4, 5), torch.ones(4), torch.zeros(()), 0, 255)
 
 
+def test_scale_and_offset_are_broadcast_against_each_other_on_the_host():
+    """The kernels read scale[e] and offset[e] with one index, so operands of different shapes are expanded to their
+    common shape before anything is launched; shapes that do not broadcast are refused."""
+    from aimet_amd.quantization.affine.backends import hip as H
+
+    scale, offset = torch.rand(6, 1) + 0.1, torch.tensor(-3.0)
+    s2, o2 = H._broadcast_encodings(scale, offset, None)
+    assert s2.shape == o2.shape == (6, 1) and bool((o2 == -3.0).all())
+    s2, o2 = H._broadcast_encodings(torch.tensor(0.5), torch.zeros(6, 1), None)
+    assert s2.shape == o2.shape == (6, 1)
+    s2, o2 = H._broadcast_encodings(torch.rand(6, 1), torch.zeros(1, 5), None)
+    assert s2.shape == o2.shape == (6, 5)
+    with pytest.raises(RuntimeError, match="cannot be broadcast"):
+        H._broadcast_encodings(torch.rand(6, 1), torch.zeros(4, 1), None)
+    with pytest.raises(RuntimeError, match="cannot be expanded"):
+        H._broadcast_encodings(torch.rand(6, 1), torch.zeros(6, 4), (1, 8))
+    s2, o2 = H._broadcast_encodings(torch.rand(6, 4), torch.tensor(0.0), (1, 8))
+    assert o2.shape == (6, 4)
+    # gradients flow back to each operand's own shape through the expansion
+    off = torch.zeros((), requires_grad=True)
+    _, o2 = H._broadcast_encodings(torch.rand(6, 1), off, None)
+    o2.sum().backward()
+    assert off.grad.shape == () and float(off.grad) == 6.0
+
+
+def test_encoding_cache_follows_tracked_writes_and_has_an_invalidate_hook():
+    """Scale / offset are cached while no gradient can reach min / max.  Tracked writes (set_range, copy_) are seen
+    through the version counter; a write through .data is not and needs invalidate_encoding_cache()."""
+    from aimet_amd.quantization.affine import QuantizeDequantize
+
+    q = QuantizeDequantize((), qmin=0, qmax=255, symmetric=False)
+    q.set_range(torch.tensor(0.0), torch.tensor(255.0))
+    with torch.no_grad():
+        assert float(q.get_encodings().scale) == 1.0
+        q.set_range(None, torch.tensor(510.0))
+        assert float(q.get_encodings().scale) == 2.0
+        q.max.copy_(torch.tensor(1020.0))
+        assert float(q.get_encodings().scale) == 4.0
+        q.max.data.fill_(255.0)  # untracked
+        q.invalidate_encoding_cache()
+        assert float(q.get_encodings().scale) == 1.0
+    # with gradients enabled nothing is cached: the reference's behaviour
+    q.max.data.fill_(510.0)
+    assert float(q.get_encodings().scale) == 2.0
+
+
 def test_quantizer_construction_and_bookkeeping_on_cpu():
     from aimet_amd.quantization.affine import QuantizeDequantize, GroupedBlockQuantizeDequantize, Quantize
 

@@ -64,6 +64,47 @@ def test_histogram_stream_single_slot(device, dtype, num_bins, growth):
         _check_hist_lists(obs.get_stats(), ref.stats, f"running statistics after batch {k}")
 
 
+def _range_whose_last_edge_rounds(num_bins, below: bool, seed):
+    """(lo, hi) in float32 such that the last bin edge B * RN((hi - lo) / B) + lo lies below (or above) hi."""
+    g = torch.Generator().manual_seed(seed)
+    for _ in range(10000):
+        lo = (torch.rand((), generator=g) * 4 - 3).float()
+        hi = (lo + torch.rand((), generator=g) * 5 + 0.5).float()
+        last = torch.tensor(float(num_bins)) * ((hi - lo) / num_bins) + lo
+        if (below and last < hi) or (not below and last > hi):
+            return lo, hi
+    raise AssertionError("no such range found")
+
+
+@pytest.mark.parametrize("num_bins", [512, 10, 100])
+@pytest.mark.parametrize("below", [True, False], ids=["last_edge_below_max", "last_edge_above_max"])
+def test_histogram_repeated_batches_and_maxima_at_the_running_maximum(device, num_bins, below):
+    """The reference clamps a batch's maximum with the last bin EDGE, which rounding can put below or above the running
+    maximum (encoding_analyzer.py:266-270).  Seeing the same tensor again, a batch whose maximum equals the running
+    maximum, and one whose maximum lies between the last edge and the running maximum must all leave the running
+    statistics as the reference has them."""
+    from aimet_amd.quantization.encoding_analyzer import _HistogramObserver
+
+    lo, hi = _range_whose_last_edge_rounds(num_bins, below, seed=num_bins)
+    g = torch.Generator().manual_seed(3)
+    n = 3 * 4099
+    base = torch.rand(n, generator=g) * (hi - lo) + lo
+    base = base.clamp(lo, hi)
+    base[17], base[n - 5] = lo, hi
+    inside = torch.rand(n, generator=g) * (hi - lo) * 0.5 + lo
+    at_max = inside.clone()
+    at_max[n // 2] = hi
+    just_below = inside.clone()
+    just_below[7] = torch.nextafter(hi, lo)  # between the last edge and the maximum when the edge rounds further down
+    batches = [base, base, at_max, just_below, inside, base * 1.25, base * 1.25, at_max]
+    obs = _HistogramObserver((1,), num_bins=num_bins)
+    ref = O.HistObserver((1,), num_bins, None)
+    for k, b in enumerate(batches):
+        ref.update(b)
+        obs.update(b.to(device))
+        _check_hist_lists(obs.get_stats(), ref.stats, f"running statistics after batch {k}")
+
+
 @pytest.mark.parametrize("case", [((4, 1), None, (4, 300)), ((2, 3), (2, 5), (4, 15)), ((3, 1, 1), None, (2, 3, 5, 7)),
                                   ((4, 1), None, (4, 5000)), ((3, 1, 1), None, (2, 3, 64, 64)), ((2, 2), (3, 2048), (6, 4096))],
                          ids=["per_channel", "blockwise", "activation_channels", "long_rows_ragged_tiles",
