@@ -110,6 +110,7 @@ _SIGNATURES = {
                                   ctypes.c_size_t, _P]),
     "ahq_minmax_copy": (ctypes.c_int, [ctypes.c_int32, ctypes.POINTER(Layout), _P, _P, _P, _P, _P, _P, ctypes.c_int, _P,
                                        ctypes.c_size_t, _P]),
+    "ahq_minmax_static": (ctypes.c_int, [ctypes.c_int32, ctypes.POINTER(Layout), _P, _P, _P, _P, _P, ctypes.c_int, _P]),
     "ahq_minmax_to_encodings": (ctypes.c_int, [ctypes.c_int32, _P, _P, ctypes.c_int64, ctypes.c_int64, ctypes.c_int32,
                                                ctypes.c_float, ctypes.c_float, ctypes.c_float, ctypes.c_float, _P, _P, _P,
                                                _P]),

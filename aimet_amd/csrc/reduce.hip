@@ -5,10 +5,18 @@
 // NaN handling follows torch.amin/amax (any NaN in a slice makes that slice's result NaN) unless `finite_only`, which
 // reproduces the histogram observer's range (non-finite values ignored).
 
+#include <mutex>
+
 #include "ahq_device.h"
 #include "ahq_host.h"
 #include "layout.h"
 #include "tiling.h"
+
+// Scratch of ahq_minmax_static: partial extrema or per-encoding keys of one reduction.  Every device the library
+// runs on holds its own copy of this array until the process ends.  In host code the name is only a handle for
+// hipGetSymbolAddress; the address the kernels receive is looked up once per device (static_scratch below).
+constexpr size_t kStaticScratchBytes = AHQ_MINMAX_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
 namespace ahq {
 
@@ -527,4 +535,55 @@ extern "C" int ahq_minmax_copy(int32_t dtype, const ahq_layout* layout, const vo
     if (y == x) return set_error("y must not alias x"), AHQ_ERR_INVALID;
     return minmax_impl(dtype, layout, x, y, out_min, out_max, run_min, run_max, finite_only, workspace, workspace_bytes,
                        stream);
+}
+
+// ------------------------------------------------------------------------------------ entry point without allocation --
+namespace {
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {nullptr};  // device address of `scratch` on each device, looked up on first use
+
+// Address of the current device's copy of `scratch`.
+int static_scratch(void** out) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
+        return set_error("ahq_minmax_static: cannot identify the current device"), AHQ_ERR_LAUNCH;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) {
+            std::snprintf(error_buffer(), 512, "ahq_minmax_static: hipGetSymbolAddress failed: %s", hipGetErrorString(e));
+            return AHQ_ERR_LAUNCH;
+        }
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return AHQ_OK;
+}
+
+}  // namespace
+
+extern "C" int ahq_minmax_static(int32_t dtype, const ahq_layout* layout, const void* x, void* out_min, void* out_max,
+                                 void* run_min, void* run_max, int finite_only, void* stream) {
+    if (dtype < AHQ_F32 || dtype > AHQ_BF16) return set_error("bad dtype"), AHQ_ERR_INVALID;
+    if (!layout) return set_error("layout is null"), AHQ_ERR_INVALID;
+    // the size check comes first and needs no device: the plan is host arithmetic
+    Plan p;
+    if (!make_plan(dtype, *layout, aligned16(x), true, &p)) return AHQ_ERR_INVALID;
+    const size_t need = p.ws_elems * 12;
+    if (need > kStaticScratchBytes) {
+        std::snprintf(error_buffer(), 512,
+                      "ahq_minmax_static: this reduction needs %zu bytes of scratch, the static buffer holds %zu; "
+                      "use ahq_minmax with a caller-provided workspace",
+                      need, kStaticScratchBytes);
+        return AHQ_ERR_WORKSPACE;
+    }
+    if (!x || !out_min || !out_max) return set_error("x, out_min or out_max is null"), AHQ_ERR_INVALID;
+    void* ws = nullptr;
+    const int rc = static_scratch(&ws);
+    if (rc != AHQ_OK) return rc;
+    return minmax_impl(dtype, layout, x, nullptr, out_min, out_max, run_min, run_max, finite_only, ws,
+                       kStaticScratchBytes, stream);
 }

@@ -134,6 +134,21 @@ int    ahq_minmax_copy(int32_t dtype, const ahq_layout* layout, const void* x, v
                        void* run_min, void* run_max, int finite_only, void* workspace, size_t workspace_bytes,
                        void* stream);
 
+/* ahq_minmax for callers that cannot allocate device memory and have no workspace to pass: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference.  Same arguments and
+ * results as ahq_minmax without the workspace pair: the partial extrema / per-encoding keys go to a file-scope
+ * device array of AHQ_MINMAX_STATIC_SCRATCH_BYTES that every device the library runs on holds until the process ends.
+ * The call allocates nothing (no hipMalloc / hipFree, no allocating library routine); the first call on a device
+ * looks the array's address up (hipGetSymbolAddress), so make that call outside a capture.
+ * A reduction whose ahq_minmax_workspace_bytes() exceeds the array returns AHQ_ERR_WORKSPACE and launches nothing
+ * (12 bytes per 4096-element tile of a per-tensor reduction, 12 bytes per encoding otherwise).
+ * All calls on one device share the array: calls that overlap on one device (different streams) race; calls on one
+ * stream are ordered and each clears what it needs.
+ */
+#define AHQ_MINMAX_STATIC_SCRATCH_BYTES (1u << 20)
+int    ahq_minmax_static(int32_t dtype, const ahq_layout* layout, const void* x, void* out_min, void* out_max,
+                         void* run_min, void* run_max, int finite_only, void* stream);
+
 /* Replaces MinMaxEncodingAnalyzer.compute_encodings_from_stats (AT/quantization/encoding_analyzer.py:425-481) and the
  * checks of _flag_extreme_min_max (:484-498): zero forced into the range, ranges narrower than the minimum scale
  * widened, symmetric grids re-centred, the result clamped to the statistics dtype.  stat_min / stat_max / out_min /

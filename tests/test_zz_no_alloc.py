@@ -1,0 +1,102 @@
+"""ahq_minmax_static, the entry point that allocates nothing (its scratch is a file-scope device array), against
+ahq_minmax with a caller-provided workspace: identical results, bit for bit, through the C ABI, on two calls in a row
+of which the second is smaller (the shared scratch keeps the first call's contents)."""
+
+import ctypes
+
+import pytest
+import torch
+
+from aimet_amd import _lib
+from aimet_amd.quantization.affine.backends.hip import _prepare
+from tests.helpers import assert_same_bits
+
+SCRATCH_BYTES = 1 << 20  # AHQ_MINMAX_STATIC_SCRATCH_BYTES
+
+
+def _both(lib, x, shape, block, finite_only, running=None):
+    """(min, max) from ahq_minmax and from ahq_minmax_static on the same tensor."""
+    xd, layout = _prepare(x, shape, block)
+    code = _lib.DTYPE_CODE[x.dtype]
+    stream = _lib.current_stream(x.device)
+    out = []
+    for static in (False, True):
+        mn = torch.full(shape, 123.0, dtype=x.dtype, device=x.device)
+        mx = torch.full(shape, -123.0, dtype=x.dtype, device=x.device)
+        run = None if running is None else [r.clone() for r in running]
+        rp = (None, None) if run is None else (run[0].data_ptr(), run[1].data_ptr())
+        if static:
+            rc = lib.ahq_minmax_static(code, layout, xd.data_ptr(), mn.data_ptr(), mx.data_ptr(), rp[0], rp[1],
+                                       finite_only, stream)
+            _lib.check(rc, "ahq_minmax_static")
+        else:
+            nbytes = lib.ahq_minmax_workspace_bytes(layout)
+            ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=x.device)
+            rc = lib.ahq_minmax(code, layout, xd.data_ptr(), mn.data_ptr(), mx.data_ptr(), rp[0], rp[1], finite_only,
+                                ws.data_ptr(), nbytes, stream)
+            _lib.check(rc, "ahq_minmax")
+        out.append((mn, mx, run))
+    torch.cuda.synchronize()
+    return out
+
+
+CASES = [
+    # (first tensor shape, second (smaller) tensor shape, encoding shape of each, block size)
+    ("per_tensor", (64, 33000), (7, 4100), (), (), None),              # partials of 516 tiles, then of 8
+    ("per_channel_rows", (48, 9000), (16, 5000), (48, 1), (16, 1), None),  # one partial per tile of each row
+    ("per_channel_short_rows", (300, 100), (40, 100), (300, 1), (40, 1), None),  # ordered keys + atomics
+    ("blockwise", (64, 1024), (8, 256), (64, 16), (8, 4), (1, 64)),     # shuffle reduction, no scratch at all
+    ("columns", (700, 512), (90, 256), (512,), (256,), None),           # column walk: keys per encoding
+]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=lambda d: str(d).split(".")[-1])
+@pytest.mark.parametrize("case", CASES, ids=lambda c: c[0])
+@pytest.mark.parametrize("finite_only", [0, 1])
+def test_static_scratch_matches_the_workspace_entry_point(device, dtype, case, finite_only):
+    _, big, small, big_enc, small_enc, block = case
+    lib = _lib.load()
+    g = torch.Generator().manual_seed(9)
+    for k, (shape, enc) in enumerate(((big, big_enc), (small, small_enc))):
+        x = (torch.randn(shape, generator=g) * (3.0 - k)).to(dtype)
+        flat = x.view(-1)
+        flat[3], flat[-2] = float("inf"), float("-inf")
+        if finite_only == 0 and k == 1:
+            flat[11] = float("nan")
+        xd = x.to(device)
+        (mn, mx, _), (smn, smx, _) = _both(lib, xd, enc, block, finite_only)
+        assert_same_bits(smn, mn, f"call {k}: minimum")
+        assert_same_bits(smx, mx, f"call {k}: maximum")
+        # and both agree with torch on the finite part (the entry point it mirrors is itself tested against the oracle)
+        if finite_only == 1 and enc == ():
+            fin = x[x.isfinite()]
+            assert smn.item() == fin.min().item() and smx.item() == fin.max().item()
+
+
+@pytest.mark.gpu
+def test_static_scratch_folds_running_statistics(device):
+    lib = _lib.load()
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(32, 70000, generator=g).to(device)
+    running = (torch.full((), -0.5, device=device), torch.full((), 9.0, device=device))
+    (mn, mx, run), (smn, smx, srun) = _both(lib, x, (), None, 0, running)
+    assert_same_bits(smn, mn, "minimum")
+    assert_same_bits(smx, mx, "maximum")
+    assert_same_bits(srun[0], run[0], "running minimum")
+    assert_same_bits(srun[1], run[1], "running maximum")
+    assert srun[1].item() == 9.0 and srun[0].item() == x.min().item()
+
+
+def test_static_scratch_rejects_reductions_beyond_its_size():
+    """Host-side check, no GPU needed: the plan is pure arithmetic and the refusal comes before any HIP call."""
+    lib = _lib.load()
+    n = (SCRATCH_BYTES // 12 + 1) * 4096  # one tile more than the scratch has partials for
+    lay = _lib.make_layout([n], [n], [0])
+    assert lib.ahq_minmax_workspace_bytes(lay) > SCRATCH_BYTES
+    rc = lib.ahq_minmax_static(_lib.AHQ_F32, lay, 16, 16, 16, None, None, 0, None)
+    assert rc == _lib.AHQ_ERR_WORKSPACE
+    assert b"static buffer" in lib.ahq_last_error()
+    enc = SCRATCH_BYTES // 12 + 1
+    lay = _lib.make_layout([enc, 40], [1, 40], [1, 0])  # per-channel with short rows: 12 bytes per encoding
+    assert lib.ahq_minmax_static(_lib.AHQ_F32, lay, 16, 16, 16, None, None, 0, None) == _lib.AHQ_ERR_WORKSPACE
