@@ -109,6 +109,59 @@ __global__ void range_to_scale_offset_kernel(const ScaleOffArgs a) {
     }
 }
 
+// ------------------------------------------------------------------------------- LPBQ: grouped block scales --
+// GroupedBlockQuantizeDequantize._get_scale / _get_per_channel_scale (aimet_torch/quantization/affine/quantizer.py:
+// 1363-1399) for a quantizer that holds min / max, dtype = float32:
+//   raw         = clamp_min(|float(max) - float(min)| / num_steps, minimum_scale)            per block
+//   per_channel = amax(raw over the group) / multipliers                                      per group
+//   scale       = clamp(round(raw / per_channel), 1, multipliers) * per_channel               per block
+// (the last line is quantize_dequantize(raw, per_channel, 0, 1, multipliers) in float32: true division, round half
+// to even).  One wave per group of neighbouring blocks; the group is read twice (it is a few hundred bytes).
+struct LpbqArgs {
+    const void* pmin;
+    const void* pmax;
+    float* scale;
+    float* per_channel;
+    int64_t groups, group_size;
+    float num_steps, minimum_scale, multipliers;
+};
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void lpbq_scale_kernel(const LpbqArgs a) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t waves = (int64_t)gridDim.x * (kBlock / kWave);
+    const T* __restrict__ pmin = static_cast<const T*>(a.pmin);
+    const T* __restrict__ pmax = static_cast<const T*>(a.pmax);
+    auto raw_at = [&](int64_t i) {
+        const float s = __builtin_fabsf((load_f32(pmax[i]) - load_f32(pmin[i])) / a.num_steps);
+        return (s != s) ? s : fmaxf(s, a.minimum_scale);
+    };
+    for (int64_t g = (int64_t)blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave; g < a.groups; g += waves) {
+        const int64_t base = g * a.group_size;
+        float largest = -__builtin_inff();
+        int nan = 0;
+        for (int64_t k = lane; k < a.group_size; k += kWave) {
+            const float s = raw_at(base + k);
+            nan |= (s != s) ? 1 : 0;
+            largest = fmaxf(largest, s);
+        }
+#pragma unroll
+        for (int m = kWave / 2; m >= 1; m >>= 1) {
+            largest = fmaxf(largest, __shfl_xor(largest, m, kWave));
+            nan |= __shfl_xor(nan, m, kWave);
+        }
+        if (nan) largest = __builtin_nanf("");  // torch.amax propagates NaN
+        const float pc = largest / a.multipliers;
+        if (lane == 0) a.per_channel[g] = pc;
+        for (int64_t k = lane; k < a.group_size; k += kWave) {
+            const float s = raw_at(base + k);
+            const float r = __builtin_rintf(s / pc);
+            const float q = (r != r) ? r : fminf(fmaxf(r, 1.0f), a.multipliers);
+            a.scale[base + k] = q * pc;
+        }
+    }
+}
+
 // --------------------------------------------------------------------- "is this tensor already on a grid" test --
 // The early exit of _decompose_prequantized_tensor (aimet_torch/utils.py:2098-2118), which runs on every weight at
 // the start of a calibration: of the first 64 blocks take the first 2 * num_levels elements each, as float
@@ -253,6 +306,42 @@ extern "C" int ahq_range_to_scale_offset(int32_t dtype, const void* range_min, c
         default: hipLaunchKernelGGL((range_to_scale_offset_kernel<bf16_t>), g, b, 0, s, a); break;
     }
     return check_launch("range_to_scale_offset");
+}
+
+extern "C" int ahq_lpbq_scale(int32_t dtype, const ahq_layout* grouping, const void* range_min, const void* range_max,
+                              int64_t qmin, int64_t qmax, double minimum_scale, int32_t num_multipliers, float* scale,
+                              float* per_channel_scale, void* stream) {
+    if (dtype < AHQ_F32 || dtype > AHQ_BF16) return set_error("bad dtype"), AHQ_ERR_INVALID;
+    if (!grouping || !range_min || !range_max || !scale || !per_channel_scale) return set_error("null argument"), AHQ_ERR_INVALID;
+    if (qmin >= qmax) return set_error("qmax must be larger than qmin"), AHQ_ERR_INVALID;
+    if (num_multipliers < 1 || num_multipliers > (1 << 24)) return set_error("num_multipliers must be in 1..2^24"), AHQ_ERR_INVALID;
+    CanonLayout c;
+    const char* err = nullptr;
+    if (!canonicalize(*grouping, &c, &err)) return set_error(err), AHQ_ERR_INVALID;
+    if (c.numel == 0) return AHQ_OK;
+    if (c.kind != kIJK || c.I != 1)
+        return set_error("groups whose blocks are not neighbours in memory are not supported by the fused LPBQ scale"), AHQ_ERR_UNSUPPORTED;
+    LpbqArgs a{};
+    a.pmin = range_min;
+    a.pmax = range_max;
+    a.scale = scale;
+    a.per_channel = per_channel_scale;
+    a.groups = c.J;
+    a.group_size = c.K;
+    a.num_steps = (float)(double)(qmax - qmin);
+    a.minimum_scale = (float)minimum_scale;
+    a.multipliers = (float)num_multipliers;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int64_t per_block = kBlock / kWave;
+    int64_t nb = (c.J + per_block - 1) / per_block;
+    if (nb > 65536) nb = 65536;
+    const dim3 g((unsigned)nb), b(kBlock);
+    switch (dtype) {
+        case AHQ_F32: hipLaunchKernelGGL((lpbq_scale_kernel<float>), g, b, 0, s, a); break;
+        case AHQ_F16: hipLaunchKernelGGL((lpbq_scale_kernel<f16_t>), g, b, 0, s, a); break;
+        default: hipLaunchKernelGGL((lpbq_scale_kernel<bf16_t>), g, b, 0, s, a); break;
+    }
+    return check_launch("lpbq_scale");
 }
 
 extern "C" int ahq_minmax_to_encodings(int32_t dtype, const void* stat_min, const void* stat_max, int64_t num_encodings,

@@ -31,6 +31,7 @@ from aimet_amd.quantization._utils import (
 )
 from aimet_amd.quantization.affine._utils import _GridMixin
 from aimet_amd.quantization.affine.backends import quantize, quantize_dequantize, dequantize, _derive_qmin_qmax
+from aimet_amd.quantization.affine.backends.hip import _build_layout
 from aimet_amd.quantization.affine.encoding import AffineEncoding, GroupedBlockEncoding
 from aimet_amd.quantization.base.quantizer import QuantizerBase
 from aimet_amd.quantization.encoding_analyzer import EncodingAnalyzer, MinMaxEncodingAnalyzer, _flag_extreme_min_max
@@ -529,7 +530,37 @@ class GroupedBlockQuantizeDequantize(QuantizeDequantize):
         raw = super().get_scale(dtype)
         return None if raw is None else self._get_per_channel_scale(raw)
 
+    def _fused_lpbq_scale(self):
+        """(scale, per-channel scale) in float32 from one launch of ahq_lpbq_scale; None when that does not apply
+        (gradients wanted, parameters not on a GPU, groups that are not runs of neighbouring blocks) and the
+        step-by-step form has to run."""
+        mn, mx = self.min, self.max
+        if torch.is_grad_enabled() and (mn.requires_grad or mx.requires_grad):
+            return None
+        if not (mn.is_cuda and mx.device == mn.device and mn.dtype == mx.dtype and mn.dtype in _lib.DTYPE_CODE
+                and mn.shape == mx.shape and mn.is_contiguous() and mx.is_contiguous() and mn.numel() > 0):
+            return None
+        if type(self).get_scale is not GroupedBlockQuantizeDequantize.get_scale:
+            return None
+        shape = tuple(mn.shape)
+        group_shape = tuple(d // g if g != -1 else 1 for d, g in zip(shape, self.block_grouping))
+        layout = _build_layout(shape, tuple(range(len(shape))), group_shape, tuple(self.block_grouping))
+        lib = _lib.load()
+        scale = torch.empty(shape, dtype=torch.float32, device=mn.device)
+        per_channel = torch.empty(group_shape, dtype=torch.float32, device=mn.device)
+        status = lib.ahq_lpbq_scale(_lib.DTYPE_CODE[mn.dtype], layout, mn.data_ptr(), mx.data_ptr(), self.qmin, self.qmax,
+                                    _get_minimum_scale(self.qmax - self.qmin), 2 ** (self.decompressed_bw - self.bitwidth),
+                                    scale.data_ptr(), per_channel.data_ptr(), _lib.current_stream(mn.device))
+        if status == _lib.AHQ_ERR_UNSUPPORTED:
+            return None
+        _lib.check(status, "ahq_lpbq_scale")
+        return scale, per_channel
+
     def _get_scale(self, dtype=None):
+        if dtype in (None, torch.float32) and self.is_initialized():
+            fused = self._fused_lpbq_scale()
+            if fused is not None:
+                return fused
         raw = super().get_scale(dtype)
         if raw is None:
             return None, None

@@ -1,21 +1,30 @@
 #!/usr/bin/env python3
 """Benchmark of the fake-quant hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload all|c1|c2|c3|c4|c5|dlq]
 
-Default workload ("c2"): per-output-channel 8-bit symmetric weight quantize-dequantize forward + straight-through
-backward (input, scale and offset gradients) on an fp32 [4096, 4096] weight.  A step is one forward plus one backward
-launched through the C ABI on tensors already resident in HBM.  Prints ONE JSON line.
+Without --workload every workload runs in this one process and ONE JSON line is printed.  Its top-level fields are
+those of c4 (blockwise 4-bit LPBQ quantize-dequantize forward + straight-through backward of a bf16 [14336, 4096]
+weight, the largest forward+backward configuration and the only one whose working set exceeds the 256 MB last-level
+cache); `configs` holds the records of c1, c2, c3, c5 and dlq (DlQuantization's TF-enhanced stream) in the same form.
 
-`value` = algorithmic bytes per step (5 * sizeof(dtype) per element: forward reads x and writes y, backward reads g
-and x and writes gx) divided by the wall time per step, in GB/s.
+A step is one pass of a workload's hot path through the C ABI on tensors already resident in HBM (c4: LPBQ scale
+derivation + forward + backward).  The K-step loop is bracketed by device synchronisation and repeated at least seven
+times (more until 10 ms have been timed); `ms_per_step` is the median loop divided by K.  `value` = algorithmic bytes
+per step / time per step.  Per record: `roofline` for the dominant kernel (HIP events on the launch stream),
+`calibration` (min/max statistics of the same tensor), `module_path` (the same step through the drop-in quantizer
+module and autograd, allocations included), `cpu_baseline` / `cpu_baseline_1thread` (the CPU oracle, i.e. the
+reference's own sequence of torch CPU calls or scalar C loops, on this host) and `parity` against that oracle.
 """
 
 from __future__ import annotations
 
 import argparse
+import gc
 import json
+import math
 import os
+import statistics
 import sys
 import time
 
@@ -25,8 +34,11 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
+METRIC = "QDQ fwd+bwd GB/s (% of HBM peak); calibration elems/s; vs host-CPU ref"
 HBM_PEAK_GBS = 8000.0
 COPY_REF_ELEMS = 1 << 26
+MIN_REPEATS = 7
+MIN_TIMED_SECONDS = 0.010
 # HBM bytes per launch of each workload's dominant kernel(s): rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE averages per
 # dispatch, scaled by what the same counters read for _copy_reference() (x2.000 for FETCH_SIZE, x1.000 for WRITE_SIZE);
 # the counter summary is profiles/hbm_traffic_pmc__qdq_c1_c2_c4__hist_c3__dlq.txt.  None where no counter run has been
@@ -43,6 +55,7 @@ MEASURED_TRAFFIC_BYTES = {
     ("c3", "hist_update"): int((262327.2 + 3216.2 + 3650.0 + 127.2 + 168.6 + 139.4) * 1024),
     ("dlq", "pdf_update"): int((262350.0 + 3072.0 + 6182.0) * 1024),
 }
+DTYPE_NAME = {torch.float32: "f32", torch.bfloat16: "bf16", torch.float16: "f16"}
 
 
 def _ensure_built():
@@ -55,50 +68,85 @@ def _ensure_built():
     return _lib.load()
 
 
-# ----------------------------------------------------------------------------------------------------- workloads --
-def _make_c1(dev):
-    g = torch.Generator().manual_seed(0)
-    x = torch.relu(torch.randn(32, 64, 112, 112, generator=g))
-    g1 = torch.Generator().manual_seed(1)
-    grad = torch.randn(x.shape, generator=g1)
-    return dict(name="c1_per_tensor_8b_asym_fp32_32x64x112x112", x=x, grad=grad, enc_shape=(), block=None,
-                bitwidth=8, symmetric=False)
+# -------------------------------------------------------------------------------------------------------- timing --
+def _sync():
+    torch.cuda.synchronize()
 
 
-def _make_c2(dev):
-    g = torch.Generator().manual_seed(0)
-    w = torch.randn(4096, 4096, generator=g) * 0.02
-    rows = torch.randperm(4096, generator=torch.Generator().manual_seed(1))[:41]
-    w[rows] *= 10
-    grad = torch.randn(4096, 4096, generator=torch.Generator().manual_seed(2)) * 1e-3
-    return dict(name="c2_per_channel_8b_sym_fp32_4096x4096", x=w, grad=grad, enc_shape=(4096, 1), block=None,
-                bitwidth=8, symmetric=True)
+def timed_steps(step, steps, warmup, min_repeats=MIN_REPEATS, min_total=MIN_TIMED_SECONDS, max_repeats=400):
+    """Median wall time of a loop of exactly ``steps`` steps, each loop bracketed by a device synchronisation.
+    Returns (seconds per loop, repeats)."""
+    for _ in range(warmup):
+        step()
+    _sync()
+    loops = []
+    total = 0.0
+    while len(loops) < min_repeats or (total < min_total and len(loops) < max_repeats):
+        _sync()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step()
+        _sync()
+        dt = time.perf_counter() - t0
+        loops.append(dt)
+        total += dt
+    return statistics.median(loops), len(loops)
 
 
-def _make_c4(dev):
-    g = torch.Generator().manual_seed(0)
-    w = (torch.randn(14336, 4096, generator=g) * 0.02).bfloat16()
-    grad = torch.randn(14336, 4096, generator=torch.Generator().manual_seed(1)).bfloat16()
-    return dict(name="c4_blockwise64_4b_sym_bf16_14336x4096", x=w, grad=grad, enc_shape=(14336, 64), block=(1, 64),
-                bitwidth=4, symmetric=True)
+def event_time(fn, reps, repeats=MIN_REPEATS):
+    """Median over ``repeats`` of the average duration of ``fn`` over ``reps`` back-to-back calls, from HIP events
+    recorded on the stream the work is launched on (torch's current stream)."""
+    fn()
+    _sync()
+    out = []
+    for _ in range(repeats):
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        _sync()
+        out.append(e0.elapsed_time(e1) / reps * 1e-3)
+    return statistics.median(out)
 
 
-WORKLOADS = {"c1": _make_c1, "c2": _make_c2, "c4": _make_c4}
+def cpu_legs(step, unit_per_step, unit, sample, budget_s=4.0, max_reps=20, one_thread_budget_s=4.0):
+    """The CPU oracle timed on this host with torch's default thread count and with one thread.
+    ``unit_per_step``: bytes (-> GB/s) or elements (-> elements/s) one call of ``step`` stands for."""
 
+    def leg(budget):
+        step()
+        t0 = time.perf_counter()
+        reps = 0
+        while True:
+            step()
+            reps += 1
+            if time.perf_counter() - t0 > budget or reps >= max_reps:
+                break
+        return (time.perf_counter() - t0) / reps, reps
 
-def _encodings_cpu(w):
-    """Min/max calibration + scale/offset derivation on the CPU oracle (same arithmetic as the product path)."""
-    from oracle import torch_ref as O
+    def record(dt, reps, cores):
+        scale = 1e9 if unit == "GB/s" else 1.0
+        return {"value": round(unit_per_step / dt / scale, 3), "unit": unit, "cores": cores, "kind": "port",
+                "sample": f"{reps} x {sample} ({dt * 1e3:.1f} ms each)"}
 
-    import math
-
-    n = 2 ** w["bitwidth"] - 1
-    qmin, qmax = (-math.ceil(n / 2), math.floor(n / 2)) if w["symmetric"] else (0, n)
-    mn, mx = O.reduce_minmax(w["x"], w["enc_shape"], w["block"])
-    emin, emax = O.minmax_encodings(mn, mx, n, w["symmetric"])
-    scale = O.scale_from_minmax(emin, emax, qmin, qmax)
-    offset = O.offset_from_minmax(emin.float(), scale, qmin, qmax, w["symmetric"])
-    return scale, offset, qmin, qmax
+    threads = torch.get_num_threads()
+    dt, reps = leg(budget_s)
+    all_cores = record(dt, reps, threads)
+    torch.set_num_threads(1)
+    try:
+        t0 = time.perf_counter()
+        step()
+        first = time.perf_counter() - t0
+        if first > one_thread_budget_s:
+            one = record(first, 1, 1)
+        else:
+            dt1, reps1 = leg(one_thread_budget_s)
+            one = record(dt1, reps1, 1)
+    finally:
+        torch.set_num_threads(threads)
+    return all_cores, one
 
 
 def _copy_reference(dev):
@@ -107,22 +155,131 @@ def _copy_reference(dev):
     src = torch.ones(COPY_REF_ELEMS, dtype=torch.float32, device=dev)
     dst = torch.empty_like(src)
     torch.mul(src, 1.0, out=dst)
-    torch.cuda.synchronize()
+    _sync()
+
+
+def _base_record(value_gbs, steps, warmup, sec_per_step, dtype, config, repeats):
+    return {
+        "metric": METRIC,
+        "value": round(value_gbs, 2),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": steps,
+        "warmup": warmup,
+        "ms_per_step": round(sec_per_step * 1e3, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": dtype,
+        "data": "synthetic",
+        "config": config,
+        "repeats": repeats,
+        "timing": f"median of {repeats} loops of {steps} steps, each loop bracketed by device synchronisation",
+        "pct_of_hbm_peak": round(100.0 * value_gbs / HBM_PEAK_GBS, 2),
+    }
+
+
+# ----------------------------------------------------------------------------------------------------- workloads --
+def _make_c1():
+    g = torch.Generator().manual_seed(0)
+    x = torch.relu(torch.randn(32, 64, 112, 112, generator=g))
+    g1 = torch.Generator().manual_seed(1)
+    grad = torch.randn(x.shape, generator=g1)
+    return dict(name="c1_per_tensor_8b_asym_fp32_32x64x112x112", x=x, grad=grad, enc_shape=(), block=None,
+                bitwidth=8, symmetric=False, lpbq=False)
+
+
+def _make_c2():
+    g = torch.Generator().manual_seed(0)
+    w = torch.randn(4096, 4096, generator=g) * 0.02
+    rows = torch.randperm(4096, generator=torch.Generator().manual_seed(1))[:41]
+    w[rows] *= 10
+    grad = torch.randn(4096, 4096, generator=torch.Generator().manual_seed(2)) * 1e-3
+    return dict(name="c2_per_channel_8b_sym_fp32_4096x4096", x=w, grad=grad, enc_shape=(4096, 1), block=None,
+                bitwidth=8, symmetric=True, lpbq=False)
+
+
+def _make_c4():
+    g = torch.Generator().manual_seed(0)
+    w = (torch.randn(14336, 4096, generator=g) * 0.02).bfloat16()
+    grad = torch.randn(14336, 4096, generator=torch.Generator().manual_seed(1)).bfloat16()
+    return dict(name="c4_lpbq_blockwise64_4b_sym_bf16_14336x4096", x=w, grad=grad, enc_shape=(14336, 64), block=(1, 64),
+                bitwidth=4, symmetric=True, lpbq=True, decompressed_bw=8, grouping=(1, -1))
+
+
+WORKLOADS = {"c1": _make_c1, "c2": _make_c2, "c4": _make_c4}
+
+
+def _grid_limits(w):
+    n = 2 ** w["bitwidth"] - 1
+    return (-math.ceil(n / 2), math.floor(n / 2), n) if w["symmetric"] else (0, n, n)
+
+
+def _range_cpu(w):
+    """Min/max statistics and the encoding range on the CPU oracle."""
+    from oracle import torch_ref as O
+
+    _, _, n = _grid_limits(w)
+    mn, mx = O.reduce_minmax(w["x"], w["enc_shape"], w["block"])
+    emin, emax = O.minmax_encodings(mn, mx, n, w["symmetric"])
+    return mn, mx, emin.float(), emax.float()  # the quantizer's min / max parameters are float32
+
+
+def _scale_offset_cpu(w, emin, emax):
+    """Scale and offset from the encoding range, through the LPBQ requantisation where the workload asks for it."""
+    from oracle import torch_ref as O
+
+    qmin, qmax, _ = _grid_limits(w)
+    scale = O.scale_from_minmax(emin, emax, qmin, qmax)
+    pcs = None
+    if w["lpbq"]:
+        scale, pcs = O.lpbq_scale(scale, w["bitwidth"], w["decompressed_bw"], w["grouping"])
+    offset = O.offset_from_minmax(emin, scale, qmin, qmax, w["symmetric"])
+    return scale, offset, pcs
+
+
+def _make_module(w, dev):
+    from aimet_amd.quantization.affine import GroupedBlockQuantizeDequantize, QuantizeDequantize
+
+    if w["lpbq"]:
+        q = GroupedBlockQuantizeDequantize(shape=w["enc_shape"], bitwidth=w["bitwidth"], symmetric=True,
+                                           decompressed_bw=w["decompressed_bw"], block_size=w["block"],
+                                           block_grouping=w["grouping"])
+    else:
+        q = QuantizeDequantize(w["enc_shape"], w["bitwidth"], w["symmetric"], block_size=w["block"])
+    return q.to(dev)
 
 
 def run_qdq_workload(key, steps, warmup, dev, with_cpu_baseline=True):
     from aimet_amd import _lib
+    from aimet_amd.quantization._utils import _get_minimum_scale
     from aimet_amd.quantization.affine.backends import hip
     from oracle import torch_ref as O
 
     lib = _ensure_built()
     _copy_reference(dev)
-    w = WORKLOADS[key](dev)
-    scale_c, offset_c, qmin, qmax = _encodings_cpu(w)
+    t_start = time.perf_counter()
+    w = WORKLOADS[key]()
+    qmin, qmax, _ = _grid_limits(w)
     x = w["x"].to(dev)
     grad = w["grad"].to(dev)
-    scale = scale_c.to(dev).contiguous()
-    offset = offset_c.to(dev).contiguous()
+    stream = _lib.current_stream(dev)
+    code = _lib.DTYPE_CODE[x.dtype]
+
+    # ---- calibration through the drop-in module: min/max statistics -> range, as compute_encodings() does
+    q = _make_module(w, dev)
+    with torch.no_grad(), q.compute_encodings():
+        q(x)
+    mn_ref, mx_ref, emin_c, emax_c = _range_cpu(w)
+    scale_c, offset_c, pcs_c = _scale_offset_cpu(w, emin_c, emax_c)
+    range_exact = bool(torch.equal(q.min.detach().cpu().view(emin_c.shape), emin_c)
+                       and torch.equal(q.max.detach().cpu().view(emax_c.shape), emax_c))
+    with torch.no_grad():
+        enc = q.get_encodings()
+    scale = enc.scale.detach().contiguous()
+    offset = enc.offset.detach().to(torch.float32).expand(scale.shape).contiguous()
+    scale_exact = bool(torch.equal(scale.cpu(), scale_c.view(scale.shape)))
+
     cd = hip._internal_dtype(x.dtype, qmin, qmax)
     grid = hip._grid(_lib.AHQ_ARITH_AUTOGRAD, _lib.AHQ_OP_QDQ, x.dtype, cd, qmin, qmax, 0.0)
     _, layout = hip._prepare(x, scale.shape, w["block"])
@@ -132,7 +289,6 @@ def run_qdq_workload(key, steps, warmup, dev, with_cpu_baseline=True):
     go = torch.empty_like(scale)
     nbytes = lib.ahq_qdq_backward_workspace_bytes(grid, layout, 1)
     ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=dev)
-    stream = _lib.current_stream(dev)
 
     def fwd():
         _lib.check(lib.ahq_qdq_forward(grid, layout, x.data_ptr(), y.data_ptr(), None, scale.data_ptr(),
@@ -143,122 +299,176 @@ def run_qdq_workload(key, steps, warmup, dev, with_cpu_baseline=True):
                                         go.data_ptr(), scale.data_ptr(), offset.data_ptr(), ws.data_ptr(), nbytes,
                                         stream), "bwd")
 
-    for _ in range(warmup):
-        fwd()
-        bwd()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        fwd()
-        bwd()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
+    derive = None
+    if w["lpbq"]:
+        # the reference derives the LPBQ scales from min / max on every forward (get_encodings()); so does the step
+        group_shape = tuple(d // g if g != -1 else 1 for d, g in zip(w["enc_shape"], w["grouping"]))
+        glayout = hip._build_layout(tuple(w["enc_shape"]), tuple(range(len(w["enc_shape"]))), group_shape,
+                                    tuple(w["grouping"]))
+        pmin, pmax = q.min.detach(), q.max.detach()
+        pcs = torch.empty(group_shape, dtype=torch.float32, device=dev)
+        mult = 2 ** (w["decompressed_bw"] - w["bitwidth"])
+        min_scale = _get_minimum_scale(qmax - qmin)
 
-    # per-kernel durations from events on the launch stream
-    def event_time(fn, reps):
-        e0 = torch.cuda.Event(enable_timing=True)
-        e1 = torch.cuda.Event(enable_timing=True)
-        fn()
-        torch.cuda.synchronize()
-        e0.record()
-        for _ in range(reps):
-            fn()
-        e1.record()
-        torch.cuda.synchronize()
-        return e0.elapsed_time(e1) / reps * 1e-3
+        def derive():
+            _lib.check(lib.ahq_lpbq_scale(_lib.DTYPE_CODE[pmin.dtype], glayout, pmin.data_ptr(), pmax.data_ptr(), qmin,
+                                          qmax, min_scale, mult, scale.data_ptr(), pcs.data_ptr(), stream), "lpbq")
+
+    def step():
+        if derive is not None:
+            derive()
+        fwd()
+        bwd()
+
+    loop_s, repeats = timed_steps(step, steps, warmup)
+    sec_per_step = loop_s / steps
 
     reps = max(steps, 20)
     t_fwd = event_time(fwd, reps)
     t_bwd = event_time(bwd, reps)
+    t_derive = event_time(derive, reps) if derive is not None else 0.0
 
-    # min/max calibration of the same tensor (one fused pass for both extrema)
+    n = x.numel()
+    S = x.element_size()
+    E = scale.numel()
+    bytes_fwd = 2 * S * n + 8 * E
+    bytes_bwd = 3 * S * n + 16 * E
+    bytes_derive = (12 * E + 4 * pcs.numel()) if derive is not None else 0
+    bytes_step = bytes_fwd + bytes_bwd + bytes_derive
+    value = bytes_step / sec_per_step / 1e9
+
+    # ---- frozen quantizer (no gradient for scale / offset): the ATen fake-quantize arithmetic, input gradient only
+    frozen = None
+    if w["block"] is None:
+        grid_a = hip._grid(_lib.AHQ_ARITH_ATEN, _lib.AHQ_OP_QDQ, x.dtype, torch.float32, qmin, qmax, 0.0)
+        nb_a = lib.ahq_qdq_backward_workspace_bytes(grid_a, layout, 0)
+        ws_a = torch.empty(max(nb_a, 16), dtype=torch.uint8, device=dev)
+        y_a = torch.empty_like(x)
+
+        def fwd_a():
+            _lib.check(lib.ahq_qdq_forward(grid_a, layout, x.data_ptr(), y_a.data_ptr(), None, scale.data_ptr(),
+                                           offset.data_ptr(), None, None, stream), "fwd aten")
+
+        def bwd_a():
+            _lib.check(lib.ahq_qdq_backward(grid_a, layout, grad.data_ptr(), x.data_ptr(), gx.data_ptr(), None, None,
+                                            scale.data_ptr(), offset.data_ptr(), ws_a.data_ptr(), nb_a, stream),
+                       "bwd aten")
+
+        ta_f, ta_b = event_time(fwd_a, reps), event_time(bwd_a, reps)
+        ref_a, mask_a = O.qdq_v1(w["x"], scale_c, offset_c, qmin, qmax)
+        frozen = {"arithmetic": "ATen fake-quantize (frozen scale / offset)",
+                  "fwd_us": round(ta_f * 1e6, 2), "bwd_us": round(ta_b * 1e6, 2),
+                  "GBps": round(5 * S * n / (ta_f + ta_b) / 1e9, 1),
+                  "y_bit_exact": bool(torch.equal(y_a.cpu(), ref_a)),
+                  "gx_bit_exact": bool(torch.equal(gx.cpu(), torch.where(mask_a, w["grad"], torch.zeros_like(w["grad"]))))}
+        bwd()  # gx of the autograd arithmetic again, for the parity check below
+
+    # ---- min/max calibration of the same tensor (one fused pass for both extrema) + the range it gives
     mm_ws_bytes = lib.ahq_minmax_workspace_bytes(layout)
     mm_ws = torch.empty(max(mm_ws_bytes, 16), dtype=torch.uint8, device=dev)
     mn_out = torch.empty(scale.shape, dtype=x.dtype, device=dev)
     mx_out = torch.empty(scale.shape, dtype=x.dtype, device=dev)
-    code = _lib.DTYPE_CODE[x.dtype]
 
     def minmax():
         _lib.check(lib.ahq_minmax(code, layout, x.data_ptr(), mn_out.data_ptr(), mx_out.data_ptr(), None, None, 0,
                                   mm_ws.data_ptr(), mm_ws_bytes, stream), "minmax")
 
+    an = q.encoding_analyzer
+
+    def calibrate():
+        an.reset_stats()
+        an.update_stats(x)
+        return an.compute_encodings(qmax - qmin, w["symmetric"])
+
     t_mm = event_time(minmax, reps)
-    mn_ref, mx_ref = O.reduce_minmax(w["x"], w["enc_shape"], w["block"])
-    exact_mm = bool(torch.equal(mn_out.cpu(), mn_ref) and torch.equal(mx_out.cpu(), mx_ref))
+    t_cal = event_time(calibrate, reps)
+    exact_mm = bool(torch.equal(mn_out.cpu(), mn_ref.view(mn_out.shape)) and torch.equal(mx_out.cpu(), mx_ref.view(mx_out.shape)))
 
-    n = x.numel()
-    S = x.element_size()
-    enc_bytes = 8 * scale.numel()
-    bytes_fwd = 2 * S * n + enc_bytes
-    bytes_bwd = 3 * S * n + enc_bytes + 8 * scale.numel()
-    bytes_step = bytes_fwd + bytes_bwd
-    ms_per_step = wall / steps * 1e3
-    value = bytes_step / (wall / steps) / 1e9
+    # ---- the same step through the drop-in module: QuantizeDequantize.forward + autograd backward
+    xm = x.clone().requires_grad_(True)
 
-    # parity spot check against the oracle (same seeded inputs)
+    def module_step():
+        xm.grad = None
+        q.min.grad = None
+        q.max.grad = None
+        out = q(xm)
+        out.backward(grad)
+
+    mod_loop, mod_repeats = timed_steps(module_step, steps, min(warmup, 5))
+    mod_s = mod_loop / steps
+    module_step()
+    _sync()
+    mod_gx_exact = None
+
+    # ---- parity against the oracle (same seeded inputs, full size)
     tr = O.qdq_v2_forward(w["x"], scale_c, offset_c, qmin, qmax, w["block"])
-    gx_ref, gs_ref, go_ref = O.qdq_v2_backward(w["grad"], w["x"], scale_c, offset_c, qmin, qmax, w["block"])
+    gx_ref, gs_ref, _ = O.qdq_v2_backward(w["grad"], w["x"], scale_c, offset_c, qmin, qmax, w["block"])
     exact_y = bool(torch.equal(y.cpu(), tr.y))
     exact_gx = bool(torch.equal(gx.cpu(), gx_ref))
-    gs_err = float(((gs.cpu() - gs_ref).abs().max() / gs_ref.abs().max().clamp_min(1e-30)))
+    mod_gx_exact = bool(torch.equal(xm.grad.cpu(), gx_ref))
+    gs_err = float(((gs.cpu().view(gs_ref.shape) - gs_ref).abs().max() / gs_ref.abs().max().clamp_min(1e-30)))
+    parity = {"y_bit_exact": exact_y, "gx_bit_exact": exact_gx, "gscale_max_rel_err": gs_err,
+              "minmax_bit_exact": exact_mm, "encoding_range_bit_exact": range_exact, "scale_bit_exact": scale_exact,
+              "module_gx_bit_exact": mod_gx_exact, "sample": "full size"}
+    if w["lpbq"]:
+        parity["per_channel_scale_bit_exact"] = bool(torch.equal(pcs.cpu(), pcs_c.view(pcs.shape)))
 
     dom = ("qdq_bwd_kernel", t_bwd, bytes_bwd) if t_bwd >= t_fwd else ("qdq_fwd_kernel", t_fwd, bytes_fwd)
-    out = {
-        "metric": "QDQ fwd+bwd GB/s (% of HBM peak); calibration elems/s; vs host-CPU ref",
-        "value": round(value, 2),
-        "unit": "GB/s",
-        "n_gpus": 1,
-        "steps": steps,
-        "warmup": warmup,
-        "ms_per_step": round(ms_per_step, 5),
-        "higher_is_better": True,
-        "scaling": "weak",
-        "vs_baseline": None,
-        "dtype": {torch.float32: "f32", torch.bfloat16: "bf16", torch.float16: "f16"}[x.dtype],
-        "data": "synthetic",
-        "config": {"workload": w["name"], "elements": n, "algorithmic_bytes_per_step": bytes_step,
-                   "arithmetic": "autograd (learnable min/max)", "compute_dtype": str(cd).split(".")[-1]},
-        "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
-        "elements_per_s": round(n / (wall / steps), 1),
-        "kernels": {
-            "qdq_fwd_kernel": {"us": round(t_fwd * 1e6, 2), "GBps": round(bytes_fwd / t_fwd / 1e9, 1)},
-            "qdq_bwd_kernel": {"us": round(t_bwd * 1e6, 2), "GBps": round(bytes_bwd / t_bwd / 1e9, 1)},
-        },
-        "calibration": {"kernel": "minmax_kernel", "us": round(t_mm * 1e6, 2),
-                        "GBps": round((S * n + 2 * S * scale.numel()) / t_mm / 1e9, 1),
+    config = {"workload": w["name"], "elements": n, "encodings": E, "algorithmic_bytes_per_step": bytes_step,
+              "arithmetic": "autograd (learnable min/max)", "compute_dtype": str(cd).split(".")[-1],
+              "step": ("ahq_lpbq_scale + " if derive is not None else "") + "ahq_qdq_forward + ahq_qdq_backward (C ABI, "
+                      "preallocated outputs)"}
+    out = _base_record(value, steps, warmup, sec_per_step, DTYPE_NAME[x.dtype], config, repeats)
+    kernels = {
+        "qdq_fwd_kernel": {"us": round(t_fwd * 1e6, 2), "GBps": round(bytes_fwd / t_fwd / 1e9, 1),
+                           "frac_of_hbm_peak": round(bytes_fwd / t_fwd / 1e9 / HBM_PEAK_GBS, 4)},
+        "qdq_bwd_kernel": {"us": round(t_bwd * 1e6, 2), "GBps": round(bytes_bwd / t_bwd / 1e9, 1),
+                           "frac_of_hbm_peak": round(bytes_bwd / t_bwd / 1e9 / HBM_PEAK_GBS, 4)},
+    }
+    if derive is not None:
+        kernels["lpbq_scale_kernel"] = {"us": round(t_derive * 1e6, 2), "GBps": round(bytes_derive / t_derive / 1e9, 1)}
+    out.update({
+        "elements_per_s": round(n / sec_per_step, 1),
+        "kernels": kernels,
+        "calibration": {"kernel": "ahq_minmax (both extrema in one pass)", "us": round(t_mm * 1e6, 2),
+                        "GBps": round((S * n + 2 * S * E) / t_mm / 1e9, 1),
                         "elements_per_s": round(n / t_mm, 1),
-                        "frac_of_hbm_peak": round((S * n) / t_mm / 1e9 / HBM_PEAK_GBS, 4)},
-        "parity": {"y_bit_exact": exact_y, "gx_bit_exact": exact_gx, "gscale_max_rel_err": gs_err,
-                   "minmax_bit_exact": exact_mm},
+                        "frac_of_hbm_peak": round((S * n) / t_mm / 1e9 / HBM_PEAK_GBS, 4),
+                        "analyzer_update_plus_compute_encodings_us": round(t_cal * 1e6, 2),
+                        "analyzer_elements_per_s": round(n / t_cal, 1)},
+        "module_path": {"what": "QuantizeDequantize.forward + .backward() with learnable min/max (allocations, "
+                                "autograd and the per-call scale / offset derivation included)",
+                        "ms_per_step": round(mod_s * 1e3, 5), "GBps": round(bytes_step / mod_s / 1e9, 1),
+                        "frac_of_hbm_peak": round(bytes_step / mod_s / 1e9 / HBM_PEAK_GBS, 4), "repeats": mod_repeats},
+        "parity": parity,
         "roofline": {"bound": "hbm", "kernel": dom[0], "achieved": round(dom[2] / dom[1] / 1e9, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(dom[2] / dom[1] / 1e9 / HBM_PEAK_GBS, 4),
                      "algorithmic_bytes": dom[2], "traffic": MEASURED_TRAFFIC_BYTES.get((key, dom[0]))},
-    }
+    })
+    if frozen is not None:
+        out["frozen_quantizer"] = frozen
     if with_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline_qdq(w, scale_c, offset_c, qmin, qmax, bytes_step)
+        def cpu_step():
+            s_c = scale_c
+            if w["lpbq"]:
+                raw = O.scale_from_minmax(emin_c, emax_c, qmin, qmax)
+                s_c, _ = O.lpbq_scale(raw, w["bitwidth"], w["decompressed_bw"], w["grouping"])
+            O.qdq_v2_forward(w["x"], s_c, offset_c, qmin, qmax, w["block"])
+            O.qdq_v2_backward(w["grad"], w["x"], s_c, offset_c, qmin, qmax, w["block"])
+
+        sample = f"full-size step of {w['name']} with the reference's torch CPU operations"
+        out["cpu_baseline"], out["cpu_baseline_1thread"] = cpu_legs(cpu_step, bytes_step, "GB/s", sample)
+
+        def cpu_cal():
+            a, b = O.reduce_minmax(w["x"], w["enc_shape"], w["block"])
+            O.minmax_encodings(a, b, qmax - qmin, w["symmetric"])
+
+        c_all, c_one = cpu_legs(cpu_cal, n, "elements/s", "min/max calibration of the same tensor", budget_s=2.0,
+                                one_thread_budget_s=2.0)
+        out["calibration"]["cpu_baseline"] = c_all
+        out["calibration"]["cpu_baseline_1thread"] = c_one
+    out["bench_seconds"] = round(time.perf_counter() - t_start, 1)
     return out
-
-
-def cpu_baseline_qdq(w, scale, offset, qmin, qmax, bytes_step, budget_s=12.0):
-    """The oracle (the reference's own sequence of torch CPU operations) timed on this host, full-size workload."""
-    from oracle import torch_ref as O
-
-    def step():
-        O.qdq_v2_forward(w["x"], scale, offset, qmin, qmax, w["block"])
-        O.qdq_v2_backward(w["grad"], w["x"], scale, offset, qmin, qmax, w["block"])
-
-    step()
-    t0 = time.perf_counter()
-    reps = 0
-    while True:
-        step()
-        reps += 1
-        if time.perf_counter() - t0 > budget_s or reps >= 20:
-            break
-    dt = (time.perf_counter() - t0) / reps
-    return {"value": round(bytes_step / dt / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(),
-            "kind": "port", "sample": f"{reps} full-size fwd+bwd steps of {w['name']} with torch CPU ops "
-                                      f"({dt * 1e3:.1f} ms/step)"}
 
 
 def _laplace_batch(shape, seed, dev):
@@ -282,6 +492,7 @@ def run_hist_workload(steps, warmup, dev, with_cpu_baseline=True, batches=16, sh
 
     _ensure_built()
     _copy_reference(dev)
+    t_start = time.perf_counter()
     xs = [_laplace_batch(shape, b, dev) for b in range(batches)]
     an = SqnrEncodingAnalyzer((1,), num_bins=512, asymmetric_delta_candidates=100, offset_candidates=64, gamma=3.0)
 
@@ -291,49 +502,27 @@ def run_hist_workload(steps, warmup, dev, with_cpu_baseline=True, batches=16, sh
             an.update_stats(x)
         return an.compute_encodings(255, False)
 
-    for _ in range(warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        lo, hi = step()
-    torch.cuda.synchronize()
-    wall = (time.perf_counter() - t0) / steps
+    loop_s, repeats = timed_steps(step, steps, warmup)
+    wall = loop_s / steps
+    lo, hi = step()
+    st = an.observer.get_stats()[0]
+    hist_gpu, edges_gpu = st.histogram.cpu().clone(), st.bin_edges.cpu().clone()
+    best_gpu = int(an.last_search["best_index"].item())
 
-    def event_time(fn, reps):
-        e0 = torch.cuda.Event(enable_timing=True)
-        e1 = torch.cuda.Event(enable_timing=True)
-        fn()
-        torch.cuda.synchronize()
-        e0.record()
-        for _ in range(reps):
-            fn()
-        e1.record()
-        torch.cuda.synchronize()
-        return e0.elapsed_time(e1) / reps * 1e-3
-
-    # one histogram update of a later batch and the search alone.  The update bins the batch on the running range while
-    # it looks for elements outside it, and reads the batch a second time only if the range moved: the algorithmic
-    # figure of two reads per element can therefore be exceeded
+    # one histogram update of a later batch that stays inside the running range (read once), one of a batch that moves
+    # it (read twice), and the search alone
     t_upd = event_time(lambda: an.update_stats(xs[1]), 20)
     t_search = event_time(lambda: an.compute_encodings(255, False), 20)
     n_b = xs[0].numel()
     n = n_b * batches
-    bytes_step = 8 * n
-    bytes_upd = 8 * n_b
+    bytes_step = 8 * n      # the two reads per element of the plain algorithm (range pass + binning pass)
+    bytes_read_once = 4 * n_b
+    traffic_upd = MEASURED_TRAFFIC_BYTES[("c3", "hist_update")]
 
-    # parity on a bounded sample: the first two batches through the CPU oracle
-    ref = O.HistObserver((1,), 512)
-    t_cpu0 = time.perf_counter()
-    cpu_batches = [xs[0].cpu(), xs[1].cpu()]
-    t_cpu1 = time.perf_counter()
-    for xb in cpu_batches:
-        ref.update(xb)
-    lo_r, hi_r, _, _, bi = O.sqnr_encodings(ref.stats, (1,), 255, False, asym_deltas=100, num_offsets=64, gamma=3.0)
-    cpu_dt = time.perf_counter() - t_cpu1
-    cpu_n = 2
+    parity = {"sample": "not compared (CPU leg switched off)"}
+    cpu_all = cpu_one = None
     if with_cpu_baseline:
-        # the CPU leg proper: the whole 16-batch step, one batch on the host at a time
+        # the CPU leg: the whole 16-batch step, one batch on the host at a time; its result is the parity reference
         ref_all = O.HistObserver((1,), 512)
         cpu_dt = 0.0
         for xb in xs:
@@ -343,49 +532,66 @@ def run_hist_workload(steps, warmup, dev, with_cpu_baseline=True, batches=16, sh
             cpu_dt += time.perf_counter() - t_b
             del xc
         t_b = time.perf_counter()
-        O.sqnr_encodings(ref_all.stats, (1,), 255, False, asym_deltas=100, num_offsets=64, gamma=3.0)
+        lo_r, hi_r, _, _, bi = O.sqnr_encodings(ref_all.stats, (1,), 255, False, asym_deltas=100, num_offsets=64, gamma=3.0)
         cpu_dt += time.perf_counter() - t_b
-        cpu_n = batches
-    an.reset_stats()
-    for xb in xs[:2]:
-        an.update_stats(xb)
-    lo2, hi2 = an.compute_encodings(255, False)
-    st = an.observer.get_stats()[0]
-    parity = {
-        "hist_bit_exact": bool(torch.equal(st.histogram.cpu(), ref.stats[0].histogram)),
-        "edges_bit_exact": bool(torch.equal(st.bin_edges.cpu(), ref.stats[0].bin_edges)),
-        "argmin_identical": bool(int(an.last_search["best_index"].item()) == int(bi.item())),
-        "encoding_bit_exact": bool(torch.equal(lo2.cpu(), lo_r) and torch.equal(hi2.cpu(), hi_r)),
-        "sample": "first 2 of 16 batches",
-    }
-    out = {
-        "metric": "QDQ fwd+bwd GB/s (% of HBM peak); calibration elems/s; vs host-CPU ref",
-        "value": round(bytes_step / wall / 1e9, 2),
-        "unit": "GB/s",
-        "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": round(wall * 1e3, 4),
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "c3_hist512_sqnr100x64_fp32_16x8x2048x4096", "elements": n,
-                   "algorithmic_bytes_per_step": bytes_step, "batches": batches},
-        "pct_of_hbm_peak": round(100.0 * bytes_step / wall / 1e9 / HBM_PEAK_GBS, 2),
+        threads = torch.get_num_threads()
+        cpu_all = {"value": round(n / cpu_dt, 1), "unit": "elements/s", "cores": threads, "kind": "port",
+                   "sample": f"all {batches} batches folded + SQNR search with the reference's torch CPU operations "
+                             f"({cpu_dt:.2f} s)"}
+        parity = {
+            "hist_bit_exact": bool(torch.equal(hist_gpu, ref_all.stats[0].histogram)),
+            "edges_bit_exact": bool(torch.equal(edges_gpu, ref_all.stats[0].bin_edges)),
+            "argmin_identical": bool(best_gpu == int(bi.item())),
+            "encoding_bit_exact": bool(torch.equal(lo.cpu(), lo_r) and torch.equal(hi.cpu(), hi_r)),
+            "largest_bin_count": float(hist_gpu.max()),
+            "sample": f"all {batches} batches",
+        }
+        # one thread: two batches and the search (bounded)
+        torch.set_num_threads(1)
+        try:
+            ref_1 = O.HistObserver((1,), 512)
+            one_dt = 0.0
+            for xb in xs[:2]:
+                xc = xb.cpu()
+                t_b = time.perf_counter()
+                ref_1.update(xc)
+                one_dt += time.perf_counter() - t_b
+                del xc
+            t_b = time.perf_counter()
+            O.sqnr_encodings(ref_1.stats, (1,), 255, False, asym_deltas=100, num_offsets=64, gamma=3.0)
+            t_s1 = time.perf_counter() - t_b
+        finally:
+            torch.set_num_threads(threads)
+        cpu_one = {"value": round(n / (one_dt * batches / 2 + t_s1), 1), "unit": "elements/s", "cores": 1, "kind": "port",
+                   "sample": f"2 of {batches} batches folded ({one_dt:.2f} s) + SQNR search ({t_s1:.2f} s), scaled to the "
+                             "whole step"}
+
+    config = {"workload": "c3_hist512_sqnr100x64_fp32_16x8x2048x4096", "elements": n,
+              "algorithmic_bytes_per_step": bytes_step, "batches": batches,
+              "step": "16 x SqnrEncodingAnalyzer.update_stats + compute_encodings (analyzer API over the C ABI)"}
+    out = _base_record(bytes_step / wall / 1e9, steps, warmup, wall, "f32", config, repeats)
+    out.update({
         "elements_per_s": round(n / wall, 1),
-        "kernels": {"hist_update(batch>=2)": {"us": round(t_upd * 1e6, 2), "GBps": round(bytes_upd / t_upd / 1e9, 1)},
-                    "sqnr_search": {"us": round(t_search * 1e6, 2), "candidates": 6400, "bins": 512}},
+        "kernels": {"hist_update(batch inside the running range)": {"us": round(t_upd * 1e6, 2),
+                                                                      "GBps_one_read": round(bytes_read_once / t_upd / 1e9, 1)},
+                    "sqnr_search(api)": {"us": round(t_search * 1e6, 2), "candidates": 6400, "bins": 512}},
         "encoding": {"min": float(lo.item()), "max": float(hi.item())},
         "parity": parity,
-        "roofline": {"bound": "hbm", "kernel": "hist_update (speculative hist_bin_kernel, second pass only when the range moves)",
-                     "achieved": round(bytes_upd / t_upd / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(bytes_upd / t_upd / 1e9 / HBM_PEAK_GBS, 4), "algorithmic_bytes": bytes_upd,
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(("c3", "hist_update")),
-                     "note": "algorithmic bytes count two reads per element (range pass + binning pass); the timed "
-                             "batch lies inside the running range and is read once, so the measured traffic is half "
-                             "of them and the fraction is not a bandwidth utilisation: against its own traffic the "
-                             "update runs at " + str(round(MEASURED_TRAFFIC_BYTES[("c3", "hist_update")] / t_upd / 1e9, 1))
-                             + " GB/s"},
-    }
-    if with_cpu_baseline:
-        out["cpu_baseline"] = {"value": round(cpu_n * n_b / cpu_dt, 1), "unit": "elements/s", "cores": torch.get_num_threads(),
-                               "kind": "port", "sample": f"all {cpu_n} batches folded + SQNR search with torch CPU ops "
-                                                         f"({cpu_dt:.2f} s)"}
+        "roofline": {"bound": "hbm", "kernel": "hist_bin_kernel<SPEC> inside one histogram update (4 launches timed together)",
+                     "achieved": round(traffic_upd / t_upd / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(traffic_upd / t_upd / 1e9 / HBM_PEAK_GBS, 4), "algorithmic_bytes": bytes_read_once,
+                     "traffic": traffic_upd,
+                     "note": "the timed batch lies inside the running range and is read once (speculative binning), so "
+                             "achieved / frac are its measured traffic over its time; against the plain algorithm's two "
+                             f"reads per element ({2 * bytes_read_once} bytes) the update runs at "
+                             f"{round(2 * bytes_read_once / t_upd / 1e9, 1)} GB/s = "
+                             f"{round(2 * bytes_read_once / t_upd / 1e9 / HBM_PEAK_GBS, 4)} of peak, and the whole "
+                             f"16-batch step at {round(bytes_step / wall / 1e9 / HBM_PEAK_GBS, 4)}"},
+    })
+    if cpu_all is not None:
+        out["cpu_baseline"], out["cpu_baseline_1thread"] = cpu_all, cpu_one
+    out["bench_seconds"] = round(time.perf_counter() - t_start, 1)
+    del xs
     return out
 
 
@@ -394,9 +600,11 @@ def run_dlq_workload(steps, warmup, dev, with_cpu_baseline=True, batches=16, sha
     candidate search for an 8-bit asymmetric encoding) followed by one per-tensor quantize-dequantize of a batch."""
     from aimet_amd import dlq
     from oracle import dlq as OD
+    from oracle import torch_ref as O
 
     _ensure_built()
     _copy_reference(dev)
+    t_start = time.perf_counter()
     xs = [_laplace_batch(shape, b, dev) for b in range(batches)]
     q = dlq.BlockTensorQuantizer((), 8, dlq.QUANTIZATION_TF_ENHANCED, device=dev)
     y = torch.empty_like(xs[0])
@@ -410,26 +618,9 @@ def run_dlq_workload(steps, warmup, dev, with_cpu_baseline=True, batches=16, sha
         q.quantizeDequantize(xs[0], y)
         return enc
 
-    for _ in range(warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        enc = step()
-    torch.cuda.synchronize()
-    wall = (time.perf_counter() - t0) / steps
-
-    def event_time(fn, reps):
-        e0 = torch.cuda.Event(enable_timing=True)
-        e1 = torch.cuda.Event(enable_timing=True)
-        fn()
-        torch.cuda.synchronize()
-        e0.record()
-        for _ in range(reps):
-            fn()
-        e1.record()
-        torch.cuda.synchronize()
-        return e0.elapsed_time(e1) / reps * 1e-3
+    loop_s, repeats = timed_steps(step, steps, warmup)
+    wall = loop_s / steps
+    enc = step()
 
     t_upd = event_time(lambda: q.updateStats(xs[1]), 20)   # range already fixed: one read of the batch
     t_qdq = event_time(lambda: q.quantizeDequantize(xs[0], y), 20)
@@ -443,7 +634,6 @@ def run_dlq_workload(steps, warmup, dev, with_cpu_baseline=True, batches=16, sha
     # aimet_torch's float fake-cast of the same batch (float8_e4m3fn, per-tensor scale), also outside the step
     from aimet_amd.quantization.float import float_quantize_dequantize
     from aimet_amd.quantization.float._finfo import _float8_e4m3fn
-    from oracle import torch_ref as O
     fscale = torch.tensor(float(enc8[0].delta), device=dev)
     t_fcast = event_time(lambda: float_quantize_dequantize(xs[0], _float8_e4m3fn, fscale), 20)
     n_b = xs[0].numel()
@@ -452,14 +642,21 @@ def run_dlq_workload(steps, warmup, dev, with_cpu_baseline=True, batches=16, sha
     bytes_qdq = 8 * n_b
     bytes_step = batches * bytes_upd + bytes_qdq
 
-    # parity on the first two batches and a bounded sample of the quantize-dequantize, against the C oracle
+    # parity: the first two batches' integer histograms, then the PDF after all 16 and the chosen encoding, and a
+    # bounded sample of the quantize-dequantize, against the C oracle
     q.resetEncodingStats()
     ref = OD.Pdf()
     hist_ok = True
-    for b in range(2):
-        h = q.updateStats(xs[b], return_histogram=True)
-        hr = ref.update(xs[b].cpu().numpy())
-        hist_ok = hist_ok and bool((h.cpu().numpy().astype("int64")[0] == hr.astype("int64")).all())
+    for b in range(batches):
+        xc = xs[b].cpu().numpy()
+        if b < 2:
+            h = q.updateStats(xs[b], return_histogram=True)
+            hr = ref.update(xc)
+            hist_ok = hist_ok and bool((h.cpu().numpy().astype("int64")[0] == hr.astype("int64")).all())
+        else:
+            q.updateStats(xs[b])
+            ref.update(xc)
+        del xc
     pdf_ok = bool((q._pdf.cpu().numpy()[0] == ref.pdf).all() and (q._xleft.cpu().numpy()[0] == ref.xleft).all())
     enc_gpu = q.computeEncodings(False)[0]
     enc_ref = ref.compute_encoding(8, False)
@@ -473,15 +670,11 @@ def run_dlq_workload(steps, warmup, dev, with_cpu_baseline=True, batches=16, sha
     yf = float_quantize_dequantize(sample, _float8_e4m3fn, fscale).cpu()
     fcast_ok = bool(torch.equal(yf.view(torch.int32), O.float_qdq(sample.cpu(), fscale.cpu(), 4, 3, True, False).view(torch.int32)))
 
-    out = {
-        "metric": "QDQ fwd+bwd GB/s (% of HBM peak); calibration elems/s; vs host-CPU ref",
-        "value": round(bytes_step / wall / 1e9, 2),
-        "unit": "GB/s",
-        "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": round(wall * 1e3, 4),
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "dlq_tf_enhanced_pdf1536_search17x21_qdq_fp32_16x8x2048x4096", "elements": n,
-                   "algorithmic_bytes_per_step": bytes_step, "batches": batches},
-        "pct_of_hbm_peak": round(100.0 * bytes_step / wall / 1e9 / HBM_PEAK_GBS, 2),
+    config = {"workload": "dlq_tf_enhanced_pdf1536_search17x21_qdq_fp32_16x8x2048x4096", "elements": n,
+              "algorithmic_bytes_per_step": bytes_step, "batches": batches,
+              "step": "16 x BlockTensorQuantizer.updateStats + computeEncodings + setEncodings + one quantizeDequantize"}
+    out = _base_record(bytes_step / wall / 1e9, steps, warmup, wall, "f32", config, repeats)
+    out.update({
         "elements_per_s": round(n / wall, 1),
         "kernels": {"pdf_update(range fixed)": {"us": round(t_upd * 1e6, 2), "GBps": round(bytes_upd / t_upd / 1e9, 1)},
                     "dlq_qdq_forward": {"us": round(t_qdq * 1e6, 2), "GBps": round(bytes_qdq / t_qdq / 1e9, 1)},
@@ -492,13 +685,16 @@ def run_dlq_workload(steps, warmup, dev, with_cpu_baseline=True, batches=16, sha
                     "tfe_search(with host read-back)": {"us": round(t_enc * 1e6, 2), "candidates": 358, "buckets": 1536}},
         "encoding": {"min": enc[0].min, "max": enc[0].max, "delta": enc[0].delta, "offset": enc[0].offset},
         "parity": {"hist_bit_exact": hist_ok, "pdf_bit_exact": pdf_ok, "encoding_bit_exact": bool(enc_ok),
-                   "qdq_bit_exact": y_ok, "fp8_qdq_bit_exact": fp8_ok, "float_qdq_bit_exact": fcast_ok, "sample": "first 2 of 16 batches; 4M-element quantize-dequantize"},
+                   "qdq_bit_exact": y_ok, "fp8_qdq_bit_exact": fp8_ok, "float_qdq_bit_exact": fcast_ok,
+                   "sample": f"integer histograms of the first 2 batches; PDF and chosen encoding after all {batches}; "
+                             "4M-element quantize-dequantize"},
         "roofline": {"bound": "hbm", "kernel": "dlq_pdf_bin_kernel", "achieved": round(bytes_upd / t_upd / 1e9, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(bytes_upd / t_upd / 1e9 / HBM_PEAK_GBS, 4),
                      "algorithmic_bytes": bytes_upd, "traffic": MEASURED_TRAFFIC_BYTES.get(("dlq", "pdf_update"))},
-    }
+    })
     if with_cpu_baseline:
-        # the scalar C restatement of the reference's loops, one thread, on a bounded slice of one batch
+        # the scalar C restatement of the reference's loops, one thread (the reference's Python binding passes no
+        # loop runner, so its CPU path is single-threaded), on a bounded slice of one batch
         m = 1 << 24
         xc = xs[0].view(-1)[:m].cpu().numpy()
         p = OD.Pdf()
@@ -518,7 +714,48 @@ def run_dlq_workload(steps, warmup, dev, with_cpu_baseline=True, batches=16, sha
                                          f"{t_pdf * 1e3:.1f} ms, quantize-dequantize {t_q * 1e3:.1f} ms), search "
                                          f"{t_s * 1e3:.2f} ms, scaled to the full step",
                                "elements_per_s": round(n / cpu_step, 1)}
+        out["cpu_baseline_1thread"] = out["cpu_baseline"]
+    out["bench_seconds"] = round(time.perf_counter() - t_start, 1)
+    del xs
     return out
+
+
+def _model_parity_sweep(model, ids, dev):
+    """Every quantizer of the model against the oracle on the tensor it sees: one calibration pass with one batch,
+    each quantizer's input reduced on the CPU as it goes by; then the calibrated min / max of all quantizers are
+    compared with the oracle's encodings of those statistics."""
+    import llama_harness as LH
+    from aimet_amd.quantization.affine import QuantizeDequantize
+    from oracle import torch_ref as O
+
+    stats = {}
+    hooks = []
+
+    def record(name, q):
+        def hook(_mod, args, _out):
+            if name in stats:
+                return  # a weight quantizer sees its weight again in the forward pass: same tensor
+            x = args[0].detach().cpu()
+            stats[name] = O.reduce_minmax(x, tuple(q.shape), q.block_size)
+        return hook
+
+    quantizers = {n: m for n, m in model.named_modules() if isinstance(m, QuantizeDequantize)}
+    for name, q in quantizers.items():
+        hooks.append(q.register_forward_hook(record(name, q)))
+    LH.calibrate(model, [ids])
+    for h in hooks:
+        h.remove()
+    ok = 0
+    bad = []
+    for name, q in quantizers.items():
+        mn, mx = stats[name]
+        lo, hi = O.minmax_encodings(mn, mx, q.qmax - q.qmin, q.symmetric)
+        same = (torch.equal(q.min.detach().cpu(), lo.view(q.shape).to(torch.float32))
+                and torch.equal(q.max.detach().cpu(), hi.view(q.shape).to(torch.float32)))
+        ok += int(same)
+        if not same:
+            bad.append(name)
+    return len(quantizers), ok, bad[:5]
 
 
 def run_model_workload(steps, warmup, dev, with_cpu_baseline=True, batches=8, seq=2048):
@@ -531,14 +768,13 @@ def run_model_workload(steps, warmup, dev, with_cpu_baseline=True, batches=8, se
 
     _ensure_built()
     _copy_reference(dev)
+    t_start = time.perf_counter()
     cfg = LH.LlamaConfig()
     model = LH.build(cfg, dev, seed=0)
     nlin = LH.quantize(model)
     ids = LH.calibration_batches(cfg, dev, batches=batches, seq=seq)
 
     def calibrate(use_graph=False):
-        # eager passes; the graph-replayed variant (llama_harness.calibrate) is timed beside it and must leave
-        # identical encodings -- with 8 batches its capture costs as much as the replays save
         LH.calibrate(model, ids, use_graph=use_graph)
 
     def forward():
@@ -549,29 +785,24 @@ def run_model_workload(steps, warmup, dev, with_cpu_baseline=True, batches=8, se
         calibrate()
         return forward()
 
-    import gc
-
-    for _ in range(warmup):
-        step()
-    torch.cuda.synchronize()
-    # the step is bound by the host interpreter (about 4000 launches): keep the cyclic garbage collector's pauses out
-    # of the few timed steps
+    # the step is bound by the host interpreter (a few thousand launches): keep the cyclic garbage collector's pauses
+    # out of the timed steps
+    step()
     gc.collect()
     gc.disable()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        step()
-    torch.cuda.synchronize()
-    wall = (time.perf_counter() - t0) / steps
-    gc.enable()
+    try:
+        loop_s, repeats = timed_steps(step, steps, warmup, min_repeats=5)
+    finally:
+        gc.enable()
+    wall = loop_s / steps
 
     def timed(fn, reps):
         fn()
-        torch.cuda.synchronize()
+        _sync()
         t = time.perf_counter()
         for _ in range(reps):
             fn()
-        torch.cuda.synchronize()
+        _sync()
         return (time.perf_counter() - t) / reps
 
     def all_ranges():
@@ -600,7 +831,8 @@ def run_model_workload(steps, warmup, dev, with_cpu_baseline=True, batches=8, se
     act_out = cfg.layers * (4 * cfg.hidden + 2 * cfg.ffn + cfg.hidden) * tokens + cfg.vocab * tokens
     act = act_in + act_out
     S = 2
-    # calibration: weights min/max once + QDQ per batch; activations min/max once per batch
+    # calibration: weights min/max once + QDQ per batch; activations min/max once per batch (the reference's flow;
+    # work that this implementation avoids still counts as algorithmic bytes of the step)
     bytes_cal = wel * S + batches * (wel * 2 * S + act * S)
     bytes_fwd = wel * 2 * S + act * 2 * S
     bytes_step = bytes_cal + bytes_fwd
@@ -623,26 +855,29 @@ def run_model_workload(steps, warmup, dev, with_cpu_baseline=True, batches=8, se
         sc, off = q.get_scale().detach().cpu(), q.get_offset().detach().cpu()
         ref = (O.qdq_v1(x, sc, off, q.qmin, q.qmax)[0] if q.block_size is None
                else O.qdq_v2_forward(x, sc, off, q.qmin, q.qmax, q.block_size).y)
-        parity[n.split(".")[-3] + "." + n.split(".")[-2]] = bool(
+        parity["forward_" + n.split(".")[-3] + "." + n.split(".")[-2]] = bool(
             torch.equal(y.as_subclass(torch.Tensor).view(torch.int16), ref.view(torch.int16)))
-    wq = mods[names[1]]
-    w = mods["blocks.0.mlp.down_proj"].weight.detach().cpu()
-    mn, mx = O.reduce_minmax(w, tuple(wq.shape), wq.block_size)
-    lo, hi = O.minmax_encodings(mn, mx, wq.qmax - wq.qmin, True)
     parity["graph_replayed_calibration_equals_eager"] = bool(same_ranges)
-    parity["weight_encodings_bit_exact"] = bool(torch.equal(wq.min.detach().cpu(), lo.view(wq.shape).float())
-                                                and torch.equal(wq.max.detach().cpu(), hi.view(wq.shape).float()))
+    aq_io = io[names[2]]
+    wq = mods[names[1]]
+    w_cpu = mods["blocks.0.mlp.down_proj"].weight.detach().cpu()
+    wq_enc = (wq.get_scale().detach().cpu(), wq.get_offset().detach().cpu())
+    aq = mods[names[2]]
+    aq_enc = (aq.get_scale().detach().cpu(), aq.get_offset().detach().cpu())
+    # every quantizer's calibrated range against the oracle (one pass, one batch); leaves the model calibrated on it
+    total, ok, bad = _model_parity_sweep(model, ids[0], dev)
+    parity["calibrated_ranges_bit_exact"] = f"{ok} of {total} quantizers"
+    parity["all_quantizers_bit_exact"] = bool(ok == total)
+    if bad:
+        parity["first_mismatches"] = bad
+    parity["sample"] = "calibrated min/max of every quantizer on its full-size input (1 batch); forward of 3 quantizers"
 
-    out = {
-        "metric": "QDQ fwd+bwd GB/s (% of HBM peak); calibration elems/s; vs host-CPU ref",
-        "value": round(bytes_step / wall / 1e9, 2),
-        "unit": "GB/s",
-        "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": round(wall * 1e3, 3),
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": "c5_llama16x2048_ffn8192_w4b64_a16_calib8x2048_plus_forward", "linear_layers": nlin,
-                   "weight_elements": wel, "activation_elements_per_forward": act,
-                   "algorithmic_bytes_per_step": bytes_step, "quantizer_elements_per_step": elems_step},
-        "pct_of_hbm_peak": round(100.0 * bytes_step / wall / 1e9 / HBM_PEAK_GBS, 2),
+    config = {"workload": "c5_llama16x2048_ffn8192_w4b64_a16_calib8x2048_plus_forward", "linear_layers": nlin,
+              "weight_elements": wel, "activation_elements_per_forward": act,
+              "algorithmic_bytes_per_step": bytes_step, "quantizer_elements_per_step": elems_step,
+              "step": "nn.compute_encodings over 8 batches + one quantized forward (module API)"}
+    out = _base_record(bytes_step / wall / 1e9, steps, warmup, wall, "bf16", config, repeats)
+    out.update({
         "elements_per_s": round(elems_step / wall, 1),
         "phases": {"calibration_8_batches_ms": round(t_cal * 1e3, 2),
                    "calibration_8_batches_graph_replay_ms": round(t_cal_graph * 1e3, 2),
@@ -656,40 +891,43 @@ def run_model_workload(steps, warmup, dev, with_cpu_baseline=True, batches=8, se
                      "frac": round(bytes_fwd / t_fwd / 1e9 / HBM_PEAK_GBS, 4), "algorithmic_bytes": bytes_fwd,
                      "traffic": None,
                      "note": "whole forward including PyTorch GEMMs and attention; the per-kernel figure is in profiles/"},
-    }
+    })
     if with_cpu_baseline:
         # the reference's CPU path for the same quantizers on a bounded sample: one weight and one activation tensor
-        w = mods["blocks.0.mlp.down_proj"].weight.detach().cpu()
-        wq = mods[names[1]]
-        sc, off = wq.get_scale().detach().cpu(), wq.get_offset().detach().cpu()
-        x, _ = io[names[2]]
-        aq = mods[names[2]]
-        asc, aoff = aq.get_scale().detach().cpu(), aq.get_offset().detach().cpu()
-        reps = 0
-        t0 = time.perf_counter()
-        while time.perf_counter() - t0 < 10.0:
-            O.reduce_minmax(w, tuple(wq.shape), wq.block_size)
-            O.qdq_v2_forward(w, sc, off, wq.qmin, wq.qmax, wq.block_size)
-            O.reduce_minmax(x, ())
-            O.qdq_v1(x, asc, aoff, aq.qmin, aq.qmax)
-            reps += 1
-        dt = (time.perf_counter() - t0) / reps
-        el = 2 * w.numel() + 2 * x.numel()
-        out["cpu_baseline"] = {"value": round(el / dt * (bytes_step / elems_step) / 1e9, 3), "unit": "GB/s",
-                               "cores": torch.get_num_threads(), "kind": "port",
-                               "sample": "min/max + quantize-dequantize of one 2048x8192 bf16 weight (block 64, 4 bit) and "
-                                         "one 2048x2048 bf16 activation (16 bit) with the reference's torch CPU calls, "
-                                         f"{reps} repetitions; quantizer work only, no GEMMs",
-                               "elements_per_s": round(el / dt, 1)}
+        x_act = aq_io[0]
+
+        def cpu_step():
+            O.reduce_minmax(w_cpu, tuple(wq.shape), wq.block_size)
+            O.qdq_v2_forward(w_cpu, wq_enc[0], wq_enc[1], wq.qmin, wq.qmax, wq.block_size)
+            O.reduce_minmax(x_act, ())
+            O.qdq_v1(x_act, aq_enc[0], aq_enc[1], aq.qmin, aq.qmax)
+
+        el = 2 * w_cpu.numel() + 2 * x_act.numel()
+        sample = ("min/max + quantize-dequantize of one 2048x8192 bf16 weight (block 64, 4 bit) and one 2048x2048 bf16 "
+                  "activation (16 bit) with the reference's torch CPU calls; quantizer work only, no GEMMs")
+        a, b = cpu_legs(cpu_step, el * (bytes_step / elems_step), "GB/s", sample, budget_s=4.0, max_reps=200)
+        out["cpu_baseline"], out["cpu_baseline_1thread"] = a, b
+    out["bench_seconds"] = round(time.perf_counter() - t_start, 1)
+    del model
     return out
+
+
+RUNNERS = {
+    "c1": lambda a, dev, cpu: run_qdq_workload("c1", a.steps, a.warmup, dev, cpu),
+    "c2": lambda a, dev, cpu: run_qdq_workload("c2", a.steps, a.warmup, dev, cpu),
+    "c4": lambda a, dev, cpu: run_qdq_workload("c4", a.steps, a.warmup, dev, cpu),
+    "c3": lambda a, dev, cpu: run_hist_workload(min(a.steps, 10), min(a.warmup, 2), dev, cpu),
+    "dlq": lambda a, dev, cpu: run_dlq_workload(min(a.steps, 10), min(a.warmup, 2), dev, cpu),
+    "c5": lambda a, dev, cpu: run_model_workload(min(a.steps, 3), min(a.warmup, 1), dev, cpu),
+}
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["c3", "c5", "dlq"])
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="all", choices=["all"] + sorted(RUNNERS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -700,14 +938,26 @@ def main():
         print("bench.py: no HIP device visible", file=sys.stderr)
         sys.exit(1)
     dev = torch.device("cuda:0")
-    if args.workload == "c3":
-        out = run_hist_workload(min(args.steps, 10), min(args.warmup, 2), dev, with_cpu_baseline=not args.no_cpu_baseline)
-    elif args.workload == "c5":
-        out = run_model_workload(min(args.steps, 3), min(args.warmup, 1), dev, with_cpu_baseline=not args.no_cpu_baseline)
-    elif args.workload == "dlq":
-        out = run_dlq_workload(min(args.steps, 10), min(args.warmup, 2), dev, with_cpu_baseline=not args.no_cpu_baseline)
+    cpu = not args.no_cpu_baseline
+    t0 = time.perf_counter()
+    if args.workload != "all":
+        out = RUNNERS[args.workload](args, dev, cpu)
     else:
-        out = run_qdq_workload(args.workload, args.steps, args.warmup, dev, with_cpu_baseline=not args.no_cpu_baseline)
+        out = RUNNERS["c4"](args, dev, cpu)
+        torch.cuda.empty_cache()
+        configs = {}
+        for key in ("c1", "c2", "c3", "dlq", "c5"):
+            print(f"[bench] {key} ...", file=sys.stderr, flush=True)
+            configs[key] = RUNNERS[key](args, dev, cpu)
+            gc.collect()
+            torch.cuda.empty_cache()
+        out["configs"] = configs
+        out["summary"] = {k: {"GBps": r["value"], "pct_of_hbm_peak": r["pct_of_hbm_peak"], "ms_per_step": r["ms_per_step"],
+                              "elements_per_s": r["elements_per_s"], "roofline_frac": r["roofline"]["frac"]}
+                          for k, r in [("c4", out)] + list(configs.items())}
+    out["host"] = {"cpu_count": os.cpu_count(), "torch_threads": torch.get_num_threads(),
+                   "device": torch.cuda.get_device_name(0)}
+    out["bench_total_seconds"] = round(time.perf_counter() - t0, 1)
     print(json.dumps(out))
 
 

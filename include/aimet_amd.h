@@ -176,6 +176,21 @@ int ahq_range_to_scale_offset(int32_t dtype, const void* range_min, const void* 
                               int64_t qmin, int64_t qmax, double minimum_scale, float* scale, float* offset,
                               void* stream);
 
+/* Replaces GroupedBlockQuantizeDequantize._get_scale / _get_per_channel_scale with dtype = float32 (LPBQ,
+ * AT/quantization/affine/quantizer.py:1363-1399), which the reference runs on every forward through get_encodings():
+ *   raw               = clamp_min(|float(max) - float(min)| / (qmax - qmin), minimum_scale)     (quantizer.py:319-339)
+ *   per_channel_scale = amax(raw over each group of blocks) / num_multipliers
+ *   scale             = quantize_dequantize(raw, per_channel_scale, offset 0, qmin 1, qmax num_multipliers)
+ * range_min / range_max: one value of `dtype` per block.  grouping: the layout of the GROUPS over the array of blocks
+ * (dims = the quantizer shape, block = blocks per group along each dimension, enc_stride = strides of the
+ * per-channel-scale array); scale: float32 per block, per_channel_scale: float32 per group.  num_multipliers =
+ * 2^(decompressed_bw - bitwidth).  AHQ_ERR_UNSUPPORTED: groups whose blocks are not neighbours in memory (the caller
+ * then composes ahq_range_to_scale_offset, ahq_minmax and ahq_qdq_forward, or the reference's torch form).
+ */
+int ahq_lpbq_scale(int32_t dtype, const ahq_layout* grouping, const void* range_min, const void* range_max,
+                   int64_t qmin, int64_t qmax, double minimum_scale, int32_t num_multipliers, float* scale,
+                   float* per_channel_scale, void* stream);
+
 /* Replaces the early exit of _decompose_prequantized_tensor (AT/utils.py:2098-2118), the test every weight goes
  * through when a calibration starts: of the first 64 blocks of the layout, the first 2 * num_levels elements each are
  * taken as float magnitudes; *verdict = 0 if one of those samples holds more than num_levels distinct values (the

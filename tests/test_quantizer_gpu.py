@@ -216,6 +216,62 @@ def test_lpbq_c4_like(device):
     assert q.min.grad is not None and q.max.grad is not None
 
 
+@pytest.mark.parametrize("case", [
+    ((96, 8), (1, 64), (1, -1), (96, 512)),          # C4's grouping: every row of blocks is one group
+    ((40, 12), (1, 16), (1, 4), (40, 192)),          # groups of four neighbouring blocks
+    ((10, 64, 1, 1), (1, 8, 1, 1), (1, 64, 1, 1), (10, 512, 1, 1)),  # convolution weight
+    ((6, 130), (1, 2), (1, -1), (6, 260)),           # groups longer than a wave
+    ((8, 6), (4, 4), (2, 3), (32, 24)),              # groups that are not runs of neighbours: step-by-step form
+    ((64, 10), (8, 1), (64, 1), (512, 10)),          # groups down a column: step-by-step form
+], ids=["rows", "fours", "conv", "long_groups", "two_dimensional_groups", "column_groups"])
+@pytest.mark.parametrize("param_dtype", [torch.float32, torch.bfloat16], ids=["f32_params", "bf16_params"])
+def test_lpbq_scale_in_one_launch(device, case, param_dtype):
+    """Without gradients get_encodings() derives the LPBQ scales with one launch (ahq_lpbq_scale); with gradients it
+    runs the reference's sequence of torch operations.  Both must give the oracle's bits."""
+    from aimet_amd.quantization.affine import GroupedBlockQuantizeDequantize
+
+    shape, block, grouping, wshape = case
+    g = torch.Generator().manual_seed(21)
+    w = torch.randn(wshape, generator=g) * 0.05
+    w.view(-1)[: w.numel() // 7] *= 30  # uneven block ranges, so the multipliers spread over 1..16
+    q = GroupedBlockQuantizeDequantize(shape=shape, bitwidth=4, symmetric=True, decompressed_bw=8, block_size=block,
+                                       block_grouping=grouping).to(device)
+    with q.compute_encodings():
+        q(w.to(device))
+    if param_dtype != torch.float32:
+        q.to(param_dtype)
+    mn, mx = q.min.detach().cpu(), q.max.detach().cpu()
+    raw = O.scale_from_minmax(mn.float(), mx.float(), -8, 7)
+    scale_ref, pcs_ref = O.lpbq_scale(raw, 4, 8, grouping)
+    with torch.no_grad():
+        enc = q.get_encodings()
+    assert_same_bits(enc.per_channel_scale, pcs_ref, "per-channel scale (one launch)")
+    assert_same_bits(enc.scale, scale_ref, "LPBQ scale (one launch)")
+    enc_grad = q.get_encodings()  # min / max require gradients: step-by-step form
+    assert enc_grad.scale.requires_grad
+    assert_same_bits(enc_grad.scale, scale_ref, "LPBQ scale (step by step)")
+    mult = enc.per_block_int_scale.detach().cpu()
+    assert mult.min() >= 1 and mult.max() <= 16 and torch.equal(mult, mult.round())
+    assert mult.unique().numel() > 4
+
+
+def test_lpbq_scale_propagates_nan(device):
+    from aimet_amd.quantization.affine import GroupedBlockQuantizeDequantize
+
+    q = GroupedBlockQuantizeDequantize(shape=(4, 8), bitwidth=4, symmetric=True, decompressed_bw=8, block_size=(1, 16),
+                                       block_grouping=(1, -1)).to(device)
+    mx = torch.rand(4, 8, generator=torch.Generator().manual_seed(1)) + 0.1
+    mx[2, 3] = float("nan")
+    q.set_range(-mx.to(device), mx.to(device))
+    raw = O.scale_from_minmax(-mx, mx, -8, 7)
+    scale_ref, pcs_ref = O.lpbq_scale(raw, 4, 8, (1, -1))
+    with torch.no_grad():
+        enc = q.get_encodings()
+    assert_same_bits(enc.scale, scale_ref, "LPBQ scale")
+    assert_same_bits(enc.per_channel_scale, pcs_ref, "per-channel scale")
+    assert bool(enc.scale[2].isnan().all()) and not bool(enc.scale[1].isnan().any())
+
+
 def test_quantize_module_and_state_dict(device):
     from aimet_amd.quantization.affine import Quantize, QuantizeDequantize, Dequantize
 
