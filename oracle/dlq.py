@@ -195,6 +195,14 @@ class Pdf:
         lib().dlq_pdf_update(self._buf, x, x.size, hist)
         return hist
 
+    def load(self, xleft, pdf, iterations=1):
+        """Replace the statistics by a given table of left edges and probabilities (tests build such tables by hand)."""
+        buf = np.frombuffer(self._buf, dtype=np.float64, count=2 * PDF_SIZE, offset=0)
+        buf[:PDF_SIZE] = np.asarray(xleft, dtype=np.float64)
+        buf[PDF_SIZE:] = np.asarray(pdf, dtype=np.float64)
+        meta = np.frombuffer(self._buf, dtype=np.int32, count=3, offset=16 * PDF_SIZE)
+        meta[:] = (int(iterations), 1, 1)
+
     @property
     def xleft(self):
         return np.frombuffer(self._buf, dtype=np.float64, count=PDF_SIZE, offset=0).copy()

@@ -9,8 +9,14 @@
  * (test/TestQuantizationFunctions.cpp:62-255), per-channel encodings and outputs (test/TestTensorQuantizer.cpp:197-300,
  * 568-728), block min/max encodings (test/TestMinMaxEncodingAnalyzer.cpp:17-130), the all-zero TF-enhanced encoding
  * (test/TestTfEnhancedEncodingAnalyzer.cpp:133-153) -- plus closed forms (uniform grids, brute-force histogram).
- * Parity unpinned: dlq_pdf_update and dlq_tfe_compute_encoding on arbitrary data; the reference's tests only bound
- * their results (test/TestTfEnhancedEncodingAnalyzer.cpp:57-286), and those bounds are checked.
+ * dlq_pdf_update and dlq_tfe_compute_encoding, whose results the reference's tests only bound
+ * (test/TestTfEnhancedEncodingAnalyzer.cpp:57-286; those bounds are checked too), are pinned exactly: the statistics
+ * on inputs at binary fractions strictly inside their buckets against a brute-force count with no slack and a
+ * hand-computed running average of three unequal batches; the search against tests/tfe_enumeration.py, an
+ * independent array-arithmetic statement of the algorithm (identical delta, offset, candidate index and candidate
+ * count on hand-built tables, for every mode and 2/4/8/16 bits), against two searches solved by hand (first of equal
+ * costs wins; the float running sum yields 101 symmetric multipliers) and on tables where the factor 3 on the
+ * saturation cost decides the winner.
  *
  * Conversions of out-of-range or NaN floats to int are undefined in C; the reference relies on what x86-64 does
  * (cvttss2si yields INT_MIN).  to_int() states that behaviour explicitly.

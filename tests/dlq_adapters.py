@@ -93,6 +93,13 @@ class OracleQuantizer:
             self.last_best.append((best, n))
         return out
 
+    def load_pdf(self, xleft, pdf, iterations=1):
+        """Put hand-built statistics ([E][1536] left edges and probabilities) in place of observed ones."""
+        xleft, pdf = np.asarray(xleft, dtype=np.float64).reshape(self.E, -1), np.asarray(pdf, dtype=np.float64).reshape(self.E, -1)
+        for e, p in enumerate(self.pdfs):
+            p.load(xleft[e], pdf[e], iterations)
+        self.valid_stats = True
+
     def setEncodings(self, encodings):
         if len(encodings) != self.E:
             raise RuntimeError("Length of encoding vector did not match BlockTensorQuantizer shape")
@@ -165,6 +172,18 @@ class HipQuantizer:
         if self.scheme == QUANTIZATION_TF_ENHANCED:
             self.last_best = [tuple(r) for r in self.q._last_best.cpu().tolist()]
         return [tuple(e) for e in encs]
+
+    def load_pdf(self, xleft, pdf, iterations=1):
+        q = self.q
+        E = q._xleft.shape[0]
+        q._xleft.copy_(torch.from_numpy(np.asarray(xleft, dtype=np.float64).reshape(E, -1)))
+        q._pdf.copy_(torch.from_numpy(np.asarray(pdf, dtype=np.float64).reshape(E, -1)))
+        q._meta.zero_()
+        q._meta[:, 0] = int(iterations)
+        q._meta[:, 1] = 1
+        q._meta[:, 2] = 1
+        q._validStats = True
+        q._all_initialized = True
 
     def setEncodings(self, encodings):
         self.q.setEncodings(encodings)

@@ -294,6 +294,157 @@ def check_tfe_properties(make):
         raise AssertionError("TF-enhanced must reject a zero-point shift")
 
 
+# ------------------------------------------------------------------ exact pins of the TF-enhanced statistics and search --
+def hand_built_pdfs():
+    """Probability tables whose candidate costs lie far apart: name -> (left edges, probabilities).  Bucket edges are
+    multiples of a power of two, so every left edge and centre is exact."""
+    from tests import tfe_enumeration as T
+
+    out = {}
+    xl = T.uniform_buckets(-12.0, 1.0 / 64)
+    pdf = np.zeros(1536)
+    pdf[640], pdf[992] = 0.7, 0.3                      # mass at the centres of two buckets: -2 and 3.5
+    out["two_centres"] = (xl, pdf)
+    pdf = np.zeros(1536)
+    pdf[600], pdf[840], pdf[1100] = 0.25, 0.5, 0.25    # three centres
+    out["three_centres"] = (xl, pdf)
+    pdf = np.zeros(1536)
+    pdf[768:1025] = np.arange(257)                     # one-sided ramp from 0 to 4
+    out["ramp"] = (xl, pdf / pdf.sum())
+    pdf = np.zeros(1536)
+    pdf[768:832] = 0.999 / 64                          # a block on [0, 1] and a lone outlier at 9
+    pdf[768 + 9 * 64] = 0.001
+    out["lone_outlier"] = (xl, pdf)
+    return out
+
+
+def _assert_search_equals_enumeration(q, xleft, pdf, bw, symmetric, strict=False, unsigned=False, what=""):
+    from tests import tfe_enumeration as T
+
+    q.load_pdf(xleft, pdf)
+    (e,) = q.computeEncodings(symmetric)
+    best, count = q.last_best[0]
+    want = T.search(xleft, pdf, bw, symmetric, strict, unsigned)
+    assert count == want["count"], f"{what}: {count} candidates, the enumeration has {want['count']}"
+    assert best == want["index"], f"{what}: candidate {best} chosen, the enumeration picks {want['index']}"
+    got = (e[0], e[1], e[2], e[3], e[4])
+    assert got == (want["min"], want["max"], want["delta"], want["offset"], bw), f"{what}: {got} vs {want}"
+    return want
+
+
+def check_tfe_exact_against_enumeration(make):
+    """The chosen (delta, offset), its index and the number of candidates against tests/tfe_enumeration.py, an
+    independent array-arithmetic statement of TfEnhancedEncodingAnalyzer.cpp:90-377: on the hand-built tables (whose
+    best and second-best costs are far apart, or tie exactly) and on the statistics of the reference tests' inputs."""
+    tables = dict(hand_built_pdfs())
+    for name in ("normal_mean2_std2", "normal_meanm2_std1"):
+        q = make((), 8, TFE)
+        q.updateStats(torch.from_numpy(INPUTS[name].copy()))
+        xl, pdf, _ = q.stats()
+        tables[name] = (xl[0].copy(), pdf[0].copy())
+    for name, (xl, pdf) in tables.items():
+        for bw in (8, 4, 2, 16):
+            for symmetric, strict, unsigned in ((False, False, False), (True, False, False), (True, True, False),
+                                                (True, False, True)):
+                q = make((), bw, TFE)
+                q.setStrictSymmetric(strict)
+                q.setUnsignedSymmetric(unsigned)
+                want = _assert_search_equals_enumeration(q, xl, pdf, bw, symmetric, strict, unsigned,
+                                                         f"{name} bw={bw} sym={symmetric} strict={strict} unsigned={unsigned}")
+                if name in ("two_centres", "three_centres", "ramp", "lone_outlier") and bw == 8:
+                    c = np.sort(want["costs"])
+                    # far apart (no rounding can swap them) or the very same candidate twice (the first one wins)
+                    assert c[1] == c[0] or (c[1] - c[0]) > 1e-6 * c[1], name
+
+
+def check_tfe_closed_forms(make):
+    """Two searches whose answer follows by hand.
+
+    All mass in the one bucket [255/16, 256/16) of a table with buckets of 1/16 starting at -32, 8 bits, asymmetric:
+    the observed range is [0, 255/16], so delta_max = 1/16 and the grid k/16 holds the range exactly.  A candidate
+    whose largest value falls into the mass's own bucket costs nothing (the bucket saturates onto its own centre);
+    every candidate with a smaller range costs something.  In the reference's order -- 17 multipliers f = 1/16 ..
+    17/16 times 21 offsets, dropping for f <= 1 only the offset -255 (empty after the clamp to the observed range) --
+    the first such candidate is f = 16/16 with offset 0: position 15 * 20 + 19 = 319.  The same (1/16, 0) comes again
+    from f = 17/16 (cut back to the observed range) and as the appended observed candidate: the FIRST of equal costs
+    has to win.  For f = 17/16 the offsets -255 (empty) and -12 (strictly contains the observed range) are dropped:
+    16 * 20 + 19 + 1 = 340 candidates.
+
+    Same table, symmetric: delta_max = (255/16) / 127.5 = 1/8, offset -128, multipliers are the running float sum
+    0.01, 0.02, ...: 100 of them stay below 1 (the float sum of 100 x 0.01 is 0.99999934), the 101st (1.0099993) is
+    still <= 1.01, a 102nd is not: 101 candidates.  Only the last one reaches past the mass's bucket (127 * 1.01 / 8 >
+    255/16), so the mass is quantised (error < delta / 2) instead of saturated onto a centre two buckets away at three
+    times the cost: the last candidate wins."""
+    from tests import tfe_enumeration as T
+
+    xl = T.uniform_buckets(-32.0, 1.0 / 16)
+    pdf = np.zeros(1536)
+    pdf[512 + 255] = 1.0
+    q = make((), 8, TFE)
+    q.load_pdf(xl, pdf)
+    (e,) = q.computeEncodings(False)
+    assert tuple(e) == (0.0, 255.0 / 16, 1.0 / 16, 0.0, 8)
+    assert tuple(q.last_best[0]) == (319, 340)
+    q = make((), 8, TFE)
+    q.load_pdf(xl, pdf)
+    (e,) = q.computeEncodings(True)
+    f = np.float32(0.01)
+    for _ in range(100):
+        f = np.float32(np.float64(f) + 0.01)
+    delta = np.float32(f * np.float32(0.125))
+    assert tuple(q.last_best[0]) == (100, 101)
+    assert (e[2], e[3]) == (float(delta), -128.0)
+    assert (e[0], e[1]) == (float(np.float32(delta * np.float32(-128))), float(np.float32(delta * np.float32(127))))
+
+
+def check_tfe_saturation_weight_decides(make):
+    """Tables on which the factor 3 on the saturation cost decides the winner: a heavy mass near zero and a light one
+    far out, on a coarse grid.  With the factor the search keeps a wider range than it would without; the enumeration
+    run with a factor of 1 confirms that the two answers differ, so a dropped or wrong factor cannot pass."""
+    from tests import tfe_enumeration as T
+
+    xl = T.uniform_buckets(-32.0, 1.0 / 16)
+    for bw, light, far in ((4, 0.05, 900), (2, 0.02, 900), (3, 0.1, 900)):
+        pdf = np.zeros(1536)
+        pdf[512 + 40], pdf[far] = 1.0 - light, light
+        q = make((), bw, TFE)
+        want = _assert_search_equals_enumeration(q, xl, pdf, bw, False, what=f"bw={bw}")
+        unweighted = T.search(xl, pdf, bw, False, gamma=1.0)
+        assert unweighted["delta"] < want["delta"] and unweighted["index"] != want["index"]
+
+
+def check_pdf_exact_binary_fractions(make):
+    """Statistics of inputs that sit on exact binary fractions strictly inside their buckets: no rounding anywhere, so
+    the counts must equal a brute-force count with no slack, and the running average of three unequal batches is what
+    a hand calculation gives.
+
+    First batch spans [-1, 1]: the range becomes three times that around the centre 0, [-3, 3], in 1536 buckets of
+    1/256 whose left edges are (i - 768) / 256."""
+    k1 = np.concatenate([np.arange(-256, 256), np.arange(-256, 256, 2)])
+    x1 = np.concatenate([(k1 + 0.5) / 256, [-1.0, 1.0]]).astype(np.float32)       # 770 values; -1 and 1 fix the range
+    k2 = np.concatenate([np.arange(-700, 700, 7), np.arange(0, 64), np.arange(0, 64)])
+    x2 = np.concatenate([(k2 + 0.25) / 256, [5.0, -5.0, 3.0, np.nan, np.inf]]).astype(np.float32)  # the last five fall outside
+    k3 = np.arange(-768, 768, 3)
+    x3 = ((k3 + 0.75) / 256).astype(np.float32)
+    q = make((), 8, TFE)
+    hists = [q.updateStats(torch.from_numpy(x.copy()), return_histogram=True)[0].numpy().astype(np.int64) for x in (x1, x2, x3)]
+    xl, pdf, meta = q.stats()
+    assert np.array_equal(xl[0], (np.arange(1536) - 768) / 256.0)
+    brute1 = np.bincount(k1 + 768, minlength=1536)
+    brute1[768 - 256] += 1          # -1.0 is the left edge of its bucket
+    brute1[768 + 256] += 1          # 1.0 likewise
+    brute2 = np.bincount(k2 + 768, minlength=1536)  # 5, -5, 3 (= the right end of the range), NaN and inf are dropped
+    brute3 = np.bincount(k3 + 768, minlength=1536)
+    for h, b, x in zip(hists, (brute1, brute2, brute3), (x1, x2, x3)):
+        assert np.array_equal(h, b)
+    assert hists[1].sum() == x2.size - 5
+    # running average by hand: ((p1 * 0 + p1) / 1 -> p1; (p1 * 1 + p2) / 2; (that * 2 + p3) / 3), p = counts / batch size
+    p1, p2, p3 = brute1 / float(x1.size), brute2 / float(x2.size), brute3 / float(x3.size)
+    expect = (((p1 * 1 + p2) / 2) * 2 + p3) / 3
+    assert np.array_equal(pdf[0], expect)
+    assert tuple(meta[0][:3]) == (3, 1, 1)
+
+
 def check_percentile(make):
     """test/TestPercentileEncodingAnalyzer.cpp:21-296: the reference's bounds and exact expectations."""
     d100k = torch.from_numpy(INPUTS["normal_mean2_std2_100k"].copy())

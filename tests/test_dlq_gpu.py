@@ -12,6 +12,8 @@ from tests.dlq_adapters import (QUANTIZATION_PERCENTILE, QUANTIZATION_TF, QUANTI
 
 pytestmark = pytest.mark.gpu
 
+TFE_MODES = [(False, False, False), (True, False, False), (True, True, False), (True, False, True)]
+
 
 @pytest.fixture()
 def make(device):
@@ -48,6 +50,48 @@ def test_tfe_reference_bounds(make):
 
 def test_percentile_reference_expectations(make):
     C.check_percentile(make)
+
+
+# ------------------------------------------------------- exact pins: independent enumeration and closed forms --------
+def test_tfe_search_equals_independent_enumeration(make):
+    C.check_tfe_exact_against_enumeration(make)
+
+
+def test_tfe_closed_forms(make):
+    C.check_tfe_closed_forms(make)
+
+
+def test_tfe_saturation_weight_decides(make):
+    C.check_tfe_saturation_weight_decides(make)
+
+
+def test_pdf_exact_on_binary_fractions(make):
+    C.check_pdf_exact_binary_fractions(make)
+
+
+@pytest.mark.parametrize("slots", [5, 24])
+def test_tfe_search_of_several_hand_built_tables_at_once(device, slots):
+    """The same pins with several slots in one call: up to 16 slots are priced with one wave per candidate, more with
+    one lane per candidate; every slot must pick what the independent enumeration picks for its table."""
+    from tests import tfe_enumeration as T
+
+    tables = list(C.hand_built_pdfs().values())
+    xl = T.uniform_buckets(-32.0, 1.0 / 16)
+    one = np.zeros(1536)
+    one[512 + 255] = 1.0
+    tables.append((xl, one))
+    xls = np.stack([tables[s % len(tables)][0] for s in range(slots)])
+    pdfs = np.stack([tables[s % len(tables)][1] for s in range(slots)])
+    for sym, strict, uns in TFE_MODES:
+        q = HipQuantizer((slots, 1), 8, QUANTIZATION_TF_ENHANCED, device)
+        q.setStrictSymmetric(strict)
+        q.setUnsignedSymmetric(uns)
+        q.load_pdf(xls, pdfs)
+        encs = q.computeEncodings(sym)
+        for s in range(slots):
+            want = T.search(xls[s], pdfs[s], 8, sym, strict, uns)
+            assert tuple(q.last_best[s]) == (want["index"], want["count"]), (s, sym, strict, uns)
+            assert tuple(encs[s]) == (want["min"], want["max"], want["delta"], want["offset"], 8), (s, sym, strict, uns)
 
 
 # ------------------------------------------------------------------------------------- bit-exact against the oracle --
@@ -247,8 +291,6 @@ def test_pdf_update_of_an_empty_tensor_through_the_c_abi(device):
     _lib.check(lib.ahq_dlq_pdf_update(_lib.AHQ_F32, lay, None, st, 1, None, None, 0, _lib.current_stream(device)), "update")
     assert meta.cpu().tolist() == [[0, 0, 1, 0]] and float(pdf.abs().sum()) == 0.0
 
-
-TFE_MODES = [(False, False, False), (True, False, False), (True, True, False), (True, False, True)]
 
 
 @pytest.mark.parametrize("bw", [4, 8, 16])

@@ -43,6 +43,22 @@ def test_tfe_reference_bounds():
     C.check_tfe_properties(make)
 
 
+def test_tfe_search_equals_independent_enumeration():
+    C.check_tfe_exact_against_enumeration(make)
+
+
+def test_tfe_closed_forms():
+    C.check_tfe_closed_forms(make)
+
+
+def test_tfe_saturation_weight_decides():
+    C.check_tfe_saturation_weight_decides(make)
+
+
+def test_pdf_exact_on_binary_fractions():
+    C.check_pdf_exact_binary_fractions(make)
+
+
 def test_percentile_reference_expectations():
     C.check_percentile(make)
 
