@@ -125,6 +125,11 @@ _SIGNATURES = {
     "ahq_sqnr_search": (ctypes.c_int, [ctypes.POINTER(SqnrParams), _P, _P, _P, _P, _P, _P, _P, _P, _P, _P]),
     "ahq_dlq_minmax_encodings": (ctypes.c_int, [_P, _P, ctypes.c_int64, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32,
                                                 ctypes.c_int32, ctypes.c_double, _P, _P]),
+    "ahq_dlq_qdq_per_tensor": (ctypes.c_int, [ctypes.c_int32, _P, _P, ctypes.c_uint64, ctypes.c_double, ctypes.c_double,
+                                              ctypes.c_double, ctypes.c_double, _P]),
+    "ahq_dlq_fp8_qdq_per_tensor": (ctypes.c_int, [ctypes.c_int32, _P, _P, ctypes.c_uint64, ctypes.c_double, ctypes.c_int32,
+                                                  ctypes.c_int32, ctypes.c_float, _P]),
+    "ahq_dlq_minmax_fold": (ctypes.c_int, [ctypes.c_int32, _P, _P, ctypes.c_int64, _P, _P, _P]),
     "ahq_dlq_pdf_update_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int32, ctypes.POINTER(Layout)]),
     "ahq_dlq_pdf_update": (ctypes.c_int, [ctypes.c_int32, ctypes.POINTER(Layout), _P, ctypes.POINTER(DlqPdfState),
                                           ctypes.c_int32, _P, _P, ctypes.c_size_t, _P]),

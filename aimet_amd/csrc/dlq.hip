@@ -1007,6 +1007,34 @@ extern "C" int ahq_dlq_pdf_update(int32_t dtype, const ahq_layout* layout, const
     return check_launch("dlq_pdf_update");
 }
 
+// Running float min / max <- std::min / std::max with a batch's extrema given in the tensor's dtype (a 16-bit tensor is
+// widened value by value before the fold, MinMaxEncodingAnalyzer.cpp:32-95 with tensor_utils.hpp's widening).
+template <typename IO>
+__global__ void dlq_minmax_fold_kernel(const IO* bmin, const IO* bmax, float* rmin, float* rmax, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const float mn = load_f32(bmin[i]), mx = load_f32(bmax[i]);
+    const float pmn = rmin[i], pmx = rmax[i];
+    rmin[i] = mn < pmn ? mn : pmn;
+    rmax[i] = pmx < mx ? mx : pmx;
+}
+
+extern "C" int ahq_dlq_minmax_fold(int32_t dtype, const void* batch_min, const void* batch_max, int64_t num_encodings,
+                                   float* run_min, float* run_max, void* stream) {
+    if (dtype < AHQ_F32 || dtype > AHQ_BF16) return set_error("bad dtype"), AHQ_ERR_INVALID;
+    if (!batch_min || !batch_max || !run_min || !run_max) return set_error("null argument"), AHQ_ERR_INVALID;
+    if (num_encodings < 0) return set_error("negative encoding count"), AHQ_ERR_INVALID;
+    if (num_encodings == 0) return AHQ_OK;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const dim3 g((unsigned)((num_encodings + 255) / 256)), b(256);
+    switch (dtype) {
+        case AHQ_F32: hipLaunchKernelGGL((dlq_minmax_fold_kernel<float>), g, b, 0, s, static_cast<const float*>(batch_min), static_cast<const float*>(batch_max), run_min, run_max, num_encodings); break;
+        case AHQ_F16: hipLaunchKernelGGL((dlq_minmax_fold_kernel<f16_t>), g, b, 0, s, static_cast<const f16_t*>(batch_min), static_cast<const f16_t*>(batch_max), run_min, run_max, num_encodings); break;
+        default: hipLaunchKernelGGL((dlq_minmax_fold_kernel<bf16_t>), g, b, 0, s, static_cast<const bf16_t*>(batch_min), static_cast<const bf16_t*>(batch_max), run_min, run_max, num_encodings); break;
+    }
+    return check_launch("dlq_minmax_fold");
+}
+
 extern "C" size_t ahq_dlq_tfe_encodings_workspace_bytes(int32_t num_slots) {
     if (num_slots <= 0) return 0;
     const size_t S = (size_t)num_slots;

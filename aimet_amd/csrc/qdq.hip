@@ -375,6 +375,10 @@ struct QdqArgs : Geom {
     GridC gc;
     int32_t red;
     int32_t out_cd;  // compute dtype the reduced gradients are rounded through
+    // one encoding handed over by value (scale, offset, min, max) instead of through the four pointers: what the
+    // per-tensor entry points use, so that their callers need no device copy of the encoding
+    int32_t by_value;
+    float value_enc[4];
 };
 
 template <typename M>
@@ -382,10 +386,10 @@ __device__ __forceinline__ void stage_encodings(const QdqArgs& a, const Tile& t,
     for (int i = threadIdx.x; i < t.nstage; i += kBlock) {
         int64_t e = t.e0 + i;
         if (e >= a.J) e %= a.J;
-        const float s = a.scale[e];
-        const float off = a.offset ? a.offset[e] : 0.f;
-        const float mn = a.emin ? a.emin[e] : 0.f;
-        const float mx = a.emax ? a.emax[e] : 0.f;
+        const float s = a.by_value ? a.value_enc[0] : a.scale[e];
+        const float off = a.by_value ? a.value_enc[1] : (a.offset ? a.offset[e] : 0.f);
+        const float mn = a.by_value ? a.value_enc[2] : (a.emin ? a.emin[e] : 0.f);
+        const float mx = a.by_value ? a.value_enc[3] : (a.emax ? a.emax[e] : 0.f);
         const EncP p = M::prep(s, off, mn, mx, a.gc);
         sp[0][i] = p.p0;
         sp[1][i] = p.p1;
@@ -408,6 +412,7 @@ __device__ __forceinline__ EncP staged(float (*sp)[kStage], int i) {
 
 template <typename M>
 __device__ __forceinline__ EncP load_enc(const QdqArgs& a, int64_t e) {
+    if (a.by_value) return M::prep(a.value_enc[0], a.value_enc[1], a.value_enc[2], a.value_enc[3], a.gc);
     return M::prep(a.scale[e], a.offset ? a.offset[e] : 0.f, a.emin ? a.emin[e] : 0.f, a.emax ? a.emax[e] : 0.f, a.gc);
 }
 
@@ -1111,6 +1116,71 @@ extern "C" int ahq_dlq_fp8_qdq(int32_t dtype, const ahq_layout* layout, const vo
     hipStream_t st = static_cast<hipStream_t>(stream);
     launch_fwd<float, MathDlqFp8>(p, a, st, aligned16(x) && aligned16(y));
     return check_launch("ahq_dlq_fp8_qdq");
+}
+
+// One encoding by value over a flat tensor of `count` elements.
+static bool flat_plan(int32_t dtype, uint64_t count, const void* x, const void* y, Plan* p, bool* aligned) {
+    if (count > (uint64_t)1 << 62) return set_error("count too large"), false;
+    ahq_layout layout{};
+    layout.ndim = 1;
+    layout.dims[0] = (int64_t)count;
+    layout.block[0] = count ? (int64_t)count : 1;
+    layout.enc_stride[0] = 0;
+    *aligned = aligned16(x) && aligned16(y);
+    return make_plan(dtype, layout, *aligned, false, p, kFwdUnroll);
+}
+
+extern "C" int ahq_dlq_qdq_per_tensor(int32_t dtype, const void* x, void* y, uint64_t count, double enc_min,
+                                      double enc_max, double delta, double offset, void* stream) {
+    if (dtype < AHQ_F32 || dtype > AHQ_BF16) return set_error("bad dtype"), AHQ_ERR_INVALID;
+    Plan p;
+    bool al;
+    if (!flat_plan(dtype, count, x, y, &p, &al)) return AHQ_ERR_INVALID;
+    if (p.cl.numel == 0) return AHQ_OK;
+    if (!x || !y) return set_error("x or y is null"), AHQ_ERR_INVALID;
+    ahq_grid grid{};
+    grid.arith = AHQ_ARITH_DLQ;
+    grid.op = AHQ_OP_QDQ;
+    grid.io_dtype = dtype;
+    grid.compute_dtype = AHQ_F32;
+    QdqArgs a{};
+    a.x = x;
+    a.y = y;
+    a.by_value = 1;
+    // the encoding's doubles narrowed to float, as quantizeDequantizeCpu / Gpu do (trim_functions.cpp:211-226)
+    a.value_enc[0] = (float)delta;
+    a.value_enc[1] = (float)offset;
+    a.value_enc[2] = (float)enc_min;
+    a.value_enc[3] = (float)enc_max;
+    fill_args(grid, p, &a);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    AHQ_IO_SWITCH(dtype, (launch_fwd<IO, MathDlq>(p, a, st, al)));
+    return check_launch("ahq_dlq_qdq_per_tensor");
+}
+
+extern "C" int ahq_dlq_fp8_qdq_per_tensor(int32_t dtype, const void* x, void* y, uint64_t count, double delta,
+                                          int32_t mantissa_bits, int32_t exponent_min, float max_value, void* stream) {
+    if (dtype != AHQ_F32) return set_error("FP8 quantize-dequantize supports float tensors only"), AHQ_ERR_UNSUPPORTED;
+    if (mantissa_bits < 0 || mantissa_bits > 23 || exponent_min < -126 || exponent_min > 127 || !(max_value > 0.f))
+        return set_error("bad FP8 format description"), AHQ_ERR_INVALID;
+    Plan p;
+    bool al;
+    if (!flat_plan(dtype, count, x, y, &p, &al)) return AHQ_ERR_INVALID;
+    if (p.cl.numel == 0) return AHQ_OK;
+    if (!x || !y) return set_error("x or y is null"), AHQ_ERR_INVALID;
+    QdqArgs a{};
+    a.x = x;
+    a.y = y;
+    a.by_value = 1;
+    a.value_enc[0] = (float)delta;
+    ahq_grid grid{};
+    grid.compute_dtype = AHQ_F32;
+    fill_args(grid, p, &a);
+    a.gc.qmin = (float)exponent_min;
+    a.gc.qmax = max_value;
+    a.gc.zps = (float)mantissa_bits;
+    launch_fwd<float, MathDlqFp8>(p, a, static_cast<hipStream_t>(stream), al);
+    return check_launch("ahq_dlq_fp8_qdq_per_tensor");
 }
 
 extern "C" int ahq_float_qdq(int32_t dtype, const ahq_layout* layout, const void* x, void* y, const float* scale,

@@ -188,8 +188,8 @@ class BlockTensorQuantizer:
                 mx = torch.empty_like(mn)
                 _lib.check(lib.ahq_minmax(code, layout, x.data_ptr(), mn.data_ptr(), mx.data_ptr(), None, None, 2,
                                           ws.data_ptr(), nbytes, stream), "ahq_minmax")
-                torch.minimum(self._min, mn.float(), out=self._min)
-                torch.maximum(self._max, mx.float(), out=self._max)
+                _lib.check(lib.ahq_dlq_minmax_fold(code, mn.data_ptr(), mx.data_ptr(), self._E, self._min.data_ptr(),
+                                                   self._max.data_ptr(), stream), "ahq_dlq_minmax_fold")
             return None
         state = self._pdf_state()
         nbytes = lib.ahq_dlq_pdf_update_workspace_bytes(code, layout)

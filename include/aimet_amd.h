@@ -100,6 +100,15 @@ int ahq_qdq_forward(const ahq_grid* grid, const ahq_layout* layout, const void* 
                     const float* scale, const float* offset, const float* enc_min, const float* enc_max,
                     void* stream);
 
+/* Replaces DlQuantization::quantizeDequantize<T>(in, cnt, encoding, out, COMP_MODE_GPU, ROUND_NEAREST, stream)
+ * (DLQ/src/trim_functions.hpp:35-37, trim_functions.cpp:108-128), the per-tensor form BlockTensorQuantizer uses when
+ * its shape has one element (DLQ/src/TensorQuantizer.cpp:106-111): the encoding travels by value, so the caller needs
+ * no device copy of it.  x / y: `count` elements of `dtype`; the four doubles are the TfEncoding fields, narrowed to
+ * float inside as the reference does.
+ */
+int ahq_dlq_qdq_per_tensor(int32_t dtype, const void* x, void* y, uint64_t count, double enc_min, double enc_max,
+                           double delta, double offset, void* stream);
+
 /* Backward of the above with the straight-through estimator (torch_builtins.py:637-655, 691-701, 779-831).  The mask
  * is recomputed from x.  gx may be NULL; gscale/goffset may be NULL (both or neither); when given they receive the
  * gradient already reduced to one fp32 value per encoding (what autograd's sum-to-size produces in the reference).
@@ -267,6 +276,13 @@ int ahq_dlq_minmax_encodings(const float* stat_min, const float* stat_max, int64
                              int32_t symmetric, int32_t strict, int32_t unsigned_sym, double zero_point_shift,
                              double* out, void* stream);
 
+/* Folds a batch's per-block extrema (values of `dtype`, e.g. the out_min / out_max of ahq_minmax with finite_only = 2
+ * on a 16-bit tensor) into the running float statistics with std::min / std::max: what MinMaxEncodingAnalyzer::
+ * updateStats does after widening a half / bfloat16 tensor (DLQ/src/MinMaxEncodingAnalyzer.cpp:32-95).
+ */
+int ahq_dlq_minmax_fold(int32_t dtype, const void* batch_min, const void* batch_max, int64_t num_encodings,
+                        float* run_min, float* run_max, void* stream);
+
 /* TF-enhanced statistics: one 1536-bucket PDF per encoding block (DLQ/src/math_functions.hpp:28-49).
  * xleft/pdf: [num_slots][AHQ_DLQ_PDF_SIZE] doubles; meta: [num_slots][4] int32 = iterations, initialized (xLeft not
  * empty), stats_updated, reserved.  All zero = a freshly constructed analyzer; resetStats zeroes everything but
@@ -311,6 +327,12 @@ int    ahq_dlq_tfe_encodings(const ahq_dlq_pdf_state* state, int32_t bw, int32_t
  */
 int ahq_dlq_fp8_qdq(int32_t dtype, const ahq_layout* layout, const void* x, void* y, const float* scale,
                     int32_t mantissa_bits, int32_t exponent_min, float max_value, void* stream);
+
+/* The per-tensor form of ahq_dlq_fp8_qdq with the scale (TfEncoding.delta) by value: quantizeDequantizeFp8
+ * (DLQ/src/trim_functions.hpp:39-41, trim_functions.cpp:243-258).
+ */
+int ahq_dlq_fp8_qdq_per_tensor(int32_t dtype, const void* x, void* y, uint64_t count, double delta,
+                               int32_t mantissa_bits, int32_t exponent_min, float max_value, void* stream);
 
 /* Replaces _float_quantize_dequantize of aimet_torch (aimet_torch/quantization/float/quantizer.py:634-716, with
  * _cast_decast :709-710 and fake_cast_to_ieee_float, aimet_torch/fp_quantization.py:148-214): in the arithmetic of
