@@ -20,20 +20,46 @@ static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
 namespace ahq {
 
-struct MmArgs : Geom {
-    const void* x;
+// Where results go (shared by every kernel family of this file).
+struct MmOut {
     void* out_min;
     void* out_max;
+    void* run_min;          // optional running statistics folded with torch.minimum / torch.maximum semantics
+    void* run_max;
+    int32_t finite_only;
+};
+
+struct MmArgs : Geom, MmOut {
+    const void* x;
     float* part_min;      // kRedTile: [nblocks]
     float* part_max;
     int* part_nan;
     unsigned int* key_min;  // kRedAtomic: [num_enc] order-preserving keys
     unsigned int* key_max;
     int32_t red;
-    void* run_min;          // optional running statistics folded with torch.minimum / torch.maximum semantics
-    void* run_max;
-    int32_t finite_only;
     void* copy;             // optional: the tensor is also copied there by the pass that reads it (single encoding)
+};
+
+// Arguments of the single-encoding kernels.
+struct MmFlatArgs : MmOut {
+    const void* x;
+    void* copy;        // optional: the tensor is also copied there by the pass that reads it
+    int64_t numel;
+    int64_t nvec;
+    float* part_min;   // [gridDim.x] partial extrema, folded by minmax_fold_kernel
+    float* part_max;
+    int* part_nan;
+};
+
+// Arguments of the two lean kernels below (runs of whole vectors on the leading axis): a few words instead of the
+// whole tile geometry, because their workgroups live for about a microsecond and every scalar load and division at
+// their start shows.
+struct MmRunArgs : MmOut {
+    const void* x;
+    int64_t nvec;      // vectors in the tensor
+    int64_t runs;      // number of encodings
+    int32_t kv;        // vectors per run
+    int32_t kv_shift;  // log2(kv) (segment kernel: kv is a power of two)
 };
 
 struct MinMax {
@@ -55,6 +81,41 @@ __device__ __forceinline__ void mm_add(MinMax& m, float v, bool finite_only) {
     }
 }
 
+// Both extrema of one 16-byte vector.  The kernels are close enough to the memory system's limit that the vector
+// instructions per element show in their run time, so: two elements per three-operand minimum / maximum, and NaN is
+// looked for with one unordered comparison per PAIR of elements whose lane mask is OR-ed on the scalar unit
+// (`unordered`: lanes that have seen a NaN), instead of a compare, a select and an OR per element.
+// MODE 0: NaN is tracked (torch.amin / amax propagate it); 1: non-finite values are ignored; 2: NaN is simply never
+// chosen (fminf / fmaxf), which is what DlQuantization's std::min / std::max folds do.
+template <typename IO, int VEC, int MODE>
+__device__ __forceinline__ void mm_pack(const Pack<IO, VEC>& p, float& mn, float& mx, uint64_t& unordered) {
+    float f[VEC];
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) f[k] = load_f32(p.v[k]);
+    if (MODE == 1) {
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) {
+            const bool fin = __builtin_fabsf(f[k]) < __builtin_inff();
+            mn = fminf(mn, fin ? f[k] : __builtin_inff());
+            mx = fmaxf(mx, fin ? f[k] : -__builtin_inff());
+        }
+        return;
+    }
+#pragma unroll
+    for (int k = 0; k + 1 < VEC; k += 2) {
+        mn = fminf(fminf(mn, f[k]), f[k + 1]);
+        mx = fmaxf(fmaxf(mx, f[k]), f[k + 1]);
+        if (MODE == 0) unordered |= __builtin_amdgcn_ballot_w64(__builtin_isunordered(f[k], f[k + 1]));
+    }
+    if (VEC & 1) {
+        mn = fminf(mn, f[VEC - 1]);
+        mx = fmaxf(mx, f[VEC - 1]);
+        if (MODE == 0) unordered |= __builtin_amdgcn_ballot_w64(f[VEC - 1] != f[VEC - 1]);
+    }
+}
+
+constexpr int mm_mode(bool finite) { return finite ? 1 : 0; }
+
 __device__ __forceinline__ MinMax mm_merge(const MinMax& a, const MinMax& b) {
     return {fminf(a.mn, b.mn), fmaxf(a.mx, b.mx), a.nan | b.nan};
 }
@@ -63,6 +124,7 @@ __device__ __forceinline__ MinMax mm_shfl_xor(const MinMax& a, int m) {
     return {__shfl_xor(a.mn, m, kWave), __shfl_xor(a.mx, m, kWave), __shfl_xor(a.nan, m, kWave)};
 }
 
+template <int BLOCK = kBlock>
 __device__ __forceinline__ MinMax mm_block_reduce(MinMax v, MinMax* smem) {
 #pragma unroll
     for (int m = kWave / 2; m >= 1; m >>= 1) v = mm_merge(v, mm_shfl_xor(v, m));
@@ -71,12 +133,12 @@ __device__ __forceinline__ MinMax mm_block_reduce(MinMax v, MinMax* smem) {
     __syncthreads();
     MinMax r = smem[0];
 #pragma unroll
-    for (int w = 1; w < kBlock / kWave; ++w) r = mm_merge(r, smem[w]);
+    for (int w = 1; w < BLOCK / kWave; ++w) r = mm_merge(r, smem[w]);
     return r;
 }
 
 template <typename IO>
-__device__ __forceinline__ void mm_write(const MmArgs& a, int64_t e, MinMax m) {
+__device__ __forceinline__ void mm_write(const MmOut& a, int64_t e, MinMax m) {
     IO* omn = static_cast<IO*>(a.out_min);
     IO* omx = static_cast<IO*>(a.out_max);
     const float qnan = __builtin_nanf("");
@@ -126,28 +188,49 @@ __device__ __forceinline__ void mm_tile(const MmArgs& a, const Tile& t, MinMax& 
         const int lv = u * kBlock + threadIdx.x;
         if (FULL || lv < t.nv) in[u] = load_pack<IO, VEC>(x + (int64_t)lv * VEC);
     }
+    // lanes of this lane's run, as a mask over the wave (kRedSeg): a NaN seen by any of them belongs to the run
+    uint64_t run_lanes = ~0ull;
+    if (RED == kRedSeg && a.Kv < kWave) run_lanes = ((1ull << a.Kv) - 1) << (threadIdx.x & (kWave - 1) & ~((int)a.Kv - 1));
+    const uint64_t my_lane = 1ull << (threadIdx.x & (kWave - 1));
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
         const int lv = u * kBlock + threadIdx.x;
         MinMax v = mm_identity();
         int si = 0;
-        if (FULL || lv < t.nv) {
-            si = stage_index(a, t, lv);
+        uint64_t unordered = 0;  // lanes of the wave whose vector holds a NaN
+        const bool live = FULL || lv < t.nv;
+        if (RED != kRedTile && live) si = stage_index(a, t, lv);
+        if (FULL) {
+            mm_pack<IO, VEC, mm_mode(FINITE)>(in[u], v.mn, v.mx, unordered);
+        } else {
+            // ragged tile: lanes without a vector contribute the identity (the ballot inside sees only live lanes'
+            // values because the others hold zeros)
+            Pack<IO, VEC> pk = in[u];
+            if (!live)
 #pragma unroll
-            for (int k = 0; k < VEC; ++k) mm_add(v, load_f32(in[u].v[k]), FINITE);
+                for (int k = 0; k < VEC; ++k) pk.v[k] = IO{};
+            float mn = __builtin_inff(), mx = -__builtin_inff();
+            mm_pack<IO, VEC, mm_mode(FINITE)>(pk, mn, mx, unordered);
+            if (live) {
+                v.mn = mn;
+                v.mx = mx;
+            }
         }
         if (RED == kRedTile) {
+            // a NaN anywhere in the wave marks the whole wave's contribution: the tile has one encoding
+            v.nan = unordered != 0 ? 1 : 0;
             acc = mm_merge(acc, v);
         } else if (RED == kRedSeg) {
+            v.nan = (unordered & run_lanes) != 0 ? 1 : 0;
             const int kv = (int)a.Kv;
             v.mn = segment_reduce(v.mn, kv, OpMinF());
             v.mx = segment_reduce(v.mx, kv, OpMaxF());
-            v.nan = segment_reduce(v.nan, kv, OpOrI());
-            if ((FULL || lv < t.nv) && (threadIdx.x & (kv - 1)) == 0) mm_write<IO>(a, t.e0 + si, v);
+            if (live && (threadIdx.x & (kv - 1)) == 0) mm_write<IO>(a, t.e0 + si, v);
         } else if (RED == kRedAtomic) {
+            v.nan = (unordered & my_lane) != 0 ? 1 : 0;
             // first into the tile's own table in LDS (one entry per run the tile touches); the table goes to the
             // global keys once per run and tile instead of once per vector
-            if (FULL || lv < t.nv) {
+            if (live) {
                 atomicMin(&stage_keys[si], f32_key(v.mn));
                 atomicMax(&stage_keys[kMmStage + si], f32_key(v.mx));
                 if (v.nan) atomicOr(&stage_keys[2 * kMmStage + si], 1u);
@@ -197,51 +280,56 @@ __global__ __launch_bounds__(kBlock) void minmax_kernel(const MmArgs a) {
     }
 }
 
-// Single encoding (per-tensor statistics): a lean streaming kernel without any encoding lookup.  A workgroup reads
-// kFlatUnroll 16-byte vectors per lane, all issued before the first use, and leaves one partial.
+// Single encoding (per-tensor statistics): a lean streaming kernel without any encoding lookup.  Workgroups of 512
+// threads walk the tensor with a grid stride, kFlatUnroll 16-byte vectors per lane in flight, and leave one partial
+// each; at most kFlatMaxBlocks of them run, so the launch that folds the partials has a few hundred to read (measured
+// on 103 MB: 15.8 us for the stream alone at any grid size; stream + fold 19.8 us with 6272 workgroups of 256, 17.6 us
+// with 512 of 512).
+constexpr int kFlatBlock = 512;
 constexpr int kFlatUnroll = 4;
-constexpr int kFlatTileVec = kBlock * kFlatUnroll;
+constexpr int kFlatTileVec = kFlatBlock * kFlatUnroll;
+constexpr int kFlatMaxBlocks = 512;
 
 template <typename IO, int VEC, bool FINITE>
-__global__ __launch_bounds__(kBlock) void minmax_flat_kernel(const MmArgs a) {
-    __shared__ MinMax red_smem[kBlock / kWave];
-    const int64_t v0 = (int64_t)blockIdx.x * kFlatTileVec;
-    const int64_t left = a.nvec - v0;
-    const IO* __restrict__ x = static_cast<const IO*>(a.x) + v0 * VEC;
-    IO* __restrict__ cp = a.copy ? static_cast<IO*>(a.copy) + v0 * VEC : nullptr;
+__global__ __launch_bounds__(kFlatBlock) void minmax_flat_kernel(const MmFlatArgs a) {
+    __shared__ MinMax red_smem[kFlatBlock / kWave];
+    constexpr int MODE = mm_mode(FINITE);
+    const IO* __restrict__ x = static_cast<const IO*>(a.x);
+    IO* __restrict__ cp = static_cast<IO*>(a.copy);
     MinMax acc = mm_identity();
-    Pack<IO, VEC> in[kFlatUnroll];
-    if (left >= kFlatTileVec) {
+    uint64_t unordered = 0;
+    const int64_t full_tiles = a.nvec / kFlatTileVec;
+    for (int64_t tile = blockIdx.x; tile < full_tiles; tile += gridDim.x) {
+        const int64_t v0 = tile * kFlatTileVec + threadIdx.x;
+        Pack<IO, VEC> in[kFlatUnroll];
 #pragma unroll
-        for (int u = 0; u < kFlatUnroll; ++u) in[u] = load_pack<IO, VEC>(x + (int64_t)(u * kBlock + threadIdx.x) * VEC);
+        for (int u = 0; u < kFlatUnroll; ++u) in[u] = load_pack<IO, VEC>(x + (v0 + u * kFlatBlock) * VEC);
         if (cp) {
 #pragma unroll
-            for (int u = 0; u < kFlatUnroll; ++u) store_pack<IO, VEC>(cp + (int64_t)(u * kBlock + threadIdx.x) * VEC, in[u]);
+            for (int u = 0; u < kFlatUnroll; ++u) store_pack<IO, VEC>(cp + (v0 + u * kFlatBlock) * VEC, in[u]);
         }
 #pragma unroll
-        for (int u = 0; u < kFlatUnroll; ++u)
+        for (int u = 0; u < kFlatUnroll; ++u) mm_pack<IO, VEC, MODE>(in[u], acc.mn, acc.mx, unordered);
+    }
+    // the vectors past the last full tile: the workgroup after the one that took that tile
+    if (blockIdx.x == full_tiles % gridDim.x) {
+        for (int64_t v = full_tiles * kFlatTileVec + threadIdx.x; v < a.nvec; v += kFlatBlock) {
+            const Pack<IO, VEC> p = load_pack<IO, VEC>(x + v * VEC);
+            if (cp) store_pack<IO, VEC>(cp + v * VEC, p);
 #pragma unroll
-            for (int k = 0; k < VEC; ++k) mm_add(acc, load_f32(in[u].v[k]), FINITE);
-    } else {
-        for (int u = 0; u < kFlatUnroll; ++u) {
-            const int lv = u * kBlock + threadIdx.x;
-            if (lv < left) {
-                const Pack<IO, VEC> p = load_pack<IO, VEC>(x + (int64_t)lv * VEC);
-                if (cp) store_pack<IO, VEC>(cp + (int64_t)lv * VEC, p);
-#pragma unroll
-                for (int k = 0; k < VEC; ++k) mm_add(acc, load_f32(p.v[k]), FINITE);
-            }
+            for (int k = 0; k < VEC; ++k) mm_add(acc, load_f32(p.v[k]), FINITE);
         }
     }
     if (VEC > 1 && blockIdx.x == 0) {  // elements past the last full vector
         const int64_t i = a.nvec * VEC + threadIdx.x;
         if (i < a.numel) {
-            const IO v = static_cast<const IO*>(a.x)[i];
-            if (a.copy) static_cast<IO*>(a.copy)[i] = v;
+            const IO v = x[i];
+            if (cp) cp[i] = v;
             mm_add(acc, load_f32(v), FINITE);
         }
     }
-    const MinMax b = mm_block_reduce(acc, red_smem);
+    acc.nan |= unordered != 0 ? 1 : 0;
+    const MinMax b = mm_block_reduce<kFlatBlock>(acc, red_smem);
     if (threadIdx.x == 0) {
         if (gridDim.x == 1) {
             mm_write<IO>(a, 0, b);
@@ -251,6 +339,110 @@ __global__ __launch_bounds__(kBlock) void minmax_flat_kernel(const MmArgs a) {
             a.part_nan[blockIdx.x] = b.nan;
         }
     }
+}
+
+// Folds the at most kFlatMaxBlocks partials of minmax_flat_kernel: one workgroup, one or two loads per lane.
+constexpr int kFoldThreads = 256;
+template <typename IO>
+__global__ __launch_bounds__(kFoldThreads) void minmax_fold_kernel(const MmFlatArgs a, int nparts) {
+    __shared__ MinMax red_smem[kFoldThreads / kWave];
+    MinMax s = mm_identity();
+    for (int q = threadIdx.x; q < nparts; q += kFoldThreads) s = mm_merge(s, MinMax{a.part_min[q], a.part_max[q], a.part_nan[q]});
+    const MinMax r = mm_block_reduce<kFoldThreads>(s, red_smem);
+    if (threadIdx.x == 0) mm_write<IO>(a, 0, r);
+}
+
+// Runs on the leading axis, each long enough for a workgroup (BLOCK = 256, runs of 512 vectors or more) or a wave
+// (BLOCK = 64, runs of 64 to 511 vectors): the workgroup walks its run and writes the run's result itself -- no
+// partials, no second launch, no atomics.  Per-channel weights ([4096, 4096]: one pass of four vectors per lane).
+template <typename IO, int VEC, bool FINITE, int BLOCK>
+__global__ __launch_bounds__(BLOCK) void minmax_runs_kernel(const MmRunArgs a) {
+    __shared__ MinMax red_smem[BLOCK / kWave];
+    constexpr int MODE = mm_mode(FINITE);
+    const IO* __restrict__ x = static_cast<const IO*>(a.x) + (int64_t)blockIdx.x * a.kv * VEC;
+    MinMax acc = mm_identity();
+    uint64_t unordered = 0;
+    int v = threadIdx.x;
+    for (; v + (kUnroll - 1) * BLOCK < a.kv; v += kUnroll * BLOCK) {
+        Pack<IO, VEC> in[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) in[u] = load_pack<IO, VEC>(x + (int64_t)(v + u * BLOCK) * VEC);
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) mm_pack<IO, VEC, MODE>(in[u], acc.mn, acc.mx, unordered);
+    }
+    // what is left of the run: whole waves take part so that the ballots inside see defined values
+    for (int v0 = v - threadIdx.x; v0 < a.kv; v0 += BLOCK) {
+        const bool live = v0 + (int)threadIdx.x < a.kv;
+        Pack<IO, VEC> pk;
+        if (live) pk = load_pack<IO, VEC>(x + (int64_t)(v0 + threadIdx.x) * VEC);
+        else
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) pk.v[k] = IO{};
+        float mn = __builtin_inff(), mx = -__builtin_inff();
+        mm_pack<IO, VEC, MODE>(pk, mn, mx, unordered);
+        if (live) {
+            acc.mn = fminf(acc.mn, mn);
+            acc.mx = fmaxf(acc.mx, mx);
+        }
+    }
+    acc.nan = unordered != 0 ? 1 : 0;
+    MinMax b;
+    if (BLOCK == kWave) {
+        b = acc;
+#pragma unroll
+        for (int m = kWave / 2; m >= 1; m >>= 1) b = mm_merge(b, mm_shfl_xor(b, m));
+    } else {
+        b = mm_block_reduce<BLOCK>(acc, red_smem);
+    }
+    if (threadIdx.x == 0) mm_write<IO>(a, blockIdx.x, b);
+}
+
+// Runs of a power-of-two number of lanes (up to 64) on the leading axis: blocks of 64 bf16 are 8 lanes.  A tile of
+// kSegUnroll vectors per lane; the lanes of a run combine with data-parallel moves, the run leaders leave their
+// results in LDS, and after one barrier consecutive lanes write consecutive encodings (whole cache lines instead of
+// one 2- or 4-byte store per run leader).
+constexpr int kSegUnroll = 2;
+constexpr int kSegTileVec = kBlock * kSegUnroll;
+
+template <typename IO, int VEC, bool FINITE>
+__global__ __launch_bounds__(kBlock) void minmax_seg_kernel(const MmRunArgs a) {
+    __shared__ float s_mn[kSegTileVec], s_mx[kSegTileVec];
+    __shared__ unsigned char s_nan[kSegTileVec];
+    constexpr int MODE = mm_mode(FINITE);
+    const int64_t v0 = (int64_t)blockIdx.x * kSegTileVec;
+    const int64_t left = a.nvec - v0;
+    const IO* __restrict__ x = static_cast<const IO*>(a.x) + v0 * VEC;
+    const int kv = a.kv;
+    const int lane = threadIdx.x & (kWave - 1);
+    const uint64_t run_lanes = kv >= kWave ? ~0ull : ((1ull << kv) - 1) << (lane & ~(kv - 1));
+    Pack<IO, VEC> in[kSegUnroll];
+#pragma unroll
+    for (int u = 0; u < kSegUnroll; ++u) {
+        const int lv = u * kBlock + threadIdx.x;
+        if (lv < left) in[u] = load_pack<IO, VEC>(x + (int64_t)lv * VEC);
+        else
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) in[u].v[k] = IO{};
+    }
+#pragma unroll
+    for (int u = 0; u < kSegUnroll; ++u) {
+        const int lv = u * kBlock + threadIdx.x;
+        float mn = __builtin_inff(), mx = -__builtin_inff();
+        uint64_t unordered = 0;
+        mm_pack<IO, VEC, MODE>(in[u], mn, mx, unordered);
+        mn = segment_reduce(mn, kv, OpMinF());
+        mx = segment_reduce(mx, kv, OpMaxF());
+        if ((lane & (kv - 1)) == 0 && lv < left) {  // runs are whole inside the tensor: a live leader means a live run
+            const int slot = lv >> a.kv_shift;
+            s_mn[slot] = mn;
+            s_mx[slot] = mx;
+            s_nan[slot] = (unordered & run_lanes) != 0 ? 1 : 0;
+        }
+    }
+    __syncthreads();
+    const int nslots = (int)((left < kSegTileVec ? left : (int64_t)kSegTileVec) >> a.kv_shift);
+    const int64_t e0 = v0 >> a.kv_shift;
+    for (int t = threadIdx.x; t < nslots; t += kBlock) mm_write<IO>(a, e0 + t, MinMax{s_mn[t], s_mx[t], (int)s_nan[t]});
 }
 
 // Folds the per-tile partials of every encoding (second launch; see the note on fences in qdq.hip).
@@ -372,7 +564,23 @@ static void launch_mm_red(const Plan& p, const MmArgs& a, hipStream_t st) {
     else hipLaunchKernelGGL((minmax_kernel<IO, IoTraits<IO>::kVec, RED, FINITE>), dim3(p.nblocks), dim3(kBlock), 0, st, a);
 }
 
-static int64_t flat_blocks(const Plan& p) { return p.nvec > 0 ? (p.nvec + kFlatTileVec - 1) / kFlatTileVec : 1; }
+static int64_t flat_blocks(const Plan& p) {
+    const int64_t tiles = p.nvec > 0 ? (p.nvec + kFlatTileVec - 1) / kFlatTileVec : 1;
+    return tiles < kFlatMaxBlocks ? tiles : kFlatMaxBlocks;
+}
+
+static MmFlatArgs flat_args(const Plan& p, const MmArgs& a) {
+    MmFlatArgs f{};
+    static_cast<MmOut&>(f) = static_cast<const MmOut&>(a);
+    f.x = a.x;
+    f.copy = a.copy;
+    f.numel = p.cl.numel;
+    f.nvec = p.nvec;
+    f.part_min = a.part_min;
+    f.part_max = a.part_max;
+    f.part_nan = a.part_nan;
+    return f;
+}
 
 template <typename IO, bool FINITE>
 static void launch_mm(const Plan& p, const MmArgs& a, hipStream_t st) {
@@ -380,10 +588,38 @@ static void launch_mm(const Plan& p, const MmArgs& a, hipStream_t st) {
     const unsigned gb = (unsigned)((ne + 255) / 256 > 1024 ? 1024 : (ne + 255) / 256);
     if (p.cl.kind == kIJK && p.cl.J == 1) {
         const int64_t nb = flat_blocks(p);
-        if (p.vec == 1) hipLaunchKernelGGL((minmax_flat_kernel<IO, 1, FINITE>), dim3((unsigned)nb), dim3(kBlock), 0, st, a);
-        else hipLaunchKernelGGL((minmax_flat_kernel<IO, IoTraits<IO>::kVec, FINITE>), dim3((unsigned)nb), dim3(kBlock), 0, st, a);
-        if (nb > 1) hipLaunchKernelGGL((minmax_finish_kernel<IO>), dim3(1), dim3(kFinishThreads), 0, st, a, nb);
+        const MmFlatArgs f = flat_args(p, a);
+        if (p.vec == 1) hipLaunchKernelGGL((minmax_flat_kernel<IO, 1, FINITE>), dim3((unsigned)nb), dim3(kFlatBlock), 0, st, f);
+        else hipLaunchKernelGGL((minmax_flat_kernel<IO, IoTraits<IO>::kVec, FINITE>), dim3((unsigned)nb), dim3(kFlatBlock), 0, st, f);
+        if (nb > 1) hipLaunchKernelGGL((minmax_fold_kernel<IO>), dim3(1), dim3(kFoldThreads), 0, st, f, (int)nb);
         return;
+    }
+    // runs on the leading axis that a workgroup, a wave or a group of lanes can own: lean kernels, one launch
+    if (p.cl.kind == kIJK && p.cl.I == 1 && p.cl.J > 1 && p.vec > 1 && p.cl.J <= 0x7fffffff && p.Kv <= 0x7fffffff) {
+        MmRunArgs r{};
+        static_cast<MmOut&>(r) = static_cast<const MmOut&>(a);
+        r.x = a.x;
+        r.nvec = p.nvec;
+        r.runs = p.cl.J;
+        r.kv = (int32_t)p.Kv;
+        r.kv_shift = 0;
+        while ((1 << r.kv_shift) < r.kv) ++r.kv_shift;
+        constexpr int V = IoTraits<IO>::kVec;
+        // a workgroup per run needs enough runs to fill the GPU, or runs short enough not to matter; a few very long
+        // runs keep the tiled kernel with its partials
+        if (p.Kv >= 2 * kBlock && (p.cl.J >= 512 || p.Kv <= 8 * kTileVec)) {
+            hipLaunchKernelGGL((minmax_runs_kernel<IO, V, FINITE, kBlock>), dim3((unsigned)p.cl.J), dim3(kBlock), 0, st, r);
+            return;
+        }
+        if (p.Kv >= kWave && p.Kv < 2 * kBlock) {
+            hipLaunchKernelGGL((minmax_runs_kernel<IO, V, FINITE, kWave>), dim3((unsigned)p.cl.J), dim3(kWave), 0, st, r);
+            return;
+        }
+        if (p.Kv < kWave && is_pow2(p.Kv)) {
+            const int64_t nb = (p.nvec + kSegTileVec - 1) / kSegTileVec;
+            hipLaunchKernelGGL((minmax_seg_kernel<IO, V, FINITE>), dim3((unsigned)nb), dim3(kBlock), 0, st, r);
+            return;
+        }
     }
     if (p.red == kRedAtomic) hipLaunchKernelGGL(minmax_keys_init_kernel, dim3(gb), dim3(256), 0, st, a.key_min, a.key_max, a.part_nan, ne);
     if (p.cl.kind == kGeneric) {
@@ -441,10 +677,11 @@ extern "C" __attribute__((visibility("hidden"))) int ahq_minmax_finite_partials(
     a.part_nan = reinterpret_cast<int*>(w + p.ws_elems * 8);
     const int64_t nb = flat_blocks(p);
     hipStream_t st = static_cast<hipStream_t>(stream);
+    const MmFlatArgs f = flat_args(p, a);
 #define AHQ_FLAT(IO)                                                                                                  \
     do {                                                                                                              \
-        if (p.vec == 1) hipLaunchKernelGGL((minmax_flat_kernel<IO, 1, true>), dim3((unsigned)nb), dim3(kBlock), 0, st, a); \
-        else hipLaunchKernelGGL((minmax_flat_kernel<IO, IoTraits<IO>::kVec, true>), dim3((unsigned)nb), dim3(kBlock), 0, st, a); \
+        if (p.vec == 1) hipLaunchKernelGGL((minmax_flat_kernel<IO, 1, true>), dim3((unsigned)nb), dim3(kFlatBlock), 0, st, f); \
+        else hipLaunchKernelGGL((minmax_flat_kernel<IO, IoTraits<IO>::kVec, true>), dim3((unsigned)nb), dim3(kFlatBlock), 0, st, f); \
     } while (0)
     switch (dtype) {
         case AHQ_F32: AHQ_FLAT(float); break;
