@@ -204,6 +204,14 @@ class QuantizedLinear(nn.Linear):
         them through unquantized, and set their ranges on exit."""
         self._compute_param_encodings(overwrite=True, verdicts=_verdicts)
         with contextlib.ExitStack() as stack:
+            # Neither the parameters nor their (just computed) encodings change inside the context, so the
+            # quantize-dequantized parameters are the same in every calibration pass: they are formed once here and
+            # the passes use them (the reference calls the parameter quantizers again in every pass, with the same
+            # result; its own _patch_quantized_parameters / fold_param_quantizers, nn/base.py:296-324, 1103-1151, are
+            # the same trade).  A caller that modifies a parameter in place inside the context sees the old values.
+            if any(q is not None and q.is_initialized() for q in self.param_quantizers.values()):
+                stack.enter_context(self._patch_quantized_parameters())
+                stack.enter_context(self._remove_param_quantizers())
             for qtzr in list(self.input_quantizers) + list(self.output_quantizers):
                 if not isinstance(qtzr, QuantizerBase) or not qtzr.is_overwrite_allowed():
                     continue

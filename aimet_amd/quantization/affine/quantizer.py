@@ -144,7 +144,7 @@ class AffineQuantizerBase(QuantizerBase, _GridMixin):
             return None
         dtype = dtype or torch.float32
         if self.symmetric:
-            device = next(p.device for p in self.parameters())
+            device = self.min.device
             return _symmetric_offset(self.qmin, self.qmax, self.shape, dtype, device)
         scale = scale if scale is not None else self.get_scale(dtype)
         offset = torch.clamp(ste_round(self.min / scale) - self.qmin, -self.qmax, -self.qmin)
@@ -304,10 +304,7 @@ class AffineQuantizerBase(QuantizerBase, _GridMixin):
             return
         inner_forward = torch.Tensor.clone if passthrough else self.forward
         shape = self.shape
-        try:
-            dtype, device = next((p.dtype, p.device) for p in self.parameters())
-        except StopIteration as e:
-            raise RuntimeError from e
+        dtype, device = self.min.dtype, self.min.device
 
         @functools.wraps(inner_forward)
         def observing_forward(input: torch.Tensor) -> torch.Tensor:
@@ -318,10 +315,10 @@ class AffineQuantizerBase(QuantizerBase, _GridMixin):
             if passthrough:
                 # the input is only observed; the dynamic encodings of this batch would go unused.  A min/max
                 # analyzer writes the clone from the pass that reads the tensor
-                fused = getattr(self.encoding_analyzer, "update_stats_and_clone", None)
+                fused = getattr(self.encoding_analyzer, "observe_and_clone", None)
                 if (fused is not None and input.is_cuda and input.dtype in _lib.DTYPE_CODE and input.is_contiguous()
                         and not (torch.is_grad_enabled() and input.requires_grad)):
-                    return fused(input)[1]
+                    return fused(input)
                 self.encoding_analyzer.update_stats(input)
                 return inner_forward(input)
             batch_stats = self.encoding_analyzer.update_stats(input)
@@ -389,7 +386,7 @@ class AffineQuantizerBase(QuantizerBase, _GridMixin):
             yield
 
     def _get_dummy_encoding(self) -> AffineEncoding:
-        device = next(p.device for p in self.parameters())
+        device = self.min.device
         return AffineEncoding(torch.ones((), device=device), torch.zeros((), device=device), self.qmin, self.qmax,
                               self._symmetric, block_size=None, zero_point_shift=self.zero_point_shift, producer=self)
 

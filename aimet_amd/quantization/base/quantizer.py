@@ -45,7 +45,16 @@ class QuantizerBase(abc.ABC, torch.nn.Module):
 
     def is_initialized(self, name: Optional[str] = None) -> bool:
         """True if every quantization parameter (or the named one) has been given a value."""
-        return all(self._is_initialized(n, p) for n, p in self.named_parameters() if name is None or n == name)
+        # a quantizer's parameters are its own (no sub-modules hold any): the dictionary is walked directly, which is
+        # an order of magnitude cheaper than named_parameters() and this runs several times per forward pass
+        params = self._parameters
+        if name is not None:
+            p = params.get(name)
+            return p is None or self._is_initialized(name, p)
+        for n, p in params.items():
+            if p is not None and not self._is_initialized(n, p):
+                return False
+        return True
 
     def _is_initialized(self, param_name: str, current: nn.Parameter) -> bool:
         ref, version = self._initial_parameters.get(param_name, (None, None))

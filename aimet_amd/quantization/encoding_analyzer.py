@@ -157,8 +157,43 @@ class _MinMaxObserver(_Observer[_MinMaxRange]):
         self.merge_stats(new)
         return new
 
+    @torch.no_grad()
+    def observe_and_clone(self, input_tensor: torch.Tensor) -> torch.Tensor:
+        """update() for a caller that throws the batch's own statistics away and wants a copy of the input (the
+        pass-through calibration of a whole model: hundreds of these per forward pass).  Once the running statistics
+        exist, everything that does not change from call to call -- layout, workspace, the two tensors the batch's
+        extrema are written to -- is kept, and a call is one allocation (the copy) and one library call."""
+        fast = self.__dict__.get("_fast")
+        cur = self.stats
+        x = input_tensor
+        key = (x.shape, x.dtype, x.device)
+        if (fast is None or fast[0] != key or fast[1] is not cur.min or fast[2] is not cur.max or not x.is_contiguous()
+                or x.requires_grad):
+            out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+            self.update(x, copy_to=out)
+            cur = self.stats
+            self.__dict__["_fast"] = None
+            if (x.is_contiguous() and x.is_cuda and cur.min is not None and cur.min.dtype == x.dtype
+                    and cur.min.device == x.device and cur.min.is_contiguous() and cur.max.is_contiguous()):
+                lib = _lib.load()
+                _, layout = _prepare(x.detach(), self.shape, self.block_size)
+                nbytes = lib.ahq_minmax_workspace_bytes(layout)
+                ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=x.device)
+                bmin, bmax = torch.empty_like(cur.min), torch.empty_like(cur.max)
+                self.__dict__["_fast"] = (key, cur.min, cur.max, layout, ws, nbytes, bmin, bmax, _lib.DTYPE_CODE[x.dtype],
+                                          lib.ahq_minmax_copy)
+            return out
+        _, rmin, rmax, layout, ws, nbytes, bmin, bmax, code, entry = fast
+        out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+        status = entry(code, layout, x.data_ptr(), out.data_ptr(), bmin.data_ptr(), bmax.data_ptr(), rmin.data_ptr(),
+                       rmax.data_ptr(), 0, ws.data_ptr(), nbytes, _lib.current_stream(x.device))
+        if status:
+            _lib.check(status, "ahq_minmax_copy")
+        return out
+
     def reset_stats(self):
         self.stats = _MinMaxRange()
+        self.__dict__["_fast"] = None
 
     def get_stats(self) -> _MinMaxRange:
         return self.stats
@@ -333,6 +368,10 @@ class MinMaxEncodingAnalyzer(EncodingAnalyzer[_MinMaxRange]):
         """update_stats(input) and input.clone() with one read of the tensor.  Returns (batch statistics, clone)."""
         out = torch.empty(input_tensor.shape, dtype=input_tensor.dtype, device=input_tensor.device)
         return self.observer.update(input_tensor, copy_to=out), out
+
+    def observe_and_clone(self, input_tensor: torch.Tensor) -> torch.Tensor:
+        """update_stats(input) whose result nobody reads, and input.clone(), with one read of the tensor."""
+        return self.observer.observe_and_clone(input_tensor)
 
     @torch.no_grad()
     def compute_encodings_from_stats(self, stats: _MinMaxRange, num_steps: int, is_symmetric: bool):
