@@ -138,6 +138,10 @@ _SIGNATURES = {
                                        ctypes.c_float, _P]),
     "ahq_float_qdq": (ctypes.c_int, [ctypes.c_int32, ctypes.POINTER(Layout), _P, _P, _P, ctypes.c_int32, ctypes.c_int32,
                                      ctypes.c_float, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32, _P]),
+    "ahq_float_quantize": (ctypes.c_int, [ctypes.c_int32, ctypes.POINTER(Layout), _P, _P, _P, ctypes.c_int32,
+                                          ctypes.c_int32, ctypes.c_float, ctypes.c_int32, ctypes.c_int32,
+                                          ctypes.c_int32, _P]),
+    "ahq_float_dequantize": (ctypes.c_int, [ctypes.c_int32, ctypes.POINTER(Layout), _P, _P, _P, _P]),
     "ahq_dlq_percentile_encodings": (ctypes.c_int, [ctypes.POINTER(DlqPdfState), ctypes.c_float, ctypes.c_int32,
                                                     ctypes.c_int32, ctypes.c_int32, ctypes.c_int32, _P, _P]),
     "ahq_dlq_tfe_encodings": (ctypes.c_int, [ctypes.POINTER(DlqPdfState), ctypes.c_int32, ctypes.c_int32, ctypes.c_int32,

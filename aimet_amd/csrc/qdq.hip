@@ -32,6 +32,8 @@ struct GridC {
 constexpr int kCastOverflowNaN = 1;    // a value that rounds past the largest one becomes NaN (else infinity)
 constexpr int kCastUnsignedZero = 2;   // the format has no negative zero
 constexpr int kCastLogForm = 4;        // 16-bit tensors: the reference's logarithm formula, rounded step by step
+constexpr int kCastKeepScaled = 8;     // stop before the multiplication by the scale (quantize only)
+constexpr int kCastRescaleOnly = 16;   // only the multiplication by the scale (dequantize)
 
 struct EncP {
     float p0, p1, p2, p3;
@@ -320,6 +322,8 @@ struct MathFloatCast {
     template <bool FAST>
     __device__ static float fwd(float x, const EncP& e, const GridC& g, bool& inr) {
         inr = true;
+        if (g.flags & kCastRescaleOnly) return x * e.p0;  // last rounding by the caller
+        const float back = (g.flags & kCastKeepScaled) ? 1.f : e.p0;
         float t = rnd<CD>(divide<FAST, AHQ_F32>(x, e.p0, e.rs));
         // the corrected quotient of divide<true> does not keep the sign of a zero
         if (FAST && t == 0.f) t = bits_to_f32((f32_to_bits(x) ^ f32_to_bits(e.p0)) & 0x80000000u);
@@ -340,7 +344,7 @@ struct MathFloatCast {
                 const float ex2 = rnd<CD>(rnd<CD>(ls - g.zps) - bias);
                 const float sc = rnd<CD>(__builtin_exp2f(ex2));
                 const float q = rnd<CD>(t / sc);
-                return rnd<CD>(__builtin_rintf(q) * sc) * e.p0;  // last rounding by the caller
+                return rnd<CD>(__builtin_rintf(q) * sc) * back;  // last rounding by the caller
             }
         }
         int ex = __builtin_amdgcn_frexp_expf(t) - 1;
@@ -350,7 +354,7 @@ struct MathFloatCast {
         if (__builtin_fabsf(v) > g.qmax)
             v = (g.flags & kCastOverflowNaN) ? __builtin_nanf("") : __builtin_copysignf(__builtin_inff(), v);
         if ((g.flags & kCastUnsignedZero) && v == 0.f) v = 0.f;
-        return rnd<CD>(v) * e.p0;  // last rounding by the caller
+        return rnd<CD>(v) * back;  // last rounding by the caller
     }
     template <bool FAST>
     __device__ static void bwd(float, float, const EncP&, const GridC&, float& gx, float& gs, float& goff) {
@@ -1183,13 +1187,14 @@ extern "C" int ahq_dlq_fp8_qdq_per_tensor(int32_t dtype, const void* x, void* y,
     return check_launch("ahq_dlq_fp8_qdq_per_tensor");
 }
 
-extern "C" int ahq_float_qdq(int32_t dtype, const ahq_layout* layout, const void* x, void* y, const float* scale,
-                             int32_t mantissa_bits, int32_t exponent_min, float max_value, int32_t overflow_to_nan,
-                             int32_t unsigned_zero, int32_t logarithm_form, void* stream) {
+static int float_cast_impl(const char* what, int stage_flags, int32_t dtype, const ahq_layout* layout, const void* x,
+                           void* y, const float* scale, int32_t mantissa_bits, int32_t exponent_min, float max_value,
+                           int32_t overflow_to_nan, int32_t unsigned_zero, int32_t logarithm_form, void* stream) {
     if (dtype < AHQ_F32 || dtype > AHQ_BF16) return set_error("bad dtype"), AHQ_ERR_INVALID;
     if (!layout) return set_error("layout is null"), AHQ_ERR_INVALID;
     if (!scale) return set_error("scale is null"), AHQ_ERR_INVALID;
-    if (mantissa_bits < 0 || mantissa_bits > 23 || exponent_min < -126 || exponent_min > 127 || !(max_value > 0.f))
+    if (!(stage_flags & kCastRescaleOnly) &&
+        (mantissa_bits < 0 || mantissa_bits > 23 || exponent_min < -126 || exponent_min > 127 || !(max_value > 0.f)))
         return set_error("bad float format description"), AHQ_ERR_INVALID;
     Plan p;
     if (!make_plan(dtype, *layout, aligned16(x) && aligned16(y), false, &p, kFwdUnroll)) return AHQ_ERR_INVALID;
@@ -1206,12 +1211,33 @@ extern "C" int ahq_float_qdq(int32_t dtype, const ahq_layout* layout, const void
     a.gc.qmax = max_value;
     a.gc.zps = (float)mantissa_bits;
     a.gc.flags = (overflow_to_nan ? kCastOverflowNaN : 0) | (unsigned_zero ? kCastUnsignedZero : 0) |
-                 (logarithm_form ? kCastLogForm : 0);
+                 (logarithm_form ? kCastLogForm : 0) | stage_flags;
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (dtype == AHQ_F32) launch_fwd<float, MathFloatCast<AHQ_F32>>(p, a, st, aligned16(x) && aligned16(y));
     else if (dtype == AHQ_F16) launch_fwd<f16_t, MathFloatCast<AHQ_F16>>(p, a, st, aligned16(x) && aligned16(y));
     else launch_fwd<bf16_t, MathFloatCast<AHQ_BF16>>(p, a, st, aligned16(x) && aligned16(y));
-    return check_launch("ahq_float_qdq");
+    return check_launch(what);
+}
+
+extern "C" int ahq_float_qdq(int32_t dtype, const ahq_layout* layout, const void* x, void* y, const float* scale,
+                             int32_t mantissa_bits, int32_t exponent_min, float max_value, int32_t overflow_to_nan,
+                             int32_t unsigned_zero, int32_t logarithm_form, void* stream) {
+    return float_cast_impl("ahq_float_qdq", 0, dtype, layout, x, y, scale, mantissa_bits, exponent_min, max_value,
+                           overflow_to_nan, unsigned_zero, logarithm_form, stream);
+}
+
+extern "C" int ahq_float_quantize(int32_t dtype, const ahq_layout* layout, const void* x, void* y, const float* scale,
+                                  int32_t mantissa_bits, int32_t exponent_min, float max_value,
+                                  int32_t overflow_to_nan, int32_t unsigned_zero, int32_t logarithm_form,
+                                  void* stream) {
+    return float_cast_impl("ahq_float_quantize", kCastKeepScaled, dtype, layout, x, y, scale, mantissa_bits,
+                           exponent_min, max_value, overflow_to_nan, unsigned_zero, logarithm_form, stream);
+}
+
+extern "C" int ahq_float_dequantize(int32_t dtype, const ahq_layout* layout, const void* x, void* y,
+                                    const float* scale, void* stream) {
+    return float_cast_impl("ahq_float_dequantize", kCastRescaleOnly, dtype, layout, x, y, scale, 0, 0, 1.f, 0, 0, 0,
+                           stream);
 }
 
 extern "C" size_t ahq_qdq_backward_workspace_bytes(const ahq_grid* grid, const ahq_layout* layout, int want_param_grads) {

@@ -73,7 +73,25 @@ class FloatEncoding(EncodingBase):
                              self.scale.to(dtype=dtype, device=device), self.block_size, producer=self.producer)
 
     def quantize(self, input: torch.Tensor) -> torch.Tensor:  # pylint: disable=redefined-builtin
-        raise NotImplementedError
+        """float/encoding.py:140-152: the values the format stores, ``cast(clamp(input / scale))``."""
+        from .quantizer import float_quantize
+
+        if type(input) is not torch.Tensor:  # pylint: disable=unidiomatic-typecheck
+            input = input.as_subclass(torch.Tensor)
+        return float_quantize(input, self._finfo, self.scale, self.block_size)
 
     def dequantize(self, input: torch.Tensor) -> torch.Tensor:  # pylint: disable=redefined-builtin
-        raise NotImplementedError
+        """float/encoding.py:154-165: ``input * scale`` blockwise."""
+        from .quantizer import float_dequantize
+
+        if type(input) is not torch.Tensor:  # pylint: disable=unidiomatic-typecheck
+            input = input.as_subclass(torch.Tensor)
+        return float_dequantize(input, self.scale, self.block_size)
+
+    def quantize_dequantize(self, input: torch.Tensor) -> torch.Tensor:  # pylint: disable=redefined-builtin
+        """float/encoding.py:167-178."""
+        from .quantizer import float_quantize_dequantize
+
+        if type(input) is not torch.Tensor:  # pylint: disable=unidiomatic-typecheck
+            input = input.as_subclass(torch.Tensor)
+        return float_quantize_dequantize(input, self._finfo, self.scale, self.block_size)

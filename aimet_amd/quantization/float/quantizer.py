@@ -27,10 +27,11 @@ from aimet_amd.quantization.tensor import DequantizedTensor
 from ._finfo import _finfo, _float4_e2m1fn, _torch_dtype_to_finfo
 from .encoding import FloatEncoding
 
-__all__ = ["FloatQuantizeDequantize", "QuantizeDequantize", "float_quantize_dequantize"]
+__all__ = ["FloatQuantizeDequantize", "QuantizeDequantize", "float_quantize_dequantize", "float_quantize",
+           "float_dequantize"]
 
 
-def _launch(x: torch.Tensor, finfo: _finfo, scale: torch.Tensor, block_size) -> torch.Tensor:
+def _launch(x: torch.Tensor, finfo: _finfo, scale: torch.Tensor, block_size, entry: str = "ahq_float_qdq") -> torch.Tensor:
     lib = _lib.load()
     x, layout = _hip._prepare(x, scale.shape, block_size)  # pylint: disable=protected-access
     y = torch.empty_like(x)
@@ -40,10 +41,42 @@ def _launch(x: torch.Tensor, finfo: _finfo, scale: torch.Tensor, block_size) -> 
         # a format without a storage type goes through the reference's logarithm formula, whose steps round to the
         # tensor's dtype: on 16-bit tensors that differs from an exact cast next to binade boundaries
         log_form = finfo.to_torch_dtype() is None and x.dtype != torch.float32
-        _lib.check(lib.ahq_float_qdq(_lib.DTYPE_CODE[x.dtype], layout, x.data_ptr(), y.data_ptr(), s.data_ptr(), mbits,
-                                     emin, mx, int(overflow_nan), int(uz), int(log_form),
-                                     _lib.current_stream(x.device)),
-                   "ahq_float_qdq")
+        _lib.check(getattr(lib, entry)(_lib.DTYPE_CODE[x.dtype], layout, x.data_ptr(), y.data_ptr(), s.data_ptr(), mbits,
+                                       emin, mx, int(overflow_nan), int(uz), int(log_form),
+                                       _lib.current_stream(x.device)),
+                   entry)
+    return y
+
+
+def _checked_operands(input: torch.Tensor, scale: torch.Tensor):  # pylint: disable=redefined-builtin
+    _lib.require_device(input, "input")
+    dtype = torch.result_type(input, scale)
+    if dtype not in _lib.DTYPE_CODE:
+        raise RuntimeError(f"float fake-cast computes in float32, float16 or bfloat16; got {dtype}")
+    return (input if input.dtype == dtype else input.to(dtype)).detach(), scale.to(input.device)
+
+
+def float_quantize(input: torch.Tensor, finfo: _finfo, scale: torch.Tensor, block_size=None) -> torch.Tensor:  # pylint: disable=redefined-builtin
+    """_float_quantize (float/quantizer.py:687-706): ``cast(clamp(input / scale, -max, max))``, i.e. the value the
+    simulated format stores.  No gradient is formed (FloatEncoding.quantize is its only caller)."""
+    if finfo.to_torch_dtype() is None and finfo.unsigned_zero:
+        raise NotImplementedError(f"Fake-casting to {finfo.to_str()} is not implemented")
+    x, scale = _checked_operands(input, scale)
+    if finfo.max > torch.finfo(x.dtype).max:
+        raise RuntimeError(f"value cannot be converted to type {x.dtype} without overflow")
+    return _launch(x, finfo, scale, tuple(block_size) if block_size else None, "ahq_float_quantize")
+
+
+def float_dequantize(input: torch.Tensor, scale: torch.Tensor, block_size=None) -> torch.Tensor:  # pylint: disable=redefined-builtin
+    """FloatEncoding.dequantize (float/encoding.py:154-165): ``input * scale`` blockwise."""
+    x, scale = _checked_operands(input, scale)
+    lib = _lib.load()
+    x, layout = _hip._prepare(x, scale.shape, tuple(block_size) if block_size else None)  # pylint: disable=protected-access
+    y = torch.empty_like(x)
+    if x.numel():
+        s = _hip._enc_f32(scale)  # pylint: disable=protected-access
+        _lib.check(lib.ahq_float_dequantize(_lib.DTYPE_CODE[x.dtype], layout, x.data_ptr(), y.data_ptr(), s.data_ptr(),
+                                            _lib.current_stream(x.device)), "ahq_float_dequantize")
     return y
 
 

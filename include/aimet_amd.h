@@ -353,6 +353,21 @@ int ahq_float_qdq(int32_t dtype, const ahq_layout* layout, const void* x, void* 
                   int32_t mantissa_bits, int32_t exponent_min, float max_value, int32_t overflow_to_nan,
                   int32_t unsigned_zero, int32_t logarithm_form, void* stream);
 
+/* Replaces _float_quantize of aimet_torch (aimet_torch/quantization/float/quantizer.py:687-706), which
+ * FloatEncoding.quantize calls (aimet_torch/quantization/float/encoding.py:140-152): ahq_float_qdq without its last
+ * multiplication, y = cast(clamp(x / scale, -max_value, max_value)); same arguments, same arithmetic.
+ */
+int ahq_float_quantize(int32_t dtype, const ahq_layout* layout, const void* x, void* y, const float* scale,
+                       int32_t mantissa_bits, int32_t exponent_min, float max_value, int32_t overflow_to_nan,
+                       int32_t unsigned_zero, int32_t logarithm_form, void* stream);
+
+/* Replaces FloatEncoding.dequantize of aimet_torch (aimet_torch/quantization/float/encoding.py:154-165, a blockwise
+ * torch.mul): y = x * scale, the product formed in float and rounded once to `dtype`; scale: one float per encoding
+ * of the layout.
+ */
+int ahq_float_dequantize(int32_t dtype, const ahq_layout* layout, const void* x, void* y, const float* scale,
+                         void* stream);
+
 /* Replaces PercentileEncodingAnalyzer::computeEncoding (DLQ/src/PercentileEncodingAnalyzer.cpp:52-169) on the same PDF
  * statistics: the range that keeps `percentile` percent of the probability mass on each side, widened to contain
  * zero, then getComputedEncodings.  out: [num_slots][5].

@@ -651,9 +651,9 @@ def fake_cast_to_ieee_float(x, maxval, exponent_bits, mantissa_bits, finite=True
     return out.to(x.dtype)
 
 
-def float_qdq(x, scale, exponent_bits, mantissa_bits, finite, unsigned_zero, block_size=None):
-    """_float_quantize_dequantize (float/quantizer.py:634-716): divide, clamp, fake-cast, multiply, every step a torch
-    op on the promoted dtype of (x, scale)."""
+def float_quantize(x, scale, exponent_bits, mantissa_bits, finite, unsigned_zero, block_size=None):
+    """_float_quantize (float/quantizer.py:687-706): divide, clamp, fake-cast, every step a torch op on the promoted
+    dtype of (x, scale)."""
     key = (exponent_bits, mantissa_bits, finite, unsigned_zero)
     mx = float_max(*key)
     shape = x.shape
@@ -661,12 +661,21 @@ def float_qdq(x, scale, exponent_bits, mantissa_bits, finite, unsigned_zero, blo
     t = torch.div(xb, sb).reshape(shape) if block_size else torch.div(x, scale)
     t = t.clamp(-mx, mx)
     if key in FLOAT_TORCH_DTYPES:
-        t = t.to(FLOAT_TORCH_DTYPES[key]).to(t.dtype)
-    elif not unsigned_zero:
-        t = fake_cast_to_ieee_float(t, mx, exponent_bits, mantissa_bits, finite=finite)
-    else:
-        raise NotImplementedError("Fake-casting to this format is not implemented")
+        return t.to(FLOAT_TORCH_DTYPES[key]).to(t.dtype)
+    if not unsigned_zero:
+        return fake_cast_to_ieee_float(t, mx, exponent_bits, mantissa_bits, finite=finite)
+    raise NotImplementedError("Fake-casting to this format is not implemented")
+
+
+def float_dequantize(t, scale, block_size=None):
+    """FloatEncoding.dequantize (float/encoding.py:154-165): blockwise torch.mul."""
     if block_size:
         tb, sb, _ = _blocked_views(t, scale, None, block_size)
-        return torch.mul(tb, sb).reshape(shape)
+        return torch.mul(tb, sb).reshape(t.shape)
     return torch.mul(t, scale)
+
+
+def float_qdq(x, scale, exponent_bits, mantissa_bits, finite, unsigned_zero, block_size=None):
+    """_float_quantize_dequantize (float/quantizer.py:634-656): quantize, then multiply by the scale."""
+    t = float_quantize(x, scale, exponent_bits, mantissa_bits, finite, unsigned_zero, block_size)
+    return float_dequantize(t, scale, block_size)

@@ -82,6 +82,35 @@ def test_kernel_matches_the_restatement(device, name, dtype, shape, scale_shape,
     assert_same_bits(got, want, name)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=lambda d: str(d)[6:])
+@pytest.mark.parametrize("name", list(FORMATS))
+@pytest.mark.parametrize("shape,scale_shape,block", [((4099,), (), None), ((64, 515), (64, 1), None),
+                                                     ((32, 256), (32, 4), (1, 64))])
+def test_encoding_quantize_and_dequantize_match_the_restatement(device, name, dtype, shape, scale_shape, block):
+    """FloatEncoding.quantize / dequantize / quantize_dequantize (float/encoding.py:140-178) bit for bit, and
+    dequantize(quantize(x)) is quantize_dequantize(x)."""
+    from aimet_amd.quantization.float.encoding import FloatEncoding
+
+    fmt, _ = FORMATS[name]
+    mx = O.float_max(*fmt)
+    x = _data(shape, dtype, seed=len(name) * 5 + len(shape), span=min(mx, 3e4))
+    g = torch.Generator().manual_seed(23)
+    scale = torch.exp(torch.rand(scale_shape, generator=g) * 6 - 4)
+    enc = FloatEncoding(fmt[1], fmt[0], fmt[2], fmt[3], scale.to(device), block)
+    if mx > torch.finfo(torch.result_type(x, scale)).max:
+        with pytest.raises(RuntimeError, match="without overflow"):
+            enc.quantize(x.to(device))
+        return
+    want_q = O.float_quantize(x, scale, *fmt, block_size=block)
+    got_q = enc.quantize(x.to(device))
+    assert got_q.dtype == want_q.dtype
+    assert_same_bits(got_q, want_q, name)
+    want = O.float_dequantize(want_q, scale, block)
+    got = enc.dequantize(got_q)
+    assert_same_bits(got, want, name)
+    assert_same_bits(enc.quantize_dequantize(x.to(device)), want, name)
+
+
 def test_bfloat16_tensor_cast_to_float16_overflows_like_the_conversion(device):
     """The clamp bound 65504 becomes 65536 in bfloat16 (a Python scalar against a bfloat16 tensor), so the largest
     inputs convert to infinity."""

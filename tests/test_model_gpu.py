@@ -127,13 +127,38 @@ def test_param_encodings_are_computed_lazily_on_first_call(device):
     assert wq.is_initialized()
 
 
-def test_prequantized_weight_is_reported(device):
+@pytest.mark.parametrize("bitwidth", [2, 4])
+def test_prequantized_weight_keeps_its_grid(device, bitwidth):
+    """test_prequantized_weight (TrainingExtensions/torch/test/python/v2/nn/test_true_quant.py:2456-2475): a weight
+    built from codes in {-1, 0, 1} and per-channel scales 0.01 ... 0.10 gets exactly those scales -- min/max
+    calibration would give absmax / 2^(bw-1), a different grid on which the weight is not representable."""
+    qmin, qmax = -(2 ** (bitwidth - 1)), 2 ** (bitwidth - 1) - 1
+    lin = qnn.QuantizedLinear(10, 10, bias=False).to(device)
+    weight_scale = torch.arange(0.01, 0.11, step=0.01, dtype=torch.float32, device=device).view(10, 1)
+    g = torch.Generator().manual_seed(bitwidth)
+    with torch.no_grad():
+        lin.weight.copy_(torch.randint(-1, 2, (10, 10), generator=g).float().to(device) * weight_scale)
+    wq = QuantizeDequantize((10, 1), qmin=qmin, qmax=qmax, symmetric=True).to(device)
+    lin.param_quantizers["weight"] = wq
+    with torch.no_grad():
+        lin._compute_param_encodings(overwrite=True)
+        assert torch.allclose(wq.get_scale(), weight_scale)
+        assert torch.allclose(wq(lin.weight), lin.weight, rtol=1e-6, atol=0)  # lossless
+
+
+def test_weight_that_passes_the_probe_but_is_on_no_grid_is_calibrated(device):
+    """Few distinct magnitudes with irrational ratios: the recovery refuses and min/max calibration takes over."""
+    g = torch.Generator().manual_seed(0)
+    values = torch.tensor([1.0, 2.0 ** 0.5, 3.0 ** 0.5, 7.0 ** 0.5])
+    w = values[torch.randint(0, 4, (8, 64), generator=g)] * (torch.randint(0, 2, (8, 64), generator=g) * 2.0 - 1)
     lin = qnn.QuantizedLinear(64, 8, bias=False).to(device)
     with torch.no_grad():
-        lin.weight.copy_(torch.randint(-8, 8, (8, 64)).float() * 0.125)
-    lin.param_quantizers["weight"] = QuantizeDequantize((8, 1), 4, symmetric=True).to(device)
-    with pytest.raises(NotImplementedError):
+        lin.weight.copy_(w)
+    wq = QuantizeDequantize((8, 1), 4, symmetric=True).to(device)
+    lin.param_quantizers["weight"] = wq
+    with torch.no_grad():
         lin(torch.randn(2, 64, device=device))
+        assert torch.allclose(wq.get_scale(), lin.weight.abs().amax(dim=1, keepdim=True) / 7)  # max / qmax
 
 
 def _calibrated_copy(device, seed=5):

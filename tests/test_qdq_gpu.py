@@ -464,3 +464,35 @@ def test_offset_and_scale_of_different_shapes_broadcast(device, dtype, case):
     assert_same_bits(y2.as_subclass(torch.Tensor), tr.y, "output without gradients")
     q = affine.quantize(x.float().to(device), scale.to(device), offset.to(device), 0, 255)
     assert_same_bits(q.as_subclass(torch.Tensor), O.quantize_forward(x.float(), scale, offset, 0, 255)[0], "codes")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=lambda d: str(d).split(".")[-1])
+@pytest.mark.parametrize("layout", [
+    ((8, 100), (8, 1), None),               # runs shorter than a tile
+    ((256, 4096), (256, 1), None),          # runs of a quarter / an eighth of a tile
+    ((4, 6, 10, 10), (6, 1, 1), None),      # short runs, each encoding met several times
+    ((8, 16), (2, 4), (4, 4)),              # generic walk
+    ((1100, 264), (1, 264), None),          # column-walking kernel
+    ((3, 40, 1536), (1536,), None),
+], ids=lambda l: "x".join(map(str, l[0])) + "_" + "x".join(map(str, l[1])))
+def test_parameter_gradients_repeat_on_layouts_that_sum_with_atomics(device, layout, dtype):
+    """Where one encoding's terms are spread over workgroups with no fixed meeting order, the scale / offset gradients
+    are summed with 64-bit floating-point atomics, whose order varies between runs.  The terms are float32 values
+    added in double precision, so two runs differ by about 1e-16 of the sum of magnitudes before the final rounding to
+    the compute dtype: repeated runs must agree to within one unit in the last place of that dtype (and in practice
+    agree exactly; a difference needs the double sums to straddle a rounding boundary of the narrower type)."""
+    from aimet_amd.quantization import affine
+
+    shape, enc_shape, block = layout
+    x, scale, offset, grad = _make_case(shape, enc_shape, dtype, -128, 127, True, seed=11)
+    xd, gd = x.to(device), grad.to(device)
+    runs = []
+    for _ in range(5):
+        sd = scale.to(device).requires_grad_(True)
+        od = offset.to(device).requires_grad_(True)
+        affine.quantize_dequantize(xd, sd, od, -128, 127, block_size=block).backward(gd)
+        runs.append((sd.grad.clone(), od.grad.clone()))
+    ulp = float(torch.finfo(torch.float32 if dtype == torch.float32 else dtype).eps)
+    for gs, go in runs[1:]:
+        assert_close_rel(gs, runs[0][0], ulp, "scale gradient of a repeated run", abs_floor=1e-30)
+        assert_close_rel(go, runs[0][1], ulp, "offset gradient of a repeated run", abs_floor=1e-30)
