@@ -114,6 +114,10 @@ _SIGNATURES = {
     "ahq_minmax_to_encodings": (ctypes.c_int, [ctypes.c_int32, _P, _P, ctypes.c_int64, ctypes.c_int64, ctypes.c_int32,
                                                ctypes.c_float, ctypes.c_float, ctypes.c_float, ctypes.c_float, _P, _P, _P,
                                                _P]),
+    "ahq_minmax_finalize": (ctypes.c_int, [ctypes.c_int32, _P, _P, ctypes.c_int64, ctypes.c_int64, ctypes.c_int32,
+                                           ctypes.c_float, ctypes.c_float, ctypes.c_float, ctypes.c_float, _P,
+                                           ctypes.c_int32, _P, _P, ctypes.c_int64, ctypes.c_int64, ctypes.c_double, _P,
+                                           _P, _P]),
     "ahq_range_to_scale_offset": (ctypes.c_int, [ctypes.c_int32, _P, _P, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
                                                  ctypes.c_double, _P, _P, _P]),
     "ahq_lpbq_scale": (ctypes.c_int, [ctypes.c_int32, ctypes.POINTER(Layout), _P, _P, ctypes.c_int64, ctypes.c_int64,

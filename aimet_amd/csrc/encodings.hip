@@ -40,13 +40,10 @@ struct RoundTo<bf16_t> { __device__ static float f(float v) { return rnd<AHQ_BF1
 
 __device__ __forceinline__ float nan_max(float a, float b) { return (a != a || b != b) ? __builtin_nanf("") : fmaxf(a, b); }
 
+// statistics (mn, mx) -> encoding range (lo, hi), both as T values widened to float; raises the flags
 template <typename T>
-__global__ void minmax_to_encodings_kernel(const EncArgs a) {
-    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= a.n) return;
+__device__ __forceinline__ void encode_range(const EncArgs& a, float mn, float mx, T& lo_t, T& hi_t) {
     using R = RoundTo<T>;
-    const float mn = load_f32(static_cast<const T*>(a.smin)[i]);
-    const float mx = load_f32(static_cast<const T*>(a.smax)[i]);
     // clamp(min, max=0), clamp(max, min=0): NaN stays NaN
     float lo = (mn != mn) ? mn : fminf(mn, 0.f);
     float hi = (mx != mx) ? mx : fmaxf(mx, 0.f);
@@ -65,9 +62,8 @@ __global__ void minmax_to_encodings_kernel(const EncArgs a) {
         lo = (lo != lo) ? lo : fmaxf(lo, -a.t_max);
     }
     hi = (hi != hi) ? hi : fminf(hi, a.t_max);
-    const T lo_t = store_cast<T>(lo), hi_t = store_cast<T>(hi);
-    static_cast<T*>(a.out_min)[i] = lo_t;
-    static_cast<T*>(a.out_max)[i] = hi_t;
+    lo_t = store_cast<T>(lo);
+    hi_t = store_cast<T>(hi);
     if (a.flags) {
         const float l = load_f32(lo_t), h = load_f32(hi_t);
         const bool nonfinite = !(__builtin_fabsf(l) < __builtin_inff()) || !(__builtin_fabsf(h) < __builtin_inff());
@@ -76,6 +72,16 @@ __global__ void minmax_to_encodings_kernel(const EncArgs a) {
         if (nonfinite) atomicOr(&a.flags[0], 1);
         if (near) atomicOr(&a.flags[1], 1);
     }
+}
+
+template <typename T>
+__global__ void minmax_to_encodings_kernel(const EncArgs a) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= a.n) return;
+    T lo_t, hi_t;
+    encode_range<T>(a, load_f32(static_cast<const T*>(a.smin)[i]), load_f32(static_cast<const T*>(a.smax)[i]), lo_t, hi_t);
+    static_cast<T*>(a.out_min)[i] = lo_t;
+    static_cast<T*>(a.out_max)[i] = hi_t;
 }
 
 // ----------------------------------------------------------------------------------- range -> (scale, offset) --
@@ -106,6 +112,36 @@ __global__ void range_to_scale_offset_kernel(const ScaleOffArgs a) {
     if (a.offset) {
         const float r = __builtin_rintf(mn / s) - a.qmin;
         a.offset[i] = (r != r) ? r : fminf(fmaxf(r, a.lo), a.hi);
+    }
+}
+
+// ------------------------------------------------ statistics -> range, quantizer parameters, scale and offset --
+// The end of a min/max calibration in one launch: the encoding range of the statistics (minmax_to_encodings_kernel),
+// stored into the quantizer's min / max parameters in their own dtype P (what Tensor.copy_ does: round to nearest
+// even), and scale / offset derived from the stored parameters (range_to_scale_offset_kernel).  A whole-model
+// calibration ends a few hundred quantizer contexts; each is a handful of values.
+struct FinalArgs {
+    void* pmin;
+    void* pmax;
+    ScaleOffArgs so;  // pmin / pmax unused
+};
+
+template <typename T, typename P>
+__global__ void minmax_finalize_kernel(const EncArgs a, const FinalArgs f) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= a.n) return;
+    T lo_t, hi_t;
+    encode_range<T>(a, load_f32(static_cast<const T*>(a.smin)[i]), load_f32(static_cast<const T*>(a.smax)[i]), lo_t, hi_t);
+    const P lo_p = store_cast<P>(load_f32(lo_t)), hi_p = store_cast<P>(load_f32(hi_t));
+    static_cast<P*>(f.pmin)[i] = lo_p;
+    static_cast<P*>(f.pmax)[i] = hi_p;
+    const float mn = load_f32(lo_p), mx = load_f32(hi_p);
+    float s = __builtin_fabsf((mx - mn) / f.so.num_steps);
+    s = (s != s) ? s : fmaxf(s, f.so.minimum_scale);
+    f.so.scale[i] = s;
+    if (f.so.offset) {
+        const float r = __builtin_rintf(mn / s) - f.so.qmin;
+        f.so.offset[i] = (r != r) ? r : fminf(fmaxf(r, f.so.lo), f.so.hi);
     }
 }
 
@@ -344,31 +380,41 @@ extern "C" int ahq_lpbq_scale(int32_t dtype, const ahq_layout* grouping, const v
     return check_launch("lpbq_scale");
 }
 
+static int fill_enc_args(EncArgs* a, int32_t dtype, const void* stat_min, const void* stat_max, int64_t num_encodings,
+                         int64_t num_steps, int32_t symmetric, float minimum_scale_in_dtype, float minimum_scale,
+                         float dtype_max, float near_max_threshold, int32_t* flags) {
+    if (dtype < AHQ_F32 || dtype > AHQ_BF16) return set_error("bad dtype"), AHQ_ERR_INVALID;
+    if (!stat_min || !stat_max) return set_error("null argument"), AHQ_ERR_INVALID;
+    if (num_encodings < 0) return set_error("negative encoding count"), AHQ_ERR_INVALID;
+    if (num_steps <= 0 || num_steps > (1ll << 24)) return set_error("num_steps must be in 1..2^24"), AHQ_ERR_INVALID;
+    a->smin = stat_min;
+    a->smax = stat_max;
+    a->flags = flags;
+    a->n = num_encodings;
+    a->num_steps = (float)num_steps;
+    a->tiny_t = minimum_scale_in_dtype;
+    a->tiny_f = minimum_scale;
+    a->pos = (float)(num_steps / 2);
+    a->neg = (float)(num_steps - num_steps / 2);
+    a->pos_extra = a->pos + (num_steps == 3 ? 1.f : 0.f);
+    a->t_max = dtype_max;
+    a->near_thr = near_max_threshold;
+    a->symmetric = symmetric ? 1 : 0;
+    return AHQ_OK;
+}
+
 extern "C" int ahq_minmax_to_encodings(int32_t dtype, const void* stat_min, const void* stat_max, int64_t num_encodings,
                                        int64_t num_steps, int32_t symmetric, float minimum_scale_in_dtype,
                                        float minimum_scale, float dtype_max, float near_max_threshold, void* out_min,
                                        void* out_max, int32_t* flags, void* stream) {
-    if (dtype < AHQ_F32 || dtype > AHQ_BF16) return set_error("bad dtype"), AHQ_ERR_INVALID;
-    if (!stat_min || !stat_max || !out_min || !out_max) return set_error("null argument"), AHQ_ERR_INVALID;
-    if (num_encodings < 0) return set_error("negative encoding count"), AHQ_ERR_INVALID;
-    if (num_steps <= 0 || num_steps > (1ll << 24)) return set_error("num_steps must be in 1..2^24"), AHQ_ERR_INVALID;
-    if (num_encodings == 0) return AHQ_OK;
     EncArgs a{};
-    a.smin = stat_min;
-    a.smax = stat_max;
+    const int rc = fill_enc_args(&a, dtype, stat_min, stat_max, num_encodings, num_steps, symmetric,
+                                 minimum_scale_in_dtype, minimum_scale, dtype_max, near_max_threshold, flags);
+    if (rc != AHQ_OK) return rc;
+    if (!out_min || !out_max) return set_error("null argument"), AHQ_ERR_INVALID;
+    if (num_encodings == 0) return AHQ_OK;
     a.out_min = out_min;
     a.out_max = out_max;
-    a.flags = flags;
-    a.n = num_encodings;
-    a.num_steps = (float)num_steps;
-    a.tiny_t = minimum_scale_in_dtype;
-    a.tiny_f = minimum_scale;
-    a.pos = (float)(num_steps / 2);
-    a.neg = (float)(num_steps - num_steps / 2);
-    a.pos_extra = a.pos + (num_steps == 3 ? 1.f : 0.f);
-    a.t_max = dtype_max;
-    a.near_thr = near_max_threshold;
-    a.symmetric = symmetric ? 1 : 0;
     hipStream_t s = static_cast<hipStream_t>(stream);
     const dim3 g((unsigned)((num_encodings + 255) / 256)), b(256);
     switch (dtype) {
@@ -377,4 +423,48 @@ extern "C" int ahq_minmax_to_encodings(int32_t dtype, const void* stat_min, cons
         default: hipLaunchKernelGGL((minmax_to_encodings_kernel<bf16_t>), g, b, 0, s, a); break;
     }
     return check_launch("minmax_to_encodings");
+}
+
+template <typename T>
+static void launch_finalize(int32_t param_dtype, const dim3& g, const dim3& b, hipStream_t s, const EncArgs& a,
+                            const FinalArgs& f) {
+    switch (param_dtype) {
+        case AHQ_F32: hipLaunchKernelGGL((minmax_finalize_kernel<T, float>), g, b, 0, s, a, f); break;
+        case AHQ_F16: hipLaunchKernelGGL((minmax_finalize_kernel<T, f16_t>), g, b, 0, s, a, f); break;
+        default: hipLaunchKernelGGL((minmax_finalize_kernel<T, bf16_t>), g, b, 0, s, a, f); break;
+    }
+}
+
+extern "C" int ahq_minmax_finalize(int32_t stat_dtype, const void* stat_min, const void* stat_max, int64_t num_encodings,
+                                   int64_t num_steps, int32_t symmetric, float minimum_scale_in_dtype,
+                                   float minimum_scale, float dtype_max, float near_max_threshold, int32_t* flags,
+                                   int32_t param_dtype, void* param_min, void* param_max, int64_t qmin, int64_t qmax,
+                                   double grid_minimum_scale, float* scale, float* offset, void* stream) {
+    EncArgs a{};
+    const int rc = fill_enc_args(&a, stat_dtype, stat_min, stat_max, num_encodings, num_steps, symmetric,
+                                 minimum_scale_in_dtype, minimum_scale, dtype_max, near_max_threshold, flags);
+    if (rc != AHQ_OK) return rc;
+    if (param_dtype < AHQ_F32 || param_dtype > AHQ_BF16) return set_error("bad parameter dtype"), AHQ_ERR_INVALID;
+    if (!param_min || !param_max || !scale) return set_error("null argument"), AHQ_ERR_INVALID;
+    if (qmin >= qmax) return set_error("qmax must be larger than qmin"), AHQ_ERR_INVALID;
+    if (num_encodings == 0) return AHQ_OK;
+    FinalArgs f{};
+    f.pmin = param_min;
+    f.pmax = param_max;
+    f.so.scale = scale;
+    f.so.offset = offset;
+    f.so.n = num_encodings;
+    f.so.num_steps = (float)(double)(qmax - qmin);
+    f.so.minimum_scale = (float)grid_minimum_scale;
+    f.so.qmin = (float)(double)qmin;
+    f.so.lo = (float)(double)(-qmax);
+    f.so.hi = (float)(double)(-qmin);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const dim3 g((unsigned)((num_encodings + 255) / 256)), b(256);
+    switch (stat_dtype) {
+        case AHQ_F32: launch_finalize<float>(param_dtype, g, b, s, a, f); break;
+        case AHQ_F16: launch_finalize<f16_t>(param_dtype, g, b, s, a, f); break;
+        default: launch_finalize<bf16_t>(param_dtype, g, b, s, a, f); break;
+    }
+    return check_launch("minmax_finalize");
 }

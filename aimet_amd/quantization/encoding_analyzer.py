@@ -438,6 +438,7 @@ def _scalar_constants(dtype: torch.dtype, tiny: float):
 
 
 _deferred_range_flags = None  # list of device flag pairs while deferred_range_warnings() is active
+_deferred_shared_flags = None  # device -> int32[2] that kernels OR into while it is active
 
 
 @contextlib.contextmanager
@@ -445,21 +446,39 @@ def deferred_range_warnings():
     """Inside this context the non-finite / near-overflow checks of every quantizer are gathered on the device and
     read back once on exit, instead of one host synchronisation per quantizer (a whole-model calibration ends
     hundreds of quantizer contexts at once).  The same warnings are issued, at the end."""
-    global _deferred_range_flags  # pylint: disable=global-statement
+    global _deferred_range_flags, _deferred_shared_flags  # pylint: disable=global-statement
     if _deferred_range_flags is not None:
         yield
         return
     _deferred_range_flags = []
+    _deferred_shared_flags = {}
     try:
         yield
     finally:
         flags, _deferred_range_flags = _deferred_range_flags, None
+        shared, _deferred_shared_flags = _deferred_shared_flags, None
+        flags += [f != 0 for f in shared.values()]
         if flags:
             by_device = {}
             for f in flags:
                 by_device.setdefault(f.device, []).append(f)
             for group in by_device.values():
                 _warn_range_flags(*torch.stack(group).any(dim=0).tolist())
+
+
+def _range_flags_buffer(device):
+    """(int32[2] on ``device`` for a kernel to OR its range flags into, whether the caller has to report it itself).
+    Inside deferred_range_warnings() all kernels on a device share one buffer, read back when the context ends."""
+    if _deferred_shared_flags is not None:
+        buf = _deferred_shared_flags.get(device)
+        if buf is None:
+            buf = _deferred_shared_flags[device] = torch.zeros(2, dtype=torch.int32, device=device)
+        return buf, False
+    return torch.zeros(2, dtype=torch.int32, device=device), True
+
+
+def _report_range_flags(flags: torch.Tensor):
+    _warn_range_flags(*(flags != 0).tolist())
 
 
 def _warn_range_flags(nonfinite: bool, extreme: bool):

@@ -185,6 +185,21 @@ int ahq_range_to_scale_offset(int32_t dtype, const void* range_min, const void* 
                               int64_t qmin, int64_t qmax, double minimum_scale, float* scale, float* offset,
                               void* stream);
 
+/* The end of a min/max calibration in one launch: replaces, for a quantizer that holds min / max, the sequence
+ * MinMaxEncodingAnalyzer.compute_encodings_from_stats (AT/quantization/encoding_analyzer.py:425-481) with the checks of
+ * _flag_extreme_min_max (:484-498), set_range (AT/quantization/affine/quantizer.py:378-438: min.copy_(lo),
+ * max.copy_(hi)) and the get_scale / _get_offset the next forward would run (:319-376).  The first ten arguments and
+ * `flags` are those of ahq_minmax_to_encodings; the range is stored into param_min / param_max (num_encodings values
+ * of `param_dtype`, rounded to nearest even from `stat_dtype` as Tensor.copy_ does), and scale / offset (float32,
+ * offset may be NULL for a symmetric grid) are derived from the stored values exactly as ahq_range_to_scale_offset
+ * derives them; qmin, qmax and grid_minimum_scale are that function's arguments.
+ */
+int ahq_minmax_finalize(int32_t stat_dtype, const void* stat_min, const void* stat_max, int64_t num_encodings,
+                        int64_t num_steps, int32_t symmetric, float minimum_scale_in_dtype, float minimum_scale,
+                        float dtype_max, float near_max_threshold, int32_t* flags, int32_t param_dtype,
+                        void* param_min, void* param_max, int64_t qmin, int64_t qmax, double grid_minimum_scale,
+                        float* scale, float* offset, void* stream);
+
 /* Replaces GroupedBlockQuantizeDequantize._get_scale / _get_per_channel_scale with dtype = float32 (LPBQ,
  * AT/quantization/affine/quantizer.py:1363-1399), which the reference runs on every forward through get_encodings():
  *   raw               = clamp_min(|float(max) - float(min)| / (qmax - qmin), minimum_scale)     (quantizer.py:319-339)

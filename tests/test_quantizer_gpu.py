@@ -3,6 +3,7 @@ closed-form expectations the reference's own quantizer tests hold
 (TrainingExtensions/torch/test/python/v2/quantization/affine/test_affine_quantizer.py)."""
 
 import math
+import warnings
 
 import pytest
 import torch
@@ -388,3 +389,92 @@ def test_scale_and_offset_from_a_range_in_one_launch(device, dtype, grid):
     # gradients wanted: the step-by-step form runs
     with torch.enable_grad():
         assert q._fused_scale_offset() is None
+
+
+@pytest.mark.parametrize("stat_dtype", [torch.float32, torch.float16, torch.bfloat16], ids=lambda d: str(d).split(".")[-1])
+@pytest.mark.parametrize("param_dtype", [torch.float32, torch.bfloat16], ids=["f32_params", "bf16_params"])
+@pytest.mark.parametrize("grid", [(0, 255, False, None), (-128, 127, True, None), (-8, 7, True, None),
+                                  (0, 65535, False, None), (-2, 1, True, 0.5), (-2, 1, True, None)], ids=str)
+def test_end_of_minmax_calibration_in_one_launch(device, monkeypatch, stat_dtype, param_dtype, grid):
+    """Leaving compute_encodings() with ahq_minmax_finalize gives the min / max parameters, scale and offset of the
+    step-by-step form (analyzer kernel, set_range, get_scale / get_offset) bit for bit, and the oracle's; the
+    encodings it leaves in the cache are the ones a later get_encodings() derives afresh."""
+    from aimet_amd.quantization.affine import QuantizeDequantize
+    from aimet_amd.quantization.affine.quantizer import AffineQuantizerBase
+
+    qmin, qmax, symmetric, zps = grid
+    g = torch.Generator().manual_seed(9)
+    rows = 512
+    x = torch.randn(rows, 96, generator=g) * torch.logspace(-9, 9, rows).view(-1, 1)
+    x[0] = 0.0
+    x[1] = 1e-12
+    x[2, 0], x[3, 0], x[4, 0] = float("inf"), -float("inf"), float("nan")
+    x[5] = x[5].abs()
+    x[6] = -x[6].abs()
+    x = x.to(stat_dtype).to(device)
+
+    def calibrated(fused: bool):
+        q = QuantizeDequantize((rows, 1), qmin=qmin, qmax=qmax, symmetric=symmetric,
+                               zero_point_shift=zps).to(device=device, dtype=param_dtype)
+        calls = []
+        real = AffineQuantizerBase._finalize_from_minmax
+        monkeypatch.setattr(AffineQuantizerBase, "_finalize_from_minmax",
+                            (lambda self: calls.append(real(self)) or calls[-1]) if fused else (lambda self: False))
+        with warnings.catch_warnings():
+            warnings.simplefilter("ignore")
+            with torch.no_grad(), q._compute_encodings(passthrough=True):
+                q(x)
+                q(x * 0.5)
+        monkeypatch.undo()
+        assert calls == ([True] if fused else [])
+        return q
+
+    fast, slow = calibrated(True), calibrated(False)
+    assert_same_bits(fast.min, slow.min, "min")
+    assert_same_bits(fast.max, slow.max, "max")
+    primed = fast.__dict__["_encoding_cache"][1]
+    with torch.no_grad():
+        assert fast.get_encodings() is primed  # the key it was stored under is the live one
+        want = slow.get_encodings()
+        assert_same_bits(primed.scale, want.scale, "scale")
+        assert_same_bits(primed.offset, want.offset, "offset")
+        fast.invalidate_encoding_cache()
+        again = fast.get_encodings()
+        assert_same_bits(again.scale, primed.scale, "scale derived afresh")
+        assert_same_bits(again.offset, primed.offset, "offset derived afresh")
+    # the oracle's analyzer on the same statistics
+    steps = (qmax - qmin) - (1 if zps else 0)
+    mn = torch.minimum(x.amin(dim=1, keepdim=True), (x * 0.5).amin(dim=1, keepdim=True)).cpu()
+    mx = torch.maximum(x.amax(dim=1, keepdim=True), (x * 0.5).amax(dim=1, keepdim=True)).cpu()
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        lo, hi = O.minmax_encodings(mn, mx, steps, symmetric)
+    # (+ 0.0: which zero the minimum of a row holding both +0 and -0 is depends on the order of the reduction)
+    assert_same_bits(fast.min.detach() + 0.0, lo.to(param_dtype) + 0.0, "min against the oracle")
+    assert_same_bits(fast.max.detach() + 0.0, hi.to(param_dtype) + 0.0, "max against the oracle")
+
+
+def test_range_warnings_of_the_fused_calibration_end(device):
+    from aimet_amd.quantization.affine import QuantizeDequantize
+    from aimet_amd.quantization.encoding_analyzer import deferred_range_warnings
+
+    def run(value, deferred):
+        q = QuantizeDequantize((), 8, symmetric=False).to(device)
+        x = torch.full((64,), value, device=device)
+        with torch.no_grad():
+            if deferred:
+                with deferred_range_warnings():
+                    with q._compute_encodings(passthrough=True):
+                        q(x)
+            else:
+                with q._compute_encodings(passthrough=True):
+                    q(x)
+
+    for deferred in (False, True):
+        with pytest.warns(UserWarning, match="Infinite or NaN"):
+            run(float("nan"), deferred)  # an infinite statistic is clamped to the largest finite value first
+        with pytest.warns(UserWarning, match="Extreme values"):
+            run(3.3e38, deferred)
+        with warnings.catch_warnings():
+            warnings.simplefilter("error")
+            run(1.0, deferred)
