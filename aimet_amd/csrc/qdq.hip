@@ -595,7 +595,7 @@ __device__ __forceinline__ float finish_sum_rt(double s, int cd) {
 template <typename IO, int VEC, typename M, int RED, bool FULL, bool FAST>
 __device__ __forceinline__ void bwd_math(const QdqArgs& a, const Tile& t, float (*sp)[kStage], const Pack<IO, VEC>* xin,
                                          const Pack<IO, VEC>* gin, IO* __restrict__ gxp, double& acc_s, double& acc_o,
-                                         double* stage_sums) {
+                                         double* stage_sums, float* vec_sums) {
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
         const int lv = u * kBlock + threadIdx.x;
@@ -673,13 +673,19 @@ __device__ __forceinline__ void bwd_math(const QdqArgs& a, const Tile& t, float 
                 atomicAdd(&stage_sums[2 * si], (double)vs);
                 atomicAdd(&stage_sums[2 * si + 1], (double)vo);
             }
+        } else if (RED == kRedRuns) {
+            // one pair per vector; the runs are added up in a fixed order once the tile is through
+            if (FULL || lv < t.nv) {
+                vec_sums[lv] = vs;
+                vec_sums[kTileVec + lv] = vo;
+            }
         }
     }
 }
 
 template <typename IO, int VEC, typename M, int RED, bool FULL>
 __device__ __forceinline__ void bwd_tile(const QdqArgs& a, const Tile& t, float (*sp)[kStage], double& acc_s, double& acc_o,
-                                         double* stage_sums) {
+                                         double* stage_sums, float* vec_sums) {
     const IO* __restrict__ x = static_cast<const IO*>(a.x) + t.v0 * VEC;
     const IO* __restrict__ g = static_cast<const IO*>(a.g) + t.v0 * VEC;
     IO* __restrict__ gxp = a.gx ? static_cast<IO*>(a.gx) + t.v0 * VEC : nullptr;
@@ -698,9 +704,9 @@ __device__ __forceinline__ void bwd_tile(const QdqArgs& a, const Tile& t, float 
         for (int i = threadIdx.x; i < 2 * t.nstage; i += kBlock) stage_sums[i] = 0.0;
     __syncthreads();
     if (!M::kDiv || __builtin_amdgcn_ballot_w64(!lane_can_divide_fast<IO, VEC, M, FULL, kUnroll>(a, t, sp, xin)) == 0)
-        bwd_math<IO, VEC, M, RED, FULL, true>(a, t, sp, xin, gin, gxp, acc_s, acc_o, stage_sums);
+        bwd_math<IO, VEC, M, RED, FULL, true>(a, t, sp, xin, gin, gxp, acc_s, acc_o, stage_sums, vec_sums);
     else
-        bwd_math<IO, VEC, M, RED, FULL, false>(a, t, sp, xin, gin, gxp, acc_s, acc_o, stage_sums);
+        bwd_math<IO, VEC, M, RED, FULL, false>(a, t, sp, xin, gin, gxp, acc_s, acc_o, stage_sums, vec_sums);
 }
 
 template <typename IO, int VEC, typename M, int RED>
@@ -708,10 +714,51 @@ __global__ __launch_bounds__(kBlock) void qdq_bwd_kernel(const QdqArgs a) {
     __shared__ float sp[M::kNP + (M::kDiv ? 1 : 0)][kStage];
     __shared__ double red_smem[kBlock / kWave];
     __shared__ double stage_sums[RED == kRedAtomic ? 2 * kStage : 1];  // kRedAtomic: (scale, offset) sums per run
+    __shared__ float vec_sums[RED == kRedRuns ? 2 * kTileVec : 1];     // kRedRuns: (scale, offset) terms per vector
     const Tile t = make_tile(a, blockIdx.x);
     double acc_s = 0.0, acc_o = 0.0;  // kRedTile: per-thread totals
-    if (t.nv == kTileVec) bwd_tile<IO, VEC, M, RED, true>(a, t, sp, acc_s, acc_o, stage_sums);
-    else bwd_tile<IO, VEC, M, RED, false>(a, t, sp, acc_s, acc_o, stage_sums);
+    if (t.nv == kTileVec) bwd_tile<IO, VEC, M, RED, true>(a, t, sp, acc_s, acc_o, stage_sums, vec_sums);
+    else bwd_tile<IO, VEC, M, RED, false>(a, t, sp, acc_s, acc_o, stage_sums, vec_sums);
+    if (RED == kRedRuns) {
+        // The tile holds t.nstage whole runs of Kv vectors.  Short runs: one thread adds a run front to back.  Longer
+        // ones: one wave per run, every lane adds its strided share front to back, then the lanes are combined in
+        // the fixed pattern of wave_reduce.  Either way the order of additions depends on the layout alone.
+        __syncthreads();
+        const int kv = (int)a.Kv;
+        const int64_t run0 = (int64_t)blockIdx.x * a.tpr;
+        auto emit = [&](int run, double s, double o) {
+            if (a.I == 1) {
+                a.gscale[run0 + run] = finish_sum_rt(s, a.out_cd);
+                a.goffset[run0 + run] = finish_sum_rt(o, a.out_cd);
+            } else {
+                a.partials[2 * (run0 + run)] = s;
+                a.partials[2 * (run0 + run) + 1] = o;
+            }
+        };
+        if (kv <= 16) {
+            for (int run = threadIdx.x; run < t.nstage; run += kBlock) {
+                double s = 0.0, o = 0.0;
+                for (int k = 0; k < kv; ++k) {
+                    s += (double)vec_sums[run * kv + k];
+                    o += (double)vec_sums[kTileVec + run * kv + k];
+                }
+                emit(run, s, o);
+            }
+        } else {
+            const int lane = threadIdx.x & (kWave - 1);
+            for (int run = threadIdx.x / kWave; run < t.nstage; run += kBlock / kWave) {
+                double s = 0.0, o = 0.0;
+                for (int k = lane; k < kv; k += kWave) {
+                    s += (double)vec_sums[run * kv + k];
+                    o += (double)vec_sums[kTileVec + run * kv + k];
+                }
+                s = wave_reduce(s, OpAddD());
+                o = wave_reduce(o, OpAddD());
+                if (lane == 0) emit(run, s, o);
+            }
+        }
+        return;
+    }
     if (RED == kRedAtomic) {
         __syncthreads();
         for (int i = threadIdx.x; i < t.nstage; i += kBlock) {
@@ -811,6 +858,29 @@ __global__ __launch_bounds__(kFinishThreads) void qdq_bwd_finish_kernel(const Qd
     }
 }
 
+// Adds, for every encoding, `count` partial pairs that lie `stride` pairs apart (the first one at the encoding's own
+// index), in a fixed order: one wave per encoding, every lane its strided share front to back, then wave_reduce.
+// kRedRuns with I > 1: count = I runs per encoding, stride = J.  Column kernel: count = row groups, stride = J.
+__global__ __launch_bounds__(kBlock) void qdq_bwd_strided_finish_kernel(const double* __restrict__ partials, int64_t count,
+                                                                        int64_t stride, int64_t num_enc, float* gscale,
+                                                                        float* goffset, int cd) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t waves = (int64_t)gridDim.x * (kBlock / kWave);
+    for (int64_t e = (int64_t)blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave; e < num_enc; e += waves) {
+        double s = 0.0, o = 0.0;
+        for (int64_t q = lane; q < count; q += kWave) {
+            s += partials[2 * (q * stride + e)];
+            o += partials[2 * (q * stride + e) + 1];
+        }
+        s = wave_reduce(s, OpAddD());
+        o = wave_reduce(o, OpAddD());
+        if (lane == 0) {
+            gscale[e] = finish_sum_rt(s, cd);
+            goffset[e] = finish_sum_rt(o, cd);
+        }
+    }
+}
+
 template <typename IO, typename M>
 __global__ __launch_bounds__(kBlock) void qdq_bwd_generic_kernel(const QdqArgs a) {
     const IO* __restrict__ x = static_cast<const IO*>(a.x);
@@ -856,7 +926,8 @@ __global__ __launch_bounds__(kBlock) void qdq_bwd_generic_kernel(const QdqArgs a
 }
 
 // Backward for run length 1 (see qdq_fwd_cols_kernel): every lane keeps the sums of its VEC encodings over the rows
-// it walks, the waves of a workgroup add theirs up in LDS, and one wave adds the workgroup's sums to the global ones.
+// it walks, the waves of a workgroup add theirs up in LDS one after the other, and the workgroup's sums go to its own
+// row of the partials ([row group][encoding]), which qdq_bwd_strided_finish_kernel adds up in order.
 template <typename IO, int VEC, typename M>
 __global__ __launch_bounds__(kColThreads) void qdq_bwd_cols_kernel(const QdqArgs a) {
     __shared__ double sums[2 * VEC * kWave];
@@ -868,18 +939,19 @@ __global__ __launch_bounds__(kColThreads) void qdq_bwd_cols_kernel(const QdqArgs
         for (int i = threadIdx.x; i < 2 * VEC * kWave; i += kColThreads) sums[i] = 0.0;
         __syncthreads();
     }
+    double acc_s[VEC], acc_o[VEC];
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) acc_s[k] = acc_o[k] = 0.0;
     if (live) {
         const IO* __restrict__ x = static_cast<const IO*>(a.x);
         const IO* __restrict__ g = static_cast<const IO*>(a.g);
         IO* __restrict__ gxp = static_cast<IO*>(a.gx);
         EncP e[VEC];
         bool enc_fast = true;
-        double acc_s[VEC], acc_o[VEC];
 #pragma unroll
         for (int k = 0; k < VEC; ++k) {
             e[k] = load_enc<M>(a, c0 + k);
             enc_fast &= !M::kDiv || e[k].rs != 0.f;
-            acc_s[k] = acc_o[k] = 0.0;
         }
         const int64_t step = (int64_t)gridDim.y * kColWaves * kColUnroll;
         for (int64_t r0 = ((int64_t)blockIdx.y * kColWaves + wave) * kColUnroll; r0 < a.I; r0 += step) {
@@ -912,21 +984,25 @@ __global__ __launch_bounds__(kColThreads) void qdq_bwd_cols_kernel(const QdqArgs
                 if (gxp) store_pack_stream<IO, VEC>(gxp + (r0 + u) * a.J + c0, out);
             }
         }
-        if (want_pg) {
-#pragma unroll
-            for (int k = 0; k < VEC; ++k) {
-                atomicAdd(&sums[(2 * k) * kWave + lane], acc_s[k]);
-                atomicAdd(&sums[(2 * k + 1) * kWave + lane], acc_o[k]);
-            }
-        }
     }
     if (!want_pg) return;
-    __syncthreads();
+    // the waves take turns, so the sums do not depend on which wave finishes first
+    for (int w = 0; w < kColWaves; ++w) {
+        if (wave == w && live) {
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) {
+                sums[(2 * k) * kWave + lane] += acc_s[k];
+                sums[(2 * k + 1) * kWave + lane] += acc_o[k];
+            }
+        }
+        __syncthreads();
+    }
     if (wave == 0 && live) {
+        double* row = a.partials + 2 * (int64_t)blockIdx.y * a.J;
 #pragma unroll
         for (int k = 0; k < VEC; ++k) {
-            atomicAdd(&a.partials[2 * (c0 + k)], sums[(2 * k) * kWave + lane]);
-            atomicAdd(&a.partials[2 * (c0 + k) + 1], sums[(2 * k + 1) * kWave + lane]);
+            row[2 * (c0 + k)] = sums[(2 * k) * kWave + lane];
+            row[2 * (c0 + k) + 1] = sums[(2 * k + 1) * kWave + lane];
         }
     }
 }
@@ -1013,6 +1089,27 @@ static void launch_fwd(const Plan& p, const QdqArgs& a, hipStream_t st, bool ali
     }
 }
 
+// the column-walking backward kernel takes run length 1 whatever reduction the plan would otherwise use for it
+template <typename IO>
+static bool bwd_cols_layout(const Plan& p, bool aligned) {
+    return cols_layout<IO>(p, aligned) && (p.red == kRedAtomic || p.red == kRedRuns || p.red == kRedNone);
+}
+
+static bool bwd_cols_layout(int io_dtype, const Plan& p, bool aligned) {
+    return io_dtype == AHQ_F32 ? bwd_cols_layout<float>(p, aligned) : bwd_cols_layout<f16_t>(p, aligned);
+}
+
+static unsigned bwd_cols_row_groups(int io_dtype, const Plan& p) {
+    return io_dtype == AHQ_F32 ? cols_grid<float>(p, 512).y : cols_grid<f16_t>(p, 512).y;
+}
+
+// pairs of doubles the backward pass needs as scratch for its parameter gradients
+static size_t bwd_scratch_pairs(int io_dtype, const Plan& p, bool aligned, bool want_pg) {
+    if (!want_pg) return 0;
+    if (bwd_cols_layout(io_dtype, p, aligned)) return (size_t)bwd_cols_row_groups(io_dtype, p) * (size_t)p.cl.J;
+    return p.ws_elems;
+}
+
 template <typename IO, typename M, int RED>
 static void launch_bwd_red(const Plan& p, const QdqArgs& a, hipStream_t st) {
     if (p.vec == 1) {
@@ -1024,8 +1121,8 @@ static void launch_bwd_red(const Plan& p, const QdqArgs& a, hipStream_t st) {
 
 template <typename IO, typename M>
 static void launch_bwd(const Plan& p, const QdqArgs& a, hipStream_t st, bool aligned) {
-    if (cols_layout<IO>(p, aligned) && (p.red == kRedAtomic || p.red == kRedNone)) {
-        // few row groups: every workgroup ends with two global atomics per encoding
+    if (bwd_cols_layout<IO>(p, aligned)) {
+        // few row groups: every workgroup ends with one row of partial sums
         hipLaunchKernelGGL((qdq_bwd_cols_kernel<IO, IoTraits<IO>::kVec, M>), cols_grid<IO>(p, 512), dim3(kColThreads), 0, st, a);
         return;
     }
@@ -1037,6 +1134,7 @@ static void launch_bwd(const Plan& p, const QdqArgs& a, hipStream_t st, bool ali
         case kRedNone: launch_bwd_red<IO, M, kRedNone>(p, a, st); break;
         case kRedTile: launch_bwd_red<IO, M, kRedTile>(p, a, st); break;
         case kRedSeg: launch_bwd_red<IO, M, kRedSeg>(p, a, st); break;
+        case kRedRuns: launch_bwd_red<IO, M, kRedRuns>(p, a, st); break;
         default: launch_bwd_red<IO, M, kRedAtomic>(p, a, st); break;
     }
 }
@@ -1242,12 +1340,16 @@ extern "C" int ahq_float_dequantize(int32_t dtype, const ahq_layout* layout, con
 
 extern "C" size_t ahq_qdq_backward_workspace_bytes(const ahq_grid* grid, const ahq_layout* layout, int want_param_grads) {
     if (!grid || !layout) return 0;
+    const bool pg = want_param_grads != 0;
     Plan p;
-    if (!make_plan(grid->io_dtype, *layout, true, want_param_grads != 0, &p)) return 0;
-    size_t a = p.ws_elems * 2 * sizeof(double);
+    if (!make_plan(grid->io_dtype, *layout, true, pg, &p, kUnroll, true)) return 0;
+    size_t a = bwd_scratch_pairs(grid->io_dtype, p, true, pg) * 2 * sizeof(double);
     // an unaligned tensor falls back to the scalar path whose strategy may need a different amount
     Plan q;
-    if (make_plan(grid->io_dtype, *layout, false, want_param_grads != 0, &q) && q.ws_elems * 2 * sizeof(double) > a) a = q.ws_elems * 2 * sizeof(double);
+    if (make_plan(grid->io_dtype, *layout, false, pg, &q, kUnroll, true)) {
+        const size_t b = bwd_scratch_pairs(grid->io_dtype, q, false, pg) * 2 * sizeof(double);
+        if (b > a) a = b;
+    }
     return a;
 }
 
@@ -1262,12 +1364,13 @@ extern "C" int ahq_qdq_backward(const ahq_grid* grid, const ahq_layout* layout, 
     if (want_pg && grid->arith == AHQ_ARITH_ATEN) return set_error("the ATen arithmetic has no scale/offset gradient"), AHQ_ERR_INVALID;
     Plan p;
     const bool al = aligned16(x) && aligned16(g) && (!gx || aligned16(gx));
-    if (!make_plan(grid->io_dtype, *layout, al, want_pg, &p)) return AHQ_ERR_INVALID;
+    if (!make_plan(grid->io_dtype, *layout, al, want_pg, &p, kUnroll, true)) return AHQ_ERR_INVALID;
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (p.cl.numel == 0) return AHQ_OK;  // nothing to read: outputs are left untouched
     if (!x || !g) return set_error("x or g is null"), AHQ_ERR_INVALID;
     if (!gx && !want_pg) return AHQ_OK;
-    const size_t ws_need = p.ws_elems * 2 * sizeof(double);
+    const bool cols = bwd_cols_layout(grid->io_dtype, p, al);
+    const size_t ws_need = bwd_scratch_pairs(grid->io_dtype, p, al, want_pg) * 2 * sizeof(double);
     if (ws_need > 0 && (!workspace || workspace_bytes < ws_need)) return set_error("workspace too small"), AHQ_ERR_WORKSPACE;
     QdqArgs a{};
     a.x = x;
@@ -1279,7 +1382,8 @@ extern "C" int ahq_qdq_backward(const ahq_grid* grid, const ahq_layout* layout, 
     a.goffset = goffset;
     a.partials = ws_need ? static_cast<double*>(workspace) : nullptr;
     fill_args(*grid, p, &a);
-    if (p.red == kRedAtomic) {
+    const bool atomic = p.red == kRedAtomic && !cols;
+    if (atomic) {
         const int64_t n = p.cl.num_enc * 2;
         hipLaunchKernelGGL(zero_f64_kernel, dim3((unsigned)((n + 255) / 256 > 1024 ? 1024 : (n + 255) / 256)), dim3(256), 0, st, a.partials, n);
     }
@@ -1292,10 +1396,17 @@ extern "C" int ahq_qdq_backward(const ahq_grid* grid, const ahq_layout* layout, 
             hipLaunchKernelGGL(qdq_bwd_finish_kernel, dim3((unsigned)(nb > 4096 ? 4096 : nb)), dim3(kFinishThreads), 0, st, a);
         }
     }
-    if (p.red == kRedAtomic) {
+    if (atomic) {
         const int64_t n = p.cl.num_enc;
         hipLaunchKernelGGL(finish_atomic_kernel, dim3((unsigned)((n + 255) / 256 > 1024 ? 1024 : (n + 255) / 256)), dim3(256), 0, st,
                            (const double*)a.partials, gscale, goffset, n, (int)grid->compute_dtype);
+    }
+    if (want_pg && (cols || (p.red == kRedRuns && p.cl.I > 1))) {
+        // one slot per (row group, encoding) or per run: added up per encoding in a fixed order
+        const int64_t count = cols ? (int64_t)bwd_cols_row_groups(grid->io_dtype, p) : p.cl.I;
+        const int64_t nb = (p.cl.J + kBlock / kWave - 1) / (kBlock / kWave);
+        hipLaunchKernelGGL(qdq_bwd_strided_finish_kernel, dim3((unsigned)(nb > 4096 ? 4096 : nb)), dim3(kBlock), 0, st,
+                           (const double*)a.partials, count, p.cl.J, p.cl.J, gscale, goffset, (int)grid->compute_dtype);
     }
     return check_launch("ahq_qdq_backward");
 }

@@ -8,13 +8,18 @@
 
 namespace ahq {
 
-enum TileMode : int { kFlat = 0, kRows = 1 };
+// kFlat: tiles of tile_vec vectors over the flat tensor; kRows: tiles never leave a run (runs of at least half a tile);
+// kRuns: a tile is a whole number of neighbouring runs (runs shorter than half a tile)
+enum TileMode : int { kFlat = 0, kRows = 1, kRuns = 2 };
 // How per-encoding reductions leave the kernel:
 //   kRedTile    every tile lies inside one run; workgroup totals go straight to the output when one tile covers the
 //               whole encoding, else to a partials array that a second small launch adds in a fixed order
 //   kRedSeg     a run is a power-of-two number (<= 64) of neighbouring lanes: shuffle reduction, direct store
 //   kRedAtomic  anything else: atomics into a per-encoding scratch array, finished by a second tiny kernel
-enum RedMode : int { kRedNone = 0, kRedTile = 1, kRedSeg = 2, kRedAtomic = 3 };
+//   kRedRuns    (only on request, for sums whose order must not vary) tiles of whole runs: every run is summed inside
+//               its tile in a fixed order and stored -- straight to the output when each encoding has one run, else to
+//               one slot per run that a second launch adds up per encoding in a fixed order
+enum RedMode : int { kRedNone = 0, kRedTile = 1, kRedSeg = 2, kRedAtomic = 3, kRedRuns = 4 };
 
 // Geometry every tiled kernel receives (flat index = (i*J + j)*K + k, encoding index = j).
 struct Geom {
@@ -25,7 +30,7 @@ struct Geom {
     int32_t kv_shift;  // log2(Kv) when Kv is a power of two below the tile size, else -1
     int32_t tile_vec;  // vectors per tile: kBlock x (vectors per thread, at most kUnroll)
     int32_t mode;
-    int32_t tpr;   // tiles per row (kRows)
+    int32_t tpr;   // tiles per row (kRows); runs per tile (kRuns)
     uint32_t nblocks;
     int64_t ntiles;  // tiles in total (== nblocks: one tile per workgroup)
     // generic layout (per-element coordinate walk)
@@ -54,6 +59,15 @@ __device__ __forceinline__ Tile make_tile(const Geom& a, int64_t tile) {
         t.rem0 = tt * a.tile_vec;
         t.e0 = a.I == 1 ? row : row % a.J;
         t.nstage = 1;
+    } else if (a.mode == kRuns) {
+        const int64_t run0 = tile * a.tpr;
+        const int64_t left = a.I * a.J - run0;
+        const int n = (int)(left < a.tpr ? left : a.tpr);
+        t.v0 = run0 * a.Kv;
+        t.nv = n > 0 ? n * (int)a.Kv : 0;
+        t.rem0 = 0;
+        t.e0 = a.I == 1 ? run0 : run0 % a.J;
+        t.nstage = n > 0 ? n : 0;
     } else {
         t.v0 = tile * a.tile_vec;
         const int64_t left = a.nvec - t.v0;
@@ -96,13 +110,13 @@ struct Plan {
     CanonLayout cl;
     int vec;       // element vector width used (16 bytes worth, or 1)
     int mode;
-    int tpr;
+    int tpr;       // kRows: tiles per row; kRuns: runs per tile
     int red;
     uint32_t nblocks;
     int64_t Kv, nvec;
     int tile_vec;  // vectors per tile
     int64_t ntiles;
-    size_t ws_elems;  // kRedTile: number of tiles; kRedAtomic: number of encodings; else 0
+    size_t ws_elems;  // kRedTile: number of tiles; kRedAtomic: number of encodings; kRedRuns: runs if I > 1; else 0
 };
 
 inline int io_vec(int dtype) { return dtype == AHQ_F32 ? 4 : 8; }
@@ -111,9 +125,11 @@ inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
 inline bool is_pow2(int64_t v) { return v > 0 && (v & (v - 1)) == 0; }
 
 // Decide tiling and reduction strategy.  `ptr_aligned`: every tensor pointer is 16-byte aligned; `unroll`: vectors per
-// thread and tile the kernel family works with (its register arrays hold that many).
+// thread and tile the kernel family works with (its register arrays hold that many).  `ordered`: the reduction is a
+// floating-point sum whose result must not depend on the order workgroups finish in: short runs get kRedRuns instead
+// of kRedAtomic, unless that needs more scratch (one slot per run) than the tensor itself occupies.
 inline bool make_plan(int io_dtype, const ahq_layout& layout, bool ptr_aligned, bool want_red, Plan* p,
-                      int unroll = kUnroll) {
+                      int unroll = kUnroll, bool ordered = false) {
     const int tile_vec = kBlock * unroll;
     p->tile_vec = tile_vec;
     const char* err = nullptr;
@@ -151,11 +167,18 @@ inline bool make_plan(int io_dtype, const ahq_layout& layout, bool ptr_aligned, 
             p->red = kRedTile;
         } else if (c.I == 1 && is_pow2(p->Kv) && p->Kv <= kWave) {
             p->red = kRedSeg;
-        } else if (p->Kv >= tile_vec / 2) {
+        } else if (p->Kv > tile_vec / 2 || (p->Kv == tile_vec / 2 && !(ordered && c.I == 1))) {
+            // (runs of exactly half a tile go two to a tile when the sum is ordered anyway: full tiles, no finish)
             p->red = kRedTile;
             p->mode = kRows;
             p->tpr = (int)((p->Kv + tile_vec - 1) / tile_vec);
             nb = c.I * c.J * (int64_t)p->tpr;
+        } else if (ordered && (c.I == 1 || c.K * (int64_t)io_size(io_dtype) >= 16)) {
+            p->red = kRedRuns;
+            p->mode = kRuns;
+            p->tpr = (int)(tile_vec / p->Kv);
+            nb = (c.I * c.J + p->tpr - 1) / p->tpr;
+            p->ws_elems = c.I > 1 ? (size_t)(c.I * c.J) : 0;
         } else {
             p->red = kRedAtomic;
         }

@@ -35,6 +35,9 @@ LAYOUTS = [
     ((1100, 264), (1, 264), None),         # same, many rows per workgroup, lanes without columns
     ((1100, 24), (1, 24), None),           # too few columns for them: tiled kernel
     ((3, 40, 1536), (1536,), None),        # same, several groups of 64 lanes across
+    ((300, 24), (300, 1), None),           # whole runs per workgroup, one thread adds a run
+    ((37, 5, 48), (5, 1), None),           # whole runs per workgroup, each encoding met 37 times
+    ((12, 4096), (12, 1), None),           # runs of half a tile and less (16-bit): one wave adds a run
 ]
 
 DTYPES = [torch.float32, torch.bfloat16, torch.float16]
@@ -468,31 +471,44 @@ def test_offset_and_scale_of_different_shapes_broadcast(device, dtype, case):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=lambda d: str(d).split(".")[-1])
 @pytest.mark.parametrize("layout", [
-    ((8, 100), (8, 1), None),               # runs shorter than a tile
-    ((256, 4096), (256, 1), None),          # runs of a quarter / an eighth of a tile
-    ((4, 6, 10, 10), (6, 1, 1), None),      # short runs, each encoding met several times
-    ((8, 16), (2, 4), (4, 4)),              # generic walk
-    ((1100, 264), (1, 264), None),          # column-walking kernel
-    ((3, 40, 1536), (1536,), None),
+    ((8, 100), (8, 1), None, True),               # runs shorter than a tile
+    ((256, 4096), (256, 1), None, True),          # runs of a quarter / an eighth of a tile
+    ((300, 24), (300, 1), None, True),            # runs of a few vectors: one thread adds a run
+    ((4, 6, 10, 10), (6, 1, 1), None, True),      # short runs, each encoding met several times
+    ((37, 5, 48), (5, 1), None, True),
+    ((1100, 264), (1, 264), None, True),          # column-walking kernel, several row groups
+    ((3, 40, 1536), (1536,), None, True),
+    ((1100, 24), (1, 24), None, False),           # run length 1 without the column kernel: atomics
+    ((8, 16), (2, 4), (4, 4), False),             # generic walk: atomics
 ], ids=lambda l: "x".join(map(str, l[0])) + "_" + "x".join(map(str, l[1])))
-def test_parameter_gradients_repeat_on_layouts_that_sum_with_atomics(device, layout, dtype):
-    """Where one encoding's terms are spread over workgroups with no fixed meeting order, the scale / offset gradients
-    are summed with 64-bit floating-point atomics, whose order varies between runs.  The terms are float32 values
-    added in double precision, so two runs differ by about 1e-16 of the sum of magnitudes before the final rounding to
-    the compute dtype: repeated runs must agree to within one unit in the last place of that dtype (and in practice
-    agree exactly; a difference needs the double sums to straddle a rounding boundary of the narrower type)."""
+def test_parameter_gradients_repeat(device, layout, dtype):
+    """Scale / offset gradients are float32 terms added in double precision and rounded once.  On every layout of the
+    flat [outer, encoding, run] form the order of the additions is fixed by the layout (whole runs per workgroup,
+    lanes and waves combined in a fixed pattern, per-run or per-row-group partial sums added up by a second launch),
+    so repeated runs agree bit for bit.  Two kinds of layout still add with 64-bit floating-point atomics, in an
+    order that varies between runs: blocks along several dimensions (the generic walk) and runs of a single element
+    that the column kernel does not take.  There two runs differ by about 1e-16 of the sum of magnitudes before the
+    final rounding: they must agree to one unit in the last place of the compute dtype."""
     from aimet_amd.quantization import affine
 
-    shape, enc_shape, block = layout
+    shape, enc_shape, block, ordered = layout
     x, scale, offset, grad = _make_case(shape, enc_shape, dtype, -128, 127, True, seed=11)
     xd, gd = x.to(device), grad.to(device)
+    # other work in between changes which workgroups finish first
+    noise = torch.randn(1 << 20, device=device)
     runs = []
-    for _ in range(5):
+    for i in range(5):
         sd = scale.to(device).requires_grad_(True)
         od = offset.to(device).requires_grad_(True)
+        if i % 2:
+            noise.mul_(1.0001)
         affine.quantize_dequantize(xd, sd, od, -128, 127, block_size=block).backward(gd)
         runs.append((sd.grad.clone(), od.grad.clone()))
     ulp = float(torch.finfo(torch.float32 if dtype == torch.float32 else dtype).eps)
     for gs, go in runs[1:]:
-        assert_close_rel(gs, runs[0][0], ulp, "scale gradient of a repeated run", abs_floor=1e-30)
-        assert_close_rel(go, runs[0][1], ulp, "offset gradient of a repeated run", abs_floor=1e-30)
+        if ordered:
+            assert_same_bits(gs, runs[0][0], "scale gradient of a repeated run")
+            assert_same_bits(go, runs[0][1], "offset gradient of a repeated run")
+        else:
+            assert_close_rel(gs, runs[0][0], ulp, "scale gradient of a repeated run", abs_floor=1e-30)
+            assert_close_rel(go, runs[0][1], ulp, "offset gradient of a repeated run", abs_floor=1e-30)
