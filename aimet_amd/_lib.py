@@ -21,6 +21,7 @@ AHQ_OP_QDQ, AHQ_OP_QUANTIZE, AHQ_OP_DEQUANTIZE = 0, 1, 2
 
 DTYPE_CODE = {torch.float32: AHQ_F32, torch.float16: AHQ_F16, torch.bfloat16: AHQ_BF16}
 
+MINMAX_SLOTS_BYTES = 12 * 512  # AHQ_MINMAX_SLOTS_BYTES
 LIB_NAME = "libaimet_amd.so"
 LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), LIB_NAME)
 
@@ -114,6 +115,8 @@ _SIGNATURES = {
     "ahq_minmax_to_encodings": (ctypes.c_int, [ctypes.c_int32, _P, _P, ctypes.c_int64, ctypes.c_int64, ctypes.c_int32,
                                                ctypes.c_float, ctypes.c_float, ctypes.c_float, ctypes.c_float, _P, _P, _P,
                                                _P]),
+    "ahq_minmax_accumulate": (ctypes.c_int, [ctypes.c_int32, _P, ctypes.c_int64, _P, _P, ctypes.c_int32, _P]),
+    "ahq_minmax_slots_read": (ctypes.c_int, [ctypes.c_int32, _P, _P, _P, _P]),
     "ahq_minmax_finalize": (ctypes.c_int, [ctypes.c_int32, _P, _P, ctypes.c_int64, ctypes.c_int64, ctypes.c_int32,
                                            ctypes.c_float, ctypes.c_float, ctypes.c_float, ctypes.c_float, _P,
                                            ctypes.c_int32, _P, _P, ctypes.c_int64, ctypes.c_int64, ctypes.c_double, _P,

@@ -1077,7 +1077,8 @@ static dim3 cols_grid(const Plan& p, int64_t target) {
 template <typename IO, typename M>
 static void launch_fwd(const Plan& p, const QdqArgs& a, hipStream_t st, bool aligned) {
     if (cols_layout<IO>(p, aligned) && (p.cl.J / IoTraits<IO>::kVec + kWave - 1) / kWave <= 0x7fffffff) {
-        hipLaunchKernelGGL((qdq_fwd_cols_kernel<IO, IoTraits<IO>::kVec, M>), cols_grid<IO>(p, 2048), dim3(kColThreads), 0, st, a);
+        // a lane prepares kVec encodings before its first row: the more of them, the more rows it should walk
+        hipLaunchKernelGGL((qdq_fwd_cols_kernel<IO, IoTraits<IO>::kVec, M>), cols_grid<IO>(p, IoTraits<IO>::kVec > 4 ? 768 : 2048), dim3(kColThreads), 0, st, a);
         return;
     }
     if (p.cl.kind == kGeneric) {

@@ -49,6 +49,10 @@ struct MmFlatArgs : MmOut {
     float* part_min;   // [gridDim.x] partial extrema, folded by minmax_fold_kernel
     float* part_max;
     int* part_nan;
+    // accumulate: the partials are running statistics, one slot per workgroup ([kFlatMaxBlocks] each): a workgroup
+    // merges its result into its slot and nothing is folded; first: the slots hold nothing yet
+    int32_t accumulate;
+    int32_t first;
 };
 
 // Arguments of the two lean kernels below (runs of whole vectors on the leading axis): a few words instead of the
@@ -330,6 +334,25 @@ __global__ __launch_bounds__(kFlatBlock) void minmax_flat_kernel(const MmFlatArg
     }
     acc.nan |= unordered != 0 ? 1 : 0;
     const MinMax b = mm_block_reduce<kFlatBlock>(acc, red_smem);
+    if (a.accumulate) {
+        // min / max are idempotent and order-free, so slot b may hold the extrema of everything workgroup b has seen
+        // in any batch; whoever wants the statistics folds the slots (minmax_fold_kernel), once
+        if (threadIdx.x == 0) {
+            MinMax s = b;
+            if (!a.first) s = mm_merge(b, MinMax{a.part_min[blockIdx.x], a.part_max[blockIdx.x], a.part_nan[blockIdx.x]});
+            a.part_min[blockIdx.x] = s.mn;
+            a.part_max[blockIdx.x] = s.mx;
+            a.part_nan[blockIdx.x] = s.nan;
+        }
+        if (a.first && blockIdx.x == 0) {
+            for (int q = gridDim.x + threadIdx.x; q < kFlatMaxBlocks; q += kFlatBlock) {
+                a.part_min[q] = __builtin_inff();
+                a.part_max[q] = -__builtin_inff();
+                a.part_nan[q] = 0;
+            }
+        }
+        return;
+    }
     if (threadIdx.x == 0) {
         if (gridDim.x == 1) {
             mm_write<IO>(a, 0, b);
@@ -772,6 +795,67 @@ extern "C" int ahq_minmax_copy(int32_t dtype, const ahq_layout* layout, const vo
     if (y == x) return set_error("y must not alias x"), AHQ_ERR_INVALID;
     return minmax_impl(dtype, layout, x, y, out_min, out_max, run_min, run_max, finite_only, workspace, workspace_bytes,
                        stream);
+}
+
+// ------------------------------------------------------------------- running extrema as one slot per workgroup --
+static_assert(AHQ_MINMAX_SLOTS == kFlatMaxBlocks, "the slots are the partials of the single-encoding kernel");
+static_assert(AHQ_MINMAX_SLOTS_BYTES == 12 * kFlatMaxBlocks, "two floats and a flag per slot");
+
+static MmFlatArgs slot_args(void* slots) {
+    MmFlatArgs f{};
+    char* w = static_cast<char*>(slots);
+    f.part_min = reinterpret_cast<float*>(w);
+    f.part_max = reinterpret_cast<float*>(w + 4 * kFlatMaxBlocks);
+    f.part_nan = reinterpret_cast<int*>(w + 8 * kFlatMaxBlocks);
+    return f;
+}
+
+extern "C" int ahq_minmax_accumulate(int32_t dtype, const void* x, int64_t count, void* copy_to, void* slots,
+                                     int32_t first, void* stream) {
+    if (dtype < AHQ_F32 || dtype > AHQ_BF16) return set_error("bad dtype"), AHQ_ERR_INVALID;
+    if (count < 0) return set_error("negative element count"), AHQ_ERR_INVALID;
+    if (!slots || (reinterpret_cast<uintptr_t>(slots) & 3u)) return set_error("slots is null or misaligned"), AHQ_ERR_INVALID;
+    if (count > 0 && !x) return set_error("x is null"), AHQ_ERR_INVALID;
+    if (copy_to && copy_to == x) return set_error("copy_to must not alias x"), AHQ_ERR_INVALID;
+    if (count == 0 && !first) return AHQ_OK;  // nothing to add; an empty first batch still clears the slots
+    MmFlatArgs f = slot_args(slots);
+    f.x = x;
+    f.copy = copy_to;
+    f.numel = count;
+    const int vec = (aligned16(x) && (!copy_to || aligned16(copy_to))) ? io_vec(dtype) : 1;
+    f.nvec = count / vec;
+    f.accumulate = 1;
+    f.first = first ? 1 : 0;
+    const int64_t tiles = f.nvec > 0 ? (f.nvec + kFlatTileVec - 1) / kFlatTileVec : 1;
+    const unsigned nb = (unsigned)(tiles < kFlatMaxBlocks ? tiles : kFlatMaxBlocks);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+#define AHQ_LAUNCH_ACC(IO)                                                                                              \
+    do {                                                                                                                \
+        if (vec == 1) hipLaunchKernelGGL((minmax_flat_kernel<IO, 1, false>), dim3(nb), dim3(kFlatBlock), 0, st, f);        \
+        else hipLaunchKernelGGL((minmax_flat_kernel<IO, IoTraits<IO>::kVec, false>), dim3(nb), dim3(kFlatBlock), 0, st, f); \
+    } while (0)
+    switch (dtype) {
+        case AHQ_F32: AHQ_LAUNCH_ACC(float); break;
+        case AHQ_F16: AHQ_LAUNCH_ACC(f16_t); break;
+        default: AHQ_LAUNCH_ACC(bf16_t); break;
+    }
+#undef AHQ_LAUNCH_ACC
+    return check_launch("ahq_minmax_accumulate");
+}
+
+extern "C" int ahq_minmax_slots_read(int32_t dtype, const void* slots, void* out_min, void* out_max, void* stream) {
+    if (dtype < AHQ_F32 || dtype > AHQ_BF16) return set_error("bad dtype"), AHQ_ERR_INVALID;
+    if (!slots || !out_min || !out_max) return set_error("null argument"), AHQ_ERR_INVALID;
+    MmFlatArgs f = slot_args(const_cast<void*>(slots));
+    f.out_min = out_min;
+    f.out_max = out_max;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    switch (dtype) {
+        case AHQ_F32: hipLaunchKernelGGL((minmax_fold_kernel<float>), dim3(1), dim3(kFoldThreads), 0, st, f, kFlatMaxBlocks); break;
+        case AHQ_F16: hipLaunchKernelGGL((minmax_fold_kernel<f16_t>), dim3(1), dim3(kFoldThreads), 0, st, f, kFlatMaxBlocks); break;
+        default: hipLaunchKernelGGL((minmax_fold_kernel<bf16_t>), dim3(1), dim3(kFoldThreads), 0, st, f, kFlatMaxBlocks); break;
+    }
+    return check_launch("ahq_minmax_slots_read");
 }
 
 // ------------------------------------------------------------------------------------ entry point without allocation --

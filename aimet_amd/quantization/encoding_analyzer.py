@@ -123,6 +123,29 @@ class _MinMaxObserver(_Observer[_MinMaxRange]):
     def __init__(self, shape, block_size=None):
         super().__init__(shape, block_size)
         self.stats = _MinMaxRange()
+        # A single encoding observed through observe_and_clone() keeps its running extrema as one slot per workgroup
+        # of the streaming kernel (ahq_minmax_accumulate): no second launch per batch; the slots are folded into
+        # `stats` when somebody asks (get_stats, or any of the other ways of adding statistics, which then take over).
+        self._single = math.prod(self.shape) == 1 and not block_size
+        self._slots = None         # the slot buffer, kept across reset_stats()
+        self._slots_of = None      # (dtype, device) of the tensors accumulated while the slots are live, else None
+        self._slots_dirty = False  # the slots hold more than `stats`
+
+    def _fold_slots(self):
+        if self._slots_of is not None and self._slots_dirty:
+            dtype, device = self._slots_of
+            mn = torch.empty(self.shape, dtype=dtype, device=device)
+            mx = torch.empty(self.shape, dtype=dtype, device=device)
+            _lib.check(_lib.load().ahq_minmax_slots_read(_lib.DTYPE_CODE[dtype], self._slots.data_ptr(), mn.data_ptr(),
+                                                         mx.data_ptr(), _lib.current_stream(device)),
+                       "ahq_minmax_slots_read")
+            self.stats = _MinMaxRange(mn, mx)
+            self._slots_dirty = False
+
+    def _leave_slots(self):
+        """`stats` becomes the one place the running extrema live in."""
+        self._fold_slots()
+        self._slots_of = None
 
     @torch.no_grad()
     def collect_stats(self, input_tensor: torch.Tensor) -> _MinMaxRange:
@@ -131,6 +154,7 @@ class _MinMaxObserver(_Observer[_MinMaxRange]):
 
     @torch.no_grad()
     def merge_stats(self, stats: _MinMaxRange):
+        self._leave_slots()
         new_min, new_max = self.stats.min, self.stats.max
         if stats.min is not None:
             new_min = stats.min.clone() if new_min is None else torch.minimum(new_min, stats.min)
@@ -142,6 +166,7 @@ class _MinMaxObserver(_Observer[_MinMaxRange]):
     def update(self, input_tensor: torch.Tensor, copy_to: Optional[torch.Tensor] = None) -> _MinMaxRange:
         """collect + merge in one launch: the running fold happens where the reduction finishes.  ``copy_to``
         receives a copy of the input from the same pass (what pass-through calibration returns)."""
+        self._leave_slots()
         cur = self.stats
         fused = (
             cur.min is not None and cur.max is not None
@@ -163,9 +188,26 @@ class _MinMaxObserver(_Observer[_MinMaxRange]):
         pass-through calibration of a whole model: hundreds of these per forward pass).  Once the running statistics
         exist, everything that does not change from call to call -- layout, workspace, the two tensors the batch's
         extrema are written to -- is kept, and a call is one allocation (the copy) and one library call."""
+        x = input_tensor
+        if (self._single and x.is_cuda and x.dtype in _lib.DTYPE_CODE and x.is_contiguous() and not x.requires_grad
+                and x.numel() > 0):
+            of = (x.dtype, x.device)
+            first = self._slots_of is None and self.stats.min is None and self.stats.max is None
+            if first or self._slots_of == of:
+                if self._slots is None or self._slots.device != x.device:
+                    self._slots = torch.empty(_lib.MINMAX_SLOTS_BYTES, dtype=torch.uint8, device=x.device)
+                out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+                status = _lib.load().ahq_minmax_accumulate(_lib.DTYPE_CODE[x.dtype], x.data_ptr(), x.numel(),
+                                                           out.data_ptr(), self._slots.data_ptr(), 1 if first else 0,
+                                                           _lib.current_stream(x.device))
+                if status:
+                    _lib.check(status, "ahq_minmax_accumulate")
+                self._slots_of = of
+                self._slots_dirty = True
+                return out
+        self._leave_slots()
         fast = self.__dict__.get("_fast")
         cur = self.stats
-        x = input_tensor
         key = (x.shape, x.dtype, x.device)
         if (fast is None or fast[0] != key or fast[1] is not cur.min or fast[2] is not cur.max or not x.is_contiguous()
                 or x.requires_grad):
@@ -193,9 +235,12 @@ class _MinMaxObserver(_Observer[_MinMaxRange]):
 
     def reset_stats(self):
         self.stats = _MinMaxRange()
+        self._slots_of = None
+        self._slots_dirty = False
         self.__dict__["_fast"] = None
 
     def get_stats(self) -> _MinMaxRange:
+        self._fold_slots()
         return self.stats
 
 

@@ -149,6 +149,35 @@ def cpu_legs(step, unit_per_step, unit, sample, budget_s=4.0, max_reps=20, one_t
     return all_cores, one
 
 
+def device_ceiling(dev, nbytes=1 << 30):
+    """What the memory system gives the simplest possible kernels (ahq_diag_read / ahq_diag_copy: 16-byte loads
+    folded into a word, and a copy) on a buffer far larger than the last-level cache: the best of a few grid sizes,
+    each the median of repeated HIP-event timings.  The library's kernels are priced against the published 8 TB/s; this
+    says how much of the distance no kernel closes on this device."""
+    from aimet_amd import _lib
+
+    lib = _lib.load()
+    x = torch.empty(nbytes, dtype=torch.uint8, device=dev).random_(0, 255)
+    y = torch.empty_like(x)
+    out = torch.empty(65536, dtype=torch.int32, device=dev)
+    stream = _lib.current_stream(dev)
+    best = {"read": (0.0, 0), "copy": (0.0, 0)}
+    for wgs in (1024, 2048, 4096, 8192, 16384):
+        t_read = event_time(lambda: lib.ahq_diag_read(x.data_ptr(), nbytes, wgs, out.data_ptr(), stream), 10)
+        t_copy = event_time(lambda: lib.ahq_diag_copy(x.data_ptr(), y.data_ptr(), nbytes, wgs, stream), 10)
+        for kind, gbs in (("read", nbytes / t_read / 1e9), ("copy", 2 * nbytes / t_copy / 1e9)):
+            if gbs > best[kind][0]:
+                best[kind] = (gbs, wgs)
+    assert torch.equal(x[:1 << 20], y[:1 << 20]) and torch.equal(x[-(1 << 20):], y[-(1 << 20):])
+    del x, y
+    return {"read_GBps": round(best["read"][0], 1), "read_frac_of_peak": round(best["read"][0] / HBM_PEAK_GBS, 4),
+            "read_workgroups": best["read"][1],
+            "copy_GBps": round(best["copy"][0], 1), "copy_frac_of_peak": round(best["copy"][0] / HBM_PEAK_GBS, 4),
+            "copy_workgroups": best["copy"][1], "buffer_bytes": nbytes,
+            "note": "bare streaming kernels of this library (no arithmetic), read = bytes read / time, copy = bytes "
+                    "read + written / time; peak = published 8 TB/s"}
+
+
 def _copy_reference(dev):
     """One plain elementwise pass of known size (256 MiB read, 256 MiB written), outside every timed region: hardware
     counter runs of this script scale FETCH_SIZE / WRITE_SIZE of the kernels below by what they read for this one."""
@@ -955,6 +984,9 @@ def main():
         out["summary"] = {k: {"GBps": r["value"], "pct_of_hbm_peak": r["pct_of_hbm_peak"], "ms_per_step": r["ms_per_step"],
                               "elements_per_s": r["elements_per_s"], "roofline_frac": r["roofline"]["frac"]}
                           for k, r in [("c4", out)] + list(configs.items())}
+    if args.workload == "all":
+        _ensure_built()
+        out["device_ceiling"] = device_ceiling(dev)
     out["host"] = {"cpu_count": os.cpu_count(), "torch_threads": torch.get_num_threads(),
                    "device": torch.cuda.get_device_name(0)}
     out["bench_total_seconds"] = round(time.perf_counter() - t0, 1)

@@ -158,6 +158,20 @@ int    ahq_minmax_copy(int32_t dtype, const ahq_layout* layout, const void* x, v
 int    ahq_minmax_static(int32_t dtype, const ahq_layout* layout, const void* x, void* out_min, void* out_max,
                          void* run_min, void* run_max, int finite_only, void* stream);
 
+/* Running per-tensor extrema without a second launch per batch.  Replaces the same reference code as ahq_minmax
+ * (_MinMaxObserver.collect_stats + merge_stats, AT/quantization/encoding_analyzer.py:69-118) for a single encoding when
+ * the caller does not need the statistics between batches: `slots` (AHQ_MINMAX_SLOTS_BYTES bytes, 4-byte aligned,
+ * owned by the caller) holds one (min, max, saw-NaN) triple per workgroup of the streaming kernel; each call folds the
+ * batch into them in place (minimum and maximum are exact in any order and grouping), `first` != 0 starts them
+ * afresh.  copy_to (optional) receives a copy of the `count` elements of x from the same pass.  ahq_minmax_slots_read
+ * folds the slots into one (min, max) of `dtype`, with torch.amin / amax semantics (NaN if any element was NaN).
+ */
+#define AHQ_MINMAX_SLOTS 512
+#define AHQ_MINMAX_SLOTS_BYTES (12 * AHQ_MINMAX_SLOTS)
+int ahq_minmax_accumulate(int32_t dtype, const void* x, int64_t count, void* copy_to, void* slots, int32_t first,
+                          void* stream);
+int ahq_minmax_slots_read(int32_t dtype, const void* slots, void* out_min, void* out_max, void* stream);
+
 /* Replaces MinMaxEncodingAnalyzer.compute_encodings_from_stats (AT/quantization/encoding_analyzer.py:425-481) and the
  * checks of _flag_extreme_min_max (:484-498): zero forced into the range, ranges narrower than the minimum scale
  * widened, symmetric grids re-centred, the result clamped to the statistics dtype.  stat_min / stat_max / out_min /
