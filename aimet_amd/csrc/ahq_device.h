@@ -67,6 +67,27 @@ template <typename T, int N>
 __device__ __forceinline__ Pack<T, N> load_pack(const T* p) {
     return *reinterpret_cast<const Pack<T, N>*>(p);
 }
+// Non-temporal load, for kernels that only read.  Which kernels gain is an empirical matter on this part (same box,
+// back-to-back runs): a bare reduction over 1 GiB goes from 6.3 to 7.0 TB/s and the per-row min/max of a 67 MB tensor
+// from 11.4 to 10.0 us, the histogram stream gains 8 %; the quantize-dequantize kernels, which write as much as they
+// read, lose 10 % and the 8-lane block min/max loses 9 %, so those keep load_pack.
+template <typename T, int N>
+__device__ __forceinline__ Pack<T, N> load_pack_stream(const T* p) {
+    constexpr int kBytes = (int)sizeof(T) * N;
+    if constexpr (kBytes == 16) {
+        typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+        return __builtin_bit_cast(Pack<T, N>, __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p)));
+    } else if constexpr (kBytes == 8) {
+        typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+        return __builtin_bit_cast(Pack<T, N>, __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(p)));
+    } else if constexpr (kBytes == 4) {
+        return __builtin_bit_cast(Pack<T, N>, __builtin_nontemporal_load(reinterpret_cast<const unsigned int*>(p)));
+    } else if constexpr (kBytes == 2) {
+        return __builtin_bit_cast(Pack<T, N>, __builtin_nontemporal_load(reinterpret_cast<const unsigned short*>(p)));
+    } else {
+        return load_pack<T, N>(p);
+    }
+}
 template <typename T, int N>
 __device__ __forceinline__ void store_pack(T* p, const Pack<T, N>& v) {
     *reinterpret_cast<Pack<T, N>*>(p) = v;

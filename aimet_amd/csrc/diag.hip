@@ -12,6 +12,7 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 constexpr int kDiagThreads = 256;
 constexpr int kDiagUnroll = 4;
 
+template <bool NT>
 __global__ __launch_bounds__(kDiagThreads) void diag_read_kernel(const u32x4* __restrict__ x, int64_t nvec,
                                                                  uint32_t* __restrict__ out) {
     uint32_t acc = 0;
@@ -21,7 +22,7 @@ __global__ __launch_bounds__(kDiagThreads) void diag_read_kernel(const u32x4* __
 #pragma unroll
         for (int u = 0; u < kDiagUnroll; ++u) {
             const int64_t i = base + (int64_t)u * kDiagThreads;
-            v[u] = i < nvec ? __builtin_nontemporal_load(x + i) : u32x4{0u, 0u, 0u, 0u};
+            v[u] = i >= nvec ? u32x4{0u, 0u, 0u, 0u} : NT ? __builtin_nontemporal_load(x + i) : x[i];
         }
 #pragma unroll
         for (int u = 0; u < kDiagUnroll; ++u) acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
@@ -60,13 +61,18 @@ __global__ __launch_bounds__(kDiagThreads) void diag_copy_kernel(const u32x4* __
 
 using namespace ahq;
 
-extern "C" int ahq_diag_read(const void* x, size_t bytes, int32_t workgroups, uint32_t* out, void* stream) {
+extern "C" int ahq_diag_read(const void* x, size_t bytes, int32_t workgroups, int32_t nontemporal, uint32_t* out,
+                             void* stream) {
     if (!x || !out) return set_error("null argument"), AHQ_ERR_INVALID;
     if (bytes % 16 != 0 || (reinterpret_cast<uintptr_t>(x) & 15u)) return set_error("x must be 16-byte aligned and a multiple of 16 bytes long"), AHQ_ERR_INVALID;
     if (workgroups < 1 || workgroups > 65536) return set_error("workgroups must be in 1..65536"), AHQ_ERR_INVALID;
     if (bytes == 0) return AHQ_OK;
-    hipLaunchKernelGGL(diag_read_kernel, dim3((unsigned)workgroups), dim3(kDiagThreads), 0, static_cast<hipStream_t>(stream),
-                       static_cast<const u32x4*>(x), (int64_t)(bytes / 16), out);
+    if (nontemporal)
+        hipLaunchKernelGGL(diag_read_kernel<true>, dim3((unsigned)workgroups), dim3(kDiagThreads), 0,
+                           static_cast<hipStream_t>(stream), static_cast<const u32x4*>(x), (int64_t)(bytes / 16), out);
+    else
+        hipLaunchKernelGGL(diag_read_kernel<false>, dim3((unsigned)workgroups), dim3(kDiagThreads), 0,
+                           static_cast<hipStream_t>(stream), static_cast<const u32x4*>(x), (int64_t)(bytes / 16), out);
     return check_launch("ahq_diag_read");
 }
 

@@ -363,7 +363,7 @@ __global__ __launch_bounds__(kBlock, 6) void hist_bin_kernel(const BinArgs a) {
     for (int64_t tile = blockIdx.x; tile < full_tiles; tile += gridDim.x) {
         Pack<IO, VEC> in[kUnroll];
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u) in[u] = load_pack<IO, VEC>(x + (tile * kTileVec + u * kBlock + threadIdx.x) * VEC);
+        for (int u = 0; u < kUnroll; ++u) in[u] = load_pack_stream<IO, VEC>(x + (tile * kTileVec + u * kBlock + threadIdx.x) * VEC);
         if (track_all) {
             for (int u = 0; u < kUnroll; ++u)
                 for (int k = 0; k < VEC; ++k) track(load_f32(in[u].v[k]));
@@ -402,7 +402,7 @@ __global__ __launch_bounds__(kBlock, 6) void hist_bin_kernel(const BinArgs a) {
         for (int u = 0; u < kUnroll; ++u) {
             const int lv = u * kBlock + threadIdx.x;
             if (lv < nv) {
-                const Pack<IO, VEC> pk = load_pack<IO, VEC>(x + (v0 + lv) * VEC);
+                const Pack<IO, VEC> pk = load_pack_stream<IO, VEC>(x + (v0 + lv) * VEC);
                 for (int k = 0; k < VEC; ++k) bin_slow(load_f32(pk.v[k]), false);
             }
         }
@@ -507,7 +507,7 @@ __global__ __launch_bounds__(kBlock, 6) void hist_bin_rows_kernel(const BinArgs 
     if (t.nv == kTileVec) {
         Pack<IO, VEC> in[kUnroll];
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u) in[u] = load_pack<IO, VEC>(x + (int64_t)(u * kBlock + threadIdx.x) * VEC);
+        for (int u = 0; u < kUnroll; ++u) in[u] = load_pack_stream<IO, VEC>(x + (int64_t)(u * kBlock + threadIdx.x) * VEC);
         uint32_t binned = 0;
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u)
@@ -532,7 +532,7 @@ __global__ __launch_bounds__(kBlock, 6) void hist_bin_rows_kernel(const BinArgs 
         for (int u = 0; u < kUnroll; ++u) {
             const int lv = u * kBlock + threadIdx.x;
             if (lv < t.nv) {
-                const Pack<IO, VEC> pk = load_pack<IO, VEC>(x + (int64_t)lv * VEC);
+                const Pack<IO, VEC> pk = load_pack_stream<IO, VEC>(x + (int64_t)lv * VEC);
                 for (int k = 0; k < VEC; ++k) bin_slow(load_f32(pk.v[k]), false);
             }
         }

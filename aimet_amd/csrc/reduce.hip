@@ -302,12 +302,17 @@ __global__ __launch_bounds__(kFlatBlock) void minmax_flat_kernel(const MmFlatArg
     IO* __restrict__ cp = static_cast<IO*>(a.copy);
     MinMax acc = mm_identity();
     uint64_t unordered = 0;
+    // accumulate: what this workgroup's slot holds is asked for before the stream starts, so that the load's latency
+    // is not left over at the end of a kernel that lasts a few microseconds
+    MinMax held = mm_identity();
+    if (a.accumulate && !a.first && threadIdx.x == 0)
+        held = MinMax{a.part_min[blockIdx.x], a.part_max[blockIdx.x], a.part_nan[blockIdx.x]};
     const int64_t full_tiles = a.nvec / kFlatTileVec;
     for (int64_t tile = blockIdx.x; tile < full_tiles; tile += gridDim.x) {
         const int64_t v0 = tile * kFlatTileVec + threadIdx.x;
         Pack<IO, VEC> in[kFlatUnroll];
 #pragma unroll
-        for (int u = 0; u < kFlatUnroll; ++u) in[u] = load_pack<IO, VEC>(x + (v0 + u * kFlatBlock) * VEC);
+        for (int u = 0; u < kFlatUnroll; ++u) in[u] = load_pack_stream<IO, VEC>(x + (v0 + u * kFlatBlock) * VEC);
         if (cp) {
 #pragma unroll
             for (int u = 0; u < kFlatUnroll; ++u) store_pack<IO, VEC>(cp + (v0 + u * kFlatBlock) * VEC, in[u]);
@@ -318,7 +323,7 @@ __global__ __launch_bounds__(kFlatBlock) void minmax_flat_kernel(const MmFlatArg
     // the vectors past the last full tile: the workgroup after the one that took that tile
     if (blockIdx.x == full_tiles % gridDim.x) {
         for (int64_t v = full_tiles * kFlatTileVec + threadIdx.x; v < a.nvec; v += kFlatBlock) {
-            const Pack<IO, VEC> p = load_pack<IO, VEC>(x + v * VEC);
+            const Pack<IO, VEC> p = load_pack_stream<IO, VEC>(x + v * VEC);
             if (cp) store_pack<IO, VEC>(cp + v * VEC, p);
 #pragma unroll
             for (int k = 0; k < VEC; ++k) mm_add(acc, load_f32(p.v[k]), FINITE);
@@ -338,8 +343,7 @@ __global__ __launch_bounds__(kFlatBlock) void minmax_flat_kernel(const MmFlatArg
         // min / max are idempotent and order-free, so slot b may hold the extrema of everything workgroup b has seen
         // in any batch; whoever wants the statistics folds the slots (minmax_fold_kernel), once
         if (threadIdx.x == 0) {
-            MinMax s = b;
-            if (!a.first) s = mm_merge(b, MinMax{a.part_min[blockIdx.x], a.part_max[blockIdx.x], a.part_nan[blockIdx.x]});
+            const MinMax s = mm_merge(b, held);
             a.part_min[blockIdx.x] = s.mn;
             a.part_max[blockIdx.x] = s.mx;
             a.part_nan[blockIdx.x] = s.nan;
@@ -389,7 +393,7 @@ __global__ __launch_bounds__(BLOCK) void minmax_runs_kernel(const MmRunArgs a) {
     for (; v + (kUnroll - 1) * BLOCK < a.kv; v += kUnroll * BLOCK) {
         Pack<IO, VEC> in[kUnroll];
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u) in[u] = load_pack<IO, VEC>(x + (int64_t)(v + u * BLOCK) * VEC);
+        for (int u = 0; u < kUnroll; ++u) in[u] = load_pack_stream<IO, VEC>(x + (int64_t)(v + u * BLOCK) * VEC);
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) mm_pack<IO, VEC, MODE>(in[u], acc.mn, acc.mx, unordered);
     }
@@ -397,7 +401,7 @@ __global__ __launch_bounds__(BLOCK) void minmax_runs_kernel(const MmRunArgs a) {
     for (int v0 = v - threadIdx.x; v0 < a.kv; v0 += BLOCK) {
         const bool live = v0 + (int)threadIdx.x < a.kv;
         Pack<IO, VEC> pk;
-        if (live) pk = load_pack<IO, VEC>(x + (int64_t)(v0 + threadIdx.x) * VEC);
+        if (live) pk = load_pack_stream<IO, VEC>(x + (int64_t)(v0 + threadIdx.x) * VEC);
         else
 #pragma unroll
             for (int k = 0; k < VEC; ++k) pk.v[k] = IO{};
@@ -555,7 +559,7 @@ __global__ __launch_bounds__(kBlock) void minmax_cols_kernel(const MmArgs a) {
     for (int k = 0; k < VEC; ++k) m[k] = mm_identity();
 #pragma unroll 4
     for (int64_t r = r0; r < r1; ++r) {
-        const Pack<IO, VEC> pk = load_pack<IO, VEC>(x + r * a.J + c0);
+        const Pack<IO, VEC> pk = load_pack_stream<IO, VEC>(x + r * a.J + c0);
 #pragma unroll
         for (int k = 0; k < VEC; ++k) mm_add(m[k], load_f32(pk.v[k]), FINITE);
     }

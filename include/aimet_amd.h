@@ -405,11 +405,12 @@ int ahq_dlq_percentile_encodings(const ahq_dlq_pdf_state* state, float percentil
                                  int32_t strict, int32_t unsigned_sym, double* out, void* stream);
 
 /* Measurement aids for the benchmark; no counterpart in the reference.  ahq_diag_read streams `bytes` bytes through
- * 16-byte loads and folds them into one word per workgroup (out: `workgroups` words); ahq_diag_copy copies them.
- * Both are persistent grid-stride kernels of `workgroups` x 256 threads.  x, y: 16-byte aligned, bytes a multiple of
- * 16.  What they reach is the ceiling the memory system offers the library's streaming kernels on this device.
+ * 16-byte loads (non-temporal ones if `nontemporal`) and folds them into one word per workgroup (out: `workgroups`
+ * words); ahq_diag_copy copies them.  Both are persistent grid-stride kernels of `workgroups` x 256 threads.  x, y:
+ * 16-byte aligned, bytes a multiple of 16.  What they reach on buffers that are not already in the last-level cache is
+ * the ceiling the memory system offers the library's streaming kernels on this device.
  */
-int ahq_diag_read(const void* x, size_t bytes, int32_t workgroups, uint32_t* out, void* stream);
+int ahq_diag_read(const void* x, size_t bytes, int32_t workgroups, int32_t nontemporal, uint32_t* out, void* stream);
 int ahq_diag_copy(const void* x, void* y, size_t bytes, int32_t workgroups, void* stream);
 
 #ifdef __cplusplus
