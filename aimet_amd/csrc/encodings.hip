@@ -115,6 +115,54 @@ __global__ void range_to_scale_offset_kernel(const ScaleOffArgs a) {
     }
 }
 
+// ------------------------------------------------------ gradients of (scale, offset) -> gradients of (min, max) --
+// What autograd derives for get_scale / _get_offset above when min / max are learned (the chain SubBackward,
+// DivBackward, AbsBackward, ClampMinBackward and, for asymmetric grids, DivBackward, the straight-through round and
+// ClampBackward: a dozen small launches per training step), operation by operation in float32:
+//   gr     = goffset where -qmax <= round(min / s) - qmin <= -qmin, else 0            (clamp, straight-through round)
+//   gmin1  = gr / s;   gs' = gscale + (-gr * ((min / s) / s))                          (min / s)
+//   ga     = gs' where |d / n| >= minimum_scale, else 0;   g0 = ga * sgn(d / n)        (clamp_min, abs; d = max - min)
+//   gd     = g0 / n;   gmax = gd;   gmin = gmin1 + (-gd)                               (division by num_steps, max - min)
+// Symmetric grids have a constant offset: gr = 0.  Gradients that leave through a parameter of a narrower dtype P
+// are rounded to P where autograd casts them (each of the two terms of gmin, then their sum).
+struct RangeGradArgs {
+    const void* pmin;
+    const void* pmax;
+    const float* gscale;
+    const float* goffset;  // null: symmetric grid
+    void* gmin;
+    void* gmax;
+    int64_t n;
+    float num_steps, minimum_scale, qmin, lo, hi;  // lo = -qmax, hi = -qmin
+};
+
+template <typename P>
+__global__ void range_grad_kernel(const RangeGradArgs a) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= a.n) return;
+    using R = RoundTo<P>;
+    const float mn = load_f32(static_cast<const P*>(a.pmin)[i]);
+    const float mx = load_f32(static_cast<const P*>(a.pmax)[i]);
+    const float s0 = (mx - mn) / a.num_steps;
+    const float ab = __builtin_fabsf(s0);
+    const float s = (ab != ab) ? ab : fmaxf(ab, a.minimum_scale);
+    float gs = a.gscale[i];
+    float gmin1 = 0.f;
+    if (a.goffset) {
+        const float r = mn / s;
+        const float u = __builtin_rintf(r) - a.qmin;
+        const float gr = (u >= a.lo && u <= a.hi) ? a.goffset[i] : 0.f;
+        gmin1 = R::f(gr / s);
+        gs = gs + (-gr) * (r / s);
+    }
+    const float ga = (ab >= a.minimum_scale) ? gs : 0.f;
+    const float sg = (s0 > 0.f) ? 1.f : (s0 < 0.f) ? -1.f : 0.f;
+    const float gd = (ga * sg) / a.num_steps;
+    static_cast<P*>(a.gmax)[i] = store_cast<P>(gd);
+    const float gmin2 = R::f(-gd);
+    static_cast<P*>(a.gmin)[i] = store_cast<P>(a.goffset ? gmin1 + gmin2 : gmin2);
+}
+
 // ------------------------------------------------ statistics -> range, quantizer parameters, scale and offset --
 // The end of a min/max calibration in one launch: the encoding range of the statistics (minmax_to_encodings_kernel),
 // stored into the quantizer's min / max parameters in their own dtype P (what Tensor.copy_ does: round to nearest
@@ -378,6 +426,37 @@ extern "C" int ahq_lpbq_scale(int32_t dtype, const ahq_layout* grouping, const v
         default: hipLaunchKernelGGL((lpbq_scale_kernel<bf16_t>), g, b, 0, s, a); break;
     }
     return check_launch("lpbq_scale");
+}
+
+extern "C" int ahq_range_backward(int32_t dtype, const void* range_min, const void* range_max, int64_t num_encodings,
+                                  int64_t qmin, int64_t qmax, double minimum_scale, const float* grad_scale,
+                                  const float* grad_offset, void* grad_min, void* grad_max, void* stream) {
+    if (dtype < AHQ_F32 || dtype > AHQ_BF16) return set_error("bad dtype"), AHQ_ERR_INVALID;
+    if (!range_min || !range_max || !grad_scale || !grad_min || !grad_max) return set_error("null argument"), AHQ_ERR_INVALID;
+    if (num_encodings < 0) return set_error("negative encoding count"), AHQ_ERR_INVALID;
+    if (qmin >= qmax) return set_error("qmax must be larger than qmin"), AHQ_ERR_INVALID;
+    if (num_encodings == 0) return AHQ_OK;
+    RangeGradArgs a{};
+    a.pmin = range_min;
+    a.pmax = range_max;
+    a.gscale = grad_scale;
+    a.goffset = grad_offset;
+    a.gmin = grad_min;
+    a.gmax = grad_max;
+    a.n = num_encodings;
+    a.num_steps = (float)(double)(qmax - qmin);
+    a.minimum_scale = (float)minimum_scale;
+    a.qmin = (float)(double)qmin;
+    a.lo = (float)(double)(-qmax);
+    a.hi = (float)(double)(-qmin);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const dim3 g((unsigned)((num_encodings + 255) / 256)), b(256);
+    switch (dtype) {
+        case AHQ_F32: hipLaunchKernelGGL((range_grad_kernel<float>), g, b, 0, s, a); break;
+        case AHQ_F16: hipLaunchKernelGGL((range_grad_kernel<f16_t>), g, b, 0, s, a); break;
+        default: hipLaunchKernelGGL((range_grad_kernel<bf16_t>), g, b, 0, s, a); break;
+    }
+    return check_launch("range_backward");
 }
 
 static int fill_enc_args(EncArgs* a, int32_t dtype, const void* stat_min, const void* stat_max, int64_t num_encodings,

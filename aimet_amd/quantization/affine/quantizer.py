@@ -49,6 +49,53 @@ def _symmetric_offset(qmin: int, qmax: int, shape, dtype, device) -> torch.Tenso
     return off
 
 
+class _RangeToScaleOffset(torch.autograd.Function):
+    """(min, max) -> (scale, offset) in float32 with one launch each way (ahq_range_to_scale_offset /
+    ahq_range_backward) instead of the dozen elementwise operations of get_scale / _get_offset and the dozen autograd
+    nodes behind them (quantizer.py:319-376); the same float32 operations, so the same bits."""
+
+    @staticmethod
+    def forward(ctx, mn, mx, qmin, qmax, symmetric, constant_offset):  # pylint: disable=arguments-differ
+        lib = _lib.load()
+        scale = torch.empty(mn.shape, dtype=torch.float32, device=mn.device)
+        offset = constant_offset if symmetric else torch.empty(mn.shape, dtype=torch.float32, device=mn.device)
+        _lib.check(
+            lib.ahq_range_to_scale_offset(_lib.DTYPE_CODE[mn.dtype], mn.data_ptr(), mx.data_ptr(), mn.numel(), qmin, qmax,
+                                          _get_minimum_scale(qmax - qmin), scale.data_ptr(),
+                                          None if symmetric else offset.data_ptr(), _lib.current_stream(mn.device)),
+            "ahq_range_to_scale_offset")
+        ctx.save_for_backward(mn, mx)
+        ctx.grid = (qmin, qmax, symmetric)
+        ctx.set_materialize_grads(False)  # an output nobody used arrives as None, not as zeros
+        if symmetric:
+            ctx.mark_non_differentiable(offset)
+        return scale, offset
+
+    @staticmethod
+    def backward(ctx, gscale, goffset):  # pylint: disable=arguments-differ
+        mn, mx = ctx.saved_tensors
+        qmin, qmax, symmetric = ctx.grid
+        if gscale is None and (symmetric or goffset is None):
+            return None, None, None, None, None, None
+        shape, device = mn.shape, mn.device
+        if gscale is None:
+            gscale = torch.zeros(shape, dtype=torch.float32, device=device)
+        # an offset that nothing downstream used has no gradient path at all (a zero gradient would still meet
+        # infinite factors on its way)
+        symmetric = symmetric or goffset is None
+        gscale = gscale.to(torch.float32).contiguous()
+        if not symmetric:
+            goffset = goffset.to(torch.float32).contiguous()
+        gmin, gmax = torch.empty_like(mn), torch.empty_like(mx)
+        _lib.check(
+            _lib.load().ahq_range_backward(_lib.DTYPE_CODE[mn.dtype], mn.data_ptr(), mx.data_ptr(), mn.numel(), qmin, qmax,
+                                           _get_minimum_scale(qmax - qmin), gscale.data_ptr(),
+                                           None if symmetric else goffset.data_ptr(), gmin.data_ptr(), gmax.data_ptr(),
+                                           _lib.current_stream(device)),
+            "ahq_range_backward")
+        return gmin, gmax, None, None, None, None
+
+
 def _get_scale_offset(min: torch.Tensor, max: torch.Tensor, qmin: int, qmax: int, symmetric: bool):
     """scale = (max - min) / (qmax - qmin); offset = round(min / scale) - qmin, or the symmetric constant
     (quantizer.py:876-900)."""
@@ -198,17 +245,20 @@ class AffineQuantizerBase(QuantizerBase, _GridMixin):
 
     def _fused_scale_offset(self):
         """get_scale(float32) and _get_offset(float32) of a quantizer that holds min / max on a GPU in one launch
-        (ahq_range_to_scale_offset); None when that does not apply (gradients wanted, a subclass with its own scale,
-        parameters that are not on a GPU or not contiguous) and the step-by-step form has to run."""
+        (ahq_range_to_scale_offset; as an autograd node with a one-launch backward when min / max are learned); None
+        when that does not apply (a subclass with its own scale, parameters that are not on a GPU or not contiguous)
+        and the step-by-step form has to run."""
         cls = type(self)
         if cls.get_scale is not AffineQuantizerBase.get_scale or cls._get_offset is not AffineQuantizerBase._get_offset:
             return None
         mn, mx = self.min, self.max
-        if torch.is_grad_enabled() and (mn.requires_grad or mx.requires_grad):
-            return None
         if not (mn.is_cuda and mx.device == mn.device and mn.dtype == mx.dtype and mn.dtype in _lib.DTYPE_CODE
                 and mn.shape == mx.shape and mn.is_contiguous() and mx.is_contiguous()):
             return None
+        if torch.is_grad_enabled() and (mn.requires_grad or mx.requires_grad):
+            # learned ranges: the same kernel as one autograd node, with a one-launch backward
+            return _RangeToScaleOffset.apply(mn, mx, self.qmin, self.qmax, bool(self.symmetric),
+                                             self._constant_offset(mn.device) if self.symmetric else None)
         lib = _lib.load()
         scale = torch.empty(mn.shape, dtype=torch.float32, device=mn.device)
         if self.symmetric:

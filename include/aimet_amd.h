@@ -214,6 +214,17 @@ int ahq_minmax_finalize(int32_t stat_dtype, const void* stat_min, const void* st
                         void* param_min, void* param_max, int64_t qmin, int64_t qmax, double grid_minimum_scale,
                         float* scale, float* offset, void* stream);
 
+/* The backward pass of ahq_range_to_scale_offset: replaces the autograd chain of get_scale / _get_offset
+ * (AT/quantization/affine/quantizer.py:319-376) when min / max are learned -- SubBackward, DivBackward, AbsBackward,
+ * ClampMinBackward and, for asymmetric grids, DivBackward, the straight-through round (AT/utils.py:1250-1257) and
+ * ClampBackward -- with one launch that evaluates the same float32 operations.  grad_scale / grad_offset: float32
+ * gradients with respect to scale and offset (grad_offset NULL: symmetric grid); grad_min / grad_max: outputs in
+ * `dtype`, the dtype of range_min / range_max.
+ */
+int ahq_range_backward(int32_t dtype, const void* range_min, const void* range_max, int64_t num_encodings,
+                       int64_t qmin, int64_t qmax, double minimum_scale, const float* grad_scale,
+                       const float* grad_offset, void* grad_min, void* grad_max, void* stream);
+
 /* Replaces GroupedBlockQuantizeDequantize._get_scale / _get_per_channel_scale with dtype = float32 (LPBQ,
  * AT/quantization/affine/quantizer.py:1363-1399), which the reference runs on every forward through get_encodings():
  *   raw               = clamp_min(|float(max) - float(min)| / (qmax - qmin), minimum_scale)     (quantizer.py:319-339)

@@ -386,9 +386,71 @@ def test_scale_and_offset_from_a_range_in_one_launch(device, dtype, grid):
     # the step-by-step form on the device gives the same answer
     assert_same_bits(q.get_scale(), scale, "get_scale")
     assert_same_bits(q.get_offset(), offset, "get_offset")
-    # gradients wanted: the step-by-step form runs
+    # learned ranges: the same values as one autograd node
     with torch.enable_grad():
-        assert q._fused_scale_offset() is None
+        fused = q._fused_scale_offset()
+        assert fused[0].grad_fn is not None
+        assert_same_bits(fused[0], scale, "scale with grad")
+        assert_same_bits(fused[1], offset, "offset with grad")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16], ids=lambda d: str(d).split(".")[-1])
+@pytest.mark.parametrize("grid", [(0, 255, False), (-128, 127, True), (0, 15, False), (0, 65535, False), (3, 11, False),
+                                  (-8, 7, False)], ids=str)
+def test_learned_range_gradients_in_one_launch(device, dtype, grid):
+    """The gradients of min / max through get_scale / _get_offset (quantizer.py:319-376): ahq_range_backward against
+    what autograd derives for the reference's composition on the CPU, bit for bit -- ranges below the minimum scale,
+    reversed, zero, huge, NaN and infinite included, offsets on and beyond both clamp bounds."""
+    from aimet_amd.quantization.affine import QuantizeDequantize
+    from aimet_amd.quantization._utils import ste_round
+
+    qmin, qmax, symmetric = grid
+    g = torch.Generator().manual_seed(4)
+    n = 4096
+    lo = -torch.rand(n, generator=g) * torch.logspace(-10, 10, n)
+    hi = torch.rand(n, generator=g) * torch.logspace(10, -10, n)
+    lo[::7] = lo[::7].abs()            # positive minima: offsets clamp at -qmax ... -qmin and beyond
+    lo[1::11] *= 300.0
+    special = torch.tensor([0.0, -0.0, 1.0, -1.0, 1e-30, -1e-30, 3e38, -3e38, float("inf"), -float("inf"), float("nan"),
+                            0.1, -0.1, 65504.0, -65504.0, 2.5, -2.5])
+    lo = torch.cat([lo, special, special.flip(0), torch.zeros(17), -torch.ones(17)]).to(dtype)
+    hi = torch.cat([hi, special, special, special, special]).to(dtype)
+    gs = torch.randn(lo.numel(), generator=g) * torch.logspace(-3, 3, lo.numel())
+    go = torch.randn(lo.numel(), generator=g)
+
+    # the reference's composition on the CPU, autograd's own backward
+    mn_c, mx_c = lo.clone().requires_grad_(True), hi.clone().requires_grad_(True)
+    steps = qmax - qmin
+    scale_c = ((mx_c.to(torch.float32) - mn_c.to(torch.float32)) / steps).abs().clamp_min_(O.minimum_scale(steps)).to(torch.float32)
+    loss = (scale_c * gs).sum()
+    if not symmetric:
+        offset_c = torch.clamp(ste_round(mn_c / scale_c) - qmin, -qmax, -qmin).to(torch.float32)
+        loss = loss + (offset_c * go).sum()
+    loss.backward()
+
+    q = QuantizeDequantize((lo.numel(),), qmin=qmin, qmax=qmax, symmetric=symmetric).to(device=device, dtype=dtype)
+    with torch.no_grad():
+        q.set_range(lo.to(device), hi.to(device))
+    enc = q.get_encodings()
+    assert enc.scale.grad_fn is not None and type(enc.scale.grad_fn).__name__.startswith("_RangeToScaleOffset")
+    assert_same_bits(enc.scale, scale_c, "scale")
+    loss = (enc.scale * gs.to(device)).sum()
+    if not symmetric:
+        assert_same_bits(enc.offset, offset_c, "offset")
+        loss = loss + (enc.offset * go.to(device)).sum()
+    else:
+        assert not enc.offset.requires_grad
+    loss.backward()
+    assert q.min.grad.dtype == dtype
+    assert_same_bits(q.max.grad, mx_c.grad, "gradient of max")
+    assert_same_bits(q.min.grad, mn_c.grad, "gradient of min")
+    # only one of the two outputs used downstream
+    q.min.grad = q.max.grad = None
+    q.get_encodings().scale.sum().backward()
+    mn_c.grad = mx_c.grad = None
+    ((mx_c.to(torch.float32) - mn_c.to(torch.float32)) / steps).abs().clamp_min_(O.minimum_scale(steps)).sum().backward()
+    assert_same_bits(q.max.grad, mx_c.grad, "gradient of max, scale only")
+    assert_same_bits(q.min.grad, mn_c.grad, "gradient of min, scale only")
 
 
 @pytest.mark.parametrize("stat_dtype", [torch.float32, torch.float16, torch.bfloat16], ids=lambda d: str(d).split(".")[-1])
