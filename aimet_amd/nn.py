@@ -160,8 +160,13 @@ class QuantizedLinear(nn.Linear):
                     with torch.no_grad():
                         qtzr.set_range(scale * qtzr.qmin, scale * qtzr.qmax)
                     continue
-            with qtzr._compute_encodings(passthrough=True):  # pylint: disable=protected-access
-                _ = qtzr(param)
+            if isinstance(qtzr, AffineQuantizerBase):
+                qtzr._calibrate_on(param)  # pylint: disable=protected-access
+            else:
+                with qtzr._compute_encodings(passthrough=True):  # pylint: disable=protected-access
+                    _ = qtzr(param)
+            if getattr(qtzr, "encoding_analyzer", None) is not None:
+                qtzr.encoding_analyzer.reset_stats()  # nn/base.py:385-386
 
     def _patch_quantized_parameters(self, param_names: Optional[Iterable[str]] = None):
         """nn/base.py:296-324: a context in which the named parameters (all by default) hold their

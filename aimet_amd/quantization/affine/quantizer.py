@@ -454,7 +454,24 @@ class AffineQuantizerBase(QuantizerBase, _GridMixin):
         self.encoding_analyzer.reset_stats()
         with patch_attr(self, "forward", observing_forward):
             yield
+        self._set_range_from_statistics()
 
+    def _calibrate_on(self, tensor: torch.Tensor) -> None:
+        """``with self._compute_encodings(passthrough=True): self(tensor)`` for a caller that drops the result (the
+        calibration of a parameter, nn/base.py:378-383): the statistics are reset, the tensor is observed and the range
+        set, without the pass-through copy of the tensor and without patching the forward method."""
+        if not any(self._is_overwrite_allowed.values()):
+            return
+        self.encoding_analyzer.reset_stats()
+        if type(tensor) != torch.Tensor:  # pylint: disable=unidiomatic-typecheck
+            tensor = tensor.as_subclass(torch.Tensor)
+        if tensor.numel():
+            self.encoding_analyzer.update_stats(tensor.detach())
+        self._set_range_from_statistics()
+
+    def _set_range_from_statistics(self) -> None:
+        """What leaving compute_encodings() does (quantizer.py:678-698)."""
+        shape = self.shape
         if self._finalize_from_minmax():
             return
         try:

@@ -58,11 +58,10 @@ def test_every_quantizer_is_calibrated_like_the_oracle(calibrated):
         xs = seen[name]
         assert q.is_initialized()
         is_weight = name.endswith("param_quantizers.weight")
-        # a weight quantizer sees its weight once for calibration and once more on entry: the quantize-dequantized
-        # weight is formed once and serves every calibration pass (nothing it depends on changes inside the context)
-        assert len(xs) == (2 if is_weight else 3), name
-        if is_weight:
-            xs = xs[:1]
+        # a weight quantizer is calibrated on its weight without a forward call and called once on entry: the
+        # quantize-dequantized weight is formed once and serves every calibration pass (nothing it depends on changes
+        # inside the context)
+        assert len(xs) == (1 if is_weight else 3), name
         mn = mx = None
         for x in xs:
             a, b = O.reduce_minmax(x, tuple(q.shape), q.block_size)
