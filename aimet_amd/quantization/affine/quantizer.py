@@ -689,7 +689,16 @@ class GroupedBlockQuantizeDequantize(QuantizeDequantize):
             fused = self._fused_lpbq_scale()
             if fused is not None:
                 return fused
-        raw = super().get_scale(dtype)
+        raw = None
+        mn, mx = self.min, self.max
+        if (dtype in (None, torch.float32) and self.is_initialized() and torch.is_grad_enabled()
+                and (mn.requires_grad or mx.requires_grad) and mn.is_cuda and mx.device == mn.device
+                and mn.dtype == mx.dtype and mn.dtype in _lib.DTYPE_CODE and mn.shape == mx.shape
+                and mn.is_contiguous() and mx.is_contiguous()):
+            # learned ranges: the block scales before snapping as one autograd node (see _RangeToScaleOffset)
+            raw = _RangeToScaleOffset.apply(mn, mx, self.qmin, self.qmax, True, self._constant_offset(mn.device))[0]
+        if raw is None:
+            raw = super().get_scale(dtype)
         if raw is None:
             return None, None
         per_channel = self._get_per_channel_scale(raw)

@@ -540,3 +540,38 @@ def test_range_warnings_of_the_fused_calibration_end(device):
         with warnings.catch_warnings():
             warnings.simplefilter("error")
             run(1.0, deferred)
+
+
+def test_lpbq_learned_range_gradients_with_the_fused_block_scale_node(device, monkeypatch):
+    """With learned ranges the LPBQ block scales before snapping come from one autograd node (_RangeToScaleOffset);
+    the min / max gradients of a training step equal those of the step-by-step composition bit for bit."""
+    from aimet_amd.quantization.affine import GroupedBlockQuantizeDequantize
+    from aimet_amd.quantization.affine import quantizer as Q
+
+    g = torch.Generator().manual_seed(8)
+    w = (torch.randn(96, 512, generator=g) * 0.02).bfloat16().to(device)
+    grad = torch.randn(96, 512, generator=g).bfloat16().to(device)
+
+    def run(fused: bool):
+        q = GroupedBlockQuantizeDequantize(shape=(96, 8), bitwidth=4, symmetric=True, decompressed_bw=8,
+                                           block_size=(1, 64), block_grouping=(1, -1)).to(device)
+        with q.compute_encodings():
+            q(w)
+        calls = []
+        real = Q._RangeToScaleOffset.apply
+        if fused:
+            monkeypatch.setattr(Q._RangeToScaleOffset, "apply", lambda *a: calls.append(1) or real(*a))
+        else:
+            # a CPU-resident check in the condition fails first, so the step-by-step form runs
+            monkeypatch.setattr(Q._RangeToScaleOffset, "apply", lambda *a: (None, None))
+        wd = w.clone().requires_grad_(True)
+        y = q(wd)
+        y.backward(grad)
+        monkeypatch.undo()
+        assert bool(calls) == fused
+        return y.detach(), wd.grad, q.min.grad, q.max.grad
+
+    a, b = run(True), run(False)
+    for got, want, what in zip(a, b, ("output", "input gradient", "gradient of min", "gradient of max")):
+        assert_same_bits(got, want, what)
+    assert float(a[2].abs().sum()) > 0 and float(a[3].abs().sum()) > 0
