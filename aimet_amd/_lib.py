@@ -115,6 +115,8 @@ _SIGNATURES = {
     "ahq_minmax_to_encodings": (ctypes.c_int, [ctypes.c_int32, _P, _P, ctypes.c_int64, ctypes.c_int64, ctypes.c_int32,
                                                ctypes.c_float, ctypes.c_float, ctypes.c_float, ctypes.c_float, _P, _P, _P,
                                                _P]),
+    "ahq_lpbq_scale_backward": (ctypes.c_int, [ctypes.c_int32, ctypes.POINTER(Layout), _P, _P, ctypes.c_int64,
+                                               ctypes.c_int64, ctypes.c_double, ctypes.c_int32, _P, _P, _P, _P, _P]),
     "ahq_range_backward": (ctypes.c_int, [ctypes.c_int32, _P, _P, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
                                           ctypes.c_double, _P, _P, _P, _P, _P]),
     "ahq_minmax_accumulate": (ctypes.c_int, [ctypes.c_int32, _P, ctypes.c_int64, _P, _P, ctypes.c_int32, _P]),

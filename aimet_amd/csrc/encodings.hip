@@ -246,6 +246,95 @@ __global__ __launch_bounds__(kBlock) void lpbq_scale_kernel(const LpbqArgs a) {
     }
 }
 
+// LPBQ with learned ranges: the gradients of min / max given the gradient of the snapped block scales, i.e. the
+// backward pass of everything lpbq_scale_kernel computes, as autograd derives it for the reference's composition
+// (quantizer.py:1363-1399 on top of :319-342), in one launch.  Per group of blocks, with r_k the raw block scales,
+// L their maximum, pc = L / M and t_k = r_k / pc:
+//   quantize-dequantize of r by pc on the grid [1, M] (torch_builtins.py:727-831, float32 arithmetic, offset 0):
+//       in_k   = 1 <= rint(t_k) <= M
+//       gr1_k  = g_k where in_k, else 0
+//       gpc    = sum_k g_k * (in_k ? rint(t_k) - t_k : clamp(rint(t_k), 1, M))      [+ the gradient of pc itself]
+//   pc = L / M and L = amax(r):   gL = gpc / M;   gr2_k = (gL / #{k: r_k == L}) * [r_k == L]
+//   r_k = clamp_min(|max_k - min_k| / n, eps):   the symmetric branch of range_grad_kernel on gr1_k + gr2_k.
+// The sum runs in double precision in a fixed order (lanes stride over the group, then the fixed butterfly) and is
+// rounded once; the reference's float32 sum differs from it in the last bits, as for every scale gradient.
+struct LpbqGradArgs {
+    const void* pmin;
+    const void* pmax;
+    const float* gscale;        // gradient of the snapped block scales
+    const float* gper_channel;  // optional: gradient of the per-group scales themselves
+    void* gmin;
+    void* gmax;
+    int64_t groups, group_size;
+    float num_steps, minimum_scale, multipliers;
+};
+
+template <typename P>
+__global__ __launch_bounds__(kBlock) void lpbq_scale_grad_kernel(const LpbqGradArgs a) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t waves = (int64_t)gridDim.x * (kBlock / kWave);
+    const P* __restrict__ pmin = static_cast<const P*>(a.pmin);
+    const P* __restrict__ pmax = static_cast<const P*>(a.pmax);
+    P* __restrict__ gmin = static_cast<P*>(a.gmin);
+    P* __restrict__ gmax = static_cast<P*>(a.gmax);
+    for (int64_t g = (int64_t)blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave; g < a.groups; g += waves) {
+        const int64_t base = g * a.group_size;
+        auto raw_at = [&](int64_t i, float& s0, float& ab) {
+            s0 = (load_f32(pmax[i]) - load_f32(pmin[i])) / a.num_steps;
+            ab = __builtin_fabsf(s0);
+            return (ab != ab) ? ab : fmaxf(ab, a.minimum_scale);
+        };
+        // the group's maximum (NaN if any member is NaN, as torch.amax)
+        float largest = -__builtin_inff();
+        int nan = 0;
+        for (int64_t k = lane; k < a.group_size; k += kWave) {
+            float s0, ab;
+            const float r = raw_at(base + k, s0, ab);
+            nan |= (r != r) ? 1 : 0;
+            largest = fmaxf(largest, r);
+        }
+#pragma unroll
+        for (int m = kWave / 2; m >= 1; m >>= 1) {
+            largest = fmaxf(largest, __shfl_xor(largest, m, kWave));
+            nan |= __shfl_xor(nan, m, kWave);
+        }
+        if (nan) largest = __builtin_nanf("");
+        const float pc = largest / a.multipliers;
+        // gradient of pc and the number of members that attain the maximum
+        double sum = 0.0;
+        int ties = 0;
+        for (int64_t k = lane; k < a.group_size; k += kWave) {
+            float s0, ab;
+            const float r = raw_at(base + k, s0, ab);
+            const float t = r / pc;
+            const float xr = __builtin_rintf(t);
+            const bool in = (xr >= 1.f) & (xr <= a.multipliers);
+            const float xc = xr < 1.f ? 1.f : (xr > a.multipliers ? a.multipliers : xr);
+            sum += (double)(a.gscale[base + k] * (in ? xr - t : xc));
+            ties += (r == largest) ? 1 : 0;
+        }
+        sum = wave_reduce(sum, OpAddD());
+#pragma unroll
+        for (int m = kWave / 2; m >= 1; m >>= 1) ties += __shfl_xor(ties, m, kWave);
+        float gpc = (float)sum;
+        if (a.gper_channel) gpc = gpc + a.gper_channel[g];
+        const float share = (gpc / a.multipliers) / (float)ties;
+        for (int64_t k = lane; k < a.group_size; k += kWave) {
+            float s0, ab;
+            const float r = raw_at(base + k, s0, ab);
+            const float t = r / pc;
+            const float xr = __builtin_rintf(t);
+            const bool in = (xr >= 1.f) & (xr <= a.multipliers);
+            const float gr = (in ? a.gscale[base + k] : 0.f) + share * ((r == largest) ? 1.f : 0.f);
+            const float ga = (ab >= a.minimum_scale) ? gr : 0.f;
+            const float sg = (s0 > 0.f) ? 1.f : (s0 < 0.f) ? -1.f : 0.f;
+            const float gd = (ga * sg) / a.num_steps;
+            gmax[base + k] = store_cast<P>(gd);
+            gmin[base + k] = store_cast<P>(-gd);
+        }
+    }
+}
+
 // --------------------------------------------------------------------- "is this tensor already on a grid" test --
 // The early exit of _decompose_prequantized_tensor (aimet_torch/utils.py:2098-2118), which runs on every weight at
 // the start of a calibration: of the first 64 blocks take the first 2 * num_levels elements each, as float
@@ -426,6 +515,46 @@ extern "C" int ahq_lpbq_scale(int32_t dtype, const ahq_layout* grouping, const v
         default: hipLaunchKernelGGL((lpbq_scale_kernel<bf16_t>), g, b, 0, s, a); break;
     }
     return check_launch("lpbq_scale");
+}
+
+extern "C" int ahq_lpbq_scale_backward(int32_t dtype, const ahq_layout* grouping, const void* range_min,
+                                       const void* range_max, int64_t qmin, int64_t qmax, double minimum_scale,
+                                       int32_t num_multipliers, const float* grad_scale,
+                                       const float* grad_per_channel_scale, void* grad_min, void* grad_max,
+                                       void* stream) {
+    if (dtype < AHQ_F32 || dtype > AHQ_BF16) return set_error("bad dtype"), AHQ_ERR_INVALID;
+    if (!grouping || !range_min || !range_max || !grad_scale || !grad_min || !grad_max) return set_error("null argument"), AHQ_ERR_INVALID;
+    if (qmin >= qmax) return set_error("qmax must be larger than qmin"), AHQ_ERR_INVALID;
+    if (num_multipliers < 1 || num_multipliers > (1 << 24)) return set_error("num_multipliers must be in 1..2^24"), AHQ_ERR_INVALID;
+    CanonLayout c;
+    const char* err = nullptr;
+    if (!canonicalize(*grouping, &c, &err)) return set_error(err), AHQ_ERR_INVALID;
+    if (c.numel == 0) return AHQ_OK;
+    if (c.kind != kIJK || c.I != 1)
+        return set_error("groups whose blocks are not neighbours in memory are not supported by the fused LPBQ scale"), AHQ_ERR_UNSUPPORTED;
+    LpbqGradArgs a{};
+    a.pmin = range_min;
+    a.pmax = range_max;
+    a.gscale = grad_scale;
+    a.gper_channel = grad_per_channel_scale;
+    a.gmin = grad_min;
+    a.gmax = grad_max;
+    a.groups = c.J;
+    a.group_size = c.K;
+    a.num_steps = (float)(double)(qmax - qmin);
+    a.minimum_scale = (float)minimum_scale;
+    a.multipliers = (float)num_multipliers;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int64_t per_block = kBlock / kWave;
+    int64_t nb = (c.J + per_block - 1) / per_block;
+    if (nb > 65536) nb = 65536;
+    const dim3 g((unsigned)nb), b(kBlock);
+    switch (dtype) {
+        case AHQ_F32: hipLaunchKernelGGL((lpbq_scale_grad_kernel<float>), g, b, 0, s, a); break;
+        case AHQ_F16: hipLaunchKernelGGL((lpbq_scale_grad_kernel<f16_t>), g, b, 0, s, a); break;
+        default: hipLaunchKernelGGL((lpbq_scale_grad_kernel<bf16_t>), g, b, 0, s, a); break;
+    }
+    return check_launch("lpbq_scale_backward");
 }
 
 extern "C" int ahq_range_backward(int32_t dtype, const void* range_min, const void* range_max, int64_t num_encodings,

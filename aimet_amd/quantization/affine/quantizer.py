@@ -96,6 +96,46 @@ class _RangeToScaleOffset(torch.autograd.Function):
         return gmin, gmax, None, None, None, None
 
 
+class _LpbqScale(torch.autograd.Function):
+    """(min, max) -> (LPBQ block scales, per-group scales) in float32 with one launch each way (ahq_lpbq_scale /
+    ahq_lpbq_scale_backward) instead of the reference's sequence -- get_scale, group maximum, division,
+    quantize-dequantize of the block scales (quantizer.py:1363-1399) -- and the autograd nodes behind it."""
+
+    @staticmethod
+    def forward(ctx, mn, mx, qmin, qmax, multipliers, layout, group_shape):  # pylint: disable=arguments-differ
+        scale = torch.empty(mn.shape, dtype=torch.float32, device=mn.device)
+        per_channel = torch.empty(group_shape, dtype=torch.float32, device=mn.device)
+        _lib.check(
+            _lib.load().ahq_lpbq_scale(_lib.DTYPE_CODE[mn.dtype], layout, mn.data_ptr(), mx.data_ptr(), qmin, qmax,
+                                       _get_minimum_scale(qmax - qmin), multipliers, scale.data_ptr(),
+                                       per_channel.data_ptr(), _lib.current_stream(mn.device)),
+            "ahq_lpbq_scale")
+        ctx.save_for_backward(mn, mx)
+        ctx.args = (qmin, qmax, multipliers, layout)
+        ctx.set_materialize_grads(False)
+        return scale, per_channel
+
+    @staticmethod
+    def backward(ctx, gscale, gper_channel):  # pylint: disable=arguments-differ
+        mn, mx = ctx.saved_tensors
+        qmin, qmax, multipliers, layout = ctx.args
+        if gscale is None and gper_channel is None:
+            return (None,) * 7
+        if gscale is None:
+            gscale = torch.zeros(mn.shape, dtype=torch.float32, device=mn.device)
+        gscale = gscale.to(torch.float32).contiguous()
+        if gper_channel is not None:
+            gper_channel = gper_channel.to(torch.float32).contiguous()
+        gmin, gmax = torch.empty_like(mn), torch.empty_like(mx)
+        _lib.check(
+            _lib.load().ahq_lpbq_scale_backward(_lib.DTYPE_CODE[mn.dtype], layout, mn.data_ptr(), mx.data_ptr(), qmin,
+                                                qmax, _get_minimum_scale(qmax - qmin), multipliers, gscale.data_ptr(),
+                                                _lib.ptr(gper_channel), gmin.data_ptr(), gmax.data_ptr(),
+                                                _lib.current_stream(mn.device)),
+            "ahq_lpbq_scale_backward")
+        return gmin, gmax, None, None, None, None, None
+
+
 def _get_scale_offset(min: torch.Tensor, max: torch.Tensor, qmin: int, qmax: int, symmetric: bool):
     """scale = (max - min) / (qmax - qmin); offset = round(min / scale) - qmin, or the symmetric constant
     (quantizer.py:876-900)."""
@@ -659,12 +699,10 @@ class GroupedBlockQuantizeDequantize(QuantizeDequantize):
         return None if raw is None else self._get_per_channel_scale(raw)
 
     def _fused_lpbq_scale(self):
-        """(scale, per-channel scale) in float32 from one launch of ahq_lpbq_scale; None when that does not apply
-        (gradients wanted, parameters not on a GPU, groups that are not runs of neighbouring blocks) and the
-        step-by-step form has to run."""
+        """(scale, per-channel scale) in float32 from one launch of ahq_lpbq_scale -- as an autograd node with a
+        one-launch backward when min / max are learned; None when that does not apply (parameters not on a GPU,
+        groups that are not runs of neighbouring blocks) and the step-by-step form has to run."""
         mn, mx = self.min, self.max
-        if torch.is_grad_enabled() and (mn.requires_grad or mx.requires_grad):
-            return None
         if not (mn.is_cuda and mx.device == mn.device and mn.dtype == mx.dtype and mn.dtype in _lib.DTYPE_CODE
                 and mn.shape == mx.shape and mn.is_contiguous() and mx.is_contiguous() and mn.numel() > 0):
             return None
@@ -673,15 +711,28 @@ class GroupedBlockQuantizeDequantize(QuantizeDequantize):
         shape = tuple(mn.shape)
         group_shape = tuple(d // g if g != -1 else 1 for d, g in zip(shape, self.block_grouping))
         layout = _build_layout(shape, tuple(range(len(shape))), group_shape, tuple(self.block_grouping))
+        multipliers = 2 ** (self.decompressed_bw - self.bitwidth)
+        unsupported = self.__dict__.get("_lpbq_unsupported")
+        if unsupported == (shape, tuple(self.block_grouping)):
+            return None
+        if torch.is_grad_enabled() and (mn.requires_grad or mx.requires_grad):
+            # the library refuses some groupings; find out once, outside autograd
+            if self.__dict__.get("_lpbq_supported") != (shape, tuple(self.block_grouping)):
+                with torch.no_grad():
+                    if self._fused_lpbq_scale() is None:
+                        return None
+            return _LpbqScale.apply(mn, mx, self.qmin, self.qmax, multipliers, layout, group_shape)
         lib = _lib.load()
         scale = torch.empty(shape, dtype=torch.float32, device=mn.device)
         per_channel = torch.empty(group_shape, dtype=torch.float32, device=mn.device)
         status = lib.ahq_lpbq_scale(_lib.DTYPE_CODE[mn.dtype], layout, mn.data_ptr(), mx.data_ptr(), self.qmin, self.qmax,
-                                    _get_minimum_scale(self.qmax - self.qmin), 2 ** (self.decompressed_bw - self.bitwidth),
+                                    _get_minimum_scale(self.qmax - self.qmin), multipliers,
                                     scale.data_ptr(), per_channel.data_ptr(), _lib.current_stream(mn.device))
         if status == _lib.AHQ_ERR_UNSUPPORTED:
+            self.__dict__["_lpbq_unsupported"] = (shape, tuple(self.block_grouping))
             return None
         _lib.check(status, "ahq_lpbq_scale")
+        self.__dict__["_lpbq_supported"] = (shape, tuple(self.block_grouping))
         return scale, per_channel
 
     def _get_scale(self, dtype=None):

@@ -214,6 +214,18 @@ int ahq_minmax_finalize(int32_t stat_dtype, const void* stat_min, const void* st
                         void* param_min, void* param_max, int64_t qmin, int64_t qmax, double grid_minimum_scale,
                         float* scale, float* offset, void* stream);
 
+/* The backward pass of ahq_lpbq_scale: replaces the autograd chain of GroupedBlockQuantizeDequantize._get_scale
+ * (AT/quantization/affine/quantizer.py:1363-1399 on top of :319-342) when min / max are learned -- the backward of
+ * the quantize-dequantize of the block scales (AT/quantization/affine/backends/torch_builtins.py:727-831), of the
+ * division by the number of multipliers, of torch.amax over each group and of get_scale -- with one launch.
+ * grad_scale: float32 gradient with respect to `scale`; grad_per_channel_scale: optional float32 gradient with respect
+ * to `per_channel_scale`; grad_min / grad_max: outputs in `dtype`.  Same grouping restriction as ahq_lpbq_scale.
+ */
+int ahq_lpbq_scale_backward(int32_t dtype, const ahq_layout* grouping, const void* range_min, const void* range_max,
+                            int64_t qmin, int64_t qmax, double minimum_scale, int32_t num_multipliers,
+                            const float* grad_scale, const float* grad_per_channel_scale, void* grad_min,
+                            void* grad_max, void* stream);
+
 /* The backward pass of ahq_range_to_scale_offset: replaces the autograd chain of get_scale / _get_offset
  * (AT/quantization/affine/quantizer.py:319-376) when min / max are learned -- SubBackward, DivBackward, AbsBackward,
  * ClampMinBackward and, for asymmetric grids, DivBackward, the straight-through round (AT/utils.py:1250-1257) and

@@ -227,8 +227,9 @@ def test_lpbq_c4_like(device):
 ], ids=["rows", "fours", "conv", "long_groups", "two_dimensional_groups", "column_groups"])
 @pytest.mark.parametrize("param_dtype", [torch.float32, torch.bfloat16], ids=["f32_params", "bf16_params"])
 def test_lpbq_scale_in_one_launch(device, case, param_dtype):
-    """Without gradients get_encodings() derives the LPBQ scales with one launch (ahq_lpbq_scale); with gradients it
-    runs the reference's sequence of torch operations.  Both must give the oracle's bits."""
+    """get_encodings() derives the LPBQ scales with one launch (ahq_lpbq_scale), as an autograd node when min / max
+    are learned; groupings the library declines run the reference's sequence of torch operations.  All must give the
+    oracle's bits."""
     from aimet_amd.quantization.affine import GroupedBlockQuantizeDequantize
 
     shape, block, grouping, wshape = case
@@ -248,9 +249,11 @@ def test_lpbq_scale_in_one_launch(device, case, param_dtype):
         enc = q.get_encodings()
     assert_same_bits(enc.per_channel_scale, pcs_ref, "per-channel scale (one launch)")
     assert_same_bits(enc.scale, scale_ref, "LPBQ scale (one launch)")
-    enc_grad = q.get_encodings()  # min / max require gradients: step-by-step form
+    enc_grad = q.get_encodings()  # min / max require gradients
     assert enc_grad.scale.requires_grad
-    assert_same_bits(enc_grad.scale, scale_ref, "LPBQ scale (step by step)")
+    assert_same_bits(enc_grad.scale, scale_ref, "LPBQ scale (with gradients)")
+    fused = type(enc_grad.scale.grad_fn).__name__.startswith("_LpbqScale")
+    assert fused == (case[0] not in ((8, 6), (64, 10)))
     mult = enc.per_block_int_scale.detach().cpu()
     assert mult.min() >= 1 and mult.max() <= 16 and torch.equal(mult, mult.round())
     assert mult.unique().numel() > 4
@@ -542,11 +545,11 @@ def test_range_warnings_of_the_fused_calibration_end(device):
             run(1.0, deferred)
 
 
-def test_lpbq_learned_range_gradients_with_the_fused_block_scale_node(device, monkeypatch):
-    """With learned ranges the LPBQ block scales before snapping come from one autograd node (_RangeToScaleOffset);
-    the min / max gradients of a training step equal those of the step-by-step composition bit for bit."""
+def test_lpbq_training_step_with_the_fused_scale_node(device):
+    """A training step of an LPBQ quantizer with learned ranges: with the block scales from the one-launch autograd
+    node (_LpbqScale) output and input gradient equal those of the step-by-step composition bit for bit, and the
+    min / max gradients agree to the tolerance of the per-group sums (double precision against float32)."""
     from aimet_amd.quantization.affine import GroupedBlockQuantizeDequantize
-    from aimet_amd.quantization.affine import quantizer as Q
 
     g = torch.Generator().manual_seed(8)
     w = (torch.randn(96, 512, generator=g) * 0.02).bfloat16().to(device)
@@ -557,21 +560,99 @@ def test_lpbq_learned_range_gradients_with_the_fused_block_scale_node(device, mo
                                            block_size=(1, 64), block_grouping=(1, -1)).to(device)
         with q.compute_encodings():
             q(w)
-        calls = []
-        real = Q._RangeToScaleOffset.apply
-        if fused:
-            monkeypatch.setattr(Q._RangeToScaleOffset, "apply", lambda *a: calls.append(1) or real(*a))
-        else:
-            # a CPU-resident check in the condition fails first, so the step-by-step form runs
-            monkeypatch.setattr(Q._RangeToScaleOffset, "apply", lambda *a: (None, None))
+        if not fused:
+            q.__dict__["_lpbq_unsupported"] = ((96, 8), (1, -1))  # what a grouping the library declines leaves behind
+        name = type(q.get_encodings().scale.grad_fn).__name__
+        assert name.startswith("_LpbqScale") == fused
         wd = w.clone().requires_grad_(True)
         y = q(wd)
         y.backward(grad)
-        monkeypatch.undo()
-        assert bool(calls) == fused
         return y.detach(), wd.grad, q.min.grad, q.max.grad
 
     a, b = run(True), run(False)
-    for got, want, what in zip(a, b, ("output", "input gradient", "gradient of min", "gradient of max")):
-        assert_same_bits(got, want, what)
+    assert_same_bits(a[0], b[0], "output")
+    assert_same_bits(a[1], b[1], "input gradient")
+    assert_close_rel(a[2], b[2], 1e-5, "gradient of min", abs_floor=1e-30)
+    assert_close_rel(a[3], b[3], 1e-5, "gradient of max", abs_floor=1e-30)
     assert float(a[2].abs().sum()) > 0 and float(a[3].abs().sum()) > 0
+
+
+class _OracleScaleQdq(torch.autograd.Function):
+    """The reference's quantize-dequantize with its hand-written backward (torch_builtins.py:727-831), on the CPU."""
+
+    @staticmethod
+    def forward(ctx, x, scale, qmin, qmax, block):
+        ctx.save_for_backward(x, scale)
+        ctx.args = (qmin, qmax, block)
+        return O.qdq_v2_forward(x.detach(), scale.detach(), torch.zeros_like(scale), qmin, qmax, block).y
+
+    @staticmethod
+    def backward(ctx, g):
+        x, scale = ctx.saved_tensors
+        qmin, qmax, block = ctx.args
+        gx, gs, _ = O.qdq_v2_backward(g, x.detach(), scale.detach(), torch.zeros_like(scale), qmin, qmax, block)
+        return gx, gs.view(scale.shape), None, None, None
+
+
+@pytest.mark.parametrize("case", [
+    ((96, 8), (1, -1), 16),           # C4's grouping
+    ((40, 12), (1, 4), 16),           # groups of four neighbouring blocks
+    ((6, 130), (1, -1), 256),         # groups longer than a wave, 8 extra bits
+    ((10, 64, 1, 1), (1, 64, 1, 1), 16),
+], ids=["rows", "fours", "long_groups", "conv"])
+@pytest.mark.parametrize("param_dtype", [torch.float32, torch.bfloat16], ids=["f32_params", "bf16_params"])
+def test_lpbq_learned_range_gradients_in_one_launch(device, case, param_dtype):
+    """ahq_lpbq_scale_backward against the CPU: autograd through get_scale, torch.amax and the division, and the
+    reference's own backward formulas for the quantize-dequantize of the block scales.  The per-group sum is taken
+    in double precision here and in float32 there: 1e-5 relative, as for every scale gradient; ties for the group
+    maximum, ranges below the minimum scale and reversed ranges included."""
+    from aimet_amd.quantization.affine import GroupedBlockQuantizeDequantize
+    from aimet_amd.quantization.affine import quantizer as Q
+
+    shape, grouping, mult = case
+    bw = 4
+    dbw = bw + {16: 4, 256: 8}[mult]
+    g = torch.Generator().manual_seed(13)
+    hi = (torch.rand(shape, generator=g) * 0.1 + 1e-3)
+    hi.view(-1)[::5] *= 7.0
+    hi.view(-1)[3] = 0.0                      # below the minimum scale
+    lo = -hi * (8.0 / 7.0)
+    lo.view(-1)[7], hi.view(-1)[7] = hi.view(-1)[7].clone(), lo.view(-1)[7].clone()   # reversed range
+    flat = hi.view(shape[0], -1)
+    flat[1, 1] = flat[1].max()                # two members attain the group maximum
+    lo.view(shape[0], -1)[1, 1] = -flat[1, 1] * (8.0 / 7.0)
+    j = int(flat[1].argmax())
+    lo.view(shape[0], -1)[1, j] = -flat[1, j] * (8.0 / 7.0)
+    lo, hi = lo.to(param_dtype), hi.to(param_dtype)
+    up = torch.randn(shape, generator=g)
+
+    # CPU: the reference's composition
+    mn_c, mx_c = lo.clone().requires_grad_(True), hi.clone().requires_grad_(True)
+    raw = ((mx_c.to(torch.float32) - mn_c.to(torch.float32)) / 15).abs().clamp_min_(O.minimum_scale(15))
+    pcs_shape = [d // gsz if gsz != -1 else 1 for d, gsz in zip(shape, grouping)]
+    cg = O.concrete_block_size(shape, pcs_shape, grouping)
+    resh = raw.reshape(*O.interleave(pcs_shape, cg))
+    pcs = torch.amax(resh, dim=tuple(range(1, resh.dim(), 2))) / mult
+    snapped = _OracleScaleQdq.apply(raw, pcs, 1, mult, grouping)
+    (snapped * up).sum().backward()
+
+    q = GroupedBlockQuantizeDequantize(shape=shape, bitwidth=bw, symmetric=True, decompressed_bw=dbw,
+                                       block_size=None if len(shape) != 2 else None, block_grouping=grouping)
+    q = q.to(device=device, dtype=param_dtype)
+    with torch.no_grad():
+        q.min.copy_(lo.to(device))
+        q.max.copy_(hi.to(device))
+    scale = q.get_encodings().scale
+    assert type(scale.grad_fn).__name__.startswith("_LpbqScale")
+    assert_same_bits(scale, snapped, "LPBQ scale")
+    (scale * up.to(device)).sum().backward()
+    tol = 1e-5 if param_dtype == torch.float32 else float(torch.finfo(param_dtype).eps)
+    assert_close_rel(q.max.grad, mx_c.grad, tol, "gradient of max", abs_floor=1e-30)
+    assert_close_rel(q.min.grad, mn_c.grad, tol, "gradient of min", abs_floor=1e-30)
+    # and the step-by-step composition on the device gives the same gradients to the same tolerance
+    q.min.grad = q.max.grad = None
+    q.__dict__["_lpbq_unsupported"] = (tuple(shape), tuple(grouping))
+    scale2 = q.get_encodings().scale
+    assert not type(scale2.grad_fn).__name__.startswith("_LpbqScale")
+    (scale2 * up.to(device)).sum().backward()
+    assert_close_rel(q.max.grad, mx_c.grad, tol, "gradient of max, step by step", abs_floor=1e-30)
