@@ -190,7 +190,7 @@ class _MinMaxObserver(_Observer[_MinMaxRange]):
         extrema are written to -- is kept, and a call is one allocation (the copy) and one library call."""
         x = input_tensor
         if (self._single and x.is_cuda and x.dtype in _lib.DTYPE_CODE and x.is_contiguous() and not x.requires_grad
-                and x.numel() > 0):
+                and x.numel() > 0 and len(self.shape) <= x.dim()):
             of = (x.dtype, x.device)
             first = self._slots_of is None and self.stats.min is None and self.stats.max is None
             if first or self._slots_of == of:
