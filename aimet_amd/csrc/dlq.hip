@@ -216,7 +216,7 @@ __global__ __launch_bounds__(THREADS) void dlq_pdf_bin_kernel(const PdfBinArgs a
     Pack<IO, VEC> bufa[kPdfUnroll], bufb[kPdfUnroll];
     auto load_tile = [&](Pack<IO, VEC>* buf, int64_t t) {
 #pragma unroll
-        for (int u = 0; u < kPdfUnroll; ++u) buf[u] = load_pack<IO, VEC>(x + (t * kTile + u * THREADS + threadIdx.x) * VEC);
+        for (int u = 0; u < kPdfUnroll; ++u) buf[u] = load_pack_stream<IO, VEC>(x + (t * kTile + u * THREADS + threadIdx.x) * VEC);
     };
     auto bin_tile = [&](const Pack<IO, VEC>* buf) {
 #pragma unroll
@@ -240,7 +240,7 @@ __global__ __launch_bounds__(THREADS) void dlq_pdf_bin_kernel(const PdfBinArgs a
     }
     if (blockIdx.x == 0) {  // ragged last tile and the elements past the last full vector
         for (int64_t v = full_tiles * kTile + threadIdx.x; v < a.nvec; v += THREADS) {
-            const Pack<IO, VEC> pk = load_pack<IO, VEC>(x + v * VEC);
+            const Pack<IO, VEC> pk = load_pack_stream<IO, VEC>(x + v * VEC);
             for (int k = 0; k < VEC; ++k) add(load_f32(pk.v[k]));
         }
         for (int64_t i = a.nvec * VEC + threadIdx.x; i < a.numel; i += THREADS) add(load_f32(x[i]));
@@ -282,7 +282,7 @@ __global__ __launch_bounds__(kBlock) void dlq_pdf_bin_runs_kernel(const PdfBinAr
         const IO* __restrict__ x = static_cast<const IO*>(a.x) + e * a.K;
         const int64_t nv = a.K / VEC;
         for (int64_t v = threadIdx.x; v < nv; v += kBlock) {
-            const Pack<IO, VEC> pk = load_pack<IO, VEC>(x + v * VEC);
+            const Pack<IO, VEC> pk = load_pack_stream<IO, VEC>(x + v * VEC);
 #pragma unroll
             for (int k = 0; k < VEC; ++k) {
                 int idx;
