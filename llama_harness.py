@@ -1,9 +1,9 @@
 """A random-init bf16 Llama-style decoder and its quantization set-up, used by bench.py and the whole-model tests.
 
 Only the quantize-dequantize and calibration kernels under test are this repository's; the GEMMs, attention, norms and
-rotary embedding below are plain PyTorch-ROCm calls.  The quantization layout is the one of the benchmark
-configuration: 4-bit symmetric blockwise weights (block 64 along the input dimension) and 16-bit asymmetric per-tensor
-quantize-dequantize at the input and output of every nn.Linear.
+rotary embedding below are plain PyTorch-ROCm calls (fused RMS norm, rotary tables formed once per sequence length).
+The quantization layout is the one of the benchmark configuration: 4-bit symmetric blockwise weights (block 64 along
+the input dimension) and 16-bit asymmetric per-tensor quantize-dequantize at the input and output of every nn.Linear.
 """
 
 from __future__ import annotations
@@ -36,20 +36,23 @@ class RMSNorm(nn.Module):
         self.eps = eps
 
     def forward(self, x):
-        v = x.float()
-        v = v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + self.eps)
-        return (v * self.weight.float()).to(x.dtype)
+        return F.rms_norm(x, self.weight.shape, self.weight, self.eps)  # one fused kernel, statistics in float32
 
 
-def rotary(x, theta):
-    # x: [B, H, T, D]
-    B, H, T, D = x.shape
-    half = D // 2
-    freqs = 1.0 / (theta ** (torch.arange(0, half, device=x.device, dtype=torch.float32) / half))
-    ang = torch.arange(T, device=x.device, dtype=torch.float32)[:, None] * freqs[None, :]
-    cos, sin = ang.cos()[None, None], ang.sin()[None, None]
-    x1, x2 = x[..., :half].float(), x[..., half:].float()
-    return torch.cat([x1 * cos - x2 * sin, x1 * sin + x2 * cos], dim=-1).to(x.dtype)
+def rotary_tables(seq: int, head_dim: int, theta: float, device, dtype):
+    """cos / sin of the rotary angles, [1, 1, seq, head_dim] in the model's dtype, the two halves of the last axis
+    alike: a function of the sequence length only, so a model forms them once and every layer uses them."""
+    half = head_dim // 2
+    freqs = 1.0 / (theta ** (torch.arange(0, half, device=device, dtype=torch.float32) / half))
+    ang = torch.arange(seq, device=device, dtype=torch.float32)[:, None] * freqs[None, :]
+    ang = torch.cat([ang, ang], dim=-1)
+    return ang.cos()[None, None].to(dtype), ang.sin()[None, None].to(dtype)
+
+
+def rotary(x, cos, sin):
+    # x: [B, H, T, D]; x * cos + rotate_half(x) * sin
+    half = x.shape[-1] // 2
+    return x * cos + torch.cat([-x[..., half:], x[..., :half]], dim=-1) * sin
 
 
 class Attention(nn.Module):
@@ -62,13 +65,13 @@ class Attention(nn.Module):
         self.v_proj = nn.Linear(h, h, bias=False)
         self.o_proj = nn.Linear(h, h, bias=False)
 
-    def forward(self, x):
+    def forward(self, x, rope):
         B, T, C = x.shape
         H = self.cfg.heads
         q = self.q_proj(x).view(B, T, H, C // H).transpose(1, 2)
         k = self.k_proj(x).view(B, T, H, C // H).transpose(1, 2)
         v = self.v_proj(x).view(B, T, H, C // H).transpose(1, 2)
-        q, k = rotary(q, self.cfg.rope_theta), rotary(k, self.cfg.rope_theta)
+        q, k = rotary(q, *rope), rotary(k, *rope)
         y = F.scaled_dot_product_attention(q, k, v, is_causal=True)
         return self.o_proj(y.transpose(1, 2).reshape(B, T, C))
 
@@ -92,8 +95,8 @@ class Block(nn.Module):
         self.post_norm = RMSNorm(cfg.hidden, cfg.eps)
         self.mlp = MLP(cfg)
 
-    def forward(self, x):
-        x = x + self.attn(self.input_norm(x))
+    def forward(self, x, rope):
+        x = x + self.attn(self.input_norm(x), rope)
         return x + self.mlp(self.post_norm(x))
 
 
@@ -105,11 +108,20 @@ class Llama(nn.Module):
         self.blocks = nn.ModuleList([Block(cfg) for _ in range(cfg.layers)])
         self.norm = RMSNorm(cfg.hidden, cfg.eps)
         self.lm_head = nn.Linear(cfg.hidden, cfg.vocab, bias=False)
+        self._rope = {}
+
+    def rope(self, seq: int, like: torch.Tensor):
+        key = (seq, like.device, like.dtype)
+        if key not in self._rope:
+            self._rope[key] = rotary_tables(seq, self.cfg.hidden // self.cfg.heads, self.cfg.rope_theta,
+                                            like.device, like.dtype)
+        return self._rope[key]
 
     def forward(self, ids):
         x = self.embed(ids)
+        rope = self.rope(ids.shape[1], x)
         for b in self.blocks:
-            x = b(x)
+            x = b(x, rope)
         return self.lm_head(self.norm(x))
 
 
