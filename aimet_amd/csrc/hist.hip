@@ -30,7 +30,6 @@ namespace ahq {
 
 constexpr int kHistBlocksMax = 1536;  // persistent workgroups of the binning pass (6 per CU)
 constexpr int kRng = 8;               // floats per slot in `ranges`
-constexpr int kFoldGroups = 32;       // partial histograms left after the first fold
 
 // ranges[slot]: lo1, hi1, thr_lo1, thr_hi1 (batch's own range), lo2, hi2, thr_lo2, thr_hi2 (updated range).
 // thr_* are the edges rounded to the tensor dtype: the reference compares `x < edge` in the tensor's dtype.
@@ -62,43 +61,61 @@ struct PrepArgs {
 // _create_bin_edges (encoding_analyzer.py:221-229).  `lo`/`hi` already hold the min==max adjustment.
 __device__ __forceinline__ float edge_at(float lo, float step, int i) { return (float)i * step + lo; }
 
+// Fold of the per-workgroup partial extrema of the min/max pass by one workgroup (saves that pass's own finishing
+// launch); min and max are exact and order-independent, and the partials already are values of the tensor's dtype.
+__device__ __forceinline__ void fold_partial_extrema(const PrepArgs& a, float& mn, float& mx) {
+    __shared__ float red_mn[16], red_mx[16];
+    mn = __builtin_inff();
+    mx = -__builtin_inff();
+    for (int64_t q = threadIdx.x; q < a.nparts; q += blockDim.x) {
+        mn = fminf(mn, a.part_min[q]);
+        mx = fmaxf(mx, a.part_max[q]);
+    }
+#pragma unroll
+    for (int m = kWave / 2; m >= 1; m >>= 1) {
+        mn = fminf(mn, __shfl_xor(mn, m, kWave));
+        mx = fmaxf(mx, __shfl_xor(mx, m, kWave));
+    }
+    if ((threadIdx.x & (kWave - 1)) == 0) {
+        red_mn[threadIdx.x / kWave] = mn;
+        red_mx[threadIdx.x / kWave] = mx;
+    }
+    __syncthreads();
+    const int nw = (blockDim.x + kWave - 1) / kWave;
+    mn = red_mn[0];
+    mx = red_mx[0];
+    for (int w = 1; w < nw; ++w) {
+        mn = fminf(mn, red_mn[w]);
+        mx = fmaxf(mx, red_mx[w]);
+    }
+}
+
+// The running range after a batch with extrema (mn, mx) (encoding_analyzer.py:266-270): clamp(min=left, max=edge0) ==
+// min(max(x, left), edge0).  Returns whether it equals the range the state holds.
+struct RunningRange {
+    float first_edge, last_edge, limit_lo, limit_hi, min, max;
+};
+
+__device__ __forceinline__ RunningRange load_running_range(const PrepArgs& a, int s) {
+    const float* ce = a.edges + (size_t)s * (a.num_bins + 1);
+    const float* lim = a.limits + (size_t)s * 2;
+    const float* mmx = a.minmax + (size_t)s * 2;
+    return RunningRange{ce[0], ce[a.num_bins], lim[0], lim[1], mmx[0], mmx[1]};
+}
+
+__device__ __forceinline__ bool updated_range(const RunningRange& r, float mn, float mx, float& umin, float& umax) {
+    umin = fminf(fmaxf(mn, r.limit_lo), r.first_edge);
+    umax = fminf(fmaxf(mx, r.last_edge), r.limit_hi);
+    return (umin == r.min) && (umax == r.max);
+}
+
+// Everything between the extrema of a batch and its binning pass, for slot `s`, by one workgroup.  `keep_minmax`: the
+// new running range goes to `ranges` only and the state's min / max stay as they are (other workgroups of the same
+// launch still compare against them; the launch that finishes the update stores them).
 template <typename IO>
-__global__ void hist_prepare_kernel(const PrepArgs a) {
-    const int s = blockIdx.x;
+__device__ void prepare_slot(const PrepArgs& a, const int s, const float mn, const float mx, const bool keep_minmax) {
     const int B = a.num_bins;
     const float Bf = (float)B;
-    float mn, mx;
-    if (a.nparts > 0) {
-        // fold the partial extrema of the min/max pass (saves that pass's own finishing launch); min and max are
-        // exact and order-independent, and the partials already are values of the tensor's dtype
-        __shared__ float red_mn[16], red_mx[16];
-        mn = __builtin_inff();
-        mx = -__builtin_inff();
-        for (int64_t q = threadIdx.x; q < a.nparts; q += blockDim.x) {
-            mn = fminf(mn, a.part_min[q]);
-            mx = fmaxf(mx, a.part_max[q]);
-        }
-#pragma unroll
-        for (int m = kWave / 2; m >= 1; m >>= 1) {
-            mn = fminf(mn, __shfl_xor(mn, m, kWave));
-            mx = fmaxf(mx, __shfl_xor(mx, m, kWave));
-        }
-        if ((threadIdx.x & (kWave - 1)) == 0) {
-            red_mn[threadIdx.x / kWave] = mn;
-            red_mx[threadIdx.x / kWave] = mx;
-        }
-        __syncthreads();
-        const int nw = (blockDim.x + kWave - 1) / kWave;
-        mn = red_mn[0];
-        mx = red_mx[0];
-        for (int w = 1; w < nw; ++w) {
-            mn = fminf(mn, red_mn[w]);
-            mx = fmaxf(mx, red_mx[w]);
-        }
-    } else {
-        mn = load_f32(static_cast<const IO*>(a.bmin)[s]);
-        mx = load_f32(static_cast<const IO*>(a.bmax)[s]);
-    }
     // the batch's own bin edges; "min - 0.5" happens in the tensor dtype before the cast to float
     const bool eq = mn == mx;
     const float lo1 = eq ? round_io<IO>(mn - 0.5f) : mn;
@@ -142,11 +159,8 @@ __global__ void hist_prepare_kernel(const PrepArgs a) {
     const float* ce = a.edges + (size_t)s * (B + 1);
     const float* ch = a.hist + (size_t)s * B;
     float* carried = a.carried + (size_t)s * B;
-    const float c_first = ce[0], c_last = ce[B];
-    // clamp(min=left, max=edge0) == min(max(x, left), edge0)
-    const float umin = fminf(fmaxf(mn, lim[0]), c_first);
-    const float umax = fminf(fmaxf(mx, c_last), lim[1]);
-    const bool same = (umin == mmx[0]) && (umax == mmx[1]);
+    float umin, umax;
+    const bool same = updated_range(load_running_range(a, s), mn, mx, umin, umax);
     if (a.rebin && threadIdx.x == 0) a.rebin[s] = same ? 0 : 1;
     if (same) {
         for (int i = threadIdx.x; i < B; i += blockDim.x) carried[i] = ch[i];
@@ -200,9 +214,24 @@ __global__ void hist_prepare_kernel(const PrepArgs a) {
         rg[5] = umax;
         rg[6] = round_io<IO>(umin);
         rg[7] = round_io<IO>(umax);
-        mmx[0] = umin;
-        mmx[1] = umax;
+        if (!keep_minmax) {
+            mmx[0] = umin;
+            mmx[1] = umax;
+        }
     }
+}
+
+template <typename IO>
+__global__ void hist_prepare_kernel(const PrepArgs a) {
+    const int s = blockIdx.x;
+    float mn, mx;
+    if (a.nparts > 0) {
+        fold_partial_extrema(a, mn, mx);
+    } else {
+        mn = load_f32(static_cast<const IO*>(a.bmin)[s]);
+        mx = load_f32(static_cast<const IO*>(a.bmax)[s]);
+    }
+    prepare_slot<IO>(a, s, mn, mx, false);
 }
 
 // ------------------------------------------------------------------------------------------------ binning pass --
@@ -593,18 +622,6 @@ __global__ void zero_u32_kernel(uint32_t* p, int64_t n) {
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) p[i] = 0;
 }
 
-// ------------------------------------------------------------------------------------ fold of the partial counts --
-// partial[p][l] (p < nparts, l < len) -> folded[g][l] = sum of the partials p with p % groups == g
-__global__ __launch_bounds__(kBlock) void hist_fold_kernel(const uint32_t* partial, uint32_t* folded, int nparts, int len, int groups) {
-    const int l = blockIdx.x * kBlock + threadIdx.x;
-    const int g = blockIdx.y;
-    if (l >= len) return;
-    uint32_t acc = 0;
-#pragma unroll 4
-    for (int p = g; p < nparts; p += groups) acc += partial[(size_t)p * len + l];
-    folded[(size_t)g * len + l] = acc;
-}
-
 // ----------------------------------------------------------------------------------------------------- finish --
 struct FinArgs {
     int32_t num_slots, num_bins, nhist, first;
@@ -615,6 +632,10 @@ struct FinArgs {
     float* hist;               // [S][B] running (out)
     float* edges;              // [S][B+1] running (out)
     float* new_hist;           // [S][B] (out)
+    // single-slot fold-and-finish only:
+    const int32_t* rebin;      // optional: leave at once when *rebin == 0 (the speculative pass already was the update)
+    const float* ranges;       // optional, with `minmax`: the new running range (ranges[4], ranges[5]) is stored into
+    float* minmax;             //   the state here, by the launch that ends the update
 };
 
 __global__ __launch_bounds__(kBlock) void hist_finish_kernel(const FinArgs a) {
@@ -671,6 +692,151 @@ __global__ __launch_bounds__(kBlock) void hist_finish_kernel(const FinArgs a) {
     }
 }
 
+// --------------------------------------------------------- single slot: fold of the partial counts and finish --
+// One launch instead of a fold and a finish: a workgroup of 1024 threads owns 8 bins, thread = (bin, one of 128 groups
+// of partial histograms); the integer sums over the partials are order-independent, the float operations per bin are
+// those of hist_finish_kernel.  `carried` may be the running histogram itself (every bin is read and written by one
+// thread); upd_edges == NULL leaves the running edges as they are.
+constexpr int kFfBins = 8;
+constexpr int kFfThreads = 1024;
+constexpr int kFfGroups = kFfThreads / kFfBins;
+
+// this thread's share of the sums: bin blockIdx.x * kFfBins + (thread % kFfBins), every kFfGroups-th partial histogram.
+// The loads are independent and the partials come from other dies' caches, so as many as possible are in flight.
+__device__ __forceinline__ void fold_load(const FinArgs& a, unsigned long long (&c)[2]) {
+    const int B = a.num_bins;
+    const int bl = threadIdx.x & (kFfBins - 1), grp = threadIdx.x / kFfBins;
+    const int b = blockIdx.x * kFfBins + bl;
+    const uint32_t* base = a.counts;
+    const size_t row = (size_t)(B + 2);
+    c[0] = c[1] = 0;
+    if (b >= B) return;
+    if (a.nhist == 1) {
+        constexpr int kFlight = 16;  // 16 * 128 = 2048 partials per round: one round for any binning grid
+        for (int p = grp; p < a.nparts; p += kFlight * kFfGroups) {
+            uint32_t v[kFlight];
+#pragma unroll
+            for (int k = 0; k < kFlight; ++k) v[k] = p + k * kFfGroups < a.nparts ? base[(size_t)(p + k * kFfGroups) * row + b] : 0u;
+#pragma unroll
+            for (int k = 0; k < kFlight; ++k) c[0] += v[k];
+        }
+    } else {
+#pragma unroll 4
+        for (int p = grp; p < a.nparts; p += kFfGroups) {
+            c[0] += base[((size_t)p * 2) * row + b];
+            c[1] += base[((size_t)p * 2 + 1) * row + b];
+        }
+    }
+}
+
+__device__ void fold_finish_bins(const FinArgs& a, unsigned long long (&c)[2]) {
+    __shared__ unsigned long long sm[kFfGroups][2][kFfBins];
+    __shared__ unsigned long long wave_edge[kFfThreads / kWave][4];
+    const int B = a.num_bins, NH = a.nhist;
+    const int bl = threadIdx.x & (kFfBins - 1), grp = threadIdx.x / kFfBins;
+    const int b = blockIdx.x * kFfBins + bl;
+    const uint32_t* base = a.counts;
+    const size_t row = (size_t)(B + 2);
+    sm[grp][0][bl] = c[0];
+    sm[grp][1][bl] = c[1];
+    const float carried_b = (grp == 0 && b < B && !a.first) ? a.carried[b] : 0.f;  // fetched ahead of the barriers
+    // below / above totals, wanted by the owners of bin 0 and of bin B - 1: thread = (histogram, side, partials)
+    const bool owns_end = blockIdx.x == 0 || (int)blockIdx.x == (B - 1) / kFfBins;
+    if (owns_end) {
+        const int combo = threadIdx.x & 3, h = combo >> 1, side = combo & 1;
+        unsigned long long t = 0;
+        if (h < NH) {
+            constexpr int kFlight = 8, kStep = kFfThreads / 4;  // 8 * 256 partials per round
+            for (int p = threadIdx.x >> 2; p < a.nparts; p += kFlight * kStep) {
+                uint32_t v[kFlight];
+#pragma unroll
+                for (int k = 0; k < kFlight; ++k)
+                    v[k] = p + k * kStep < a.nparts ? base[((size_t)(p + k * kStep) * NH + h) * row + B + side] : 0u;
+#pragma unroll
+                for (int k = 0; k < kFlight; ++k) t += v[k];
+            }
+        }
+#pragma unroll
+        for (int m = 32; m >= 4; m >>= 1) t += __shfl_xor(t, m, kWave);
+        if ((threadIdx.x & (kWave - 1)) < 4) wave_edge[threadIdx.x / kWave][combo] = t;
+    }
+    __syncthreads();
+    if (grp < 8) {
+        for (int h = 0; h < NH; ++h) {
+            unsigned long long t = 0;
+#pragma unroll
+            for (int k = 0; k < kFfGroups / 8; ++k) t += sm[grp + 8 * k][h][bl];
+            c[h] = t;
+        }
+    }
+    __syncthreads();
+    if (grp < 8) {
+        sm[grp][0][bl] = c[0];
+        sm[grp][1][bl] = c[1];
+    }
+    __syncthreads();
+    if (grp != 0 || b >= B) return;
+    unsigned long long tot[2] = {0, 0};
+    for (int h = 0; h < NH; ++h)
+        for (int k = 0; k < 8; ++k) tot[h] += sm[k][h][bl];
+    unsigned long long edge_cnt[2][2] = {{0, 0}, {0, 0}};
+    if (b == 0 || b == B - 1)
+        for (int w = 0; w < kFfThreads / kWave; ++w)
+            for (int q = 0; q < 4; ++q) edge_cnt[q >> 1][q & 1] += wave_edge[w][q];
+    // the batch's own histogram: counts, then "+= below" on bin 0 and "+= above" on the last bin
+    float nh = (float)tot[0];
+    if (b == 0) nh += (float)edge_cnt[0][0];
+    if (b == B - 1) nh += (float)edge_cnt[0][1];
+    if (a.new_hist) a.new_hist[b] = nh;
+    float uh;
+    if (a.first) {
+        uh = nh;
+    } else {
+        const int h = NH - 1;
+        uh = (float)tot[h] + carried_b;
+        if (b == 0) uh += (float)edge_cnt[h][0];
+        if (b == B - 1) uh += (float)edge_cnt[h][1];
+    }
+    a.hist[b] = uh;
+    if (a.upd_edges) {
+        a.edges[b] = a.upd_edges[b];
+        if (b == B - 1) a.edges[B] = a.upd_edges[B];
+    }
+}
+
+__global__ __launch_bounds__(kFfThreads) void hist_fold_finish_kernel(const FinArgs a) {
+    if (a.rebin && *a.rebin == 0) return;
+    if (a.minmax && blockIdx.x == 0 && threadIdx.x == 0) {
+        a.minmax[0] = a.ranges[4];
+        a.minmax[1] = a.ranges[5];
+    }
+    unsigned long long c[2];
+    fold_load(a, c);
+    fold_finish_bins(a, c);
+}
+
+// After a speculative binning pass (hist_bin_kernel<SPEC>), single slot.  Every workgroup folds the pass's partial
+// extrema and decides, from the same unchanged state, whether the running range holds.  If it does, the pass's counts
+// are the batch's contribution: the workgroups fold them into the running histogram (16 bins each) and the update is
+// complete -- the launches that follow see *rebin == 0 and leave at once.  If it does not, workgroup 0 prepares the
+// second pass (new range and edges, running counts carried over to the new bins), the others leave; the state's min /
+// max are left alone in this launch because the other workgroups compare against them.
+template <typename IO>
+__global__ __launch_bounds__(kFfThreads) void hist_resolve_kernel(const PrepArgs pa, const FinArgs fa) {
+    float mn, mx, umin, umax;
+    unsigned long long c[2];
+    const RunningRange running = load_running_range(pa, 0);
+    fold_load(fa, c);  // ahead of the decision: reading the counts is harmless, and the latencies overlap
+    fold_partial_extrema(pa, mn, mx);
+    const bool same = updated_range(running, mn, mx, umin, umax);
+    if (same) {
+        if (blockIdx.x == 0 && threadIdx.x == 0) pa.rebin[0] = 0;
+        fold_finish_bins(fa, c);
+    } else if (blockIdx.x == 0) {
+        prepare_slot<IO>(pa, 0, mn, mx, true);
+    }
+}
+
 }  // namespace ahq
 
 using namespace ahq;
@@ -685,7 +851,7 @@ struct HistPlan {
     int copies;
     int nblocks;
     int64_t ntiles;
-    size_t off_mm_ws, off_bmin, off_bmax, off_ranges, off_carried, off_upd_edges, off_scratch, off_rebin, off_counts, off_folded, total;
+    size_t off_mm_ws, off_bmin, off_bmax, off_ranges, off_carried, off_upd_edges, off_scratch, off_rebin, off_counts, total;
 };
 
 size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
@@ -742,8 +908,6 @@ bool make_hist_plan(int dtype, const ahq_layout& layout, const void* x, int num_
     hp->off_counts = o;
     const size_t nparts = hp->fast ? (size_t)hp->nblocks : 1;
     o = align_up(o + (size_t)S * nparts * 2 * (B + 2) * 4);
-    hp->off_folded = o;
-    o = align_up(o + (size_t)kFoldGroups * 2 * (B + 2) * 4);
     hp->total = o;
     return true;
 }
@@ -853,11 +1017,30 @@ extern "C" int ahq_hist_update(int32_t dtype, const ahq_layout* layout, const vo
     pa.ranges = reinterpret_cast<float*>(w + hp.off_ranges);
     pa.scratch = reinterpret_cast<int32_t*>(w + hp.off_scratch);
     pa.rebin = speculative ? rebin : nullptr;
-    const int pthreads = nparts > 0 ? 1024 : (B >= 512 ? 512 : (B >= 64 ? ((B + 63) / 64) * 64 : 64));
-    switch (dtype) {
-        case AHQ_F32: hipLaunchKernelGGL((hist_prepare_kernel<float>), dim3(S), dim3(pthreads), 0, s, pa); break;
-        case AHQ_F16: hipLaunchKernelGGL((hist_prepare_kernel<f16_t>), dim3(S), dim3(pthreads), 0, s, pa); break;
-        default: hipLaunchKernelGGL((hist_prepare_kernel<bf16_t>), dim3(S), dim3(pthreads), 0, s, pa); break;
+    FinArgs fa{};
+    fa.num_slots = S;
+    fa.num_bins = B;
+    const dim3 ffgrid((B + kFfBins - 1) / kFfBins);
+    if (speculative) {
+        // the counts of the speculative pass, folded straight into the running histogram if the range holds
+        fa.nhist = 1;
+        fa.first = 0;
+        fa.nparts = hp.nblocks;
+        fa.counts = counts;
+        fa.carried = st->hist;
+        fa.hist = st->hist;
+        switch (dtype) {
+            case AHQ_F32: hipLaunchKernelGGL((hist_resolve_kernel<float>), ffgrid, dim3(kFfThreads), 0, s, pa, fa); break;
+            case AHQ_F16: hipLaunchKernelGGL((hist_resolve_kernel<f16_t>), ffgrid, dim3(kFfThreads), 0, s, pa, fa); break;
+            default: hipLaunchKernelGGL((hist_resolve_kernel<bf16_t>), ffgrid, dim3(kFfThreads), 0, s, pa, fa); break;
+        }
+    } else {
+        const int pthreads = nparts > 0 ? 1024 : (B >= 512 ? 512 : (B >= 64 ? ((B + 63) / 64) * 64 : 64));
+        switch (dtype) {
+            case AHQ_F32: hipLaunchKernelGGL((hist_prepare_kernel<float>), dim3(S), dim3(pthreads), 0, s, pa); break;
+            case AHQ_F16: hipLaunchKernelGGL((hist_prepare_kernel<f16_t>), dim3(S), dim3(pthreads), 0, s, pa); break;
+            default: hipLaunchKernelGGL((hist_prepare_kernel<bf16_t>), dim3(S), dim3(pthreads), 0, s, pa); break;
+        }
     }
 
     // 3. binning pass (after a speculative pass: only if the range changed)
@@ -916,9 +1099,6 @@ extern "C" int ahq_hist_update(int32_t dtype, const ahq_layout* layout, const vo
     }
 
     // 4. counts -> fp32 statistics
-    FinArgs fa{};
-    fa.num_slots = S;
-    fa.num_bins = B;
     fa.nhist = NH;
     fa.first = first_batch ? 1 : 0;
     fa.nparts = hp.fast ? hp.nblocks : 1;
@@ -928,19 +1108,15 @@ extern "C" int ahq_hist_update(int32_t dtype, const ahq_layout* layout, const vo
     fa.hist = st->hist;
     fa.edges = st->edges;
     fa.new_hist = st->new_hist;
-    if (hp.fast && hp.nblocks > kFoldGroups) {
-        uint32_t* folded = reinterpret_cast<uint32_t*>(w + hp.off_folded);
-        const int len = NH * (B + 2);
-        hipLaunchKernelGGL(hist_fold_kernel, dim3((len + kBlock - 1) / kBlock, kFoldGroups), dim3(kBlock), 0, s, counts,
-                           folded, hp.nblocks, len, kFoldGroups);
-        fa.nparts = kFoldGroups;
-        fa.counts = folded;
+    if (hp.fast) {
+        if (speculative) {  // only if the range moved; ends the update by storing the new range into the state
+            fa.rebin = rebin;
+            fa.ranges = pa.ranges;
+            fa.minmax = st->minmax;
+        }
+        hipLaunchKernelGGL(hist_fold_finish_kernel, ffgrid, dim3(kFfThreads), 0, s, fa);
+    } else {
+        hipLaunchKernelGGL(hist_finish_kernel, dim3((B + 63) / 64, S < 65535 ? S : 65535), dim3(kBlock), 0, s, fa);
     }
-    fa.carried = pa.carried;
-    fa.upd_edges = pa.upd_edges;
-    fa.hist = st->hist;
-    fa.edges = st->edges;
-    fa.new_hist = st->new_hist;
-    hipLaunchKernelGGL(hist_finish_kernel, dim3((B + 63) / 64, S < 65535 ? S : 65535), dim3(kBlock), 0, s, fa);
     return check_launch("ahq_hist_update");
 }
