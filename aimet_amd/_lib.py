@@ -129,6 +129,8 @@ _SIGNATURES = {
                                                  ctypes.c_double, _P, _P, _P]),
     "ahq_lpbq_scale": (ctypes.c_int, [ctypes.c_int32, ctypes.POINTER(Layout), _P, _P, ctypes.c_int64, ctypes.c_int64,
                                       ctypes.c_double, ctypes.c_int32, _P, _P, _P]),
+    "ahq_lpbq_qdq_forward": (ctypes.c_int, [ctypes.POINTER(Grid), ctypes.POINTER(Layout), _P, _P, _P, ctypes.c_int32, _P,
+                                            _P, ctypes.c_int64, ctypes.c_double, ctypes.c_int32, _P, _P, _P, _P]),
     "ahq_grid_probe": (ctypes.c_int, [ctypes.c_int32, ctypes.POINTER(Layout), _P, ctypes.c_int64, _P, _P]),
     "ahq_hist_update_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int32, ctypes.POINTER(Layout), ctypes.c_int32]),
     "ahq_hist_update": (ctypes.c_int, [ctypes.c_int32, ctypes.POINTER(Layout), _P, ctypes.POINTER(HistState),

@@ -403,6 +403,119 @@ __device__ __forceinline__ void stage_encodings(const QdqArgs& a, const Tile& t,
     }
 }
 
+// LPBQ forward with the grouped block scales derived by the kernel itself (GroupedBlockQuantizeDequantize._get_scale,
+// aimet_torch/quantization/affine/quantizer.py:1363-1399, which the reference runs before every forward): a tile's
+// workgroup evaluates, for the groups its blocks belong to, the largest raw block scale (a group is a run of
+// neighbouring blocks, a few hundred bytes of min / max), then snaps the raw scales of its own blocks to integer
+// multiples of the group's per-channel scale, writes them out for the backward pass and stages them.  The float
+// operations are those of lpbq_scale_kernel, in the same order.
+struct LpbqFuse {
+    const void* pmin;        // per block, `dtype`
+    const void* pmax;
+    float* scale_out;        // per block
+    float* per_channel_out;  // per group, optional
+    int64_t group;           // neighbouring blocks per group
+    int32_t dtype;
+    float num_steps, minimum_scale, multipliers;
+};
+
+__device__ __forceinline__ void lpbq_load_range(const LpbqFuse& f, int64_t i, float& mn, float& mx) {
+    if (f.dtype == AHQ_F32) {
+        mn = static_cast<const float*>(f.pmin)[i];
+        mx = static_cast<const float*>(f.pmax)[i];
+    } else if (f.dtype == AHQ_F16) {
+        mn = load_f32(static_cast<const f16_t*>(f.pmin)[i]);
+        mx = load_f32(static_cast<const f16_t*>(f.pmax)[i]);
+    } else {
+        mn = load_f32(static_cast<const bf16_t*>(f.pmin)[i]);
+        mx = load_f32(static_cast<const bf16_t*>(f.pmax)[i]);
+    }
+}
+
+__device__ __forceinline__ float lpbq_raw_from(const LpbqFuse& f, float mn, float mx) {
+    const float s = __builtin_fabsf((mx - mn) / f.num_steps);
+    return (s != s) ? s : fmaxf(s, f.minimum_scale);
+}
+
+__device__ __forceinline__ float lpbq_raw_scale(const LpbqFuse& f, int64_t i) {
+    float mn, mx;
+    lpbq_load_range(f, i, mn, mx);
+    return lpbq_raw_from(f, mn, mx);
+}
+
+// min / max of the block this thread stages first, requested ahead of the tile's elements: loads return in the order
+// they were issued, so the scale derivation can then run while the elements are still in flight
+__device__ __forceinline__ void lpbq_preload(const LpbqFuse& f, const Tile& t, float& mn, float& mx) {
+    mn = mx = 0.f;
+    if ((int)threadIdx.x < t.nstage) lpbq_load_range(f, t.e0 + threadIdx.x, mn, mx);
+}
+
+template <typename M>
+__device__ __forceinline__ void stage_lpbq(const QdqArgs& a, const LpbqFuse& f, const Tile& t, float (*sp)[kStage],
+                                           const float pre_mn, const float pre_mx) {
+    __shared__ float per_channel[kStage];  // of the groups this tile touches
+    const int64_t G = f.group;
+    const int64_t g0 = t.e0 / G;
+    const int ng = t.nstage > 0 ? (int)((t.e0 + t.nstage - 1) / G - g0) + 1 : 0;
+    const int lane = threadIdx.x & (kWave - 1);
+    auto stage_one = [&](int i, int64_t e, int64_t g, float raw, float pc) {
+        const float r = __builtin_rintf(raw / pc);
+        const float q = (r != r) ? r : fminf(fmaxf(r, 1.0f), f.multipliers);
+        const float s = q * pc;
+        f.scale_out[e] = s;  // a block lies in one tile, or in two neighbouring ones that store the same value
+        if (f.per_channel_out && e == g * G) f.per_channel_out[g] = pc;
+        const EncP p = M::prep(s, a.offset ? a.offset[e] : 0.f, 0.f, 0.f, a.gc);
+        sp[0][i] = p.p0;
+        sp[1][i] = p.p1;
+        if (M::kNP > 2) sp[2][i] = p.p2;
+        if (M::kNP > 3) sp[3][i] = p.p3;
+        if (M::kDiv) sp[M::kNP][i] = p.rs;
+    };
+    if (G <= kWave && (G & (G - 1)) == 0 && t.e0 % G == 0 && t.nstage % G == 0) {
+        // whole groups, each inside a power-of-two run of lanes: one read of min / max per block, the group's largest
+        // raw scale by shuffles (a maximum does not depend on the order), no second barrier
+        const int padded = (t.nstage + kWave - 1) & ~(kWave - 1);
+        for (int i = threadIdx.x; i < padded; i += kBlock) {
+            const bool live = i < t.nstage;
+            const int64_t e = t.e0 + i;
+            const float raw = !live ? -__builtin_inff()
+                              : i == (int)threadIdx.x ? lpbq_raw_from(f, pre_mn, pre_mx) : lpbq_raw_scale(f, e);
+            float largest = raw;
+            int nan = (raw != raw) ? 1 : 0;
+            for (int m = 1; m < (int)G; m <<= 1) {
+                largest = fmaxf(largest, __shfl_xor(largest, m, kWave));
+                nan |= __shfl_xor(nan, m, kWave);
+            }
+            if (nan) largest = __builtin_nanf("");  // torch.amax propagates NaN
+            if (live) stage_one(i, e, e / G, raw, largest / f.multipliers);
+        }
+        return;
+    }
+    for (int gi = threadIdx.x / kWave; gi < ng; gi += kBlock / kWave) {
+        const int64_t base = (g0 + gi) * G;
+        float largest = -__builtin_inff();
+        int nan = 0;
+        for (int64_t k = lane; k < G; k += kWave) {
+            const float s = lpbq_raw_scale(f, base + k);
+            nan |= (s != s) ? 1 : 0;
+            largest = fmaxf(largest, s);
+        }
+#pragma unroll
+        for (int m = kWave / 2; m >= 1; m >>= 1) {
+            largest = fmaxf(largest, __shfl_xor(largest, m, kWave));
+            nan |= __shfl_xor(nan, m, kWave);
+        }
+        if (nan) largest = __builtin_nanf("");  // torch.amax propagates NaN
+        if (lane == 0) per_channel[gi] = largest / f.multipliers;
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < t.nstage; i += kBlock) {
+        const int64_t e = t.e0 + i;
+        const int64_t g = e / G;
+        stage_one(i, e, g, lpbq_raw_scale(f, e), per_channel[g - g0]);
+    }
+}
+
 template <typename M>
 __device__ __forceinline__ EncP staged(float (*sp)[kStage], int i) {
     EncP e;
@@ -470,18 +583,22 @@ __device__ __forceinline__ void fwd_math(const QdqArgs& a, const Tile& t, float 
 // FULL: every lane of the tile has work, so loads and stores carry no per-lane bounds checks (all tiles but the last).
 // The tile's elements are requested first; the encodings are fetched, prepared and staged while those loads are in
 // flight, and the workgroup meets at the barrier once before the arithmetic.
-template <typename IO, int VEC, typename M, bool FULL, int U>
-__device__ __forceinline__ void fwd_tile(const QdqArgs& a, const Tile& t, float (*sp)[kStage]) {
+template <typename IO, int VEC, typename M, bool FULL, int U, bool LPBQ = false>
+__device__ __forceinline__ void fwd_tile(const QdqArgs& a, const Tile& t, float (*sp)[kStage],
+                                         const LpbqFuse* lpbq = nullptr) {
     const IO* __restrict__ x = static_cast<const IO*>(a.x) + t.v0 * VEC;
     IO* __restrict__ y = static_cast<IO*>(a.y) + t.v0 * VEC;
     uint8_t* __restrict__ mask = a.mask ? a.mask + t.v0 * VEC : nullptr;
     Pack<IO, VEC> in[U];
+    float pre_mn = 0.f, pre_mx = 0.f;
+    if constexpr (LPBQ) lpbq_preload(*lpbq, t, pre_mn, pre_mx);
 #pragma unroll
     for (int u = 0; u < U; ++u) {
         const int lv = u * kBlock + threadIdx.x;
         if (FULL || lv < t.nv) in[u] = load_pack<IO, VEC>(x + (int64_t)lv * VEC);
     }
-    stage_encodings<M>(a, t, sp);
+    if constexpr (LPBQ) stage_lpbq<M>(a, *lpbq, t, sp, pre_mn, pre_mx);
+    else stage_encodings<M>(a, t, sp);
     __syncthreads();
     // one wave-uniform choice per tile: huge or infinite inputs and out-of-range scales take the general division
     if (!M::kDiv || __builtin_amdgcn_ballot_w64(!lane_can_divide_fast<IO, VEC, M, FULL, U>(a, t, sp, in)) == 0)
@@ -509,6 +626,16 @@ __global__ __launch_bounds__(kBlock) void qdq_fwd_kernel(const QdqArgs a) {
             if (a.mask) a.mask[i] = inr ? 1 : 0;
         }
     }
+}
+
+// The tiled forward kernel with the LPBQ block scales derived in place of read (no elements past the last full vector:
+// the host side sends such tensors to the two-launch form).
+template <typename IO, int VEC, typename M>
+__global__ __launch_bounds__(kBlock) void qdq_fwd_lpbq_kernel(const QdqArgs a, const LpbqFuse f) {
+    __shared__ float sp[M::kNP + (M::kDiv ? 1 : 0)][kStage];
+    const Tile t = make_tile(a, blockIdx.x);
+    if (t.nv == kBlock * kFwdUnroll) fwd_tile<IO, VEC, M, true, kFwdUnroll, true>(a, t, sp, &f);
+    else fwd_tile<IO, VEC, M, false, kFwdUnroll, true>(a, t, sp, &f);
 }
 
 // Encodings that change with every element (run length 1: per-channel along the fastest axis).  The tiled kernel
@@ -1193,6 +1320,58 @@ extern "C" int ahq_qdq_forward(const ahq_grid* grid, const ahq_layout* layout, c
     hipStream_t st = static_cast<hipStream_t>(stream);
     AHQ_IO_SWITCH(grid->io_dtype, AHQ_MATH_SWITCH(*grid, (launch_fwd<IO, M>(p, a, st, al))));
     return check_launch("ahq_qdq_forward");
+}
+
+template <typename IO, typename M>
+static void launch_fwd_lpbq(const Plan& p, const QdqArgs& a, const LpbqFuse& f, hipStream_t st) {
+    if (p.vec == 1) hipLaunchKernelGGL((qdq_fwd_lpbq_kernel<IO, 1, M>), dim3(p.nblocks), dim3(kBlock), 0, st, a, f);
+    else hipLaunchKernelGGL((qdq_fwd_lpbq_kernel<IO, IoTraits<IO>::kVec, M>), dim3(p.nblocks), dim3(kBlock), 0, st, a, f);
+}
+
+extern "C" int ahq_lpbq_qdq_forward(const ahq_grid* grid, const ahq_layout* layout, const void* x, void* y,
+                                    uint8_t* mask_out, int32_t range_dtype, const void* range_min,
+                                    const void* range_max, int64_t blocks_per_group, double minimum_scale,
+                                    int32_t num_multipliers, const float* offset, float* scale,
+                                    float* per_channel_scale, void* stream) {
+    if (!validate_grid(grid, false)) return AHQ_ERR_INVALID;
+    if (!layout || !range_min || !range_max || !scale) return set_error("null argument"), AHQ_ERR_INVALID;
+    if (range_dtype < AHQ_F32 || range_dtype > AHQ_BF16) return set_error("bad range dtype"), AHQ_ERR_INVALID;
+    if (blocks_per_group < 1) return set_error("blocks_per_group must be positive"), AHQ_ERR_INVALID;
+    if (grid->qmin >= grid->qmax) return set_error("qmax must be larger than qmin"), AHQ_ERR_INVALID;
+    if (num_multipliers < 1 || num_multipliers > (1 << 24)) return set_error("num_multipliers must be in 1..2^24"), AHQ_ERR_INVALID;
+    if (grid->arith != AHQ_ARITH_AUTOGRAD || grid->op != AHQ_OP_QDQ || grid->zero_point_shift != 0.0 ||
+        grid->compute_dtype != grid->io_dtype)
+        return set_error("the fused LPBQ forward covers the autograd quantize-dequantize arithmetic computed in the tensor's dtype"), AHQ_ERR_UNSUPPORTED;
+    Plan p;
+    const bool al = aligned16(x) && aligned16(y) && (!mask_out || (reinterpret_cast<uintptr_t>(mask_out) & 7u) == 0);
+    if (!make_plan(grid->io_dtype, *layout, al, false, &p, kFwdUnroll)) return AHQ_ERR_INVALID;
+    if (p.cl.numel == 0) return AHQ_OK;
+    if (!x || !y) return set_error("x or y is null"), AHQ_ERR_INVALID;
+    if (p.cl.kind != kIJK || p.cl.I != 1 || p.cl.J % blocks_per_group != 0 || p.nvec * p.vec != p.cl.numel)
+        return set_error("the fused LPBQ forward needs blocks that follow each other in memory, in whole groups"), AHQ_ERR_UNSUPPORTED;
+    QdqArgs a{};
+    a.x = x;
+    a.y = y;
+    a.mask = mask_out;
+    a.offset = offset;
+    fill_args(*grid, p, &a);
+    LpbqFuse f{};
+    f.pmin = range_min;
+    f.pmax = range_max;
+    f.scale_out = scale;
+    f.per_channel_out = per_channel_scale;
+    f.group = blocks_per_group;
+    f.dtype = range_dtype;
+    f.num_steps = (float)(double)(grid->qmax - grid->qmin);
+    f.minimum_scale = (float)minimum_scale;
+    f.multipliers = (float)num_multipliers;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    switch (grid->io_dtype) {
+        case AHQ_F32: launch_fwd_lpbq<float, MathAutogradQdq<AHQ_F32, false>>(p, a, f, st); break;
+        case AHQ_F16: launch_fwd_lpbq<f16_t, MathAutogradQdq<AHQ_F16, false>>(p, a, f, st); break;
+        default: launch_fwd_lpbq<bf16_t, MathAutogradQdq<AHQ_BF16, false>>(p, a, f, st); break;
+    }
+    return check_launch("ahq_lpbq_qdq_forward");
 }
 
 extern "C" int ahq_dlq_fp8_qdq(int32_t dtype, const ahq_layout* layout, const void* x, void* y, const float* scale,

@@ -370,10 +370,24 @@ def run_qdq_workload(key, steps, warmup, dev, with_cpu_baseline=True):
             _lib.check(lib.ahq_lpbq_scale(_lib.DTYPE_CODE[pmin.dtype], glayout, pmin.data_ptr(), pmax.data_ptr(), qmin,
                                           qmax, min_scale, mult, scale.data_ptr(), pcs.data_ptr(), stream), "lpbq")
 
+    # LPBQ: the scale derivation inside the forward launch (ahq_lpbq_qdq_forward); the separate launches are timed too
+    fused = None
+    if derive is not None:
+        blocks_per_group = q._blocks_per_group()
+        if blocks_per_group is not None:
+            def fused():
+                _lib.check(lib.ahq_lpbq_qdq_forward(grid, layout, x.data_ptr(), y.data_ptr(), None,
+                                                    _lib.DTYPE_CODE[pmin.dtype], pmin.data_ptr(), pmax.data_ptr(),
+                                                    blocks_per_group, min_scale, mult, None, scale.data_ptr(),
+                                                    pcs.data_ptr(), stream), "lpbq forward")
+
     def step():
-        if derive is not None:
-            derive()
-        fwd()
+        if fused is not None:
+            fused()
+        else:
+            if derive is not None:
+                derive()
+            fwd()
         bwd()
 
     loop_s, repeats = timed_steps(step, steps, warmup)
@@ -383,6 +397,7 @@ def run_qdq_workload(key, steps, warmup, dev, with_cpu_baseline=True):
     t_fwd = event_time(fwd, reps)
     t_bwd = event_time(bwd, reps)
     t_derive = event_time(derive, reps) if derive is not None else 0.0
+    t_fused = event_time(fused, reps) if fused is not None else 0.0
 
     n = x.numel()
     S = x.element_size()
@@ -390,7 +405,9 @@ def run_qdq_workload(key, steps, warmup, dev, with_cpu_baseline=True):
     bytes_fwd = 2 * S * n + 8 * E
     bytes_bwd = 3 * S * n + 16 * E
     bytes_derive = (12 * E + 4 * pcs.numel()) if derive is not None else 0
-    bytes_step = bytes_fwd + bytes_bwd + bytes_derive
+    # fused: x, y, min / max of every block read, scale and per-channel scale written (the offset is the constant 0)
+    bytes_fused = (2 * S * n + 2 * pmin.element_size() * E + 4 * E + 4 * pcs.numel()) if fused is not None else 0
+    bytes_step = (bytes_fused + bytes_bwd) if fused is not None else (bytes_fwd + bytes_bwd + bytes_derive)
     value = bytes_step / sec_per_step / 1e9
 
     # ---- frozen quantizer (no gradient for scale / offset): the ATen fake-quantize arithmetic, input gradient only
@@ -487,12 +504,21 @@ def run_qdq_workload(key, steps, warmup, dev, with_cpu_baseline=True):
               "module_gx_bit_exact": mod_gx_exact, "sample": "full size"}
     if w["lpbq"]:
         parity["per_channel_scale_bit_exact"] = bool(torch.equal(pcs.cpu(), pcs_c.view(pcs.shape)))
+    if fused is not None:
+        y.zero_()
+        scale.zero_()
+        pcs.zero_()
+        fused()
+        parity["fused_forward_bit_exact"] = bool(torch.equal(y.cpu(), tr.y) and torch.equal(scale.cpu(), scale_c.view(scale.shape))
+                                                 and torch.equal(pcs.cpu(), pcs_c.view(pcs.shape)))
 
     dom = ("qdq_bwd_kernel", t_bwd, bytes_bwd) if t_bwd >= t_fwd else ("qdq_fwd_kernel", t_fwd, bytes_fwd)
     config = {"workload": w["name"], "elements": n, "encodings": E, "algorithmic_bytes_per_step": bytes_step,
               "arithmetic": "autograd (learnable min/max)", "compute_dtype": str(cd).split(".")[-1],
-              "step": ("ahq_lpbq_scale + " if derive is not None else "") + "ahq_qdq_forward + ahq_qdq_backward (C ABI, "
-                      "preallocated outputs)"}
+              "step": ("ahq_lpbq_qdq_forward (block scales derived inside the forward launch) + ahq_qdq_backward"
+                       if fused is not None else
+                       ("ahq_lpbq_scale + " if derive is not None else "") + "ahq_qdq_forward + ahq_qdq_backward")
+                      + " (C ABI, preallocated outputs)"}
     out = _base_record(value, steps, warmup, sec_per_step, DTYPE_NAME[x.dtype], config, repeats)
     kernels = {
         "qdq_fwd_kernel": {"us": round(t_fwd * 1e6, 2), "GBps": round(bytes_fwd / t_fwd / 1e9, 1),
@@ -502,6 +528,11 @@ def run_qdq_workload(key, steps, warmup, dev, with_cpu_baseline=True):
     }
     if derive is not None:
         kernels["lpbq_scale_kernel"] = {"us": round(t_derive * 1e6, 2), "GBps": round(bytes_derive / t_derive / 1e9, 1)}
+    if fused is not None:
+        kernels["qdq_fwd_lpbq_kernel"] = {"us": round(t_fused * 1e6, 2), "GBps": round(bytes_fused / t_fused / 1e9, 1),
+                                          "frac_of_hbm_peak": round(bytes_fused / t_fused / 1e9 / HBM_PEAK_GBS, 4)}
+        kernels["qdq_fwd_kernel"]["note"] = kernels["lpbq_scale_kernel"]["note"] = \
+            "the two-launch form of the forward pass, not part of the timed step"
     out.update({
         "elements_per_s": round(n / sec_per_step, 1),
         "kernels": kernels,

@@ -252,6 +252,23 @@ int ahq_lpbq_scale(int32_t dtype, const ahq_layout* grouping, const void* range_
                    int64_t qmin, int64_t qmax, double minimum_scale, int32_t num_multipliers, float* scale,
                    float* per_channel_scale, void* stream);
 
+/* ahq_lpbq_scale and ahq_qdq_forward in one launch: the forward pass of GroupedBlockQuantizeDequantize
+ * (AT/quantization/affine/quantizer.py:1363-1399 for the scale, which the reference derives before every forward, then
+ * AT/quantization/affine/backends/torch_builtins.py:705-725).  Every workgroup derives the grouped scales of the blocks
+ * its tile touches from range_min / range_max (one value of `range_dtype` per block, in the order of the encodings of
+ * `layout`), stores them into `scale` (float32 per block, bit for bit what ahq_lpbq_scale stores; the backward pass
+ * reads them) and `per_channel_scale` (float32 per group, may be NULL), and quantize-dequantizes x with them.  A group
+ * is blocks_per_group encodings that follow each other in that order.  offset: float32 per block or NULL (zero).
+ * minimum_scale / num_multipliers as for ahq_lpbq_scale.
+ * AHQ_ERR_UNSUPPORTED (the caller then makes the two calls): another arithmetic than the autograd quantize-dequantize
+ * computed in the tensor's dtype without zero-point shift, blocks that do not follow each other in memory (encodings
+ * that repeat over a leading dimension, strided layouts), a number of blocks that is no multiple of blocks_per_group.
+ */
+int ahq_lpbq_qdq_forward(const ahq_grid* grid, const ahq_layout* layout, const void* x, void* y, uint8_t* mask_out,
+                         int32_t range_dtype, const void* range_min, const void* range_max, int64_t blocks_per_group,
+                         double minimum_scale, int32_t num_multipliers, const float* offset, float* scale,
+                         float* per_channel_scale, void* stream);
+
 /* Replaces the early exit of _decompose_prequantized_tensor (AT/utils.py:2098-2118), the test every weight goes
  * through when a calibration starts: of the first 64 blocks of the layout, the first 2 * num_levels elements each are
  * taken as float magnitudes; *verdict = 0 if one of those samples holds more than num_levels distinct values (the

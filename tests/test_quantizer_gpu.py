@@ -656,3 +656,99 @@ def test_lpbq_learned_range_gradients_in_one_launch(device, case, param_dtype):
     assert not type(scale2.grad_fn).__name__.startswith("_LpbqScale")
     (scale2 * up.to(device)).sum().backward()
     assert_close_rel(q.max.grad, mx_c.grad, tol, "gradient of max, step by step", abs_floor=1e-30)
+
+
+LPBQ_FORWARD_CASES = [
+    # (quantizer shape, block size, block grouping, weight shape)
+    ((96, 8), (1, 64), (1, -1), (96, 512)),       # a group is a row of blocks
+    ((6, 24), (1, 64), (1, -1), (6, 1536)),       # tiles end inside a group
+    ((16, 32), (1, 16), (1, 4), (16, 512)),       # four neighbouring blocks to a group
+    ((5, 3), (1, 2), (1, -1), (5, 6)),            # blocks shorter than a vector
+    ((8, 6), (4, 4), (2, 3), (32, 24)),           # blocks along two dimensions: two launches
+    ((64, 10), (8, 1), (64, 1), (512, 10)),       # groups down a column: two launches
+]
+
+
+@pytest.mark.parametrize("case", LPBQ_FORWARD_CASES, ids=["rows", "split_groups", "fours", "short_blocks",
+                                                            "two_dimensional", "column_groups"])
+@pytest.mark.parametrize("dtype,param_dtype", [(torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16),
+                                               (torch.float16, torch.float32), (torch.bfloat16, torch.float32)],
+                         ids=["f32", "bf16", "f16_f32params", "bf16_f32params"])
+def test_lpbq_forward_in_one_launch(device, case, dtype, param_dtype):
+    """Without gradients the LPBQ forward pass is one launch (ahq_lpbq_qdq_forward: block scales from min / max,
+    snapped to the group's multiples, quantize-dequantize).  Output, block scales and per-channel scales must be the
+    oracle's bits, and equal to what the two-launch form (get_encodings(), then quantize_dequantize) gives."""
+    from aimet_amd.quantization.affine import GroupedBlockQuantizeDequantize
+    from aimet_amd.quantization.affine import quantize_dequantize
+
+    shape, block, grouping, wshape = case
+    g = torch.Generator().manual_seed(33)
+    w = torch.randn(wshape, generator=g) * 0.05
+    w.view(-1)[: w.numel() // 7] *= 30
+    q = GroupedBlockQuantizeDequantize(shape=shape, bitwidth=4, symmetric=True, decompressed_bw=8, block_size=block,
+                                       block_grouping=grouping).to(device)
+    with q.compute_encodings():
+        q(w.to(device))
+    q.to(param_dtype)
+    x = (torch.randn(wshape, generator=g) * 0.08).to(dtype)
+    x.view(-1)[-1] = 1e30
+    x.view(-1)[0] = float("nan")
+    mn, mx = q.min.detach().cpu(), q.max.detach().cpu()
+    raw = O.scale_from_minmax(mn.float(), mx.float(), -8, 7)
+    scale_ref, pcs_ref = O.lpbq_scale(raw, 4, 8, grouping)
+    y_ref = O.qdq_v2_forward(x, scale_ref, torch.zeros_like(scale_ref), -8, 7, block_size=block).y
+    with torch.no_grad():
+        out = q(x.to(device))
+        enc = q.get_encodings()
+        two = quantize_dequantize(x.to(device), enc.scale, enc.offset, -8, 7, block_size=block)
+    assert type(out).__name__ == "DequantizedTensor" and out.dtype == dtype
+    assert_same_bits(out.encoding.scale, scale_ref, "block scales written by the forward launch")
+    assert_same_bits(out.encoding.per_channel_scale, pcs_ref, "per-channel scales written by the forward launch")
+    assert_same_bits(out.as_subclass(torch.Tensor), y_ref, "output against the oracle")
+    assert_same_bits(out.as_subclass(torch.Tensor), two.as_subclass(torch.Tensor), "output against the two-launch form")
+    fused = q.__dict__.get("_lpbq_forward_unsupported") is None and q._blocks_per_group() is not None
+    assert fused == (case[0] not in ((8, 6), (64, 10)))
+    codes = out.quantize()
+    assert float(codes.as_subclass(torch.Tensor)[~x.isnan().to(device)].abs().max()) <= 8
+
+
+def test_lpbq_forward_misaligned_and_refused_layouts(device):
+    """ahq_lpbq_qdq_forward on a tensor that is not 16-byte aligned (scalar loads), and its refusals: encodings that
+    repeat over a leading dimension, a block count that is no multiple of the group, arithmetic in float32 on a
+    16-bit tensor."""
+    from aimet_amd import _lib
+    from aimet_amd.quantization.affine.backends import hip
+    from aimet_amd.quantization._utils import _get_minimum_scale
+
+    lib = _lib.load()
+    g = torch.Generator().manual_seed(5)
+    base = (torch.randn(16 * 256 + 1, generator=g) * 0.1).to(device)
+    x = base[1:].view(16, 256)
+    mx = (torch.rand(16, 4, generator=g) + 0.05).to(device)
+    mn = -mx
+    raw = O.scale_from_minmax(mn.cpu(), mx.cpu(), -8, 7)
+    scale_ref, pcs_ref = O.lpbq_scale(raw, 4, 8, (1, -1))
+    y_ref = O.qdq_v2_forward(x.cpu(), scale_ref, torch.zeros_like(scale_ref), -8, 7, block_size=(1, 64)).y
+
+    def call(xx, enc_shape, block, group, cd=None, mn_=mn, mx_=mx):
+        xd, layout = hip._prepare(xx, enc_shape, block)
+        grid = hip._grid(_lib.AHQ_ARITH_AUTOGRAD, _lib.AHQ_OP_QDQ, xd.dtype, cd or xd.dtype, -8, 7, 0.0)
+        y = torch.empty_like(xd)
+        scale = torch.empty(enc_shape, dtype=torch.float32, device=device)
+        pcs = torch.empty(max(1, scale.numel() // group), dtype=torch.float32, device=device)
+        status = lib.ahq_lpbq_qdq_forward(grid, layout, xd.data_ptr(), y.data_ptr(), None, _lib.DTYPE_CODE[mn_.dtype],
+                                          mn_.data_ptr(), mx_.data_ptr(), group, _get_minimum_scale(15), 16, None,
+                                          scale.data_ptr(), pcs.data_ptr(), _lib.current_stream(device))
+        return status, y, scale, pcs
+
+    status, y, scale, pcs = call(x, (16, 4), (1, 64), 4)
+    assert status == _lib.AHQ_OK
+    assert_same_bits(scale, scale_ref, "scales")
+    assert_same_bits(pcs.view(16, 1), pcs_ref, "per-channel scales")
+    assert_same_bits(y, y_ref, "output of the scalar-load path")
+    x3 = torch.randn(3, 16, 256, generator=g).to(device)
+    assert call(x3, (16, 4), (1, 64), 4)[0] == _lib.AHQ_ERR_UNSUPPORTED       # encodings repeat over the leading dimension
+    assert call(x.contiguous(), (16, 4), (1, 64), 3)[0] == _lib.AHQ_ERR_UNSUPPORTED   # 64 blocks, groups of 3
+    xb = x.contiguous().bfloat16()
+    assert call(xb, (16, 4), (1, 64), 4, cd=torch.float32)[0] == _lib.AHQ_ERR_UNSUPPORTED
+    assert call(xb, (16, 4), (1, 64), 4)[0] == _lib.AHQ_OK
