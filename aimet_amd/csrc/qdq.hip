@@ -415,6 +415,7 @@ struct LpbqFuse {
     float* scale_out;        // per block
     float* per_channel_out;  // per group, optional
     int64_t group;           // neighbouring blocks per group
+    int32_t group_shift;     // log2(group) when it is a power of two, else -1
     int32_t dtype;
     float num_steps, minimum_scale, multipliers;
 };
@@ -455,8 +456,6 @@ __device__ __forceinline__ void stage_lpbq(const QdqArgs& a, const LpbqFuse& f, 
                                            const float pre_mn, const float pre_mx) {
     __shared__ float per_channel[kStage];  // of the groups this tile touches
     const int64_t G = f.group;
-    const int64_t g0 = t.e0 / G;
-    const int ng = t.nstage > 0 ? (int)((t.e0 + t.nstage - 1) / G - g0) + 1 : 0;
     const int lane = threadIdx.x & (kWave - 1);
     auto stage_one = [&](int i, int64_t e, int64_t g, float raw, float pc) {
         const float r = __builtin_rintf(raw / pc);
@@ -471,7 +470,7 @@ __device__ __forceinline__ void stage_lpbq(const QdqArgs& a, const LpbqFuse& f, 
         if (M::kNP > 3) sp[3][i] = p.p3;
         if (M::kDiv) sp[M::kNP][i] = p.rs;
     };
-    if (G <= kWave && (G & (G - 1)) == 0 && t.e0 % G == 0 && t.nstage % G == 0) {
+    if (f.group_shift >= 0 && G <= kWave && (t.e0 & (G - 1)) == 0 && (t.nstage & (G - 1)) == 0) {
         // whole groups, each inside a power-of-two run of lanes: one read of min / max per block, the group's largest
         // raw scale by shuffles (a maximum does not depend on the order), no second barrier
         const int padded = (t.nstage + kWave - 1) & ~(kWave - 1);
@@ -487,10 +486,12 @@ __device__ __forceinline__ void stage_lpbq(const QdqArgs& a, const LpbqFuse& f, 
                 nan |= __shfl_xor(nan, m, kWave);
             }
             if (nan) largest = __builtin_nanf("");  // torch.amax propagates NaN
-            if (live) stage_one(i, e, e / G, raw, largest / f.multipliers);
+            if (live) stage_one(i, e, e >> f.group_shift, raw, largest / f.multipliers);
         }
         return;
     }
+    const int64_t g0 = t.e0 / G;
+    const int ng = t.nstage > 0 ? (int)((t.e0 + t.nstage - 1) / G - g0) + 1 : 0;
     for (int gi = threadIdx.x / kWave; gi < ng; gi += kBlock / kWave) {
         const int64_t base = (g0 + gi) * G;
         float largest = -__builtin_inff();
@@ -1361,6 +1362,10 @@ extern "C" int ahq_lpbq_qdq_forward(const ahq_grid* grid, const ahq_layout* layo
     f.scale_out = scale;
     f.per_channel_out = per_channel_scale;
     f.group = blocks_per_group;
+    f.group_shift = -1;
+    if (is_pow2(blocks_per_group))
+        for (int b = 0; b < 62; ++b)
+            if (((int64_t)1 << b) == blocks_per_group) f.group_shift = b;
     f.dtype = range_dtype;
     f.num_steps = (float)(double)(grid->qmax - grid->qmin);
     f.minimum_scale = (float)minimum_scale;

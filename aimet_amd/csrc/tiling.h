@@ -78,10 +78,13 @@ __device__ __forceinline__ Tile make_tile(const Geom& a, int64_t tile) {
             t.e0 = 0;
             t.nstage = 1;
         } else {
-            const int64_t row0 = t.v0 / a.Kv;
+            // (the usual block sizes are powers of two: shifts instead of 64-bit divisions, which cost a workgroup a
+            // few hundred instructions each)
+            const int64_t row0 = a.kv_shift >= 0 ? t.v0 >> a.kv_shift : t.v0 / a.Kv;
             t.rem0 = t.v0 - row0 * a.Kv;
             t.e0 = a.I == 1 ? row0 : row0 % a.J;
-            t.nstage = t.nv > 0 ? (int)((t.rem0 + t.nv - 1) / a.Kv) + 1 : 0;
+            const int64_t last = t.rem0 + t.nv - 1;
+            t.nstage = t.nv > 0 ? (int)(a.kv_shift >= 0 ? last >> a.kv_shift : last / a.Kv) + 1 : 0;
         }
     }
     return t;
