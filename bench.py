@@ -48,13 +48,14 @@ MEASURED_TRAFFIC_BYTES = {
     ("c1", "qdq_fwd_kernel"): int((100492.8 + 100756.7) * 1024),
     ("c2", "qdq_bwd_kernel"): int((131497.3 + 65843.5) * 1024),
     ("c2", "qdq_fwd_kernel"): int((65968.2 + 65954.8) * 1024),
-    ("c4", "qdq_bwd_kernel"): int((236861.6 + 121868.1) * 1024),
-    ("c4", "qdq_fwd_kernel"): int((122043.3 + 114935.4) * 1024),
-    # the timed update (a batch inside the running range): speculative binning pass (read + write) + the fold, finish
-    # and prepare kernels; a batch that moves the range is read a second time (about a quarter of the batches of the
-    # c3 stream)
-    ("c3", "hist_update"): int((262288.2 + 3216.0 + 3649.5 + 66.5 + 160.5 + 4.1 + 22.1 + 4.9) * 1024),
-    ("dlq", "pdf_update"): int((262317.6 + 3072.0 + 6191.2) * 1024),
+    ("c4", "qdq_bwd_kernel"): int((236827.4 + 121867.3) * 1024),
+    ("c4", "qdq_fwd_kernel"): int((122024.0 + 114935.4) * 1024),
+    ("c4", "qdq_fwd_lpbq_kernel"): int((122050.8 + 118776.6) * 1024),
+    # the timed update (a batch inside the running range): speculative binning pass (read + write) + the launch that
+    # folds its extrema and partial histograms into the running state; a batch that moves the range is read a second
+    # time (about a quarter of the batches of the c3 stream)
+    ("c3", "hist_update"): int((262288.0 + 3216.0 + 14862.3 + 3.5) * 1024),
+    ("dlq", "pdf_update"): int((262675.2 + 3072.0 + 6191.2 + 12.0) * 1024),
 }
 DTYPE_NAME = {torch.float32: "f32", torch.bfloat16: "bf16", torch.float16: "f16"}
 
