@@ -30,6 +30,7 @@ namespace ahq {
 
 constexpr int kHistBlocksMax = 1536;  // persistent workgroups of the binning pass (6 per CU)
 constexpr int kRng = 8;               // floats per slot in `ranges`
+constexpr int kPartBins = 8;          // entries per block of the single-slot partial counts
 
 // ranges[slot]: lo1, hi1, thr_lo1, thr_hi1 (batch's own range), lo2, hi2, thr_lo2, thr_hi2 (updated range).
 // thr_* are the edges rounded to the tensor dtype: the reference compares `x < edge` in the tensor's dtype.
@@ -238,7 +239,7 @@ __global__ void hist_prepare_kernel(const PrepArgs a) {
 struct BinArgs : Geom {
     const void* x;
     const float* ranges;   // [S][8]
-    uint32_t* partials;    // single slot: [nblocks][NH][B + 2]  (bins, below, above)
+    uint32_t* partials;    // single slot: [NH][blocks of kPartBins entries][nblocks][kPartBins]  (bins, below, above)
     uint32_t* counts;      // several slots: [S][NH][B + 2], zero-initialised
     int32_t num_bins;
     int32_t nhist;
@@ -480,18 +481,25 @@ __global__ __launch_bounds__(kBlock, 6) void hist_bin_kernel(const BinArgs a) {
         a.part_min[blockIdx.x] = mn;
         a.part_max[blockIdx.x] = mx;
     }
-    uint32_t* out = a.partials + (size_t)blockIdx.x * NH * (B + 2);
+    // partial counts in blocks of kPartBins entries (an entry: a bin, or one of the two edge counters behind the bins):
+    // [NH][blocks][gridDim.x][kPartBins] -- a workgroup stores 32-byte pieces, and the launch that folds the partials
+    // reads all workgroups' counts of a block as one contiguous run
+    const size_t np = gridDim.x;
+    const int nblk = (B + 2 + kPartBins - 1) / kPartBins;
+    auto slot = [&](int h, int entry) {
+        return a.partials + (((size_t)h * nblk + entry / kPartBins) * np + blockIdx.x) * kPartBins + entry % kPartBins;
+    };
     for (int i = threadIdx.x; i < NH * B; i += kBlock) {
         const int h = i / B, b = i - h * B;
         uint32_t c = 0;
         for (int cp = 0; cp < copies; ++cp) c += lds[(size_t)i * copies + cp];
-        out[h * (B + 2) + b] = c;
+        *slot(h, b) = c;
     }
     if (threadIdx.x < NH * 2) {
         const int h = threadIdx.x / 2, w = threadIdx.x & 1;
         uint32_t c = 0;
         for (int wv = 0; wv < kBlock / kWave; ++wv) c += cnt_smem[wv][h][w];
-        out[h * (B + 2) + B + w] = c;
+        *slot(h, B + w) = c;
     }
 }
 
@@ -626,7 +634,7 @@ __global__ void zero_u32_kernel(uint32_t* p, int64_t n) {
 struct FinArgs {
     int32_t num_slots, num_bins, nhist, first;
     int32_t nparts;            // partial histograms per slot (1 when `counts` is used)
-    const uint32_t* counts;    // [S][nparts][NH][B + 2]
+    const uint32_t* counts;    // several slots: [S][NH][B + 2] (nparts == 1); one slot: see hist_bin_kernel
     const float* carried;      // [S][B]
     const float* upd_edges;    // [S][B+1]
     float* hist;               // [S][B] running (out)
@@ -693,92 +701,84 @@ __global__ __launch_bounds__(kBlock) void hist_finish_kernel(const FinArgs a) {
 }
 
 // --------------------------------------------------------- single slot: fold of the partial counts and finish --
-// One launch instead of a fold and a finish: a workgroup of 1024 threads owns 8 bins, thread = (bin, one of 128 groups
-// of partial histograms); the integer sums over the partials are order-independent, the float operations per bin are
-// those of hist_finish_kernel.  `carried` may be the running histogram itself (every bin is read and written by one
-// thread); upd_edges == NULL leaves the running edges as they are.
-constexpr int kFfBins = 8;
+// One launch instead of a fold and a finish: a workgroup of 1024 threads owns one block of kPartBins bins, whose
+// partial counts from all workgroups of the binning pass are one contiguous run of memory (see hist_bin_kernel), so
+// the threads read it as whole cache lines, every thread always the same bin.  The integer sums are order-independent,
+// the float operations per bin are those of hist_finish_kernel.  `carried` may be the running histogram itself (a
+// bin is read and written by one thread); upd_edges == NULL leaves the running edges as they are.
 constexpr int kFfThreads = 1024;
-constexpr int kFfGroups = kFfThreads / kFfBins;
 
-// this thread's share of the sums: bin blockIdx.x * kFfBins + (thread % kFfBins), every kFfGroups-th partial histogram.
-// The loads are independent and the partials come from other dies' caches, so as many as possible are in flight.
+__device__ __forceinline__ const uint32_t* part_block(const FinArgs& a, int h, int blk) {
+    const int nblk = (a.num_bins + 2 + kPartBins - 1) / kPartBins;
+    return a.counts + ((size_t)h * nblk + blk) * (size_t)a.nparts * kPartBins;
+}
+
+// this thread's share of the sums of bin blockIdx.x * kPartBins + thread % kPartBins; all its loads in flight at once
 __device__ __forceinline__ void fold_load(const FinArgs& a, unsigned long long (&c)[2]) {
-    const int B = a.num_bins;
-    const int bl = threadIdx.x & (kFfBins - 1), grp = threadIdx.x / kFfBins;
-    const int b = blockIdx.x * kFfBins + bl;
-    const uint32_t* base = a.counts;
-    const size_t row = (size_t)(B + 2);
     c[0] = c[1] = 0;
-    if (b >= B) return;
-    if (a.nhist == 1) {
-        constexpr int kFlight = 16;  // 16 * 128 = 2048 partials per round: one round for any binning grid
-        for (int p = grp; p < a.nparts; p += kFlight * kFfGroups) {
+    const int n = a.nparts * kPartBins;
+    constexpr int kFlight = 16;  // 16 * 1024 entries = 2048 workgroups per round: one round for any binning grid
+    for (int h = 0; h < a.nhist; ++h) {
+        const uint32_t* run = part_block(a, h, blockIdx.x);
+        unsigned long long t = 0;
+        for (int j = threadIdx.x; j < n; j += kFlight * kFfThreads) {
             uint32_t v[kFlight];
 #pragma unroll
-            for (int k = 0; k < kFlight; ++k) v[k] = p + k * kFfGroups < a.nparts ? base[(size_t)(p + k * kFfGroups) * row + b] : 0u;
+            for (int k = 0; k < kFlight; ++k) v[k] = j + k * kFfThreads < n ? run[j + k * kFfThreads] : 0u;
 #pragma unroll
-            for (int k = 0; k < kFlight; ++k) c[0] += v[k];
+            for (int k = 0; k < kFlight; ++k) t += v[k];
         }
-    } else {
-#pragma unroll 4
-        for (int p = grp; p < a.nparts; p += kFfGroups) {
-            c[0] += base[((size_t)p * 2) * row + b];
-            c[1] += base[((size_t)p * 2 + 1) * row + b];
-        }
+        c[h] = t;
     }
 }
 
 __device__ void fold_finish_bins(const FinArgs& a, unsigned long long (&c)[2]) {
-    __shared__ unsigned long long sm[kFfGroups][2][kFfBins];
+    __shared__ unsigned long long sm[kFfThreads / kWave][2][kPartBins];
     __shared__ unsigned long long wave_edge[kFfThreads / kWave][4];
     const int B = a.num_bins, NH = a.nhist;
-    const int bl = threadIdx.x & (kFfBins - 1), grp = threadIdx.x / kFfBins;
-    const int b = blockIdx.x * kFfBins + bl;
-    const uint32_t* base = a.counts;
-    const size_t row = (size_t)(B + 2);
-    sm[grp][0][bl] = c[0];
-    sm[grp][1][bl] = c[1];
-    const float carried_b = (grp == 0 && b < B && !a.first) ? a.carried[b] : 0.f;  // fetched ahead of the barriers
-    // below / above totals, wanted by the owners of bin 0 and of bin B - 1: thread = (histogram, side, partials)
-    const bool owns_end = blockIdx.x == 0 || (int)blockIdx.x == (B - 1) / kFfBins;
+    const int wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
+    const int b = blockIdx.x * kPartBins + threadIdx.x;  // for the threads that finish a bin (the first kPartBins)
+    const bool owner = threadIdx.x < kPartBins && b < B;
+    const float carried_b = (owner && !a.first) ? a.carried[b] : 0.f;  // fetched ahead of the barrier
+#pragma unroll
+    for (int m = kWave / 2; m >= kPartBins; m >>= 1) {
+        c[0] += __shfl_xor(c[0], m, kWave);
+        c[1] += __shfl_xor(c[1], m, kWave);
+    }
+    if (lane < kPartBins) {
+        sm[wave][0][lane] = c[0];
+        sm[wave][1][lane] = c[1];
+    }
+    // below / above totals (entries B and B + 1 of every partial histogram), wanted by the owners of bin 0 and of
+    // bin B - 1: thread = (histogram, side, workgroups of the binning pass)
+    const bool owns_end = blockIdx.x == 0 || (int)blockIdx.x == (B - 1) / kPartBins;
     if (owns_end) {
         const int combo = threadIdx.x & 3, h = combo >> 1, side = combo & 1;
         unsigned long long t = 0;
         if (h < NH) {
-            constexpr int kFlight = 8, kStep = kFfThreads / 4;  // 8 * 256 partials per round
+            const int entry = B + side;
+            const uint32_t* run = part_block(a, h, entry / kPartBins) + entry % kPartBins;
+            constexpr int kFlight = 8, kStep = kFfThreads / 4;  // 8 * 256 workgroups per round
             for (int p = threadIdx.x >> 2; p < a.nparts; p += kFlight * kStep) {
                 uint32_t v[kFlight];
 #pragma unroll
                 for (int k = 0; k < kFlight; ++k)
-                    v[k] = p + k * kStep < a.nparts ? base[((size_t)(p + k * kStep) * NH + h) * row + B + side] : 0u;
+                    v[k] = p + k * kStep < a.nparts ? run[(size_t)(p + k * kStep) * kPartBins] : 0u;
 #pragma unroll
                 for (int k = 0; k < kFlight; ++k) t += v[k];
             }
         }
 #pragma unroll
-        for (int m = 32; m >= 4; m >>= 1) t += __shfl_xor(t, m, kWave);
-        if ((threadIdx.x & (kWave - 1)) < 4) wave_edge[threadIdx.x / kWave][combo] = t;
+        for (int m = kWave / 2; m >= 4; m >>= 1) t += __shfl_xor(t, m, kWave);
+        if (lane < 4) wave_edge[wave][lane] = t;
     }
     __syncthreads();
-    if (grp < 8) {
-        for (int h = 0; h < NH; ++h) {
-            unsigned long long t = 0;
-#pragma unroll
-            for (int k = 0; k < kFfGroups / 8; ++k) t += sm[grp + 8 * k][h][bl];
-            c[h] = t;
-        }
-    }
-    __syncthreads();
-    if (grp < 8) {
-        sm[grp][0][bl] = c[0];
-        sm[grp][1][bl] = c[1];
-    }
-    __syncthreads();
-    if (grp != 0 || b >= B) return;
+    if (!owner) return;
     unsigned long long tot[2] = {0, 0};
-    for (int h = 0; h < NH; ++h)
-        for (int k = 0; k < 8; ++k) tot[h] += sm[k][h][bl];
+    for (int w = 0; w < kFfThreads / kWave; ++w) {
+        tot[0] += sm[w][0][threadIdx.x];
+        tot[1] += sm[w][1][threadIdx.x];
+    }
     unsigned long long edge_cnt[2][2] = {{0, 0}, {0, 0}};
     if (b == 0 || b == B - 1)
         for (int w = 0; w < kFfThreads / kWave; ++w)
@@ -907,7 +907,8 @@ bool make_hist_plan(int dtype, const ahq_layout& layout, const void* x, int num_
     hp->off_rebin = o;     o = align_up(o + (size_t)S * 4);
     hp->off_counts = o;
     const size_t nparts = hp->fast ? (size_t)hp->nblocks : 1;
-    o = align_up(o + (size_t)S * nparts * 2 * (B + 2) * 4);
+    const size_t entries = ((B + 2 + kPartBins - 1) / kPartBins) * kPartBins;  // the single-slot layout is in whole blocks
+    o = align_up(o + (size_t)S * nparts * 2 * entries * 4);
     hp->total = o;
     return true;
 }
@@ -1020,7 +1021,7 @@ extern "C" int ahq_hist_update(int32_t dtype, const ahq_layout* layout, const vo
     FinArgs fa{};
     fa.num_slots = S;
     fa.num_bins = B;
-    const dim3 ffgrid((B + kFfBins - 1) / kFfBins);
+    const dim3 ffgrid((B + kPartBins - 1) / kPartBins);
     if (speculative) {
         // the counts of the speculative pass, folded straight into the running histogram if the range holds
         fa.nhist = 1;

@@ -487,8 +487,11 @@ def run_qdq_workload(key, steps, warmup, dev, with_cpu_baseline=True):
         out = q(xm)
         out.backward(grad)
 
-    mod_loop, mod_repeats = timed_steps(module_step, steps, min(warmup, 5))
-    mod_s = mod_loop / steps
+    # loops of at least 200 steps: the first steps after a synchronisation wait for autograd's device thread to wake up
+    # (about a millisecond), which a loop of twenty 0.1 ms steps would report as half as much again per step
+    mod_steps = max(steps, 200)
+    mod_loop, mod_repeats = timed_steps(module_step, mod_steps, min(warmup, 5))
+    mod_s = mod_loop / mod_steps
     module_step()
     _sync()
     mod_gx_exact = None
@@ -547,7 +550,8 @@ def run_qdq_workload(key, steps, warmup, dev, with_cpu_baseline=True):
         "module_path": {"what": "QuantizeDequantize.forward + .backward() with learnable min/max (allocations, "
                                 "autograd and the per-call scale / offset derivation included)",
                         "ms_per_step": round(mod_s * 1e3, 5), "GBps": round(bytes_step / mod_s / 1e9, 1),
-                        "frac_of_hbm_peak": round(bytes_step / mod_s / 1e9 / HBM_PEAK_GBS, 4), "repeats": mod_repeats},
+                        "frac_of_hbm_peak": round(bytes_step / mod_s / 1e9 / HBM_PEAK_GBS, 4), "repeats": mod_repeats,
+                        "steps_per_timed_loop": mod_steps},
         "parity": parity,
         "roofline": {"bound": "hbm", "kernel": dom[0], "achieved": round(dom[2] / dom[1] / 1e9, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(dom[2] / dom[1] / 1e9 / HBM_PEAK_GBS, 4),
