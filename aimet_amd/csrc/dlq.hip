@@ -173,6 +173,7 @@ __device__ __forceinline__ bool pdf_index(float v, float inv, float off, int& id
 // adds to copy l % copies, so with many copies the lanes of a wave land in different banks whatever the data looks
 // like: real activations put most elements into a few dozen buckets, and with few copies the wave's 64 atomic adds
 // pile onto a handful of banks and are replayed bank conflict by bank conflict.
+constexpr int kFfBins = 16;    // buckets per block of the single-slot partial counts
 constexpr int kPdfUnroll = 4;  // 16-byte loads in flight per lane: the workgroups are persistent, so this sets the bytes in flight
 
 template <typename IO, int VEC, int THREADS>
@@ -254,11 +255,12 @@ __global__ __launch_bounds__(THREADS) void dlq_pdf_bin_kernel(const PdfBinArgs a
         for (int64_t i = a.nvec * VEC + threadIdx.x; i < a.numel; i += THREADS) add(load_f32(x[i]));
     }
     __syncthreads();
-    uint32_t* out = a.partials + (size_t)blockIdx.x * kPdf;
+    // partial counts in blocks of kFfBins buckets, [block][workgroup][kFfBins]: a workgroup stores 64-byte pieces, and
+    // the launch that folds the partials reads all workgroups' counts of a block as one contiguous run
     for (int i = threadIdx.x; i < kPdf; i += THREADS) {
         uint32_t c = 0;
         for (int cp = 0; cp < copies; ++cp) c += lds[(size_t)i * copies + cp];
-        out[i] = c;
+        a.partials[((size_t)(i / kFfBins) * gridDim.x + blockIdx.x) * kFfBins + i % kFfBins] = c;
     }
 }
 
@@ -312,18 +314,6 @@ __global__ void dlq_zero_u32_kernel(uint32_t* p, int64_t n) {
 
 constexpr int kPdfFoldGroups = 16;
 
-// partial[p][kPdf] -> folded[g][kPdf], g = p % groups
-__global__ __launch_bounds__(kBlock) void dlq_pdf_fold_kernel(const uint32_t* partial, uint32_t* folded, const float* params,
-                                                             int nparts) {
-    if (params[2] == 0.f) return;
-    const int l = blockIdx.x * kBlock + threadIdx.x;
-    const int g = blockIdx.y;
-    uint32_t acc = 0;
-#pragma unroll 4
-    for (int p = g; p < nparts; p += kPdfFoldGroups) acc += partial[(size_t)p * kPdf + l];
-    folded[(size_t)g * kPdf + l] = acc;
-}
-
 struct PdfFinArgs {
     const uint32_t* counts;  // [S][nparts][kPdf]
     int32_t nparts;
@@ -356,10 +346,12 @@ __global__ __launch_bounds__(kBlock) void dlq_pdf_finish_kernel(const PdfFinArgs
     }
 }
 
-// Single slot, many partial histograms: fold and average in one launch.  A workgroup owns kFfBins neighbouring
-// buckets; its lanes split the partials kFfGroups ways (64-byte segments per partial), then one lane per bucket adds
-// the group sums in a fixed order and does what dlq_pdf_finish_kernel does.
-constexpr int kFfBins = 16, kFfGroups = kBlock / kFfBins;
+// Single slot, many partial histograms: fold and average in one launch.  A workgroup owns one block of kFfBins
+// neighbouring buckets, whose partial counts from all workgroups of the binning pass are one contiguous run (see
+// dlq_pdf_bin_kernel): its threads read it as whole cache lines, every thread always the same bucket, all loads in
+// flight at once; then one lane per bucket adds the group sums (integers: the order does not matter) and does what
+// dlq_pdf_finish_kernel does.
+constexpr int kFfGroups = kBlock / kFfBins;
 __global__ __launch_bounds__(kBlock) void dlq_pdf_fold_finish_kernel(const PdfFinArgs a) {
     __shared__ uint32_t sm[kFfGroups][kFfBins];
     const int bl = threadIdx.x & (kFfBins - 1), grp = threadIdx.x / kFfBins;
@@ -367,8 +359,16 @@ __global__ __launch_bounds__(kBlock) void dlq_pdf_fold_finish_kernel(const PdfFi
     const bool active = a.params[2] != 0.f;
     uint32_t acc = 0;
     if (active) {
-#pragma unroll 8
-        for (int p = grp; p < a.nparts; p += kFfGroups) acc += a.counts[(size_t)p * kPdf + i];
+        const uint32_t* run = a.counts + (size_t)blockIdx.x * a.nparts * kFfBins;
+        const int n = a.nparts * kFfBins;
+        constexpr int kFlight = 16;
+        for (int j = threadIdx.x; j < n; j += kFlight * kBlock) {
+            uint32_t v[kFlight];
+#pragma unroll
+            for (int k = 0; k < kFlight; ++k) v[k] = j + k * kBlock < n ? run[j + k * kBlock] : 0u;
+#pragma unroll
+            for (int k = 0; k < kFlight; ++k) acc += v[k];
+        }
     }
     sm[grp][bl] = acc;
     __syncthreads();
@@ -816,7 +816,7 @@ struct PdfPlan {
     Plan plan;
     bool fast;
     int copies, nblocks;
-    size_t off_mm_ws, off_bmin, off_bmax, off_params, off_counts, off_folded, total;
+    size_t off_mm_ws, off_bmin, off_bmax, off_params, off_counts, total;
 };
 
 bool make_pdf_plan(int dtype, const ahq_layout& layout, const void* x, PdfPlan* pp) {
@@ -836,7 +836,6 @@ bool make_pdf_plan(int dtype, const ahq_layout& layout, const void* x, PdfPlan* 
     pp->off_bmax = o;    o = up256(o + S * 4);
     pp->off_params = o;  o = up256(o + S * 16);
     pp->off_counts = o;  o = up256(o + (pp->fast ? (size_t)pp->nblocks : S) * kPdf * 4);
-    pp->off_folded = o;  o = up256(o + (size_t)kPdfFoldGroups * kPdf * 4);
     pp->total = o;
     return true;
 }
@@ -966,19 +965,11 @@ extern "C" int ahq_dlq_pdf_update(int32_t dtype, const ahq_layout* layout, const
         }
 #undef AHQ_LAUNCH_PDF
 #undef AHQ_LAUNCH_PDF_K
+        // (one slot: the layout of the partial counts is the one dlq_pdf_fold_finish_kernel reads)
         fa.counts = counts;
         fa.nparts = pp.nblocks;
-        if (S == 1 && pp.nblocks > kPdfFoldGroups) {
-            hipLaunchKernelGGL(dlq_pdf_fold_finish_kernel, dim3(kPdf / kFfBins), dim3(kBlock), 0, s, fa);
-            return check_launch("dlq_pdf_update");
-        }
-        if (pp.nblocks > kPdfFoldGroups) {
-            uint32_t* folded = reinterpret_cast<uint32_t*>(w + pp.off_folded);
-            hipLaunchKernelGGL(dlq_pdf_fold_kernel, dim3(kPdf / kBlock, kPdfFoldGroups), dim3(kBlock), 0, s, counts, folded,
-                               params, pp.nblocks);
-            fa.counts = folded;
-            fa.nparts = kPdfFoldGroups;
-        }
+        hipLaunchKernelGGL(dlq_pdf_fold_finish_kernel, dim3(kPdf / kFfBins), dim3(kBlock), 0, s, fa);
+        return check_launch("dlq_pdf_update");
     } else if (pp.plan.cl.kind == kIJK && pp.plan.cl.I == 1 && pp.plan.cl.J > 1 && pp.plan.cl.K >= kBlock &&
                pp.plan.cl.J <= 0x7fffffff) {
         // one run per slot
