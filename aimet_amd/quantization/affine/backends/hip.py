@@ -225,36 +225,43 @@ class _HipAffineFunction(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, grad):
-        lib = _lib.load()
         x, s, o = ctx.saved_tensors
         need_x, need_s, need_o = ctx.needs_input_grad[:3]
         none7 = (None,) * 7
         if not (need_x or need_s or need_o):
             return (None, None, None) + none7
         want_pg = (need_s or need_o) and ctx.grid.arith == _lib.AHQ_ARITH_AUTOGRAD
-        g = _like(x, grad)
-        gx = torch.empty_like(x) if need_x else None
-        gs = go = None
-        if want_pg:
-            gs = torch.empty(s.shape, dtype=torch.float32, device=x.device)
-            go = torch.empty(s.shape, dtype=torch.float32, device=x.device)
-        if x.numel() == 0:
-            if want_pg:
-                gs.zero_()
-                go.zero_()
-        else:
-            nbytes = lib.ahq_qdq_backward_workspace_bytes(ctx.grid, ctx.layout, 1 if want_pg else 0)
-            ws = _workspace(nbytes, x.device)
-            _lib.check(
-                lib.ahq_qdq_backward(ctx.grid, ctx.layout, g.data_ptr(), x.data_ptr(), _lib.ptr(gx), _lib.ptr(gs),
-                                     _lib.ptr(go), s.data_ptr(), o.data_ptr(), _lib.ptr(ws), nbytes,
-                                     _lib.current_stream(x.device)),
-                "ahq_qdq_backward",
-            )
+        gx, gs, go = _launch_backward(ctx.grid, ctx.layout, x, s, o, grad, need_x, want_pg)
         s_shape, o_shape, s_dtype, o_dtype = ctx.enc_shapes
         gs_out = gs.view(s_shape).to(s_dtype) if (need_s and want_pg) else None
         go_out = go.view(o_shape).to(o_dtype) if (need_o and want_pg) else None
         return (gx, gs_out, go_out) + none7
+
+
+def _launch_backward(grid, layout, x, s, o, grad, need_x: bool, want_pg: bool):
+    """One launch for the input gradient and (``want_pg``) the float32 gradients of scale and offset; x, s, o as
+    _launch_forward returned them."""
+    lib = _lib.load()
+    g = _like(x, grad)
+    gx = torch.empty_like(x) if need_x else None
+    gs = go = None
+    if want_pg:
+        gs = torch.empty(s.shape, dtype=torch.float32, device=x.device)
+        go = torch.empty(s.shape, dtype=torch.float32, device=x.device)
+    if x.numel() == 0:
+        if want_pg:
+            gs.zero_()
+            go.zero_()
+    else:
+        nbytes = lib.ahq_qdq_backward_workspace_bytes(grid, layout, 1 if want_pg else 0)
+        ws = _workspace(nbytes, x.device)
+        _lib.check(
+            lib.ahq_qdq_backward(grid, layout, g.data_ptr(), x.data_ptr(), _lib.ptr(gx), _lib.ptr(gs),
+                                 _lib.ptr(go), s.data_ptr(), o.data_ptr(), _lib.ptr(ws), nbytes,
+                                 _lib.current_stream(x.device)),
+            "ahq_qdq_backward",
+        )
+    return gx, gs, go
 
 
 def _broadcast_encodings(scale: torch.Tensor, offset: torch.Tensor, block_size):

@@ -97,6 +97,139 @@ class _RangeToScaleOffset(torch.autograd.Function):
         return gmin, gmax, None, None, None, None
 
 
+class _QdqFromRange(torch.autograd.Function):
+    """QuantizeDequantize.forward with learned min / max as one autograd node: (x, min, max) -> (y, scale, offset).
+    Forward: ahq_range_to_scale_offset, then ahq_qdq_forward; backward: ahq_qdq_backward (input, scale and offset
+    gradients in one launch), then ahq_range_backward.  The same four launches as _RangeToScaleOffset followed by the
+    backend's quantize_dequantize, so the same bits; one node, one apply() and one encoding object less per step of a
+    host-bound training loop.  scale and offset are outputs too, for whoever differentiates through the encoding the
+    output tensor carries; offset is None on a symmetric grid (the caller holds the constant)."""
+
+    @staticmethod
+    def forward(ctx, x, mn, mx, qmin, qmax, symmetric, constant_offset, block_size, zps, compute_dtype):  # pylint: disable=arguments-differ
+        from aimet_amd.quantization.affine.backends import hip as _hip
+
+        scale = torch.empty(mn.shape, dtype=torch.float32, device=mn.device)
+        offset = constant_offset if symmetric else torch.empty(mn.shape, dtype=torch.float32, device=mn.device)
+        _lib.check(
+            _lib.load().ahq_range_to_scale_offset(_lib.DTYPE_CODE[mn.dtype], mn.data_ptr(), mx.data_ptr(), mn.numel(),
+                                                  qmin, qmax, _get_minimum_scale(qmax - qmin), scale.data_ptr(),
+                                                  None if symmetric else offset.data_ptr(),
+                                                  _lib.current_stream(mn.device)),
+            "ahq_range_to_scale_offset")
+        y, xd, s, o, grid, layout = _hip._launch_forward(  # pylint: disable=protected-access
+            x, scale, offset, _lib.AHQ_ARITH_AUTOGRAD, _lib.AHQ_OP_QDQ, compute_dtype, qmin, qmax, block_size, zps)
+        ctx.save_for_backward(xd, s, o, mn, mx)
+        ctx.grid, ctx.layout, ctx.range_grid = grid, layout, (qmin, qmax, symmetric)
+        ctx.set_materialize_grads(False)  # an output nobody used arrives as None, not as zeros
+        return y, scale, (None if symmetric else offset)
+
+    @staticmethod
+    def backward(ctx, gy, gscale, goffset):  # pylint: disable=arguments-differ
+        from aimet_amd.quantization.affine.backends import hip as _hip
+
+        xd, s, o, mn, mx = ctx.saved_tensors
+        qmin, qmax, symmetric = ctx.range_grid
+        need_x, need_mn, need_mx = ctx.needs_input_grad[:3]
+        none7 = (None,) * 7
+        want_pg = need_mn or need_mx
+        gx = gs = go = None
+        if gy is not None and (need_x or want_pg):
+            gx, gs, go = _hip._launch_backward(ctx.grid, ctx.layout, xd, s, o, gy, need_x, want_pg)  # pylint: disable=protected-access
+        if not want_pg:
+            return (gx, None, None) + none7
+        # gradients that reached scale / offset through the encoding object add to the kernel's
+        if gscale is not None:
+            gscale = gscale.to(torch.float32).reshape(s.shape)
+            gs = gscale if gs is None else gs + gscale
+        if goffset is not None and not symmetric:
+            goffset = goffset.to(torch.float32).reshape(s.shape)
+            go = goffset if go is None else go + goffset
+        if gs is None and (symmetric or go is None):
+            return (gx, None, None) + none7
+        if gs is None:
+            gs = torch.zeros(s.shape, dtype=torch.float32, device=s.device)
+        # an offset that nothing downstream used has no gradient path at all (a zero gradient would still meet
+        # infinite factors on its way)
+        symmetric = symmetric or go is None
+        gmin, gmax = torch.empty_like(mn), torch.empty_like(mx)
+        _lib.check(
+            _lib.load().ahq_range_backward(_lib.DTYPE_CODE[mn.dtype], mn.data_ptr(), mx.data_ptr(), mn.numel(), qmin, qmax,
+                                           _get_minimum_scale(qmax - qmin), gs.contiguous().data_ptr(),
+                                           None if symmetric else go.contiguous().data_ptr(), gmin.data_ptr(),
+                                           gmax.data_ptr(), _lib.current_stream(mn.device)),
+            "ahq_range_backward")
+        return (gx, gmin if need_mn else None, gmax if need_mx else None) + none7
+
+
+def _lpbq_forward_launch(x, mn, mx, qmin, qmax, block_size, group, group_shape, multipliers, offset):
+    """ahq_lpbq_qdq_forward on a plain tensor: (status, y, x dense in memory, scale, per-channel scale, grid, layout).
+    ``offset``: the quantizer's constant float32 offset (not passed to the kernel when it is zero)."""
+    from aimet_amd.quantization.affine.backends import hip as _hip
+
+    x, layout = _hip._prepare(x.detach(), tuple(mn.shape), block_size)  # pylint: disable=protected-access
+    grid = _hip._grid(_lib.AHQ_ARITH_AUTOGRAD, _lib.AHQ_OP_QDQ, x.dtype, x.dtype, qmin, qmax, 0.0)  # pylint: disable=protected-access
+    y = torch.empty_like(x)
+    scale = torch.empty(mn.shape, dtype=torch.float32, device=x.device)
+    per_channel = torch.empty(group_shape, dtype=torch.float32, device=x.device)
+    offset_ptr = None if getattr(offset, "_ahq_constant", None) == 0 else offset.data_ptr()
+    status = _lib.load().ahq_lpbq_qdq_forward(
+        grid, layout, x.data_ptr(), y.data_ptr(), None, _lib.DTYPE_CODE[mn.dtype], mn.data_ptr(), mx.data_ptr(), group,
+        _get_minimum_scale(qmax - qmin), multipliers, offset_ptr, scale.data_ptr(), per_channel.data_ptr(),
+        _lib.current_stream(x.device))
+    return status, y, x, scale, per_channel, grid, layout
+
+
+class _LpbqQdqFromRange(torch.autograd.Function):
+    """GroupedBlockQuantizeDequantize.forward with gradients as one autograd node: (x, min, max) -> (y, block scales,
+    per-channel scales) with ahq_lpbq_qdq_forward; backward: ahq_qdq_backward (input and scale gradients in one
+    launch), then ahq_lpbq_scale_backward down to min / max.  The launches compute what _LpbqScale followed by the
+    backend's quantize_dequantize computes, bit for bit."""
+
+    @staticmethod
+    def forward(ctx, x, mn, mx, qmin, qmax, block_size, group, group_shape, multipliers, offset, group_layout):  # pylint: disable=arguments-differ
+        status, y, xd, scale, per_channel, grid, layout = _lpbq_forward_launch(
+            x, mn, mx, qmin, qmax, block_size, group, group_shape, multipliers, offset)
+        _lib.check(status, "ahq_lpbq_qdq_forward")
+        ctx.save_for_backward(xd, scale, mn, mx)
+        ctx.grid, ctx.layout, ctx.offset = grid, layout, offset
+        ctx.args = (qmin, qmax, multipliers, group_layout)
+        ctx.set_materialize_grads(False)
+        return y, scale, per_channel
+
+    @staticmethod
+    def backward(ctx, gy, gscale, gper_channel):  # pylint: disable=arguments-differ
+        from aimet_amd.quantization.affine.backends import hip as _hip
+
+        xd, s, mn, mx = ctx.saved_tensors
+        qmin, qmax, multipliers, group_layout = ctx.args
+        need_x, need_mn, need_mx = ctx.needs_input_grad[:3]
+        none8 = (None,) * 8
+        want_pg = need_mn or need_mx
+        gx = gs = None
+        if gy is not None and (need_x or want_pg):
+            gx, gs, _ = _hip._launch_backward(ctx.grid, ctx.layout, xd, s.detach(), ctx.offset, gy, need_x, want_pg)  # pylint: disable=protected-access
+        if not want_pg:
+            return (gx, None, None) + none8
+        if gscale is not None:
+            gscale = gscale.to(torch.float32).reshape(s.shape)
+            gs = gscale if gs is None else gs + gscale
+        if gs is None and gper_channel is None:
+            return (gx, None, None) + none8
+        if gs is None:
+            gs = torch.zeros(s.shape, dtype=torch.float32, device=s.device)
+        if gper_channel is not None:
+            gper_channel = gper_channel.to(torch.float32).contiguous()
+        gmin, gmax = torch.empty_like(mn), torch.empty_like(mx)
+        _lib.check(
+            _lib.load().ahq_lpbq_scale_backward(_lib.DTYPE_CODE[mn.dtype], group_layout, mn.data_ptr(), mx.data_ptr(),
+                                                qmin, qmax, _get_minimum_scale(qmax - qmin), multipliers,
+                                                gs.contiguous().data_ptr(), _lib.ptr(gper_channel), gmin.data_ptr(),
+                                                gmax.data_ptr(), _lib.current_stream(mn.device)),
+            "ahq_lpbq_scale_backward")
+        return (gx, gmin if need_mn else None, gmax if need_mx else None) + none8
+
+
 class _LpbqScale(torch.autograd.Function):
     """(min, max) -> (LPBQ block scales, per-group scales) in float32 with one launch each way (ahq_lpbq_scale /
     ahq_lpbq_scale_backward) instead of the reference's sequence -- get_scale, group maximum, division,
@@ -638,7 +771,44 @@ class QuantizeDequantize(AffineQuantizerBase):
     def __init__(self, shape, *args, **kwargs):  # pylint: disable=useless-parent-delegation
         super().__init__(shape, *args, **kwargs)
 
+    def _forward_from_range(self, input: torch.Tensor) -> Optional[DequantizedTensor]:
+        """The forward pass with learned min / max as one autograd node (_QdqFromRange); None when that does not
+        apply (nothing learned, a subclass or a patched get_encodings(), another backend, tensors the library does
+        not take, a grid that needs another compute dtype check) and the step-by-step form has to run."""
+        from aimet_amd.quantization.affine.backends import get_backend, hip as _hip
+
+        cls = type(self)
+        mn, mx = self.min, self.max
+        if not (torch.is_grad_enabled() and (mn.requires_grad or mx.requires_grad)):
+            return None
+        if (cls.get_scale is not AffineQuantizerBase.get_scale or cls._get_offset is not AffineQuantizerBase._get_offset
+                or cls.get_encodings is not AffineQuantizerBase.get_encodings or "get_encodings" in self.__dict__
+                or get_backend() is not _hip or not self.is_initialized()):
+            return None
+        if not (input.is_cuda and input.dtype in _lib.DTYPE_CODE and input.numel() > 0 and mn.device == input.device
+                and mx.device == input.device and mn.dtype == mx.dtype and mn.dtype in _lib.DTYPE_CODE
+                and mn.shape == mx.shape and mn.is_contiguous() and mx.is_contiguous()):
+            return None
+        cd = _hip._internal_dtype(input.dtype, self.qmin, self.qmax)  # pylint: disable=protected-access
+        if cd == torch.float64 or not _hip._is_grid_representable(cd, self.qmin, self.qmax):  # pylint: disable=protected-access
+            return None  # the step-by-step form raises what the reference raises
+        x = input if type(input) == torch.Tensor else input.as_subclass(torch.Tensor)  # pylint: disable=unidiomatic-typecheck
+        _hip._validate_arguments(x, mn, self.qmin, self.qmax, self.block_size)  # pylint: disable=protected-access
+        symmetric = bool(self.symmetric)
+        constant = self._constant_offset(mn.device) if symmetric else None
+        bs = tuple(self.block_size) if self.block_size else None
+        y, scale, offset = _QdqFromRange.apply(x, mn, mx, self.qmin, self.qmax, symmetric, constant, bs,
+                                               float(self.zero_point_shift or 0.0), cd)
+        encoding = AffineEncoding(scale, constant if symmetric else offset, self.qmin, self.qmax, self._symmetric,
+                                  self.block_size, self.zero_point_shift, producer=self)
+        output = y.as_subclass(DequantizedTensor)
+        output.encoding = encoding
+        return output
+
     def forward(self, input: torch.Tensor) -> DequantizedTensor:
+        fused = self._forward_from_range(input)
+        if fused is not None:
+            return fused
         encoding = self._forward_encoding(input, "QuantizeDequantize")
         if type(input) != torch.Tensor:  # pylint: disable=unidiomatic-typecheck
             input = input.as_subclass(torch.Tensor)
@@ -754,23 +924,24 @@ class GroupedBlockQuantizeDequantize(QuantizeDequantize):
 
     def _fused_forward(self, input: torch.Tensor) -> Optional[DequantizedTensor]:
         """The whole forward pass -- block scales from min / max, snapped to the group's multiples, then
-        quantize-dequantize -- in one launch (ahq_lpbq_qdq_forward) when no gradient is wanted; None when that does
-        not apply and get_encodings() followed by quantize_dequantize() has to run."""
-        from aimet_amd.quantization.affine.backends import hip as _hip
+        quantize-dequantize -- in one launch (ahq_lpbq_qdq_forward), as one autograd node (_LpbqQdqFromRange) when a
+        gradient is wanted; None when that does not apply and get_encodings() followed by quantize_dequantize() has
+        to run."""
+        from aimet_amd.quantization.affine.backends import get_backend, hip as _hip
 
         cls = type(self)
         if (cls.get_scale is not GroupedBlockQuantizeDequantize.get_scale
                 or cls.get_encodings is not GroupedBlockQuantizeDequantize.get_encodings
-                or "get_encodings" in self.__dict__ or not self.is_initialized() or self.zero_point_shift):
+                or "get_encodings" in self.__dict__ or not self.is_initialized() or self.zero_point_shift
+                or get_backend() is not _hip):
             return None
         mn, mx = self.min, self.max
-        if torch.is_grad_enabled() and (input.requires_grad or mn.requires_grad or mx.requires_grad):
-            return None
         if not (input.is_cuda and input.dtype in _lib.DTYPE_CODE and input.numel() > 0 and mn.device == input.device
                 and mx.device == input.device and mn.dtype == mx.dtype and mn.dtype in _lib.DTYPE_CODE
                 and mn.shape == mx.shape and mn.is_contiguous() and mx.is_contiguous()):
             return None
-        key = (tuple(input.shape), input.dtype, tuple(mn.shape), self.block_size, tuple(self.block_grouping))
+        shape = tuple(mn.shape)
+        key = (tuple(input.shape), input.dtype, shape, self.block_size, tuple(self.block_grouping))
         if self.__dict__.get("_lpbq_forward_unsupported") == key:
             return None
         group = self._blocks_per_group()
@@ -778,28 +949,30 @@ class GroupedBlockQuantizeDequantize(QuantizeDequantize):
             return None
         x = input if type(input) == torch.Tensor else input.as_subclass(torch.Tensor)  # pylint: disable=unidiomatic-typecheck
         _hip._validate_arguments(x, mn, self.qmin, self.qmax, self.block_size)  # pylint: disable=protected-access
-        x, layout = _hip._prepare(x.detach(), tuple(mn.shape), self.block_size)  # pylint: disable=protected-access
         offset = self._constant_offset(x.device)  # symmetric grid (the constructor accepts no other)
-        if getattr(offset, "_ahq_constant", None) == 0:
-            offset_ptr = None
-        elif offset.is_contiguous() and offset.numel() == mn.numel() and offset.dtype == torch.float32:
-            offset_ptr = offset.data_ptr()
-        else:
+        if not (offset.is_contiguous() and offset.numel() == mn.numel() and offset.dtype == torch.float32):
             return None
-        shape = tuple(mn.shape)
         group_shape = tuple(d // g if g != -1 else 1 for d, g in zip(shape, self.block_grouping))
-        grid = _hip._grid(_lib.AHQ_ARITH_AUTOGRAD, _lib.AHQ_OP_QDQ, x.dtype, x.dtype, self.qmin, self.qmax, 0.0)  # pylint: disable=protected-access
-        y = torch.empty_like(x)
-        scale = torch.empty(shape, dtype=torch.float32, device=x.device)
-        per_channel = torch.empty(group_shape, dtype=torch.float32, device=x.device)
-        status = _lib.load().ahq_lpbq_qdq_forward(
-            grid, layout, x.data_ptr(), y.data_ptr(), None, _lib.DTYPE_CODE[mn.dtype], mn.data_ptr(), mx.data_ptr(),
-            group, _get_minimum_scale(self.qmax - self.qmin), 2 ** (self.decompressed_bw - self.bitwidth), offset_ptr,
-            scale.data_ptr(), per_channel.data_ptr(), _lib.current_stream(x.device))
-        if status == _lib.AHQ_ERR_UNSUPPORTED:
-            self.__dict__["_lpbq_forward_unsupported"] = key
-            return None
-        _lib.check(status, "ahq_lpbq_qdq_forward")
+        multipliers = 2 ** (self.decompressed_bw - self.bitwidth)
+        bs = tuple(self.block_size) if self.block_size else None
+        if torch.is_grad_enabled() and (input.requires_grad or mn.requires_grad or mx.requires_grad):
+            # the library refuses some layouts and groupings: find out once per shape, outside autograd
+            if self.__dict__.get("_lpbq_forward_supported") != key:
+                with torch.no_grad():
+                    if self._fused_forward(x.detach()) is None or self._fused_lpbq_scale() is None:
+                        self.__dict__["_lpbq_forward_unsupported"] = key
+                        return None
+            group_layout = _build_layout(shape, tuple(range(len(shape))), group_shape, tuple(self.block_grouping))
+            y, scale, per_channel = _LpbqQdqFromRange.apply(x, mn, mx, self.qmin, self.qmax, bs, group, group_shape,
+                                                            multipliers, offset, group_layout)
+        else:
+            status, y, _, scale, per_channel, _, _ = _lpbq_forward_launch(x, mn, mx, self.qmin, self.qmax, bs, group,
+                                                                          group_shape, multipliers, offset)
+            if status == _lib.AHQ_ERR_UNSUPPORTED:
+                self.__dict__["_lpbq_forward_unsupported"] = key
+                return None
+            _lib.check(status, "ahq_lpbq_qdq_forward")
+            self.__dict__["_lpbq_forward_supported"] = key
         encoding = GroupedBlockEncoding(scale=scale, offset=offset, bitwidth=self.bitwidth, signed=self.signed,
                                         symmetry=self.symmetric, block_size=self.block_size,
                                         block_grouping=self.block_grouping, decompressed_bw=self.decompressed_bw,

@@ -752,3 +752,101 @@ def test_lpbq_forward_misaligned_and_refused_layouts(device):
     xb = x.contiguous().bfloat16()
     assert call(xb, (16, 4), (1, 64), 4, cd=torch.float32)[0] == _lib.AHQ_ERR_UNSUPPORTED
     assert call(xb, (16, 4), (1, 64), 4)[0] == _lib.AHQ_OK
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("case", [
+    ((37, 129), (), None, 8, False),
+    ((64, 512), (64, 1), None, 8, True),
+    ((32, 256), (32, 4), (1, 64), 4, True),
+    ((4, 6, 10, 10), (6, 1, 1), None, 8, False),
+    ((16, 64), (16, 1), None, 16, False),
+], ids=["per_tensor", "per_channel", "blockwise", "activation_channels", "sixteen_bit"])
+def test_forward_with_learned_ranges_as_one_autograd_node(device, monkeypatch, dtype, case):
+    """With learned min / max, QuantizeDequantize.forward is one autograd node (_QdqFromRange: scale / offset
+    derivation and quantize-dequantize forward, their two backward launches behind it).  Output, input gradient and
+    the gradients of min / max must equal, bit for bit, what the two-node form gives -- get_encodings() followed by
+    the backend's quantize_dequantize -- also when the loss uses the scale and offset of the encoding the output
+    carries."""
+    from aimet_amd.quantization.affine import QuantizeDequantize
+    from aimet_amd.quantization.affine.quantizer import QuantizeDequantize as QdqClass
+
+    shape, enc_shape, block, bitwidth, symmetric = case
+    g = torch.Generator().manual_seed(17)
+    x = (torch.randn(shape, generator=g) * 0.7).to(dtype)
+    grad = torch.randn(shape, generator=g).to(dtype)
+    q = QuantizeDequantize(enc_shape, bitwidth, symmetric, block_size=block).to(device)
+    with q.compute_encodings():
+        q(x.to(device) * 0.5)          # narrower ranges than the data: clipped elements carry the range gradients
+    w = torch.randn(enc_shape, generator=g).to(device)
+
+    def run(through_encoding):
+        xd = x.to(device).requires_grad_(True)
+        q.min.grad = q.max.grad = None
+        out = q(xd)
+        loss = (out.as_subclass(torch.Tensor).float() * grad.to(device).float()).sum()
+        if through_encoding:
+            loss = loss + (out.encoding.scale * w).sum()
+            if not symmetric:
+                loss = loss + (out.encoding.offset * w).sum() * 1e-3
+        loss.backward()
+        return (out.detach().as_subclass(torch.Tensor).clone(), xd.grad.clone(), q.min.grad.clone(), q.max.grad.clone(),
+                type(out.encoding.scale.grad_fn).__name__)
+
+    for through_encoding in (False, True):
+        one = run(through_encoding)
+        assert one[4].startswith("_QdqFromRange")
+        with monkeypatch.context() as m:
+            m.setattr(QdqClass, "_forward_from_range", lambda self, input: None)
+            two = run(through_encoding)
+        assert not two[4].startswith("_QdqFromRange")
+        for a, b, what in zip(one[:4], two[:4], ("output", "input gradient", "gradient of min", "gradient of max")):
+            assert_same_bits(a, b, f"{what} (loss through the encoding: {through_encoding})")
+        assert float(one[2].abs().sum()) > 0 and float(one[3].abs().sum()) > 0
+
+
+@pytest.mark.parametrize("dtype,param_dtype", [(torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16),
+                                               (torch.bfloat16, torch.float32)], ids=["f32", "bf16", "bf16_f32params"])
+@pytest.mark.parametrize("case", LPBQ_FORWARD_CASES[:4], ids=["rows", "split_groups", "fours", "short_blocks"])
+def test_lpbq_forward_with_gradients_as_one_autograd_node(device, monkeypatch, case, dtype, param_dtype):
+    """With gradients wanted the LPBQ forward pass is one autograd node (_LpbqQdqFromRange: ahq_lpbq_qdq_forward, then
+    ahq_qdq_backward and ahq_lpbq_scale_backward).  Output, input gradient and the gradients of min / max must equal,
+    bit for bit, what the two-node form gives (_LpbqScale, then the backend's quantize_dequantize), also when the loss
+    uses the scales of the encoding the output carries."""
+    from aimet_amd.quantization.affine import GroupedBlockQuantizeDequantize
+    from aimet_amd.quantization.affine.quantizer import GroupedBlockQuantizeDequantize as Cls
+
+    shape, block, grouping, wshape = case
+    g = torch.Generator().manual_seed(29)
+    w = torch.randn(wshape, generator=g) * 0.05
+    w.view(-1)[: w.numel() // 7] *= 30
+    q = GroupedBlockQuantizeDequantize(shape=shape, bitwidth=4, symmetric=True, decompressed_bw=8, block_size=block,
+                                       block_grouping=grouping).to(device)
+    with q.compute_encodings():
+        q(w.to(device) * 0.6)
+    q.to(param_dtype)
+    x = w.to(dtype)
+    grad = torch.randn(wshape, generator=g).to(dtype)
+    ws = torch.randn(shape, generator=g).to(device)
+
+    def run(through_encoding):
+        xd = x.to(device).requires_grad_(True)
+        q.min.grad = q.max.grad = None
+        out = q(xd)
+        loss = (out.as_subclass(torch.Tensor).float() * grad.to(device).float()).sum()
+        if through_encoding:
+            loss = loss + (out.encoding.scale * ws).sum() + out.encoding.per_channel_scale.sum()
+        loss.backward()
+        return (out.detach().as_subclass(torch.Tensor).clone(), xd.grad.clone(), q.min.grad.clone(), q.max.grad.clone(),
+                type(out.encoding.scale.grad_fn).__name__)
+
+    for through_encoding in (False, True):
+        one = run(through_encoding)
+        assert one[4].startswith("_LpbqQdqFromRange")
+        with monkeypatch.context() as m:
+            m.setattr(Cls, "_fused_forward", lambda self, input: None)
+            two = run(through_encoding)
+        assert two[4].startswith("_LpbqScale")
+        for a, b, what in zip(one[:4], two[:4], ("output", "input gradient", "gradient of min", "gradient of max")):
+            assert_same_bits(a, b, f"{what} (loss through the encoding: {through_encoding})")
+        assert float(one[2].abs().sum()) > 0 and float(one[3].abs().sum()) > 0
