@@ -54,8 +54,8 @@ MEASURED_TRAFFIC_BYTES = {
     # the timed update (a batch inside the running range): speculative binning pass (read + write) + the launch that
     # folds its extrema and partial histograms into the running state; a batch that moves the range is read a second
     # time (about a quarter of the batches of the c3 stream)
-    ("c3", "hist_update"): int((262288.0 + 3216.0 + 14862.3 + 3.5) * 1024),
-    ("dlq", "pdf_update"): int((262675.2 + 3072.0 + 6191.2 + 12.0) * 1024),
+    ("c3", "hist_update"): int((262285.2 + 3216.0 + 3370.9 + 3.5) * 1024),
+    ("dlq", "pdf_update"): int((262674.4 + 3072.0 + 3127.6 + 12.0) * 1024),
 }
 DTYPE_NAME = {torch.float32: "f32", torch.bfloat16: "bf16", torch.float16: "f16"}
 
