@@ -64,6 +64,25 @@ def test_argument_validation_without_a_gpu(lib):
     assert lib.ahq_minmax(0, lay, None, None, None, None, None, 0, None, 0, None) == 1
     assert lib.ahq_hist_update(0, lay, None, None, 1, None, 0, None) == 1
     assert lib.ahq_sqnr_search(None, None, None, None, None, None, None, None, None, None, None) == 1
+    # the fused LPBQ forward: validation, then the refusals that send a caller to the two-launch form
+    g.arith, g.op, g.io_dtype, g.compute_dtype, g.qmin, g.qmax = _lib.AHQ_ARITH_AUTOGRAD, 0, 0, 0, -8, 7
+    blocks = _lib.make_layout([4, 64], [1, 16], [4, 1])   # 4 x 4 blocks of 16 elements
+
+    def fused(grid, layout, group, mult=16):
+        return lib.ahq_lpbq_qdq_forward(grid, layout, 1, 1, None, 0, 1, 1, group, 1e-9, mult, None, 1, None, None)
+
+    assert lib.ahq_lpbq_qdq_forward(g, blocks, 1, 1, None, 0, None, 1, 4, 1e-9, 16, None, 1, None, None) == 1  # no min
+    assert fused(g, blocks, 0) == 1 and fused(g, blocks, 4, mult=0) == 1
+    assert fused(g, blocks, 3) == _lib.AHQ_ERR_UNSUPPORTED        # 16 blocks, groups of 3
+    g.compute_dtype = _lib.AHQ_F32
+    g.io_dtype = _lib.AHQ_BF16
+    assert fused(g, blocks, 4) == _lib.AHQ_ERR_UNSUPPORTED        # arithmetic in float32 on a 16-bit tensor
+    g.io_dtype = g.compute_dtype = 0
+    g.arith = _lib.AHQ_ARITH_ATEN
+    assert fused(g, blocks, 4) == _lib.AHQ_ERR_UNSUPPORTED
+    g.arith = _lib.AHQ_ARITH_AUTOGRAD
+    repeated = _lib.make_layout([3, 4, 64], [3, 1, 16], [0, 4, 1])
+    assert fused(g, repeated, 4) == _lib.AHQ_ERR_UNSUPPORTED      # encodings repeat over the leading dimension
 
 
 def test_workspace_queries_and_planning(lib):
@@ -207,6 +226,14 @@ def test_quantizer_construction_and_bookkeeping_on_cpu():
         GroupedBlockQuantizeDequantize((4, 2), 8, True, 4, None, (1, 8), (1, -1))
     with pytest.raises(TypeError):
         QuantizeDequantize((), 8, True, bogus=1)
+    # a group of LPBQ blocks is a run of neighbours in the scale array, or the one-launch forward does not apply
+    def per_group(shape, grouping):
+        return GroupedBlockQuantizeDequantize(shape, 4, True, 8, None, None, grouping)._blocks_per_group()
+
+    assert per_group((96, 8), (1, -1)) == 8 and per_group((96, 8), (1, 4)) == 4 and per_group((96, 8), (1, 1)) == 1
+    assert per_group((10, 64, 1, 1), (1, 64, 1, 1)) == 64 and per_group((4, 6, 8), (1, 3, -1)) == 24
+    assert per_group((8, 6), (2, 3)) is None and per_group((64, 10), (64, 1)) is None
+    assert per_group((1, 8), (-1, 4)) == 4
     sd = q.state_dict()
     q3 = QuantizeDequantize((3, 1), 8, True)
     q3.load_state_dict(sd)
