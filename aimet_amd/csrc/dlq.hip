@@ -174,7 +174,7 @@ __device__ __forceinline__ bool pdf_index(float v, float inv, float off, int& id
 // like: real activations put most elements into a few dozen buckets, and with few copies the wave's 64 atomic adds
 // pile onto a handful of banks and are replayed bank conflict by bank conflict.
 constexpr int kFfBins = 16;    // buckets per block of the single-slot partial counts
-constexpr int kPdfUnroll = 4;  // 16-byte loads in flight per lane: the workgroups are persistent, so this sets the bytes in flight
+constexpr int kPdfUnroll = 1;  // 16-byte loads in flight per lane: the workgroups are persistent, so this sets the bytes in flight
 
 template <typename IO, int VEC, int THREADS>
 __global__ __launch_bounds__(THREADS) void dlq_pdf_bin_kernel(const PdfBinArgs a) {

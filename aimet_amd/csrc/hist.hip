@@ -31,6 +31,7 @@ namespace ahq {
 constexpr int kHistBlocksMax = 1536;  // persistent workgroups of the binning pass (6 per CU)
 constexpr int kRng = 8;               // floats per slot in `ranges`
 constexpr int kPartBins = 8;          // entries per block of the single-slot partial counts
+constexpr int kHistBinU = 1;          // 16-byte vectors per lane and tile of the single-slot binning pass
 
 // ranges[slot]: lo1, hi1, thr_lo1, thr_hi1 (batch's own range), lo2, hi2, thr_lo2, thr_hi2 (updated range).
 // thr_* are the edges rounded to the tensor dtype: the reference compares `x < edge` in the tensor's dtype.
@@ -389,18 +390,37 @@ __global__ __launch_bounds__(kBlock, 6) void hist_bin_kernel(const BinArgs a) {
         }
     };
 
-    const int64_t full_tiles = a.nvec / kTileVec;
-    for (int64_t tile = blockIdx.x; tile < full_tiles; tile += gridDim.x) {
-        Pack<IO, VEC> in[kUnroll];
+    // Tiles of kBinU vectors per lane, software-pipelined with two register buffers used alternately: the next tile's
+    // loads are in flight while the current tile is binned, and no more than 2 * kBinU 16-byte loads per lane are
+    // outstanding (more in flight made this kernel slower, as they do the quantize-dequantize kernels).  The prefetch
+    // is unconditional, so the number of loads in flight is known at every wait; past the end it reads the tensor's
+    // first tile with ordinary loads (cache hits after the first workgroup) and the data is dropped.
+    constexpr int kBinU = kHistBinU;
+    constexpr int kBinVec = kBlock * kBinU;
+    const int64_t full_tiles = a.nvec / kBinVec;
+    auto load_tile = [&](Pack<IO, VEC>* buf, int64_t t, bool real) {
+        if (real) {
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u) in[u] = load_pack_stream<IO, VEC>(x + (tile * kTileVec + u * kBlock + threadIdx.x) * VEC);
+            for (int u = 0; u < kBinU; ++u) buf[u] = load_pack_stream<IO, VEC>(x + (t * kBinVec + u * kBlock + threadIdx.x) * VEC);
+        } else {
+#pragma unroll
+            for (int u = 0; u < kBinU; ++u) buf[u] = load_pack<IO, VEC>(x + (u * kBlock + threadIdx.x) * VEC);
+        }
+    };
+    auto bin_tile = [&](const Pack<IO, VEC>* in) {
         if (track_all) {
-            for (int u = 0; u < kUnroll; ++u)
-                for (int k = 0; k < VEC; ++k) track(load_f32(in[u].v[k]));
+            // (the empty asm keeps the elements' comparisons inside this rarely taken branch: hoisted above it they
+            // cost three instructions per element on every tile and spill the masks)
+            for (int u = 0; u < kBinU; ++u)
+                for (int k = 0; k < VEC; ++k) {
+                    float v = load_f32(in[u].v[k]);
+                    asm volatile("" : "+v"(v));
+                    track(v);
+                }
         }
         uint32_t binned = 0;  // this lane's elements that took the fast path
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
+        for (int u = 0; u < kBinU; ++u) {
 #pragma unroll
             for (int k = 0; k < VEC; ++k) {
                 const float v = load_f32(in[u].v[k]);
@@ -420,16 +440,31 @@ __global__ __launch_bounds__(kBlock, 6) void hist_bin_kernel(const BinArgs a) {
                 }
             }
         }
-        if (__builtin_amdgcn_ballot_w64(binned != (uint32_t)(kUnroll * VEC * NH)) != 0) {
-            for (int u = 0; u < kUnroll; ++u)
+        if (__builtin_amdgcn_ballot_w64(binned != (uint32_t)(kBinU * VEC * NH)) != 0) {
+            for (int u = 0; u < kBinU; ++u)
                 for (int k = 0; k < VEC; ++k) bin_slow(load_f32(in[u].v[k]), true);
+        }
+    };
+    {
+        Pack<IO, VEC> bufa[kBinU], bufb[kBinU];
+        const int64_t step = gridDim.x;
+        int64_t tile = blockIdx.x;
+        if (tile < full_tiles) load_tile(bufa, tile, true);
+        while (tile < full_tiles) {
+            load_tile(bufb, tile + step, tile + step < full_tiles);
+            bin_tile(bufa);
+            tile += step;
+            if (tile >= full_tiles) break;
+            load_tile(bufa, tile + step, tile + step < full_tiles);
+            bin_tile(bufb);
+            tile += step;
         }
     }
     // the ragged last tile
-    if (blockIdx.x == 0 && full_tiles * kTileVec < a.nvec) {
-        const int64_t v0 = full_tiles * kTileVec;
+    if (blockIdx.x == 0 && full_tiles * kBinVec < a.nvec) {
+        const int64_t v0 = full_tiles * kBinVec;
         const int nv = (int)(a.nvec - v0);
-        for (int u = 0; u < kUnroll; ++u) {
+        for (int u = 0; u < kBinU; ++u) {
             const int lv = u * kBlock + threadIdx.x;
             if (lv < nv) {
                 const Pack<IO, VEC> pk = load_pack_stream<IO, VEC>(x + (v0 + lv) * VEC);
@@ -890,7 +925,7 @@ bool make_hist_plan(int dtype, const ahq_layout& layout, const void* x, int num_
             hp->copies = copies;
         }
     }
-    hp->ntiles = (hp->plan.nvec + kTileVec - 1) / kTileVec;
+    hp->ntiles = (hp->plan.nvec + kBlock * kHistBinU - 1) / (kBlock * kHistBinU);
     int64_t nb = hp->fast ? hp->ntiles : (c.numel + kBlock - 1) / kBlock;
     if (nb > kHistBlocksMax) nb = kHistBlocksMax;
     if (nb < 1) nb = 1;
