@@ -212,8 +212,8 @@ __global__ __launch_bounds__(THREADS) void dlq_pdf_bin_kernel(const PdfBinArgs a
         if (pdf_index(v, inv, off, idx)) atomicAdd(reinterpret_cast<uint32_t*>(mine + ((uint32_t)idx << bshift)), 1u);
     };
     const int64_t full_tiles = a.nvec / kTile;
-    // software pipeline with two register buffers used alternately (no copies between them, which would force a full
-    // wait): the next tile's loads are in flight while the current tile is binned
+    // two register buffers used alternately, a tile's load issued one round ahead of its binning, one vector per lane
+    // and buffer: the shape and the reasons are those of the histogram's binning pass (hist_bin_kernel)
     Pack<IO, VEC> bufa[kPdfUnroll], bufb[kPdfUnroll];
     // `real` false: the prefetch past the end.  It reads the tensor's first tile with ordinary loads -- every
     // workgroup the same 64 KB, cache hits after the first -- where a streaming load of the current tile again was
