@@ -775,11 +775,13 @@ class QuantizeDequantize(AffineQuantizerBase):
         """The forward pass with learned min / max as one autograd node (_QdqFromRange); None when that does not
         apply (nothing learned, a subclass or a patched get_encodings(), another backend, tensors the library does
         not take, a grid that needs another compute dtype check) and the step-by-step form has to run."""
+        if not torch.is_grad_enabled():
+            return None
         from aimet_amd.quantization.affine.backends import get_backend, hip as _hip
 
         cls = type(self)
         mn, mx = self.min, self.max
-        if not (torch.is_grad_enabled() and (mn.requires_grad or mx.requires_grad)):
+        if not (mn.requires_grad or mx.requires_grad):
             return None
         if (cls.get_scale is not AffineQuantizerBase.get_scale or cls._get_offset is not AffineQuantizerBase._get_offset
                 or cls.get_encodings is not AffineQuantizerBase.get_encodings or "get_encodings" in self.__dict__
