@@ -641,10 +641,13 @@ __global__ __launch_bounds__(kBlock) void qdq_fwd_lpbq_kernel(const QdqArgs a, c
 
 // Encodings that change with every element (run length 1: per-channel along the fastest axis).  The tiled kernel
 // would prepare one encoding per element; here a lane owns VEC neighbouring encodings, prepares them once and walks
-// down the rows, so loads and stores stay coalesced 16-byte vectors.  A workgroup is 64 lanes across x kColWaves waves
-// down; each wave takes kColUnroll rows per step.
+// down the rows, so loads and stores stay coalesced 16-byte vectors.  A workgroup is 64 lanes across x a few waves
+// down; each wave takes kColUnroll rows per step.  kColWaves is the unit the grids are sized in (workgroups of sixteen
+// waves, the first shape); the kernels run with fewer waves per workgroup and correspondingly more workgroups, which
+// measured faster (forward 8192 x 4096 fp32: 43.6 us with sixteen waves, 40.8 us with four) and leaves a lane more
+// registers.
 constexpr int kColWaves = 16;
-constexpr int kColThreads = kWave * kColWaves;
+constexpr int kFwdColWaves = 4;
 constexpr int kColUnroll = 2;
 
 // the division-free form is allowed for this lane's VEC elements of one row
@@ -656,8 +659,8 @@ __device__ __forceinline__ bool row_can_divide_fast(const Pack<IO, VEC>& p) {
     return sum <= kFastDivMax;  // fails for NaN and infinity
 }
 
-template <typename IO, int VEC, typename M>
-__global__ __launch_bounds__(kColThreads) void qdq_fwd_cols_kernel(const QdqArgs a) {
+template <typename IO, int VEC, typename M, int WAVES>
+__global__ __launch_bounds__(WAVES * kWave) void qdq_fwd_cols_kernel(const QdqArgs a) {
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     const int64_t c0 = ((int64_t)blockIdx.x * kWave + lane) * VEC;
     if (c0 >= a.J) return;
@@ -670,8 +673,8 @@ __global__ __launch_bounds__(kColThreads) void qdq_fwd_cols_kernel(const QdqArgs
         e[k] = load_enc<M>(a, c0 + k);
         enc_fast &= !M::kDiv || e[k].rs != 0.f;
     }
-    const int64_t step = (int64_t)gridDim.y * kColWaves * kColUnroll;
-    for (int64_t r0 = ((int64_t)blockIdx.y * kColWaves + wave) * kColUnroll; r0 < a.I; r0 += step) {
+    const int64_t step = (int64_t)gridDim.y * WAVES * kColUnroll;
+    for (int64_t r0 = ((int64_t)blockIdx.y * WAVES + wave) * kColUnroll; r0 < a.I; r0 += step) {
         Pack<IO, VEC> in[kColUnroll];
         bool ok = enc_fast;
 #pragma unroll
@@ -1056,15 +1059,15 @@ __global__ __launch_bounds__(kBlock) void qdq_bwd_generic_kernel(const QdqArgs a
 // Backward for run length 1 (see qdq_fwd_cols_kernel): every lane keeps the sums of its VEC encodings over the rows
 // it walks, the waves of a workgroup add theirs up in LDS one after the other, and the workgroup's sums go to its own
 // row of the partials ([row group][encoding]), which qdq_bwd_strided_finish_kernel adds up in order.
-template <typename IO, int VEC, typename M>
-__global__ __launch_bounds__(kColThreads) void qdq_bwd_cols_kernel(const QdqArgs a) {
+template <typename IO, int VEC, typename M, int WAVES>
+__global__ __launch_bounds__(WAVES * kWave) void qdq_bwd_cols_kernel(const QdqArgs a) {
     __shared__ double sums[2 * VEC * kWave];
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     const int64_t c0 = ((int64_t)blockIdx.x * kWave + lane) * VEC;
     const bool live = c0 < a.J;
     const bool want_pg = a.partials != nullptr;
     if (want_pg) {
-        for (int i = threadIdx.x; i < 2 * VEC * kWave; i += kColThreads) sums[i] = 0.0;
+        for (int i = threadIdx.x; i < 2 * VEC * kWave; i += WAVES * kWave) sums[i] = 0.0;
         __syncthreads();
     }
     double acc_s[VEC], acc_o[VEC];
@@ -1081,8 +1084,8 @@ __global__ __launch_bounds__(kColThreads) void qdq_bwd_cols_kernel(const QdqArgs
             e[k] = load_enc<M>(a, c0 + k);
             enc_fast &= !M::kDiv || e[k].rs != 0.f;
         }
-        const int64_t step = (int64_t)gridDim.y * kColWaves * kColUnroll;
-        for (int64_t r0 = ((int64_t)blockIdx.y * kColWaves + wave) * kColUnroll; r0 < a.I; r0 += step) {
+        const int64_t step = (int64_t)gridDim.y * WAVES * kColUnroll;
+        for (int64_t r0 = ((int64_t)blockIdx.y * WAVES + wave) * kColUnroll; r0 < a.I; r0 += step) {
             Pack<IO, VEC> xin[kColUnroll], gin[kColUnroll];
             bool ok = enc_fast;
 #pragma unroll
@@ -1115,7 +1118,7 @@ __global__ __launch_bounds__(kColThreads) void qdq_bwd_cols_kernel(const QdqArgs
     }
     if (!want_pg) return;
     // the waves take turns, so the sums do not depend on which wave finishes first
-    for (int w = 0; w < kColWaves; ++w) {
+    for (int w = 0; w < WAVES; ++w) {
         if (wave == w && live) {
 #pragma unroll
             for (int k = 0; k < VEC; ++k) {
@@ -1192,10 +1195,10 @@ static bool cols_layout(const Plan& p, bool aligned) {
 // grid of the column-walking kernels: x over groups of 64 lanes x VEC encodings, y over row groups; about `target`
 // workgroups, every wave with at least one step of rows
 template <typename IO>
-static dim3 cols_grid(const Plan& p, int64_t target) {
+static dim3 cols_grid(const Plan& p, int64_t target, int waves = kColWaves) {
     constexpr int V = IoTraits<IO>::kVec;
     const int64_t gx = (p.cl.J / V + kWave - 1) / kWave;
-    const int64_t row_groups = (p.cl.I + (int64_t)kColWaves * kColUnroll - 1) / ((int64_t)kColWaves * kColUnroll);
+    const int64_t row_groups = (p.cl.I + (int64_t)waves * kColUnroll - 1) / ((int64_t)waves * kColUnroll);
     int64_t gy = (target + gx - 1) / gx;
     gy = gy < 1 ? 1 : (gy > row_groups ? row_groups : gy);
     if (gy > 65535) gy = 65535;
@@ -1206,7 +1209,9 @@ template <typename IO, typename M>
 static void launch_fwd(const Plan& p, const QdqArgs& a, hipStream_t st, bool aligned) {
     if (cols_layout<IO>(p, aligned) && (p.cl.J / IoTraits<IO>::kVec + kWave - 1) / kWave <= 0x7fffffff) {
         // a lane prepares kVec encodings before its first row: the more of them, the more rows it should walk
-        hipLaunchKernelGGL((qdq_fwd_cols_kernel<IO, IoTraits<IO>::kVec, M>), cols_grid<IO>(p, IoTraits<IO>::kVec > 4 ? 768 : 2048), dim3(kColThreads), 0, st, a);
+        constexpr int W = kFwdColWaves;
+        hipLaunchKernelGGL((qdq_fwd_cols_kernel<IO, IoTraits<IO>::kVec, M, W>),
+                           cols_grid<IO>(p, (IoTraits<IO>::kVec > 4 ? 768 : 2048) * (kColWaves / W), W), dim3(W * kWave), 0, st, a);
         return;
     }
     if (p.cl.kind == kGeneric) {
@@ -1228,8 +1233,20 @@ static bool bwd_cols_layout(int io_dtype, const Plan& p, bool aligned) {
     return io_dtype == AHQ_F32 ? bwd_cols_layout<float>(p, aligned) : bwd_cols_layout<f16_t>(p, aligned);
 }
 
+// The backward kernel keeps eight encodings, sixteen double sums and two rows of two tensors per lane on a 16-bit
+// tensor: more than the 128 registers a workgroup of sixteen waves leaves a lane (36 of them were spilled: 92 us on
+// 8192 x 4096 bf16 with learned encodings; 73 us with eight waves, 62 us with four, 71 us with two).  float32:
+// 73.6 us with sixteen waves, 69.5 us with eight, 72 us with four.
+template <typename IO>
+constexpr int bwd_cols_waves() { return IoTraits<IO>::kVec > 4 ? kColWaves / 4 : kColWaves / 2; }
+
+template <typename IO>
+static dim3 bwd_cols_grid(const Plan& p) {
+    return cols_grid<IO>(p, 512 * (kColWaves / bwd_cols_waves<IO>()), bwd_cols_waves<IO>());
+}
+
 static unsigned bwd_cols_row_groups(int io_dtype, const Plan& p) {
-    return io_dtype == AHQ_F32 ? cols_grid<float>(p, 512).y : cols_grid<f16_t>(p, 512).y;
+    return io_dtype == AHQ_F32 ? bwd_cols_grid<float>(p).y : bwd_cols_grid<f16_t>(p).y;
 }
 
 // pairs of doubles the backward pass needs as scratch for its parameter gradients
@@ -1252,7 +1269,8 @@ template <typename IO, typename M>
 static void launch_bwd(const Plan& p, const QdqArgs& a, hipStream_t st, bool aligned) {
     if (bwd_cols_layout<IO>(p, aligned)) {
         // few row groups: every workgroup ends with one row of partial sums
-        hipLaunchKernelGGL((qdq_bwd_cols_kernel<IO, IoTraits<IO>::kVec, M>), cols_grid<IO>(p, 512), dim3(kColThreads), 0, st, a);
+        constexpr int W = bwd_cols_waves<IO>();
+        hipLaunchKernelGGL((qdq_bwd_cols_kernel<IO, IoTraits<IO>::kVec, M, W>), bwd_cols_grid<IO>(p), dim3(W * kWave), 0, st, a);
         return;
     }
     if (p.cl.kind == kGeneric) {
