@@ -27,7 +27,7 @@ struct Geom {
     int64_t nvec;  // numel / VEC
     int64_t I, J, K;
     int64_t Kv;    // vectors per run of one encoding (K / VEC); 2^62 when J == 1
-    int32_t kv_shift;  // log2(Kv) when Kv is a power of two below the tile size, else -1
+    int32_t kv_shift;  // log2(Kv) when Kv is a power of two below 2^31, else -1
     int32_t tile_vec;  // vectors per tile: kBlock x (vectors per thread, at most kUnroll)
     int32_t mode;
     int32_t tpr;   // tiles per row (kRows); runs per tile (kRuns)
@@ -51,7 +51,7 @@ struct Tile {
 __device__ __forceinline__ Tile make_tile(const Geom& a, int64_t tile) {
     Tile t;
     if (a.mode == kRows) {
-        const int64_t row = tile / a.tpr;
+        const int64_t row = a.tpr == 1 ? tile : tile / a.tpr;  // (a 64-bit division costs a workgroup a few hundred instructions)
         const int64_t tt = tile - row * a.tpr;
         t.v0 = row * a.Kv + tt * a.tile_vec;
         const int64_t left = a.Kv - tt * a.tile_vec;
@@ -208,7 +208,7 @@ inline void fill_geom(const Plan& p, Geom* g) {
     g->Kv = p.Kv;
     g->kv_shift = -1;
     g->tile_vec = p.tile_vec;
-    if (p.Kv < p.tile_vec && is_pow2(p.Kv))
+    if (p.Kv < ((int64_t)1 << 31) && is_pow2(p.Kv))
         for (int b = 0; b < 31; ++b)
             if (((int64_t)1 << b) == p.Kv) g->kv_shift = b;
     g->mode = p.mode;
