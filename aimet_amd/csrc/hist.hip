@@ -13,6 +13,9 @@
 // Bin index formula = torch.histc on CPU:  pos = int64(((x - lo) * B) / (hi - lo)) in fp32, the top edge belongs to the
 // last bin, values outside [lo, hi] and NaN are not counted.
 
+
+#include <algorithm>
+
 #include "ahq_device.h"
 #include "ahq_host.h"
 #include "layout.h"
@@ -542,6 +545,125 @@ __global__ __launch_bounds__(kBlock, 6) void hist_bin_kernel(const BinArgs a) {
     }
 }
 
+// Single slot, 16-bit tensors, one histogram: binning through a table.  A 16-bit element has 65536 possible bit
+// patterns, and the bin of a pattern is the same for the whole batch, so each workgroup first fills a table in LDS --
+// pattern -> bin, or one of three further entries: below the range, above it, neither (NaN, or outside the float
+// range but not beyond the thresholds) -- with the exact reference arithmetic (128 KB of the compute unit's 160 KB),
+// and an element then costs one table read and one LDS add instead of the thirteen vector instructions of
+// hist_bin_kernel, which is what binds that kernel on 16-bit tensors (twice the elements per byte).  Workgroups of
+// 1024 threads, one per compute unit; partial counts leave in the layout of hist_bin_kernel.  SPEC as there: the
+// elements the table sends outside the range leave their finite extrema, looked at one by one (they are rare).
+constexpr int kLutThreads = 1024;
+constexpr int kLutEntries = 65536;
+constexpr size_t kLutBytes = (size_t)kLutEntries * 2;
+constexpr size_t kLdsMax = 160 * 1024;
+
+template <typename IO, int VEC, bool SPEC>
+__global__ __launch_bounds__(kLutThreads) void hist_bin16_kernel(const BinArgs a) {
+    extern __shared__ uint32_t lds[];
+    __shared__ float ext_smem[kLutThreads / kWave][2];
+    if (!SPEC && a.rebin && *a.rebin == 0) return;
+    uint16_t* lut = reinterpret_cast<uint16_t*>(lds);
+    uint32_t* cnt = lds + kLutBytes / 4;  // [B + 3][copies], lane l adds to copy l % copies
+    const int B = a.num_bins;
+    const float Bf = (float)B;
+    const int copies = a.copies, cshift = a.copy_shift;
+    for (int i = threadIdx.x; i < (B + 3) * copies; i += kLutThreads) cnt[i] = 0;
+    RangeC r;
+    float run_lo = 0.f, run_hi = 0.f, thr_min = 0.f, thr_max = 0.f;
+    bool track_all = false;
+    if (SPEC) {
+        run_lo = a.state_minmax[0];
+        run_hi = a.state_minmax[1];
+        const float rg[4] = {run_lo, run_hi, round_io<IO>(run_lo), round_io<IO>(run_hi)};
+        r = load_range(rg, 0);
+        thr_min = a.state_edges[0];
+        thr_max = a.state_edges[B];
+        track_all = (run_lo == run_hi) | (thr_max < run_hi) | (thr_min > run_lo);
+    } else {
+        r = load_range(a.ranges, 0);
+    }
+    auto value_of = [](uint32_t pattern) {
+        IO v;
+        v.bits = (uint16_t)pattern;
+        return load_f32(v);
+    };
+    for (int p = threadIdx.x; p < kLutEntries; p += kLutThreads) {
+        const float v = value_of((uint32_t)p);
+        int e;
+        if ((v >= r.lo) & (v <= r.hi)) e = bin_exact(v, r, Bf, B);
+        else e = v < r.thr_lo ? B : (v > r.thr_hi ? B + 1 : B + 2);
+        lut[p] = (uint16_t)e;
+    }
+    __syncthreads();
+    float ext_min = __builtin_inff(), ext_max = -__builtin_inff();
+    auto track = [&](float v) {  // finite elements beyond the outermost edges (see hist_bin_kernel)
+        const bool fin = __builtin_fabsf(v) < __builtin_inff();
+        ext_min = fminf(ext_min, (fin & (v < thr_min)) ? v : __builtin_inff());
+        ext_max = fmaxf(ext_max, (fin & (v > thr_max)) ? v : -__builtin_inff());
+    };
+    uint32_t* mine = cnt + (threadIdx.x & (copies - 1));
+    uint32_t zeros = 0;   // exact zeros are counted here and added once (they would all meet in one LDS word)
+    bool outside = false;  // SPEC: this lane met an element the table sent outside the range
+    const bool zero_outside = lut[0] >= (uint32_t)B;
+    auto count = [&](uint32_t pattern) {
+        if ((pattern & 0x7fffu) == 0) {
+            ++zeros;
+            if (SPEC) outside |= zero_outside;
+        } else {
+            const uint32_t e = lut[pattern];
+            atomicAdd(mine + (e << cshift), 1u);
+            if (SPEC) outside |= e >= (uint32_t)B;
+        }
+    };
+    const IO* __restrict__ x = static_cast<const IO*>(a.x);
+    const int64_t full_tiles = a.nvec / kLutThreads;
+    for (int64_t tile = blockIdx.x; tile < full_tiles; tile += gridDim.x) {
+        const Pack<IO, VEC> in = load_pack_stream<IO, VEC>(x + (tile * kLutThreads + threadIdx.x) * VEC);
+        outside = false;
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) count(in.v[k].bits);
+        if (SPEC && (track_all || __builtin_amdgcn_ballot_w64(outside) != 0)) {
+            for (int k = 0; k < VEC; ++k) track(load_f32(in.v[k]));
+        }
+    }
+    if (blockIdx.x == 0) {  // the vectors past the last full tile and the elements past the last full vector
+        for (int64_t i = full_tiles * kLutThreads * VEC + threadIdx.x; i < a.numel; i += kLutThreads) {
+            count(x[i].bits);
+            if (SPEC) track(load_f32(x[i]));
+        }
+    }
+    if (zeros != 0) atomicAdd(mine + ((uint32_t)lut[0] << cshift), zeros);
+    if (SPEC) {
+#pragma unroll
+        for (int m = kWave / 2; m >= 1; m >>= 1) {
+            ext_min = fminf(ext_min, __shfl_xor(ext_min, m, kWave));
+            ext_max = fmaxf(ext_max, __shfl_xor(ext_max, m, kWave));
+        }
+        if ((threadIdx.x & (kWave - 1)) == 0) {
+            ext_smem[threadIdx.x / kWave][0] = ext_min;
+            ext_smem[threadIdx.x / kWave][1] = ext_max;
+        }
+    }
+    __syncthreads();
+    if (SPEC && threadIdx.x == 0) {
+        float mn = ext_smem[0][0], mx = ext_smem[0][1];
+        for (int wv = 1; wv < kLutThreads / kWave; ++wv) {
+            mn = fminf(mn, ext_smem[wv][0]);
+            mx = fmaxf(mx, ext_smem[wv][1]);
+        }
+        a.part_min[blockIdx.x] = mn;
+        a.part_max[blockIdx.x] = mx;
+    }
+    // partial counts in the layout hist_bin_kernel leaves them in: entries 0..B-1 the bins, B below, B + 1 above
+    const size_t np = gridDim.x;
+    for (int e = threadIdx.x; e < B + 2; e += kLutThreads) {
+        uint32_t c = 0;
+        for (int cp = 0; cp < copies; ++cp) c += cnt[((size_t)e << cshift) + cp];
+        a.partials[(((size_t)(e / kPartBins)) * np + blockIdx.x) * kPartBins + e % kPartBins] = c;
+    }
+}
+
 // Several slots whose runs are long enough that a tile lies inside one run (per-channel weights, per-channel
 // activations with large feature maps): one workgroup per tile bins into LDS sub-histograms of its slot and adds the
 // non-empty bins to the slot's zero-initialised counters in global memory.
@@ -1003,6 +1125,42 @@ extern "C" int ahq_hist_update(int32_t dtype, const ahq_layout* layout, const vo
     uint32_t* counts = reinterpret_cast<uint32_t*>(w + hp.off_counts);
     int32_t* rebin = reinterpret_cast<int32_t*>(w + hp.off_rebin);
 
+    // 16-bit tensors, one histogram: the binning kernel that looks the bin up in a table (hist_bin16_kernel)
+    int lut_copies = 0;
+    if (hp.fast && NH == 1 && dtype != AHQ_F32) {
+        const size_t room = kLdsMax - kLutBytes - 1024;
+        for (int c2 = 8; c2 >= 1 && lut_copies == 0; c2 >>= 1)
+            if ((size_t)c2 * (B + 3) * 4 <= room) lut_copies = c2;
+    }
+    const int lut_blocks = lut_copies > 0 ? (int)std::min<int64_t>(std::max<int64_t>(hp.plan.nvec / kLutThreads, 1), std::min(256, hp.nblocks)) : 0;
+    auto launch_lut = [&](BinArgs args, bool spec) {
+        args.copies = lut_copies;
+        args.copy_shift = 0;
+        while ((1 << args.copy_shift) < lut_copies) ++args.copy_shift;
+        const size_t lds = kLutBytes + (size_t)lut_copies * (B + 3) * 4;
+        const dim3 g(lut_blocks), b(kLutThreads);
+#define AHQ_LAUNCH_LUT_K(K)                                                                                         \
+    do {                                                                                                            \
+        hipFuncSetAttribute(reinterpret_cast<const void*>(&K), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
+        hipLaunchKernelGGL(K, g, b, lds, s, args);                                                                  \
+    } while (0)
+#define AHQ_LAUNCH_LUT(IO)                                                                                          \
+    do {                                                                                                            \
+        if (hp.plan.vec == 1) {                                                                                     \
+            if (spec) AHQ_LAUNCH_LUT_K((hist_bin16_kernel<IO, 1, true>));                                           \
+            else AHQ_LAUNCH_LUT_K((hist_bin16_kernel<IO, 1, false>));                                               \
+        } else {                                                                                                    \
+            if (spec) AHQ_LAUNCH_LUT_K((hist_bin16_kernel<IO, 8, true>));                                           \
+            else AHQ_LAUNCH_LUT_K((hist_bin16_kernel<IO, 8, false>));                                               \
+        }                                                                                                           \
+    } while (0)
+        if (dtype == AHQ_F16) AHQ_LAUNCH_LUT(f16_t);
+        else AHQ_LAUNCH_LUT(bf16_t);
+#undef AHQ_LAUNCH_LUT
+#undef AHQ_LAUNCH_LUT_K
+    };
+    const int bin_blocks = lut_copies > 0 ? lut_blocks : hp.nblocks;  // partial histograms the binning pass leaves
+
     // 1. finite range of the batch, in the tensor's dtype
     const float *part_min = nullptr, *part_max = nullptr;
     int64_t nparts = 0;
@@ -1011,7 +1169,7 @@ extern "C" int ahq_hist_update(int32_t dtype, const ahq_layout* layout, const vo
         ba.state_minmax = st->minmax;
         ba.state_edges = st->edges;
         ba.part_min = reinterpret_cast<float*>(w + hp.off_mm_ws);
-        ba.part_max = ba.part_min + hp.nblocks;
+        ba.part_max = ba.part_min + bin_blocks;
         const size_t lds = (size_t)hp.copies * B * 4;
         const dim3 g(hp.nblocks), b(kBlock);
 #define AHQ_LAUNCH_SPEC(IO)                                                                                         \
@@ -1019,15 +1177,19 @@ extern "C" int ahq_hist_update(int32_t dtype, const ahq_layout* layout, const vo
         if (hp.plan.vec == 1) hipLaunchKernelGGL((hist_bin_kernel<IO, 1, 1, true>), g, b, lds, s, ba);              \
         else hipLaunchKernelGGL((hist_bin_kernel<IO, IoTraits<IO>::kVec, 1, true>), g, b, lds, s, ba);              \
     } while (0)
-        switch (dtype) {
-            case AHQ_F32: AHQ_LAUNCH_SPEC(float); break;
-            case AHQ_F16: AHQ_LAUNCH_SPEC(f16_t); break;
-            default: AHQ_LAUNCH_SPEC(bf16_t); break;
+        if (lut_copies > 0) {
+            launch_lut(ba, true);
+        } else {
+            switch (dtype) {
+                case AHQ_F32: AHQ_LAUNCH_SPEC(float); break;
+                case AHQ_F16: AHQ_LAUNCH_SPEC(f16_t); break;
+                default: AHQ_LAUNCH_SPEC(bf16_t); break;
+            }
         }
 #undef AHQ_LAUNCH_SPEC
         part_min = ba.part_min;
         part_max = ba.part_max;
-        nparts = hp.nblocks;
+        nparts = bin_blocks;
         ba.rebin = rebin;  // for the second pass
     } else {
         int rc = ahq_minmax_finite_partials(dtype, layout, x, w + hp.off_bmin, w + hp.off_bmax, w + hp.off_mm_ws,
@@ -1065,7 +1227,7 @@ extern "C" int ahq_hist_update(int32_t dtype, const ahq_layout* layout, const vo
         // the counts of the speculative pass, folded straight into the running histogram if the range holds
         fa.nhist = 1;
         fa.first = 0;
-        fa.nparts = hp.nblocks;
+        fa.nparts = bin_blocks;
         fa.counts = counts;
         fa.carried = st->hist;
         fa.hist = st->hist;
@@ -1099,10 +1261,14 @@ extern "C" int ahq_hist_update(int32_t dtype, const ahq_layout* layout, const vo
             else hipLaunchKernelGGL((hist_bin_kernel<IO, IoTraits<IO>::kVec, 2>), g, b, lds, s, ba);                \
         }                                                                                                           \
     } while (0)
-        switch (dtype) {
-            case AHQ_F32: AHQ_LAUNCH_BIN(float); break;
-            case AHQ_F16: AHQ_LAUNCH_BIN(f16_t); break;
-            default: AHQ_LAUNCH_BIN(bf16_t); break;
+        if (lut_copies > 0) {
+            launch_lut(ba, false);
+        } else {
+            switch (dtype) {
+                case AHQ_F32: AHQ_LAUNCH_BIN(float); break;
+                case AHQ_F16: AHQ_LAUNCH_BIN(f16_t); break;
+                default: AHQ_LAUNCH_BIN(bf16_t); break;
+            }
         }
 #undef AHQ_LAUNCH_BIN
     } else {
@@ -1141,7 +1307,7 @@ extern "C" int ahq_hist_update(int32_t dtype, const ahq_layout* layout, const vo
     // 4. counts -> fp32 statistics
     fa.nhist = NH;
     fa.first = first_batch ? 1 : 0;
-    fa.nparts = hp.fast ? hp.nblocks : 1;
+    fa.nparts = hp.fast ? bin_blocks : 1;
     fa.counts = counts;
     fa.carried = pa.carried;
     fa.upd_edges = pa.upd_edges;
