@@ -133,6 +133,7 @@ _SIGNATURES = {
                                             _P, ctypes.c_int64, ctypes.c_double, ctypes.c_int32, _P, _P, _P, _P]),
     "ahq_grid_probe": (ctypes.c_int, [ctypes.c_int32, ctypes.POINTER(Layout), _P, ctypes.c_int64, _P, _P]),
     "ahq_hist_update_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int32, ctypes.POINTER(Layout), ctypes.c_int32]),
+    "ahq_hist_table_min_numel": (ctypes.c_int64, [ctypes.c_int64]),
     "ahq_hist_update": (ctypes.c_int, [ctypes.c_int32, ctypes.POINTER(Layout), _P, ctypes.POINTER(HistState),
                                        ctypes.c_int, _P, ctypes.c_size_t, _P]),
     "ahq_sqnr_search": (ctypes.c_int, [ctypes.POINTER(SqnrParams), _P, _P, _P, _P, _P, _P, _P, _P, _P, _P]),

@@ -311,6 +311,14 @@ size_t ahq_hist_update_workspace_bytes(int32_t dtype, const ahq_layout* layout, 
 int    ahq_hist_update(int32_t dtype, const ahq_layout* layout, const void* x, const ahq_hist_state* state,
                        int first_batch, void* workspace, size_t workspace_bytes, void* stream);
 
+/* No counterpart in the reference: a tuning knob of ahq_hist_update.  A single-slot update of a 16-bit tensor that
+ * forms one histogram is binned through a 64K-entry table in LDS once the tensor has at least this many elements
+ * (default 48 Mi; below it filling the table costs more than it saves), and arithmetically below.  Both ways give the
+ * same counts.  set >= 0 replaces the threshold (0: always the table), set < 0 only reads it; returns the value that
+ * was in force before the call.  Process-wide.
+ */
+int64_t ahq_hist_table_min_numel(int64_t set);
+
 /* ---------------------------------------------------------------- SQNR / TF-enhanced search ------------------------
  * Replaces: _LpNormEncodingAnalyzer._pick_test_candidates / _clamp_delta_offset_values /
  * _estimate_clip_and_quant_noise / _select_best_candidates (encoding_analyzer.py:728-899).

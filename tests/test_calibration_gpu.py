@@ -166,6 +166,70 @@ def test_histogram_update_with_and_without_the_batch_histogram(device, case):
             assert_same_bits(only._state["hist"][s_], r.histogram, f"running histogram after batch {k} slot {s_}")
 
 
+@pytest.fixture
+def table_binning():
+    """Route every eligible 16-bit histogram update through the table kernel, whatever the tensor's size."""
+    from aimet_amd import _lib
+
+    lib = _lib.load()
+    before = lib.ahq_hist_table_min_numel(0)
+    yield
+    lib.ahq_hist_table_min_numel(before)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=lambda d: str(d).split(".")[-1])
+@pytest.mark.parametrize("num_bins", [512, 2048, 7, 5000])
+@pytest.mark.parametrize("numel", [8 * 1024 * 37 + 13, 1024 * 8, 1001, 5], ids=lambda n: f"n{n}")
+def test_histogram_of_16_bit_tensors_through_the_table(device, table_binning, dtype, num_bins, numel):
+    """Running statistics only, one slot, 16-bit elements: the kernel that looks bins up in a 64K-entry table.  Batches
+    inside the running range (binned speculatively), beyond it on either side (binned again), with zeros of both signs,
+    infinities and NaN, with and without a ragged tail; counts, edges and min/max bit-exact against the oracle, and
+    the same with the table switched off."""
+    from aimet_amd import _lib
+    from aimet_amd.quantization.encoding_analyzer import _HistogramObserver
+
+    table = _HistogramObserver((1,), num_bins=num_bins)
+    arith = _HistogramObserver((1,), num_bins=num_bins)
+    ref = O.HistObserver((1,), num_bins, None)
+    g = torch.Generator().manual_seed(numel + num_bins)
+    scales = [(1.0, 0.0), (0.5, 0.1), (3.0, 0.0), (1.0, -9.0), (0.2, 0.0), (1.0, 0.0)]
+    lib = _lib.load()
+    for k, (s_, shift) in enumerate(scales):
+        x = torch.randn(numel, generator=g) * s_ + shift
+        if k == 4:
+            x = torch.relu(x)
+            x[::5] = -0.0
+        if k == 5 and numel >= 5:
+            x[0], x[1], x[-1] = float("inf"), float("nan"), -float("inf")
+        x = x.to(dtype)
+        ref.update(x)
+        xd = x.to(device)
+        for obs, threshold in ((table, 0), (arith, 1 << 62)):
+            if obs._state is None:
+                obs._state = obs._alloc(xd.device)
+            lib.ahq_hist_table_min_numel(threshold)
+            obs._run(xd, obs._state, first=(k == 0), batch_hist=False, batch_stats=False)
+        lib.ahq_hist_table_min_numel(0)
+        for key in ("hist", "edges", "minmax", "limits"):
+            assert_same_bits(table._state[key], arith._state[key], f"running {key} after batch {k}")
+        r = ref.stats[0]
+        assert_same_bits(table._state["hist"][0], r.histogram, f"running histogram after batch {k}")
+        assert_same_bits(table._state["edges"][0], r.bin_edges, f"running edges after batch {k}")
+        assert table._state["minmax"][0, 0].item() == r.min.float().item()
+        assert table._state["minmax"][0, 1].item() == r.max.float().item()
+
+
+def test_table_threshold_knob(device):
+    from aimet_amd import _lib
+
+    lib = _lib.load()
+    default = lib.ahq_hist_table_min_numel(-1)
+    assert default == 48 << 20
+    assert lib.ahq_hist_table_min_numel(123) == default
+    assert lib.ahq_hist_table_min_numel(-1) == 123
+    assert lib.ahq_hist_table_min_numel(default) == 123
+
+
 @pytest.mark.parametrize("case", ["nested", "straddle"])
 def test_histogram_merge_closed_forms(device, case):
     """The merges whose result is known by hand (tests/helpers.py), on the HIP path."""
