@@ -638,9 +638,37 @@ def run_hist_workload(steps, warmup, dev, with_cpu_baseline=True, batches=16, sh
     bytes_read_once = 4 * n_b
     traffic_upd = MEASURED_TRAFFIC_BYTES[("c3", "hist_update")]
 
+    # the same stream in bf16: twice the elements per byte, and an update that holds the range bins them through a
+    # table in LDS (hist_bin16_kernel) instead of computing each element's bin
+    xs16 = [x.bfloat16() for x in xs[:4]]
+    an16 = SqnrEncodingAnalyzer((1,), num_bins=512, asymmetric_delta_candidates=100, offset_candidates=64, gamma=3.0)
+    for x in xs16[:2]:
+        an16.update_stats(x)
+    st16 = an16.observer.get_stats()[0]
+    hist16_gpu, edges16_gpu = st16.histogram.cpu().clone(), st16.bin_edges.cpu().clone()
+    for x in xs16[2:] + xs16:
+        an16.update_stats(x)
+    turn16 = [0]
+
+    def update_next16():
+        turn16[0] = (turn16[0] + 1) % len(xs16)
+        an16.update_stats(xs16[turn16[0]])
+
+    t_upd16 = event_time(update_next16, 20)
+    bf16_stream = {"update_us": round(t_upd16 * 1e6, 2), "GBps_one_read": round(2 * n_b / t_upd16 / 1e9, 1),
+                   "elements_per_s": round(n_b / t_upd16, 1), "kernel": "hist_bin16_kernel<SPEC>",
+                   "sample": "the first 4 batches rounded to bf16, in turn"}
+
     parity = {"sample": "not compared (CPU leg switched off)"}
     cpu_all = cpu_one = None
     if with_cpu_baseline:
+        ref16 = O.HistObserver((1,), 512)
+        for xb in xs16[:2]:
+            ref16.update(xb.cpu())
+        bf16_stream["parity"] = {"hist_bit_exact": bool(torch.equal(hist16_gpu, ref16.stats[0].histogram)),
+                                 "edges_bit_exact": bool(torch.equal(edges16_gpu, ref16.stats[0].bin_edges)),
+                                 "sample": "after 2 batches"}
+        del ref16
         # the CPU leg: the whole 16-batch step, one batch on the host at a time; its result is the parity reference
         ref_all = O.HistObserver((1,), 512)
         cpu_dt = 0.0
@@ -696,6 +724,7 @@ def run_hist_workload(steps, warmup, dev, with_cpu_baseline=True, batches=16, sh
                     "sqnr_search(api)": {"us": round(t_search * 1e6, 2), "candidates": 6400, "bins": 512}},
         "encoding": {"min": float(lo.item()), "max": float(hi.item())},
         "parity": parity,
+        "bf16_stream": bf16_stream,
         "roofline": {"bound": "hbm", "kernel": "hist_bin_kernel<SPEC> inside one histogram update (4 launches timed together)",
                      "achieved": round(traffic_upd / t_upd / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(traffic_upd / t_upd / 1e9 / HBM_PEAK_GBS, 4), "algorithmic_bytes": bytes_read_once,
@@ -710,7 +739,7 @@ def run_hist_workload(steps, warmup, dev, with_cpu_baseline=True, batches=16, sh
     if cpu_all is not None:
         out["cpu_baseline"], out["cpu_baseline_1thread"] = cpu_all, cpu_one
     out["bench_seconds"] = round(time.perf_counter() - t_start, 1)
-    del xs
+    del xs, xs16
     return out
 
 
