@@ -125,6 +125,14 @@ _SIGNATURES = {
                                            ctypes.c_float, ctypes.c_float, ctypes.c_float, ctypes.c_float, _P,
                                            ctypes.c_int32, _P, _P, ctypes.c_int64, ctypes.c_int64, ctypes.c_double, _P,
                                            _P, _P]),
+    "ahq_minmax_slots_finalize": (ctypes.c_int, [ctypes.c_int32, _P, ctypes.c_int64, ctypes.c_int32, ctypes.c_float,
+                                                 ctypes.c_float, ctypes.c_float, ctypes.c_float, _P, ctypes.c_int32, _P,
+                                                 _P, ctypes.c_int64, ctypes.c_int64, ctypes.c_double, _P, _P, _P]),
+    "ahq_minmax_calibrate_qdq_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int32, ctypes.POINTER(Layout)]),
+    "ahq_minmax_calibrate_qdq": (ctypes.c_int, [ctypes.POINTER(Grid), ctypes.POINTER(Layout), _P, _P, ctypes.c_int64,
+                                                ctypes.c_int32, ctypes.c_float, ctypes.c_float, ctypes.c_float,
+                                                ctypes.c_float, _P, ctypes.c_int32, _P, _P, ctypes.c_double, _P, _P, _P,
+                                                ctypes.c_size_t, _P]),
     "ahq_range_to_scale_offset": (ctypes.c_int, [ctypes.c_int32, _P, _P, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
                                                  ctypes.c_double, _P, _P, _P]),
     "ahq_lpbq_scale": (ctypes.c_int, [ctypes.c_int32, ctypes.POINTER(Layout), _P, _P, ctypes.c_int64, ctypes.c_int64,

@@ -175,11 +175,61 @@ struct FinalArgs {
 };
 
 template <typename T, typename P>
+__device__ __forceinline__ void finalize_one(const EncArgs& a, const FinalArgs& f, int64_t i, float smin, float smax);
+
+template <typename T, typename P>
 __global__ void minmax_finalize_kernel(const EncArgs a, const FinalArgs f) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= a.n) return;
+    finalize_one<T, P>(a, f, i, load_f32(static_cast<const T*>(a.smin)[i]), load_f32(static_cast<const T*>(a.smax)[i]));
+}
+
+// The same for a single encoding whose running extrema still lie in the slots of ahq_minmax_accumulate (min, max and
+// a NaN flag per workgroup of that kernel): one workgroup folds the slots the way ahq_minmax_slots_read does -- a
+// NaN seen anywhere makes both statistics NaN, as torch.amin / amax would -- and its first thread goes on.
+constexpr int kSlotThreads = 256;
+
+template <typename T, typename P>
+__global__ __launch_bounds__(kSlotThreads) void minmax_slots_finalize_kernel(const float* slot_min, const float* slot_max,
+                                                                             const int* slot_nan, const EncArgs a,
+                                                                             const FinalArgs f) {
+    __shared__ float red[kSlotThreads / kWave][2];
+    __shared__ int red_nan[kSlotThreads / kWave];
+    float mn = __builtin_inff(), mx = -__builtin_inff();
+    int nan = 0;
+    for (int q = threadIdx.x; q < AHQ_MINMAX_SLOTS; q += kSlotThreads) {
+        mn = fminf(mn, slot_min[q]);
+        mx = fmaxf(mx, slot_max[q]);
+        nan |= slot_nan[q];
+    }
+#pragma unroll
+    for (int m = kWave / 2; m >= 1; m >>= 1) {
+        mn = fminf(mn, __shfl_xor(mn, m, kWave));
+        mx = fmaxf(mx, __shfl_xor(mx, m, kWave));
+        nan |= __shfl_xor(nan, m, kWave);
+    }
+    if ((threadIdx.x & (kWave - 1)) == 0) {
+        red[threadIdx.x / kWave][0] = mn;
+        red[threadIdx.x / kWave][1] = mx;
+        red_nan[threadIdx.x / kWave] = nan;
+    }
+    __syncthreads();
+    if (threadIdx.x != 0) return;
+    for (int w = 1; w < kSlotThreads / kWave; ++w) {
+        mn = fminf(mn, red[w][0]);
+        mx = fmaxf(mx, red[w][1]);
+        nan |= red_nan[w];
+    }
+    const float qnan = __builtin_nanf("");
+    // the statistics as the fold would have stored them: values of the tensor's dtype
+    finalize_one<T, P>(a, f, 0, load_f32(store_cast<T>(nan ? qnan : mn)), load_f32(store_cast<T>(nan ? qnan : mx)));
+}
+
+template <typename T, typename P>
+__device__ __forceinline__ void finalize_one(const EncArgs& a, const FinalArgs& f, const int64_t i, const float smin,
+                                             const float smax) {
     T lo_t, hi_t;
-    encode_range<T>(a, load_f32(static_cast<const T*>(a.smin)[i]), load_f32(static_cast<const T*>(a.smax)[i]), lo_t, hi_t);
+    encode_range<T>(a, smin, smax, lo_t, hi_t);
     const P lo_p = store_cast<P>(load_f32(lo_t)), hi_p = store_cast<P>(load_f32(hi_t));
     static_cast<P*>(f.pmin)[i] = lo_p;
     static_cast<P*>(f.pmax)[i] = hi_p;
@@ -675,4 +725,53 @@ extern "C" int ahq_minmax_finalize(int32_t stat_dtype, const void* stat_min, con
         default: launch_finalize<bf16_t>(param_dtype, g, b, s, a, f); break;
     }
     return check_launch("minmax_finalize");
+}
+
+template <typename T>
+static void launch_slots_finalize(int32_t param_dtype, hipStream_t s, const float* mn, const float* mx, const int* nan,
+                                  const EncArgs& a, const FinalArgs& f) {
+    const dim3 g(1), b(kSlotThreads);
+    switch (param_dtype) {
+        case AHQ_F32: hipLaunchKernelGGL((minmax_slots_finalize_kernel<T, float>), g, b, 0, s, mn, mx, nan, a, f); break;
+        case AHQ_F16: hipLaunchKernelGGL((minmax_slots_finalize_kernel<T, f16_t>), g, b, 0, s, mn, mx, nan, a, f); break;
+        default: hipLaunchKernelGGL((minmax_slots_finalize_kernel<T, bf16_t>), g, b, 0, s, mn, mx, nan, a, f); break;
+    }
+}
+
+extern "C" int ahq_minmax_slots_finalize(int32_t stat_dtype, const void* slots, int64_t num_steps, int32_t symmetric,
+                                         float minimum_scale_in_dtype, float minimum_scale, float dtype_max,
+                                         float near_max_threshold, int32_t* flags, int32_t param_dtype, void* param_min,
+                                         void* param_max, int64_t qmin, int64_t qmax, double grid_minimum_scale,
+                                         float* scale, float* offset, void* stream) {
+    if (!slots || (reinterpret_cast<uintptr_t>(slots) & 3u)) return set_error("slots is null or misaligned"), AHQ_ERR_INVALID;
+    EncArgs a{};
+    const int rc = fill_enc_args(&a, stat_dtype, slots, slots, 1, num_steps, symmetric, minimum_scale_in_dtype,
+                                 minimum_scale, dtype_max, near_max_threshold, flags);
+    if (rc != AHQ_OK) return rc;
+    if (param_dtype < AHQ_F32 || param_dtype > AHQ_BF16) return set_error("bad parameter dtype"), AHQ_ERR_INVALID;
+    if (!param_min || !param_max || !scale) return set_error("null argument"), AHQ_ERR_INVALID;
+    if (qmin >= qmax) return set_error("qmax must be larger than qmin"), AHQ_ERR_INVALID;
+    a.smin = a.smax = nullptr;  // the statistics come from the slots
+    FinalArgs f{};
+    f.pmin = param_min;
+    f.pmax = param_max;
+    f.so.scale = scale;
+    f.so.offset = offset;
+    f.so.n = 1;
+    f.so.num_steps = (float)(double)(qmax - qmin);
+    f.so.minimum_scale = (float)grid_minimum_scale;
+    f.so.qmin = (float)(double)qmin;
+    f.so.lo = (float)(double)(-qmax);
+    f.so.hi = (float)(double)(-qmin);
+    const char* w = static_cast<const char*>(slots);
+    const float* mn = reinterpret_cast<const float*>(w);
+    const float* mx = reinterpret_cast<const float*>(w + 4 * AHQ_MINMAX_SLOTS);
+    const int* nan = reinterpret_cast<const int*>(w + 8 * AHQ_MINMAX_SLOTS);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    switch (stat_dtype) {
+        case AHQ_F32: launch_slots_finalize<float>(param_dtype, s, mn, mx, nan, a, f); break;
+        case AHQ_F16: launch_slots_finalize<f16_t>(param_dtype, s, mn, mx, nan, a, f); break;
+        default: launch_slots_finalize<bf16_t>(param_dtype, s, mn, mx, nan, a, f); break;
+    }
+    return check_launch("minmax_slots_finalize");
 }

@@ -140,8 +140,10 @@ class QuantizedLinear(nn.Linear):
                 out[name] = _may_be_prequantized(param.detach(), qtzr)
         return out
 
-    def _compute_param_encodings(self, overwrite: bool, verdicts=None):
-        """nn/base.py:331-383.  ``verdicts``: already read-back results of _prequantized_verdicts()."""
+    def _compute_param_encodings(self, overwrite: bool, verdicts=None, quantized=None):
+        """nn/base.py:331-383.  ``verdicts``: already read-back results of _prequantized_verdicts().  ``quantized``:
+        a dictionary that receives, by name, the quantize-dequantized parameters that came out of the calibration
+        itself (one library call for both, where the quantizer offers it), for a caller that wants them next."""
         todo = list(self._params_to_calibrate(overwrite))
         if not todo:
             return
@@ -161,16 +163,21 @@ class QuantizedLinear(nn.Linear):
                         qtzr.set_range(scale * qtzr.qmin, scale * qtzr.qmax)
                     continue
             if isinstance(qtzr, AffineQuantizerBase):
-                qtzr._calibrate_on(param)  # pylint: disable=protected-access
+                fused = getattr(qtzr, "_calibrate_and_quantize", None) if quantized is not None else None
+                out = fused(param) if fused is not None else None
+                if out is not None:
+                    quantized[name] = out
+                else:
+                    qtzr._calibrate_on(param)  # pylint: disable=protected-access
             else:
                 with qtzr._compute_encodings(passthrough=True):  # pylint: disable=protected-access
                     _ = qtzr(param)
             if getattr(qtzr, "encoding_analyzer", None) is not None:
                 qtzr.encoding_analyzer.reset_stats()  # nn/base.py:385-386
 
-    def _patch_quantized_parameters(self, param_names: Optional[Iterable[str]] = None):
+    def _patch_quantized_parameters(self, param_names: Optional[Iterable[str]] = None, _quantized=None):
         """nn/base.py:296-324: a context in which the named parameters (all by default) hold their
-        quantize-dequantized values, computed once on entry."""
+        quantize-dequantized values, computed once on entry (``_quantized``: those already at hand, by name)."""
         names = self.param_quantizers.keys() if param_names is None else param_names
         stack = contextlib.ExitStack()
         for name in names:
@@ -178,7 +185,9 @@ class QuantizedLinear(nn.Linear):
             param = getattr(self, name)
             if qtzr is None or param is None:
                 continue
-            if qtzr.is_initialized():
+            if _quantized and name in _quantized:
+                param = _quantized[name]
+            elif qtzr.is_initialized():
                 param = qtzr(param)
             stack.enter_context(patch_attr(self, name, param))
         return stack
@@ -215,7 +224,8 @@ class QuantizedLinear(nn.Linear):
     def compute_encodings(self, _verdicts=None):
         """nn/base.py:392-427: weights are calibrated on entry; activation quantizers observe their inputs and pass
         them through unquantized, and set their ranges on exit."""
-        self._compute_param_encodings(overwrite=True, verdicts=_verdicts)
+        quantized = {}
+        self._compute_param_encodings(overwrite=True, verdicts=_verdicts, quantized=quantized)
         with contextlib.ExitStack() as stack:
             # Neither the parameters nor their (just computed) encodings change inside the context, so the
             # quantize-dequantized parameters are the same in every calibration pass: they are formed once here and
@@ -223,7 +233,7 @@ class QuantizedLinear(nn.Linear):
             # result; its own _patch_quantized_parameters / fold_param_quantizers, nn/base.py:296-324, 1103-1151, are
             # the same trade).  A caller that modifies a parameter in place inside the context sees the old values.
             if any(q is not None and q.is_initialized() for q in self.param_quantizers.values()):
-                stack.enter_context(self._patch_quantized_parameters())
+                stack.enter_context(self._patch_quantized_parameters(_quantized=quantized))
                 stack.enter_context(self._remove_param_quantizers())
             for qtzr in list(self.input_quantizers) + list(self.output_quantizers):
                 if not isinstance(qtzr, QuantizerBase) or not qtzr.is_overwrite_allowed():

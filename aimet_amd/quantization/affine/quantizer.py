@@ -475,33 +475,52 @@ class AffineQuantizerBase(QuantizerBase, _GridMixin):
                 or cls.set_range is not AffineQuantizerBase.set_range
                 or not all(self._is_overwrite_allowed.values())):
             return False
-        stats = an.observer.get_stats()
-        smin, smax = stats.min, stats.max
         mn, mx = self.min, self.max
         num_steps = self._num_steps_for_calibration()
-        if (smin is None or smax is None or not smin.is_cuda or smin.dtype not in _lib.DTYPE_CODE
-                or smax.dtype != smin.dtype or smax.device != smin.device or smin.shape != smax.shape
-                or mn.device != smin.device or mx.device != smin.device or mn.dtype not in _lib.DTYPE_CODE
-                or mx.dtype != mn.dtype or mn.shape != mx.shape or mn.numel() != smin.numel()
-                or not (smin.is_contiguous() and smax.is_contiguous() and mn.is_contiguous() and mx.is_contiguous())
+        if (not mn.is_cuda or mx.device != mn.device or mn.dtype not in _lib.DTYPE_CODE or mx.dtype != mn.dtype
+                or mn.shape != mx.shape or not (mn.is_contiguous() and mx.is_contiguous())
                 or num_steps <= 0 or num_steps > (1 << 24)):
             return False
+        # a single encoding observed through observe_and_clone(): the running extrema still lie in the observer's
+        # slots, and the launch folds them itself (the observer is left as it is and folds them if anybody asks)
+        slots = an.observer.live_slots()
+        if slots is not None and (slots[1] != mn.device or mn.numel() != 1):
+            slots = None
+        if slots is None:
+            stats = an.observer.get_stats()
+            smin, smax = stats.min, stats.max
+            if (smin is None or smax is None or smin.dtype not in _lib.DTYPE_CODE or smax.dtype != smin.dtype
+                    or smin.device != mn.device or smax.device != mn.device or smin.shape != smax.shape
+                    or mn.numel() != smin.numel() or not (smin.is_contiguous() and smax.is_contiguous())):
+                return False
+            stat_dtype = smin.dtype
+        else:
+            stat_dtype = slots[0]
         from aimet_amd.quantization.encoding_analyzer import _scalar_constants, _range_flags_buffer, _report_range_flags
 
         device = mn.device
-        consts = _scalar_constants(smin.dtype, _get_minimum_scale(num_steps))
+        consts = _scalar_constants(stat_dtype, _get_minimum_scale(num_steps))
         scale = torch.empty(mn.shape, dtype=torch.float32, device=device)
         offset = self._constant_offset(device) if self.symmetric else torch.empty(mn.shape, dtype=torch.float32,
                                                                                   device=device)
         flags, own = _range_flags_buffer(device)
-        _lib.check(
-            _lib.load().ahq_minmax_finalize(
-                _lib.DTYPE_CODE[smin.dtype], smin.data_ptr(), smax.data_ptr(), smin.numel(), num_steps,
-                1 if self.symmetric else 0, consts[0], consts[1], consts[2], consts[3], flags.data_ptr(),
-                _lib.DTYPE_CODE[mn.dtype], mn.data_ptr(), mx.data_ptr(), self.qmin, self.qmax,
-                _get_minimum_scale(self.qmax - self.qmin), scale.data_ptr(),
-                None if self.symmetric else offset.data_ptr(), _lib.current_stream(device)),
-            "ahq_minmax_finalize")
+        if slots is not None:
+            _lib.check(
+                _lib.load().ahq_minmax_slots_finalize(
+                    _lib.DTYPE_CODE[stat_dtype], slots[2].data_ptr(), num_steps, 1 if self.symmetric else 0,
+                    consts[0], consts[1], consts[2], consts[3], flags.data_ptr(), _lib.DTYPE_CODE[mn.dtype],
+                    mn.data_ptr(), mx.data_ptr(), self.qmin, self.qmax, _get_minimum_scale(self.qmax - self.qmin),
+                    scale.data_ptr(), None if self.symmetric else offset.data_ptr(), _lib.current_stream(device)),
+                "ahq_minmax_slots_finalize")
+        else:
+            _lib.check(
+                _lib.load().ahq_minmax_finalize(
+                    _lib.DTYPE_CODE[stat_dtype], smin.data_ptr(), smax.data_ptr(), smin.numel(), num_steps,
+                    1 if self.symmetric else 0, consts[0], consts[1], consts[2], consts[3], flags.data_ptr(),
+                    _lib.DTYPE_CODE[mn.dtype], mn.data_ptr(), mx.data_ptr(), self.qmin, self.qmax,
+                    _get_minimum_scale(self.qmax - self.qmin), scale.data_ptr(),
+                    None if self.symmetric else offset.data_ptr(), _lib.current_stream(device)),
+                "ahq_minmax_finalize")
         # min / max were written behind torch's back: tell autograd, and everyone who keys on the version counters
         torch.autograd.graph.increment_version((mn, mx))
         enc = AffineEncoding(scale, offset, self.qmin, self.qmax, self._symmetric, self.block_size,
@@ -805,6 +824,95 @@ class QuantizeDequantize(AffineQuantizerBase):
                                   self.block_size, self.zero_point_shift, producer=self)
         output = y.as_subclass(DequantizedTensor)
         output.encoding = encoding
+        return output
+
+    def _calibrate_and_quantize(self, tensor: torch.Tensor) -> Optional[DequantizedTensor]:
+        """``self._calibrate_on(tensor)`` followed by ``self(tensor)`` -- what a quantized module does with each of
+        its parameters when a calibration starts (nn/base.py:331-386, 296-324) -- as one library call
+        (ahq_minmax_calibrate_qdq: the three launches of the step-by-step form, same results).  None, with nothing
+        changed, when that does not apply and the two steps have to run: gradients switched on, a subclass or a
+        patched method, hooks on the quantizer, another backend or analyzer, an end that may not be overwritten,
+        tensors the library does not take, or an arithmetic that would depend on the offsets' values."""
+        if torch.is_grad_enabled() or type(self) is not QuantizeDequantize:  # pylint: disable=unidiomatic-typecheck
+            return None
+        from aimet_amd.quantization._stats import _check_reducible
+        from aimet_amd.quantization.affine.backends import get_backend, hip as _hip
+        from aimet_amd.quantization.encoding_analyzer import _scalar_constants, _range_flags_buffer, _report_range_flags
+        from torch.nn.modules import module as _module
+
+        an = self.encoding_analyzer
+        mn, mx = self.min, self.max
+        own = self.__dict__
+        if (type(an) is not MinMaxEncodingAnalyzer  # pylint: disable=unidiomatic-typecheck
+                or not all(self._is_overwrite_allowed.values()) or get_backend() is not _hip
+                or "forward" in own or "get_encodings" in own or "is_initialized" in own
+                or self._forward_hooks or self._forward_pre_hooks
+                or _module._global_forward_hooks or _module._global_forward_pre_hooks):  # pylint: disable=protected-access
+            return None
+        x = tensor.detach()
+        if type(x) != torch.Tensor:  # pylint: disable=unidiomatic-typecheck
+            x = x.as_subclass(torch.Tensor)
+        num_steps = self._num_steps_for_calibration()
+        if not (x.is_cuda and x.dtype in _lib.DTYPE_CODE and x.is_contiguous() and x.numel() > 0
+                and mn.device == x.device and mx.device == x.device and mn.dtype == mx.dtype
+                and mn.dtype in _lib.DTYPE_CODE and mn.shape == mx.shape and mn.is_contiguous() and mx.is_contiguous()
+                and 0 < num_steps <= (1 << 24)):
+            return None
+        symmetric = bool(self.symmetric)
+        zps = float(self.zero_point_shift or 0.0)
+        bs = tuple(self.block_size) if self.block_size else None
+        held = own.get("_calibrate_qdq_plan")
+        key = (tuple(x.shape), x.dtype, x.device, tuple(mn.shape), self.qmin, self.qmax, symmetric, bs, zps)
+        if held is None or held[0] != key:
+            try:
+                _check_reducible(x, tuple(self.shape), bs)
+                _hip._validate_arguments(x, mn, self.qmin, self.qmax, bs)  # pylint: disable=protected-access
+            except RuntimeError:
+                return None  # the step-by-step form raises what the reference raises
+            # the arithmetic the forward pass would choose (backends/hip.py: quantize_dequantize)
+            per_tensor = mn.numel() == 1
+            if bs is None and zps == 0.0 and (per_tensor or symmetric):
+                aten = per_tensor or _hip._aten_arithmetic_applies(  # pylint: disable=protected-access
+                    x, mn, self._constant_offset(x.device), self.qmin, self.qmax)
+            elif bs is None and zps == 0.0:
+                return None  # per-channel, asymmetric: the choice looks at the offsets
+            else:
+                aten = False
+            if aten:
+                arith, cd = _lib.AHQ_ARITH_ATEN, torch.float32
+            else:
+                arith, cd = _lib.AHQ_ARITH_AUTOGRAD, _hip._internal_dtype(x.dtype, self.qmin, self.qmax)  # pylint: disable=protected-access
+                if cd == torch.float64 or not _hip._is_grid_representable(cd, self.qmin, self.qmax):  # pylint: disable=protected-access
+                    return None
+            grid = _hip._grid(arith, _lib.AHQ_OP_QDQ, x.dtype, cd, self.qmin, self.qmax, 0.0 if aten else zps)  # pylint: disable=protected-access
+            layout = _build_layout(tuple(x.shape), tuple(range(x.dim())), tuple(mn.shape), None if aten else bs)
+            nbytes = _lib.load().ahq_minmax_calibrate_qdq_workspace_bytes(_lib.DTYPE_CODE[x.dtype], layout)
+            ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=x.device)
+            held = own["_calibrate_qdq_plan"] = (key, grid, layout, nbytes, ws)
+        _, grid, layout, nbytes, ws = held
+        device = x.device
+        an.reset_stats()
+        consts = _scalar_constants(x.dtype, _get_minimum_scale(num_steps))
+        y = torch.empty_like(x)
+        scale = torch.empty(mn.shape, dtype=torch.float32, device=device)
+        offset = self._constant_offset(device) if symmetric else torch.empty(mn.shape, dtype=torch.float32,
+                                                                             device=device)
+        flags, own_flags = _range_flags_buffer(device)
+        _lib.check(
+            _lib.load().ahq_minmax_calibrate_qdq(
+                grid, layout, x.data_ptr(), y.data_ptr(), num_steps, 1 if symmetric else 0, consts[0], consts[1],
+                consts[2], consts[3], flags.data_ptr(), _lib.DTYPE_CODE[mn.dtype], mn.data_ptr(), mx.data_ptr(),
+                _get_minimum_scale(self.qmax - self.qmin), scale.data_ptr(), offset.data_ptr(), ws.data_ptr(), nbytes,
+                _lib.current_stream(device)),
+            "ahq_minmax_calibrate_qdq")
+        torch.autograd.graph.increment_version((mn, mx))
+        enc = AffineEncoding(scale, offset, self.qmin, self.qmax, self._symmetric, self.block_size,
+                             self.zero_point_shift, producer=self)
+        own["_encoding_cache"] = (self._encoding_cache_key(), enc)
+        if own_flags:
+            _report_range_flags(flags)
+        output = y.as_subclass(DequantizedTensor)
+        output.encoding = enc
         return output
 
     def forward(self, input: torch.Tensor) -> DequantizedTensor:

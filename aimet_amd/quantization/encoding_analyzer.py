@@ -142,6 +142,12 @@ class _MinMaxObserver(_Observer[_MinMaxRange]):
             self.stats = _MinMaxRange(mn, mx)
             self._slots_dirty = False
 
+    def live_slots(self):
+        """(dtype, device, slot buffer) while the slots hold running extrema that `stats` does not, else None."""
+        if self._slots_of is not None and self._slots_dirty:
+            return (*self._slots_of, self._slots)
+        return None
+
     def _leave_slots(self):
         """`stats` becomes the one place the running extrema live in."""
         self._fold_slots()
@@ -475,6 +481,7 @@ class MinMaxEncodingAnalyzer(EncodingAnalyzer[_MinMaxRange]):
 
 
 @functools.lru_cache(maxsize=256)
+@functools.lru_cache(maxsize=None)
 def _scalar_constants(dtype: torch.dtype, tiny: float):
     """(minimum scale as `dtype` sees it, as float32, finfo(dtype).max, the near-overflow threshold in `dtype`)."""
     big = torch.finfo(dtype).max

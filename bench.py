@@ -880,6 +880,7 @@ def _model_parity_sweep(model, ids, dev):
     each quantizer's input reduced on the CPU as it goes by; then the calibrated min / max of all quantizers are
     compared with the oracle's encodings of those statistics."""
     import llama_harness as LH
+    from aimet_amd import nn as qnn
     from aimet_amd.quantization.affine import QuantizeDequantize
     from oracle import torch_ref as O
 
@@ -895,8 +896,15 @@ def _model_parity_sweep(model, ids, dev):
         return hook
 
     quantizers = {n: m for n, m in model.named_modules() if isinstance(m, QuantizeDequantize)}
+    weights = {f"{n}.param_quantizers.weight": m.weight for n, m in model.named_modules()
+               if isinstance(m, qnn.QuantizedLinear) and m.param_quantizers["weight"] is not None}
     for name, q in quantizers.items():
-        hooks.append(q.register_forward_hook(record(name, q)))
+        if name in weights:
+            # no hook: a hooked parameter quantizer is calibrated and called in two steps, and the timed step uses
+            # the one-call form; its input is the weight itself
+            stats[name] = O.reduce_minmax(weights[name].detach().cpu(), tuple(q.shape), q.block_size)
+        else:
+            hooks.append(q.register_forward_hook(record(name, q)))
     LH.calibrate(model, [ids])
     for h in hooks:
         h.remove()
@@ -1025,7 +1033,15 @@ def run_model_workload(steps, warmup, dev, with_cpu_baseline=True, batches=8, se
     parity["all_quantizers_bit_exact"] = bool(ok == total)
     if bad:
         parity["first_mismatches"] = bad
-    parity["sample"] = "calibrated min/max of every quantizer on its full-size input (1 batch); forward of 3 quantizers"
+    # the weight a calibration pass multiplies with (quantize-dequantized by the call that calibrated its quantizer)
+    with torch.no_grad(), qnn.compute_encodings(model):
+        held = mods["blocks.0.mlp.down_proj"].weight.detach().as_subclass(torch.Tensor).cpu()
+        model(ids[0])
+    ref_w = O.qdq_v2_forward(w_cpu, wq.get_scale().detach().cpu(), wq.get_offset().detach().cpu(), wq.qmin, wq.qmax,
+                             wq.block_size).y
+    parity["calibration_pass_weight_bit_exact"] = bool(torch.equal(held.view(torch.int16), ref_w.view(torch.int16)))
+    parity["sample"] = ("calibrated min/max of every quantizer on its full-size input (1 batch); forward of 3 "
+                        "quantizers; the down_proj weight of block 0 as the calibration passes see it")
 
     config = {"workload": "c5_llama16x2048_ffn8192_w4b64_a16_calib8x2048_plus_forward", "linear_layers": nlin,
               "weight_elements": wel, "activation_elements_per_forward": act,

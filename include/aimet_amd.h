@@ -214,6 +214,35 @@ int ahq_minmax_finalize(int32_t stat_dtype, const void* stat_min, const void* st
                         void* param_min, void* param_max, int64_t qmin, int64_t qmax, double grid_minimum_scale,
                         float* scale, float* offset, void* stream);
 
+/* ahq_minmax_finalize for a single encoding whose running extrema still lie in the slots of ahq_minmax_accumulate:
+ * the launch folds the slots (as ahq_minmax_slots_read would: a NaN seen in any batch makes both statistics NaN) and
+ * goes on from there, so that leaving a whole-model calibration costs one launch per activation quantizer instead of
+ * two.  The slots are only read.  Remaining arguments as in ahq_minmax_finalize with num_encodings = 1.
+ */
+int ahq_minmax_slots_finalize(int32_t stat_dtype, const void* slots, int64_t num_steps, int32_t symmetric,
+                              float minimum_scale_in_dtype, float minimum_scale, float dtype_max,
+                              float near_max_threshold, int32_t* flags, int32_t param_dtype, void* param_min,
+                              void* param_max, int64_t qmin, int64_t qmax, double grid_minimum_scale, float* scale,
+                              float* offset, void* stream);
+
+/* The calibration of a parameter followed by its first quantize-dequantize, as one call: what
+ * BaseQuantizationMixin._compute_param_encodings (AT/nn/base.py:331-386: the parameter quantizer observes the
+ * parameter inside its compute_encodings() context and sets its range on leaving it) and the quantizer's next forward
+ * pass do for a min/max-calibrated affine quantizer.  The launches and the results are those of ahq_minmax on x,
+ * ahq_minmax_finalize on the extrema and ahq_qdq_forward with the scale / offset just derived; a whole-model
+ * calibration makes this call once per weight, and the host time of three calls with their arguments was the larger
+ * part of entering it.  grid: AHQ_OP_QDQ, AHQ_ARITH_ATEN or AHQ_ARITH_AUTOGRAD, as the forward pass would choose;
+ * num_steps .. grid_minimum_scale as in ahq_minmax_finalize (qmin / qmax are the grid's); scale: float32 output;
+ * offset: float32, written for an asymmetric grid, READ for a symmetric one (the caller's constant offsets), one
+ * value per encoding either way.  workspace: ahq_minmax_calibrate_qdq_workspace_bytes(grid->io_dtype, layout) bytes.
+ */
+size_t ahq_minmax_calibrate_qdq_workspace_bytes(int32_t dtype, const ahq_layout* layout);
+int    ahq_minmax_calibrate_qdq(const ahq_grid* grid, const ahq_layout* layout, const void* x, void* y,
+                                int64_t num_steps, int32_t symmetric, float minimum_scale_in_dtype,
+                                float minimum_scale, float dtype_max, float near_max_threshold, int32_t* flags,
+                                int32_t param_dtype, void* param_min, void* param_max, double grid_minimum_scale,
+                                float* scale, float* offset, void* workspace, size_t workspace_bytes, void* stream);
+
 /* The backward pass of ahq_lpbq_scale: replaces the autograd chain of GroupedBlockQuantizeDequantize._get_scale
  * (AT/quantization/affine/quantizer.py:1363-1399 on top of :319-342) when min / max are learned -- the backward of
  * the quantize-dequantize of the block scales (AT/quantization/affine/backends/torch_builtins.py:727-831), of the

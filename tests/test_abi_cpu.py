@@ -83,6 +83,22 @@ def test_argument_validation_without_a_gpu(lib):
     g.arith = _lib.AHQ_ARITH_AUTOGRAD
     repeated = _lib.make_layout([3, 4, 64], [3, 1, 16], [0, 4, 1])
     assert fused(g, repeated, 4) == _lib.AHQ_ERR_UNSUPPORTED      # encodings repeat over the leading dimension
+    # calibration and first quantize-dequantize of a parameter in one call
+    def calibrate(grid, layout, x=1, y=1, offset=1, ws=1, ws_bytes=1 << 20):
+        return lib.ahq_minmax_calibrate_qdq(grid, layout, x, y, 15, 1, 1e-9, 1e-9, 3e38, 1e37, 1, 0, 1, 1, 1e-9, 1,
+                                            offset, ws, ws_bytes, None)
+
+    assert calibrate(None, blocks) == 1 and calibrate(g, None) == 1
+    assert calibrate(g, blocks, x=None) == 1 and calibrate(g, blocks, y=None) == 1 and calibrate(g, blocks, offset=None) == 1
+    g.arith = _lib.AHQ_ARITH_DLQ
+    assert calibrate(g, blocks) == 1 and b"arithmetic" in lib.ahq_last_error()
+    g.arith, g.op = _lib.AHQ_ARITH_AUTOGRAD, 1
+    assert calibrate(g, blocks) == 1
+    g.op = 0
+    assert calibrate(g, bad) == 1
+    assert calibrate(g, blocks, ws=None) == _lib.AHQ_ERR_WORKSPACE
+    assert calibrate(g, blocks, ws_bytes=8) == _lib.AHQ_ERR_WORKSPACE
+    assert calibrate(g, _lib.make_layout([0, 64], [1, 16], [4, 1])) == 1   # nothing to calibrate on
 
 
 def test_workspace_queries_and_planning(lib):
@@ -102,6 +118,11 @@ def test_workspace_queries_and_planning(lib):
     assert lib.ahq_minmax_workspace_bytes(per_tensor) >= tiles * 12
     assert lib.ahq_hist_update_workspace_bytes(0, per_tensor, 512) > 1024 * 2 * 514 * 4
     assert lib.ahq_qdq_backward_workspace_bytes(g, blockwise, 1) >= 0
+    # statistics of every encoding (two aligned arrays) in front of the reduction's own workspace
+    assert (lib.ahq_minmax_calibrate_qdq_workspace_bytes(_lib.AHQ_BF16, blockwise)
+            >= 2 * 14336 * 64 * 2 + lib.ahq_minmax_workspace_bytes(blockwise))
+    assert lib.ahq_minmax_calibrate_qdq_workspace_bytes(0, per_tensor) >= 512 + lib.ahq_minmax_workspace_bytes(per_tensor)
+    assert lib.ahq_minmax_calibrate_qdq_workspace_bytes(9, per_tensor) == 0
 
 
 def test_backend_registry():

@@ -519,6 +519,155 @@ def test_end_of_minmax_calibration_in_one_launch(device, monkeypatch, stat_dtype
     assert_same_bits(fast.max.detach() + 0.0, hi.to(param_dtype) + 0.0, "max against the oracle")
 
 
+PARAM_CALIBRATION_CASES = {
+    # tensor shape, quantizer shape, block size, (qmin, qmax, symmetric, zero-point shift)
+    "blocks_of_64_4bit": ((96, 256), (96, 4), (1, 64), (-8, 7, True, None)),
+    "blocks_of_16_shifted_2bit": ((33, 64), (33, 4), (1, 16), (-2, 1, True, 0.5)),
+    "per_row_8bit": ((130, 77), (130, 1), None, (-128, 127, True, None)),
+    "per_tensor_8bit_asymmetric": ((57, 129), (), None, (0, 255, False, None)),
+    "per_tensor_16bit_asymmetric": ((57, 129), (1,), None, (0, 65535, False, None)),
+    "blocks_asymmetric": ((64, 128), (64, 2), (1, 64), (0, 15, False, None)),
+    "blocks_along_rows": ((128, 40), (4, 40), (32, 1), (-8, 7, True, None)),
+}
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16], ids=lambda d: str(d).split(".")[-1])
+@pytest.mark.parametrize("param_dtype", [torch.float32, torch.bfloat16], ids=["f32_params", "bf16_params"])
+@pytest.mark.parametrize("case", list(PARAM_CALIBRATION_CASES), ids=str)
+def test_parameter_calibration_and_first_quantization_in_one_call(device, case, dtype, param_dtype):
+    """_calibrate_and_quantize (ahq_minmax_calibrate_qdq) against the two steps it stands for -- calibrate on the
+    parameter, then call the quantizer on it: min / max, scale, offset and the quantize-dequantized parameter bit for
+    bit, the encodings left in the cache are the ones the next forward pass uses, and the result against the oracle's
+    quantize-dequantize with those encodings."""
+    from aimet_amd.quantization.affine import QuantizeDequantize
+
+    xshape, qshape, block, (qmin, qmax, symmetric, zps) = PARAM_CALIBRATION_CASES[case]
+    g = torch.Generator().manual_seed(len(case))
+    w = (torch.randn(xshape, generator=g) * torch.logspace(-3, 1, xshape[0]).view(-1, 1)).to(dtype)
+    w[0, :3] = 0.0
+    wd = torch.nn.Parameter(w.to(device))
+
+    def make():
+        return QuantizeDequantize(qshape, qmin=qmin, qmax=qmax, symmetric=symmetric, block_size=block,
+                                  zero_point_shift=zps).to(device=device, dtype=param_dtype)
+
+    one, two = make(), make()
+    with torch.no_grad():
+        y1 = one._calibrate_and_quantize(wd)
+        assert y1 is not None
+        two._calibrate_on(wd)
+        y2 = two(wd)
+        assert type(y1) is type(y2) and y1.shape == y2.shape and y1.dtype == y2.dtype
+        assert_same_bits(one.min, two.min, "min")
+        assert_same_bits(one.max, two.max, "max")
+        assert_same_bits(y1.as_subclass(torch.Tensor), y2.as_subclass(torch.Tensor), "quantize-dequantized parameter")
+        assert_same_bits(y1.encoding.scale, y2.encoding.scale, "scale")
+        assert_same_bits(y1.encoding.offset, y2.encoding.offset, "offset")
+        assert one.is_initialized() and one.get_encodings() is y1.encoding
+        assert one.encoding_analyzer.observer.get_stats().min is None  # nothing is left behind in the analyzer
+        again = one(wd)
+        assert_same_bits(again.as_subclass(torch.Tensor), y1.as_subclass(torch.Tensor), "next forward pass")
+    scale, offset = y1.encoding.scale.cpu(), y1.encoding.offset.cpu()
+    if block is None and (len(qshape) == 0 or math.prod(qshape) == 1 or symmetric):
+        ref = O.qdq_v1(w, scale, offset, qmin, qmax)[0]
+    else:
+        ref = O.qdq_v2_forward(w, scale, offset, qmin, qmax, block, zero_point_shift=zps or 0.0).y
+    assert_same_bits(y1.as_subclass(torch.Tensor).cpu(), ref, "against the oracle")
+    # a second calibration reuses the plan and follows a changed parameter
+    with torch.no_grad():
+        wd.mul_(0.5)
+        y3 = one._calibrate_and_quantize(wd)
+        two._calibrate_on(wd)
+        assert_same_bits(one.min, two.min, "min after the parameter changed")
+        assert_same_bits(y3.as_subclass(torch.Tensor), two(wd).as_subclass(torch.Tensor), "after the parameter changed")
+
+
+def test_parameter_calibration_in_one_call_steps_aside(device):
+    """The cases _calibrate_and_quantize leaves to the two-step form, with nothing touched."""
+    from aimet_amd.quantization.affine import QuantizeDequantize
+    from aimet_amd.quantization.encoding_analyzer import SqnrEncodingAnalyzer
+
+    w = torch.randn(32, 64, device=device)
+
+    def untouched(q, x=w, grad=False):
+        with torch.set_grad_enabled(grad):
+            out = q._calibrate_and_quantize(x)
+        return out is None and not q.is_initialized()
+
+    base = dict(bitwidth=4, symmetric=True, block_size=(1, 16))
+    assert untouched(QuantizeDequantize((32, 4), **base).to(device), grad=True)
+    hooked = QuantizeDequantize((32, 4), **base).to(device)
+    hooked.register_forward_hook(lambda m, a, o: None)
+    assert untouched(hooked)
+
+    class Mine(QuantizeDequantize):
+        pass
+
+    assert untouched(Mine((32, 4), **base).to(device))
+    assert untouched(QuantizeDequantize((32, 1), 8, symmetric=False).to(device))  # per row, asymmetric
+    sq = QuantizeDequantize((32, 4), encoding_analyzer=SqnrEncodingAnalyzer((32, 4), block_size=(1, 16)), **base)
+    assert untouched(sq.to(device))
+    frozen = QuantizeDequantize((32, 4), **base).to(device)
+    frozen.allow_overwrite(False)
+    assert untouched(frozen)
+    assert untouched(QuantizeDequantize((32, 4), **base).to(device), x=w.t())          # not contiguous
+    assert untouched(QuantizeDequantize((32, 4), **base).to(device), x=w.double())
+    assert untouched(QuantizeDequantize((32, 4), **base).to(device), x=w[:, :60].contiguous())  # shape does not fit
+    with torch.no_grad():
+        assert QuantizeDequantize((32, 4), **base).to(device)._calibrate_and_quantize(w) is not None
+
+
+@pytest.mark.parametrize("stat_dtype", [torch.float32, torch.float16, torch.bfloat16], ids=lambda d: str(d).split(".")[-1])
+@pytest.mark.parametrize("param_dtype", [torch.float32, torch.bfloat16], ids=["f32_params", "bf16_params"])
+@pytest.mark.parametrize("grid", [(0, 255, False), (-128, 127, True), (0, 65535, False), (-2, 1, True)], ids=str)
+@pytest.mark.parametrize("special", [None, "nan", "inf", "zeros"])
+def test_end_of_a_per_tensor_calibration_straight_from_the_slots(device, monkeypatch, stat_dtype, param_dtype, grid,
+                                                                 special):
+    """A per-tensor quantizer that observed its batches through observe_and_clone() leaves the calibration with one
+    launch that folds the observer's slots itself (ahq_minmax_slots_finalize): same min / max / scale / offset as
+    folding first (ahq_minmax_slots_read + ahq_minmax_finalize), the observer's statistics are still there for whoever
+    asks, and they are the extrema of everything seen."""
+    from aimet_amd.quantization.affine import QuantizeDequantize
+    from aimet_amd.quantization.encoding_analyzer import _MinMaxObserver
+
+    qmin, qmax, symmetric = grid
+    g = torch.Generator().manual_seed(17)
+    batches = [torch.randn(3, 70001, generator=g) * s_ for s_ in (1.0, 3.0, 0.2)]
+    if special == "nan":
+        batches[1][2, 5] = float("nan")
+    elif special == "inf":
+        batches[0][0, 0], batches[2][1, 1] = float("inf"), -float("inf")
+    elif special == "zeros":
+        batches = [torch.zeros(3, 1000) for _ in range(3)]
+    batches = [b.to(stat_dtype).to(device) for b in batches]
+
+    def calibrated(from_slots: bool):
+        q = QuantizeDequantize((), qmin=qmin, qmax=qmax, symmetric=symmetric).to(device=device, dtype=param_dtype)
+        seen = []
+        real = _MinMaxObserver.live_slots
+        monkeypatch.setattr(_MinMaxObserver, "live_slots",
+                            (lambda self: seen.append(real(self)) or seen[-1]) if from_slots else (lambda self: None))
+        with warnings.catch_warnings():
+            warnings.simplefilter("ignore")
+            with torch.no_grad(), q._compute_encodings(passthrough=True):
+                for b in batches:
+                    assert_same_bits(q(b), b, "pass-through copy")
+        monkeypatch.undo()
+        assert (len(seen) == 1 and seen[0] is not None) if from_slots else not seen
+        return q
+
+    fast, slow = calibrated(True), calibrated(False)
+    assert_same_bits(fast.min, slow.min, "min")
+    assert_same_bits(fast.max, slow.max, "max")
+    with torch.no_grad():
+        assert_same_bits(fast.get_encodings().scale, slow.get_encodings().scale, "scale")
+        assert_same_bits(fast.get_encodings().offset, slow.get_encodings().offset, "offset")
+    stats = fast.encoding_analyzer.observer.get_stats()
+    everything = torch.cat([b.flatten() for b in batches])
+    assert_same_bits(stats.min, everything.amin(), "the observer's minimum, read afterwards")
+    assert_same_bits(stats.max, everything.amax(), "the observer's maximum, read afterwards")
+
+
 def test_range_warnings_of_the_fused_calibration_end(device):
     from aimet_amd.quantization.affine import QuantizeDequantize
     from aimet_amd.quantization.encoding_analyzer import deferred_range_warnings
