@@ -611,7 +611,6 @@ class AffineQuantizerBase(QuantizerBase, _GridMixin):
         shape = self.shape
         dtype, device = self.min.dtype, self.min.device
 
-        @functools.wraps(inner_forward)
         def observing_forward(input: torch.Tensor) -> torch.Tensor:
             if type(input) != torch.Tensor:  # pylint: disable=unidiomatic-typecheck
                 input = input.as_subclass(torch.Tensor)
@@ -644,6 +643,8 @@ class AffineQuantizerBase(QuantizerBase, _GridMixin):
                 ret.encoding = encoding
             return ret
 
+        if not passthrough:  # (a whole-model calibration enters hundreds of these contexts: nothing it does not need)
+            functools.update_wrapper(observing_forward, inner_forward)
         self.encoding_analyzer.reset_stats()
         with patch_attr(self, "forward", observing_forward):
             yield
