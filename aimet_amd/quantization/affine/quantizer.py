@@ -31,7 +31,8 @@ from aimet_amd.quantization._utils import (
     true_divide,
 )
 from aimet_amd.quantization.affine._utils import _GridMixin
-from aimet_amd.quantization.affine.backends import quantize, quantize_dequantize, dequantize, _derive_qmin_qmax
+from aimet_amd.quantization.affine.backends import quantize, quantize_dequantize, dequantize, _derive_qmin_qmax, get_backend
+from aimet_amd.quantization.affine.backends import hip as _hip_backend
 from aimet_amd.quantization.affine.backends.hip import _build_layout
 from aimet_amd.quantization.affine.encoding import AffineEncoding, GroupedBlockEncoding
 from aimet_amd.quantization.base.quantizer import QuantizerBase
@@ -888,10 +889,10 @@ class QuantizeDequantize(AffineQuantizerBase):
             grid = _hip._grid(arith, _lib.AHQ_OP_QDQ, x.dtype, cd, self.qmin, self.qmax, 0.0 if aten else zps)  # pylint: disable=protected-access
             layout = _build_layout(tuple(x.shape), tuple(range(x.dim())), tuple(mn.shape), None if aten else bs)
             nbytes = _lib.load().ahq_minmax_calibrate_qdq_workspace_bytes(_lib.DTYPE_CODE[x.dtype], layout)
-            ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=x.device)
-            held = own["_calibrate_qdq_plan"] = (key, grid, layout, nbytes, ws)
-        _, grid, layout, nbytes, ws = held
+            held = own["_calibrate_qdq_plan"] = (key, grid, layout, nbytes)
+        _, grid, layout, nbytes = held
         device = x.device
+        ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=device)  # two statistics per encoding: not kept
         an.reset_stats()
         consts = _scalar_constants(x.dtype, _get_minimum_scale(num_steps))
         y = torch.empty_like(x)
@@ -916,7 +917,91 @@ class QuantizeDequantize(AffineQuantizerBase):
         output.encoding = enc
         return output
 
+    def _forward_steady(self, input: torch.Tensor) -> Optional[DequantizedTensor]:
+        """The forward pass of an inference loop -- no gradients, cached encodings, an input of the shape seen before:
+        the library call of the step-by-step form with the grid and layout of an earlier call, and nothing else (a
+        whole-model forward makes hundreds of these calls and is bound by their host time).  Grid and layout depend
+        on the quantizer's grid and on shapes, not on the encodings' values, so they outlive a new calibration.  None
+        whenever anything differs; the step-by-step form then runs."""
+        own = self.__dict__
+        plan = own.get("_forward_plan")
+        cached = own.get("_encoding_cache")
+        if plan is None or cached is None or torch.is_grad_enabled() or "get_encodings" in own:
+            return None
+        x = input if type(input) == torch.Tensor else input.as_subclass(torch.Tensor)  # pylint: disable=unidiomatic-typecheck
+        key = self._encoding_cache_key()
+        if (cached[0] != key or plan[1] != x.shape or plan[2] != x.dtype or plan[3] != x.device
+                or not x.is_contiguous() or get_backend() is not _hip_backend):
+            return None
+        enc = cached[1]
+        scale, offset = enc.scale, enc.offset
+        if plan[0] is not enc:
+            # other encodings than last time (a calibration, a new range): they have to fit the plan as they are
+            f32 = torch.float32
+            if (plan[6] != key[6:] or scale.dtype != f32 or offset.dtype != f32 or scale.shape != plan[7]
+                    or offset.shape != plan[7] or not (scale.is_contiguous() and offset.is_contiguous())
+                    or scale.device != x.device or offset.device != x.device or scale.requires_grad
+                    or offset.requires_grad or (plan[8] and getattr(offset, "_ahq_constant", None) is None)):
+                del own["_forward_plan"]
+                return None
+            own["_forward_plan"] = (enc,) + plan[1:]
+        y = torch.empty_like(x)
+        status = _lib.load().ahq_qdq_forward(plan[4], plan[5], x.data_ptr(), y.data_ptr(), None, scale.data_ptr(),
+                                             offset.data_ptr(), None, None, _lib.current_stream(x.device))
+        if status:
+            _lib.check(status, "ahq_qdq_forward")
+        output = y.as_subclass(DequantizedTensor)
+        output.encoding = enc
+        return output
+
+    def _plan_steady_forward(self, input: torch.Tensor, encoding: AffineEncoding) -> None:
+        """After a step-by-step forward pass without gradients, the second in a row with the same input shape: keep
+        what the next one can reuse (see _forward_steady).  Nothing is kept where the choice of the arithmetic looks
+        at tensor values, where scale or offset would have to be converted or broadcast first, or for anything but
+        the plain class on this backend."""
+        _hip = _hip_backend
+        own = self.__dict__
+        if "get_encodings" in own:
+            return  # a pass with borrowed encodings (dynamic ones of a calibration batch, precomputed ones)
+        own.pop("_forward_plan", None)
+        seen = own.get("_forward_seen")
+        if seen is None or seen[0] != input.shape or seen[1] != input.dtype:
+            own["_forward_seen"] = (input.shape, input.dtype)
+            return
+        cached = own.get("_encoding_cache")
+        scale, offset = encoding.scale, encoding.offset
+        if (type(self) is not QuantizeDequantize  # pylint: disable=unidiomatic-typecheck
+                or cached is None or cached[1] is not encoding or get_backend() is not _hip
+                or not (input.is_cuda and input.is_contiguous() and input.numel() > 0 and input.dtype in _lib.DTYPE_CODE)
+                or scale.dtype != torch.float32 or offset.dtype != torch.float32 or scale.shape != offset.shape
+                or not (scale.is_contiguous() and offset.is_contiguous())
+                or scale.device != input.device or offset.device != input.device
+                or scale.requires_grad or offset.requires_grad):
+            return
+        bs = tuple(encoding.block_size) if encoding.block_size else None
+        zps = float(encoding.zero_point_shift or 0.0)
+        qmin, qmax = encoding.qmin, encoding.qmax
+        aten = needs_constant = False
+        if bs is None and zps == 0.0:
+            needs_constant = scale.numel() != 1
+            if needs_constant and getattr(offset, "_ahq_constant", None) is None:
+                return  # per-channel with offsets of its own: the choice reads them on every call
+            aten = _hip._aten_arithmetic_applies(input, scale, offset, qmin, qmax)  # pylint: disable=protected-access
+        if aten:
+            arith, cd = _lib.AHQ_ARITH_ATEN, torch.float32
+        else:
+            arith, cd = _lib.AHQ_ARITH_AUTOGRAD, _hip._internal_dtype(input.dtype, qmin, qmax)  # pylint: disable=protected-access
+            if cd == torch.float64 or not _hip._is_grid_representable(cd, qmin, qmax):  # pylint: disable=protected-access
+                return
+        grid = _hip._grid(arith, _lib.AHQ_OP_QDQ, input.dtype, cd, qmin, qmax, 0.0 if aten else zps)  # pylint: disable=protected-access
+        layout = _build_layout(tuple(input.shape), tuple(range(input.dim())), tuple(scale.shape), None if aten else bs)
+        own["_forward_plan"] = (encoding, input.shape, input.dtype, input.device, grid, layout, cached[0][6:],
+                                scale.shape, needs_constant)
+
     def forward(self, input: torch.Tensor) -> DequantizedTensor:
+        steady = self._forward_steady(input)
+        if steady is not None:
+            return steady
         fused = self._forward_from_range(input)
         if fused is not None:
             return fused
@@ -925,6 +1010,8 @@ class QuantizeDequantize(AffineQuantizerBase):
             input = input.as_subclass(torch.Tensor)
         output = quantize_dequantize(input, encoding.scale, encoding.offset, encoding.qmin, encoding.qmax,
                                      block_size=encoding.block_size, zero_point_shift=encoding.zero_point_shift)
+        if not torch.is_grad_enabled():
+            self._plan_steady_forward(input, encoding)
         output = output.as_subclass(DequantizedTensor)
         output.encoding = encoding
         return output

@@ -668,6 +668,86 @@ def test_end_of_a_per_tensor_calibration_straight_from_the_slots(device, monkeyp
     assert_same_bits(stats.max, everything.amax(), "the observer's maximum, read afterwards")
 
 
+STEADY_CASES = {
+    "per_tensor_asymmetric": ((3, 64, 96), (), None, dict(bitwidth=16, symmetric=False)),
+    "per_tensor_symmetric": ((3, 64, 96), (1,), None, dict(bitwidth=8, symmetric=True)),
+    "per_row_symmetric": ((48, 200), (48, 1), None, dict(bitwidth=8, symmetric=True)),
+    "per_row_asymmetric": ((48, 200), (48, 1), None, dict(bitwidth=8, symmetric=False)),   # never planned
+    "blocks_4bit": ((48, 256), (48, 4), (1, 64), dict(bitwidth=4, symmetric=True)),
+}
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=lambda d: str(d).split(".")[-1])
+@pytest.mark.parametrize("case", list(STEADY_CASES), ids=str)
+def test_repeated_forward_without_gradients_reuses_the_previous_call(device, monkeypatch, case, dtype):
+    """From the third identical call on, a forward pass without gradients is the library call alone
+    (_forward_steady): same bits as the step-by-step form; a changed range, another shape, a strided input or a
+    wanted gradient go back to it; copies of the quantizer work."""
+    import copy
+
+    from aimet_amd.quantization.affine import QuantizeDequantize
+    from aimet_amd.quantization.affine import quantizer as Q
+
+    xshape, qshape, block, kw = STEADY_CASES[case]
+    g = torch.Generator().manual_seed(21)
+    x = (torch.randn(xshape, generator=g) * 3).to(dtype).to(device)
+    q = QuantizeDequantize(qshape, block_size=block, **kw).to(device)
+    with torch.no_grad(), q.compute_encodings():
+        q(x)
+    planned = case != "per_row_asymmetric"
+    q.__dict__.pop("_forward_seen", None)  # (the calibration pass has already shown the shape once)
+    calls = []
+    real = Q.quantize_dequantize
+    monkeypatch.setattr(Q, "quantize_dequantize", lambda *a, **k: calls.append(1) or real(*a, **k))
+    with torch.no_grad():
+        first, second, third = q(x), q(x), q(x)
+        assert len(calls) == (2 if planned else 3)
+        assert ("_forward_plan" in q.__dict__) == planned
+        assert type(third) is type(first) and third.encoding is first.encoding
+        assert_same_bits(second.as_subclass(torch.Tensor), first.as_subclass(torch.Tensor), "second call")
+        assert_same_bits(third.as_subclass(torch.Tensor), first.as_subclass(torch.Tensor), "third call")
+        other = torch.randn(xshape, generator=g).to(dtype).to(device)
+        want = real(other, first.encoding.scale, first.encoding.offset, q.qmin, q.qmax, block_size=q.block_size)
+        assert_same_bits(q(other).as_subclass(torch.Tensor), want, "other values, same shape")
+        n = len(calls)
+        # a strided input of the same shape, and another shape: the step-by-step form
+        strided = torch.empty(xshape[:-1] + (2 * xshape[-1],), dtype=dtype, device=device)[..., ::2].copy_(x)
+        assert_same_bits(q(strided).as_subclass(torch.Tensor), first.as_subclass(torch.Tensor), "strided input")
+        assert len(calls) == n + 1
+        if block is None and len(qshape) < 2:
+            q(x[:2])
+            assert len(calls) == n + 2
+        # a new range is followed
+        q.set_range(q.min * 0.5, q.max * 0.5)
+        n = len(calls)
+        moved = q(x)
+        assert len(calls) == n + 1
+        fresh = QuantizeDequantize(qshape, block_size=block, **kw).to(device)
+        fresh.set_range(q.min, q.max)
+        assert_same_bits(moved.as_subclass(torch.Tensor), fresh(x).as_subclass(torch.Tensor), "after set_range")
+        q(x)
+        clone = copy.deepcopy(q)
+        assert_same_bits(clone(x).as_subclass(torch.Tensor), moved.as_subclass(torch.Tensor), "deep copy")
+        assert_same_bits(q(x).as_subclass(torch.Tensor), moved.as_subclass(torch.Tensor), "steady again")
+        # grid and layout outlive new encodings (a calibration between two forward passes)
+        for passthrough in (True, False):
+            with q._compute_encodings(passthrough=passthrough):
+                q(x * 4)
+            n = len(calls)
+            wider = q(x)
+            assert len(calls) == (n if planned else n + 1)
+        fresh = QuantizeDequantize(qshape, block_size=block, **kw).to(device)
+        fresh.set_range(q.min, q.max)
+        assert_same_bits(wider.as_subclass(torch.Tensor), fresh(x).as_subclass(torch.Tensor), "new range, old plan")
+        assert wider.encoding is q.get_encodings() and wider.encoding is not moved.encoding
+    # gradients wanted: the autograd forms
+    xg = x.clone().requires_grad_(True)
+    out = q(xg)
+    assert out.requires_grad
+    out.sum().backward()
+    assert xg.grad is not None
+
+
 def test_range_warnings_of_the_fused_calibration_end(device):
     from aimet_amd.quantization.affine import QuantizeDequantize
     from aimet_amd.quantization.encoding_analyzer import deferred_range_warnings
