@@ -925,24 +925,33 @@ class QuantizeDequantize(AffineQuantizerBase):
         whenever anything differs; the step-by-step form then runs."""
         own = self.__dict__
         plan = own.get("_forward_plan")
-        cached = own.get("_encoding_cache")
-        if plan is None or cached is None or torch.is_grad_enabled() or "get_encodings" in own:
+        if plan is None or torch.is_grad_enabled():
             return None
+        borrowed = "get_encodings" in own  # precomputed encodings, or the dynamic ones of a calibration batch
+        if borrowed:
+            enc = self.get_encodings()
+            if enc is None:
+                return None
+        else:
+            cached = own.get("_encoding_cache")
+            if cached is None or cached[0] != self._encoding_cache_key():
+                return None
+            enc = cached[1]
         x = input if type(input) == torch.Tensor else input.as_subclass(torch.Tensor)  # pylint: disable=unidiomatic-typecheck
-        key = self._encoding_cache_key()
-        if (cached[0] != key or plan[1] != x.shape or plan[2] != x.dtype or plan[3] != x.device
-                or not x.is_contiguous() or get_backend() is not _hip_backend):
+        if (plan[1] != x.shape or plan[2] != x.dtype or plan[3] != x.device or not x.is_contiguous()
+                or get_backend() is not _hip_backend):
             return None
-        enc = cached[1]
         scale, offset = enc.scale, enc.offset
         if plan[0] is not enc:
             # other encodings than last time (a calibration, a new range): they have to fit the plan as they are
             f32 = torch.float32
-            if (plan[6] != key[6:] or scale.dtype != f32 or offset.dtype != f32 or scale.shape != plan[7]
+            if (plan[6] != (enc.qmin, enc.qmax, enc.symmetry, enc.block_size, enc.zero_point_shift)
+                    or scale.dtype != f32 or offset.dtype != f32 or scale.shape != plan[7]
                     or offset.shape != plan[7] or not (scale.is_contiguous() and offset.is_contiguous())
                     or scale.device != x.device or offset.device != x.device or scale.requires_grad
                     or offset.requires_grad or (plan[8] and getattr(offset, "_ahq_constant", None) is None)):
-                del own["_forward_plan"]
+                if not borrowed:
+                    del own["_forward_plan"]
                 return None
             own["_forward_plan"] = (enc,) + plan[1:]
         y = torch.empty_like(x)
@@ -995,7 +1004,8 @@ class QuantizeDequantize(AffineQuantizerBase):
                 return
         grid = _hip._grid(arith, _lib.AHQ_OP_QDQ, input.dtype, cd, qmin, qmax, 0.0 if aten else zps)  # pylint: disable=protected-access
         layout = _build_layout(tuple(input.shape), tuple(range(input.dim())), tuple(scale.shape), None if aten else bs)
-        own["_forward_plan"] = (encoding, input.shape, input.dtype, input.device, grid, layout, cached[0][6:],
+        own["_forward_plan"] = (encoding, input.shape, input.dtype, input.device, grid, layout,
+                                (qmin, qmax, encoding.symmetry, encoding.block_size, encoding.zero_point_shift),
                                 scale.shape, needs_constant)
 
     def forward(self, input: torch.Tensor) -> DequantizedTensor:

@@ -739,6 +739,13 @@ def test_repeated_forward_without_gradients_reuses_the_previous_call(device, mon
         fresh = QuantizeDequantize(qshape, block_size=block, **kw).to(device)
         fresh.set_range(q.min, q.max)
         assert_same_bits(wider.as_subclass(torch.Tensor), fresh(x).as_subclass(torch.Tensor), "new range, old plan")
+        # precomputed encodings (inference mode) go the same way
+        n = len(calls)
+        with q._precompute_encodings(dtype=torch.float32):
+            held = q(x)
+            assert held.encoding is q.get_encodings()
+        assert len(calls) == (n if planned else n + 1)
+        assert_same_bits(held.as_subclass(torch.Tensor), wider.as_subclass(torch.Tensor), "precomputed encodings")
         assert wider.encoding is q.get_encodings() and wider.encoding is not moved.encoding
     # gradients wanted: the autograd forms
     xg = x.clone().requires_grad_(True)
