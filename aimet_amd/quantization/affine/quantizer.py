@@ -14,7 +14,7 @@ from __future__ import annotations
 import functools
 import math
 from contextlib import contextmanager, nullcontext
-from typing import Optional, Tuple
+from typing import NamedTuple, Optional, Tuple
 
 import torch
 from torch import nn
@@ -785,6 +785,19 @@ class Quantize(AffineQuantizerBase):
         return output
 
 
+class _ForwardPlan(NamedTuple):
+    """What a forward pass without gradients can take over from an earlier one (QuantizeDequantize._forward_steady)."""
+    encoding: AffineEncoding   # the encodings last checked against the rest
+    shape: torch.Size          # of the input
+    dtype: torch.dtype
+    device: torch.device
+    grid: "_lib.Grid"
+    layout: "_lib.Layout"
+    grid_key: tuple            # (qmin, qmax, symmetry, block_size, zero_point_shift) the grid and layout were made for
+    enc_shape: torch.Size      # of scale and offset
+    needs_constant: bool       # the arithmetic was chosen knowing that the offsets are the grid's constant
+
+
 class QuantizeDequantize(AffineQuantizerBase):
     r"""out = (clamp(round(input / scale) - offset, qmin, qmax) + offset) * scale, returned as a
     :class:`DequantizedTensor`; scale and offset derive from the learnable ``min`` / ``max``."""
@@ -938,24 +951,24 @@ class QuantizeDequantize(AffineQuantizerBase):
                 return None
             enc = cached[1]
         x = input if type(input) == torch.Tensor else input.as_subclass(torch.Tensor)  # pylint: disable=unidiomatic-typecheck
-        if (plan[1] != x.shape or plan[2] != x.dtype or plan[3] != x.device or not x.is_contiguous()
+        if (plan.shape != x.shape or plan.dtype != x.dtype or plan.device != x.device or not x.is_contiguous()
                 or get_backend() is not _hip_backend):
             return None
         scale, offset = enc.scale, enc.offset
-        if plan[0] is not enc:
+        if plan.encoding is not enc:
             # other encodings than last time (a calibration, a new range): they have to fit the plan as they are
             f32 = torch.float32
-            if (plan[6] != (enc.qmin, enc.qmax, enc.symmetry, enc.block_size, enc.zero_point_shift)
-                    or scale.dtype != f32 or offset.dtype != f32 or scale.shape != plan[7]
-                    or offset.shape != plan[7] or not (scale.is_contiguous() and offset.is_contiguous())
+            if (plan.grid_key != (enc.qmin, enc.qmax, enc.symmetry, enc.block_size, enc.zero_point_shift)
+                    or scale.dtype != f32 or offset.dtype != f32 or scale.shape != plan.enc_shape
+                    or offset.shape != plan.enc_shape or not (scale.is_contiguous() and offset.is_contiguous())
                     or scale.device != x.device or offset.device != x.device or scale.requires_grad
-                    or offset.requires_grad or (plan[8] and getattr(offset, "_ahq_constant", None) is None)):
+                    or offset.requires_grad or (plan.needs_constant and getattr(offset, "_ahq_constant", None) is None)):
                 if not borrowed:
                     del own["_forward_plan"]
                 return None
-            own["_forward_plan"] = (enc,) + plan[1:]
+            own["_forward_plan"] = plan._replace(encoding=enc)
         y = torch.empty_like(x)
-        status = _lib.load().ahq_qdq_forward(plan[4], plan[5], x.data_ptr(), y.data_ptr(), None, scale.data_ptr(),
+        status = _lib.load().ahq_qdq_forward(plan.grid, plan.layout, x.data_ptr(), y.data_ptr(), None, scale.data_ptr(),
                                              offset.data_ptr(), None, None, _lib.current_stream(x.device))
         if status:
             _lib.check(status, "ahq_qdq_forward")
@@ -1004,9 +1017,9 @@ class QuantizeDequantize(AffineQuantizerBase):
                 return
         grid = _hip._grid(arith, _lib.AHQ_OP_QDQ, input.dtype, cd, qmin, qmax, 0.0 if aten else zps)  # pylint: disable=protected-access
         layout = _build_layout(tuple(input.shape), tuple(range(input.dim())), tuple(scale.shape), None if aten else bs)
-        own["_forward_plan"] = (encoding, input.shape, input.dtype, input.device, grid, layout,
-                                (qmin, qmax, encoding.symmetry, encoding.block_size, encoding.zero_point_shift),
-                                scale.shape, needs_constant)
+        own["_forward_plan"] = _ForwardPlan(
+            encoding, input.shape, input.dtype, input.device, grid, layout,
+            (qmin, qmax, encoding.symmetry, encoding.block_size, encoding.zero_point_shift), scale.shape, needs_constant)
 
     def forward(self, input: torch.Tensor) -> DequantizedTensor:
         steady = self._forward_steady(input)
