@@ -13,8 +13,9 @@ inline size_t align_up(size_t v) { return (v + kAlign - 1) / kAlign * kAlign; }
 inline size_t dtype_bytes(int32_t dtype) { return dtype == AHQ_F32 ? 4 : 2; }
 
 // statistics (minimum, then maximum, each aligned) in front of the reduction's own workspace
-bool calibrate_qdq_offsets(int32_t dtype, const ahq_layout* layout, size_t* off_max, size_t* off_reduce, size_t* total) {
-    ahq::CanonLayout c;
+bool calibrate_qdq_offsets(int32_t dtype, const ahq_layout* layout, ahq::CanonLayout* canon, size_t* off_max,
+                           size_t* off_reduce, size_t* total) {
+    ahq::CanonLayout& c = *canon;
     const char* err = nullptr;
     if (!ahq::canonicalize(*layout, &c, &err)) return ahq::set_error(err), false;
     const size_t stats = align_up((size_t)c.num_enc * dtype_bytes(dtype));
@@ -28,8 +29,9 @@ bool calibrate_qdq_offsets(int32_t dtype, const ahq_layout* layout, size_t* off_
 
 extern "C" size_t ahq_minmax_calibrate_qdq_workspace_bytes(int32_t dtype, const ahq_layout* layout) {
     if (!layout || dtype < AHQ_F32 || dtype > AHQ_BF16) return 0;
+    ahq::CanonLayout c;
     size_t off_max, off_reduce, total;
-    return calibrate_qdq_offsets(dtype, layout, &off_max, &off_reduce, &total) ? total : 0;
+    return calibrate_qdq_offsets(dtype, layout, &c, &off_max, &off_reduce, &total) ? total : 0;
 }
 
 extern "C" int ahq_minmax_calibrate_qdq(const ahq_grid* grid, const ahq_layout* layout, const void* x, void* y,
@@ -44,12 +46,10 @@ extern "C" int ahq_minmax_calibrate_qdq(const ahq_grid* grid, const ahq_layout* 
     if (dtype < AHQ_F32 || dtype > AHQ_BF16) return set_error("bad dtype"), AHQ_ERR_INVALID;
     if (grid->op != AHQ_OP_QDQ || grid->arith == AHQ_ARITH_DLQ)
         return set_error("a quantize-dequantize grid of the ATen or autograd arithmetic is expected"), AHQ_ERR_INVALID;
-    size_t off_max, off_reduce, total;
-    if (!calibrate_qdq_offsets(dtype, layout, &off_max, &off_reduce, &total)) return AHQ_ERR_INVALID;
-    if (!workspace || workspace_bytes < total) return set_error("workspace too small"), AHQ_ERR_WORKSPACE;
     ahq::CanonLayout c;
-    const char* err = nullptr;
-    ahq::canonicalize(*layout, &c, &err);
+    size_t off_max, off_reduce, total;
+    if (!calibrate_qdq_offsets(dtype, layout, &c, &off_max, &off_reduce, &total)) return AHQ_ERR_INVALID;
+    if (!workspace || workspace_bytes < total) return set_error("workspace too small"), AHQ_ERR_WORKSPACE;
     if (c.numel == 0) return set_error("cannot calibrate on an empty tensor"), AHQ_ERR_INVALID;
     char* w = static_cast<char*>(workspace);
     void* stat_min = w;
