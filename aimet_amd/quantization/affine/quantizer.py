@@ -647,8 +647,18 @@ class AffineQuantizerBase(QuantizerBase, _GridMixin):
         if not passthrough:  # (a whole-model calibration enters hundreds of these contexts: nothing it does not need)
             functools.update_wrapper(observing_forward, inner_forward)
         self.encoding_analyzer.reset_stats()
-        with patch_attr(self, "forward", observing_forward):
+        # (patch_attr(self, "forward", ...) without its generality: a plain function goes into the instance's own
+        # dictionary, which is where Module.__setattr__ would put it after its checks)
+        own = self.__dict__
+        outer = own.get("forward")
+        own["forward"] = observing_forward
+        try:
             yield
+        finally:
+            if outer is None:
+                del own["forward"]
+            else:
+                own["forward"] = outer
         self._set_range_from_statistics()
 
     def _calibrate_on(self, tensor: torch.Tensor) -> None:
