@@ -50,6 +50,13 @@ class OracleImpl:
                                       gamma=float(gamma))
         return lo, hi
 
+    def percentile(self, batches, shape, num_bins, percentile, num_steps, symmetric):
+        obs = O.HistObserver(shape, num_bins)
+        for b in batches:
+            obs.update(b)
+        lo, hi = O.percentile_encodings(obs.stats, shape, percentile, num_steps, symmetric)
+        return lo, hi, [s.histogram for s in obs.stats], [s.bin_edges for s in obs.stats]
+
 
 class HipImpl:
     """The product path on cuda:0, results brought back to the CPU."""
@@ -118,3 +125,12 @@ class HipImpl:
             an.update_stats(self._d(b))
         lo, hi = an.compute_encodings(num_steps, symmetric)
         return lo.cpu(), hi.cpu()
+
+    def percentile(self, batches, shape, num_bins, percentile, num_steps, symmetric):
+        from aimet_amd.quantization.encoding_analyzer import PercentileEncodingAnalyzer
+        an = PercentileEncodingAnalyzer(shape, num_bins=num_bins, percentile=percentile)
+        for b in batches:
+            an.update_stats(self._d(b))
+        lo, hi = an.compute_encodings(num_steps, symmetric)
+        stats = an.observer.get_stats()
+        return lo.cpu(), hi.cpu(), [s.histogram.cpu() for s in stats], [s.bin_edges.cpu() for s in stats]

@@ -10,6 +10,8 @@ An adapter provides:
     minmax_encodings(x, num_steps, symmetric) -> (min, max)           per-tensor min-max analyzer
     hist_observer(num_bins) -> object with update(x) and stat() -> (histogram, bin_edges, min, max) as CPU tensors
     sqnr(x_batches, num_steps, symmetric, **analyzer kwargs) -> (min, max)
+    percentile(x_batches, shape, num_bins, percentile, num_steps, symmetric) -> (min, max, histograms, bin_edges)
+        histograms / bin_edges: one CPU tensor per slot of the analyzer's statistics
 """
 
 import json
@@ -125,6 +127,10 @@ def _named_input(name):
         return torch.full((1,), 3.0)
     if name == "pair(-10.5, 10.5)":
         return torch.tensor([-10.5, 10.5])
+    if name == "arange(0, 1001)":
+        return torch.arange(start=0, end=1001, step=1, dtype=torch.float)
+    if name == "zeros()":
+        return torch.zeros(())
     if name == "arange(-50, 51)":
         return torch.arange(-50, 51, dtype=torch.float)
     if name == "arange(-50, 51) * 1.5":
@@ -260,3 +266,72 @@ def check_sqnr_brute_force(impl):
                 best = (c, dd, oo)
     sel_cost = cost(delta_sel, round(lo.item() / delta_sel))
     assert sel_cost <= best[0] * (1 + 1e-4), (sel_cost, best)
+
+
+def check_percentile(impl):
+    """The percentile analyzer on the cases the reference's tests hold (test_encoding_analyzer.py:556-612, 886-971),
+    plus two results derived by hand that fix which side of a tie the cumulative search takes."""
+    pv = VECTORS["percentile"]
+    for c in pv["exact"]:
+        lo, hi, _, _ = impl.percentile([_named_input(c["input"])], (), c["num_bins"], c["percentile"], c["num_steps"],
+                                       c["symmetric"])
+        assert lo.item() == c["min"] and hi.item() == c["max"], (c, lo, hi)
+    for c in pv["close"]:
+        lo, hi, _, _ = impl.percentile([_named_input(c["input"])], (), c["num_bins"], c["percentile"], c["num_steps"],
+                                       c["symmetric"])
+        assert torch.allclose(lo, torch.full_like(lo, c["min"])) and torch.allclose(hi, torch.full_like(hi, c["max"])), c
+    for c in pv["quantile_index"]:
+        x = _named_input(c["input"])
+        if c["input"] == "full(3.0)":
+            x = x.reshape(())
+        n = c["num_steps"]
+        lo_a, hi_a, hists, edges = impl.percentile([x], (), c["num_bins"], c["percentile"], n, False)
+        cs = torch.cumsum(hists[0], dim=0)
+        value = edges[0][torch.searchsorted(cs, torch.quantile(cs, c["q"]))]
+        if c["expect"] == "constant":
+            # :556-583: asymmetric (0, v); symmetric (-v - max / (n // 2), v)
+            lo_s, hi_s, _, _ = impl.percentile([x], (), c["num_bins"], c["percentile"], n, True)
+            assert torch.allclose(lo_a, torch.zeros_like(lo_a)) and torch.allclose(hi_a, torch.full_like(hi_a, value))
+            assert torch.allclose(hi_s, torch.full_like(hi_s, value))
+            assert torch.allclose(lo_s, torch.full_like(lo_s, -value) - hi_s / (n // 2))
+        elif c["expect"] == "zero":
+            # :585-612: asymmetric (v, 0); symmetric with n - 1 steps (v, -v)
+            lo_s, hi_s, _, _ = impl.percentile([x], (), c["num_bins"], c["percentile"], n - 1, True)
+            assert torch.allclose(lo_a, torch.full_like(lo_a, value)) and torch.allclose(hi_a, torch.zeros_like(hi_a))
+            assert torch.allclose(lo_s, torch.full_like(lo_s, value)) and torch.allclose(hi_s, torch.full_like(hi_s, -value))
+        else:
+            # :933-955: symmetric with n - 1 steps gives -+ the middle edge; asymmetric (0, middle edge), exactly
+            lo_s, hi_s, _, _ = impl.percentile([x], (), c["num_bins"], c["percentile"], n - 1, True)
+            assert lo_s.item() == -value.item() and hi_s.item() == value.item()
+            assert lo_a.item() == 0 and hi_a.item() == value.item()
+    # :913-931: the 100th percentile is the observed range
+    x = torch.randn(10000, generator=torch.Generator().manual_seed(11)) * 2 + 2
+    lo, hi, _, _ = impl.percentile([x], (), 3, 100, 254, True)
+    assert torch.allclose(lo, -x.abs().max()) and torch.allclose(hi, x.abs().max())
+    lo, hi, _, _ = impl.percentile([x], (), 3, 100, 255, False)
+    assert torch.allclose(lo, x.min()) and torch.allclose(hi, x.max())
+    # :957-971: two outliers above a ramp
+    o = pv["outliers"]
+    x = torch.arange(start=0, end=101, step=1, dtype=torch.float)
+    x[-1] = 1000
+    x[-2] = 800
+    _, hi, _, _ = impl.percentile([x], tuple(o["shape"]), o["num_bins"], o["percentile"], o["num_steps"], False)
+    assert o["max_above"] < hi.item() < o["max_below"]
+    # By hand.  Eight values in four bins of width 2 over [0, 8] give counts 2, 2, 2, 2 and cumulative counts 2, 4,
+    # 6, 8.  At 50 % both targets are exactly 4.0 = the second cumulative count: the first position whose count is
+    # NOT BELOW the target is bin 1, whose left edge is 2.0 (a search for the first count ABOVE it would give 4.0).
+    x = torch.tensor([0.0, 1.0, 2.0, 3.0, 4.0, 5.0, 6.0, 8.0])
+    lo, hi, hists, edges = impl.percentile([x], (), 4, 50, 255, False)
+    assert hists[0].tolist() == [2.0, 2.0, 2.0, 2.0] and edges[0].tolist() == [0.0, 2.0, 4.0, 6.0, 8.0]
+    assert lo.item() == 0.0 and hi.item() == 2.0, (lo, hi)
+    # Shifted to [-8, 0]: the lower edge survives the "zero in range" rule, the upper one is raised to 0.  At 75 %
+    # the targets are 6.0 (upper: bin 2, edge -4) and 2.0 (lower: bin 0, edge -8): (-8, 0).  Symmetric with 254
+    # steps: delta = max(0 / 127, 8 / 127), so (-8, 8) up to the rounding of 127 * (8 / 127).
+    lo, hi, _, _ = impl.percentile([x - 8.0], (), 4, 75, 255, False)
+    assert lo.item() == -8.0 and hi.item() == 0.0, (lo, hi)
+    lo, hi, _, _ = impl.percentile([x - 8.0], (), 4, 75, 254, True)
+    assert abs(lo.item() + 8.0) < 1e-6 and abs(hi.item() - 8.0) < 1e-6
+    # Two slots of one analyzer are independent: slot 0 is the ramp above, slot 1 its mirror image.
+    both = torch.stack([x, -x])
+    lo, hi, _, _ = impl.percentile([both], (2, 1), 4, 50, 255, False)
+    assert lo.flatten().tolist() == [0.0, -4.0] and hi.flatten().tolist() == [2.0, 0.0], (lo, hi)

@@ -55,3 +55,7 @@ def test_sqnr_outlier(impl):
 
 def test_sqnr_brute_force(impl):
     G.check_sqnr_brute_force(impl)
+
+
+def test_percentile(impl):
+    G.check_percentile(impl)
