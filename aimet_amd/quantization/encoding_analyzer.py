@@ -228,13 +228,15 @@ class _MinMaxObserver(_Observer[_MinMaxRange]):
                 nbytes = lib.ahq_minmax_workspace_bytes(layout)
                 ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=x.device)
                 bmin, bmax = torch.empty_like(cur.min), torch.empty_like(cur.max)
-                self.__dict__["_fast"] = (key, cur.min, cur.max, layout, ws, nbytes, bmin, bmax, _lib.DTYPE_CODE[x.dtype],
-                                          lib.ahq_minmax_copy)
+                # plain data only: the observer is deep-copied and pickled with its quantizer, and a ctypes function
+                # pointer can be neither
+                self.__dict__["_fast"] = (key, cur.min, cur.max, layout, ws, nbytes, bmin, bmax, _lib.DTYPE_CODE[x.dtype])
             return out
-        _, rmin, rmax, layout, ws, nbytes, bmin, bmax, code, entry = fast
+        _, rmin, rmax, layout, ws, nbytes, bmin, bmax, code = fast
         out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
-        status = entry(code, layout, x.data_ptr(), out.data_ptr(), bmin.data_ptr(), bmax.data_ptr(), rmin.data_ptr(),
-                       rmax.data_ptr(), 0, ws.data_ptr(), nbytes, _lib.current_stream(x.device))
+        status = _lib.load().ahq_minmax_copy(code, layout, x.data_ptr(), out.data_ptr(), bmin.data_ptr(),
+                                             bmax.data_ptr(), rmin.data_ptr(), rmax.data_ptr(), 0, ws.data_ptr(), nbytes,
+                                             _lib.current_stream(x.device))
         if status:
             _lib.check(status, "ahq_minmax_copy")
         return out
@@ -481,7 +483,6 @@ class MinMaxEncodingAnalyzer(EncodingAnalyzer[_MinMaxRange]):
 
 
 @functools.lru_cache(maxsize=256)
-@functools.lru_cache(maxsize=None)
 def _scalar_constants(dtype: torch.dtype, tiny: float):
     """(minimum scale as `dtype` sees it, as float32, finfo(dtype).max, the near-overflow threshold in `dtype`)."""
     big = torch.finfo(dtype).max

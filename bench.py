@@ -37,6 +37,7 @@ if ROOT not in sys.path:
 METRIC = "QDQ fwd+bwd GB/s (% of HBM peak); calibration elems/s; vs host-CPU ref"
 HBM_PEAK_GBS = 8000.0
 COPY_REF_ELEMS = 1 << 26
+ROTATION_BYTES = 1 << 31    # tensors a timed loop goes through before it comes back to the first
 MIN_REPEATS = 7
 MIN_TIMED_SECONDS = 0.010
 # HBM bytes per launch of each workload's dominant kernel(s): rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE averages per
@@ -307,7 +308,31 @@ def _make_module(w, dev):
     return q.to(dev)
 
 
-def run_qdq_workload(key, steps, warmup, dev, with_cpu_baseline=True):
+def _host_time_of_module_step(q, xm, grad, reps=60):
+    """Python time of QuantizeDequantize.forward and of .backward() with the GPU idle when each starts (device
+    synchronised before both): what the interpreter, autograd and the library's host code cost per call, the floor of
+    a module-API step however fast the kernels are.  Medians, microseconds."""
+    fwd_t, bwd_t = [], []
+    for _ in range(reps):
+        xm.grad = None
+        q.min.grad = None
+        q.max.grad = None
+        _sync()
+        t0 = time.perf_counter()
+        out = q(xm)
+        t1 = time.perf_counter()
+        _sync()
+        t2 = time.perf_counter()
+        out.backward(grad)
+        t3 = time.perf_counter()
+        fwd_t.append(t1 - t0)
+        bwd_t.append(t3 - t2)
+    _sync()
+    return {"host_us_forward": round(statistics.median(fwd_t[5:]) * 1e6, 1),
+            "host_us_backward": round(statistics.median(bwd_t[5:]) * 1e6, 1)}
+
+
+def run_qdq_workload(key, steps, warmup, dev, with_cpu_baseline=True, with_cached=True):
     from aimet_amd import _lib
     from aimet_amd.quantization._utils import _get_minimum_scale
     from aimet_amd.quantization.affine.backends import hip
@@ -340,21 +365,40 @@ def run_qdq_workload(key, steps, warmup, dev, with_cpu_baseline=True):
     cd = hip._internal_dtype(x.dtype, qmin, qmax)
     grid = hip._grid(_lib.AHQ_ARITH_AUTOGRAD, _lib.AHQ_OP_QDQ, x.dtype, cd, qmin, qmax, 0.0)
     _, layout = hip._prepare(x, scale.shape, w["block"])
-    y = torch.empty_like(x)
-    gx = torch.empty_like(x)
     gs = torch.empty_like(scale)
     go = torch.empty_like(scale)
     nbytes = lib.ahq_qdq_backward_workspace_bytes(grid, layout, 1)
     ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=dev)
+    # Every timed launch works on the next of `rot` sets of (x, y, grad, gx) at addresses of their own, at least 2 GiB
+    # in rotation (eight and more times the 256 MB last-level cache), and the backward pass of a step takes the set
+    # half a rotation away from its forward pass: nothing a launch reads was touched by any of the launches before it
+    # that the caches could still hold, so bytes / time is what HBM delivered.  Set 0 is the one compared with the
+    # oracle; the others hold the same values.
+    rot = max(6, -(-ROTATION_BYTES // (4 * x.numel() * x.element_size())))
+    rot += rot % 2
+    sets = [(x, torch.empty_like(x), grad, torch.empty_like(x))]
+    sets += [(x.clone(), torch.empty_like(x), grad.clone(), torch.empty_like(x)) for _ in range(rot - 1)]
+    y, gx = sets[0][1], sets[0][3]
+    turn = {"fwd": 0, "bwd": rot // 2, "mm": 0, "mod": 0}
 
-    def fwd():
-        _lib.check(lib.ahq_qdq_forward(grid, layout, x.data_ptr(), y.data_ptr(), None, scale.data_ptr(),
+    def nxt(which):
+        turn[which] = k = (turn[which] + 1) % rot
+        return sets[k]
+
+    def fwd_on(t):
+        _lib.check(lib.ahq_qdq_forward(grid, layout, t[0].data_ptr(), t[1].data_ptr(), None, scale.data_ptr(),
                                        offset.data_ptr(), None, None, stream), "fwd")
 
-    def bwd():
-        _lib.check(lib.ahq_qdq_backward(grid, layout, grad.data_ptr(), x.data_ptr(), gx.data_ptr(), gs.data_ptr(),
+    def bwd_on(t):
+        _lib.check(lib.ahq_qdq_backward(grid, layout, t[2].data_ptr(), t[0].data_ptr(), t[3].data_ptr(), gs.data_ptr(),
                                         go.data_ptr(), scale.data_ptr(), offset.data_ptr(), ws.data_ptr(), nbytes,
                                         stream), "bwd")
+
+    def fwd():
+        fwd_on(nxt("fwd"))
+
+    def bwd():
+        bwd_on(nxt("bwd"))
 
     derive = None
     if w["lpbq"]:
@@ -376,20 +420,26 @@ def run_qdq_workload(key, steps, warmup, dev, with_cpu_baseline=True):
     if derive is not None:
         blocks_per_group = q._blocks_per_group()
         if blocks_per_group is not None:
-            def fused():
-                _lib.check(lib.ahq_lpbq_qdq_forward(grid, layout, x.data_ptr(), y.data_ptr(), None,
+            def fused_on(t):
+                _lib.check(lib.ahq_lpbq_qdq_forward(grid, layout, t[0].data_ptr(), t[1].data_ptr(), None,
                                                     _lib.DTYPE_CODE[pmin.dtype], pmin.data_ptr(), pmax.data_ptr(),
                                                     blocks_per_group, min_scale, mult, None, scale.data_ptr(),
                                                     pcs.data_ptr(), stream), "lpbq forward")
 
-    def step():
+            def fused():
+                fused_on(nxt("fwd"))
+
+    def step_on(tf, tb):
         if fused is not None:
-            fused()
+            fused_on(tf)
         else:
             if derive is not None:
                 derive()
-            fwd()
-        bwd()
+            fwd_on(tf)
+        bwd_on(tb)
+
+    def step():
+        step_on(nxt("fwd"), nxt("bwd"))
 
     loop_s, repeats = timed_steps(step, steps, warmup)
     sec_per_step = loop_s / steps
@@ -399,6 +449,23 @@ def run_qdq_workload(key, steps, warmup, dev, with_cpu_baseline=True):
     t_bwd = event_time(bwd, reps)
     t_derive = event_time(derive, reps) if derive is not None else 0.0
     t_fused = event_time(fused, reps) if fused is not None else 0.0
+    # the same launches over ONE set again and again: the tensors then partly come from the last-level cache
+    cached = None
+    if with_cached:
+        c_loop, _ = timed_steps(lambda: step_on(sets[0], sets[0]), steps, warmup)
+        tc_fwd = event_time(lambda: (fused_on if fused is not None else fwd_on)(sets[0]), reps)
+        tc_bwd = event_time(lambda: bwd_on(sets[0]), reps)
+        cached = {"ms_per_step": round(c_loop / steps * 1e3, 5), "fwd_us": round(tc_fwd * 1e6, 2),
+                  "bwd_us": round(tc_bwd * 1e6, 2)}
+    # every set must hold what set 0 holds (compared with the oracle below)
+    _sync()
+    for t in sets[1:]:
+        fwd_on(t)
+        bwd_on(t)
+    fwd_on(sets[0])
+    bwd_on(sets[0])
+    _sync()
+    sets_agree = all(torch.equal(t[1], y) and torch.equal(t[3], gx) for t in sets[1:])
 
     n = x.numel()
     S = x.element_size()
@@ -417,25 +484,29 @@ def run_qdq_workload(key, steps, warmup, dev, with_cpu_baseline=True):
         grid_a = hip._grid(_lib.AHQ_ARITH_ATEN, _lib.AHQ_OP_QDQ, x.dtype, torch.float32, qmin, qmax, 0.0)
         nb_a = lib.ahq_qdq_backward_workspace_bytes(grid_a, layout, 0)
         ws_a = torch.empty(max(nb_a, 16), dtype=torch.uint8, device=dev)
-        y_a = torch.empty_like(x)
 
-        def fwd_a():
-            _lib.check(lib.ahq_qdq_forward(grid_a, layout, x.data_ptr(), y_a.data_ptr(), None, scale.data_ptr(),
+        def fwd_a_on(t):
+            _lib.check(lib.ahq_qdq_forward(grid_a, layout, t[0].data_ptr(), t[1].data_ptr(), None, scale.data_ptr(),
                                            offset.data_ptr(), None, None, stream), "fwd aten")
 
-        def bwd_a():
-            _lib.check(lib.ahq_qdq_backward(grid_a, layout, grad.data_ptr(), x.data_ptr(), gx.data_ptr(), None, None,
-                                            scale.data_ptr(), offset.data_ptr(), ws_a.data_ptr(), nb_a, stream),
+        def bwd_a_on(t):
+            _lib.check(lib.ahq_qdq_backward(grid_a, layout, t[2].data_ptr(), t[0].data_ptr(), t[3].data_ptr(), None,
+                                            None, scale.data_ptr(), offset.data_ptr(), ws_a.data_ptr(), nb_a, stream),
                        "bwd aten")
 
-        ta_f, ta_b = event_time(fwd_a, reps), event_time(bwd_a, reps)
+        ta_f = event_time(lambda: fwd_a_on(nxt("fwd")), reps)
+        ta_b = event_time(lambda: bwd_a_on(nxt("bwd")), reps)
+        y_a = torch.empty_like(x)
+        fwd_a_on((x, y_a))
+        bwd_a_on(sets[0])
         ref_a, mask_a = O.qdq_v1(w["x"], scale_c, offset_c, qmin, qmax)
         frozen = {"arithmetic": "ATen fake-quantize (frozen scale / offset)",
                   "fwd_us": round(ta_f * 1e6, 2), "bwd_us": round(ta_b * 1e6, 2),
                   "GBps": round(5 * S * n / (ta_f + ta_b) / 1e9, 1),
                   "y_bit_exact": bool(torch.equal(y_a.cpu(), ref_a)),
                   "gx_bit_exact": bool(torch.equal(gx.cpu(), torch.where(mask_a, w["grad"], torch.zeros_like(w["grad"]))))}
-        bwd()  # gx of the autograd arithmetic again, for the parity check below
+        del y_a
+        bwd_on(sets[0])  # gx of the autograd arithmetic again, for the parity check below
 
     # ---- min/max calibration of the same tensor (one fused pass for both extrema) + the range it gives
     mm_ws_bytes = lib.ahq_minmax_workspace_bytes(layout)
@@ -443,19 +514,33 @@ def run_qdq_workload(key, steps, warmup, dev, with_cpu_baseline=True):
     mn_out = torch.empty(scale.shape, dtype=x.dtype, device=dev)
     mx_out = torch.empty(scale.shape, dtype=x.dtype, device=dev)
 
-    def minmax():
-        _lib.check(lib.ahq_minmax(code, layout, x.data_ptr(), mn_out.data_ptr(), mx_out.data_ptr(), None, None, 0,
+    # the statistics pass reads one tensor: it goes through the inputs and the upstream gradients of all sets in turn
+    # (2 * rot tensors of the workload's shape and dtype, 0.8 to 1.4 GB)
+    mm_inputs = [t[0] for t in sets] + [t[2] for t in sets]
+    mm_turn = [0]
+
+    def mm_next():
+        mm_turn[0] = k = (mm_turn[0] + 1) % len(mm_inputs)
+        return mm_inputs[k]
+
+    def minmax_on(t):
+        _lib.check(lib.ahq_minmax(code, layout, t.data_ptr(), mn_out.data_ptr(), mx_out.data_ptr(), None, None, 0,
                                   mm_ws.data_ptr(), mm_ws_bytes, stream), "minmax")
 
     an = q.encoding_analyzer
 
-    def calibrate():
+    def calibrate_on(t):
         an.reset_stats()
-        an.update_stats(x)
+        an.update_stats(t)
         return an.compute_encodings(qmax - qmin, w["symmetric"])
 
-    t_mm = event_time(minmax, reps)
-    t_cal = event_time(calibrate, reps)
+    t_mm = event_time(lambda: minmax_on(mm_next()), reps)
+    t_cal = event_time(lambda: calibrate_on(mm_next()), reps)
+    mm_cached = None
+    if with_cached:
+        mm_cached = {"us": round(event_time(lambda: minmax_on(x), reps) * 1e6, 2),
+                     "analyzer_update_plus_compute_encodings_us": round(event_time(lambda: calibrate_on(x), reps) * 1e6, 2)}
+    minmax_on(x)
     # a calibration stream only needs the running extrema: per-tensor statistics keep them as one slot per workgroup
     # and skip the launch that folds a batch's partials (ahq_minmax_accumulate); folded once, at the end
     running = None
@@ -463,11 +548,21 @@ def run_qdq_workload(key, steps, warmup, dev, with_cpu_baseline=True):
         slots = torch.empty(_lib.MINMAX_SLOTS_BYTES, dtype=torch.uint8, device=dev)
         lib.ahq_minmax_accumulate(code, x.data_ptr(), n_elems := x.numel(), None, slots.data_ptr(), 1, stream)
 
-        def accumulate():
-            _lib.check(lib.ahq_minmax_accumulate(code, x.data_ptr(), n_elems, None, slots.data_ptr(), 0, stream),
+        def accumulate_on(t):
+            _lib.check(lib.ahq_minmax_accumulate(code, t.data_ptr(), n_elems, None, slots.data_ptr(), 0, stream),
                        "minmax accumulate")
 
+        x_copies = [t[0] for t in sets]  # the running extrema must stay those of x
+        acc_turn = [0]
+
+        def accumulate():
+            acc_turn[0] = k = (acc_turn[0] + 1) % (2 * rot)
+            accumulate_on(x_copies[k % rot] if k < rot else sets[k - rot][1])
+
+        # (the outputs y hold quantize-dequantized x: inside x's range, so they leave the running extrema alone)
         t_acc = event_time(accumulate, reps)
+        if with_cached:
+            mm_cached["running_us"] = round(event_time(lambda: accumulate_on(x), reps) * 1e6, 2)
         r_mn, r_mx = torch.empty_like(mn_out), torch.empty_like(mx_out)
         _lib.check(lib.ahq_minmax_slots_read(code, slots.data_ptr(), r_mn.data_ptr(), r_mx.data_ptr(), stream), "read")
         running = {"kernel": "ahq_minmax_accumulate (running extrema in per-workgroup slots, no fold launch)",
@@ -478,21 +573,34 @@ def run_qdq_workload(key, steps, warmup, dev, with_cpu_baseline=True):
     exact_mm = bool(torch.equal(mn_out.cpu(), mn_ref.view(mn_out.shape)) and torch.equal(mx_out.cpu(), mx_ref.view(mx_out.shape)))
 
     # ---- the same step through the drop-in module: QuantizeDequantize.forward + autograd backward
-    xm = x.clone().requires_grad_(True)
+    xms = [t[0].clone().requires_grad_(True) for t in sets]
+    xm = xms[0]
 
-    def module_step():
-        xm.grad = None
+    def module_step_on(k):
+        xk = xms[k]
+        xk.grad = None
         q.min.grad = None
         q.max.grad = None
-        out = q(xm)
-        out.backward(grad)
+        out = q(xk)
+        out.backward(sets[(k + rot // 2) % rot][2])
+
+    def module_step():
+        turn["mod"] = k = (turn["mod"] + 1) % rot
+        module_step_on(k)
 
     # loops of at least 200 steps: the first steps after a synchronisation wait for autograd's device thread to wake up
     # (about a millisecond), which a loop of twenty 0.1 ms steps would report as half as much again per step
     mod_steps = max(steps, 200)
     mod_loop, mod_repeats = timed_steps(module_step, mod_steps, min(warmup, 5))
     mod_s = mod_loop / mod_steps
-    module_step()
+    mod_cached = None
+    if with_cached:
+        mc_loop, _ = timed_steps(lambda: module_step_on(0), mod_steps, min(warmup, 5))
+        mod_cached = round(mc_loop / mod_steps * 1e3, 5)
+    host = _host_time_of_module_step(q, xm, sets[0][2])
+    for xk in xms[1:]:
+        xk.grad = None
+    module_step_on(0)
     _sync()
     mod_gx_exact = None
 
@@ -503,7 +611,8 @@ def run_qdq_workload(key, steps, warmup, dev, with_cpu_baseline=True):
     exact_gx = bool(torch.equal(gx.cpu(), gx_ref))
     mod_gx_exact = bool(torch.equal(xm.grad.cpu(), gx_ref))
     gs_err = float(((gs.cpu().view(gs_ref.shape) - gs_ref).abs().max() / gs_ref.abs().max().clamp_min(1e-30)))
-    parity = {"y_bit_exact": exact_y, "gx_bit_exact": exact_gx, "gscale_max_rel_err": gs_err,
+    parity = {"y_bit_exact": exact_y, "gx_bit_exact": exact_gx, "all_sets_in_rotation_agree": bool(sets_agree),
+              "gscale_max_rel_err": gs_err,
               "minmax_bit_exact": exact_mm, "encoding_range_bit_exact": range_exact, "scale_bit_exact": scale_exact,
               "module_gx_bit_exact": mod_gx_exact, "sample": "full size"}
     if w["lpbq"]:
@@ -512,12 +621,18 @@ def run_qdq_workload(key, steps, warmup, dev, with_cpu_baseline=True):
         y.zero_()
         scale.zero_()
         pcs.zero_()
-        fused()
+        fused_on(sets[0])
         parity["fused_forward_bit_exact"] = bool(torch.equal(y.cpu(), tr.y) and torch.equal(scale.cpu(), scale_c.view(scale.shape))
                                                  and torch.equal(pcs.cpu(), pcs_c.view(pcs.shape)))
 
-    dom = ("qdq_bwd_kernel", t_bwd, bytes_bwd) if t_bwd >= t_fwd else ("qdq_fwd_kernel", t_fwd, bytes_fwd)
+    t_fwd_step, bytes_fwd_step, fwd_name = ((t_fused, bytes_fused, "qdq_fwd_lpbq_kernel") if fused is not None
+                                            else (t_fwd, bytes_fwd, "qdq_fwd_kernel"))
+    dom = (("qdq_bwd_kernel", t_bwd, bytes_bwd) if t_bwd >= t_fwd_step else (fwd_name, t_fwd_step, bytes_fwd_step))
+    # the bytes the step's definition counts: 2 S forward + 3 S backward per element, 8 bytes per encoding
+    bytes_step_plain = 5 * S * n + 8 * E
     config = {"workload": w["name"], "elements": n, "encodings": E, "algorithmic_bytes_per_step": bytes_step,
+              "algorithmic_bytes_per_step_without_side_outputs": bytes_step_plain,
+              "tensor_sets_in_rotation": rot, "bytes_in_rotation": rot * 4 * S * n,
               "arithmetic": "autograd (learnable min/max)", "compute_dtype": str(cd).split(".")[-1],
               "step": ("ahq_lpbq_qdq_forward (block scales derived inside the forward launch) + ahq_qdq_backward"
                        if fused is not None else
@@ -546,17 +661,30 @@ def run_qdq_workload(key, steps, warmup, dev, with_cpu_baseline=True):
                         "frac_of_hbm_peak": round((S * n) / t_mm / 1e9 / HBM_PEAK_GBS, 4),
                         "analyzer_update_plus_compute_encodings_us": round(t_cal * 1e6, 2),
                         "analyzer_elements_per_s": round(n / t_cal, 1),
+                        "analyzer_frac_of_hbm_peak": round((S * n) / t_cal / 1e9 / HBM_PEAK_GBS, 4),
+                        "inputs_in_rotation": len(mm_inputs),
+                        **({"same_tensor_again_and_again": mm_cached} if mm_cached is not None else {}),
                         **({"running": running} if running is not None else {})},
         "module_path": {"what": "QuantizeDequantize.forward + .backward() with learnable min/max (allocations, "
                                 "autograd and the per-call scale / offset derivation included)",
                         "ms_per_step": round(mod_s * 1e3, 5), "GBps": round(bytes_step / mod_s / 1e9, 1),
                         "frac_of_hbm_peak": round(bytes_step / mod_s / 1e9 / HBM_PEAK_GBS, 4), "repeats": mod_repeats,
-                        "steps_per_timed_loop": mod_steps},
+                        "steps_per_timed_loop": mod_steps, **host,
+                        **({"same_tensor_again_and_again_ms_per_step": mod_cached} if mod_cached is not None else {})},
         "parity": parity,
         "roofline": {"bound": "hbm", "kernel": dom[0], "achieved": round(dom[2] / dom[1] / 1e9, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(dom[2] / dom[1] / 1e9 / HBM_PEAK_GBS, 4),
-                     "algorithmic_bytes": dom[2], "traffic": MEASURED_TRAFFIC_BYTES.get((key, dom[0]))},
+                     "algorithmic_bytes": dom[2], "traffic": MEASURED_TRAFFIC_BYTES.get((key, dom[0])),
+                     "memory": f"HBM: every launch takes the next of {rot} tensor sets, {rot * 4 * S * n >> 20} MiB in rotation"},
     })
+    out["pct_of_hbm_peak_without_side_outputs"] = round(100.0 * bytes_step_plain / sec_per_step / 1e9 / HBM_PEAK_GBS, 2)
+    if cached is not None:
+        t_c_dom = cached["bwd_us"] if dom[0] == "qdq_bwd_kernel" else cached["fwd_us"]
+        out["roofline"]["cached"] = {
+            "what": "the same launches over one tensor set again and again (partly served by the 256 MB last-level cache)",
+            "frac": round(dom[2] / (t_c_dom * 1e-6) / 1e9 / HBM_PEAK_GBS, 4), "us": t_c_dom,
+            "step_ms": cached["ms_per_step"],
+            "step_pct_of_hbm_peak": round(100.0 * bytes_step / (cached["ms_per_step"] * 1e-3) / 1e9 / HBM_PEAK_GBS, 2)}
     if frozen is not None:
         out["frozen_quantizer"] = frozen
     if with_cpu_baseline:
@@ -1084,9 +1212,9 @@ def run_model_workload(steps, warmup, dev, with_cpu_baseline=True, batches=8, se
 
 
 RUNNERS = {
-    "c1": lambda a, dev, cpu: run_qdq_workload("c1", a.steps, a.warmup, dev, cpu),
-    "c2": lambda a, dev, cpu: run_qdq_workload("c2", a.steps, a.warmup, dev, cpu),
-    "c4": lambda a, dev, cpu: run_qdq_workload("c4", a.steps, a.warmup, dev, cpu),
+    "c1": lambda a, dev, cpu: run_qdq_workload("c1", a.steps, a.warmup, dev, cpu, not a.no_cached),
+    "c2": lambda a, dev, cpu: run_qdq_workload("c2", a.steps, a.warmup, dev, cpu, not a.no_cached),
+    "c4": lambda a, dev, cpu: run_qdq_workload("c4", a.steps, a.warmup, dev, cpu, not a.no_cached),
     "c3": lambda a, dev, cpu: run_hist_workload(min(a.steps, 10), min(a.warmup, 2), dev, cpu),
     "dlq": lambda a, dev, cpu: run_dlq_workload(min(a.steps, 10), min(a.warmup, 2), dev, cpu),
     "c5": lambda a, dev, cpu: run_model_workload(min(a.steps, 3), min(a.warmup, 1), dev, cpu),
@@ -1100,6 +1228,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="all", choices=["all"] + sorted(RUNNERS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-cached", action="store_true",
+                    help="c1 / c2 / c4: leave out the legs that go over one tensor set again and again (the figures "
+                         "under 'cached' / 'same_tensor_again_and_again'), so that every launch of a profiled run "
+                         "reads from HBM")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no collectives exist on this path); use --gpus 1",

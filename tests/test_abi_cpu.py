@@ -270,3 +270,30 @@ def test_product_never_imports_the_oracle():
     code = "import sys; import aimet_amd.quantization, aimet_amd.quantization.affine, aimet_amd.quantization.encoding_analyzer; print(any(m.startswith('oracle') for m in sys.modules))"
     res = subprocess.run([sys.executable, "-c", code], cwd=ROOT, capture_output=True, text=True)
     assert res.stdout.strip() == "False", res.stdout + res.stderr
+
+
+def test_a_quantizer_whose_observer_holds_call_state_can_be_copied_and_pickled():
+    """After a pass-through calibration of a per-channel quantizer its observer keeps what the next call reuses
+    (layout, workspace, result tensors).  Deep copies and pickles of the quantizer go through that state, so it must
+    be plain data: ctypes structures of integers are, a ctypes function pointer is not."""
+    import copy
+    import pickle
+
+    from aimet_amd import _lib
+    from aimet_amd.quantization.affine import QuantizeDequantize
+
+    q = QuantizeDequantize((3, 1), 8, True)
+    q.set_range(torch.tensor([[-1.0], [-2.0], [-3.0]]), torch.tensor([[1.0], [2.0], [3.0]]))
+    obs = q.encoding_analyzer.observer
+    layout = _lib.Layout()
+    layout.ndim = 2
+    mn, mx = torch.zeros(3, 1), torch.ones(3, 1)
+    obs.__dict__["_fast"] = ((torch.Size([3, 8]), torch.float32, torch.device("cpu")), mn, mx, layout,
+                             torch.empty(16, dtype=torch.uint8), 16, torch.empty(3, 1), torch.empty(3, 1), 0)
+    for twin in (copy.deepcopy(q), pickle.loads(pickle.dumps(q))):
+        assert twin.is_initialized() and torch.equal(twin.max, q.max)
+        kept = twin.encoding_analyzer.observer.__dict__["_fast"]
+        assert kept[3].ndim == 2 and kept[0] == obs.__dict__["_fast"][0]
+    # what this guards against
+    with pytest.raises(ValueError):
+        pickle.dumps(_lib.load().ahq_minmax_copy)

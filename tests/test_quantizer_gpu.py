@@ -755,6 +755,33 @@ def test_repeated_forward_without_gradients_reuses_the_previous_call(device, mon
     assert xg.grad is not None
 
 
+@pytest.mark.parametrize("qshape,block", [((16, 1), None), ((16, 4), (1, 8)), ((), None)])
+def test_copy_and_pickle_after_passthrough_calibration(device, qshape, block):
+    """A quantizer (and so a whole model) is deep-copied and pickled after calibration: the observer's kept call state
+    must survive both, and the twins must go on working."""
+    import copy
+    import pickle
+
+    from aimet_amd.quantization.affine import QuantizeDequantize
+
+    g = torch.Generator().manual_seed(21)
+    x = torch.randn(16, 32, generator=g).to(device)
+    q = QuantizeDequantize(qshape, 8, True, block_size=block).to(device)
+    with q._compute_encodings(passthrough=True):
+        for k in range(3):  # the third call is the one that reuses the kept state
+            out = q(x * (k + 1))
+            assert_same_bits(out, x * (k + 1), "pass-through")
+    want = q(x).as_subclass(torch.Tensor)
+    for twin in (copy.deepcopy(q), pickle.loads(pickle.dumps(q))):
+        assert twin.is_initialized()
+        assert_same_bits(twin(x).as_subclass(torch.Tensor), want, "twin forward")
+        with twin._compute_encodings(passthrough=True):
+            for k in range(3):
+                twin(x * (k + 4))
+        assert_same_bits(twin.max, q.max * 2, "twin calibrates on its own")
+    assert_same_bits(q(x).as_subclass(torch.Tensor), want, "original untouched")
+
+
 def test_range_warnings_of_the_fused_calibration_end(device):
     from aimet_amd.quantization.affine import QuantizeDequantize
     from aimet_amd.quantization.encoding_analyzer import deferred_range_warnings
