@@ -23,8 +23,8 @@ PKG = os.path.dirname(HERE)
 OBJ_DIR = os.path.join(HERE, "build")
 LIB_PATH = os.path.join(PKG, "libaimet_amd.so")
 
-SOURCES = ["capi.hip", "qdq.hip", "reduce.hip", "hist.hip", "sqnr.hip", "dlq.hip", "encodings.hip", "diag.hip"]
-HEADERS = ["ahq_device.h", "ahq_host.h", "layout.h", "tiling.h", os.path.join("..", "..", "include", "aimet_amd.h")]
+SOURCES = ["capi.hip", "qdq.hip", "qdq_bwd.hip", "reduce.hip", "hist.hip", "sqnr.hip", "dlq.hip", "encodings.hip", "diag.hip"]
+HEADERS = ["ahq_device.h", "ahq_host.h", "layout.h", "tiling.h", "qdq_common.h", os.path.join("..", "..", "include", "aimet_amd.h")]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",

@@ -1,0 +1,605 @@
+// Fake-quantization backward kernels: straight-through input gradient and the per-encoding scale / offset gradients
+// (arithmetic and arguments: qdq_common.h).
+
+#include "qdq_common.h"
+
+namespace ahq {
+
+__device__ __forceinline__ float finish_sum_rt(double s, int cd) {
+    if (cd == AHQ_BF16) return rnd<AHQ_BF16>((float)s);
+    if (cd == AHQ_F16) return rnd<AHQ_F16>((float)s);
+    return (float)s;
+}
+
+template <typename IO, int VEC, typename M, int RED, bool FULL, bool FAST>
+__device__ __forceinline__ void bwd_math(const QdqArgs& a, const Tile& t, float (*sp)[kStage], const Pack<IO, VEC>* xin,
+                                         const Pack<IO, VEC>* gin, IO* __restrict__ gxp, double& acc_s, double& acc_o,
+                                         double* stage_sums, float* vec_sums, int base) {
+#pragma unroll
+    for (int u = 0; u < kBwdUnroll; ++u) {
+        const int lv = base + u * kBlock + threadIdx.x;
+        float vs = 0.f, vo = 0.f;
+        int si = 0;
+        bool wave_all_in = false;  // only the split form below sets it
+        if constexpr (FAST && M::kSplitBwd) {
+            const bool work = FULL || lv < t.nv;
+            EncP e{};
+            float tq[VEC], xr[VEC], m[VEC];
+            bool all_in = true;
+            if (work) {
+                si = stage_index(a, t, lv);
+                e = staged<M>(sp, si);
+                const float lo = e.p1 + a.gc.qmin, hi = e.p1 + a.gc.qmax;
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) {
+                    M::bwd_pre(load_f32(xin[u].v[k]), e, lo, hi, tq[k], xr[k], m[k]);
+                    all_in &= (m[k] == xr[k]);
+                }
+            }
+            wave_all_in = __builtin_amdgcn_ballot_w64(!all_in) == 0;
+            if (wave_all_in) {
+                // every element of this vector, in every lane, is inside the grid: the input gradient is the output
+                // gradient, the offset gradient gets no term
+                if (work) {
+#pragma unroll
+                    for (int k = 0; k < VEC; ++k) vs += M::bwd_gs_in(load_f32(gin[u].v[k]), tq[k], xr[k]);
+                    if (gxp) store_pack_stream<IO, VEC>(gxp + (int64_t)lv * VEC, gin[u]);
+                }
+            } else if (work) {
+                Pack<IO, VEC> out;
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) {
+                    const float gr = load_f32(gin[u].v[k]);
+                    const bool in = (m[k] == xr[k]);
+                    out.v[k] = store_cast<IO>(in ? gr : 0.f);
+                    vs += in ? M::bwd_gs_in(gr, tq[k], xr[k]) : M::bwd_gs_out(gr, m[k]);
+                    vo += in ? 0.f : M::bwd_goff_out(gr, e);
+                }
+                if (gxp) store_pack_stream<IO, VEC>(gxp + (int64_t)lv * VEC, out);
+            }
+        } else if (FULL || lv < t.nv) {
+            si = stage_index(a, t, lv);
+            const EncP e = staged<M>(sp, si);
+            Pack<IO, VEC> out;
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) {
+                float gx, gs, go;
+                M::template bwd<FAST>(load_f32(gin[u].v[k]), load_f32(xin[u].v[k]), e, a.gc, gx, gs, go);
+                out.v[k] = store_cast<IO>(gx);
+                vs += gs;
+                vo += go;
+            }
+            if (gxp) store_pack_stream<IO, VEC>(gxp + (int64_t)lv * VEC, out);
+        }
+        if (RED == kRedTile) {
+            acc_s += (double)vs;
+            acc_o += (double)vo;
+        } else if (RED == kRedSeg) {
+            // runs of Kv (power of two <= 64) neighbouring lanes share an encoding; runs never straddle a wave.  At most
+            // 64 x VEC terms per encoding, so single precision (what the reference's own sum accumulates in) is enough
+            const int kv = (int)a.Kv;
+            const float fs = segment_reduce(vs, kv, OpAddF());
+            const float fo = wave_all_in ? 0.f : segment_reduce(vo, kv, OpAddF());
+            if ((FULL || lv < t.nv) && (threadIdx.x & (kv - 1)) == 0) {
+                const int64_t e = t.e0 + si;
+                a.gscale[e] = finish_sum_rt((double)fs, a.out_cd);
+                a.goffset[e] = finish_sum_rt((double)fo, a.out_cd);
+            }
+        } else if (RED == kRedAtomic) {
+            // into the tile's own table in LDS first (one entry per run the tile touches); the table is added to the
+            // global sums once per run and tile instead of once per vector
+            if (FULL || lv < t.nv) {
+                atomicAdd(&stage_sums[2 * si], (double)vs);
+                atomicAdd(&stage_sums[2 * si + 1], (double)vo);
+            }
+        } else if (RED == kRedRuns) {
+            // one pair per vector; the runs are added up in a fixed order once the tile is through
+            if (FULL || lv < t.nv) {
+                vec_sums[lv] = vs;
+                vec_sums[kBwdTileVec + lv] = vo;
+            }
+        }
+    }
+}
+
+template <typename IO, int VEC, typename M, int RED, bool FULL, int ROUNDS>
+__device__ __forceinline__ void bwd_tile(const QdqArgs& a, const Tile& t, float (*sp)[kStage], double& acc_s, double& acc_o,
+                                         double* stage_sums, float* vec_sums) {
+    const IO* __restrict__ x = static_cast<const IO*>(a.x) + t.v0 * VEC;
+    const IO* __restrict__ g = static_cast<const IO*>(a.g) + t.v0 * VEC;
+    IO* __restrict__ gxp = a.gx ? static_cast<IO*>(a.gx) + t.v0 * VEC : nullptr;
+    Pack<IO, VEC> xin[kBwdUnroll], gin[kBwdUnroll];
+#pragma unroll
+    for (int r = 0; r < ROUNDS; ++r) {
+        const int base = r * kBlock * kBwdUnroll;
+        if (!FULL && r > 0 && base >= t.nv) break;
+#pragma unroll
+        for (int u = 0; u < kBwdUnroll; ++u) {
+            const int lv = base + u * kBlock + threadIdx.x;
+            if (FULL || lv < t.nv) {
+                xin[u] = load_pack_hinted<IO, VEC>(x + (int64_t)lv * VEC, a.stream_loads != 0);
+                gin[u] = load_pack_hinted<IO, VEC>(g + (int64_t)lv * VEC, a.stream_loads != 0);
+            }
+        }
+        if (r == 0) {
+            // the encodings are staged while the first loads are in flight
+            stage_encodings<M>(a, t, sp);
+            if (RED == kRedAtomic)
+                for (int i = threadIdx.x; i < 2 * t.nstage; i += kBlock) stage_sums[i] = 0.0;
+            __syncthreads();
+        }
+        if (!M::kDiv || __builtin_amdgcn_ballot_w64(!lane_can_divide_fast<IO, VEC, M, FULL, kBwdUnroll>(a, t, sp, xin, base)) == 0)
+            bwd_math<IO, VEC, M, RED, FULL, true>(a, t, sp, xin, gin, gxp, acc_s, acc_o, stage_sums, vec_sums, base);
+        else
+            bwd_math<IO, VEC, M, RED, FULL, false>(a, t, sp, xin, gin, gxp, acc_s, acc_o, stage_sums, vec_sums, base);
+    }
+}
+
+template <typename IO, int VEC, typename M, int RED, int ROUNDS>
+__global__ __launch_bounds__(kBlock) void qdq_bwd_kernel(const QdqArgs a) {
+    __shared__ float sp[M::kNP + (M::kDiv ? 1 : 0)][kStage];
+    __shared__ double red_smem[kBlock / kWave];
+    __shared__ double stage_sums[RED == kRedAtomic ? 2 * kStage : 1];  // kRedAtomic: (scale, offset) sums per run
+    __shared__ float vec_sums[RED == kRedRuns ? 2 * kBwdTileVec : 1];     // kRedRuns: (scale, offset) terms per vector
+    const Tile t = make_tile(a, blockIdx.x);
+    double acc_s = 0.0, acc_o = 0.0;  // kRedTile: per-thread totals
+    if (t.nv == kBlock * kBwdUnroll * ROUNDS) bwd_tile<IO, VEC, M, RED, true, ROUNDS>(a, t, sp, acc_s, acc_o, stage_sums, vec_sums);
+    else bwd_tile<IO, VEC, M, RED, false, ROUNDS>(a, t, sp, acc_s, acc_o, stage_sums, vec_sums);
+    if (RED == kRedRuns) {
+        // The tile holds t.nstage whole runs of Kv vectors.  Short runs: one thread adds a run front to back.  Longer
+        // ones: one wave per run, every lane adds its strided share front to back, then the lanes are combined in
+        // the fixed pattern of wave_reduce.  Either way the order of additions depends on the layout alone.
+        __syncthreads();
+        const int kv = (int)a.Kv;
+        const int64_t run0 = (int64_t)blockIdx.x * a.tpr;
+        auto emit = [&](int run, double s, double o) {
+            if (a.I == 1) {
+                a.gscale[run0 + run] = finish_sum_rt(s, a.out_cd);
+                a.goffset[run0 + run] = finish_sum_rt(o, a.out_cd);
+            } else {
+                a.partials[2 * (run0 + run)] = s;
+                a.partials[2 * (run0 + run) + 1] = o;
+            }
+        };
+        if (kv <= 16) {
+            for (int run = threadIdx.x; run < t.nstage; run += kBlock) {
+                double s = 0.0, o = 0.0;
+                for (int k = 0; k < kv; ++k) {
+                    s += (double)vec_sums[run * kv + k];
+                    o += (double)vec_sums[kBwdTileVec + run * kv + k];
+                }
+                emit(run, s, o);
+            }
+        } else {
+            const int lane = threadIdx.x & (kWave - 1);
+            for (int run = threadIdx.x / kWave; run < t.nstage; run += kBlock / kWave) {
+                double s = 0.0, o = 0.0;
+                for (int k = lane; k < kv; k += kWave) {
+                    s += (double)vec_sums[run * kv + k];
+                    o += (double)vec_sums[kBwdTileVec + run * kv + k];
+                }
+                s = wave_reduce(s, OpAddD());
+                o = wave_reduce(o, OpAddD());
+                if (lane == 0) emit(run, s, o);
+            }
+        }
+        return;
+    }
+    if (RED == kRedAtomic) {
+        __syncthreads();
+        for (int i = threadIdx.x; i < t.nstage; i += kBlock) {
+            int64_t e = t.e0 + i;
+            if (e >= a.J) e %= a.J;
+            atomicAdd(&a.partials[2 * e], stage_sums[2 * i]);
+            atomicAdd(&a.partials[2 * e + 1], stage_sums[2 * i + 1]);
+        }
+    }
+    if (VEC > 1 && blockIdx.x == 0) {  // tail elements, single encoding only
+        const int64_t i = a.nvec * VEC + threadIdx.x;
+        if (i < a.numel) {
+            const IO* x = static_cast<const IO*>(a.x);
+            const IO* g = static_cast<const IO*>(a.g);
+            IO* gxp = static_cast<IO*>(a.gx);
+            const EncP e = staged<M>(sp, 0);
+            float gx, gs, go;
+            M::template bwd<false>(load_f32(g[i]), load_f32(x[i]), e, a.gc, gx, gs, go);
+            if (gxp) gxp[i] = store_cast<IO>(gx);
+            if (RED == kRedTile) {
+                acc_s += (double)gs;
+                acc_o += (double)go;
+            } else if (RED == kRedAtomic) {
+                atomicAdd(&a.partials[0], (double)gs);
+                atomicAdd(&a.partials[1], (double)go);
+            }
+        }
+    }
+    if (RED == kRedTile) {
+        const double bs = block_reduce(acc_s, OpAddD(), red_smem);
+        const double bo = block_reduce(acc_o, OpAddD(), red_smem);
+        // number of tiles that feed one encoding
+        const int64_t per_enc = a.mode == kRows ? a.I * (int64_t)a.tpr : (int64_t)a.nblocks;
+        if (per_enc == 1) {
+            if (threadIdx.x == 0) {
+                a.gscale[t.e0] = finish_sum_rt(bs, a.out_cd);
+                a.goffset[t.e0] = finish_sum_rt(bo, a.out_cd);
+            }
+            return;
+        }
+        if (threadIdx.x == 0) {
+            a.partials[2 * (int64_t)blockIdx.x] = bs;
+            a.partials[2 * (int64_t)blockIdx.x + 1] = bo;
+        }
+    }
+}
+
+// Adds the per-tile partial sums of every encoding in a fixed order (second launch: a kernel boundary makes the
+// partials visible without any in-kernel fence, which on a multi-die GPU would flush the L2 once per workgroup).
+constexpr int kFinishThreads = 1024;
+__global__ __launch_bounds__(kFinishThreads) void qdq_bwd_finish_kernel(const QdqArgs a) {
+    __shared__ double red_smem[2][kFinishThreads / kWave];
+    const int64_t per_enc = a.mode == kRows ? a.I * (int64_t)a.tpr : (int64_t)a.nblocks;
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    if (a.mode != kRows) {
+        // single encoding: independent loads per thread, then one tree
+        double s = 0.0, o = 0.0;
+#pragma unroll 4
+        for (int64_t q = threadIdx.x; q < per_enc; q += kFinishThreads) {
+            s += a.partials[2 * q];
+            o += a.partials[2 * q + 1];
+        }
+        s = wave_reduce(s, OpAddD());
+        o = wave_reduce(o, OpAddD());
+        if (lane == 0) {
+            red_smem[0][wave] = s;
+            red_smem[1][wave] = o;
+        }
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            double ts = 0.0, to = 0.0;
+            for (int w = 0; w < kFinishThreads / kWave; ++w) {
+                ts += red_smem[0][w];
+                to += red_smem[1][w];
+            }
+            a.gscale[0] = finish_sum_rt(ts, a.out_cd);
+            a.goffset[0] = finish_sum_rt(to, a.out_cd);
+        }
+        return;
+    }
+    // one wave per encoding, lanes stride over that encoding's tiles
+    const int64_t wave0 = (int64_t)blockIdx.x * (kFinishThreads / kWave) + wave;
+    for (int64_t j = wave0; j < a.J; j += (int64_t)gridDim.x * (kFinishThreads / kWave)) {
+        double s = 0.0, o = 0.0;
+        for (int64_t q = lane; q < per_enc; q += kWave) {
+            const int64_t i = q / a.tpr, tt = q - i * a.tpr;
+            const int64_t blk = (i * a.J + j) * a.tpr + tt;
+            s += a.partials[2 * blk];
+            o += a.partials[2 * blk + 1];
+        }
+        s = wave_reduce(s, OpAddD());
+        o = wave_reduce(o, OpAddD());
+        if (lane == 0) {
+            a.gscale[j] = finish_sum_rt(s, a.out_cd);
+            a.goffset[j] = finish_sum_rt(o, a.out_cd);
+        }
+    }
+}
+
+// Adds, for every encoding, `count` partial pairs that lie `stride` pairs apart (the first one at the encoding's own
+// index), in a fixed order: one wave per encoding, every lane its strided share front to back, then wave_reduce.
+// kRedRuns with I > 1: count = I runs per encoding, stride = J.  Column kernel: count = row groups, stride = J.
+__global__ __launch_bounds__(kBlock) void qdq_bwd_strided_finish_kernel(const double* __restrict__ partials, int64_t count,
+                                                                        int64_t stride, int64_t num_enc, float* gscale,
+                                                                        float* goffset, int cd) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t waves = (int64_t)gridDim.x * (kBlock / kWave);
+    for (int64_t e = (int64_t)blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave; e < num_enc; e += waves) {
+        double s = 0.0, o = 0.0;
+        for (int64_t q = lane; q < count; q += kWave) {
+            s += partials[2 * (q * stride + e)];
+            o += partials[2 * (q * stride + e) + 1];
+        }
+        s = wave_reduce(s, OpAddD());
+        o = wave_reduce(o, OpAddD());
+        if (lane == 0) {
+            gscale[e] = finish_sum_rt(s, cd);
+            goffset[e] = finish_sum_rt(o, cd);
+        }
+    }
+}
+
+template <typename IO, typename M>
+__global__ __launch_bounds__(kBlock) void qdq_bwd_generic_kernel(const QdqArgs a) {
+    const IO* __restrict__ x = static_cast<const IO*>(a.x);
+    const IO* __restrict__ g = static_cast<const IO*>(a.g);
+    IO* __restrict__ gxp = static_cast<IO*>(a.gx);
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t stride = (int64_t)gridDim.x * kBlock;
+    const int64_t first = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    // whole waves iterate together (lanes past the end carry zeros), so the exchanges below are wave-wide
+    for (int64_t base = first - lane; base < a.numel; base += stride) {
+        const int64_t i = base + lane;
+        const bool active = i < a.numel;
+        int64_t ei = -1;
+        float gx = 0.f, gs = 0.f, go = 0.f;
+        if (active) {
+            ei = generic_enc_index(a, i);
+            const EncP e = load_enc<M>(a, ei);
+            M::template bwd<false>(load_f32(g[i]), load_f32(x[i]), e, a.gc, gx, gs, go);
+            if (gxp) gxp[i] = store_cast<IO>(gx);
+        }
+        if (a.partials) {
+            // neighbouring elements mostly share an encoding: the lanes of each distinct encoding are summed first
+            // and one lane issues the two atomics
+            uint64_t todo = __builtin_amdgcn_ballot_w64(active);
+            while (todo != 0) {
+                const int lead = __builtin_ctzll(todo);
+                const int64_t el = __shfl(ei, lead, kWave);
+                const bool mine = active && ei == el;
+                double ss = mine ? (double)gs : 0.0, so = mine ? (double)go : 0.0;
+#pragma unroll
+                for (int k = kWave / 2; k >= 1; k >>= 1) {
+                    ss += __shfl_xor(ss, k, kWave);
+                    so += __shfl_xor(so, k, kWave);
+                }
+                if (lane == lead) {
+                    atomicAdd(&a.partials[2 * el], ss);
+                    atomicAdd(&a.partials[2 * el + 1], so);
+                }
+                todo &= ~__builtin_amdgcn_ballot_w64(mine);
+            }
+        }
+    }
+}
+
+// Backward for run length 1 (see qdq_fwd_cols_kernel): every lane keeps the sums of its VEC encodings over the rows
+// it walks, the waves of a workgroup add theirs up in LDS one after the other, and the workgroup's sums go to its own
+// row of the partials ([row group][encoding]), which qdq_bwd_strided_finish_kernel adds up in order.
+template <typename IO, int VEC, typename M, int WAVES>
+__global__ __launch_bounds__(WAVES * kWave) void qdq_bwd_cols_kernel(const QdqArgs a) {
+    __shared__ double sums[2 * VEC * kWave];
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int64_t c0 = ((int64_t)blockIdx.x * kWave + lane) * VEC;
+    const bool live = c0 < a.J;
+    const bool want_pg = a.partials != nullptr;
+    if (want_pg) {
+        for (int i = threadIdx.x; i < 2 * VEC * kWave; i += WAVES * kWave) sums[i] = 0.0;
+        __syncthreads();
+    }
+    double acc_s[VEC], acc_o[VEC];
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) acc_s[k] = acc_o[k] = 0.0;
+    if (live) {
+        const IO* __restrict__ x = static_cast<const IO*>(a.x);
+        const IO* __restrict__ g = static_cast<const IO*>(a.g);
+        IO* __restrict__ gxp = static_cast<IO*>(a.gx);
+        EncP e[VEC];
+        bool enc_fast = true;
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) {
+            e[k] = load_enc<M>(a, c0 + k);
+            enc_fast &= !M::kDiv || e[k].rs != 0.f;
+        }
+        const int64_t step = (int64_t)gridDim.y * WAVES * kColUnroll;
+        for (int64_t r0 = ((int64_t)blockIdx.y * WAVES + wave) * kColUnroll; r0 < a.I; r0 += step) {
+            Pack<IO, VEC> xin[kColUnroll], gin[kColUnroll];
+            bool ok = enc_fast;
+#pragma unroll
+            for (int u = 0; u < kColUnroll; ++u)
+                if (r0 + u < a.I) {
+                    xin[u] = load_pack<IO, VEC>(x + (r0 + u) * a.J + c0);
+                    gin[u] = load_pack<IO, VEC>(g + (r0 + u) * a.J + c0);
+                }
+#pragma unroll
+            for (int u = 0; u < kColUnroll; ++u)
+                if (M::kDiv && r0 + u < a.I) ok &= row_can_divide_fast<IO, VEC>(xin[u]);
+            const bool fast = !M::kDiv || __builtin_amdgcn_ballot_w64(!ok) == 0;
+#pragma unroll
+            for (int u = 0; u < kColUnroll; ++u) {
+                if (r0 + u >= a.I) continue;
+                Pack<IO, VEC> out;
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) {
+                    float gx, gs, go;
+                    const float gr = load_f32(gin[u].v[k]), v = load_f32(xin[u].v[k]);
+                    if (fast) M::template bwd<true>(gr, v, e[k], a.gc, gx, gs, go);
+                    else M::template bwd<false>(gr, v, e[k], a.gc, gx, gs, go);
+                    out.v[k] = store_cast<IO>(gx);
+                    acc_s[k] += (double)gs;
+                    acc_o[k] += (double)go;
+                }
+                if (gxp) store_pack_stream<IO, VEC>(gxp + (r0 + u) * a.J + c0, out);
+            }
+        }
+    }
+    if (!want_pg) return;
+    // the waves take turns, so the sums do not depend on which wave finishes first
+    for (int w = 0; w < WAVES; ++w) {
+        if (wave == w && live) {
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) {
+                sums[(2 * k) * kWave + lane] += acc_s[k];
+                sums[(2 * k + 1) * kWave + lane] += acc_o[k];
+            }
+        }
+        __syncthreads();
+    }
+    if (wave == 0 && live) {
+        double* row = a.partials + 2 * (int64_t)blockIdx.y * a.J;
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) {
+            row[2 * (c0 + k)] = sums[(2 * k) * kWave + lane];
+            row[2 * (c0 + k) + 1] = sums[(2 * k + 1) * kWave + lane];
+        }
+    }
+}
+
+__global__ void zero_f64_kernel(double* p, int64_t n) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) p[i] = 0.0;
+}
+
+__global__ void finish_atomic_kernel(const double* acc, float* gscale, float* goffset, int64_t nenc, int cd) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < nenc; i += (int64_t)gridDim.x * blockDim.x) {
+        gscale[i] = finish_sum_rt(acc[2 * i], cd);
+        goffset[i] = finish_sum_rt(acc[2 * i + 1], cd);
+    }
+}
+
+
+// the column-walking backward kernel takes run length 1 whatever reduction the plan would otherwise use for it
+template <typename IO>
+static bool bwd_cols_layout(const Plan& p, bool aligned) {
+    return cols_layout<IO>(p, aligned) && (p.red == kRedAtomic || p.red == kRedRuns || p.red == kRedNone);
+}
+
+static bool bwd_cols_layout(int io_dtype, const Plan& p, bool aligned) {
+    return io_dtype == AHQ_F32 ? bwd_cols_layout<float>(p, aligned) : bwd_cols_layout<f16_t>(p, aligned);
+}
+
+// The backward kernel keeps eight encodings, sixteen double sums and two rows of two tensors per lane on a 16-bit
+// tensor: more than the 128 registers a workgroup of sixteen waves leaves a lane (36 of them were spilled: 92 us on
+// 8192 x 4096 bf16 with learned encodings; 73 us with eight waves, 62 us with four, 71 us with two).  float32:
+// 73.6 us with sixteen waves, 69.5 us with eight, 72 us with four.
+template <typename IO>
+constexpr int bwd_cols_waves() { return IoTraits<IO>::kVec > 4 ? kColWaves / 4 : kColWaves / 2; }
+
+template <typename IO>
+static dim3 bwd_cols_grid(const Plan& p) {
+    return cols_grid<IO>(p, 512 * (kColWaves / bwd_cols_waves<IO>()), bwd_cols_waves<IO>());
+}
+
+static unsigned bwd_cols_row_groups(int io_dtype, const Plan& p) {
+    return io_dtype == AHQ_F32 ? bwd_cols_grid<float>(p).y : bwd_cols_grid<f16_t>(p).y;
+}
+
+// pairs of doubles the backward pass needs as scratch for its parameter gradients
+static size_t bwd_scratch_pairs(int io_dtype, const Plan& p, bool aligned, bool want_pg) {
+    if (!want_pg) return 0;
+    if (bwd_cols_layout(io_dtype, p, aligned)) return (size_t)bwd_cols_row_groups(io_dtype, p) * (size_t)p.cl.J;
+    return p.ws_elems;
+}
+
+template <typename IO, typename M, int RED>
+static void launch_bwd_red(const Plan& p, const QdqArgs& a, hipStream_t st) {
+    if constexpr (RED == kRedTile) {
+        if (p.tile_vec == kBwdTileVec) {  // a whole row per tile, in kBwdRounds rounds (plan_bwd)
+            if (p.vec == 1) hipLaunchKernelGGL((qdq_bwd_kernel<IO, 1, M, RED, kBwdRounds>), dim3(p.nblocks), dim3(kBlock), 0, st, a);
+            else hipLaunchKernelGGL((qdq_bwd_kernel<IO, IoTraits<IO>::kVec, M, RED, kBwdRounds>), dim3(p.nblocks), dim3(kBlock), 0, st, a);
+            return;
+        }
+    }
+    if (p.vec == 1) {
+        hipLaunchKernelGGL((qdq_bwd_kernel<IO, 1, M, RED, 1>), dim3(p.nblocks), dim3(kBlock), 0, st, a);
+    } else {
+        hipLaunchKernelGGL((qdq_bwd_kernel<IO, IoTraits<IO>::kVec, M, RED, 1>), dim3(p.nblocks), dim3(kBlock), 0, st, a);
+    }
+}
+
+template <typename IO, typename M>
+static void launch_bwd(const Plan& p, const QdqArgs& a, hipStream_t st, bool aligned) {
+    if (bwd_cols_layout<IO>(p, aligned)) {
+        // few row groups: every workgroup ends with one row of partial sums
+        constexpr int W = bwd_cols_waves<IO>();
+        hipLaunchKernelGGL((qdq_bwd_cols_kernel<IO, IoTraits<IO>::kVec, M, W>), bwd_cols_grid<IO>(p), dim3(W * kWave), 0, st, a);
+        return;
+    }
+    if (p.cl.kind == kGeneric) {
+        hipLaunchKernelGGL((qdq_bwd_generic_kernel<IO, M>), dim3(p.nblocks), dim3(kBlock), 0, st, a);
+        return;
+    }
+    switch (p.red) {
+        case kRedNone: launch_bwd_red<IO, M, kRedNone>(p, a, st); break;
+        case kRedTile: launch_bwd_red<IO, M, kRedTile>(p, a, st); break;
+        case kRedSeg: launch_bwd_red<IO, M, kRedSeg>(p, a, st); break;
+        case kRedRuns: launch_bwd_red<IO, M, kRedRuns>(p, a, st); break;
+        default: launch_bwd_red<IO, M, kRedAtomic>(p, a, st); break;
+    }
+}
+
+}  // namespace ahq
+
+using namespace ahq;
+
+// The tiling of the backward pass: tiles of one round, of kBwdRounds rounds where a row then is one tile instead of two.
+static bool plan_bwd(int io_dtype, const ahq_layout& layout, bool aligned, bool want_pg, Plan* p) {
+    if (!make_plan(io_dtype, layout, aligned, want_pg, p, kBwdUnroll, true)) return false;
+    if (p->red == kRedTile && p->mode == kRows && p->tpr > 1 && p->tpr <= kBwdRounds) {
+        Plan q;
+        if (make_plan(io_dtype, layout, aligned, want_pg, &q, kBwdTileUnroll, true) && q.red == kRedTile &&
+            q.mode == kRows && q.tpr == 1)
+            *p = q;
+    }
+    return true;
+}
+
+extern "C" size_t ahq_qdq_backward_workspace_bytes(const ahq_grid* grid, const ahq_layout* layout, int want_param_grads) {
+    if (!grid || !layout) return 0;
+    const bool pg = want_param_grads != 0;
+    Plan p;
+    if (!plan_bwd(grid->io_dtype, *layout, true, pg, &p)) return 0;
+    size_t a = bwd_scratch_pairs(grid->io_dtype, p, true, pg) * 2 * sizeof(double);
+    // an unaligned tensor falls back to the scalar path whose strategy may need a different amount
+    Plan q;
+    if (plan_bwd(grid->io_dtype, *layout, false, pg, &q)) {
+        const size_t b = bwd_scratch_pairs(grid->io_dtype, q, false, pg) * 2 * sizeof(double);
+        if (b > a) a = b;
+    }
+    return a;
+}
+
+extern "C" int ahq_qdq_backward(const ahq_grid* grid, const ahq_layout* layout, const void* g, const void* x, void* gx,
+                                float* gscale, float* goffset, const float* scale, const float* offset, void* workspace,
+                                size_t workspace_bytes, void* stream) {
+    if (!validate_grid(grid, true)) return AHQ_ERR_INVALID;
+    if (!layout) return set_error("layout is null"), AHQ_ERR_INVALID;
+    if (!scale) return set_error("scale is null"), AHQ_ERR_INVALID;
+    if ((gscale == nullptr) != (goffset == nullptr)) return set_error("gscale and goffset must be given together"), AHQ_ERR_INVALID;
+    const bool want_pg = gscale != nullptr;
+    if (want_pg && grid->arith == AHQ_ARITH_ATEN) return set_error("the ATen arithmetic has no scale/offset gradient"), AHQ_ERR_INVALID;
+    Plan p;
+    const bool al = aligned16(x) && aligned16(g) && (!gx || aligned16(gx));
+    if (!plan_bwd(grid->io_dtype, *layout, al, want_pg, &p)) return AHQ_ERR_INVALID;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (p.cl.numel == 0) return AHQ_OK;  // nothing to read: outputs are left untouched
+    if (!x || !g) return set_error("x or g is null"), AHQ_ERR_INVALID;
+    if (!gx && !want_pg) return AHQ_OK;
+    const bool cols = bwd_cols_layout(grid->io_dtype, p, al);
+    const size_t ws_need = bwd_scratch_pairs(grid->io_dtype, p, al, want_pg) * 2 * sizeof(double);
+    if (ws_need > 0 && (!workspace || workspace_bytes < ws_need)) return set_error("workspace too small"), AHQ_ERR_WORKSPACE;
+    QdqArgs a{};
+    a.x = x;
+    a.g = g;
+    a.gx = gx;
+    a.scale = scale;
+    a.offset = offset;
+    a.gscale = gscale;
+    a.goffset = goffset;
+    a.partials = ws_need ? static_cast<double*>(workspace) : nullptr;
+    fill_args(*grid, p, &a);
+    const bool atomic = p.red == kRedAtomic && !cols;
+    if (atomic) {
+        const int64_t n = p.cl.num_enc * 2;
+        hipLaunchKernelGGL(zero_f64_kernel, dim3((unsigned)((n + 255) / 256 > 1024 ? 1024 : (n + 255) / 256)), dim3(256), 0, st, a.partials, n);
+    }
+    AHQ_IO_SWITCH(grid->io_dtype, AHQ_MATH_SWITCH(*grid, (launch_bwd<IO, M>(p, a, st, al))));
+    if (p.red == kRedTile) {
+        const int64_t per_enc = p.mode == kRows ? p.cl.I * (int64_t)p.tpr : (int64_t)p.nblocks;
+        if (per_enc > 1) {
+            const int64_t waves = kFinishThreads / kWave;
+            const int64_t nb = p.mode == kRows ? (p.cl.J + waves - 1) / waves : 1;
+            hipLaunchKernelGGL(qdq_bwd_finish_kernel, dim3((unsigned)(nb > 4096 ? 4096 : nb)), dim3(kFinishThreads), 0, st, a);
+        }
+    }
+    if (atomic) {
+        const int64_t n = p.cl.num_enc;
+        hipLaunchKernelGGL(finish_atomic_kernel, dim3((unsigned)((n + 255) / 256 > 1024 ? 1024 : (n + 255) / 256)), dim3(256), 0, st,
+                           (const double*)a.partials, gscale, goffset, n, (int)grid->compute_dtype);
+    }
+    if (want_pg && (cols || (p.red == kRedRuns && p.cl.I > 1))) {
+        // one slot per (row group, encoding) or per run: added up per encoding in a fixed order
+        const int64_t count = cols ? (int64_t)bwd_cols_row_groups(grid->io_dtype, p) : p.cl.I;
+        const int64_t nb = (p.cl.J + kBlock / kWave - 1) / (kBlock / kWave);
+        hipLaunchKernelGGL(qdq_bwd_strided_finish_kernel, dim3((unsigned)(nb > 4096 ? 4096 : nb)), dim3(kBlock), 0, st,
+                           (const double*)a.partials, count, p.cl.J, p.cl.J, gscale, goffset, (int)grid->compute_dtype);
+    }
+    return check_launch("ahq_qdq_backward");
+}

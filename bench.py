@@ -506,7 +506,8 @@ def run_qdq_workload(key, steps, warmup, dev, with_cpu_baseline=True, with_cache
                   "y_bit_exact": bool(torch.equal(y_a.cpu(), ref_a)),
                   "gx_bit_exact": bool(torch.equal(gx.cpu(), torch.where(mask_a, w["grad"], torch.zeros_like(w["grad"]))))}
         del y_a
-        bwd_on(sets[0])  # gx of the autograd arithmetic again, for the parity check below
+        fwd_on(sets[0])  # y and gx of the autograd arithmetic again, for the parity check below
+        bwd_on(sets[0])
 
     # ---- min/max calibration of the same tensor (one fused pass for both extrema) + the range it gives
     mm_ws_bytes = lib.ahq_minmax_workspace_bytes(layout)
