@@ -119,7 +119,10 @@ _SIGNATURES = {
                                                ctypes.c_int64, ctypes.c_double, ctypes.c_int32, _P, _P, _P, _P, _P]),
     "ahq_range_backward": (ctypes.c_int, [ctypes.c_int32, _P, _P, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
                                           ctypes.c_double, _P, _P, _P, _P, _P]),
-    "ahq_minmax_accumulate": (ctypes.c_int, [ctypes.c_int32, _P, ctypes.c_int64, _P, _P, ctypes.c_int32, _P]),
+    "ahq_minmax_accumulate": (ctypes.c_int, [ctypes.c_int32, _P, ctypes.c_int64, _P, _P, _P, ctypes.c_int32, _P]),
+    "ahq_minmax_slots_to_encodings": (ctypes.c_int, [ctypes.c_int32, _P, ctypes.c_int64, ctypes.c_int32, ctypes.c_float,
+                                                     ctypes.c_float, ctypes.c_float, ctypes.c_float, _P, _P, _P, _P, _P,
+                                                     _P]),
     "ahq_minmax_slots_read": (ctypes.c_int, [ctypes.c_int32, _P, _P, _P, _P]),
     "ahq_minmax_finalize": (ctypes.c_int, [ctypes.c_int32, _P, _P, ctypes.c_int64, ctypes.c_int64, ctypes.c_int32,
                                            ctypes.c_float, ctypes.c_float, ctypes.c_float, ctypes.c_float, _P,

@@ -13,6 +13,10 @@ constexpr int kBlock = 256;          // threads per workgroup = 4 waves of 64
 constexpr int kWave = 64;
 constexpr int kUnroll = 4;           // 16-byte vectors per thread per tile
 constexpr int kTileVec = kBlock * kUnroll;  // vectors per tile
+// Tensors of at least this many bytes are read with non-temporal loads by the kernels that take the hint: they do not
+// fit the caches anyway, and a streamed line that is not kept leaves room for what the rest of the step reads again.
+// Smaller tensors are often still resident from the kernel that produced them and keep the ordinary loads.
+constexpr long long kStreamLoadBytes = 32ll << 20;
 
 // ------------------------------------------------------------------------------------------------ storage types --
 struct f16_t { uint16_t bits; };

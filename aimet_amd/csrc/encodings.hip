@@ -189,13 +189,15 @@ __global__ void minmax_finalize_kernel(const EncArgs a, const FinalArgs f) {
 // NaN seen anywhere makes both statistics NaN, as torch.amin / amax would -- and its first thread goes on.
 constexpr int kSlotThreads = 256;
 
-template <typename T, typename P>
-__global__ __launch_bounds__(kSlotThreads) void minmax_slots_finalize_kernel(const float* slot_min, const float* slot_max,
-                                                                             const int* slot_nan, const EncArgs a,
-                                                                             const FinalArgs f) {
+// Folds the slots; true in the one thread that holds the result (mn, mx as values of the tensor's dtype T: what the
+// fold would have stored).
+template <typename T>
+__device__ __forceinline__ bool fold_slots(const float* slot_min, const float* slot_max, const int* slot_nan, float& mn,
+                                           float& mx) {
     __shared__ float red[kSlotThreads / kWave][2];
     __shared__ int red_nan[kSlotThreads / kWave];
-    float mn = __builtin_inff(), mx = -__builtin_inff();
+    mn = __builtin_inff();
+    mx = -__builtin_inff();
     int nan = 0;
     for (int q = threadIdx.x; q < AHQ_MINMAX_SLOTS; q += kSlotThreads) {
         mn = fminf(mn, slot_min[q]);
@@ -214,15 +216,40 @@ __global__ __launch_bounds__(kSlotThreads) void minmax_slots_finalize_kernel(con
         red_nan[threadIdx.x / kWave] = nan;
     }
     __syncthreads();
-    if (threadIdx.x != 0) return;
+    if (threadIdx.x != 0) return false;
     for (int w = 1; w < kSlotThreads / kWave; ++w) {
         mn = fminf(mn, red[w][0]);
         mx = fmaxf(mx, red[w][1]);
         nan |= red_nan[w];
     }
     const float qnan = __builtin_nanf("");
-    // the statistics as the fold would have stored them: values of the tensor's dtype
-    finalize_one<T, P>(a, f, 0, load_f32(store_cast<T>(nan ? qnan : mn)), load_f32(store_cast<T>(nan ? qnan : mx)));
+    mn = load_f32(store_cast<T>(nan ? qnan : mn));
+    mx = load_f32(store_cast<T>(nan ? qnan : mx));
+    return true;
+}
+
+template <typename T, typename P>
+__global__ __launch_bounds__(kSlotThreads) void minmax_slots_finalize_kernel(const float* slot_min, const float* slot_max,
+                                                                             const int* slot_nan, const EncArgs a,
+                                                                             const FinalArgs f) {
+    float mn, mx;
+    if (fold_slots<T>(slot_min, slot_max, slot_nan, mn, mx)) finalize_one<T, P>(a, f, 0, mn, mx);
+}
+
+// minmax_to_encodings_kernel for one encoding whose statistics lie in such slots; stat_min / stat_max (optional)
+// receive the folded statistics themselves.
+template <typename T>
+__global__ __launch_bounds__(kSlotThreads) void minmax_slots_to_encodings_kernel(const float* slot_min, const float* slot_max,
+                                                                                 const int* slot_nan, const EncArgs a,
+                                                                                 T* stat_min, T* stat_max) {
+    float mn, mx;
+    if (!fold_slots<T>(slot_min, slot_max, slot_nan, mn, mx)) return;
+    T lo_t, hi_t;
+    encode_range<T>(a, mn, mx, lo_t, hi_t);
+    static_cast<T*>(a.out_min)[0] = lo_t;
+    static_cast<T*>(a.out_max)[0] = hi_t;
+    if (stat_min) stat_min[0] = store_cast<T>(mn);
+    if (stat_max) stat_max[0] = store_cast<T>(mx);
 }
 
 template <typename T, typename P>
@@ -774,4 +801,31 @@ extern "C" int ahq_minmax_slots_finalize(int32_t stat_dtype, const void* slots, 
         default: launch_slots_finalize<bf16_t>(param_dtype, s, mn, mx, nan, a, f); break;
     }
     return check_launch("minmax_slots_finalize");
+}
+
+extern "C" int ahq_minmax_slots_to_encodings(int32_t dtype, const void* slots, int64_t num_steps, int32_t symmetric,
+                                             float minimum_scale_in_dtype, float minimum_scale, float dtype_max,
+                                             float near_max_threshold, void* out_min, void* out_max, void* stat_min,
+                                             void* stat_max, int32_t* flags, void* stream) {
+    if (!slots || (reinterpret_cast<uintptr_t>(slots) & 3u)) return set_error("slots is null or misaligned"), AHQ_ERR_INVALID;
+    EncArgs a{};
+    const int rc = fill_enc_args(&a, dtype, slots, slots, 1, num_steps, symmetric, minimum_scale_in_dtype, minimum_scale,
+                                 dtype_max, near_max_threshold, flags);
+    if (rc != AHQ_OK) return rc;
+    if (!out_min || !out_max) return set_error("null argument"), AHQ_ERR_INVALID;
+    a.smin = a.smax = nullptr;  // the statistics come from the slots
+    a.out_min = out_min;
+    a.out_max = out_max;
+    const char* w = static_cast<const char*>(slots);
+    const float* mn = reinterpret_cast<const float*>(w);
+    const float* mx = reinterpret_cast<const float*>(w + 4 * AHQ_MINMAX_SLOTS);
+    const int* nan = reinterpret_cast<const int*>(w + 8 * AHQ_MINMAX_SLOTS);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const dim3 g(1), b(kSlotThreads);
+    switch (dtype) {
+        case AHQ_F32: hipLaunchKernelGGL((minmax_slots_to_encodings_kernel<float>), g, b, 0, s, mn, mx, nan, a, static_cast<float*>(stat_min), static_cast<float*>(stat_max)); break;
+        case AHQ_F16: hipLaunchKernelGGL((minmax_slots_to_encodings_kernel<f16_t>), g, b, 0, s, mn, mx, nan, a, static_cast<f16_t*>(stat_min), static_cast<f16_t*>(stat_max)); break;
+        default: hipLaunchKernelGGL((minmax_slots_to_encodings_kernel<bf16_t>), g, b, 0, s, mn, mx, nan, a, static_cast<bf16_t*>(stat_min), static_cast<bf16_t*>(stat_max)); break;
+    }
+    return check_launch("minmax_slots_to_encodings");
 }

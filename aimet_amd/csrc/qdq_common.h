@@ -39,10 +39,6 @@ constexpr int kBwdRounds = 2;
 constexpr int kBwdTileUnroll = kBwdUnroll * kBwdRounds;
 constexpr int kBwdTileVec = kBlock * kBwdTileUnroll;
 constexpr int kStage = kBwdTileVec + 2;  // most encodings a tile can touch
-// Tensors of at least this many bytes are read with non-temporal loads: they do not fit the caches anyway, and a
-// streamed line that is not kept leaves room for what the rest of the step reads again.  Smaller tensors are often
-// still resident from the kernel that produced them and keep the ordinary loads.
-constexpr int64_t kStreamLoadBytes = (int64_t)32 << 20;
 
 struct GridC {
     float qmin, qmax, zps;

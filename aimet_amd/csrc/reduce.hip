@@ -53,6 +53,10 @@ struct MmFlatArgs : MmOut {
     // merges its result into its slot and nothing is folded; first: the slots hold nothing yet
     int32_t accumulate;
     int32_t first;
+    // accumulate, optional: slots of the same shape that receive this batch's own partials (nothing merged into them)
+    float* batch_min;
+    float* batch_max;
+    int* batch_nan;
 };
 
 // Arguments of the two lean kernels below (runs of whole vectors on the leading axis): a few words instead of the
@@ -64,6 +68,7 @@ struct MmRunArgs : MmOut {
     int64_t runs;      // number of encodings
     int32_t kv;        // vectors per run
     int32_t kv_shift;  // log2(kv) (segment kernel: kv is a power of two)
+    int32_t stream_loads;  // segment kernel: non-temporal loads (tensors too large to be resident in the caches)
 };
 
 struct MinMax {
@@ -347,12 +352,24 @@ __global__ __launch_bounds__(kFlatBlock) void minmax_flat_kernel(const MmFlatArg
             a.part_min[blockIdx.x] = s.mn;
             a.part_max[blockIdx.x] = s.mx;
             a.part_nan[blockIdx.x] = s.nan;
+            if (a.batch_min) {
+                a.batch_min[blockIdx.x] = b.mn;
+                a.batch_max[blockIdx.x] = b.mx;
+                a.batch_nan[blockIdx.x] = b.nan;
+            }
         }
-        if (a.first && blockIdx.x == 0) {
+        if (blockIdx.x == 0) {
             for (int q = gridDim.x + threadIdx.x; q < kFlatMaxBlocks; q += kFlatBlock) {
-                a.part_min[q] = __builtin_inff();
-                a.part_max[q] = -__builtin_inff();
-                a.part_nan[q] = 0;
+                if (a.first) {
+                    a.part_min[q] = __builtin_inff();
+                    a.part_max[q] = -__builtin_inff();
+                    a.part_nan[q] = 0;
+                }
+                if (a.batch_min) {
+                    a.batch_min[q] = __builtin_inff();
+                    a.batch_max[q] = -__builtin_inff();
+                    a.batch_nan[q] = 0;
+                }
             }
         }
         return;
@@ -428,6 +445,9 @@ __global__ __launch_bounds__(BLOCK) void minmax_runs_kernel(const MmRunArgs a) {
 // kSegUnroll vectors per lane; the lanes of a run combine with data-parallel moves, the run leaders leave their
 // results in LDS, and after one barrier consecutive lanes write consecutive encodings (whole cache lines instead of
 // one 2- or 4-byte store per run leader).
+// Loads: non-temporal for tensors of kStreamLoadBytes or more, which come from HBM whatever the caches hold (23.9 ->
+// about 20 us on a 117 MB bf16 weight that is not resident); ordinary ones below, where a tensor is often still in
+// the last-level cache from the kernel that wrote it and the ordinary load is the faster one (by 9 %).
 constexpr int kSegUnroll = 2;
 constexpr int kSegTileVec = kBlock * kSegUnroll;
 
@@ -446,7 +466,7 @@ __global__ __launch_bounds__(kBlock) void minmax_seg_kernel(const MmRunArgs a) {
 #pragma unroll
     for (int u = 0; u < kSegUnroll; ++u) {
         const int lv = u * kBlock + threadIdx.x;
-        if (lv < left) in[u] = load_pack<IO, VEC>(x + (int64_t)lv * VEC);
+        if (lv < left) in[u] = a.stream_loads ? load_pack_stream<IO, VEC>(x + (int64_t)lv * VEC) : load_pack<IO, VEC>(x + (int64_t)lv * VEC);
         else
 #pragma unroll
             for (int k = 0; k < VEC; ++k) in[u].v[k] = IO{};
@@ -596,6 +616,14 @@ static int64_t flat_blocks(const Plan& p) {
     return tiles < kFlatMaxBlocks ? tiles : kFlatMaxBlocks;
 }
 
+// Partial triples (min, max, saw-NaN: 12 bytes) a reduction keeps in its workspace: one per workgroup of the
+// single-encoding kernel (at most kFlatMaxBlocks, whatever the tensor's size), else what the plan says (one per tile
+// or per encoding).
+static size_t mm_ws_elems(const Plan& p) {
+    if (p.cl.kind == kIJK && p.cl.J == 1) return (size_t)flat_blocks(p);
+    return p.ws_elems;
+}
+
 static MmFlatArgs flat_args(const Plan& p, const MmArgs& a) {
     MmFlatArgs f{};
     static_cast<MmOut&>(f) = static_cast<const MmOut&>(a);
@@ -631,6 +659,7 @@ static void launch_mm(const Plan& p, const MmArgs& a, hipStream_t st) {
         r.kv = (int32_t)p.Kv;
         r.kv_shift = 0;
         while ((1 << r.kv_shift) < r.kv) ++r.kv_shift;
+        r.stream_loads = p.cl.numel * (int64_t)sizeof(IO) >= kStreamLoadBytes ? 1 : 0;
         constexpr int V = IoTraits<IO>::kVec;
         // a workgroup per run needs enough runs to fill the GPU, or runs short enough not to matter; a few very long
         // runs keep the tiled kernel with its partials
@@ -691,7 +720,7 @@ extern "C" __attribute__((visibility("hidden"))) int ahq_minmax_finite_partials(
     Plan p;
     if (dtype < AHQ_F32 || dtype > AHQ_BF16 || !layout || !make_plan(dtype, *layout, aligned16(x), true, &p) ||
         !(p.cl.kind == kIJK && p.cl.J == 1) || flat_blocks(p) <= 1 || !x || !workspace ||
-        workspace_bytes < p.ws_elems * 12)
+        workspace_bytes < mm_ws_elems(p) * 12)
         return ahq_minmax(dtype, layout, x, out_min, out_max, nullptr, nullptr, 1, workspace, workspace_bytes, stream);
     MmArgs a{};
     fill_geom(p, &a);
@@ -700,8 +729,8 @@ extern "C" __attribute__((visibility("hidden"))) int ahq_minmax_finite_partials(
     a.finite_only = 1;
     char* w = static_cast<char*>(workspace);
     a.part_min = reinterpret_cast<float*>(w);
-    a.part_max = reinterpret_cast<float*>(w + p.ws_elems * 4);
-    a.part_nan = reinterpret_cast<int*>(w + p.ws_elems * 8);
+    a.part_max = reinterpret_cast<float*>(w + mm_ws_elems(p) * 4);
+    a.part_nan = reinterpret_cast<int*>(w + mm_ws_elems(p) * 8);
     const int64_t nb = flat_blocks(p);
     hipStream_t st = static_cast<hipStream_t>(stream);
     const MmFlatArgs f = flat_args(p, a);
@@ -729,7 +758,7 @@ extern "C" size_t ahq_minmax_workspace_bytes(const ahq_layout* layout) {
     for (int dt = AHQ_F32; dt <= AHQ_BF16; ++dt)
         for (int al = 0; al < 2; ++al) {
             Plan p;
-            if (make_plan(dt, *layout, al != 0, true, &p) && p.ws_elems * 12 > need) need = p.ws_elems * 12;
+            if (make_plan(dt, *layout, al != 0, true, &p) && mm_ws_elems(p) * 12 > need) need = mm_ws_elems(p) * 12;
         }
     return need;
 }
@@ -745,7 +774,8 @@ static int minmax_impl(int32_t dtype, const ahq_layout* layout, const void* x, v
     if (!make_plan(dtype, *layout, aligned16(x) && aligned16(copy), true, &p)) return AHQ_ERR_INVALID;
     if (p.cl.numel == 0) return set_error("cannot reduce an empty tensor"), AHQ_ERR_INVALID;
     if (!x) return set_error("x is null"), AHQ_ERR_INVALID;
-    const size_t need = p.ws_elems * 12;
+    const size_t ws_elems = mm_ws_elems(p);
+    const size_t need = ws_elems * 12;
     const int64_t per_enc = p.red == kRedTile ? (p.mode == kRows ? p.cl.I * (int64_t)p.tpr : (int64_t)p.nblocks) : 0;
     const bool uses_ws = p.red == kRedAtomic || (p.red == kRedTile && per_enc > 1);
     if (uses_ws && (!workspace || workspace_bytes < need)) return set_error("workspace too small"), AHQ_ERR_WORKSPACE;
@@ -761,10 +791,10 @@ static int minmax_impl(int32_t dtype, const ahq_layout* layout, const void* x, v
     if (uses_ws) {
         char* w = static_cast<char*>(workspace);
         a.part_min = reinterpret_cast<float*>(w);
-        a.part_max = reinterpret_cast<float*>(w + p.ws_elems * 4);
-        a.part_nan = reinterpret_cast<int*>(w + p.ws_elems * 8);
+        a.part_max = reinterpret_cast<float*>(w + ws_elems * 4);
+        a.part_nan = reinterpret_cast<int*>(w + ws_elems * 8);
         a.key_min = reinterpret_cast<unsigned int*>(w);
-        a.key_max = reinterpret_cast<unsigned int*>(w + p.ws_elems * 4);
+        a.key_max = reinterpret_cast<unsigned int*>(w + ws_elems * 4);
     }
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (copy) {
@@ -815,14 +845,22 @@ static MmFlatArgs slot_args(void* slots) {
 }
 
 extern "C" int ahq_minmax_accumulate(int32_t dtype, const void* x, int64_t count, void* copy_to, void* slots,
-                                     int32_t first, void* stream) {
+                                     void* batch_slots, int32_t first, void* stream) {
     if (dtype < AHQ_F32 || dtype > AHQ_BF16) return set_error("bad dtype"), AHQ_ERR_INVALID;
     if (count < 0) return set_error("negative element count"), AHQ_ERR_INVALID;
     if (!slots || (reinterpret_cast<uintptr_t>(slots) & 3u)) return set_error("slots is null or misaligned"), AHQ_ERR_INVALID;
+    if (batch_slots && ((reinterpret_cast<uintptr_t>(batch_slots) & 3u) || batch_slots == slots))
+        return set_error("batch_slots is misaligned or aliases slots"), AHQ_ERR_INVALID;
     if (count > 0 && !x) return set_error("x is null"), AHQ_ERR_INVALID;
     if (copy_to && copy_to == x) return set_error("copy_to must not alias x"), AHQ_ERR_INVALID;
-    if (count == 0 && !first) return AHQ_OK;  // nothing to add; an empty first batch still clears the slots
+    if (count == 0 && !first && !batch_slots) return AHQ_OK;  // nothing to add; an empty first batch still clears the slots
     MmFlatArgs f = slot_args(slots);
+    if (batch_slots) {
+        const MmFlatArgs b = slot_args(batch_slots);
+        f.batch_min = b.part_min;
+        f.batch_max = b.part_max;
+        f.batch_nan = b.part_nan;
+    }
     f.x = x;
     f.copy = copy_to;
     f.numel = count;
@@ -897,7 +935,7 @@ extern "C" int ahq_minmax_static(int32_t dtype, const ahq_layout* layout, const 
     // the size check comes first and needs no device: the plan is host arithmetic
     Plan p;
     if (!make_plan(dtype, *layout, aligned16(x), true, &p)) return AHQ_ERR_INVALID;
-    const size_t need = p.ws_elems * 12;
+    const size_t need = mm_ws_elems(p) * 12;
     if (need > kStaticScratchBytes) {
         std::snprintf(error_buffer(), 512,
                       "ahq_minmax_static: this reduction needs %zu bytes of scratch, the static buffer holds %zu; "

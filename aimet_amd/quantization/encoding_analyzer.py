@@ -30,10 +30,82 @@ from aimet_amd.quantization._stats import reduce_min_max, _check_reducible
 from aimet_amd.quantization.affine.backends.hip import _prepare
 
 
-@dataclass
 class _MinMaxRange:
-    min: Optional[torch.Tensor] = None
-    max: Optional[torch.Tensor] = None
+    """The reference's ``_MinMaxRange(min, max)`` (encoding_analyzer.py:46-50).  A single encoding's statistics may
+    still lie in the per-workgroup slots of the streaming kernel (``from_slots``): ``min`` / ``max`` fold them when they
+    are first read, and a consumer that takes slots (MinMaxEncodingAnalyzer.compute_encodings_from_stats, the end of
+    a quantizer's calibration) folds them inside its own launch, so that nothing is launched for statistics nobody
+    reads."""
+
+    __slots__ = ("_min", "_max", "_slots", "_of")
+
+    def __init__(self, min: Optional[torch.Tensor] = None, max: Optional[torch.Tensor] = None):
+        self._min, self._max, self._slots, self._of = min, max, None, None
+
+    @classmethod
+    def from_slots(cls, slots: torch.Tensor, dtype, device, shape) -> "_MinMaxRange":
+        r = cls()
+        r._slots, r._of = slots, (dtype, device, tuple(shape))
+        return r
+
+    def unfolded(self):
+        """(dtype, device, shape, slot buffer) while the statistics have not been folded, else None."""
+        return (*self._of, self._slots) if self._slots is not None else None
+
+    def adopt(self, mn: torch.Tensor, mx: torch.Tensor) -> None:
+        """The folded statistics, from the launch of a consumer that formed them on its way."""
+        self._min, self._max, self._slots = mn, mx, None
+
+    def _fold(self) -> None:
+        if self._slots is None:
+            return
+        dtype, device, shape = self._of
+        mn = torch.empty(shape, dtype=dtype, device=device)
+        mx = torch.empty(shape, dtype=dtype, device=device)
+        _lib.check(_lib.load().ahq_minmax_slots_read(_lib.DTYPE_CODE[dtype], self._slots.data_ptr(), mn.data_ptr(),
+                                                     mx.data_ptr(), _lib.current_stream(device)),
+                   "ahq_minmax_slots_read")
+        self.adopt(mn, mx)
+
+    @property
+    def min(self) -> Optional[torch.Tensor]:
+        self._fold()
+        return self._min
+
+    @min.setter
+    def min(self, value):
+        self._fold()
+        self._min = value
+
+    @property
+    def max(self) -> Optional[torch.Tensor]:
+        self._fold()
+        return self._max
+
+    @max.setter
+    def max(self, value):
+        self._fold()
+        self._max = value
+
+    def is_empty(self) -> bool:
+        """Nothing observed (without folding anything)."""
+        return self._slots is None and self._min is None and self._max is None
+
+    def __eq__(self, other):
+        return isinstance(other, _MinMaxRange) and self.min is other.min and self.max is other.max
+
+    __hash__ = None
+
+    def __repr__(self):
+        return f"_MinMaxRange(min={self.min!r}, max={self.max!r})"
+
+    def __getstate__(self):
+        self._fold()
+        return (self._min, self._max)
+
+    def __setstate__(self, state):
+        self._min, self._max = state
+        self._slots = self._of = None
 
 
 @dataclass
@@ -123,28 +195,33 @@ class _MinMaxObserver(_Observer[_MinMaxRange]):
     def __init__(self, shape, block_size=None):
         super().__init__(shape, block_size)
         self.stats = _MinMaxRange()
-        # A single encoding observed through observe_and_clone() keeps its running extrema as one slot per workgroup
-        # of the streaming kernel (ahq_minmax_accumulate): no second launch per batch; the slots are folded into
-        # `stats` when somebody asks (get_stats, or any of the other ways of adding statistics, which then take over).
+        # A single encoding keeps its running extrema as one slot per workgroup of the streaming kernel
+        # (ahq_minmax_accumulate): one launch per batch, no launch that folds a batch's partials.  The batch's own
+        # extrema come back as slots of their own (a _MinMaxRange that folds them if they are read), and `stats`
+        # becomes a view of the running slots when somebody asks for it (get_stats), folded at the latest before the
+        # next batch changes the slots.  Any other way of adding statistics (merge_stats, tensors the streaming
+        # kernel does not take) folds the slots into `stats` and takes over.
         self._single = math.prod(self.shape) == 1 and not block_size
         self._slots = None         # the slot buffer, kept across reset_stats()
         self._slots_of = None      # (dtype, device) of the tensors accumulated while the slots are live, else None
         self._slots_dirty = False  # the slots hold more than `stats`
 
+    def _stats_view_live(self) -> bool:
+        """`stats` is an unfolded view of the running slots."""
+        u = self.stats.unfolded()
+        return u is not None and u[3] is self._slots
+
     def _fold_slots(self):
+        """`stats` = everything the slots hold, as tensors."""
         if self._slots_of is not None and self._slots_dirty:
-            dtype, device = self._slots_of
-            mn = torch.empty(self.shape, dtype=dtype, device=device)
-            mx = torch.empty(self.shape, dtype=dtype, device=device)
-            _lib.check(_lib.load().ahq_minmax_slots_read(_lib.DTYPE_CODE[dtype], self._slots.data_ptr(), mn.data_ptr(),
-                                                         mx.data_ptr(), _lib.current_stream(device)),
-                       "ahq_minmax_slots_read")
-            self.stats = _MinMaxRange(mn, mx)
+            self.stats = _MinMaxRange.from_slots(self._slots, *self._slots_of, self.shape)
             self._slots_dirty = False
+        if self._stats_view_live():
+            self.stats._fold()  # pylint: disable=protected-access
 
     def live_slots(self):
-        """(dtype, device, slot buffer) while the slots hold running extrema that `stats` does not, else None."""
-        if self._slots_of is not None and self._slots_dirty:
+        """(dtype, device, slot buffer) while the running extrema lie in the slots and nowhere else, else None."""
+        if self._slots_of is not None and (self._slots_dirty or self._stats_view_live()):
             return (*self._slots_of, self._slots)
         return None
 
@@ -152,6 +229,33 @@ class _MinMaxObserver(_Observer[_MinMaxRange]):
         """`stats` becomes the one place the running extrema live in."""
         self._fold_slots()
         self._slots_of = None
+
+    def _takes_slots(self, x: torch.Tensor) -> bool:
+        return (self._single and x.is_cuda and x.dtype in _lib.DTYPE_CODE and x.is_contiguous() and x.numel() > 0
+                and len(self.shape) <= x.dim())
+
+    def _accumulate(self, x: torch.Tensor, copy_to: Optional[torch.Tensor], want_batch: bool):
+        """One launch: the batch folded into the running slots, its copy written if asked for, its own extrema left
+        in slots of their own if asked for.  False when the running statistics do not lie in slots of this dtype and
+        device (the caller then takes the general route)."""
+        of = (x.dtype, x.device)
+        first = self._slots_of is None and self.stats.is_empty()
+        if not (first or self._slots_of == of):
+            return False
+        if self._stats_view_live():
+            self.stats._fold()  # pylint: disable=protected-access  (a view handed out earlier keeps what it saw)
+        if self._slots is None or self._slots.device != x.device:
+            self._slots = torch.empty(_lib.MINMAX_SLOTS_BYTES, dtype=torch.uint8, device=x.device)
+        batch = torch.empty(_lib.MINMAX_SLOTS_BYTES, dtype=torch.uint8, device=x.device) if want_batch else None
+        status = _lib.load().ahq_minmax_accumulate(_lib.DTYPE_CODE[x.dtype], x.data_ptr(), x.numel(),
+                                                   None if copy_to is None else copy_to.data_ptr(),
+                                                   self._slots.data_ptr(), None if batch is None else batch.data_ptr(),
+                                                   1 if first else 0, _lib.current_stream(x.device))
+        if status:
+            _lib.check(status, "ahq_minmax_accumulate")
+        self._slots_of = of
+        self._slots_dirty = True
+        return _MinMaxRange.from_slots(batch, x.dtype, x.device, self.shape) if want_batch else True
 
     @torch.no_grad()
     def collect_stats(self, input_tensor: torch.Tensor) -> _MinMaxRange:
@@ -172,6 +276,12 @@ class _MinMaxObserver(_Observer[_MinMaxRange]):
     def update(self, input_tensor: torch.Tensor, copy_to: Optional[torch.Tensor] = None) -> _MinMaxRange:
         """collect + merge in one launch: the running fold happens where the reduction finishes.  ``copy_to``
         receives a copy of the input from the same pass (what pass-through calibration returns)."""
+        x = input_tensor
+        if self._takes_slots(x) and (copy_to is None or (copy_to.dtype == x.dtype and copy_to.device == x.device
+                                                         and copy_to.shape == x.shape and copy_to.is_contiguous())):
+            batch = self._accumulate(x.detach(), copy_to, True)
+            if batch is not False:
+                return batch
         self._leave_slots()
         cur = self.stats
         fused = (
@@ -195,21 +305,9 @@ class _MinMaxObserver(_Observer[_MinMaxRange]):
         exist, everything that does not change from call to call -- layout, workspace, the two tensors the batch's
         extrema are written to -- is kept, and a call is one allocation (the copy) and one library call."""
         x = input_tensor
-        if (self._single and x.is_cuda and x.dtype in _lib.DTYPE_CODE and x.is_contiguous() and not x.requires_grad
-                and x.numel() > 0 and len(self.shape) <= x.dim()):
-            of = (x.dtype, x.device)
-            first = self._slots_of is None and self.stats.min is None and self.stats.max is None
-            if first or self._slots_of == of:
-                if self._slots is None or self._slots.device != x.device:
-                    self._slots = torch.empty(_lib.MINMAX_SLOTS_BYTES, dtype=torch.uint8, device=x.device)
-                out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
-                status = _lib.load().ahq_minmax_accumulate(_lib.DTYPE_CODE[x.dtype], x.data_ptr(), x.numel(),
-                                                           out.data_ptr(), self._slots.data_ptr(), 1 if first else 0,
-                                                           _lib.current_stream(x.device))
-                if status:
-                    _lib.check(status, "ahq_minmax_accumulate")
-                self._slots_of = of
-                self._slots_dirty = True
+        if self._takes_slots(x) and not x.requires_grad:
+            out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+            if self._accumulate(x, out, False) is not False:
                 return out
         self._leave_slots()
         fast = self.__dict__.get("_fast")
@@ -248,7 +346,11 @@ class _MinMaxObserver(_Observer[_MinMaxRange]):
         self.__dict__["_fast"] = None
 
     def get_stats(self) -> _MinMaxRange:
-        self._fold_slots()
+        if self._slots_of is not None and self._slots_dirty:
+            # a view of the running slots: folded when it is read, or inside the launch of a consumer that takes
+            # slots, and at the latest before the next batch changes them
+            self.stats = _MinMaxRange.from_slots(self._slots, *self._slots_of, self.shape)
+            self._slots_dirty = False
         return self.stats
 
 
@@ -430,7 +532,7 @@ class MinMaxEncodingAnalyzer(EncodingAnalyzer[_MinMaxRange]):
     def compute_encodings_from_stats(self, stats: _MinMaxRange, num_steps: int, is_symmetric: bool):
         if num_steps <= 0:
             raise ValueError("The number of quantization bins cannot be less than or equal to 0.")
-        if stats.min is None or stats.max is None:
+        if stats.is_empty() or (stats.unfolded() is None and (stats.min is None or stats.max is None)):
             raise StatisticsNotFoundError("No statistics present to compute encodings.")
 
         fused = self._fused_encodings(stats, num_steps, is_symmetric)
@@ -461,7 +563,26 @@ class MinMaxEncodingAnalyzer(EncodingAnalyzer[_MinMaxRange]):
     @staticmethod
     def _fused_encodings(stats: _MinMaxRange, num_steps: int, is_symmetric: bool):
         """The arithmetic below in one kernel launch (ahq_minmax_to_encodings); None when the statistics are not a
-        pair of same-shaped 16/32-bit float tensors, in which case the elementwise formulation runs."""
+        pair of same-shaped 16/32-bit float tensors, in which case the elementwise formulation runs.  Statistics that
+        still lie in the streaming kernel's slots are folded by the same launch (ahq_minmax_slots_to_encodings)."""
+        slots = stats.unfolded()
+        if slots is not None and 0 < num_steps <= (1 << 24) and num_steps == int(num_steps):
+            dt, device, shape, buf = slots
+            num_steps = int(num_steps)
+            consts = _scalar_constants(dt, _get_minimum_scale(num_steps))
+            out = torch.empty((4,) + tuple(shape), dtype=dt, device=device)  # lo, hi and the folded statistics
+            flags = torch.zeros(2, dtype=torch.int32, device=device)
+            base, step = out.data_ptr(), out.element_size()
+            status = _lib.load().ahq_minmax_slots_to_encodings(
+                _lib.DTYPE_CODE[dt], buf.data_ptr(), num_steps, 1 if is_symmetric else 0, consts[0], consts[1],
+                consts[2], consts[3], base, base + step, base + 2 * step, base + 3 * step, flags.data_ptr(),
+                _lib.current_stream(device))
+            if status:
+                _lib.check(status, "ahq_minmax_slots_to_encodings")
+            lo, hi = out[0], out[1]
+            stats.adopt(out[2], out[3])
+            lo._ahq_range_flags = hi._ahq_range_flags = flags  # pylint: disable=protected-access
+            return lo, hi
         mn, mx = stats.min, stats.max
         if (mn.dtype not in _lib.DTYPE_CODE or mx.dtype != mn.dtype or mn.shape != mx.shape or not mn.is_cuda
                 or num_steps > (1 << 24) or num_steps != int(num_steps)):

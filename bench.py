@@ -547,10 +547,10 @@ def run_qdq_workload(key, steps, warmup, dev, with_cpu_baseline=True, with_cache
     running = None
     if E == 1:
         slots = torch.empty(_lib.MINMAX_SLOTS_BYTES, dtype=torch.uint8, device=dev)
-        lib.ahq_minmax_accumulate(code, x.data_ptr(), n_elems := x.numel(), None, slots.data_ptr(), 1, stream)
+        lib.ahq_minmax_accumulate(code, x.data_ptr(), n_elems := x.numel(), None, slots.data_ptr(), None, 1, stream)
 
         def accumulate_on(t):
-            _lib.check(lib.ahq_minmax_accumulate(code, t.data_ptr(), n_elems, None, slots.data_ptr(), 0, stream),
+            _lib.check(lib.ahq_minmax_accumulate(code, t.data_ptr(), n_elems, None, slots.data_ptr(), None, 0, stream),
                        "minmax accumulate")
 
         x_copies = [t[0] for t in sets]  # the running extrema must stay those of x
@@ -562,6 +562,20 @@ def run_qdq_workload(key, steps, warmup, dev, with_cpu_baseline=True, with_cache
 
         # (the outputs y hold quantize-dequantized x: inside x's range, so they leave the running extrema alone)
         t_acc = event_time(accumulate, reps)
+        # what _MinMaxObserver.update() launches per batch: the same with the batch's own extrema left in a second
+        # slot array (update_stats() returns them; they are folded when somebody reads them)
+        own = torch.empty(_lib.MINMAX_SLOTS_BYTES, dtype=torch.uint8, device=dev)
+
+        def observe():
+            acc_turn[0] = k = (acc_turn[0] + 1) % (2 * rot)
+            t = x_copies[k % rot] if k < rot else sets[k - rot][1]
+            _lib.check(lib.ahq_minmax_accumulate(code, t.data_ptr(), n_elems, None, slots.data_ptr(), own.data_ptr(), 0,
+                                                 stream), "minmax accumulate")
+
+        t_obs = event_time(observe, reps)
+        b_mn, b_mx = torch.empty_like(mn_out), torch.empty_like(mx_out)
+        lib.ahq_minmax_accumulate(code, x.data_ptr(), n_elems, None, slots.data_ptr(), own.data_ptr(), 0, stream)
+        _lib.check(lib.ahq_minmax_slots_read(code, own.data_ptr(), b_mn.data_ptr(), b_mx.data_ptr(), stream), "read")
         if with_cached:
             mm_cached["running_us"] = round(event_time(lambda: accumulate_on(x), reps) * 1e6, 2)
         r_mn, r_mx = torch.empty_like(mn_out), torch.empty_like(mx_out)
@@ -570,7 +584,13 @@ def run_qdq_workload(key, steps, warmup, dev, with_cpu_baseline=True, with_cache
                    "us": round(t_acc * 1e6, 2), "GBps": round(x.element_size() * n_elems / t_acc / 1e9, 1),
                    "frac_of_hbm_peak": round(x.element_size() * n_elems / t_acc / 1e9 / HBM_PEAK_GBS, 4),
                    "bit_exact": bool(torch.equal(r_mn.cpu(), mn_ref.view(r_mn.shape))
-                                     and torch.equal(r_mx.cpu(), mx_ref.view(r_mx.shape)))}
+                                     and torch.equal(r_mx.cpu(), mx_ref.view(r_mx.shape))),
+                   "with_the_batch_extrema_in_slots_of_their_own": {
+                       "what": "the launch of MinMaxEncodingAnalyzer.update_stats() on a per-tensor analyzer",
+                       "us": round(t_obs * 1e6, 2),
+                       "frac_of_hbm_peak": round(x.element_size() * n_elems / t_obs / 1e9 / HBM_PEAK_GBS, 4),
+                       "bit_exact": bool(torch.equal(b_mn.cpu(), mn_ref.view(b_mn.shape))
+                                         and torch.equal(b_mx.cpu(), mx_ref.view(b_mx.shape)))}}
     exact_mm = bool(torch.equal(mn_out.cpu(), mn_ref.view(mn_out.shape)) and torch.equal(mx_out.cpu(), mx_ref.view(mx_out.shape)))
 
     # ---- the same step through the drop-in module: QuantizeDequantize.forward + autograd backward
@@ -594,6 +614,12 @@ def run_qdq_workload(key, steps, warmup, dev, with_cpu_baseline=True, with_cache
     mod_steps = max(steps, 200)
     mod_loop, mod_repeats = timed_steps(module_step, mod_steps, min(warmup, 5))
     mod_s = mod_loop / mod_steps
+    # the same loop with autograd's engine running the backward pass on the calling thread: by default PyTorch hands
+    # the backward pass of a GPU tensor to a worker thread and the caller sleeps until it is done, two thread wake-ups
+    # per step that cost more than the kernels on most hosts
+    with torch.autograd.set_multithreading_enabled(False):
+        st_loop, _ = timed_steps(module_step, mod_steps, min(warmup, 5))
+    mod_st = st_loop / mod_steps
     mod_cached = None
     if with_cached:
         mc_loop, _ = timed_steps(lambda: module_step_on(0), mod_steps, min(warmup, 5))
@@ -656,7 +682,10 @@ def run_qdq_workload(key, steps, warmup, dev, with_cpu_baseline=True, with_cache
     out.update({
         "elements_per_s": round(n / sec_per_step, 1),
         "kernels": kernels,
-        "calibration": {"kernel": "ahq_minmax (both extrema in one pass)", "us": round(t_mm * 1e6, 2),
+        "calibration": {"kernel": "ahq_minmax (both extrema in one pass"
+                                  + ("; two launches for a single encoding: stream + fold of the partials; the "
+                                     "analyzers use the one-launch form under 'running')" if E == 1 else ")"),
+                        "us": round(t_mm * 1e6, 2),
                         "GBps": round((S * n + 2 * S * E) / t_mm / 1e9, 1),
                         "elements_per_s": round(n / t_mm, 1),
                         "frac_of_hbm_peak": round((S * n) / t_mm / 1e9 / HBM_PEAK_GBS, 4),
@@ -670,7 +699,12 @@ def run_qdq_workload(key, steps, warmup, dev, with_cpu_baseline=True, with_cache
                                 "autograd and the per-call scale / offset derivation included)",
                         "ms_per_step": round(mod_s * 1e3, 5), "GBps": round(bytes_step / mod_s / 1e9, 1),
                         "frac_of_hbm_peak": round(bytes_step / mod_s / 1e9 / HBM_PEAK_GBS, 4), "repeats": mod_repeats,
-                        "steps_per_timed_loop": mod_steps, **host,
+                        "steps_per_timed_loop": mod_steps,
+                        "autograd_on_the_calling_thread": {
+                            "what": "the same loop inside torch.autograd.set_multithreading_enabled(False)",
+                            "ms_per_step": round(mod_st * 1e3, 5), "GBps": round(bytes_step / mod_st / 1e9, 1),
+                            "frac_of_hbm_peak": round(bytes_step / mod_st / 1e9 / HBM_PEAK_GBS, 4)},
+                        **host,
                         **({"same_tensor_again_and_again_ms_per_step": mod_cached} if mod_cached is not None else {})},
         "parity": parity,
         "roofline": {"bound": "hbm", "kernel": dom[0], "achieved": round(dom[2] / dom[1] / 1e9, 1),

@@ -150,7 +150,7 @@ int    ahq_minmax_copy(int32_t dtype, const ahq_layout* layout, const void* x, v
  * The call allocates nothing (no hipMalloc / hipFree, no allocating library routine); the first call on a device
  * looks the array's address up (hipGetSymbolAddress), so make that call outside a capture.
  * A reduction whose ahq_minmax_workspace_bytes() exceeds the array returns AHQ_ERR_WORKSPACE and launches nothing
- * (12 bytes per 4096-element tile of a per-tensor reduction, 12 bytes per encoding otherwise).
+ * (a per-tensor reduction needs 6 KB whatever its size; others 12 bytes per encoding or per tile).
  * All calls on one device share the array: calls that overlap on one device (different streams) race; calls on one
  * stream are ordered and each clears what it needs.
  */
@@ -163,13 +163,17 @@ int    ahq_minmax_static(int32_t dtype, const ahq_layout* layout, const void* x,
  * the caller does not need the statistics between batches: `slots` (AHQ_MINMAX_SLOTS_BYTES bytes, 4-byte aligned,
  * owned by the caller) holds one (min, max, saw-NaN) triple per workgroup of the streaming kernel; each call folds the
  * batch into them in place (minimum and maximum are exact in any order and grouping), `first` != 0 starts them
- * afresh.  copy_to (optional) receives a copy of the `count` elements of x from the same pass.  ahq_minmax_slots_read
- * folds the slots into one (min, max) of `dtype`, with torch.amin / amax semantics (NaN if any element was NaN).
+ * afresh.  copy_to (optional) receives a copy of the `count` elements of x from the same pass.  batch_slots
+ * (optional, a second array of the same size that must not alias `slots`) receives the batch's OWN partial extrema,
+ * written, not merged: what update_stats() returns (the statistics of this tensor alone, :369-374) without a launch
+ * that folds them.  ahq_minmax_slots_read folds either array into one (min, max) of `dtype`, with torch.amin / amax
+ * semantics (NaN if any element was NaN); ahq_minmax_slots_to_encodings and ahq_minmax_slots_finalize fold them inside
+ * the launch that consumes them.
  */
 #define AHQ_MINMAX_SLOTS 512
 #define AHQ_MINMAX_SLOTS_BYTES (12 * AHQ_MINMAX_SLOTS)
-int ahq_minmax_accumulate(int32_t dtype, const void* x, int64_t count, void* copy_to, void* slots, int32_t first,
-                          void* stream);
+int ahq_minmax_accumulate(int32_t dtype, const void* x, int64_t count, void* copy_to, void* slots, void* batch_slots,
+                          int32_t first, void* stream);
 int ahq_minmax_slots_read(int32_t dtype, const void* slots, void* out_min, void* out_max, void* stream);
 
 /* Replaces MinMaxEncodingAnalyzer.compute_encodings_from_stats (AT/quantization/encoding_analyzer.py:425-481) and the
@@ -185,6 +189,16 @@ int ahq_minmax_to_encodings(int32_t dtype, const void* stat_min, const void* sta
                             int64_t num_steps, int32_t symmetric, float minimum_scale_in_dtype, float minimum_scale,
                             float dtype_max, float near_max_threshold, void* out_min, void* out_max, int32_t* flags,
                             void* stream);
+
+/* ahq_minmax_to_encodings for one encoding whose statistics lie in the slots of ahq_minmax_accumulate (the running
+ * ones or a batch's own): the launch folds the slots as ahq_minmax_slots_read would and goes on from there, so a
+ * per-tensor analyzer's update_stats() + compute_encodings() are two launches, not four.  stat_min / stat_max
+ * (optional, one value of `dtype` each) receive the folded statistics.  The slots are only read.
+ */
+int ahq_minmax_slots_to_encodings(int32_t dtype, const void* slots, int64_t num_steps, int32_t symmetric,
+                                  float minimum_scale_in_dtype, float minimum_scale, float dtype_max,
+                                  float near_max_threshold, void* out_min, void* out_max, void* stat_min,
+                                  void* stat_max, int32_t* flags, void* stream);
 
 /* Replaces AffineQuantizerBase.get_scale / _get_offset with dtype = float32 for a quantizer that holds min / max
  * (AT/quantization/affine/quantizer.py:319-376), the half-dozen elementwise launches a quantizer spends on its first

@@ -556,14 +556,30 @@ def test_per_tensor_extrema_kept_as_slots(device, dtype, shape):
             assert_same_bits(st.min.reshape(()), lo, f"min after batch {i}")
             assert_same_bits(st.max.reshape(()), hi, f"max after batch {i}")
     assert an.observer._slots_of is not None  # the slots stayed the running statistics throughout
-    # the other ways of adding statistics take over from the slots and carry on from their content
+    # update_stats() goes the same way and hands back the batch's own extrema, which fold when they are read
     extra = (torch.randn(1000, generator=g) * 50).to(dtype).to(device)
-    an.update_stats(extra)
-    assert an.observer._slots_of is None
+    own = an.update_stats(extra)
+    assert an.observer._slots_of is not None and own.unfolded() is not None
+    assert_same_bits(own.min.reshape(()), extra.amin(), "the batch's own min")
+    assert_same_bits(own.max.reshape(()), extra.amax(), "the batch's own max")
+    assert own.unfolded() is None and own.min.shape == shape
     lo, hi = torch.minimum(lo, extra.amin()), torch.maximum(hi, extra.amax())
+    # a view of the running statistics handed out before a batch keeps what it saw
+    view = an.observer.get_stats()
+    assert view.unfolded() is not None
+    more = (torch.randn(3000, generator=g) * 80).to(dtype).to(device)
+    an.update_stats(more)
+    assert_same_bits(view.min.reshape(()), lo, "view taken before the batch: min")
+    assert_same_bits(view.max.reshape(()), hi, "view taken before the batch: max")
+    lo, hi = torch.minimum(lo, more.amin()), torch.maximum(hi, more.amax())
+    # the other ways of adding statistics take over from the slots and carry on from their content
+    last = (torch.randn(500, generator=g) * 200).to(dtype).to(device)
+    an.observer.merge_stats(an.observer.collect_stats(last))
+    assert an.observer._slots_of is None
+    lo, hi = torch.minimum(lo, last.amin()), torch.maximum(hi, last.amax())
     st = an.observer.get_stats()
-    assert_same_bits(st.min.reshape(()), lo, "min after update_stats")
-    assert_same_bits(st.max.reshape(()), hi, "max after update_stats")
+    assert_same_bits(st.min.reshape(()), lo, "min after merge_stats")
+    assert_same_bits(st.max.reshape(()), hi, "max after merge_stats")
     y = an.observe_and_clone(extra * 2)   # statistics exist outside the slots: the running-tensor form continues
     assert an.observer._slots_of is None and torch.equal(y, extra * 2)
     st = an.observer.get_stats()

@@ -91,12 +91,45 @@ def test_static_scratch_folds_running_statistics(device):
 def test_static_scratch_rejects_reductions_beyond_its_size():
     """Host-side check, no GPU needed: the plan is pure arithmetic and the refusal comes before any HIP call."""
     lib = _lib.load()
-    n = (SCRATCH_BYTES // 12 + 1) * 4096  # one tile more than the scratch has partials for
-    lay = _lib.make_layout([n], [n], [0])
+    enc = SCRATCH_BYTES // 12 + 1
+    lay = _lib.make_layout([enc, 40], [1, 40], [1, 0])  # per-channel with short rows: 12 bytes per encoding
     assert lib.ahq_minmax_workspace_bytes(lay) > SCRATCH_BYTES
     rc = lib.ahq_minmax_static(_lib.AHQ_F32, lay, 16, 16, 16, None, None, 0, None)
     assert rc == _lib.AHQ_ERR_WORKSPACE
     assert b"static buffer" in lib.ahq_last_error()
-    enc = SCRATCH_BYTES // 12 + 1
-    lay = _lib.make_layout([enc, 40], [1, 40], [1, 0])  # per-channel with short rows: 12 bytes per encoding
+    rows = SCRATCH_BYTES // 12 // 3 + 1
+    lay = _lib.make_layout([rows, 3 * 4096], [1, 3 * 4096], [1, 0])  # long rows: one partial per tile of each row
     assert lib.ahq_minmax_static(_lib.AHQ_F32, lay, 16, 16, 16, None, None, 0, None) == _lib.AHQ_ERR_WORKSPACE
+    # a per-tensor reduction keeps one partial per workgroup of its streaming kernel, 6 KB whatever the size: never
+    # refused for its size (the null pointers are what this call is refused for)
+    n = 1 << 36
+    lay = _lib.make_layout([n], [n], [0])
+    assert lib.ahq_minmax_workspace_bytes(lay) == 512 * 12
+    assert lib.ahq_minmax_static(_lib.AHQ_F32, lay, None, None, None, None, None, 0, None) == _lib.AHQ_ERR_INVALID
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", CASES, ids=lambda c: c[0])
+def test_static_scratch_allocates_no_device_memory(device, case):
+    """What the entry point exists for: after the first call on the device (which looks the array's address up), calls
+    leave the device's free memory and torch's allocator statistics where they were."""
+    _, big, _, big_enc, _, block = case
+    lib = _lib.load()
+    x = torch.randn(big, generator=torch.Generator().manual_seed(5)).to(device)
+    _, layout = _prepare(x, big_enc, block)
+    mn = torch.empty(big_enc, dtype=x.dtype, device=device)
+    mx = torch.empty(big_enc, dtype=x.dtype, device=device)
+    stream = _lib.current_stream(device)
+
+    def call():
+        return lib.ahq_minmax_static(_lib.DTYPE_CODE[x.dtype], layout, x.data_ptr(), mn.data_ptr(), mx.data_ptr(), None,
+                                     None, 0, stream)
+
+    assert call() == 0
+    torch.cuda.synchronize()
+    free0, allocated0, reserved0 = torch.cuda.mem_get_info()[0], torch.cuda.memory_allocated(), torch.cuda.memory_reserved()
+    for _ in range(20):
+        assert call() == 0
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free0
+    assert torch.cuda.memory_allocated() == allocated0 and torch.cuda.memory_reserved() == reserved0
