@@ -150,6 +150,36 @@ __device__ __forceinline__ T segment_reduce(T v, int kv, Op op) {
     return v;
 }
 
+// Minimum / maximum of a float over runs of KV lanes (KV a power of two <= 16, known at compile time), every lane
+// receiving the result: one vector instruction per step, the exchange being the instruction's own data-parallel
+// operand (quad permutes, then the mirrored lane of each 8 and each 16; see segment_reduce for why those are valid as
+// later steps of a butterfly).  The compiler's own form of such a step is four instructions: a move through the
+// data-parallel network and two operand canonicalisations in front of the minimum.  v_min_f32 / v_max_f32 return the
+// other operand when one is NaN, so NaN never wins; the callers track NaN separately.  The two wait states a
+// data-parallel operand needs after the vector instruction that wrote it are spelled out, since the assembler does
+// not add them inside an asm statement.
+#define AHQ_DPP_STEP(OPC, CTRL) \
+    asm volatile("s_nop 1\n\t" OPC " %0, %1, %1 " CTRL " row_mask:0xf bank_mask:0xf" : "=v"(v) : "v"(v))
+template <int KV>
+__device__ __forceinline__ float segment_min_f32(float v) {
+    static_assert(KV >= 1 && KV <= 16 && (KV & (KV - 1)) == 0, "runs of 1, 2, 4, 8 or 16 lanes");
+    if constexpr (KV > 1) AHQ_DPP_STEP("v_min_f32_dpp", "quad_perm:[1,0,3,2]");
+    if constexpr (KV > 2) AHQ_DPP_STEP("v_min_f32_dpp", "quad_perm:[2,3,0,1]");
+    if constexpr (KV > 4) AHQ_DPP_STEP("v_min_f32_dpp", "row_half_mirror");
+    if constexpr (KV > 8) AHQ_DPP_STEP("v_min_f32_dpp", "row_mirror");
+    return v;
+}
+template <int KV>
+__device__ __forceinline__ float segment_max_f32(float v) {
+    static_assert(KV >= 1 && KV <= 16 && (KV & (KV - 1)) == 0, "runs of 1, 2, 4, 8 or 16 lanes");
+    if constexpr (KV > 1) AHQ_DPP_STEP("v_max_f32_dpp", "quad_perm:[1,0,3,2]");
+    if constexpr (KV > 2) AHQ_DPP_STEP("v_max_f32_dpp", "quad_perm:[2,3,0,1]");
+    if constexpr (KV > 4) AHQ_DPP_STEP("v_max_f32_dpp", "row_half_mirror");
+    if constexpr (KV > 8) AHQ_DPP_STEP("v_max_f32_dpp", "row_mirror");
+    return v;
+}
+#undef AHQ_DPP_STEP
+
 template <typename T, typename Op>
 __device__ __forceinline__ T wave_reduce(T v, Op op) {
 #pragma unroll

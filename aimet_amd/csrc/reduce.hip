@@ -53,6 +53,9 @@ struct MmFlatArgs : MmOut {
     // merges its result into its slot and nothing is folded; first: the slots hold nothing yet
     int32_t accumulate;
     int32_t first;
+    // the workgroup that takes the vectors past the last full tile: (nvec / kFlatTileVec) % gridDim.x, formed on the
+    // host (a 64-bit remainder is a hundred instructions that every workgroup would run as its last act)
+    uint32_t tail_block;
     // accumulate, optional: slots of the same shape that receive this batch's own partials (nothing merged into them)
     float* batch_min;
     float* batch_max;
@@ -133,10 +136,25 @@ __device__ __forceinline__ MinMax mm_shfl_xor(const MinMax& a, int m) {
     return {__shfl_xor(a.mn, m, kWave), __shfl_xor(a.mx, m, kWave), __shfl_xor(a.nan, m, kWave)};
 }
 
+// Extrema over the 64 lanes of a wave, every lane receiving them: the four steps inside a row of 16 lanes are one
+// instruction each (segment_min_f32), two exchanges across rows follow; the NaN flags are one ballot.  (Eighteen
+// dependent trips through the LDS permute network before: the tail of every workgroup of kernels that last a
+// microsecond or two.)
+__device__ __forceinline__ MinMax mm_wave_reduce(MinMax v) {
+    v.mn = segment_min_f32<16>(v.mn);
+    v.mx = segment_max_f32<16>(v.mx);
+#pragma unroll
+    for (int m = 16; m <= 32; m <<= 1) {
+        v.mn = fminf(v.mn, __shfl_xor(v.mn, m, kWave));
+        v.mx = fmaxf(v.mx, __shfl_xor(v.mx, m, kWave));
+    }
+    v.nan = __builtin_amdgcn_ballot_w64(v.nan != 0) != 0 ? 1 : 0;
+    return v;
+}
+
 template <int BLOCK = kBlock>
 __device__ __forceinline__ MinMax mm_block_reduce(MinMax v, MinMax* smem) {
-#pragma unroll
-    for (int m = kWave / 2; m >= 1; m >>= 1) v = mm_merge(v, mm_shfl_xor(v, m));
+    v = mm_wave_reduce(v);
     __syncthreads();
     if ((threadIdx.x & (kWave - 1)) == 0) smem[threadIdx.x / kWave] = v;
     __syncthreads();
@@ -326,7 +344,7 @@ __global__ __launch_bounds__(kFlatBlock) void minmax_flat_kernel(const MmFlatArg
         for (int u = 0; u < kFlatUnroll; ++u) mm_pack<IO, VEC, MODE>(in[u], acc.mn, acc.mx, unordered);
     }
     // the vectors past the last full tile: the workgroup after the one that took that tile
-    if (blockIdx.x == full_tiles % gridDim.x) {
+    if (blockIdx.x == a.tail_block) {
         for (int64_t v = full_tiles * kFlatTileVec + threadIdx.x; v < a.nvec; v += kFlatBlock) {
             const Pack<IO, VEC> p = load_pack_stream<IO, VEC>(x + v * VEC);
             if (cp) store_pack<IO, VEC>(cp + v * VEC, p);
@@ -432,9 +450,7 @@ __global__ __launch_bounds__(BLOCK) void minmax_runs_kernel(const MmRunArgs a) {
     acc.nan = unordered != 0 ? 1 : 0;
     MinMax b;
     if (BLOCK == kWave) {
-        b = acc;
-#pragma unroll
-        for (int m = kWave / 2; m >= 1; m >>= 1) b = mm_merge(b, mm_shfl_xor(b, m));
+        b = mm_wave_reduce(acc);
     } else {
         b = mm_block_reduce<BLOCK>(acc, red_smem);
     }
@@ -451,7 +467,9 @@ __global__ __launch_bounds__(BLOCK) void minmax_runs_kernel(const MmRunArgs a) {
 constexpr int kSegUnroll = 2;
 constexpr int kSegTileVec = kBlock * kSegUnroll;
 
-template <typename IO, int VEC, bool FINITE>
+// KV: lanes per run when that is at most 16 (the exchanges are then one instruction each, segment_min_f32), else 0
+// (the general butterfly over a.kv lanes).  A full tile issues all its loads before it looks at any of them.
+template <typename IO, int VEC, bool FINITE, int KV>
 __global__ __launch_bounds__(kBlock) void minmax_seg_kernel(const MmRunArgs a) {
     __shared__ float s_mn[kSegTileVec], s_mx[kSegTileVec];
     __shared__ unsigned char s_nan[kSegTileVec];
@@ -459,17 +477,28 @@ __global__ __launch_bounds__(kBlock) void minmax_seg_kernel(const MmRunArgs a) {
     const int64_t v0 = (int64_t)blockIdx.x * kSegTileVec;
     const int64_t left = a.nvec - v0;
     const IO* __restrict__ x = static_cast<const IO*>(a.x) + v0 * VEC;
-    const int kv = a.kv;
+    const int kv = KV ? KV : a.kv;
+    const int kv_shift = KV ? __builtin_ctz(KV ? KV : 1) : a.kv_shift;
     const int lane = threadIdx.x & (kWave - 1);
     const uint64_t run_lanes = kv >= kWave ? ~0ull : ((1ull << kv) - 1) << (lane & ~(kv - 1));
     Pack<IO, VEC> in[kSegUnroll];
+    if (left >= kSegTileVec) {
+        if (a.stream_loads) {
 #pragma unroll
-    for (int u = 0; u < kSegUnroll; ++u) {
-        const int lv = u * kBlock + threadIdx.x;
-        if (lv < left) in[u] = a.stream_loads ? load_pack_stream<IO, VEC>(x + (int64_t)lv * VEC) : load_pack<IO, VEC>(x + (int64_t)lv * VEC);
-        else
+            for (int u = 0; u < kSegUnroll; ++u) in[u] = load_pack_stream<IO, VEC>(x + (int64_t)(u * kBlock + threadIdx.x) * VEC);
+        } else {
 #pragma unroll
-            for (int k = 0; k < VEC; ++k) in[u].v[k] = IO{};
+            for (int u = 0; u < kSegUnroll; ++u) in[u] = load_pack<IO, VEC>(x + (int64_t)(u * kBlock + threadIdx.x) * VEC);
+        }
+    } else {
+#pragma unroll
+        for (int u = 0; u < kSegUnroll; ++u) {
+            const int lv = u * kBlock + threadIdx.x;
+            if (lv < left) in[u] = load_pack<IO, VEC>(x + (int64_t)lv * VEC);
+            else
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) in[u].v[k] = IO{};
+        }
     }
 #pragma unroll
     for (int u = 0; u < kSegUnroll; ++u) {
@@ -477,18 +506,23 @@ __global__ __launch_bounds__(kBlock) void minmax_seg_kernel(const MmRunArgs a) {
         float mn = __builtin_inff(), mx = -__builtin_inff();
         uint64_t unordered = 0;
         mm_pack<IO, VEC, MODE>(in[u], mn, mx, unordered);
-        mn = segment_reduce(mn, kv, OpMinF());
-        mx = segment_reduce(mx, kv, OpMaxF());
+        if constexpr (KV != 0) {
+            mn = segment_min_f32<KV>(mn);
+            mx = segment_max_f32<KV>(mx);
+        } else {
+            mn = segment_reduce(mn, kv, OpMinF());
+            mx = segment_reduce(mx, kv, OpMaxF());
+        }
         if ((lane & (kv - 1)) == 0 && lv < left) {  // runs are whole inside the tensor: a live leader means a live run
-            const int slot = lv >> a.kv_shift;
+            const int slot = lv >> kv_shift;
             s_mn[slot] = mn;
             s_mx[slot] = mx;
             s_nan[slot] = (unordered & run_lanes) != 0 ? 1 : 0;
         }
     }
     __syncthreads();
-    const int nslots = (int)((left < kSegTileVec ? left : (int64_t)kSegTileVec) >> a.kv_shift);
-    const int64_t e0 = v0 >> a.kv_shift;
+    const int nslots = (int)((left < kSegTileVec ? left : (int64_t)kSegTileVec) >> kv_shift);
+    const int64_t e0 = v0 >> kv_shift;
     for (int t = threadIdx.x; t < nslots; t += kBlock) mm_write<IO>(a, e0 + t, MinMax{s_mn[t], s_mx[t], (int)s_nan[t]});
 }
 
@@ -631,6 +665,7 @@ static MmFlatArgs flat_args(const Plan& p, const MmArgs& a) {
     f.copy = a.copy;
     f.numel = p.cl.numel;
     f.nvec = p.nvec;
+    f.tail_block = (uint32_t)((p.nvec / kFlatTileVec) % flat_blocks(p));
     f.part_min = a.part_min;
     f.part_max = a.part_max;
     f.part_nan = a.part_nan;
@@ -673,7 +708,15 @@ static void launch_mm(const Plan& p, const MmArgs& a, hipStream_t st) {
         }
         if (p.Kv < kWave && is_pow2(p.Kv)) {
             const int64_t nb = (p.nvec + kSegTileVec - 1) / kSegTileVec;
-            hipLaunchKernelGGL((minmax_seg_kernel<IO, V, FINITE>), dim3((unsigned)nb), dim3(kBlock), 0, st, r);
+            const dim3 g((unsigned)nb), b(kBlock);
+            switch (r.kv) {
+                case 1: hipLaunchKernelGGL((minmax_seg_kernel<IO, V, FINITE, 1>), g, b, 0, st, r); break;
+                case 2: hipLaunchKernelGGL((minmax_seg_kernel<IO, V, FINITE, 2>), g, b, 0, st, r); break;
+                case 4: hipLaunchKernelGGL((minmax_seg_kernel<IO, V, FINITE, 4>), g, b, 0, st, r); break;
+                case 8: hipLaunchKernelGGL((minmax_seg_kernel<IO, V, FINITE, 8>), g, b, 0, st, r); break;
+                case 16: hipLaunchKernelGGL((minmax_seg_kernel<IO, V, FINITE, 16>), g, b, 0, st, r); break;
+                default: hipLaunchKernelGGL((minmax_seg_kernel<IO, V, FINITE, 0>), g, b, 0, st, r); break;
+            }
             return;
         }
     }
@@ -870,6 +913,7 @@ extern "C" int ahq_minmax_accumulate(int32_t dtype, const void* x, int64_t count
     f.first = first ? 1 : 0;
     const int64_t tiles = f.nvec > 0 ? (f.nvec + kFlatTileVec - 1) / kFlatTileVec : 1;
     const unsigned nb = (unsigned)(tiles < kFlatMaxBlocks ? tiles : kFlatMaxBlocks);
+    f.tail_block = (uint32_t)((f.nvec / kFlatTileVec) % nb);
     hipStream_t st = static_cast<hipStream_t>(stream);
 #define AHQ_LAUNCH_ACC(IO)                                                                                              \
     do {                                                                                                                \
