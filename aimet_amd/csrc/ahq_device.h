@@ -180,6 +180,23 @@ __device__ __forceinline__ float segment_max_f32(float v) {
 }
 #undef AHQ_DPP_STEP
 
+// Maximum of a float over runs of `kv` lanes (a power of two up to 64, uniform across the wave), in every lane: the
+// steps inside a row of 16 lanes are one instruction each, the two across rows go through the LDS permute network.
+// NaN never wins (see segment_max_f32).
+__device__ __forceinline__ float segment_max_any(float v, int kv) {
+    switch (kv) {
+        case 1: return v;
+        case 2: return segment_max_f32<2>(v);
+        case 4: return segment_max_f32<4>(v);
+        case 8: return segment_max_f32<8>(v);
+        default: break;
+    }
+    v = segment_max_f32<16>(v);
+    if (kv > 16) v = fmaxf(v, __shfl_xor(v, 16, kWave));
+    if (kv > 32) v = fmaxf(v, __shfl_xor(v, 32, kWave));
+    return v;
+}
+
 template <typename T, typename Op>
 __device__ __forceinline__ T wave_reduce(T v, Op op) {
 #pragma unroll

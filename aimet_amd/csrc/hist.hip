@@ -563,17 +563,22 @@ constexpr size_t kLdsMax = 160 * 1024;
 // against 42.9 at 32M, 70.9 against 62.3 at 64M).
 std::atomic<int64_t> g_table_min_numel{(int64_t)48 << 20};
 
+constexpr int kLutU = 2;  // 16-byte vectors per lane and round of the aligned form
+
 template <typename IO, int VEC, bool SPEC>
 __global__ __launch_bounds__(kLutThreads) void hist_bin16_kernel(const BinArgs a) {
     extern __shared__ uint32_t lds[];
     __shared__ float ext_smem[kLutThreads / kWave][2];
+    __shared__ uint16_t chunk_entry[kLutEntries / 64];
     if (!SPEC && a.rebin && *a.rebin == 0) return;
     uint16_t* lut = reinterpret_cast<uint16_t*>(lds);
     uint32_t* cnt = lds + kLutBytes / 4;  // [B + 3][copies], lane l adds to copy l % copies
     const int B = a.num_bins;
     const float Bf = (float)B;
     const int copies = a.copies, cshift = a.copy_shift;
-    for (int i = threadIdx.x; i < (B + 3) * copies; i += kLutThreads) cnt[i] = 0;
+    // behind the counters: one word per thread for its exact zeros (see below)
+    uint32_t* zero_words = cnt + ((size_t)(B + 3) << cshift);
+    for (int i = threadIdx.x; i < (B + 3) * copies + kLutThreads; i += kLutThreads) cnt[i] = 0;
     RangeC r;
     float run_lo = 0.f, run_hi = 0.f, thr_min = 0.f, thr_max = 0.f;
     bool track_all = false;
@@ -588,17 +593,29 @@ __global__ __launch_bounds__(kLutThreads) void hist_bin16_kernel(const BinArgs a
     } else {
         r = load_range(a.ranges, 0);
     }
-    auto value_of = [](uint32_t pattern) {
-        IO v;
-        v.bits = (uint16_t)pattern;
-        return load_f32(v);
+    auto entry_of = [&](uint32_t pattern) -> uint32_t {
+        IO io;
+        io.bits = (uint16_t)pattern;
+        const float v = load_f32(io);
+        if ((v >= r.lo) & (v <= r.hi)) return (uint32_t)bin_exact(v, r, Bf, B);
+        return v < r.thr_lo ? (uint32_t)B : (v > r.thr_hi ? (uint32_t)B + 1u : (uint32_t)B + 2u);
     };
-    for (int p = threadIdx.x; p < kLutEntries; p += kLutThreads) {
-        const float v = value_of((uint32_t)p);
-        int e;
-        if ((v >= r.lo) & (v <= r.hi)) e = bin_exact(v, r, Bf, B);
-        else e = v < r.thr_lo ? B : (v > r.thr_hi ? B + 1 : B + 2);
-        lut[p] = (uint16_t)e;
+    // The table.  The entry is a monotone function of the value on either side of zero, and a run of 64 neighbouring
+    // patterns (one sign, rising magnitude) almost always lies inside one bin or outside the range altogether: only
+    // the few binades the range's bins are as narrow as 16-bit values are dense in need their entries one by one.
+    // So a thread first looks at the two ends of one run; where they agree the run is filled with that entry.  (The
+    // entry "neither below nor above" sits on both sides of the range, so agreement on it proves nothing.)  The exact
+    // arithmetic per pattern -- a division -- for all 65536 of them cost every workgroup 4 us of a 50 us kernel.
+    {
+        const uint32_t first = entry_of(threadIdx.x * 64u), last = entry_of(threadIdx.x * 64u + 63u);
+        chunk_entry[threadIdx.x] = (uint16_t)((first == last && first != (uint32_t)B + 2u) ? first : 0xffffu);
+    }
+    __syncthreads();
+    for (uint32_t q = threadIdx.x; q < kLutEntries / 2; q += kLutThreads) {
+        const uint32_t same = chunk_entry[q >> 5];
+        const uint32_t e0 = same != 0xffffu ? same : entry_of(2u * q);
+        const uint32_t e1 = same != 0xffffu ? same : entry_of(2u * q + 1u);
+        lds[q] = e0 | (e1 << 16);
     }
     __syncthreads();
     float ext_min = __builtin_inff(), ext_max = -__builtin_inff();
@@ -607,38 +624,56 @@ __global__ __launch_bounds__(kLutThreads) void hist_bin16_kernel(const BinArgs a
         ext_min = fminf(ext_min, (fin & (v < thr_min)) ? v : __builtin_inff());
         ext_max = fmaxf(ext_max, (fin & (v > thr_max)) ? v : -__builtin_inff());
     };
-    uint32_t* mine = cnt + (threadIdx.x & (copies - 1));
-    uint32_t zeros = 0;   // exact zeros are counted here and added once (they would all meet in one LDS word)
-    bool outside = false;  // SPEC: this lane met an element the table sent outside the range
-    const bool zero_outside = lut[0] >= (uint32_t)B;
-    auto count = [&](uint32_t pattern) {
-        if ((pattern & 0x7fffu) == 0) {
-            ++zeros;
-            if (SPEC) outside |= zero_outside;
-        } else {
-            const uint32_t e = lut[pattern];
-            atomicAdd(mine + (e << cshift), 1u);
-            if (SPEC) outside |= e >= (uint32_t)B;
-        }
-    };
+    const uint32_t copy = threadIdx.x & (copies - 1);
+    uint32_t* mine = cnt + copy;
+    // Exact zeros (half of a rectified activation) would all meet in one LDS word; each thread adds them to a word
+    // of its own instead and moves the sum to the bin of zero once, at the end.
+    const uint32_t zero_at = (uint32_t)((B + 3) << cshift) + threadIdx.x;
     const IO* __restrict__ x = static_cast<const IO*>(a.x);
-    const int64_t full_tiles = a.nvec / kLutThreads;
-    for (int64_t tile = blockIdx.x; tile < full_tiles; tile += gridDim.x) {
-        const Pack<IO, VEC> in = load_pack_stream<IO, VEC>(x + (tile * kLutThreads + threadIdx.x) * VEC);
-        outside = false;
+    int64_t done = 0;  // elements binned by the vector loop
+    if (VEC > 1) {
+        // Rounds of kLutU vectors per lane: all the round's table reads are issued before the first increment, so
+        // the LDS unit always has independent work queued (an increment waits for its table read).
+        const int64_t rounds = a.nvec / (kLutThreads * kLutU);
+        for (int64_t t = blockIdx.x; t < rounds; t += gridDim.x) {
+            Pack<IO, VEC> in[kLutU];
 #pragma unroll
-        for (int k = 0; k < VEC; ++k) count(in.v[k].bits);
-        if (SPEC && (track_all || __builtin_amdgcn_ballot_w64(outside) != 0)) {
-            for (int k = 0; k < VEC; ++k) track(load_f32(in.v[k]));
+            for (int u = 0; u < kLutU; ++u) in[u] = load_pack_stream<IO, VEC>(x + ((t * kLutU + u) * kLutThreads + threadIdx.x) * VEC);
+            uint32_t e[kLutU][VEC];
+#pragma unroll
+            for (int u = 0; u < kLutU; ++u)
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) e[u][k] = lut[in[u].v[k].bits];
+            bool outside = false;
+#pragma unroll
+            for (int u = 0; u < kLutU; ++u)
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) {
+                    const bool zero = (in[u].v[k].bits & 0x7fffu) == 0;
+                    atomicAdd(cnt + (zero ? zero_at : (e[u][k] << cshift) + copy), 1u);
+                    if (SPEC) outside |= e[u][k] >= (uint32_t)B;
+                }
+            if (SPEC && (track_all || __builtin_amdgcn_ballot_w64(outside) != 0)) {
+#pragma unroll
+                for (int u = 0; u < kLutU; ++u)
+                    for (int k = 0; k < VEC; ++k) track(load_f32(in[u].v[k]));
+            }
         }
+        done = rounds * kLutThreads * kLutU * VEC;
     }
-    if (blockIdx.x == 0) {  // the vectors past the last full tile and the elements past the last full vector
-        for (int64_t i = full_tiles * kLutThreads * VEC + threadIdx.x; i < a.numel; i += kLutThreads) {
-            count(x[i].bits);
-            if (SPEC) track(load_f32(x[i]));
-        }
+    // what the rounds leave (less than one round; everything when the tensor is not 16-byte aligned), element by
+    // element, spread over the workgroups
+    for (int64_t i = done + (int64_t)blockIdx.x * kLutThreads + threadIdx.x; i < a.numel; i += (int64_t)gridDim.x * kLutThreads) {
+        const uint32_t bits = x[i].bits;
+        const uint32_t e = lut[bits];
+        atomicAdd(cnt + ((bits & 0x7fffu) == 0 ? zero_at : (e << cshift) + copy), 1u);
+        if (SPEC && (track_all || e >= (uint32_t)B)) track(load_f32(x[i]));
     }
-    if (zeros != 0) atomicAdd(mine + ((uint32_t)lut[0] << cshift), zeros);
+    __syncthreads();
+    {
+        const uint32_t zeros = zero_words[threadIdx.x];
+        if (zeros != 0) atomicAdd(mine + ((uint32_t)lut[0] << cshift), zeros);
+    }
     if (SPEC) {
 #pragma unroll
         for (int m = kWave / 2; m >= 1; m >>= 1) {
@@ -667,6 +702,32 @@ __global__ __launch_bounds__(kLutThreads) void hist_bin16_kernel(const BinArgs a
         for (int cp = 0; cp < copies; ++cp) c += cnt[((size_t)e << cshift) + cp];
         a.partials[(((size_t)(e / kPartBins)) * np + blockIdx.x) * kPartBins + e % kPartBins] = c;
     }
+}
+
+// The table kernels need more dynamic LDS than a kernel gets by default: asked for once per device and dtype, for
+// the most any launch uses; false when the runtime refuses (the callers then keep the arithmetic kernels).
+static bool lut_lds_available(int dtype) {
+    constexpr int kMost = (int)(kLdsMax - 4096);
+    constexpr int kMaxDevices = 64;
+    static std::atomic<int> state[kMaxDevices][2];  // 0 not asked yet, 1 granted, 2 refused
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return false;
+    std::atomic<int>& st = state[dev][dtype == AHQ_F16 ? 0 : 1];
+    int v = st.load(std::memory_order_acquire);
+    if (v == 0) {
+        auto allow = [](auto kernel) {
+            return hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kMost) == hipSuccess;
+        };
+        const bool ok = dtype == AHQ_F16
+            ? allow(&hist_bin16_kernel<f16_t, 1, true>) && allow(&hist_bin16_kernel<f16_t, 1, false>) &&
+              allow(&hist_bin16_kernel<f16_t, 8, true>) && allow(&hist_bin16_kernel<f16_t, 8, false>)
+            : allow(&hist_bin16_kernel<bf16_t, 1, true>) && allow(&hist_bin16_kernel<bf16_t, 1, false>) &&
+              allow(&hist_bin16_kernel<bf16_t, 8, true>) && allow(&hist_bin16_kernel<bf16_t, 8, false>);
+        if (!ok) (void)hipGetLastError();  // the refusal is handled here, not reported by the next launch check
+        v = ok ? 1 : 2;
+        st.store(v, std::memory_order_release);
+    }
+    return v == 1;
 }
 
 // Several slots whose runs are long enough that a tile lies inside one run (per-channel weights, per-channel
@@ -1063,7 +1124,8 @@ bool make_hist_plan(int dtype, const ahq_layout& layout, const void* x, int num_
     hp->nblocks = (int)nb;
     const size_t B = (size_t)num_bins;
     size_t o = 0;
-    hp->off_mm_ws = o;     o = align_up(o + ahq_minmax_workspace_bytes(&layout));
+    // (the same region holds the speculative pass's partial extrema: two floats per workgroup)
+    hp->off_mm_ws = o;     o = align_up(o + std::max(ahq_minmax_workspace_bytes(&layout), (size_t)kHistBlocksMax * 8));
     hp->off_bmin = o;      o = align_up(o + (size_t)S * 4);
     hp->off_bmax = o;      o = align_up(o + (size_t)S * 4);
     hp->off_ranges = o;    o = align_up(o + (size_t)S * kRng * 4);
@@ -1137,22 +1199,20 @@ extern "C" int ahq_hist_update(int32_t dtype, const ahq_layout* layout, const vo
     // 16-bit tensors, one histogram: the binning kernel that looks the bin up in a table (hist_bin16_kernel)
     int lut_copies = 0;
     if (hp.fast && NH == 1 && dtype != AHQ_F32 && c.numel >= g_table_min_numel.load(std::memory_order_relaxed)) {
-        const size_t room = kLdsMax - kLutBytes - 1024;
+        // static arrays of the kernel (4 KB), one word per thread for its zeros, then the counters
+        const size_t room = kLdsMax - kLutBytes - 4096 - (size_t)kLutThreads * 4;
         for (int c2 = 8; c2 >= 1 && lut_copies == 0; c2 >>= 1)
             if ((size_t)c2 * (B + 3) * 4 <= room) lut_copies = c2;
+        if (lut_copies > 0 && !lut_lds_available(dtype)) lut_copies = 0;  // refused: the arithmetic kernels bin
     }
     const int lut_blocks = lut_copies > 0 ? (int)std::min<int64_t>(std::max<int64_t>(hp.plan.nvec / kLutThreads, 1), std::min(256, hp.nblocks)) : 0;
     auto launch_lut = [&](BinArgs args, bool spec) {
         args.copies = lut_copies;
         args.copy_shift = 0;
         while ((1 << args.copy_shift) < lut_copies) ++args.copy_shift;
-        const size_t lds = kLutBytes + (size_t)lut_copies * (B + 3) * 4;
+        const size_t lds = kLutBytes + (size_t)lut_copies * (B + 3) * 4 + (size_t)kLutThreads * 4;
         const dim3 g(lut_blocks), b(kLutThreads);
-#define AHQ_LAUNCH_LUT_K(K)                                                                                         \
-    do {                                                                                                            \
-        hipFuncSetAttribute(reinterpret_cast<const void*>(&K), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
-        hipLaunchKernelGGL(K, g, b, lds, s, args);                                                                  \
-    } while (0)
+#define AHQ_LAUNCH_LUT_K(K) hipLaunchKernelGGL(K, g, b, lds, s, args)
 #define AHQ_LAUNCH_LUT(IO)                                                                                          \
     do {                                                                                                            \
         if (hp.plan.vec == 1) {                                                                                     \

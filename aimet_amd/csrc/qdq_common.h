@@ -501,13 +501,10 @@ __device__ __forceinline__ void stage_lpbq(const QdqArgs& a, const LpbqFuse& f, 
             const int64_t e = t.e0 + i;
             const float raw = !live ? -__builtin_inff()
                               : i == (int)threadIdx.x ? lpbq_raw_from(f, pre_mn, pre_mx) : lpbq_raw_scale(f, e);
-            float largest = raw;
-            int nan = (raw != raw) ? 1 : 0;
-            for (int m = 1; m < (int)G; m <<= 1) {
-                largest = fmaxf(largest, __shfl_xor(largest, m, kWave));
-                nan |= __shfl_xor(nan, m, kWave);
-            }
-            if (nan) largest = __builtin_nanf("");  // torch.amax propagates NaN
+            // (one ballot says which lanes hold NaN; a lane looks at the bits of its own group)
+            float largest = segment_max_any(raw, (int)G);
+            const uint64_t group_lanes = G >= kWave ? ~0ull : (((1ull << G) - 1) << (lane & ~((int)G - 1)));
+            if (__builtin_amdgcn_ballot_w64(raw != raw) & group_lanes) largest = __builtin_nanf("");  // torch.amax propagates NaN
             if (live) stage_one(i, e, e >> f.group_shift, raw, largest / f.multipliers);
         }
         return;

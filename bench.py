@@ -802,15 +802,17 @@ def run_hist_workload(steps, warmup, dev, with_cpu_baseline=True, batches=16, sh
     traffic_upd = MEASURED_TRAFFIC_BYTES[("c3", "hist_update")]
 
     # the same stream in bf16: twice the elements per byte, and an update that holds the range bins them through a
-    # table in LDS (hist_bin16_kernel) instead of computing each element's bin
-    xs16 = [x.bfloat16() for x in xs[:4]]
+    # table in LDS (hist_bin16_kernel) instead of computing each element's bin.  All 16 batches are folded (one at a
+    # time is converted: 16 more resident batches would not fit beside the float32 ones on every box) and the result
+    # is compared with the oracle below; the timed updates then go through four resident bf16 batches in turn.
     an16 = SqnrEncodingAnalyzer((1,), num_bins=512, asymmetric_delta_candidates=100, offset_candidates=64, gamma=3.0)
-    for x in xs16[:2]:
-        an16.update_stats(x)
+    for x in xs:
+        an16.update_stats(x.bfloat16())
     st16 = an16.observer.get_stats()[0]
     hist16_gpu, edges16_gpu = st16.histogram.cpu().clone(), st16.bin_edges.cpu().clone()
-    for x in xs16[2:] + xs16:
-        an16.update_stats(x)
+    lo16, hi16 = an16.compute_encodings(255, False)
+    best16_gpu = int(an16.last_search["best_index"].item())
+    xs16 = [x.bfloat16() for x in xs[:4]]
     turn16 = [0]
 
     def update_next16():
@@ -819,18 +821,25 @@ def run_hist_workload(steps, warmup, dev, with_cpu_baseline=True, batches=16, sh
 
     t_upd16 = event_time(update_next16, 20)
     bf16_stream = {"update_us": round(t_upd16 * 1e6, 2), "GBps_one_read": round(2 * n_b / t_upd16 / 1e9, 1),
+                   "frac_of_hbm_peak": round(2 * n_b / t_upd16 / 1e9 / HBM_PEAK_GBS, 4),
                    "elements_per_s": round(n_b / t_upd16, 1), "kernel": "hist_bin16_kernel<SPEC>",
-                   "sample": "the first 4 batches rounded to bf16, in turn"}
+                   "sample": "the first 4 batches rounded to bf16, in turn",
+                   "bound": "LDS instruction issue: a table read and an increment per element; bare LDS increments "
+                            "alone take 28 us for 67 M elements on this device (16 cycles per wave instruction)"}
 
     parity = {"sample": "not compared (CPU leg switched off)"}
     cpu_all = cpu_one = None
     if with_cpu_baseline:
         ref16 = O.HistObserver((1,), 512)
-        for xb in xs16[:2]:
-            ref16.update(xb.cpu())
+        for xb in xs:
+            ref16.update(xb.bfloat16().cpu())
+        lo16_r, hi16_r, _, _, bi16 = O.sqnr_encodings(ref16.stats, (1,), 255, False, asym_deltas=100, num_offsets=64, gamma=3.0)
         bf16_stream["parity"] = {"hist_bit_exact": bool(torch.equal(hist16_gpu, ref16.stats[0].histogram)),
                                  "edges_bit_exact": bool(torch.equal(edges16_gpu, ref16.stats[0].bin_edges)),
-                                 "sample": "after 2 batches"}
+                                 "argmin_identical": bool(best16_gpu == int(bi16.item())),
+                                 "encoding_bit_exact": bool(torch.equal(lo16.cpu(), lo16_r) and torch.equal(hi16.cpu(), hi16_r)),
+                                 "largest_bin_count": float(hist16_gpu.max()),
+                                 "sample": f"all {batches} batches rounded to bf16"}
         del ref16
         # the CPU leg: the whole 16-batch step, one batch on the host at a time; its result is the parity reference
         ref_all = O.HistObserver((1,), 512)
