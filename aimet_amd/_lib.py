@@ -88,6 +88,39 @@ class DlqPdfState(ctypes.Structure):
     ]
 
 
+class GridProbeItem(ctypes.Structure):
+    """ahq_grid_probe_item"""
+
+    _fields_ = [("dtype", ctypes.c_int32), ("layout", Layout), ("x", ctypes.c_void_p), ("num_levels", ctypes.c_int64)]
+
+
+class CalibrateQdqItem(ctypes.Structure):
+    """ahq_calibrate_qdq_item"""
+
+    _fields_ = [
+        ("grid", Grid), ("layout", Layout), ("x", ctypes.c_void_p), ("y", ctypes.c_void_p),
+        ("num_steps", ctypes.c_int64), ("symmetric", ctypes.c_int32),
+        ("minimum_scale_in_dtype", ctypes.c_float), ("minimum_scale", ctypes.c_float), ("dtype_max", ctypes.c_float),
+        ("near_max_threshold", ctypes.c_float), ("param_dtype", ctypes.c_int32),
+        ("param_min", ctypes.c_void_p), ("param_max", ctypes.c_void_p), ("grid_minimum_scale", ctypes.c_double),
+        ("scale", ctypes.c_void_p), ("offset", ctypes.c_void_p), ("workspace", ctypes.c_void_p),
+        ("workspace_bytes", ctypes.c_size_t),
+    ]
+
+
+class SlotsFinalizeItem(ctypes.Structure):
+    """ahq_slots_finalize_item"""
+
+    _fields_ = [
+        ("stat_dtype", ctypes.c_int32), ("symmetric", ctypes.c_int32), ("slots", ctypes.c_void_p),
+        ("num_steps", ctypes.c_int64),
+        ("minimum_scale_in_dtype", ctypes.c_float), ("minimum_scale", ctypes.c_float), ("dtype_max", ctypes.c_float),
+        ("near_max_threshold", ctypes.c_float), ("param_dtype", ctypes.c_int32), ("reserved", ctypes.c_int32),
+        ("param_min", ctypes.c_void_p), ("param_max", ctypes.c_void_p), ("qmin", ctypes.c_int64), ("qmax", ctypes.c_int64),
+        ("grid_minimum_scale", ctypes.c_double), ("scale", ctypes.c_void_p), ("offset", ctypes.c_void_p),
+    ]
+
+
 DLQ_PDF_SIZE = 1536
 
 
@@ -143,6 +176,9 @@ _SIGNATURES = {
     "ahq_lpbq_qdq_forward": (ctypes.c_int, [ctypes.POINTER(Grid), ctypes.POINTER(Layout), _P, _P, _P, ctypes.c_int32, _P,
                                             _P, ctypes.c_int64, ctypes.c_double, ctypes.c_int32, _P, _P, _P, _P]),
     "ahq_grid_probe": (ctypes.c_int, [ctypes.c_int32, ctypes.POINTER(Layout), _P, ctypes.c_int64, _P, _P]),
+    "ahq_grid_probe_many": (ctypes.c_int, [ctypes.POINTER(GridProbeItem), ctypes.c_int64, _P, _P, _P]),
+    "ahq_minmax_calibrate_qdq_many": (ctypes.c_int, [ctypes.POINTER(CalibrateQdqItem), ctypes.c_int64, _P, _P]),
+    "ahq_minmax_slots_finalize_many": (ctypes.c_int, [ctypes.POINTER(SlotsFinalizeItem), ctypes.c_int64, _P, _P]),
     "ahq_hist_update_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int32, ctypes.POINTER(Layout), ctypes.c_int32]),
     "ahq_hist_table_min_numel": (ctypes.c_int64, [ctypes.c_int64]),
     "ahq_hist_update": (ctypes.c_int, [ctypes.c_int32, ctypes.POINTER(Layout), _P, ctypes.POINTER(HistState),

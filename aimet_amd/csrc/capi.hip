@@ -1,4 +1,6 @@
 // Entry points that do not belong to one kernel family.
+#include <cstdio>
+
 #include "ahq_host.h"
 #include "layout.h"
 
@@ -62,4 +64,47 @@ extern "C" int ahq_minmax_calibrate_qdq(const ahq_grid* grid, const ahq_layout* 
                              grid->qmin, grid->qmax, grid_minimum_scale, scale, symmetric ? nullptr : offset, stream);
     if (rc != AHQ_OK) return rc;
     return ahq_qdq_forward(grid, layout, x, y, nullptr, scale, offset, nullptr, nullptr, stream);
+}
+
+extern "C" int ahq_grid_probe_many(const ahq_grid_probe_item* items, int64_t count, uint8_t* verdicts,
+                                   uint8_t* unsupported, void* stream) {
+    using ahq::set_error;
+    if (count < 0 || (count > 0 && (!items || !verdicts))) return set_error("null argument"), AHQ_ERR_INVALID;
+    for (int64_t i = 0; i < count; ++i) {
+        const ahq_grid_probe_item& it = items[i];
+        if (unsupported) unsupported[i] = 0;
+        const int rc = ahq_grid_probe(it.dtype, &it.layout, it.x, it.num_levels, verdicts + i, stream);
+        if (rc == AHQ_ERR_UNSUPPORTED && unsupported) {
+            unsupported[i] = 1;
+            continue;
+        }
+        if (rc != AHQ_OK) {
+            char msg[512];
+            std::snprintf(msg, sizeof msg, "item %lld: %s", (long long)i, ahq::error_buffer());
+            set_error(msg);
+            return rc;
+        }
+    }
+    return AHQ_OK;
+}
+
+extern "C" int ahq_minmax_calibrate_qdq_many(const ahq_calibrate_qdq_item* items, int64_t count, int32_t* flags,
+                                             void* stream) {
+    using ahq::set_error;
+    if (count < 0 || (count > 0 && !items)) return set_error("null argument"), AHQ_ERR_INVALID;
+    for (int64_t i = 0; i < count; ++i) {
+        const ahq_calibrate_qdq_item& it = items[i];
+        const int rc = ahq_minmax_calibrate_qdq(&it.grid, &it.layout, it.x, it.y, it.num_steps, it.symmetric,
+                                                it.minimum_scale_in_dtype, it.minimum_scale, it.dtype_max,
+                                                it.near_max_threshold, flags, it.param_dtype, it.param_min,
+                                                it.param_max, it.grid_minimum_scale, it.scale, it.offset, it.workspace,
+                                                it.workspace_bytes, stream);
+        if (rc != AHQ_OK) {
+            char msg[512];
+            std::snprintf(msg, sizeof msg, "item %lld: %s", (long long)i, ahq::error_buffer());
+            set_error(msg);
+            return rc;
+        }
+    }
+    return AHQ_OK;
 }

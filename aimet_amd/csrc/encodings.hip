@@ -7,6 +7,8 @@
 // statistics arithmetic in the statistics dtype T (rounded after each operation), everything after the float32
 // "widen" term in float32, the result rounded to T once.
 
+#include <cstdio>
+
 #include "ahq_device.h"
 #include "ahq_host.h"
 #include "layout.h"
@@ -234,6 +236,38 @@ __global__ __launch_bounds__(kSlotThreads) void minmax_slots_finalize_kernel(con
                                                                              const FinalArgs f) {
     float mn, mx;
     if (fold_slots<T>(slot_min, slot_max, slot_nan, mn, mx)) finalize_one<T, P>(a, f, 0, mn, mx);
+}
+
+// minmax_slots_finalize_kernel for up to kManySlots quantizers per launch, one workgroup each; every item carries
+// its own dtypes, so the type dispatch happens in the kernel.
+constexpr int kManySlots = 16;  // what fits the 4 KB a kernel takes as arguments
+struct ManySlotItem {
+    const float* slot_min;
+    const float* slot_max;
+    const int* slot_nan;
+    EncArgs a;
+    FinalArgs f;
+    int32_t stat_dtype, param_dtype;
+};
+struct ManySlotArgs {
+    ManySlotItem items[kManySlots];
+};
+static_assert(sizeof(ManySlotArgs) <= 4096, "kernel arguments are limited to 4 KB");
+
+template <typename T>
+__device__ __forceinline__ void many_slots_one(const ManySlotItem& it) {
+    float mn, mx;
+    if (!fold_slots<T>(it.slot_min, it.slot_max, it.slot_nan, mn, mx)) return;
+    if (it.param_dtype == AHQ_F32) finalize_one<T, float>(it.a, it.f, 0, mn, mx);
+    else if (it.param_dtype == AHQ_F16) finalize_one<T, f16_t>(it.a, it.f, 0, mn, mx);
+    else finalize_one<T, bf16_t>(it.a, it.f, 0, mn, mx);
+}
+
+__global__ __launch_bounds__(kSlotThreads) void minmax_slots_finalize_many_kernel(const ManySlotArgs m) {
+    const ManySlotItem& it = m.items[blockIdx.x];
+    if (it.stat_dtype == AHQ_F32) many_slots_one<float>(it);
+    else if (it.stat_dtype == AHQ_F16) many_slots_one<f16_t>(it);
+    else many_slots_one<bf16_t>(it);
 }
 
 // minmax_to_encodings_kernel for one encoding whose statistics lie in such slots; stat_min / stat_max (optional)
@@ -828,4 +862,49 @@ extern "C" int ahq_minmax_slots_to_encodings(int32_t dtype, const void* slots, i
         default: hipLaunchKernelGGL((minmax_slots_to_encodings_kernel<bf16_t>), g, b, 0, s, mn, mx, nan, a, static_cast<bf16_t*>(stat_min), static_cast<bf16_t*>(stat_max)); break;
     }
     return check_launch("minmax_slots_to_encodings");
+}
+
+extern "C" int ahq_minmax_slots_finalize_many(const ahq_slots_finalize_item* items, int64_t count, int32_t* flags,
+                                              void* stream) {
+    if (count < 0 || (count > 0 && !items)) return set_error("null argument"), AHQ_ERR_INVALID;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    for (int64_t base = 0; base < count; base += kManySlots) {
+        const int n = (int)(count - base < kManySlots ? count - base : kManySlots);
+        ManySlotArgs m{};
+        for (int k = 0; k < n; ++k) {
+            const ahq_slots_finalize_item& it = items[base + k];
+            ManySlotItem& d = m.items[k];
+            auto fail = [&](const char* what) {
+                std::snprintf(error_buffer(), 512, "item %lld: %s", (long long)(base + k), what);
+                return AHQ_ERR_INVALID;
+            };
+            if (!it.slots || (reinterpret_cast<uintptr_t>(it.slots) & 3u)) return fail("slots is null or misaligned");
+            const int rc = fill_enc_args(&d.a, it.stat_dtype, it.slots, it.slots, 1, it.num_steps, it.symmetric,
+                                         it.minimum_scale_in_dtype, it.minimum_scale, it.dtype_max,
+                                         it.near_max_threshold, flags);
+            if (rc != AHQ_OK) return fail(error_buffer());
+            if (it.param_dtype < AHQ_F32 || it.param_dtype > AHQ_BF16) return fail("bad parameter dtype");
+            if (!it.param_min || !it.param_max || !it.scale) return fail("null argument");
+            if (it.qmin >= it.qmax) return fail("qmax must be larger than qmin");
+            d.a.smin = d.a.smax = nullptr;
+            d.f.pmin = it.param_min;
+            d.f.pmax = it.param_max;
+            d.f.so.scale = it.scale;
+            d.f.so.offset = it.offset;
+            d.f.so.n = 1;
+            d.f.so.num_steps = (float)(double)(it.qmax - it.qmin);
+            d.f.so.minimum_scale = (float)it.grid_minimum_scale;
+            d.f.so.qmin = (float)(double)it.qmin;
+            d.f.so.lo = (float)(double)(-it.qmax);
+            d.f.so.hi = (float)(double)(-it.qmin);
+            const char* w = static_cast<const char*>(it.slots);
+            d.slot_min = reinterpret_cast<const float*>(w);
+            d.slot_max = reinterpret_cast<const float*>(w + 4 * AHQ_MINMAX_SLOTS);
+            d.slot_nan = reinterpret_cast<const int*>(w + 8 * AHQ_MINMAX_SLOTS);
+            d.stat_dtype = it.stat_dtype;
+            d.param_dtype = it.param_dtype;
+        }
+        hipLaunchKernelGGL(minmax_slots_finalize_many_kernel, dim3((unsigned)n), dim3(kSlotThreads), 0, s, m);
+    }
+    return check_launch("minmax_slots_finalize_many");
 }

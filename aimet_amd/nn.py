@@ -131,12 +131,17 @@ class QuantizedLinear(nn.Linear):
             if param is not None:
                 yield name, qtzr, param
 
+    @staticmethod
+    def _wants_grid_recovery(qtzr) -> bool:
+        """The parameters whose grid the reference would first try to recover (nn/base.py:355-383)."""
+        return (isinstance(qtzr, AffineQuantizerBase) and not isinstance(qtzr, GroupedBlockQuantizeDequantize)
+                and bool(qtzr.symmetric) and math.ceil((qtzr.qmin + qtzr.qmax) / 2) == 0)
+
     def _prequantized_verdicts(self, overwrite: bool):
         """name -> True / device flag for the parameters whose grid the reference would first try to recover."""
         out = {}
         for name, qtzr, param in self._params_to_calibrate(overwrite):
-            if (isinstance(qtzr, AffineQuantizerBase) and not isinstance(qtzr, GroupedBlockQuantizeDequantize)
-                    and qtzr.symmetric and math.ceil((qtzr.qmin + qtzr.qmax) / 2) == 0):
+            if self._wants_grid_recovery(qtzr):
                 out[name] = _may_be_prequantized(param.detach(), qtzr)
         return out
 
@@ -150,6 +155,8 @@ class QuantizedLinear(nn.Linear):
         if verdicts is None:
             verdicts = {k: bool(v) for k, v in self._prequantized_verdicts(overwrite).items()}
         for name, qtzr, param in todo:
+            if quantized is not None and name in quantized:
+                continue  # calibrated and quantize-dequantized already (aimet_amd.nn.compute_encodings)
             if verdicts.get(name, False):
                 try:
                     _, scale = _decompose_prequantized_tensor(
@@ -246,22 +253,208 @@ def quantized_linears(model: nn.Module) -> Iterable[QuantizedLinear]:
     return (m for m in model.modules() if isinstance(m, QuantizedLinear))
 
 
+def _probe_parameters_together(candidates):
+    """_may_be_prequantized() for many (parameter, quantizer) pairs with one library call (ahq_grid_probe_many) and
+    one read-back.  Returns the verdicts as Python booleans, in order."""
+    import ctypes
+
+    from aimet_amd import _lib
+    from aimet_amd.quantization.affine.backends.hip import _prepare
+
+    verdicts = [None] * len(candidates)
+    batched = []  # (index, item fields)
+    for i, (param, qtzr) in enumerate(candidates):
+        num_levels = max(abs(qtzr.qmax), abs(qtzr.qmin)) + 1
+        p = param.detach()
+        shape = tuple(qtzr.shape)
+        if (p.is_cuda and p.dtype in _lib.DTYPE_CODE and p.is_contiguous() and p.numel() > 0 and num_levels <= 4096
+                and p.numel() // max(1, math.prod(shape)) > num_levels):
+            xd, layout = _prepare(p, shape, qtzr.block_size)
+            batched.append((i, _lib.DTYPE_CODE[p.dtype], layout, xd, num_levels))
+        else:
+            verdicts[i] = _may_be_prequantized(p, qtzr)
+    by_device = {}
+    for entry in batched:
+        by_device.setdefault(entry[3].device, []).append(entry)
+    pending = []
+    for device, entries in by_device.items():
+        items = (_lib.GridProbeItem * len(entries))()
+        for it, (_, code, layout, xd, num_levels) in zip(items, entries):
+            it.dtype, it.layout, it.x, it.num_levels = code, layout, xd.data_ptr(), num_levels
+        out = torch.empty(len(entries), dtype=torch.bool, device=device)
+        unsupported = (ctypes.c_uint8 * len(entries))()
+        with torch.cuda.device(device):
+            _lib.check(_lib.load().ahq_grid_probe_many(items, len(entries), out.data_ptr(), unsupported,
+                                                       _lib.current_stream(device)), "ahq_grid_probe_many")
+        pending.append((entries, out, unsupported))
+    for entries, out, unsupported in pending:
+        answers = out.tolist()
+        for (i, *_), answer, skipped in zip(entries, answers, unsupported):
+            verdicts[i] = _may_be_prequantized(candidates[i][0].detach(), candidates[i][1], on_device=False) if skipped else answer
+    return [bool(v) for v in verdicts]
+
+
+def _calibrate_parameters_together(work):
+    """Calibration and first quantize-dequantize of many parameters with one library call
+    (ahq_minmax_calibrate_qdq_many).  ``work``: (module, name, quantizer, parameter) of parameters that are not on a
+    grid already.  Returns {(id(module), name): quantize-dequantized parameter} for those the call covered; the
+    others are left to QuantizedLinear._compute_param_encodings()."""
+    from aimet_amd import _lib
+    from aimet_amd.quantization._utils import _get_minimum_scale
+    from aimet_amd.quantization.encoding_analyzer import _scalar_constants, _range_flags_buffer, _report_range_flags
+
+    done = {}
+    if torch.is_grad_enabled():
+        return done
+    by_device = {}
+    for module, name, qtzr, param in work:
+        prepare = getattr(qtzr, "_calibrate_qdq_prepare", None)
+        plan = prepare(param) if prepare is not None else None
+        if plan is not None:
+            by_device.setdefault(plan[0].device, []).append((module, name, qtzr, plan))
+    for device, entries in by_device.items():
+        n = len(entries)
+        items = (_lib.CalibrateQdqItem * n)()
+        # one allocation each for the scales, the offsets of asymmetric grids and the workspaces of all parameters
+        enc_sizes = [q.min.numel() for _, _, q, _ in entries]
+        ws_sizes = [(max(plan[3], 16) + 255) // 256 * 256 for *_, plan in entries]
+        scales = torch.empty(sum(enc_sizes), dtype=torch.float32, device=device)
+        offsets = torch.empty(sum(e for e, (*_, plan) in zip(enc_sizes, entries) if not plan[5]) or 1,
+                              dtype=torch.float32, device=device)
+        ws = torch.empty(sum(ws_sizes), dtype=torch.uint8, device=device)
+        flags, own_flags = _range_flags_buffer(device)
+        outputs = []
+        s_at = o_at = w_at = 0
+        for it, (module, name, qtzr, plan), ne, nw in zip(items, entries, enc_sizes, ws_sizes):
+            x, grid, layout, nbytes, num_steps, symmetric = plan
+            mn, mx = qtzr.min, qtzr.max
+            consts = _scalar_constants(x.dtype, _get_minimum_scale(num_steps))
+            y = torch.empty_like(x)
+            scale = scales[s_at:s_at + ne].view(mn.shape)
+            s_at += ne
+            if symmetric:
+                offset = qtzr._constant_offset(device)  # pylint: disable=protected-access
+            else:
+                offset = offsets[o_at:o_at + ne].view(mn.shape)
+                o_at += ne
+            qtzr.encoding_analyzer.reset_stats()
+            it.grid, it.layout, it.x, it.y = grid, layout, x.data_ptr(), y.data_ptr()
+            it.num_steps, it.symmetric = num_steps, 1 if symmetric else 0
+            it.minimum_scale_in_dtype, it.minimum_scale, it.dtype_max, it.near_max_threshold = consts
+            it.param_dtype, it.param_min, it.param_max = _lib.DTYPE_CODE[mn.dtype], mn.data_ptr(), mx.data_ptr()
+            it.grid_minimum_scale = _get_minimum_scale(qtzr.qmax - qtzr.qmin)
+            it.scale, it.offset = scale.data_ptr(), offset.data_ptr()
+            it.workspace, it.workspace_bytes = ws.data_ptr() + w_at, nbytes
+            w_at += nw
+            outputs.append((y, scale, offset))
+        with torch.cuda.device(device):
+            _lib.check(_lib.load().ahq_minmax_calibrate_qdq_many(items, n, flags.data_ptr(), _lib.current_stream(device)),
+                       "ahq_minmax_calibrate_qdq_many")
+        for (module, name, qtzr, _), (y, scale, offset) in zip(entries, outputs):
+            done[(id(module), name)] = qtzr._calibrate_qdq_adopt(y, scale, offset)  # pylint: disable=protected-access
+            qtzr.encoding_analyzer.reset_stats()  # nn/base.py:385-386
+        if own_flags:
+            _report_range_flags(flags)
+    return done
+
+
+def _finalize_together(quantizers):
+    """What leaving their compute_encodings() contexts does for many activation quantizers
+    (_set_range_from_statistics), with one library call for all per-tensor min/max quantizers whose running extrema
+    lie in their observers' slots (ahq_minmax_slots_finalize_many); the others one by one."""
+    from aimet_amd import _lib
+    from aimet_amd.quantization._utils import _get_minimum_scale
+    from aimet_amd.quantization.encoding_analyzer import _scalar_constants, _range_flags_buffer, _report_range_flags
+
+    by_device = {}
+    for q in quantizers:
+        item = q._slots_finalize_item() if hasattr(q, "_slots_finalize_item") else None  # pylint: disable=protected-access
+        if item is None:
+            q._set_range_from_statistics()  # pylint: disable=protected-access
+        else:
+            by_device.setdefault(q.min.device, []).append((q, item))
+    for device, entries in by_device.items():
+        n = len(entries)
+        items = (_lib.SlotsFinalizeItem * n)()
+        scales = torch.empty(n, dtype=torch.float32, device=device)
+        n_asym = sum(1 for q, _ in entries if not q.symmetric)
+        offsets = torch.empty(max(n_asym, 1), dtype=torch.float32, device=device)
+        flags, own_flags = _range_flags_buffer(device)
+        s_ptr, o_ptr = scales.data_ptr(), offsets.data_ptr()
+        scale_views, offset_views = scales.unbind(0), offsets.unbind(0)  # all 0-dim views with one call each
+        outputs = []
+        o_at = 0
+        for k, (it, (q, (stat_dtype, slots, num_steps))) in enumerate(zip(items, entries)):
+            mn, mx = q.min, q.max
+            symmetric = bool(q.symmetric)
+            consts = _scalar_constants(stat_dtype, _get_minimum_scale(num_steps))
+            it.stat_dtype, it.symmetric, it.slots, it.num_steps = _lib.DTYPE_CODE[stat_dtype], 1 if symmetric else 0, slots.data_ptr(), num_steps
+            it.minimum_scale_in_dtype, it.minimum_scale, it.dtype_max, it.near_max_threshold = consts
+            it.param_dtype, it.param_min, it.param_max = _lib.DTYPE_CODE[mn.dtype], mn.data_ptr(), mx.data_ptr()
+            it.qmin, it.qmax, it.grid_minimum_scale = q.qmin, q.qmax, _get_minimum_scale(q.qmax - q.qmin)
+            it.scale = s_ptr + 4 * k
+            scale = scale_views[k] if mn.dim() == 0 else scale_views[k].view(mn.shape)
+            if symmetric:
+                it.offset = None
+                offset = q._constant_offset(device)  # pylint: disable=protected-access
+            else:
+                it.offset = o_ptr + 4 * o_at
+                offset = offset_views[o_at] if mn.dim() == 0 else offset_views[o_at].view(mn.shape)
+                o_at += 1
+            outputs.append((scale, offset))
+        with torch.cuda.device(device):
+            _lib.check(_lib.load().ahq_minmax_slots_finalize_many(items, n, flags.data_ptr(), _lib.current_stream(device)),
+                       "ahq_minmax_slots_finalize_many")
+        for (q, _), (scale, offset) in zip(entries, outputs):
+            q._finalize_adopt(scale, offset)  # pylint: disable=protected-access
+        if own_flags:
+            _report_range_flags(flags)
+
+
 @contextlib.contextmanager
 def compute_encodings(model: nn.Module):
-    """aimet_torch.nn.compute_encodings (nn/base.py): the compute_encodings context of every quantized module."""
+    """aimet_torch.nn.compute_encodings (nn/base.py): the compute_encodings context of every quantized module.  The
+    modules enter and leave together, so the work of all their quantizers is handed to the library in three calls
+    (the "already on a grid?" test of every weight, calibration + quantize-dequantize of every weight, the ranges of
+    all per-tensor activation quantizers at the end); whatever those calls do not cover goes the quantizer's own way,
+    with the same results."""
     from aimet_amd.quantization.encoding_analyzer import deferred_range_warnings
 
     modules = list(quantized_linears(model))
-    # the "is this weight already quantized" tests of all layers are evaluated on the device and read back together
-    pending = [(m, m._prequantized_verdicts(True)) for m in modules]  # pylint: disable=protected-access
-    flags = [v for _, d in pending for v in d.values() if isinstance(v, torch.Tensor)]
-    answers = iter(torch.stack(flags).tolist()) if flags else iter(())
-    verdicts = {id(m): {k: (next(answers) if isinstance(v, torch.Tensor) else bool(v)) for k, v in d.items()}
-                for m, d in pending}
     with deferred_range_warnings(), contextlib.ExitStack() as stack:
+        # 1. parameters: the reference's early exit of the grid recovery, then min/max calibration (nn/base.py:331-386)
+        todo = [(m, name, qtzr, param) for m in modules for name, qtzr, param in m._params_to_calibrate(True)]  # pylint: disable=protected-access
+        probe = [k for k, (m, name, qtzr, param) in enumerate(todo) if m._wants_grid_recovery(qtzr)]  # pylint: disable=protected-access
+        answers = _probe_parameters_together([(todo[k][3], todo[k][2]) for k in probe])
+        verdicts = {id(m): {} for m in modules}
+        for k, answer in zip(probe, answers):
+            verdicts[id(todo[k][0])][todo[k][1]] = answer
+        plain = [w for w in todo if not verdicts[id(w[0])].get(w[1], False) and isinstance(w[2], AffineQuantizerBase)]
+        quantized = _calibrate_parameters_together(plain)
         for m in modules:
-            stack.enter_context(m.compute_encodings(_verdicts=verdicts[id(m)]))
-        yield
+            mine = {name: t for (mid, name), t in quantized.items() if mid == id(m)}
+            m._compute_param_encodings(overwrite=True, verdicts=verdicts[id(m)], quantized=mine)  # pylint: disable=protected-access
+            if any(q is not None and q.is_initialized() for q in m.param_quantizers.values()):
+                stack.enter_context(m._patch_quantized_parameters(_quantized=mine))  # pylint: disable=protected-access
+                stack.enter_context(m._remove_param_quantizers())  # pylint: disable=protected-access
+        # 2. activations: observed and passed through unquantized; ranges set on leaving (nn/base.py:392-427)
+        observing = []
+        for m in modules:
+            for qtzr in list(m.input_quantizers) + list(m.output_quantizers):
+                if not isinstance(qtzr, QuantizerBase) or not qtzr.is_overwrite_allowed():
+                    continue
+                begin = getattr(qtzr, "_begin_passthrough_calibration", None)
+                if begin is not None and "forward" not in qtzr.__dict__:
+                    if begin():
+                        observing.append(qtzr)
+                else:
+                    stack.enter_context(qtzr._compute_encodings(passthrough=True))  # pylint: disable=protected-access
+        try:
+            yield
+        finally:
+            for qtzr in observing:
+                qtzr._end_passthrough_calibration()  # pylint: disable=protected-access
+            _finalize_together(observing)
 
 
 def fold_param_quantizers(model: nn.Module):

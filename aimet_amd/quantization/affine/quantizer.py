@@ -522,14 +522,40 @@ class AffineQuantizerBase(QuantizerBase, _GridMixin):
                     _get_minimum_scale(self.qmax - self.qmin), scale.data_ptr(),
                     None if self.symmetric else offset.data_ptr(), _lib.current_stream(device)),
                 "ahq_minmax_finalize")
-        # min / max were written behind torch's back: tell autograd, and everyone who keys on the version counters
-        torch.autograd.graph.increment_version((mn, mx))
-        enc = AffineEncoding(scale, offset, self.qmin, self.qmax, self._symmetric, self.block_size,
-                             self.zero_point_shift, producer=self)
-        self.__dict__["_encoding_cache"] = (self._encoding_cache_key(), enc)
+        self._finalize_adopt(scale, offset)
         if own:
             _report_range_flags(flags)
         return True
+
+    def _finalize_adopt(self, scale: torch.Tensor, offset: torch.Tensor) -> None:
+        """What follows a finalize launch on the host: min / max were written behind torch's back (tell autograd, and
+        everyone who keys on the version counters), and the encodings the next forward would derive are at hand."""
+        torch.autograd.graph.increment_version((self.min, self.max))
+        enc = AffineEncoding(scale, offset, self.qmin, self.qmax, self._symmetric, self.block_size,
+                             self.zero_point_shift, producer=self)
+        self.__dict__["_encoding_cache"] = (self._encoding_cache_key(), enc)
+
+    def _slots_finalize_item(self):
+        """The arguments of ahq_minmax_slots_finalize for this quantizer as (item fields..., scale, offset), for a
+        caller that finalizes many quantizers with one call (aimet_amd.nn.compute_encodings); None where
+        _set_range_from_statistics() has to run: the conditions of _finalize_from_minmax(), with the running extrema
+        of a single encoding in the observer's slots."""
+        an = self.encoding_analyzer
+        cls = type(self)
+        if (type(an) is not MinMaxEncodingAnalyzer  # pylint: disable=unidiomatic-typecheck
+                or cls.get_scale is not AffineQuantizerBase.get_scale
+                or cls._get_offset is not AffineQuantizerBase._get_offset
+                or cls.set_range is not AffineQuantizerBase.set_range
+                or not all(self._is_overwrite_allowed.values())):
+            return None
+        mn, mx = self.min, self.max
+        num_steps = self._num_steps_for_calibration()
+        slots = an.observer.live_slots()
+        if (slots is None or mn.numel() != 1 or not mn.is_cuda or slots[1] != mn.device or mx.device != mn.device
+                or mn.dtype not in _lib.DTYPE_CODE or mx.dtype != mn.dtype or mn.shape != mx.shape
+                or num_steps <= 0 or num_steps > (1 << 24)):
+            return None
+        return slots[0], slots[2], num_steps
 
     def _derive_encodings(self) -> Optional[AffineEncoding]:
         if not self.is_initialized():
@@ -617,15 +643,6 @@ class AffineQuantizerBase(QuantizerBase, _GridMixin):
                 input = input.as_subclass(torch.Tensor)
             if input.numel() == 0:
                 return inner_forward(input)
-            if passthrough:
-                # the input is only observed; the dynamic encodings of this batch would go unused.  A min/max
-                # analyzer writes the clone from the pass that reads the tensor
-                fused = getattr(self.encoding_analyzer, "observe_and_clone", None)
-                if (fused is not None and input.is_cuda and input.dtype in _lib.DTYPE_CODE and input.is_contiguous()
-                        and not (torch.is_grad_enabled() and input.requires_grad)):
-                    return fused(input)
-                self.encoding_analyzer.update_stats(input)
-                return inner_forward(input)
             batch_stats = self.encoding_analyzer.update_stats(input)
             lo, hi = self.encoding_analyzer.compute_encodings_from_stats(
                 batch_stats, self._num_steps_for_calibration(), self.symmetric
@@ -644,6 +661,8 @@ class AffineQuantizerBase(QuantizerBase, _GridMixin):
                 ret.encoding = encoding
             return ret
 
+        if passthrough:
+            observing_forward = self._observe_passthrough
         if not passthrough:  # (a whole-model calibration enters hundreds of these contexts: nothing it does not need)
             functools.update_wrapper(observing_forward, inner_forward)
         self.encoding_analyzer.reset_stats()
@@ -660,6 +679,43 @@ class AffineQuantizerBase(QuantizerBase, _GridMixin):
             else:
                 own["forward"] = outer
         self._set_range_from_statistics()
+
+    def _observe_passthrough(self, input: torch.Tensor) -> torch.Tensor:
+        """The forward pass of a whole-model calibration (quantizer.py:601-640 with passthrough): the input is only
+        observed and comes back as a copy; the dynamic encodings of this batch would go unused.  A min/max analyzer
+        writes the copy from the pass that reads the tensor."""
+        if type(input) != torch.Tensor:  # pylint: disable=unidiomatic-typecheck
+            input = input.as_subclass(torch.Tensor)
+        if input.numel() == 0:
+            return input.clone()
+        fused = getattr(self.encoding_analyzer, "observe_and_clone", None)
+        if (fused is not None and input.is_cuda and input.dtype in _lib.DTYPE_CODE and input.is_contiguous()
+                and not (torch.is_grad_enabled() and input.requires_grad)):
+            return fused(input)
+        self.encoding_analyzer.update_stats(input)
+        return input.clone()
+
+    def _begin_passthrough_calibration(self) -> bool:
+        """Entering ``_compute_encodings(passthrough=True)`` without the context manager around it, for a caller
+        that enters hundreds of them and leaves them together (aimet_amd.nn.compute_encodings): statistics reset,
+        forward replaced by the observing one.  False, with nothing changed, when no end may be overwritten.  The
+        caller ends with _end_passthrough_calibration() and sets the range (_set_range_from_statistics(), or a
+        launch of its own that does the same for many quantizers)."""
+        if not any(self._is_overwrite_allowed.values()):
+            return False
+        self.encoding_analyzer.reset_stats()
+        own = self.__dict__
+        own["_forward_before_calibration"] = own.get("forward")
+        own["forward"] = self._observe_passthrough
+        return True
+
+    def _end_passthrough_calibration(self) -> None:
+        own = self.__dict__
+        outer = own.pop("_forward_before_calibration", None)
+        if outer is None:
+            own.pop("forward", None)
+        else:
+            own["forward"] = outer
 
     def _calibrate_on(self, tensor: torch.Tensor) -> None:
         """``with self._compute_encodings(passthrough=True): self(tensor)`` for a caller that drops the result (the
@@ -851,18 +907,16 @@ class QuantizeDequantize(AffineQuantizerBase):
         output.encoding = encoding
         return output
 
-    def _calibrate_and_quantize(self, tensor: torch.Tensor) -> Optional[DequantizedTensor]:
-        """``self._calibrate_on(tensor)`` followed by ``self(tensor)`` -- what a quantized module does with each of
-        its parameters when a calibration starts (nn/base.py:331-386, 296-324) -- as one library call
-        (ahq_minmax_calibrate_qdq: the three launches of the step-by-step form, same results).  None, with nothing
-        changed, when that does not apply and the two steps have to run: gradients switched on, a subclass or a
-        patched method, hooks on the quantizer, another backend or analyzer, an end that may not be overwritten,
+    def _calibrate_qdq_prepare(self, tensor: torch.Tensor):
+        """Whether calibration on `tensor` followed by its quantize-dequantize can be one library call
+        (ahq_minmax_calibrate_qdq), and with which arguments: (tensor as the library takes it, grid, layout, workspace
+        bytes, calibration steps, symmetric).  None when the two steps have to run: gradients switched on, a subclass
+        or a patched method, hooks on the quantizer, another backend or analyzer, an end that may not be overwritten,
         tensors the library does not take, or an arithmetic that would depend on the offsets' values."""
         if torch.is_grad_enabled() or type(self) is not QuantizeDequantize:  # pylint: disable=unidiomatic-typecheck
             return None
         from aimet_amd.quantization._stats import _check_reducible
         from aimet_amd.quantization.affine.backends import get_backend, hip as _hip
-        from aimet_amd.quantization.encoding_analyzer import _scalar_constants, _range_flags_buffer, _report_range_flags
         from torch.nn.modules import module as _module
 
         an = self.encoding_analyzer
@@ -914,9 +968,34 @@ class QuantizeDequantize(AffineQuantizerBase):
             nbytes = _lib.load().ahq_minmax_calibrate_qdq_workspace_bytes(_lib.DTYPE_CODE[x.dtype], layout)
             held = own["_calibrate_qdq_plan"] = (key, grid, layout, nbytes)
         _, grid, layout, nbytes = held
+        return x, grid, layout, nbytes, num_steps, symmetric
+
+    def _calibrate_qdq_adopt(self, y: torch.Tensor, scale: torch.Tensor, offset: torch.Tensor) -> DequantizedTensor:
+        """What follows the launches of ahq_minmax_calibrate_qdq on the host: min / max were written behind torch's
+        back, the encodings the next forward would derive are at hand, and `y` is the quantizer's output."""
+        torch.autograd.graph.increment_version((self.min, self.max))
+        enc = AffineEncoding(scale, offset, self.qmin, self.qmax, self._symmetric, self.block_size,
+                             self.zero_point_shift, producer=self)
+        self.__dict__["_encoding_cache"] = (self._encoding_cache_key(), enc)
+        output = y.as_subclass(DequantizedTensor)
+        output.encoding = enc
+        return output
+
+    def _calibrate_and_quantize(self, tensor: torch.Tensor) -> Optional[DequantizedTensor]:
+        """``self._calibrate_on(tensor)`` followed by ``self(tensor)`` -- what a quantized module does with each of
+        its parameters when a calibration starts (nn/base.py:331-386, 296-324) -- as one library call
+        (ahq_minmax_calibrate_qdq: the three launches of the step-by-step form, same results).  None, with nothing
+        changed, when that does not apply and the two steps have to run (see _calibrate_qdq_prepare)."""
+        from aimet_amd.quantization.encoding_analyzer import _scalar_constants, _range_flags_buffer, _report_range_flags
+
+        plan = self._calibrate_qdq_prepare(tensor)
+        if plan is None:
+            return None
+        x, grid, layout, nbytes, num_steps, symmetric = plan
+        mn, mx = self.min, self.max
         device = x.device
         ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=device)  # two statistics per encoding: not kept
-        an.reset_stats()
+        self.encoding_analyzer.reset_stats()
         consts = _scalar_constants(x.dtype, _get_minimum_scale(num_steps))
         y = torch.empty_like(x)
         scale = torch.empty(mn.shape, dtype=torch.float32, device=device)
@@ -930,14 +1009,9 @@ class QuantizeDequantize(AffineQuantizerBase):
                 _get_minimum_scale(self.qmax - self.qmin), scale.data_ptr(), offset.data_ptr(), ws.data_ptr(), nbytes,
                 _lib.current_stream(device)),
             "ahq_minmax_calibrate_qdq")
-        torch.autograd.graph.increment_version((mn, mx))
-        enc = AffineEncoding(scale, offset, self.qmin, self.qmax, self._symmetric, self.block_size,
-                             self.zero_point_shift, producer=self)
-        own["_encoding_cache"] = (self._encoding_cache_key(), enc)
+        output = self._calibrate_qdq_adopt(y, scale, offset)
         if own_flags:
             _report_range_flags(flags)
-        output = y.as_subclass(DequantizedTensor)
-        output.encoding = enc
         return output
 
     def _forward_steady(self, input: torch.Tensor) -> Optional[DequantizedTensor]:

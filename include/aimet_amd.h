@@ -257,6 +257,63 @@ int    ahq_minmax_calibrate_qdq(const ahq_grid* grid, const ahq_layout* layout, 
                                 int32_t param_dtype, void* param_min, void* param_max, double grid_minimum_scale,
                                 float* scale, float* offset, void* workspace, size_t workspace_bytes, void* stream);
 
+/* Whole-model calibration, where a model's quantized modules enter and leave their compute_encodings() contexts
+ * together (AT/nn/base.py:392-427 for every module of a QuantizationSimModel, AT/quantsim/quantsim.py:514-560): the
+ * calls above for ALL quantizers behind one call each, in the order given, so that the host spends one call on
+ * entering (every parameter: the grid test of _decompose_prequantized_tensor, then calibration + first
+ * quantize-dequantize) and one on leaving (every per-tensor activation quantizer) instead of one per quantizer.
+ * Each item holds the arguments of the single call of the same name; `flags` is shared by all items.  The items are
+ * read on the host during the call.  Returns the first failing item's status (its index is in ahq_last_error());
+ * items before it have been launched.
+ * ahq_grid_probe_many: item i writes verdicts[i]; an item the single call would answer with AHQ_ERR_UNSUPPORTED gets
+ * unsupported[i] = 1 (host array, optional) and no launch, and the call goes on.
+ * ahq_minmax_slots_finalize_many launches one workgroup per item, 16 items per launch.
+ */
+typedef struct {
+    int32_t dtype;
+    ahq_layout layout;
+    const void* x;
+    int64_t num_levels;
+} ahq_grid_probe_item;
+int ahq_grid_probe_many(const ahq_grid_probe_item* items, int64_t count, uint8_t* verdicts, uint8_t* unsupported,
+                        void* stream);
+
+typedef struct {
+    ahq_grid grid;
+    ahq_layout layout;
+    const void* x;
+    void* y;
+    int64_t num_steps;
+    int32_t symmetric;
+    float minimum_scale_in_dtype, minimum_scale, dtype_max, near_max_threshold;
+    int32_t param_dtype;
+    void* param_min;
+    void* param_max;
+    double grid_minimum_scale;
+    float* scale;
+    float* offset;
+    void* workspace;
+    size_t workspace_bytes;
+} ahq_calibrate_qdq_item;
+int ahq_minmax_calibrate_qdq_many(const ahq_calibrate_qdq_item* items, int64_t count, int32_t* flags, void* stream);
+
+typedef struct {
+    int32_t stat_dtype;
+    int32_t symmetric;
+    const void* slots;
+    int64_t num_steps;
+    float minimum_scale_in_dtype, minimum_scale, dtype_max, near_max_threshold;
+    int32_t param_dtype;
+    int32_t reserved;
+    void* param_min;
+    void* param_max;
+    int64_t qmin, qmax;
+    double grid_minimum_scale;
+    float* scale;
+    float* offset;   /* NULL for a symmetric grid */
+} ahq_slots_finalize_item;
+int ahq_minmax_slots_finalize_many(const ahq_slots_finalize_item* items, int64_t count, int32_t* flags, void* stream);
+
 /* The backward pass of ahq_lpbq_scale: replaces the autograd chain of GroupedBlockQuantizeDequantize._get_scale
  * (AT/quantization/affine/quantizer.py:1363-1399 on top of :319-342) when min / max are learned -- the backward of
  * the quantize-dequantize of the block scales (AT/quantization/affine/backends/torch_builtins.py:727-831), of the

@@ -290,3 +290,54 @@ def test_grid_probe_matches_the_sorted_sample_test(device, case, dtype):
         want = _may_be_prequantized(w, q, on_device=False)
         got = _may_be_prequantized(w.to(device), q)
         assert bool(got) == bool(want), (name, bool(got), bool(want))
+
+
+def test_calibrating_all_modules_together_equals_module_by_module(device):
+    """aimet_amd.nn.compute_encodings hands the quantizers of all modules to the library in three calls
+    (ahq_grid_probe_many, ahq_minmax_calibrate_qdq_many, ahq_minmax_slots_finalize_many); every module entering its
+    own compute_encodings() context makes one call per quantizer.  Same ranges, encodings, calibration-pass outputs and
+    quantized forward, bit for bit -- also with a weight that is already on a grid (kept), a per-channel activation
+    quantizer and one that may not be overwritten (left to their own ways)."""
+    import contextlib
+
+    batches = LH.calibration_batches(CFG, device, batches=3, seq=64)
+    results = []
+    for together in (True, False):
+        model = LH.build(CFG, device, seed=5)
+        LH.quantize(model)
+        lin = model.blocks[0].mlp.down_proj
+        # a weight already on a 4-bit grid of its quantizer's blocks
+        with torch.no_grad():
+            w = lin.weight
+            step = (w.abs().reshape(w.shape[0], -1, 64).amax(dim=2, keepdim=True) / 7).clamp_min(1e-3)
+            w.copy_((torch.round(w.reshape(w.shape[0], -1, 64) / step).clamp(-8, 7) * step).reshape(w.shape))
+        model.blocks[1].attn.q_proj.output_quantizers[0] = QuantizeDequantize((CFG.hidden,), 8, symmetric=True).to(device)
+        frozen = model.blocks[1].mlp.up_proj.input_quantizers[0]
+        frozen.set_range(torch.tensor(-3.0, device=device), torch.tensor(5.0, device=device))
+        frozen.allow_overwrite(False)
+        outs = []
+        with torch.no_grad():
+            if together:
+                ctx = qnn.compute_encodings(model)
+            else:
+                ctx = contextlib.ExitStack()
+                for m in qnn.quantized_linears(model):
+                    ctx.enter_context(m.compute_encodings())
+            with ctx:
+                for ids in batches:
+                    outs.append(model(ids))
+            outs.append(model(batches[0]))
+        quantizers = {n: m for n, m in model.named_modules() if isinstance(m, QuantizeDequantize)}
+        state = {n: (q.min.detach().clone(), q.max.detach().clone(), q.get_scale().detach().clone(),
+                     q.get_offset().detach().clone()) for n, q in quantizers.items()}
+        assert all(q.is_initialized() for q in quantizers.values())
+        assert "forward" not in frozen.__dict__ and all("forward" not in q.__dict__ for q in quantizers.values())
+        results.append((state, outs))
+    (a_state, a_outs), (b_state, b_outs) = results
+    assert a_state.keys() == b_state.keys()
+    for name in a_state:
+        for x, y in zip(a_state[name], b_state[name]):
+            assert torch.equal(_bits(x), _bits(y)), name
+    for x, y in zip(a_outs, b_outs):
+        assert torch.equal(_bits(x), _bits(y))
+    assert float(a_state["blocks.1.mlp.up_proj.input_quantizers.0"][0]) == -3.0
