@@ -157,36 +157,13 @@ def calibration_batches(cfg: LlamaConfig, device, batches: int = 8, seq: int = 2
     return [torch.randint(0, cfg.vocab, (batch, seq), generator=g).to(device) for _ in range(batches)]
 
 
-def calibrate(model: nn.Module, batches, use_graph: bool = False):
-    """compute_encodings over ``batches`` (the reference flow: aimet_torch.nn.compute_encodings around forward passes).
-
-    ``use_graph``: the passes are host-bound (a few hundred small launches per pass), so after one eager pass -- which
-    creates every observer's running statistics -- the second pass is captured into a HIP graph and replayed for it
-    and every later batch.  Inside a pass the observers only fold the batch's extrema into their running tensors in
-    place and pass the activations through, and the weight quantizers reuse their cached encodings, so a replay does
-    exactly what the eager pass would.  Needs batches of one shape; fewer than three batches run eagerly."""
+def calibrate(model: nn.Module, batches):
+    """compute_encodings over ``batches`` (the reference flow: aimet_torch.nn.compute_encodings around forward passes)."""
     from aimet_amd import nn as qnn
 
-    batches = list(batches)
     with torch.no_grad(), qnn.compute_encodings(model):
-        if not use_graph or len(batches) < 3 or any(b.shape != batches[0].shape for b in batches):
-            for b in batches:
-                model(b)
-            return
-        model(batches[0])
-        static_ids = batches[1].clone()
-        side = torch.cuda.Stream()
-        side.wait_stream(torch.cuda.current_stream())
-        with torch.cuda.stream(side):
-            model(static_ids)  # warm-up on the capture stream (allocator pools, GEMM heuristics); observes batch 1
-        torch.cuda.current_stream().wait_stream(side)
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph, stream=side):
-            model(static_ids)
-        for b in batches[2:]:
-            static_ids.copy_(b)
-            graph.replay()
-        torch.cuda.current_stream().synchronize()
+        for b in batches:
+            model(b)
 
 
 def linear_flops(cfg: LlamaConfig, tokens: int) -> float:

@@ -141,3 +141,106 @@ def test_histogram_counts_are_additive_at_full_size(device):
     # the batch's own histogram against torch.histc on the device (same formula, counts below 2^24 are exact)
     lo, hi = float(first.min), float(first.max)
     assert torch.equal(first.histogram.view(-1), torch.histc(x, 512, lo, hi))
+
+
+def _laplace_with_outliers(shape, seed, device):
+    """One batch of the calibration stream: Laplace(0, 1), 0.1 % of the elements replaced by +-U(20, 60)."""
+    g = torch.Generator(device=device).manual_seed(seed)
+    u = (torch.rand(shape, generator=g, device=device) - 0.5).clamp_(-0.4999999, 0.4999999)
+    x = -torch.sign(u) * torch.log1p(-2 * u.abs())
+    n = x.numel()
+    k = n // 1000
+    idx = torch.randint(0, n, (k,), generator=g, device=device)
+    out = (torch.rand(k, generator=g, device=device) * 40 + 20) * torch.sign(torch.rand(k, generator=g, device=device) - 0.5)
+    x.view(-1)[idx] = out
+    return x
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+def test_histogram_stream_and_candidate_search_at_the_benchmark_shape(device, dtype):
+    """Four batches of [8, 2048, 4096] through SqnrEncodingAnalyzer(512 bins, 100 x 64 candidates, 8-bit asymmetric)
+    against the oracle on the same batches: running counts (the fullest bin passes 2^24 with the third batch, from
+    where float32 counts round), edges, range, the candidate chosen and the encoding, bit for bit.  bf16: the same
+    through the table-binning kernel."""
+    from aimet_amd.quantization.encoding_analyzer import SqnrEncodingAnalyzer
+
+    an = SqnrEncodingAnalyzer((1,), num_bins=512, asymmetric_delta_candidates=100, offset_candidates=64, gamma=3.0)
+    ref = O.HistObserver((1,), 512)
+    for b in range(4):
+        x = _laplace_with_outliers((8, 2048, 4096), b, device).to(dtype)
+        an.update_stats(x)
+        ref.update(x.cpu())
+        del x
+    st, st_ref = an.observer.get_stats()[0], ref.stats[0]
+    assert float(st_ref.histogram.max()) > 2 ** 24
+    assert_same_bits(st.histogram, st_ref.histogram, "running counts")
+    assert_same_bits(st.bin_edges, st_ref.bin_edges, "bin edges")
+    assert_same_bits(st.min, st_ref.min, "min")
+    assert_same_bits(st.max, st_ref.max, "max")
+    lo, hi = an.compute_encodings(255, False)
+    lo_r, hi_r, _, _, best = O.sqnr_encodings(ref.stats, (1,), 255, False, asym_deltas=100, num_offsets=64, gamma=3.0)
+    assert int(an.last_search["best_index"].item()) == int(best.item())
+    assert_same_bits(lo, lo_r, "encoding min")
+    assert_same_bits(hi, hi_r, "encoding max")
+
+
+def test_decoder_layer_at_the_benchmark_shape(device):
+    """One decoder layer of the whole-model configuration (hidden 2048, FFN 8192, 32 heads, sequence 2048, bf16;
+    W4 blocks of 64, A16 per tensor at every Linear input and output; a small vocabulary keeps the CPU side short):
+    two calibration batches through aimet_amd.nn.compute_encodings, then a quantized forward.  Every quantizer's
+    calibrated range, scale and offset, and its output in the quantized forward, against the oracle on the very
+    tensors it saw."""
+    import llama_harness as LH
+    from aimet_amd import nn as qnn
+    from aimet_amd.quantization.affine import QuantizeDequantize
+
+    cfg = LH.LlamaConfig(layers=1, hidden=2048, ffn=8192, heads=32, vocab=4096)
+    model = LH.build(cfg, device, seed=0)
+    assert LH.quantize(model) == 8
+    quantizers = {n: m for n, m in model.named_modules() if isinstance(m, QuantizeDequantize)}
+    weights = {f"{n}.param_quantizers.weight": m.weight for n, m in model.named_modules()
+               if isinstance(m, qnn.QuantizedLinear)}
+    assert len(quantizers) == 24 and len(weights) == 8
+    stats = {}
+
+    def observe(name, q):
+        def hook(_mod, args, _out):
+            a, b = O.reduce_minmax(args[0].detach().cpu(), tuple(q.shape), q.block_size)
+            if name in stats:
+                a, b = torch.minimum(a, stats[name][0]), torch.maximum(b, stats[name][1])
+            stats[name] = (a, b)
+        return hook
+
+    hooks = [q.register_forward_hook(observe(n, q)) for n, q in quantizers.items() if n not in weights]
+    batches = LH.calibration_batches(cfg, device, batches=2, seq=2048)
+    LH.calibrate(model, batches)
+    for h in hooks:
+        h.remove()
+    for name, w in weights.items():  # (no hook on these: they take the one-call form, on the weight itself)
+        q = quantizers[name]
+        stats[name] = O.reduce_minmax(w.detach().cpu(), tuple(q.shape), q.block_size)
+    for name, q in quantizers.items():
+        lo, hi = O.minmax_encodings(*stats[name], q.qmax - q.qmin, q.symmetric)
+        assert_same_bits(q.min.detach(), lo.view(q.shape).to(torch.float32), f"{name}: min")
+        assert_same_bits(q.max.detach(), hi.view(q.shape).to(torch.float32), f"{name}: max")
+        scale = O.scale_from_minmax(q.min.detach().cpu(), q.max.detach().cpu(), q.qmin, q.qmax)
+        assert_same_bits(q.get_scale().detach(), scale, f"{name}: scale")
+        assert_same_bits(q.get_offset().detach(),
+                         O.offset_from_minmax(q.min.detach().cpu(), scale, q.qmin, q.qmax, q.symmetric), f"{name}: offset")
+    io = {}
+    hooks = [q.register_forward_hook(lambda _m, args, out, key=n: io.__setitem__(key, (args[0].detach().cpu(),
+                                                                                        out.detach().cpu())))
+             for n, q in quantizers.items()]
+    with torch.no_grad():
+        logits = model(batches[0])
+    for h in hooks:
+        h.remove()
+    assert torch.isfinite(logits.float()).all() and len(io) == 24
+    for name, q in quantizers.items():
+        x, y = io[name]
+        scale, offset = q.get_scale().detach().cpu(), q.get_offset().detach().cpu()
+        if q.block_size is None:
+            want = O.qdq_v1(x, scale, offset, q.qmin, q.qmax)[0]   # no gradients: the ATen fake-quantize arithmetic
+        else:
+            want = O.qdq_v2_forward(x, scale, offset, q.qmin, q.qmax, q.block_size).y
+        assert_same_bits(y.as_subclass(torch.Tensor), want, f"{name}: forward")
