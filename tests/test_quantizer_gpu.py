@@ -1113,3 +1113,154 @@ def test_lpbq_forward_with_gradients_as_one_autograd_node(device, monkeypatch, c
         for a, b, what in zip(one[:4], two[:4], ("output", "input gradient", "gradient of min", "gradient of max")):
             assert_same_bits(a, b, f"{what} (loss through the encoding: {through_encoding})")
         assert float(one[2].abs().sum()) > 0 and float(one[3].abs().sum()) > 0
+
+
+# ------------------------------------------------------- quantizers that hold their encoding as scale / offset --
+@pytest.mark.parametrize("case", CASES, ids=lambda c: c[0])
+def test_scale_offset_parametrisation_forward_backward(device, case):
+    """A quantizer reparametrized to (scale, offset) computes what it computed before (same scale, same offset, hence
+    the same bits out and the same input gradient), and its gradients reach scale and offset themselves: those are the
+    oracle's scale and offset gradients (offset through the straight-through rounding, i.e. unchanged)."""
+    from aimet_amd.quantization.affine import QuantizeDequantize
+
+    _, xshape, dtype, qshape, bw, sym, block = case
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(xshape, generator=g)
+    if not sym:
+        x = torch.relu(x)
+    x = x.to(dtype)
+    grad = torch.randn(xshape, generator=g).to(dtype)
+    n = 2 ** bw - 1
+    qmin, qmax = (-math.ceil(n / 2), math.floor(n / 2)) if sym else (0, n)
+
+    q = QuantizeDequantize(qshape, bw, sym, block_size=block).to(device)
+    xd = x.to(device)
+    with q.compute_encodings():
+        q(xd)
+    scale, offset = q.get_scale().detach().clone(), q.get_offset().detach().clone()
+    with torch.no_grad():
+        y_min_max = q(xd).clone()
+    y_learning = q(xd).detach().clone()  # learned encodings take the composed arithmetic: other bits in 16-bit types
+    q._reparametrize_to_scale_offset()
+    assert q._is_scale_offset_quantizer() and q.is_initialized() and q.scale.device == xd.device
+    assert_same_bits(q.get_scale(), scale, "scale after reparametrizing")
+    assert_same_bits(q.get_offset(), offset, "offset after reparametrizing")
+    with torch.no_grad():
+        assert_same_bits(q(xd), y_min_max, "forward without gradients")
+
+    xg = xd.clone().requires_grad_(True)
+    y = q(xg)
+    assert type(y).__name__ == "DequantizedTensor"
+    assert_same_bits(y, y_learning, "forward with gradients")
+    y.backward(grad.to(device))
+    sc, of = scale.cpu(), offset.cpu()
+    ref_y = O.qdq_v2_forward(x, sc, of, qmin, qmax, block, 0.0).y
+    assert_same_bits(y, ref_y, "forward against the oracle")
+    gx, gs, go = O.qdq_v2_backward(grad, x, sc, of, qmin, qmax, block, 0.0)
+    assert_same_bits(xg.grad, gx, "input gradient")
+    D = O.internal_dtype(dtype, qmin, qmax)
+    # float32: up to 25088 signed terms per encoding, summed in two different orders and cancelling to a few percent
+    # of their absolute sum -- 4e-5 of the result is a few units in the last place of that absolute sum
+    tol = 4e-5 if D == torch.float32 else float(torch.finfo(D).eps)
+    assert_close_rel(q.scale.grad, gs.view(qshape), tol, "scale gradient", abs_floor=1e-30)
+    if sym:
+        assert q.offset is None
+    else:
+        assert_close_rel(q.offset.grad, go.view(qshape), tol, "offset gradient", abs_floor=1e-30)
+
+    # calibrating again goes through set_range(): the same encodings as a min/max quantizer finds
+    fresh = QuantizeDequantize(qshape, bw, sym, block_size=block).to(device)
+    fresh._reparametrize_to_scale_offset()
+    with fresh.compute_encodings():
+        fresh(xd)
+    assert_same_bits(fresh.get_scale(), scale, "scale of a calibrated scale/offset quantizer")
+    assert_same_bits(fresh.get_offset(), offset, "offset of a calibrated scale/offset quantizer")
+    q._reparametrize_to_min_max()
+    with torch.no_grad():
+        assert_same_bits(q(xd), y_min_max, "forward after reparametrizing back")
+
+
+@pytest.mark.parametrize("params", ["min_max", "scale_offset"])
+def test_import_signed_flag(device, params):
+    """Reference expectation: test_affine_quantizer.py:1592-1627."""
+    from aimet_amd.quantization.affine import QuantizeDequantize
+
+    symmetric_quantizer = QuantizeDequantize((1,), 8, symmetric=True).to(device)
+    asymmetric_quantizer = QuantizeDequantize((1,), 8, symmetric=False).to(device)
+    if params == "scale_offset":
+        symmetric_quantizer._reparametrize_to_scale_offset()
+        asymmetric_quantizer._reparametrize_to_scale_offset()
+    assert symmetric_quantizer.signed
+    g = torch.Generator().manual_seed(0)
+    with symmetric_quantizer.compute_encodings():
+        symmetric_quantizer(torch.randn(10, generator=g).to(device))
+    asymmetric_quantizer.set_legacy_encodings(symmetric_quantizer.get_legacy_encodings())
+    assert asymmetric_quantizer.signed and asymmetric_quantizer.symmetric
+    x = torch.randn(10, generator=g).to(device)
+    assert_same_bits(asymmetric_quantizer(x), symmetric_quantizer(x), "the same encodings after the import")
+
+    asymmetric_quantizer = QuantizeDequantize((), 8, symmetric=False).to(device)
+    if params == "scale_offset":
+        asymmetric_quantizer._reparametrize_to_scale_offset()
+    with asymmetric_quantizer.compute_encodings():
+        asymmetric_quantizer(torch.randn(10, generator=g).to(device))
+    symmetric_quantizer.set_legacy_encodings(asymmetric_quantizer.get_legacy_encodings())
+    assert not symmetric_quantizer.signed and not symmetric_quantizer.symmetric
+
+
+def test_grouped_block_quantizer_held_as_scale_offset(device):
+    from aimet_amd.quantization.affine import GroupedBlockQuantizeDequantize
+
+    g = torch.Generator().manual_seed(3)
+    w = torch.randn(16, 256, generator=g).to(device)
+    q = GroupedBlockQuantizeDequantize((16, 8), 4, True, 8, block_size=(1, 32), block_grouping=(1, 8)).to(device)
+    with q.compute_encodings():
+        q(w)
+    scale, per_channel = q.get_scale().clone(), q.get_per_channel_scale().clone()
+    with torch.no_grad():
+        y = q(w).clone()
+    q._reparametrize_to_scale_offset()
+    assert_same_bits(q.get_scale(), scale, "snapped block scales")
+    assert_same_bits(q.get_per_channel_scale(), per_channel, "per-channel scales")
+    with torch.no_grad():
+        assert_same_bits(q(w), y, "forward without gradients")
+    wg = w.clone().requires_grad_(True)
+    out = q(wg)
+    assert_same_bits(out, y, "forward with gradients")
+    out.sum().backward()
+    assert q.scale.grad is not None and torch.isfinite(q.scale.grad).all()
+
+
+def test_model_calibration_with_a_scale_offset_parameter_quantizer(device):
+    """The batched calibration of a whole model leaves a quantizer held as scale / offset to the generic route; its
+    encodings come out as those of its min/max twin."""
+    import copy as _copy
+
+    import aimet_amd.nn as qnn
+    from aimet_amd.quantization.affine import QuantizeDequantize
+
+    torch.manual_seed(0)
+
+    def build():
+        lin = qnn.QuantizedLinear(64, 32, bias=False).to(device)
+        lin.param_quantizers["weight"] = QuantizeDequantize((32, 1), 8, True).to(device)
+        lin.input_quantizers[0] = QuantizeDequantize((), 8, False).to(device)
+        lin.output_quantizers[0] = QuantizeDequantize((), 8, False).to(device)
+        return lin
+
+    a = build()
+    b = _copy.deepcopy(a)
+    for qz in (b.param_quantizers["weight"], b.input_quantizers[0]):
+        qz._reparametrize_to_scale_offset()
+    x = torch.randn(8, 64, device=device)
+    for m in (a, b):
+        with qnn.compute_encodings(m):
+            m(x)
+    for qa, qb in ((a.param_quantizers["weight"], b.param_quantizers["weight"]),
+                   (a.input_quantizers[0], b.input_quantizers[0]), (a.output_quantizers[0], b.output_quantizers[0])):
+        assert qb.is_initialized()
+        assert_same_bits(qb.get_scale(), qa.get_scale(), "scale")
+        assert_same_bits(qb.get_offset(), qa.get_offset(), "offset")
+    assert b.param_quantizers["weight"]._is_scale_offset_quantizer()
+    with torch.no_grad():
+        assert_same_bits(b(x), a(x), "layer output")

@@ -1,0 +1,221 @@
+"""Host logic of the two ways a quantizer can hold its encoding -- (min, max) or (scale, offset) -- and of the legacy
+list-of-dictionaries form: nothing here launches a kernel.  Expectations follow the reference's own tests
+(TrainingExtensions/torch/test/python/v2/quantization/affine/test_affine_quantizer.py: the "scale_offset" fixtures,
+the state-dict cross-loading case and test_import_signed_flag) and quantizer.py:195-285, 319-438, 480-571."""
+
+import copy
+import pickle
+
+import pytest
+import torch
+
+from aimet_amd.quantization.affine import Quantize, QuantizeDequantize
+
+LO = torch.tensor([[-1.0], [-2.0], [-0.5], [0.0]])
+HI = torch.tensor([[1.0], [3.0], [0.25], [4.0]])
+
+
+def _initialized(cls, symmetric):
+    q = cls((4, 1), 8, symmetric=symmetric)
+    q.set_range(LO, HI)
+    return q
+
+
+@pytest.mark.parametrize("cls", [Quantize, QuantizeDequantize])
+@pytest.mark.parametrize("symmetric", [True, False])
+def test_a_new_quantizer_holds_min_and_max(cls, symmetric):
+    q = cls((4, 1), 8, symmetric=symmetric)
+    assert q._is_min_max_quantizer() and not q._is_scale_offset_quantizer()
+    assert list(q._parameters) == ["min", "max"]
+    q._reparametrize_to_min_max()  # no change, no error
+    assert list(q._parameters) == ["min", "max"] and not q.is_initialized()
+
+
+@pytest.mark.parametrize("cls", [Quantize, QuantizeDequantize])
+@pytest.mark.parametrize("symmetric", [True, False])
+def test_reparametrizing_before_initialisation(cls, symmetric):
+    q = cls((4, 1), 8, symmetric=symmetric)
+    q._reparametrize_to_scale_offset()
+    assert q._is_scale_offset_quantizer() and not q._is_min_max_quantizer()
+    assert list(q._parameters) == ["scale", "offset"]
+    assert (q.offset is None) == symmetric and q.symmetric == symmetric
+    assert not q.is_initialized()
+    assert q.get_scale() is None and q.get_offset() is None and q.get_min() is None and q.get_max() is None
+    assert q.get_encodings() is None and q.get_legacy_encodings() is None
+    # a range in part cannot be given to a quantizer that holds no range to complete it with
+    with pytest.raises(ValueError):
+        q.set_range(0.0, None)
+    with pytest.raises(ValueError):
+        q.set_range(None, 1.0)
+    q.set_range(LO, HI)
+    assert q.is_initialized()
+
+
+@pytest.mark.parametrize("cls", [Quantize, QuantizeDequantize])
+@pytest.mark.parametrize("symmetric", [True, False])
+def test_reparametrizing_keeps_the_encoding(cls, symmetric):
+    q = _initialized(cls, symmetric)
+    scale, offset, lo, hi = q.get_scale(), q.get_offset(), q.get_min(), q.get_max()
+    q._reparametrize_to_scale_offset()
+    assert q.is_initialized()
+    assert q.scale.dtype == torch.float32 and tuple(q.scale.shape) == (4, 1)
+    assert torch.equal(q.scale, scale)
+    if symmetric:
+        assert q.offset is None
+    else:
+        assert torch.equal(q.offset, offset)
+    for got, want in ((q.get_scale(), scale), (q.get_offset(), offset), (q.get_min(), lo), (q.get_max(), hi)):
+        assert torch.equal(got, want)
+    enc = q.get_encodings()
+    assert torch.equal(enc.scale, scale) and torch.equal(enc.offset, offset) and enc.symmetry == symmetric
+    # and back: min = scale * (offset + qmin), max = scale * (offset + qmax)
+    q._reparametrize_to_min_max()
+    assert list(q._parameters) == ["min", "max"] and q.is_initialized()
+    assert torch.equal(q.min, scale * (offset + q.qmin)) and torch.equal(q.max, scale * (offset + q.qmax))
+    assert torch.equal(q.get_scale(), scale) and torch.equal(q.get_offset(), offset)
+
+
+def test_closed_form_of_an_asymmetric_range():
+    # 8 bit over [0, 255]: scale 1 and offset 0; over [-128, 127]: scale 1, offset -128
+    q = QuantizeDequantize((), 8, symmetric=False)
+    q._reparametrize_to_scale_offset()
+    q.set_range(0.0, 255.0)
+    assert q.scale.item() == 1.0 and q.offset.item() == 0.0
+    q.set_range(-128.0, 127.0)
+    assert q.scale.item() == 1.0 and q.offset.item() == -128.0
+    # one end only: the other is the one held
+    q.set_range(None, 382.0)  # [-128, 382] -> scale 2, offset -64
+    assert q.scale.item() == 2.0 and q.offset.item() == -64.0
+    assert q.get_min().item() == -128.0 and q.get_max().item() == 382.0
+    s = QuantizeDequantize((), 8, symmetric=True)
+    s._reparametrize_to_scale_offset()
+    s.set_range(-128.0, 127.0)
+    assert s.scale.item() == 1.0 and s.offset is None and s.get_offset().item() == 0.0  # a signed grid is centred
+
+
+@pytest.mark.parametrize("symmetric", [True, False])
+def test_which_parameters_learn_is_kept(symmetric):
+    q = _initialized(QuantizeDequantize, symmetric)
+    q.requires_grad_(False)
+    q._reparametrize_to_scale_offset()
+    assert not q.scale.requires_grad and (q.offset is None or not q.offset.requires_grad)
+    q._reparametrize_to_min_max()
+    assert not q.min.requires_grad and not q.max.requires_grad
+    q.min.requires_grad_(True)  # one learned end is enough
+    q._reparametrize_to_scale_offset()
+    assert q.scale.requires_grad and (q.offset is None or q.offset.requires_grad)
+
+
+def test_scale_and_offset_stay_float32_whatever_min_and_max_were():
+    q = _initialized(QuantizeDequantize, False).to(torch.bfloat16)
+    q._reparametrize_to_scale_offset()
+    assert q.scale.dtype == torch.float32 and q.offset.dtype == torch.float32
+
+
+@pytest.mark.parametrize("symmetric", [True, False])
+def test_attribute_errors_name_the_way_out(symmetric):
+    q = _initialized(QuantizeDequantize, symmetric)
+    with pytest.raises(AttributeError, match=r"parametrized with min/max.*get_scale\(\)"):
+        q.scale  # pylint: disable=pointless-statement
+    q._reparametrize_to_scale_offset()
+    with pytest.raises(AttributeError, match=r"parametrized with scale/offset.*get_min\(\).*set_range\(\)"):
+        q.min  # pylint: disable=pointless-statement
+    with pytest.raises(AttributeError) as e:
+        q.no_such_thing  # pylint: disable=pointless-statement
+    assert "parametrized" not in str(e.value)
+
+
+@pytest.mark.parametrize("symmetric", [True, False])
+@pytest.mark.parametrize("strict", [True, False])
+def test_state_dicts_do_not_cross_parametrisations(symmetric, strict):
+    """test_affine_quantizer.py:1050-1075: a min/max state dict into a scale/offset quantizer, and the other way round,
+    is an error in either strictness."""
+    min_max = _initialized(QuantizeDequantize, symmetric)
+    scale_offset = copy.deepcopy(min_max)
+    scale_offset._reparametrize_to_scale_offset()
+    with pytest.raises(RuntimeError):
+        min_max.load_state_dict(scale_offset.state_dict(), strict=strict)
+    with pytest.raises(RuntimeError):
+        scale_offset.load_state_dict(min_max.state_dict(), strict=strict)
+    # the same parametrisation loads, and marks the parameters initialised
+    fresh = QuantizeDequantize((4, 1), 8, symmetric=symmetric)
+    fresh._reparametrize_to_scale_offset()
+    assert not fresh.is_initialized()
+    fresh.load_state_dict(scale_offset.state_dict(), strict=strict)
+    assert fresh.is_initialized() and torch.equal(fresh.get_min(), min_max.get_min())
+
+
+def test_a_non_strict_load_may_change_the_shape_of_scale_and_offset():
+    src = _initialized(QuantizeDequantize, False)
+    src._reparametrize_to_scale_offset()
+    dst = QuantizeDequantize((), 8, symmetric=False)
+    dst._reparametrize_to_scale_offset()
+    with pytest.raises(RuntimeError):
+        dst.load_state_dict(src.state_dict(), strict=True)
+    dst.load_state_dict(src.state_dict(), strict=False)
+    assert dst.shape == (4, 1) and torch.equal(dst.scale, src.scale) and torch.equal(dst.offset, src.offset)
+
+
+@pytest.mark.parametrize("symmetric", [True, False])
+def test_copies_and_pickles_keep_the_parametrisation(symmetric):
+    q = _initialized(QuantizeDequantize, symmetric)
+    q._reparametrize_to_scale_offset()
+    for clone in (copy.deepcopy(q), pickle.loads(pickle.dumps(q))):
+        assert clone._is_scale_offset_quantizer() and clone.is_initialized() and clone.symmetric == symmetric
+        assert torch.equal(clone.get_min(), q.get_min()) and torch.equal(clone.get_max(), q.get_max())
+    blank = QuantizeDequantize((4, 1), 8, symmetric=symmetric)
+    blank._reparametrize_to_scale_offset()
+    assert not copy.deepcopy(blank).is_initialized()
+
+
+def test_symmetry_of_a_scale_offset_quantizer_is_whether_it_holds_an_offset():
+    q = _initialized(QuantizeDequantize, False)
+    q._reparametrize_to_scale_offset()
+    q.symmetric = True
+    assert q.offset is None and q.symmetric
+    q.symmetric = False
+    assert q.offset is not None and not q.symmetric
+    assert torch.equal(q.offset, torch.full((4, 1), -128.0))  # starts from the symmetric grid's constant
+    q.symmetric = True
+    q._reparametrize_to_min_max()
+    assert q.symmetric
+
+
+@pytest.mark.parametrize("params", ["min_max", "scale_offset"])
+def test_legacy_encodings_carry_grid_and_range(params):
+    """The legacy form knows signed-symmetric and unsigned-asymmetric grids; loading one into a quantizer of the
+    other kind converts it (test_affine_quantizer.py:1592-1627, with set_range in place of a calibration pass)."""
+    sym = QuantizeDequantize((1,), 8, symmetric=True)
+    asym = QuantizeDequantize((1,), 8, symmetric=False)
+    if params == "scale_offset":
+        sym._reparametrize_to_scale_offset()
+        asym._reparametrize_to_scale_offset()
+    assert sym.signed and sym.get_legacy_encodings() is None
+    sym.set_range(torch.tensor([-2.0]), torch.tensor([2.0 * 127 / 128]))
+    legacy = sym.get_legacy_encodings()
+    assert len(legacy) == 1 and set(legacy[0]) == {"min", "max", "scale", "offset", "bitwidth", "dtype", "is_symmetric"}
+    assert legacy[0]["bitwidth"] == 8 and legacy[0]["dtype"] == "int" and legacy[0]["is_symmetric"] == "True"
+    assert legacy[0]["offset"] == -128 and legacy[0]["scale"] == pytest.approx(2.0 / 128)
+    asym.set_legacy_encodings(legacy)
+    assert asym.signed and asym.symmetric and (asym.qmin, asym.qmax) == (-128, 127)
+    assert torch.equal(asym.get_min(), sym.get_min()) and torch.equal(asym.get_max(), sym.get_max())
+
+    asym = QuantizeDequantize((), 8, symmetric=False)
+    if params == "scale_offset":
+        asym._reparametrize_to_scale_offset()
+    asym.set_range(-1.0, 3.0)
+    sym.set_legacy_encodings(asym.get_legacy_encodings())
+    assert not sym.signed and not sym.symmetric and (sym.qmin, sym.qmax) == (0, 255)
+    assert sym.get_min().item() == pytest.approx(asym.get_min().item(), abs=1e-6)
+    assert sym.get_max().item() == pytest.approx(asym.get_max().item(), abs=1e-6)
+    with pytest.raises(ValueError):
+        sym.set_legacy_encodings([dict(asym.get_legacy_encodings()[0], is_symmetric="maybe")])
+
+
+def test_legacy_encodings_one_dictionary_per_channel():
+    q = _initialized(QuantizeDequantize, False)
+    legacy = q.get_legacy_encodings()
+    assert len(legacy) == 4
+    other = QuantizeDequantize((4, 1), 8, symmetric=True)
+    other.set_legacy_encodings(legacy)
+    assert torch.allclose(other.get_min(), q.get_min(), atol=1e-6) and torch.allclose(other.get_max(), q.get_max(), atol=1e-6)
