@@ -199,6 +199,23 @@ class QuantizedLinear(nn.Linear):
             stack.enter_context(patch_attr(self, name, param))
         return stack
 
+    def _params_quantized_once(self):
+        """Names of the parameters whose quantize-dequantized value may be formed once for a whole calibration context
+        instead of in every pass: the quantizer holds encodings, and no gradient can be wanted through it (gradients
+        are switched off, or neither the parameter nor the quantizer learns).  Every other parameter quantizer stays
+        in place and runs in every pass, as in the reference (nn/base.py:392-427): a pass then builds its own graph,
+        and a quantizer without encodings raises in forward."""
+        names = []
+        grad = torch.is_grad_enabled()
+        for name, qtzr in self.param_quantizers.items():
+            param = getattr(self, name)
+            if qtzr is None or param is None or not qtzr.is_initialized():
+                continue
+            if grad and (param.requires_grad or any(p.requires_grad for p in qtzr.parameters())):
+                continue
+            names.append(name)
+        return names
+
     @contextlib.contextmanager
     def _remove_param_quantizers(self, keys=None):
         """nn/base.py:995-1005."""
@@ -234,14 +251,16 @@ class QuantizedLinear(nn.Linear):
         quantized = {}
         self._compute_param_encodings(overwrite=True, verdicts=_verdicts, quantized=quantized)
         with contextlib.ExitStack() as stack:
-            # Neither the parameters nor their (just computed) encodings change inside the context, so the
-            # quantize-dequantized parameters are the same in every calibration pass: they are formed once here and
-            # the passes use them (the reference calls the parameter quantizers again in every pass, with the same
-            # result; its own _patch_quantized_parameters / fold_param_quantizers, nn/base.py:296-324, 1103-1151, are
-            # the same trade).  A caller that modifies a parameter in place inside the context sees the old values.
-            if any(q is not None and q.is_initialized() for q in self.param_quantizers.values()):
-                stack.enter_context(self._patch_quantized_parameters(_quantized=quantized))
-                stack.enter_context(self._remove_param_quantizers())
+            # Neither the parameters nor their (just computed) encodings change inside the context, so where no
+            # gradient can be wanted the quantize-dequantized parameters are the same in every calibration pass: they
+            # are formed once here and the passes use them (the reference calls the parameter quantizers again in
+            # every pass, with the same result; its own _patch_quantized_parameters / fold_param_quantizers,
+            # nn/base.py:296-324, 1103-1151, are the same trade).  A caller that modifies such a parameter in place
+            # inside the context sees the old values, and reads None for its quantizer.
+            once = self._params_quantized_once()
+            if once:
+                stack.enter_context(self._patch_quantized_parameters(once, _quantized=quantized))
+                stack.enter_context(self._remove_param_quantizers(once))
             for qtzr in list(self.input_quantizers) + list(self.output_quantizers):
                 if not isinstance(qtzr, QuantizerBase) or not qtzr.is_overwrite_allowed():
                     continue
@@ -434,9 +453,10 @@ def compute_encodings(model: nn.Module):
         for m in modules:
             mine = {name: t for (mid, name), t in quantized.items() if mid == id(m)}
             m._compute_param_encodings(overwrite=True, verdicts=verdicts[id(m)], quantized=mine)  # pylint: disable=protected-access
-            if any(q is not None and q.is_initialized() for q in m.param_quantizers.values()):
-                stack.enter_context(m._patch_quantized_parameters(_quantized=mine))  # pylint: disable=protected-access
-                stack.enter_context(m._remove_param_quantizers())  # pylint: disable=protected-access
+            once = m._params_quantized_once()  # pylint: disable=protected-access
+            if once:
+                stack.enter_context(m._patch_quantized_parameters(once, _quantized=mine))  # pylint: disable=protected-access
+                stack.enter_context(m._remove_param_quantizers(once))  # pylint: disable=protected-access
         # 2. activations: observed and passed through unquantized; ranges set on leaving (nn/base.py:392-427)
         observing = []
         for m in modules:

@@ -552,7 +552,9 @@ int ahq_float_dequantize(int32_t dtype, const ahq_layout* layout, const void* x,
 int ahq_dlq_percentile_encodings(const ahq_dlq_pdf_state* state, float percentile, int32_t bw, int32_t symmetric,
                                  int32_t strict, int32_t unsigned_sym, double* out, void* stream);
 
-/* Measurement aids for the benchmark; no counterpart in the reference.  ahq_diag_read streams `bytes` bytes through
+/* Diagnostics, outside the drop-in boundary: measurement aids for the benchmark with no counterpart in the reference;
+ * nothing that replaces a reference call uses them and a binding of the reference need not declare them.
+ * ahq_diag_read streams `bytes` bytes through
  * 16-byte loads (non-temporal ones if `nontemporal`) and folds them into one word per workgroup (out: `workgroups`
  * words); ahq_diag_copy copies them.  Both are persistent grid-stride kernels of `workgroups` x 256 threads.  x, y:
  * 16-byte aligned, bytes a multiple of 16.  What they reach on buffers that are not already in the last-level cache is

@@ -318,3 +318,51 @@ def test_calibrating_all_modules_together_equals_module_by_module(device):
     for x, y in zip(a_outs, b_outs):
         assert torch.equal(_bits(x), _bits(y))
     assert float(a_state["blocks.1.mlp.up_proj.input_quantizers.0"][0]) == -3.0
+
+
+@pytest.mark.parametrize("together", [True, False], ids=["model_context", "module_context"])
+def test_calibration_context_with_gradients_wanted(device, together):
+    """With gradients switched on and a weight (or its quantizer) that learns, the parameter quantizers stay in place
+    and run in every pass, as in the reference (nn/base.py:392-427): each pass builds its own graph, so a backward in
+    every pass works, and the quantizers are there to be read.  Without gradients the quantize-dequantized weight is
+    formed once and the quantizer steps aside for the length of the context; the outputs are the same."""
+    torch.manual_seed(0)
+    lin = qnn.QuantizedLinear(64, 32, bias=False).to(device)
+    lin.param_quantizers["weight"] = QuantizeDequantize((32, 1), 8, True).to(device)
+    lin.input_quantizers[0] = QuantizeDequantize((), 8, False).to(device)
+    ctx = (lambda: qnn.compute_encodings(lin)) if together else lin.compute_encodings
+    x = torch.randn(8, 64, device=device)
+    wq = lin.param_quantizers["weight"]
+    with ctx():
+        assert lin.param_quantizers["weight"] is wq
+        outs = []
+        for _ in range(2):
+            out = lin(x)
+            out.sum().backward()
+            outs.append(out.detach())
+        assert lin.weight.grad is not None and wq.min.grad is not None
+    assert wq.is_initialized() and lin.input_quantizers[0].is_initialized()
+    with torch.no_grad(), ctx():
+        assert lin.param_quantizers["weight"] is None  # formed once for the whole context
+        again = lin(x)
+    assert lin.param_quantizers["weight"] is wq
+    for out in outs:
+        assert torch.equal(_bits(out), _bits(again))
+    # a frozen weight with a frozen quantizer wants no gradient either, whatever the mode
+    lin.requires_grad_(False)
+    with ctx():
+        assert lin.param_quantizers["weight"] is None
+        assert torch.equal(_bits(lin(x)), _bits(again))
+
+
+@pytest.mark.parametrize("together", [True, False], ids=["model_context", "module_context"])
+def test_parameter_quantizer_without_encodings_still_raises_inside_the_context(device, together):
+    """A parameter quantizer that holds no encodings and may not be overwritten cannot be calibrated; the forward pass
+    says so inside the calibration context as it does outside (quantizer.py:760-775)."""
+    lin = qnn.QuantizedLinear(16, 8, bias=False).to(device)
+    lin.param_quantizers["weight"] = QuantizeDequantize((), 8, True).to(device)
+    lin.param_quantizers["weight"].allow_overwrite(False)
+    ctx = (lambda: qnn.compute_encodings(lin)) if together else lin.compute_encodings
+    with torch.no_grad(), ctx():
+        with pytest.raises(RuntimeError, match="not initialized"):
+            lin(torch.randn(2, 16, device=device))
