@@ -235,17 +235,28 @@ __global__ __launch_bounds__(kBlock) void qdq_bwd_kernel(const QdqArgs a) {
 // Adds the per-tile partial sums of every encoding in a fixed order (second launch: a kernel boundary makes the
 // partials visible without any in-kernel fence, which on a multi-die GPU would flush the L2 once per workgroup).
 constexpr int kFinishThreads = 1024;
+constexpr int kFinishLoads = 16;
 __global__ __launch_bounds__(kFinishThreads) void qdq_bwd_finish_kernel(const QdqArgs a) {
     __shared__ double red_smem[2][kFinishThreads / kWave];
     const int64_t per_enc = a.mode == kRows ? a.I * (int64_t)a.tpr : (int64_t)a.nblocks;
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     if (a.mode != kRows) {
-        // single encoding: independent loads per thread, then one tree
+        // single encoding: every thread issues the loads of up to kFinishLoads pairs before it adds the first (the
+        // launch is a chain of memory latencies and little else), front to back, then one tree
         double s = 0.0, o = 0.0;
-#pragma unroll 4
-        for (int64_t q = threadIdx.x; q < per_enc; q += kFinishThreads) {
-            s += a.partials[2 * q];
-            o += a.partials[2 * q + 1];
+        const double2* __restrict__ pairs = reinterpret_cast<const double2*>(a.partials);
+        for (int64_t q0 = threadIdx.x; q0 < per_enc; q0 += (int64_t)kFinishThreads * kFinishLoads) {
+            double2 v[kFinishLoads];
+#pragma unroll
+            for (int u = 0; u < kFinishLoads; ++u) {
+                const int64_t q = q0 + (int64_t)u * kFinishThreads;
+                v[u] = q < per_enc ? pairs[q] : double2{0.0, 0.0};
+            }
+#pragma unroll
+            for (int u = 0; u < kFinishLoads; ++u) {
+                s += v[u].x;
+                o += v[u].y;
+            }
         }
         s = wave_reduce(s, OpAddD());
         o = wave_reduce(o, OpAddD());
@@ -565,6 +576,7 @@ extern "C" int ahq_qdq_backward(const ahq_grid* grid, const ahq_layout* layout, 
     const bool cols = bwd_cols_layout(grid->io_dtype, p, al);
     const size_t ws_need = bwd_scratch_pairs(grid->io_dtype, p, al, want_pg) * 2 * sizeof(double);
     if (ws_need > 0 && (!workspace || workspace_bytes < ws_need)) return set_error("workspace too small"), AHQ_ERR_WORKSPACE;
+    if (ws_need > 0 && !aligned16(workspace)) return set_error("workspace must be 16-byte aligned"), AHQ_ERR_INVALID;
     QdqArgs a{};
     a.x = x;
     a.g = g;

@@ -316,7 +316,7 @@ def _probe_parameters_together(candidates):
 def _calibrate_parameters_together(work):
     """Calibration and first quantize-dequantize of many parameters with one library call
     (ahq_minmax_calibrate_qdq_many).  ``work``: (module, name, quantizer, parameter) of parameters that are not on a
-    grid already.  Returns {(id(module), name): quantize-dequantized parameter} for those the call covered; the
+    grid already.  Returns {id(module): {name: quantize-dequantized parameter}} for those the call covered; the
     others are left to QuantizedLinear._compute_param_encodings()."""
     from aimet_amd import _lib
     from aimet_amd.quantization._utils import _get_minimum_scale
@@ -370,7 +370,7 @@ def _calibrate_parameters_together(work):
             _lib.check(_lib.load().ahq_minmax_calibrate_qdq_many(items, n, flags.data_ptr(), _lib.current_stream(device)),
                        "ahq_minmax_calibrate_qdq_many")
         for (module, name, qtzr, _), (y, scale, offset) in zip(entries, outputs):
-            done[(id(module), name)] = qtzr._calibrate_qdq_adopt(y, scale, offset)  # pylint: disable=protected-access
+            done.setdefault(id(module), {})[name] = qtzr._calibrate_qdq_adopt(y, scale, offset)  # pylint: disable=protected-access
             qtzr.encoding_analyzer.reset_stats()  # nn/base.py:385-386
         if own_flags:
             _report_range_flags(flags)
@@ -451,7 +451,7 @@ def compute_encodings(model: nn.Module):
         plain = [w for w in todo if not verdicts[id(w[0])].get(w[1], False) and isinstance(w[2], AffineQuantizerBase)]
         quantized = _calibrate_parameters_together(plain)
         for m in modules:
-            mine = {name: t for (mid, name), t in quantized.items() if mid == id(m)}
+            mine = quantized.get(id(m), {})
             m._compute_param_encodings(overwrite=True, verdicts=verdicts[id(m)], quantized=mine)  # pylint: disable=protected-access
             once = m._params_quantized_once()  # pylint: disable=protected-access
             if once:

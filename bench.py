@@ -45,18 +45,19 @@ MIN_TIMED_SECONDS = 0.010
 # the counter summary is profiles/hbm_traffic_pmc__qdq_c1_c2_c4__hist_c3__dlq.txt.  None where no counter run has been
 # made.
 MEASURED_TRAFFIC_BYTES = {
-    ("c1", "qdq_bwd_kernel"): int((200859.8 + 100603.6) * 1024),
-    ("c1", "qdq_fwd_kernel"): int((100492.8 + 100756.7) * 1024),
-    ("c2", "qdq_bwd_kernel"): int((131497.3 + 65843.5) * 1024),
-    ("c2", "qdq_fwd_kernel"): int((65968.2 + 65954.8) * 1024),
-    ("c4", "qdq_bwd_kernel"): int((236827.4 + 121867.3) * 1024),
-    ("c4", "qdq_fwd_kernel"): int((122024.0 + 114935.4) * 1024),
-    ("c4", "qdq_fwd_lpbq_kernel"): int((122050.8 + 118776.6) * 1024),
+    ("c1", "qdq_bwd_kernel"): int((200862.2 + 100749.3) * 1024),
+    ("c1", "qdq_fwd_kernel"): int((100494.1 + 100398.9) * 1024),
+    ("c2", "qdq_bwd_kernel"): int((131570.4 + 65794.4) * 1024),
+    ("c2", "qdq_fwd_kernel"): int((65956.2 + 65591.0) * 1024),
+    ("c4", "qdq_bwd_kernel"): int((236756.8 + 121856.5) * 1024),
+    ("c4", "qdq_fwd_kernel"): int((122033.5 + 114695.3) * 1024),
+    ("c4", "qdq_fwd_lpbq_kernel"): int((122082.5 + 118720.7) * 1024),
     # the timed update (a batch inside the running range): speculative binning pass (read + write) + the launch that
     # folds its extrema and partial histograms into the running state; a batch that moves the range is read a second
     # time (about a quarter of the batches of the c3 stream)
-    ("c3", "hist_update"): int((262285.2 + 3216.0 + 3370.9 + 3.5) * 1024),
-    ("dlq", "pdf_update"): int((262674.4 + 3072.0 + 3127.6 + 12.0) * 1024),
+    ("c3", "hist_update"): int((262267.2 + 3216.0 + 3370.9 + 3.5) * 1024),
+    ("c3", "hist_update_bf16"): int((131158.4 + 536.0 + 680.9 + 2.0) * 1024),
+    ("dlq", "pdf_update"): int((262284.3 + 3072.0 + 3127.6 + 12.0) * 1024),
 }
 DTYPE_NAME = {torch.float32: "f32", torch.bfloat16: "bf16", torch.float16: "f16"}
 
@@ -824,6 +825,7 @@ def run_hist_workload(steps, warmup, dev, with_cpu_baseline=True, batches=16, sh
                    "frac_of_hbm_peak": round(2 * n_b / t_upd16 / 1e9 / HBM_PEAK_GBS, 4),
                    "elements_per_s": round(n_b / t_upd16, 1), "kernel": "hist_bin16_kernel<SPEC>",
                    "sample": "the first 4 batches rounded to bf16, in turn",
+                   "algorithmic_bytes": 2 * n_b, "traffic": MEASURED_TRAFFIC_BYTES.get(("c3", "hist_update_bf16")),
                    "bound": "LDS instruction issue: a table read and an increment per element; bare LDS increments "
                             "alone take 28 us for 67 M elements on this device (16 cycles per wave instruction)"}
 

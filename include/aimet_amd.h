@@ -112,6 +112,7 @@ int ahq_dlq_qdq_per_tensor(int32_t dtype, const void* x, void* y, uint64_t count
 /* Backward of the above with the straight-through estimator (torch_builtins.py:637-655, 691-701, 779-831).  The mask
  * is recomputed from x.  gx may be NULL; gscale/goffset may be NULL (both or neither); when given they receive the
  * gradient already reduced to one fp32 value per encoding (what autograd's sum-to-size produces in the reference).
+ * workspace: ahq_qdq_backward_workspace_bytes() bytes of device memory, 16-byte aligned (NULL if that is 0).
  */
 size_t ahq_qdq_backward_workspace_bytes(const ahq_grid* grid, const ahq_layout* layout, int want_param_grads);
 int    ahq_qdq_backward(const ahq_grid* grid, const ahq_layout* layout, const void* g, const void* x, void* gx,
