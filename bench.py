@@ -40,6 +40,7 @@ COPY_REF_ELEMS = 1 << 26
 ROTATION_BYTES = 1 << 31    # tensors a timed loop goes through before it comes back to the first
 MIN_REPEATS = 7
 MIN_TIMED_SECONDS = 0.010
+DEVICE_WARM_SECONDS = 0.100  # untimed steps before the timed loops of a workload, beyond the --warmup steps
 # HBM bytes per launch of each workload's dominant kernel(s): rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE averages per
 # dispatch, scaled by what the same counters read for _copy_reference() (x2.000 for FETCH_SIZE, x1.000 for WRITE_SIZE);
 # the counter summary is profiles/hbm_traffic_pmc__qdq_c1_c2_c4__hist_c3__dlq.txt.  None where no counter run has been
@@ -82,7 +83,15 @@ def timed_steps(step, steps, warmup, min_repeats=MIN_REPEATS, min_total=MIN_TIME
     Returns (seconds per loop, repeats)."""
     for _ in range(warmup):
         step()
+    # ... and, still untimed, more of the same steps until the device has been busy for DEVICE_WARM_SECONDS: after the
+    # idle stretch of a workload's set-up the first tens of milliseconds of launches run below the steady rate (five
+    # steps of 0.1 ms are over long before that), and a loop of 20 such steps would be timed inside that ramp
     _sync()
+    t_warm = time.perf_counter()
+    while time.perf_counter() - t_warm < DEVICE_WARM_SECONDS:
+        for _ in range(max(1, warmup)):
+            step()
+        _sync()
     loops = []
     total = 0.0
     while len(loops) < min_repeats or (total < min_total and len(loops) < max_repeats):
@@ -233,7 +242,9 @@ def _base_record(value_gbs, steps, warmup, sec_per_step, dtype, config, repeats)
         "data": "synthetic",
         "config": config,
         "repeats": repeats,
-        "timing": f"median of {repeats} loops of {steps} steps, each loop bracketed by device synchronisation",
+        "timing": f"median of {repeats} loops of {steps} steps, each loop bracketed by device synchronisation; before "
+                  f"them the {warmup} warm-up steps and further untimed steps until the device has been busy for "
+                  f"{int(DEVICE_WARM_SECONDS * 1e3)} ms",
         "pct_of_hbm_peak": round(100.0 * value_gbs / HBM_PEAK_GBS, 2),
     }
 

@@ -299,3 +299,45 @@ def test_a_quantizer_whose_observer_holds_call_state_can_be_copied_and_pickled()
     # what this guards against
     with pytest.raises(ValueError):
         pickle.dumps(_lib.load().ahq_minmax_copy)
+
+
+def test_ctypes_structures_have_the_layout_the_header_declares(tmp_path):
+    """Every struct of include/aimet_amd.h, compiled by the C compiler, against its ctypes mirror in aimet_amd/_lib.py:
+    same size and the same offset for every field (a field added or reordered on one side only would otherwise hand
+    the library shifted pointers)."""
+    import ctypes
+    import os
+    import re
+    import shutil
+    import subprocess
+
+    from aimet_amd import _lib
+
+    if shutil.which("gcc") is None:
+        pytest.skip("no C compiler")
+    pairs = {"ahq_layout": _lib.Layout, "ahq_grid": _lib.Grid, "ahq_hist_state": _lib.HistState,
+             "ahq_sqnr_params": _lib.SqnrParams, "ahq_dlq_pdf_state": _lib.DlqPdfState,
+             "ahq_grid_probe_item": _lib.GridProbeItem, "ahq_calibrate_qdq_item": _lib.CalibrateQdqItem,
+             "ahq_slots_finalize_item": _lib.SlotsFinalizeItem}
+    header = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "include", "aimet_amd.h")
+    declared = set(re.findall(r"^\} (ahq_\w+);", open(header).read(), flags=re.M)) - {"ahq_status", "ahq_arith", "ahq_op"}
+    assert declared == set(pairs), "a struct of the header has no ctypes mirror in this test (or the other way round)"
+    lines = ['#include <stdio.h>', '#include <stddef.h>', f'#include "{header}"', "int main(void) {"]
+    for cname, cls in pairs.items():
+        lines.append(f'  printf("{cname} size %zu\\n", sizeof({cname}));')
+        for field, _ in cls._fields_:
+            lines.append(f'  printf("{cname} {field} %zu\\n", offsetof({cname}, {field}));')
+    lines += ["  return 0;", "}"]
+    src = tmp_path / "layout.c"
+    src.write_text("\n".join(lines))
+    exe = tmp_path / "layout"
+    subprocess.run(["gcc", "-std=c11", "-o", str(exe), str(src)], check=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout
+    seen = {}
+    for line in out.splitlines():
+        cname, what, value = line.split()
+        seen[(cname, what)] = int(value)
+    for cname, cls in pairs.items():
+        assert seen[(cname, "size")] == ctypes.sizeof(cls), cname
+        for field, _ in cls._fields_:
+            assert seen[(cname, field)] == getattr(cls, field).offset, f"{cname}.{field}"
