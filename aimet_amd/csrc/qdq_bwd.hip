@@ -138,7 +138,7 @@ __device__ __forceinline__ void bwd_tile(const QdqArgs& a, const Tile& t, float 
 template <typename IO, int VEC, typename M, int RED, int ROUNDS>
 __global__ __launch_bounds__(kBlock) void qdq_bwd_kernel(const QdqArgs a) {
     __shared__ float sp[M::kNP + (M::kDiv ? 1 : 0)][kStage];
-    __shared__ double red_smem[kBlock / kWave];
+    __shared__ double red_smem[2][kBlock / kWave];
     __shared__ double stage_sums[RED == kRedAtomic ? 2 * kStage : 1];  // kRedAtomic: (scale, offset) sums per run
     __shared__ float vec_sums[RED == kRedRuns ? 2 * kBwdTileVec : 1];     // kRedRuns: (scale, offset) terms per vector
     const Tile t = make_tile(a, blockIdx.x);
@@ -214,8 +214,25 @@ __global__ __launch_bounds__(kBlock) void qdq_bwd_kernel(const QdqArgs a) {
         }
     }
     if (RED == kRedTile) {
-        const double bs = block_reduce(acc_s, OpAddD(), red_smem);
-        const double bo = block_reduce(acc_o, OpAddD(), red_smem);
+        // both sums through one barrier (the waves' results are added in wave order by thread 0, which alone needs
+        // them; red_smem is not used before this point)
+        const double ws = wave_reduce(acc_s, OpAddD());
+        const double wo = wave_reduce(acc_o, OpAddD());
+        if ((threadIdx.x & (kWave - 1)) == 0) {
+            red_smem[0][threadIdx.x / kWave] = ws;
+            red_smem[1][threadIdx.x / kWave] = wo;
+        }
+        __syncthreads();
+        double bs = 0.0, bo = 0.0;
+        if (threadIdx.x == 0) {
+            bs = red_smem[0][0];
+            bo = red_smem[1][0];
+#pragma unroll
+            for (int w = 1; w < kBlock / kWave; ++w) {
+                bs += red_smem[0][w];
+                bo += red_smem[1][w];
+            }
+        }
         // number of tiles that feed one encoding
         const int64_t per_enc = a.mode == kRows ? a.I * (int64_t)a.tpr : (int64_t)a.nblocks;
         if (per_enc == 1) {
