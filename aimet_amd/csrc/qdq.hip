@@ -29,8 +29,8 @@ __device__ __forceinline__ void fwd_math(const QdqArgs& a, const Tile& t, float 
 }
 
 // FULL: every lane of the tile has work, so loads and stores carry no per-lane bounds checks (all tiles but the last).
-// The tile's elements are requested first; the encodings are fetched, prepared and staged while those loads are in
-// flight, and the workgroup meets at the barrier once before the arithmetic.
+// The encodings a thread stages are requested first, then the tile's elements; the encodings are prepared and staged
+// while the elements are in flight, and the workgroup meets at the barrier once before the arithmetic.
 template <typename IO, int VEC, typename M, bool FULL, int U, bool LPBQ = false>
 __device__ __forceinline__ void fwd_tile(const QdqArgs& a, const Tile& t, float (*sp)[kStage],
                                          const LpbqFuse* lpbq = nullptr) {
@@ -39,14 +39,16 @@ __device__ __forceinline__ void fwd_tile(const QdqArgs& a, const Tile& t, float 
     uint8_t* __restrict__ mask = a.mask ? a.mask + t.v0 * VEC : nullptr;
     Pack<IO, VEC> in[U];
     float pre_mn = 0.f, pre_mx = 0.f;
+    EncRaw pre{};
     if constexpr (LPBQ) lpbq_preload(*lpbq, t, pre_mn, pre_mx);
+    else pre = preload_encoding(a, t);
 #pragma unroll
     for (int u = 0; u < U; ++u) {
         const int lv = u * kBlock + threadIdx.x;
         if (FULL || lv < t.nv) in[u] = load_pack_hinted<IO, VEC>(x + (int64_t)lv * VEC, a.stream_loads != 0);
     }
     if constexpr (LPBQ) stage_lpbq<M>(a, *lpbq, t, sp, pre_mn, pre_mx);
-    else stage_encodings<M>(a, t, sp);
+    else stage_encodings<M>(a, t, sp, pre);
     __syncthreads();
     // one wave-uniform choice per tile: huge or infinite inputs and out-of-range scales take the general division
     if (!M::kDiv || __builtin_amdgcn_ballot_w64(!lane_can_divide_fast<IO, VEC, M, FULL, U>(a, t, sp, in)) == 0)

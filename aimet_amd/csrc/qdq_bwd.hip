@@ -109,6 +109,7 @@ __device__ __forceinline__ void bwd_tile(const QdqArgs& a, const Tile& t, float 
     const IO* __restrict__ g = static_cast<const IO*>(a.g) + t.v0 * VEC;
     IO* __restrict__ gxp = a.gx ? static_cast<IO*>(a.gx) + t.v0 * VEC : nullptr;
     Pack<IO, VEC> xin[kBwdUnroll], gin[kBwdUnroll];
+    const EncRaw pre = preload_encoding(a, t);  // ahead of the elements: see preload_encoding
 #pragma unroll
     for (int r = 0; r < ROUNDS; ++r) {
         const int base = r * kBlock * kBwdUnroll;
@@ -123,7 +124,7 @@ __device__ __forceinline__ void bwd_tile(const QdqArgs& a, const Tile& t, float 
         }
         if (r == 0) {
             // the encodings are staged while the first loads are in flight
-            stage_encodings<M>(a, t, sp);
+            stage_encodings<M>(a, t, sp, pre);
             if (RED == kRedAtomic)
                 for (int i = threadIdx.x; i < 2 * t.nstage; i += kBlock) stage_sums[i] = 0.0;
             __syncthreads();

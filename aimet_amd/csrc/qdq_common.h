@@ -407,16 +407,36 @@ __device__ __forceinline__ Pack<IO, VEC> load_pack_hinted(const IO* p, bool stre
     return stream ? load_pack_stream<IO, VEC>(p) : load_pack<IO, VEC>(p);
 }
 
+// The values of one encoding as the caller passed them.
+struct EncRaw {
+    float s, off, mn, mx;
+};
+
+__device__ __forceinline__ EncRaw load_raw_encoding(const QdqArgs& a, const Tile& t, int i) {
+    int64_t e = t.e0 + i;
+    if (e >= a.J) e %= a.J;
+    EncRaw r;
+    r.s = a.by_value ? a.value_enc[0] : a.scale[e];
+    r.off = a.by_value ? a.value_enc[1] : (a.offset ? a.offset[e] : 0.f);
+    r.mn = a.by_value ? a.value_enc[2] : (a.emin ? a.emin[e] : 0.f);
+    r.mx = a.by_value ? a.value_enc[3] : (a.emax ? a.emax[e] : 0.f);
+    return r;
+}
+
+// The encoding this thread stages first, requested ahead of the tile's elements: loads return in the order they were
+// issued, so the preparation of the encodings (a division among other things) and the barrier behind it can then
+// run while the elements are still in flight instead of after the last of them has arrived.
+__device__ __forceinline__ EncRaw preload_encoding(const QdqArgs& a, const Tile& t) {
+    EncRaw r{1.f, 0.f, 0.f, 0.f};
+    if ((int)threadIdx.x < t.nstage) r = load_raw_encoding(a, t, threadIdx.x);
+    return r;
+}
+
 template <typename M>
-__device__ __forceinline__ void stage_encodings(const QdqArgs& a, const Tile& t, float (*sp)[kStage]) {
+__device__ __forceinline__ void stage_encodings(const QdqArgs& a, const Tile& t, float (*sp)[kStage], const EncRaw& pre) {
     for (int i = threadIdx.x; i < t.nstage; i += kBlock) {
-        int64_t e = t.e0 + i;
-        if (e >= a.J) e %= a.J;
-        const float s = a.by_value ? a.value_enc[0] : a.scale[e];
-        const float off = a.by_value ? a.value_enc[1] : (a.offset ? a.offset[e] : 0.f);
-        const float mn = a.by_value ? a.value_enc[2] : (a.emin ? a.emin[e] : 0.f);
-        const float mx = a.by_value ? a.value_enc[3] : (a.emax ? a.emax[e] : 0.f);
-        const EncP p = M::prep(s, off, mn, mx, a.gc);
+        const EncRaw r = i == (int)threadIdx.x ? pre : load_raw_encoding(a, t, i);
+        const EncP p = M::prep(r.s, r.off, r.mn, r.mx, a.gc);
         sp[0][i] = p.p0;
         sp[1][i] = p.p1;
         if (M::kNP > 2) sp[2][i] = p.p2;
