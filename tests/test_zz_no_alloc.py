@@ -133,3 +133,66 @@ def test_static_scratch_allocates_no_device_memory(device, case):
     torch.cuda.synchronize()
     assert torch.cuda.mem_get_info()[0] == free0
     assert torch.cuda.memory_allocated() == allocated0 and torch.cuda.memory_reserved() == reserved0
+
+
+@pytest.mark.gpu
+def test_calibrate_forward_backward_replayed_from_a_captured_graph(device):
+    """What the static entry point is for: ahq_minmax_static, ahq_range_to_scale_offset, ahq_qdq_forward and
+    ahq_qdq_backward (preallocated outputs and workspace) recorded once into a HIP graph and replayed on new contents
+    of the same buffers.  Every replay is compared with the eager calls on the same data, with eager work and
+    synchronisations of the process between the replays; the first call of the static entry point happens outside
+    the capture (it looks its scratch array up)."""
+    from aimet_amd.quantization.affine.backends import hip
+
+    lib = _lib.load()
+    g0 = torch.Generator().manual_seed(21)
+    shape, enc = (256, 4096), (256, 1)
+    x = torch.randn(shape, generator=g0).to(device)
+    g = torch.randn(shape, generator=g0).to(device)
+    y, gx = torch.empty_like(x), torch.empty_like(x)
+    mn, mx, scale, gs, go = (torch.empty(enc, device=device) for _ in range(5))
+    offset = torch.zeros(enc, device=device)
+    xd, layout = hip._prepare(x, enc, None)
+    assert xd.data_ptr() == x.data_ptr()
+    grid = hip._grid(_lib.AHQ_ARITH_AUTOGRAD, _lib.AHQ_OP_QDQ, x.dtype, torch.float32, -128, 127, 0.0)
+    nbytes = lib.ahq_qdq_backward_workspace_bytes(grid, layout, 1)
+    ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=device)
+    code = _lib.DTYPE_CODE[x.dtype]
+    outputs = (mn, mx, scale, y, gx, gs, go)
+
+    def work():
+        st = _lib.current_stream(device)
+        _lib.check(lib.ahq_minmax_static(code, layout, x.data_ptr(), mn.data_ptr(), mx.data_ptr(), None, None, 0, st),
+                   "ahq_minmax_static")
+        _lib.check(lib.ahq_range_to_scale_offset(code, mn.data_ptr(), mx.data_ptr(), mn.numel(), -128, 127, 1e-10,
+                                                 scale.data_ptr(), None, st), "ahq_range_to_scale_offset")
+        _lib.check(lib.ahq_qdq_forward(grid, layout, x.data_ptr(), y.data_ptr(), None, scale.data_ptr(),
+                                       offset.data_ptr(), None, None, st), "ahq_qdq_forward")
+        _lib.check(lib.ahq_qdq_backward(grid, layout, g.data_ptr(), x.data_ptr(), gx.data_ptr(), gs.data_ptr(),
+                                        go.data_ptr(), scale.data_ptr(), offset.data_ptr(), ws.data_ptr(), nbytes, st),
+                   "ahq_qdq_backward")
+
+    work()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        work()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        work()
+    for rep in range(3):
+        x.copy_(torch.randn(shape, generator=g0).to(device) * (rep + 1))
+        g.copy_(torch.randn(shape, generator=g0).to(device))
+        work()
+        torch.cuda.synchronize()
+        eager = [t.clone() for t in outputs]
+        for t in outputs:
+            t.fill_(7.0)
+        assert float((x * 2).sum()) == float((x * 2).sum())  # eager work and a synchronisation between the replays
+        graph.replay()
+        torch.cuda.synchronize()
+        for name, want, got in zip(("min", "max", "scale", "y", "gx", "gscale", "goffset"), eager, outputs):
+            assert_same_bits(got, want, f"replay {rep}: {name}")
