@@ -175,7 +175,9 @@ def _like(ref: torch.Tensor, t: torch.Tensor) -> torch.Tensor:
     return out
 
 
+@functools.lru_cache(maxsize=1024)
 def _grid(arith, op, io_dtype, compute_dtype, qmin, qmax, zps) -> _lib.Grid:
+    """The ahq_grid of a call; shared between calls with the same arguments, so nobody writes into it."""
     g = _lib.Grid()
     g.arith = arith
     g.op = op
@@ -187,10 +189,36 @@ def _grid(arith, op, io_dtype, compute_dtype, qmin, qmax, zps) -> _lib.Grid:
     return g
 
 
+_WORKSPACES = {}  # (device, stream, bytes) -> tensor
+_BACKWARD_BYTES = {}  # (id(grid), id(layout), parameter gradients wanted) -> (grid, layout, bytes)
+
+
 def _workspace(nbytes: int, device) -> Optional[torch.Tensor]:
+    """Scratch of ``nbytes`` for a launch on the current stream of ``device``.  The library neither expects anything
+    in a workspace nor leaves anything there for a later call, and launches on one stream run in order, so one buffer
+    per (device, stream, size) serves every call (a step of a training loop asks for the same size again and
+    again); a handful of sizes are kept."""
     if nbytes == 0:
         return None
-    return torch.empty(nbytes, dtype=torch.uint8, device=device)
+    key = (device, _lib.current_stream(device), nbytes)
+    ws = _WORKSPACES.get(key)
+    if ws is None:
+        if len(_WORKSPACES) >= 64:
+            _WORKSPACES.clear()
+        ws = _WORKSPACES[key] = torch.empty(nbytes, dtype=torch.uint8, device=device)
+    return ws
+
+
+def _backward_workspace_bytes(grid, layout, want_pg: bool) -> int:
+    """ahq_qdq_backward_workspace_bytes, asked once per (grid, layout): both objects come out of caches and live on."""
+    key = (id(grid), id(layout), want_pg)
+    held = _BACKWARD_BYTES.get(key)
+    if held is None or held[0] is not grid or held[1] is not layout:
+        if len(_BACKWARD_BYTES) >= 4096:
+            _BACKWARD_BYTES.clear()
+        held = _BACKWARD_BYTES[key] = (grid, layout,
+                                       _lib.load().ahq_qdq_backward_workspace_bytes(grid, layout, 1 if want_pg else 0))
+    return held[2]
 
 
 def _launch_forward(tensor, scale, offset, arith, op, compute_dtype, qmin, qmax, block_size, zps):
@@ -246,14 +274,13 @@ def _launch_backward(grid, layout, x, s, o, grad, need_x: bool, want_pg: bool):
     gx = torch.empty_like(x) if need_x else None
     gs = go = None
     if want_pg:
-        gs = torch.empty(s.shape, dtype=torch.float32, device=x.device)
-        go = torch.empty(s.shape, dtype=torch.float32, device=x.device)
+        gs, go = torch.empty((2,) + tuple(s.shape), dtype=torch.float32, device=x.device).unbind(0)
     if x.numel() == 0:
         if want_pg:
             gs.zero_()
             go.zero_()
     else:
-        nbytes = lib.ahq_qdq_backward_workspace_bytes(grid, layout, 1 if want_pg else 0)
+        nbytes = _backward_workspace_bytes(grid, layout, want_pg)
         ws = _workspace(nbytes, x.device)
         _lib.check(
             lib.ahq_qdq_backward(grid, layout, g.data_ptr(), x.data_ptr(), _lib.ptr(gx), _lib.ptr(gs),
