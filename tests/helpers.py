@@ -63,3 +63,34 @@ def histogram_merge_closed_forms():
     new = [1 + 2, 1, 3, 1]
     straddle = (4, first, second, [o + n for o, n in zip(old, new)], (-0.375, 1.625))
     return {"nested": nested, "straddle": straddle}
+
+
+def nested_range_batches(num_bins: int, seed: int, dtype=None):
+    """Three batches whose ranges are [-a, a], [-2a, 2a], [-8a, 8a] for a power of two a, values on a dyadic grid
+    fine enough that none lies on a bin edge except the range ends: every old bin then lies inside one bin of the
+    next range, no count is ever split, and the merged histogram is -- exactly -- the plain histogram of all the
+    data over the last range (with each earlier batch's maximum counted below the edge it sits on).  Returns (batches, expected counts as float32, (lo, hi))."""
+    import torch
+
+    g = torch.Generator().manual_seed(seed)
+    a = 2.0 ** (seed % 5 - 2)
+    batches = []
+    for k, width in enumerate((1, 2, 8)):
+        n = 3000 + 500 * k
+        half = width * a
+        # odd multiples of half / (4 * num_bins): never on an edge of any of the three bin grids
+        steps = torch.randint(-2 * num_bins, 2 * num_bins, (n,), generator=g) * 2 + 1
+        x = steps.to(torch.float32) * (half / (4 * num_bins))
+        x[0], x[1] = -half, half
+        if dtype is not None:
+            x = x.to(dtype)
+        batches.append(x)
+    lo, hi = -8 * a, 8 * a
+    # a batch's maximum is counted in the last bin of its own range (torch.histc closes the range on the right) and
+    # stays with that bin's counts from then on, although the value is the left edge of the next bin of a wider grid:
+    # for the plain histogram it is therefore taken just below
+    inside = [b.to(torch.float32).clone() for b in batches]
+    for k, width in enumerate((1, 2)):
+        inside[k][1] = width * a * (1 - 1 / (8 * num_bins))
+    expected = torch.histc(torch.cat(inside), bins=num_bins, min=lo, max=hi)
+    return batches, expected, (lo, hi)

@@ -246,6 +246,27 @@ def test_histogram_merge_closed_forms(device, case):
     assert st.min.item() == lo and st.max.item() == hi
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["float32", "bfloat16"])
+@pytest.mark.parametrize("num_bins", [8, 64, 512])
+@pytest.mark.parametrize("seed", range(3))
+def test_histogram_merge_of_nested_ranges_is_the_histogram_of_all_the_data(device, num_bins, seed, dtype):
+    """The randomized closed form of tests/test_oracle_golden.py on the HIP path (every value of the dyadic grid is
+    a bfloat16 value too while num_bins <= 64; beyond that the float32 case alone applies)."""
+    from aimet_amd.quantization.encoding_analyzer import _HistogramObserver
+    from tests.helpers import nested_range_batches
+
+    if dtype == torch.bfloat16 and num_bins > 64:
+        pytest.skip("the grid needs more mantissa bits than bfloat16 has")
+    batches, expected, (lo, hi) = nested_range_batches(num_bins, seed, dtype)
+    obs = _HistogramObserver((1,), num_bins=num_bins)
+    for b in batches:
+        obs.update(b.to(device))
+    st = obs.get_stats()[0]
+    assert torch.equal(st.histogram.cpu().float(), expected)
+    assert st.min.item() == lo and st.max.item() == hi
+    assert st.bin_edges[0].item() == lo and st.bin_edges[-1].item() == hi
+
+
 def test_batch_histogram_is_formed_on_first_read(device):
     from aimet_amd.quantization.encoding_analyzer import _HistogramObserver
 

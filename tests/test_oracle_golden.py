@@ -242,6 +242,25 @@ def test_histogram_merge_closed_forms(case):
     assert st.min.item() == lo and st.max.item() == hi
 
 
+@pytest.mark.parametrize("num_bins", [8, 64, 512])
+@pytest.mark.parametrize("seed", range(6))
+def test_histogram_merge_of_nested_ranges_is_the_histogram_of_all_the_data(num_bins, seed):
+    """Re-binning on data nobody chose by hand: ranges that double and then quadruple keep every old bin inside one
+    new bin, so whatever the merge does must add up to torch.histc of all the data over the final range (a wrong
+    destination index, a dropped or doubled source bin, or a split where none belongs all break the equality)."""
+    from tests.helpers import nested_range_batches
+
+    batches, expected, (lo, hi) = nested_range_batches(num_bins, seed)
+    obs = O.HistObserver((1,), num_bins)
+    for b in batches:
+        obs.update(b)
+    st = obs.stats[0]
+    assert torch.equal(st.histogram, expected)
+    assert st.min.item() == lo and st.max.item() == hi
+    assert st.bin_edges[0].item() == lo and st.bin_edges[-1].item() == hi
+    assert int(st.histogram.sum()) == sum(b.numel() for b in batches)
+
+
 def test_lpbq_closed_form():
     """Reference: test_affine_quantizer.py:1426-1474."""
     g = torch.Generator().manual_seed(6)
