@@ -242,6 +242,22 @@ def test_histogram_merge_closed_forms(case):
     assert st.min.item() == lo and st.max.item() == hi
 
 
+@pytest.mark.parametrize("seed", range(12))
+def test_histogram_merges_conserve_every_count(seed):
+    """On arbitrary data the ranges grow by arbitrary factors and most old bins are split between two new ones.  A
+    split hands round(share * count) to one bin and the REST to the other, so no merge may gain or lose a single
+    count: after every batch the histogram sums to the number of values seen, exactly."""
+    g = torch.Generator().manual_seed(100 + seed)
+    obs = O.HistObserver((1,), [7, 64, 512][seed % 3])
+    total = 0
+    for _ in range(5):
+        spread = 1 + 3 * torch.rand((), generator=g).item()
+        x = torch.randn(10000, generator=g) * spread + torch.rand((), generator=g).item()
+        obs.update(x)
+        total += x.numel()
+        assert obs.stats[0].histogram.double().sum().item() == total
+
+
 @pytest.mark.parametrize("num_bins", [8, 64, 512])
 @pytest.mark.parametrize("seed", range(6))
 def test_histogram_merge_of_nested_ranges_is_the_histogram_of_all_the_data(num_bins, seed):
