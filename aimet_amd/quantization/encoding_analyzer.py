@@ -265,6 +265,7 @@ class _MinMaxObserver(_Observer[_MinMaxRange]):
     @torch.no_grad()
     def merge_stats(self, stats: _MinMaxRange):
         self._leave_slots()
+        self.__dict__["_stats_shared"] = False  # new tensors below
         new_min, new_max = self.stats.min, self.stats.max
         if stats.min is not None:
             new_min = stats.min.clone() if new_min is None else torch.minimum(new_min, stats.min)
@@ -284,12 +285,21 @@ class _MinMaxObserver(_Observer[_MinMaxRange]):
                 return batch
         self._leave_slots()
         cur = self.stats
+        if cur.min is None and cur.max is None:
+            # the first batch: its extrema ARE the running statistics.  The two objects share their tensors until
+            # somebody is about to write into the running ones (_own_stats), so a calibration on one batch -- every
+            # weight -- makes no copies
+            mn, mx = reduce_min_max(input_tensor, self.shape, self.block_size, copy_to=copy_to)
+            self.stats = _MinMaxRange(mn, mx)
+            self.__dict__["_stats_shared"] = True
+            return _MinMaxRange(mn, mx)
         fused = (
             cur.min is not None and cur.max is not None
             and cur.min.dtype == input_tensor.dtype and cur.min.device == input_tensor.device
             and cur.min.is_contiguous() and cur.max.is_contiguous()
         )
         if fused:
+            cur = self._own_stats()
             mn, mx = reduce_min_max(input_tensor, self.shape, self.block_size, running=(cur.min, cur.max),
                                     copy_to=copy_to)
             return _MinMaxRange(mn, mx)
@@ -297,6 +307,15 @@ class _MinMaxObserver(_Observer[_MinMaxRange]):
         new = _MinMaxRange(mn, mx)
         self.merge_stats(new)
         return new
+
+    def _own_stats(self) -> _MinMaxRange:
+        """The running statistics as tensors nobody else holds: whoever writes into them in place asks here first."""
+        if self.__dict__.get("_stats_shared"):
+            cur = self.stats
+            self.stats = _MinMaxRange(None if cur.min is None else cur.min.clone(),
+                                      None if cur.max is None else cur.max.clone())
+            self.__dict__["_stats_shared"] = False
+        return self.stats
 
     @torch.no_grad()
     def observe_and_clone(self, input_tensor: torch.Tensor) -> torch.Tensor:
@@ -316,7 +335,8 @@ class _MinMaxObserver(_Observer[_MinMaxRange]):
         if (fast is None or fast[0] != key or fast[1] is not cur.min or fast[2] is not cur.max or not x.is_contiguous()
                 or x.requires_grad):
             out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
-            self.update(x, copy_to=out)
+            self.update(x, copy_to=out)  # (the batch's own extrema are dropped here, so nobody shares the tensors)
+            self.__dict__["_stats_shared"] = False
             cur = self.stats
             self.__dict__["_fast"] = None
             if (x.is_contiguous() and x.is_cuda and cur.min is not None and cur.min.dtype == x.dtype

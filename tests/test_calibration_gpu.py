@@ -648,3 +648,27 @@ def test_slot_statistics_through_a_quantizer(device):
     with torch.no_grad(), fresh._compute_encodings(passthrough=True):
         pass
     assert not fresh.is_initialized()
+
+
+@pytest.mark.parametrize("shape,block", [((6, 1), None), ((6, 4), (1, 8))], ids=["per_channel", "blockwise"])
+def test_first_batch_statistics_are_not_changed_by_later_batches(device, shape, block):
+    """The first batch's extrema are the running statistics, and the two share their tensors until the running ones
+    are written to: what update() returned for the first batch must still be that batch's extrema after the second,
+    and the running statistics the fold of both."""
+    from aimet_amd.quantization.encoding_analyzer import _MinMaxObserver
+
+    g = torch.Generator().manual_seed(17)
+    a = torch.randn(6, 32, generator=g)
+    b = torch.randn(6, 32, generator=g) * 3
+    obs = _MinMaxObserver(shape, block) if block else _MinMaxObserver(shape)
+    first = obs.update(a.to(device))
+    want = O.reduce_minmax(a, shape, block)
+    assert_same_bits(first.min, want[0].view(shape), "first batch minimum")
+    assert_same_bits(obs.get_stats().min, want[0].view(shape), "running minimum after one batch")
+    second = obs.update(b.to(device))
+    assert_same_bits(first.min, want[0].view(shape), "first batch minimum after the second batch")
+    assert_same_bits(first.max, want[1].view(shape), "first batch maximum after the second batch")
+    wb = O.reduce_minmax(b, shape, block)
+    assert_same_bits(second.min, wb[0].view(shape), "second batch minimum")
+    assert_same_bits(obs.get_stats().min, torch.minimum(want[0], wb[0]).view(shape), "running minimum")
+    assert_same_bits(obs.get_stats().max, torch.maximum(want[1], wb[1]).view(shape), "running maximum")
