@@ -672,7 +672,7 @@ def _range_flags_buffer(device):
 
 
 def _report_range_flags(flags: torch.Tensor):
-    _warn_range_flags(*(flags != 0).tolist())
+    _warn_range_flags(*(v != 0 for v in flags.tolist()))  # one device-to-host read, no launch
 
 
 def _warn_range_flags(nonfinite: bool, extreme: bool):
@@ -686,11 +686,11 @@ def _flag_extreme_min_max(curr_min, curr_max):
     """Warn about non-finite or near-overflow encodings (reference: encoding_analyzer.py:484-498)."""
     flags = getattr(curr_min, "_ahq_range_flags", None)
     if flags is not None and getattr(curr_max, "_ahq_range_flags", None) is flags:
-        flags = flags != 0  # already evaluated by the kernel that produced this pair
+        # already evaluated by the kernel that produced this pair
         if _deferred_range_flags is not None:
-            _deferred_range_flags.append(flags)
+            _deferred_range_flags.append(flags != 0)
             return
-        _warn_range_flags(*flags.tolist())
+        _report_range_flags(flags)
         return
     big = torch.finfo(curr_min.dtype).max
     both = torch.stack([curr_min.reshape(-1), curr_max.reshape(-1)]).abs()
