@@ -1264,3 +1264,40 @@ def test_model_calibration_with_a_scale_offset_parameter_quantizer(device):
     assert b.param_quantizers["weight"]._is_scale_offset_quantizer()
     with torch.no_grad():
         assert_same_bits(b(x), a(x), "layer output")
+
+
+@pytest.mark.parametrize("symmetric", [True, False])
+def test_quantize_held_as_scale_offset(device, symmetric):
+    """Quantize (integer codes out) with its encoding held as scale / offset: the codes, the dequantized values and
+    the gradients of scale and offset are those of the oracle at the same scale and offset."""
+    from aimet_amd.quantization.affine import Quantize
+
+    g = torch.Generator().manual_seed(8)
+    x = torch.randn(12, 40, generator=g)
+    if not symmetric:
+        x = torch.relu(x)
+    grad = torch.randn(12, 40, generator=g)
+    q = Quantize((12, 1), 8, symmetric).to(device)
+    with q.compute_encodings():
+        q(x.to(device))
+    scale, offset = q.get_scale().detach().cpu(), q.get_offset().detach().cpu()
+    q._reparametrize_to_scale_offset()
+    xd = x.to(device).requires_grad_(True)
+    out = q(xd)
+    assert type(out).__name__ == "QuantizedTensor"
+    qmin, qmax = (-128, 127) if symmetric else (0, 255)
+    codes = torch.clamp(torch.round(x / scale) - offset, qmin, qmax)  # torch_builtins.py:588-632 on the CPU
+    assert_same_bits(out, codes, "codes")
+    assert_same_bits(out.dequantize(), (codes + offset) * scale, "dequantized codes")
+    out.backward(grad.to(device))
+    # plain autograd of clamp(round_ste(x / s) - o, qmin, qmax)
+    s = scale.clone().requires_grad_(True)
+    o = offset.clone().requires_grad_(True)
+    xr = x.clone().requires_grad_(True)
+    t = xr / s
+    ref = torch.clamp(t + (torch.round(t) - t).detach() - o, qmin, qmax)
+    ref.backward(grad)
+    assert_same_bits(xd.grad, xr.grad, "input gradient")
+    assert_close_rel(q.scale.grad, s.grad, 1e-5, "scale gradient", abs_floor=1e-30)
+    if not symmetric:
+        assert_close_rel(q.offset.grad, o.grad, 1e-5, "offset gradient", abs_floor=1e-30)
