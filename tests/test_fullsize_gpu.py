@@ -288,3 +288,76 @@ def test_tf_enhanced_pdf_at_the_benchmark_shape(device):
     y = q.quantizeDequantize(x)
     assert float(y.amin()) >= e_min - 1e-3 and float(y.amax()) <= e_max + 1e-3
     assert float((y - x).abs()[(x > e_min) & (x < e_max)].max()) <= (e_max - e_min) / 255 * 0.5001
+
+
+def test_tensors_of_more_than_two_to_the_31_elements(device):
+    """A 288 GB device holds tensors whose element index does not fit 32 bits.  One bfloat16 tensor of 2^31 + 98760
+    elements (4.3 GB): min/max finds values planted past the 2^31st element and in the last one; the forward and the
+    input gradient of chunks at the start, across the 2^31 boundary and at the end equal those chunks computed alone;
+    the offset gradient counts the clipped elements; per-row statistics and encodings on a [65537, 32768] view of the
+    same memory; the histogram counts every element."""
+    from aimet_amd.quantization import affine
+    from aimet_amd.quantization._stats import reduce_min_max
+    from aimet_amd.quantization.encoding_analyzer import _HistogramObserver
+
+    free, _ = torch.cuda.mem_get_info()
+    if free < 40 << 30:
+        pytest.skip("needs 40 GB of free device memory")
+    n = (1 << 31) + 8 * 12345
+    g = torch.Generator(device=device).manual_seed(0)
+    x = torch.empty(n, dtype=torch.bfloat16, device=device)
+    step = 1 << 28
+    for i in range(0, n, step):
+        x[i:i + step] = torch.randn(min(step, n - i), generator=g, device=device).to(torch.bfloat16)
+    x[(1 << 31) + 5] = 300.0
+    x[n - 1] = -400.0
+    mn, mx = reduce_min_max(x, ())
+    assert float(mn) == -400.0 and float(mx) == 300.0
+
+    scale = torch.tensor(0.05, device=device)
+    offset = torch.tensor(-128.0, device=device)
+    with torch.no_grad():
+        y = affine.quantize_dequantize(x, scale, offset, 0, 255)
+    m = 1 << 20
+    starts = (0, (1 << 31) - m // 2, n - m)
+    for lo in starts:
+        with torch.no_grad():
+            part = affine.quantize_dequantize(x[lo:lo + m].clone(), scale, offset, 0, 255)
+        assert torch.equal(part.view(torch.int16), y[lo:lo + m].view(torch.int16)), lo
+    del y
+
+    xg = x.requires_grad_(True)
+    s = scale.clone().requires_grad_(True)
+    o = offset.clone().requires_grad_(True)
+    out = affine.quantize_dequantize(xg, s, o, 0, 255)
+    out.backward(torch.ones(1, dtype=torch.bfloat16, device=device).expand(n))
+    del out
+    x = x.detach()
+    clipped = 0
+    for lo in range(0, n, step):
+        q = (x[lo:lo + step].float() / 0.05).round() + 128
+        clipped += int(((q < 0) | (q > 255)).sum())
+    for lo in starts:
+        q = (x[lo:lo + m].float() / 0.05).round() + 128
+        assert torch.equal(xg.grad[lo:lo + m], ((q >= 0) & (q <= 255)).to(torch.bfloat16)), lo
+    assert clipped >= 2 and abs(float(o.grad) - 0.05 * clipped) <= 1e-3 * 0.05 * clipped  # a clipped element adds scale
+    del xg
+
+    rows, cols = 65537, 32768
+    xr = x[:rows * cols].view(rows, cols)
+    mn, mx = reduce_min_max(xr, (rows, 1))
+    for r in (0, 12345, rows - 1):
+        assert float(mn[r]) == float(xr[r].amin()) and float(mx[r]) == float(xr[r].amax()), r
+    sc = (mx.float() - mn.float()).clamp_min(1e-3) / 255
+    of = torch.round(mn.float() / sc)
+    with torch.no_grad():
+        yr = affine.quantize_dequantize(xr, sc, of, 0, 255)
+        for r in (0, 40000, rows - 1):
+            part = affine.quantize_dequantize(xr[r:r + 1].clone(), sc[r:r + 1], of[r:r + 1], 0, 255)
+            assert torch.equal(part.view(torch.int16), yr[r:r + 1].view(torch.int16)), r
+    del yr
+
+    obs = _HistogramObserver((1,), num_bins=512)
+    first = obs.update(x)[0]
+    assert float(first.min) == -400.0 and float(first.max) == 300.0
+    assert abs(float(first.histogram.double().sum()) - n) <= n * 1e-6  # float32 counts: every bin rounds once
