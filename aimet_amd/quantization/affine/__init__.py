@@ -11,6 +11,8 @@ from aimet_amd.quantization.affine.backends import (  # noqa: F401
 from aimet_amd.quantization.affine.encoding import AffineEncoding, GroupedBlockEncoding  # noqa: F401,E402
 from aimet_amd.quantization.affine.quantizer import (  # noqa: F401,E402
     AffineQuantizerBase,
+    MinMaxQuantizer,
+    ScaleOffsetQuantizer,
     Quantize,
     QuantizeDequantize,
     Dequantize,

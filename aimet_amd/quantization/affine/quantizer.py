@@ -14,7 +14,7 @@ from __future__ import annotations
 import functools
 import math
 from contextlib import contextmanager, nullcontext
-from typing import NamedTuple, Optional, Tuple
+from typing import Any, NamedTuple, Optional, Protocol, Tuple, runtime_checkable
 
 import torch
 from torch import nn
@@ -39,7 +39,8 @@ from aimet_amd.quantization.base.quantizer import QuantizerBase
 from aimet_amd.quantization.encoding_analyzer import EncodingAnalyzer, MinMaxEncodingAnalyzer, _flag_extreme_min_max
 from aimet_amd.quantization.tensor import QuantizedTensor, DequantizedTensor
 
-__all__ = ["AffineQuantizerBase", "Quantize", "QuantizeDequantize", "Dequantize", "GroupedBlockQuantizeDequantize"]
+__all__ = ["AffineQuantizerBase", "MinMaxQuantizer", "ScaleOffsetQuantizer", "Quantize", "QuantizeDequantize",
+           "Dequantize", "GroupedBlockQuantizeDequantize"]
 
 
 def _symmetric_offset(qmin: int, qmax: int, shape, dtype, device) -> torch.Tensor:
@@ -411,6 +412,9 @@ class AffineQuantizerBase(QuantizerBase, _GridMixin):
             self.to(device=mn.device, dtype=torch.float32)
             if was_initialized:
                 self.set_range(mn, mx)
+        # the marker the runtime-checkable protocols below look for (quantizer.py:252-254)
+        self.__dict__.pop("_is_min_max", None)
+        self.__dict__["_is_scale_offset"] = True
 
     def _reparametrize_to_min_max(self):
         """The encoding held as (min, max) (quantizer.py:263-285), the form every quantizer starts in."""
@@ -431,6 +435,8 @@ class AffineQuantizerBase(QuantizerBase, _GridMixin):
             if was_initialized:
                 mn, mx = _get_min_max(scale.detach(), None if offset is None else offset.detach(), self.qmin, self.qmax)
                 self.set_range(mn, mx)
+        self.__dict__.pop("_is_scale_offset", None)
+        self.__dict__["_is_min_max"] = True
 
     # ------------------------------------------------------------------------------------- derived quantities --
     def get_scale(self, dtype=None) -> Optional[torch.Tensor]:
@@ -1001,6 +1007,31 @@ class AffineQuantizerBase(QuantizerBase, _GridMixin):
                 elif new.shape != cur.shape:
                     setattr(self, name, nn.Parameter(new.clone().to(device=cur.device, dtype=cur.dtype)))
         return super().load_state_dict(state_dict, strict, **kwargs)
+
+
+@runtime_checkable
+class MinMaxQuantizer(Protocol):
+    """An affine quantizer that holds its encoding as min and max (quantizer.py:903-914): isinstance() looks for the
+    marker the reparametrisation leaves."""
+
+    _is_min_max: Any
+
+    shape: Tuple[int, ...]
+    qmin: int
+    qmax: int
+    symmetric: bool
+
+
+@runtime_checkable
+class ScaleOffsetQuantizer(Protocol):
+    """An affine quantizer that holds its encoding as scale and offset (quantizer.py:917-928)."""
+
+    _is_scale_offset: Any
+
+    shape: Tuple[int, ...]
+    qmin: int
+    qmax: int
+    symmetric: bool
 
 
 class Quantize(AffineQuantizerBase):

@@ -10,6 +10,7 @@ from __future__ import annotations
 import abc
 import contextlib
 import copy
+import warnings
 import weakref
 from collections import OrderedDict
 from typing import Optional
@@ -37,6 +38,28 @@ class QuantizerBase(abc.ABC, torch.nn.Module):
     @abc.abstractmethod
     def get_encodings(self):
         """Return the quantizer's encodings as an encoding object."""
+
+    def get_encoding(self):
+        """Deprecated alias of get_encodings() (base/quantizer.py:81-86)."""
+        warnings.warn("get_encoding is deprecated: use get_encodings instead", DeprecationWarning, stacklevel=2)
+        return self.get_encodings()
+
+    def set_encodings(self, encodings):
+        """Set the quantizer's encodings (base/quantizer.py:88-92: not implemented by the reference either)."""
+        raise NotImplementedError
+
+    @abc.abstractmethod
+    def get_legacy_encodings(self):
+        """The encodings as a list of dictionaries, one per channel; None before initialisation."""
+
+    @abc.abstractmethod
+    def set_legacy_encodings(self, encodings):
+        """Take the encodings from a list in the form get_legacy_encodings() gives."""
+
+    @classmethod
+    @abc.abstractmethod
+    def from_encodings(cls, encodings):
+        """A quantizer that holds the given encoding object's encodings."""
 
     def register_quantization_parameter(self, name: str, param: Optional[nn.Parameter]):
         self.register_parameter(name, param)
@@ -124,6 +147,17 @@ class QuantizerBase(abc.ABC, torch.nn.Module):
         if name is None:
             return any(self._is_overwrite_allowed.values())
         return self._is_overwrite_allowed[name]
+
+    @property
+    def _allow_overwrite(self) -> bool:
+        """Deprecated spelling of is_overwrite_allowed() / allow_overwrite() (base/quantizer.py:293-302)."""
+        warnings.warn("_allow_overwrite is deprecated: use is_overwrite_allowed() instead", DeprecationWarning, stacklevel=2)
+        return self.is_overwrite_allowed()
+
+    @_allow_overwrite.setter
+    def _allow_overwrite(self, mode: bool):
+        warnings.warn("_allow_overwrite is deprecated: use allow_overwrite() instead", DeprecationWarning, stacklevel=2)
+        self.allow_overwrite(mode)
 
     @contextlib.contextmanager
     def _precompute_encodings(self, dtype=None):  # pylint: disable=unused-argument

@@ -219,3 +219,34 @@ def test_legacy_encodings_one_dictionary_per_channel():
     other = QuantizeDequantize((4, 1), 8, symmetric=True)
     other.set_legacy_encodings(legacy)
     assert torch.allclose(other.get_min(), q.get_min(), atol=1e-6) and torch.allclose(other.get_max(), q.get_max(), atol=1e-6)
+
+
+def test_runtime_checkable_protocols_follow_the_parametrisation():
+    """quantizer.py:903-928: isinstance(q, MinMaxQuantizer) / isinstance(q, ScaleOffsetQuantizer) tell which
+    parameters a quantizer holds, also after copies."""
+    from aimet_amd.quantization.affine import MinMaxQuantizer, ScaleOffsetQuantizer
+
+    q = QuantizeDequantize((4, 1), 8, symmetric=False)
+    assert isinstance(q, MinMaxQuantizer) and not isinstance(q, ScaleOffsetQuantizer)
+    q._reparametrize_to_scale_offset()
+    assert isinstance(q, ScaleOffsetQuantizer) and not isinstance(q, MinMaxQuantizer)
+    for clone in (copy.deepcopy(q), pickle.loads(pickle.dumps(q))):
+        assert isinstance(clone, ScaleOffsetQuantizer) and not isinstance(clone, MinMaxQuantizer)
+    q._reparametrize_to_min_max()
+    assert isinstance(q, MinMaxQuantizer) and not isinstance(q, ScaleOffsetQuantizer)
+    assert not isinstance(torch.nn.Linear(2, 2), MinMaxQuantizer)
+
+
+def test_deprecated_spellings_of_the_base_class_still_work():
+    """base/quantizer.py:81-92, 293-302: get_encoding(), the _allow_overwrite property, set_encodings()."""
+    q = _initialized(QuantizeDequantize, True)
+    with pytest.warns(DeprecationWarning):
+        enc = q.get_encoding()
+    assert torch.equal(enc.scale, q.get_encodings().scale)
+    with pytest.warns(DeprecationWarning):
+        assert q._allow_overwrite is True
+    with pytest.warns(DeprecationWarning):
+        q._allow_overwrite = False
+    assert not q.is_overwrite_allowed() and not q.is_overwrite_allowed("min")
+    with pytest.raises(NotImplementedError):
+        q.set_encodings(enc)
