@@ -8,7 +8,7 @@ from aimet_amd.quantization.affine.backends import (  # noqa: F401
     get_backend,
     add_backend,
 )
-from aimet_amd.quantization.affine.encoding import AffineEncoding, GroupedBlockEncoding  # noqa: F401,E402
+from aimet_amd.quantization.affine.encoding import AffineEncoding, GroupedBlockEncoding, VectorEncoding  # noqa: F401,E402
 from aimet_amd.quantization.affine.quantizer import (  # noqa: F401,E402
     AffineQuantizerBase,
     MinMaxQuantizer,

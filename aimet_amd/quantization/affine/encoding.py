@@ -1,13 +1,15 @@
 """Affine encodings: the (scale, offset, grid) description attached to quantizer outputs.
 
-Counterpart of aimet_torch/quantization/affine/encoding.py:33-458 and :579-684, including the export of an encoding to
-the dictionary formats "0.6.1", "1.0.0", "2.0.0" and "2.1.0" (`to_qnn_encoding_dict`).
+Counterpart of aimet_torch/quantization/affine/encoding.py:33-740, including the export of an encoding to the
+dictionary formats "0.6.1", "1.0.0", "2.0.0" and "2.1.0" (`to_qnn_encoding_dict`), the way back from a per-tensor
+2.0.0 / 2.1.0 dictionary, the vector-quantization encoding (a record of its extra fields) and the reading of a
+blockwise encoding as a grouped one.
 """
 
 from __future__ import annotations
 
 import math
-from typing import Dict, List, Optional, Tuple, Union
+from typing import Any, Dict, List, Optional, Tuple, Union
 
 import torch
 
@@ -15,7 +17,7 @@ from aimet_amd.quantization.base.encoding import EncodingBase
 from aimet_amd.quantization.affine._utils import _GridMixin
 from aimet_amd.quantization.affine.backends import quantize, dequantize, quantize_dequantize, _derive_qmin_qmax
 
-__all__ = ["AffineEncoding", "GroupedBlockEncoding"]
+__all__ = ["AffineEncoding", "VectorEncoding", "GroupedBlockEncoding"]
 
 
 class AffineEncoding(EncodingBase, _GridMixin):
@@ -94,6 +96,17 @@ class AffineEncoding(EncodingBase, _GridMixin):
     def signed(self) -> bool:
         return self._get_signed()
 
+    @property
+    def dtype(self) -> torch.dtype:
+        """The narrowest of uint8, int8, int16, int32 that holds the grid (encoding.py:178-192)."""
+        if 0 <= self.qmin < self.qmax < 2 ** 8:
+            return torch.uint8
+        if -(2 ** 7) <= self.qmin < self.qmax < 2 ** 7:
+            return torch.int8
+        if -(2 ** 15) <= self.qmin < self.qmax < 2 ** 15:
+            return torch.int16
+        return torch.int32
+
     def to(self, *args, **kwargs):
         """Same encoding with scale/offset moved to another device and/or floating-point dtype."""
         scale = self.scale.to(*args, **kwargs)
@@ -159,6 +172,30 @@ class AffineEncoding(EncodingBase, _GridMixin):
                 enc["zero_point_shift"] = self.zero_point_shift
             out.append(enc)
         return out
+
+    def _get_additional_properties(self) -> Dict[str, Any]:
+        """Fields a subclass adds to the exported dictionaries (encoding.py:359-360)."""
+        return {}
+
+    @classmethod
+    def _from_qnn_encoding_dict(cls, encoding_dict, version=None) -> "AffineEncoding":
+        """A per-tensor encoding from its 2.0.0 / 2.1.0 dictionary (encoding.py:460-497)."""
+        if version is None:
+            version = "2.0.0" if "y_scale" in encoding_dict or "per_block_int_scale" in encoding_dict else "unknown"
+        if version not in ("2.0.0", "2.1.0"):
+            raise NotImplementedError(f"Only 2.0.0 and 2.1.0 encodings are supported; got {version}")
+        if "per_block_int_scale" in encoding_dict or "axis" in encoding_dict:
+            raise NotImplementedError("Only per-tensor encodings are supported")
+        unsigned, bw = encoding_dict["output_dtype"].split("int")
+        bw = int(bw)
+        if unsigned:
+            qmin, qmax = 0, 2 ** bw - 1
+        else:
+            qmin, qmax = -(2 ** (bw - 1)), 2 ** (bw - 1) - 1
+        offset = -encoding_dict.get("y_zero_point", 0)
+        return AffineEncoding(scale=torch.tensor(encoding_dict["y_scale"], dtype=torch.float32),
+                              offset=torch.tensor(offset, dtype=torch.float32), qmin=qmin, qmax=qmax,
+                              symmetry=(not unsigned) and offset == 0)
 
     def to_qnn_encoding_dict(self, encoding_version=None) -> Union[List, Dict]:
         """The encoding as a dictionary of the given format version (encoding.py:362-458)."""
@@ -232,6 +269,40 @@ class AffineEncoding(EncodingBase, _GridMixin):
                                    zero_point_shift=self._zero_point_shift)
 
 
+class VectorEncoding(AffineEncoding):
+    """Affine encoding of a vector-quantized tensor (encoding.py:500-575): the codebook geometry travels with it into
+    the legacy and 1.0.0 dictionaries."""
+
+    _FIELDS = ("rows_per_block", "cols_per_block", "vector_dim", "vector_stride", "index_bw")
+
+    def __init__(self, scale: torch.Tensor, offset: torch.Tensor, bitwidth: int, signed=False, symmetry=False,
+                 block_size: Optional[Tuple[int, ...]] = None, **kwargs):
+        extra = {k: kwargs.pop(k) for k in self._FIELDS}  # all five are required
+        super().__init__(scale, offset, bitwidth, signed, symmetry, block_size, **kwargs)
+        for k, v in extra.items():
+            setattr(self, k, v)
+
+    def _get_additional_properties(self) -> Dict[str, Any]:
+        return {k: getattr(self, k) for k in self._FIELDS}
+
+    def _to_legacy_format(self) -> List[Dict]:
+        encoding = super()._to_legacy_format()
+        for e in encoding:
+            e.update(self._get_additional_properties())
+        return encoding
+
+    def to_qnn_encoding_dict(self, encoding_version=None):
+        encodings = super().to_qnn_encoding_dict(encoding_version)
+        if encoding_version == "1.0.0":
+            encodings.update(self._get_additional_properties())
+            encodings["enc_type"] = "VECTOR"
+        return encodings
+
+    def _rebuilt(self, scale, offset):
+        return VectorEncoding(scale, offset, self.bitwidth, self.signed, self._symmetry, self.block_size,
+                              producer=self.producer, **self._get_additional_properties())
+
+
 class GroupedBlockEncoding(AffineEncoding):
     """Blockwise encoding whose block scales are integer multiples of a per-channel scale (LPBQ)."""
 
@@ -279,6 +350,41 @@ class GroupedBlockEncoding(AffineEncoding):
                                     "axis": channel_axis},
                         "output_dtype": output_dtype})
         return enc
+
+    @classmethod
+    def _from_affine_encoding(cls, encoding: AffineEncoding) -> "GroupedBlockEncoding":
+        """A symmetric blockwise encoding read as a grouped one (encoding.py:686-735): the groups run along the block
+        axis, the block scales expand to twice the bitwidth, and the reading is accepted if snapping the scales to
+        integer multiples of the per-channel scale leaves them where they are."""
+        from aimet_amd.quantization.affine.quantizer import GroupedBlockQuantizeDequantize
+
+        if isinstance(encoding, GroupedBlockEncoding):
+            return encoding
+        if not isinstance(encoding, AffineEncoding):
+            raise ValueError(f"Only AffineEncoding can be converted to GroupedBlockEncoding; got {type(encoding)}")
+        if encoding.block_size is None:
+            raise ValueError("Only blockwise AffineEncodings can be converted to GroupedBlockEncoding; "
+                             f"got block_size={encoding.block_size}")
+        if not encoding.symmetry:
+            raise ValueError("Only symmetric AffineEncodings can be converted to GroupedBlockEncoding; "
+                             "asymmetric encodings are not supported")
+        _, block_axis = encoding._safe_get_channel_and_block_axis()
+        ndim = encoding.scale.dim()
+        block_grouping = tuple(d if block_axis in (axis, axis - ndim) else 1
+                               for axis, d in enumerate(encoding.scale.shape))
+        qtzr = GroupedBlockQuantizeDequantize(shape=encoding.scale.shape, bitwidth=encoding.bitwidth,
+                                              symmetric=encoding.symmetry, decompressed_bw=encoding.bitwidth * 2,
+                                              block_size=encoding.block_size, block_grouping=block_grouping)
+        qtzr.to(encoding.scale.device)
+        with torch.no_grad():
+            qtzr.min.copy_(encoding.min)
+            qtzr.max.copy_(encoding.max)
+        lpbq = qtzr.get_encodings()
+        if torch.allclose(encoding.scale, lpbq.scale):
+            if encoding._input_shape_hint is not None:
+                lpbq._hint_input_shape(encoding._input_shape_hint)
+            return lpbq
+        raise ValueError("Failed to interpret encoding as GroupedBlockEncoding.")
 
     def _rebuilt(self, scale, offset):
         return GroupedBlockEncoding(scale, offset, self.bitwidth, self.signed, self._symmetry, self.block_size,

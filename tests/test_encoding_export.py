@@ -109,3 +109,58 @@ def test_zero_point_shift_and_errors():
     two_block_axes = AffineEncoding(torch.ones(2, 2), torch.zeros(2, 2), 0, 255, False, (5, 5))._hint_input_shape((10, 10))
     with pytest.raises(RuntimeError, match="Multiple non-trivial block axes"):
         two_block_axes.to_qnn_encoding_dict("2.0.0")
+
+
+def test_from_qnn_encoding_dict():
+    """Reference expectation: test_affine_quantizer.py:2788-2826."""
+    e = AffineEncoding._from_qnn_encoding_dict({"y_scale": 0.1, "output_dtype": "int8"}, version="2.0.0")
+    assert e.scale == 0.1 and e.offset == 0 and e.symmetry and (e.qmin, e.qmax) == (-128, 127)
+    e = AffineEncoding._from_qnn_encoding_dict({"y_scale": 0.1, "output_dtype": "uint8"}, version="2.0.0")
+    assert e.scale == 0.1 and e.offset == 0 and not e.symmetry and (e.qmin, e.qmax) == (0, 255)
+    e = AffineEncoding._from_qnn_encoding_dict({"y_scale": 0.1, "y_zero_point": 0, "output_dtype": "int8"}, version="2.0.0")
+    assert e.scale == 0.1 and e.offset == 0 and e.symmetry
+    e = AffineEncoding._from_qnn_encoding_dict({"y_scale": 0.1, "y_zero_point": 128, "output_dtype": "uint8"}, version="2.0.0")
+    assert e.scale == 0.1 and e.offset == -128 and not e.symmetry
+    # the version is recognised from the keys; everything but per-tensor 2.x dictionaries is refused
+    assert AffineEncoding._from_qnn_encoding_dict({"y_scale": 0.5, "output_dtype": "uint4"}).qmax == 15
+    with pytest.raises(NotImplementedError):
+        AffineEncoding._from_qnn_encoding_dict({"scale": [0.1], "bw": 8}, version=None)
+    with pytest.raises(NotImplementedError):
+        AffineEncoding._from_qnn_encoding_dict({"y_scale": [0.1, 0.2], "axis": 0, "output_dtype": "int8"}, version="2.1.0")
+    # and a per-tensor encoding survives the round trip
+    src = AffineEncoding(torch.tensor(0.25), torch.tensor(-3.0), 0, 255)
+    back = AffineEncoding._from_qnn_encoding_dict(src.to_qnn_encoding_dict("2.0.0"), version="2.0.0")
+    assert back.scale == src.scale and back.offset == src.offset and (back.qmin, back.qmax) == (0, 255)
+
+
+def test_encoding_dtype_is_the_narrowest_integer_type_that_holds_the_grid():
+    """encoding.py:178-192."""
+    one, zero = torch.tensor(1.0), torch.tensor(0.0)
+    assert AffineEncoding(one, zero, 0, 255).dtype == torch.uint8
+    assert AffineEncoding(one, zero, 0, 15).dtype == torch.uint8
+    assert AffineEncoding(one, zero, -128, 127).dtype == torch.int8
+    assert AffineEncoding(one, zero, -8, 7).dtype == torch.int8
+    assert AffineEncoding(one, zero, 0, 256).dtype == torch.int16
+    assert AffineEncoding(one, zero, -32768, 32767).dtype == torch.int16
+    assert AffineEncoding(one, zero, 0, 65535).dtype == torch.int32
+    assert AffineEncoding(one, zero, -(2 ** 31), 2 ** 31 - 1).dtype == torch.int32
+
+
+def test_vector_encoding_carries_its_codebook_geometry():
+    """encoding.py:500-575."""
+    from aimet_amd.quantization.affine import VectorEncoding
+
+    geometry = dict(rows_per_block=64, cols_per_block=2, vector_dim=2, vector_stride=1, index_bw=8)
+    e = VectorEncoding(torch.tensor([0.5, 0.25]), torch.zeros(2), 8, signed=True, symmetry=True, **geometry)
+    assert e._get_additional_properties() == geometry
+    legacy = e.to_qnn_encoding_dict("0.6.1")
+    assert len(legacy) == 2 and all(all(entry[k] == v for k, v in geometry.items()) for entry in legacy)
+    v1 = e._hint_input_shape((2, 8)).to_qnn_encoding_dict("1.0.0")
+    assert v1["enc_type"] == "VECTOR" and all(v1[k] == v for k, v in geometry.items())
+    assert "rows_per_block" not in e.to_qnn_encoding_dict("2.0.0")
+    moved = e.to(torch.float64)
+    assert isinstance(moved, VectorEncoding) and moved.scale.dtype == torch.float64
+    assert moved._get_additional_properties() == geometry
+    assert AffineEncoding(torch.tensor(1.0), torch.tensor(0.0), 0, 255)._get_additional_properties() == {}
+    with pytest.raises(KeyError):
+        VectorEncoding(torch.tensor(1.0), torch.tensor(0.0), 8, rows_per_block=1)

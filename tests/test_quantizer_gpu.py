@@ -1301,3 +1301,35 @@ def test_quantize_held_as_scale_offset(device, symmetric):
     assert_close_rel(q.scale.grad, s.grad, 1e-5, "scale gradient", abs_floor=1e-30)
     if not symmetric:
         assert_close_rel(q.offset.grad, o.grad, 1e-5, "offset gradient", abs_floor=1e-30)
+
+
+def test_blockwise_encoding_read_as_a_grouped_one(device):
+    """GroupedBlockEncoding._from_affine_encoding (encoding.py:686-735): block scales that ARE integer multiples of a
+    per-channel scale convert (with the same scales, the grouping along the block axis and twice the bitwidth);
+    scales that are not, asymmetric and per-channel encodings are refused."""
+    from aimet_amd.quantization.affine import AffineEncoding, GroupedBlockEncoding
+
+    per_channel = torch.tensor([[0.01], [0.02], [0.04]], device=device)
+    multipliers = torch.tensor([[16.0, 3.0, 7.0, 1.0], [16.0, 16.0, 2.0, 9.0], [5.0, 16.0, 11.0, 4.0]], device=device)
+    scale = per_channel * multipliers  # 4-bit grid, 8-bit expansion: multipliers 1..16, the largest one is 16
+    enc = AffineEncoding(scale, torch.zeros_like(scale), -8, 7, True, (1, 32))._hint_input_shape((3, 128))
+    lpbq = GroupedBlockEncoding._from_affine_encoding(enc)
+    assert isinstance(lpbq, GroupedBlockEncoding)
+    assert lpbq.block_grouping == (1, 4) and lpbq.decompressed_bw == 8 and lpbq.bitwidth == 4
+    assert torch.allclose(lpbq.scale, scale) and torch.allclose(lpbq.per_channel_scale, per_channel)
+    assert torch.equal(lpbq.per_block_int_scale.float(), multipliers)
+    assert GroupedBlockEncoding._from_affine_encoding(lpbq) is lpbq
+    exported = lpbq.to_qnn_encoding_dict("2.0.0")
+    assert exported["per_block_int_scale"] == multipliers.int().tolist()
+
+    off_grid = AffineEncoding(scale * torch.tensor([[1.0, 1.03, 1.0, 1.0]], device=device), torch.zeros_like(scale), -8, 7,
+                              True, (1, 32))._hint_input_shape((3, 128))
+    with pytest.raises(ValueError, match="Failed to interpret"):
+        GroupedBlockEncoding._from_affine_encoding(off_grid)
+    with pytest.raises(ValueError, match="blockwise"):
+        GroupedBlockEncoding._from_affine_encoding(AffineEncoding(per_channel, torch.zeros_like(per_channel), -8, 7, True))
+    with pytest.raises(ValueError, match="symmetric"):
+        GroupedBlockEncoding._from_affine_encoding(
+            AffineEncoding(scale, torch.full_like(scale, -3.0), 0, 15, False, (1, 32))._hint_input_shape((3, 128)))
+    with pytest.raises(ValueError, match="Only AffineEncoding"):
+        GroupedBlockEncoding._from_affine_encoding(object())
