@@ -867,6 +867,7 @@ extern "C" int ahq_minmax_slots_to_encodings(int32_t dtype, const void* slots, i
 extern "C" int ahq_minmax_slots_finalize_many(const ahq_slots_finalize_item* items, int64_t count, int32_t* flags,
                                               void* stream) {
     if (count < 0 || (count > 0 && !items)) return set_error("null argument"), AHQ_ERR_INVALID;
+    if (count == 0) return AHQ_OK;
     hipStream_t s = static_cast<hipStream_t>(stream);
     for (int64_t base = 0; base < count; base += kManySlots) {
         const int n = (int)(count - base < kManySlots ? count - base : kManySlots);

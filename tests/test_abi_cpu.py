@@ -341,3 +341,46 @@ def test_ctypes_structures_have_the_layout_the_header_declares(tmp_path):
         assert seen[(cname, "size")] == ctypes.sizeof(cls), cname
         for field, _ in cls._fields_:
             assert seen[(cname, field)] == getattr(cls, field).offset, f"{cname}.{field}"
+
+
+def test_argument_validation_of_the_batched_entry_points(lib):
+    """ahq_grid_probe_many / ahq_minmax_calibrate_qdq_many / ahq_minmax_slots_finalize_many refuse bad arguments on
+    the host, name the failing item and launch nothing (no GPU here)."""
+    import ctypes
+
+    from aimet_amd import _lib
+
+    assert lib.ahq_grid_probe_many(None, 0, None, None, None) == 0          # nothing to do
+    assert lib.ahq_minmax_calibrate_qdq_many(None, 0, None, None) == 0
+    assert lib.ahq_minmax_slots_finalize_many(None, 0, None, None) == 0
+    assert lib.ahq_grid_probe_many(None, 2, None, None, None) == 1
+    assert lib.ahq_grid_probe_many(None, -1, None, None, None) == 1
+    assert lib.ahq_minmax_calibrate_qdq_many(None, 3, None, None) == 1
+    assert lib.ahq_minmax_slots_finalize_many(None, 1, None, None) == 1
+
+    probes = (_lib.GridProbeItem * 2)()
+    for it in probes:
+        it.dtype, it.layout, it.x, it.num_levels = 0, _lib.make_layout([64, 64], [1, 64], [1, 0]), 256, 8
+    probes[1].dtype = 9
+    verdicts = (ctypes.c_uint8 * 2)()
+    assert lib.ahq_grid_probe_many(probes, 2, None, None, None) == 1        # nowhere to put the verdicts
+    probes[0].dtype = 9                                                      # the first item fails before any launch
+    assert lib.ahq_grid_probe_many(probes, 2, verdicts, None, None) == 1
+    assert b"item 0" in lib.ahq_last_error()
+
+    items = (_lib.SlotsFinalizeItem * 2)()
+    for it in items:
+        it.stat_dtype, it.symmetric, it.slots, it.num_steps = 0, 0, 256, 255
+        it.minimum_scale_in_dtype = it.minimum_scale = 1e-9
+        it.dtype_max, it.near_max_threshold = 3e38, 1e37
+        it.param_dtype, it.param_min, it.param_max = 0, 256, 256
+        it.qmin, it.qmax, it.grid_minimum_scale, it.scale, it.offset = 0, 255, 1e-9, 256, 256
+    items[0].slots = None
+    assert lib.ahq_minmax_slots_finalize_many(items, 2, 256, None) == 1
+    assert b"item 0" in lib.ahq_last_error() and b"slots" in lib.ahq_last_error()
+    items[0].slots = 258                                                     # not 4-byte aligned
+    assert lib.ahq_minmax_slots_finalize_many(items, 2, 256, None) == 1
+    items[0].slots, items[0].qmin = 256, 300
+    assert lib.ahq_minmax_slots_finalize_many(items, 2, 256, None) == 1 and b"qmax" in lib.ahq_last_error()
+    items[0].qmin, items[0].param_dtype = 0, 7
+    assert lib.ahq_minmax_slots_finalize_many(items, 2, 256, None) == 1 and b"dtype" in lib.ahq_last_error()
