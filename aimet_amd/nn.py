@@ -83,6 +83,35 @@ def _may_be_prequantized(param: torch.Tensor, qtzr: AffineQuantizerBase, on_devi
     return ~torch.any(distinct > num_levels)
 
 
+class _Removed:
+    """Quantizers taken out of a ModuleList / ModuleDict at once (aimet_torch/nn/base.py:1240-1265 with
+    utils._ContextManager): the slots read None from the moment of the call; leaving a ``with`` block puts them back,
+    a bare call leaves them out for good."""
+
+    def __init__(self, container, keys):
+        slots = container._modules  # pylint: disable=protected-access
+        self._restore = [(slots, k, slots[k]) for k in keys]
+        for k in keys:
+            slots[k] = None
+
+    @classmethod
+    def both(cls, first: "_Removed", second: "_Removed") -> "_Removed":
+        merged = cls.__new__(cls)
+        merged._restore = first._restore + second._restore  # pylint: disable=protected-access
+        return merged
+
+    def _cleanup(self):
+        for slots, k, q in self._restore:
+            slots[k] = q
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self._cleanup()
+        return False
+
+
 class QuantizedLinear(nn.Linear):
     """``nn.Linear`` with quantizers at its input, weight and output (any of them may be None)."""
 
@@ -216,18 +245,77 @@ class QuantizedLinear(nn.Linear):
             names.append(name)
         return names
 
-    @contextlib.contextmanager
+    def _remove_input_quantizers(self, indices=None):
+        """nn/base.py:983-993: the input quantizers (all, one index or several) are taken out at once; used as a
+        context manager, the call puts them back on leaving."""
+        if isinstance(indices, int):
+            indices = [indices]
+        elif indices is None:
+            indices = list(range(len(self.input_quantizers)))
+        return _Removed(self.input_quantizers, [str(i) for i in indices])
+
     def _remove_param_quantizers(self, keys=None):
         """nn/base.py:995-1005."""
         keys = list(self.param_quantizers.keys()) if keys is None else ([keys] if isinstance(keys, str) else list(keys))
-        slots = self.param_quantizers._modules  # pylint: disable=protected-access
-        saved = {k: slots[k] for k in keys}
-        try:
-            for k in keys:
-                slots[k] = None
-            yield
-        finally:
-            slots.update(saved)
+        return _Removed(self.param_quantizers, keys)
+
+    def _remove_output_quantizers(self, indices=None):
+        """nn/base.py:1007-1017."""
+        if isinstance(indices, int):
+            indices = [indices]
+        elif indices is None:
+            indices = list(range(len(self.output_quantizers)))
+        return _Removed(self.output_quantizers, [str(i) for i in indices])
+
+    def _remove_activation_quantizers(self):
+        """nn/base.py:1019-1026."""
+        return _Removed.both(self._remove_output_quantizers(), self._remove_input_quantizers())
+
+    def _remove_all_quantizers(self):
+        """nn/base.py:1028-1035."""
+        return _Removed.both(self._remove_activation_quantizers(), self._remove_param_quantizers())
+
+    def compute_param_encodings(self):
+        """Compute the encodings of the parameter quantizers (nn/base.py:388-390)."""
+        self._compute_param_encodings(overwrite=True)
+
+    def export_input_encodings(self, encoding_version: str):
+        """One exported dictionary (or None) per input quantizer (nn/base.py:527-539)."""
+        return [q.get_encodings().to_qnn_encoding_dict(encoding_version)
+                if isinstance(q, QuantizerBase) and q.is_initialized() else None for q in self.input_quantizers]
+
+    def export_output_encodings(self, encoding_version: str):
+        """nn/base.py:586-598."""
+        return [q.get_encodings().to_qnn_encoding_dict(encoding_version)
+                if isinstance(q, QuantizerBase) and q.is_initialized() else None for q in self.output_quantizers]
+
+    def export_param_encodings(self, encoding_version: str):
+        """{parameter name: exported dictionary or None} (nn/base.py:645-678); a parameter that is an already
+        quantized tensor without a quantizer exports the encoding it carries."""
+        from aimet_amd.quantization.tensor import QuantizedTensorBase
+
+        out = {}
+        for name, q in self.param_quantizers.items():
+            param = getattr(self, name)
+            if isinstance(q, QuantizerBase):
+                out[name] = (q.get_encodings()._hint_input_shape(param.shape).to_qnn_encoding_dict(encoding_version)  # pylint: disable=protected-access
+                             if q.is_initialized() else None)
+            elif isinstance(param, QuantizedTensorBase) and param.encoding is not None:
+                out[name] = param.encoding._hint_input_shape(param.shape).to_qnn_encoding_dict(encoding_version)  # pylint: disable=protected-access
+            else:
+                out[name] = None
+        return out
+
+    def get_original_module(self) -> nn.Linear:
+        """The floating-point layer with the quantizers removed; parameters are shared (nn/base.py:757-794)."""
+        orig = nn.Linear.__new__(nn.Linear)
+        orig.__dict__ = self.__dict__.copy()
+        orig.__dict__.pop("forward", None)
+        orig._parameters = self._parameters.copy()  # pylint: disable=protected-access
+        orig._buffers = self._buffers.copy()  # pylint: disable=protected-access
+        orig._modules = {k: v for k, v in self._modules.items()  # pylint: disable=protected-access
+                         if k not in ("input_quantizers", "output_quantizers", "param_quantizers")}
+        return orig
 
     def fold_param_quantizers(self):
         """nn/base.py:1103-1151: bake each parameter quantizer into its parameter (the parameter becomes the

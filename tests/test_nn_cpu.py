@@ -1,0 +1,75 @@
+"""Host logic of the quantized-module glue that needs no kernel: taking quantizers out and putting them back, the
+exported encoding dictionaries of a module, the floating-point twin.  Reference: aimet_torch/nn/base.py:388-390,
+527-539, 586-598, 645-678, 757-794, 983-1035."""
+
+import torch
+
+import aimet_amd.nn as qnn
+from aimet_amd.quantization.affine import QuantizeDequantize
+
+
+def _layer():
+    lin = qnn.QuantizedLinear(8, 4, bias=True)
+    lin.input_quantizers[0] = QuantizeDequantize((), 8, False)
+    lin.output_quantizers[0] = QuantizeDequantize((), 8, False)
+    lin.param_quantizers["weight"] = QuantizeDequantize((4, 1), 4, True)
+    return lin
+
+
+def test_removed_quantizers_come_back_after_a_with_block_and_stay_out_after_a_bare_call():
+    lin = _layer()
+    iq, oq, wq = lin.input_quantizers[0], lin.output_quantizers[0], lin.param_quantizers["weight"]
+    with lin._remove_input_quantizers():
+        assert lin.input_quantizers[0] is None and lin.output_quantizers[0] is oq
+    assert lin.input_quantizers[0] is iq
+    with lin._remove_output_quantizers(0):
+        assert lin.output_quantizers[0] is None
+    assert lin.output_quantizers[0] is oq
+    with lin._remove_param_quantizers("weight"):
+        assert lin.param_quantizers["weight"] is None
+    assert lin.param_quantizers["weight"] is wq
+    with lin._remove_activation_quantizers():
+        assert lin.input_quantizers[0] is None and lin.output_quantizers[0] is None
+        assert lin.param_quantizers["weight"] is wq
+    assert lin.input_quantizers[0] is iq and lin.output_quantizers[0] is oq
+    with lin._remove_all_quantizers():
+        assert lin.input_quantizers[0] is None and lin.output_quantizers[0] is None
+        assert lin.param_quantizers["weight"] is None
+    assert (lin.input_quantizers[0], lin.output_quantizers[0], lin.param_quantizers["weight"]) == (iq, oq, wq)
+    # the reference's removal acts when it is called; without a with block nothing puts the quantizers back
+    lin._remove_param_quantizers()
+    assert lin.param_quantizers["weight"] is None and lin.input_quantizers[0] is iq
+    with qnn.remove_param_quantizers(lin):
+        pass
+    lin._remove_all_quantizers()
+    assert lin.input_quantizers[0] is None and lin.output_quantizers[0] is None
+
+
+def test_exported_encodings_of_a_module():
+    lin = _layer()
+    assert lin.export_input_encodings("1.0.0") == [None]          # nothing calibrated yet
+    assert lin.export_param_encodings("1.0.0") == {"weight": None, "bias": None}
+    lin.input_quantizers[0].set_range(0.0, 2.55)
+    lin.output_quantizers[0] = None
+    lin.param_quantizers["weight"].set_range(torch.full((4, 1), -0.8), torch.full((4, 1), 0.7))
+    (inp,) = lin.export_input_encodings("1.0.0")
+    assert inp["enc_type"] == "PER_TENSOR" and inp["bw"] == 8 and not inp["is_sym"]
+    assert abs(inp["scale"][0] - 0.01) < 1e-9 and inp["offset"] == [0]
+    assert lin.export_output_encodings("2.0.0") == [None]
+    params = lin.export_param_encodings("2.0.0")
+    assert params["bias"] is None
+    assert params["weight"]["output_dtype"] == "int4" and params["weight"]["axis"] in (0, -2)  # the output-channel axis
+    assert len(params["weight"]["y_scale"]) == 4 and abs(params["weight"]["y_scale"][0] - 0.1) < 1e-7
+    legacy = lin.export_param_encodings("0.6.1")["weight"]
+    assert len(legacy) == 4 and legacy[0]["bitwidth"] == 4 and legacy[0]["is_symmetric"] == "True"
+
+
+def test_the_floating_point_twin_shares_the_parameters():
+    lin = _layer()
+    plain = lin.get_original_module()
+    assert type(plain) is torch.nn.Linear
+    assert plain.weight is lin.weight and plain.bias is lin.bias
+    assert not hasattr(plain, "param_quantizers") and not hasattr(plain, "input_quantizers")
+    x = torch.randn(3, 8)
+    assert torch.equal(plain(x), torch.nn.functional.linear(x, lin.weight, lin.bias))
+    assert lin.param_quantizers["weight"] is not None  # the quantized module is left as it was
