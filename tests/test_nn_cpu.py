@@ -73,3 +73,28 @@ def test_the_floating_point_twin_shares_the_parameters():
     x = torch.randn(3, 8)
     assert torch.equal(plain(x), torch.nn.functional.linear(x, lin.weight, lin.bias))
     assert lin.param_quantizers["weight"] is not None  # the quantized module is left as it was
+
+
+def test_model_level_removal_utilities():
+    """aimet_torch.utils.remove_{input,output,param,activation,all}_quantizers (utils.py:1305-1540)."""
+    model = torch.nn.Sequential(_layer(), torch.nn.ReLU(), _layer())
+    layers = [model[0], model[2]]
+    kept = [(m.input_quantizers[0], m.output_quantizers[0], m.param_quantizers["weight"]) for m in layers]
+
+    def state():
+        return [(m.input_quantizers[0] is not None, m.output_quantizers[0] is not None,
+                 m.param_quantizers["weight"] is not None) for m in layers]
+
+    for remove, want in ((qnn.remove_input_quantizers, (False, True, True)),
+                         (qnn.remove_output_quantizers, (True, False, True)),
+                         (qnn.remove_param_quantizers, (True, True, False)),
+                         (qnn.remove_activation_quantizers, (False, False, True)),
+                         (qnn.remove_all_quantizers, (False, False, False))):
+        with remove(model):
+            assert state() == [want, want]
+        assert state() == [(True, True, True)] * 2
+    assert [(m.input_quantizers[0], m.output_quantizers[0], m.param_quantizers["weight"]) for m in layers] == kept
+    qnn.remove_activation_quantizers(model)  # a bare call is for good
+    assert state() == [(False, False, True)] * 2
+    with qnn.remove_all_quantizers(torch.nn.Sequential(torch.nn.ReLU())):
+        pass  # a model without quantized modules
