@@ -88,6 +88,26 @@ __global__ __launch_bounds__(kBlock) void qdq_fwd_lpbq_kernel(const QdqArgs a, c
     else fwd_tile<IO, VEC, M, false, kFwdUnroll, true>(a, t, sp, &f);
 }
 
+template <typename IO, int VEC, typename M, bool FAST>
+__device__ __forceinline__ void fwd_cols_rows(const QdqArgs& a, const Pack<IO, VEC>* in, const EncP* e, IO* __restrict__ y,
+                                              int64_t r0, int64_t c0) {
+#pragma unroll
+    for (int u = 0; u < kColUnroll; ++u) {
+        if (r0 + u >= a.I) continue;
+        Pack<IO, VEC> out;
+        Pack<uint8_t, VEC> mk;
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) {
+            bool inr;
+            const float r = M::template fwd<FAST>(load_f32(in[u].v[k]), e[k], a.gc, inr);
+            out.v[k] = store_rounded<IO, M::kCD>(r);
+            mk.v[k] = inr ? 1 : 0;
+        }
+        store_pack_stream<IO, VEC>(y + (r0 + u) * a.J + c0, out);
+        if (a.mask) store_pack_stream<uint8_t, VEC>(a.mask + (r0 + u) * a.J + c0, mk);
+    }
+}
+
 template <typename IO, int VEC, typename M, int WAVES>
 __global__ __launch_bounds__(WAVES * kWave) void qdq_fwd_cols_kernel(const QdqArgs a) {
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
@@ -97,38 +117,24 @@ __global__ __launch_bounds__(WAVES * kWave) void qdq_fwd_cols_kernel(const QdqAr
     IO* __restrict__ y = static_cast<IO*>(a.y);
     EncP e[VEC];
     bool enc_fast = true;
+    load_col_encodings<M, VEC>(a, c0, e);
 #pragma unroll
-    for (int k = 0; k < VEC; ++k) {
-        e[k] = load_enc<M>(a, c0 + k);
-        enc_fast &= !M::kDiv || e[k].rs != 0.f;
-    }
+    for (int k = 0; k < VEC; ++k) enc_fast &= !M::kDiv || e[k].rs != 0.f;
     const int64_t step = (int64_t)gridDim.y * WAVES * kColUnroll;
     for (int64_t r0 = ((int64_t)blockIdx.y * WAVES + wave) * kColUnroll; r0 < a.I; r0 += step) {
         Pack<IO, VEC> in[kColUnroll];
         bool ok = enc_fast;
 #pragma unroll
         for (int u = 0; u < kColUnroll; ++u)
-            if (r0 + u < a.I) in[u] = load_pack<IO, VEC>(x + (r0 + u) * a.J + c0);
+            if (r0 + u < a.I) in[u] = load_pack_hinted<IO, VEC>(x + (r0 + u) * a.J + c0, a.stream_loads != 0);
 #pragma unroll
         for (int u = 0; u < kColUnroll; ++u)
             if (M::kDiv && r0 + u < a.I) ok &= row_can_divide_fast<IO, VEC>(in[u]);
-        const bool fast = !M::kDiv || __builtin_amdgcn_ballot_w64(!ok) == 0;  // wave-uniform, like the tiled kernel
-#pragma unroll
-        for (int u = 0; u < kColUnroll; ++u) {
-            if (r0 + u >= a.I) continue;
-            Pack<IO, VEC> out;
-            Pack<uint8_t, VEC> mk;
-#pragma unroll
-            for (int k = 0; k < VEC; ++k) {
-                bool inr;
-                const float v = load_f32(in[u].v[k]);
-                const float r = fast ? M::template fwd<true>(v, e[k], a.gc, inr) : M::template fwd<false>(v, e[k], a.gc, inr);
-                out.v[k] = store_rounded<IO, M::kCD>(r);
-                mk.v[k] = inr ? 1 : 0;
-            }
-            store_pack_stream<IO, VEC>(y + (r0 + u) * a.J + c0, out);
-            if (a.mask) store_pack_stream<uint8_t, VEC>(a.mask + (r0 + u) * a.J + c0, mk);
-        }
+        // wave-uniform, like the tiled kernel: one branch per step, and each side a straight run of arithmetic over
+        // all its elements (a choice per element costs a branch per element and keeps the compiler from interleaving
+        // the elements' instruction chains)
+        if (!M::kDiv || __builtin_amdgcn_ballot_w64(!ok) == 0) fwd_cols_rows<IO, VEC, M, true>(a, in, e, y, r0, c0);
+        else fwd_cols_rows<IO, VEC, M, false>(a, in, e, y, r0, c0);
     }
 }
 
@@ -148,10 +154,13 @@ __global__ __launch_bounds__(kBlock) void qdq_fwd_generic_kernel(const QdqArgs a
 template <typename IO, typename M>
 static void launch_fwd(const Plan& p, const QdqArgs& a, hipStream_t st, bool aligned) {
     if (cols_layout<IO>(p, aligned) && (p.cl.J / IoTraits<IO>::kVec + kWave - 1) / kWave <= 0x7fffffff) {
-        // a lane prepares kVec encodings before its first row: the more of them, the more rows it should walk
-        constexpr int W = kFwdColWaves;
-        hipLaunchKernelGGL((qdq_fwd_cols_kernel<IO, IoTraits<IO>::kVec, M, W>),
-                           cols_grid<IO>(p, (IoTraits<IO>::kVec > 4 ? 768 : 2048) * (kColWaves / W), W), dim3(W * kWave), 0, st, a);
+        // About as many workgroups as the chip holds at once (256 CUs; the 16-bit kernels run four waves per SIMD,
+        // the float32 ones eight): every wave prepares its encodings before its first row, and a second round of
+        // waves pays that set-up while the memory pipes drain (8192 x 4096 bf16: 25.5 us with 1024 workgroups,
+        // 28.7 us with 3072, 32.3 us with 384; float32: 44.3 us with 8192, 45.6 us with 4096 or 16384).
+        constexpr int V = IoTraits<IO>::kVec;
+        hipLaunchKernelGGL((qdq_fwd_cols_kernel<IO, V, M, kFwdColWaves>), (cols_grid<IO, V>(p, V > 4 ? 1024 : 8192, kFwdColWaves)),
+                           dim3(kFwdColWaves * kWave), 0, st, a);
         return;
     }
     if (p.cl.kind == kGeneric) {

@@ -336,6 +336,49 @@ __global__ __launch_bounds__(kBlock) void qdq_bwd_strided_finish_kernel(const do
     }
 }
 
+// The same sums for many encodings (at least half a wave of them): a lane per encoding, so that a wave reads 64
+// neighbouring pairs, one kilobyte, per load (a wave per encoding reads 64 pairs that lie `stride` apart: a cache line
+// fetched for every 16 bytes used).  The waves of a workgroup take contiguous shares of the `count` rows, a few loads
+// in flight each, and wave 0 adds the shares up in wave order.
+constexpr int kRowsFinishWaves = 16;
+constexpr int kRowsFinishLoads = 4;
+__global__ __launch_bounds__(kRowsFinishWaves * kWave) void qdq_bwd_rows_finish_kernel(const double* __restrict__ partials,
+                                                                                       int64_t count, int64_t num_enc,
+                                                                                       float* gscale, float* goffset, int cd) {
+    __shared__ double shares[kRowsFinishWaves][2][kWave];
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int64_t e = (int64_t)blockIdx.x * kWave + lane;
+    const int64_t share = (count + kRowsFinishWaves - 1) / kRowsFinishWaves;
+    const int64_t q0 = wave * share, q1 = q0 + share < count ? q0 + share : count;
+    double s = 0.0, o = 0.0;
+    if (e < num_enc) {
+        const double2* __restrict__ pairs = reinterpret_cast<const double2*>(partials) + e;
+        for (int64_t q = q0; q < q1; q += kRowsFinishLoads) {
+            double2 v[kRowsFinishLoads];
+#pragma unroll
+            for (int u = 0; u < kRowsFinishLoads; ++u) v[u] = q + u < q1 ? pairs[(q + u) * num_enc] : double2{0.0, 0.0};
+#pragma unroll
+            for (int u = 0; u < kRowsFinishLoads; ++u) {
+                s += v[u].x;
+                o += v[u].y;
+            }
+        }
+    }
+    shares[wave][0][lane] = s;
+    shares[wave][1][lane] = o;
+    __syncthreads();
+    if (wave == 0 && e < num_enc) {
+        s = o = 0.0;
+#pragma unroll
+        for (int w = 0; w < kRowsFinishWaves; ++w) {
+            s += shares[w][0][lane];
+            o += shares[w][1][lane];
+        }
+        gscale[e] = finish_sum_rt(s, cd);
+        goffset[e] = finish_sum_rt(o, cd);
+    }
+}
+
 template <typename IO, typename M>
 __global__ __launch_bounds__(kBlock) void qdq_bwd_generic_kernel(const QdqArgs a) {
     const IO* __restrict__ x = static_cast<const IO*>(a.x);
@@ -380,34 +423,111 @@ __global__ __launch_bounds__(kBlock) void qdq_bwd_generic_kernel(const QdqArgs a
     }
 }
 
-// Backward for run length 1 (see qdq_fwd_cols_kernel): every lane keeps the sums of its VEC encodings over the rows
-// it walks, the waves of a workgroup add theirs up in LDS one after the other, and the workgroup's sums go to its own
-// row of the partials ([row group][encoding]), which qdq_bwd_strided_finish_kernel adds up in order.
+// Backward for run length 1 (see qdq_fwd_cols_kernel).  A lane keeps the sums of its VEC encodings over the rows it
+// walks: in single precision in registers for kColFlushSteps steps (kColFlushSteps * kColUnroll terms per encoding,
+// about what the tiled kernel adds in single precision per vector), then added to double-precision sums that live in
+// LDS, a table per wave (sixteen double accumulators per lane in registers leave the 16-bit kernels two waves per
+// SIMD).  At the end the first waves add the tables up in wave order and the workgroup's sums go to its own row of the
+// partials ([row group][encoding]), which qdq_bwd_rows_finish_kernel adds up in order.
+constexpr int kColFlushSteps = 4;
+
+// One step of a wave: kColUnroll rows of VEC elements per lane.  Like the tiled kernel, the division-free form looks
+// at a whole row of the wave before it spends work on out-of-range terms: when every element is inside the grid the
+// input gradient is the output gradient as loaded and the offset gradient gets no term.  r0 is the same for all lanes
+// of a wave, so the row test is wave-uniform.  Returns whether vo received terms (wave-uniform).
+template <typename IO, int VEC, typename M, bool FAST>
+__device__ __forceinline__ bool bwd_cols_rows(const QdqArgs& a, const Pack<IO, VEC>* xin, const Pack<IO, VEC>* gin,
+                                              const EncP* e, IO* __restrict__ gxp, int64_t r0, int64_t c0, float* vs,
+                                              float* vo) {
+    bool offset_terms = false;
+#pragma unroll
+    for (int u = 0; u < kColUnroll; ++u) {
+        if (r0 + u >= a.I) continue;
+        IO* const out_row = gxp ? gxp + (r0 + u) * a.J + c0 : nullptr;
+        if constexpr (FAST && M::kSplitBwd) {
+            float tq[VEC], xr[VEC], m[VEC];
+            bool all_in = true;
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) {
+                M::bwd_pre(load_f32(xin[u].v[k]), e[k], e[k].p1 + a.gc.qmin, e[k].p1 + a.gc.qmax, tq[k], xr[k], m[k]);
+                all_in &= (m[k] == xr[k]);
+            }
+            if (__builtin_amdgcn_ballot_w64(!all_in) == 0) {
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) vs[k] += M::bwd_gs_in(load_f32(gin[u].v[k]), tq[k], xr[k]);
+                if (out_row) store_pack_stream<IO, VEC>(out_row, gin[u]);
+            } else {
+                offset_terms = true;
+                Pack<IO, VEC> out;
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) {
+                    const float gr = load_f32(gin[u].v[k]);
+                    const bool in = (m[k] == xr[k]);
+                    out.v[k] = store_cast<IO>(in ? gr : 0.f);
+                    vs[k] += in ? M::bwd_gs_in(gr, tq[k], xr[k]) : M::bwd_gs_out(gr, m[k]);
+                    vo[k] += in ? 0.f : M::bwd_goff_out(gr, e[k]);
+                }
+                if (out_row) store_pack_stream<IO, VEC>(out_row, out);
+            }
+        } else {
+            offset_terms = true;
+            Pack<IO, VEC> out;
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) {
+                float gx, gs, go;
+                M::template bwd<FAST>(load_f32(gin[u].v[k]), load_f32(xin[u].v[k]), e[k], a.gc, gx, gs, go);
+                out.v[k] = store_cast<IO>(gx);
+                vs[k] += gs;
+                vo[k] += go;
+            }
+            if (out_row) store_pack_stream<IO, VEC>(out_row, out);
+        }
+    }
+    return offset_terms;
+}
+
+// adds a lane's single-precision sums to its double-precision ones in the wave's table and clears them
+template <int VEC>
+__device__ __forceinline__ void flush_col_sums(double (*table)[kWave], int lane, float* vs, float* vo, bool offset_terms) {
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) {
+        table[2 * k][lane] += (double)vs[k];
+        vs[k] = 0.f;
+    }
+    if (offset_terms) {
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) {
+            table[2 * k + 1][lane] += (double)vo[k];
+            vo[k] = 0.f;
+        }
+    }
+}
+
 template <typename IO, int VEC, typename M, int WAVES>
 __global__ __launch_bounds__(WAVES * kWave) void qdq_bwd_cols_kernel(const QdqArgs a) {
-    __shared__ double sums[2 * VEC * kWave];
+    __shared__ double sums[WAVES][2 * VEC][kWave];  // [wave][2 * k: scale sum, 2 * k + 1: offset sum][lane]
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     const int64_t c0 = ((int64_t)blockIdx.x * kWave + lane) * VEC;
     const bool live = c0 < a.J;
     const bool want_pg = a.partials != nullptr;
-    if (want_pg) {
-        for (int i = threadIdx.x; i < 2 * VEC * kWave; i += WAVES * kWave) sums[i] = 0.0;
-        __syncthreads();
-    }
-    double acc_s[VEC], acc_o[VEC];
+    if (want_pg) {  // a wave clears its own table: nobody else touches it before the barrier below
 #pragma unroll
-    for (int k = 0; k < VEC; ++k) acc_s[k] = acc_o[k] = 0.0;
+        for (int i = 0; i < 2 * VEC; ++i) sums[wave][i][lane] = 0.0;
+    }
     if (live) {
         const IO* __restrict__ x = static_cast<const IO*>(a.x);
         const IO* __restrict__ g = static_cast<const IO*>(a.g);
         IO* __restrict__ gxp = static_cast<IO*>(a.gx);
         EncP e[VEC];
         bool enc_fast = true;
+        load_col_encodings<M, VEC>(a, c0, e);
 #pragma unroll
-        for (int k = 0; k < VEC; ++k) {
-            e[k] = load_enc<M>(a, c0 + k);
-            enc_fast &= !M::kDiv || e[k].rs != 0.f;
-        }
+        for (int k = 0; k < VEC; ++k) enc_fast &= !M::kDiv || e[k].rs != 0.f;
+        float vs[VEC], vo[VEC];
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) vs[k] = vo[k] = 0.f;
+        bool offset_terms = false;
+        int pending = 0;
         const int64_t step = (int64_t)gridDim.y * WAVES * kColUnroll;
         for (int64_t r0 = ((int64_t)blockIdx.y * WAVES + wave) * kColUnroll; r0 < a.I; r0 += step) {
             Pack<IO, VEC> xin[kColUnroll], gin[kColUnroll];
@@ -415,50 +535,39 @@ __global__ __launch_bounds__(WAVES * kWave) void qdq_bwd_cols_kernel(const QdqAr
 #pragma unroll
             for (int u = 0; u < kColUnroll; ++u)
                 if (r0 + u < a.I) {
-                    xin[u] = load_pack<IO, VEC>(x + (r0 + u) * a.J + c0);
-                    gin[u] = load_pack<IO, VEC>(g + (r0 + u) * a.J + c0);
+                    xin[u] = load_pack_hinted<IO, VEC>(x + (r0 + u) * a.J + c0, a.stream_loads != 0);
+                    gin[u] = load_pack_hinted<IO, VEC>(g + (r0 + u) * a.J + c0, a.stream_loads != 0);
                 }
 #pragma unroll
             for (int u = 0; u < kColUnroll; ++u)
                 if (M::kDiv && r0 + u < a.I) ok &= row_can_divide_fast<IO, VEC>(xin[u]);
-            const bool fast = !M::kDiv || __builtin_amdgcn_ballot_w64(!ok) == 0;
-#pragma unroll
-            for (int u = 0; u < kColUnroll; ++u) {
-                if (r0 + u >= a.I) continue;
-                Pack<IO, VEC> out;
-#pragma unroll
-                for (int k = 0; k < VEC; ++k) {
-                    float gx, gs, go;
-                    const float gr = load_f32(gin[u].v[k]), v = load_f32(xin[u].v[k]);
-                    if (fast) M::template bwd<true>(gr, v, e[k], a.gc, gx, gs, go);
-                    else M::template bwd<false>(gr, v, e[k], a.gc, gx, gs, go);
-                    out.v[k] = store_cast<IO>(gx);
-                    acc_s[k] += (double)gs;
-                    acc_o[k] += (double)go;
-                }
-                if (gxp) store_pack_stream<IO, VEC>(gxp + (r0 + u) * a.J + c0, out);
+            // one wave-uniform branch per step, each side a straight run of arithmetic over all its elements
+            if (!M::kDiv || __builtin_amdgcn_ballot_w64(!ok) == 0)
+                offset_terms |= bwd_cols_rows<IO, VEC, M, true>(a, xin, gin, e, gxp, r0, c0, vs, vo);
+            else
+                offset_terms |= bwd_cols_rows<IO, VEC, M, false>(a, xin, gin, e, gxp, r0, c0, vs, vo);
+            if (want_pg && ++pending == kColFlushSteps) {
+                flush_col_sums<VEC>(sums[wave], lane, vs, vo, offset_terms);
+                pending = 0;
+                offset_terms = false;
             }
         }
+        if (want_pg && pending) flush_col_sums<VEC>(sums[wave], lane, vs, vo, offset_terms);
     }
     if (!want_pg) return;
-    // the waves take turns, so the sums do not depend on which wave finishes first
-    for (int w = 0; w < WAVES; ++w) {
-        if (wave == w && live) {
+    __syncthreads();
+    // the tables are added up in wave order, whichever wave finished first; the 2 * VEC sums of a lane are shared out
+    // over the waves, and a lane's pair of sums for one encoding is one 16-byte store
+    double* row = a.partials + 2 * (int64_t)blockIdx.y * a.J;
+    for (int k = wave; k < VEC; k += WAVES) {
+        if (!live) break;
+        double ps = 0.0, po = 0.0;
 #pragma unroll
-            for (int k = 0; k < VEC; ++k) {
-                sums[(2 * k) * kWave + lane] += acc_s[k];
-                sums[(2 * k + 1) * kWave + lane] += acc_o[k];
-            }
+        for (int w = 0; w < WAVES; ++w) {
+            ps += sums[w][2 * k][lane];
+            po += sums[w][2 * k + 1][lane];
         }
-        __syncthreads();
-    }
-    if (wave == 0 && live) {
-        double* row = a.partials + 2 * (int64_t)blockIdx.y * a.J;
-#pragma unroll
-        for (int k = 0; k < VEC; ++k) {
-            row[2 * (c0 + k)] = sums[(2 * k) * kWave + lane];
-            row[2 * (c0 + k) + 1] = sums[(2 * k + 1) * kWave + lane];
-        }
+        store_pack<double, 2>(row + 2 * (c0 + k), Pack<double, 2>{{ps, po}});
     }
 }
 
@@ -484,16 +593,18 @@ static bool bwd_cols_layout(int io_dtype, const Plan& p, bool aligned) {
     return io_dtype == AHQ_F32 ? bwd_cols_layout<float>(p, aligned) : bwd_cols_layout<f16_t>(p, aligned);
 }
 
-// The backward kernel keeps eight encodings, sixteen double sums and two rows of two tensors per lane on a 16-bit
-// tensor: more than the 128 registers a workgroup of sixteen waves leaves a lane (36 of them were spilled: 92 us on
-// 8192 x 4096 bf16 with learned encodings; 73 us with eight waves, 62 us with four, 71 us with two).  float32:
-// 73.6 us with sixteen waves, 69.5 us with eight, 72 us with four.
+// On a 16-bit tensor a lane of the backward kernel takes four encodings (8-byte vectors), not eight: with eight, the
+// encodings, the two rows of two tensors and the temporaries of the split form need about 170 registers, two or three
+// waves per SIMD (8192 x 4096 bf16 with learned encodings: 47.6 us against 42 us, same tensors every launch).
+// Workgroups of eight waves, about as many as the chip holds at once, for the reason given at the forward launch
+// (bf16: 42.0 us with 1024 workgroups, 45.0 us with 2048; float32: 72.8 us with 256, 74.9 us with 512, 75.9 us with 1024).
+constexpr int kBwdColWaves = 8;
 template <typename IO>
-constexpr int bwd_cols_waves() { return IoTraits<IO>::kVec > 4 ? kColWaves / 4 : kColWaves / 2; }
+constexpr int bwd_cols_vec() { return IoTraits<IO>::kVec > 4 ? 4 : IoTraits<IO>::kVec; }
 
 template <typename IO>
 static dim3 bwd_cols_grid(const Plan& p) {
-    return cols_grid<IO>(p, 512 * (kColWaves / bwd_cols_waves<IO>()), bwd_cols_waves<IO>());
+    return cols_grid<IO, bwd_cols_vec<IO>()>(p, IoTraits<IO>::kVec > 4 ? 1024 : 256, kBwdColWaves);
 }
 
 static unsigned bwd_cols_row_groups(int io_dtype, const Plan& p) {
@@ -527,8 +638,12 @@ template <typename IO, typename M>
 static void launch_bwd(const Plan& p, const QdqArgs& a, hipStream_t st, bool aligned) {
     if (bwd_cols_layout<IO>(p, aligned)) {
         // few row groups: every workgroup ends with one row of partial sums
-        constexpr int W = bwd_cols_waves<IO>();
-        hipLaunchKernelGGL((qdq_bwd_cols_kernel<IO, IoTraits<IO>::kVec, M, W>), bwd_cols_grid<IO>(p), dim3(W * kWave), 0, st, a);
+        constexpr int W = kBwdColWaves, V = bwd_cols_vec<IO>();
+        dim3 g = bwd_cols_grid<IO>(p);
+        // arithmetic without a division and no sums to keep: few registers, eight waves per SIMD, so the chip holds
+        // more workgroups at once (8192 x 4096 fp32: 70.3 us against 81.8 us)
+        if (!M::kDiv && !a.partials) g = cols_grid<IO, V>(p, IoTraits<IO>::kVec > 4 ? 2048 : 1024, W);
+        hipLaunchKernelGGL((qdq_bwd_cols_kernel<IO, V, M, W>), g, dim3(W * kWave), 0, st, a);
         return;
     }
     if (p.cl.kind == kGeneric) {
@@ -627,9 +742,15 @@ extern "C" int ahq_qdq_backward(const ahq_grid* grid, const ahq_layout* layout, 
     if (want_pg && (cols || (p.red == kRedRuns && p.cl.I > 1))) {
         // one slot per (row group, encoding) or per run: added up per encoding in a fixed order
         const int64_t count = cols ? (int64_t)bwd_cols_row_groups(grid->io_dtype, p) : p.cl.I;
-        const int64_t nb = (p.cl.J + kBlock / kWave - 1) / (kBlock / kWave);
-        hipLaunchKernelGGL(qdq_bwd_strided_finish_kernel, dim3((unsigned)(nb > 4096 ? 4096 : nb)), dim3(kBlock), 0, st,
-                           (const double*)a.partials, count, p.cl.J, p.cl.J, gscale, goffset, (int)grid->compute_dtype);
+        if (p.cl.J >= kWave / 2 && (p.cl.J + kWave - 1) / kWave <= 0x7fffffff) {
+            hipLaunchKernelGGL(qdq_bwd_rows_finish_kernel, dim3((unsigned)((p.cl.J + kWave - 1) / kWave)),
+                               dim3(kRowsFinishWaves * kWave), 0, st, (const double*)a.partials, count, p.cl.J, gscale, goffset,
+                               (int)grid->compute_dtype);
+        } else {
+            const int64_t nb = (p.cl.J + kBlock / kWave - 1) / (kBlock / kWave);
+            hipLaunchKernelGGL(qdq_bwd_strided_finish_kernel, dim3((unsigned)(nb > 4096 ? 4096 : nb)), dim3(kBlock), 0, st,
+                               (const double*)a.partials, count, p.cl.J, p.cl.J, gscale, goffset, (int)grid->compute_dtype);
+        }
     }
     return check_launch("ahq_qdq_backward");
 }

@@ -599,14 +599,56 @@ __device__ __forceinline__ bool lane_can_divide_fast(const QdqArgs& a, const Til
 
 // Encodings that change with every element (run length 1: per-channel along the fastest axis).  The tiled kernel
 // would prepare one encoding per element; here a lane owns VEC neighbouring encodings, prepares them once and walks
-// down the rows, so loads and stores stay coalesced 16-byte vectors.  A workgroup is 64 lanes across x a few waves
-// down; each wave takes kColUnroll rows per step.  kColWaves is the unit the grids are sized in (workgroups of sixteen
-// waves, the first shape); the kernels run with fewer waves per workgroup and correspondingly more workgroups, which
-// measured faster (forward 8192 x 4096 fp32: 43.6 us with sixteen waves, 40.8 us with four) and leaves a lane more
-// registers.
-constexpr int kColWaves = 16;
+// down the rows, so loads and stores stay coalesced vectors.  A workgroup is 64 lanes across x a few waves down; each
+// wave takes kColUnroll rows per step.  Few waves per workgroup measured faster than many (forward 8192 x 4096 fp32:
+// 43.6 us with sixteen waves, 40.8 us with four) and leave a lane more registers.
 constexpr int kFwdColWaves = 4;
 constexpr int kColUnroll = 2;
+
+// The VEC neighbouring encodings of a lane, starting at column c0 (a multiple of VEC; VEC is 4 or 8).  Read as 16-byte
+// vectors when the arrays allow it: read one float at a time, a wave's load touches sixteen cache lines for 256 useful
+// bytes, and the 2 * VEC such loads of the set-up move as many lines through the vector cache as sixteen steps of rows.
+template <typename M, int VEC>
+__device__ __forceinline__ void load_col_encodings(const QdqArgs& a, int64_t c0, EncP* e) {
+    if (a.by_value) {
+        const EncP p = M::prep(a.value_enc[0], a.value_enc[1], a.value_enc[2], a.value_enc[3], a.gc);
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) e[k] = p;
+        return;
+    }
+    float s[VEC], off[VEC], mn[VEC], mx[VEC];
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) off[k] = mn[k] = mx[k] = 0.f;
+    const bool wide = ((reinterpret_cast<uintptr_t>(a.scale) | reinterpret_cast<uintptr_t>(a.offset) |
+                        reinterpret_cast<uintptr_t>(a.emin) | reinterpret_cast<uintptr_t>(a.emax)) & 15) == 0;
+    if (VEC % 4 == 0 && wide) {
+#pragma unroll
+        for (int k = 0; k < VEC; k += 4) {
+            const Pack<float, 4> ps = load_pack<float, 4>(a.scale + c0 + k);
+            Pack<float, 4> po = ps, pn = ps, px = ps;
+            if (a.offset) po = load_pack<float, 4>(a.offset + c0 + k);
+            if (M::kNP > 3 && a.emin) pn = load_pack<float, 4>(a.emin + c0 + k);
+            if (M::kNP > 3 && a.emax) px = load_pack<float, 4>(a.emax + c0 + k);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                s[k + j] = ps.v[j];
+                if (a.offset) off[k + j] = po.v[j];
+                if (M::kNP > 3 && a.emin) mn[k + j] = pn.v[j];
+                if (M::kNP > 3 && a.emax) mx[k + j] = px.v[j];
+            }
+        }
+    } else {
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) {
+            s[k] = a.scale[c0 + k];
+            if (a.offset) off[k] = a.offset[c0 + k];
+            if (M::kNP > 3 && a.emin) mn[k] = a.emin[c0 + k];
+            if (M::kNP > 3 && a.emax) mx[k] = a.emax[c0 + k];
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) e[k] = M::prep(s[k], off[k], mn[k], mx[k], a.gc);
+}
 
 // the division-free form is allowed for this lane's VEC elements of one row
 template <typename IO, int VEC>
@@ -663,9 +705,8 @@ static bool cols_layout(const Plan& p, bool aligned) {
 
 // grid of the column-walking kernels: x over groups of 64 lanes x VEC encodings, y over row groups; about `target`
 // workgroups, every wave with at least one step of rows
-template <typename IO>
-static dim3 cols_grid(const Plan& p, int64_t target, int waves = kColWaves) {
-    constexpr int V = IoTraits<IO>::kVec;
+template <typename IO, int V = IoTraits<IO>::kVec>
+static dim3 cols_grid(const Plan& p, int64_t target, int waves) {
     const int64_t gx = (p.cl.J / V + kWave - 1) / kWave;
     const int64_t row_groups = (p.cl.I + (int64_t)waves * kColUnroll - 1) / ((int64_t)waves * kColUnroll);
     int64_t gy = (target + gx - 1) / gx;

@@ -253,6 +253,36 @@ def test_non_dense_and_misaligned_inputs(device):
         assert_same_bits(y, tr.y, "output")
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_column_kernels_with_encodings_off_16_byte_alignment(device, dtype):
+    """Per-channel encodings along the fastest axis are read as 16-byte vectors when their arrays allow it and one
+    float at a time when a view starts in the middle of such a vector: both must give the same bits, forward and
+    backward."""
+    from aimet_amd.quantization import affine
+
+    g = torch.Generator().manual_seed(11)
+    x = (torch.randn(300, 256, generator=g) * 3).to(dtype).to(device)
+    grad = torch.randn(300, 256, generator=g).to(dtype).to(device)
+    sbuf = (torch.rand(257, generator=g) * 0.04 + 0.01).to(device)
+    obuf = torch.randint(-3, 4, (257,), generator=g).float().to(device)
+    results = []
+    for off_view in (False, True):
+        if off_view:
+            s, o = sbuf[1:], obuf[1:]
+            assert s.data_ptr() % 16 == 4 and s.is_contiguous()
+        else:
+            s, o = sbuf[1:].clone(), obuf[1:].clone()
+            assert s.data_ptr() % 16 == 0
+        s = s.detach().requires_grad_(True)
+        o = o.detach().requires_grad_(True)
+        xi = x.clone().requires_grad_(True)
+        y = affine.quantize_dequantize(xi, s, o, -8, 7)
+        y.backward(grad)
+        results.append((y.detach(), xi.grad, s.grad, o.grad))
+    for name, a, b in zip(("output", "input gradient", "scale gradient", "offset gradient"), *results):
+        assert_same_bits(b, a, name)
+
+
 def test_errors(device):
     from aimet_amd.quantization import affine
 
