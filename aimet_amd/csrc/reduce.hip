@@ -598,30 +598,114 @@ __global__ __launch_bounds__(kBlock) void minmax_generic_kernel(const MmArgs a) 
 }
 
 // Encodings that change with every element (run length 1, e.g. per-channel along the fastest axis): a lane owns VEC
-// neighbouring encodings and walks down the rows of its slab, so loads stay coalesced 16-byte vectors and each lane
-// ends with one pair of atomics per encoding instead of one per element.
-constexpr int kColRows = 64;  // rows per slab
+// neighbouring encodings and walks down rows, so loads stay coalesced 16-byte vectors.  A workgroup is 64 lanes
+// across x kMmColWaves waves down; the waves take rows in turn, kMmColUnroll loads in flight each, and the grid's y
+// axis splits the rows into row groups.  The waves' extrema meet in LDS, the workgroup's go to its row of the
+// partials ([row group][encoding]: no atomics, nothing to clear) and minmax_cols_finish_kernel folds the row groups.
+constexpr int kMmColWaves = 16;
+constexpr int kMmColUnroll = 4;  // even: rows are taken in pairs
 template <typename IO, int VEC, bool FINITE>
-__global__ __launch_bounds__(kBlock) void minmax_cols_kernel(const MmArgs a) {
-    const int64_t c0 = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * VEC;
-    if (c0 >= a.J) return;
-    const int64_t r0 = (int64_t)blockIdx.y * kColRows;
-    const int64_t r1 = r0 + kColRows < a.I ? r0 + kColRows : a.I;
+__global__ __launch_bounds__(kMmColWaves * kWave) void minmax_cols_kernel(const MmArgs a, int stream_loads) {
+    constexpr int kHalf = kMmColWaves / 2;  // the upper half of the waves hands over to the lower half first
+    __shared__ float smn[kHalf][kWave * VEC], smx[kHalf][kWave * VEC];
+    __shared__ unsigned char snan[kHalf][kWave * VEC];
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int64_t cbase = (int64_t)blockIdx.x * kWave * VEC;  // first column of the workgroup
+    const int64_t c0 = cbase + (int64_t)lane * VEC;
     const IO* __restrict__ x = static_cast<const IO*>(a.x);
     MinMax m[VEC];
 #pragma unroll
     for (int k = 0; k < VEC; ++k) m[k] = mm_identity();
-#pragma unroll 4
-    for (int64_t r = r0; r < r1; ++r) {
-        const Pack<IO, VEC> pk = load_pack_stream<IO, VEC>(x + r * a.J + c0);
+    if (c0 < a.J) {
+        // NaN is looked for with one unordered comparison per pair of rows; the comparison's lane mask is OR-ed on the
+        // scalar unit, one mask per encoding of the lane (see mm_pack)
+        uint64_t unordered[VEC];
 #pragma unroll
-        for (int k = 0; k < VEC; ++k) mm_add(m[k], load_f32(pk.v[k]), FINITE);
+        for (int k = 0; k < VEC; ++k) unordered[k] = 0;
+        const int64_t step = (int64_t)gridDim.y * kMmColWaves * kMmColUnroll;
+        for (int64_t r0 = ((int64_t)blockIdx.y * kMmColWaves + wave) * kMmColUnroll; r0 < a.I; r0 += step) {
+            Pack<IO, VEC> pk[kMmColUnroll];
+#pragma unroll
+            for (int u = 0; u < kMmColUnroll; ++u) {
+                // rows past the end are read as the step's first row again: extrema do not mind
+                const int64_t r = r0 + u < a.I ? r0 + u : r0;
+                pk[u] = stream_loads ? load_pack_stream<IO, VEC>(x + r * a.J + c0) : load_pack<IO, VEC>(x + r * a.J + c0);
+            }
+#pragma unroll
+            for (int u = 0; u < kMmColUnroll; u += 2) {
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) {
+                    const float f0 = load_f32(pk[u].v[k]), f1 = load_f32(pk[u + 1].v[k]);
+                    if (FINITE) {
+                        mm_add(m[k], f0, true);
+                        mm_add(m[k], f1, true);
+                    } else {
+                        m[k].mn = fminf(fminf(m[k].mn, f0), f1);
+                        m[k].mx = fmaxf(fmaxf(m[k].mx, f0), f1);
+                        unordered[k] |= __builtin_amdgcn_ballot_w64(__builtin_isunordered(f0, f1));
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) m[k].nan = (int)((unordered[k] >> lane) & 1);
     }
+    if (wave >= kHalf) {
 #pragma unroll
-    for (int k = 0; k < VEC; ++k) {
-        atomicMin(&a.key_min[c0 + k], f32_key(m[k].mn));
-        atomicMax(&a.key_max[c0 + k], f32_key(m[k].mx));
-        if (m[k].nan) atomicOr(&a.part_nan[c0 + k], 1);
+        for (int k = 0; k < VEC; ++k) {
+            smn[wave - kHalf][lane * VEC + k] = m[k].mn;
+            smx[wave - kHalf][lane * VEC + k] = m[k].mx;
+            snan[wave - kHalf][lane * VEC + k] = (unsigned char)m[k].nan;
+        }
+    }
+    __syncthreads();
+    if (wave < kHalf) {
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) {
+            const int c = lane * VEC + k;
+            m[k] = mm_merge(m[k], MinMax{smn[wave][c], smx[wave][c], snan[wave][c]});
+            smn[wave][c] = m[k].mn;
+            smx[wave][c] = m[k].mx;
+            snan[wave][c] = (unsigned char)m[k].nan;
+        }
+    }
+    __syncthreads();
+    // a thread per column of the workgroup: neighbouring threads read neighbouring LDS words and store neighbouring
+    // partials
+    for (int c = threadIdx.x; c < kWave * VEC; c += kMmColWaves * kWave) {
+        if (cbase + c >= a.J) break;
+        MinMax r = mm_identity();
+#pragma unroll
+        for (int w = 0; w < kHalf; ++w) r = mm_merge(r, MinMax{smn[w][c], smx[w][c], snan[w][c]});
+        const int64_t slot = (int64_t)blockIdx.y * a.J + cbase + c;
+        a.part_min[slot] = r.mn;
+        a.part_max[slot] = r.mx;
+        a.part_nan[slot] = r.nan;
+    }
+}
+
+// Folds the row groups of minmax_cols_kernel: a lane per encoding (coalesced reads), the waves of a workgroup take
+// the row groups in turn and meet in LDS.
+constexpr int kMmColFinishWaves = 4;
+template <typename IO>
+__global__ __launch_bounds__(kMmColFinishWaves * kWave) void minmax_cols_finish_kernel(const MmArgs a, int groups) {
+    __shared__ MinMax shares[kMmColFinishWaves][kWave];
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int64_t e = (int64_t)blockIdx.x * kWave + lane;
+    MinMax r = mm_identity();
+    if (e < a.J) {
+#pragma unroll 4
+        for (int q = wave; q < groups; q += kMmColFinishWaves) {
+            const int64_t slot = (int64_t)q * a.J + e;
+            r = mm_merge(r, MinMax{a.part_min[slot], a.part_max[slot], a.part_nan[slot]});
+        }
+    }
+    shares[wave][lane] = r;
+    __syncthreads();
+    if (wave == 0 && e < a.J) {
+#pragma unroll
+        for (int w = 1; w < kMmColFinishWaves; ++w) r = mm_merge(r, shares[w][lane]);
+        mm_write<IO>(a, e, r);
     }
 }
 
@@ -658,6 +742,26 @@ static size_t mm_ws_elems(const Plan& p) {
     return p.ws_elems;
 }
 
+// The column-walking kernel applies: run length 1 over several rows, whole 16-byte vectors per row.
+static bool mm_cols_layout(int io_dtype, const Plan& p) {
+    const int V = io_vec(io_dtype);
+    return p.ptr_aligned && p.cl.kind == kIJK && p.red == kRedAtomic && p.cl.K == 1 && p.cl.I > 1 && p.cl.J % V == 0 &&
+           p.cl.J / V >= kWave / 2 && (p.cl.J / V + kWave - 1) / kWave <= 0x7fffffff;
+}
+
+// Row groups the column-walking kernel would like (about 256 workgroups of sixteen waves, four waves per SIMD of 256
+// CUs, every wave at least one step of rows: 8192 x 4096 bf16 17.9 us, 18.6 us with 512 workgroups, 21.4 us with 1024;
+// fp32 25.9 / 27.5 / 27.7 us) and the partial triples they need.  The workspace every reduction of this layout needs
+// is one row of partials (12 bytes per encoding); with less than the preferred size the kernel runs with as many row
+// groups as fit.
+static int64_t mm_cols_row_groups(int io_dtype, const Plan& p) {
+    const int64_t gx = (p.cl.J / io_vec(io_dtype) + kWave - 1) / kWave;
+    const int64_t most = (p.cl.I + kMmColWaves * kMmColUnroll - 1) / (kMmColWaves * kMmColUnroll);
+    int64_t gy = (256 + gx - 1) / gx;
+    gy = gy > most ? most : gy;
+    return gy < 1 ? 1 : (gy > 65535 ? 65535 : gy);
+}
+
 static MmFlatArgs flat_args(const Plan& p, const MmArgs& a) {
     MmFlatArgs f{};
     static_cast<MmOut&>(f) = static_cast<const MmOut&>(a);
@@ -673,7 +777,7 @@ static MmFlatArgs flat_args(const Plan& p, const MmArgs& a) {
 }
 
 template <typename IO, bool FINITE>
-static void launch_mm(const Plan& p, const MmArgs& a, hipStream_t st) {
+static void launch_mm(const Plan& p, const MmArgs& a, hipStream_t st, int cols_groups) {
     const int64_t ne = p.cl.num_enc;
     const unsigned gb = (unsigned)((ne + 255) / 256 > 1024 ? 1024 : (ne + 255) / 256);
     if (p.cl.kind == kIJK && p.cl.J == 1) {
@@ -720,6 +824,15 @@ static void launch_mm(const Plan& p, const MmArgs& a, hipStream_t st) {
             return;
         }
     }
+    if (cols_groups > 0) {
+        constexpr int V = IoTraits<IO>::kVec;
+        const dim3 g((unsigned)((p.cl.J / V + kWave - 1) / kWave), (unsigned)cols_groups);
+        const int stream_loads = p.cl.numel * (int64_t)sizeof(IO) >= kStreamLoadBytes ? 1 : 0;
+        hipLaunchKernelGGL((minmax_cols_kernel<IO, V, FINITE>), g, dim3(kMmColWaves * kWave), 0, st, a, stream_loads);
+        hipLaunchKernelGGL((minmax_cols_finish_kernel<IO>), dim3((unsigned)((p.cl.J + kWave - 1) / kWave)),
+                           dim3(kMmColFinishWaves * kWave), 0, st, a, cols_groups);
+        return;
+    }
     if (p.red == kRedAtomic) hipLaunchKernelGGL(minmax_keys_init_kernel, dim3(gb), dim3(256), 0, st, a.key_min, a.key_max, a.part_nan, ne);
     if (p.cl.kind == kGeneric) {
         hipLaunchKernelGGL((minmax_generic_kernel<IO>), dim3(p.nblocks), dim3(kBlock), 0, st, a);
@@ -733,11 +846,6 @@ static void launch_mm(const Plan& p, const MmArgs& a, hipStream_t st) {
         }
     } else if (p.red == kRedSeg) {
         launch_mm_red<IO, kRedSeg, FINITE>(p, a, st);
-    } else if (p.cl.K == 1 && p.cl.J % IoTraits<IO>::kVec == 0 && p.cl.J / IoTraits<IO>::kVec >= kWave / 2 && aligned16(a.x) && p.cl.I > 1 &&
-               (p.cl.I + kColRows - 1) / kColRows <= 65535) {
-        constexpr int V = IoTraits<IO>::kVec;
-        const dim3 g((unsigned)((p.cl.J / V + kBlock - 1) / kBlock), (unsigned)((p.cl.I + kColRows - 1) / kColRows));
-        hipLaunchKernelGGL((minmax_cols_kernel<IO, V, FINITE>), g, dim3(kBlock), 0, st, a);
     } else {
         launch_mm_red<IO, kRedAtomic, FINITE>(p, a, st);
     }
@@ -801,7 +909,10 @@ extern "C" size_t ahq_minmax_workspace_bytes(const ahq_layout* layout) {
     for (int dt = AHQ_F32; dt <= AHQ_BF16; ++dt)
         for (int al = 0; al < 2; ++al) {
             Plan p;
-            if (make_plan(dt, *layout, al != 0, true, &p) && mm_ws_elems(p) * 12 > need) need = mm_ws_elems(p) * 12;
+            if (!make_plan(dt, *layout, al != 0, true, &p)) continue;
+            size_t n = mm_ws_elems(p) * 12;
+            if (mm_cols_layout(dt, p)) n = (size_t)mm_cols_row_groups(dt, p) * (size_t)p.cl.J * 12;  // the preferred size
+            if (n > need) need = n;
         }
     return need;
 }
@@ -831,13 +942,21 @@ static int minmax_impl(int32_t dtype, const ahq_layout* layout, const void* x, v
     a.run_min = run_min;
     a.run_max = run_max;
     a.finite_only = finite_only;
+    int cols_groups = 0;  // > 0: the column-walking kernel with that many row groups
     if (uses_ws) {
+        size_t slots = ws_elems;
+        if (mm_cols_layout(dtype, p)) {
+            const int64_t fit = (int64_t)(workspace_bytes / ((size_t)p.cl.J * 12));
+            const int64_t want = mm_cols_row_groups(dtype, p);
+            cols_groups = (int)(fit < want ? fit : want);
+            slots = (size_t)cols_groups * (size_t)p.cl.J;
+        }
         char* w = static_cast<char*>(workspace);
         a.part_min = reinterpret_cast<float*>(w);
-        a.part_max = reinterpret_cast<float*>(w + ws_elems * 4);
-        a.part_nan = reinterpret_cast<int*>(w + ws_elems * 8);
+        a.part_max = reinterpret_cast<float*>(w + slots * 4);
+        a.part_nan = reinterpret_cast<int*>(w + slots * 8);
         a.key_min = reinterpret_cast<unsigned int*>(w);
-        a.key_max = reinterpret_cast<unsigned int*>(w + ws_elems * 4);
+        a.key_max = reinterpret_cast<unsigned int*>(w + slots * 4);
     }
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (copy) {
@@ -848,7 +967,7 @@ static int minmax_impl(int32_t dtype, const ahq_layout* layout, const void* x, v
             return set_error("device-to-device copy failed"), AHQ_ERR_LAUNCH;
         }
     }
-#define AHQ_MM(IO) do { if (finite_only == 1) launch_mm<IO, true>(p, a, st); else launch_mm<IO, false>(p, a, st); } while (0)
+#define AHQ_MM(IO) do { if (finite_only == 1) launch_mm<IO, true>(p, a, st, cols_groups); else launch_mm<IO, false>(p, a, st, cols_groups); } while (0)
     switch (dtype) {
         case AHQ_F32: AHQ_MM(float); break;
         case AHQ_F16: AHQ_MM(f16_t); break;

@@ -120,6 +120,7 @@ struct Plan {
     int tile_vec;  // vectors per tile
     int64_t ntiles;
     size_t ws_elems;  // kRedTile: number of tiles; kRedAtomic: number of encodings; kRedRuns: runs if I > 1; else 0
+    bool ptr_aligned; // what the caller said of its pointers: all 16-byte aligned
 };
 
 inline int io_vec(int dtype) { return dtype == AHQ_F32 ? 4 : 8; }
@@ -135,6 +136,7 @@ inline bool make_plan(int io_dtype, const ahq_layout& layout, bool ptr_aligned, 
                       int unroll = kUnroll, bool ordered = false) {
     const int tile_vec = kBlock * unroll;
     p->tile_vec = tile_vec;
+    p->ptr_aligned = ptr_aligned;
     const char* err = nullptr;
     if (!canonicalize(layout, &p->cl, &err)) {
         set_error(err);

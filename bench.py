@@ -277,7 +277,17 @@ def _make_c4():
                 bitwidth=4, symmetric=True, lpbq=True, decompressed_bw=8, grouping=(1, -1))
 
 
-WORKLOADS = {"c1": _make_c1, "c2": _make_c2, "c4": _make_c4}
+def _make_cols():
+    """Not one of the benchmark configurations: per-channel encodings along the fastest axis, the layout the
+    column-walking kernels serve (run with --workload cols; left out of the default run)."""
+    g = torch.Generator().manual_seed(0)
+    x = (torch.randn(8192, 4096, generator=g) * torch.linspace(0.5, 2.0, 4096)).bfloat16()
+    grad = torch.randn(8192, 4096, generator=torch.Generator().manual_seed(1)).bfloat16()
+    return dict(name="per_column_8b_sym_bf16_8192x4096", x=x, grad=grad, enc_shape=(1, 4096), block=None,
+                bitwidth=8, symmetric=True, lpbq=False)
+
+
+WORKLOADS = {"c1": _make_c1, "c2": _make_c2, "c4": _make_c4, "cols": _make_cols}
 
 
 def _grid_limits(w):
@@ -1284,6 +1294,7 @@ RUNNERS = {
     "c1": lambda a, dev, cpu: run_qdq_workload("c1", a.steps, a.warmup, dev, cpu, not a.no_cached),
     "c2": lambda a, dev, cpu: run_qdq_workload("c2", a.steps, a.warmup, dev, cpu, not a.no_cached),
     "c4": lambda a, dev, cpu: run_qdq_workload("c4", a.steps, a.warmup, dev, cpu, not a.no_cached),
+    "cols": lambda a, dev, cpu: run_qdq_workload("cols", a.steps, a.warmup, dev, cpu, not a.no_cached),
     "c3": lambda a, dev, cpu: run_hist_workload(min(a.steps, 10), min(a.warmup, 2), dev, cpu),
     "dlq": lambda a, dev, cpu: run_dlq_workload(min(a.steps, 10), min(a.warmup, 2), dev, cpu),
     "c5": lambda a, dev, cpu: run_model_workload(min(a.steps, 3), min(a.warmup, 1), dev, cpu),

@@ -150,8 +150,10 @@ int    ahq_minmax_copy(int32_t dtype, const ahq_layout* layout, const void* x, v
  * device array of AHQ_MINMAX_STATIC_SCRATCH_BYTES that every device the library runs on holds until the process ends.
  * The call allocates nothing (no hipMalloc / hipFree, no allocating library routine); the first call on a device
  * looks the array's address up (hipGetSymbolAddress), so make that call outside a capture.
- * A reduction whose ahq_minmax_workspace_bytes() exceeds the array returns AHQ_ERR_WORKSPACE and launches nothing
- * (a per-tensor reduction needs 6 KB whatever its size; others 12 bytes per encoding or per tile).
+ * A reduction that needs more scratch than the array holds returns AHQ_ERR_WORKSPACE and launches nothing (a
+ * per-tensor reduction needs 6 KB whatever its size; others 12 bytes per encoding or per tile; per-channel along the
+ * fastest axis needs 12 bytes per encoding and uses more when it is there, which is what
+ * ahq_minmax_workspace_bytes() reports for that layout).
  * All calls on one device share the array: calls that overlap on one device (different streams) race; calls on one
  * stream are ordered and each clears what it needs.
  */

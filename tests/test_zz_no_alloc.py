@@ -46,7 +46,10 @@ CASES = [
     ("per_channel_rows", (48, 9000), (16, 5000), (48, 1), (16, 1), None),  # one partial per tile of each row
     ("per_channel_short_rows", (300, 100), (40, 100), (300, 1), (40, 1), None),  # ordered keys + atomics
     ("blockwise", (64, 1024), (8, 256), (64, 16), (8, 4), (1, 64)),     # shuffle reduction, no scratch at all
-    ("columns", (700, 512), (90, 256), (512,), (256,), None),           # column walk: keys per encoding
+    ("columns", (700, 512), (90, 256), (512,), (256,), None),           # column walk: a row of partials per row group
+    # column walk whose preferred scratch (8 row groups x 16384 x 12 bytes for the 16-bit dtypes) is more than the
+    # static array holds: that entry point runs it with the 5 row groups that fit
+    ("wide_columns", (600, 16384), (90, 256), (16384,), (256,), None),
 ]
 
 
@@ -72,6 +75,19 @@ def test_static_scratch_matches_the_workspace_entry_point(device, dtype, case, f
         if finite_only == 1 and enc == ():
             fin = x[x.isfinite()]
             assert smn.item() == fin.min().item() and smx.item() == fin.max().item()
+
+
+def test_column_walk_prefers_more_scratch_than_it_needs():
+    """Host-side: for per-channel along the fastest axis the workspace query reports the preferred size, the static
+    entry point accepts the layout as long as one row of partials fits."""
+    lib = _lib.load()
+    lay = _lib.make_layout([600, 16384], [600, 1], [0, 1])
+    assert lib.ahq_minmax_workspace_bytes(lay) == 8 * 16384 * 12 > SCRATCH_BYTES
+    # accepted for its size: the null pointers are what this call is refused for
+    assert lib.ahq_minmax_static(_lib.AHQ_BF16, lay, None, None, None, None, None, 0, None) == _lib.AHQ_ERR_INVALID
+    cols = SCRATCH_BYTES // 12 + 8
+    lay = _lib.make_layout([600, cols], [600, 1], [0, 1])
+    assert lib.ahq_minmax_static(_lib.AHQ_BF16, lay, 16, 16, 16, None, None, 0, None) == _lib.AHQ_ERR_WORKSPACE
 
 
 @pytest.mark.gpu
