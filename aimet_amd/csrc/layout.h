@@ -7,7 +7,10 @@
 //   IJK      flat index = (i*J + j)*K + k  and encoding index = j      (I, J, K >= 1)
 //            per-tensor is J == 1; per-channel on the leading axis is I == 1; blocks along the fastest axis
 //            with one row of blocks per leading coordinate collapse to I == 1, J = #blocks, K = block size
-//   GENERIC  anything else (2-D blocks, several channel axes): per-element coordinate walk
+//   GENERIC  anything else (2-D blocks, several channel axes): per-element coordinate walk.  One generic form is also
+//            described as STACKED COLUMNS: flat index = (a*I + i)*J + j and encoding index = a*J + j  (A > 1: blocks
+//            along a leading axis with one encoding per element of the fastest axis), which the column-walking
+//            kernels take as A problems of the IJK form with K == 1
 #pragma once
 
 #include <cstdint>
@@ -30,6 +33,8 @@ struct CanonLayout {
     int64_t num_enc = 1;
     // IJK form
     int64_t I = 1, J = 1, K = 1;
+    // stacked columns (kind == kGeneric and A > 1): I, J as above, K == 1
+    int64_t A = 1;
     // generic form: segments outermost first, with the flat stride of each
     int32_t nseg = 0;
     int64_t seg_extent[2 * AHQ_MAX_DIMS];
@@ -132,10 +137,16 @@ inline bool canonicalize(const ahq_layout& in, CanonLayout* out, const char** er
             out->seg_flat_stride[i] = stride;
             stride *= merged[i].extent;
         }
+        if (m == 3 && !is_b(0) && is_b(1) && !is_b(2) && merged[2].enc_stride == 1 &&
+            merged[0].enc_stride == merged[2].extent) {
+            out->A = merged[0].extent;
+            out->I = merged[1].extent;
+            out->J = merged[2].extent;
+        }
     }
     if (numel == 0) {
         out->kind = kIJK;
-        out->I = out->J = 1;
+        out->A = out->I = out->J = 1;
         out->K = 0;
     }
     return true;

@@ -90,7 +90,7 @@ __global__ __launch_bounds__(kBlock) void qdq_fwd_lpbq_kernel(const QdqArgs a, c
 
 template <typename IO, int VEC, typename M, bool FAST>
 __device__ __forceinline__ void fwd_cols_rows(const QdqArgs& a, const Pack<IO, VEC>* in, const EncP* e, IO* __restrict__ y,
-                                              int64_t r0, int64_t c0) {
+                                              uint8_t* __restrict__ mask, int64_t r0, int64_t c0) {
 #pragma unroll
     for (int u = 0; u < kColUnroll; ++u) {
         if (r0 + u >= a.I) continue;
@@ -104,7 +104,7 @@ __device__ __forceinline__ void fwd_cols_rows(const QdqArgs& a, const Pack<IO, V
             mk.v[k] = inr ? 1 : 0;
         }
         store_pack_stream<IO, VEC>(y + (r0 + u) * a.J + c0, out);
-        if (a.mask) store_pack_stream<uint8_t, VEC>(a.mask + (r0 + u) * a.J + c0, mk);
+        if (mask) store_pack_stream<uint8_t, VEC>(mask + (r0 + u) * a.J + c0, mk);
     }
 }
 
@@ -113,11 +113,13 @@ __global__ __launch_bounds__(WAVES * kWave) void qdq_fwd_cols_kernel(const QdqAr
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     const int64_t c0 = ((int64_t)blockIdx.x * kWave + lane) * VEC;
     if (c0 >= a.J) return;
-    const IO* __restrict__ x = static_cast<const IO*>(a.x);
-    IO* __restrict__ y = static_cast<IO*>(a.y);
+    const int64_t z = blockIdx.z;  // stacked columns: problem z has its own I x J elements and J encodings
+    const IO* __restrict__ x = static_cast<const IO*>(a.x) + z * a.I * a.J;
+    IO* __restrict__ y = static_cast<IO*>(a.y) + z * a.I * a.J;
+    uint8_t* __restrict__ mask = a.mask ? a.mask + z * a.I * a.J : nullptr;
     EncP e[VEC];
     bool enc_fast = true;
-    load_col_encodings<M, VEC>(a, c0, e);
+    load_col_encodings<M, VEC>(a, z * a.J + c0, e);
 #pragma unroll
     for (int k = 0; k < VEC; ++k) enc_fast &= !M::kDiv || e[k].rs != 0.f;
     const int64_t step = (int64_t)gridDim.y * WAVES * kColUnroll;
@@ -133,8 +135,8 @@ __global__ __launch_bounds__(WAVES * kWave) void qdq_fwd_cols_kernel(const QdqAr
         // wave-uniform, like the tiled kernel: one branch per step, and each side a straight run of arithmetic over
         // all its elements (a choice per element costs a branch per element and keeps the compiler from interleaving
         // the elements' instruction chains)
-        if (!M::kDiv || __builtin_amdgcn_ballot_w64(!ok) == 0) fwd_cols_rows<IO, VEC, M, true>(a, in, e, y, r0, c0);
-        else fwd_cols_rows<IO, VEC, M, false>(a, in, e, y, r0, c0);
+        if (!M::kDiv || __builtin_amdgcn_ballot_w64(!ok) == 0) fwd_cols_rows<IO, VEC, M, true>(a, in, e, y, mask, r0, c0);
+        else fwd_cols_rows<IO, VEC, M, false>(a, in, e, y, mask, r0, c0);
     }
 }
 

@@ -348,6 +348,10 @@ __global__ __launch_bounds__(kRowsFinishWaves * kWave) void qdq_bwd_rows_finish_
     __shared__ double shares[kRowsFinishWaves][2][kWave];
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     const int64_t e = (int64_t)blockIdx.x * kWave + lane;
+    // stacked problems (the grid's y axis): each has its own `count` rows of partials and its own num_enc results
+    partials += 2 * (int64_t)blockIdx.y * count * num_enc;
+    gscale += (int64_t)blockIdx.y * num_enc;
+    goffset += (int64_t)blockIdx.y * num_enc;
     const int64_t share = (count + kRowsFinishWaves - 1) / kRowsFinishWaves;
     const int64_t q0 = wave * share, q1 = q0 + share < count ? q0 + share : count;
     double s = 0.0, o = 0.0;
@@ -515,12 +519,13 @@ __global__ __launch_bounds__(WAVES * kWave) void qdq_bwd_cols_kernel(const QdqAr
         for (int i = 0; i < 2 * VEC; ++i) sums[wave][i][lane] = 0.0;
     }
     if (live) {
-        const IO* __restrict__ x = static_cast<const IO*>(a.x);
-        const IO* __restrict__ g = static_cast<const IO*>(a.g);
-        IO* __restrict__ gxp = static_cast<IO*>(a.gx);
+        const int64_t zoff = (int64_t)blockIdx.z * a.I * a.J;  // stacked columns: problem z has its own I x J elements
+        const IO* __restrict__ x = static_cast<const IO*>(a.x) + zoff;
+        const IO* __restrict__ g = static_cast<const IO*>(a.g) + zoff;
+        IO* __restrict__ gxp = a.gx ? static_cast<IO*>(a.gx) + zoff : nullptr;
         EncP e[VEC];
         bool enc_fast = true;
-        load_col_encodings<M, VEC>(a, c0, e);
+        load_col_encodings<M, VEC>(a, (int64_t)blockIdx.z * a.J + c0, e);
 #pragma unroll
         for (int k = 0; k < VEC; ++k) enc_fast &= !M::kDiv || e[k].rs != 0.f;
         float vs[VEC], vo[VEC];
@@ -558,7 +563,7 @@ __global__ __launch_bounds__(WAVES * kWave) void qdq_bwd_cols_kernel(const QdqAr
     __syncthreads();
     // the tables are added up in wave order, whichever wave finished first; the 2 * VEC sums of a lane are shared out
     // over the waves, and a lane's pair of sums for one encoding is one 16-byte store
-    double* row = a.partials + 2 * (int64_t)blockIdx.y * a.J;
+    double* row = a.partials + 2 * ((int64_t)blockIdx.z * gridDim.y + blockIdx.y) * a.J;
     for (int k = wave; k < VEC; k += WAVES) {
         if (!live) break;
         double ps = 0.0, po = 0.0;
@@ -567,7 +572,13 @@ __global__ __launch_bounds__(WAVES * kWave) void qdq_bwd_cols_kernel(const QdqAr
             ps += sums[w][2 * k][lane];
             po += sums[w][2 * k + 1][lane];
         }
-        store_pack<double, 2>(row + 2 * (c0 + k), Pack<double, 2>{{ps, po}});
+        if (gridDim.y == 1) {  // a single row group: these are the sums themselves, no finish launch follows
+            const int64_t enc = (int64_t)blockIdx.z * a.J + c0 + k;
+            a.gscale[enc] = finish_sum_rt(ps, a.out_cd);
+            a.goffset[enc] = finish_sum_rt(po, a.out_cd);
+        } else {
+            store_pack<double, 2>(row + 2 * (c0 + k), Pack<double, 2>{{ps, po}});
+        }
     }
 }
 
@@ -614,7 +625,7 @@ static unsigned bwd_cols_row_groups(int io_dtype, const Plan& p) {
 // pairs of doubles the backward pass needs as scratch for its parameter gradients
 static size_t bwd_scratch_pairs(int io_dtype, const Plan& p, bool aligned, bool want_pg) {
     if (!want_pg) return 0;
-    if (bwd_cols_layout(io_dtype, p, aligned)) return (size_t)bwd_cols_row_groups(io_dtype, p) * (size_t)p.cl.J;
+    if (bwd_cols_layout(io_dtype, p, aligned)) return (size_t)p.cl.A * (size_t)bwd_cols_row_groups(io_dtype, p) * (size_t)p.cl.J;
     return p.ws_elems;
 }
 
@@ -739,11 +750,13 @@ extern "C" int ahq_qdq_backward(const ahq_grid* grid, const ahq_layout* layout, 
         hipLaunchKernelGGL(finish_atomic_kernel, dim3((unsigned)((n + 255) / 256 > 1024 ? 1024 : (n + 255) / 256)), dim3(256), 0, st,
                            (const double*)a.partials, gscale, goffset, n, (int)grid->compute_dtype);
     }
-    if (want_pg && (cols || (p.red == kRedRuns && p.cl.I > 1))) {
-        // one slot per (row group, encoding) or per run: added up per encoding in a fixed order
-        const int64_t count = cols ? (int64_t)bwd_cols_row_groups(grid->io_dtype, p) : p.cl.I;
+    const int64_t col_groups = cols ? (int64_t)bwd_cols_row_groups(grid->io_dtype, p) : 0;
+    if (want_pg && ((cols && col_groups > 1) || (!cols && p.red == kRedRuns && p.cl.I > 1))) {
+        // one slot per (row group, encoding) or per run: added up per encoding in a fixed order (the column kernel
+        // with a single row group has stored the sums itself)
+        const int64_t count = cols ? col_groups : p.cl.I;
         if (p.cl.J >= kWave / 2 && (p.cl.J + kWave - 1) / kWave <= 0x7fffffff) {
-            hipLaunchKernelGGL(qdq_bwd_rows_finish_kernel, dim3((unsigned)((p.cl.J + kWave - 1) / kWave)),
+            hipLaunchKernelGGL(qdq_bwd_rows_finish_kernel, dim3((unsigned)((p.cl.J + kWave - 1) / kWave), cols ? (unsigned)p.cl.A : 1u),
                                dim3(kRowsFinishWaves * kWave), 0, st, (const double*)a.partials, count, p.cl.J, gscale, goffset,
                                (int)grid->compute_dtype);
         } else {

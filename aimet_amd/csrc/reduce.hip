@@ -612,7 +612,8 @@ __global__ __launch_bounds__(kMmColWaves * kWave) void minmax_cols_kernel(const 
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     const int64_t cbase = (int64_t)blockIdx.x * kWave * VEC;  // first column of the workgroup
     const int64_t c0 = cbase + (int64_t)lane * VEC;
-    const IO* __restrict__ x = static_cast<const IO*>(a.x);
+    // stacked columns: problem blockIdx.z has its own I x J elements, J encodings and gridDim.y rows of partials
+    const IO* __restrict__ x = static_cast<const IO*>(a.x) + (int64_t)blockIdx.z * a.I * a.J;
     MinMax m[VEC];
 #pragma unroll
     for (int k = 0; k < VEC; ++k) m[k] = mm_identity();
@@ -677,7 +678,11 @@ __global__ __launch_bounds__(kMmColWaves * kWave) void minmax_cols_kernel(const 
         MinMax r = mm_identity();
 #pragma unroll
         for (int w = 0; w < kHalf; ++w) r = mm_merge(r, MinMax{smn[w][c], smx[w][c], snan[w][c]});
-        const int64_t slot = (int64_t)blockIdx.y * a.J + cbase + c;
+        if (gridDim.y == 1) {  // a single row group: these are the extrema themselves, no finish launch follows
+            mm_write<IO>(a, (int64_t)blockIdx.z * a.J + cbase + c, r);
+            continue;
+        }
+        const int64_t slot = ((int64_t)blockIdx.z * gridDim.y + blockIdx.y) * a.J + cbase + c;
         a.part_min[slot] = r.mn;
         a.part_max[slot] = r.mx;
         a.part_nan[slot] = r.nan;
@@ -696,7 +701,7 @@ __global__ __launch_bounds__(kMmColFinishWaves * kWave) void minmax_cols_finish_
     if (e < a.J) {
 #pragma unroll 4
         for (int q = wave; q < groups; q += kMmColFinishWaves) {
-            const int64_t slot = (int64_t)q * a.J + e;
+            const int64_t slot = ((int64_t)blockIdx.y * groups + q) * a.J + e;
             r = mm_merge(r, MinMax{a.part_min[slot], a.part_max[slot], a.part_nan[slot]});
         }
     }
@@ -705,7 +710,7 @@ __global__ __launch_bounds__(kMmColFinishWaves * kWave) void minmax_cols_finish_
     if (wave == 0 && e < a.J) {
 #pragma unroll
         for (int w = 1; w < kMmColFinishWaves; ++w) r = mm_merge(r, shares[w][lane]);
-        mm_write<IO>(a, e, r);
+        mm_write<IO>(a, (int64_t)blockIdx.y * a.J + e, r);  // blockIdx.y: the stacked problem
     }
 }
 
@@ -745,7 +750,8 @@ static size_t mm_ws_elems(const Plan& p) {
 // The column-walking kernel applies: run length 1 over several rows, whole 16-byte vectors per row.
 static bool mm_cols_layout(int io_dtype, const Plan& p) {
     const int V = io_vec(io_dtype);
-    return p.ptr_aligned && p.cl.kind == kIJK && p.red == kRedAtomic && p.cl.K == 1 && p.cl.I > 1 && p.cl.J % V == 0 &&
+    const bool form = p.cl.kind == kIJK || (p.cl.kind == kGeneric && p.cl.A > 1 && p.cl.A <= 65535);  // stacked: z axis
+    return p.ptr_aligned && form && p.red == kRedAtomic && p.cl.K == 1 && p.cl.I > 1 && p.cl.J % V == 0 &&
            p.cl.J / V >= kWave / 2 && (p.cl.J / V + kWave - 1) / kWave <= 0x7fffffff;
 }
 
@@ -757,7 +763,7 @@ static bool mm_cols_layout(int io_dtype, const Plan& p) {
 static int64_t mm_cols_row_groups(int io_dtype, const Plan& p) {
     const int64_t gx = (p.cl.J / io_vec(io_dtype) + kWave - 1) / kWave;
     const int64_t most = (p.cl.I + kMmColWaves * kMmColUnroll - 1) / (kMmColWaves * kMmColUnroll);
-    int64_t gy = (256 + gx - 1) / gx;
+    int64_t gy = (256 + gx * p.cl.A - 1) / (gx * p.cl.A);
     gy = gy > most ? most : gy;
     return gy < 1 ? 1 : (gy > 65535 ? 65535 : gy);
 }
@@ -826,10 +832,11 @@ static void launch_mm(const Plan& p, const MmArgs& a, hipStream_t st, int cols_g
     }
     if (cols_groups > 0) {
         constexpr int V = IoTraits<IO>::kVec;
-        const dim3 g((unsigned)((p.cl.J / V + kWave - 1) / kWave), (unsigned)cols_groups);
+        const dim3 g((unsigned)((p.cl.J / V + kWave - 1) / kWave), (unsigned)cols_groups, (unsigned)p.cl.A);
         const int stream_loads = p.cl.numel * (int64_t)sizeof(IO) >= kStreamLoadBytes ? 1 : 0;
         hipLaunchKernelGGL((minmax_cols_kernel<IO, V, FINITE>), g, dim3(kMmColWaves * kWave), 0, st, a, stream_loads);
-        hipLaunchKernelGGL((minmax_cols_finish_kernel<IO>), dim3((unsigned)((p.cl.J + kWave - 1) / kWave)),
+        if (cols_groups > 1)
+            hipLaunchKernelGGL((minmax_cols_finish_kernel<IO>), dim3((unsigned)((p.cl.J + kWave - 1) / kWave), (unsigned)p.cl.A),
                            dim3(kMmColFinishWaves * kWave), 0, st, a, cols_groups);
         return;
     }
@@ -911,7 +918,7 @@ extern "C" size_t ahq_minmax_workspace_bytes(const ahq_layout* layout) {
             Plan p;
             if (!make_plan(dt, *layout, al != 0, true, &p)) continue;
             size_t n = mm_ws_elems(p) * 12;
-            if (mm_cols_layout(dt, p)) n = (size_t)mm_cols_row_groups(dt, p) * (size_t)p.cl.J * 12;  // the preferred size
+            if (mm_cols_layout(dt, p)) n = (size_t)p.cl.A * (size_t)mm_cols_row_groups(dt, p) * (size_t)p.cl.J * 12;  // the preferred size
             if (n > need) need = n;
         }
     return need;
@@ -946,10 +953,10 @@ static int minmax_impl(int32_t dtype, const ahq_layout* layout, const void* x, v
     if (uses_ws) {
         size_t slots = ws_elems;
         if (mm_cols_layout(dtype, p)) {
-            const int64_t fit = (int64_t)(workspace_bytes / ((size_t)p.cl.J * 12));
+            const int64_t fit = (int64_t)(workspace_bytes / ((size_t)p.cl.A * (size_t)p.cl.J * 12));
             const int64_t want = mm_cols_row_groups(dtype, p);
             cols_groups = (int)(fit < want ? fit : want);
-            slots = (size_t)cols_groups * (size_t)p.cl.J;
+            slots = (size_t)p.cl.A * (size_t)cols_groups * (size_t)p.cl.J;
         }
         char* w = static_cast<char*>(workspace);
         a.part_min = reinterpret_cast<float*>(w);

@@ -27,6 +27,8 @@ CASES = [
     ((3, 5), (3, 5), None),
     ((200, 2056), (2056,), None),          # one encoding per element of the fastest axis: lanes walk down columns
     ((3, 70, 512), (512,), None),          # the same with several slabs of rows and leading dimensions folded in
+    ((192, 256), (3, 256), (64, 1)),       # blocks along the leading axis, run length 1: stacked column problems
+    ((5, 300, 512), (5, 1, 512), None),    # the same from a batch axis with encodings of its own, several row groups
     ((256, 256), (2, 2), (128, 128)),      # two-dimensional blocks wider than a wave (generic walk, wave pre-reduction)
     ((96, 100), (3, 4), (32, 25)),         # two-dimensional blocks narrower than a wave
     ((32, 512, 14, 14), (512, 1, 1), None),  # short runs, many per tile (LDS table of the tile's runs)
