@@ -155,14 +155,19 @@ __global__ __launch_bounds__(kBlock) void qdq_fwd_generic_kernel(const QdqArgs a
 
 template <typename IO, typename M>
 static void launch_fwd(const Plan& p, const QdqArgs& a, hipStream_t st, bool aligned) {
-    if (cols_layout<IO>(p, aligned) && (p.cl.J / IoTraits<IO>::kVec + kWave - 1) / kWave <= 0x7fffffff) {
+    const int lane_elems = cols_lane_elems(IoTraits<IO>::kDtype, p, aligned);
+    if (lane_elems > 0) {
         // About as many workgroups as the chip holds at once (256 CUs; the 16-bit kernels run four waves per SIMD,
         // the float32 ones eight): every wave prepares its encodings before its first row, and a second round of
         // waves pays that set-up while the memory pipes drain (8192 x 4096 bf16: 25.5 us with 1024 workgroups,
         // 28.7 us with 3072, 32.3 us with 384; float32: 44.3 us with 8192, 45.6 us with 4096 or 16384).
         constexpr int V = IoTraits<IO>::kVec;
-        hipLaunchKernelGGL((qdq_fwd_cols_kernel<IO, V, M, kFwdColWaves>), (cols_grid<IO, V>(p, V > 4 ? 1024 : 8192, kFwdColWaves)),
-                           dim3(kFwdColWaves * kWave), 0, st, a);
+        if (lane_elems == V)
+            hipLaunchKernelGGL((qdq_fwd_cols_kernel<IO, V, M, kFwdColWaves>), (cols_grid<V>(p, V > 4 ? 1024 : 8192, kFwdColWaves)),
+                               dim3(kFwdColWaves * kWave), 0, st, a);
+        else
+            hipLaunchKernelGGL((qdq_fwd_cols_kernel<IO, 1, M, kFwdColWaves>), (cols_grid<1>(p, 8192, kFwdColWaves)),
+                               dim3(kFwdColWaves * kWave), 0, st, a);
         return;
     }
     if (p.cl.kind == kGeneric) {

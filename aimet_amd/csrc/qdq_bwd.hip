@@ -594,38 +594,30 @@ __global__ void finish_atomic_kernel(const double* acc, float* gscale, float* go
 }
 
 
-// the column-walking backward kernel takes run length 1 whatever reduction the plan would otherwise use for it
-template <typename IO>
-static bool bwd_cols_layout(const Plan& p, bool aligned) {
-    return cols_layout<IO>(p, aligned) && (p.red == kRedAtomic || p.red == kRedRuns || p.red == kRedNone);
+// Elements per lane of the column-walking backward kernel, 0 where it does not apply.  It takes run length 1 whatever
+// reduction the plan would otherwise use for it.  On a 16-bit tensor a lane takes four encodings (8-byte vectors), not
+// eight: with eight, the encodings, the two rows of two tensors and the temporaries of the split form need about 170
+// registers, two or three waves per SIMD (8192 x 4096 bf16 with learned encodings: 47.6 us against 42 us, same tensors
+// every launch).
+static int bwd_cols_lane_elems(int io_dtype, const Plan& p, bool aligned) {
+    if (!(p.red == kRedAtomic || p.red == kRedRuns || p.red == kRedNone)) return 0;
+    const int n = cols_lane_elems(io_dtype, p, aligned);
+    return n > 4 ? 4 : n;
 }
 
-static bool bwd_cols_layout(int io_dtype, const Plan& p, bool aligned) {
-    return io_dtype == AHQ_F32 ? bwd_cols_layout<float>(p, aligned) : bwd_cols_layout<f16_t>(p, aligned);
-}
-
-// On a 16-bit tensor a lane of the backward kernel takes four encodings (8-byte vectors), not eight: with eight, the
-// encodings, the two rows of two tensors and the temporaries of the split form need about 170 registers, two or three
-// waves per SIMD (8192 x 4096 bf16 with learned encodings: 47.6 us against 42 us, same tensors every launch).
 // Workgroups of eight waves, about as many as the chip holds at once, for the reason given at the forward launch
 // (bf16: 42.0 us with 1024 workgroups, 45.0 us with 2048; float32: 72.8 us with 256, 74.9 us with 512, 75.9 us with 1024).
 constexpr int kBwdColWaves = 8;
-template <typename IO>
-constexpr int bwd_cols_vec() { return IoTraits<IO>::kVec > 4 ? 4 : IoTraits<IO>::kVec; }
-
-template <typename IO>
-static dim3 bwd_cols_grid(const Plan& p) {
-    return cols_grid<IO, bwd_cols_vec<IO>()>(p, IoTraits<IO>::kVec > 4 ? 1024 : 256, kBwdColWaves);
-}
-
-static unsigned bwd_cols_row_groups(int io_dtype, const Plan& p) {
-    return io_dtype == AHQ_F32 ? bwd_cols_grid<float>(p).y : bwd_cols_grid<f16_t>(p).y;
+static dim3 bwd_cols_grid(int io_dtype, const Plan& p, int lane_elems) {
+    const int64_t target = io_dtype == AHQ_F32 ? 256 : 1024;
+    return lane_elems == 4 ? cols_grid<4>(p, target, kBwdColWaves) : cols_grid<1>(p, target, kBwdColWaves);
 }
 
 // pairs of doubles the backward pass needs as scratch for its parameter gradients
 static size_t bwd_scratch_pairs(int io_dtype, const Plan& p, bool aligned, bool want_pg) {
     if (!want_pg) return 0;
-    if (bwd_cols_layout(io_dtype, p, aligned)) return (size_t)p.cl.A * (size_t)bwd_cols_row_groups(io_dtype, p) * (size_t)p.cl.J;
+    const int lane_elems = bwd_cols_lane_elems(io_dtype, p, aligned);
+    if (lane_elems > 0) return (size_t)p.cl.A * (size_t)bwd_cols_grid(io_dtype, p, lane_elems).y * (size_t)p.cl.J;
     return p.ws_elems;
 }
 
@@ -647,14 +639,20 @@ static void launch_bwd_red(const Plan& p, const QdqArgs& a, hipStream_t st) {
 
 template <typename IO, typename M>
 static void launch_bwd(const Plan& p, const QdqArgs& a, hipStream_t st, bool aligned) {
-    if (bwd_cols_layout<IO>(p, aligned)) {
-        // few row groups: every workgroup ends with one row of partial sums
-        constexpr int W = kBwdColWaves, V = bwd_cols_vec<IO>();
-        dim3 g = bwd_cols_grid<IO>(p);
+    const int lane_elems = bwd_cols_lane_elems(IoTraits<IO>::kDtype, p, aligned);
+    if (lane_elems > 0) {
+        constexpr int W = kBwdColWaves;
+        dim3 g = bwd_cols_grid(IoTraits<IO>::kDtype, p, lane_elems);
         // arithmetic without a division and no sums to keep: few registers, eight waves per SIMD, so the chip holds
         // more workgroups at once (8192 x 4096 fp32: 70.3 us against 81.8 us)
-        if (!M::kDiv && !a.partials) g = cols_grid<IO, V>(p, IoTraits<IO>::kVec > 4 ? 2048 : 1024, W);
-        hipLaunchKernelGGL((qdq_bwd_cols_kernel<IO, V, M, W>), g, dim3(W * kWave), 0, st, a);
+        const int64_t light = IoTraits<IO>::kVec > 4 ? 2048 : 1024;
+        if (lane_elems == 4) {
+            if (!M::kDiv && !a.partials) g = cols_grid<4>(p, light, W);
+            hipLaunchKernelGGL((qdq_bwd_cols_kernel<IO, 4, M, W>), g, dim3(W * kWave), 0, st, a);
+        } else {
+            if (!M::kDiv && !a.partials) g = cols_grid<1>(p, light, W);
+            hipLaunchKernelGGL((qdq_bwd_cols_kernel<IO, 1, M, W>), g, dim3(W * kWave), 0, st, a);
+        }
         return;
     }
     if (p.cl.kind == kGeneric) {
@@ -717,7 +715,8 @@ extern "C" int ahq_qdq_backward(const ahq_grid* grid, const ahq_layout* layout, 
     if (p.cl.numel == 0) return AHQ_OK;  // nothing to read: outputs are left untouched
     if (!x || !g) return set_error("x or g is null"), AHQ_ERR_INVALID;
     if (!gx && !want_pg) return AHQ_OK;
-    const bool cols = bwd_cols_layout(grid->io_dtype, p, al);
+    const int col_lane_elems = bwd_cols_lane_elems(grid->io_dtype, p, al);
+    const bool cols = col_lane_elems > 0;
     const size_t ws_need = bwd_scratch_pairs(grid->io_dtype, p, al, want_pg) * 2 * sizeof(double);
     if (ws_need > 0 && (!workspace || workspace_bytes < ws_need)) return set_error("workspace too small"), AHQ_ERR_WORKSPACE;
     if (ws_need > 0 && !aligned16(workspace)) return set_error("workspace must be 16-byte aligned"), AHQ_ERR_INVALID;
@@ -750,7 +749,7 @@ extern "C" int ahq_qdq_backward(const ahq_grid* grid, const ahq_layout* layout, 
         hipLaunchKernelGGL(finish_atomic_kernel, dim3((unsigned)((n + 255) / 256 > 1024 ? 1024 : (n + 255) / 256)), dim3(256), 0, st,
                            (const double*)a.partials, gscale, goffset, n, (int)grid->compute_dtype);
     }
-    const int64_t col_groups = cols ? (int64_t)bwd_cols_row_groups(grid->io_dtype, p) : 0;
+    const int64_t col_groups = cols ? (int64_t)bwd_cols_grid(grid->io_dtype, p, col_lane_elems).y : 0;
     if (want_pg && ((cols && col_groups > 1) || (!cols && p.red == kRedRuns && p.cl.I > 1))) {
         // one slot per (row group, encoding) or per run: added up per encoding in a fixed order (the column kernel
         // with a single row group has stored the sums itself)

@@ -695,21 +695,11 @@ static bool validate_grid(const ahq_grid* g, bool backward) {
         default: { using IO = bf16_t; CALL; } break;                    \
     }
 
-// Run length 1 over several rows, whole 16-byte vectors per row: the column-walking kernels apply.
-template <typename IO>
-static bool cols_layout(const Plan& p, bool aligned) {
-    constexpr int V = IoTraits<IO>::kVec;
-    // at least half a wave of lanes must own columns, or the tiled kernel's full waves win
-    // (stacked columns, A > 1, are A such problems side by side: the grid's z axis)
-    const bool form = p.cl.kind == kIJK || (p.cl.kind == kGeneric && p.cl.A > 1 && p.cl.A <= 65535);
-    return aligned && form && p.cl.K == 1 && p.cl.I > 1 && p.cl.J % V == 0 && p.cl.J / V >= kWave / 2;
-}
-
 // grid of the column-walking kernels: x over groups of 64 lanes x VEC encodings, y over row groups, z over stacked
 // problems; about `target` workgroups, every wave with at least one step of rows
-template <typename IO, int V = IoTraits<IO>::kVec>
+template <int V>
 static dim3 cols_grid(const Plan& p, int64_t target, int waves) {
-    const int64_t gx = (p.cl.J / V + kWave - 1) / kWave;
+    const int64_t gx = ((p.cl.J + V - 1) / V + kWave - 1) / kWave;
     const int64_t row_groups = (p.cl.I + (int64_t)waves * kColUnroll - 1) / ((int64_t)waves * kColUnroll);
     int64_t gy = (target + gx * p.cl.A - 1) / (gx * p.cl.A);
     gy = gy < 1 ? 1 : (gy > row_groups ? row_groups : gy);

@@ -747,12 +747,9 @@ static size_t mm_ws_elems(const Plan& p) {
     return p.ws_elems;
 }
 
-// The column-walking kernel applies: run length 1 over several rows, whole 16-byte vectors per row.
-static bool mm_cols_layout(int io_dtype, const Plan& p) {
-    const int V = io_vec(io_dtype);
-    const bool form = p.cl.kind == kIJK || (p.cl.kind == kGeneric && p.cl.A > 1 && p.cl.A <= 65535);  // stacked: z axis
-    return p.ptr_aligned && form && p.red == kRedAtomic && p.cl.K == 1 && p.cl.I > 1 && p.cl.J % V == 0 &&
-           p.cl.J / V >= kWave / 2 && (p.cl.J / V + kWave - 1) / kWave <= 0x7fffffff;
+// Elements per lane of the column-walking kernel, 0 where it does not apply.
+static int mm_cols_lane_elems(int io_dtype, const Plan& p) {
+    return p.red == kRedAtomic ? cols_lane_elems(io_dtype, p, p.ptr_aligned) : 0;
 }
 
 // Row groups the column-walking kernel would like (about 256 workgroups of sixteen waves, four waves per SIMD of 256
@@ -761,7 +758,8 @@ static bool mm_cols_layout(int io_dtype, const Plan& p) {
 // is one row of partials (12 bytes per encoding); with less than the preferred size the kernel runs with as many row
 // groups as fit.
 static int64_t mm_cols_row_groups(int io_dtype, const Plan& p) {
-    const int64_t gx = (p.cl.J / io_vec(io_dtype) + kWave - 1) / kWave;
+    const int n = mm_cols_lane_elems(io_dtype, p);
+    const int64_t gx = ((p.cl.J + n - 1) / n + kWave - 1) / kWave;
     const int64_t most = (p.cl.I + kMmColWaves * kMmColUnroll - 1) / (kMmColWaves * kMmColUnroll);
     int64_t gy = (256 + gx * p.cl.A - 1) / (gx * p.cl.A);
     gy = gy > most ? most : gy;
@@ -832,9 +830,11 @@ static void launch_mm(const Plan& p, const MmArgs& a, hipStream_t st, int cols_g
     }
     if (cols_groups > 0) {
         constexpr int V = IoTraits<IO>::kVec;
-        const dim3 g((unsigned)((p.cl.J / V + kWave - 1) / kWave), (unsigned)cols_groups, (unsigned)p.cl.A);
+        const int n = mm_cols_lane_elems(IoTraits<IO>::kDtype, p);
+        const dim3 g((unsigned)(((p.cl.J + n - 1) / n + kWave - 1) / kWave), (unsigned)cols_groups, (unsigned)p.cl.A);
         const int stream_loads = p.cl.numel * (int64_t)sizeof(IO) >= kStreamLoadBytes ? 1 : 0;
-        hipLaunchKernelGGL((minmax_cols_kernel<IO, V, FINITE>), g, dim3(kMmColWaves * kWave), 0, st, a, stream_loads);
+        if (n == V) hipLaunchKernelGGL((minmax_cols_kernel<IO, V, FINITE>), g, dim3(kMmColWaves * kWave), 0, st, a, stream_loads);
+        else hipLaunchKernelGGL((minmax_cols_kernel<IO, 1, FINITE>), g, dim3(kMmColWaves * kWave), 0, st, a, stream_loads);
         if (cols_groups > 1)
             hipLaunchKernelGGL((minmax_cols_finish_kernel<IO>), dim3((unsigned)((p.cl.J + kWave - 1) / kWave), (unsigned)p.cl.A),
                            dim3(kMmColFinishWaves * kWave), 0, st, a, cols_groups);
@@ -918,7 +918,7 @@ extern "C" size_t ahq_minmax_workspace_bytes(const ahq_layout* layout) {
             Plan p;
             if (!make_plan(dt, *layout, al != 0, true, &p)) continue;
             size_t n = mm_ws_elems(p) * 12;
-            if (mm_cols_layout(dt, p)) n = (size_t)p.cl.A * (size_t)mm_cols_row_groups(dt, p) * (size_t)p.cl.J * 12;  // the preferred size
+            if (mm_cols_lane_elems(dt, p) > 0) n = (size_t)p.cl.A * (size_t)mm_cols_row_groups(dt, p) * (size_t)p.cl.J * 12;  // the preferred size
             if (n > need) need = n;
         }
     return need;
@@ -952,7 +952,7 @@ static int minmax_impl(int32_t dtype, const ahq_layout* layout, const void* x, v
     int cols_groups = 0;  // > 0: the column-walking kernel with that many row groups
     if (uses_ws) {
         size_t slots = ws_elems;
-        if (mm_cols_layout(dtype, p)) {
+        if (mm_cols_lane_elems(dtype, p) > 0) {
             const int64_t fit = (int64_t)(workspace_bytes / ((size_t)p.cl.A * (size_t)p.cl.J * 12));
             const int64_t want = mm_cols_row_groups(dtype, p);
             cols_groups = (int)(fit < want ? fit : want);

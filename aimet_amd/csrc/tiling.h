@@ -200,6 +200,19 @@ inline bool make_plan(int io_dtype, const ahq_layout& layout, bool ptr_aligned, 
     return true;
 }
 
+// Elements a lane of the column-walking kernels owns per row of this layout: a 16-byte vector where the rows allow
+// it, one element where they do not (row length no multiple of the vector, tensors off 16-byte alignment), 0 where
+// those kernels do not apply (run length above 1, a single row, fewer than half a wave of columns: there the tiled
+// kernel's full waves win).  Stacked columns (A > 1) are A such problems side by side, the grid's z axis.
+inline int cols_lane_elems(int io_dtype, const Plan& p, bool aligned) {
+    const CanonLayout& c = p.cl;
+    const bool form = c.kind == kIJK || (c.kind == kGeneric && c.A > 1 && c.A <= 65535);
+    if (!form || c.K != 1 || c.I <= 1) return 0;
+    const int V = io_vec(io_dtype);
+    if (aligned && c.J % V == 0 && c.J / V >= kWave / 2 && (c.J / V + kWave - 1) / kWave <= 0x7fffffff) return V;
+    return (c.J >= kWave / 2 && (c.J + kWave - 1) / kWave <= 0x7fffffff) ? 1 : 0;
+}
+
 inline void fill_geom(const Plan& p, Geom* g) {
     const CanonLayout& c = p.cl;
     g->numel = c.numel;

@@ -27,6 +27,7 @@ CASES = [
     ((3, 5), (3, 5), None),
     ((200, 2056), (2056,), None),          # one encoding per element of the fastest axis: lanes walk down columns
     ((3, 70, 512), (512,), None),          # the same with several slabs of rows and leading dimensions folded in
+    ((301, 203), (203,), None),            # rows no multiple of a vector: the column walk with one element per lane
     ((192, 256), (3, 256), (64, 1)),       # blocks along the leading axis, run length 1: stacked column problems
     ((5, 300, 512), (5, 1, 512), None),    # the same from a batch axis with encodings of its own, several row groups
     ((256, 256), (2, 2), (128, 128)),      # two-dimensional blocks wider than a wave (generic walk, wave pre-reduction)

@@ -38,6 +38,7 @@ LAYOUTS = [
     ((300, 24), (300, 1), None),           # whole runs per workgroup, one thread adds a run
     ((37, 5, 48), (5, 1), None),           # whole runs per workgroup, each encoding met 37 times
     ((12, 4096), (12, 1), None),           # runs of half a tile and less (16-bit): one wave adds a run
+    ((301, 203), (1, 203), None),          # run length 1, rows no multiple of a vector: one element per lane
     ((192, 256), (3, 256), (64, 1)),       # blocks along the leading axis, run length 1: stacked column problems
     ((5, 70, 512), (5, 1, 512), None),     # the same from a batch axis with encodings of its own
 ]
@@ -513,6 +514,7 @@ def test_offset_and_scale_of_different_shapes_broadcast(device, dtype, case):
     ((1100, 264), (1, 264), None, True),          # column-walking kernel, several row groups
     ((3, 40, 1536), (1536,), None, True),
     ((640, 256), (2, 256), (320, 1), True),       # stacked column problems (blocks along the leading axis)
+    ((700, 203), (1, 203), None, True),           # column-walking kernel, one element per lane (odd row length)
     ((1100, 24), (1, 24), None, False),           # run length 1 without the column kernel: atomics
     ((8, 16), (2, 4), (4, 4), False),             # generic walk: atomics
 ], ids=lambda l: "x".join(map(str, l[0])) + "_" + "x".join(map(str, l[1])))
