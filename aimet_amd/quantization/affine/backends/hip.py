@@ -334,11 +334,14 @@ def _apply(tensor, scale, offset, arith, op, compute_dtype, qmin, qmax, block_si
 # --------------------------------------------------------------------------------------- ATen-arithmetic decision --
 def _offsets_fit_grid(offset: torch.Tensor, qmin: int, qmax: int) -> bool:
     """ATen's per-channel fake-quantize refuses zero points outside [qmin, qmax]; the reference then leaves the fast
-    path (torch_builtins.py:425-429).  Quantizer-made symmetric offsets carry their constant value so that this needs
-    no device read."""
+    path (torch_builtins.py:425-429).  Quantizer-made offsets say so themselves -- symmetric ones carry their constant
+    value, those derived from a min / max pair the grid they were clamped into -- so that this needs no device read
+    (a read is a synchronisation: 78 instead of 43 us for a no-grad forward over 134 MB)."""
     const = getattr(offset, "_ahq_constant", None)
     if const is not None:
         return qmin <= -int(const) <= qmax
+    if getattr(offset, "_ahq_in_grid", None) == (qmin, qmax):
+        return True  # derived from a min / max pair by a formula that ends in clamp(., -qmax, -qmin)
     zp = -offset.detach().to(torch.int32)
     return bool(((zp >= qmin) & (zp <= qmax)).all())
 

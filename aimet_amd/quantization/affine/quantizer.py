@@ -653,6 +653,7 @@ class AffineQuantizerBase(QuantizerBase, _GridMixin):
         """What follows a finalize launch on the host: min / max were written behind torch's back (tell autograd, and
         everyone who keys on the version counters), and the encodings the next forward would derive are at hand."""
         torch.autograd.graph.increment_version((self.min, self.max))
+        self._mark_offset_in_grid(offset)
         enc = AffineEncoding(scale, offset, self.qmin, self.qmax, self._symmetric, self.block_size,
                              self.zero_point_shift, producer=self)
         self.__dict__["_encoding_cache"] = (self._encoding_cache_key(), enc)
@@ -691,8 +692,18 @@ class AffineQuantizerBase(QuantizerBase, _GridMixin):
             offset = self._get_offset(scale=scale, dtype=torch.float32)
         if scale is None or offset is None:
             return None
+        self._mark_offset_in_grid(offset)
         return AffineEncoding(scale, offset, self.qmin, self.qmax, self.symmetric, self.block_size,
                               self.zero_point_shift, producer=self)
+
+    def _mark_offset_in_grid(self, offset: torch.Tensor) -> None:
+        """An asymmetric offset derived from min / max is clamp(round(min / scale) - qmin, -qmax, -qmin)
+        (_get_offset, and the kernels that compute the same): its zero point lies in [qmin, qmax] by construction,
+        which is what the backend would otherwise read back from the device before it chooses the arithmetic."""
+        if (not self.symmetric and self._is_min_max_quantizer()
+                and type(self)._get_offset is AffineQuantizerBase._get_offset  # pylint: disable=protected-access
+                and getattr(offset, "_ahq_constant", None) is None):
+            offset._ahq_in_grid = (self.qmin, self.qmax)  # pylint: disable=protected-access
 
     @classmethod
     def from_encodings(cls, encodings: AffineEncoding) -> "AffineQuantizerBase":
@@ -1180,6 +1191,7 @@ class QuantizeDequantize(AffineQuantizerBase):
         """What follows the launches of ahq_minmax_calibrate_qdq on the host: min / max were written behind torch's
         back, the encodings the next forward would derive are at hand, and `y` is the quantizer's output."""
         torch.autograd.graph.increment_version((self.min, self.max))
+        self._mark_offset_in_grid(offset)
         enc = AffineEncoding(scale, offset, self.qmin, self.qmax, self._symmetric, self.block_size,
                              self.zero_point_shift, producer=self)
         self.__dict__["_encoding_cache"] = (self._encoding_cache_key(), enc)
@@ -1252,7 +1264,9 @@ class QuantizeDequantize(AffineQuantizerBase):
                     or scale.dtype != f32 or offset.dtype != f32 or scale.shape != plan.enc_shape
                     or offset.shape != plan.enc_shape or not (scale.is_contiguous() and offset.is_contiguous())
                     or scale.device != x.device or offset.device != x.device or scale.requires_grad
-                    or offset.requires_grad or (plan.needs_constant and getattr(offset, "_ahq_constant", None) is None)):
+                    or offset.requires_grad
+                    or (plan.needs_constant and getattr(offset, "_ahq_constant", None) is None
+                        and getattr(offset, "_ahq_in_grid", None) != (enc.qmin, enc.qmax))):
                 if not borrowed:
                     del own["_forward_plan"]
                 return None
@@ -1296,8 +1310,9 @@ class QuantizeDequantize(AffineQuantizerBase):
         aten = needs_constant = False
         if bs is None and zps == 0.0:
             needs_constant = scale.numel() != 1
-            if needs_constant and getattr(offset, "_ahq_constant", None) is None:
-                return  # per-channel with offsets of its own: the choice reads them on every call
+            if (needs_constant and getattr(offset, "_ahq_constant", None) is None
+                    and getattr(offset, "_ahq_in_grid", None) != (qmin, qmax)):
+                return  # per-channel with offsets of unknown range: the choice reads them on every call
             aten = _hip._aten_arithmetic_applies(input, scale, offset, qmin, qmax)  # pylint: disable=protected-access
         if aten:
             arith, cd = _lib.AHQ_ARITH_ATEN, torch.float32

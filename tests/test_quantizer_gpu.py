@@ -672,7 +672,7 @@ STEADY_CASES = {
     "per_tensor_asymmetric": ((3, 64, 96), (), None, dict(bitwidth=16, symmetric=False)),
     "per_tensor_symmetric": ((3, 64, 96), (1,), None, dict(bitwidth=8, symmetric=True)),
     "per_row_symmetric": ((48, 200), (48, 1), None, dict(bitwidth=8, symmetric=True)),
-    "per_row_asymmetric": ((48, 200), (48, 1), None, dict(bitwidth=8, symmetric=False)),   # never planned
+    "per_row_asymmetric": ((48, 200), (48, 1), None, dict(bitwidth=8, symmetric=False)),   # offsets known to be in the grid
     "blocks_4bit": ((48, 256), (48, 4), (1, 64), dict(bitwidth=4, symmetric=True)),
 }
 
@@ -694,7 +694,7 @@ def test_repeated_forward_without_gradients_reuses_the_previous_call(device, mon
     q = QuantizeDequantize(qshape, block_size=block, **kw).to(device)
     with torch.no_grad(), q.compute_encodings():
         q(x)
-    planned = case != "per_row_asymmetric"
+    planned = True
     q.__dict__.pop("_forward_seen", None)  # (the calibration pass has already shown the shape once)
     calls = []
     real = Q.quantize_dequantize
@@ -1333,3 +1333,45 @@ def test_blockwise_encoding_read_as_a_grouped_one(device):
             AffineEncoding(scale, torch.full_like(scale, -3.0), 0, 15, False, (1, 32))._hint_input_shape((3, 128)))
     with pytest.raises(ValueError, match="Only AffineEncoding"):
         GroupedBlockEncoding._from_affine_encoding(object())
+
+
+def test_asymmetric_per_channel_forward_needs_no_device_read(device):
+    """The offsets an asymmetric min/max quantizer derives are clamped into the grid, and say so: the backend takes the
+    ATen arithmetic for a no-grad forward without reading them back (a synchronisation per forward otherwise).  The
+    result is what the reference's fast path gives, bit for bit; offsets of unknown origin are still read."""
+    from aimet_amd.quantization.affine import QuantizeDequantize
+    from aimet_amd.quantization.affine.backends import hip
+
+    g = torch.Generator().manual_seed(5)
+    x = (torch.randn(4, 64, 96, generator=g) * 2 + 0.7)
+    q = QuantizeDequantize((64, 1), 8, symmetric=False).to(device)
+    with q.compute_encodings():
+        q(x.to(device))
+    with torch.no_grad():
+        enc = q.get_encodings()
+    assert getattr(enc.offset, "_ahq_in_grid", None) == (q.qmin, q.qmax)
+    reads = []
+    real = hip._offsets_fit_grid  # pylint: disable=protected-access
+
+    def counting(offset, qmin, qmax):
+        reads.append(getattr(offset, "_ahq_in_grid", None) is None and getattr(offset, "_ahq_constant", None) is None)
+        return real(offset, qmin, qmax)
+
+    hip._offsets_fit_grid = counting  # pylint: disable=protected-access
+    try:
+        with torch.no_grad():
+            y = q(x.to(device))
+            y2 = q(x.to(device))
+            y3 = q(x.to(device))
+    finally:
+        hip._offsets_fit_grid = real  # pylint: disable=protected-access
+    assert not any(reads), "an offset derived from min / max was read back from the device"
+    ref = O.qdq_v1(x, enc.scale.detach().cpu(), enc.offset.detach().cpu(), q.qmin, q.qmax)
+    assert ref is not None
+    for out in (y, y2, y3):
+        assert_same_bits(out.as_subclass(torch.Tensor), ref[0], "no-grad forward")
+    # a plain tensor of offsets is still checked by reading it
+    off = enc.offset.detach().clone()
+    assert getattr(off, "_ahq_in_grid", None) is None
+    assert real(off, q.qmin, q.qmax) is True
+    assert real(off - 1000.0, q.qmin, q.qmax) is False
