@@ -361,3 +361,64 @@ def test_tensors_of_more_than_two_to_the_31_elements(device):
     first = obs.update(x)[0]
     assert float(first.min) == -400.0 and float(first.max) == 300.0
     assert abs(float(first.histogram.double().sum()) - n) <= n * 1e-6  # float32 counts: every bin rounds once
+
+
+# (name, tensor shape, dtype, encoding shape, block size): one encoding per element of the fastest axis, which the
+# column-walking kernels serve -- 16-byte vectors per lane, stacked problems (blocks along the leading axis), and one
+# element per lane where the rows are no multiple of a vector
+COLUMN_CONFIGS = [
+    ("per_column_bf16", (8192, 4096), torch.bfloat16, (1, 4096), None),
+    ("blocks_64x1_bf16", (8192, 4096), torch.bfloat16, (128, 4096), (64, 1)),
+    ("per_column_odd_fp32", (4099, 4099), torch.float32, (1, 4099), None),
+]
+
+
+@pytest.mark.parametrize("cfg", COLUMN_CONFIGS, ids=lambda c: c[0])
+def test_column_layouts_at_full_size(device, cfg):
+    """Min/max against torch's reductions; forward output and input gradient of a sample of rows, and scale / offset
+    gradients of a sample of columns (a column's sums involve no other column), against the oracle."""
+    from aimet_amd.quantization._stats import reduce_min_max
+    from tests.helpers import assert_close_rel
+
+    A = _affine()
+    name, shape, dtype, enc_shape, block = cfg
+    qmin, qmax = -128, 127
+    g = torch.Generator(device=device).manual_seed(3)
+    x = (torch.randn(shape, generator=g, device=device) * torch.linspace(0.5, 2.0, shape[1], device=device)).to(dtype)
+    grad = torch.randn(shape, generator=g, device=device).to(dtype)
+    groups = enc_shape[0]                       # 1, or the number of blocks along the leading axis
+    rows_per_group = shape[0] // groups
+    xv = x.view(groups, rows_per_group, shape[1])
+
+    mn, mx = reduce_min_max(x, enc_shape, block)
+    assert torch.equal(mn, xv.amin(dim=1)) and torch.equal(mx, xv.amax(dim=1))
+
+    # encodings that clip a few per cent of the values, so that every gradient term occurs
+    scale = (torch.maximum(mn.float().abs(), mx.float().abs()) / qmax * 0.6).clamp_min(1e-6)
+    offset = torch.zeros_like(scale)
+    xd = x.clone().requires_grad_(True)
+    sd = scale.clone().requires_grad_(True)
+    od = offset.clone().requires_grad_(True)
+    y = A.quantize_dequantize(xd, sd, od, qmin, qmax, block_size=block)
+    y.backward(grad)
+
+    # rows: a few whole groups, or every 85th row (elementwise results)
+    if groups > 1:
+        gsel = sorted({0, groups // 2, groups - 1})
+        rsel = torch.cat([torch.arange(i * rows_per_group, (i + 1) * rows_per_group) for i in gsel])
+        sub_scale, sub_off, sub_block = scale[gsel].cpu(), offset[gsel].cpu(), block
+    else:
+        rsel = torch.arange(0, shape[0], max(1, shape[0] // 96))
+        sub_scale, sub_off, sub_block = scale.cpu(), offset.cpu(), None
+    ref = O.qdq_v2_forward(x[rsel].cpu(), sub_scale, sub_off, qmin, qmax, sub_block)
+    assert_same_bits(y.detach()[rsel].as_subclass(torch.Tensor), ref.y, f"{name}: output, sample of rows")
+    gx_ref, _, _ = O.qdq_v2_backward(grad[rsel].cpu(), x[rsel].cpu(), sub_scale, sub_off, qmin, qmax, sub_block)
+    assert_same_bits(xd.grad[rsel], gx_ref, f"{name}: input gradient, sample of rows")
+
+    # columns: all rows of 48 columns spread over the width, with their own encodings
+    csel = torch.arange(0, shape[1], max(1, shape[1] // 48))[:48]
+    _, gs_ref, go_ref = O.qdq_v2_backward(grad[:, csel].cpu(), x[:, csel].cpu(), scale[:, csel].cpu(), offset[:, csel].cpu(),
+                                          qmin, qmax, block)
+    assert bool((xd.grad == 0).any()) and bool((od.grad != 0).any())
+    assert_close_rel(sd.grad[:, csel], gs_ref, 4e-5, f"{name}: scale gradient, sample of columns")
+    assert_close_rel(od.grad[:, csel], go_ref, 4e-5, f"{name}: offset gradient, sample of columns")
