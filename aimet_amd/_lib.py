@@ -197,11 +197,13 @@ _SIGNATURES = {
     "ahq_dlq_tfe_encodings_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int32]),
     "ahq_dlq_fp8_qdq": (ctypes.c_int, [ctypes.c_int32, ctypes.POINTER(Layout), _P, _P, _P, ctypes.c_int32, ctypes.c_int32,
                                        ctypes.c_float, _P]),
+    "ahq_float_cast_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int32, ctypes.POINTER(Layout)]),
     "ahq_float_qdq": (ctypes.c_int, [ctypes.c_int32, ctypes.POINTER(Layout), _P, _P, _P, ctypes.c_int32, ctypes.c_int32,
-                                     ctypes.c_float, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32, _P]),
+                                     ctypes.c_float, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32, _P, ctypes.c_size_t,
+                                     _P]),
     "ahq_float_quantize": (ctypes.c_int, [ctypes.c_int32, ctypes.POINTER(Layout), _P, _P, _P, ctypes.c_int32,
                                           ctypes.c_int32, ctypes.c_float, ctypes.c_int32, ctypes.c_int32,
-                                          ctypes.c_int32, _P]),
+                                          ctypes.c_int32, _P, ctypes.c_size_t, _P]),
     "ahq_float_dequantize": (ctypes.c_int, [ctypes.c_int32, ctypes.POINTER(Layout), _P, _P, _P, _P]),
     "ahq_diag_read": (ctypes.c_int, [_P, ctypes.c_size_t, ctypes.c_int32, ctypes.c_int32, _P, _P]),
     "ahq_diag_copy": (ctypes.c_int, [_P, _P, ctypes.c_size_t, ctypes.c_int32, _P]),

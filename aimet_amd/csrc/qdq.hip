@@ -1,6 +1,8 @@
 // Fake-quantization forward kernels: quantize-dequantize / quantize / dequantize, the LPBQ forward that derives its
 // block scales in the launch, the DlQuantization and float fake-casts (arithmetic and arguments: qdq_common.h).
 
+#include <atomic>
+
 #include "qdq_common.h"
 
 namespace ahq {
@@ -356,9 +358,107 @@ extern "C" int ahq_dlq_fp8_qdq_per_tensor(int32_t dtype, const void* x, void* y,
     return check_launch("ahq_dlq_fp8_qdq_per_tensor");
 }
 
+// ----------------------------------------------------------------------- float fake-cast of 16-bit tensors by table --
+// With one encoding the result is a function of the element's 16 bits alone, and the cast is arithmetic-bound on
+// 16-bit tensors (eight elements per 16 bytes, a logarithm, an exponential and a dozen roundings each: 71 to 117 us
+// for 134 MB where the memory system needs 43).  So the function is tabulated first -- one launch evaluates
+// MathFloatCast::fwd, the very code of the elementwise kernel, on all 65536 bit patterns and leaves the 128 KB table in
+// the caller's workspace -- and the tensor is then streamed through a copy of the table in LDS: a 16-byte load, eight
+// two-byte LDS reads, a 16-byte store.
+namespace ahq {
+constexpr int kCastTableEntries = 65536;
+constexpr size_t kCastTableBytes = (size_t)kCastTableEntries * 2;
+constexpr int64_t kCastTableMinNumel = (int64_t)1 << 22;  // below that the two extra launches cost more than they save
+constexpr int kCastTableThreads = 1024;
+constexpr int kCastTableUnroll = 2;
+
+template <typename IO, int CD>
+__global__ __launch_bounds__(256) void float_cast_table_kernel(const QdqArgs a, uint16_t* __restrict__ table) {
+    using M = MathFloatCast<CD>;
+    const int p = blockIdx.x * 256 + threadIdx.x;
+    if (p >= kCastTableEntries) return;
+    const EncP e = M::prep(a.scale[0], 0.f, 0.f, 0.f, a.gc);
+    IO in;
+    in.bits = (uint16_t)p;
+    bool inr;
+    const IO out = store_rounded<IO, CD>(M::template fwd<false>(load_f32(in), e, a.gc, inr));
+    table[p] = out.bits;
+}
+
+template <typename IO>
+__global__ __launch_bounds__(kCastTableThreads) void float_cast_lookup_kernel(const IO* __restrict__ x, IO* __restrict__ y,
+                                                                              int64_t numel, const uint16_t* __restrict__ table) {
+    extern __shared__ uint16_t lut[];
+    {
+        // 128 KB / 1024 threads: eight 16-byte vectors each, neighbouring threads neighbouring vectors
+        const Pack<uint16_t, 8>* src = reinterpret_cast<const Pack<uint16_t, 8>*>(table);
+        Pack<uint16_t, 8>* dst = reinterpret_cast<Pack<uint16_t, 8>*>(lut);
+#pragma unroll
+        for (int i = 0; i < kCastTableEntries / 8 / kCastTableThreads; ++i) dst[i * kCastTableThreads + threadIdx.x] = src[i * kCastTableThreads + threadIdx.x];
+    }
+    __syncthreads();
+    const int64_t nvec = numel / 8;
+    const int64_t stride = (int64_t)gridDim.x * kCastTableThreads * kCastTableUnroll;
+    for (int64_t v0 = (int64_t)blockIdx.x * kCastTableThreads * kCastTableUnroll + threadIdx.x; v0 < nvec; v0 += stride) {
+        Pack<IO, 8> in[kCastTableUnroll];
+#pragma unroll
+        for (int u = 0; u < kCastTableUnroll; ++u)
+            if (v0 + u * kCastTableThreads < nvec) in[u] = load_pack_stream<IO, 8>(x + (v0 + u * kCastTableThreads) * 8);
+#pragma unroll
+        for (int u = 0; u < kCastTableUnroll; ++u) {
+            if (v0 + u * kCastTableThreads >= nvec) continue;
+            Pack<IO, 8> out;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) out.v[k].bits = lut[in[u].v[k].bits];
+            store_pack_stream<IO, 8>(y + (v0 + u * kCastTableThreads) * 8, out);
+        }
+    }
+    // the elements behind the last whole vector, straight from the table in memory
+    if (blockIdx.x == 0 && threadIdx.x < (int)(numel - nvec * 8)) {
+        const int64_t i = nvec * 8 + threadIdx.x;
+        IO out;
+        out.bits = table[x[i].bits];
+        y[i] = out;
+    }
+}
+
+// The lookup kernel's 128 KB of dynamic LDS are more than a kernel gets by default: asked for once per device and
+// dtype; false when the runtime refuses (the elementwise kernel then does the work).
+static bool cast_table_lds_available(int dtype) {
+    constexpr int kMaxDevices = 64;
+    static std::atomic<int> state[kMaxDevices][2];  // 0 not asked yet, 1 granted, 2 refused
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return false;
+    std::atomic<int>& st = state[dev][dtype == AHQ_F16 ? 0 : 1];
+    int v = st.load(std::memory_order_acquire);
+    if (v == 0) {
+        const void* k = dtype == AHQ_F16 ? reinterpret_cast<const void*>(&float_cast_lookup_kernel<f16_t>)
+                                         : reinterpret_cast<const void*>(&float_cast_lookup_kernel<bf16_t>);
+        const bool ok = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kCastTableBytes) == hipSuccess;
+        if (!ok) (void)hipGetLastError();  // the refusal is handled here, not reported by the next launch check
+        v = ok ? 1 : 2;
+        st.store(v, std::memory_order_release);
+    }
+    return v == 1;
+}
+
+// the table applies: a 16-bit tensor, dense and 16-byte aligned, one encoding, enough elements
+static bool cast_table_applies(int dtype, const Plan& p) {
+    return dtype != AHQ_F32 && p.cl.kind == kIJK && p.cl.J == 1 && p.cl.numel >= kCastTableMinNumel;
+}
+}  // namespace ahq
+
+extern "C" size_t ahq_float_cast_workspace_bytes(int32_t dtype, const ahq_layout* layout) {
+    if (dtype < AHQ_F32 || dtype > AHQ_BF16 || !layout) return 0;
+    Plan p;
+    if (!make_plan(dtype, *layout, true, false, &p, kFwdUnroll)) return 0;
+    return cast_table_applies(dtype, p) ? kCastTableBytes : 0;
+}
+
 static int float_cast_impl(const char* what, int stage_flags, int32_t dtype, const ahq_layout* layout, const void* x,
                            void* y, const float* scale, int32_t mantissa_bits, int32_t exponent_min, float max_value,
-                           int32_t overflow_to_nan, int32_t unsigned_zero, int32_t logarithm_form, void* stream) {
+                           int32_t overflow_to_nan, int32_t unsigned_zero, int32_t logarithm_form, void* workspace,
+                           size_t workspace_bytes, void* stream) {
     if (dtype < AHQ_F32 || dtype > AHQ_BF16) return set_error("bad dtype"), AHQ_ERR_INVALID;
     if (!layout) return set_error("layout is null"), AHQ_ERR_INVALID;
     if (!scale) return set_error("scale is null"), AHQ_ERR_INVALID;
@@ -383,6 +483,25 @@ static int float_cast_impl(const char* what, int stage_flags, int32_t dtype, con
     a.gc.flags = (overflow_to_nan ? kCastOverflowNaN : 0) | (unsigned_zero ? kCastUnsignedZero : 0) |
                  (logarithm_form ? kCastLogForm : 0) | stage_flags;
     hipStream_t st = static_cast<hipStream_t>(stream);
+    if (workspace && workspace_bytes >= kCastTableBytes && aligned16(workspace) && aligned16(x) && aligned16(y) &&
+        cast_table_applies(dtype, p) && cast_table_lds_available(dtype)) {
+        uint16_t* table = static_cast<uint16_t*>(workspace);
+        const dim3 tg(kCastTableEntries / 256), tb(256);
+        // one workgroup per compute unit and 128 KB of LDS each; fewer for tensors that would leave them idle
+        const int64_t nvec = p.cl.numel / 8;
+        int64_t nb = (nvec + (int64_t)kCastTableThreads * kCastTableUnroll - 1) / ((int64_t)kCastTableThreads * kCastTableUnroll);
+        nb = nb < 1 ? 1 : (nb > 256 ? 256 : nb);
+        if (dtype == AHQ_F16) {
+            hipLaunchKernelGGL((float_cast_table_kernel<f16_t, AHQ_F16>), tg, tb, 0, st, a, table);
+            hipLaunchKernelGGL((float_cast_lookup_kernel<f16_t>), dim3((unsigned)nb), dim3(kCastTableThreads), kCastTableBytes, st,
+                               static_cast<const f16_t*>(x), static_cast<f16_t*>(y), p.cl.numel, (const uint16_t*)table);
+        } else {
+            hipLaunchKernelGGL((float_cast_table_kernel<bf16_t, AHQ_BF16>), tg, tb, 0, st, a, table);
+            hipLaunchKernelGGL((float_cast_lookup_kernel<bf16_t>), dim3((unsigned)nb), dim3(kCastTableThreads), kCastTableBytes, st,
+                               static_cast<const bf16_t*>(x), static_cast<bf16_t*>(y), p.cl.numel, (const uint16_t*)table);
+        }
+        return check_launch(what);
+    }
     if (dtype == AHQ_F32) launch_fwd<float, MathFloatCast<AHQ_F32>>(p, a, st, aligned16(x) && aligned16(y));
     else if (dtype == AHQ_F16) launch_fwd<f16_t, MathFloatCast<AHQ_F16>>(p, a, st, aligned16(x) && aligned16(y));
     else launch_fwd<bf16_t, MathFloatCast<AHQ_BF16>>(p, a, st, aligned16(x) && aligned16(y));
@@ -391,21 +510,23 @@ static int float_cast_impl(const char* what, int stage_flags, int32_t dtype, con
 
 extern "C" int ahq_float_qdq(int32_t dtype, const ahq_layout* layout, const void* x, void* y, const float* scale,
                              int32_t mantissa_bits, int32_t exponent_min, float max_value, int32_t overflow_to_nan,
-                             int32_t unsigned_zero, int32_t logarithm_form, void* stream) {
+                             int32_t unsigned_zero, int32_t logarithm_form, void* workspace, size_t workspace_bytes,
+                             void* stream) {
     return float_cast_impl("ahq_float_qdq", 0, dtype, layout, x, y, scale, mantissa_bits, exponent_min, max_value,
-                           overflow_to_nan, unsigned_zero, logarithm_form, stream);
+                           overflow_to_nan, unsigned_zero, logarithm_form, workspace, workspace_bytes, stream);
 }
 
 extern "C" int ahq_float_quantize(int32_t dtype, const ahq_layout* layout, const void* x, void* y, const float* scale,
                                   int32_t mantissa_bits, int32_t exponent_min, float max_value,
                                   int32_t overflow_to_nan, int32_t unsigned_zero, int32_t logarithm_form,
-                                  void* stream) {
+                                  void* workspace, size_t workspace_bytes, void* stream) {
     return float_cast_impl("ahq_float_quantize", kCastKeepScaled, dtype, layout, x, y, scale, mantissa_bits,
-                           exponent_min, max_value, overflow_to_nan, unsigned_zero, logarithm_form, stream);
+                           exponent_min, max_value, overflow_to_nan, unsigned_zero, logarithm_form, workspace,
+                           workspace_bytes, stream);
 }
 
 extern "C" int ahq_float_dequantize(int32_t dtype, const ahq_layout* layout, const void* x, void* y,
                                     const float* scale, void* stream) {
     return float_cast_impl("ahq_float_dequantize", kCastRescaleOnly, dtype, layout, x, y, scale, 0, 0, 1.f, 0, 0, 0,
-                           stream);
+                           nullptr, 0, stream);
 }

@@ -31,6 +31,18 @@ __all__ = ["FloatQuantizeDequantize", "QuantizeDequantize", "float_quantize_dequ
            "float_dequantize"]
 
 
+_TABLE_BYTES = {}
+
+
+def _table_bytes(dtype_code: int, layout) -> int:
+    """ahq_float_cast_workspace_bytes, asked once per (dtype, layout object): layouts are cached by shape."""
+    key = (dtype_code, id(layout))
+    held = _TABLE_BYTES.get(key)
+    if held is None or held[0] is not layout:
+        held = _TABLE_BYTES[key] = (layout, int(_lib.load().ahq_float_cast_workspace_bytes(dtype_code, layout)))
+    return held[1]
+
+
 def _launch(x: torch.Tensor, finfo: _finfo, scale: torch.Tensor, block_size, entry: str = "ahq_float_qdq") -> torch.Tensor:
     lib = _lib.load()
     x, layout = _hip._prepare(x, scale.shape, block_size)  # pylint: disable=protected-access
@@ -41,8 +53,13 @@ def _launch(x: torch.Tensor, finfo: _finfo, scale: torch.Tensor, block_size, ent
         # a format without a storage type goes through the reference's logarithm formula, whose steps round to the
         # tensor's dtype: on 16-bit tensors that differs from an exact cast next to binade boundaries
         log_form = finfo.to_torch_dtype() is None and x.dtype != torch.float32
+        # large 16-bit tensors with one encoding go through a table of the cast's 65536 values, which lives in a
+        # workspace (0 bytes: the table does not apply)
+        nbytes = _table_bytes(_lib.DTYPE_CODE[x.dtype], layout) if scale.numel() == 1 else 0
+        ws = _hip._workspace(nbytes, x.device) if nbytes else None  # pylint: disable=protected-access
         _lib.check(getattr(lib, entry)(_lib.DTYPE_CODE[x.dtype], layout, x.data_ptr(), y.data_ptr(), s.data_ptr(), mbits,
                                        emin, mx, int(overflow_nan), int(uz), int(log_form),
+                                       ws.data_ptr() if ws is not None else None, nbytes,
                                        _lib.current_stream(x.device)),
                    entry)
     return y
@@ -250,11 +267,24 @@ class FloatQuantizeDequantize(QuantizerBase):  # pylint: disable=abstract-method
         return torch.log2(self.maxval.abs().double()) - math.log2(self._finfo.max)
 
     def get_encodings(self) -> Optional[FloatEncoding]:
-        if self.is_initialized():
-            fi = self._finfo
-            return FloatEncoding(fi.mantissa_bits, fi.exponent_bits, fi.finite, fi.unsigned_zero, self.get_scale(),
-                                 block_size=self.block_size, producer=self)
-        return None
+        if not self.is_initialized():
+            return None
+        fi = self._finfo
+        mv = self.maxval
+        # the scale is six small launches' worth of arithmetic on maxval: derived once per value of maxval unless a
+        # gradient has to flow through the derivation (the key follows the tensor object, its version and its memory)
+        reuse = (type(self).get_scale is FloatQuantizeDequantize.get_scale and isinstance(mv, torch.Tensor)
+                 and not (torch.is_grad_enabled() and mv.requires_grad))
+        if reuse:
+            key = (id(mv), mv._version, mv.data_ptr(), tuple(fi), self.block_size)  # pylint: disable=protected-access
+            held = self.__dict__.get("_encoding_cache")
+            if held is not None and held[0] == key:
+                return held[1]
+        enc = FloatEncoding(fi.mantissa_bits, fi.exponent_bits, fi.finite, fi.unsigned_zero, self.get_scale(),
+                            block_size=self.block_size, producer=self)
+        if reuse:
+            self.__dict__["_encoding_cache"] = (key, enc)
+        return enc
 
     def _get_dummy_encoding(self) -> FloatEncoding:
         fi = self._finfo

@@ -528,10 +528,16 @@ int ahq_dlq_fp8_qdq_per_tensor(int32_t dtype, const void* x, void* y, uint64_t c
  * round(x / scales) * scales with bias = 1 - exponent_min and every operation rounded to `dtype`: values within one
  * unit of `dtype` below a power of two land on the next binade's grid and a clamp bound that `dtype` rounds upward is
  * returned as it is, as in the reference; overflow_to_nan and unsigned_zero do not apply.
+ * workspace (optional): ahq_float_cast_workspace_bytes() bytes of 16-byte aligned device memory, or null.  With it,
+ * a 16-bit tensor with a single encoding and at least 2^22 elements is cast through a table of the function's value
+ * for each of the 65536 bit patterns (filled by the same arithmetic, so the results are the same bits) instead of
+ * once per element; without it, and for every other tensor, the arithmetic runs per element.  The query returns 0
+ * where the table does not apply.
  */
+size_t ahq_float_cast_workspace_bytes(int32_t dtype, const ahq_layout* layout);
 int ahq_float_qdq(int32_t dtype, const ahq_layout* layout, const void* x, void* y, const float* scale,
                   int32_t mantissa_bits, int32_t exponent_min, float max_value, int32_t overflow_to_nan,
-                  int32_t unsigned_zero, int32_t logarithm_form, void* stream);
+                  int32_t unsigned_zero, int32_t logarithm_form, void* workspace, size_t workspace_bytes, void* stream);
 
 /* Replaces _float_quantize of aimet_torch (aimet_torch/quantization/float/quantizer.py:687-706), which
  * FloatEncoding.quantize calls (aimet_torch/quantization/float/encoding.py:140-152): ahq_float_qdq without its last
@@ -539,7 +545,8 @@ int ahq_float_qdq(int32_t dtype, const ahq_layout* layout, const void* x, void* 
  */
 int ahq_float_quantize(int32_t dtype, const ahq_layout* layout, const void* x, void* y, const float* scale,
                        int32_t mantissa_bits, int32_t exponent_min, float max_value, int32_t overflow_to_nan,
-                       int32_t unsigned_zero, int32_t logarithm_form, void* stream);
+                       int32_t unsigned_zero, int32_t logarithm_form, void* workspace, size_t workspace_bytes,
+                       void* stream);
 
 /* Replaces FloatEncoding.dequantize of aimet_torch (aimet_torch/quantization/float/encoding.py:154-165, a blockwise
  * torch.mul): y = x * scale, the product formed in float and rounded once to `dtype`; scale: one float per encoding

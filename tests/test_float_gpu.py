@@ -56,6 +56,42 @@ def test_every_16bit_value_through_a_format_without_a_storage_type(device, fmt, 
     assert_same_bits(got, want, str(fmt))
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=lambda d: str(d)[6:])
+@pytest.mark.parametrize("name", list(FORMATS))
+@pytest.mark.parametrize("scale", [1.0, 0.7451069355010986, 2.0 ** -70])
+def test_large_16bit_tensors_go_through_a_table_with_the_same_bits(device, name, dtype, scale):
+    """A 16-bit tensor with one encoding and at least 2^22 elements is cast through a table of the cast's value for
+    every bit pattern.  Every pattern, repeated until the tensor is large enough (plus a ragged tail), against the
+    per-element arithmetic on a tensor below the threshold and against the CPU restatement; quantize as well."""
+    from aimet_amd import _lib
+    from aimet_amd.quantization.affine.backends.hip import _prepare
+
+    fmt, _ = FORMATS[name]
+    fi = _finfo(name)
+    if O.float_max(*fmt) > torch.finfo(dtype).max:
+        pytest.skip("the format's largest value does not fit the tensor's dtype")
+    pats = torch.arange(-32768, 32768, dtype=torch.int32).to(torch.int16).view(dtype)
+    big = torch.cat([pats.repeat(65), pats[:4099]]).to(device)          # 4 264 003 elements: table
+    assert _lib.load().ahq_float_cast_workspace_bytes(_lib.DTYPE_CODE[dtype], _prepare(big, (), None)[1]) == 131072
+    assert _lib.load().ahq_float_cast_workspace_bytes(_lib.DTYPE_CODE[dtype], _prepare(pats.to(device), (), None)[1]) == 0
+    sc = torch.tensor(scale, device=device)
+    small = _fq().float_quantize_dequantize(pats.to(device), fi, sc)      # 65 536 elements: per-element arithmetic
+    got = _fq().float_quantize_dequantize(big, fi, sc)
+    assert_same_bits(got[:65536], small, f"{name}: first copy of the patterns")
+    assert_same_bits(got[64 * 65536:65 * 65536], small, f"{name}: last whole copy")
+    assert_same_bits(got[65 * 65536:], small[:4099], f"{name}: tail")
+    assert_same_bits(small, O.float_qdq(pats, torch.tensor(scale), *fmt), f"{name}: against the restatement")
+    from aimet_amd.quantization.float.quantizer import float_quantize
+    q_small = float_quantize(pats.to(device), fi, sc)
+    q_big = float_quantize(big, fi, sc)
+    assert_same_bits(q_big[:65536], q_small, f"{name}: quantize")
+    assert_same_bits(q_big[65 * 65536:], q_small[:4099], f"{name}: quantize, tail")
+    # per-channel scales, a float32 tensor and a tensor off 16-byte alignment keep the per-element arithmetic
+    off = torch.cat([big[:1], big])[1:]
+    assert off.data_ptr() % 16 != 0
+    assert_same_bits(_fq().float_quantize_dequantize(off, fi, sc)[:65536], small, f"{name}: unaligned tensor")
+
+
 # ------------------------------------------------------------------------------------- kernel against the oracle --
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=lambda d: str(d)[6:])
 @pytest.mark.parametrize("name", list(FORMATS))
