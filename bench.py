@@ -53,6 +53,10 @@ MEASURED_TRAFFIC_BYTES = {
     ("c4", "qdq_bwd_kernel"): int((236756.8 + 121856.5) * 1024),
     ("c4", "qdq_fwd_kernel"): int((122033.5 + 114695.3) * 1024),
     ("c4", "qdq_fwd_lpbq_kernel"): int((122082.5 + 118720.7) * 1024),
+    # (profiles/hbm_traffic_pmc__per_column_bf16_8192x4096_column_walking_kernels.txt; the backward launch and its
+    # finish launch)
+    ("cols", "qdq_bwd_kernel"): int((131203.3 + 69632.0 + 4136.5 + 32.0) * 1024),
+    ("cols", "qdq_fwd_kernel"): int((65673.6 + 65537.5) * 1024),
     # the timed update (a batch inside the running range): speculative binning pass (read + write) + the launch that
     # folds its extrema and partial histograms into the running state; a batch that moves the range is read a second
     # time (about a quarter of the batches of the c3 stream)
