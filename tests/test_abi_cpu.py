@@ -127,6 +127,41 @@ def test_workspace_queries_and_planning(lib):
     assert lib.ahq_minmax_calibrate_qdq_workspace_bytes(9, per_tensor) == 0
 
 
+def test_planning_of_the_column_layouts(lib):
+    """Host arithmetic only: one encoding per element of the fastest axis is planned as a column walk with row groups,
+    blocks along the leading axis as that many stacked problems, and the scratch follows."""
+    from aimet_amd import _lib
+
+    g = _lib.Grid()
+    g.arith, g.op, g.io_dtype, g.compute_dtype, g.qmin, g.qmax = _lib.AHQ_ARITH_AUTOGRAD, 0, _lib.AHQ_BF16, _lib.AHQ_BF16, -8, 7
+    per_column = _lib.make_layout([8192, 4096], [8192, 1], [0, 1])
+    # min/max: about 256 workgroups of 64 lanes x 8 columns (16-bit) -> 8 across, 32 row groups of 12-byte triples;
+    # the float32 plan has 16 across and 16 row groups: the larger one is reported
+    assert lib.ahq_minmax_workspace_bytes(per_column) == 32 * 4096 * 12
+    # backward, 16-bit: four columns per lane -> 16 workgroups across, 1024 / 16 = 64 row groups of double pairs
+    assert lib.ahq_qdq_backward_workspace_bytes(g, per_column, 1) == 64 * 4096 * 16
+    assert lib.ahq_qdq_backward_workspace_bytes(g, per_column, 0) == 0
+    # 64 x 1 blocks: 128 stacked problems of 64 rows; 64 rows are one row group in both passes
+    stacked = _lib.make_layout([8192, 4096], [64, 1], [4096, 1])
+    assert lib.ahq_minmax_workspace_bytes(stacked) == 128 * 4096 * 12
+    assert lib.ahq_qdq_backward_workspace_bytes(g, stacked, 1) == 128 * 4096 * 16
+    # the same with a batch axis that has encodings of its own
+    batched = _lib.make_layout([5, 70, 512], [1, 70, 1], [512, 0, 1])
+    assert lib.ahq_minmax_workspace_bytes(batched) >= 5 * 512 * 12
+    # an odd row length: one element per lane, the kernels still apply (scratch per row group and encoding)
+    odd = _lib.make_layout([4099, 4099], [4099, 1], [0, 1])
+    assert lib.ahq_minmax_workspace_bytes(odd) % (4099 * 12) == 0 and lib.ahq_minmax_workspace_bytes(odd) >= 4099 * 12
+    # too few columns for a column walk: one slot per encoding (ordered keys)
+    assert lib.ahq_minmax_workspace_bytes(_lib.make_layout([1100, 24], [1100, 1], [0, 1])) == 24 * 12
+    # float fake-cast by table: 16-bit tensors of 2^22 elements and more with one encoding
+    big, small = _lib.make_layout([1 << 22], [1 << 22], [0]), _lib.make_layout([(1 << 22) - 1], [(1 << 22) - 1], [0])
+    assert lib.ahq_float_cast_workspace_bytes(_lib.AHQ_BF16, big) == 131072
+    assert lib.ahq_float_cast_workspace_bytes(_lib.AHQ_F16, big) == 131072
+    assert lib.ahq_float_cast_workspace_bytes(_lib.AHQ_F32, big) == 0
+    assert lib.ahq_float_cast_workspace_bytes(_lib.AHQ_BF16, small) == 0
+    assert lib.ahq_float_cast_workspace_bytes(_lib.AHQ_BF16, _lib.make_layout([4096, 4096], [1, 4096], [1, 0])) == 0
+
+
 def test_backend_registry():
     import aimet_amd.quantization as Q
     from aimet_amd.quantization.affine.backends import hip
