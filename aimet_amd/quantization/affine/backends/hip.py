@@ -342,8 +342,19 @@ def _offsets_fit_grid(offset: torch.Tensor, qmin: int, qmax: int) -> bool:
         return qmin <= -int(const) <= qmax
     if getattr(offset, "_ahq_in_grid", None) == (qmin, qmax):
         return True  # derived from a min / max pair by a formula that ends in clamp(., -qmax, -qmin)
+    # the answer is kept on the tensor object, for the version of its contents that was read (like autograd, this
+    # follows writes torch knows of; a write through .data or by a foreign kernel into the same memory is not seen)
+    key = (offset._version, offset.data_ptr(), qmin, qmax)  # pylint: disable=protected-access
+    held = getattr(offset, "_ahq_fit_checked", None)
+    if held is not None and held[0] == key:
+        return held[1]
     zp = -offset.detach().to(torch.int32)
-    return bool(((zp >= qmin) & (zp <= qmax)).all())
+    fits = bool(((zp >= qmin) & (zp <= qmax)).all())
+    try:
+        offset._ahq_fit_checked = (key, fits)  # pylint: disable=protected-access
+    except (AttributeError, RuntimeError):
+        pass
+    return fits
 
 
 def _aten_arithmetic_applies(tensor, scale, offset, qmin, qmax) -> bool:

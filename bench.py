@@ -1294,11 +1294,87 @@ def run_model_workload(steps, warmup, dev, with_cpu_baseline=True, batches=8, se
     return out
 
 
+def run_ops_workload(dev):
+    """Not one of the benchmark configurations (run with --workload ops; left out of the default run): the public
+    operations the driver line does not time -- quantize, dequantize, the ATen-arithmetic quantize-dequantize of frozen
+    encodings (per tensor and per channel) and the float fake-cast -- on an [8, 2048, 4096] tensor in the three dtypes,
+    every launch on the next of six tensors (HBM figures: one read + one write of the tensor), each checked against
+    the oracle on a sample of rows."""
+    from aimet_amd.quantization import affine
+    from aimet_amd.quantization.float import FloatQuantizeDequantize
+    from oracle import torch_ref as O
+
+    _ensure_built()
+    t_start = time.perf_counter()
+    records = {}
+    shape = (8, 2048, 4096)
+    for dt in (torch.float32, torch.bfloat16, torch.float16):
+        g = torch.Generator().manual_seed(0)
+        base = torch.randn(shape, generator=g).to(dt)
+        xs = [base.to(dev)] + [base.to(dev).clone() for _ in range(5)]
+        nbytes = base.numel() * base.element_size()
+        turn = [0]
+
+        def nxt():
+            turn[0] = (turn[0] + 1) % len(xs)
+            return xs[turn[0]]
+
+        s0, o0 = torch.tensor(0.02), torch.tensor(-3.0)
+        sc = torch.rand(2048, 1, generator=g) * 0.02 + 0.01
+        oc = torch.zeros(2048, 1)
+        sd, od, scd, ocd = s0.to(dev), o0.to(dev), sc.to(dev), oc.to(dev)
+        codes = affine.quantize(xs[0], sd, od, -128, 127)
+        sample = slice(0, 2048, 256)  # rows 0, 256, ... of every batch entry
+        cases = {
+            "quantize_per_tensor": (lambda: affine.quantize(nxt(), sd, od, -128, 127),
+                                    lambda y: torch.equal(y[:, sample].cpu(), O.quantize_forward(base[:, sample], s0, o0, -128, 127)[0])),
+            "quantize_per_channel": (lambda: affine.quantize(nxt(), scd, ocd, -128, 127),
+                                     lambda y: torch.equal(y[:, sample].cpu(), O.quantize_forward(base[:, sample], sc[sample], oc[sample], -128, 127)[0])),
+            "dequantize_per_tensor": (lambda: affine.dequantize(codes, sd, od),
+                                      lambda y: torch.equal(y[:, sample].cpu(), O.dequantize_forward(codes[:, sample].cpu(), s0, o0))),
+            "qdq_frozen_per_tensor": (lambda: affine.quantize_dequantize(nxt(), sd, od, -128, 127),
+                                      lambda y: torch.equal(y[:, sample].cpu(), O.qdq_v1(base[:, sample], s0, o0, -128, 127)[0])),
+            "qdq_frozen_per_channel": (lambda: affine.quantize_dequantize(nxt(), scd, ocd, -128, 127),
+                                       lambda y: torch.equal(y[:, sample].cpu(), O.qdq_v1(base[:, sample], sc[sample], oc[sample], -128, 127)[0])),
+        }
+        for name, kw, fmt in (("float_cast_e4m3fn", dict(dtype=torch.float8_e4m3fn), (4, 3, True, False)),
+                              ("float_cast_e5m2", dict(dtype=torch.float8_e5m2), (5, 2, False, False)),
+                              ("float_cast_e3m4", dict(exponent_bits=3, mantissa_bits=4), (3, 4, False, False))):
+            fq = FloatQuantizeDequantize(**kw).to(dev)
+            with torch.no_grad(), fq.compute_encodings():
+                fq(xs[0])
+            with torch.no_grad():
+                fscale = fq.get_encodings().scale.detach().cpu()
+            cases[name] = ((lambda fq=fq: fq(nxt())),
+                           (lambda y, fmt=fmt, fscale=fscale: torch.equal(y[:, sample].as_subclass(torch.Tensor).cpu().view(torch.int16 if dt != torch.float32 else torch.int32),
+                                                                          O.float_qdq(base[:, sample], fscale, *fmt).view(torch.int16 if dt != torch.float32 else torch.int32))))
+        rec = {}
+        with torch.no_grad():
+            for name, (fn, check) in cases.items():
+                y = fn()
+                turn[0] = len(xs) - 1  # the checked call ran on xs[0]
+                ok = bool(check(fn().as_subclass(torch.Tensor)))
+                t = event_time(fn, 20)
+                rec[name] = {"us": round(t * 1e6, 2), "GBps": round(2 * nbytes / t / 1e9, 1),
+                             "frac_of_hbm_peak": round(2 * nbytes / t / 1e9 / HBM_PEAK_GBS, 4), "bit_exact_on_sample": ok}
+                del y
+        records[DTYPE_NAME[dt]] = rec
+        del xs, codes
+        torch.cuda.empty_cache()
+    worst = min(r["frac_of_hbm_peak"] for rec in records.values() for r in rec.values())
+    return {"metric": "HBM GB/s of the operations outside the timed step (one read + one write of the tensor)",
+            "unit": "GB/s", "config": {"workload": "ops_8x2048x4096_f32_bf16_f16"}, "data": "synthetic",
+            "operations": records, "lowest_frac_of_hbm_peak": worst,
+            "all_bit_exact_on_sample": all(r["bit_exact_on_sample"] for rec in records.values() for r in rec.values()),
+            "bench_seconds": round(time.perf_counter() - t_start, 1)}
+
+
 RUNNERS = {
     "c1": lambda a, dev, cpu: run_qdq_workload("c1", a.steps, a.warmup, dev, cpu, not a.no_cached),
     "c2": lambda a, dev, cpu: run_qdq_workload("c2", a.steps, a.warmup, dev, cpu, not a.no_cached),
     "c4": lambda a, dev, cpu: run_qdq_workload("c4", a.steps, a.warmup, dev, cpu, not a.no_cached),
     "cols": lambda a, dev, cpu: run_qdq_workload("cols", a.steps, a.warmup, dev, cpu, not a.no_cached),
+    "ops": lambda a, dev, cpu: run_ops_workload(dev),
     "c3": lambda a, dev, cpu: run_hist_workload(min(a.steps, 10), min(a.warmup, 2), dev, cpu),
     "dlq": lambda a, dev, cpu: run_dlq_workload(min(a.steps, 10), min(a.warmup, 2), dev, cpu),
     "c5": lambda a, dev, cpu: run_model_workload(min(a.steps, 3), min(a.warmup, 1), dev, cpu),

@@ -1370,8 +1370,13 @@ def test_asymmetric_per_channel_forward_needs_no_device_read(device):
     assert ref is not None
     for out in (y, y2, y3):
         assert_same_bits(out.as_subclass(torch.Tensor), ref[0], "no-grad forward")
-    # a plain tensor of offsets is still checked by reading it
+    # a plain tensor of offsets is still checked by reading it -- once per version of its contents
     off = enc.offset.detach().clone()
     assert getattr(off, "_ahq_in_grid", None) is None
     assert real(off, q.qmin, q.qmax) is True
     assert real(off - 1000.0, q.qmin, q.qmax) is False
+    assert off._ahq_fit_checked[1] is True  # pylint: disable=protected-access
+    off.sub_(1000.0)  # a tracked write: the kept answer no longer applies
+    assert real(off, q.qmin, q.qmax) is False
+    off.add_(1000.0)
+    assert real(off, q.qmin, q.qmax) is True
