@@ -205,6 +205,8 @@ _SIGNATURES = {
                                           ctypes.c_int32, ctypes.c_float, ctypes.c_int32, ctypes.c_int32,
                                           ctypes.c_int32, _P, ctypes.c_size_t, _P]),
     "ahq_float_dequantize": (ctypes.c_int, [ctypes.c_int32, ctypes.POINTER(Layout), _P, _P, _P, _P]),
+    "ahq_float_qdq_backward": (ctypes.c_int, [ctypes.c_int32, ctypes.POINTER(Layout), _P, _P, _P, _P, ctypes.c_int32,
+                                              ctypes.c_int32, ctypes.c_float, ctypes.c_int32, ctypes.c_int32, _P]),
     "ahq_diag_read": (ctypes.c_int, [_P, ctypes.c_size_t, ctypes.c_int32, ctypes.c_int32, _P, _P]),
     "ahq_diag_copy": (ctypes.c_int, [_P, _P, ctypes.c_size_t, ctypes.c_int32, _P]),
     "ahq_dlq_percentile_encodings": (ctypes.c_int, [ctypes.POINTER(DlqPdfState), ctypes.c_float, ctypes.c_int32,

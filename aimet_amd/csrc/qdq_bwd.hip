@@ -668,9 +668,60 @@ static void launch_bwd(const Plan& p, const QdqArgs& a, hipStream_t st, bool ali
     }
 }
 
+// The input gradient alone (no sums): the kernels of launch_bwd that need no reduction.
+template <typename IO, typename M>
+static void launch_bwd_input_only(const Plan& p, const QdqArgs& a, hipStream_t st, bool aligned) {
+    const int lane_elems = bwd_cols_lane_elems(IoTraits<IO>::kDtype, p, aligned);
+    if (lane_elems > 0) {
+        constexpr int W = kBwdColWaves;
+        const dim3 g = bwd_cols_grid(IoTraits<IO>::kDtype, p, lane_elems);
+        if (lane_elems == 4) hipLaunchKernelGGL((qdq_bwd_cols_kernel<IO, 4, M, W>), g, dim3(W * kWave), 0, st, a);
+        else hipLaunchKernelGGL((qdq_bwd_cols_kernel<IO, 1, M, W>), g, dim3(W * kWave), 0, st, a);
+        return;
+    }
+    if (p.cl.kind == kGeneric) {
+        hipLaunchKernelGGL((qdq_bwd_generic_kernel<IO, M>), dim3(p.nblocks), dim3(kBlock), 0, st, a);
+        return;
+    }
+    launch_bwd_red<IO, M, kRedNone>(p, a, st);
+}
+
 }  // namespace ahq
 
 using namespace ahq;
+
+extern "C" int ahq_float_qdq_backward(int32_t dtype, const ahq_layout* layout, const void* g, const void* x, void* gx,
+                                      const float* scale, int32_t mantissa_bits, int32_t exponent_min, float max_value,
+                                      int32_t overflow_to_nan, int32_t unsigned_zero, void* stream) {
+    if (dtype < AHQ_F32 || dtype > AHQ_BF16) return set_error("bad dtype"), AHQ_ERR_INVALID;
+    if (!layout) return set_error("layout is null"), AHQ_ERR_INVALID;
+    if (!scale) return set_error("scale is null"), AHQ_ERR_INVALID;
+    if (mantissa_bits < 0 || mantissa_bits > 23 || exponent_min < -126 || exponent_min > 127 || !(max_value > 0.f))
+        return set_error("bad float format description"), AHQ_ERR_INVALID;
+    Plan p;
+    const bool al = aligned16(x) && aligned16(g) && aligned16(gx);
+    if (!make_plan(dtype, *layout, al, false, &p, kBwdUnroll, true)) return AHQ_ERR_INVALID;
+    if (p.cl.numel == 0) return AHQ_OK;
+    if (!x || !g || !gx) return set_error("x, g or gx is null"), AHQ_ERR_INVALID;
+    QdqArgs a{};
+    a.x = x;
+    a.g = g;
+    a.gx = gx;
+    a.scale = scale;
+    ahq_grid grid{};
+    grid.io_dtype = dtype;
+    grid.compute_dtype = dtype;
+    fill_args(grid, p, &a);
+    a.gc.qmin = (float)exponent_min;
+    a.gc.qmax = max_value;
+    a.gc.zps = (float)mantissa_bits;
+    a.gc.flags = (overflow_to_nan ? kCastOverflowNaN : 0) | (unsigned_zero ? kCastUnsignedZero : 0);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (dtype == AHQ_F32) launch_bwd_input_only<float, MathFloatCast<AHQ_F32>>(p, a, st, al);
+    else if (dtype == AHQ_F16) launch_bwd_input_only<f16_t, MathFloatCast<AHQ_F16>>(p, a, st, al);
+    else launch_bwd_input_only<bf16_t, MathFloatCast<AHQ_BF16>>(p, a, st, al);
+    return check_launch("ahq_float_qdq_backward");
+}
 
 // The tiling of the backward pass: tiles of one round, of kBwdRounds rounds where a row then is one tile instead of two.
 static bool plan_bwd(int io_dtype, const ahq_layout& layout, bool aligned, bool want_pg, Plan* p) {

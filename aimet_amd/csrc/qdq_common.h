@@ -329,7 +329,7 @@ struct MathFloatCast {
     static constexpr int kCD = CD;
     static constexpr int kNP = 2;
     static constexpr bool kDiv = true;
-    static constexpr bool kHasBwd = false;
+    static constexpr bool kHasBwd = true;  // the input gradient of the exact form (formats with a storage type)
     // The scale stays a float whatever CD is: a float32 scale with one element per tensor is an operand torch keeps
     // at full precision next to a 16-bit tensor (and any larger float32 scale widens the whole computation), so the
     // quotient is the correctly rounded float one, rounded once more to CD.
@@ -362,6 +362,10 @@ struct MathFloatCast {
                 return rnd<CD>(__builtin_rintf(q) * sc) * back;  // last rounding by the caller
             }
         }
+        return rnd<CD>(to_format(t, g)) * back;  // last rounding by the caller
+    }
+    // the conversion to the simulated storage type and back: round to nearest even on its grid, overflow as it does
+    __device__ static float to_format(float t, const GridC& g) {
         int ex = __builtin_amdgcn_frexp_expf(t) - 1;
         ex = ex < (int)g.qmin ? (int)g.qmin : ex;
         const int sh = ex - (int)g.zps;
@@ -369,11 +373,21 @@ struct MathFloatCast {
         if (__builtin_fabsf(v) > g.qmax)
             v = (g.flags & kCastOverflowNaN) ? __builtin_nanf("") : __builtin_copysignf(__builtin_inff(), v);
         if ((g.flags & kCastUnsignedZero) && v == 0.f) v = 0.f;
-        return rnd<CD>(v) * back;  // last rounding by the caller
+        return v;
     }
+    // What autograd derives for the reference's composition with a storage type (float/quantizer.py:687-710:
+    // div, clamp, .to(storage type), .to(dtype), mul), operation by operation and each rounded to CD:
+    //   g * scale  ->  through the two casts backwards, i.e. converted to the storage type and back (the gradient
+    //   is rounded onto the simulated format's grid, and overflows like any other value)  ->  times the clamp's mask
+    //   (bounds included; a NaN quotient is outside)  ->  / scale.
     template <bool FAST>
-    __device__ static void bwd(float, float, const EncP&, const GridC&, float& gx, float& gs, float& goff) {
-        gx = gs = goff = 0.f;
+    __device__ static void bwd(float gr, float x, const EncP& e, const GridC& g, float& gx, float& gs, float& goff) {
+        const float t = rnd<CD>(divide<FAST, AHQ_F32>(x, e.p0, e.rs));
+        const float mx = rnd<CD>(g.qmax);
+        const float c = rnd<CD>(to_format(rnd<CD>(gr * e.p0), g));
+        const float masked = ((t >= -mx) & (t <= mx)) ? c : 0.f;  // clamp's backward selects: +0 outside, whatever c is
+        gx = rnd<CD>(masked / e.p0);  // the gradient's magnitude is not bounded like x: general division
+        gs = goff = 0.f;
     }
 };
 

@@ -539,6 +539,18 @@ int ahq_float_qdq(int32_t dtype, const ahq_layout* layout, const void* x, void* 
                   int32_t mantissa_bits, int32_t exponent_min, float max_value, int32_t overflow_to_nan,
                   int32_t unsigned_zero, int32_t logarithm_form, void* workspace, size_t workspace_bytes, void* stream);
 
+/* The input gradient autograd derives for _float_quantize_dequantize with a format that has a torch storage type
+ * (aimet_torch/quantization/float/quantizer.py:634-710: div, clamp, _cast_decast = .to(storage type).to(dtype), mul),
+ * in one pass: gx = (cast(g * scale) * [ -max_value <= x / scale <= max_value ]) / scale, every operation rounded to
+ * `dtype` as torch's would be.  The backward of the two conversions converts the gradient to the storage type and
+ * back, so the reference's gradient is rounded onto the simulated format's grid (and overflows like any other
+ * value); this is reproduced.  Format arguments as for ahq_float_qdq.  (Formats without a storage type go through the
+ * reference's logarithm formula, whose gradient is zero everywhere: no kernel needed.)
+ */
+int ahq_float_qdq_backward(int32_t dtype, const ahq_layout* layout, const void* g, const void* x, void* gx,
+                           const float* scale, int32_t mantissa_bits, int32_t exponent_min, float max_value,
+                           int32_t overflow_to_nan, int32_t unsigned_zero, void* stream);
+
 /* Replaces _float_quantize of aimet_torch (aimet_torch/quantization/float/quantizer.py:687-706), which
  * FloatEncoding.quantize calls (aimet_torch/quantization/float/encoding.py:140-152): ahq_float_qdq without its last
  * multiplication, y = cast(clamp(x / scale, -max_value, max_value)); same arguments, same arithmetic.

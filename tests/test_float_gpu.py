@@ -175,6 +175,33 @@ def test_input_gradient(device):
     assert_same_bits(xd.grad, xr.grad)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=lambda d: str(d)[6:])
+@pytest.mark.parametrize("name", [n for n, f in FORMATS.items() if f[1] is not None])
+@pytest.mark.parametrize("shape,scale_shape,block", [((4099,), (), None), ((64, 515), (64, 1), None),
+                                                     ((32, 256), (32, 4), (1, 64)), ((300, 256), (1, 256), None)])
+def test_input_gradient_is_what_autograd_derives_for_the_composition(device, name, dtype, shape, scale_shape, block):
+    """The backward of .to(storage type).to(dtype) converts the gradient to the storage type and back, so the
+    reference's input gradient lies on the simulated format's grid: g * scale, rounded to the format, masked by the
+    clamp, divided by the scale.  Arbitrary gradients (not representable in the format, huge, infinite, NaN) against
+    autograd through the CPU restatement, bit for bit."""
+    fmt, _ = FORMATS[name]
+    mx = O.float_max(*fmt)
+    x = _data(shape, dtype, seed=len(name) * 3 + len(shape), span=min(mx, 3e4))
+    g = torch.Generator().manual_seed(31)
+    scale = torch.exp(torch.rand(scale_shape, generator=g) * 6 - 4)
+    grad = _data(shape, dtype, seed=77, span=min(mx, 3e4) * 4)
+    if mx > torch.finfo(torch.result_type(x, scale)).max:
+        pytest.skip("the format's largest value does not fit the computation's dtype")
+    xr = x.clone().requires_grad_(True)
+    y = O.float_qdq(xr, scale, *fmt, block_size=block)
+    y.backward(grad.to(y.dtype))
+    xd = x.to(device).requires_grad_(True)
+    yd = _fq().float_quantize_dequantize(xd, _finfo(name), scale.to(device), block)
+    yd.backward(grad.to(device).to(yd.dtype))
+    assert xd.grad.dtype == xr.grad.dtype
+    assert_same_bits(xd.grad, xr.grad, f"{name}: input gradient")
+
+
 # ------------------------------------------------------------------------- the reference's quantizer scenarios --
 @pytest.fixture()
 def x(device):
