@@ -98,9 +98,10 @@ def float_dequantize(input: torch.Tensor, scale: torch.Tensor, block_size=None) 
 
 
 class _FloatQdqFunction(torch.autograd.Function):
-    """Forward: one kernel.  Backward: what autograd derives for the reference's composition -- the clamp passes the
-    gradient where |x / scale| <= max, the conversion to a storage type and back is an identity for it, and the
-    rounding of the logarithm-based cast (formats without a storage type) has a zero derivative."""
+    """Forward: one kernel.  Backward: what autograd derives for the reference's composition (float/quantizer.py:634-710)
+    -- g * scale, converted to the storage type and back (the backward of the two conversions: the gradient lands on
+    the simulated format's grid), passed by the clamp where |x / scale| <= max, divided by the scale -- in one kernel;
+    the rounding of the logarithm-based cast (formats without a storage type) has a zero derivative."""
 
     @staticmethod
     def forward(ctx, x, scale, finfo, block_size):
